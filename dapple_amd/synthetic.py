@@ -1,0 +1,113 @@
+"""Seeded synthetic inputs, weights and upstream gradients for the stage configs.
+
+Every array comes from ``numpy.random.Generator(PCG64(seed))``: inputs use seed
+1000+config, weights 2000+config, upstream gradients 3000+config, and micro-batch
+``m`` adds ``m`` to the seed, so a CPU checker and the GPU stage see identical
+bits without exchanging files.
+
+Weight keys follow the reference's TF variable scopes
+(bert/models/bert/modeling_slice.py:945-996), so a checkpoint name map applies
+unchanged.
+"""
+import numpy as np
+
+SEED_INPUT = 1000
+SEED_WEIGHT = 2000
+SEED_GRAD = 3000
+
+
+def _rng(seed):
+    return np.random.Generator(np.random.PCG64(seed))
+
+
+# --------------------------------------------------------------------------- BERT
+def bert_layer_shapes(hidden, ffn):
+    """Per-encoder-layer variable shapes, in the reference's scope order."""
+    return [
+        ("attention/self/query/kernel", (hidden, hidden)),
+        ("attention/self/query/bias", (hidden,)),
+        ("attention/self/key/kernel", (hidden, hidden)),
+        ("attention/self/key/bias", (hidden,)),
+        ("attention/self/value/kernel", (hidden, hidden)),
+        ("attention/self/value/bias", (hidden,)),
+        ("attention/output/dense/kernel", (hidden, hidden)),
+        ("attention/output/dense/bias", (hidden,)),
+        ("attention/output/LayerNorm/gamma", (hidden,)),
+        ("attention/output/LayerNorm/beta", (hidden,)),
+        ("intermediate/dense/kernel", (hidden, ffn)),
+        ("intermediate/dense/bias", (ffn,)),
+        ("output/dense/kernel", (ffn, hidden)),
+        ("output/dense/bias", (hidden,)),
+        ("output/LayerNorm/gamma", (hidden,)),
+        ("output/LayerNorm/beta", (hidden,)),
+    ]
+
+
+def bert_embedding_shapes(vocab, hidden, type_vocab, max_pos):
+    return [
+        ("bert/embeddings/word_embeddings", (vocab, hidden)),
+        ("bert/embeddings/token_type_embeddings", (type_vocab, hidden)),
+        ("bert/embeddings/position_embeddings", (max_pos, hidden)),
+        ("bert/embeddings/LayerNorm/gamma", (hidden,)),
+        ("bert/embeddings/LayerNorm/beta", (hidden,)),
+    ]
+
+
+def bert_weights(seed, num_layers, hidden, ffn, first_layer=0, embeddings=None,
+                 stddev=0.02, perturb=False):
+    """N(0, stddev) kernels/tables, zero biases, LayerNorm gamma 1 / beta 0.
+
+    ``perturb=True`` draws biases, gamma and beta at random too, so that a test
+    can tell a dropped bias or a swapped gamma/beta apart from a correct result.
+    ``embeddings`` = (vocab, type_vocab, max_pos) adds the embedding tables.
+    """
+    rng = _rng(seed)
+    w = {}
+
+    def fill(name, shape):
+        if name.endswith("kernel") or name.endswith("embeddings"):
+            w[name] = (rng.standard_normal(shape) * stddev).astype(np.float32)
+        elif name.endswith("gamma"):
+            w[name] = (1.0 + 0.1 * rng.standard_normal(shape)).astype(np.float32) if perturb \
+                else np.ones(shape, np.float32)
+        else:
+            w[name] = (0.1 * rng.standard_normal(shape)).astype(np.float32) if perturb \
+                else np.zeros(shape, np.float32)
+
+    if embeddings is not None:
+        vocab, type_vocab, max_pos = embeddings
+        for name, shape in bert_embedding_shapes(vocab, hidden, type_vocab, max_pos):
+            fill(name, shape)
+    for l in range(first_layer, first_layer + num_layers):
+        for name, shape in bert_layer_shapes(hidden, ffn):
+            fill("bert/encoder/layer_%d/%s" % (l, name), shape)
+    return w
+
+
+def bert_activation_inputs(seed, num_micro_batches, batch, seq, hidden):
+    """Stage-boundary activations N(0,1), one [batch*seq, hidden] per micro-batch."""
+    return [_rng(seed + m).standard_normal((batch * seq, hidden)).astype(np.float32)
+            for m in range(num_micro_batches)]
+
+
+def bert_id_inputs(seed, num_micro_batches, batch, seq, vocab):
+    return [_rng(seed + m).integers(0, vocab, size=(batch, seq)).astype(np.int32)
+            for m in range(num_micro_batches)]
+
+
+def upstream_grads(seed, num_micro_batches, shape):
+    return [_rng(seed + m).standard_normal(shape).astype(np.float32)
+            for m in range(num_micro_batches)]
+
+
+# --------------------------------------------------------------------------- configs
+CONFIGS = {
+    # BASELINE configs[0]: BERT-Large 2-layer encoder stage behind the embedding
+    "bert_large_2l": dict(index=0, kind="bert", num_layers=2, hidden=1024, heads=16, ffn=4096,
+                          seq=128, micro_batch=2, num_micro_batches=4, dtype="fp32",
+                          embeddings=(30522, 2, 512)),
+    # BASELINE configs[3]: BERT-48 half-stage
+    "bert48_half": dict(index=3, kind="bert", num_layers=24, hidden=1024, heads=16, ffn=4096,
+                        seq=512, micro_batch=2, num_micro_batches=8, dtype="bf16",
+                        embeddings=None),
+}
