@@ -1,0 +1,115 @@
+"""ctypes binding of libdapple_hip.so (the C ABI declared in include/dapple_stage.h).
+
+There is no CPU fallback: if the library is missing or a call fails, this module
+raises.  Build it with ``python -m dapple_amd.build`` (hipcc, gfx950).
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libdapple_hip.so")
+
+DS_F32, DS_BF16 = 0, 1
+DS_K_MAJOR, DS_MN_MAJOR = 0, 1
+DS_EPI_BIAS, DS_EPI_RESIDUAL, DS_EPI_GELU, DS_EPI_DGELU = 1, 2, 4, 8
+DS_EPI_OUT_F32, DS_EPI_ACCUM, DS_EPI_RELU = 16, 32, 64
+DS_STAGE_BERT = 0
+
+
+class DappleError(RuntimeError):
+    pass
+
+
+class GemmDesc(C.Structure):
+    _fields_ = [
+        ("dtype", C.c_int), ("a_major", C.c_int), ("b_major", C.c_int),
+        ("m", C.c_int), ("n", C.c_int), ("k", C.c_int),
+        ("lda", C.c_int64), ("ldb", C.c_int64), ("ldc", C.c_int64),
+        ("batch", C.c_int), ("batch_inner", C.c_int),
+        ("a_stride_outer", C.c_int64), ("a_stride_inner", C.c_int64),
+        ("b_stride_outer", C.c_int64), ("b_stride_inner", C.c_int64),
+        ("c_stride_outer", C.c_int64), ("c_stride_inner", C.c_int64),
+        ("flags", C.c_int), ("alpha", C.c_float),
+        ("a", C.c_void_p), ("b", C.c_void_p), ("c", C.c_void_p),
+        ("bias", C.c_void_p), ("residual", C.c_void_p), ("c2", C.c_void_p),
+    ]
+
+
+class StageCfg(C.Structure):
+    _fields_ = [
+        ("kind", C.c_int), ("dtype", C.c_int), ("num_layers", C.c_int),
+        ("hidden", C.c_int), ("heads", C.c_int), ("ffn", C.c_int),
+        ("batch", C.c_int), ("seq", C.c_int), ("with_embedding", C.c_int),
+        ("vocab", C.c_int), ("type_vocab", C.c_int), ("max_pos", C.c_int),
+        ("ln_eps", C.c_float), ("stash_slots", C.c_int), ("first_layer", C.c_int),
+        ("reserved", C.c_int * 7),
+    ]
+
+
+# name -> (restype, argtypes); every symbol include/dapple_stage.h declares
+PROTOTYPES = {
+    "ds_last_error": (C.c_char_p, []),
+    "ds_build_target": (C.c_char_p, []),
+    "ds_grad_accumulate": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]),
+    "ds_cast_f32_to_bf16": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "ds_cast_bf16_to_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "ds_gemm": (C.c_int, [C.POINTER(GemmDesc), C.c_void_p]),
+    "ds_layernorm_fwd": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_float,
+                                   C.c_void_p, C.c_void_p, C.c_void_p]),
+    "ds_layernorm_bwd": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                   C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "ds_softmax_fwd": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_float, C.c_void_p,
+                                 C.c_float, C.c_void_p, C.c_void_p]),
+    "ds_softmax_bwd": (C.c_int, [C.c_int, C.c_int64, C.c_int, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p,
+                                 C.c_void_p]),
+    "ds_colsum_accum": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]),
+    "ds_stage_create": (C.c_int, [C.POINTER(StageCfg), C.c_void_p, C.POINTER(C.c_void_p)]),
+    "ds_stage_destroy": (C.c_int, [C.c_void_p]),
+    "ds_stage_num_weights": (C.c_int, [C.c_void_p]),
+    "ds_stage_weight_info": (C.c_int, [C.c_void_p, C.c_int, C.c_char_p, C.c_size_t, C.POINTER(C.c_int64),
+                                       C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
+    "ds_stage_bind_weights": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p)]),
+    "ds_stage_refresh_weights": (C.c_int, [C.c_void_p]),
+    "ds_stage_forward": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "ds_stage_set_token_types": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p]),
+    "ds_stage_backward": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
+    "ds_stage_workspace_bytes": (C.c_size_t, [C.c_void_p]),
+    "ds_stage_stash_bytes": (C.c_size_t, [C.c_void_p, C.c_int]),
+    "ds_stage_sync": (C.c_int, [C.c_void_p]),
+}
+
+_lib = None
+
+
+def load():
+    """Loads the shared library and sets the prototypes; raises if it is not built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise DappleError("%s not found: build it with `python -m dapple_amd.build` "
+                          "(there is no CPU fallback)" % LIB_PATH)
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in PROTOTYPES.items():
+        fn = getattr(lib, name)          # AttributeError if the symbol is missing
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(rc, what=""):
+    if rc != 0:
+        msg = load().ds_last_error().decode("utf-8", "replace")
+        kind = {-1: ValueError, -2: DappleError, -3: DappleError}.get(rc, DappleError)
+        raise kind("%s failed (%d): %s" % (what or "libdapple_hip call", rc, msg))
+
+
+def ptr(t):
+    """Device pointer of a torch tensor (or None)."""
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def current_stream():
+    import torch
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)

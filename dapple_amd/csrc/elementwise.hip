@@ -1,0 +1,462 @@
+// HBM-bound kernels: gradient accumulation, casts, LayerNorm, softmax, column sums.
+// All move data as 16-byte vectors per lane with grid-stride or one-wave-per-row mappings.
+#include "common.h"
+
+namespace {
+
+// ------------------------------------------------------------------ accumulate / cast
+// acc[i] += g[i]; 12 B/element (fp32 g) or 10 B/element (bf16 g) of HBM traffic.
+template <typename G>
+__global__ __launch_bounds__(256) void accumulate_kernel(float* __restrict__ acc, const G* __restrict__ g, size_t n) {
+  constexpr int VEC = Vec16<G>::N;
+  typedef typename Vec16<G>::type GV;
+  const size_t nvec = n / VEC;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t v = (size_t)blockIdx.x * blockDim.x + threadIdx.x; v < nvec; v += stride) {
+    const GV gv = reinterpret_cast<const GV*>(g)[v];
+    f32x4* ap = reinterpret_cast<f32x4*>(acc) + v * (VEC / 4);
+#pragma unroll
+    for (int q = 0; q < VEC / 4; ++q) {
+      f32x4 a = ap[q];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) a[e] += to_f32(gv[q * 4 + e]);
+      ap[q] = a;
+    }
+  }
+  // tail (n not a multiple of the vector width)
+  const size_t tail0 = nvec * VEC;
+  const size_t t = tail0 + (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < n) acc[t] += to_f32(g[t]);
+}
+
+template <typename D, typename S>
+__global__ __launch_bounds__(256) void cast_kernel(D* __restrict__ dst, const S* __restrict__ src, size_t n) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x * 4;
+  for (size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4; i < n; i += stride) {
+    if (i + 4 <= n) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dst[i + e] = from_f32<D>(to_f32(src[i + e]));
+    } else {
+      for (size_t e = i; e < n; ++e) dst[e] = from_f32<D>(to_f32(src[e]));
+    }
+  }
+}
+
+inline int grid_for(size_t work_items, int per_block) {
+  size_t b = (work_items + per_block - 1) / per_block;
+  if (b < 1) b = 1;
+  if (b > 256 * 16) b = 256 * 16;
+  return (int)b;
+}
+
+// ------------------------------------------------------------------ LayerNorm
+// One wave per row; a lane keeps NV 16-byte vectors of the row in registers.
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void layernorm_fwd_kernel(int rows, int cols, const T* __restrict__ x,
+                                                           const float* __restrict__ gamma,
+                                                           const float* __restrict__ beta, float eps,
+                                                           T* __restrict__ y, float* __restrict__ stats) {
+  constexpr int VEC = Vec16<T>::N;
+  typedef typename Vec16<T>::type V;
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const T* xr = x + (int64_t)row * cols;
+  float v[NV][VEC];
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = (lane + i * 64) * VEC;
+    if (c < cols) {
+      const V t = *reinterpret_cast<const V*>(xr + c);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) { v[i][e] = to_f32(t[e]); sum += v[i][e]; }
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) v[i][e] = 0.f;
+    }
+  }
+  const float mean = wave_sum(sum) / cols;
+  float sq = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = (lane + i * 64) * VEC;
+    if (c < cols) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) { const float d = v[i][e] - mean; sq += d * d; }
+    }
+  }
+  const float rstd = rsqrtf(wave_sum(sq) / cols + eps);
+  if (lane == 0 && stats) { stats[2 * row] = mean; stats[2 * row + 1] = rstd; }
+  T* yr = y + (int64_t)row * cols;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = (lane + i * 64) * VEC;
+    if (c < cols) {
+      V o;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) o[e] = from_f32<T>((v[i][e] - mean) * rstd * gamma[c + e] + beta[c + e]);
+      *reinterpret_cast<V*>(yr + c) = o;
+    }
+  }
+}
+
+// Backward: each wave walks ROWS_PER_WAVE rows and keeps the column partial sums of
+// d_gamma, d_beta and dx in registers; the 4 waves of a block combine through LDS and
+// issue one atomicAdd per column and quantity.
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void layernorm_bwd_kernel(int rows, int cols, int rows_per_wave,
+                                                           const T* __restrict__ dy, const T* __restrict__ x,
+                                                           const float* __restrict__ gamma,
+                                                           const float* __restrict__ stats,
+                                                           const T* __restrict__ dx_add, T* __restrict__ dx,
+                                                           float* __restrict__ d_gamma, float* __restrict__ d_beta,
+                                                           float* __restrict__ d_colsum) {
+  constexpr int VEC = Vec16<T>::N;
+  typedef typename Vec16<T>::type V;
+  extern __shared__ float red[];  // [3][cols]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int c = threadIdx.x; c < 3 * cols; c += 256) red[c] = 0.f;
+  __syncthreads();
+
+  float g[NV][VEC], pg[NV][VEC], pb[NV][VEC], ps[NV][VEC];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = (lane + i * 64) * VEC;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      g[i][e] = (c < cols) ? gamma[c + e] : 0.f;
+      pg[i][e] = pb[i][e] = ps[i][e] = 0.f;
+    }
+  }
+  const int row0 = (blockIdx.x * 4 + wave) * rows_per_wave;
+  for (int r = 0; r < rows_per_wave; ++r) {
+    const int row = row0 + r;
+    if (row >= rows) break;
+    const float mean = stats[2 * row], rstd = stats[2 * row + 1];
+    const T* dyr = dy + (int64_t)row * cols;
+    const T* xr = x + (int64_t)row * cols;
+    float dyv[NV][VEC], xh[NV][VEC];
+    float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int c = (lane + i * 64) * VEC;
+      if (c < cols) {
+        const V a = *reinterpret_cast<const V*>(dyr + c);
+        const V b = *reinterpret_cast<const V*>(xr + c);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          dyv[i][e] = to_f32(a[e]);
+          xh[i][e] = (to_f32(b[e]) - mean) * rstd;
+          const float dxh = dyv[i][e] * g[i][e];
+          s1 += dxh;
+          s2 += dxh * xh[i][e];
+          pg[i][e] += dyv[i][e] * xh[i][e];
+          pb[i][e] += dyv[i][e];
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) { dyv[i][e] = 0.f; xh[i][e] = 0.f; }
+      }
+    }
+    s1 = wave_sum(s1) / cols;
+    s2 = wave_sum(s2) / cols;
+    T* dxr = dx + (int64_t)row * cols;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int c = (lane + i * 64) * VEC;
+      if (c < cols) {
+        V o;
+        V add = {};
+        if (dx_add) add = *reinterpret_cast<const V*>(dx_add + (int64_t)row * cols + c);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const float d = rstd * (dyv[i][e] * g[i][e] - s1 - xh[i][e] * s2);
+          ps[i][e] += d;
+          o[e] = from_f32<T>(d + (dx_add ? to_f32(add[e]) : 0.f));
+        }
+        *reinterpret_cast<V*>(dxr + c) = o;
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = (lane + i * 64) * VEC;
+    if (c < cols) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        atomicAdd(&red[c + e], pg[i][e]);
+        atomicAdd(&red[cols + c + e], pb[i][e]);
+        atomicAdd(&red[2 * cols + c + e], ps[i][e]);
+      }
+    }
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < cols; c += 256) {
+    atomicAdd(d_gamma + c, red[c]);
+    atomicAdd(d_beta + c, red[cols + c]);
+    if (d_colsum) atomicAdd(d_colsum + c, red[2 * cols + c]);
+  }
+}
+
+// ------------------------------------------------------------------ softmax
+// One wave per row of fp32 scores; NV 16-byte vectors (4 floats) per lane.
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void softmax_fwd_kernel(int64_t rows, int k, int rows_per_batch,
+                                                         const float* __restrict__ scores, float scale,
+                                                         const float* __restrict__ key_mask, float mask_value,
+                                                         T* __restrict__ p) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const float* sr = scores + row * k;
+  const float* mk = key_mask ? key_mask + (row / rows_per_batch) * k : nullptr;
+  float v[NV][4];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = (lane + i * 64) * 4;
+    if (c < k) {
+      const f32x4 t = *reinterpret_cast<const f32x4*>(sr + c);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float s = t[e] * scale;
+        if (mk) s += (1.0f - mk[c + e]) * mask_value;
+        v[i][e] = s;
+        mx = fmaxf(mx, s);
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[i][e] = -INFINITY;
+    }
+  }
+  mx = wave_max(mx);
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { v[i][e] = expf(v[i][e] - mx); sum += v[i][e]; }
+  const float inv = 1.0f / wave_sum(sum);
+  T* pr = p + row * k;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = (lane + i * 64) * 4;
+    if (c < k) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) pr[c + e] = from_f32<T>(v[i][e] * inv);
+    }
+  }
+}
+
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void softmax_bwd_kernel(int64_t rows, int k, const T* __restrict__ p,
+                                                         const float* __restrict__ dp, float scale,
+                                                         T* __restrict__ ds) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const T* pr = p + row * k;
+  const float* dr = dp + row * k;
+  float pv[NV][4], dv[NV][4];
+  float dot = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = (lane + i * 64) * 4;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (c < k) { pv[i][e] = to_f32(pr[c + e]); dv[i][e] = dr[c + e]; } else { pv[i][e] = 0.f; dv[i][e] = 0.f; }
+      dot += pv[i][e] * dv[i][e];
+    }
+  }
+  dot = wave_sum(dot);
+  T* out = ds + row * k;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = (lane + i * 64) * 4;
+    if (c < k) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) out[c + e] = from_f32<T>(scale * pv[i][e] * (dv[i][e] - dot));
+    }
+  }
+}
+
+// ------------------------------------------------------------------ column sums
+// Block = 64 columns x 4 row groups; each thread strides down the rows, LDS-combines, then
+// one atomicAdd per column.
+template <typename T>
+__global__ __launch_bounds__(256) void colsum_kernel(int rows, int cols, const T* __restrict__ x, int64_t ldx,
+                                                    int rows_per_block, float* __restrict__ out) {
+  __shared__ float red[4][64];
+  const int c = blockIdx.x * 64 + (threadIdx.x & 63);
+  const int g = threadIdx.x >> 6;
+  const int r0 = blockIdx.y * rows_per_block;
+  int r1 = r0 + rows_per_block;
+  if (r1 > rows) r1 = rows;
+  float s = 0.f;
+  if (c < cols)
+    for (int r = r0 + g; r < r1; r += 4) s += to_f32(x[(int64_t)r * ldx + c]);
+  red[g][threadIdx.x & 63] = s;
+  __syncthreads();
+  if (g == 0 && c < cols) atomicAdd(out + c, red[0][threadIdx.x] + red[1][threadIdx.x] + red[2][threadIdx.x] + red[3][threadIdx.x]);
+}
+
+}  // namespace
+
+// =================================================================== C ABI
+extern "C" int ds_grad_accumulate(void* acc, const void* g, size_t n, int g_dtype, void* stream) {
+  DS_CHECK_ARG(acc && g, "ds_grad_accumulate: null pointer");
+  DS_CHECK_ARG(g_dtype == DS_F32 || g_dtype == DS_BF16, "ds_grad_accumulate: g_dtype %d", g_dtype);
+  DS_CHECK_ARG(ds_aligned16(acc) && ds_aligned16(g), "ds_grad_accumulate: pointers must be 16-byte aligned");
+  if (n == 0) return DS_OK;
+  hipStream_t s = (hipStream_t)stream;
+  if (g_dtype == DS_F32) {
+    const int grid = grid_for((n + 3) / 4, 256 * 4);
+    hipLaunchKernelGGL(accumulate_kernel<float>, dim3(grid), dim3(256), 0, s, (float*)acc, (const float*)g, n);
+  } else {
+    const int grid = grid_for((n + 7) / 8, 256 * 4);
+    hipLaunchKernelGGL(accumulate_kernel<bf16>, dim3(grid), dim3(256), 0, s, (float*)acc, (const bf16*)g, n);
+  }
+  DS_CHECK_LAUNCH();
+  return DS_OK;
+}
+
+extern "C" int ds_cast_f32_to_bf16(void* dst, const void* src, size_t n, void* stream) {
+  DS_CHECK_ARG(dst && src, "ds_cast_f32_to_bf16: null pointer");
+  if (n == 0) return DS_OK;
+  hipLaunchKernelGGL((cast_kernel<bf16, float>), dim3(grid_for((n + 3) / 4, 256)), dim3(256), 0, (hipStream_t)stream,
+                     (bf16*)dst, (const float*)src, n);
+  DS_CHECK_LAUNCH();
+  return DS_OK;
+}
+extern "C" int ds_cast_bf16_to_f32(void* dst, const void* src, size_t n, void* stream) {
+  DS_CHECK_ARG(dst && src, "ds_cast_bf16_to_f32: null pointer");
+  if (n == 0) return DS_OK;
+  hipLaunchKernelGGL((cast_kernel<float, bf16>), dim3(grid_for((n + 3) / 4, 256)), dim3(256), 0, (hipStream_t)stream,
+                     (float*)dst, (const bf16*)src, n);
+  DS_CHECK_LAUNCH();
+  return DS_OK;
+}
+
+template <typename T> static int max_cols_rowkernel(int nv) { return 64 * Vec16<T>::N * nv; }
+
+#define DISPATCH_NV(T, need, CALL)                                   \
+  do {                                                               \
+    if ((need) <= 1) { constexpr int NV = 1; CALL; }                 \
+    else if ((need) <= 2) { constexpr int NV = 2; CALL; }            \
+    else if ((need) <= 4) { constexpr int NV = 4; CALL; }            \
+    else { constexpr int NV = 8; CALL; }                             \
+  } while (0)
+
+template <typename T>
+static int layernorm_fwd_t(int rows, int cols, const void* x, const float* gamma, const float* beta, float eps, void* y,
+                           float* stats, hipStream_t s) {
+  const int vec = Vec16<T>::N;
+  const int need = (cols / vec + 63) / 64;
+  dim3 grid((rows + 3) / 4);
+  DISPATCH_NV(T, need, hipLaunchKernelGGL((layernorm_fwd_kernel<T, NV>), grid, dim3(256), 0, s, rows, cols, (const T*)x,
+                                          gamma, beta, eps, (T*)y, stats));
+  DS_CHECK_LAUNCH();
+  return DS_OK;
+}
+
+static int check_rows(const char* who, int dtype, int rows, int cols) {
+  DS_CHECK_ARG(dtype == DS_F32 || dtype == DS_BF16, "%s: dtype %d", who, dtype);
+  const int vec = dtype == DS_BF16 ? 8 : 4;
+  DS_CHECK_ARG(rows > 0 && cols > 0, "%s: rows/cols must be positive", who);
+  DS_CHECK_ARG(cols % vec == 0, "%s: cols=%d must be a multiple of %d", who, cols, vec);
+  DS_CHECK_ARG(cols <= 64 * vec * 8, "%s: cols=%d exceeds the %d this kernel keeps in registers", who, cols, 64 * vec * 8);
+  return DS_OK;
+}
+
+extern "C" int ds_layernorm_fwd(int dtype, int rows, int cols, const void* x, const float* gamma, const float* beta,
+                                float eps, void* y, float* stats, void* stream) {
+  DS_PROPAGATE(check_rows("ds_layernorm_fwd", dtype, rows, cols));
+  DS_CHECK_ARG(x && gamma && beta && y, "ds_layernorm_fwd: null pointer");
+  DS_CHECK_ARG(ds_aligned16(x) && ds_aligned16(y), "ds_layernorm_fwd: x/y must be 16-byte aligned");
+  if (dtype == DS_BF16) return layernorm_fwd_t<bf16>(rows, cols, x, gamma, beta, eps, y, stats, (hipStream_t)stream);
+  return layernorm_fwd_t<float>(rows, cols, x, gamma, beta, eps, y, stats, (hipStream_t)stream);
+}
+
+template <typename T>
+static int layernorm_bwd_t(int rows, int cols, const void* dy, const void* x, const float* gamma, const float* stats,
+                           const void* dx_add, void* dx, float* dg, float* db, float* dcs, hipStream_t s) {
+  const int vec = Vec16<T>::N;
+  const int need = (cols / vec + 63) / 64;
+  // aim for ~512 blocks of 4 waves; each wave walks rows_per_wave rows
+  int rpw = rows / (512 * 4);
+  if (rpw < 1) rpw = 1;
+  if (rpw > 16) rpw = 16;
+  dim3 grid((rows + 4 * rpw - 1) / (4 * rpw));
+  const size_t lds = 3 * (size_t)cols * sizeof(float);
+  DISPATCH_NV(T, need, hipLaunchKernelGGL((layernorm_bwd_kernel<T, NV>), grid, dim3(256), lds, s, rows, cols, rpw,
+                                          (const T*)dy, (const T*)x, gamma, stats, (const T*)dx_add, (T*)dx, dg, db, dcs));
+  DS_CHECK_LAUNCH();
+  return DS_OK;
+}
+
+extern "C" int ds_layernorm_bwd(int dtype, int rows, int cols, const void* dy, const void* x, const float* gamma,
+                                const float* stats, const void* dx_add, void* dx, float* d_gamma, float* d_beta,
+                                float* d_colsum, void* stream) {
+  DS_PROPAGATE(check_rows("ds_layernorm_bwd", dtype, rows, cols));
+  DS_CHECK_ARG(dy && x && gamma && stats && dx && d_gamma && d_beta, "ds_layernorm_bwd: null pointer");
+  DS_CHECK_ARG(ds_aligned16(dy) && ds_aligned16(x) && ds_aligned16(dx) && ds_aligned16(dx_add),
+               "ds_layernorm_bwd: tensors must be 16-byte aligned");
+  if (dtype == DS_BF16)
+    return layernorm_bwd_t<bf16>(rows, cols, dy, x, gamma, stats, dx_add, dx, d_gamma, d_beta, d_colsum, (hipStream_t)stream);
+  return layernorm_bwd_t<float>(rows, cols, dy, x, gamma, stats, dx_add, dx, d_gamma, d_beta, d_colsum, (hipStream_t)stream);
+}
+
+template <typename T>
+static int softmax_fwd_t(int64_t rows, int k, int rpb, const float* scores, float scale, const float* mask, float mv,
+                         void* p, hipStream_t s) {
+  const int need = (k / 4 + 63) / 64;
+  dim3 grid((unsigned)((rows + 3) / 4));
+  DISPATCH_NV(T, need, hipLaunchKernelGGL((softmax_fwd_kernel<T, NV>), grid, dim3(256), 0, s, rows, k, rpb, scores, scale,
+                                          mask, mv, (T*)p));
+  DS_CHECK_LAUNCH();
+  return DS_OK;
+}
+
+extern "C" int ds_softmax_fwd(int dtype, int batch, int heads, int q, int k, const float* scores, float scale,
+                              const float* key_mask, float mask_value, void* p, void* stream) {
+  DS_CHECK_ARG(dtype == DS_F32 || dtype == DS_BF16, "ds_softmax_fwd: dtype %d", dtype);
+  DS_CHECK_ARG(batch > 0 && heads > 0 && q > 0 && k > 0, "ds_softmax_fwd: non-positive shape");
+  DS_CHECK_ARG(k % 4 == 0 && k <= 64 * 4 * 8, "ds_softmax_fwd: k=%d must be a multiple of 4 and at most 2048", k);
+  DS_CHECK_ARG(scores && p && ds_aligned16(scores), "ds_softmax_fwd: null or unaligned pointer");
+  const int64_t rows = (int64_t)batch * heads * q;
+  if (dtype == DS_BF16)
+    return softmax_fwd_t<bf16>(rows, k, heads * q, scores, scale, key_mask, mask_value, p, (hipStream_t)stream);
+  return softmax_fwd_t<float>(rows, k, heads * q, scores, scale, key_mask, mask_value, p, (hipStream_t)stream);
+}
+
+template <typename T>
+static int softmax_bwd_t(int64_t rows, int k, const void* p, const float* dp, float scale, void* ds, hipStream_t s) {
+  const int need = (k / 4 + 63) / 64;
+  dim3 grid((unsigned)((rows + 3) / 4));
+  DISPATCH_NV(T, need, hipLaunchKernelGGL((softmax_bwd_kernel<T, NV>), grid, dim3(256), 0, s, rows, k, (const T*)p, dp,
+                                          scale, (T*)ds));
+  DS_CHECK_LAUNCH();
+  return DS_OK;
+}
+
+extern "C" int ds_softmax_bwd(int dtype, int64_t rows, int k, const void* p, const float* dp, float scale, void* ds,
+                              void* stream) {
+  DS_CHECK_ARG(dtype == DS_F32 || dtype == DS_BF16, "ds_softmax_bwd: dtype %d", dtype);
+  DS_CHECK_ARG(rows > 0 && k > 0 && k % 4 == 0 && k <= 2048, "ds_softmax_bwd: bad shape rows=%lld k=%d", (long long)rows, k);
+  DS_CHECK_ARG(p && dp && ds, "ds_softmax_bwd: null pointer");
+  if (dtype == DS_BF16) return softmax_bwd_t<bf16>(rows, k, p, dp, scale, ds, (hipStream_t)stream);
+  return softmax_bwd_t<float>(rows, k, p, dp, scale, ds, (hipStream_t)stream);
+}
+
+extern "C" int ds_colsum_accum(int dtype, int rows, int cols, const void* x, int64_t ldx, float* out, void* stream) {
+  DS_CHECK_ARG(dtype == DS_F32 || dtype == DS_BF16, "ds_colsum_accum: dtype %d", dtype);
+  DS_CHECK_ARG(rows > 0 && cols > 0 && ldx >= cols && x && out, "ds_colsum_accum: bad argument");
+  int rpb = 64;
+  dim3 grid((cols + 63) / 64, (rows + rpb - 1) / rpb);
+  if (dtype == DS_BF16)
+    hipLaunchKernelGGL(colsum_kernel<bf16>, grid, dim3(256), 0, (hipStream_t)stream, rows, cols, (const bf16*)x, ldx, rpb, out);
+  else
+    hipLaunchKernelGGL(colsum_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, rows, cols, (const float*)x, ldx, rpb, out);
+  DS_CHECK_LAUNCH();
+  return DS_OK;
+}

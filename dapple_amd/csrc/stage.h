@@ -1,0 +1,42 @@
+// Stage handle behind ds_stage_*: weights (fp32 masters owned by the caller), compute copies,
+// workspace and the K-slot activation stash (owned by the handle).
+#pragma once
+#include <string>
+#include <vector>
+
+#include "common.h"
+
+struct WeightInfo {
+  std::string name;
+  int64_t rows, cols;  // cols == 1 row vector for biases: rows = 1, cols = n
+  int64_t numel() const { return rows * cols; }
+};
+
+// Bump allocator over one hipMalloc'd arena; every carve is 256-byte aligned.
+struct Arena {
+  char* base = nullptr;
+  size_t cap = 0, used = 0;
+  size_t reserve(size_t bytes) {  // planning pass: returns the offset
+    const size_t off = used;
+    used += (bytes + 255) & ~size_t(255);
+    return off;
+  }
+};
+
+struct ds_stage {
+  ds_stage_cfg cfg;
+  hipStream_t stream = nullptr;
+  std::vector<WeightInfo> winfo;
+  std::vector<const float*> w;  // fp32 masters
+  std::vector<float*> g;        // fp32 master grads
+  bool bound = false;
+  std::vector<char> slot_forwarded;
+  virtual ~ds_stage() {}
+  virtual int refresh_weights() = 0;
+  virtual int forward(int slot, const void* in, const float* key_mask, void* out) = 0;
+  virtual int backward(int slot, const void* d_out, void* d_in) = 0;
+  virtual size_t workspace_bytes() const = 0;
+  virtual size_t stash_bytes(int slots) const = 0;
+};
+
+int ds_bert_stage_create(const ds_stage_cfg* cfg, hipStream_t stream, ds_stage** out);

@@ -1,0 +1,140 @@
+"""Torch-tensor front ends of the per-kernel C-ABI entry points.
+
+Each function takes CUDA (ROCm) tensors, passes raw device pointers through
+ctypes and launches on torch's current stream.  Nothing here computes on the
+host and nothing falls back to torch ops.
+"""
+import ctypes as C
+
+import torch
+
+from . import _lib
+from ._lib import (DS_BF16, DS_EPI_ACCUM, DS_EPI_BIAS, DS_EPI_DGELU, DS_EPI_GELU, DS_EPI_OUT_F32,
+                   DS_EPI_RELU, DS_EPI_RESIDUAL, DS_F32, DS_K_MAJOR, DS_MN_MAJOR, GemmDesc, check, ptr)
+
+
+def dtype_code(t):
+    if t.dtype == torch.float32:
+        return DS_F32
+    if t.dtype == torch.bfloat16:
+        return DS_BF16
+    raise ValueError("unsupported element type %s (fp32 or bf16)" % t.dtype)
+
+
+def _need_cuda(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise ValueError("tensor must live on the GPU")
+        if t is not None and not t.is_contiguous():
+            raise ValueError("tensor must be contiguous")
+
+
+def grad_accumulate(acc, g):
+    """acc (fp32) += g, in place (tf.accumulate_n of bert/graph.py:159, one micro-batch at a time)."""
+    _need_cuda(acc, g)
+    if acc.dtype != torch.float32 or acc.numel() != g.numel():
+        raise ValueError("acc must be fp32 with as many elements as g")
+    check(_lib.load().ds_grad_accumulate(ptr(acc), ptr(g), g.numel(), dtype_code(g), _lib.current_stream()),
+          "ds_grad_accumulate")
+    return acc
+
+
+def cast_to_bf16(src):
+    _need_cuda(src)
+    dst = torch.empty_like(src, dtype=torch.bfloat16)
+    check(_lib.load().ds_cast_f32_to_bf16(ptr(dst), ptr(src), src.numel(), _lib.current_stream()), "ds_cast_f32_to_bf16")
+    return dst
+
+
+def cast_to_f32(src):
+    _need_cuda(src)
+    dst = torch.empty_like(src, dtype=torch.float32)
+    check(_lib.load().ds_cast_bf16_to_f32(ptr(dst), ptr(src), src.numel(), _lib.current_stream()), "ds_cast_bf16_to_f32")
+    return dst
+
+
+def gemm(a, b, c, m, n, k, a_major=DS_K_MAJOR, b_major=DS_MN_MAJOR, lda=None, ldb=None, ldc=None, flags=0,
+         alpha=1.0, bias=None, residual=None, c2=None, batch=1, batch_inner=1, a_strides=(0, 0), b_strides=(0, 0),
+         c_strides=(0, 0)):
+    """Raw ds_gemm: C[m][n] (+)= alpha * sum_k A(m,k) B(n,k); see include/dapple_stage.h."""
+    _need_cuda(a, b, c, bias, residual, c2)
+    d = GemmDesc()
+    d.dtype = dtype_code(a)
+    d.a_major, d.b_major = a_major, b_major
+    d.m, d.n, d.k = m, n, k
+    d.lda = lda if lda is not None else (k if a_major == DS_K_MAJOR else m)
+    d.ldb = ldb if ldb is not None else (k if b_major == DS_K_MAJOR else n)
+    d.ldc = ldc if ldc is not None else n
+    d.batch, d.batch_inner = batch, batch_inner
+    d.a_stride_outer, d.a_stride_inner = a_strides
+    d.b_stride_outer, d.b_stride_inner = b_strides
+    d.c_stride_outer, d.c_stride_inner = c_strides
+    d.flags, d.alpha = flags, alpha
+    d.a, d.b, d.c = a.data_ptr(), b.data_ptr(), c.data_ptr()
+    d.bias = bias.data_ptr() if bias is not None else None
+    d.residual = residual.data_ptr() if residual is not None else None
+    d.c2 = c2.data_ptr() if c2 is not None else None
+    check(_lib.load().ds_gemm(C.byref(d), _lib.current_stream()), "ds_gemm")
+    return c
+
+
+def dense(x, kernel, bias=None, residual=None, gelu=False):
+    """tf.layers.dense: x[m,k] @ kernel[k,n] + bias (+ residual) (gelu -> returns (pre, act))."""
+    m, k = x.shape
+    n = kernel.shape[1]
+    y = torch.empty(m, n, dtype=x.dtype, device=x.device)
+    flags = (DS_EPI_BIAS if bias is not None else 0) | (DS_EPI_RESIDUAL if residual is not None else 0)
+    act = None
+    if gelu:
+        flags |= DS_EPI_GELU
+        act = torch.empty_like(y)
+    gemm(x, kernel, y, m, n, k, DS_K_MAJOR, DS_MN_MAJOR, flags=flags, bias=bias, residual=residual, c2=act)
+    return (y, act) if gelu else y
+
+
+def layernorm_fwd(x, gamma, beta, eps=1e-12):
+    _need_cuda(x, gamma, beta)
+    rows, cols = x.shape
+    y = torch.empty_like(x)
+    stats = torch.empty(rows, 2, dtype=torch.float32, device=x.device)
+    check(_lib.load().ds_layernorm_fwd(dtype_code(x), rows, cols, ptr(x), ptr(gamma), ptr(beta), eps, ptr(y), ptr(stats),
+                                       _lib.current_stream()), "ds_layernorm_fwd")
+    return y, stats
+
+
+def layernorm_bwd(dy, x, gamma, stats, d_gamma, d_beta, d_colsum=None, dx_add=None):
+    _need_cuda(dy, x, gamma, stats, d_gamma, d_beta, d_colsum, dx_add)
+    rows, cols = x.shape
+    dx = torch.empty_like(x)
+    check(_lib.load().ds_layernorm_bwd(dtype_code(x), rows, cols, ptr(dy), ptr(x), ptr(gamma), ptr(stats), ptr(dx_add),
+                                       ptr(dx), ptr(d_gamma), ptr(d_beta), ptr(d_colsum), _lib.current_stream()),
+          "ds_layernorm_bwd")
+    return dx
+
+
+def softmax_fwd(scores, scale, key_mask=None, mask_value=-10000.0, out_dtype=torch.float32):
+    """scores fp32 [B, N, Q, K] -> probabilities of out_dtype."""
+    _need_cuda(scores, key_mask)
+    b, n, q, k = scores.shape
+    p = torch.empty(b, n, q, k, dtype=out_dtype, device=scores.device)
+    check(_lib.load().ds_softmax_fwd(dtype_code(p), b, n, q, k, ptr(scores), scale, ptr(key_mask), mask_value, ptr(p),
+                                     _lib.current_stream()), "ds_softmax_fwd")
+    return p
+
+
+def softmax_bwd(p, dp, scale):
+    _need_cuda(p, dp)
+    k = p.shape[-1]
+    rows = p.numel() // k
+    ds = torch.empty_like(p)
+    check(_lib.load().ds_softmax_bwd(dtype_code(p), rows, k, ptr(p), ptr(dp), scale, ptr(ds), _lib.current_stream()),
+          "ds_softmax_bwd")
+    return ds
+
+
+def colsum_accum(x, out):
+    _need_cuda(x, out)
+    rows, cols = x.shape
+    check(_lib.load().ds_colsum_accum(dtype_code(x), rows, cols, ptr(x), cols, ptr(out), _lib.current_stream()),
+          "ds_colsum_accum")
+    return out

@@ -1,0 +1,201 @@
+"""The explicit per-stage runtime the reference only implies with graph edges.
+
+``schedule_ops`` states the early-backward rule of bert/graph.py:126-132 (and the
+``2S-1`` variant of vgg19/tf-keras-dapple.py:292) as the op order of one stage;
+``StageRuntime.step`` issues ``ds_stage_forward`` / ``ds_stage_backward`` in that
+order with a stash of K = S - i slots, and the weight gradients accumulate in
+place in one flat fp32 buffer (bert/graph.py:145-161: a sum over micro-batches).
+"""
+import ctypes as C
+
+import torch
+
+from . import _lib
+from ._lib import DS_BF16, DS_F32, DS_STAGE_BERT, StageCfg, check, ptr
+
+
+def stash_depth(stage_index, num_stages, variant="S"):
+    """In-flight micro-batches at a stage: S - i (bert/graph.py:129) or 2S - 1 - i (vgg19/tf-keras-dapple.py:292)."""
+    if variant not in ("S", "2S-1"):
+        raise ValueError("variant must be 'S' or '2S-1'")
+    return (num_stages if variant == "S" else 2 * num_stages - 1) - stage_index
+
+
+def schedule_ops(stage_index, num_stages, num_micro_batches, variant="S"):
+    """[('F', j) | ('B', j)] in execution order: K warm-up forwards, then one backward per forward."""
+    if not (0 <= stage_index < num_stages):
+        raise ValueError("stage_index %d outside [0, %d)" % (stage_index, num_stages))
+    if num_micro_batches < 1:
+        raise ValueError("num_micro_batches must be >= 1")
+    k = min(stash_depth(stage_index, num_stages, variant), num_micro_batches)
+    ops = [("F", j) for j in range(k)]
+    for j in range(num_micro_batches):
+        ops.append(("B", j))
+        if j + k < num_micro_batches:
+            ops.append(("F", j + k))
+    return ops
+
+
+_TORCH_DTYPE = {DS_F32: torch.float32, DS_BF16: torch.bfloat16}
+
+
+class Stage:
+    """Owns a ``ds_stage`` handle plus the flat fp32 master weights / gradients it is bound to."""
+
+    def __init__(self, kind, dtype, num_layers, hidden, heads, ffn, batch, seq, stash_slots, with_embedding=False,
+                 vocab=0, type_vocab=0, max_pos=0, ln_eps=1e-12, first_layer=0, device="cuda:0"):
+        self.lib = _lib.load()
+        self.device = torch.device(device)
+        self.dtype_code = {"fp32": DS_F32, "bf16": DS_BF16, DS_F32: DS_F32, DS_BF16: DS_BF16}[dtype]
+        self.act_dtype = _TORCH_DTYPE[self.dtype_code]
+        cfg = StageCfg()
+        cfg.kind, cfg.dtype, cfg.num_layers = kind, self.dtype_code, num_layers
+        cfg.hidden, cfg.heads, cfg.ffn, cfg.batch, cfg.seq = hidden, heads, ffn, batch, seq
+        cfg.with_embedding = 1 if with_embedding else 0
+        cfg.vocab, cfg.type_vocab, cfg.max_pos = vocab, type_vocab, max_pos
+        cfg.ln_eps, cfg.stash_slots, cfg.first_layer = ln_eps, stash_slots, first_layer
+        self.cfg = cfg
+        self.rows, self.hidden, self.stash_slots = batch * seq, hidden, stash_slots
+        self.with_embedding = bool(with_embedding)
+        self._h = C.c_void_p()
+        with torch.cuda.device(self.device):
+            self._stream = _lib.current_stream()
+            check(self.lib.ds_stage_create(C.byref(cfg), self._stream, C.byref(self._h)), "ds_stage_create")
+        n = self.lib.ds_stage_num_weights(self._h)
+        self.weight_names, self.weight_shapes = [], []
+        buf = C.create_string_buffer(256)
+        numel, rows, cols = C.c_int64(), C.c_int64(), C.c_int64()
+        for i in range(n):
+            check(self.lib.ds_stage_weight_info(self._h, i, buf, 256, C.byref(numel), C.byref(rows), C.byref(cols)),
+                  "ds_stage_weight_info")
+            self.weight_names.append(buf.value.decode())
+            self.weight_shapes.append((rows.value, cols.value) if rows.value > 1 or "kernel" in buf.value.decode()
+                                      or "embeddings" in buf.value.decode() else (cols.value,))
+        self.weights, self.grads = {}, {}
+        self.flat_weights = self.flat_grads = None
+
+    # -- weights ---------------------------------------------------------------------------
+    def bind(self, weights):
+        """weights: {reference variable name: array/tensor}. Copies into one flat fp32 buffer,
+        allocates the flat master-gradient buffer (zeroed) and binds both."""
+        missing = [n for n in self.weight_names if n not in weights]
+        if missing:
+            raise KeyError("missing weights: %s" % missing[:4])
+        sizes = []
+        for n, shp in zip(self.weight_names, self.weight_shapes):
+            numel = 1
+            for s in shp:
+                numel *= s
+            w = weights[n]
+            if tuple(w.shape) != tuple(shp):
+                raise ValueError("weight %s has shape %s, stage expects %s" % (n, tuple(w.shape), tuple(shp)))
+            sizes.append((numel + 63) // 64 * 64)          # keep every view 256-byte aligned
+        total = sum(sizes)
+        self.flat_weights = torch.empty(total, dtype=torch.float32, device=self.device)
+        self.flat_grads = torch.zeros(total, dtype=torch.float32, device=self.device)
+        off = 0
+        wp = (C.c_void_p * len(sizes))()
+        gp = (C.c_void_p * len(sizes))()
+        for i, (n, shp, sz) in enumerate(zip(self.weight_names, self.weight_shapes, sizes)):
+            numel = 1
+            for s in shp:
+                numel *= s
+            wv = self.flat_weights[off:off + numel].view(*shp)
+            wv.copy_(torch.as_tensor(weights[n], dtype=torch.float32))
+            self.weights[n] = wv
+            self.grads[n] = self.flat_grads[off:off + numel].view(*shp)
+            wp[i], gp[i] = wv.data_ptr(), self.grads[n].data_ptr()
+            off += sz
+        check(self.lib.ds_stage_bind_weights(self._h, len(sizes), wp, gp), "ds_stage_bind_weights")
+
+    def refresh_weights(self):
+        check(self.lib.ds_stage_refresh_weights(self._h), "ds_stage_refresh_weights")
+
+    def zero_grads(self):
+        self.flat_grads.zero_()
+
+    # -- one micro-batch ---------------------------------------------------------------------
+    def forward(self, slot, x, out, key_mask=None, token_type_ids=None):
+        if self.with_embedding:
+            if x.dtype != torch.int32 or x.numel() != self.rows:
+                raise ValueError("an embedding stage takes int32 ids of %d elements" % self.rows)
+            if token_type_ids is not None:
+                check(self.lib.ds_stage_set_token_types(self._h, slot, ptr(token_type_ids)), "ds_stage_set_token_types")
+        elif x.dtype != self.act_dtype or x.numel() != self.rows * self.hidden:
+            raise ValueError("stage input must be %s [%d, %d]" % (self.act_dtype, self.rows, self.hidden))
+        if out.dtype != self.act_dtype or out.numel() != self.rows * self.hidden:
+            raise ValueError("stage output must be %s [%d, %d]" % (self.act_dtype, self.rows, self.hidden))
+        if key_mask is not None and (key_mask.dtype != torch.float32 or key_mask.numel() != self.cfg.batch * self.cfg.seq):
+            raise ValueError("key_mask must be fp32 [batch, seq]")
+        check(self.lib.ds_stage_forward(self._h, slot, ptr(x), ptr(key_mask), ptr(out)), "ds_stage_forward")
+
+    def backward(self, slot, d_out, d_in=None):
+        if d_out.dtype != self.act_dtype or d_out.numel() != self.rows * self.hidden:
+            raise ValueError("upstream gradient must be %s [%d, %d]" % (self.act_dtype, self.rows, self.hidden))
+        if d_in is not None and (d_in.dtype != self.act_dtype or d_in.numel() != self.rows * self.hidden):
+            raise ValueError("input gradient must be %s [%d, %d]" % (self.act_dtype, self.rows, self.hidden))
+        check(self.lib.ds_stage_backward(self._h, slot, ptr(d_out), ptr(d_in)), "ds_stage_backward")
+
+    def sync(self):
+        check(self.lib.ds_stage_sync(self._h), "ds_stage_sync")
+
+    def workspace_bytes(self):
+        return self.lib.ds_stage_workspace_bytes(self._h)
+
+    def stash_bytes(self, slots=None):
+        return self.lib.ds_stage_stash_bytes(self._h, self.stash_slots if slots is None else slots)
+
+    def close(self):
+        if self._h:
+            self.lib.ds_stage_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def bert_stage(num_layers, hidden, heads, ffn, batch, seq, dtype, stash_slots, embeddings=None, first_layer=0,
+               ln_eps=1e-12, device="cuda:0"):
+    """A BERT stage: ``num_layers`` encoder layers, behind the embedding when ``embeddings`` =
+    (vocab, type_vocab, max_pos) is given."""
+    if hidden % heads != 0:
+        raise ValueError("The hidden size (%d) is not a multiple of the number of attention heads (%d)" % (hidden, heads))
+    kw = {}
+    if embeddings is not None:
+        kw = dict(with_embedding=True, vocab=embeddings[0], type_vocab=embeddings[1], max_pos=embeddings[2])
+    return Stage(DS_STAGE_BERT, dtype, num_layers, hidden, heads, ffn, batch, seq, stash_slots, ln_eps=ln_eps,
+                 first_layer=first_layer, device=device, **kw)
+
+
+class StageRuntime:
+    """Runs one stage over M micro-batches in the early-backward order."""
+
+    def __init__(self, stage, stage_index=0, num_stages=2, num_micro_batches=8, variant="S", needs_input_grad=True):
+        self.stage = stage
+        self.ops = schedule_ops(stage_index, num_stages, num_micro_batches, variant)
+        self.k = min(stash_depth(stage_index, num_stages, variant), num_micro_batches)
+        if stage.stash_slots < self.k:
+            raise ValueError("stage has %d stash slots, the schedule needs %d" % (stage.stash_slots, self.k))
+        self.m = num_micro_batches
+        self.needs_input_grad = needs_input_grad and not stage.with_embedding
+
+    def step(self, inputs, upstream, outputs, input_grads=None, key_masks=None):
+        """inputs[M], upstream[M]: device tensors; outputs[M] (and input_grads[M]) are filled.
+        Weight gradients add into ``stage.grads`` (call ``stage.zero_grads()`` between steps)."""
+        if len(inputs) != self.m or len(upstream) != self.m or len(outputs) != self.m:
+            raise ValueError("expected %d micro-batches" % self.m)
+        slot_of, free = {}, list(range(self.stage.stash_slots))
+        for op, j in self.ops:
+            if op == "F":
+                slot = free.pop(0)
+                slot_of[j] = slot
+                self.stage.forward(slot, inputs[j], outputs[j], None if key_masks is None else key_masks[j])
+            else:
+                slot = slot_of.pop(j)
+                d_in = input_grads[j] if (self.needs_input_grad and input_grads is not None) else None
+                self.stage.backward(slot, upstream[j], d_in)
+                free.append(slot)
+        return outputs

@@ -1,0 +1,169 @@
+/*
+ * C ABI of libdapple_hip.so: one DAPPLE pipeline stage on one MI355X.
+ *
+ * The reference (AlibabaPAI/DAPPLE) has no FFI for this path: src/api/capi.rs is
+ * empty and its runtime is TF1 graph construction.  Every entry point below
+ * therefore cites the reference Python/TF interface it replaces.  All pointers
+ * are device pointers unless the comment says "host"; the caller owns every
+ * buffer it passes in; the stage handle owns its compute copies of the weights,
+ * its workspace and its K-slot activation stash.  Every function returns 0 on
+ * success and a negative DS_E* code on failure, never throws, and leaves a
+ * message for ds_last_error() (thread-local).  A handle is used from one host
+ * thread at a time.  Launches are asynchronous on the given stream.
+ */
+#ifndef DAPPLE_STAGE_H
+#define DAPPLE_STAGE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DS_OK 0
+#define DS_EINVAL (-1)  /* bad argument: shape, alignment, null pointer, unknown enum */
+#define DS_EHIP (-2)    /* a HIP runtime call failed */
+#define DS_ESTATE (-3)  /* call order: slot not forwarded, weights not bound, ... */
+
+/* element types of activations / compute copies */
+#define DS_F32 0
+#define DS_BF16 1
+
+/* operand storage for ds_gemm: which index is contiguous in memory */
+#define DS_K_MAJOR 0  /* reduction index contiguous: A[m][k] / B[n][k] */
+#define DS_MN_MAJOR 1 /* free index contiguous:      A[k][m] / B[k][n] */
+
+/* epilogue flags for ds_gemm */
+#define DS_EPI_BIAS 1      /* + bias[n] (fp32) */
+#define DS_EPI_RESIDUAL 2  /* + residual[m][n] (element type) */
+#define DS_EPI_GELU 4      /* C = pre-activation, C2 = gelu_erf(C) */
+#define DS_EPI_DGELU 8     /* C = acc * gelu_erf'(aux[m][n]) */
+#define DS_EPI_OUT_F32 16  /* C is fp32 even when dtype is bf16 */
+#define DS_EPI_ACCUM 32    /* C (fp32) += acc, split-K allowed (atomic) */
+#define DS_EPI_RELU 64     /* C = max(acc + bias, 0) */
+
+const char* ds_last_error(void);
+
+/* Version / build probe; returns the gfx target the library was built for ("gfx950"). */
+const char* ds_build_target(void);
+
+/* ---------------------------------------------------------------------------
+ * Gradient accumulation: acc[i] (fp32) += g[i], i < n.
+ * Replaces tf.accumulate_n(grad_i_set) at bert/graph.py:159 (and its copies at
+ * vgg19/tf-keras-dapple.py:311, gnmt/nmt/model.py:288, xlnet/main_tf_estimator.py:226),
+ * applied in place as each micro-batch's backward finishes: a sum, no 1/M.
+ * g_dtype is DS_F32 or DS_BF16.  Pointers must be 16-byte aligned. */
+int ds_grad_accumulate(void* acc_fp32, const void* g, size_t n, int g_dtype, void* stream);
+
+/* fp32 -> bf16 copy of n elements (compute copies of the fp32 master weights). */
+int ds_cast_f32_to_bf16(void* dst_bf16, const void* src_f32, size_t n, void* stream);
+int ds_cast_bf16_to_f32(void* dst_f32, const void* src_bf16, size_t n, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * GEMM on the matrix cores: C[m][n] (+)= sum_k A(m,k) * B(n,k), optionally batched.
+ * Replaces tf.layers.dense (bert/models/bert/modeling_slice.py:464-485, 974-994),
+ * tf.matmul (:499, :533) and their tf.gradients.  Batch index z in [0, batch) is
+ * split as (z / batch_inner, z % batch_inner) with separate strides, which
+ * addresses [B, heads] views of a [B*S, hidden] matrix without copies. */
+typedef struct ds_gemm_desc {
+  int dtype;            /* DS_F32 or DS_BF16: element type of A, B (and C unless OUT_F32/ACCUM) */
+  int a_major, b_major; /* DS_K_MAJOR / DS_MN_MAJOR */
+  int m, n, k;
+  int64_t lda, ldb, ldc; /* leading dimensions in elements */
+  int batch, batch_inner;
+  int64_t a_stride_outer, a_stride_inner;
+  int64_t b_stride_outer, b_stride_inner;
+  int64_t c_stride_outer, c_stride_inner;
+  int flags;            /* DS_EPI_* */
+  float alpha;          /* acc is scaled by alpha before the epilogue */
+  const void* a;
+  const void* b;
+  void* c;
+  const float* bias;    /* [n] fp32, DS_EPI_BIAS */
+  const void* residual; /* same layout and strides as C, DS_EPI_RESIDUAL */
+  void* c2;             /* DS_EPI_GELU second output / DS_EPI_DGELU aux input, layout of C */
+} ds_gemm_desc;
+int ds_gemm(const ds_gemm_desc* d, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * LayerNorm over the last axis, y = (x - mean) * rsqrt(var + eps) * gamma + beta,
+ * biased variance.  Replaces layer_norm() at modeling_slice.py:152-155
+ * (tf.contrib.layers.layer_norm, eps 1e-12) and xlnet/layers/layer_normalization.py:69-78.
+ * stats receives (mean, rstd) per row for the backward pass. */
+int ds_layernorm_fwd(int dtype, int rows, int cols, const void* x, const float* gamma,
+                     const float* beta, float eps, void* y, float* stats, void* stream);
+/* dx = LN backward; d_gamma/d_beta (fp32, [cols]) are accumulated (+=); d_colsum (nullable,
+ * fp32 [cols]) += column sums of dx (the bias gradient of the dense layer that fed x);
+ * dx_add (nullable) is added to dx before it is written (gradient of a residual branch). */
+int ds_layernorm_bwd(int dtype, int rows, int cols, const void* dy, const void* x,
+                     const float* gamma, const float* stats, const void* dx_add, void* dx,
+                     float* d_gamma, float* d_beta, float* d_colsum, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Softmax over the last axis of fp32 scores [batch*heads*q, k]:
+ *   p = softmax(scores * scale + (1 - key_mask[b][j]) * mask_value)
+ * Replaces modeling_slice.py:499-518 (scale 1/sqrt(d), mask_value -10000).
+ * key_mask is [batch, k] fp32 of 0/1 or NULL. p has element type dtype. */
+int ds_softmax_fwd(int dtype, int batch, int heads, int q, int k, const float* scores,
+                   float scale, const float* key_mask, float mask_value, void* p, void* stream);
+/* ds = scale * p * (dp - sum_j dp*p), dp fp32, ds element type dtype */
+int ds_softmax_bwd(int dtype, int64_t rows, int k, const void* p, const float* dp, float scale,
+                   void* ds, void* stream);
+
+/* Column sums: out[n] (fp32) += sum_m x[m][n]; the bias gradient of tf.layers.dense. */
+int ds_colsum_accum(int dtype, int rows, int cols, const void* x, int64_t ldx, float* out,
+                    void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Stage handle: the explicit form of what the reference's unrolled graph implies.
+ * ds_stage_forward(slot) = stages[k](prev_output) for every k the planner put on this
+ * device (bert/models/bert/bert.py:437-456); ds_stage_backward(slot) =
+ * tf.gradients(ys, [prev_y] + vars_i, grad_ys) of bert/graph.py:110-123 with the
+ * accumulation of :145-161 fused in (master grads are updated in place). */
+#define DS_STAGE_BERT 0
+
+typedef struct ds_stage_cfg {
+  int kind;        /* DS_STAGE_* */
+  int dtype;       /* compute type: DS_F32 or DS_BF16; master weights/grads are always fp32 */
+  int num_layers;  /* encoder layers on this stage */
+  int hidden, heads, ffn;
+  int batch, seq;  /* micro-batch shape; activations are [batch*seq, hidden] */
+  int with_embedding; /* 1: the stage starts at token ids (embedding_stage, modeling_slice.py:794) */
+  int vocab, type_vocab, max_pos;
+  float ln_eps;
+  int stash_slots; /* K: in-flight micro-batches (S - i, bert/graph.py:129) */
+  int first_layer; /* index of this stage's first encoder layer in the whole model (names only) */
+  int reserved[7];
+} ds_stage_cfg;
+
+typedef struct ds_stage ds_stage;
+
+int ds_stage_create(const ds_stage_cfg* cfg, void* stream, ds_stage** out);
+int ds_stage_destroy(ds_stage* h);
+/* Number of weight tensors and, per tensor, its name (reference variable scope,
+ * modeling_slice.py:945-996) and element count. name_buf is host memory. */
+int ds_stage_num_weights(const ds_stage* h);
+int ds_stage_weight_info(const ds_stage* h, int i, char* name_buf, size_t name_cap, int64_t* numel,
+                         int64_t* rows, int64_t* cols);
+/* weights[i] / master_grads[i]: fp32 device tensors in ds_stage_weight_info order (host arrays of
+ * device pointers).  The handle keeps the pointers; it never frees them. */
+int ds_stage_bind_weights(ds_stage* h, int n, const void* const* weights, void* const* master_grads);
+/* Refresh the compute copies (bf16 casts, fused QKV packing) after the master weights changed. */
+int ds_stage_refresh_weights(ds_stage* h);
+/* key_mask: [batch, seq] fp32 0/1 input_mask for this slot's micro-batch, or NULL (all ones). */
+int ds_stage_forward(ds_stage* h, int slot, const void* in, const float* key_mask, void* out);
+/* token_type_ids [batch, seq] int32 for the micro-batch that will be forwarded into `slot`
+ * (segment_ids of bert/models/bert/bert.py:390); NULL or never called: all zeros
+ * (modeling_slice.py:785-786).  Only for stages with an embedding. */
+int ds_stage_set_token_types(ds_stage* h, int slot, const int32_t* token_type_ids);
+/* d_in may be NULL for a first stage (bert/graph.py:121 takes no input gradient there). */
+int ds_stage_backward(ds_stage* h, int slot, const void* d_out, void* d_in);
+size_t ds_stage_workspace_bytes(const ds_stage* h);
+size_t ds_stage_stash_bytes(const ds_stage* h, int slots);
+int ds_stage_sync(ds_stage* h);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DAPPLE_STAGE_H */

@@ -1,0 +1,182 @@
+"""Per-kernel parity through the C ABI against fp64 host arithmetic.
+
+Tolerances: fp32 kernels 1e-4 relative (1e-5 where only summation order differs);
+bf16 kernels 2e-2 relative to the fp32/fp64 result on the same bf16-rounded inputs.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from dapple_amd import ops
+from dapple_amd._lib import (DS_EPI_ACCUM, DS_EPI_BIAS, DS_EPI_DGELU, DS_EPI_GELU, DS_EPI_OUT_F32, DS_EPI_RELU,
+                             DS_EPI_RESIDUAL, DS_K_MAJOR, DS_MN_MAJOR)
+from oracle import bert as ob
+from util import assert_close, dev
+
+pytestmark = pytest.mark.gpu
+DT = {"fp32": torch.float32, "bf16": torch.bfloat16}
+TOL = {"fp32": 1e-5, "bf16": 1e-2}
+
+
+def rng(seed):
+    return np.random.Generator(np.random.PCG64(seed))
+
+
+@pytest.mark.parametrize("n", [0, 1, 5, 1024, 4099, 12596224])
+@pytest.mark.parametrize("gdt", ["fp32", "bf16"])
+def test_grad_accumulate_bit_exact(n, gdt):
+    r = rng(n + 1)
+    acc = r.standard_normal(n).astype(np.float32)
+    gs = [r.standard_normal(n).astype(np.float32) for _ in range(3)]
+    a = dev(acc)
+    want = torch.from_numpy(acc.copy())
+    for g in gs:
+        gd = dev(g, DT[gdt])
+        ops.grad_accumulate(a, gd)
+        want += gd.cpu().to(torch.float32)          # exact: fp32 add of the same operands, same order
+    assert torch.equal(a.cpu(), want)
+
+
+def test_grad_accumulate_rejects_bad_arguments():
+    a = torch.zeros(8, device="cuda")
+    with pytest.raises(ValueError):
+        ops.grad_accumulate(a, torch.zeros(9, device="cuda"))
+    with pytest.raises(ValueError):
+        ops.grad_accumulate(a[1:], torch.zeros(7, device="cuda"))       # not 16-byte aligned
+
+
+def test_cast_round_trip():
+    x = dev(rng(3).standard_normal(100003).astype(np.float32))
+    b = ops.cast_to_bf16(x)
+    assert torch.equal(b.cpu(), x.cpu().to(torch.bfloat16))
+    assert torch.equal(ops.cast_to_f32(b).cpu(), b.cpu().to(torch.float32))
+
+
+SHAPES = [(128, 128, 64), (256, 384, 128), (1024, 1024, 1024), (72, 40, 24), (8, 8, 8), (200, 136, 72), (64, 3072, 256)]
+
+
+@pytest.mark.parametrize("dt", ["fp32", "bf16"])
+@pytest.mark.parametrize("am,bm", [(0, 0), (0, 1), (1, 1), (1, 0)])
+@pytest.mark.parametrize("m,n,k", SHAPES)
+def test_gemm_layouts(dt, am, bm, m, n, k):
+    r = rng(m * 7 + n * 3 + k + am * 2 + bm)
+    A = r.standard_normal((m, k)).astype(np.float32)
+    B = r.standard_normal((n, k)).astype(np.float32)
+    a = dev(A if am == DS_K_MAJOR else A.T, DT[dt])
+    b = dev(B if bm == DS_K_MAJOR else B.T, DT[dt])
+    c = torch.full((m, n), float("nan"), dtype=DT[dt], device="cuda")
+    ops.gemm(a, b, c, m, n, k, am, bm)
+    Ar = (a if am == DS_K_MAJOR else a.T).cpu().double()
+    Br = (b if bm == DS_K_MAJOR else b.T).cpu().double()
+    assert_close(c, Ar @ Br.T, TOL[dt], "gemm")
+
+
+@pytest.mark.parametrize("dt", ["fp32", "bf16"])
+def test_gemm_epilogues(dt):
+    m, n, k = 192, 160, 96
+    r = rng(5)
+    x = dev(r.standard_normal((m, k)), DT[dt])
+    w = dev(r.standard_normal((k, n)) * 0.2, DT[dt])
+    bias = dev(r.standard_normal(n), torch.float32)
+    res = dev(r.standard_normal((m, n)), DT[dt])
+    ref = x.cpu().double() @ w.cpu().double() + bias.cpu().double()
+    y = ops.dense(x, w, bias, residual=res)
+    assert_close(y, ref + res.cpu().double(), TOL[dt], "bias+residual")
+    pre, act = ops.dense(x, w, bias, gelu=True)
+    assert_close(pre, ref, TOL[dt], "pre-gelu")
+    assert_close(act, ob.gelu(ref), TOL[dt], "gelu")
+    # relu
+    c = torch.empty(m, n, dtype=DT[dt], device="cuda")
+    ops.gemm(x, w, c, m, n, k, DS_K_MAJOR, DS_MN_MAJOR, flags=DS_EPI_BIAS | DS_EPI_RELU, bias=bias)
+    assert_close(c, ref.clamp(min=0), TOL[dt], "relu")
+    # dgelu: c = (x w) * gelu'(aux)
+    aux = dev(r.standard_normal((m, n)), DT[dt])
+    ops.gemm(x, w, c, m, n, k, DS_K_MAJOR, DS_MN_MAJOR, flags=DS_EPI_DGELU, c2=aux)
+    a64 = aux.cpu().double().requires_grad_(True)
+    (gp,) = torch.autograd.grad(ob.gelu(a64).sum(), a64)
+    assert_close(c, (x.cpu().double() @ w.cpu().double()) * gp, TOL[dt], "dgelu")
+    # fp32 output and accumulate (wgrad form: both operands MN-major), twice -> 2x + initial
+    acc0 = r.standard_normal((k, n)).astype(np.float32)
+    acc = dev(acc0)
+    dy = dev(r.standard_normal((m, n)), DT[dt])
+    for _ in range(2):
+        ops.gemm(x, dy, acc, k, n, m, DS_MN_MAJOR, DS_MN_MAJOR, lda=k, ldb=n, ldc=n, flags=DS_EPI_ACCUM)
+    assert_close(acc, torch.from_numpy(acc0).double() + 2 * (x.cpu().double().T @ dy.cpu().double()), 1e-5, "accum")
+    out32 = torch.empty(m, n, dtype=torch.float32, device="cuda")
+    ops.gemm(x, w, out32, m, n, k, DS_K_MAJOR, DS_MN_MAJOR, flags=DS_EPI_OUT_F32, alpha=0.5)
+    assert_close(out32, 0.5 * (x.cpu().double() @ w.cpu().double()), 1e-5, "out_f32 alpha")
+
+
+@pytest.mark.parametrize("dt", ["fp32", "bf16"])
+def test_gemm_batched_head_views(dt):
+    B, N, S, D = 2, 4, 32, 16
+    H = N * D
+    r = rng(9)
+    qkv = dev(r.standard_normal((B * S, 3 * H)), DT[dt])
+    scores = torch.empty(B, N, S, S, dtype=torch.float32, device="cuda")
+    kview = qkv.view(-1)[H:]
+    ops.gemm(qkv, kview, scores, S, S, D, DS_K_MAJOR, DS_K_MAJOR, lda=3 * H, ldb=3 * H, ldc=S, flags=DS_EPI_OUT_F32,
+             batch=B * N, batch_inner=N, a_strides=(S * 3 * H, D), b_strides=(S * 3 * H, D), c_strides=(N * S * S, S * S))
+    q = qkv[:, :H].cpu().double().reshape(B, S, N, D).permute(0, 2, 1, 3)
+    k = qkv[:, H:2 * H].cpu().double().reshape(B, S, N, D).permute(0, 2, 1, 3)
+    assert_close(scores, q @ k.transpose(-1, -2), 1e-5, "scores")
+
+
+@pytest.mark.parametrize("dt", ["fp32", "bf16"])
+@pytest.mark.parametrize("rows,cols", [(7, 64), (256, 1024), (33, 512), (5, 2048)])
+def test_layernorm_fwd_bwd(dt, rows, cols):
+    r = rng(rows + cols)
+    x = dev(r.standard_normal((rows, cols)) * 2 + 0.5, DT[dt])
+    g = dev(1 + 0.2 * r.standard_normal(cols), torch.float32)
+    b = dev(0.3 * r.standard_normal(cols), torch.float32)
+    dy = dev(r.standard_normal((rows, cols)), DT[dt])
+    add = dev(r.standard_normal((rows, cols)), DT[dt])
+    y, stats = ops.layernorm_fwd(x, g, b, 1e-12)
+    x64 = x.cpu().double().requires_grad_(True)
+    g64 = g.cpu().double().requires_grad_(True)
+    b64 = b.cpu().double().requires_grad_(True)
+    ref = ob.layer_norm(x64, g64, b64)
+    tol = 1e-5 if dt == "fp32" else 1e-2
+    assert_close(y, ref, tol, "ln fwd")
+    dx_ref, dg_ref, db_ref = torch.autograd.grad(ref, [x64, g64, b64], dy.cpu().double())
+    dg = torch.ones(cols, device="cuda")
+    db = torch.ones(cols, device="cuda")
+    dcs = torch.ones(cols, device="cuda")
+    dx = ops.layernorm_bwd(dy, x, g, stats, dg, db, dcs, dx_add=add)
+    assert_close(dx, dx_ref + add.cpu().double(), tol, "ln dx")
+    assert_close(dg, dg_ref + 1, 1e-4, "ln dgamma (accumulates)")
+    assert_close(db, db_ref + 1, 1e-4, "ln dbeta")
+    assert_close(dcs, dx_ref.sum(0) + 1, 1e-4 if dt == "fp32" else 1e-2, "ln colsum")
+
+
+@pytest.mark.parametrize("dt", ["fp32", "bf16"])
+@pytest.mark.parametrize("k", [16, 128, 512, 896])
+def test_softmax_fwd_bwd(dt, k):
+    B, N, Q = 2, 3, 5
+    r = rng(k)
+    s = dev(r.standard_normal((B, N, Q, k)) * 3, torch.float32)
+    mask = dev((r.random((B, k)) > 0.3), torch.float32)
+    scale = 0.125
+    p = ops.softmax_fwd(s, scale, mask, -10000.0, DT[dt])
+    s64 = (s.cpu().double() * scale + (1 - mask.cpu().double())[:, None, None, :] * -10000.0).requires_grad_(True)
+    ref = torch.softmax(s64, -1)
+    tol = 1e-5 if dt == "fp32" else 1e-2
+    assert_close(p, ref, tol, "softmax")
+    assert (p.float().sum(-1) - 1).abs().max().item() < (1e-5 if dt == "fp32" else 2e-2)
+    p0 = ops.softmax_fwd(s, scale, None, 0.0, DT[dt])
+    assert_close(p0, torch.softmax(s.cpu().double() * scale, -1), tol, "softmax no mask")
+    dp = dev(r.standard_normal((B, N, Q, k)), torch.float32)
+    ds = ops.softmax_bwd(p, dp, scale)
+    pr = p.cpu().double()
+    want = scale * pr * (dp.cpu().double() - (dp.cpu().double() * pr).sum(-1, keepdim=True))
+    assert_close(ds, want, tol, "softmax bwd")
+
+
+@pytest.mark.parametrize("dt", ["fp32", "bf16"])
+def test_colsum(dt):
+    x = dev(rng(4).standard_normal((1000, 200)), DT[dt])
+    out = torch.ones(200, device="cuda")
+    ops.colsum_accum(x, out)
+    assert_close(out, x.cpu().double().sum(0) + 1, 1e-5, "colsum")
