@@ -304,8 +304,9 @@ __global__ __launch_bounds__(256) void colsum_kernel(int rows, int cols, const T
 
 // =================================================================== C ABI
 extern "C" int ds_grad_accumulate(void* acc, const void* g, size_t n, int g_dtype, void* stream) {
-  DS_CHECK_ARG(acc && g, "ds_grad_accumulate: null pointer");
   DS_CHECK_ARG(g_dtype == DS_F32 || g_dtype == DS_BF16, "ds_grad_accumulate: g_dtype %d", g_dtype);
+  if (n == 0) return DS_OK;  // an empty tensor has no storage to point at
+  DS_CHECK_ARG(acc && g, "ds_grad_accumulate: null pointer");
   DS_CHECK_ARG(ds_aligned16(acc) && ds_aligned16(g), "ds_grad_accumulate: pointers must be 16-byte aligned");
   if (n == 0) return DS_OK;
   hipStream_t s = (hipStream_t)stream;

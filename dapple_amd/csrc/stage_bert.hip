@@ -166,7 +166,7 @@ struct BertStage : ds_stage {
       emb_st = sa.reserve(stats);
     }
     ls.resize(L);
-    size_t next_x = sa.reserve(act);
+    size_t next_x = L ? sa.reserve(act) : 0;
     for (int l = 0; l < L; ++l) {
       LayerStash& t = ls[l];
       t.x = next_x;
@@ -284,7 +284,7 @@ struct BertStage : ds_stage {
       mask = (const float*)(sp + mask_off);
     }
     slot_has_mask[slot] = key_mask != nullptr;
-    char* x0 = sp + ls[0].x;
+    char* x0 = L ? sp + ls[0].x : nullptr;
     if (emb) {
       DS_CHECK_HIP(hipMemcpyAsync(sp + emb_ids, in, (size_t)rows * 4, hipMemcpyDeviceToDevice, stream));
       const int32_t* tt = slot_has_tt[slot] ? (const int32_t*)(sp + emb_tt) : nullptr;

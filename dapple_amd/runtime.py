@@ -69,8 +69,9 @@ class Stage:
             check(self.lib.ds_stage_weight_info(self._h, i, buf, 256, C.byref(numel), C.byref(rows), C.byref(cols)),
                   "ds_stage_weight_info")
             self.weight_names.append(buf.value.decode())
-            self.weight_shapes.append((rows.value, cols.value) if rows.value > 1 or "kernel" in buf.value.decode()
-                                      or "embeddings" in buf.value.decode() else (cols.value,))
+            name = buf.value.decode()
+            vector = name.endswith(("/bias", "/gamma", "/beta"))
+            self.weight_shapes.append((cols.value,) if vector else (rows.value, cols.value))
         self.weights, self.grads = {}, {}
         self.flat_weights = self.flat_grads = None
 

@@ -63,7 +63,10 @@ def run_case(dtype, L, H, N, F, B, S, M, embeddings=None, use_mask=False, K=2, s
             acc[n] = g.clone() if n not in acc else acc[n] + g
     worst = 0.0
     for n in stage.weight_names:
-        mx, l2 = assert_close(stage.grads[n], acc[n], TOL[dtype], "accumulated grad " + n)
+        # the key bias shifts every score of a query row equally, so its gradient is identically 0:
+        # judge it against the size of the query-bias gradient instead of against rounding noise
+        floor = acc[n.replace("/key/", "/query/")].abs().max().item() if n.endswith("/key/bias") else None
+        mx, l2 = assert_close(stage.grads[n], acc[n], TOL[dtype], "accumulated grad " + n, floor=floor)
         worst = max(worst, mx, l2)
     stage.close()
     return worst
