@@ -50,6 +50,8 @@ class StageCfg(C.Structure):
 PROTOTYPES = {
     "ds_last_error": (C.c_char_p, []),
     "ds_build_target": (C.c_char_p, []),
+    "ds_profile_enable": (C.c_int, [C.c_int]),
+    "ds_profile_dump": (C.c_int, [C.c_char_p, C.c_size_t]),
     "ds_grad_accumulate": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]),
     "ds_cast_f32_to_bf16": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "ds_cast_bf16_to_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
@@ -103,6 +105,21 @@ def check(rc, what=""):
         msg = load().ds_last_error().decode("utf-8", "replace")
         kind = {-1: ValueError, -2: DappleError, -3: DappleError}.get(rc, DappleError)
         raise kind("%s failed (%d): %s" % (what or "libdapple_hip call", rc, msg))
+
+
+def profile(on):
+    check(load().ds_profile_enable(1 if on else 0), "ds_profile_enable")
+
+
+def profile_dump():
+    """{tag: (launches, total_ms, total_work, unit)} of the launches since the last dump."""
+    buf = C.create_string_buffer(1 << 16)
+    check(load().ds_profile_dump(buf, len(buf)), "ds_profile_dump")
+    out = {}
+    for line in buf.value.decode().splitlines():
+        tag, n, ms, work, unit = line.split("\t")
+        out[tag] = (int(n), float(ms), float(work), unit)
+    return out
 
 
 def ptr(t):

@@ -10,6 +10,65 @@ void ds_set_error(const char* fmt, ...) {
   va_end(ap);
 }
 
+// ---------------------------------------------------------------- per-launch timing
+#include <map>
+#include <string>
+#include <vector>
+
+namespace {
+struct ProfEntry { std::string tag; const char* unit; double work; hipEvent_t a, b; };
+bool g_prof_on = false;
+std::vector<ProfEntry> g_prof;
+std::vector<hipEvent_t> g_event_pool;
+hipEvent_t take_event() {
+  if (!g_event_pool.empty()) { hipEvent_t e = g_event_pool.back(); g_event_pool.pop_back(); return e; }
+  hipEvent_t e = nullptr;
+  (void)hipEventCreate(&e);
+  return e;
+}
+}  // namespace
+
+ds_prof_scope::ds_prof_scope(hipStream_t s, const char* tag, double work, const char* unit) : on(g_prof_on), stream(s) {
+  if (!on) return;
+  ProfEntry e{tag, unit, work, take_event(), take_event()};
+  (void)hipEventRecord(e.a, s);
+  g_prof.push_back(e);
+}
+ds_prof_scope::~ds_prof_scope() {
+  if (on) (void)hipEventRecord(g_prof.back().b, stream);
+}
+
+extern "C" int ds_profile_enable(int on) {
+  g_prof_on = on != 0;
+  return DS_OK;
+}
+
+// Writes one line per kernel tag: "tag<TAB>launches<TAB>total_ms<TAB>total_work<TAB>unit\n" and clears the log.
+extern "C" int ds_profile_dump(char* buf, size_t cap) {
+  DS_CHECK_ARG(buf != nullptr && cap > 0, "ds_profile_dump: null buffer");
+  struct Agg { long n = 0; double ms = 0, work = 0; const char* unit = ""; };
+  std::map<std::string, Agg> agg;
+  for (ProfEntry& e : g_prof) {
+    DS_CHECK_HIP(hipEventSynchronize(e.b));
+    float ms = 0.f;
+    DS_CHECK_HIP(hipEventElapsedTime(&ms, e.a, e.b));
+    Agg& a = agg[e.tag];
+    a.n++; a.ms += ms; a.work += e.work; a.unit = e.unit;
+    g_event_pool.push_back(e.a);
+    g_event_pool.push_back(e.b);
+  }
+  g_prof.clear();
+  size_t off = 0;
+  buf[0] = 0;
+  for (auto& kv : agg) {
+    const int w = snprintf(buf + off, cap - off, "%s\t%ld\t%.6f\t%.6e\t%s\n", kv.first.c_str(), kv.second.n, kv.second.ms,
+                           kv.second.work, kv.second.unit);
+    if (w < 0 || (size_t)w >= cap - off) { ds_set_error("ds_profile_dump: buffer too small"); return DS_EINVAL; }
+    off += w;
+  }
+  return DS_OK;
+}
+
 extern "C" const char* ds_last_error(void) { return g_err; }
 extern "C" const char* ds_build_target(void) { return "gfx950"; }
 

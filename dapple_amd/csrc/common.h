@@ -43,6 +43,14 @@ void ds_set_error(const char* fmt, ...);
     if (rc_ != DS_OK) return rc_; \
   } while (0)
 
+// ---- optional per-launch timing (host): HIP events around each kernel launch on its own stream
+struct ds_prof_scope {
+  bool on;
+  hipStream_t stream;
+  ds_prof_scope(hipStream_t s, const char* tag, double work, const char* unit);
+  ~ds_prof_scope();
+};
+
 static inline bool ds_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 // ---- device helpers ----

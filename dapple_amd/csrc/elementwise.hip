@@ -310,6 +310,8 @@ extern "C" int ds_grad_accumulate(void* acc, const void* g, size_t n, int g_dtyp
   DS_CHECK_ARG(ds_aligned16(acc) && ds_aligned16(g), "ds_grad_accumulate: pointers must be 16-byte aligned");
   if (n == 0) return DS_OK;
   hipStream_t s = (hipStream_t)stream;
+  ds_prof_scope prof(s, g_dtype == DS_F32 ? "accumulate_kernel<float>" : "accumulate_kernel<bf16>",
+                     (double)n * (g_dtype == DS_F32 ? 12 : 10), "B");
   if (g_dtype == DS_F32) {
     const int grid = grid_for((n + 3) / 4, 256 * 4);
     hipLaunchKernelGGL(accumulate_kernel<float>, dim3(grid), dim3(256), 0, s, (float*)acc, (const float*)g, n);
@@ -324,6 +326,7 @@ extern "C" int ds_grad_accumulate(void* acc, const void* g, size_t n, int g_dtyp
 extern "C" int ds_cast_f32_to_bf16(void* dst, const void* src, size_t n, void* stream) {
   DS_CHECK_ARG(dst && src, "ds_cast_f32_to_bf16: null pointer");
   if (n == 0) return DS_OK;
+  ds_prof_scope prof((hipStream_t)stream, "cast_kernel<bf16,float>", (double)n * 6, "B");
   hipLaunchKernelGGL((cast_kernel<bf16, float>), dim3(grid_for((n + 3) / 4, 256)), dim3(256), 0, (hipStream_t)stream,
                      (bf16*)dst, (const float*)src, n);
   DS_CHECK_LAUNCH();
@@ -332,6 +335,7 @@ extern "C" int ds_cast_f32_to_bf16(void* dst, const void* src, size_t n, void* s
 extern "C" int ds_cast_bf16_to_f32(void* dst, const void* src, size_t n, void* stream) {
   DS_CHECK_ARG(dst && src, "ds_cast_bf16_to_f32: null pointer");
   if (n == 0) return DS_OK;
+  ds_prof_scope prof((hipStream_t)stream, "cast_kernel<float,bf16>", (double)n * 6, "B");
   hipLaunchKernelGGL((cast_kernel<float, bf16>), dim3(grid_for((n + 3) / 4, 256)), dim3(256), 0, (hipStream_t)stream,
                      (float*)dst, (const bf16*)src, n);
   DS_CHECK_LAUNCH();
@@ -354,6 +358,8 @@ static int layernorm_fwd_t(int rows, int cols, const void* x, const float* gamma
   const int vec = Vec16<T>::N;
   const int need = (cols / vec + 63) / 64;
   dim3 grid((rows + 3) / 4);
+  ds_prof_scope prof(s, sizeof(T) == 2 ? "layernorm_fwd_kernel<bf16>" : "layernorm_fwd_kernel<float>",
+                     (double)rows * cols * sizeof(T) * 2, "B");
   DISPATCH_NV(T, need, hipLaunchKernelGGL((layernorm_fwd_kernel<T, NV>), grid, dim3(256), 0, s, rows, cols, (const T*)x,
                                           gamma, beta, eps, (T*)y, stats));
   DS_CHECK_LAUNCH();
@@ -389,6 +395,8 @@ static int layernorm_bwd_t(int rows, int cols, const void* dy, const void* x, co
   if (rpw > 16) rpw = 16;
   dim3 grid((rows + 4 * rpw - 1) / (4 * rpw));
   const size_t lds = 3 * (size_t)cols * sizeof(float);
+  ds_prof_scope prof(s, sizeof(T) == 2 ? "layernorm_bwd_kernel<bf16>" : "layernorm_bwd_kernel<float>",
+                     (double)rows * cols * sizeof(T) * (dx_add ? 4 : 3), "B");
   DISPATCH_NV(T, need, hipLaunchKernelGGL((layernorm_bwd_kernel<T, NV>), grid, dim3(256), lds, s, rows, cols, rpw,
                                           (const T*)dy, (const T*)x, gamma, stats, (const T*)dx_add, (T*)dx, dg, db, dcs));
   DS_CHECK_LAUNCH();
@@ -412,6 +420,8 @@ static int softmax_fwd_t(int64_t rows, int k, int rpb, const float* scores, floa
                          void* p, hipStream_t s) {
   const int need = (k / 4 + 63) / 64;
   dim3 grid((unsigned)((rows + 3) / 4));
+  ds_prof_scope prof(s, sizeof(T) == 2 ? "softmax_fwd_kernel<bf16>" : "softmax_fwd_kernel<float>",
+                     (double)rows * k * (4 + sizeof(T)), "B");
   DISPATCH_NV(T, need, hipLaunchKernelGGL((softmax_fwd_kernel<T, NV>), grid, dim3(256), 0, s, rows, k, rpb, scores, scale,
                                           mask, mv, (T*)p));
   DS_CHECK_LAUNCH();
@@ -434,6 +444,8 @@ template <typename T>
 static int softmax_bwd_t(int64_t rows, int k, const void* p, const float* dp, float scale, void* ds, hipStream_t s) {
   const int need = (k / 4 + 63) / 64;
   dim3 grid((unsigned)((rows + 3) / 4));
+  ds_prof_scope prof(s, sizeof(T) == 2 ? "softmax_bwd_kernel<bf16>" : "softmax_bwd_kernel<float>",
+                     (double)rows * k * (4 + 2 * sizeof(T)), "B");
   DISPATCH_NV(T, need, hipLaunchKernelGGL((softmax_bwd_kernel<T, NV>), grid, dim3(256), 0, s, rows, k, (const T*)p, dp,
                                           scale, (T*)ds));
   DS_CHECK_LAUNCH();
@@ -454,6 +466,8 @@ extern "C" int ds_colsum_accum(int dtype, int rows, int cols, const void* x, int
   DS_CHECK_ARG(rows > 0 && cols > 0 && ldx >= cols && x && out, "ds_colsum_accum: bad argument");
   int rpb = 64;
   dim3 grid((cols + 63) / 64, (rows + rpb - 1) / rpb);
+  ds_prof_scope prof((hipStream_t)stream, dtype == DS_BF16 ? "colsum_kernel<bf16>" : "colsum_kernel<float>",
+                     (double)rows * cols * (dtype == DS_BF16 ? 2 : 4), "B");
   if (dtype == DS_BF16)
     hipLaunchKernelGGL(colsum_kernel<bf16>, grid, dim3(256), 0, (hipStream_t)stream, rows, cols, (const bf16*)x, ldx, rpb, out);
   else

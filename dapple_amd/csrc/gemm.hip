@@ -12,6 +12,8 @@
 //   MN-major operand: [k row][free index contiguous]; 32-byte granule g of row r lives at
 //                     g ^ (((r & 3) << 1) & (granules-1)).  bf16 fragments come from
 //                     ds_read_b64_tr_b16 (a 4x16 transpose per 16 lanes), fp32 from 4-byte loads.
+#include <stdlib.h>
+
 #include "common.h"
 
 namespace {
@@ -48,6 +50,8 @@ struct GemmArgs {
   float alpha;
   int splitk;
   int ktiles_per_split;
+  int grid_m, grid_n;
+  int vec_epi;
 };
 
 __device__ __forceinline__ int kmajor_off(int row, int chunk) { return row * 128 + ((chunk ^ (row & 7)) << 4); }
@@ -133,6 +137,158 @@ template <typename T, int W, int MAJOR> struct OperandTile {
   }
 };
 
+template <typename T, int BM, int BN>
+__device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, f32x16 (&acc)[BM / 64][BN / 64], int m0, int n0, int wm,
+                                              int wn, int lane, int64_t c_off) {
+  constexpr int TM = BM / 64, TN = BN / 64;
+  // epilogue: lane holds column (lane & 31), rows (e/4)*8 + (lane>>5)*4 + (e&3) of each 32x32 tile
+  const int flags = p.flags;
+  const bool out_f32 = (flags & (DS_EPI_OUT_F32 | DS_EPI_ACCUM)) != 0 || sizeof(T) == 4;
+  float* Cf = reinterpret_cast<float*>(p.c) + c_off;
+  T* Ct = reinterpret_cast<T*>(p.c) + c_off;
+  const T* R = reinterpret_cast<const T*>(p.residual) + c_off;
+  T* C2 = reinterpret_cast<T*>(p.c2) + c_off;
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int col = n0 + wn * (BN / 2) + j * 32 + (lane & 31);
+      if (col >= p.n) continue;
+      const float bias = (flags & DS_EPI_BIAS) ? p.bias[col] : 0.f;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = m0 + wm * (BM / 2) + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+        if (row >= p.m) continue;
+        const int64_t idx = (int64_t)row * p.ldc + col;
+        float v = acc[i][j][e] * p.alpha + bias;
+        if (flags & DS_EPI_RESIDUAL) v += to_f32(R[idx]);
+        if (flags & DS_EPI_DGELU) v *= gelu_erf_grad(to_f32(C2[idx]));
+        if (flags & DS_EPI_RELU) v = fmaxf(v, 0.f);
+        if (flags & DS_EPI_ACCUM) {
+          if (p.splitk > 1) atomicAdd(Cf + idx, v); else Cf[idx] += v;
+        } else if (out_f32) {
+          Cf[idx] = v;
+        } else {
+          Ct[idx] = from_f32<T>(v);
+        }
+        if (flags & DS_EPI_GELU) C2[idx] = from_f32<T>(gelu_erf(v));
+      }
+    }
+}
+
+
+// Epilogue through LDS: accumulators (scaled, biased) are parked as fp32 rows in LDS, then every
+// thread handles 8 consecutive columns of one row, so residual / aux reads and C writes are
+// 16-byte vectors that cover whole rows of the tile.  Needs n, ldc and the C-side batch strides
+// to be multiples of 8 and 16-byte aligned bases (checked on the host: GemmArgs::vec_epi).
+template <typename T, int BM, int BN>
+__device__ __forceinline__ void gemm_epilogue_staged(const GemmArgs& p, f32x16 (&acc)[BM / 64][BN / 64], int m0, int n0,
+                                                     int wm, int wn, int lane, int tid, int64_t c_off, char* lds) {
+  constexpr int TM = BM / 64, TN = BN / 64;
+  constexpr int LDW = BN + 4;
+  float* sc = reinterpret_cast<float*>(lds);
+  const int flags = p.flags;
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int cl = wn * (BN / 2) + j * 32 + (lane & 31);
+      const int col = n0 + cl;
+      const float bias = ((flags & DS_EPI_BIAS) && col < p.n) ? p.bias[col] : 0.f;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int rl = wm * (BM / 2) + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+        sc[rl * LDW + cl] = acc[i][j][e] * p.alpha + bias;
+      }
+    }
+  __syncthreads();
+  const bool out_f32 = (flags & (DS_EPI_OUT_F32 | DS_EPI_ACCUM)) != 0 || sizeof(T) == 4;
+  float* Cf = reinterpret_cast<float*>(p.c) + c_off;
+  T* Ct = reinterpret_cast<T*>(p.c) + c_off;
+  const T* R = reinterpret_cast<const T*>(p.residual) + c_off;
+  T* C2 = reinterpret_cast<T*>(p.c2) + c_off;
+  constexpr int VPR = BN / 8;  // 8-column vectors per tile row
+#pragma unroll 2
+  for (int v = tid; v < BM * VPR; v += 256) {
+    const int rl = v / VPR, cl = (v % VPR) * 8;
+    const int row = m0 + rl, col = n0 + cl;
+    if (row >= p.m || col >= p.n) continue;
+    const int64_t idx = (int64_t)row * p.ldc + col;
+    float x[8];
+    {
+      const f32x4 lo = *reinterpret_cast<const f32x4*>(sc + rl * LDW + cl);
+      const f32x4 hi = *reinterpret_cast<const f32x4*>(sc + rl * LDW + cl + 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { x[e] = lo[e]; x[4 + e] = hi[e]; }
+    }
+    if (flags & DS_EPI_RESIDUAL) {
+      if (sizeof(T) == 2) {
+        const bf16x8 r = *reinterpret_cast<const bf16x8*>(R + idx);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] += (float)r[e];
+      } else {
+        const f32x4 r0 = *reinterpret_cast<const f32x4*>(R + idx), r1 = *reinterpret_cast<const f32x4*>(R + idx + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { x[e] += r0[e]; x[4 + e] += r1[e]; }
+      }
+    }
+    if (flags & DS_EPI_DGELU) {
+      if (sizeof(T) == 2) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(C2 + idx);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] *= gelu_erf_grad((float)a[e]);
+      } else {
+        const f32x4 a0 = *reinterpret_cast<const f32x4*>(C2 + idx), a1 = *reinterpret_cast<const f32x4*>(C2 + idx + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { x[e] *= gelu_erf_grad(a0[e]); x[4 + e] *= gelu_erf_grad(a1[e]); }
+      }
+    }
+    if (flags & DS_EPI_RELU) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[e] = fmaxf(x[e], 0.f);
+    }
+    if (flags & DS_EPI_ACCUM) {
+      if (p.splitk > 1) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) atomicAdd(Cf + idx + e, x[e]);
+      } else {
+        f32x4 c0 = *reinterpret_cast<f32x4*>(Cf + idx), c1 = *reinterpret_cast<f32x4*>(Cf + idx + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { c0[e] += x[e]; c1[e] += x[4 + e]; }
+        *reinterpret_cast<f32x4*>(Cf + idx) = c0;
+        *reinterpret_cast<f32x4*>(Cf + idx + 4) = c1;
+      }
+    } else if (out_f32) {
+      f32x4 c0, c1;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { c0[e] = x[e]; c1[e] = x[4 + e]; }
+      *reinterpret_cast<f32x4*>(Cf + idx) = c0;
+      *reinterpret_cast<f32x4*>(Cf + idx + 4) = c1;
+    } else {
+      bf16x8 o;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = (bf16)x[e];
+      *reinterpret_cast<bf16x8*>(reinterpret_cast<bf16*>(p.c) + c_off + idx) = o;
+    }
+    if (flags & DS_EPI_GELU) {
+      if (sizeof(T) == 2) {
+        bf16x8 o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = (bf16)gelu_erf(x[e]);
+        *reinterpret_cast<bf16x8*>(reinterpret_cast<bf16*>(p.c2) + c_off + idx) = o;
+      } else {
+        f32x4 c0, c1;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { c0[e] = gelu_erf(x[e]); c1[e] = gelu_erf(x[4 + e]); }
+        *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.c2) + c_off + idx) = c0;
+        *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.c2) + c_off + idx + 4) = c1;
+      }
+    }
+  }
+  (void)Ct;
+}
+
 template <typename T, int BM, int BN, int AMAJ, int BMAJ>
 __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
   typedef OperandTile<T, BM, AMAJ> TA;
@@ -144,7 +300,18 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  // XCD-aware tile order: consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with
+  // its own L2.  Give every XCD a contiguous run of tile ids, and walk tile ids M-fastest, so
+  // one XCD works on a few whole columns of C tiles and re-reads only its own slice of B from L2.
+  int tile_id;
+  {
+    const int tiles = p.grid_m * p.grid_n;
+    const int w = blockIdx.x;
+    const int per = (tiles + 7) >> 3, tall = (tiles & 7) ? (tiles & 7) : 8;
+    const int xcd = w & 7, local = w >> 3;
+    tile_id = xcd < tall ? xcd * per + local : tall * per + (xcd - tall) * (per - 1) + local;
+  }
+  const int m0 = (tile_id % p.grid_m) * BM, n0 = (tile_id / p.grid_m) * BN;
   const int z = blockIdx.z / p.splitk, ks_id = blockIdx.z % p.splitk;
   const int zo = z / p.batch_inner, zi = z % p.batch_inner;
   const T* A = reinterpret_cast<const T*>(p.a) + zo * p.a_so + zi * p.a_si;
@@ -195,46 +362,262 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
     }
   }
 
-  // epilogue: lane holds column (lane & 31), rows (e/4)*8 + (lane>>5)*4 + (e&3) of each 32x32 tile
-  const int flags = p.flags;
-  const bool out_f32 = (flags & (DS_EPI_OUT_F32 | DS_EPI_ACCUM)) != 0 || sizeof(T) == 4;
-  float* Cf = reinterpret_cast<float*>(p.c) + c_off;
-  T* Ct = reinterpret_cast<T*>(p.c) + c_off;
-  const T* R = reinterpret_cast<const T*>(p.residual) + c_off;
-  T* C2 = reinterpret_cast<T*>(p.c2) + c_off;
+  gemm_epilogue<T, BM, BN>(p, acc, m0, n0, wm, wn, lane, c_off);
+}
+
+
+// LDS fragment reads as inline asm: the compiler's wait-count pass would otherwise put a full
+// vmcnt(0) in front of LDS reads that follow an LDS-DMA load, which serialises the pipeline.
+// lds_wait() is the matching s_waitcnt; it names the fragment registers as in/out operands so
+// that no MFMA using them can be scheduled above it.
+__device__ __forceinline__ uint32_t lds_addr(const void* p) {
+  return (uint32_t)(uintptr_t)((__attribute__((address_space(3))) const char*)p);
+}
+__device__ __forceinline__ void lds_read(bf16x8& f, uint32_t a) { asm volatile("ds_read_b128 %0, %1" : "=v"(f) : "v"(a)); }
+__device__ __forceinline__ void lds_read(f32x4& f, uint32_t a) { asm volatile("ds_read_b128 %0, %1" : "=v"(f) : "v"(a)); }
+__device__ __forceinline__ void lds_read_tr(s16x4& f, uint32_t a) { asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(f) : "v"(a)); }
+__device__ __forceinline__ void lds_read_b32(float& f, uint32_t a) { asm volatile("ds_read_b32 %0, %1" : "=v"(f) : "v"(a)); }
+template <typename F> __device__ __forceinline__ void lds_wait1(F& a) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a)); }
+
+// Registers an LDS read lands in, kept apart from the MFMA operand until lds_wait() has run: any
+// register copy the compiler makes to assemble the operand then happens after the data arrived.
+template <typename T, int MAJOR> struct RawFrag { typename Mma<T>::Frag v; };
+template <> struct RawFrag<bf16, DS_MN_MAJOR> { s16x4 lo, hi; };
+template <> struct RawFrag<float, DS_MN_MAJOR> { float e0, e1, e2, e3; };
+
+template <typename T> __device__ __forceinline__ void lds_wait(RawFrag<T, DS_K_MAJOR>& r) { lds_wait1(r.v); }
+__device__ __forceinline__ void lds_wait(RawFrag<bf16, DS_MN_MAJOR>& r) {
+  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r.lo), "+v"(r.hi));
+}
+__device__ __forceinline__ void lds_wait(RawFrag<float, DS_MN_MAJOR>& r) {
+  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r.e0), "+v"(r.e1), "+v"(r.e2), "+v"(r.e3));
+}
+template <typename T> __device__ __forceinline__ typename Mma<T>::Frag to_frag(const RawFrag<T, DS_K_MAJOR>& r) { return r.v; }
+__device__ __forceinline__ bf16x8 to_frag(const RawFrag<bf16, DS_MN_MAJOR>& r) {
+  union { s16x4 v[2]; bf16x8 f; } u;
+  u.v[0] = r.lo; u.v[1] = r.hi;
+  return u.f;
+}
+__device__ __forceinline__ f32x4 to_frag(const RawFrag<float, DS_MN_MAJOR>& r) {
+  f32x4 f = {r.e0, r.e1, r.e2, r.e3};
+  return f;
+}
+
+// Per-lane byte offsets (inside one operand tile) of the MFMA fragments a wave reads.
+template <typename T, int W, int MAJOR, int NF> struct FragReader {
+  static constexpr int ROW_BYTES = W * (int)sizeof(T);
+  typedef RawFrag<T, MAJOR> Raw;
+  uint32_t off[MAJOR == DS_K_MAJOR ? 4 : NF];
+
+  __device__ __forceinline__ void init(int ft0, int lane) {
+    const int h = lane >> 5;
+    if (MAJOR == DS_K_MAJOR) {
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) off[ks] = kmajor_off(ft0 + (lane & 31), 2 * ks + h);
+    } else if (sizeof(T) == 2) {
+      const int s = lane & 15;
+#pragma unroll
+      for (int i = 0; i < NF; ++i) {
+        const int col = ft0 + i * 32 + (((lane >> 4) & 1) << 4) + ((s & 3) << 2);
+        off[i] = mnmajor_off<ROW_BYTES>(8 * h + (s >> 2), col * 2);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NF; ++i) off[i] = mnmajor_off<ROW_BYTES>(4 * h, (ft0 + i * 32 + (lane & 31)) * 4);
+    }
+  }
+  // issues the reads of fragment i, k-step ks from the tile at LDS byte address `tile`
+  __device__ __forceinline__ void read(RawFrag<T, DS_K_MAJOR>& f, uint32_t tile, int i, int ks) const {
+    lds_read(f.v, tile + off[ks] + i * (32 * 128));
+  }
+  __device__ __forceinline__ void read(RawFrag<bf16, DS_MN_MAJOR>& f, uint32_t tile, int i, int ks) const {
+    // rows r and r+4 (and r+16) share (r & 3), so the swizzle term is the same: constant byte offsets
+    lds_read_tr(f.lo, tile + off[i] + (16 * ks) * ROW_BYTES);
+    lds_read_tr(f.hi, tile + off[i] + (16 * ks + 4) * ROW_BYTES);
+  }
+  __device__ __forceinline__ void read(RawFrag<float, DS_MN_MAJOR>& f, uint32_t tile, int i, int ks) const {
+    // rows 4h..4h+3 differ in (r & 3): redo the granule swizzle per row (off[i] is row 4h, unswizzled)
+    constexpr int NG = ROW_BYTES / 32;
+    const uint32_t base = off[i];
+    const uint32_t g = (base % ROW_BYTES) >> 5, within = base & 31, row0 = base / ROW_BYTES;
+    lds_read_b32(f.e0, tile + (row0 + 8 * ks + 0) * ROW_BYTES + ((g ^ (0 & (NG - 1))) << 5) + within);
+    lds_read_b32(f.e1, tile + (row0 + 8 * ks + 1) * ROW_BYTES + ((g ^ (2 & (NG - 1))) << 5) + within);
+    lds_read_b32(f.e2, tile + (row0 + 8 * ks + 2) * ROW_BYTES + ((g ^ (4 & (NG - 1))) << 5) + within);
+    lds_read_b32(f.e3, tile + (row0 + 8 * ks + 3) * ROW_BYTES + ((g ^ (6 & (NG - 1))) << 5) + within);
+  }
+};
+
+// ------------------------------------------------------------------------------------------
+// Pipelined variant for k % KT == 0: tiles go global -> LDS directly (global_load_lds_dwordx4,
+// no VGPR staging), STAGES k-tiles deep, so several k-tiles of loads are in flight while one is
+// multiplied.  A wave's DMA writes 64 consecutive 16-byte LDS slots, so the swizzle is applied
+// to the global address each lane fetches instead of to the LDS address it stores to.
+// Out-of-range free indices are clamped to the last valid row/vector: they only feed
+// accumulators of rows/columns the epilogue never stores.
+typedef __attribute__((address_space(3))) void* lds_vptr;
+typedef __attribute__((address_space(1))) void* glb_vptr;
+
+template <typename T, int W, int MAJOR> struct DmaTile {
+  static constexpr int VEC = Vec16<T>::N;
+  static constexpr int KT = Mma<T>::KT;
+  static constexpr int NV = W / 32;
+  static constexpr int ROW_BYTES = W * (int)sizeof(T);
+  static constexpr int CPR = ROW_BYTES / 16;
+
+  // per-lane source pointers for k-tile 0; slot i of wave w covers LDS positions (i*4+w)*64 + lane
+  static __device__ __forceinline__ void init(const T* (&src)[NV], const T* base, int64_t ld, int f0, int F, int k0,
+                                              int wave, int lane) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int p = (i * 4 + wave) * 64 + lane;
+      if (MAJOR == DS_K_MAJOR) {
+        const int row = p >> 3, c = (p & 7) ^ (row & 7);
+        int f = f0 + row;
+        if (f > F - 1) f = F - 1;
+        src[i] = base + (int64_t)f * ld + k0 + c * VEC;
+      } else {
+        constexpr int NG = ROW_BYTES / 32;
+        const int r = p / CPR, pc = p % CPR;
+        const int g = (pc >> 1) ^ (((r & 3) << 1) & (NG - 1));
+        int f = f0 + (g * 2 + (pc & 1)) * VEC;
+        if (f > F - VEC) f = F - VEC;
+        src[i] = base + (int64_t)(k0 + r) * ld + f;
+      }
+    }
+  }
+  static __device__ __forceinline__ void issue(const T* (&src)[NV], char* lds, int64_t ld, int wave) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      __builtin_amdgcn_global_load_lds((glb_vptr)src[i], (lds_vptr)(lds + (i * 4 + wave) * 1024), 16, 0, 0);
+      src[i] += (MAJOR == DS_K_MAJOR) ? (int64_t)KT : (int64_t)KT * ld;
+    }
+  }
+};
+
+// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[15:14])
+#define DS_VMCNT(n) (((n) & 15) | (((n) >> 4) << 14) | (7 << 4) | (15 << 8))
+
+template <typename T, int BM, int BN, int AMAJ, int BMAJ, int STAGES>
+__global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
+  typedef OperandTile<T, BM, AMAJ> TA;
+  typedef OperandTile<T, BN, BMAJ> TB;
+  typedef DmaTile<T, BM, AMAJ> DA;
+  typedef DmaTile<T, BN, BMAJ> DB;
+  constexpr int KT = Mma<T>::KT;
+  constexpr int TM = BM / 64, TN = BN / 64;
+  constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE_BYTES = A_BYTES + B_BYTES;
+  constexpr int LPT = DA::NV + DB::NV;  // DMA loads per thread per k-tile
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  int tile_id;
+  {
+    const int tiles = p.grid_m * p.grid_n;
+    const int w = blockIdx.x;
+    const int per = (tiles + 7) >> 3, tall = (tiles & 7) ? (tiles & 7) : 8;
+    const int xcd = w & 7, local = w >> 3;
+    tile_id = xcd < tall ? xcd * per + local : tall * per + (xcd - tall) * (per - 1) + local;
+  }
+  const int m0 = (tile_id % p.grid_m) * BM, n0 = (tile_id / p.grid_m) * BN;
+  const int z = blockIdx.z / p.splitk, ks_id = blockIdx.z % p.splitk;
+  const int zo = z / p.batch_inner, zi = z % p.batch_inner;
+  const T* A = reinterpret_cast<const T*>(p.a) + zo * p.a_so + zi * p.a_si;
+  const T* B = reinterpret_cast<const T*>(p.b) + zo * p.b_so + zi * p.b_si;
+  const int64_t c_off = zo * p.c_so + zi * p.c_si;
+
+  const int kt_begin = ks_id * p.ktiles_per_split;
+  const int kt_total = p.k / KT;
+  int kt_end = kt_begin + p.ktiles_per_split;
+  if (kt_end > kt_total) kt_end = kt_total;
+  const int nkt = kt_end - kt_begin;
+
+  f32x16 acc[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int col = n0 + wn * (BN / 2) + j * 32 + (lane & 31);
-      if (col >= p.n) continue;
-      const float bias = (flags & DS_EPI_BIAS) ? p.bias[col] : 0.f;
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int row = m0 + wm * (BM / 2) + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-        if (row >= p.m) continue;
-        const int64_t idx = (int64_t)row * p.ldc + col;
-        float v = acc[i][j][e] * p.alpha + bias;
-        if (flags & DS_EPI_RESIDUAL) v += to_f32(R[idx]);
-        if (flags & DS_EPI_DGELU) v *= gelu_erf_grad(to_f32(C2[idx]));
-        if (flags & DS_EPI_RELU) v = fmaxf(v, 0.f);
-        if (flags & DS_EPI_ACCUM) {
-          if (p.splitk > 1) atomicAdd(Cf + idx, v); else Cf[idx] += v;
-        } else if (out_f32) {
-          Cf[idx] = v;
-        } else {
-          Ct[idx] = from_f32<T>(v);
-        }
-        if (flags & DS_EPI_GELU) C2[idx] = from_f32<T>(gelu_erf(v));
-      }
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  const T* sa_src[DA::NV];
+  const T* sb_src[DB::NV];
+  DA::init(sa_src, A, p.lda, m0, p.m, kt_begin * KT, wave, lane);
+  DB::init(sb_src, B, p.ldb, n0, p.n, kt_begin * KT, wave, lane);
+#pragma unroll
+  for (int s = 0; s < STAGES - 1; ++s) {
+    if (s < nkt) {
+      DA::issue(sa_src, lds + s * STAGE_BYTES, p.lda, wave);
+      DB::issue(sb_src, lds + s * STAGE_BYTES + A_BYTES, p.ldb, wave);
     }
+  }
+  FragReader<T, BM, AMAJ, TM> ra;
+  FragReader<T, BN, BMAJ, TN> rb;
+  ra.init(wm * (BM / 2), lane);
+  rb.init(wn * (BN / 2), lane);
+  const uint32_t lds0 = lds_addr(lds);
+  int buf = 0;  // kt % STAGES
+  for (int kt = 0; kt < nkt; ++kt) {
+    // tile kt is complete once at most the tiles issued after it are outstanding
+    if (kt + STAGES - 2 < nkt) __builtin_amdgcn_s_waitcnt(DS_VMCNT(LPT * (STAGES - 2)));
+    else __builtin_amdgcn_s_waitcnt(DS_VMCNT(0));
+    __builtin_amdgcn_s_barrier();
+    if (kt + STAGES - 1 < nkt) {
+      int nb = buf + STAGES - 1;
+      if (nb >= STAGES) nb -= STAGES;
+      DA::issue(sa_src, lds + nb * STAGE_BYTES, p.lda, wave);
+      DB::issue(sb_src, lds + nb * STAGE_BYTES + A_BYTES, p.ldb, wave);
+    }
+    const uint32_t sa = lds0 + buf * STAGE_BYTES, sb = sa + A_BYTES;
+    RawFrag<T, AMAJ> fa[2][TM];
+    RawFrag<T, BMAJ> fb[2][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) ra.read(fa[0][i], sa, i, 0);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) rb.read(fb[0][j], sb, j, 0);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const int cur = ks & 1, nxt = cur ^ 1;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) lds_wait(fa[cur][i]);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) lds_wait(fb[cur][j]);
+      if (ks < 3) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) ra.read(fa[nxt][i], sa, i, ks + 1);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) rb.read(fb[nxt][j], sb, j, ks + 1);
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) Mma<T>::mma(acc[i][j], to_frag(fa[cur][i]), to_frag(fb[cur][j]));
+    }
+    if (++buf == STAGES) buf = 0;
+  }
+  if (p.vec_epi) gemm_epilogue_staged<T, BM, BN>(p, acc, m0, n0, wm, wn, lane, tid, c_off, lds);
+  else gemm_epilogue<T, BM, BN>(p, acc, m0, n0, wm, wn, lane, c_off);
 }
 
 template <typename T, int BM, int BN, int AMAJ, int BMAJ>
-int launch_cfg(const GemmArgs& a, int batch, hipStream_t stream) {
-  dim3 grid((a.n + BN - 1) / BN, (a.m + BM - 1) / BM, batch * a.splitk);
-  const size_t lds = 2 * (BM + BN) * 128;
-  hipLaunchKernelGGL((gemm_kernel<T, BM, BN, AMAJ, BMAJ>), grid, dim3(256), lds, stream, a);
+int launch_cfg(GemmArgs a, int batch, hipStream_t stream) {
+  a.grid_m = (a.m + BM - 1) / BM;
+  a.grid_n = (a.n + BN - 1) / BN;
+  dim3 grid(a.grid_m * a.grid_n, 1, batch * a.splitk);
+  if (a.k % Mma<T>::KT == 0) {
+    constexpr int STAGES = 4;
+    constexpr size_t lds = (size_t)STAGES * (BM + BN) * 128;
+    static bool attr_set = false;
+    if (!attr_set) {
+      DS_CHECK_HIP(hipFuncSetAttribute((const void*)gemm_dma_kernel<T, BM, BN, AMAJ, BMAJ, STAGES>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      attr_set = true;
+    }
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, AMAJ, BMAJ, STAGES>), grid, dim3(256), lds, stream, a);
+  } else {
+    const size_t lds = 2 * (BM + BN) * 128;
+    hipLaunchKernelGGL((gemm_kernel<T, BM, BN, AMAJ, BMAJ>), grid, dim3(256), lds, stream, a);
+  }
   DS_CHECK_LAUNCH();
   return DS_OK;
 }
@@ -258,24 +641,22 @@ int launch_major(const GemmArgs& a, int batch, int tile, int am, int bm, hipStre
 
 }  // namespace
 
-// Picks the tile shape (and split-K for accumulating outputs) that keeps the 256 CUs busiest.
+// Picks the tile shape.  Measured on MI355X (bf16, 4-stage pipeline): one k-tile costs about 0.6 us in
+// a 128x128 block alone on its CU, 1.06 us in two co-resident 128x64 blocks and 0.45 us in two
+// co-resident 64x64 blocks; the k-loop repeats once per round of resident blocks.  Split-K is never
+// chosen: its atomic epilogue was slower than the under-filled grid on every shape tried.
 static void choose_tiling(int m, int n, int k, int kt, int batch, bool can_split, int* tile, int* splitk) {
   static const int bm[3] = {128, 128, 64}, bn[3] = {128, 64, 64};
-  static const double eff[3] = {1.0, 0.8, 0.55};
-  const double slots = 512.0;  // 256 CUs x 2 resident blocks
+  static const double slots[3] = {256, 512, 512}, t_round[3] = {0.6, 1.06, 0.45};
+  (void)k; (void)kt; (void)can_split;
   double best = 1e300;
   *tile = 0;
   *splitk = 1;
-  const int ktiles = (k + kt - 1) / kt;
   for (int t = 0; t < 3; ++t) {
     const double blocks = (double)((m + bm[t] - 1) / bm[t]) * ((n + bn[t] - 1) / bn[t]) * batch;
-    for (int s = 1; s <= (can_split ? 8 : 1); s *= 2) {
-      if (s > ktiles) break;
-      const double rounds = (double)((long long)((blocks * s + slots - 1) / slots));
-      const double per_block = (double)bm[t] * bn[t] * ((ktiles + s - 1) / s) / eff[t] + 4.0 * bm[t] * bn[t] / 64;
-      const double cost = rounds * per_block;
-      if (cost < best) { best = cost; *tile = t; *splitk = s; }
-    }
+    const double rounds = (double)((long long)((blocks + slots[t] - 1) / slots[t]));
+    const double cost = rounds * t_round[t];
+    if (cost < best) { best = cost; *tile = t; }
   }
 }
 
@@ -323,13 +704,27 @@ extern "C" int ds_gemm(const ds_gemm_desc* d, void* stream) {
   a.c_so = d->c_stride_outer; a.c_si = d->c_stride_inner;
   a.flags = f;
   a.alpha = d->alpha;
+  a.vec_epi = d->n % 8 == 0 && d->ldc % 8 == 0 && d->c_stride_outer % 8 == 0 && d->c_stride_inner % 8 == 0 &&
+              ds_aligned16(d->c) && ds_aligned16(d->residual) && ds_aligned16(d->c2);
   const int kt = d->dtype == DS_BF16 ? 64 : 32;
   int tile, splitk;
   choose_tiling(d->m, d->n, d->k, kt, batch, (f & DS_EPI_ACCUM) != 0, &tile, &splitk);
+  {  // tuning overrides: DS_GEMM_TILE=0|1|2, DS_GEMM_SPLITK=n (accumulating outputs only)
+    static const char* env_tile = getenv("DS_GEMM_TILE");
+    static const char* env_split = getenv("DS_GEMM_SPLITK");
+    if (env_tile) tile = atoi(env_tile) % 3;
+    if (env_split && (f & DS_EPI_ACCUM)) splitk = atoi(env_split) > 0 ? atoi(env_split) : 1;
+  }
   const int ktiles = (d->k + kt - 1) / kt;
+  if (splitk > 1) a.vec_epi = 0;  // atomics want neighbouring lanes on neighbouring addresses
   a.splitk = splitk;
   a.ktiles_per_split = (ktiles + splitk - 1) / splitk;
   hipStream_t s = (hipStream_t)stream;
+  static const int tbm[3] = {128, 128, 64}, tbn[3] = {128, 64, 64};
+  char tag[96];
+  snprintf(tag, sizeof(tag), "gemm_kernel<%s,%d,%d,%s,%s>", d->dtype == DS_BF16 ? "bf16" : "float", tbm[tile], tbn[tile],
+           d->a_major == DS_K_MAJOR ? "K" : "MN", d->b_major == DS_K_MAJOR ? "K" : "MN");
+  ds_prof_scope prof(s, tag, 2.0 * d->m * d->n * d->k * batch, "FLOP");
   if (d->dtype == DS_BF16) return launch_major<bf16>(a, batch, tile, d->a_major, d->b_major, s);
   return launch_major<float>(a, batch, tile, d->a_major, d->b_major, s);
 }

@@ -48,6 +48,14 @@ const char* ds_last_error(void);
 /* Version / build probe; returns the gfx target the library was built for ("gfx950"). */
 const char* ds_build_target(void);
 
+/* Per-launch timing for roofline reports (no counterpart in the reference, which relied on
+ * tf.train.ProfilerHook, bert/utils/hooks/hooks_helper.py:72-88).  While enabled, every kernel
+ * launch made through this library is bracketed by HIP events on the stream it is launched on.
+ * ds_profile_dump writes "tag<TAB>launches<TAB>total_ms<TAB>total_work<TAB>unit" lines (work =
+ * algorithmic FLOP or bytes) into a host buffer and clears the log.  Not thread safe. */
+int ds_profile_enable(int on);
+int ds_profile_dump(char* buf, size_t cap);
+
 /* ---------------------------------------------------------------------------
  * Gradient accumulation: acc[i] (fp32) += g[i], i < n.
  * Replaces tf.accumulate_n(grad_i_set) at bert/graph.py:159 (and its copies at
