@@ -281,23 +281,35 @@ __global__ __launch_bounds__(256) void softmax_bwd_kernel(int64_t rows, int k, c
 }
 
 // ------------------------------------------------------------------ column sums
-// Block = 64 columns x 4 row groups; each thread strides down the rows, LDS-combines, then
-// one atomicAdd per column.
+// Block = 4 row groups x 64 lanes; a lane owns one 16-byte vector of columns and strides down the
+// rows of its group; groups combine through LDS, then one atomicAdd per column.
 template <typename T>
 __global__ __launch_bounds__(256) void colsum_kernel(int rows, int cols, const T* __restrict__ x, int64_t ldx,
                                                     int rows_per_block, float* __restrict__ out) {
-  __shared__ float red[4][64];
-  const int c = blockIdx.x * 64 + (threadIdx.x & 63);
-  const int g = threadIdx.x >> 6;
+  constexpr int VEC = Vec16<T>::N;
+  typedef typename Vec16<T>::type V;
+  __shared__ float red[4][64 * VEC];
+  const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
+  const int c = (blockIdx.x * 64 + lane) * VEC;
   const int r0 = blockIdx.y * rows_per_block;
   int r1 = r0 + rows_per_block;
   if (r1 > rows) r1 = rows;
-  float s = 0.f;
+  float s[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) s[e] = 0.f;
   if (c < cols)
-    for (int r = r0 + g; r < r1; r += 4) s += to_f32(x[(int64_t)r * ldx + c]);
-  red[g][threadIdx.x & 63] = s;
+    for (int r = r0 + g; r < r1; r += 4) {
+      const V v = *reinterpret_cast<const V*>(x + (int64_t)r * ldx + c);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) s[e] += to_f32(v[e]);
+    }
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) red[g][lane * VEC + e] = s[e];
   __syncthreads();
-  if (g == 0 && c < cols) atomicAdd(out + c, red[0][threadIdx.x] + red[1][threadIdx.x] + red[2][threadIdx.x] + red[3][threadIdx.x]);
+  for (int i = threadIdx.x; i < 64 * VEC; i += 256) {
+    const int cc = blockIdx.x * 64 * VEC + i;
+    if (cc < cols) atomicAdd(out + cc, red[0][i] + red[1][i] + red[2][i] + red[3][i]);
+  }
 }
 
 }  // namespace
@@ -389,8 +401,8 @@ static int layernorm_bwd_t(int rows, int cols, const void* dy, const void* x, co
                            const void* dx_add, void* dx, float* dg, float* db, float* dcs, hipStream_t s) {
   const int vec = Vec16<T>::N;
   const int need = (cols / vec + 63) / 64;
-  // aim for ~512 blocks of 4 waves; each wave walks rows_per_wave rows
-  int rpw = rows / (512 * 4);
+  // aim for ~64 blocks of 4 waves (the column atomics at the end cost more than the row work)
+  int rpw = rows / (64 * 4);
   if (rpw < 1) rpw = 1;
   if (rpw > 16) rpw = 16;
   dim3 grid((rows + 4 * rpw - 1) / (4 * rpw));
@@ -464,8 +476,10 @@ extern "C" int ds_softmax_bwd(int dtype, int64_t rows, int k, const void* p, con
 extern "C" int ds_colsum_accum(int dtype, int rows, int cols, const void* x, int64_t ldx, float* out, void* stream) {
   DS_CHECK_ARG(dtype == DS_F32 || dtype == DS_BF16, "ds_colsum_accum: dtype %d", dtype);
   DS_CHECK_ARG(rows > 0 && cols > 0 && ldx >= cols && x && out, "ds_colsum_accum: bad argument");
-  int rpb = 64;
-  dim3 grid((cols + 63) / 64, (rows + rpb - 1) / rpb);
+  const int vec = dtype == DS_BF16 ? 8 : 4;
+  DS_CHECK_ARG(cols % vec == 0 && ldx % vec == 0 && ds_aligned16(x), "ds_colsum_accum: cols and ldx must be multiples of %d and x 16-byte aligned", vec);
+  int rpb = 32;
+  dim3 grid((cols + 64 * vec - 1) / (64 * vec), (rows + rpb - 1) / rpb);
   ds_prof_scope prof((hipStream_t)stream, dtype == DS_BF16 ? "colsum_kernel<bf16>" : "colsum_kernel<float>",
                      (double)rows * cols * (dtype == DS_BF16 ? 2 : 4), "B");
   if (dtype == DS_BF16)

@@ -384,9 +384,24 @@ struct BertStage : ds_stage {
       DS_PROPAGATE(gemm_heads(DS_MN_MAJOR, DS_MN_MAJOR, S, D, S, dsm, S, soP, siP, q, 3 * H, so3, D,
                               dqkv + (size_t)H * esz, 3 * H, so3, D, 0));
       // projection gradients: three [H,H] kernels and three biases fed by the columns of dqkv
-      for (int j = 0; j < 3; ++j) {
-        DS_PROPAGATE(ds_colsum_accum(dtype, rows, H, dqkv + (size_t)j * H * esz, 3 * H, g[b + B_Q + j], stream));
-        DS_PROPAGATE(gemm_wgrad(rows, H, H, sp + t.x, H, dqkv + (size_t)j * H * esz, 3 * H, g[b + W_Q + j], H));
+      const bool adjacent = g[b + B_K] == g[b + B_Q] + H && g[b + B_V] == g[b + B_Q] + 2 * H &&
+                            g[b + W_K] == g[b + W_Q] + (size_t)H * H && g[b + W_V] == g[b + W_Q] + (size_t)2 * H * H;
+      if (adjacent) {
+        // q, k, v master gradients lie back to back: one column sum over [rows, 3H] and one GEMM batched
+        // over the three column blocks of dqkv
+        DS_PROPAGATE(ds_colsum_accum(dtype, rows, 3 * H, dqkv, 3 * H, g[b + B_Q], stream));
+        ds_gemm_desc d;
+        memset(&d, 0, sizeof(d));
+        d.dtype = dtype; d.a_major = DS_MN_MAJOR; d.b_major = DS_MN_MAJOR;
+        d.m = H; d.n = H; d.k = rows; d.lda = H; d.ldb = 3 * H; d.ldc = H; d.batch = 3; d.batch_inner = 3;
+        d.b_stride_inner = H; d.c_stride_inner = (int64_t)H * H;
+        d.flags = DS_EPI_ACCUM; d.alpha = 1.f; d.a = sp + t.x; d.b = dqkv; d.c = g[b + W_Q];
+        DS_PROPAGATE(ds_gemm(&d, stream));
+      } else {
+        for (int j = 0; j < 3; ++j) {
+          DS_PROPAGATE(ds_colsum_accum(dtype, rows, H, dqkv + (size_t)j * H * esz, 3 * H, g[b + B_Q + j], stream));
+          DS_PROPAGATE(gemm_wgrad(rows, H, H, sp + t.x, H, dqkv + (size_t)j * H * esz, 3 * H, g[b + W_Q + j], H));
+        }
       }
       // dx = dqkv Wqkv^T + dz1 (x also feeds the residual into z1)
       const bool first = (l == 0);
