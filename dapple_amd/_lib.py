@@ -12,8 +12,8 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libdapple_hip.so")
 DS_F32, DS_BF16 = 0, 1
 DS_K_MAJOR, DS_MN_MAJOR = 0, 1
 DS_EPI_BIAS, DS_EPI_RESIDUAL, DS_EPI_GELU, DS_EPI_DGELU = 1, 2, 4, 8
-DS_EPI_OUT_F32, DS_EPI_ACCUM, DS_EPI_RELU = 16, 32, 64
-DS_STAGE_BERT = 0
+DS_EPI_OUT_F32, DS_EPI_ACCUM, DS_EPI_RELU, DS_EPI_MASK = 16, 32, 64, 128
+DS_STAGE_BERT, DS_STAGE_VGG19 = 0, 1
 
 
 class DappleError(RuntimeError):
@@ -46,6 +46,14 @@ class StageCfg(C.Structure):
     ]
 
 
+class VggCfg(C.Structure):
+    _fields_ = [
+        ("dtype", C.c_int), ("batch", C.c_int), ("height", C.c_int), ("width", C.c_int), ("in_channels", C.c_int),
+        ("num_ops", C.c_int), ("ops", C.c_int * 40), ("stash_slots", C.c_int), ("need_input_grad", C.c_int),
+        ("reserved", C.c_int * 8),
+    ]
+
+
 # name -> (restype, argtypes); every symbol include/dapple_stage.h declares
 PROTOTYPES = {
     "ds_last_error": (C.c_char_p, []),
@@ -65,6 +73,15 @@ PROTOTYPES = {
     "ds_softmax_bwd": (C.c_int, [C.c_int, C.c_int64, C.c_int, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p,
                                  C.c_void_p]),
     "ds_colsum_accum": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]),
+    "ds_conv3x3_fwd": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p,
+                                 C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "ds_conv3x3_wgrad": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
+                                   C.c_void_p, C.c_void_p]),
+    "ds_conv3x3_flip": (C.c_int, [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "ds_maxpool2x2_fwd": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "ds_maxpool2x2_bwd": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int,
+                                    C.c_void_p]),
+    "ds_vgg_stage_create": (C.c_int, [C.POINTER(VggCfg), C.c_void_p, C.POINTER(C.c_void_p)]),
     "ds_stage_create": (C.c_int, [C.POINTER(StageCfg), C.c_void_p, C.POINTER(C.c_void_p)]),
     "ds_stage_destroy": (C.c_int, [C.c_void_p]),
     "ds_stage_num_weights": (C.c_int, [C.c_void_p]),

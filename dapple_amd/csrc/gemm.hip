@@ -13,6 +13,7 @@
 //                     g ^ (((r & 3) << 1) & (granules-1)).  bf16 fragments come from
 //                     ds_read_b64_tr_b16 (a 4x16 transpose per 16 lanes), fp32 from 4-byte loads.
 #include <stdlib.h>
+#include <string.h>
 
 #include "common.h"
 
@@ -52,6 +53,7 @@ struct GemmArgs {
   int ktiles_per_split;
   int grid_m, grid_n;
   int vec_epi;
+  int conv_h, conv_w, conv_c;  // implicit 3x3 'same' convolution: extent of the gathered NHWC tensor
 };
 
 __device__ __forceinline__ int kmajor_off(int row, int chunk) { return row * 128 + ((chunk ^ (row & 7)) << 4); }
@@ -164,6 +166,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, f32x16 (&acc)[B
         if (flags & DS_EPI_RESIDUAL) v += to_f32(R[idx]);
         if (flags & DS_EPI_DGELU) v *= gelu_erf_grad(to_f32(C2[idx]));
         if (flags & DS_EPI_RELU) v = fmaxf(v, 0.f);
+        if (flags & DS_EPI_MASK) v = to_f32(C2[idx]) > 0.f ? v : 0.f;
         if (flags & DS_EPI_ACCUM) {
           if (p.splitk > 1) atomicAdd(Cf + idx, v); else Cf[idx] += v;
         } else if (out_f32) {
@@ -247,6 +250,17 @@ __device__ __forceinline__ void gemm_epilogue_staged(const GemmArgs& p, f32x16 (
     if (flags & DS_EPI_RELU) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) x[e] = fmaxf(x[e], 0.f);
+    }
+    if (flags & DS_EPI_MASK) {
+      if (sizeof(T) == 2) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(C2 + idx);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = (float)a[e] > 0.f ? x[e] : 0.f;
+      } else {
+        const f32x4 a0 = *reinterpret_cast<const f32x4*>(C2 + idx), a1 = *reinterpret_cast<const f32x4*>(C2 + idx + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { x[e] = a0[e] > 0.f ? x[e] : 0.f; x[4 + e] = a1[e] > 0.f ? x[4 + e] : 0.f; }
+      }
     }
     if (flags & DS_EPI_ACCUM) {
       if (p.splitk > 1) {
@@ -457,16 +471,20 @@ template <typename T, int W, int MAJOR, int NF> struct FragReader {
 typedef __attribute__((address_space(3))) void* lds_vptr;
 typedef __attribute__((address_space(1))) void* glb_vptr;
 
-template <typename T, int W, int MAJOR> struct DmaTile {
+template <typename T, int W, int MAJOR> struct PlainDma {
   static constexpr int VEC = Vec16<T>::N;
   static constexpr int KT = Mma<T>::KT;
   static constexpr int NV = W / 32;
   static constexpr int ROW_BYTES = W * (int)sizeof(T);
   static constexpr int CPR = ROW_BYTES / 16;
+  const T* src[NV];
+  int64_t step;
 
-  // per-lane source pointers for k-tile 0; slot i of wave w covers LDS positions (i*4+w)*64 + lane
-  static __device__ __forceinline__ void init(const T* (&src)[NV], const T* base, int64_t ld, int f0, int F, int k0,
-                                              int wave, int lane) {
+  // per-lane source pointers for k-tile kt0; slot i of wave w covers LDS positions (i*4+w)*64 + lane
+  __device__ __forceinline__ void init(const GemmArgs&, const T* base, int64_t ld, int f0, int F, int kt0, int wave,
+                                       int lane) {
+    const int k0 = kt0 * KT;
+    step = (MAJOR == DS_K_MAJOR) ? (int64_t)KT : (int64_t)KT * ld;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int p = (i * 4 + wave) * 64 + lane;
@@ -485,24 +503,115 @@ template <typename T, int W, int MAJOR> struct DmaTile {
       }
     }
   }
-  static __device__ __forceinline__ void issue(const T* (&src)[NV], char* lds, int64_t ld, int wave) {
+  __device__ __forceinline__ void issue(char* lds, int wave) {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       __builtin_amdgcn_global_load_lds((glb_vptr)src[i], (lds_vptr)(lds + (i * 4 + wave) * 1024), 16, 0, 0);
-      src[i] += (MAJOR == DS_K_MAJOR) ? (int64_t)KT : (int64_t)KT * ld;
+      src[i] += step;
     }
   }
 };
 
+// Source of zeros for the taps of a 3x3 'same' convolution that fall outside the image.
+__device__ __attribute__((aligned(16))) float g_zero16[4] = {0.f, 0.f, 0.f, 0.f};
+
+// Implicit-GEMM gather of a 3x3, stride 1, 'same' convolution over an NHWC tensor X[P = N*H*W, C]:
+//   MODE 1 (K-major A, forward / dgrad): A(m = pixel p, k = (tap, c)) = X[p shifted by tap][c];
+//           one k-tile is KT consecutive channels of one tap (needs C % KT == 0).
+//   MODE 2 (MN-major A, wgrad): A(m = (tap, c), k = pixel p) = X[p shifted by tap][c]; a 16-byte
+//           vector is VEC consecutive channels of one tap (needs C % VEC == 0).
+// Shifted pixels outside the image read g_zero16 instead.
+template <typename T, int W, int MODE> struct ConvDma {
+  static constexpr int VEC = Vec16<T>::N;
+  static constexpr int KT = Mma<T>::KT;
+  static constexpr int NV = W / 32;
+  static constexpr int ROW_BYTES = W * (int)sizeof(T);
+  static constexpr int CPR = ROW_BYTES / 16;
+  const T* base;
+  int H, Wd, C;
+  // MODE 1
+  int64_t off[NV];
+  int y[NV], x[NV];
+  int tap, c0;
+  // MODE 2
+  int shift[NV];  // (dy * Wd + dx) * C + c
+  int dyx[NV];    // (dy + 1) * 4 + (dx + 1)
+  int r[NV];
+  int64_t pix0;
+
+  __device__ __forceinline__ void init(const GemmArgs& p, const T* b, int64_t, int f0, int F, int kt0, int wave, int lane) {
+    base = b; H = p.conv_h; Wd = p.conv_w; C = p.conv_c;
+    if (MODE == 1) {
+      const int kpt = C / KT;
+      tap = kt0 / kpt;
+      c0 = (kt0 - tap * kpt) * KT;
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const int pos = (i * 4 + wave) * 64 + lane;
+        const int row = pos >> 3, c = (pos & 7) ^ (row & 7);
+        int pix = f0 + row;
+        if (pix > F - 1) pix = F - 1;
+        x[i] = pix % Wd;
+        y[i] = (pix / Wd) % H;
+        off[i] = (int64_t)pix * C + c * VEC;
+      }
+    } else {
+      pix0 = (int64_t)kt0 * KT;
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        constexpr int NG = ROW_BYTES / 32;
+        const int pos = (i * 4 + wave) * 64 + lane;
+        const int rr = pos / CPR, pc = pos % CPR;
+        const int g = (pc >> 1) ^ (((rr & 3) << 1) & (NG - 1));
+        int mi = f0 + (g * 2 + (pc & 1)) * VEC;
+        if (mi > F - VEC) mi = F - VEC;
+        const int t = mi / C, c = mi - t * C;
+        const int dy = t / 3 - 1, dx = t - (t / 3) * 3 - 1;
+        shift[i] = (dy * Wd + dx) * C + c;
+        dyx[i] = (dy + 1) * 4 + (dx + 1);
+        r[i] = rr;
+      }
+    }
+  }
+  __device__ __forceinline__ void issue(char* lds, int wave) {
+    if (MODE == 1) {
+      const int dy = tap / 3 - 1, dx = tap - (tap / 3) * 3 - 1;
+      const int sh = (dy * Wd + dx) * C + c0;
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const bool ok = (unsigned)(y[i] + dy) < (unsigned)H && (unsigned)(x[i] + dx) < (unsigned)Wd;
+        const T* src = ok ? base + off[i] + sh : reinterpret_cast<const T*>(g_zero16);
+        __builtin_amdgcn_global_load_lds((glb_vptr)src, (lds_vptr)(lds + (i * 4 + wave) * 1024), 16, 0, 0);
+      }
+      c0 += KT;
+      if (c0 == C) { c0 = 0; ++tap; }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const int64_t pix = pix0 + r[i];
+        const int q = (int)(pix / Wd);
+        const int xx = (int)(pix - (int64_t)q * Wd), yy = q % H;
+        const int dy = (dyx[i] >> 2) - 1, dx = (dyx[i] & 3) - 1;
+        const bool ok = (unsigned)(yy + dy) < (unsigned)H && (unsigned)(xx + dx) < (unsigned)Wd;
+        const T* src = ok ? base + pix * C + shift[i] : reinterpret_cast<const T*>(g_zero16);
+        __builtin_amdgcn_global_load_lds((glb_vptr)src, (lds_vptr)(lds + (i * 4 + wave) * 1024), 16, 0, 0);
+      }
+      pix0 += KT;
+    }
+  }
+};
+
+template <typename T, int W, int MAJOR, int CONV> struct DmaSelect { typedef PlainDma<T, W, MAJOR> type; };
+template <typename T, int W> struct DmaSelect<T, W, DS_K_MAJOR, 1> { typedef ConvDma<T, W, 1> type; };
+template <typename T, int W> struct DmaSelect<T, W, DS_MN_MAJOR, 2> { typedef ConvDma<T, W, 2> type; };
+
 // s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[15:14])
 #define DS_VMCNT(n) (((n) & 15) | (((n) >> 4) << 14) | (7 << 4) | (15 << 8))
 
-template <typename T, int BM, int BN, int AMAJ, int BMAJ, int STAGES>
+template <typename T, int BM, int BN, int AMAJ, int BMAJ, int STAGES, int CONVA = 0>
 __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
-  typedef OperandTile<T, BM, AMAJ> TA;
-  typedef OperandTile<T, BN, BMAJ> TB;
-  typedef DmaTile<T, BM, AMAJ> DA;
-  typedef DmaTile<T, BN, BMAJ> DB;
+  typedef typename DmaSelect<T, BM, AMAJ, CONVA>::type DA;
+  typedef PlainDma<T, BN, BMAJ> DB;
   constexpr int KT = Mma<T>::KT;
   constexpr int TM = BM / 64, TN = BN / 64;
   constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE_BYTES = A_BYTES + B_BYTES;
@@ -540,15 +649,15 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  const T* sa_src[DA::NV];
-  const T* sb_src[DB::NV];
-  DA::init(sa_src, A, p.lda, m0, p.m, kt_begin * KT, wave, lane);
-  DB::init(sb_src, B, p.ldb, n0, p.n, kt_begin * KT, wave, lane);
+  DA da;
+  DB db;
+  da.init(p, A, p.lda, m0, p.m, kt_begin, wave, lane);
+  db.init(p, B, p.ldb, n0, p.n, kt_begin, wave, lane);
 #pragma unroll
   for (int s = 0; s < STAGES - 1; ++s) {
     if (s < nkt) {
-      DA::issue(sa_src, lds + s * STAGE_BYTES, p.lda, wave);
-      DB::issue(sb_src, lds + s * STAGE_BYTES + A_BYTES, p.ldb, wave);
+      da.issue(lds + s * STAGE_BYTES, wave);
+      db.issue(lds + s * STAGE_BYTES + A_BYTES, wave);
     }
   }
   FragReader<T, BM, AMAJ, TM> ra;
@@ -565,8 +674,8 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
     if (kt + STAGES - 1 < nkt) {
       int nb = buf + STAGES - 1;
       if (nb >= STAGES) nb -= STAGES;
-      DA::issue(sa_src, lds + nb * STAGE_BYTES, p.lda, wave);
-      DB::issue(sb_src, lds + nb * STAGE_BYTES + A_BYTES, p.ldb, wave);
+      da.issue(lds + nb * STAGE_BYTES, wave);
+      db.issue(lds + nb * STAGE_BYTES + A_BYTES, wave);
     }
     const uint32_t sa = lds0 + buf * STAGE_BYTES, sb = sa + A_BYTES;
     RawFrag<T, AMAJ> fa[2][TM];
@@ -660,7 +769,7 @@ static void choose_tiling(int m, int n, int k, int kt, int batch, bool can_split
   }
 }
 
-extern "C" int ds_gemm(const ds_gemm_desc* d, void* stream) {
+static int gemm_run(const ds_gemm_desc* d, int splitk_req, void* stream) {
   DS_CHECK_ARG(d != nullptr, "ds_gemm: null descriptor");
   DS_CHECK_ARG(d->dtype == DS_F32 || d->dtype == DS_BF16, "ds_gemm: dtype %d", d->dtype);
   DS_CHECK_ARG((d->a_major | 1) == 1 && (d->b_major | 1) == 1, "ds_gemm: operand major must be 0 or 1");
@@ -716,15 +825,107 @@ extern "C" int ds_gemm(const ds_gemm_desc* d, void* stream) {
     if (env_split && (f & DS_EPI_ACCUM)) splitk = atoi(env_split) > 0 ? atoi(env_split) : 1;
   }
   const int ktiles = (d->k + kt - 1) / kt;
+  if (splitk_req > 1 && (f & DS_EPI_ACCUM)) splitk = splitk_req < ktiles ? splitk_req : ktiles;
   if (splitk > 1) a.vec_epi = 0;  // atomics want neighbouring lanes on neighbouring addresses
   a.splitk = splitk;
   a.ktiles_per_split = (ktiles + splitk - 1) / splitk;
   hipStream_t s = (hipStream_t)stream;
   static const int tbm[3] = {128, 128, 64}, tbn[3] = {128, 64, 64};
   char tag[96];
-  snprintf(tag, sizeof(tag), "gemm_kernel<%s,%d,%d,%s,%s>", d->dtype == DS_BF16 ? "bf16" : "float", tbm[tile], tbn[tile],
+  snprintf(tag, sizeof(tag), "%s<%s,%d,%d,%s,%s>", d->k % kt == 0 ? "gemm_dma_kernel" : "gemm_kernel",
+           d->dtype == DS_BF16 ? "bf16" : "float", tbm[tile], tbn[tile],
            d->a_major == DS_K_MAJOR ? "K" : "MN", d->b_major == DS_K_MAJOR ? "K" : "MN");
   ds_prof_scope prof(s, tag, 2.0 * d->m * d->n * d->k * batch, "FLOP");
   if (d->dtype == DS_BF16) return launch_major<bf16>(a, batch, tile, d->a_major, d->b_major, s);
   return launch_major<float>(a, batch, tile, d->a_major, d->b_major, s);
+}
+
+
+extern "C" int ds_gemm(const ds_gemm_desc* d, void* stream) { return gemm_run(d, 1, stream); }
+
+// Split-K variant for accumulating outputs whose reduction dimension dwarfs m*n (atomic fp32 adds).
+int ds_gemm_splitk(const ds_gemm_desc* d, int splitk, void* stream) { return gemm_run(d, splitk, stream); }
+
+// ------------------------------------------------------------------------------------------
+// 3x3 / stride 1 / 'same' convolution over NHWC tensors as an implicit GEMM (fp32 MFMA).
+namespace {
+template <int BM, int BN, int AMAJ, int MODE>
+int launch_conv_cfg(GemmArgs a, hipStream_t stream) {
+  a.grid_m = (a.m + BM - 1) / BM;
+  a.grid_n = (a.n + BN - 1) / BN;
+  dim3 grid(a.grid_m * a.grid_n, 1, a.splitk);
+  constexpr int STAGES = 4;
+  constexpr size_t lds = (size_t)STAGES * (BM + BN) * 128;
+  static bool attr_set = false;
+  if (!attr_set) {
+    DS_CHECK_HIP(hipFuncSetAttribute((const void*)gemm_dma_kernel<float, BM, BN, AMAJ, DS_MN_MAJOR, STAGES, MODE>,
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_set = true;
+  }
+  hipLaunchKernelGGL((gemm_dma_kernel<float, BM, BN, AMAJ, DS_MN_MAJOR, STAGES, MODE>), grid, dim3(256), lds, stream, a);
+  DS_CHECK_LAUNCH();
+  return DS_OK;
+}
+
+int conv_check(const char* who, int dtype, int n, int h, int w, int cin, int cout) {
+  DS_CHECK_ARG(dtype == DS_F32, "%s: only fp32 is built (dtype %d)", who, dtype);
+  DS_CHECK_ARG(n > 0 && h > 0 && w > 0 && cin > 0 && cout > 0, "%s: non-positive shape", who);
+  DS_CHECK_ARG(cin % 32 == 0, "%s: input channels (%d) must be a multiple of 32 (use ds_im2col3x3 + ds_gemm otherwise)", who, cin);
+  DS_CHECK_ARG(cout % 4 == 0, "%s: output channels (%d) must be a multiple of 4", who, cout);
+  DS_CHECK_ARG((int64_t)n * h * w < (int64_t)1 << 31, "%s: more than 2^31 pixels", who);
+  return DS_OK;
+}
+}  // namespace
+
+extern "C" int ds_conv3x3_fwd(int dtype, int n, int h, int w, int cin, int cout, const void* x, const void* kernel_hwio,
+                              const float* bias, int flags, const void* mask_src, void* y, void* stream) {
+  DS_PROPAGATE(conv_check("ds_conv3x3_fwd", dtype, n, h, w, cin, cout));
+  DS_CHECK_ARG(x && kernel_hwio && y, "ds_conv3x3_fwd: null pointer");
+  DS_CHECK_ARG((flags & ~(DS_EPI_BIAS | DS_EPI_RELU | DS_EPI_MASK)) == 0, "ds_conv3x3_fwd: unsupported flags %d", flags);
+  if (flags & DS_EPI_BIAS) DS_CHECK_ARG(bias != nullptr, "ds_conv3x3_fwd: DS_EPI_BIAS without bias");
+  if (flags & DS_EPI_MASK) DS_CHECK_ARG(mask_src != nullptr, "ds_conv3x3_fwd: DS_EPI_MASK without mask_src");
+  DS_CHECK_ARG(ds_aligned16(x) && ds_aligned16(kernel_hwio) && ds_aligned16(y) && ds_aligned16(mask_src),
+               "ds_conv3x3_fwd: tensors must be 16-byte aligned");
+  GemmArgs a;
+  memset(&a, 0, sizeof(a));
+  a.a = (const char*)x; a.b = (const char*)kernel_hwio; a.c = (char*)y;
+  a.bias = bias; a.c2 = (char*)mask_src;
+  a.m = n * h * w; a.n = cout; a.k = 9 * cin;
+  a.lda = cin; a.ldb = cout; a.ldc = cout;
+  a.batch_inner = 1; a.flags = flags; a.alpha = 1.f; a.splitk = 1; a.ktiles_per_split = a.k / 32;
+  a.vec_epi = cout % 8 == 0;
+  a.conv_h = h; a.conv_w = w; a.conv_c = cin;
+  hipStream_t s = (hipStream_t)stream;
+  ds_prof_scope prof(s, cout <= 64 ? "conv3x3_fwd<float,128,64>" : "conv3x3_fwd<float,128,128>", 2.0 * a.m * a.n * a.k, "FLOP");
+  if (cout <= 64) return launch_conv_cfg<128, 64, DS_K_MAJOR, 1>(a, s);
+  return launch_conv_cfg<128, 128, DS_K_MAJOR, 1>(a, s);
+}
+
+extern "C" int ds_conv3x3_wgrad(int dtype, int n, int h, int w, int cin, int cout, const void* x, const void* dz,
+                                float* dkernel_hwio, void* stream) {
+  DS_PROPAGATE(conv_check("ds_conv3x3_wgrad", dtype, n, h, w, cin, cout));
+  DS_CHECK_ARG(x && dz && dkernel_hwio, "ds_conv3x3_wgrad: null pointer");
+  DS_CHECK_ARG(ds_aligned16(x) && ds_aligned16(dz) && ds_aligned16(dkernel_hwio), "ds_conv3x3_wgrad: tensors must be 16-byte aligned");
+  const int64_t pixels = (int64_t)n * h * w;
+  DS_CHECK_ARG(pixels % 32 == 0, "ds_conv3x3_wgrad: n*h*w (%lld) must be a multiple of 32", (long long)pixels);
+  GemmArgs a;
+  memset(&a, 0, sizeof(a));
+  a.a = (const char*)x; a.b = (const char*)dz; a.c = (char*)dkernel_hwio;
+  a.m = 9 * cin; a.n = cout; a.k = (int)pixels;
+  a.lda = cin; a.ldb = cout; a.ldc = cout;
+  a.batch_inner = 1; a.flags = DS_EPI_ACCUM; a.alpha = 1.f;
+  a.conv_h = h; a.conv_w = w; a.conv_c = cin;
+  const int bn = cout <= 64 ? 64 : 128;
+  const int tiles = ((a.m + 127) / 128) * ((a.n + bn - 1) / bn);
+  const int ktiles = a.k / 32;
+  int splitk = 1024 / tiles;  // the reduction runs over every pixel of the micro-batch: split it across the chip
+  if (splitk > ktiles / 8) splitk = ktiles / 8;
+  if (splitk < 1) splitk = 1;
+  a.splitk = splitk;
+  a.ktiles_per_split = (ktiles + splitk - 1) / splitk;
+  a.vec_epi = splitk == 1 && cout % 8 == 0;
+  hipStream_t s = (hipStream_t)stream;
+  ds_prof_scope prof(s, cout <= 64 ? "conv3x3_wgrad<float,128,64>" : "conv3x3_wgrad<float,128,128>", 2.0 * a.m * a.n * a.k, "FLOP");
+  if (cout <= 64) return launch_conv_cfg<128, 64, DS_MN_MAJOR, 2>(a, s);
+  return launch_conv_cfg<128, 128, DS_MN_MAJOR, 2>(a, s);
 }

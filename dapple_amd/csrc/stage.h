@@ -40,3 +40,4 @@ struct ds_stage {
 };
 
 int ds_bert_stage_create(const ds_stage_cfg* cfg, hipStream_t stream, ds_stage** out);
+int ds_gemm_splitk(const ds_gemm_desc* d, int splitk, void* stream);

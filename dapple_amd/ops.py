@@ -138,3 +138,50 @@ def colsum_accum(x, out):
     check(_lib.load().ds_colsum_accum(dtype_code(x), rows, cols, ptr(x), cols, ptr(out), _lib.current_stream()),
           "ds_colsum_accum")
     return out
+
+
+def conv3x3(x, kernel, bias=None, relu=False, mask_src=None):
+    """NHWC fp32 3x3 'same' convolution (keras Conv2D of vgg19_slice_model.py:137); kernel HWIO."""
+    _need_cuda(x, kernel, bias, mask_src)
+    n, h, w, cin = x.shape
+    cout = kernel.shape[-1]
+    y = torch.empty(n, h, w, cout, dtype=x.dtype, device=x.device)
+    flags = (DS_EPI_BIAS if bias is not None else 0) | (DS_EPI_RELU if relu else 0) | (128 if mask_src is not None else 0)
+    check(_lib.load().ds_conv3x3_fwd(dtype_code(x), n, h, w, cin, cout, ptr(x), ptr(kernel), ptr(bias), flags, ptr(mask_src),
+                                     ptr(y), _lib.current_stream()), "ds_conv3x3_fwd")
+    return y
+
+
+def conv3x3_wgrad(x, dz, dkernel):
+    """dkernel (HWIO fp32) += correlation of x with dz."""
+    _need_cuda(x, dz, dkernel)
+    n, h, w, cin = x.shape
+    cout = dz.shape[-1]
+    check(_lib.load().ds_conv3x3_wgrad(dtype_code(x), n, h, w, cin, cout, ptr(x), ptr(dz), ptr(dkernel),
+                                       _lib.current_stream()), "ds_conv3x3_wgrad")
+    return dkernel
+
+
+def conv3x3_flip(kernel):
+    _need_cuda(kernel)
+    cin, cout = kernel.shape[2], kernel.shape[3]
+    out = torch.empty(3, 3, cout, cin, dtype=torch.float32, device=kernel.device)
+    check(_lib.load().ds_conv3x3_flip(cin, cout, ptr(kernel), ptr(out), _lib.current_stream()), "ds_conv3x3_flip")
+    return out
+
+
+def maxpool2x2(x):
+    _need_cuda(x)
+    n, h, w, c = x.shape
+    y = torch.empty(n, h // 2, w // 2, c, dtype=x.dtype, device=x.device)
+    check(_lib.load().ds_maxpool2x2_fwd(n, h, w, c, ptr(x), ptr(y), _lib.current_stream()), "ds_maxpool2x2_fwd")
+    return y
+
+
+def maxpool2x2_bwd(x, dy, relu_mask=False):
+    _need_cuda(x, dy)
+    n, h, w, c = x.shape
+    dx = torch.empty_like(x)
+    check(_lib.load().ds_maxpool2x2_bwd(n, h, w, c, ptr(x), ptr(dy), ptr(dx), 1 if relu_mask else 0, _lib.current_stream()),
+          "ds_maxpool2x2_bwd")
+    return dx

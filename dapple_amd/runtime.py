@@ -11,7 +11,7 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._lib import DS_BF16, DS_F32, DS_STAGE_BERT, StageCfg, check, ptr
+from ._lib import DS_BF16, DS_F32, DS_STAGE_BERT, StageCfg, VggCfg, check, ptr
 
 
 def stash_depth(stage_index, num_stages, variant="S"):
@@ -42,25 +42,18 @@ _TORCH_DTYPE = {DS_F32: torch.float32, DS_BF16: torch.bfloat16}
 class Stage:
     """Owns a ``ds_stage`` handle plus the flat fp32 master weights / gradients it is bound to."""
 
-    def __init__(self, kind, dtype, num_layers, hidden, heads, ffn, batch, seq, stash_slots, with_embedding=False,
-                 vocab=0, type_vocab=0, max_pos=0, ln_eps=1e-12, first_layer=0, device="cuda:0"):
+    def __init__(self, handle, act_dtype, in_numel, out_numel, stash_slots, in_dtype=None, takes_input_grad=True,
+                 device="cuda:0", cfg=None):
         self.lib = _lib.load()
         self.device = torch.device(device)
-        self.dtype_code = {"fp32": DS_F32, "bf16": DS_BF16, DS_F32: DS_F32, DS_BF16: DS_BF16}[dtype]
-        self.act_dtype = _TORCH_DTYPE[self.dtype_code]
-        cfg = StageCfg()
-        cfg.kind, cfg.dtype, cfg.num_layers = kind, self.dtype_code, num_layers
-        cfg.hidden, cfg.heads, cfg.ffn, cfg.batch, cfg.seq = hidden, heads, ffn, batch, seq
-        cfg.with_embedding = 1 if with_embedding else 0
-        cfg.vocab, cfg.type_vocab, cfg.max_pos = vocab, type_vocab, max_pos
-        cfg.ln_eps, cfg.stash_slots, cfg.first_layer = ln_eps, stash_slots, first_layer
+        self._h = handle
         self.cfg = cfg
-        self.rows, self.hidden, self.stash_slots = batch * seq, hidden, stash_slots
-        self.with_embedding = bool(with_embedding)
-        self._h = C.c_void_p()
-        with torch.cuda.device(self.device):
-            self._stream = _lib.current_stream()
-            check(self.lib.ds_stage_create(C.byref(cfg), self._stream, C.byref(self._h)), "ds_stage_create")
+        self.act_dtype = act_dtype
+        self.in_dtype = act_dtype if in_dtype is None else in_dtype
+        self.in_numel, self.out_numel = in_numel, out_numel
+        self.stash_slots = stash_slots
+        self.takes_input_grad = takes_input_grad
+        self.with_embedding = not takes_input_grad
         n = self.lib.ds_stage_num_weights(self._h)
         self.weight_names, self.weight_shapes = [], []
         buf = C.create_string_buffer(256)
@@ -68,8 +61,8 @@ class Stage:
         for i in range(n):
             check(self.lib.ds_stage_weight_info(self._h, i, buf, 256, C.byref(numel), C.byref(rows), C.byref(cols)),
                   "ds_stage_weight_info")
-            self.weight_names.append(buf.value.decode())
             name = buf.value.decode()
+            self.weight_names.append(name)
             vector = name.endswith(("/bias", "/gamma", "/beta"))
             self.weight_shapes.append((cols.value,) if vector else (rows.value, cols.value))
         self.weights, self.grads = {}, {}
@@ -78,18 +71,23 @@ class Stage:
     # -- weights ---------------------------------------------------------------------------
     def bind(self, weights):
         """weights: {reference variable name: array/tensor}. Copies into one flat fp32 buffer,
-        allocates the flat master-gradient buffer (zeroed) and binds both."""
+        allocates the flat master-gradient buffer (zeroed) and binds both.  A weight may come in the
+        reference's own shape (e.g. an HWIO conv kernel) as long as its element count matches."""
         missing = [n for n in self.weight_names if n not in weights]
         if missing:
             raise KeyError("missing weights: %s" % missing[:4])
-        sizes = []
+        sizes, shapes = [], []
         for n, shp in zip(self.weight_names, self.weight_shapes):
             numel = 1
             for s in shp:
                 numel *= s
             w = weights[n]
-            if tuple(w.shape) != tuple(shp):
+            wn = 1
+            for s in tuple(w.shape):
+                wn *= s
+            if wn != numel:
                 raise ValueError("weight %s has shape %s, stage expects %s" % (n, tuple(w.shape), tuple(shp)))
+            shapes.append(tuple(w.shape))
             sizes.append((numel + 63) // 64 * 64)          # keep every view 256-byte aligned
         total = sum(sizes)
         self.flat_weights = torch.empty(total, dtype=torch.float32, device=self.device)
@@ -97,7 +95,7 @@ class Stage:
         off = 0
         wp = (C.c_void_p * len(sizes))()
         gp = (C.c_void_p * len(sizes))()
-        for i, (n, shp, sz) in enumerate(zip(self.weight_names, self.weight_shapes, sizes)):
+        for i, (n, shp, sz) in enumerate(zip(self.weight_names, shapes, sizes)):
             numel = 1
             for s in shp:
                 numel *= s
@@ -117,24 +115,21 @@ class Stage:
 
     # -- one micro-batch ---------------------------------------------------------------------
     def forward(self, slot, x, out, key_mask=None, token_type_ids=None):
-        if self.with_embedding:
-            if x.dtype != torch.int32 or x.numel() != self.rows:
-                raise ValueError("an embedding stage takes int32 ids of %d elements" % self.rows)
-            if token_type_ids is not None:
-                check(self.lib.ds_stage_set_token_types(self._h, slot, ptr(token_type_ids)), "ds_stage_set_token_types")
-        elif x.dtype != self.act_dtype or x.numel() != self.rows * self.hidden:
-            raise ValueError("stage input must be %s [%d, %d]" % (self.act_dtype, self.rows, self.hidden))
-        if out.dtype != self.act_dtype or out.numel() != self.rows * self.hidden:
-            raise ValueError("stage output must be %s [%d, %d]" % (self.act_dtype, self.rows, self.hidden))
-        if key_mask is not None and (key_mask.dtype != torch.float32 or key_mask.numel() != self.cfg.batch * self.cfg.seq):
+        if x.dtype != self.in_dtype or x.numel() != self.in_numel:
+            raise ValueError("stage input must be %s with %d elements" % (self.in_dtype, self.in_numel))
+        if token_type_ids is not None:
+            check(self.lib.ds_stage_set_token_types(self._h, slot, ptr(token_type_ids)), "ds_stage_set_token_types")
+        if out.dtype != self.act_dtype or out.numel() != self.out_numel:
+            raise ValueError("stage output must be %s with %d elements" % (self.act_dtype, self.out_numel))
+        if key_mask is not None and key_mask.dtype != torch.float32:
             raise ValueError("key_mask must be fp32 [batch, seq]")
         check(self.lib.ds_stage_forward(self._h, slot, ptr(x), ptr(key_mask), ptr(out)), "ds_stage_forward")
 
     def backward(self, slot, d_out, d_in=None):
-        if d_out.dtype != self.act_dtype or d_out.numel() != self.rows * self.hidden:
-            raise ValueError("upstream gradient must be %s [%d, %d]" % (self.act_dtype, self.rows, self.hidden))
-        if d_in is not None and (d_in.dtype != self.act_dtype or d_in.numel() != self.rows * self.hidden):
-            raise ValueError("input gradient must be %s [%d, %d]" % (self.act_dtype, self.rows, self.hidden))
+        if d_out.dtype != self.act_dtype or d_out.numel() != self.out_numel:
+            raise ValueError("upstream gradient must be %s with %d elements" % (self.act_dtype, self.out_numel))
+        if d_in is not None and (d_in.dtype != self.act_dtype or d_in.numel() != self.in_numel):
+            raise ValueError("input gradient must be %s with %d elements" % (self.act_dtype, self.in_numel))
         check(self.lib.ds_stage_backward(self._h, slot, ptr(d_out), ptr(d_in)), "ds_stage_backward")
 
     def sync(self):
@@ -158,17 +153,63 @@ class Stage:
             pass
 
 
+def _dtype_code(dtype):
+    return {"fp32": DS_F32, "bf16": DS_BF16, DS_F32: DS_F32, DS_BF16: DS_BF16}[dtype]
+
+
 def bert_stage(num_layers, hidden, heads, ffn, batch, seq, dtype, stash_slots, embeddings=None, first_layer=0,
                ln_eps=1e-12, device="cuda:0"):
     """A BERT stage: ``num_layers`` encoder layers, behind the embedding when ``embeddings`` =
     (vocab, type_vocab, max_pos) is given."""
     if hidden % heads != 0:
         raise ValueError("The hidden size (%d) is not a multiple of the number of attention heads (%d)" % (hidden, heads))
-    kw = {}
+    lib = _lib.load()
+    cfg = StageCfg()
+    cfg.kind, cfg.dtype, cfg.num_layers = DS_STAGE_BERT, _dtype_code(dtype), num_layers
+    cfg.hidden, cfg.heads, cfg.ffn, cfg.batch, cfg.seq = hidden, heads, ffn, batch, seq
     if embeddings is not None:
-        kw = dict(with_embedding=True, vocab=embeddings[0], type_vocab=embeddings[1], max_pos=embeddings[2])
-    return Stage(DS_STAGE_BERT, dtype, num_layers, hidden, heads, ffn, batch, seq, stash_slots, ln_eps=ln_eps,
-                 first_layer=first_layer, device=device, **kw)
+        cfg.with_embedding = 1
+        cfg.vocab, cfg.type_vocab, cfg.max_pos = embeddings
+    cfg.ln_eps, cfg.stash_slots, cfg.first_layer = ln_eps, stash_slots, first_layer
+    h = C.c_void_p()
+    with torch.cuda.device(torch.device(device)):
+        check(lib.ds_stage_create(C.byref(cfg), _lib.current_stream(), C.byref(h)), "ds_stage_create")
+    act = _TORCH_DTYPE[cfg.dtype]
+    rows = batch * seq
+    if embeddings is not None:
+        return Stage(h, act, rows, rows * hidden, stash_slots, in_dtype=torch.int32, takes_input_grad=False,
+                     device=device, cfg=cfg)
+    return Stage(h, act, rows * hidden, rows * hidden, stash_slots, device=device, cfg=cfg)
+
+
+def vgg_stage(layers, batch, height, width, in_channels, stash_slots, need_input_grad=False, dtype="fp32",
+              device="cuda:0"):
+    """A VGG19 conv stack: ``layers`` = [(name, out_channels | None for a 2x2 max-pool), ...] in the
+    order vgg19/applications/vgg19_slice_model.py:280-302 applies them."""
+    lib = _lib.load()
+    cfg = VggCfg()
+    cfg.dtype = _dtype_code(dtype)
+    cfg.batch, cfg.height, cfg.width, cfg.in_channels = batch, height, width, in_channels
+    if len(layers) > 40:
+        raise ValueError("at most 40 ops")
+    cfg.num_ops = len(layers)
+    h_, w_, c_ = height, width, in_channels
+    for i, (_, cout) in enumerate(layers):
+        cfg.ops[i] = 0 if cout is None else cout
+        if cout is None:
+            h_, w_ = h_ // 2, w_ // 2
+        else:
+            c_ = cout
+    cfg.stash_slots, cfg.need_input_grad = stash_slots, 1 if need_input_grad else 0
+    h = C.c_void_p()
+    with torch.cuda.device(torch.device(device)):
+        check(lib.ds_vgg_stage_create(C.byref(cfg), _lib.current_stream(), C.byref(h)), "ds_vgg_stage_create")
+    st = Stage(h, _TORCH_DTYPE[cfg.dtype], batch * height * width * in_channels, batch * h_ * w_ * c_, stash_slots,
+               takes_input_grad=need_input_grad, device=device, cfg=cfg)
+    st.out_shape = (batch, h_, w_, c_)
+    # the stage names convs block%d_conv%d like keras; map the caller's layer names onto them
+    st.layer_names = [n for n, c in layers if c is not None]
+    return st
 
 
 class StageRuntime:
@@ -181,7 +222,7 @@ class StageRuntime:
         if stage.stash_slots < self.k:
             raise ValueError("stage has %d stash slots, the schedule needs %d" % (stage.stash_slots, self.k))
         self.m = num_micro_batches
-        self.needs_input_grad = needs_input_grad and not stage.with_embedding
+        self.needs_input_grad = needs_input_grad and stage.takes_input_grad
 
     def step(self, inputs, upstream, outputs, input_grads=None, key_masks=None):
         """inputs[M], upstream[M]: device tensors; outputs[M] (and input_grads[M]) are filled.

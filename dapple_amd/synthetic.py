@@ -100,12 +100,66 @@ def upstream_grads(seed, num_micro_batches, shape):
             for m in range(num_micro_batches)]
 
 
+# --------------------------------------------------------------------------- VGG19
+# (name, out_channels | None for a 2x2 max-pool) in the order a stage-0 replica applies them
+# (vgg19/applications/vgg19_slice_model.py:280-302); the 15:1 split of the reference ends at
+# block5_conv2, BASELINE configs[1] runs the whole conv stack.
+VGG19_STAGE0_15_1 = [
+    ("block1_conv1", 64), ("block1_conv2", 64), ("block1_pool", None),
+    ("block2_conv1", 128), ("block2_conv2", 128), ("block2_pool", None),
+    ("block3_conv1", 256), ("block3_conv2", 256), ("block3_conv3", 256), ("block3_conv4", 256), ("block3_pool", None),
+    ("block4_conv1", 512), ("block4_conv2", 512), ("block4_conv3", 512), ("block4_conv4", 512), ("block4_pool", None),
+    ("block5_conv1", 512), ("block5_conv2", 512),
+]
+VGG19_CONV_STACK = VGG19_STAGE0_15_1 + [("block5_conv3", 512), ("block5_conv4", 512)]
+
+
+def vgg_weights(seed, layers, in_channels=3, perturb=False):
+    """He-normal kernels (sigma = sqrt(2 / (9 Cin))), HWIO [3,3,Cin,Cout]; biases 0 (or random)."""
+    rng = _rng(seed)
+    w, cin = {}, in_channels
+    for name, cout in layers:
+        if cout is None:
+            continue
+        w[name + "/kernel"] = (rng.standard_normal((3, 3, cin, cout)) * np.sqrt(2.0 / (9 * cin))).astype(np.float32)
+        w[name + "/bias"] = (0.1 * rng.standard_normal(cout)).astype(np.float32) if perturb else np.zeros(cout, np.float32)
+        cin = cout
+    return w
+
+
+def vgg_inputs(seed, num_micro_batches, batch, height, width, channels=3):
+    return [_rng(seed + m).standard_normal((batch, height, width, channels)).astype(np.float32)
+            for m in range(num_micro_batches)]
+
+
+def vgg_layers(channels):
+    """[(keras-style name, out_channels | None)] for a list like [64, 64, None, 128]: convs are named
+    block%d_conv%d and pools block%d_pool, the block index growing after every pool."""
+    out, block, k = [], 1, 0
+    for c in channels:
+        if c is None:
+            out.append(("block%d_pool" % block, None))
+            block, k = block + 1, 0
+        else:
+            k += 1
+            out.append(("block%d_conv%d" % (block, k), c))
+    return out
+
+
+def scale_layers(layers, divisor):
+    """Same topology with every channel count divided (reduced-size fixtures and tests)."""
+    return [(n, None if c is None else max(c // divisor, 1)) for n, c in layers]
+
+
 # --------------------------------------------------------------------------- configs
 CONFIGS = {
     # BASELINE configs[0]: BERT-Large 2-layer encoder stage behind the embedding
     "bert_large_2l": dict(index=0, kind="bert", num_layers=2, hidden=1024, heads=16, ffn=4096,
                           seq=128, micro_batch=2, num_micro_batches=4, dtype="fp32",
                           embeddings=(30522, 2, 512)),
+    # BASELINE configs[1]: VGG19 conv stack (stage 0 of the 15:1 split, widened to conv5_4)
+    "vgg19_stage0": dict(index=1, kind="vgg", layers=VGG19_CONV_STACK, height=224, width=224, in_channels=3,
+                         micro_batch=32, num_micro_batches=4, dtype="fp32"),
     # BASELINE configs[3]: BERT-48 half-stage
     "bert48_half": dict(index=3, kind="bert", num_layers=24, hidden=1024, heads=16, ffn=4096,
                         seq=512, micro_batch=2, num_micro_batches=8, dtype="bf16",

@@ -42,6 +42,7 @@ extern "C" {
 #define DS_EPI_OUT_F32 16  /* C is fp32 even when dtype is bf16 */
 #define DS_EPI_ACCUM 32    /* C (fp32) += acc, split-K allowed (atomic) */
 #define DS_EPI_RELU 64     /* C = max(acc + bias, 0) */
+#define DS_EPI_MASK 128    /* C = aux[m][n] > 0 ? acc : 0 (ReLU backward), aux = c2 */
 
 const char* ds_last_error(void);
 
@@ -130,6 +131,7 @@ int ds_colsum_accum(int dtype, int rows, int cols, const void* x, int64_t ldx, f
  * tf.gradients(ys, [prev_y] + vars_i, grad_ys) of bert/graph.py:110-123 with the
  * accumulation of :145-161 fused in (master grads are updated in place). */
 #define DS_STAGE_BERT 0
+#define DS_STAGE_VGG19 1
 
 typedef struct ds_stage_cfg {
   int kind;        /* DS_STAGE_* */
@@ -170,6 +172,42 @@ int ds_stage_backward(ds_stage* h, int slot, const void* d_out, void* d_in);
 size_t ds_stage_workspace_bytes(const ds_stage* h);
 size_t ds_stage_stash_bytes(const ds_stage* h, int slots);
 int ds_stage_sync(ds_stage* h);
+
+/* ---------------------------------------------------------------------------
+ * 3x3, stride 1, 'same' convolution over NHWC fp32 tensors as an implicit GEMM on the matrix cores.
+ * Replaces keras Conv2D(C, (3,3), activation='relu', padding='same') of
+ * vgg19/applications/vgg19_slice_model.py:137-212 and its tf.gradients.
+ *   fwd  : y[n,h,w,co] = epi(sum_{dy,dx,c} x[n,h+dy,w+dx,c] * kernel[dy+1][dx+1][c][co] (+ bias[co]))
+ *          flags: DS_EPI_BIAS | DS_EPI_RELU | DS_EPI_MASK (y = mask_src > 0 ? y : 0).  The input
+ *          gradient of a convolution is the same call on dz with ds_conv3x3_flip(kernel).
+ *   wgrad: dkernel[dy+1][dx+1][c][co] (fp32) += sum_{n,h,w} x[n,h+dy,w+dx,c] * dz[n,h,w,co]
+ * cin must be a multiple of 32, cout of 4; wgrad needs n*h*w to be a multiple of 32. */
+int ds_conv3x3_fwd(int dtype, int n, int h, int w, int cin, int cout, const void* x,
+                   const void* kernel_hwio, const float* bias, int flags, const void* mask_src,
+                   void* y, void* stream);
+int ds_conv3x3_wgrad(int dtype, int n, int h, int w, int cin, int cout, const void* x,
+                     const void* dz, float* dkernel_hwio, void* stream);
+/* flipped[8 - tap][co][c] = kernel[tap][c][co]: the kernel of the transposed convolution */
+int ds_conv3x3_flip(int cin, int cout, const float* kernel_hwio, float* flipped, void* stream);
+/* keras MaxPooling2D((2,2), strides=(2,2)) (vgg19_slice_model.py:145) on NHWC fp32; backward sends
+ * the gradient to the first maximum of each window, optionally masked by x > 0 (fused ReLU'). */
+int ds_maxpool2x2_fwd(int n, int h, int w, int c, const float* x, float* y, void* stream);
+int ds_maxpool2x2_bwd(int n, int h, int w, int c, const float* x, const float* dy, float* dx,
+                      int relu_mask, void* stream);
+
+/* VGG19 stage 0 (vgg19_slice_model.py:274-309): ops[i] > 0 is a conv3x3 + bias + ReLU with that many
+ * output channels, ops[i] == 0 a 2x2 max-pool.  Weights are named block%d_conv%d/{kernel,bias}
+ * (HWIO kernels flattened to [9*cin, cout]).  The handle works with every ds_stage_* call. */
+typedef struct ds_vgg_cfg {
+  int dtype;  /* DS_F32 */
+  int batch, height, width, in_channels;
+  int num_ops;
+  int ops[40];
+  int stash_slots;     /* K = 2S-1-i for this model (vgg19/tf-keras-dapple.py:292) */
+  int need_input_grad; /* 0 for a first stage fed with images */
+  int reserved[8];
+} ds_vgg_cfg;
+int ds_vgg_stage_create(const ds_vgg_cfg* cfg, void* stream, ds_stage** out);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,60 @@
+"""CPU restatement of the reference's VGG19 stage-0 slice. TEST INFRASTRUCTURE ONLY.
+
+Follows vgg19/applications/vgg19_slice_model.py:135-213 (layer definitions: keras
+Conv2D(C, (3,3), activation='relu', padding='same'), MaxPooling2D((2,2), strides=(2,2)),
+channels_last, kernel HWIO [3,3,Cin,Cout] + bias) and :274-309 (the order they are applied
+in on a stage-0 replica).  Tensors are NHWC like the reference; torch's NCHW conv is
+reached by permutation.  Backward is torch.autograd.
+
+Pins (tests/test_oracle_vgg.py): conv vs a brute-force 7-deep loop; 'same' padding = 1;
+max-pool vs brute force; ReLU gradient 0 at exactly 0; parameter counts vs
+profiling_results/vgg-19-pbs-32.txt of the reference.
+"""
+import torch
+
+# (name, out_channels) or (name, None) for a pool, in application order (:280-302)
+VGG19_STAGE0_15_1 = [
+    ("block1_conv1", 64), ("block1_conv2", 64), ("block1_pool", None),
+    ("block2_conv1", 128), ("block2_conv2", 128), ("block2_pool", None),
+    ("block3_conv1", 256), ("block3_conv2", 256), ("block3_conv3", 256), ("block3_conv4", 256), ("block3_pool", None),
+    ("block4_conv1", 512), ("block4_conv2", 512), ("block4_conv3", 512), ("block4_conv4", 512), ("block4_pool", None),
+    ("block5_conv1", 512), ("block5_conv2", 512),
+]
+# BASELINE configs[1]: conv1_1..conv5_4 (16 convs, 4 pools)
+VGG19_CONV_STACK = VGG19_STAGE0_15_1 + [("block5_conv3", 512), ("block5_conv4", 512)]
+
+
+def conv3x3_relu(x, kernel, bias):
+    """keras Conv2D(3x3, 'same', relu) on NHWC x with HWIO kernel."""
+    y = torch.nn.functional.conv2d(x.permute(0, 3, 1, 2), kernel.permute(3, 2, 0, 1), bias, stride=1, padding=1)
+    return torch.relu(y).permute(0, 2, 3, 1)
+
+
+def max_pool_2x2(x):
+    """keras MaxPooling2D((2,2), strides=(2,2)), 'valid'."""
+    return torch.nn.functional.max_pool2d(x.permute(0, 3, 1, 2), 2, 2).permute(0, 2, 3, 1)
+
+
+def stage_forward(x, w, layers):
+    for name, cout in layers:
+        if cout is None:
+            x = max_pool_2x2(x)
+        else:
+            x = conv3x3_relu(x, w[name + "/kernel"], w[name + "/bias"])
+    return x
+
+
+def to_torch(weights, dtype=torch.float64, requires_grad=False):
+    return {k: torch.as_tensor(v).to(dtype).clone().requires_grad_(requires_grad) for k, v in weights.items()}
+
+
+def stage_vjp(x, w, d_out, layers, need_input_grad=False):
+    """tf.gradients(ys=out, xs=vars (+ input), grad_ys=d_out): (out, d_x or None, {name: d_w})."""
+    names = sorted(w)
+    if need_input_grad:
+        x = x.clone().requires_grad_(True)
+    out = stage_forward(x, w, layers)
+    xs = ([x] if need_input_grad else []) + [w[n] for n in names]
+    grads = torch.autograd.grad(out, xs, grad_outputs=d_out, allow_unused=True)
+    off = 1 if need_input_grad else 0
+    return out.detach(), (grads[0] if need_input_grad else None), {n: g for n, g in zip(names, grads[off:]) if g is not None}

@@ -1,0 +1,80 @@
+"""Pins the VGG oracle: brute-force conv / pool, padding, ReLU-at-zero, parameter counts."""
+import numpy as np
+import torch
+
+from dapple_amd import synthetic
+from oracle import vgg as ov
+
+D = torch.float64
+
+
+def test_conv_same_padding_vs_brute_force():
+    r = np.random.Generator(np.random.PCG64(1))
+    x = r.standard_normal((2, 5, 4, 3))
+    k = r.standard_normal((3, 3, 3, 2))
+    b = r.standard_normal(2)
+    want = np.zeros((2, 5, 4, 2))
+    for n in range(2):
+        for y in range(5):
+            for xx in range(4):
+                for co in range(2):
+                    s = b[co]
+                    for ky in range(3):
+                        for kx in range(3):
+                            yy, xc = y + ky - 1, xx + kx - 1
+                            if 0 <= yy < 5 and 0 <= xc < 4:
+                                for c in range(3):
+                                    s += x[n, yy, xc, c] * k[ky, kx, c, co]
+                    want[n, y, xx, co] = max(s, 0.0)
+    got = ov.conv3x3_relu(torch.tensor(x), torch.tensor(k), torch.tensor(b))
+    assert np.allclose(got.numpy(), want, atol=1e-12)
+
+
+def test_max_pool_vs_brute_force_and_first_max_gradient():
+    x = torch.randn(2, 6, 4, 3, dtype=D)
+    got = ov.max_pool_2x2(x)
+    for n in range(2):
+        for y in range(3):
+            for xx in range(2):
+                for c in range(3):
+                    assert got[n, y, xx, c] == x[n, 2 * y:2 * y + 2, 2 * xx:2 * xx + 2, c].max()
+    xr = x.clone().requires_grad_(True)
+    (g,) = torch.autograd.grad(ov.max_pool_2x2(xr).sum(), xr)
+    assert g.sum().item() == 2 * 3 * 2 * 3 and set(g.unique().tolist()) == {0.0, 1.0}
+
+
+def test_relu_gradient_is_zero_at_zero():
+    x = torch.zeros(1, 2, 2, 1, dtype=D, requires_grad=True)
+    k = torch.zeros(3, 3, 1, 1, dtype=D)
+    b = torch.zeros(1, dtype=D, requires_grad=True)
+    (gb,) = torch.autograd.grad(ov.conv3x3_relu(x, k, b).sum(), b)
+    assert gb.item() == 0.0
+
+
+def test_parameter_counts_match_reference_profile():
+    # SURVEY: 16 convs = 20 024 384 parameters, the reference's 14-conv split 15 304 768
+    def count(layers):
+        return sum(v.size for v in synthetic.vgg_weights(0, synthetic.scale_layers(layers, 1)).values())
+    assert count(synthetic.VGG19_CONV_STACK) == 20024384
+    assert count(synthetic.VGG19_STAGE0_15_1) == 15304768
+    assert ov.VGG19_CONV_STACK == synthetic.VGG19_CONV_STACK
+
+
+def test_stage_vjp_finite_differences():
+    layers = [("c1", 4), ("c2", 4), ("p1", None), ("c3", 8)]
+    w = ov.to_torch(synthetic.vgg_weights(3, layers, perturb=True), requires_grad=True)
+    x = torch.randn(1, 4, 4, 3, dtype=D)
+    dy = torch.randn(1, 2, 2, 8, dtype=D)
+    out, dx, dw = ov.stage_vjp(x, w, dy, layers, need_input_grad=True)
+    assert out.shape == (1, 2, 2, 8)
+    f = lambda xx, ww: (ov.stage_forward(xx, ww, layers) * dy).sum().item()
+    eps = 1e-6
+    for name in w:
+        wd = {k: v.detach().clone() for k, v in w.items()}
+        flat = wd[name].view(-1)
+        i = flat.numel() // 3
+        flat[i] += eps
+        fp = f(x, wd)
+        flat[i] -= 2 * eps
+        fm = f(x, wd)
+        assert abs((fp - fm) / (2 * eps) - dw[name].reshape(-1)[i].item()) < 1e-5, name
