@@ -13,7 +13,7 @@ DS_F32, DS_BF16 = 0, 1
 DS_K_MAJOR, DS_MN_MAJOR = 0, 1
 DS_EPI_BIAS, DS_EPI_RESIDUAL, DS_EPI_GELU, DS_EPI_DGELU = 1, 2, 4, 8
 DS_EPI_OUT_F32, DS_EPI_ACCUM, DS_EPI_RELU, DS_EPI_MASK = 16, 32, 64, 128
-DS_STAGE_BERT, DS_STAGE_VGG19 = 0, 1
+DS_STAGE_BERT, DS_STAGE_VGG19, DS_STAGE_GNMT = 0, 1, 2
 
 
 class DappleError(RuntimeError):
@@ -54,6 +54,13 @@ class VggCfg(C.Structure):
     ]
 
 
+class GnmtCfg(C.Structure):
+    _fields_ = [
+        ("dtype", C.c_int), ("num_layers", C.c_int), ("units", C.c_int), ("vocab", C.c_int), ("batch", C.c_int),
+        ("seq", C.c_int), ("forget_bias", C.c_float), ("stash_slots", C.c_int), ("reserved", C.c_int * 8),
+    ]
+
+
 # name -> (restype, argtypes); every symbol include/dapple_stage.h declares
 PROTOTYPES = {
     "ds_last_error": (C.c_char_p, []),
@@ -82,6 +89,7 @@ PROTOTYPES = {
     "ds_maxpool2x2_bwd": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int,
                                     C.c_void_p]),
     "ds_vgg_stage_create": (C.c_int, [C.POINTER(VggCfg), C.c_void_p, C.POINTER(C.c_void_p)]),
+    "ds_gnmt_stage_create": (C.c_int, [C.POINTER(GnmtCfg), C.c_void_p, C.POINTER(C.c_void_p)]),
     "ds_stage_create": (C.c_int, [C.POINTER(StageCfg), C.c_void_p, C.POINTER(C.c_void_p)]),
     "ds_stage_destroy": (C.c_int, [C.c_void_p]),
     "ds_stage_num_weights": (C.c_int, [C.c_void_p]),

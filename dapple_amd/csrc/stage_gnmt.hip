@@ -1,0 +1,315 @@
+// GNMT encoder pipeline stage: embedding lookup, one bidirectional LSTM layer, uni-directional LSTM
+// layers (residual from the third layer on), forward and BPTT backward, fp32.
+//
+// Follows gnmt/nmt/gnmt_model.py:61-221 (DAPPLE branch) and gnmt/nmt/model_helper.py:399-456 of the
+// reference; the cell is TensorFlow's BasicLSTMCell: gates = [x, h] @ kernel[in+U, 4U] + bias, gate
+// order i, j, f, o, c' = c*sigmoid(f + forget_bias) + sigmoid(i)*tanh(j), h' = tanh(c')*sigmoid(o).
+// All sequences are full length (the config passes no lengths), so dynamic_rnn is a plain scan.
+//
+// Per layer: the input half of the gates for all T steps is ONE GEMM [T*B, in] x [in, 4U] (+bias);
+// each step then adds h[t-1] @ Wh (a [B, U] x [U, 4U] GEMM whose epilogue adds the precomputed
+// half in place) and runs the fused cell kernel.  Backward walks the steps in reverse with the cell
+// backward kernel and dh = dgates @ Wh^T, then finishes with three big GEMMs over all steps:
+// dX = dG @ Wx^T, dWx += X^T dG, dWh += Hprev^T dG.
+#include <string.h>
+
+#include "stage.h"
+
+namespace {
+
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + __expf(-x)); }
+
+// table rows -> time-major activations: x[(t*B + b), :] = table[ids[b*T + t], :]
+__global__ __launch_bounds__(256) void gnmt_embed_fwd_kernel(int B, int T, int U, int vocab, const int32_t* __restrict__ ids,
+                                                            const float* __restrict__ table, float* __restrict__ x) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= B * T) return;
+  const int t = row / B, b = row % B;
+  int id = ids[b * T + t];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  const f32x4* src = reinterpret_cast<const f32x4*>(table + (int64_t)id * U);
+  f32x4* dst = reinterpret_cast<f32x4*>(x + (int64_t)row * U);
+  for (int c = threadIdx.x & 63; c < U / 4; c += 64) dst[c] = src[c];
+}
+
+__global__ __launch_bounds__(256) void gnmt_embed_bwd_kernel(int B, int T, int U, int vocab, const int32_t* __restrict__ ids,
+                                                            const float* __restrict__ dx, float* __restrict__ dtable) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= B * T) return;
+  const int t = row / B, b = row % B;
+  int id = ids[b * T + t];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  for (int c = threadIdx.x & 63; c < U; c += 64) atomicAdd(dtable + (int64_t)id * U + c, dx[(int64_t)row * U + c]);
+}
+
+// One time step of the cell.  gates [B,4U] holds the pre-activations (bias included) and is
+// overwritten with the activated gates (sigmoid(i), tanh(j), sigmoid(f + forget_bias), sigmoid(o));
+// h is written with row stride ldh, and y = h + x_res when the cell has a residual connection.
+__global__ __launch_bounds__(256) void lstm_cell_fwd_kernel(int B, int U, float forget_bias, float* __restrict__ gates,
+                                                           const float* __restrict__ c_prev, float* __restrict__ c,
+                                                           float* __restrict__ h, int ldh, const float* __restrict__ x_res,
+                                                           int ldx, float* __restrict__ y, int ldy) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= B * U) return;
+  const int b = idx / U, u = idx % U;
+  float* g = gates + (int64_t)b * 4 * U;
+  const float i = sigmoidf_(g[u]), j = tanhf(g[U + u]), f = sigmoidf_(g[2 * U + u] + forget_bias), o = sigmoidf_(g[3 * U + u]);
+  const float cp = c_prev ? c_prev[idx] : 0.f;
+  const float cn = cp * f + i * j;
+  const float hn = tanhf(cn) * o;
+  g[u] = i; g[U + u] = j; g[2 * U + u] = f; g[3 * U + u] = o;
+  c[idx] = cn;
+  h[(int64_t)b * ldh + u] = hn;
+  if (y) y[(int64_t)b * ldy + u] = hn + x_res[(int64_t)b * ldx + u];
+}
+
+// Backward of one step: dh = dy[t] + dh_rec, dc = dc_rec + dh*o*(1 - tanh(c)^2); writes the four
+// pre-activation gate gradients and leaves dc*f in dc_rec for step t-1.
+__global__ __launch_bounds__(256) void lstm_cell_bwd_kernel(int B, int U, const float* __restrict__ gact,
+                                                           const float* __restrict__ c, const float* __restrict__ c_prev,
+                                                           const float* __restrict__ dy, int lddy,
+                                                           const float* __restrict__ dh_rec, float* __restrict__ dc_rec,
+                                                           int first, float* __restrict__ dgates) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= B * U) return;
+  const int b = idx / U, u = idx % U;
+  const float* g = gact + (int64_t)b * 4 * U;
+  const float i = g[u], j = g[U + u], f = g[2 * U + u], o = g[3 * U + u];
+  const float tc = tanhf(c[idx]);
+  const float dh = dy[(int64_t)b * lddy + u] + (first ? 0.f : dh_rec[idx]);
+  const float dc = (first ? 0.f : dc_rec[idx]) + dh * o * (1.f - tc * tc);
+  const float cp = c_prev ? c_prev[idx] : 0.f;
+  float* d = dgates + (int64_t)b * 4 * U;
+  d[u] = dc * j * i * (1.f - i);
+  d[U + u] = dc * i * (1.f - j * j);
+  d[2 * U + u] = dc * cp * f * (1.f - f);
+  d[3 * U + u] = dh * tc * o * (1.f - o);
+  dc_rec[idx] = dc * f;
+}
+
+struct Cell {
+  int widx;        // kernel index in the weight list (bias = widx + 1)
+  int n_in;        // input width
+  bool reverse, residual;
+  // byte offsets into a slot
+  size_t x_off; int ldx;     // input activations [T*B, n_in]
+  size_t h_off; int ldh;     // outputs h [T*B, U] (row stride ldh)
+  size_t y_off;              // residual output y = h + x (residual cells only)
+  size_t g_off, c_off;       // activated gates [T*B,4U], cell states [T*B,U]
+};
+
+struct GnmtStage : ds_stage {
+  ds_gnmt_cfg gc;
+  int B, T, U, L, R;  // R = T*B rows
+  std::vector<Cell> cells;
+  char* stash_base = nullptr;
+  size_t slot_bytes = 0, ids_off = 0, x0_off = 0, xb_off = 0;
+  char* ws_base = nullptr;
+  size_t ws_bytes = 0, ws_dg, ws_dx[2], ws_dh[2], ws_dc;
+
+  ~GnmtStage() override {
+    if (stash_base) (void)hipFree(stash_base);
+    if (ws_base) (void)hipFree(ws_base);
+  }
+
+  int init() {
+    B = gc.batch; T = gc.seq; U = gc.units; L = gc.num_layers; R = B * T;
+    const char* P = "dynamic_seq2seq/encoder/";
+    char name[160];
+    snprintf(name, sizeof(name), "%sembedding_encoder", P);
+    winfo.push_back({name, gc.vocab, U});
+    Arena sa;
+    ids_off = sa.reserve((size_t)R * 4);
+    x0_off = sa.reserve((size_t)R * U * 4);
+    xb_off = sa.reserve((size_t)R * 2 * U * 4);
+    size_t prev_out = 0;
+    for (int i = 0; i < L + 1; ++i) {
+      Cell c;
+      memset(&c, 0, sizeof(c));
+      const char* scope;
+      char buf[96];
+      if (i == 0) scope = "bidirectional_rnn/fw/basic_lstm_cell";
+      else if (i == 1) scope = "bidirectional_rnn/bw/basic_lstm_cell";
+      else { snprintf(buf, sizeof(buf), "rnn/multi_rnn_cell/cell_%d/rnn/basic_lstm_cell", i - 1); scope = buf; }
+      c.n_in = (i == 2) ? 2 * U : U;
+      c.reverse = (i == 1);
+      c.residual = (i >= 3);
+      c.widx = (int)winfo.size();
+      snprintf(name, sizeof(name), "%s%s/kernel", P, scope);
+      winfo.push_back({name, c.n_in + U, 4 * U});
+      snprintf(name, sizeof(name), "%s%s/bias", P, scope);
+      winfo.push_back({name, 1, 4 * U});
+      c.g_off = sa.reserve((size_t)R * 4 * U * 4);
+      c.c_off = sa.reserve((size_t)R * U * 4);
+      if (i < 2) {
+        c.x_off = x0_off; c.ldx = U;
+        c.h_off = xb_off + (size_t)i * U * 4; c.ldh = 2 * U;
+      } else if (i == 2) {
+        c.x_off = xb_off; c.ldx = 2 * U;
+        c.h_off = sa.reserve((size_t)R * U * 4); c.ldh = U;
+        prev_out = c.h_off;
+      } else {
+        c.x_off = prev_out; c.ldx = U;
+        c.h_off = sa.reserve((size_t)R * U * 4); c.ldh = U;
+        c.y_off = sa.reserve((size_t)R * U * 4);
+        prev_out = c.y_off;
+      }
+      cells.push_back(c);
+    }
+    slot_bytes = sa.used;
+    DS_CHECK_HIP(hipMalloc((void**)&stash_base, slot_bytes * gc.stash_slots));
+    slot_forwarded.assign(gc.stash_slots, 0);
+    Arena wa;
+    ws_dg = wa.reserve((size_t)R * 4 * U * 4);
+    ws_dx[0] = wa.reserve((size_t)R * 2 * U * 4);
+    ws_dx[1] = wa.reserve((size_t)R * 2 * U * 4);
+    ws_dh[0] = wa.reserve((size_t)B * U * 4);
+    ws_dh[1] = wa.reserve((size_t)B * U * 4);
+    ws_dc = wa.reserve((size_t)B * U * 4);
+    ws_bytes = wa.used;
+    DS_CHECK_HIP(hipMalloc((void**)&ws_base, ws_bytes));
+    return DS_OK;
+  }
+
+  size_t workspace_bytes() const override { return ws_bytes; }
+  size_t stash_bytes(int slots) const override { return slot_bytes * (size_t)slots; }
+  int refresh_weights() override { return DS_OK; }  // fp32 kernels are used in place
+
+  int gemm(int am, int bm, int m, int n, int k, const void* a, int64_t lda, const void* b, int64_t ldb, void* c, int64_t ldc,
+           int flags, const float* bias, const void* residual) {
+    ds_gemm_desc d;
+    memset(&d, 0, sizeof(d));
+    d.dtype = DS_F32; d.a_major = am; d.b_major = bm; d.m = m; d.n = n; d.k = k; d.lda = lda; d.ldb = ldb; d.ldc = ldc;
+    d.batch = 1; d.batch_inner = 1; d.flags = flags; d.alpha = 1.f; d.a = a; d.b = b; d.c = c; d.bias = bias; d.residual = residual;
+    return ds_gemm(&d, stream);
+  }
+
+  int forward(int slot, const void* in, const float*, void* out) override {
+    char* sp = stash_base + (size_t)slot * slot_bytes;
+    DS_CHECK_HIP(hipMemcpyAsync(sp + ids_off, in, (size_t)R * 4, hipMemcpyDeviceToDevice, stream));
+    hipLaunchKernelGGL(gnmt_embed_fwd_kernel, dim3((R + 3) / 4), dim3(256), 0, stream, B, T, U, gc.vocab,
+                       (const int32_t*)(sp + ids_off), w[0], (float*)(sp + x0_off));
+    DS_CHECK_LAUNCH();
+    const int cell_grid = (B * U + 255) / 256;
+    for (size_t ci = 0; ci < cells.size(); ++ci) {
+      const Cell& c = cells[ci];
+      const float* kernel = w[c.widx];
+      const float* wh = kernel + (size_t)c.n_in * 4 * U;
+      float* G = (float*)(sp + c.g_off);
+      float* Cs = (float*)(sp + c.c_off);
+      float* H = (float*)(sp + c.h_off);
+      const float* X = (const float*)(sp + c.x_off);
+      const bool last = ci + 1 == cells.size();
+      float* Y = c.residual ? (last ? (float*)out : (float*)(sp + c.y_off)) : nullptr;
+      // input half of the gates for every step: [T*B, n_in] x [n_in, 4U] + bias
+      DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, R, 4 * U, c.n_in, X, c.ldx, kernel, 4 * U, G, 4 * U, DS_EPI_BIAS, w[c.widx + 1], nullptr));
+      for (int s = 0; s < T; ++s) {
+        const int t = c.reverse ? T - 1 - s : s;
+        const int tp = c.reverse ? t + 1 : t - 1;  // the step whose state feeds this one
+        float* g = G + (size_t)t * B * 4 * U;
+        if (s > 0) {
+          // recurrent half, added in place: g += h[tp] @ Wh
+          DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, B, 4 * U, U, H + (size_t)tp * B * c.ldh, c.ldh, wh, 4 * U, g, 4 * U,
+                            DS_EPI_RESIDUAL, nullptr, g));
+        }
+        ds_prof_scope prof(stream, "lstm_cell_fwd_kernel", (double)B * U * 4 * (4 + 4 + 2 + (c.residual ? 2 : 1)), "B");
+        hipLaunchKernelGGL(lstm_cell_fwd_kernel, dim3(cell_grid), dim3(256), 0, stream, B, U, gc.forget_bias, g,
+                           s > 0 ? Cs + (size_t)tp * B * U : nullptr, Cs + (size_t)t * B * U, H + (size_t)t * B * c.ldh, c.ldh,
+                           c.residual ? X + (size_t)t * B * c.ldx : nullptr, c.ldx, Y ? Y + (size_t)t * B * U : nullptr, U);
+        DS_CHECK_LAUNCH();
+      }
+      if (last && !c.residual)
+        DS_CHECK_HIP(hipMemcpyAsync(out, H, (size_t)R * U * 4, hipMemcpyDeviceToDevice, stream));
+    }
+    return DS_OK;
+  }
+
+  int backward(int slot, const void* d_out, void*) override {
+    char* sp = stash_base + (size_t)slot * slot_bytes;
+    float* dG = (float*)(ws_base + ws_dg);
+    float* dc = (float*)(ws_base + ws_dc);
+    const int cell_grid = (B * U + 255) / 256;
+    const float* dY = (const float*)d_out;  // gradient w.r.t. the output of the cell being processed
+    int lddy = U;
+    int pp = 0;
+    float* dXB = nullptr;  // gradient w.r.t. the fw|bw concatenation [R, 2U]
+    float* dX0 = nullptr;
+    for (int ci = (int)cells.size() - 1; ci >= 0; --ci) {
+      const Cell& c = cells[ci];
+      const float* kernel = w[c.widx];
+      const float* wh = kernel + (size_t)c.n_in * 4 * U;
+      const float* G = (const float*)(sp + c.g_off);
+      const float* Cs = (const float*)(sp + c.c_off);
+      const float* H = (const float*)(sp + c.h_off);
+      const float* X = (const float*)(sp + c.x_off);
+      if (ci < 2) { dY = dXB + (size_t)ci * U; lddy = 2 * U; }
+      for (int s = T - 1; s >= 0; --s) {
+        const int t = c.reverse ? T - 1 - s : s;
+        const int tp = c.reverse ? t + 1 : t - 1;
+        const int first = (s == T - 1);  // no recurrent gradient flows into the last step of the scan
+        float* dh_in = (float*)(ws_base + ws_dh[s & 1]);
+        float* dh_out = (float*)(ws_base + ws_dh[(s & 1) ^ 1]);
+        {
+          ds_prof_scope prof(stream, "lstm_cell_bwd_kernel", (double)B * U * 4 * (4 + 4 + 6), "B");
+          hipLaunchKernelGGL(lstm_cell_bwd_kernel, dim3(cell_grid), dim3(256), 0, stream, B, U, G + (size_t)t * B * 4 * U,
+                             Cs + (size_t)t * B * U, s > 0 ? Cs + (size_t)tp * B * U : nullptr, dY + (size_t)t * B * lddy, lddy,
+                             dh_in, dc, first, dG + (size_t)t * B * 4 * U);
+          DS_CHECK_LAUNCH();
+        }
+        if (s > 0)  // dh for step tp: dgates[t] @ Wh^T
+          DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, B, U, 4 * U, dG + (size_t)t * B * 4 * U, 4 * U, wh, 4 * U, dh_out, U, 0, nullptr, nullptr));
+      }
+      // parameter gradients over all steps
+      DS_PROPAGATE(ds_colsum_accum(DS_F32, R, 4 * U, dG, 4 * U, g[c.widx + 1], stream));
+      DS_PROPAGATE(gemm(DS_MN_MAJOR, DS_MN_MAJOR, c.n_in, 4 * U, R, X, c.ldx, dG, 4 * U, g[c.widx], 4 * U, DS_EPI_ACCUM, nullptr, nullptr));
+      // dWh += Hprev^T dG: the state feeding step t is h[tp]; pair rows of H with the rows of dG one step later in scan order
+      if (T > 1) {
+        const float* Hp = c.reverse ? H + (size_t)B * c.ldh : H;
+        const float* dGp = c.reverse ? dG : dG + (size_t)B * 4 * U;
+        DS_PROPAGATE(gemm(DS_MN_MAJOR, DS_MN_MAJOR, U, 4 * U, (T - 1) * B, Hp, c.ldh, dGp, 4 * U, g[c.widx] + (size_t)c.n_in * 4 * U,
+                          4 * U, DS_EPI_ACCUM, nullptr, nullptr));
+      }
+      // input gradient dX = dG @ Wx^T (+ dY through the residual connection)
+      if (ci >= 2) {
+        float* dX = (float*)(ws_base + ws_dx[pp]);
+        DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, R, c.n_in, 4 * U, dG, 4 * U, kernel, 4 * U, dX, c.n_in,
+                          c.residual ? DS_EPI_RESIDUAL : 0, nullptr, c.residual ? dY : nullptr));
+        if (ci == 2) dXB = dX; else { dY = dX; lddy = U; }
+        pp ^= 1;
+      } else {
+        // both directions read the embedding: dX0 = dG_bw Wx_bw^T, then += dG_fw Wx_fw^T
+        if (ci == 1) dX0 = (float*)(ws_base + ws_dx[pp]);
+        DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, R, U, 4 * U, dG, 4 * U, kernel, 4 * U, dX0, U, ci == 0 ? DS_EPI_RESIDUAL : 0,
+                          nullptr, ci == 0 ? dX0 : nullptr));
+      }
+    }
+    hipLaunchKernelGGL(gnmt_embed_bwd_kernel, dim3((R + 3) / 4), dim3(256), 0, stream, B, T, U, gc.vocab,
+                       (const int32_t*)(sp + ids_off), dX0, g[0]);
+    DS_CHECK_LAUNCH();
+    return DS_OK;
+  }
+};
+
+}  // namespace
+
+extern "C" int ds_gnmt_stage_create(const ds_gnmt_cfg* c, void* stream, ds_stage** out) {
+  DS_CHECK_ARG(c != nullptr && out != nullptr, "ds_gnmt_stage_create: null argument");
+  *out = nullptr;
+  DS_CHECK_ARG(c->dtype == DS_F32, "ds_gnmt_stage_create: only fp32 is built (dtype %d)", c->dtype);
+  DS_CHECK_ARG(c->num_layers >= 2, "ds_gnmt_stage_create: the GNMT encoder has a bidirectional layer and at least one uni-directional layer");
+  DS_CHECK_ARG(c->units > 0 && c->units % 4 == 0, "ds_gnmt_stage_create: num_units (%d) must be a positive multiple of 4", c->units);
+  DS_CHECK_ARG(c->batch > 0 && c->seq > 0 && c->vocab > 0, "ds_gnmt_stage_create: non-positive shape");
+  DS_CHECK_ARG(c->batch % 4 == 0, "ds_gnmt_stage_create: batch (%d) must be a multiple of 4", c->batch);
+  DS_CHECK_ARG(c->stash_slots >= 1, "ds_gnmt_stage_create: stash_slots must be >= 1");
+  GnmtStage* s = new GnmtStage();
+  memset(&s->cfg, 0, sizeof(s->cfg));
+  s->cfg.kind = DS_STAGE_GNMT;
+  s->cfg.dtype = c->dtype;
+  s->cfg.stash_slots = c->stash_slots;
+  s->gc = *c;
+  s->stream = (hipStream_t)stream;
+  const int rc = s->init();
+  if (rc != DS_OK) { delete s; return rc; }
+  *out = s;
+  return DS_OK;
+}

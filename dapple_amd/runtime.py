@@ -11,7 +11,7 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._lib import DS_BF16, DS_F32, DS_STAGE_BERT, StageCfg, VggCfg, check, ptr
+from ._lib import DS_BF16, DS_F32, DS_STAGE_BERT, GnmtCfg, StageCfg, VggCfg, check, ptr
 
 
 def stash_depth(stage_index, num_stages, variant="S"):
@@ -209,6 +209,21 @@ def vgg_stage(layers, batch, height, width, in_channels, stash_slots, need_input
     st.out_shape = (batch, h_, w_, c_)
     # the stage names convs block%d_conv%d like keras; map the caller's layer names onto them
     st.layer_names = [n for n, c in layers if c is not None]
+    return st
+
+
+def gnmt_stage(num_layers, units, vocab, batch, seq, stash_slots, forget_bias=1.0, dtype="fp32", device="cuda:0"):
+    """The GNMT encoder stage (gnmt/nmt/gnmt_model.py:61-221): ids [batch, seq] int32 -> [seq, batch, units]."""
+    lib = _lib.load()
+    cfg = GnmtCfg()
+    cfg.dtype, cfg.num_layers, cfg.units, cfg.vocab = _dtype_code(dtype), num_layers, units, vocab
+    cfg.batch, cfg.seq, cfg.forget_bias, cfg.stash_slots = batch, seq, forget_bias, stash_slots
+    h = C.c_void_p()
+    with torch.cuda.device(torch.device(device)):
+        check(lib.ds_gnmt_stage_create(C.byref(cfg), _lib.current_stream(), C.byref(h)), "ds_gnmt_stage_create")
+    st = Stage(h, _TORCH_DTYPE[cfg.dtype], batch * seq, seq * batch * units, stash_slots, in_dtype=torch.int32,
+               takes_input_grad=False, device=device, cfg=cfg)
+    st.out_shape = (seq, batch, units)
     return st
 
 

@@ -151,6 +151,34 @@ def scale_layers(layers, divisor):
     return [(n, None if c is None else max(c // divisor, 1)) for n, c in layers]
 
 
+# --------------------------------------------------------------------------- GNMT encoder
+GNMT_SCOPE = "dynamic_seq2seq/encoder/"
+
+
+def gnmt_cell_scopes(num_layers):
+    """Variable scopes of the encoder's LSTM cells (gnmt/nmt/gnmt_model.py:96-166): the fw and bw cell
+    of the bidirectional layer, then uni layers 1..num_layers-1."""
+    s = [GNMT_SCOPE + "bidirectional_rnn/fw/basic_lstm_cell", GNMT_SCOPE + "bidirectional_rnn/bw/basic_lstm_cell"]
+    s += [GNMT_SCOPE + "rnn/multi_rnn_cell/cell_%d/rnn/basic_lstm_cell" % l for l in range(1, num_layers)]
+    return s
+
+
+def gnmt_weights(seed, num_layers, units, vocab, init_weight=0.1, perturb=False):
+    """U(-init_weight, init_weight) embedding table and LSTM kernels [in+units, 4*units]; biases 0."""
+    rng = _rng(seed)
+    w = {GNMT_SCOPE + "embedding_encoder": rng.uniform(-init_weight, init_weight, (vocab, units)).astype(np.float32)}
+    for i, scope in enumerate(gnmt_cell_scopes(num_layers)):
+        n_in = 2 * units if i == 2 else units           # uni layer 1 reads the fw|bw concatenation
+        w[scope + "/kernel"] = rng.uniform(-init_weight, init_weight, (n_in + units, 4 * units)).astype(np.float32)
+        w[scope + "/bias"] = rng.uniform(-init_weight, init_weight, 4 * units).astype(np.float32) if perturb \
+            else np.zeros(4 * units, np.float32)
+    return w
+
+
+def gnmt_id_inputs(seed, num_micro_batches, batch, seq, vocab):
+    return [_rng(seed + m).integers(0, vocab, size=(batch, seq)).astype(np.int32) for m in range(num_micro_batches)]
+
+
 # --------------------------------------------------------------------------- configs
 CONFIGS = {
     # BASELINE configs[0]: BERT-Large 2-layer encoder stage behind the embedding
@@ -160,6 +188,9 @@ CONFIGS = {
     # BASELINE configs[1]: VGG19 conv stack (stage 0 of the 15:1 split, widened to conv5_4)
     "vgg19_stage0": dict(index=1, kind="vgg", layers=VGG19_CONV_STACK, height=224, width=224, in_channels=3,
                          micro_batch=32, num_micro_batches=4, dtype="fp32"),
+    # BASELINE configs[2]: GNMT-16 encoder stage (8 LSTM layers, the first bidirectional)
+    "gnmt16_encoder": dict(index=2, kind="gnmt", num_layers=8, units=1024, vocab=32000, seq=50, micro_batch=64,
+                           num_micro_batches=4, dtype="fp32", forget_bias=1.0),
     # BASELINE configs[3]: BERT-48 half-stage
     "bert48_half": dict(index=3, kind="bert", num_layers=24, hidden=1024, heads=16, ffn=4096,
                         seq=512, micro_batch=2, num_micro_batches=8, dtype="bf16",

@@ -132,6 +132,7 @@ int ds_colsum_accum(int dtype, int rows, int cols, const void* x, int64_t ldx, f
  * accumulation of :145-161 fused in (master grads are updated in place). */
 #define DS_STAGE_BERT 0
 #define DS_STAGE_VGG19 1
+#define DS_STAGE_GNMT 2
 
 typedef struct ds_stage_cfg {
   int kind;        /* DS_STAGE_* */
@@ -208,6 +209,21 @@ typedef struct ds_vgg_cfg {
   int reserved[8];
 } ds_vgg_cfg;
 int ds_vgg_stage_create(const ds_vgg_cfg* cfg, void* stream, ds_stage** out);
+
+/* GNMT encoder stage (gnmt/nmt/gnmt_model.py:61-221, DAPPLE branch): embedding lookup, one
+ * bidirectional BasicLSTMCell layer, then num_layers-1 uni-directional layers, residual from the
+ * third layer on (model_helper.py:445-448); ids [batch, seq] int32 in, [seq, batch, units] out
+ * (time-major like the reference).  Kernels are TF's [in+units, 4*units] with gate order i, j, f, o.
+ * Sequences are full length.  The handle works with every ds_stage_* call; it takes no input gradient. */
+typedef struct ds_gnmt_cfg {
+  int dtype;       /* DS_F32 */
+  int num_layers;  /* encoder layers incl. the bidirectional one (8 for GNMT-16's encoder) */
+  int units, vocab, batch, seq;
+  float forget_bias; /* 1.0 in gnmt/nmt/standard_hparams/wmt16_gnmt_8_layer.json */
+  int stash_slots;
+  int reserved[8];
+} ds_gnmt_cfg;
+int ds_gnmt_stage_create(const ds_gnmt_cfg* cfg, void* stream, ds_stage** out);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,83 @@
+"""Pins the GNMT encoder oracle against torch's LSTM (gate blocks permuted), an explicit loop and
+the kernel shape the reference's own test holds."""
+import numpy as np
+import torch
+
+from dapple_amd import synthetic
+from oracle import gnmt as og
+
+D = torch.float64
+
+
+def _to_torch_lstm(kernel, bias, n_in, forget_bias):
+    """TF BasicLSTMCell kernel [in+U,4U] gate order i,j,f,o -> torch weight_ih/hh, bias; torch order i,f,g,o."""
+    U = kernel.shape[1] // 4
+    i, j, f, o = kernel.chunk(4, 1)
+    k = torch.cat([i, f, j, o], 1)
+    bi, bj, bf, bo = bias.chunk(4)
+    b = torch.cat([bi, bf + forget_bias, bj, bo])
+    return k[:n_in].t().contiguous(), k[n_in:].t().contiguous(), b, U
+
+
+def test_cell_matches_torch_lstmcell_and_kernel_layout():
+    I, U, B = 5, 5, 3
+    kernel = torch.randn(I + U, 4 * U, dtype=D)
+    assert tuple(kernel.shape) == (10, 20)              # gnmt/nmt/model_test.py:86 last_enc_weight shape
+    bias = torch.randn(4 * U, dtype=D)
+    x, h, c = torch.randn(B, I, dtype=D), torch.randn(B, U, dtype=D), torch.randn(B, U, dtype=D)
+    h1, c1 = og.lstm_cell(x, h, c, kernel, bias, forget_bias=1.0)
+    wih, whh, b, _ = _to_torch_lstm(kernel, bias, I, 1.0)
+    cell = torch.nn.LSTMCell(I, U).double()
+    with torch.no_grad():
+        cell.weight_ih.copy_(wih); cell.weight_hh.copy_(whh); cell.bias_ih.copy_(b); cell.bias_hh.zero_()
+    h2, c2 = cell(x, (h, c))
+    assert torch.allclose(h1, h2, atol=1e-12) and torch.allclose(c1, c2, atol=1e-12)
+    # forget_bias matters: without it the result differs
+    h3, _ = og.lstm_cell(x, h, c, kernel, bias, forget_bias=0.0)
+    assert (h3 - h1).abs().max() > 1e-3
+
+
+def test_bidirectional_layer_matches_torch_lstm():
+    T, B, I, U = 6, 2, 4, 4
+    x = torch.randn(T, B, I, dtype=D)
+    ks = [torch.randn(I + U, 4 * U, dtype=D) * 0.5 for _ in range(2)]
+    bs = [torch.randn(4 * U, dtype=D) * 0.5 for _ in range(2)]
+    fw = og.dynamic_rnn(x, ks[0], bs[0], 1.0)
+    bw = og.dynamic_rnn(x, ks[1], bs[1], 1.0, reverse=True)
+    lstm = torch.nn.LSTM(I, U, bidirectional=True).double()
+    with torch.no_grad():
+        for sfx, k, b in (("", ks[0], bs[0]), ("_reverse", ks[1], bs[1])):
+            wih, whh, bb, _ = _to_torch_lstm(k, b, I, 1.0)
+            getattr(lstm, "weight_ih_l0" + sfx).copy_(wih)
+            getattr(lstm, "weight_hh_l0" + sfx).copy_(whh)
+            getattr(lstm, "bias_ih_l0" + sfx).copy_(bb)
+            getattr(lstm, "bias_hh_l0" + sfx).zero_()
+    ref, _ = lstm(x)
+    assert torch.allclose(torch.cat([fw, bw], -1), ref, atol=1e-12)
+
+
+def test_encoder_structure_residual_from_third_layer():
+    T, B, U, V, L = 4, 2, 4, 9, 4
+    w = og.to_torch(synthetic.gnmt_weights(1, L, U, V, init_weight=0.5, perturb=True))
+    ids = torch.randint(0, V, (B, T), dtype=torch.int32)
+    out = og.encoder_forward(ids, w, L)
+    assert out.shape == (T, B, U)
+    # explicit restatement: bi layer -> uni 1 (input 2U, no residual) -> uni 2, 3 (residual)
+    scopes = synthetic.gnmt_cell_scopes(L)
+    assert w[scopes[2] + "/kernel"].shape == (3 * U, 4 * U) and w[scopes[3] + "/kernel"].shape == (2 * U, 4 * U)
+    emb = w[og.EMB][ids.long().t()]
+    x = torch.cat([og.dynamic_rnn(emb, w[scopes[0] + "/kernel"], w[scopes[0] + "/bias"]),
+                   og.dynamic_rnn(emb, w[scopes[1] + "/kernel"], w[scopes[1] + "/bias"], reverse=True)], -1)
+    x = og.dynamic_rnn(x, w[scopes[2] + "/kernel"], w[scopes[2] + "/bias"])
+    for s in scopes[3:]:
+        x = og.dynamic_rnn(x, w[s + "/kernel"], w[s + "/bias"]) + x
+    assert torch.equal(out, x)
+    assert [c[0] for c in og.cell_names(L)] == scopes
+
+
+def test_parameter_count_of_config():
+    # C3 = 79.7 M LSTM parameters + 32000 x 1024 embedding
+    w = synthetic.gnmt_weights(0, 8, 1024, 32)          # tiny vocab: count the cells only
+    cells = sum(v.size for k, v in w.items() if "embedding" not in k)
+    assert cells == 2 * (2048 * 4096 + 4096) + (3072 * 4096 + 4096) + 6 * (2048 * 4096 + 4096)
+    assert abs(cells - 79.7e6) < 0.1e6
