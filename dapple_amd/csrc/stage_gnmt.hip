@@ -183,6 +183,23 @@ struct GnmtStage : ds_stage {
     d.batch = 1; d.batch_inner = 1; d.flags = flags; d.alpha = 1.f; d.a = a; d.b = b; d.c = c; d.bias = bias; d.residual = residual;
     return ds_gemm(&d, stream);
   }
+  // c (fp32) += a[m,k] x b: the per-step recurrent products have only B rows, so the reduction is
+  // split across the chip and added with fp32 atomics
+  int gemm_accum_splitk(int bm, int m, int n, int k, const void* a, int64_t lda, const void* b, int64_t ldb, float* c,
+                        int64_t ldc, int splitk) {
+    ds_gemm_desc d;
+    memset(&d, 0, sizeof(d));
+    d.dtype = DS_F32; d.a_major = DS_K_MAJOR; d.b_major = bm; d.m = m; d.n = n; d.k = k; d.lda = lda; d.ldb = ldb; d.ldc = ldc;
+    d.batch = 1; d.batch_inner = 1; d.flags = DS_EPI_ACCUM; d.alpha = 1.f; d.a = a; d.b = b; d.c = c;
+    return ds_gemm_splitk(&d, splitk, stream);
+  }
+  static int split_for(int m, int n, int k) {
+    const int tiles = ((m + 63) / 64) * ((n + 63) / 64);
+    int s = 256 / (tiles > 0 ? tiles : 1);
+    const int ktiles = k / 32;
+    if (s > ktiles / 4) s = ktiles / 4;
+    return s < 1 ? 1 : s;
+  }
 
   int forward(int slot, const void* in, const float*, void* out) override {
     char* sp = stash_base + (size_t)slot * slot_bytes;
@@ -209,8 +226,8 @@ struct GnmtStage : ds_stage {
         float* g = G + (size_t)t * B * 4 * U;
         if (s > 0) {
           // recurrent half, added in place: g += h[tp] @ Wh
-          DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, B, 4 * U, U, H + (size_t)tp * B * c.ldh, c.ldh, wh, 4 * U, g, 4 * U,
-                            DS_EPI_RESIDUAL, nullptr, g));
+          DS_PROPAGATE(gemm_accum_splitk(DS_MN_MAJOR, B, 4 * U, U, H + (size_t)tp * B * c.ldh, c.ldh, wh, 4 * U, g, 4 * U,
+                                         split_for(B, 4 * U, U)));
         }
         ds_prof_scope prof(stream, "lstm_cell_fwd_kernel", (double)B * U * 4 * (4 + 4 + 2 + (c.residual ? 2 : 1)), "B");
         hipLaunchKernelGGL(lstm_cell_fwd_kernel, dim3(cell_grid), dim3(256), 0, stream, B, U, gc.forget_bias, g,
@@ -256,8 +273,11 @@ struct GnmtStage : ds_stage {
                              dh_in, dc, first, dG + (size_t)t * B * 4 * U);
           DS_CHECK_LAUNCH();
         }
-        if (s > 0)  // dh for step tp: dgates[t] @ Wh^T
-          DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, B, U, 4 * U, dG + (size_t)t * B * 4 * U, 4 * U, wh, 4 * U, dh_out, U, 0, nullptr, nullptr));
+        if (s > 0) {  // dh for step tp: dgates[t] @ Wh^T
+          DS_CHECK_HIP(hipMemsetAsync(dh_out, 0, (size_t)B * U * 4, stream));
+          DS_PROPAGATE(gemm_accum_splitk(DS_K_MAJOR, B, U, 4 * U, dG + (size_t)t * B * 4 * U, 4 * U, wh, 4 * U, dh_out, U,
+                                         split_for(B, U, 4 * U)));
+        }
       }
       // parameter gradients over all steps
       DS_PROPAGATE(ds_colsum_accum(DS_F32, R, 4 * U, dG, 4 * U, g[c.widx + 1], stream));
