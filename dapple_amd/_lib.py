@@ -12,8 +12,8 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libdapple_hip.so")
 DS_F32, DS_BF16 = 0, 1
 DS_K_MAJOR, DS_MN_MAJOR = 0, 1
 DS_EPI_BIAS, DS_EPI_RESIDUAL, DS_EPI_GELU, DS_EPI_DGELU = 1, 2, 4, 8
-DS_EPI_OUT_F32, DS_EPI_ACCUM, DS_EPI_RELU, DS_EPI_MASK = 16, 32, 64, 128
-DS_STAGE_BERT, DS_STAGE_VGG19, DS_STAGE_GNMT = 0, 1, 2
+DS_EPI_OUT_F32, DS_EPI_ACCUM, DS_EPI_RELU, DS_EPI_MASK, DS_EPI_TANH_FORM = 16, 32, 64, 128, 256
+DS_STAGE_BERT, DS_STAGE_VGG19, DS_STAGE_GNMT, DS_STAGE_XLNET = 0, 1, 2, 3
 
 
 class DappleError(RuntimeError):
@@ -61,6 +61,14 @@ class GnmtCfg(C.Structure):
     ]
 
 
+class XlnetCfg(C.Structure):
+    _fields_ = [
+        ("dtype", C.c_int), ("num_layers", C.c_int), ("hidden", C.c_int), ("heads", C.c_int), ("ffn", C.c_int),
+        ("batch", C.c_int), ("seq", C.c_int), ("mem_len", C.c_int), ("streams", C.c_int), ("ln_eps", C.c_float),
+        ("first_layer", C.c_int), ("stash_slots", C.c_int), ("reserved", C.c_int * 8),
+    ]
+
+
 # name -> (restype, argtypes); every symbol include/dapple_stage.h declares
 PROTOTYPES = {
     "ds_last_error": (C.c_char_p, []),
@@ -90,6 +98,8 @@ PROTOTYPES = {
                                     C.c_void_p]),
     "ds_vgg_stage_create": (C.c_int, [C.POINTER(VggCfg), C.c_void_p, C.POINTER(C.c_void_p)]),
     "ds_gnmt_stage_create": (C.c_int, [C.POINTER(GnmtCfg), C.c_void_p, C.POINTER(C.c_void_p)]),
+    "ds_xlnet_stage_create": (C.c_int, [C.POINTER(XlnetCfg), C.c_void_p, C.POINTER(C.c_void_p)]),
+    "ds_xlnet_stage_set_inputs": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
     "ds_stage_create": (C.c_int, [C.POINTER(StageCfg), C.c_void_p, C.POINTER(C.c_void_p)]),
     "ds_stage_destroy": (C.c_int, [C.c_void_p]),
     "ds_stage_num_weights": (C.c_int, [C.c_void_p]),

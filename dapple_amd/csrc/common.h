@@ -82,3 +82,15 @@ __device__ __forceinline__ float gelu_erf_grad(float x) {
   const float pdf = 0.39894228040143267794f * __expf(-0.5f * x * x);
   return cdf + x * pdf;
 }
+
+// tanh-form GELU of the reference's XLNet layers (xlnet/activations/gelu.py:6-11) and its derivative
+__device__ __forceinline__ float gelu_tanh(float x) {
+  const float t = tanhf(0.79788456080286535588f * (x + 0.044715f * x * x * x));
+  return 0.5f * x * (1.0f + t);
+}
+__device__ __forceinline__ float gelu_tanh_grad(float x) {
+  const float t = tanhf(0.79788456080286535588f * (x + 0.044715f * x * x * x));
+  return 0.5f * (1.0f + t) + 0.5f * x * (1.0f - t * t) * 0.79788456080286535588f * (1.0f + 3.0f * 0.044715f * x * x);
+}
+__device__ __forceinline__ float gelu_any(float x, bool tanh_form) { return tanh_form ? gelu_tanh(x) : gelu_erf(x); }
+__device__ __forceinline__ float gelu_any_grad(float x, bool tanh_form) { return tanh_form ? gelu_tanh_grad(x) : gelu_erf_grad(x); }

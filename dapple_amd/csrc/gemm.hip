@@ -145,6 +145,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, f32x16 (&acc)[B
   constexpr int TM = BM / 64, TN = BN / 64;
   // epilogue: lane holds column (lane & 31), rows (e/4)*8 + (lane>>5)*4 + (e&3) of each 32x32 tile
   const int flags = p.flags;
+  const bool tanh_form = (flags & DS_EPI_TANH_FORM) != 0;
   const bool out_f32 = (flags & (DS_EPI_OUT_F32 | DS_EPI_ACCUM)) != 0 || sizeof(T) == 4;
   float* Cf = reinterpret_cast<float*>(p.c) + c_off;
   T* Ct = reinterpret_cast<T*>(p.c) + c_off;
@@ -164,7 +165,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, f32x16 (&acc)[B
         const int64_t idx = (int64_t)row * p.ldc + col;
         float v = acc[i][j][e] * p.alpha + bias;
         if (flags & DS_EPI_RESIDUAL) v += to_f32(R[idx]);
-        if (flags & DS_EPI_DGELU) v *= gelu_erf_grad(to_f32(C2[idx]));
+        if (flags & DS_EPI_DGELU) v *= gelu_any_grad(to_f32(C2[idx]), tanh_form);
         if (flags & DS_EPI_RELU) v = fmaxf(v, 0.f);
         if (flags & DS_EPI_MASK) v = to_f32(C2[idx]) > 0.f ? v : 0.f;
         if (flags & DS_EPI_ACCUM) {
@@ -174,7 +175,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, f32x16 (&acc)[B
         } else {
           Ct[idx] = from_f32<T>(v);
         }
-        if (flags & DS_EPI_GELU) C2[idx] = from_f32<T>(gelu_erf(v));
+        if (flags & DS_EPI_GELU) C2[idx] = from_f32<T>(gelu_any(v, tanh_form));
       }
     }
 }
@@ -191,6 +192,7 @@ __device__ __forceinline__ void gemm_epilogue_staged(const GemmArgs& p, f32x16 (
   constexpr int LDW = BN + 4;
   float* sc = reinterpret_cast<float*>(lds);
   const int flags = p.flags;
+  const bool tanh_form = (flags & DS_EPI_TANH_FORM) != 0;
   __syncthreads();
 #pragma unroll
   for (int i = 0; i < TM; ++i)
@@ -240,11 +242,11 @@ __device__ __forceinline__ void gemm_epilogue_staged(const GemmArgs& p, f32x16 (
       if (sizeof(T) == 2) {
         const bf16x8 a = *reinterpret_cast<const bf16x8*>(C2 + idx);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) x[e] *= gelu_erf_grad((float)a[e]);
+        for (int e = 0; e < 8; ++e) x[e] *= gelu_any_grad((float)a[e], tanh_form);
       } else {
         const f32x4 a0 = *reinterpret_cast<const f32x4*>(C2 + idx), a1 = *reinterpret_cast<const f32x4*>(C2 + idx + 4);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) { x[e] *= gelu_erf_grad(a0[e]); x[4 + e] *= gelu_erf_grad(a1[e]); }
+        for (int e = 0; e < 4; ++e) { x[e] *= gelu_any_grad(a0[e], tanh_form); x[4 + e] *= gelu_any_grad(a1[e], tanh_form); }
       }
     }
     if (flags & DS_EPI_RELU) {
@@ -289,12 +291,12 @@ __device__ __forceinline__ void gemm_epilogue_staged(const GemmArgs& p, f32x16 (
       if (sizeof(T) == 2) {
         bf16x8 o;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) o[e] = (bf16)gelu_erf(x[e]);
+        for (int e = 0; e < 8; ++e) o[e] = (bf16)gelu_any(x[e], tanh_form);
         *reinterpret_cast<bf16x8*>(reinterpret_cast<bf16*>(p.c2) + c_off + idx) = o;
       } else {
         f32x4 c0, c1;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) { c0[e] = gelu_erf(x[e]); c1[e] = gelu_erf(x[4 + e]); }
+        for (int e = 0; e < 4; ++e) { c0[e] = gelu_any(x[e], tanh_form); c1[e] = gelu_any(x[4 + e], tanh_form); }
         *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.c2) + c_off + idx) = c0;
         *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.c2) + c_off + idx + 4) = c1;
       }

@@ -1,0 +1,551 @@
+// XLNet pipeline stage: relative-position multi-head attention layers (content stream and, optionally,
+// the query stream sharing keys/values/weights), with optional memory, forward and backward.
+//
+// Follows xlnet/layers/rel_multihead_attn.py:71-149 of the reference (einsums of _rel_attn_core and
+// call), lambda_funcs.py:85-93 (rel_shift), position_wise_feed_forward.py:92-105, layer_normalization.py:
+// 69-78 (eps 1e-14), activations/gelu.py:6-11 (tanh GELU) and the layer body of
+// models/slice_xlnet.py:164-180.  The reference builds the content stream with memory length 0; memory
+// (keys/values from concat(mem, h), positions klen .. -qlen+1) and the query stream follow the XLNet
+// formulation those layers were transcribed from.
+//
+// Activations are sequence-major rows (stream, i, b) of width H.  Scores are never shifted in memory:
+// the position term is computed unshifted as (q + r_r) k_r^T [qlen, rlen] and the softmax kernel reads
+// column j + qlen - i of it (rel_shift as index arithmetic); backward scatters with the same map.
+#include <string.h>
+
+#include "stage.h"
+
+namespace {
+
+enum XW { X_Q = 0, X_K, X_V, X_R, X_O, X_RW, X_RR, X_RS, X_SEG, X_LN1_G, X_LN1_B, X_W1, X_B1, X_W2, X_B2, X_LN2_G, X_LN2_B, X_NW };
+
+// qw = q + r_w, qr = q + r_r, qs = q + r_s (biases broadcast over rows)
+template <typename T>
+__global__ __launch_bounds__(256) void xl_bias_q_kernel(int64_t total, int H, const T* __restrict__ q, const float* __restrict__ rw,
+                                                       const float* __restrict__ rr, const float* __restrict__ rs,
+                                                       T* __restrict__ qw, T* __restrict__ qr, T* __restrict__ qs) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int c = (int)(i % H);
+    const float v = to_f32(q[i]);
+    qw[i] = from_f32<T>(v + rw[c]);
+    qr[i] = from_f32<T>(v + rr[c]);
+    qs[i] = from_f32<T>(v + rs[c]);
+  }
+}
+
+// Kernel pack: wkv[h][0:H] = wk[h][:], wkv[h][H:2H] = wv[h][:]; other weights cast to T
+template <typename T>
+__global__ __launch_bounds__(256) void xl_pack_kv_kernel(int H, const float* __restrict__ wk, const float* __restrict__ wv,
+                                                        T* __restrict__ wkv) {
+  const int64_t total = (int64_t)H * 2 * H;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int h = (int)(i / (2 * H)), j = (int)(i % (2 * H));
+    wkv[i] = from_f32<T>(j < H ? wk[(int64_t)h * H + j] : wv[(int64_t)h * H + j - H]);
+  }
+}
+
+// pe[r][t] = sin((klen - r) * f_t), pe[r][H/2 + t] = cos(...), f_t = 10000^(-2t/H)  (lambda_funcs.py:50-79)
+template <typename T>
+__global__ __launch_bounds__(256) void xl_pos_emb_kernel(int R, int H, int klen, T* __restrict__ pe) {
+  const int64_t total = (int64_t)R * (H / 2);
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int r = (int)(i / (H / 2)), t = (int)(i % (H / 2));
+    const double f = pow(10000.0, -2.0 * t / H);
+    const double a = (double)(klen - r) * f;
+    pe[(int64_t)r * H + t] = from_f32<T>((float)sin(a));
+    pe[(int64_t)r * H + H / 2 + t] = from_f32<T>((float)cos(a));
+  }
+}
+
+// One wave per (query row i, batch b, head n) of one stream:
+//   score[j] = (ac[i][j] + bd[i][j + Q - i] + ef[seg(i,j,b)]) * scale - 1e30 * mask[i][j][b],  p = softmax_j
+// with ef[s] = (q + r_s)[i,b,n,:] . seg_emb[s,n,:].  ac is [B*N][Q][K], bd [B*N][Q][R] (fp32).
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void xl_softmax_fwd_kernel(int Q, int K, int R, int B, int N, int D, const float* __restrict__ ac,
+                                                            const float* __restrict__ bd, const T* __restrict__ qs,
+                                                            const float* __restrict__ seg_emb, const uint8_t* __restrict__ seg_mat,
+                                                            const float* __restrict__ mask, float scale, T* __restrict__ p) {
+  const int lane = threadIdx.x & 63;
+  const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // = (b*N + n)*Q + i
+  if (w >= (int64_t)B * N * Q) return;
+  const int i = (int)(w % Q);
+  const int bn = (int)(w / Q), n = bn % N, b = bn / N;
+  const int H = N * D;
+  float e0 = 0.f, e1 = 0.f;
+  if (lane < D) {
+    const float qv = to_f32(qs[((int64_t)i * B + b) * H + n * D + lane]);
+    e0 = qv * seg_emb[n * D + lane];
+    e1 = qv * seg_emb[H + n * D + lane];
+  }
+  e0 = wave_sum(e0);
+  e1 = wave_sum(e1);
+  const float* acr = ac + w * K;
+  const float* bdr = bd + w * R + (Q - i);
+  float v[NV * 4];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int t = 0; t < NV * 4; ++t) {
+    const int j = lane + t * 64;
+    if (j < K) {
+      const int64_t ijb = ((int64_t)i * K + j) * B + b;
+      const float ef = (seg_mat && seg_mat[ijb]) ? e1 : e0;
+      float s = (acr[j] + bdr[j] + ef) * scale;
+      if (mask) s -= 1e30f * mask[ijb];
+      v[t] = s;
+      mx = fmaxf(mx, s);
+    } else {
+      v[t] = -INFINITY;
+    }
+  }
+  mx = wave_max(mx);
+  float sum = 0.f;
+#pragma unroll
+  for (int t = 0; t < NV * 4; ++t) { v[t] = expf(v[t] - mx); sum += v[t]; }
+  const float inv = 1.0f / wave_sum(sum);
+  T* pr = p + w * K;
+#pragma unroll
+  for (int t = 0; t < NV * 4; ++t) {
+    const int j = lane + t * 64;
+    if (j < K) pr[j] = from_f32<T>(v[t] * inv);
+  }
+}
+
+// dbd[i][r] = ds[i][r - Q + i] when that column exists, else 0 (transpose of the rel_shift index map)
+template <typename T>
+__global__ __launch_bounds__(256) void xl_unshift_kernel(int64_t rows, int Q, int K, int R, const T* __restrict__ ds, T* __restrict__ dbd) {
+  const int64_t total = rows * R;
+  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
+    const int r = (int)(idx % R);
+    const int64_t w = idx / R;
+    const int i = (int)(w % Q);
+    const int j = r - Q + i;
+    dbd[idx] = (j >= 0 && j < K) ? ds[w * K + j] : from_f32<T>(0.f);
+  }
+}
+
+// One wave per (i, b, n): def[s] = sum_j [seg(i,j,b) == s] ds[i][j]; writes def to deft[(n*2+s)][row] for the
+// seg_emb gradient GEMM, dqs = def[0]*seg_emb[0] + def[1]*seg_emb[1], and dq = dqw + dqr + dqs.
+template <typename T>
+__global__ __launch_bounds__(256) void xl_seg_bwd_kernel(int Q, int K, int B, int N, int D, int64_t rows_total, int64_t row0,
+                                                        const T* __restrict__ ds, const uint8_t* __restrict__ seg_mat,
+                                                        const float* __restrict__ seg_emb, const T* __restrict__ dqw,
+                                                        const T* __restrict__ dqr, T* __restrict__ dqs, T* __restrict__ dq,
+                                                        T* __restrict__ deft) {
+  const int lane = threadIdx.x & 63;
+  const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (w >= (int64_t)B * N * Q) return;
+  const int i = (int)(w % Q);
+  const int bn = (int)(w / Q), n = bn % N, b = bn / N;
+  const int H = N * D;
+  const T* dr = ds + w * K;
+  float d0 = 0.f, d1 = 0.f;
+  for (int j = lane; j < K; j += 64) {
+    const float v = to_f32(dr[j]);
+    if (seg_mat && seg_mat[((int64_t)i * K + j) * B + b]) d1 += v; else d0 += v;
+  }
+  d0 = wave_sum(d0);
+  d1 = wave_sum(d1);
+  const int64_t row = (int64_t)i * B + b;  // row inside this stream
+  if (lane == 0) {
+    deft[(int64_t)(n * 2 + 0) * rows_total + row0 + row] = from_f32<T>(d0);
+    deft[(int64_t)(n * 2 + 1) * rows_total + row0 + row] = from_f32<T>(d1);
+  }
+  if (lane < D) {
+    const int64_t o = row * H + n * D + lane;
+    const float s = d0 * seg_emb[n * D + lane] + d1 * seg_emb[H + n * D + lane];
+    dqs[o] = from_f32<T>(s);
+    dq[o] = from_f32<T>(to_f32(dqw[o]) + to_f32(dqr[o]) + s);
+  }
+}
+
+struct LayerOff { size_t x, qw, qr, qs, kv, p, vec, z1, y1, u, hh, z2, st1, st2; };
+
+struct XlnetStage : ds_stage {
+  ds_xlnet_cfg xc;
+  int L, H, F, N, D, B, Q, Mm, K, R, S, rowsS, rows, krows;  // rowsS = Q*B (one stream), rows = S*Q*B, krows = K*B
+  int dtype;
+  size_t esz;
+  // compute copies
+  char* wc_base = nullptr;
+  std::vector<char*> wq, wkv, wr, wo, w1, w2, kr;
+  char* pe = nullptr;
+  // stash
+  char* stash_base = nullptr;
+  size_t slot_bytes = 0, mask_off = 0, seg_off = 0, mem_off = 0;
+  std::vector<LayerOff> lo;
+  std::vector<char> has_mask, has_seg;
+  // workspace
+  char* ws_base = nullptr;
+  size_t ws_bytes = 0, ws_qall, ws_ac, ws_bd, ws_ds, ws_dbd, ws_dz2, ws_du, ws_dy1, ws_dz1, ws_dvec, ws_dqw, ws_dqr, ws_dqs, ws_dq,
+         ws_dkv, ws_dkr, ws_deft, ws_dx[2];
+
+  ~XlnetStage() override {
+    if (wc_base) (void)hipFree(wc_base);
+    if (stash_base) (void)hipFree(stash_base);
+    if (ws_base) (void)hipFree(ws_base);
+  }
+  int base(int l) const { return l * X_NW; }
+
+  int init() {
+    L = xc.num_layers; H = xc.hidden; F = xc.ffn; N = xc.heads; D = H / N; B = xc.batch; Q = xc.seq; Mm = xc.mem_len;
+    K = Mm + Q; R = K + Q; S = xc.streams; rowsS = Q * B; rows = S * rowsS; krows = K * B;
+    dtype = xc.dtype; esz = dtype == DS_BF16 ? 2 : 4;
+    char name[96];
+    static const char* names[X_NW] = {"q", "k", "v", "r", "o", "bias_context", "bias_relative", "bias_segment", "seg_emb",
+                                      "attn_ln/gamma", "attn_ln/beta", "ff/W1", "ff/b1", "ff/W2", "ff/b2", "ff_ln/gamma", "ff_ln/beta"};
+    for (int l = 0; l < L; ++l)
+      for (int k = 0; k < X_NW; ++k) {
+        snprintf(name, sizeof(name), "layer_%d/%s", xc.first_layer + l, names[k]);
+        int64_t r = 1, c = H;
+        if (k <= X_O) r = H;
+        else if (k == X_SEG) r = 2;
+        else if (k == X_W1) { r = H; c = F; }
+        else if (k == X_B1) c = F;
+        else if (k == X_W2) { r = F; c = H; }
+        winfo.push_back({name, r, c});
+      }
+    Arena ca;
+    std::vector<size_t> o_q(L), o_kv(L), o_r(L), o_o(L), o_1(L), o_2(L), o_kr(L);
+    const size_t o_pe = ca.reserve((size_t)R * H * esz);
+    for (int l = 0; l < L; ++l) {
+      o_kv[l] = ca.reserve((size_t)H * 2 * H * esz);
+      o_kr[l] = ca.reserve((size_t)R * H * esz);
+      if (dtype == DS_BF16) {
+        o_q[l] = ca.reserve((size_t)H * H * esz); o_r[l] = ca.reserve((size_t)H * H * esz); o_o[l] = ca.reserve((size_t)H * H * esz);
+        o_1[l] = ca.reserve((size_t)H * F * esz); o_2[l] = ca.reserve((size_t)F * H * esz);
+      }
+    }
+    DS_CHECK_HIP(hipMalloc((void**)&wc_base, ca.used));
+    pe = wc_base + o_pe;
+    wq.resize(L); wkv.resize(L); wr.resize(L); wo.resize(L); w1.resize(L); w2.resize(L); kr.resize(L);
+    for (int l = 0; l < L; ++l) {
+      wkv[l] = wc_base + o_kv[l]; kr[l] = wc_base + o_kr[l];
+      if (dtype == DS_BF16) { wq[l] = wc_base + o_q[l]; wr[l] = wc_base + o_r[l]; wo[l] = wc_base + o_o[l]; w1[l] = wc_base + o_1[l]; w2[l] = wc_base + o_2[l]; }
+    }
+    // stash
+    Arena sa;
+    const size_t act = (size_t)rows * H * esz, actF = (size_t)rows * F * esz, stats = (size_t)rows * 2 * 4;
+    mask_off = sa.reserve((size_t)S * Q * K * B * 4);
+    seg_off = sa.reserve((size_t)Q * K * B);
+    mem_off = sa.reserve((size_t)L * (Mm > 0 ? Mm : 1) * B * H * esz);
+    lo.resize(L);
+    size_t next_x = sa.reserve(act);
+    for (int l = 0; l < L; ++l) {
+      LayerOff& t = lo[l];
+      t.x = next_x;
+      t.qw = sa.reserve(act); t.qr = sa.reserve(act); t.qs = sa.reserve(act);
+      t.kv = sa.reserve((size_t)krows * 2 * H * esz);
+      t.p = sa.reserve((size_t)S * B * N * Q * K * esz);
+      t.vec = sa.reserve(act); t.z1 = sa.reserve(act); t.y1 = sa.reserve(act);
+      t.u = sa.reserve(actF); t.hh = sa.reserve(actF); t.z2 = sa.reserve(act);
+      t.st1 = sa.reserve(stats); t.st2 = sa.reserve(stats);
+      if (l + 1 < L) next_x = sa.reserve(act);
+    }
+    slot_bytes = sa.used;
+    DS_CHECK_HIP(hipMalloc((void**)&stash_base, slot_bytes * xc.stash_slots));
+    slot_forwarded.assign(xc.stash_slots, 0);
+    has_mask.assign(xc.stash_slots, 0);
+    has_seg.assign(xc.stash_slots, 0);
+    // workspace
+    Arena w;
+    ws_qall = w.reserve(act);
+    ws_ac = w.reserve((size_t)B * N * Q * K * 4);
+    ws_bd = w.reserve((size_t)B * N * Q * R * 4);
+    ws_ds = w.reserve((size_t)B * N * Q * K * esz);
+    ws_dbd = w.reserve((size_t)B * N * Q * R * esz);
+    ws_dz2 = w.reserve(act); ws_du = w.reserve(actF); ws_dy1 = w.reserve(act); ws_dz1 = w.reserve(act); ws_dvec = w.reserve(act);
+    ws_dqw = w.reserve(act); ws_dqr = w.reserve(act); ws_dqs = w.reserve(act); ws_dq = w.reserve(act);
+    ws_dkv = w.reserve((size_t)krows * 2 * H * esz);
+    ws_dkr = w.reserve((size_t)R * H * esz);
+    ws_deft = w.reserve((size_t)N * 2 * rows * esz);
+    ws_dx[0] = w.reserve(act); ws_dx[1] = w.reserve(act);
+    ws_bytes = w.used;
+    DS_CHECK_HIP(hipMalloc((void**)&ws_base, ws_bytes));
+    return DS_OK;
+  }
+
+  size_t workspace_bytes() const override { return ws_bytes; }
+  size_t stash_bytes(int slots) const override { return slot_bytes * (size_t)slots; }
+
+  const void* WT(int l, int which) const {
+    if (dtype == DS_BF16) {
+      switch (which) { case X_Q: return wq[l]; case X_R: return wr[l]; case X_O: return wo[l]; case X_W1: return w1[l]; default: return w2[l]; }
+    }
+    return w[base(l) + which];
+  }
+
+  int gemm(int am, int bm, int m, int n, int k, const void* a, int64_t lda, const void* b, int64_t ldb, void* c, int64_t ldc,
+           int flags = 0, const float* bias = nullptr, const void* residual = nullptr, void* c2 = nullptr) {
+    ds_gemm_desc d;
+    memset(&d, 0, sizeof(d));
+    d.dtype = dtype; d.a_major = am; d.b_major = bm; d.m = m; d.n = n; d.k = k; d.lda = lda; d.ldb = ldb; d.ldc = ldc;
+    d.batch = 1; d.batch_inner = 1; d.flags = flags; d.alpha = 1.f; d.a = a; d.b = b; d.c = c; d.bias = bias; d.residual = residual; d.c2 = c2;
+    return ds_gemm(&d, stream);
+  }
+  // batched over (b, n): zo = b, zi = n
+  int gemm_bn(int am, int bm, int m, int n, int k, const void* a, int64_t lda, int64_t a_so, int64_t a_si, const void* b,
+              int64_t ldb, int64_t b_so, int64_t b_si, void* c, int64_t ldc, int64_t c_so, int64_t c_si, int flags,
+              const void* residual = nullptr, int nb = -1) {
+    ds_gemm_desc d;
+    memset(&d, 0, sizeof(d));
+    d.dtype = dtype; d.a_major = am; d.b_major = bm; d.m = m; d.n = n; d.k = k; d.lda = lda; d.ldb = ldb; d.ldc = ldc;
+    d.batch = (nb < 0 ? B : nb) * N; d.batch_inner = N;
+    d.a_stride_outer = a_so; d.a_stride_inner = a_si; d.b_stride_outer = b_so; d.b_stride_inner = b_si;
+    d.c_stride_outer = c_so; d.c_stride_inner = c_si;
+    d.flags = flags; d.alpha = 1.f; d.a = a; d.b = b; d.c = c; d.residual = residual;
+    return ds_gemm(&d, stream);
+  }
+  static int g1(int64_t n) { int64_t b = (n + 255) / 256; return (int)(b > 8192 ? 8192 : (b < 1 ? 1 : b)); }
+
+  int refresh_weights() override {
+    if (dtype == DS_BF16) hipLaunchKernelGGL(xl_pos_emb_kernel<bf16>, dim3(g1((int64_t)R * H / 2)), dim3(256), 0, stream, R, H, K, (bf16*)pe);
+    else hipLaunchKernelGGL(xl_pos_emb_kernel<float>, dim3(g1((int64_t)R * H / 2)), dim3(256), 0, stream, R, H, K, (float*)pe);
+    DS_CHECK_LAUNCH();
+    for (int l = 0; l < L; ++l) {
+      const int b = base(l);
+      if (dtype == DS_BF16) {
+        hipLaunchKernelGGL(xl_pack_kv_kernel<bf16>, dim3(1024), dim3(256), 0, stream, H, w[b + X_K], w[b + X_V], (bf16*)wkv[l]);
+        DS_CHECK_LAUNCH();
+        DS_PROPAGATE(ds_cast_f32_to_bf16(wq[l], w[b + X_Q], (size_t)H * H, stream));
+        DS_PROPAGATE(ds_cast_f32_to_bf16(wr[l], w[b + X_R], (size_t)H * H, stream));
+        DS_PROPAGATE(ds_cast_f32_to_bf16(wo[l], w[b + X_O], (size_t)H * H, stream));
+        DS_PROPAGATE(ds_cast_f32_to_bf16(w1[l], w[b + X_W1], (size_t)H * F, stream));
+        DS_PROPAGATE(ds_cast_f32_to_bf16(w2[l], w[b + X_W2], (size_t)F * H, stream));
+      } else {
+        hipLaunchKernelGGL(xl_pack_kv_kernel<float>, dim3(1024), dim3(256), 0, stream, H, w[b + X_K], w[b + X_V], (float*)wkv[l]);
+        DS_CHECK_LAUNCH();
+      }
+      // k_r = pos_emb @ Wr does not depend on the micro-batch: once per refresh
+      DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, R, H, H, pe, H, WT(l, X_R), H, kr[l], H));
+    }
+    return DS_OK;
+  }
+
+  int set_aux(int slot, const float* masks, const uint8_t* seg_mat, const void* mems) {
+    char* sp = stash_base + (size_t)slot * slot_bytes;
+    if (masks) DS_CHECK_HIP(hipMemcpyAsync(sp + mask_off, masks, (size_t)S * Q * K * B * 4, hipMemcpyDeviceToDevice, stream));
+    if (seg_mat) DS_CHECK_HIP(hipMemcpyAsync(sp + seg_off, seg_mat, (size_t)Q * K * B, hipMemcpyDeviceToDevice, stream));
+    if (Mm > 0) {
+      if (!mems) { ds_set_error("ds_xlnet_stage_set_inputs: mem_len is %d but mems is NULL", Mm); return DS_EINVAL; }
+      DS_CHECK_HIP(hipMemcpyAsync(sp + mem_off, mems, (size_t)L * Mm * B * H * esz, hipMemcpyDeviceToDevice, stream));
+    }
+    has_mask[slot] = masks != nullptr;
+    has_seg[slot] = seg_mat != nullptr;
+    return DS_OK;
+  }
+
+  template <typename T> int softmax_fwd_t(const float* ac, const float* bd, const T* qs, const float* seg_emb, const uint8_t* seg,
+                                          const float* mask, float scale, T* p) {
+    const int64_t waves = (int64_t)B * N * Q;
+    dim3 grid((unsigned)((waves + 3) / 4));
+    const int need = (K + 255) / 256;
+    ds_prof_scope prof(stream, sizeof(T) == 2 ? "xl_softmax_fwd_kernel<bf16>" : "xl_softmax_fwd_kernel<float>",
+                       (double)waves * K * (8 + sizeof(T) + 5), "B");
+    if (need <= 1) hipLaunchKernelGGL((xl_softmax_fwd_kernel<T, 1>), grid, dim3(256), 0, stream, Q, K, R, B, N, D, ac, bd, qs, seg_emb, seg, mask, scale, p);
+    else if (need <= 2) hipLaunchKernelGGL((xl_softmax_fwd_kernel<T, 2>), grid, dim3(256), 0, stream, Q, K, R, B, N, D, ac, bd, qs, seg_emb, seg, mask, scale, p);
+    else if (need <= 4) hipLaunchKernelGGL((xl_softmax_fwd_kernel<T, 4>), grid, dim3(256), 0, stream, Q, K, R, B, N, D, ac, bd, qs, seg_emb, seg, mask, scale, p);
+    else hipLaunchKernelGGL((xl_softmax_fwd_kernel<T, 8>), grid, dim3(256), 0, stream, Q, K, R, B, N, D, ac, bd, qs, seg_emb, seg, mask, scale, p);
+    DS_CHECK_LAUNCH();
+    return DS_OK;
+  }
+
+  int forward(int slot, const void* in, const float*, void* out) override {
+    char* sp = stash_base + (size_t)slot * slot_bytes;
+    const size_t act = (size_t)rows * H * esz;
+    const float scale = 1.0f / sqrtf((float)D);
+    const uint8_t* seg = has_seg[slot] ? (const uint8_t*)(sp + seg_off) : nullptr;
+    DS_CHECK_HIP(hipMemcpyAsync(sp + lo[0].x, in, act, hipMemcpyDeviceToDevice, stream));
+    char* qall = ws_base + ws_qall;
+    float* ac = (float*)(ws_base + ws_ac);
+    float* bd = (float*)(ws_base + ws_bd);
+    for (int l = 0; l < L; ++l) {
+      const LayerOff& t = lo[l];
+      const int b = base(l);
+      char* x = sp + t.x;
+      char* y = (l + 1 < L) ? sp + lo[l + 1].x : (char*)out;
+      // q for every stream row; k|v for memory rows and for the content-stream rows
+      DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, rows, H, H, x, H, WT(l, X_Q), H, qall, H));
+      if (Mm > 0)
+        DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, Mm * B, 2 * H, H, sp + mem_off + (size_t)l * Mm * B * H * esz, H, wkv[l], 2 * H, sp + t.kv, 2 * H));
+      DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, rowsS, 2 * H, H, x, H, wkv[l], 2 * H, sp + t.kv + (size_t)Mm * B * 2 * H * esz, 2 * H));
+      {
+        const int64_t total = (int64_t)rows * H;
+        if (dtype == DS_BF16)
+          hipLaunchKernelGGL(xl_bias_q_kernel<bf16>, dim3(g1(total)), dim3(256), 0, stream, total, H, (const bf16*)qall, w[b + X_RW],
+                             w[b + X_RR], w[b + X_RS], (bf16*)(sp + t.qw), (bf16*)(sp + t.qr), (bf16*)(sp + t.qs));
+        else
+          hipLaunchKernelGGL(xl_bias_q_kernel<float>, dim3(g1(total)), dim3(256), 0, stream, total, H, (const float*)qall, w[b + X_RW],
+                             w[b + X_RR], w[b + X_RS], (float*)(sp + t.qw), (float*)(sp + t.qr), (float*)(sp + t.qs));
+        DS_CHECK_LAUNCH();
+      }
+      for (int s = 0; s < S; ++s) {
+        const size_t so = (size_t)s * rowsS * H * esz;
+        // ac = (q + r_w) k^T ; bd (unshifted) = (q + r_r) k_r^T
+        DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_K_MAJOR, Q, K, D, sp + t.qw + so, (int64_t)B * H, H, D, sp + t.kv, (int64_t)B * 2 * H, 2 * H, D,
+                             ac, K, (int64_t)N * Q * K, (int64_t)Q * K, DS_EPI_OUT_F32));
+        DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_K_MAJOR, Q, R, D, sp + t.qr + so, (int64_t)B * H, H, D, kr[l], H, 0, D,
+                             bd, R, (int64_t)N * Q * R, (int64_t)Q * R, DS_EPI_OUT_F32));
+        const float* mask = has_mask[slot] ? (const float*)(sp + mask_off) + (size_t)s * Q * K * B : nullptr;
+        char* p = sp + t.p + (size_t)s * B * N * Q * K * esz;
+        if (dtype == DS_BF16) DS_PROPAGATE(softmax_fwd_t<bf16>(ac, bd, (const bf16*)(sp + t.qs + so), w[b + X_SEG], seg, mask, scale, (bf16*)p));
+        else DS_PROPAGATE(softmax_fwd_t<float>(ac, bd, (const float*)(sp + t.qs + so), w[b + X_SEG], seg, mask, scale, (float*)p));
+        // vec = P v
+        DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_MN_MAJOR, Q, D, K, p, K, (int64_t)N * Q * K, (int64_t)Q * K, sp + t.kv + (size_t)H * esz,
+                             (int64_t)B * 2 * H, 2 * H, D, sp + t.vec + so, (int64_t)B * H, H, D, 0));
+      }
+      // attn_out = vec Wo^T (einsum ibnd,hnd->ibh) + x, LayerNorm
+      DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rows, H, H, sp + t.vec, H, WT(l, X_O), H, sp + t.z1, H, DS_EPI_RESIDUAL, nullptr, x));
+      DS_PROPAGATE(ds_layernorm_fwd(dtype, rows, H, sp + t.z1, w[b + X_LN1_G], w[b + X_LN1_B], xc.ln_eps, sp + t.y1, (float*)(sp + t.st1), stream));
+      DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, rows, F, H, sp + t.y1, H, WT(l, X_W1), F, sp + t.u, F,
+                        DS_EPI_BIAS | DS_EPI_GELU | DS_EPI_TANH_FORM, w[b + X_B1], nullptr, sp + t.hh));
+      DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, rows, H, F, sp + t.hh, F, WT(l, X_W2), H, sp + t.z2, H, DS_EPI_BIAS | DS_EPI_RESIDUAL,
+                        w[b + X_B2], sp + t.y1));
+      DS_PROPAGATE(ds_layernorm_fwd(dtype, rows, H, sp + t.z2, w[b + X_LN2_G], w[b + X_LN2_B], xc.ln_eps, y, (float*)(sp + t.st2), stream));
+    }
+    return DS_OK;
+  }
+
+  int backward(int slot, const void* d_out, void* d_in) override {
+    char* sp = stash_base + (size_t)slot * slot_bytes;
+    const float scale = 1.0f / sqrtf((float)D);
+    const uint8_t* seg = has_seg[slot] ? (const uint8_t*)(sp + seg_off) : nullptr;
+    const char* dy = (const char*)d_out;
+    char* dz2 = ws_base + ws_dz2; char* du = ws_base + ws_du; char* dy1 = ws_base + ws_dy1; char* dz1 = ws_base + ws_dz1;
+    char* dvec = ws_base + ws_dvec; char* dqw = ws_base + ws_dqw; char* dqr = ws_base + ws_dqr; char* dqs = ws_base + ws_dqs;
+    char* dq = ws_base + ws_dq; char* dkv = ws_base + ws_dkv; char* dkr = ws_base + ws_dkr; char* deft = ws_base + ws_deft;
+    float* dp = (float*)(ws_base + ws_ac);
+    char* dsm = ws_base + ws_ds; char* dbd = ws_base + ws_dbd;
+    for (int l = L - 1; l >= 0; --l) {
+      const LayerOff& t = lo[l];
+      const int b = base(l);
+      char* x = sp + t.x;
+      DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, dy, sp + t.z2, w[b + X_LN2_G], (const float*)(sp + t.st2), nullptr, dz2,
+                                    g[b + X_LN2_G], g[b + X_LN2_B], g[b + X_B2], stream));
+      DS_PROPAGATE(gemm(DS_MN_MAJOR, DS_MN_MAJOR, F, H, rows, sp + t.hh, F, dz2, H, g[b + X_W2], H, DS_EPI_ACCUM));
+      DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rows, F, H, dz2, H, WT(l, X_W2), H, du, F, DS_EPI_DGELU | DS_EPI_TANH_FORM, nullptr, nullptr, sp + t.u));
+      DS_PROPAGATE(ds_colsum_accum(dtype, rows, F, du, F, g[b + X_B1], stream));
+      DS_PROPAGATE(gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, F, rows, sp + t.y1, H, du, F, g[b + X_W1], F, DS_EPI_ACCUM));
+      DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rows, H, F, du, F, WT(l, X_W1), F, dy1, H, DS_EPI_RESIDUAL, nullptr, dz2));
+      DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, dy1, sp + t.z1, w[b + X_LN1_G], (const float*)(sp + t.st1), nullptr, dz1,
+                                    g[b + X_LN1_G], g[b + X_LN1_B], nullptr, stream));
+      // o projection: attn_out[row,h] = sum_nd vec[row,nd] Wo[h,nd]
+      DS_PROPAGATE(gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, rows, dz1, H, sp + t.vec, H, g[b + X_O], H, DS_EPI_ACCUM));
+      DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, rows, H, H, dz1, H, WT(l, X_O), H, dvec, H));
+      for (int s = 0; s < S; ++s) {
+        const size_t so = (size_t)s * rowsS * H * esz;
+        const char* p = sp + t.p + (size_t)s * B * N * Q * K * esz;
+        const int acc = s > 0 ? DS_EPI_RESIDUAL : 0;  // k, v, k_r are shared by the streams: add in place
+        // dP = dvec v^T ; dv (+)= P^T dvec
+        DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_K_MAJOR, Q, K, D, dvec + so, (int64_t)B * H, H, D, sp + t.kv + (size_t)H * esz, (int64_t)B * 2 * H,
+                             2 * H, D, dp, K, (int64_t)N * Q * K, (int64_t)Q * K, DS_EPI_OUT_F32));
+        DS_PROPAGATE(gemm_bn(DS_MN_MAJOR, DS_MN_MAJOR, K, D, Q, p, K, (int64_t)N * Q * K, (int64_t)Q * K, dvec + so, (int64_t)B * H, H, D,
+                             dkv + (size_t)H * esz, (int64_t)B * 2 * H, 2 * H, D, acc, dkv + (size_t)H * esz));
+        DS_PROPAGATE(ds_softmax_bwd(dtype, (int64_t)B * N * Q, K, p, dp, scale, dsm, stream));
+        // content term: dqw = dS k ; dk (+)= dS^T qw
+        DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_MN_MAJOR, Q, D, K, dsm, K, (int64_t)N * Q * K, (int64_t)Q * K, sp + t.kv, (int64_t)B * 2 * H, 2 * H, D,
+                             dqw + so, (int64_t)B * H, H, D, 0));
+        DS_PROPAGATE(gemm_bn(DS_MN_MAJOR, DS_MN_MAJOR, K, D, Q, dsm, K, (int64_t)N * Q * K, (int64_t)Q * K, sp + t.qw + so, (int64_t)B * H, H, D,
+                             dkv, (int64_t)B * 2 * H, 2 * H, D, acc, dkv));
+        // position term through the shift: dbd[i][r] = dS[i][r - Q + i]
+        {
+          const int64_t wr_ = (int64_t)B * N * Q;
+          if (dtype == DS_BF16) hipLaunchKernelGGL(xl_unshift_kernel<bf16>, dim3(g1(wr_ * R)), dim3(256), 0, stream, wr_, Q, K, R, (const bf16*)dsm, (bf16*)dbd);
+          else hipLaunchKernelGGL(xl_unshift_kernel<float>, dim3(g1(wr_ * R)), dim3(256), 0, stream, wr_, Q, K, R, (const float*)dsm, (float*)dbd);
+          DS_CHECK_LAUNCH();
+        }
+        DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_MN_MAJOR, Q, D, R, dbd, R, (int64_t)N * Q * R, (int64_t)Q * R, kr[l], H, 0, D,
+                             dqr + so, (int64_t)B * H, H, D, 0));
+        for (int bb = 0; bb < B; ++bb) {  // k_r is shared by the batch too: one launch per batch entry, added in place
+          const int a2 = (s > 0 || bb > 0) ? DS_EPI_RESIDUAL : 0;
+          DS_PROPAGATE(gemm_bn(DS_MN_MAJOR, DS_MN_MAJOR, R, D, Q, dbd + (size_t)bb * N * Q * R * esz, R, 0, (int64_t)Q * R,
+                               sp + t.qr + so + (size_t)bb * H * esz, (int64_t)B * H, 0, D, dkr, H, 0, D, a2, dkr, 1));
+        }
+        // segment term + dq = dqw + dqr + dqs
+        {
+          const int64_t waves = (int64_t)B * N * Q;
+          dim3 grid((unsigned)((waves + 3) / 4));
+          if (dtype == DS_BF16)
+            hipLaunchKernelGGL(xl_seg_bwd_kernel<bf16>, grid, dim3(256), 0, stream, Q, K, B, N, D, (int64_t)rows, (int64_t)s * rowsS,
+                               (const bf16*)dsm, seg, w[b + X_SEG], (const bf16*)(dqw + so), (const bf16*)(dqr + so), (bf16*)(dqs + so),
+                               (bf16*)(dq + so), (bf16*)deft);
+          else
+            hipLaunchKernelGGL(xl_seg_bwd_kernel<float>, grid, dim3(256), 0, stream, Q, K, B, N, D, (int64_t)rows, (int64_t)s * rowsS,
+                               (const float*)dsm, seg, w[b + X_SEG], (const float*)(dqw + so), (const float*)(dqr + so), (float*)(dqs + so),
+                               (float*)(dq + so), (float*)deft);
+          DS_CHECK_LAUNCH();
+        }
+      }
+      // relative biases: column sums of the three query-gradient pieces
+      DS_PROPAGATE(ds_colsum_accum(dtype, rows, H, dqw, H, g[b + X_RW], stream));
+      DS_PROPAGATE(ds_colsum_accum(dtype, rows, H, dqr, H, g[b + X_RR], stream));
+      DS_PROPAGATE(ds_colsum_accum(dtype, rows, H, dqs, H, g[b + X_RS], stream));
+      // seg_emb[s][n][:] += sum_rows def[row][n][s] * qs[row][n][:]   (batched over heads)
+      {
+        ds_gemm_desc d;
+        memset(&d, 0, sizeof(d));
+        d.dtype = dtype; d.a_major = DS_K_MAJOR; d.b_major = DS_MN_MAJOR; d.m = 2; d.n = D; d.k = rows;
+        d.lda = rows; d.ldb = H; d.ldc = H; d.batch = N; d.batch_inner = N;
+        d.a_stride_inner = (int64_t)2 * rows; d.b_stride_inner = D; d.c_stride_inner = D;
+        d.flags = DS_EPI_ACCUM; d.alpha = 1.f; d.a = deft; d.b = sp + t.qs; d.c = g[b + X_SEG];
+        DS_PROPAGATE(ds_gemm(&d, stream));
+      }
+      // projections
+      DS_PROPAGATE(gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, rows, x, H, dq, H, g[b + X_Q], H, DS_EPI_ACCUM));
+      DS_PROPAGATE(gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, R, pe, H, dkr, H, g[b + X_R], H, DS_EPI_ACCUM));
+      const char* dkv_h = dkv + (size_t)Mm * B * 2 * H * esz;
+      for (int j = 0; j < 2; ++j) {  // j = 0: k, 1: v
+        float* gw = g[b + X_K + j];
+        if (Mm > 0)
+          DS_PROPAGATE(gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, Mm * B, sp + mem_off + (size_t)l * Mm * B * H * esz, H, dkv + (size_t)j * H * esz,
+                            2 * H, gw, H, DS_EPI_ACCUM));
+        DS_PROPAGATE(gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, rowsS, x, H, dkv_h + (size_t)j * H * esz, 2 * H, gw, H, DS_EPI_ACCUM));
+      }
+      // dx = dq Wq^T + dz1 (residual); the content-stream rows also receive dkv Wkv^T
+      const bool first = l == 0;
+      if (first && d_in == nullptr) break;
+      char* dx = first ? (char*)d_in : ws_base + ws_dx[l & 1];
+      DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rows, H, H, dq, H, WT(l, X_Q), H, dx, H, DS_EPI_RESIDUAL, nullptr, dz1));
+      DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rowsS, H, 2 * H, dkv_h, 2 * H, wkv[l], 2 * H, dx, H, DS_EPI_RESIDUAL, nullptr, dx));
+      dy = dx;
+    }
+    return DS_OK;
+  }
+};
+
+}  // namespace
+
+extern "C" int ds_xlnet_stage_create(const ds_xlnet_cfg* c, void* stream, ds_stage** out) {
+  DS_CHECK_ARG(c != nullptr && out != nullptr, "ds_xlnet_stage_create: null argument");
+  *out = nullptr;
+  DS_CHECK_ARG(c->dtype == DS_F32 || c->dtype == DS_BF16, "ds_xlnet_stage_create: dtype %d", c->dtype);
+  DS_CHECK_ARG(c->num_layers > 0 && c->hidden > 0 && c->heads > 0 && c->ffn > 0 && c->batch > 0 && c->seq > 0 && c->mem_len >= 0,
+               "ds_xlnet_stage_create: non-positive shape");
+  DS_CHECK_ARG(c->streams == 1 || c->streams == 2, "ds_xlnet_stage_create: streams must be 1 (content) or 2 (content + query)");
+  DS_CHECK_ARG(c->hidden % c->heads == 0, "ds_xlnet_stage_create: hidden %d is not a multiple of heads %d", c->hidden, c->heads);
+  const int vec = c->dtype == DS_BF16 ? 8 : 4;
+  const int d = c->hidden / c->heads;
+  DS_CHECK_ARG(d % vec == 0 && d <= 64, "ds_xlnet_stage_create: head size %d must be a multiple of %d and at most 64", d, vec);
+  DS_CHECK_ARG(c->seq % vec == 0 && c->mem_len % vec == 0 && c->hidden % vec == 0 && c->ffn % vec == 0,
+               "ds_xlnet_stage_create: seq %d, mem_len %d, hidden %d, ffn %d must be multiples of %d", c->seq, c->mem_len, c->hidden, c->ffn, vec);
+  DS_CHECK_ARG(c->seq + c->mem_len <= 2048, "ds_xlnet_stage_create: klen %d exceeds 2048", c->seq + c->mem_len);
+  DS_CHECK_ARG(c->hidden <= 64 * vec * 8, "ds_xlnet_stage_create: hidden %d too large for the LayerNorm kernel", c->hidden);
+  DS_CHECK_ARG(c->stash_slots >= 1, "ds_xlnet_stage_create: stash_slots must be >= 1");
+  XlnetStage* s = new XlnetStage();
+  memset(&s->cfg, 0, sizeof(s->cfg));
+  s->cfg.kind = DS_STAGE_XLNET;
+  s->cfg.dtype = c->dtype;
+  s->cfg.stash_slots = c->stash_slots;
+  s->xc = *c;
+  s->stream = (hipStream_t)stream;
+  const int rc = s->init();
+  if (rc != DS_OK) { delete s; return rc; }
+  *out = s;
+  return DS_OK;
+}
+
+extern "C" int ds_xlnet_stage_set_inputs(ds_stage* h, int slot, const float* masks, const uint8_t* seg_mat, const void* mems) {
+  DS_CHECK_ARG(h != nullptr, "ds_xlnet_stage_set_inputs: null handle");
+  DS_CHECK_ARG(h->cfg.kind == DS_STAGE_XLNET, "ds_xlnet_stage_set_inputs: not an XLNet stage");
+  DS_CHECK_ARG(slot >= 0 && slot < h->cfg.stash_slots, "ds_xlnet_stage_set_inputs: slot %d out of range", slot);
+  return static_cast<XlnetStage*>(h)->set_aux(slot, masks, seg_mat, mems);
+}

@@ -11,7 +11,7 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._lib import DS_BF16, DS_F32, DS_STAGE_BERT, GnmtCfg, StageCfg, VggCfg, check, ptr
+from ._lib import DS_BF16, DS_F32, DS_STAGE_BERT, GnmtCfg, StageCfg, VggCfg, XlnetCfg, check, ptr
 
 
 def stash_depth(stage_index, num_stages, variant="S"):
@@ -227,6 +227,33 @@ def gnmt_stage(num_layers, units, vocab, batch, seq, stash_slots, forget_bias=1.
     return st
 
 
+class XlnetStage(Stage):
+    def set_inputs(self, slot, masks=None, seg_mat=None, mems=None):
+        """Side inputs of the micro-batch about to be forwarded into ``slot``: masks fp32
+        [streams, seq, klen, batch] (1 = masked), seg_mat uint8 [seq, klen, batch], mems [layers, mem_len, batch, hidden]."""
+        for t, dt in ((masks, torch.float32), (seg_mat, torch.uint8), (mems, self.act_dtype)):
+            if t is not None and (t.dtype != dt or not t.is_cuda or not t.is_contiguous()):
+                raise ValueError("side input must be a contiguous GPU tensor of %s" % dt)
+        check(self.lib.ds_xlnet_stage_set_inputs(self._h, slot, ptr(masks), ptr(seg_mat), ptr(mems)), "ds_xlnet_stage_set_inputs")
+
+
+def xlnet_stage(num_layers, hidden, heads, ffn, batch, seq, dtype, stash_slots, mem_len=0, streams=1, first_layer=0,
+                ln_eps=1e-14, device="cuda:0"):
+    """An XLNet stage of ``num_layers`` relative-attention layers (xlnet/models/slice_xlnet.py:164-180)."""
+    lib = _lib.load()
+    cfg = XlnetCfg()
+    cfg.dtype, cfg.num_layers, cfg.hidden, cfg.heads, cfg.ffn = _dtype_code(dtype), num_layers, hidden, heads, ffn
+    cfg.batch, cfg.seq, cfg.mem_len, cfg.streams = batch, seq, mem_len, streams
+    cfg.ln_eps, cfg.first_layer, cfg.stash_slots = ln_eps, first_layer, stash_slots
+    h = C.c_void_p()
+    with torch.cuda.device(torch.device(device)):
+        check(lib.ds_xlnet_stage_create(C.byref(cfg), _lib.current_stream(), C.byref(h)), "ds_xlnet_stage_create")
+    n = streams * seq * batch * hidden
+    st = XlnetStage(h, _TORCH_DTYPE[cfg.dtype], n, n, stash_slots, device=device, cfg=cfg)
+    st.out_shape = (streams, seq, batch, hidden)
+    return st
+
+
 class StageRuntime:
     """Runs one stage over M micro-batches in the early-backward order."""
 
@@ -239,7 +266,7 @@ class StageRuntime:
         self.m = num_micro_batches
         self.needs_input_grad = needs_input_grad and stage.takes_input_grad
 
-    def step(self, inputs, upstream, outputs, input_grads=None, key_masks=None):
+    def step(self, inputs, upstream, outputs, input_grads=None, key_masks=None, before_forward=None):
         """inputs[M], upstream[M]: device tensors; outputs[M] (and input_grads[M]) are filled.
         Weight gradients add into ``stage.grads`` (call ``stage.zero_grads()`` between steps)."""
         if len(inputs) != self.m or len(upstream) != self.m or len(outputs) != self.m:
@@ -249,6 +276,8 @@ class StageRuntime:
             if op == "F":
                 slot = free.pop(0)
                 slot_of[j] = slot
+                if before_forward is not None:
+                    before_forward(slot, j)          # e.g. XlnetStage.set_inputs for this micro-batch
                 self.stage.forward(slot, inputs[j], outputs[j], None if key_masks is None else key_masks[j])
             else:
                 slot = slot_of.pop(j)

@@ -179,6 +179,58 @@ def gnmt_id_inputs(seed, num_micro_batches, batch, seq, vocab):
     return [_rng(seed + m).integers(0, vocab, size=(batch, seq)).astype(np.int32) for m in range(num_micro_batches)]
 
 
+# --------------------------------------------------------------------------- XLNet
+def xlnet_layer_shapes(hidden, heads, ffn):
+    """Per-layer tensors of an XLNet layer (xlnet/layers/rel_multihead_attn.py:35-67, rel_bias.py:30-63,
+    segment_embed.py:23-31, position_wise_feed_forward.py:56-90, layer_normalization.py:47-67); q/k/v/r/o are
+    [hidden, heads, head_dim] flattened to [hidden, hidden]; the [num_layer, ...] bias and segment tables
+    of the reference are held one slice per layer."""
+    return [("q", (hidden, hidden)), ("k", (hidden, hidden)), ("v", (hidden, hidden)), ("r", (hidden, hidden)),
+            ("o", (hidden, hidden)), ("bias_context", (hidden,)), ("bias_relative", (hidden,)), ("bias_segment", (hidden,)),
+            ("seg_emb", (2, hidden)), ("attn_ln/gamma", (hidden,)), ("attn_ln/beta", (hidden,)),
+            ("ff/W1", (hidden, ffn)), ("ff/b1", (ffn,)), ("ff/W2", (ffn, hidden)), ("ff/b2", (hidden,)),
+            ("ff_ln/gamma", (hidden,)), ("ff_ln/beta", (hidden,))]
+
+
+def xlnet_weights(seed, num_layers, hidden, heads, ffn, first_layer=0, stddev=0.02, perturb=False):
+    rng = _rng(seed)
+    w = {}
+    for l in range(first_layer, first_layer + num_layers):
+        for name, shape in xlnet_layer_shapes(hidden, heads, ffn):
+            key = "layer_%d/%s" % (l, name)
+            if name.endswith("gamma"):
+                w[key] = (1 + 0.1 * rng.standard_normal(shape)).astype(np.float32) if perturb else np.ones(shape, np.float32)
+            elif name.endswith("beta") or name in ("ff/b1", "ff/b2"):
+                w[key] = (0.1 * rng.standard_normal(shape)).astype(np.float32) if perturb else np.zeros(shape, np.float32)
+            else:
+                w[key] = (rng.standard_normal(shape) * stddev).astype(np.float32)
+    return w
+
+
+def xlnet_perm_masks(seed, qlen, mlen, batch):
+    """Content- and query-stream masks [qlen, mlen+qlen, batch] (1 = masked) of a random factorization
+    order: position i sees j when j comes no later (content) / strictly earlier (query) in the order;
+    memory is always visible."""
+    rng = _rng(seed)
+    mh = np.zeros((qlen, mlen + qlen, batch), np.float32)
+    mg = np.zeros_like(mh)
+    for b in range(batch):
+        rank = np.empty(qlen, np.int64)
+        rank[rng.permutation(qlen)] = np.arange(qlen)
+        mh[:, mlen:, b] = (rank[None, :] > rank[:, None]).astype(np.float32)
+        mg[:, mlen:, b] = (rank[None, :] >= rank[:, None]).astype(np.float32)
+    return mh, mg
+
+
+def xlnet_stream_inputs(seed, num_micro_batches, qlen, batch, hidden, streams=2):
+    return [[_rng(seed + m + 100 * s).standard_normal((qlen, batch, hidden)).astype(np.float32) for s in range(streams)]
+            for m in range(num_micro_batches)]
+
+
+def xlnet_mems(seed, num_layers, mlen, batch, hidden):
+    return [_rng(seed + 7 * l).standard_normal((mlen, batch, hidden)).astype(np.float32) for l in range(num_layers)]
+
+
 # --------------------------------------------------------------------------- configs
 CONFIGS = {
     # BASELINE configs[0]: BERT-Large 2-layer encoder stage behind the embedding
@@ -195,4 +247,7 @@ CONFIGS = {
     "bert48_half": dict(index=3, kind="bert", num_layers=24, hidden=1024, heads=16, ffn=4096,
                         seq=512, micro_batch=2, num_micro_batches=8, dtype="bf16",
                         embeddings=None),
+    # BASELINE configs[4]: XLNet-36 half-stage, two streams, memory 384
+    "xlnet36_half": dict(index=4, kind="xlnet", num_layers=18, hidden=1024, heads=16, ffn=4096, seq=512, mem_len=384,
+                         micro_batch=1, num_micro_batches=8, dtype="bf16", streams=2),
 }

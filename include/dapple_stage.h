@@ -42,6 +42,7 @@ extern "C" {
 #define DS_EPI_OUT_F32 16  /* C is fp32 even when dtype is bf16 */
 #define DS_EPI_ACCUM 32    /* C (fp32) += acc, split-K allowed (atomic) */
 #define DS_EPI_RELU 64     /* C = max(acc + bias, 0) */
+#define DS_EPI_TANH_FORM 256 /* GELU / DGELU use the tanh approximation (xlnet/activations/gelu.py:6-11) */
 #define DS_EPI_MASK 128    /* C = aux[m][n] > 0 ? acc : 0 (ReLU backward), aux = c2 */
 
 const char* ds_last_error(void);
@@ -133,6 +134,7 @@ int ds_colsum_accum(int dtype, int rows, int cols, const void* x, int64_t ldx, f
 #define DS_STAGE_BERT 0
 #define DS_STAGE_VGG19 1
 #define DS_STAGE_GNMT 2
+#define DS_STAGE_XLNET 3
 
 typedef struct ds_stage_cfg {
   int kind;        /* DS_STAGE_* */
@@ -224,6 +226,29 @@ typedef struct ds_gnmt_cfg {
   int reserved[8];
 } ds_gnmt_cfg;
 int ds_gnmt_stage_create(const ds_gnmt_cfg* cfg, void* stream, ds_stage** out);
+
+/* XLNet stage (xlnet/models/slice_xlnet.py:164-180 layer body; xlnet/layers/rel_multihead_attn.py:71-149).
+ * Activations are sequence-major like the reference: in/out are [streams][seq][batch][hidden] (stream 0 =
+ * content stream h, stream 1 = query stream g).  Per-layer weights, in ds_stage_weight_info order:
+ * q, k, v, r, o ([hidden, heads*head_dim]), bias_context, bias_relative, bias_segment ([hidden]),
+ * seg_emb ([2, hidden]), attn_ln/{gamma,beta}, ff/{W1,b1,W2,b2}, ff_ln/{gamma,beta}.
+ * mem_len > 0 and streams == 2 go beyond what the reference builds (it hard-wires memory length 0 and has
+ * the content stream only, lambda_funcs.py:20,36) and follow the XLNet formulation. */
+typedef struct ds_xlnet_cfg {
+  int dtype;
+  int num_layers, hidden, heads, ffn;
+  int batch, seq, mem_len, streams;
+  float ln_eps;     /* 1e-14 = K.epsilon()**2 (layer_normalization.py:37-39) */
+  int first_layer;  /* names only */
+  int stash_slots;
+  int reserved[8];
+} ds_xlnet_cfg;
+int ds_xlnet_stage_create(const ds_xlnet_cfg* cfg, void* stream, ds_stage** out);
+/* Side inputs of the micro-batch that will be forwarded into `slot` (copied into the slot):
+ *   masks   [streams][seq][mem_len+seq][batch] fp32, 1 = masked (get_attn_mask, lambda_funcs.py:7-44); NULL = none
+ *   seg_mat [seq][mem_len+seq][batch] uint8, 1 = different segment (segment_embed.py:41-52); NULL = all equal
+ *   mems    [num_layers][mem_len][batch][hidden] in the compute type; required when mem_len > 0 */
+int ds_xlnet_stage_set_inputs(ds_stage* h, int slot, const float* masks, const uint8_t* seg_mat, const void* mems);
 
 #ifdef __cplusplus
 }
