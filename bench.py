@@ -2,11 +2,14 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload bert48_half] [--no-cpu-baseline]
 
-One step = the whole 1F1B pass of the stage over its M micro-batches: refresh the bf16
-compute copies of the fp32 master weights, zero the master gradients, then M forwards
-and M backwards in the early-backward order with in-place fp32 gradient accumulation.
-Inputs, weights and upstream gradients are synthetic, seeded and already resident in HBM.
-Prints ONE JSON line.
+One step = the whole early-backward (1F1B) pass of one stage over its M micro-batches: refresh
+the compute copies of the fp32 master weights, zero the master gradients, then M forwards and M
+backwards in schedule order with in-place fp32 gradient accumulation.  Inputs, weights and
+upstream gradients are synthetic, seeded and already resident in HBM.  Prints ONE JSON line.
+
+Workloads (BASELINE.json configs): bert48_half (configs[3], the one the metric is quoted on and
+the default), bert_large_2l (configs[0]), vgg19_stage0 (configs[1]), gnmt16_encoder (configs[2]),
+xlnet36_half (configs[4]).
 """
 import argparse
 import json
@@ -20,68 +23,28 @@ sys.path.insert(0, ROOT)
 PEAK = {"bf16": 2.5e15, "fp32": 157.3e12, "hbm": 8.0e12}  # MI355X dense MFMA FLOP/s and HBM B/s
 
 
-def stage_flops_per_sample(c):
-    """fwd+bwd algorithmic FLOPs of one sample: 3 x 2 x MACs of every contraction in the layers."""
-    S, H, F = c["seq"], c["hidden"], c["ffn"]
-    fwd = 2 * S * (4 * H * H + 2 * H * F) + 4 * S * S * H
-    return 3 * fwd * c["num_layers"]
-
-
-def cpu_baseline(c, layers_timed=None):
-    """Times the fp32 torch-CPU restatement of the same stage on the host cores (a baseline only)."""
-    import torch
-    from dapple_amd import synthetic
-    from oracle import bert as ob
-    B, S, H, F, N = c["micro_batch"], c["seq"], c["hidden"], c["ffn"], c["heads"]
-    L = c["num_layers"] if layers_timed is None else layers_timed
+def host_cores():
     cores = os.cpu_count() or 1
     try:
         cores = min(cores, len(os.sched_getaffinity(0)))
     except Exception:
         pass
-    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
-    torch.set_num_threads(cores)
-    w = ob.to_torch(synthetic.bert_weights(synthetic.SEED_WEIGHT + c["index"], L, H, F), torch.float32, requires_grad=True)
-    x = torch.as_tensor(synthetic.bert_activation_inputs(synthetic.SEED_INPUT + c["index"], 1, B, S, H)[0])
-    dy = torch.as_tensor(synthetic.upstream_grads(synthetic.SEED_GRAD + c["index"], 1, (B * S, H))[0])
-    layers = list(range(L))
-    ob.stage_vjp(x, w, dy, layers[:1], B, S, N)          # warm-up: one layer
-    t0 = time.perf_counter()
-    ob.stage_vjp(x, w, dy, layers, B, S, N)
-    dt = time.perf_counter() - t0
-    dt_full = dt * c["num_layers"] / L
-    return {"value": B / dt_full, "unit": "samples/s", "cores": cores, "kind": "port",
-            "sample": "1 of %d micro-batches (%d samples) fwd+bwd through %d of %d layers, fp32 torch-CPU restatement, "
-                      "%.1f s, scaled to the full stage" % (c["num_micro_batches"], B, L, c["num_layers"], dt)}
+    return min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=5)
-    ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="bert48_half")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--layers", type=int, default=None, help="override the layer count (debugging only; marks the line invalid)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build runs one pipeline stage on ONE GPU; --gpus %d is not supported "
-              "(no collectives or sharding are part of it)" % args.gpus, file=sys.stderr)
-        sys.exit(2)
+# ------------------------------------------------------------------------------------------ workloads
+class Workload:
+    """step(): one stage step on the GPU; cpu_baseline(): (seconds, samples, description) of the fp32
+    torch-CPU restatement on a bounded sample of the same workload."""
 
+
+def make_bert(c, args):
     import torch
-    from dapple_amd import _lib, runtime, synthetic
-
-    c = dict(synthetic.CONFIGS[args.workload])
-    if args.layers is not None:
-        c["num_layers"] = args.layers
-    dtype = c["dtype"]
-    adt = torch.bfloat16 if dtype == "bf16" else torch.float32
+    from dapple_amd import runtime, synthetic
     B, S, H, F, N, L, M = c["micro_batch"], c["seq"], c["hidden"], c["ffn"], c["heads"], c["num_layers"], c["num_micro_batches"]
-    num_stages, stage_index = 2, 0
-    K = runtime.stash_depth(stage_index, num_stages)
-
-    stage = runtime.bert_stage(L, H, N, F, B, S, dtype, stash_slots=K, embeddings=c["embeddings"])
+    adt = torch.bfloat16 if c["dtype"] == "bf16" else torch.float32
+    K = runtime.stash_depth(0, 2)
+    stage = runtime.bert_stage(L, H, N, F, B, S, c["dtype"], stash_slots=K, embeddings=c["embeddings"])
     stage.bind(synthetic.bert_weights(synthetic.SEED_WEIGHT + c["index"], L, H, F, embeddings=c["embeddings"]))
     if c["embeddings"] is None:
         xs = [torch.as_tensor(x).cuda().to(adt) for x in synthetic.bert_activation_inputs(synthetic.SEED_INPUT + c["index"], M, B, S, H)]
@@ -91,27 +54,190 @@ def main():
         dxs = None
     dys = [torch.as_tensor(x).cuda().to(adt) for x in synthetic.upstream_grads(synthetic.SEED_GRAD + c["index"], M, (B * S, H))]
     outs = [torch.empty(B * S, H, dtype=adt, device="cuda") for _ in range(M)]
-    rt = runtime.StageRuntime(stage, stage_index, num_stages, M)
+    rt = runtime.StageRuntime(stage, 0, 2, M)
+    wl = Workload()
+    wl.stage = stage
+    wl.step = lambda: (stage.refresh_weights(), stage.zero_grads(), rt.step(xs, dys, outs, dxs))
+    wl.samples = B * M
+    fwd = 2 * S * (4 * H * H + 2 * H * F) + 4 * S * S * H
+    wl.flops_per_sample = 3 * fwd * L
+    wl.config = {"layers": L, "hidden": H, "heads": N, "ffn": F, "seq": S, "micro_batch": B, "micro_batches": M,
+                 "embedding": c["embeddings"] is not None, "schedule": "1F1B stage 0 of 2, stash K=%d" % K}
 
-    def step():
-        stage.refresh_weights()
-        stage.zero_grads()
-        rt.step(xs, dys, outs, dxs)
+    def cpu():
+        from oracle import bert as ob
+        Lt = min(L, 24)
+        w = ob.to_torch(synthetic.bert_weights(synthetic.SEED_WEIGHT + c["index"], Lt, H, F, embeddings=c["embeddings"]),
+                        torch.float32, requires_grad=True)
+        x = xs[0].cpu() if c["embeddings"] is not None else xs[0].cpu().float()
+        dy = dys[0].cpu().float()
+        ob.stage_vjp(x, w, dy, [0], B, S, N)
+        t0 = time.perf_counter()
+        ob.stage_vjp(x, w, dy, list(range(Lt)), B, S, N)
+        dt = time.perf_counter() - t0
+        return dt, B, "1 of %d micro-batches (%d samples) fwd+bwd through all %d layers" % (M, B, Lt)
+    wl.cpu = cpu
+    return wl
+
+
+def make_vgg(c, args):
+    import torch
+    from dapple_amd import runtime, synthetic
+    B, M, layers = c["micro_batch"], c["num_micro_batches"], c["layers"]
+    Hh, Ww, Cin = c["height"], c["width"], c["in_channels"]
+    K = runtime.stash_depth(0, 2, "2S-1")
+    stage = runtime.vgg_stage(layers, B, Hh, Ww, Cin, stash_slots=K)
+    stage.bind(synthetic.vgg_weights(synthetic.SEED_WEIGHT + c["index"], layers, Cin))
+    xs = [torch.as_tensor(x).cuda() for x in synthetic.vgg_inputs(synthetic.SEED_INPUT + c["index"], M, B, Hh, Ww, Cin)]
+    dys = [torch.as_tensor(x).cuda() for x in synthetic.upstream_grads(synthetic.SEED_GRAD + c["index"], M, stage.out_shape)]
+    outs = [torch.empty(stage.out_shape, device="cuda") for _ in range(M)]
+    rt = runtime.StageRuntime(stage, 0, 2, M, variant="2S-1", needs_input_grad=False)
+    wl = Workload()
+    wl.stage = stage
+    wl.step = lambda: (stage.refresh_weights(), stage.zero_grads(), rt.step(xs, dys, outs))
+    wl.samples = B * M
+    macs, h, w_, cin, first = 0, Hh, Ww, Cin, None
+    for _, cout in layers:
+        if cout is None:
+            h, w_ = h // 2, w_ // 2
+        else:
+            m = h * w_ * 9 * cin * cout
+            first = m if first is None else first
+            macs += m
+            cin = cout
+    wl.flops_per_sample = 2 * (3 * macs - first)       # no input gradient through the first conv
+    wl.config = {"convs": sum(1 for _, c_ in layers if c_), "pools": sum(1 for _, c_ in layers if c_ is None),
+                 "image": [Hh, Ww, Cin], "micro_batch": B, "micro_batches": M, "schedule": "1F1B (2S-1 variant) stage 0 of 2, stash K=%d" % K}
+
+    def cpu():
+        from oracle import vgg as ov
+        nb = 4
+        w = ov.to_torch(synthetic.vgg_weights(synthetic.SEED_WEIGHT + c["index"], layers, Cin), torch.float32, requires_grad=True)
+        x, dy = xs[0][:nb].cpu(), dys[0][:nb].cpu()
+        t0 = time.perf_counter()
+        ov.stage_vjp(x, w, dy, layers)
+        dt = time.perf_counter() - t0
+        return dt, nb, "%d of %d images of one micro-batch, fwd+bwd through all %d ops" % (nb, B, len(layers))
+    wl.cpu = cpu
+    return wl
+
+
+def make_gnmt(c, args):
+    import torch
+    from dapple_amd import runtime, synthetic
+    L, U, V, B, T, M = c["num_layers"], c["units"], c["vocab"], c["micro_batch"], c["seq"], c["num_micro_batches"]
+    K = runtime.stash_depth(0, 2)
+    stage = runtime.gnmt_stage(L, U, V, B, T, stash_slots=K, forget_bias=c["forget_bias"])
+    stage.bind(synthetic.gnmt_weights(synthetic.SEED_WEIGHT + c["index"], L, U, V))
+    ids = [torch.as_tensor(x).cuda() for x in synthetic.gnmt_id_inputs(synthetic.SEED_INPUT + c["index"], M, B, T, V)]
+    dys = [torch.as_tensor(x).cuda() for x in synthetic.upstream_grads(synthetic.SEED_GRAD + c["index"], M, (T, B, U))]
+    outs = [torch.empty(T, B, U, device="cuda") for _ in range(M)]
+    rt = runtime.StageRuntime(stage, 0, 2, M)
+    wl = Workload()
+    wl.stage = stage
+    wl.step = lambda: (stage.refresh_weights(), stage.zero_grads(), rt.step(ids, dys, outs))
+    wl.samples = B * M
+    per_token = 2 * 4 * U * (2 * (U + U) + (2 * U + U) + (L - 2) * (U + U))
+    wl.flops_per_sample = 3 * per_token * T
+    wl.config = {"layers": L, "units": U, "vocab": V, "seq": T, "micro_batch": B, "micro_batches": M,
+                 "schedule": "1F1B stage 0 of 2, stash K=%d" % K}
+
+    def cpu():
+        from oracle import gnmt as og
+        nb = 16
+        w = og.to_torch(synthetic.gnmt_weights(synthetic.SEED_WEIGHT + c["index"], L, U, V), torch.float32, requires_grad=True)
+        t0 = time.perf_counter()
+        og.stage_vjp(ids[0][:nb].cpu(), w, dys[0][:, :nb].cpu().contiguous(), L, c["forget_bias"])
+        dt = time.perf_counter() - t0
+        return dt, nb, "%d of %d sequences of one micro-batch, fwd+BPTT through all %d layers" % (nb, B, L)
+    wl.cpu = cpu
+    return wl
+
+
+def make_xlnet(c, args):
+    import numpy as np
+    import torch
+    from dapple_amd import runtime, synthetic
+    L, H, N, F, B, Q, Mm, S, M = (c["num_layers"], c["hidden"], c["heads"], c["ffn"], c["micro_batch"], c["seq"], c["mem_len"],
+                                  c["streams"], c["num_micro_batches"])
+    adt = torch.bfloat16 if c["dtype"] == "bf16" else torch.float32
+    K = runtime.stash_depth(0, 2)
+    stage = runtime.xlnet_stage(L, H, N, F, B, Q, c["dtype"], stash_slots=K, mem_len=Mm, streams=S)
+    stage.bind(synthetic.xlnet_weights(synthetic.SEED_WEIGHT + c["index"], L, H, N, F))
+    xs = [torch.as_tensor(np.stack(x)).cuda().to(adt) for x in synthetic.xlnet_stream_inputs(synthetic.SEED_INPUT + c["index"], M, Q, B, H, S)]
+    dys = [torch.as_tensor(np.stack(x)).cuda().to(adt) for x in synthetic.xlnet_stream_inputs(synthetic.SEED_GRAD + c["index"], M, Q, B, H, S)]
+    outs = [torch.empty(S, Q, B, H, dtype=adt, device="cuda") for _ in range(M)]
+    dxs = [torch.empty_like(o) for o in outs]
+    masks_np = synthetic.xlnet_perm_masks(90 + c["index"], Q, Mm, B)[:S]
+    masks = torch.as_tensor(np.stack(masks_np)).cuda()
+    mems_np = synthetic.xlnet_mems(50 + c["index"], L, Mm, B, H)
+    mems = torch.as_tensor(np.stack(mems_np)).cuda().to(adt)
+    rt = runtime.StageRuntime(stage, 0, 2, M)
+    hook = lambda slot, j: stage.set_inputs(slot, masks, None, mems)
+    wl = Workload()
+    wl.stage = stage
+    wl.step = lambda: (stage.refresh_weights(), stage.zero_grads(), rt.step(xs, dys, outs, dxs, before_forward=hook))
+    wl.samples = B * M
+    Kl, R = Mm + Q, Mm + 2 * Q
+    # per layer fwd: q (S streams), k|v over klen, k_r over rlen, o (S streams), scores/values and position term per stream, FFN
+    fwd = 2 * H * H * (S * Q + 2 * Kl + R + S * Q) + S * (2 * 2 * Q * Kl * H + 2 * Q * R * H) + S * 4 * Q * H * F
+    wl.flops_per_sample = 3 * fwd * L
+    wl.config = {"layers": L, "hidden": H, "heads": N, "ffn": F, "seq": Q, "mem_len": Mm, "streams": S, "micro_batch": B,
+                 "micro_batches": M, "schedule": "1F1B stage 0 of 2, stash K=%d" % K, "flops": "two-stream count"}
+
+    def cpu():
+        from oracle import xlnet as ox
+        Lt = 4
+        w = ox.to_torch(synthetic.xlnet_weights(synthetic.SEED_WEIGHT + c["index"], Lt, H, N, F), torch.float32, requires_grad=True)
+        streams = [xs[0][s].cpu().float() for s in range(S)]
+        d_outs = [dys[0][s].cpu().float() for s in range(S)]
+        mm = [torch.as_tensor(m) for m in mems_np[:Lt]]
+        mk = [torch.as_tensor(m) for m in masks_np]
+        t0 = time.perf_counter()
+        ox.stage_vjp(streams, mm, w, d_outs, list(range(Lt)), N, mk, torch.zeros(Q, B, dtype=torch.int64))
+        dt = time.perf_counter() - t0
+        return dt * L / Lt, B, "1 of %d micro-batches (%d sample) fwd+bwd through %d of %d layers, scaled to %d" % (M, B, Lt, L, L)
+    wl.cpu = cpu
+    return wl
+
+
+MAKERS = {"bert": make_bert, "vgg": make_vgg, "gnmt": make_gnmt, "xlnet": make_xlnet}
+METRIC = {"bert48_half": "stage samples/sec fwd+bwd+grad-accum, BERT-48 half-stage; MFMA util %"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", default="bert48_half")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs one pipeline stage on ONE GPU; --gpus %d is not supported "
+              "(no collectives or sharding are part of it)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from dapple_amd import _lib, synthetic
+
+    c = dict(synthetic.CONFIGS[args.workload])
+    dtype = c["dtype"]
+    wl = MAKERS[c["kind"]](c, args)
 
     for _ in range(args.warmup):
-        step()
+        wl.step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        step()
+        wl.step()
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / args.steps
-    samples = B * M
-    value = samples / dt
+    value = wl.samples / dt
 
     # per-kernel durations: one more step with HIP events around every launch (same stream)
     _lib.profile(True)
-    step()
+    wl.step()
     torch.cuda.synchronize()
     prof = _lib.profile_dump()
     _lib.profile(False)
@@ -119,40 +245,40 @@ def main():
     dom = max(prof, key=lambda t: prof[t][1])
     n, ms, work, unit = prof[dom]
     if unit == "FLOP":
-        peak = PEAK[dtype]
-        roof = {"bound": "mfma", "achieved": work / (ms * 1e-3) / 1e12, "peak": peak / 1e12, "unit": "TFLOP/s"}
+        roof = {"bound": "mfma", "achieved": work / (ms * 1e-3) / 1e12, "peak": PEAK[dtype] / 1e12, "unit": "TFLOP/s"}
     else:
-        peak = PEAK["hbm"]
-        roof = {"bound": "hbm", "achieved": work / (ms * 1e-3) / 1e9, "peak": peak / 1e9, "unit": "GB/s"}
+        roof = {"bound": "hbm", "achieved": work / (ms * 1e-3) / 1e9, "peak": PEAK["hbm"] / 1e9, "unit": "GB/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
     roof["traffic"] = None
-    roof["kernel"] = dom
-    roof["launches"] = n
-    roof["avg_launch_us"] = ms * 1e3 / n
-    roof["share_of_kernel_time"] = ms / total_ms
-    stage_flops = stage_flops_per_sample(c) * samples
+    roof.update({"kernel": dom, "launches": n, "avg_launch_us": ms * 1e3 / n, "share_of_kernel_time": ms / total_ms})
+    stage_flops = wl.flops_per_sample * wl.samples
     roof["stage_achieved_TFLOPs"] = stage_flops / dt / 1e12
     roof["stage_frac_of_mfma_peak"] = stage_flops / dt / PEAK[dtype]
     kernels = {t: {"launches": v[0], "ms": round(v[1], 3),
                    "rate": round(v[2] / (v[1] * 1e-3) / (1e12 if v[3] == "FLOP" else 1e9), 2),
                    "unit": "TFLOP/s" if v[3] == "FLOP" else "GB/s"} for t, v in sorted(prof.items(), key=lambda kv: -kv[1][1])}
-
+    cfg = {"workload": args.workload, "grad_accum": "fp32 in place", "flops_per_sample": wl.flops_per_sample}
+    cfg.update(wl.config)
     line = {
-        "metric": "stage samples/sec fwd+bwd+grad-accum, BERT-48 half-stage; MFMA util %",
+        "metric": METRIC.get(args.workload, "stage samples/sec fwd+bwd+grad-accum, %s; MFMA util %%" % args.workload),
         "value": value, "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": dtype, "data": "synthetic",
-        "config": {"workload": args.workload + ("" if args.layers is None else "[layers=%d: NOT the baseline config]" % args.layers),
-                   "layers": L, "hidden": H, "heads": N, "ffn": F, "seq": S, "micro_batch": B, "micro_batches": M,
-                   "schedule": "1F1B stage %d of %d, stash K=%d" % (stage_index, num_stages, K),
-                   "grad_accum": "fp32 in place"},
-        "roofline": roof,
-        "kernels": kernels,
+        "dtype": dtype, "data": "synthetic", "config": cfg, "roofline": roof, "kernels": kernels,
     }
-    stage.close()
-    del stage
+    cpu = wl.cpu
+    wl.stage.close()
+    del wl
+    torch.cuda.empty_cache()
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(c, layers_timed=min(L, 4))
+        cores = host_cores()
+        torch.set_num_threads(cores)
+        secs, samples, what = 0.0, 0, ""
+        while secs < 10.0:          # repeat the bounded sample until it amounts to >= 10 s of CPU work
+            t, n_, what = cpu()
+            secs += t
+            samples += n_
+        line["cpu_baseline"] = {"value": samples / secs, "unit": "samples/s", "cores": cores, "kind": "port",
+                                "sample": "%s, fp32 torch-CPU restatement, %.1f s" % (what, secs)}
     else:
         line["cpu_baseline"] = None
     print(json.dumps(line))

@@ -1,0 +1,346 @@
+// Fused softmax attention for bf16, head size 64 (gfx950 MFMA): forward, and backward as two kernels
+// (dQ parallel over queries, dK/dV parallel over keys).  Replaces the score matmul, scale, mask adder,
+// softmax and context matmul of bert/models/bert/modeling_slice.py:499-533 and their tf.gradients,
+// without materialising the [B, N, S, S] probabilities.
+//
+// Every kernel keeps the MFMA output "transposed": the tile it produces has the softmax axis (keys in
+// forward/dQ, queries in dK/dV) running down the 16 accumulator registers of a lane and the other
+// axis across lanes.  Row statistics (max, sum, logsumexp, delta) are then per-lane scalars, and the
+// accumulator registers, converted to bf16, ARE the B operand of the next MFMA (k = softmax axis) -
+// no shuffle, no LDS round trip.  The matching A operands (V^T, K^T, Q^T, dO^T) are read from
+// row-major LDS tiles with ds_read_b64_tr_b16.
+//
+// q, k, v are column blocks of one [B*S, ld] matrix (the fused QKV projection); head h owns columns
+// h*64 .. h*64+63 of each block.
+#include "common.h"
+
+namespace {
+
+typedef __attribute__((address_space(3))) void* lds_vptr;
+typedef __attribute__((address_space(1))) void* glb_vptr;
+#define VMCNT0 ((0 & 15) | ((0 >> 4) << 14) | (7 << 4) | (15 << 8))
+
+constexpr int HD = 64;        // head size
+constexpr int ROWB = 128;     // bytes per tile row (64 bf16)
+constexpr int CHUNK = 512;    // rows of K/V (or Q/dO) resident in LDS at a time
+
+// LDS tile layout: row-major [row][64 bf16], 32-byte granules XOR-swizzled by the row
+__device__ __forceinline__ int tile_off(int row, int byte) {
+  const int g = (byte >> 5) ^ (((row & 3) << 1) & 3);
+  return row * ROWB + (g << 5) + (byte & 31);
+}
+
+// Fills `rows` tile rows (multiple of 16) from global rows of stride ld (elements); 128 threads.
+__device__ __forceinline__ void tile_fill(char* lds, const bf16* src, int64_t ld, int rows, int wave, int lane) {
+  for (int c = wave; c < rows / 8; c += 2) {  // each call: one wave writes 64 consecutive 16-byte slots = 8 rows
+    const int p = c * 64 + lane;
+    const int r = p >> 3, pc = p & 7;
+    const int g = (pc >> 1) ^ (((r & 3) << 1) & 3);
+    const bf16* s = src + (int64_t)r * ld + (g * 2 + (pc & 1)) * 8;
+    __builtin_amdgcn_global_load_lds((glb_vptr)s, (lds_vptr)(lds + c * 1024), 16, 0, 0);
+  }
+}
+
+// A operand, rows = tile rows (row0 + lane%32), k = 8 consecutive columns starting at 16*ks + 8*half
+__device__ __forceinline__ bf16x8 frag_rows(const char* lds, int row0, int ks, int lane) {
+  return *reinterpret_cast<const bf16x8*>(lds + tile_off(row0 + (lane & 31), (2 * ks + (lane >> 5)) * 16));
+}
+// A operand of the transposed use: rows = tile columns (col0 + lane%32), k = tile rows in the order the
+// accumulator layout hands them over: elements 0-3 -> rows r0 + 4*half + 0..3, elements 4-7 -> r0 + 8 + 4*half + 0..3
+__device__ __forceinline__ bf16x8 frag_cols(const char* lds, int r0, int col0, int lane) {
+  const int h = lane >> 5, s = lane & 15;
+  const int col = col0 + (((lane >> 4) & 1) << 4) + ((s & 3) << 2);
+  typedef __attribute__((address_space(3))) s16x4* lp;
+  union { s16x4 v[2]; bf16x8 f; } u;
+  u.v[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lp)(lds + tile_off(r0 + 4 * h + (s >> 2), col * 2)));
+  u.v[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lp)(lds + tile_off(r0 + 8 + 4 * h + (s >> 2), col * 2)));
+  return u.f;
+}
+__device__ __forceinline__ bf16x8 pack8(const float* p) {
+  bf16x8 r;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) r[j] = (bf16)p[j];
+  return r;
+}
+__device__ __forceinline__ f32x16 mfma(bf16x8 a, bf16x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+// index along the softmax axis of accumulator element e for this lane's half: (e/4)*8 + 4*half + e%4
+__device__ __forceinline__ int acc_row(int e, int half) { return (e >> 2) * 8 + half * 4 + (e & 3); }
+
+struct AttnArgs {
+  const bf16* qkv; int64_t ld;   // q at column 0, k at H, v at 2H
+  const float* key_mask;         // [B, S] 0/1 or null
+  bf16* ctx;                     // [B*S, H]
+  float* lse;                    // [B, N, S]
+  const bf16* dctx;              // backward
+  bf16* dqkv;
+  float* delta;                  // [B, N, S]
+  int B, N, S, H;
+  float scale, mask_value;
+};
+
+// store a transposed 64 x 32 accumulator pair (rows d, columns = this lane's row index) as out[row][d]
+__device__ __forceinline__ void store_t(bf16* out_row, const f32x16 (&acc)[2], float mul, int half) {
+#pragma unroll
+  for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      bf16x4 v;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] = (bf16)(acc[dt][g * 4 + j] * mul);
+      *reinterpret_cast<bf16x4*>(out_row + dt * 32 + g * 8 + half * 4) = v;
+    }
+}
+
+// ----------------------------------------------------------------------------------- forward
+// grid (S/64, B*N), 128 threads: each wave owns 32 queries, walks all keys.
+__global__ __launch_bounds__(128) void attn_fwd_kernel(AttnArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5;
+  const int b = blockIdx.y / a.N, hd = blockIdx.y % a.N;
+  const int q = blockIdx.x * 64 + wave * 32 + (lane & 31);
+  const bf16* base = a.qkv + (int64_t)b * a.S * a.ld + hd * HD;
+  char* sk = lds;
+  char* sv = lds + CHUNK * ROWB;
+  float* adder = reinterpret_cast<float*>(lds + 2 * CHUNK * ROWB);
+  for (int j = threadIdx.x; j < a.S; j += 128)
+    adder[j] = a.key_mask ? (1.0f - a.key_mask[(int64_t)b * a.S + j]) * a.mask_value : 0.f;
+  bf16x8 qf[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(base + (int64_t)q * a.ld + 16 * ks + 8 * half);
+  f32x16 o[2];
+#pragma unroll
+  for (int e = 0; e < 16; ++e) { o[0][e] = 0.f; o[1][e] = 0.f; }
+  float m = -INFINITY, l = 0.f;
+  for (int k0 = 0; k0 < a.S; k0 += CHUNK) {
+    const int rows = a.S - k0 < CHUNK ? a.S - k0 : CHUNK;
+    __syncthreads();
+    tile_fill(sk, base + a.H + (int64_t)k0 * a.ld, a.ld, rows, wave, lane);
+    tile_fill(sv, base + 2 * a.H + (int64_t)k0 * a.ld, a.ld, rows, wave, lane);
+    __builtin_amdgcn_s_waitcnt(VMCNT0);
+    __syncthreads();
+    for (int kt = 0; kt < rows; kt += 32) {
+      f32x16 s;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) s[e] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) s = mfma(frag_rows(sk, kt, ks, lane), qf[ks], s);
+      float p[16];
+      float mt = -INFINITY;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        p[e] = s[e] * a.scale + adder[k0 + kt + acc_row(e, half)];
+        mt = fmaxf(mt, p[e]);
+      }
+      mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+      const float mn = fmaxf(m, mt);
+      const float alpha = __expf(m - mn);
+      m = mn;
+      float rs = 0.f;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) { p[e] = __expf(p[e] - mn); rs += p[e]; }
+      l = l * alpha + rs;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) { o[0][e] *= alpha; o[1][e] *= alpha; }
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        const bf16x8 pf = pack8(p + 8 * s2);
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt) o[dt] = mfma(frag_cols(sv, kt + 16 * s2, dt * 32, lane), pf, o[dt]);
+      }
+    }
+  }
+  l += __shfl_xor(l, 32, 64);
+  store_t(a.ctx + ((int64_t)b * a.S + q) * a.H + hd * HD, o, 1.0f / l, half);
+  if (half == 0) a.lse[((int64_t)b * a.N + hd) * a.S + q] = m + __logf(l);
+}
+
+// ----------------------------------------------------------------------------------- backward: dQ
+// grid (S/64, B*N), 128 threads: each wave owns 32 queries.  Also writes delta[q] = sum_d dO[q,d] O[q,d].
+__global__ __launch_bounds__(128) void attn_bwd_dq_kernel(AttnArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5;
+  const int b = blockIdx.y / a.N, hd = blockIdx.y % a.N;
+  const int q = blockIdx.x * 64 + wave * 32 + (lane & 31);
+  const bf16* base = a.qkv + (int64_t)b * a.S * a.ld + hd * HD;
+  char* sk = lds;
+  char* sv = lds + CHUNK * ROWB;
+  float* adder = reinterpret_cast<float*>(lds + 2 * CHUNK * ROWB);
+  for (int j = threadIdx.x; j < a.S; j += 128)
+    adder[j] = a.key_mask ? (1.0f - a.key_mask[(int64_t)b * a.S + j]) * a.mask_value : 0.f;
+  bf16x8 qf[4], dof[4];
+  float delta = 0.f;
+  const int64_t orow = ((int64_t)b * a.S + q) * a.H + hd * HD;
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) {
+    qf[ks] = *reinterpret_cast<const bf16x8*>(base + (int64_t)q * a.ld + 16 * ks + 8 * half);
+    dof[ks] = *reinterpret_cast<const bf16x8*>(a.dctx + orow + 16 * ks + 8 * half);
+    const bf16x8 of = *reinterpret_cast<const bf16x8*>(a.ctx + orow + 16 * ks + 8 * half);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) delta += (float)dof[ks][j] * (float)of[j];
+  }
+  delta += __shfl_xor(delta, 32, 64);
+  const float lse = a.lse[((int64_t)b * a.N + hd) * a.S + q];
+  if (half == 0) a.delta[((int64_t)b * a.N + hd) * a.S + q] = delta;
+  f32x16 dq[2];
+#pragma unroll
+  for (int e = 0; e < 16; ++e) { dq[0][e] = 0.f; dq[1][e] = 0.f; }
+  for (int k0 = 0; k0 < a.S; k0 += CHUNK) {
+    const int rows = a.S - k0 < CHUNK ? a.S - k0 : CHUNK;
+    __syncthreads();
+    tile_fill(sk, base + a.H + (int64_t)k0 * a.ld, a.ld, rows, wave, lane);
+    tile_fill(sv, base + 2 * a.H + (int64_t)k0 * a.ld, a.ld, rows, wave, lane);
+    __builtin_amdgcn_s_waitcnt(VMCNT0);
+    __syncthreads();
+    for (int kt = 0; kt < rows; kt += 32) {
+      f32x16 s, dp;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) { s[e] = 0.f; dp[e] = 0.f; }
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        s = mfma(frag_rows(sk, kt, ks, lane), qf[ks], s);     // S^T[key][q]
+        dp = mfma(frag_rows(sv, kt, ks, lane), dof[ks], dp);  // dP^T[key][q] = V dO^T
+      }
+      float ds[16];
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const float p = __expf(s[e] * a.scale + adder[k0 + kt + acc_row(e, half)] - lse);
+        ds[e] = p * (dp[e] - delta) * a.scale;
+      }
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        const bf16x8 df = pack8(ds + 8 * s2);
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt) dq[dt] = mfma(frag_cols(sk, kt + 16 * s2, dt * 32, lane), df, dq[dt]);  // dQ^T += K^T dS^T
+      }
+    }
+  }
+  store_t(a.dqkv + ((int64_t)b * a.S + q) * a.ld + hd * HD, dq, 1.0f, half);
+}
+
+// ----------------------------------------------------------------------------------- backward: dK, dV
+// grid (S/64, B*N), 128 threads: each wave owns 32 keys, walks all queries (Q and dO tiles in LDS).
+__global__ __launch_bounds__(128) void attn_bwd_dkv_kernel(AttnArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5;
+  const int b = blockIdx.y / a.N, hd = blockIdx.y % a.N;
+  const int key = blockIdx.x * 64 + wave * 32 + (lane & 31);
+  const bf16* base = a.qkv + (int64_t)b * a.S * a.ld + hd * HD;
+  const bf16* dobase = a.dctx + (int64_t)b * a.S * a.H + hd * HD;
+  char* sq = lds;
+  char* sdo = lds + CHUNK * ROWB;
+  float* slse = reinterpret_cast<float*>(lds + 2 * CHUNK * ROWB);
+  float* sdelta = slse + a.S;
+  for (int j = threadIdx.x; j < a.S; j += 128) {
+    slse[j] = a.lse[((int64_t)b * a.N + hd) * a.S + j];
+    sdelta[j] = a.delta[((int64_t)b * a.N + hd) * a.S + j];
+  }
+  const float adder = a.key_mask ? (1.0f - a.key_mask[(int64_t)b * a.S + key]) * a.mask_value : 0.f;
+  bf16x8 kf[4], vf[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) {
+    kf[ks] = *reinterpret_cast<const bf16x8*>(base + a.H + (int64_t)key * a.ld + 16 * ks + 8 * half);
+    vf[ks] = *reinterpret_cast<const bf16x8*>(base + 2 * a.H + (int64_t)key * a.ld + 16 * ks + 8 * half);
+  }
+  f32x16 dk[2], dv[2];
+#pragma unroll
+  for (int e = 0; e < 16; ++e) { dk[0][e] = 0.f; dk[1][e] = 0.f; dv[0][e] = 0.f; dv[1][e] = 0.f; }
+  for (int q0 = 0; q0 < a.S; q0 += CHUNK) {
+    const int rows = a.S - q0 < CHUNK ? a.S - q0 : CHUNK;
+    __syncthreads();
+    tile_fill(sq, base + (int64_t)q0 * a.ld, a.ld, rows, wave, lane);
+    tile_fill(sdo, dobase + (int64_t)q0 * a.H, a.H, rows, wave, lane);
+    __builtin_amdgcn_s_waitcnt(VMCNT0);
+    __syncthreads();
+    for (int qt = 0; qt < rows; qt += 32) {
+      f32x16 s, dp;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) { s[e] = 0.f; dp[e] = 0.f; }
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        s = mfma(frag_rows(sq, qt, ks, lane), kf[ks], s);      // S[q][key]
+        dp = mfma(frag_rows(sdo, qt, ks, lane), vf[ks], dp);   // dP[q][key] = dO V^T
+      }
+      float p[16], ds[16];
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int qq = q0 + qt + acc_row(e, half);
+        p[e] = __expf(s[e] * a.scale + adder - slse[qq]);
+        ds[e] = p[e] * (dp[e] - sdelta[qq]) * a.scale;
+      }
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        const bf16x8 pf = pack8(p + 8 * s2), df = pack8(ds + 8 * s2);
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt) {
+          dv[dt] = mfma(frag_cols(sdo, qt + 16 * s2, dt * 32, lane), pf, dv[dt]);  // dV^T += dO^T P
+          dk[dt] = mfma(frag_cols(sq, qt + 16 * s2, dt * 32, lane), df, dk[dt]);   // dK^T += Q^T dS
+        }
+      }
+    }
+  }
+  bf16* orow = a.dqkv + ((int64_t)b * a.S + key) * a.ld + hd * HD;
+  store_t(orow + a.H, dk, 1.0f, half);
+  store_t(orow + 2 * a.H, dv, 1.0f, half);
+}
+
+int check(const char* who, int dtype, int B, int N, int S, int D) {
+  DS_CHECK_ARG(dtype == DS_BF16, "%s: the fused kernels are bf16 only (dtype %d)", who, dtype);
+  DS_CHECK_ARG(D == HD, "%s: head size must be %d (got %d)", who, HD, D);
+  DS_CHECK_ARG(B > 0 && N > 0 && S > 0 && S % 64 == 0, "%s: seq (%d) must be a positive multiple of 64", who, S);
+  DS_CHECK_ARG(S <= 2048, "%s: seq %d exceeds 2048", who, S);
+  return DS_OK;
+}
+size_t lds_bytes(int S) { return (size_t)2 * CHUNK * ROWB + (size_t)2 * S * sizeof(float); }
+
+}  // namespace
+
+extern "C" int ds_attention_fwd(int dtype, int batch, int heads, int seq, int head_dim, const void* qkv, int64_t ld,
+                                const float* key_mask, float scale, float mask_value, void* ctx, float* lse, void* stream) {
+  DS_PROPAGATE(check("ds_attention_fwd", dtype, batch, heads, seq, head_dim));
+  DS_CHECK_ARG(qkv && ctx && lse, "ds_attention_fwd: null pointer");
+  DS_CHECK_ARG(ld >= 3 * heads * head_dim && ld % 8 == 0 && ds_aligned16(qkv) && ds_aligned16(ctx), "ds_attention_fwd: bad ld or alignment");
+  AttnArgs a;
+  a.qkv = (const bf16*)qkv; a.ld = ld; a.key_mask = key_mask; a.ctx = (bf16*)ctx; a.lse = lse; a.dctx = nullptr; a.dqkv = nullptr;
+  a.delta = nullptr; a.B = batch; a.N = heads; a.S = seq; a.H = heads * head_dim; a.scale = scale; a.mask_value = mask_value;
+  static bool attr = false;
+  if (!attr) {
+    DS_CHECK_HIP(hipFuncSetAttribute((const void*)attn_fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(2048)));
+    attr = true;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  ds_prof_scope prof(s, "attn_fwd_kernel", 4.0 * batch * heads * (double)seq * seq * head_dim, "FLOP");
+  hipLaunchKernelGGL(attn_fwd_kernel, dim3(seq / 64, batch * heads), dim3(128), lds_bytes(seq), s, a);
+  DS_CHECK_LAUNCH();
+  return DS_OK;
+}
+
+extern "C" int ds_attention_bwd(int dtype, int batch, int heads, int seq, int head_dim, const void* qkv, int64_t ld,
+                                const float* key_mask, float scale, float mask_value, const void* ctx, const float* lse,
+                                const void* dctx, void* dqkv, float* delta, void* stream) {
+  DS_PROPAGATE(check("ds_attention_bwd", dtype, batch, heads, seq, head_dim));
+  DS_CHECK_ARG(qkv && ctx && lse && dctx && dqkv && delta, "ds_attention_bwd: null pointer");
+  DS_CHECK_ARG(ld >= 3 * heads * head_dim && ld % 8 == 0 && ds_aligned16(qkv) && ds_aligned16(ctx) && ds_aligned16(dctx) &&
+               ds_aligned16(dqkv), "ds_attention_bwd: bad ld or alignment");
+  AttnArgs a;
+  a.qkv = (const bf16*)qkv; a.ld = ld; a.key_mask = key_mask; a.ctx = (bf16*)ctx; a.lse = (float*)lse; a.dctx = (const bf16*)dctx;
+  a.dqkv = (bf16*)dqkv; a.delta = delta; a.B = batch; a.N = heads; a.S = seq; a.H = heads * head_dim; a.scale = scale;
+  a.mask_value = mask_value;
+  static bool attr = false;
+  if (!attr) {
+    DS_CHECK_HIP(hipFuncSetAttribute((const void*)attn_bwd_dq_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(2048)));
+    DS_CHECK_HIP(hipFuncSetAttribute((const void*)attn_bwd_dkv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(2048)));
+    attr = true;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  {
+    ds_prof_scope prof(s, "attn_bwd_dq_kernel", 6.0 * batch * heads * (double)seq * seq * head_dim, "FLOP");
+    hipLaunchKernelGGL(attn_bwd_dq_kernel, dim3(seq / 64, batch * heads), dim3(128), lds_bytes(seq), s, a);
+    DS_CHECK_LAUNCH();
+  }
+  {
+    ds_prof_scope prof(s, "attn_bwd_dkv_kernel", 8.0 * batch * heads * (double)seq * seq * head_dim, "FLOP");
+    hipLaunchKernelGGL(attn_bwd_dkv_kernel, dim3(seq / 64, batch * heads), dim3(128), lds_bytes(seq), s, a);
+    DS_CHECK_LAUNCH();
+  }
+  return DS_OK;
+}

@@ -1,5 +1,7 @@
 // HBM-bound kernels: gradient accumulation, casts, LayerNorm, softmax, column sums.
 // All move data as 16-byte vectors per lane with grid-stride or one-wave-per-row mappings.
+#include <stdlib.h>
+
 #include "common.h"
 
 namespace {
@@ -111,14 +113,11 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(int rows, int cols, 
                                                            const float* __restrict__ stats,
                                                            const T* __restrict__ dx_add, T* __restrict__ dx,
                                                            float* __restrict__ d_gamma, float* __restrict__ d_beta,
-                                                           float* __restrict__ d_colsum) {
+                                                           float* __restrict__ d_colsum, int dbg) {
   constexpr int VEC = Vec16<T>::N;
   typedef typename Vec16<T>::type V;
-  extern __shared__ float red[];  // [3][cols]
+  extern __shared__ __attribute__((aligned(16))) float red[];  // [3][cols]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int c = threadIdx.x; c < 3 * cols; c += 256) red[c] = 0.f;
-  __syncthreads();
-
   float g[NV][VEC], pg[NV][VEC], pb[NV][VEC], ps[NV][VEC];
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
@@ -179,19 +178,32 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(int rows, int cols, 
       }
     }
   }
+  if (dbg & 1) return;
+  // combine the 4 waves' column partials in LDS, one wave at a time (plain vector stores / read-modify-writes:
+  // LDS float atomics on 32-byte-strided addresses serialise 16 ways)
+  for (int wv = 0; wv < 4; ++wv) {
+    if (wave == wv) {
 #pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    const int c = (lane + i * 64) * VEC;
-    if (c < cols) {
+      for (int i = 0; i < NV; ++i) {
+        const int c = (lane + i * 64) * VEC;
+        if (c < cols) {
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        atomicAdd(&red[c + e], pg[i][e]);
-        atomicAdd(&red[cols + c + e], pb[i][e]);
-        atomicAdd(&red[2 * cols + c + e], ps[i][e]);
+          for (int e = 0; e < VEC; e += 4) {
+            f32x4* r0 = reinterpret_cast<f32x4*>(&red[c + e]);
+            f32x4* r1 = reinterpret_cast<f32x4*>(&red[cols + c + e]);
+            f32x4* r2 = reinterpret_cast<f32x4*>(&red[2 * cols + c + e]);
+            f32x4 a0 = {pg[i][e], pg[i][e + 1], pg[i][e + 2], pg[i][e + 3]};
+            f32x4 a1 = {pb[i][e], pb[i][e + 1], pb[i][e + 2], pb[i][e + 3]};
+            f32x4 a2 = {ps[i][e], ps[i][e + 1], ps[i][e + 2], ps[i][e + 3]};
+            if (wv > 0) { a0 += *r0; a1 += *r1; a2 += *r2; }
+            *r0 = a0; *r1 = a1; *r2 = a2;
+          }
+        }
       }
     }
+    __syncthreads();
   }
-  __syncthreads();
+  if (dbg & 2) return;
   for (int c = threadIdx.x; c < cols; c += 256) {
     atomicAdd(d_gamma + c, red[c]);
     atomicAdd(d_beta + c, red[cols + c]);
@@ -402,15 +414,18 @@ static int layernorm_bwd_t(int rows, int cols, const void* dy, const void* x, co
   const int vec = Vec16<T>::N;
   const int need = (cols / vec + 63) / 64;
   // aim for ~64 blocks of 4 waves (the column atomics at the end cost more than the row work)
-  int rpw = rows / (64 * 4);
+  int rpw = rows / (128 * 4);
   if (rpw < 1) rpw = 1;
   if (rpw > 16) rpw = 16;
   dim3 grid((rows + 4 * rpw - 1) / (4 * rpw));
   const size_t lds = 3 * (size_t)cols * sizeof(float);
+  static const char* env = getenv("DS_LN_DEBUG");
+  const int dbg = env ? atoi(env) : 0;
+  if (env && getenv("DS_LN_RPW")) { rpw = atoi(getenv("DS_LN_RPW")); grid = dim3((rows + 4 * rpw - 1) / (4 * rpw)); }
   ds_prof_scope prof(s, sizeof(T) == 2 ? "layernorm_bwd_kernel<bf16>" : "layernorm_bwd_kernel<float>",
                      (double)rows * cols * sizeof(T) * (dx_add ? 4 : 3), "B");
   DISPATCH_NV(T, need, hipLaunchKernelGGL((layernorm_bwd_kernel<T, NV>), grid, dim3(256), lds, s, rows, cols, rpw,
-                                          (const T*)dy, (const T*)x, gamma, stats, (const T*)dx_add, (T*)dx, dg, db, dcs));
+                                          (const T*)dy, (const T*)x, gamma, stats, (const T*)dx_add, (T*)dx, dg, db, dcs, dbg));
   DS_CHECK_LAUNCH();
   return DS_OK;
 }

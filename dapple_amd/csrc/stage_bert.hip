@@ -68,7 +68,7 @@ __global__ __launch_bounds__(256) void embed_bwd_kernel(int rows, int H, int seq
 }
 
 struct LayerStash {  // byte offsets into a slot
-  size_t x, qkv, p, ctx, z1, a, u, h, z2, st1, st2;
+  size_t x, qkv, p, ctx, z1, a, u, h, z2, st1, st2, lse;
 };
 
 struct BertStage : ds_stage {
@@ -76,6 +76,7 @@ struct BertStage : ds_stage {
   int dtype;
   size_t esz;
   bool emb;
+  bool fused_attn;  // bf16, head size 64: fused attention kernels, no [B,N,S,S] tensors at all
   // compute copies
   char* wc_base = nullptr;
   std::vector<char*> wqkv, wo, w1, w2;  // element type T
@@ -104,6 +105,7 @@ struct BertStage : ds_stage {
     const ds_stage_cfg& c = cfg;
     L = c.num_layers; H = c.hidden; F = c.ffn; NH = c.heads; B = c.batch; S = c.seq;
     D = H / NH; rows = B * S; dtype = c.dtype; esz = dtype == DS_BF16 ? 2 : 4; emb = c.with_embedding != 0;
+    fused_attn = dtype == DS_BF16 && D == 64 && S % 64 == 0 && S <= 2048;
     char name[160];
     if (emb) {
       winfo.push_back({"bert/embeddings/word_embeddings", c.vocab, H});
@@ -171,7 +173,8 @@ struct BertStage : ds_stage {
       LayerStash& t = ls[l];
       t.x = next_x;
       t.qkv = sa.reserve(3 * act);
-      t.p = sa.reserve(probs);
+      t.p = fused_attn ? 0 : sa.reserve(probs);
+      t.lse = fused_attn ? sa.reserve((size_t)B * NH * S * 4) : 0;
       t.ctx = sa.reserve(act);
       t.z1 = sa.reserve(act);
       t.a = sa.reserve(act);
@@ -190,8 +193,8 @@ struct BertStage : ds_stage {
     slot_has_tt.assign(K, 0);
     // ---- workspace
     Arena w;
-    ws_scores = w.reserve((size_t)B * NH * S * S * 4);
-    ws_ds = w.reserve(probs);
+    ws_scores = w.reserve(fused_attn ? (size_t)B * NH * S * 4 : (size_t)B * NH * S * S * 4);  // fused: delta
+    ws_ds = fused_attn ? 0 : w.reserve(probs);
     ws_dz2 = w.reserve(act);
     ws_du = w.reserve(actF);
     ws_da = w.reserve(act);
@@ -308,6 +311,11 @@ struct BertStage : ds_stage {
       char* y = (l + 1 < L) ? sp + ls[l + 1].x : (char*)out;
       // fused Q|K|V projection (modeling_slice.py:464-485)
       DS_PROPAGATE(gemm_fwd(rows, 3 * H, H, x, wqkv[l], sp + t.qkv, DS_EPI_BIAS, bqkv[l], nullptr, nullptr));
+      if (fused_attn) {
+        // scores, scale, mask adder, softmax and context in one kernel (:499-533)
+        DS_PROPAGATE(ds_attention_fwd(dtype, B, NH, S, D, sp + t.qkv, 3 * H, mask, scale, -10000.0f, sp + t.ctx,
+                                      (float*)(sp + t.lse), stream));
+      } else {
       // scores = Q K^T (:499), fp32
       DS_PROPAGATE(gemm_heads(DS_K_MAJOR, DS_K_MAJOR, S, S, D, sp + t.qkv, 3 * H, (int64_t)S * 3 * H, D,
                               sp + t.qkv + (size_t)H * esz, 3 * H, (int64_t)S * 3 * H, D, ws_base + ws_scores, S,
@@ -319,6 +327,7 @@ struct BertStage : ds_stage {
       DS_PROPAGATE(gemm_heads(DS_K_MAJOR, DS_MN_MAJOR, S, D, S, sp + t.p, S, (int64_t)NH * S * S, (int64_t)S * S,
                               sp + t.qkv + (size_t)2 * H * esz, 3 * H, (int64_t)S * 3 * H, D, sp + t.ctx, H,
                               (int64_t)S * H, D, 0));
+      }
       // attention output dense + residual (:974-978), then layer_norm (:979)
       DS_PROPAGATE(gemm_fwd(rows, H, H, sp + t.ctx, weight_T(l, W_AO), sp + t.z1, DS_EPI_BIAS | DS_EPI_RESIDUAL,
                             w[b + B_AO], x, nullptr));
@@ -371,6 +380,11 @@ struct BertStage : ds_stage {
       const char* k = q + (size_t)H * esz;
       const char* v = q + (size_t)2 * H * esz;
       const int64_t so3 = (int64_t)S * 3 * H, soH = (int64_t)S * H, soP = (int64_t)NH * S * S, siP = (int64_t)S * S;
+      if (fused_attn) {
+        const float* mask = slot_has_mask[slot] ? (const float*)(sp + mask_off) : nullptr;
+        DS_PROPAGATE(ds_attention_bwd(dtype, B, NH, S, D, q, 3 * H, mask, scale, -10000.0f, sp + t.ctx, (const float*)(sp + t.lse),
+                                      dctx, dqkv, dp, stream));
+      } else {
       // dP = dctx V^T (fp32)
       DS_PROPAGATE(gemm_heads(DS_K_MAJOR, DS_K_MAJOR, S, S, D, dctx, H, soH, D, v, 3 * H, so3, D, dp, S, soP, siP,
                               DS_EPI_OUT_F32));
@@ -383,6 +397,7 @@ struct BertStage : ds_stage {
       DS_PROPAGATE(gemm_heads(DS_K_MAJOR, DS_MN_MAJOR, S, D, S, dsm, S, soP, siP, k, 3 * H, so3, D, dqkv, 3 * H, so3, D, 0));
       DS_PROPAGATE(gemm_heads(DS_MN_MAJOR, DS_MN_MAJOR, S, D, S, dsm, S, soP, siP, q, 3 * H, so3, D,
                               dqkv + (size_t)H * esz, 3 * H, so3, D, 0));
+      }
       // projection gradients: three [H,H] kernels and three biases fed by the columns of dqkv
       const bool adjacent = g[b + B_K] == g[b + B_Q] + H && g[b + B_V] == g[b + B_Q] + 2 * H &&
                             g[b + W_K] == g[b + W_Q] + (size_t)H * H && g[b + W_V] == g[b + W_Q] + (size_t)2 * H * H;

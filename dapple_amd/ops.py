@@ -185,3 +185,25 @@ def maxpool2x2_bwd(x, dy, relu_mask=False):
     check(_lib.load().ds_maxpool2x2_bwd(n, h, w, c, ptr(x), ptr(dy), ptr(dx), 1 if relu_mask else 0, _lib.current_stream()),
           "ds_maxpool2x2_bwd")
     return dx
+
+
+def attention_fwd(qkv, batch, heads, seq, scale, key_mask=None, mask_value=-10000.0):
+    """Fused bf16 attention on the fused projection qkv [batch*seq, 3*heads*64] -> (ctx, lse)."""
+    _need_cuda(qkv, key_mask)
+    hidden = qkv.shape[1] // 3
+    ctx = torch.empty(batch * seq, hidden, dtype=qkv.dtype, device=qkv.device)
+    lse = torch.empty(batch, heads, seq, dtype=torch.float32, device=qkv.device)
+    check(_lib.load().ds_attention_fwd(dtype_code(qkv), batch, heads, seq, hidden // heads, ptr(qkv), qkv.shape[1], ptr(key_mask),
+                                       scale, mask_value, ptr(ctx), ptr(lse), _lib.current_stream()), "ds_attention_fwd")
+    return ctx, lse
+
+
+def attention_bwd(qkv, ctx, lse, dctx, batch, heads, seq, scale, key_mask=None, mask_value=-10000.0):
+    _need_cuda(qkv, ctx, lse, dctx, key_mask)
+    hidden = qkv.shape[1] // 3
+    dqkv = torch.empty_like(qkv)
+    delta = torch.empty_like(lse)
+    check(_lib.load().ds_attention_bwd(dtype_code(qkv), batch, heads, seq, hidden // heads, ptr(qkv), qkv.shape[1], ptr(key_mask),
+                                       scale, mask_value, ptr(ctx), ptr(lse), ptr(dctx), ptr(dqkv), ptr(delta),
+                                       _lib.current_stream()), "ds_attention_bwd")
+    return dqkv

@@ -121,6 +121,19 @@ int ds_softmax_fwd(int dtype, int batch, int heads, int q, int k, const float* s
 int ds_softmax_bwd(int dtype, int64_t rows, int k, const void* p, const float* dp, float scale,
                    void* ds, void* stream);
 
+/* Fused attention for bf16 and head size 64: ctx = softmax(q k^T * scale + (1 - key_mask) * mask_value) v
+ * per (batch, head), without materialising the probabilities (modeling_slice.py:499-533 in one kernel).
+ * qkv is the fused projection [batch*seq, ld]: q in columns [0,H), k in [H,2H), v in [2H,3H), H = heads*64;
+ * head h owns columns h*64..h*64+63 of each.  lse [batch, heads, seq] receives the row logsumexp for the
+ * backward pass; ds_attention_bwd writes dq|dk|dv into dqkv (same layout as qkv) and uses delta
+ * [batch, heads, seq] as scratch.  seq must be a multiple of 64, at most 2048. */
+int ds_attention_fwd(int dtype, int batch, int heads, int seq, int head_dim, const void* qkv, int64_t ld,
+                     const float* key_mask, float scale, float mask_value, void* ctx, float* lse,
+                     void* stream);
+int ds_attention_bwd(int dtype, int batch, int heads, int seq, int head_dim, const void* qkv, int64_t ld,
+                     const float* key_mask, float scale, float mask_value, const void* ctx,
+                     const float* lse, const void* dctx, void* dqkv, float* delta, void* stream);
+
 /* Column sums: out[n] (fp32) += sum_m x[m][n]; the bias gradient of tf.layers.dense. */
 int ds_colsum_accum(int dtype, int rows, int cols, const void* x, int64_t ldx, float* out,
                     void* stream);

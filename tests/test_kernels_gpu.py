@@ -180,3 +180,38 @@ def test_colsum(dt):
     out = torch.ones(200, device="cuda")
     ops.colsum_accum(x, out)
     assert_close(out, x.cpu().double().sum(0) + 1, 1e-5, "colsum")
+
+
+@pytest.mark.parametrize("B,N,S,use_mask", [(1, 1, 64, False), (2, 3, 128, True), (2, 16, 512, True), (1, 2, 1024, False)])
+def test_fused_attention_fwd_bwd(B, N, S, use_mask):
+    D, H = 64, N * 64
+    r = rng(S + N)
+    qkv = dev(r.standard_normal((B * S, 3 * H)) * 0.7, torch.bfloat16)
+    dctx = dev(r.standard_normal((B * S, H)), torch.bfloat16)
+    mask = None
+    if use_mask:
+        m = (r.random((B, S)) > 0.2).astype(np.float32)
+        m[:, 0] = 1
+        mask = dev(m)
+    scale = 1.0 / math.sqrt(D)
+    ctx, lse = ops.attention_fwd(qkv, B, N, S, scale, mask)
+    x = qkv.cpu().double().requires_grad_(True)
+    q, k, v = (x[:, i * H:(i + 1) * H].reshape(B, S, N, D).permute(0, 2, 1, 3) for i in range(3))
+    sc = q @ k.transpose(-1, -2) * scale
+    if use_mask:
+        sc = sc + (1.0 - mask.cpu().double())[:, None, None, :] * -10000.0
+    ref = (torch.softmax(sc, -1) @ v).permute(0, 2, 1, 3).reshape(B * S, H)
+    assert_close(ctx, ref, 1e-2, "fused attention fwd")
+    assert_close(lse, torch.logsumexp(sc, -1), 1e-3, "logsumexp")
+    (dx,) = torch.autograd.grad(ref, x, dctx.cpu().double())
+    dqkv = ops.attention_bwd(qkv, ctx, lse, dctx, B, N, S, scale, mask)
+    for i, name in enumerate(("dq", "dk", "dv")):
+        assert_close(dqkv[:, i * H:(i + 1) * H], dx[:, i * H:(i + 1) * H], 2e-2, "fused attention " + name)
+
+
+def test_fused_attention_rejects_other_shapes():
+    qkv = torch.zeros(64, 3 * 32, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ValueError, match="head size"):
+        ops.attention_fwd(qkv, 1, 1, 64, 1.0)
+    with pytest.raises(ValueError, match="multiple of 64"):
+        ops.attention_fwd(torch.zeros(48, 192, dtype=torch.bfloat16, device="cuda"), 1, 1, 48, 1.0)
