@@ -1,0 +1,364 @@
+"""Host-side mirror of the reference's stage-slice interfaces, on top of the HIP stage runtime.
+
+Same class / function names, argument names and error behaviour as the reference's slice files, so
+a driver written against them finds what it expects; what they return are GPU tensors computed
+eagerly through ``libdapple_hip.so`` instead of TF graph symbols.
+
+    BertConfig, BertModelSlice          bert/models/bert/modeling_slice.py:646-717, 722-1009
+    BertFinetuneSlice                   bert/models/bert/bert.py:385-479 (calc_device :419-430)
+    SliceVGG19                          vgg19/applications/vgg19_slice_model.py:38-357
+    XlnetSlice                          xlnet/models/slice_xlnet.py:22-246 (calc_device :106-121)
+    _single_cell_dapple, GNMTEncoderSlice   gnmt/nmt/model_helper.py:399-456, gnmt_model.py:61-221
+    calc_reduction_layers, BaseCell, build_network   amoeba_net/network_utils_slice.py:83-90, 294-313,
+                                        model_builder_slice.py:292-345 (API shell: no config runs it)
+
+``dep_outputs`` arguments are accepted and ignored on purpose: in the reference they only add TF
+control dependencies (values unused, bert.py:439-449); here ordering is the launch order that
+``dapple_amd.runtime.StageRuntime`` issues.
+"""
+import copy
+import json
+import sys
+
+import torch
+
+from . import runtime, synthetic
+
+
+# =========================================================================== BERT
+class BertConfig(object):
+    """Configuration for `BertModel` (modeling_slice.py:646-717)."""
+
+    def __init__(self, vocab_size, hidden_size=768, num_hidden_layers=12, num_attention_heads=12,
+                 intermediate_size=3072, hidden_act="gelu", hidden_dropout_prob=0.1,
+                 attention_probs_dropout_prob=0.1, max_position_embeddings=512, type_vocab_size=16,
+                 initializer_range=0.02):
+        self.vocab_size = vocab_size
+        self.hidden_size = hidden_size
+        self.num_hidden_layers = num_hidden_layers
+        self.num_attention_heads = num_attention_heads
+        self.hidden_act = hidden_act
+        self.intermediate_size = intermediate_size
+        self.hidden_dropout_prob = hidden_dropout_prob
+        self.attention_probs_dropout_prob = attention_probs_dropout_prob
+        self.max_position_embeddings = max_position_embeddings
+        self.type_vocab_size = type_vocab_size
+        self.initializer_range = initializer_range
+
+    @classmethod
+    def from_dict(cls, json_object):
+        config = BertConfig(vocab_size=None)
+        for (key, value) in json_object.items():
+            config.__dict__[key] = value
+        return config
+
+    @classmethod
+    def from_json_file(cls, json_file):
+        with open(json_file, "r") as reader:
+            text = reader.read()
+        return cls.from_dict(json.loads(text))
+
+    def to_dict(self):
+        return copy.deepcopy(self.__dict__)
+
+    def to_json_string(self):
+        return json.dumps(self.to_dict(), indent=2, sort_keys=True) + "\n"
+
+
+class BertModelSlice(object):
+    """``stages`` = [embedding_stage, reshape_input, layer_0 .. layer_{L-1}, pooler_stage]
+    (modeling_slice.py:792, 823, 837, 870), each ``f(prev_output, *args) -> tensor``.
+
+    ``weights`` maps the reference's variable names to arrays; absent, N(0, initializer_range) /
+    zeros / ones are drawn from ``seed``.  ``dtype`` is the compute type ("fp32" or "bf16")."""
+
+    def __init__(self, config, is_training, input_ids, input_mask=None, token_type_ids=None,
+                 use_one_hot_embeddings=True, scope=None, weights=None, dtype="fp32", seed=0):
+        config = copy.deepcopy(config)
+        if not is_training:
+            config.hidden_dropout_prob = 0.0
+            config.attention_probs_dropout_prob = 0.0
+        if config.hidden_dropout_prob or config.attention_probs_dropout_prob:
+            raise ValueError("dropout is not part of this runtime: build the model with is_training=False "
+                             "or zero dropout probabilities")
+        if config.hidden_act != "gelu":
+            raise ValueError("Unsupported activation: %s" % config.hidden_act)
+        if input_ids.dim() != 2:
+            raise ValueError("For the tensor `input_ids`, the actual rank `%d` (shape = %s) is not equal to the "
+                             "expected rank `2`" % (input_ids.dim(), tuple(input_ids.shape)))
+        if config.hidden_size % config.num_attention_heads != 0:
+            raise ValueError("The hidden size (%d) is not a multiple of the number of attention heads (%d)"
+                             % (config.hidden_size, config.num_attention_heads))
+        self.config, self.dtype = config, dtype
+        self.batch_size, self.seq_length = input_ids.shape
+        if self.seq_length > config.max_position_embeddings:
+            raise ValueError("The seq length (%d) cannot be greater than `max_position_embeddings` (%d)"
+                             % (self.seq_length, config.max_position_embeddings))
+        self.input_ids = input_ids.to(torch.int32).contiguous()
+        if input_mask is None:
+            input_mask = torch.ones_like(self.input_ids)
+        if token_type_ids is None:
+            token_type_ids = torch.zeros_like(self.input_ids)
+        self.input_mask = input_mask
+        self.token_type_ids = token_type_ids.to(torch.int32).contiguous()
+        # [B, F, T] float mask of modeling_slice.py:323-354; the kernels take its [B, T] key form
+        self.attention_mask = torch.ones(self.batch_size, self.seq_length, 1, device=input_ids.device) * \
+            input_mask.reshape(self.batch_size, 1, self.seq_length).float()
+        self._key_mask = None if bool((input_mask != 0).all()) else input_mask.float().contiguous()
+        emb = (config.vocab_size, config.type_vocab_size, config.max_position_embeddings)
+        self.weights = weights if weights is not None else synthetic.bert_weights(
+            seed, config.num_hidden_layers, config.hidden_size, config.intermediate_size, embeddings=emb,
+            stddev=config.initializer_range)
+        self.all_encoder_layers = []
+        self.sequence_output = self.embedding_output = self.pooled_output = None
+        self._handles = {}
+
+        def embedding_stage(*args):
+            st = self._op_stage("emb")
+            out = torch.empty(self.batch_size * self.seq_length, config.hidden_size, dtype=st.act_dtype, device=input_ids.device)
+            st.forward(0, self.input_ids, out, token_type_ids=self.token_type_ids)
+            st.backward(0, torch.zeros_like(out))         # frees the slot; gradients of a zero upstream are zero
+            self.embedding_output = out.reshape(self.batch_size, self.seq_length, config.hidden_size)
+            return self.embedding_output
+
+        def reshape_input(input_tensor, *args):
+            if input_tensor.dim() != 3:
+                raise ValueError("For the tensor `input_tensor`, the actual rank `%d` is not equal to the expected rank `3`"
+                                 % input_tensor.dim())
+            self.input_shape = list(input_tensor.shape)
+            if self.input_shape[2] != config.hidden_size:
+                raise ValueError("The width of the input tensor (%d) != hidden size (%d)" % (self.input_shape[2], config.hidden_size))
+            return input_tensor.reshape(-1, config.hidden_size)
+
+        def create_layer(idx):
+            def encoder_layer(layer_input, *args):
+                st = self._op_stage(idx)
+                out = torch.empty_like(layer_input)
+                st.forward(0, layer_input.contiguous(), out, key_mask=self._key_mask)
+                st.backward(0, torch.zeros_like(out), None)
+                final = out.reshape(self.batch_size, self.seq_length, config.hidden_size)
+                self.all_encoder_layers.append(final)
+                self.sequence_output = final
+                return out
+            return encoder_layer
+
+        def pooler_stage(sequence_output, *args):
+            raise NotImplementedError("the pooler belongs to the last pipeline stage (bert.py:669-718), which this "
+                                      "runtime does not build")
+
+        self.stages = [embedding_stage, reshape_input]
+        self.stages += [create_layer(i) for i in range(config.num_hidden_layers)]
+        self.stages.append(pooler_stage)
+
+    def _op_stage(self, which):
+        """A one-op stage handle (the embedding, or encoder layer ``which``), created on first use."""
+        if which not in self._handles:
+            c = self.config
+            if which == "emb":
+                st = runtime.bert_stage(0, c.hidden_size, c.num_attention_heads, c.intermediate_size, self.batch_size,
+                                        self.seq_length, self.dtype, 1,
+                                        embeddings=(c.vocab_size, c.type_vocab_size, c.max_position_embeddings))
+            else:
+                st = runtime.bert_stage(1, c.hidden_size, c.num_attention_heads, c.intermediate_size, self.batch_size,
+                                        self.seq_length, self.dtype, 1, first_layer=which)
+            st.bind(self.weights)
+            self._handles[which] = st
+        return self._handles[which]
+
+    def get_pooled_output(self):
+        return self.pooled_output
+
+    def get_sequence_output(self):
+        return self.sequence_output
+
+    def get_all_encoder_layers(self):
+        return self.all_encoder_layers
+
+    def get_embedding_output(self):
+        return self.embedding_output
+
+    def get_embedding_table(self):
+        return self.weights["bert/embeddings/word_embeddings"]
+
+
+def bert_calc_device(i, nstage):
+    """Stage -> device map of bert.py:419-430: BERT-24 (27 stages) splits 11:13 encoder layers, BERT-48 (51
+    stages) 23:25; anything else ends the process like the reference (sys.exit(0))."""
+    if nstage == 27:
+        return 0 if i < 13 else 1
+    elif nstage == 51:
+        return 0 if i < 25 else 1
+    print("Unrecognized nstage, only bert-24 and bert-48 are supported.")
+    sys.exit(0)
+
+
+class BertFinetuneSlice(object):
+    """Places ``model.stages`` on the pipeline devices and builds the HIP stage of ``local_device``
+    (bert.py:390-456).  ``stage`` is a ``runtime.Stage`` holding every op the planner put on that device."""
+
+    def __init__(self, bert_config_file, max_seq_length, is_training, input_ids, input_mask, segment_ids, labels,
+                 use_one_hot_embeddings, model_type='classification', slice_devices="/device:GPU:0",
+                 dep_outputs=None, kwargs=None, local_device=0, dtype="bf16", stash_slots=None, weights=None, seed=0):
+        bert_config = bert_config_file if isinstance(bert_config_file, BertConfig) else BertConfig.from_json_file(bert_config_file)
+        if max_seq_length > bert_config.max_position_embeddings:
+            raise ValueError("Cannot use sequence length %d because the BERT model was only trained up to sequence "
+                             "length %d" % (max_seq_length, bert_config.max_position_embeddings))
+        self.devices = slice_devices if isinstance(slice_devices, list) else slice_devices.split(",")
+        self.bert_config, self.kwargs, self.labels, self.input_ids = bert_config, kwargs, labels, input_ids
+        L = bert_config.num_hidden_layers
+        nstage = L + 3
+        self.device_of = [bert_calc_device(i, nstage) for i in range(nstage)]
+        mine = [i for i in range(nstage) if self.device_of[i] == local_device]
+        layers = [i - 2 for i in mine if 2 <= i < 2 + L]
+        with_emb = 0 in mine
+        B, S = input_ids.shape
+        ndev = max(self.device_of) + 1
+        K = stash_slots if stash_slots is not None else runtime.stash_depth(local_device, ndev)
+        emb = (bert_config.vocab_size, bert_config.type_vocab_size, bert_config.max_position_embeddings) if with_emb else None
+        self.stage = runtime.bert_stage(len(layers), bert_config.hidden_size, bert_config.num_attention_heads,
+                                        bert_config.intermediate_size, B, S, dtype, K, embeddings=emb,
+                                        first_layer=layers[0] if layers else 0)
+        if weights is None:
+            weights = synthetic.bert_weights(seed, L, bert_config.hidden_size, bert_config.intermediate_size,
+                                             embeddings=(bert_config.vocab_size, bert_config.type_vocab_size,
+                                                         bert_config.max_position_embeddings),
+                                             stddev=bert_config.initializer_range)
+        self.stage.bind(weights)
+        self.layers, self.local_device, self.model_type = layers, local_device, model_type
+        self.stage_outputs = []
+
+
+# =========================================================================== VGG19
+class SliceVGG19(object):
+    """vgg19_slice_model.py:38-357.  ``build`` runs stage 0 (the replicated conv stack) on one replica's share
+    of the batch and returns ``(None, [stage0_output])`` - the loss is stage 1's."""
+
+    def __init__(self, include_top=True, weights='imagenet', input_tensor=None, input_shape=None, pooling=None,
+                 classes=1000, num_replica=15, batch_size=None, weight_values=None, seed=0, stash_slots=3, **kwargs):
+        if num_replica not in (2, 15):
+            print("For VGG19 only 2:1 and 15:1 pipeline are supported currently!")
+            sys.exit(-1)
+        self.include_top, self.weights, self.pooling, self.classes = include_top, weights, pooling, classes
+        self.num_replica = num_replica
+        # 15:1 keeps conv1_1..conv5_2 on stage 0, 2:1 only blocks 1-3 (:280-302)
+        self.layers = synthetic.VGG19_STAGE0_15_1 if num_replica == 15 else synthetic.VGG19_STAGE0_15_1[:11]
+        self._weight_values, self._seed, self._stash = weight_values, seed, stash_slots
+        self.stage = None
+
+    def build(self, features, label, input_shape=None, dep_outputs=None):
+        n, h, w, c = features.shape
+        if self.stage is None:
+            self.stage = runtime.vgg_stage(self.layers, n, h, w, c, self._stash)
+            self.stage.bind(self._weight_values or synthetic.vgg_weights(self._seed, self.layers, c))
+        out = torch.empty(self.stage.out_shape, device=features.device)
+        self.stage.forward(0, features.contiguous(), out)
+        self.stage.backward(0, torch.zeros_like(out))
+        return None, [out]
+
+
+# =========================================================================== XLNet
+def xlnet_calc_device(i, num_layer):
+    """slice_xlnet.py:106-121: stage-function index i (layer l is i = l + 2) -> device; the split is 13
+    (XLNet-24: 11 + 13 layers) or 19 (XLNet-36: 17 + 19 layers)."""
+    split_layer_id = 13 if num_layer == 24 else 19
+    return 0 if i < split_layer_id else 1
+
+
+class XlnetSlice(object):
+    """slice_xlnet.py:22-246: builds the HIP stage holding this device's layers."""
+
+    def __init__(self, num_token, num_layer, num_head, embedding_dim, attention_head_dim, feed_forward_dim, target_len,
+                 is_training, memory_len=None, dropout=0.0, attention_dropout=0.0, attention_type=None,
+                 shared_biases=True, local_device=0, batch_size=1, dtype="bf16", streams=1, stash_slots=None,
+                 weights=None, seed=0):
+        if dropout or attention_dropout:
+            raise ValueError("dropout is not part of this runtime")
+        if num_head * attention_head_dim != embedding_dim:
+            raise ValueError("embedding_dim (%d) must equal num_head * attention_head_dim (%d)" % (embedding_dim, num_head * attention_head_dim))
+        self.num_layer = num_layer
+        layers = [l for l in range(num_layer) if xlnet_calc_device(l + 2, num_layer) == local_device]
+        K = stash_slots if stash_slots is not None else runtime.stash_depth(local_device, 2)
+        self.layers = layers
+        self.stage = runtime.xlnet_stage(len(layers), embedding_dim, num_head, feed_forward_dim, batch_size, target_len, dtype,
+                                         K, mem_len=memory_len or 0, streams=streams, first_layer=layers[0])
+        w = weights or synthetic.xlnet_weights(seed, len(layers), embedding_dim, num_head, feed_forward_dim, first_layer=layers[0])
+        self.stage.bind(w)
+
+    def build(self, inputs, dep_outputs=None, is_training=True):
+        """inputs: the boundary activation(s) [streams, seq, batch, hidden]; returns (None, [stage_output])."""
+        out = torch.empty(self.stage.out_shape, dtype=self.stage.act_dtype, device=inputs.device)
+        self.stage.forward(0, inputs.contiguous(), out)
+        self.stage.backward(0, torch.zeros_like(out), None)
+        return None, [out]
+
+
+# =========================================================================== GNMT
+class LSTMCellSpec(object):
+    """What ``_single_cell`` describes: BasicLSTMCell(num_units, forget_bias) (+ ResidualWrapper)."""
+
+    def __init__(self, layer_id, num_units, forget_bias, residual_connection, device_str):
+        self.layer_id, self.num_units, self.forget_bias = layer_id, num_units, forget_bias
+        self.residual_connection, self.device_str = residual_connection, device_str
+
+
+def _single_cell_dapple(hparams, mode, layer_id, residual_connection=False, device_str=None, residual_fn=None):
+    """model_helper.py:399-456.  hparams needs unit_type, num_units, forget_bias, dropout."""
+    if hparams.unit_type != "lstm":
+        raise ValueError("Unknown unit type %s!" % hparams.unit_type)
+    if getattr(hparams, "dropout", 0.0) and mode == "train":
+        raise ValueError("dropout is not part of this runtime")
+    if residual_fn is not None:
+        raise ValueError("custom residual_fn is not supported: the wrapper adds inputs and outputs")
+    return LSTMCellSpec(layer_id, hparams.num_units, hparams.forget_bias, residual_connection, device_str)
+
+
+class GNMTEncoderSlice(object):
+    """The encoder stage GNMTModel._build_encoder (gnmt_model.py:61-221) builds under ``dapple_test``:
+    cells 0 (fw/bw, no residual), 1 (no residual), 2.. (residual), from ``_single_cell_dapple`` specs."""
+
+    def __init__(self, hparams, batch_size, src_max_len, stash_slots=2, weights=None, seed=0):
+        n = hparams.num_encoder_layers
+        self.cells = [_single_cell_dapple(hparams, "infer", 0), _single_cell_dapple(hparams, "infer", 0)]
+        self.cells += [_single_cell_dapple(hparams, "infer", l, residual_connection=(l >= 2)) for l in range(1, n)]
+        self.stage = runtime.gnmt_stage(n, hparams.num_units, hparams.src_vocab_size, batch_size, src_max_len, stash_slots,
+                                        forget_bias=hparams.forget_bias)
+        self.stage.bind(weights or synthetic.gnmt_weights(seed, n, hparams.num_units, hparams.src_vocab_size,
+                                                          init_weight=getattr(hparams, "init_weight", 0.1)))
+
+    def build_graph(self, source_ids, scope=None, dep_outputs=None):
+        out = torch.empty(self.stage.out_shape, device=source_ids.device)
+        self.stage.forward(0, source_ids.to(torch.int32).contiguous(), out)
+        self.stage.backward(0, torch.zeros_like(out))
+        return out
+
+
+# =========================================================================== AmoebaNet (API shell)
+def calc_reduction_layers(num_cells, num_reduction_layers):
+    """network_utils_slice.py:83-90."""
+    reduction_layers = []
+    for pool_num in range(1, num_reduction_layers + 1):
+        layer_num = (float(pool_num) / (num_reduction_layers + 1)) * num_cells
+        reduction_layers.append(int(layer_num))
+    return reduction_layers
+
+
+class BaseCell(object):
+    """network_utils_slice.py:294-313: a NAS cell cut by the pipeline at ``cell_3``/``cell_7`` with two boundary
+    tensors (``cut_outputs``).  Shape of the interface only: no BASELINE config exercises AmoebaNet and its
+    kernels (separable / dilated conv, batch norm) are not built."""
+
+    def __init__(self, num_conv_filters, operations, used_hiddenstates, hiddenstate_indices, drop_path_keep_prob,
+                 total_num_cells, drop_path_burn_in_steps, dep_outputs=None):
+        self._num_conv_filters, self._operations = num_conv_filters, operations
+        self._used_hiddenstates, self._hiddenstate_indices = used_hiddenstates, hiddenstate_indices
+        self._drop_path_keep_prob, self._total_num_cells = drop_path_keep_prob, total_num_cells
+        self._drop_path_burn_in_steps, self._dep_outputs = drop_path_burn_in_steps, dep_outputs
+        self.cut_outputs = []
+
+    def __call__(self, net, scope=None, filter_scaling=1, stride=1, prev_layer=None, cell_num=-1):
+        raise NotImplementedError("AmoebaNet cells are not built: none of the measured configurations runs them")
+
+
+def build_network(inputs, num_classes, is_training=True, hparams=None, dep_outputs=None):
+    """model_builder_slice.py:292-345 (signature only)."""
+    raise NotImplementedError("AmoebaNet is an interface shell in this runtime: none of the measured configurations runs it")

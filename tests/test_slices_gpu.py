@@ -1,0 +1,71 @@
+"""The mirrored reference interfaces drive the HIP stages (GPU)."""
+import types
+
+import numpy as np
+import pytest
+import torch
+
+from dapple_amd import slices, synthetic
+from oracle import bert as ob
+from util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def test_bert_model_slice_stages_like_modeling_test():
+    # bert/models/bert/modeling_test.py:114-124 pins the shapes: embedding / sequence output [B, S, H]
+    B, S = 2, 8
+    cfg = slices.BertConfig(vocab_size=99, hidden_size=32, num_hidden_layers=2, num_attention_heads=4, intermediate_size=64,
+                            type_vocab_size=16, max_position_embeddings=64)
+    ids = torch.randint(0, 99, (B, S), dtype=torch.int32, device="cuda")
+    model = slices.BertModelSlice(cfg, False, ids)
+    assert len(model.stages) == cfg.num_hidden_layers + 3
+    x = ids
+    for f in model.stages[:-1]:
+        x = f(x)
+    assert model.get_embedding_output().shape == (B, S, 32) and model.get_sequence_output().shape == (B, S, 32)
+    assert len(model.get_all_encoder_layers()) == 2
+    w = ob.to_torch(model.weights)
+    want = ob.stage_forward(ids.cpu(), w, [0, 1], B, S, 4)
+    assert_close(x, want, 1e-4, "stages chained")
+    with pytest.raises(NotImplementedError):
+        model.stages[-1](x)
+    bad = slices.BertConfig(vocab_size=9, hidden_size=30, num_attention_heads=4)
+    with pytest.raises(ValueError, match="not a multiple of the number of attention"):
+        slices.BertModelSlice(bad, False, ids)
+    with pytest.raises(ValueError, match="cannot be greater than `max_position_embeddings`"):
+        slices.BertModelSlice(slices.BertConfig(vocab_size=9, hidden_size=32, num_attention_heads=4, max_position_embeddings=4), False, ids)
+
+
+def test_bert_finetune_slice_puts_the_planner_split_on_each_device():
+    cfg = slices.BertConfig(vocab_size=50, hidden_size=32, num_hidden_layers=24, num_attention_heads=4, intermediate_size=64,
+                            type_vocab_size=2, max_position_embeddings=16)
+    ids = torch.randint(0, 50, (2, 8), dtype=torch.int32, device="cuda")
+    s0 = slices.BertFinetuneSlice(cfg, 8, False, ids, None, None, None, False, model_type="mrc",
+                                  slice_devices="/gpu:0,/gpu:1", local_device=0, dtype="fp32")
+    s1 = slices.BertFinetuneSlice(cfg, 8, False, ids, None, None, None, False, model_type="mrc",
+                                  slice_devices=["/gpu:0", "/gpu:1"], local_device=1, dtype="fp32")
+    assert s0.layers == list(range(11)) and s1.layers == list(range(11, 24))
+    assert s0.stage.takes_input_grad is False and s1.stage.takes_input_grad is True
+    assert s0.stage.stash_slots == 2 and s1.stage.stash_slots == 1          # K = S - i
+    assert s0.stage.weight_names[0] == "bert/embeddings/word_embeddings"
+    assert s1.stage.weight_names[0] == "bert/encoder/layer_11/attention/self/query/kernel"
+    with pytest.raises(ValueError, match="Cannot use sequence length"):
+        slices.BertFinetuneSlice(cfg, 32, False, ids, None, None, None, False)
+    s0.stage.close(); s1.stage.close()
+
+
+def test_vgg_xlnet_gnmt_slices_build():
+    v = slices.SliceVGG19(num_replica=2)
+    assert [n for n, _ in v.layers][-1] == "block3_pool"
+    _, outs = v.build(torch.randn(2, 32, 32, 3, device="cuda"), None)
+    assert outs[0].shape == (2, 4, 4, 256)
+    x = slices.XlnetSlice(32000, 24, 4, 64, 16, 128, 16, False, memory_len=0, local_device=0, batch_size=2, dtype="fp32")
+    assert x.layers == list(range(11))
+    _, outs = x.build(torch.randn(1, 16, 2, 64, device="cuda"))
+    assert outs[0].shape == (1, 16, 2, 64) and torch.isfinite(outs[0]).all()
+    hp = types.SimpleNamespace(unit_type="lstm", num_units=16, forget_bias=1.0, dropout=0.0, num_encoder_layers=3, src_vocab_size=40)
+    g = slices.GNMTEncoderSlice(hp, batch_size=4, src_max_len=5)
+    assert [c.residual_connection for c in g.cells] == [False, False, False, True]
+    out = g.build_graph(torch.randint(0, 40, (4, 5), device="cuda"))
+    assert out.shape == (5, 4, 16)
