@@ -113,7 +113,7 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(int rows, int cols, 
                                                            const float* __restrict__ stats,
                                                            const T* __restrict__ dx_add, T* __restrict__ dx,
                                                            float* __restrict__ d_gamma, float* __restrict__ d_beta,
-                                                           float* __restrict__ d_colsum, int dbg) {
+                                                           float* __restrict__ d_colsum) {
   constexpr int VEC = Vec16<T>::N;
   typedef typename Vec16<T>::type V;
   extern __shared__ __attribute__((aligned(16))) float red[];  // [3][cols]
@@ -178,7 +178,6 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(int rows, int cols, 
       }
     }
   }
-  if (dbg & 1) return;
   // combine the 4 waves' column partials in LDS, one wave at a time (plain vector stores / read-modify-writes:
   // LDS float atomics on 32-byte-strided addresses serialise 16 ways)
   for (int wv = 0; wv < 4; ++wv) {
@@ -203,7 +202,6 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(int rows, int cols, 
     }
     __syncthreads();
   }
-  if (dbg & 2) return;
   for (int c = threadIdx.x; c < cols; c += 256) {
     atomicAdd(d_gamma + c, red[c]);
     atomicAdd(d_beta + c, red[cols + c]);
@@ -419,13 +417,10 @@ static int layernorm_bwd_t(int rows, int cols, const void* dy, const void* x, co
   if (rpw > 16) rpw = 16;
   dim3 grid((rows + 4 * rpw - 1) / (4 * rpw));
   const size_t lds = 3 * (size_t)cols * sizeof(float);
-  static const char* env = getenv("DS_LN_DEBUG");
-  const int dbg = env ? atoi(env) : 0;
-  if (env && getenv("DS_LN_RPW")) { rpw = atoi(getenv("DS_LN_RPW")); grid = dim3((rows + 4 * rpw - 1) / (4 * rpw)); }
   ds_prof_scope prof(s, sizeof(T) == 2 ? "layernorm_bwd_kernel<bf16>" : "layernorm_bwd_kernel<float>",
                      (double)rows * cols * sizeof(T) * (dx_add ? 4 : 3), "B");
   DISPATCH_NV(T, need, hipLaunchKernelGGL((layernorm_bwd_kernel<T, NV>), grid, dim3(256), lds, s, rows, cols, rpw,
-                                          (const T*)dy, (const T*)x, gamma, stats, (const T*)dx_add, (T*)dx, dg, db, dcs, dbg));
+                                          (const T*)dy, (const T*)x, gamma, stats, (const T*)dx_add, (T*)dx, dg, db, dcs));
   DS_CHECK_LAUNCH();
   return DS_OK;
 }
