@@ -212,6 +212,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="bert48_half")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-overlap", action="store_true", help="keep forward and backward passes on one stream")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs one pipeline stage on ONE GPU; --gpus %d is not supported "
@@ -224,6 +225,9 @@ def main():
     c = dict(synthetic.CONFIGS[args.workload])
     dtype = c["dtype"]
     wl = MAKERS[c["kind"]](c, args)
+    overlap = not args.no_overlap and wl.stage.overlap_supported()
+    if overlap:
+        wl.stage.enable_overlap()   # backward passes on a second stream: F(j+K) runs beside B(j+1)
 
     for _ in range(args.warmup):
         wl.step()
@@ -259,6 +263,7 @@ def main():
                    "unit": "TFLOP/s" if v[3] == "FLOP" else "GB/s"} for t, v in sorted(prof.items(), key=lambda kv: -kv[1][1])}
     cfg = {"workload": args.workload, "grad_accum": "fp32 in place", "flops_per_sample": wl.flops_per_sample}
     cfg.update(wl.config)
+    cfg["fwd_bwd_overlap"] = overlap
     line = {
         "metric": METRIC.get(args.workload, "stage samples/sec fwd+bwd+grad-accum, %s; MFMA util %%" % args.workload),
         "value": value, "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

@@ -89,8 +89,54 @@ extern "C" int ds_stage_create(const ds_stage_cfg* cfg, void* stream, ds_stage**
 extern "C" int ds_stage_destroy(ds_stage* h) {
   if (!h) return DS_OK;
   (void)hipStreamSynchronize(h->stream);
+  if (h->bwd_stream) {
+    (void)hipStreamSynchronize(h->bwd_stream);
+    for (hipEvent_t e : h->ev_forwarded) (void)hipEventDestroy(e);
+    for (hipEvent_t e : h->ev_released) (void)hipEventDestroy(e);
+    if (h->ev_join) (void)hipEventDestroy(h->ev_join);
+    (void)hipStreamDestroy(h->bwd_stream);
+  }
   delete h;
   return DS_OK;
+}
+
+extern "C" int ds_stage_overlap_supported(const ds_stage* h) { return h && h->overlap_safe() ? 1 : 0; }
+
+extern "C" int ds_stage_enable_overlap(ds_stage* h) {
+  DS_CHECK_ARG(h != nullptr, "ds_stage_enable_overlap: null handle");
+  if (!h->overlap_safe()) {
+    ds_set_error("ds_stage_enable_overlap: this stage's forward and backward passes share workspace");
+    return DS_EINVAL;
+  }
+  if (h->bwd_stream) return DS_OK;
+  for (char f : h->slot_forwarded)
+    if (f) { ds_set_error("ds_stage_enable_overlap: micro-batches in flight"); return DS_ESTATE; }
+  DS_CHECK_HIP(hipStreamCreateWithFlags(&h->bwd_stream, hipStreamNonBlocking));
+  const int K = h->cfg.stash_slots;
+  h->ev_forwarded.resize(K);
+  h->ev_released.resize(K);
+  h->released_valid.assign(K, 0);
+  for (int i = 0; i < K; ++i) {
+    DS_CHECK_HIP(hipEventCreateWithFlags(&h->ev_forwarded[i], hipEventDisableTiming));
+    DS_CHECK_HIP(hipEventCreateWithFlags(&h->ev_released[i], hipEventDisableTiming));
+  }
+  DS_CHECK_HIP(hipEventCreateWithFlags(&h->ev_join, hipEventDisableTiming));
+  return DS_OK;
+}
+
+// Orders everything queued on the backward stream before whatever is queued next on the stage's stream.
+static int stage_join(ds_stage* h) {
+  if (h->bwd_stream && h->bwd_pending) {
+    DS_CHECK_HIP(hipEventRecord(h->ev_join, h->bwd_stream));
+    DS_CHECK_HIP(hipStreamWaitEvent(h->stream, h->ev_join, 0));
+    h->bwd_pending = false;
+  }
+  return DS_OK;
+}
+
+extern "C" int ds_stage_join(ds_stage* h) {
+  DS_CHECK_ARG(h != nullptr, "ds_stage_join: null handle");
+  return stage_join(h);
 }
 
 extern "C" int ds_stage_num_weights(const ds_stage* h) { return h ? (int)h->winfo.size() : 0; }
@@ -131,6 +177,7 @@ extern "C" int ds_stage_bind_weights(ds_stage* h, int n, const void* const* weig
 extern "C" int ds_stage_refresh_weights(ds_stage* h) {
   DS_CHECK_ARG(h != nullptr, "ds_stage_refresh_weights: null handle");
   if (!h->bound) { ds_set_error("ds_stage_refresh_weights: weights not bound"); return DS_ESTATE; }
+  DS_PROPAGATE(stage_join(h));  // a backward pass still queued reads the compute copies
   return h->refresh_weights();
 }
 
@@ -143,8 +190,10 @@ extern "C" int ds_stage_forward(ds_stage* h, int slot, const void* in, const flo
     return DS_ESTATE;
   }
   DS_CHECK_ARG(ds_aligned16(in) && ds_aligned16(out), "ds_stage_forward: in/out must be 16-byte aligned");
+  if (h->bwd_stream && h->released_valid[slot]) DS_CHECK_HIP(hipStreamWaitEvent(h->stream, h->ev_released[slot], 0));
   const int rc = h->forward(slot, in, key_mask, out);
   if (rc == DS_OK) h->slot_forwarded[slot] = 1;
+  if (rc == DS_OK && h->bwd_stream) DS_CHECK_HIP(hipEventRecord(h->ev_forwarded[slot], h->stream));
   return rc;
 }
 
@@ -156,7 +205,19 @@ extern "C" int ds_stage_backward(ds_stage* h, int slot, const void* d_out, void*
     return DS_ESTATE;
   }
   DS_CHECK_ARG(ds_aligned16(d_out) && ds_aligned16(d_in), "ds_stage_backward: d_out/d_in must be 16-byte aligned");
-  const int rc = h->backward(slot, d_out, d_in);
+  int rc;
+  if (h->bwd_stream) {
+    DS_CHECK_HIP(hipStreamWaitEvent(h->bwd_stream, h->ev_forwarded[slot], 0));
+    hipStream_t fwd = h->stream;
+    h->stream = h->bwd_stream;
+    rc = h->backward(slot, d_out, d_in);
+    h->stream = fwd;
+    (void)hipEventRecord(h->ev_released[slot], h->bwd_stream);
+    h->released_valid[slot] = 1;
+    h->bwd_pending = true;
+  } else {
+    rc = h->backward(slot, d_out, d_in);
+  }
   h->slot_forwarded[slot] = 0;
   return rc;
 }
@@ -166,6 +227,7 @@ extern "C" size_t ds_stage_stash_bytes(const ds_stage* h, int slots) { return h 
 
 extern "C" int ds_stage_sync(ds_stage* h) {
   DS_CHECK_ARG(h != nullptr, "ds_stage_sync: null handle");
+  DS_PROPAGATE(stage_join(h));
   DS_CHECK_HIP(hipStreamSynchronize(h->stream));
   return DS_OK;
 }

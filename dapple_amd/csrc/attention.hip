@@ -24,10 +24,19 @@ constexpr int HD = 64;        // head size
 constexpr int ROWB = 128;     // bytes per tile row (64 bf16)
 constexpr int CHUNK = 512;    // rows of K/V (or Q/dO) resident in LDS at a time
 
-// LDS tile layout: row-major [row][64 bf16], 32-byte granules XOR-swizzled by the row
+// LDS tile layout: row-major [row][64 bf16], the 16-byte chunk index XOR-swizzled by the row.  The
+// LDS has 64 banks (a 256-byte line = two tile rows).  The swizzle serves both read patterns:
+//   frag_rows: 16 lanes read one chunk column of 16 consecutive rows -> the 8 rows of equal parity
+//              need 8 different chunks: any bijection of t = (row >> 1) & 7;
+//   frag_cols: 32 lanes read 4 consecutive rows x 4 adjacent chunks -> rows r and r+2 (same half
+//              line, t differs in bit 0) must land in different 64-byte quarters: bit 0 of t is
+//              moved to bit 2 of the chunk index.
+__device__ __forceinline__ int tile_swz(int row) {
+  const int t = (row >> 1) & 7;
+  return ((t & 1) << 2) | (t >> 1);
+}
 __device__ __forceinline__ int tile_off(int row, int byte) {
-  const int g = (byte >> 5) ^ (((row & 3) << 1) & 3);
-  return row * ROWB + (g << 5) + (byte & 31);
+  return row * ROWB + ((((byte >> 4) ^ tile_swz(row))) << 4) + (byte & 15);
 }
 
 // Fills `rows` tile rows (multiple of 16) from global rows of stride ld (elements); 128 threads.
@@ -35,8 +44,7 @@ __device__ __forceinline__ void tile_fill(char* lds, const bf16* src, int64_t ld
   for (int c = wave; c < rows / 8; c += 2) {  // each call: one wave writes 64 consecutive 16-byte slots = 8 rows
     const int p = c * 64 + lane;
     const int r = p >> 3, pc = p & 7;
-    const int g = (pc >> 1) ^ (((r & 3) << 1) & 3);
-    const bf16* s = src + (int64_t)r * ld + (g * 2 + (pc & 1)) * 8;
+    const bf16* s = src + (int64_t)r * ld + (pc ^ tile_swz(r)) * 8;
     __builtin_amdgcn_global_load_lds((glb_vptr)s, (lds_vptr)(lds + c * 1024), 16, 0, 0);
   }
 }

@@ -7,7 +7,7 @@
 // k-tile; the next k-tile's global loads are in flight while the current one is multiplied.
 //
 // LDS layouts (both XOR-swizzled so that fragment reads and tile stores are conflict free):
-//   K-major operand : [free row][128 B of k]; 16-byte chunk c of row r lives at chunk c ^ (r & 7).
+//   K-major operand : [free row][128 B of k]; 16-byte chunk c of row r lives at chunk c ^ ((r >> 1) & 7).
 //                     A lane reads its MFMA fragment as one 16-byte load.
 //   MN-major operand: [k row][free index contiguous]; 32-byte granule g of row r lives at
 //                     g ^ (((r & 3) << 1) & (granules-1)).  bf16 fragments come from
@@ -56,10 +56,20 @@ struct GemmArgs {
   int conv_h, conv_w, conv_c;  // implicit 3x3 'same' convolution: extent of the gathered NHWC tensor
 };
 
-__device__ __forceinline__ int kmajor_off(int row, int chunk) { return row * 128 + ((chunk ^ (row & 7)) << 4); }
-template <int ROW_BYTES> __device__ __forceinline__ int mnmajor_off(int r, int cbyte) {
+// LDS has 64 banks of 4 bytes: one bank line is 256 bytes = two 128-byte K-major rows.
+// K-major: a 16-lane phase of a 16-byte fragment read covers 16 consecutive rows of one chunk
+// column; rows of equal parity share a half line, so the chunk is rotated by (row >> 1).
+__device__ __forceinline__ int kmajor_swz(int row) { return (row >> 1) & 7; }
+__device__ __forceinline__ int kmajor_off(int row, int chunk) { return row * 128 + ((chunk ^ kmajor_swz(row)) << 4); }
+// MN-major: a transposing read touches 4 consecutive rows x two 32-byte granules per 32 lanes.
+// Rows of 256 bytes or more start on a bank line: rotate the granule pair by (r & 3).  Rows of 128
+// bytes alternate between the halves of a line: only rows r and r+2 collide, rotate by bit 1 of r.
+template <int ROW_BYTES> __device__ __forceinline__ int mnmajor_swz(int r) {
   constexpr int NG = ROW_BYTES / 32;
-  const int g = (cbyte >> 5) ^ (((r & 3) << 1) & (NG - 1));
+  return ROW_BYTES >= 256 ? (((r & 3) << 1) & (NG - 1)) : (((r >> 1) & 1) << 1);
+}
+template <int ROW_BYTES> __device__ __forceinline__ int mnmajor_off(int r, int cbyte) {
+  const int g = (cbyte >> 5) ^ mnmajor_swz<ROW_BYTES>(r);
   return r * ROW_BYTES + (g << 5) + (cbyte & 31);
 }
 
@@ -456,10 +466,10 @@ template <typename T, int W, int MAJOR, int NF> struct FragReader {
     constexpr int NG = ROW_BYTES / 32;
     const uint32_t base = off[i];
     const uint32_t g = (base % ROW_BYTES) >> 5, within = base & 31, row0 = base / ROW_BYTES;
-    lds_read_b32(f.e0, tile + (row0 + 8 * ks + 0) * ROW_BYTES + ((g ^ (0 & (NG - 1))) << 5) + within);
-    lds_read_b32(f.e1, tile + (row0 + 8 * ks + 1) * ROW_BYTES + ((g ^ (2 & (NG - 1))) << 5) + within);
-    lds_read_b32(f.e2, tile + (row0 + 8 * ks + 2) * ROW_BYTES + ((g ^ (4 & (NG - 1))) << 5) + within);
-    lds_read_b32(f.e3, tile + (row0 + 8 * ks + 3) * ROW_BYTES + ((g ^ (6 & (NG - 1))) << 5) + within);
+    lds_read_b32(f.e0, tile + (row0 + 8 * ks + 0) * ROW_BYTES + ((g ^ mnmajor_swz<ROW_BYTES>(0)) << 5) + within);
+    lds_read_b32(f.e1, tile + (row0 + 8 * ks + 1) * ROW_BYTES + ((g ^ mnmajor_swz<ROW_BYTES>(1)) << 5) + within);
+    lds_read_b32(f.e2, tile + (row0 + 8 * ks + 2) * ROW_BYTES + ((g ^ mnmajor_swz<ROW_BYTES>(2)) << 5) + within);
+    lds_read_b32(f.e3, tile + (row0 + 8 * ks + 3) * ROW_BYTES + ((g ^ mnmajor_swz<ROW_BYTES>(3)) << 5) + within);
   }
 };
 
@@ -491,26 +501,30 @@ template <typename T, int W, int MAJOR> struct PlainDma {
     for (int i = 0; i < NV; ++i) {
       const int p = (i * 4 + wave) * 64 + lane;
       if (MAJOR == DS_K_MAJOR) {
-        const int row = p >> 3, c = (p & 7) ^ (row & 7);
+        const int row = p >> 3, c = (p & 7) ^ kmajor_swz(row);
         int f = f0 + row;
         if (f > F - 1) f = F - 1;
         src[i] = base + (int64_t)f * ld + k0 + c * VEC;
       } else {
         constexpr int NG = ROW_BYTES / 32;
         const int r = p / CPR, pc = p % CPR;
-        const int g = (pc >> 1) ^ (((r & 3) << 1) & (NG - 1));
+        const int g = (pc >> 1) ^ mnmajor_swz<ROW_BYTES>(r);
         int f = f0 + (g * 2 + (pc & 1)) * VEC;
         if (f > F - VEC) f = F - VEC;
         src[i] = base + (int64_t)(k0 + r) * ld + f;
       }
     }
   }
+  // load i of the current k-tile (i = 0 .. NV-1, each exactly once per k-tile), then advance()
+  __device__ __forceinline__ void issue_one(char* lds, int wave, int i) {
+    __builtin_amdgcn_global_load_lds((glb_vptr)src[i], (lds_vptr)(lds + (i * 4 + wave) * 1024), 16, 0, 0);
+    src[i] += step;
+  }
+  __device__ __forceinline__ void advance() {}
   __device__ __forceinline__ void issue(char* lds, int wave) {
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      __builtin_amdgcn_global_load_lds((glb_vptr)src[i], (lds_vptr)(lds + (i * 4 + wave) * 1024), 16, 0, 0);
-      src[i] += step;
-    }
+    for (int i = 0; i < NV; ++i) issue_one(lds, wave, i);
+    advance();
   }
 };
 
@@ -550,7 +564,7 @@ template <typename T, int W, int MODE> struct ConvDma {
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
         const int pos = (i * 4 + wave) * 64 + lane;
-        const int row = pos >> 3, c = (pos & 7) ^ (row & 7);
+        const int row = pos >> 3, c = (pos & 7) ^ kmajor_swz(row);
         int pix = f0 + row;
         if (pix > F - 1) pix = F - 1;
         x[i] = pix % Wd;
@@ -564,7 +578,7 @@ template <typename T, int W, int MODE> struct ConvDma {
         constexpr int NG = ROW_BYTES / 32;
         const int pos = (i * 4 + wave) * 64 + lane;
         const int rr = pos / CPR, pc = pos % CPR;
-        const int g = (pc >> 1) ^ (((rr & 3) << 1) & (NG - 1));
+        const int g = (pc >> 1) ^ mnmajor_swz<ROW_BYTES>(rr);
         int mi = f0 + (g * 2 + (pc & 1)) * VEC;
         if (mi > F - VEC) mi = F - VEC;
         const int t = mi / C, c = mi - t * C;
@@ -575,31 +589,36 @@ template <typename T, int W, int MODE> struct ConvDma {
       }
     }
   }
-  __device__ __forceinline__ void issue(char* lds, int wave) {
+  // load i of the current k-tile (i = 0 .. NV-1, each exactly once per k-tile), then advance()
+  __device__ __forceinline__ void issue_one(char* lds, int wave, int i) {
     if (MODE == 1) {
       const int dy = tap / 3 - 1, dx = tap - (tap / 3) * 3 - 1;
       const int sh = (dy * Wd + dx) * C + c0;
-#pragma unroll
-      for (int i = 0; i < NV; ++i) {
-        const bool ok = (unsigned)(y[i] + dy) < (unsigned)H && (unsigned)(x[i] + dx) < (unsigned)Wd;
-        const T* src = ok ? base + off[i] + sh : reinterpret_cast<const T*>(g_zero16);
-        __builtin_amdgcn_global_load_lds((glb_vptr)src, (lds_vptr)(lds + (i * 4 + wave) * 1024), 16, 0, 0);
-      }
+      const bool ok = (unsigned)(y[i] + dy) < (unsigned)H && (unsigned)(x[i] + dx) < (unsigned)Wd;
+      const T* src = ok ? base + off[i] + sh : reinterpret_cast<const T*>(g_zero16);
+      __builtin_amdgcn_global_load_lds((glb_vptr)src, (lds_vptr)(lds + (i * 4 + wave) * 1024), 16, 0, 0);
+    } else {
+      const int64_t pix = pix0 + r[i];
+      const int q = (int)(pix / Wd);
+      const int xx = (int)(pix - (int64_t)q * Wd), yy = q % H;
+      const int dy = (dyx[i] >> 2) - 1, dx = (dyx[i] & 3) - 1;
+      const bool ok = (unsigned)(yy + dy) < (unsigned)H && (unsigned)(xx + dx) < (unsigned)Wd;
+      const T* src = ok ? base + pix * C + shift[i] : reinterpret_cast<const T*>(g_zero16);
+      __builtin_amdgcn_global_load_lds((glb_vptr)src, (lds_vptr)(lds + (i * 4 + wave) * 1024), 16, 0, 0);
+    }
+  }
+  __device__ __forceinline__ void advance() {
+    if (MODE == 1) {
       c0 += KT;
       if (c0 == C) { c0 = 0; ++tap; }
     } else {
-#pragma unroll
-      for (int i = 0; i < NV; ++i) {
-        const int64_t pix = pix0 + r[i];
-        const int q = (int)(pix / Wd);
-        const int xx = (int)(pix - (int64_t)q * Wd), yy = q % H;
-        const int dy = (dyx[i] >> 2) - 1, dx = (dyx[i] & 3) - 1;
-        const bool ok = (unsigned)(yy + dy) < (unsigned)H && (unsigned)(xx + dx) < (unsigned)Wd;
-        const T* src = ok ? base + pix * C + shift[i] : reinterpret_cast<const T*>(g_zero16);
-        __builtin_amdgcn_global_load_lds((glb_vptr)src, (lds_vptr)(lds + (i * 4 + wave) * 1024), 16, 0, 0);
-      }
       pix0 += KT;
     }
+  }
+  __device__ __forceinline__ void issue(char* lds, int wave) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) issue_one(lds, wave, i);
+    advance();
   }
 };
 
@@ -673,12 +692,14 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
     if (kt + STAGES - 2 < nkt) __builtin_amdgcn_s_waitcnt(DS_VMCNT(LPT * (STAGES - 2)));
     else __builtin_amdgcn_s_waitcnt(DS_VMCNT(0));
     __builtin_amdgcn_s_barrier();
-    if (kt + STAGES - 1 < nkt) {
-      int nb = buf + STAGES - 1;
-      if (nb >= STAGES) nb -= STAGES;
-      da.issue(lds + nb * STAGE_BYTES, wave);
-      db.issue(lds + nb * STAGE_BYTES + A_BYTES, wave);
-    }
+    // The loads of tile kt+STAGES-1 are issued one at a time between the MFMAs: a wave stalls on a
+    // load instruction while the address unit is busy, and issued as one burst those stalls would
+    // sit in front of the MFMAs instead of underneath them.
+    const bool more = kt + STAGES - 1 < nkt;
+    int nb = buf + STAGES - 1;
+    if (nb >= STAGES) nb -= STAGES;
+    char* const na = lds + nb * STAGE_BYTES;
+    char* const nbp = na + A_BYTES;
     const uint32_t sa = lds0 + buf * STAGE_BYTES, sb = sa + A_BYTES;
     RawFrag<T, AMAJ> fa[2][TM];
     RawFrag<T, BMAJ> fb[2][TN];
@@ -702,8 +723,21 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j) Mma<T>::mma(acc[i][j], to_frag(fa[cur][i]), to_frag(fb[cur][j]));
+        for (int j = 0; j < TN; ++j) {
+          Mma<T>::mma(acc[i][j], to_frag(fa[cur][i]), to_frag(fb[cur][j]));
+          constexpr int NMMA = 4 * TM * TN;
+          const int q = (ks * TM + i) * TN + j;  // compile-time after unrolling
+          if (more) {
+#pragma unroll
+            for (int l = 0; l < LPT; ++l)
+              if ((l * NMMA) / LPT == q) {
+                if (l < DA::NV) da.issue_one(na, wave, l);
+                else db.issue_one(nbp, wave, l - DA::NV);
+              }
+          }
+        }
     }
+    if (more) { da.advance(); db.advance(); }
     if (++buf == STAGES) buf = 0;
   }
   if (p.vec_epi) gemm_epilogue_staged<T, BM, BN>(p, acc, m0, n0, wm, wn, lane, tid, c_off, lds);

@@ -31,7 +31,17 @@ struct ds_stage {
   std::vector<float*> g;        // fp32 master grads
   bool bound = false;
   std::vector<char> slot_forwarded;
+  // optional forward/backward overlap: backward passes run on a second stream, ordered against the
+  // forward passes by one event pair per stash slot
+  hipStream_t bwd_stream = nullptr;
+  std::vector<hipEvent_t> ev_forwarded, ev_released;
+  std::vector<char> released_valid;
+  hipEvent_t ev_join = nullptr;
+  bool bwd_pending = false;
   virtual ~ds_stage() {}
+  // true when forward and backward passes of different slots touch disjoint memory (apart from
+  // read-only weights), so they may run concurrently
+  virtual bool overlap_safe() const { return false; }
   virtual int refresh_weights() = 0;
   virtual int forward(int slot, const void* in, const float* key_mask, void* out) = 0;
   virtual int backward(int slot, const void* d_out, void* d_in) = 0;

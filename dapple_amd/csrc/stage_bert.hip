@@ -77,6 +77,8 @@ struct BertStage : ds_stage {
   size_t esz;
   bool emb;
   bool fused_attn;  // bf16, head size 64: fused attention kernels, no [B,N,S,S] tensors at all
+  // the fused forward pass writes only its stash slot and its output; the workspace belongs to backward
+  bool overlap_safe() const override { return fused_attn; }
   // compute copies
   char* wc_base = nullptr;
   std::vector<char*> wqkv, wo, w1, w2;  // element type T

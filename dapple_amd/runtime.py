@@ -135,6 +135,18 @@ class Stage:
     def sync(self):
         check(self.lib.ds_stage_sync(self._h), "ds_stage_sync")
 
+    # -- forward/backward overlap (backward passes on a second stream of the handle) --------------
+    def overlap_supported(self):
+        return bool(self.lib.ds_stage_overlap_supported(self._h))
+
+    def enable_overlap(self):
+        check(self.lib.ds_stage_enable_overlap(self._h), "ds_stage_enable_overlap")
+        self.overlap = True
+
+    def join(self):
+        """Orders queued backward work before whatever is queued next on the stage's stream."""
+        check(self.lib.ds_stage_join(self._h), "ds_stage_join")
+
     def workspace_bytes(self):
         return self.lib.ds_stage_workspace_bytes(self._h)
 
@@ -284,4 +296,5 @@ class StageRuntime:
                 d_in = input_grads[j] if (self.needs_input_grad and input_grads is not None) else None
                 self.stage.backward(slot, upstream[j], d_in)
                 free.append(slot)
+        self.stage.join()
         return outputs

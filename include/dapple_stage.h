@@ -188,6 +188,19 @@ int ds_stage_backward(ds_stage* h, int slot, const void* d_out, void* d_in);
 size_t ds_stage_workspace_bytes(const ds_stage* h);
 size_t ds_stage_stash_bytes(const ds_stage* h, int slots);
 int ds_stage_sync(ds_stage* h);
+/* Forward/backward overlap.  The reference leaves the order of one stage's forward and backward
+ * passes of different micro-batches to TensorFlow's inter-op scheduler: only the control
+ * dependencies of bert/graph.py:126-132 constrain it (256 inter-op threads,
+ * bert/train_flags.py:183-186), so F(j+K) and B(j+1) may run at the same time.
+ * ds_stage_enable_overlap puts the backward passes on a second stream owned by the handle (default
+ * priority); per-slot events keep B(slot) after F(slot) and the next F(slot) after B(slot).
+ * ds_stage_join orders all queued backward work before what is queued next on the stage's stream
+ * (call it at the end of a step, before reading gradients on that stream); ds_stage_sync and
+ * ds_stage_refresh_weights join by themselves.  Stages whose forward and backward passes share
+ * workspace report 0 from ds_stage_overlap_supported and DS_EINVAL from ds_stage_enable_overlap. */
+int ds_stage_overlap_supported(const ds_stage* h);
+int ds_stage_enable_overlap(ds_stage* h);
+int ds_stage_join(ds_stage* h);
 
 /* ---------------------------------------------------------------------------
  * 3x3, stride 1, 'same' convolution over NHWC fp32 tensors as an implicit GEMM on the matrix cores.

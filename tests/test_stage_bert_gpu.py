@@ -149,3 +149,48 @@ def test_call_order_errors():
     with pytest.raises(ValueError, match="not a multiple"):
         runtime.bert_stage(1, 100, 3, 128, 2, 16, "fp32", stash_slots=1)
     stage.close()
+
+
+@pytest.mark.gpu
+def test_forward_backward_overlap_matches_serial():
+    """Backward passes on the handle's second stream: same outputs and input gradients bit for bit,
+    weight gradients equal up to the order of the atomic adds."""
+    import numpy as np
+    import torch
+    from dapple_amd import runtime, synthetic
+    L, H, N, F, B, S, M = 2, 256, 4, 512, 2, 128, 6
+    w = synthetic.bert_weights(11, L, H, F)
+    xs = [torch.as_tensor(x).cuda().bfloat16() for x in synthetic.bert_activation_inputs(12, M, B, S, H)]
+    dys = [torch.as_tensor(x).cuda().bfloat16() for x in synthetic.upstream_grads(13, M, (B * S, H))]
+    res = []
+    for overlap in (False, True):
+        st = runtime.bert_stage(L, H, N, F, B, S, "bf16", stash_slots=2)
+        st.bind(w)
+        assert st.overlap_supported()
+        if overlap:
+            st.enable_overlap()
+        outs = [torch.empty(B * S, H, dtype=torch.bfloat16, device="cuda") for _ in range(M)]
+        dxs = [torch.empty_like(o) for o in outs]
+        rt = runtime.StageRuntime(st, 0, 2, M)
+        for _ in range(3):                       # several steps: slot events are reused across steps
+            st.refresh_weights()
+            st.zero_grads()
+            rt.step(xs, dys, outs, dxs)
+        st.sync()
+        res.append(([o.float().cpu() for o in outs], [d.float().cpu() for d in dxs], {k: v.cpu().clone() for k, v in st.grads.items()}))
+        st.close()
+    for a, b in zip(res[0][0] + res[0][1], res[1][0] + res[1][1]):
+        assert torch.equal(a, b)
+    for k in res[0][2]:
+        a, b = res[0][2][k], res[1][2][k]
+        assert float((a - b).abs().max()) <= 1e-5 * float(a.abs().max()) + 1e-12, k
+
+
+@pytest.mark.gpu
+def test_overlap_refused_where_passes_share_workspace():
+    from dapple_amd import runtime
+    st = runtime.bert_stage(1, 64, 2, 128, 1, 16, "fp32", stash_slots=1)
+    assert not st.overlap_supported()
+    with pytest.raises(ValueError):
+        st.enable_overlap()
+    st.close()
