@@ -245,6 +245,16 @@ def main():
     torch.cuda.synchronize()
     prof = _lib.profile_dump()
     _lib.profile(False)
+    iso = None
+    if overlap:
+        # the same kernels with the stage back on one stream: durations free of the other streams' traffic
+        wl.stage.enable_overlap(False)
+        wl.step()
+        _lib.profile(True)
+        wl.step()
+        torch.cuda.synchronize()
+        iso = _lib.profile_dump()
+        _lib.profile(False)
     total_ms = sum(v[1] for v in prof.values())
     dom = max(prof, key=lambda t: prof[t][1])
     n, ms, work, unit = prof[dom]
@@ -255,6 +265,11 @@ def main():
     roof["frac"] = roof["achieved"] / roof["peak"]
     roof["traffic"] = None
     roof.update({"kernel": dom, "launches": n, "avg_launch_us": ms * 1e3 / n, "share_of_kernel_time": ms / total_ms})
+    if iso is not None and dom in iso:
+        n2, ms2, work2, _ = iso[dom]
+        rate = work2 / (ms2 * 1e-3) / (1e12 if unit == "FLOP" else 1e9)
+        roof["one_stream"] = {"achieved": rate, "frac": rate / roof["peak"], "avg_launch_us": ms2 * 1e3 / n2,
+                              "note": "same kernel with forward, backward and weight-gradient work serialised on one stream"}
     stage_flops = wl.flops_per_sample * wl.samples
     roof["stage_achieved_TFLOPs"] = stage_flops / dt / 1e12
     roof["stage_frac_of_mfma_peak"] = stage_flops / dt / PEAK[dtype]

@@ -118,7 +118,7 @@ PROTOTYPES = {
     "ds_stage_stash_bytes": (C.c_size_t, [C.c_void_p, C.c_int]),
     "ds_stage_sync": (C.c_int, [C.c_void_p]),
     "ds_stage_overlap_supported": (C.c_int, [C.c_void_p]),
-    "ds_stage_enable_overlap": (C.c_int, [C.c_void_p]),
+    "ds_stage_enable_overlap": (C.c_int, [C.c_void_p, C.c_int]),
     "ds_stage_join": (C.c_int, [C.c_void_p]),
 }
 

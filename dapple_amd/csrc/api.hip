@@ -89,40 +89,20 @@ extern "C" int ds_stage_create(const ds_stage_cfg* cfg, void* stream, ds_stage**
 extern "C" int ds_stage_destroy(ds_stage* h) {
   if (!h) return DS_OK;
   (void)hipStreamSynchronize(h->stream);
-  if (h->bwd_stream) {
-    (void)hipStreamSynchronize(h->bwd_stream);
+  if (h->bwd_owned) {
+    (void)hipStreamSynchronize(h->bwd_owned);
+    (void)hipStreamSynchronize(h->wgrad_owned);
     for (hipEvent_t e : h->ev_forwarded) (void)hipEventDestroy(e);
     for (hipEvent_t e : h->ev_released) (void)hipEventDestroy(e);
     if (h->ev_join) (void)hipEventDestroy(h->ev_join);
-    (void)hipStreamDestroy(h->bwd_stream);
+    (void)hipStreamDestroy(h->bwd_owned);
+    (void)hipStreamDestroy(h->wgrad_owned);
   }
   delete h;
   return DS_OK;
 }
 
 extern "C" int ds_stage_overlap_supported(const ds_stage* h) { return h && h->overlap_safe() ? 1 : 0; }
-
-extern "C" int ds_stage_enable_overlap(ds_stage* h) {
-  DS_CHECK_ARG(h != nullptr, "ds_stage_enable_overlap: null handle");
-  if (!h->overlap_safe()) {
-    ds_set_error("ds_stage_enable_overlap: this stage's forward and backward passes share workspace");
-    return DS_EINVAL;
-  }
-  if (h->bwd_stream) return DS_OK;
-  for (char f : h->slot_forwarded)
-    if (f) { ds_set_error("ds_stage_enable_overlap: micro-batches in flight"); return DS_ESTATE; }
-  DS_CHECK_HIP(hipStreamCreateWithFlags(&h->bwd_stream, hipStreamNonBlocking));
-  const int K = h->cfg.stash_slots;
-  h->ev_forwarded.resize(K);
-  h->ev_released.resize(K);
-  h->released_valid.assign(K, 0);
-  for (int i = 0; i < K; ++i) {
-    DS_CHECK_HIP(hipEventCreateWithFlags(&h->ev_forwarded[i], hipEventDisableTiming));
-    DS_CHECK_HIP(hipEventCreateWithFlags(&h->ev_released[i], hipEventDisableTiming));
-  }
-  DS_CHECK_HIP(hipEventCreateWithFlags(&h->ev_join, hipEventDisableTiming));
-  return DS_OK;
-}
 
 // Orders everything queued on the backward stream before whatever is queued next on the stage's stream.
 static int stage_join(ds_stage* h) {
@@ -131,6 +111,38 @@ static int stage_join(ds_stage* h) {
     DS_CHECK_HIP(hipStreamWaitEvent(h->stream, h->ev_join, 0));
     h->bwd_pending = false;
   }
+  return DS_OK;
+}
+
+extern "C" int ds_stage_enable_overlap(ds_stage* h, int on) {
+  DS_CHECK_ARG(h != nullptr, "ds_stage_enable_overlap: null handle");
+  if (on && !h->overlap_safe()) {
+    ds_set_error("ds_stage_enable_overlap: this stage's forward and backward passes share workspace");
+    return DS_EINVAL;
+  }
+  for (char f : h->slot_forwarded)
+    if (f) { ds_set_error("ds_stage_enable_overlap: micro-batches in flight"); return DS_ESTATE; }
+  if (!on) {
+    DS_PROPAGATE(stage_join(h));
+    h->bwd_stream = nullptr;
+    h->wgrad_stream = nullptr;
+    return DS_OK;
+  }
+  if (!h->bwd_owned) {
+    DS_CHECK_HIP(hipStreamCreateWithFlags(&h->bwd_owned, hipStreamNonBlocking));
+    DS_CHECK_HIP(hipStreamCreateWithFlags(&h->wgrad_owned, hipStreamNonBlocking));
+    const int K = h->cfg.stash_slots;
+    h->ev_forwarded.resize(K);
+    h->ev_released.resize(K);
+    for (int i = 0; i < K; ++i) {
+      DS_CHECK_HIP(hipEventCreateWithFlags(&h->ev_forwarded[i], hipEventDisableTiming));
+      DS_CHECK_HIP(hipEventCreateWithFlags(&h->ev_released[i], hipEventDisableTiming));
+    }
+    DS_CHECK_HIP(hipEventCreateWithFlags(&h->ev_join, hipEventDisableTiming));
+  }
+  h->released_valid.assign(h->cfg.stash_slots, 0);  // everything queued so far is ordered on h->stream
+  h->bwd_stream = h->bwd_owned;
+  h->wgrad_stream = h->wgrad_owned;
   return DS_OK;
 }
 

@@ -34,6 +34,8 @@ struct ds_stage {
   // optional forward/backward overlap: backward passes run on a second stream, ordered against the
   // forward passes by one event pair per stash slot
   hipStream_t bwd_stream = nullptr;
+  hipStream_t wgrad_stream = nullptr;  // weight-gradient GEMMs of a backward pass (stages that support it)
+  hipStream_t bwd_owned = nullptr, wgrad_owned = nullptr;  // created once, kept while overlap is switched off
   std::vector<hipEvent_t> ev_forwarded, ev_released;
   std::vector<char> released_valid;
   hipEvent_t ev_join = nullptr;

@@ -93,12 +93,20 @@ struct BertStage : ds_stage {
   // workspace
   char* ws_base = nullptr;
   size_t ws_bytes = 0;
-  size_t ws_scores, ws_ds, ws_dz2, ws_du, ws_da, ws_dz1, ws_dctx, ws_dqkv, ws_dx[2];
+  size_t ws_scores, ws_ds, ws_dz2[2], ws_du[2], ws_da, ws_dz1[2], ws_dctx, ws_dqkv[2], ws_dx[2];
+  // weight-gradient stream bookkeeping: per layer parity, "dgrad chain produced the wgrad operands" and
+  // "wgrads consumed them"
+  hipEvent_t ev_ready[2] = {nullptr, nullptr}, ev_done[2] = {nullptr, nullptr};
+  bool done_valid[2] = {false, false};
 
   ~BertStage() override {
     if (wc_base) (void)hipFree(wc_base);
     if (stash_base) (void)hipFree(stash_base);
     if (ws_base) (void)hipFree(ws_base);
+    for (int p = 0; p < 2; ++p) {
+      if (ev_ready[p]) (void)hipEventDestroy(ev_ready[p]);
+      if (ev_done[p]) (void)hipEventDestroy(ev_done[p]);
+    }
   }
   int base(int l) const { return (emb ? EMB_NW : 0) + l * LAYER_NW; }
   char* slotp(int slot) const { return stash_base + (size_t)slot * slot_bytes; }
@@ -197,12 +205,14 @@ struct BertStage : ds_stage {
     Arena w;
     ws_scores = w.reserve(fused_attn ? (size_t)B * NH * S * 4 : (size_t)B * NH * S * S * 4);  // fused: delta
     ws_ds = fused_attn ? 0 : w.reserve(probs);
-    ws_dz2 = w.reserve(act);
-    ws_du = w.reserve(actF);
+    for (int p = 0; p < 2; ++p) {  // the operands of the weight-gradient GEMMs alternate by layer parity
+      ws_dz2[p] = w.reserve(act);
+      ws_du[p] = w.reserve(actF);
+      ws_dz1[p] = w.reserve(act);
+      ws_dqkv[p] = w.reserve(3 * act);
+    }
     ws_da = w.reserve(act);
-    ws_dz1 = w.reserve(act);
     ws_dctx = w.reserve(act);
-    ws_dqkv = w.reserve(3 * act);
     ws_dx[0] = w.reserve(act);
     ws_dx[1] = w.reserve(act);
     ws_bytes = w.used;
@@ -351,31 +361,39 @@ struct BertStage : ds_stage {
     char* sp = slotp(slot);
     const float scale = 1.0f / sqrtf((float)D);
     const char* dy = (const char*)d_out;
+    // With a weight-gradient stream the wgrad GEMMs and bias column sums of a layer run beside the
+    // dgrad chain of the layers below it: they only feed the master gradients.
+    hipStream_t ws = wgrad_stream;
+    if (ws && !ev_ready[0]) {
+      for (int p = 0; p < 2; ++p) {
+        DS_CHECK_HIP(hipEventCreateWithFlags(&ev_ready[p], hipEventDisableTiming));
+        DS_CHECK_HIP(hipEventCreateWithFlags(&ev_done[p], hipEventDisableTiming));
+      }
+    }
     for (int l = L - 1; l >= 0; --l) {
       const LayerStash& t = ls[l];
       const int b = base(l);
-      char* dz2 = ws_base + ws_dz2;
-      char* du = ws_base + ws_du;
+      const int par = l & 1;
+      char* dz2 = ws_base + ws_dz2[par];
+      char* du = ws_base + ws_du[par];
       char* da = ws_base + ws_da;
-      char* dz1 = ws_base + ws_dz1;
+      char* dz1 = ws_base + ws_dz1[par];
       char* dctx = ws_base + ws_dctx;
-      char* dqkv = ws_base + ws_dqkv;
+      char* dqkv = ws_base + ws_dqkv[par];
       float* dp = (float*)(ws_base + ws_scores);
       char* dsm = ws_base + ws_ds;
+      // the wgrads that read this parity's buffers two layers up must have run
+      if (ws && done_valid[par]) DS_CHECK_HIP(hipStreamWaitEvent(stream, ev_done[par], 0));
       // output LayerNorm; the column sums of dz2 are the gradient of output/dense/bias
       DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, dy, sp + t.z2, w[b + LN2_G], (const float*)(sp + t.st2), nullptr, dz2,
                                     g[b + LN2_G], g[b + LN2_B], g[b + B_FF2], stream));
-      DS_PROPAGATE(gemm_wgrad(rows, H, F, sp + t.h, F, dz2, H, g[b + W_FF2], H));
       // du = (dz2 W2^T) * gelu'(u)
       DS_PROPAGATE(gemm_dgrad(rows, H, F, dz2, weight_T(l, W_FF2), du, DS_EPI_DGELU, nullptr, sp + t.u));
-      DS_PROPAGATE(ds_colsum_accum(dtype, rows, F, du, F, g[b + B_FF1], stream));
-      DS_PROPAGATE(gemm_wgrad(rows, F, H, sp + t.a, H, du, F, g[b + W_FF1], F));
       // da = du W1^T + dz2 (a also feeds the residual into z2)
       DS_PROPAGATE(gemm_dgrad(rows, F, H, du, weight_T(l, W_FF1), da, DS_EPI_RESIDUAL, dz2, nullptr));
       // attention-output LayerNorm; column sums of dz1 = gradient of attention/output/dense/bias
       DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, da, sp + t.z1, w[b + LN1_G], (const float*)(sp + t.st1), nullptr, dz1,
                                     g[b + LN1_G], g[b + LN1_B], g[b + B_AO], stream));
-      DS_PROPAGATE(gemm_wgrad(rows, H, H, sp + t.ctx, H, dz1, H, g[b + W_AO], H));
       DS_PROPAGATE(gemm_dgrad(rows, H, H, dz1, weight_T(l, W_AO), dctx, 0, nullptr, nullptr));
       // attention backward per (batch, head)
       const char* q = sp + t.qkv;
@@ -400,25 +418,45 @@ struct BertStage : ds_stage {
       DS_PROPAGATE(gemm_heads(DS_MN_MAJOR, DS_MN_MAJOR, S, D, S, dsm, S, soP, siP, q, 3 * H, so3, D,
                               dqkv + (size_t)H * esz, 3 * H, so3, D, 0));
       }
-      // projection gradients: three [H,H] kernels and three biases fed by the columns of dqkv
-      const bool adjacent = g[b + B_K] == g[b + B_Q] + H && g[b + B_V] == g[b + B_Q] + 2 * H &&
-                            g[b + W_K] == g[b + W_Q] + (size_t)H * H && g[b + W_V] == g[b + W_Q] + (size_t)2 * H * H;
-      if (adjacent) {
-        // q, k, v master gradients lie back to back: one column sum over [rows, 3H] and one GEMM batched
-        // over the three column blocks of dqkv
-        DS_PROPAGATE(ds_colsum_accum(dtype, rows, 3 * H, dqkv, 3 * H, g[b + B_Q], stream));
-        ds_gemm_desc d;
-        memset(&d, 0, sizeof(d));
-        d.dtype = dtype; d.a_major = DS_MN_MAJOR; d.b_major = DS_MN_MAJOR;
-        d.m = H; d.n = H; d.k = rows; d.lda = H; d.ldb = 3 * H; d.ldc = H; d.batch = 3; d.batch_inner = 3;
-        d.b_stride_inner = H; d.c_stride_inner = (int64_t)H * H;
-        d.flags = DS_EPI_ACCUM; d.alpha = 1.f; d.a = sp + t.x; d.b = dqkv; d.c = g[b + W_Q];
-        DS_PROPAGATE(ds_gemm(&d, stream));
-      } else {
-        for (int j = 0; j < 3; ++j) {
-          DS_PROPAGATE(ds_colsum_accum(dtype, rows, H, dqkv + (size_t)j * H * esz, 3 * H, g[b + B_Q + j], stream));
-          DS_PROPAGATE(gemm_wgrad(rows, H, H, sp + t.x, H, dqkv + (size_t)j * H * esz, 3 * H, g[b + W_Q + j], H));
+      // ---- weight gradients of this layer (on the weight-gradient stream when there is one)
+      hipStream_t chain = stream;
+      if (ws) {
+        DS_CHECK_HIP(hipEventRecord(ev_ready[par], chain));
+        DS_CHECK_HIP(hipStreamWaitEvent(ws, ev_ready[par], 0));
+        stream = ws;  // gemm_wgrad and the column sums below launch on `stream`
+      }
+      int rc = DS_OK;
+      do {
+        if ((rc = gemm_wgrad(rows, H, F, sp + t.h, F, dz2, H, g[b + W_FF2], H)) != DS_OK) break;
+        if ((rc = ds_colsum_accum(dtype, rows, F, du, F, g[b + B_FF1], stream)) != DS_OK) break;
+        if ((rc = gemm_wgrad(rows, F, H, sp + t.a, H, du, F, g[b + W_FF1], F)) != DS_OK) break;
+        if ((rc = gemm_wgrad(rows, H, H, sp + t.ctx, H, dz1, H, g[b + W_AO], H)) != DS_OK) break;
+        // projection gradients: three [H,H] kernels and three biases fed by the columns of dqkv
+        const bool adjacent = g[b + B_K] == g[b + B_Q] + H && g[b + B_V] == g[b + B_Q] + 2 * H &&
+                              g[b + W_K] == g[b + W_Q] + (size_t)H * H && g[b + W_V] == g[b + W_Q] + (size_t)2 * H * H;
+        if (adjacent) {
+          // q, k, v master gradients lie back to back: one column sum over [rows, 3H] and one GEMM batched
+          // over the three column blocks of dqkv
+          if ((rc = ds_colsum_accum(dtype, rows, 3 * H, dqkv, 3 * H, g[b + B_Q], stream)) != DS_OK) break;
+          ds_gemm_desc d;
+          memset(&d, 0, sizeof(d));
+          d.dtype = dtype; d.a_major = DS_MN_MAJOR; d.b_major = DS_MN_MAJOR;
+          d.m = H; d.n = H; d.k = rows; d.lda = H; d.ldb = 3 * H; d.ldc = H; d.batch = 3; d.batch_inner = 3;
+          d.b_stride_inner = H; d.c_stride_inner = (int64_t)H * H;
+          d.flags = DS_EPI_ACCUM; d.alpha = 1.f; d.a = sp + t.x; d.b = dqkv; d.c = g[b + W_Q];
+          if ((rc = ds_gemm(&d, stream)) != DS_OK) break;
+        } else {
+          for (int j = 0; j < 3 && rc == DS_OK; ++j) {
+            rc = ds_colsum_accum(dtype, rows, H, dqkv + (size_t)j * H * esz, 3 * H, g[b + B_Q + j], stream);
+            if (rc == DS_OK) rc = gemm_wgrad(rows, H, H, sp + t.x, H, dqkv + (size_t)j * H * esz, 3 * H, g[b + W_Q + j], H);
+          }
         }
+      } while (0);
+      stream = chain;
+      if (rc != DS_OK) return rc;
+      if (ws) {
+        DS_CHECK_HIP(hipEventRecord(ev_done[par], ws));
+        done_valid[par] = true;
       }
       // dx = dqkv Wqkv^T + dz1 (x also feeds the residual into z1)
       const bool first = (l == 0);
@@ -427,9 +465,13 @@ struct BertStage : ds_stage {
       DS_PROPAGATE(gemm_dgrad(rows, 3 * H, H, dqkv, wqkv[l], dx, DS_EPI_RESIDUAL, dz1, nullptr));
       dy = dx;
     }
+    // the stash slot and the master gradients are released to the caller in the order of `stream`
+    if (ws)
+      for (int p = 0; p < 2; ++p)
+        if (done_valid[p]) DS_CHECK_HIP(hipStreamWaitEvent(stream, ev_done[p], 0));
     if (emb) {
       // embedding LayerNorm backward, then scatter-add into the three tables
-      char* de = ws_base + ws_dz2;
+      char* de = ws_base + ws_dz2[0];
       DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, dy, sp + emb_e, w[E_LN_G], (const float*)(sp + emb_st), nullptr, de,
                                     g[E_LN_G], g[E_LN_B], nullptr, stream));
       const int32_t* tt = slot_has_tt[slot] ? (const int32_t*)(sp + emb_tt) : nullptr;

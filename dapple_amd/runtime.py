@@ -139,9 +139,9 @@ class Stage:
     def overlap_supported(self):
         return bool(self.lib.ds_stage_overlap_supported(self._h))
 
-    def enable_overlap(self):
-        check(self.lib.ds_stage_enable_overlap(self._h), "ds_stage_enable_overlap")
-        self.overlap = True
+    def enable_overlap(self, on=True):
+        check(self.lib.ds_stage_enable_overlap(self._h, 1 if on else 0), "ds_stage_enable_overlap")
+        self.overlap = bool(on)
 
     def join(self):
         """Orders queued backward work before whatever is queued next on the stage's stream."""

@@ -192,14 +192,16 @@ int ds_stage_sync(ds_stage* h);
  * passes of different micro-batches to TensorFlow's inter-op scheduler: only the control
  * dependencies of bert/graph.py:126-132 constrain it (256 inter-op threads,
  * bert/train_flags.py:183-186), so F(j+K) and B(j+1) may run at the same time.
- * ds_stage_enable_overlap puts the backward passes on a second stream owned by the handle (default
- * priority); per-slot events keep B(slot) after F(slot) and the next F(slot) after B(slot).
+ * ds_stage_enable_overlap(h, 1) puts the backward passes on a second stream owned by the handle and
+ * their weight-gradient GEMMs on a third (default priority); per-slot events keep B(slot) after
+ * F(slot) and the next F(slot) after B(slot); (h, 0) returns to one stream (no micro-batch may be
+ * in flight for either call).
  * ds_stage_join orders all queued backward work before what is queued next on the stage's stream
  * (call it at the end of a step, before reading gradients on that stream); ds_stage_sync and
  * ds_stage_refresh_weights join by themselves.  Stages whose forward and backward passes share
  * workspace report 0 from ds_stage_overlap_supported and DS_EINVAL from ds_stage_enable_overlap. */
 int ds_stage_overlap_supported(const ds_stage* h);
-int ds_stage_enable_overlap(ds_stage* h);
+int ds_stage_enable_overlap(ds_stage* h, int on);
 int ds_stage_join(ds_stage* h);
 
 /* ---------------------------------------------------------------------------

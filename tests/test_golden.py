@@ -22,12 +22,26 @@ def load(name):
     return z, meta, w, g
 
 
+def _floors(g):
+    """Gradients that are zero in exact arithmetic (softmax is invariant to the key bias; one-segment
+    XLNet inputs never touch the segment terms) hold only rounding noise: compare them on the scale of
+    their non-degenerate sibling."""
+    fl = {}
+    for k in g:
+        if k.endswith("/key/bias"):
+            fl[k] = float(np.abs(g[k.replace("/key/", "/query/")]).max())
+        if k.endswith("/bias_segment") or k.endswith("/seg_emb"):
+            fl[k] = float(np.abs(g[k.rsplit("/", 1)[0] + "/bias_context"]).max())
+    return fl
+
+
 def _check(acc, g, outs, z, tol):
     for m, o in enumerate(outs):
         assert_close(o, z["out_%d" % m], tol, "output mb%d" % m)
     assert set(acc) == set(g)
+    fl = _floors(g)
     for k in g:
-        assert_close(acc[k].reshape(g[k].shape), g[k], tol, "grad " + k)
+        assert_close(acc[k].reshape(g[k].shape), g[k], tol, "grad " + k, floor=fl.get(k))
 
 
 def _sum(acc, dw):
