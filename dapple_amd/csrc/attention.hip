@@ -23,6 +23,13 @@ typedef __attribute__((address_space(1))) void* glb_vptr;
 constexpr int HD = 64;        // head size
 constexpr int ROWB = 128;     // bytes per tile row (64 bf16)
 constexpr int CHUNK = 512;    // rows of K/V (or Q/dO) resident in LDS at a time
+// A block owns 64 rows of the parallel axis (two groups of 32) and splits the walked axis SPLIT ways:
+// wave w works for group (w & 1) on every SPLIT-th 32-row step starting at (w >> 1).  2*SPLIT waves
+// give every SIMD two waves, so one wave's softmax arithmetic runs under the other's MFMAs.  The
+// partial results are combined through LDS at the end.
+constexpr int SPLIT = 4;
+constexpr int NWAVES = 2 * SPLIT;
+constexpr int NTHREADS = 64 * NWAVES;
 
 // LDS tile layout: row-major [row][64 bf16], the 16-byte chunk index XOR-swizzled by the row.  The
 // LDS has 64 banks (a 256-byte line = two tile rows).  The swizzle serves both read patterns:
@@ -39,9 +46,9 @@ __device__ __forceinline__ int tile_off(int row, int byte) {
   return row * ROWB + ((((byte >> 4) ^ tile_swz(row))) << 4) + (byte & 15);
 }
 
-// Fills `rows` tile rows (multiple of 16) from global rows of stride ld (elements); 128 threads.
+// Fills `rows` tile rows (multiple of 16) from global rows of stride ld (elements); all waves of the block.
 __device__ __forceinline__ void tile_fill(char* lds, const bf16* src, int64_t ld, int rows, int wave, int lane) {
-  for (int c = wave; c < rows / 8; c += 2) {  // each call: one wave writes 64 consecutive 16-byte slots = 8 rows
+  for (int c = wave; c < rows / 8; c += NWAVES) {  // each call: one wave writes 64 consecutive 16-byte slots = 8 rows
     const int p = c * 64 + lane;
     const int r = p >> 3, pc = p & 7;
     const bf16* s = src + (int64_t)r * ld + (pc ^ tile_swz(r)) * 8;
@@ -99,18 +106,53 @@ __device__ __forceinline__ void store_t(bf16* out_row, const f32x16 (&acc)[2], f
     }
 }
 
+// Partial accumulators of one wave parked in LDS: piece (i, g) of lane l at ((i*4+g)*64 + l)*16, then
+// two floats per lane.  PART_BYTES covers up to 4 accumulators.
+constexpr int PART_BYTES = 64 * (4 * 64 + 16);
+template <int NACC>
+__device__ __forceinline__ void part_store(char* slot, const f32x16 (&acc)[NACC], int lane) {
+#pragma unroll
+  for (int i = 0; i < NACC; ++i)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      f32x4 v = {acc[i][4 * g], acc[i][4 * g + 1], acc[i][4 * g + 2], acc[i][4 * g + 3]};
+      *reinterpret_cast<f32x4*>(slot + ((i * 4 + g) * 64 + lane) * 16) = v;
+    }
+}
+__device__ __forceinline__ void part_store_xy(char* slot, float x, float y, int lane) {
+  float* xy = reinterpret_cast<float*>(slot + 4 * 4 * 64 * 16) + lane * 2;
+  xy[0] = x; xy[1] = y;
+}
+// acc = acc * wa + parked * wb
+template <int NACC>
+__device__ __forceinline__ void part_merge(const char* slot, f32x16 (&acc)[NACC], float wa, float wb, int lane) {
+#pragma unroll
+  for (int i = 0; i < NACC; ++i)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const f32x4 v = *reinterpret_cast<const f32x4*>(slot + ((i * 4 + g) * 64 + lane) * 16);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][4 * g + j] = acc[i][4 * g + j] * wa + v[j] * wb;
+    }
+}
+__device__ __forceinline__ void part_xy(const char* slot, float& x, float& y, int lane) {
+  const float* xy = reinterpret_cast<const float*>(slot + 4 * 4 * 64 * 16) + lane * 2;
+  x = xy[0]; y = xy[1];
+}
+
 // ----------------------------------------------------------------------------------- forward
-// grid (S/64, B*N), 128 threads: each wave owns 32 queries, walks all keys.
-__global__ __launch_bounds__(128) void attn_fwd_kernel(AttnArgs a) {
+// grid (S/64, B*N): each wave owns 32 queries and every SPLIT-th 32-key step.
+__global__ __launch_bounds__(NTHREADS) void attn_fwd_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5;
+  const int grp = wave & 1, part = wave >> 1;
   const int b = blockIdx.y / a.N, hd = blockIdx.y % a.N;
-  const int q = blockIdx.x * 64 + wave * 32 + (lane & 31);
+  const int q = blockIdx.x * 64 + grp * 32 + (lane & 31);
   const bf16* base = a.qkv + (int64_t)b * a.S * a.ld + hd * HD;
   char* sk = lds;
   char* sv = lds + CHUNK * ROWB;
   float* adder = reinterpret_cast<float*>(lds + 2 * CHUNK * ROWB);
-  for (int j = threadIdx.x; j < a.S; j += 128)
+  for (int j = threadIdx.x; j < a.S; j += NTHREADS)
     adder[j] = a.key_mask ? (1.0f - a.key_mask[(int64_t)b * a.S + j]) * a.mask_value : 0.f;
   bf16x8 qf[4];
 #pragma unroll
@@ -126,7 +168,7 @@ __global__ __launch_bounds__(128) void attn_fwd_kernel(AttnArgs a) {
     tile_fill(sv, base + 2 * a.H + (int64_t)k0 * a.ld, a.ld, rows, wave, lane);
     __builtin_amdgcn_s_waitcnt(VMCNT0);
     __syncthreads();
-    for (int kt = 0; kt < rows; kt += 32) {
+    for (int kt = part * 32; kt < rows; kt += 32 * SPLIT) {
       f32x16 s;
 #pragma unroll
       for (int e = 0; e < 16; ++e) s[e] = 0.f;
@@ -157,23 +199,44 @@ __global__ __launch_bounds__(128) void attn_fwd_kernel(AttnArgs a) {
       }
     }
   }
+  // combine the SPLIT partial softmaxes of each query group (part 0 always saw key step 0: m is finite)
+  __syncthreads();
+  if (part > 0) {
+    part_store<2>(lds + ((part - 1) * 2 + grp) * PART_BYTES, o, lane);
+    part_store_xy(lds + ((part - 1) * 2 + grp) * PART_BYTES, m, l, lane);
+  }
+  __syncthreads();
+  if (part > 0) return;
+#pragma unroll
+  for (int pp = 1; pp < SPLIT; ++pp) {
+    const char* slot = lds + ((pp - 1) * 2 + grp) * PART_BYTES;
+    float mp, lp;
+    part_xy(slot, mp, lp, lane);
+    const float mn = fmaxf(m, mp);
+    const float wa = __expf(m - mn), wb = __expf(mp - mn);
+    part_merge<2>(slot, o, wa, wb, lane);
+    l = l * wa + lp * wb;
+    m = mn;
+  }
   l += __shfl_xor(l, 32, 64);
   store_t(a.ctx + ((int64_t)b * a.S + q) * a.H + hd * HD, o, 1.0f / l, half);
   if (half == 0) a.lse[((int64_t)b * a.N + hd) * a.S + q] = m + __logf(l);
 }
 
 // ----------------------------------------------------------------------------------- backward: dQ
-// grid (S/64, B*N), 128 threads: each wave owns 32 queries.  Also writes delta[q] = sum_d dO[q,d] O[q,d].
-__global__ __launch_bounds__(128) void attn_bwd_dq_kernel(AttnArgs a) {
+// grid (S/64, B*N): each wave owns 32 queries and every SPLIT-th 32-key step.  Also writes
+// delta[q] = sum_d dO[q,d] O[q,d].
+__global__ __launch_bounds__(NTHREADS) void attn_bwd_dq_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5;
+  const int grp = wave & 1, part = wave >> 1;
   const int b = blockIdx.y / a.N, hd = blockIdx.y % a.N;
-  const int q = blockIdx.x * 64 + wave * 32 + (lane & 31);
+  const int q = blockIdx.x * 64 + grp * 32 + (lane & 31);
   const bf16* base = a.qkv + (int64_t)b * a.S * a.ld + hd * HD;
   char* sk = lds;
   char* sv = lds + CHUNK * ROWB;
   float* adder = reinterpret_cast<float*>(lds + 2 * CHUNK * ROWB);
-  for (int j = threadIdx.x; j < a.S; j += 128)
+  for (int j = threadIdx.x; j < a.S; j += NTHREADS)
     adder[j] = a.key_mask ? (1.0f - a.key_mask[(int64_t)b * a.S + j]) * a.mask_value : 0.f;
   bf16x8 qf[4], dof[4];
   float delta = 0.f;
@@ -188,7 +251,7 @@ __global__ __launch_bounds__(128) void attn_bwd_dq_kernel(AttnArgs a) {
   }
   delta += __shfl_xor(delta, 32, 64);
   const float lse = a.lse[((int64_t)b * a.N + hd) * a.S + q];
-  if (half == 0) a.delta[((int64_t)b * a.N + hd) * a.S + q] = delta;
+  if (half == 0 && part == 0) a.delta[((int64_t)b * a.N + hd) * a.S + q] = delta;
   f32x16 dq[2];
 #pragma unroll
   for (int e = 0; e < 16; ++e) { dq[0][e] = 0.f; dq[1][e] = 0.f; }
@@ -199,7 +262,7 @@ __global__ __launch_bounds__(128) void attn_bwd_dq_kernel(AttnArgs a) {
     tile_fill(sv, base + 2 * a.H + (int64_t)k0 * a.ld, a.ld, rows, wave, lane);
     __builtin_amdgcn_s_waitcnt(VMCNT0);
     __syncthreads();
-    for (int kt = 0; kt < rows; kt += 32) {
+    for (int kt = part * 32; kt < rows; kt += 32 * SPLIT) {
       f32x16 s, dp;
 #pragma unroll
       for (int e = 0; e < 16; ++e) { s[e] = 0.f; dp[e] = 0.f; }
@@ -222,23 +285,30 @@ __global__ __launch_bounds__(128) void attn_bwd_dq_kernel(AttnArgs a) {
       }
     }
   }
+  __syncthreads();
+  if (part > 0) part_store<2>(lds + ((part - 1) * 2 + grp) * PART_BYTES, dq, lane);
+  __syncthreads();
+  if (part > 0) return;
+#pragma unroll
+  for (int pp = 1; pp < SPLIT; ++pp) part_merge<2>(lds + ((pp - 1) * 2 + grp) * PART_BYTES, dq, 1.f, 1.f, lane);
   store_t(a.dqkv + ((int64_t)b * a.S + q) * a.ld + hd * HD, dq, 1.0f, half);
 }
 
 // ----------------------------------------------------------------------------------- backward: dK, dV
-// grid (S/64, B*N), 128 threads: each wave owns 32 keys, walks all queries (Q and dO tiles in LDS).
-__global__ __launch_bounds__(128) void attn_bwd_dkv_kernel(AttnArgs a) {
+// grid (S/64, B*N): each wave owns 32 keys and every SPLIT-th 32-query step (Q and dO tiles in LDS).
+__global__ __launch_bounds__(NTHREADS) void attn_bwd_dkv_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5;
+  const int grp = wave & 1, part = wave >> 1;
   const int b = blockIdx.y / a.N, hd = blockIdx.y % a.N;
-  const int key = blockIdx.x * 64 + wave * 32 + (lane & 31);
+  const int key = blockIdx.x * 64 + grp * 32 + (lane & 31);
   const bf16* base = a.qkv + (int64_t)b * a.S * a.ld + hd * HD;
   const bf16* dobase = a.dctx + (int64_t)b * a.S * a.H + hd * HD;
   char* sq = lds;
   char* sdo = lds + CHUNK * ROWB;
   float* slse = reinterpret_cast<float*>(lds + 2 * CHUNK * ROWB);
   float* sdelta = slse + a.S;
-  for (int j = threadIdx.x; j < a.S; j += 128) {
+  for (int j = threadIdx.x; j < a.S; j += NTHREADS) {
     slse[j] = a.lse[((int64_t)b * a.N + hd) * a.S + j];
     sdelta[j] = a.delta[((int64_t)b * a.N + hd) * a.S + j];
   }
@@ -259,7 +329,7 @@ __global__ __launch_bounds__(128) void attn_bwd_dkv_kernel(AttnArgs a) {
     tile_fill(sdo, dobase + (int64_t)q0 * a.H, a.H, rows, wave, lane);
     __builtin_amdgcn_s_waitcnt(VMCNT0);
     __syncthreads();
-    for (int qt = 0; qt < rows; qt += 32) {
+    for (int qt = part * 32; qt < rows; qt += 32 * SPLIT) {
       f32x16 s, dp;
 #pragma unroll
       for (int e = 0; e < 16; ++e) { s[e] = 0.f; dp[e] = 0.f; }
@@ -285,6 +355,20 @@ __global__ __launch_bounds__(128) void attn_bwd_dkv_kernel(AttnArgs a) {
         }
       }
     }
+  }
+  __syncthreads();
+  if (part > 0) {
+    char* slot = lds + ((part - 1) * 2 + grp) * PART_BYTES;
+    part_store<2>(slot, dk, lane);
+    part_store<2>(slot + 2 * 4 * 64 * 16, dv, lane);
+  }
+  __syncthreads();
+  if (part > 0) return;
+#pragma unroll
+  for (int pp = 1; pp < SPLIT; ++pp) {
+    const char* slot = lds + ((pp - 1) * 2 + grp) * PART_BYTES;
+    part_merge<2>(slot, dk, 1.f, 1.f, lane);
+    part_merge<2>(slot + 2 * 4 * 64 * 16, dv, 1.f, 1.f, lane);
   }
   bf16* orow = a.dqkv + ((int64_t)b * a.S + key) * a.ld + hd * HD;
   store_t(orow + a.H, dk, 1.0f, half);
@@ -317,7 +401,7 @@ extern "C" int ds_attention_fwd(int dtype, int batch, int heads, int seq, int he
   }
   hipStream_t s = (hipStream_t)stream;
   ds_prof_scope prof(s, "attn_fwd_kernel", 4.0 * batch * heads * (double)seq * seq * head_dim, "FLOP");
-  hipLaunchKernelGGL(attn_fwd_kernel, dim3(seq / 64, batch * heads), dim3(128), lds_bytes(seq), s, a);
+  hipLaunchKernelGGL(attn_fwd_kernel, dim3(seq / 64, batch * heads), dim3(NTHREADS), lds_bytes(seq), s, a);
   DS_CHECK_LAUNCH();
   return DS_OK;
 }
@@ -342,12 +426,12 @@ extern "C" int ds_attention_bwd(int dtype, int batch, int heads, int seq, int he
   hipStream_t s = (hipStream_t)stream;
   {
     ds_prof_scope prof(s, "attn_bwd_dq_kernel", 6.0 * batch * heads * (double)seq * seq * head_dim, "FLOP");
-    hipLaunchKernelGGL(attn_bwd_dq_kernel, dim3(seq / 64, batch * heads), dim3(128), lds_bytes(seq), s, a);
+    hipLaunchKernelGGL(attn_bwd_dq_kernel, dim3(seq / 64, batch * heads), dim3(NTHREADS), lds_bytes(seq), s, a);
     DS_CHECK_LAUNCH();
   }
   {
     ds_prof_scope prof(s, "attn_bwd_dkv_kernel", 8.0 * batch * heads * (double)seq * seq * head_dim, "FLOP");
-    hipLaunchKernelGGL(attn_bwd_dkv_kernel, dim3(seq / 64, batch * heads), dim3(128), lds_bytes(seq), s, a);
+    hipLaunchKernelGGL(attn_bwd_dkv_kernel, dim3(seq / 64, batch * heads), dim3(NTHREADS), lds_bytes(seq), s, a);
     DS_CHECK_LAUNCH();
   }
   return DS_OK;
