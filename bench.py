@@ -201,6 +201,14 @@ def make_xlnet(c, args):
     return wl
 
 
+# HBM bytes per launch from rocprofv3 --pmc runs (counters cannot be read from inside this process)
+TRAFFIC_SOURCE = "profiles/gemm_bert48_layer_hbm_traffic.txt"
+TRAFFIC = {
+    "gemm_dma_kernel<bf16,128,128,MN,MN>": 59.0e6,   # ffn weight-gradient shape: 42.2 MB read + 16.8 MB written
+    "gemm_dma_kernel<bf16,128,128,K,MN>": 33.9e6,    # ffn1 forward shape
+    "gemm_dma_kernel<bf16,128,128,K,K>": 33.8e6,     # ffn2 dgrad shape
+}
+
 MAKERS = {"bert": make_bert, "vgg": make_vgg, "gnmt": make_gnmt, "xlnet": make_xlnet}
 METRIC = {"bert48_half": "stage samples/sec fwd+bwd+grad-accum, BERT-48 half-stage; MFMA util %"}
 
@@ -263,7 +271,9 @@ def main():
     else:
         roof = {"bound": "hbm", "achieved": work / (ms * 1e-3) / 1e9, "peak": PEAK["hbm"] / 1e9, "unit": "GB/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["traffic"] = None
+    roof["traffic"] = TRAFFIC.get(dom)
+    if roof["traffic"] is not None:
+        roof["traffic_unit"] = "bytes per launch (FETCH_SIZE + WRITE_SIZE, scaled by a known-traffic kernel), see " + TRAFFIC_SOURCE
     roof.update({"kernel": dom, "launches": n, "avg_launch_us": ms * 1e3 / n, "share_of_kernel_time": ms / total_ms})
     if iso is not None and dom in iso:
         n2, ms2, work2, _ = iso[dom]

@@ -1,0 +1,52 @@
+"""Small fixed launches for hardware-counter runs.
+
+``accumulate N``: ``ds_grad_accumulate`` over N fp32 elements - known traffic (reads 8*N bytes, writes
+4*N bytes), used to scale the FETCH_SIZE / WRITE_SIZE counters.
+``gemms``: the GEMMs of one BERT-48 half-stage layer at their real shapes (2x512 rows, hidden 1024,
+ffn 4096, bf16), three launches each, so a counter run can report HBM traffic per launch.
+
+    rocprofv3 --pmc FETCH_SIZE --output-format csv -d out -o c -- python3 -m dapple_amd.calib accumulate 67108864
+    rocprofv3 --pmc FETCH_SIZE --output-format csv -d out -o g -- python3 -m dapple_amd.calib gemms
+"""
+import sys
+
+import torch
+
+from . import ops
+from ._lib import DS_EPI_ACCUM, DS_K_MAJOR, DS_MN_MAJOR
+
+
+def accumulate(n):
+    acc = torch.zeros(n, device="cuda")
+    g = torch.ones(n, device="cuda")
+    for _ in range(3):
+        ops.grad_accumulate(acc, g)
+    torch.cuda.synchronize()
+    print("accumulate_kernel<float>: %d elements, reads %d bytes, writes %d bytes per launch" % (n, 8 * n, 4 * n))
+
+
+def gemms():
+    rows, h, f = 1024, 1024, 4096
+    bf = torch.bfloat16
+    shapes = [  # name, m, n, k, a_major, b_major, accumulate
+        ("fwd ffn1", rows, f, h, DS_K_MAJOR, DS_MN_MAJOR, False),
+        ("fwd ffn2", rows, h, f, DS_K_MAJOR, DS_MN_MAJOR, False),
+        ("dgrad ffn2", rows, f, h, DS_K_MAJOR, DS_K_MAJOR, False),
+        ("wgrad ffn1", h, f, rows, DS_MN_MAJOR, DS_MN_MAJOR, True),
+    ]
+    for name, m, n, k, am, bm, acc in shapes:
+        a = torch.randn((m, k) if am == DS_K_MAJOR else (k, m), device="cuda").to(bf)
+        b = torch.randn((n, k) if bm == DS_K_MAJOR else (k, n), device="cuda").to(bf)
+        c = torch.zeros(m, n, device="cuda", dtype=torch.float32 if acc else bf)
+        for _ in range(3):
+            ops.gemm(a, b, c, m, n, k, am, bm, flags=DS_EPI_ACCUM if acc else 0)
+        torch.cuda.synchronize()
+        alg = 2 * (m * k + n * k) + (8 if acc else 2) * m * n
+        print("%s: m=%d n=%d k=%d, algorithmic bytes %d" % (name, m, n, k, alg))
+
+
+if __name__ == "__main__":
+    if len(sys.argv) > 1 and sys.argv[1] == "gemms":
+        gemms()
+    else:
+        accumulate(int(sys.argv[2]) if len(sys.argv) > 2 else 1 << 26)

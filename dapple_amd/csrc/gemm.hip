@@ -52,6 +52,7 @@ struct GemmArgs {
   int splitk;
   int ktiles_per_split;
   int grid_m, grid_n;
+  int xcd_rm, xcd_cn;  // tiles per XCD as an xcd_rm x xcd_cn block of the tile grid (0: contiguous runs)
   int vec_epi;
   int conv_h, conv_w, conv_c;  // implicit 3x3 'same' convolution: extent of the gathered NHWC tensor
 };
@@ -71,6 +72,25 @@ template <int ROW_BYTES> __device__ __forceinline__ int mnmajor_swz(int r) {
 template <int ROW_BYTES> __device__ __forceinline__ int mnmajor_off(int r, int cbyte) {
   const int g = (cbyte >> 5) ^ mnmajor_swz<ROW_BYTES>(r);
   return r * ROW_BYTES + (g << 5) + (cbyte & 31);
+}
+
+// XCD-aware tile order: consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with its
+// own L2.  Every XCD gets a compact xcd_rm x xcd_cn block of the tile grid (chosen on the host to
+// minimise the operand bytes the 8 L2s fetch between them), walked M-fastest; when the grid does not
+// split that way, a contiguous run of M-fastest tile ids instead.
+__device__ __forceinline__ void xcd_tile(const GemmArgs& p, int w, int& tile_m, int& tile_n) {
+  const int xcd = w & 7, local = w >> 3;
+  if (p.xcd_rm) {
+    const int nbx = p.grid_m / p.xcd_rm;
+    tile_m = (xcd % nbx) * p.xcd_rm + local % p.xcd_rm;
+    tile_n = (xcd / nbx) * p.xcd_cn + local / p.xcd_rm;
+  } else {
+    const int tiles = p.grid_m * p.grid_n;
+    const int per = (tiles + 7) >> 3, tall = (tiles & 7) ? (tiles & 7) : 8;
+    const int tile_id = xcd < tall ? xcd * per + local : tall * per + (xcd - tall) * (per - 1) + local;
+    tile_m = tile_id % p.grid_m;
+    tile_n = tile_id / p.grid_m;
+  }
 }
 
 // One operand tile: W free indices x KT reduction elements = W*128 bytes, moved as W/32 16-byte
@@ -326,18 +346,9 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  // XCD-aware tile order: consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with
-  // its own L2.  Give every XCD a contiguous run of tile ids, and walk tile ids M-fastest, so
-  // one XCD works on a few whole columns of C tiles and re-reads only its own slice of B from L2.
-  int tile_id;
-  {
-    const int tiles = p.grid_m * p.grid_n;
-    const int w = blockIdx.x;
-    const int per = (tiles + 7) >> 3, tall = (tiles & 7) ? (tiles & 7) : 8;
-    const int xcd = w & 7, local = w >> 3;
-    tile_id = xcd < tall ? xcd * per + local : tall * per + (xcd - tall) * (per - 1) + local;
-  }
-  const int m0 = (tile_id % p.grid_m) * BM, n0 = (tile_id / p.grid_m) * BN;
+  int tile_m, tile_n;
+  xcd_tile(p, blockIdx.x, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int z = blockIdx.z / p.splitk, ks_id = blockIdx.z % p.splitk;
   const int zo = z / p.batch_inner, zi = z % p.batch_inner;
   const T* A = reinterpret_cast<const T*>(p.a) + zo * p.a_so + zi * p.a_si;
@@ -641,15 +652,9 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  int tile_id;
-  {
-    const int tiles = p.grid_m * p.grid_n;
-    const int w = blockIdx.x;
-    const int per = (tiles + 7) >> 3, tall = (tiles & 7) ? (tiles & 7) : 8;
-    const int xcd = w & 7, local = w >> 3;
-    tile_id = xcd < tall ? xcd * per + local : tall * per + (xcd - tall) * (per - 1) + local;
-  }
-  const int m0 = (tile_id % p.grid_m) * BM, n0 = (tile_id / p.grid_m) * BN;
+  int tile_m, tile_n;
+  xcd_tile(p, blockIdx.x, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int z = blockIdx.z / p.splitk, ks_id = blockIdx.z % p.splitk;
   const int zo = z / p.batch_inner, zi = z % p.batch_inner;
   const T* A = reinterpret_cast<const T*>(p.a) + zo * p.a_so + zi * p.a_si;
@@ -744,10 +749,29 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
   else gemm_epilogue<T, BM, BN>(p, acc, m0, n0, wm, wn, lane, c_off);
 }
 
+// Splits the tile grid into 8 equal rm x cn blocks, one per XCD.  An XCD's L2 fetches the A rows of
+// its rm row tiles and the B columns of its cn column tiles once: total operand traffic is
+// proportional to m * (grid_n / cn) + n * (grid_m / rm).
+static void choose_xcd_block(GemmArgs& a) {
+  a.xcd_rm = a.xcd_cn = 0;
+  const int tiles = a.grid_m * a.grid_n;
+  if (tiles % 8) return;
+  const int per = tiles / 8;
+  double best = 1e300;
+  for (int rm = 1; rm <= a.grid_m; ++rm) {
+    if (a.grid_m % rm || per % rm) continue;
+    const int cn = per / rm;
+    if (cn > a.grid_n || a.grid_n % cn) continue;
+    const double cost = (double)a.m * (a.grid_n / cn) + (double)a.n * (a.grid_m / rm);
+    if (cost < best) { best = cost; a.xcd_rm = rm; a.xcd_cn = cn; }
+  }
+}
+
 template <typename T, int BM, int BN, int AMAJ, int BMAJ>
 int launch_cfg(GemmArgs a, int batch, hipStream_t stream) {
   a.grid_m = (a.m + BM - 1) / BM;
   a.grid_n = (a.n + BN - 1) / BN;
+  choose_xcd_block(a);
   dim3 grid(a.grid_m * a.grid_n, 1, batch * a.splitk);
   if (a.k % Mma<T>::KT == 0) {
     constexpr int STAGES = 4;
@@ -889,6 +913,7 @@ template <int BM, int BN, int AMAJ, int MODE>
 int launch_conv_cfg(GemmArgs a, hipStream_t stream) {
   a.grid_m = (a.m + BM - 1) / BM;
   a.grid_n = (a.n + BN - 1) / BN;
+  choose_xcd_block(a);
   dim3 grid(a.grid_m * a.grid_n, 1, a.splitk);
   constexpr int STAGES = 4;
   constexpr size_t lds = (size_t)STAGES * (BM + BN) * 128;

@@ -1,6 +1,7 @@
 """Per-kernel summary of a rocprofv3 ``--kernel-trace`` rocpd database (``*_results.db``).
 
-    python -m dapple_amd.profsum gpurun_out/prof/bench_results.db
+    python -m dapple_amd.profsum <dir>/bench_results.db
+    python -m dapple_amd.profsum pmc <dir>/x_counter_collection.csv <kernel name substring>
 """
 import re
 import sqlite3
@@ -21,5 +22,29 @@ def summarize(path, top=40):
     return "\n".join(out)
 
 
+def pmc(path, needle):
+    """Per-dispatch average of every counter in a rocprofv3 ``--pmc ... --output-format csv`` file, over
+    the dispatches whose kernel name contains ``needle`` (counter values are summed over the rows of one
+    dispatch: rocprofv3 writes one row per counter instance)."""
+    import collections
+    import csv
+    per = collections.defaultdict(lambda: collections.defaultdict(float))
+    names = {}
+    with open(path) as f:
+        for r in csv.DictReader(f):
+            per[r["Dispatch_Id"]][r["Counter_Name"]] += float(r["Counter_Value"])
+            names[r["Dispatch_Id"]] = r["Kernel_Name"]
+    sel = [d for d in per if needle in names[d]]
+    out = ["%d dispatches matching %r" % (len(sel), needle)]
+    if sel:
+        for c in sorted(per[sel[0]]):
+            vals = [per[d][c] for d in sel]
+            out.append("%-24s avg %.1f  min %.1f  max %.1f" % (c, sum(vals) / len(vals), min(vals), max(vals)))
+    return "\n".join(out)
+
+
 if __name__ == "__main__":
-    print(summarize(sys.argv[1]))
+    if sys.argv[1] == "pmc":
+        print(pmc(sys.argv[2], sys.argv[3]))
+    else:
+        print(summarize(sys.argv[1]))
