@@ -22,7 +22,7 @@ typedef __attribute__((address_space(1))) void* glb_vptr;
 
 constexpr int HD = 64;        // head size
 constexpr int ROWB = 128;     // bytes per tile row (64 bf16)
-constexpr int CHUNK = 512;    // rows of K/V (or Q/dO) resident in LDS at a time
+constexpr int CHUNK = 256;    // rows of K/V (or Q/dO) resident in LDS at a time
 // A block owns 64 rows of the parallel axis (two groups of 32) and splits the walked axis SPLIT ways:
 // wave w works for group (w & 1) on every SPLIT-th 32-row step starting at (w >> 1).  2*SPLIT waves
 // give every SIMD two waves, so one wave's softmax arithmetic runs under the other's MFMAs.  The
@@ -107,8 +107,10 @@ __device__ __forceinline__ void store_t(bf16* out_row, const f32x16 (&acc)[2], f
 }
 
 // Partial accumulators of one wave parked in LDS: piece (i, g) of lane l at ((i*4+g)*64 + l)*16, then
-// two floats per lane.  PART_BYTES covers up to 4 accumulators.
-constexpr int PART_BYTES = 64 * (4 * 64 + 16);
+// two floats per lane.  PART_BYTES covers two accumulators; the (SPLIT-1)*2 slots overlay the K/V tiles.
+constexpr int PART_XY = 2 * 4 * 64 * 16;
+constexpr int PART_BYTES = PART_XY + 64 * 16;
+static_assert((SPLIT - 1) * 2 * PART_BYTES <= 2 * CHUNK * ROWB, "merge slots must fit in the tile region");
 template <int NACC>
 __device__ __forceinline__ void part_store(char* slot, const f32x16 (&acc)[NACC], int lane) {
 #pragma unroll
@@ -120,7 +122,7 @@ __device__ __forceinline__ void part_store(char* slot, const f32x16 (&acc)[NACC]
     }
 }
 __device__ __forceinline__ void part_store_xy(char* slot, float x, float y, int lane) {
-  float* xy = reinterpret_cast<float*>(slot + 4 * 4 * 64 * 16) + lane * 2;
+  float* xy = reinterpret_cast<float*>(slot + PART_XY) + lane * 2;
   xy[0] = x; xy[1] = y;
 }
 // acc = acc * wa + parked * wb
@@ -136,7 +138,7 @@ __device__ __forceinline__ void part_merge(const char* slot, f32x16 (&acc)[NACC]
     }
 }
 __device__ __forceinline__ void part_xy(const char* slot, float& x, float& y, int lane) {
-  const float* xy = reinterpret_cast<const float*>(slot + 4 * 4 * 64 * 16) + lane * 2;
+  const float* xy = reinterpret_cast<const float*>(slot + PART_XY) + lane * 2;
   x = xy[0]; y = xy[1];
 }
 
@@ -356,20 +358,21 @@ __global__ __launch_bounds__(NTHREADS) void attn_bwd_dkv_kernel(AttnArgs a) {
       }
     }
   }
+  // two merge rounds through the same slots: dK, then dV
+  char* slot = lds + ((part - 1) * 2 + grp) * PART_BYTES;
   __syncthreads();
-  if (part > 0) {
-    char* slot = lds + ((part - 1) * 2 + grp) * PART_BYTES;
-    part_store<2>(slot, dk, lane);
-    part_store<2>(slot + 2 * 4 * 64 * 16, dv, lane);
+  if (part > 0) part_store<2>(slot, dk, lane);
+  __syncthreads();
+  if (part == 0) {
+#pragma unroll
+    for (int pp = 1; pp < SPLIT; ++pp) part_merge<2>(lds + ((pp - 1) * 2 + grp) * PART_BYTES, dk, 1.f, 1.f, lane);
   }
+  __syncthreads();
+  if (part > 0) part_store<2>(slot, dv, lane);
   __syncthreads();
   if (part > 0) return;
 #pragma unroll
-  for (int pp = 1; pp < SPLIT; ++pp) {
-    const char* slot = lds + ((pp - 1) * 2 + grp) * PART_BYTES;
-    part_merge<2>(slot, dk, 1.f, 1.f, lane);
-    part_merge<2>(slot + 2 * 4 * 64 * 16, dv, 1.f, 1.f, lane);
-  }
+  for (int pp = 1; pp < SPLIT; ++pp) part_merge<2>(lds + ((pp - 1) * 2 + grp) * PART_BYTES, dv, 1.f, 1.f, lane);
   bf16* orow = a.dqkv + ((int64_t)b * a.S + key) * a.ld + hd * HD;
   store_t(orow + a.H, dk, 1.0f, half);
   store_t(orow + 2 * a.H, dv, 1.0f, half);

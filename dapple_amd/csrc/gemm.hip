@@ -17,6 +17,13 @@
 
 #include "common.h"
 
+#ifndef DS_ST_BIG
+#define DS_ST_BIG 3
+#endif
+#ifndef DS_ST_SMALL
+#define DS_ST_SMALL 3
+#endif
+
 namespace {
 
 template <typename T> struct Mma;
@@ -774,7 +781,7 @@ int launch_cfg(GemmArgs a, int batch, hipStream_t stream) {
   choose_xcd_block(a);
   dim3 grid(a.grid_m * a.grid_n, 1, batch * a.splitk);
   if (a.k % Mma<T>::KT == 0) {
-    constexpr int STAGES = 4;
+    constexpr int STAGES = (BM + BN >= 256) ? DS_ST_BIG : DS_ST_SMALL;
     constexpr size_t lds = (size_t)STAGES * (BM + BN) * 128;
     static bool attr_set = false;
     if (!attr_set) {
