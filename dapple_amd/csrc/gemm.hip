@@ -17,12 +17,6 @@
 
 #include "common.h"
 
-#ifndef DS_ST_BIG
-#define DS_ST_BIG 3
-#endif
-#ifndef DS_ST_SMALL
-#define DS_ST_SMALL 3
-#endif
 
 namespace {
 
@@ -686,8 +680,16 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
   DB db;
   da.init(p, A, p.lda, m0, p.m, kt_begin, wave, lane);
   db.init(p, B, p.ldb, n0, p.n, kt_begin, wave, lane);
+  // Ring of STAGES tile buffers, tile t in buffer t % STAGES.  All STAGES buffers are filled up front.
+  // Inside tile kt, before the MFMAs of its last k-step: every wave has read all of tile kt (its
+  // fragment reads are waited for), waits for its own loads of tile kt+1 and meets the others at the
+  // one barrier of the k-tile.  After it, tile kt+1 is visible, its first fragments are fetched under
+  // the remaining MFMAs of tile kt, and buffer kt % STAGES is free: the loads of tile kt+STAGES go
+  // there, issued one at a time between the next 4*TM*TN MFMAs (last k-step of tile kt, first three of
+  // tile kt+1).  A wave stalls on a load instruction while the address unit is busy; issued as one
+  // burst those stalls would sit in front of the MFMAs instead of underneath them.
 #pragma unroll
-  for (int s = 0; s < STAGES - 1; ++s) {
+  for (int s = 0; s < STAGES; ++s) {
     if (s < nkt) {
       da.issue(lds + s * STAGE_BYTES, wave);
       db.issue(lds + s * STAGE_BYTES + A_BYTES, wave);
@@ -698,27 +700,33 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
   ra.init(wm * (BM / 2), lane);
   rb.init(wn * (BN / 2), lane);
   const uint32_t lds0 = lds_addr(lds);
-  int buf = 0;  // kt % STAGES
-  for (int kt = 0; kt < nkt; ++kt) {
-    // tile kt is complete once at most the tiles issued after it are outstanding
-    if (kt + STAGES - 2 < nkt) __builtin_amdgcn_s_waitcnt(DS_VMCNT(LPT * (STAGES - 2)));
+  constexpr int NMMA = 4 * TM * TN;   // MFMA groups per k-tile
+  constexpr int TAIL = TM * TN;       // of which the last k-step holds this many
+  RawFrag<T, AMAJ> fa[2][TM];
+  RawFrag<T, BMAJ> fb[2][TN];
+  {
+    // tile 0 is complete once only the tiles issued after it are outstanding
+    const int later = (nkt < STAGES ? nkt : STAGES) - 1;
+    if (later >= 3) __builtin_amdgcn_s_waitcnt(DS_VMCNT(LPT * 3));
+    else if (later == 2) __builtin_amdgcn_s_waitcnt(DS_VMCNT(LPT * 2));
+    else if (later == 1) __builtin_amdgcn_s_waitcnt(DS_VMCNT(LPT));
     else __builtin_amdgcn_s_waitcnt(DS_VMCNT(0));
     __builtin_amdgcn_s_barrier();
-    // The loads of tile kt+STAGES-1 are issued one at a time between the MFMAs: a wave stalls on a
-    // load instruction while the address unit is busy, and issued as one burst those stalls would
-    // sit in front of the MFMAs instead of underneath them.
-    const bool more = kt + STAGES - 1 < nkt;
-    int nb = buf + STAGES - 1;
-    if (nb >= STAGES) nb -= STAGES;
-    char* const na = lds + nb * STAGE_BYTES;
-    char* const nbp = na + A_BYTES;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) ra.read(fa[0][i], lds0, i, 0);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) rb.read(fb[0][j], lds0 + A_BYTES, j, 0);
+  }
+  int buf = 0;  // kt % STAGES
+  for (int kt = 0; kt < nkt; ++kt) {
     const uint32_t sa = lds0 + buf * STAGE_BYTES, sb = sa + A_BYTES;
-    RawFrag<T, AMAJ> fa[2][TM];
-    RawFrag<T, BMAJ> fb[2][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i) ra.read(fa[0][i], sa, i, 0);
-#pragma unroll
-    for (int j = 0; j < TN; ++j) rb.read(fb[0][j], sb, j, 0);
+    int pb = buf - 1;  // buffer of tile kt-1, being refilled with tile kt-1+STAGES
+    if (pb < 0) pb += STAGES;
+    const bool refill_prev = kt >= 1 && kt - 1 + STAGES < nkt;
+    const bool refill_cur = kt + STAGES < nkt;
+    const bool has_next = kt + 1 < nkt;
+    int nbuf = buf + 1;
+    if (nbuf == STAGES) nbuf = 0;
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
       const int cur = ks & 1, nxt = cur ^ 1;
@@ -731,26 +739,54 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
         for (int i = 0; i < TM; ++i) ra.read(fa[nxt][i], sa, i, ks + 1);
 #pragma unroll
         for (int j = 0; j < TN; ++j) rb.read(fb[nxt][j], sb, j, ks + 1);
+      } else if (has_next) {
+        // tile kt+1 is complete once only the tiles issued after it are outstanding:
+        // kt+2 .. kt-1+STAGES, as far as they exist
+        int later = nkt - (kt + 2);
+        if (later > STAGES - 2) later = STAGES - 2;
+        if (later >= 2) __builtin_amdgcn_s_waitcnt(DS_VMCNT(LPT * 2));
+        else if (later == 1) __builtin_amdgcn_s_waitcnt(DS_VMCNT(LPT));
+        else __builtin_amdgcn_s_waitcnt(DS_VMCNT(0));
+        __builtin_amdgcn_s_barrier();
+        const uint32_t na = lds0 + nbuf * STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) ra.read(fa[nxt][i], na, i, 0);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) rb.read(fb[nxt][j], na + A_BYTES, j, 0);
       }
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
           Mma<T>::mma(acc[i][j], to_frag(fa[cur][i]), to_frag(fb[cur][j]));
-          constexpr int NMMA = 4 * TM * TN;
           const int q = (ks * TM + i) * TN + j;  // compile-time after unrolling
-          if (more) {
+          if (ks < 3) {
+            // slots TAIL .. NMMA-1 of the window that refills the buffer of tile kt-1
+            if (refill_prev) {
+              char* const ra_dst = lds + pb * STAGE_BYTES;
 #pragma unroll
-            for (int l = 0; l < LPT; ++l)
-              if ((l * NMMA) / LPT == q) {
-                if (l < DA::NV) da.issue_one(na, wave, l);
-                else db.issue_one(nbp, wave, l - DA::NV);
-              }
+              for (int l = 0; l < LPT; ++l)
+                if ((l * NMMA) / LPT == q + TAIL) {
+                  if (l < DA::NV) da.issue_one(ra_dst, wave, l);
+                  else db.issue_one(ra_dst + A_BYTES, wave, l - DA::NV);
+                }
+            }
+          } else {
+            // slots 0 .. TAIL-1 of the window that refills the buffer of tile kt
+            if (refill_cur) {
+              char* const rc_dst = lds + buf * STAGE_BYTES;
+#pragma unroll
+              for (int l = 0; l < LPT; ++l)
+                if ((l * NMMA) / LPT == q - 3 * TAIL) {
+                  if (l < DA::NV) da.issue_one(rc_dst, wave, l);
+                  else db.issue_one(rc_dst + A_BYTES, wave, l - DA::NV);
+                }
+            }
           }
         }
+      if (ks == 2 && refill_prev) { da.advance(); db.advance(); }
     }
-    if (more) { da.advance(); db.advance(); }
-    if (++buf == STAGES) buf = 0;
+    buf = nbuf;
   }
   if (p.vec_epi) gemm_epilogue_staged<T, BM, BN>(p, acc, m0, n0, wm, wn, lane, tid, c_off, lds);
   else gemm_epilogue<T, BM, BN>(p, acc, m0, n0, wm, wn, lane, c_off);
@@ -781,7 +817,9 @@ int launch_cfg(GemmArgs a, int batch, hipStream_t stream) {
   choose_xcd_block(a);
   dim3 grid(a.grid_m * a.grid_n, 1, batch * a.splitk);
   if (a.k % Mma<T>::KT == 0) {
-    constexpr int STAGES = (BM + BN >= 256) ? DS_ST_BIG : DS_ST_SMALL;
+    // 3 buffers: 96 KB for a 128x128 block, 48 KB for 64x64 - a CU's 160 KB of LDS then holds blocks of two
+    // kernels at once, which measured better than a deeper ring when several streams feed the GPU
+    constexpr int STAGES = 3;
     constexpr size_t lds = (size_t)STAGES * (BM + BN) * 128;
     static bool attr_set = false;
     if (!attr_set) {
@@ -817,10 +855,11 @@ int launch_major(const GemmArgs& a, int batch, int tile, int am, int bm, hipStre
 
 }  // namespace
 
-// Picks the tile shape.  Measured on MI355X (bf16, 4-stage pipeline): one k-tile costs about 0.6 us in
-// a 128x128 block alone on its CU, 1.06 us in two co-resident 128x64 blocks and 0.45 us in two
-// co-resident 64x64 blocks; the k-loop repeats once per round of resident blocks.  Split-K is never
-// chosen: its atomic epilogue was slower than the under-filled grid on every shape tried.
+// Picks the tile shape.  Measured on MI355X (bf16, 3-buffer ring): one k-tile costs about 0.5 us in a
+// 128x128 block, and roughly in proportion to the tile's bytes below that; the k-loop repeats once
+// per round of resident blocks.  With several streams feeding the GPU the choice is flat between
+// 128x64 and 64x64 for narrow outputs; 128x128 on a grid of fewer than ~256 tiles loses.  Split-K is
+// never chosen: its atomic epilogue was slower than the under-filled grid on every shape tried.
 static void choose_tiling(int m, int n, int k, int kt, int batch, bool can_split, int* tile, int* splitk) {
   static const int bm[3] = {128, 128, 64}, bn[3] = {128, 64, 64};
   static const double slots[3] = {256, 512, 512}, t_round[3] = {0.6, 1.06, 0.45};
@@ -889,6 +928,7 @@ static int gemm_run(const ds_gemm_desc* d, int splitk_req, void* stream) {
     static const char* env_tile = getenv("DS_GEMM_TILE");
     static const char* env_split = getenv("DS_GEMM_SPLITK");
     if (env_tile) tile = atoi(env_tile) % 3;
+
     if (env_split && (f & DS_EPI_ACCUM)) splitk = atoi(env_split) > 0 ? atoi(env_split) : 1;
   }
   const int ktiles = (d->k + kt - 1) / kt;
