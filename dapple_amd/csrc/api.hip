@@ -202,7 +202,7 @@ extern "C" int ds_stage_forward(ds_stage* h, int slot, const void* in, const flo
     return DS_ESTATE;
   }
   DS_CHECK_ARG(ds_aligned16(in) && ds_aligned16(out), "ds_stage_forward: in/out must be 16-byte aligned");
-  if (h->bwd_stream && h->released_valid[slot]) DS_CHECK_HIP(hipStreamWaitEvent(h->stream, h->ev_released[slot], 0));
+  DS_PROPAGATE(ds_stage_acquire_slot(h, slot));
   const int rc = h->forward(slot, in, key_mask, out);
   if (rc == DS_OK) h->slot_forwarded[slot] = 1;
   if (rc == DS_OK && h->bwd_stream) DS_CHECK_HIP(hipEventRecord(h->ev_forwarded[slot], h->stream));

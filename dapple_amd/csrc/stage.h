@@ -51,5 +51,12 @@ struct ds_stage {
   virtual size_t stash_bytes(int slots) const = 0;
 };
 
+// With overlap on, anything that writes into a stash slot on the stage's stream must first wait for the
+// backward pass that last used the slot.
+static inline int ds_stage_acquire_slot(ds_stage* h, int slot) {
+  if (h->bwd_stream && h->released_valid[slot]) DS_CHECK_HIP(hipStreamWaitEvent(h->stream, h->ev_released[slot], 0));
+  return DS_OK;
+}
+
 int ds_bert_stage_create(const ds_stage_cfg* cfg, hipStream_t stream, ds_stage** out);
 int ds_gemm_splitk(const ds_gemm_desc* d, int splitk, void* stream);

@@ -529,5 +529,6 @@ extern "C" int ds_stage_set_token_types(ds_stage* h, int slot, const int32_t* to
   DS_CHECK_ARG(h != nullptr, "ds_stage_set_token_types: null handle");
   DS_CHECK_ARG(h->cfg.kind == DS_STAGE_BERT, "ds_stage_set_token_types: not a BERT stage");
   DS_CHECK_ARG(slot >= 0 && slot < h->cfg.stash_slots, "ds_stage_set_token_types: slot %d out of range", slot);
+  DS_PROPAGATE(ds_stage_acquire_slot(h, slot));
   return static_cast<BertStage*>(h)->set_token_types(slot, token_type_ids);
 }

@@ -176,7 +176,7 @@ struct XlnetStage : ds_stage {
   std::vector<char> has_mask, has_seg;
   // workspace
   char* ws_base = nullptr;
-  size_t ws_bytes = 0, ws_qall, ws_ac, ws_bd, ws_ds, ws_dbd, ws_dz2, ws_du, ws_dy1, ws_dz1, ws_dvec, ws_dqw, ws_dqr, ws_dqs, ws_dq,
+  size_t ws_bytes = 0, ws_qall, ws_ac, ws_dp, ws_bd, ws_ds, ws_dbd, ws_dz2, ws_du, ws_dy1, ws_dz1, ws_dvec, ws_dqw, ws_dqr, ws_dqs, ws_dq,
          ws_dkv, ws_dkr, ws_deft, ws_dx[2];
 
   ~XlnetStage() override {
@@ -250,6 +250,7 @@ struct XlnetStage : ds_stage {
     Arena w;
     ws_qall = w.reserve(act);
     ws_ac = w.reserve((size_t)B * N * Q * K * 4);
+    ws_dp = w.reserve((size_t)B * N * Q * K * 4);  // backward's own score-gradient buffer: forward keeps ws_ac
     ws_bd = w.reserve((size_t)B * N * Q * R * 4);
     ws_ds = w.reserve((size_t)B * N * Q * K * esz);
     ws_dbd = w.reserve((size_t)B * N * Q * R * esz);
@@ -265,6 +266,8 @@ struct XlnetStage : ds_stage {
   }
 
   size_t workspace_bytes() const override { return ws_bytes; }
+  // forward writes qall / ac / bd and its stash slot, backward everything else: disjoint
+  bool overlap_safe() const override { return true; }
   size_t stash_bytes(int slots) const override { return slot_bytes * (size_t)slots; }
 
   const void* WT(int l, int which) const {
@@ -413,7 +416,7 @@ struct XlnetStage : ds_stage {
     char* dz2 = ws_base + ws_dz2; char* du = ws_base + ws_du; char* dy1 = ws_base + ws_dy1; char* dz1 = ws_base + ws_dz1;
     char* dvec = ws_base + ws_dvec; char* dqw = ws_base + ws_dqw; char* dqr = ws_base + ws_dqr; char* dqs = ws_base + ws_dqs;
     char* dq = ws_base + ws_dq; char* dkv = ws_base + ws_dkv; char* dkr = ws_base + ws_dkr; char* deft = ws_base + ws_deft;
-    float* dp = (float*)(ws_base + ws_ac);
+    float* dp = (float*)(ws_base + ws_dp);
     char* dsm = ws_base + ws_ds; char* dbd = ws_base + ws_dbd;
     for (int l = L - 1; l >= 0; --l) {
       const LayerOff& t = lo[l];
@@ -547,5 +550,6 @@ extern "C" int ds_xlnet_stage_set_inputs(ds_stage* h, int slot, const float* mas
   DS_CHECK_ARG(h != nullptr, "ds_xlnet_stage_set_inputs: null handle");
   DS_CHECK_ARG(h->cfg.kind == DS_STAGE_XLNET, "ds_xlnet_stage_set_inputs: not an XLNet stage");
   DS_CHECK_ARG(slot >= 0 && slot < h->cfg.stash_slots, "ds_xlnet_stage_set_inputs: slot %d out of range", slot);
+  DS_PROPAGATE(ds_stage_acquire_slot(h, slot));
   return static_cast<XlnetStage*>(h)->set_aux(slot, masks, seg_mat, mems);
 }

@@ -14,7 +14,7 @@ ADT = {"fp32": torch.float32, "bf16": torch.bfloat16}
 
 
 def run_case(dtype, L, H, N, F, B, Q, Mm, S, M, K=2, seed=0, use_seg=True, mask_kind="perm", stddev=0.1, perturb=True,
-             odtype=torch.float64):
+             odtype=torch.float64, overlap=False):
     adt = ADT[dtype]
     klen = Mm + Q
     w_np = synthetic.xlnet_weights(synthetic.SEED_WEIGHT + seed, L, H, N, F, stddev=stddev, perturb=perturb)
@@ -33,6 +33,8 @@ def run_case(dtype, L, H, N, F, B, Q, Mm, S, M, K=2, seed=0, use_seg=True, mask_
 
     stage = runtime.xlnet_stage(L, H, N, F, B, Q, dtype, stash_slots=K, mem_len=Mm, streams=S)
     stage.bind(w_np)
+    if overlap:
+        stage.enable_overlap()     # backward passes on the handle's second stream
     xs = [dev(np.stack(x), adt) for x in xs_np]
     dys = [dev(np.stack(d), adt) for d in dys_np]
     outs = [torch.empty(S, Q, B, H, dtype=adt, device="cuda") for _ in range(M)]
@@ -89,3 +91,9 @@ def test_config4_shape_one_layer_bf16():
     c = synthetic.CONFIGS["xlnet36_half"]
     run_case("bf16", 1, c["hidden"], c["heads"], c["ffn"], c["micro_batch"], c["seq"], c["mem_len"], c["streams"], M=1, K=1,
              seed=c["index"], stddev=0.02, perturb=False, odtype=torch.float32)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_forward_backward_overlap(dtype):
+    # backward passes on the second stream, slots (and their masks / memories) reused three times over
+    run_case(dtype, L=2, H=64, N=4, F=128, B=2, Q=16, Mm=8, S=2, M=6, seed=3, overlap=True)
