@@ -51,6 +51,51 @@ struct ds_stage {
   virtual size_t stash_bytes(int slots) const = 0;
 };
 
+// Bookkeeping for running a layer's weight-gradient work on ds_stage::wgrad_stream beside the dgrad
+// chain of the layers below.  The buffers the weight-gradient kernels read alternate by layer parity;
+// per parity one event says "the chain produced them" and one "the weight-gradient kernels are done
+// with them".
+struct WgradLane {
+  hipEvent_t ready[2] = {nullptr, nullptr}, done[2] = {nullptr, nullptr};
+  bool valid[2] = {false, false};
+  ~WgradLane() {
+    for (int p = 0; p < 2; ++p) {
+      if (ready[p]) (void)hipEventDestroy(ready[p]);
+      if (done[p]) (void)hipEventDestroy(done[p]);
+    }
+  }
+  int ensure() {
+    if (ready[0]) return DS_OK;
+    for (int p = 0; p < 2; ++p) {
+      DS_CHECK_HIP(hipEventCreateWithFlags(&ready[p], hipEventDisableTiming));
+      DS_CHECK_HIP(hipEventCreateWithFlags(&done[p], hipEventDisableTiming));
+    }
+    return DS_OK;
+  }
+  // chain: before it overwrites the parity's buffers
+  int reuse(hipStream_t chain, int par) {
+    if (valid[par]) DS_CHECK_HIP(hipStreamWaitEvent(chain, done[par], 0));
+    return DS_OK;
+  }
+  // the parity's buffers are complete on `chain`: the weight-gradient stream may read them
+  int begin(hipStream_t chain, hipStream_t ws, int par) {
+    DS_CHECK_HIP(hipEventRecord(ready[par], chain));
+    DS_CHECK_HIP(hipStreamWaitEvent(ws, ready[par], 0));
+    return DS_OK;
+  }
+  int end(hipStream_t ws, int par) {
+    DS_CHECK_HIP(hipEventRecord(done[par], ws));
+    valid[par] = true;
+    return DS_OK;
+  }
+  // chain: everything on the weight-gradient stream so far is ordered before what follows
+  int finish(hipStream_t chain) {
+    for (int p = 0; p < 2; ++p)
+      if (valid[p]) DS_CHECK_HIP(hipStreamWaitEvent(chain, done[p], 0));
+    return DS_OK;
+  }
+};
+
 // With overlap on, anything that writes into a stash slot on the stage's stream must first wait for the
 // backward pass that last used the slot.
 static inline int ds_stage_acquire_slot(ds_stage* h, int slot) {

@@ -94,19 +94,12 @@ struct BertStage : ds_stage {
   char* ws_base = nullptr;
   size_t ws_bytes = 0;
   size_t ws_scores, ws_ds, ws_dz2[2], ws_du[2], ws_da, ws_dz1[2], ws_dctx, ws_dqkv[2], ws_dx[2];
-  // weight-gradient stream bookkeeping: per layer parity, "dgrad chain produced the wgrad operands" and
-  // "wgrads consumed them"
-  hipEvent_t ev_ready[2] = {nullptr, nullptr}, ev_done[2] = {nullptr, nullptr};
-  bool done_valid[2] = {false, false};
+  WgradLane lane;
 
   ~BertStage() override {
     if (wc_base) (void)hipFree(wc_base);
     if (stash_base) (void)hipFree(stash_base);
     if (ws_base) (void)hipFree(ws_base);
-    for (int p = 0; p < 2; ++p) {
-      if (ev_ready[p]) (void)hipEventDestroy(ev_ready[p]);
-      if (ev_done[p]) (void)hipEventDestroy(ev_done[p]);
-    }
   }
   int base(int l) const { return (emb ? EMB_NW : 0) + l * LAYER_NW; }
   char* slotp(int slot) const { return stash_base + (size_t)slot * slot_bytes; }
@@ -364,12 +357,7 @@ struct BertStage : ds_stage {
     // With a weight-gradient stream the wgrad GEMMs and bias column sums of a layer run beside the
     // dgrad chain of the layers below it: they only feed the master gradients.
     hipStream_t ws = wgrad_stream;
-    if (ws && !ev_ready[0]) {
-      for (int p = 0; p < 2; ++p) {
-        DS_CHECK_HIP(hipEventCreateWithFlags(&ev_ready[p], hipEventDisableTiming));
-        DS_CHECK_HIP(hipEventCreateWithFlags(&ev_done[p], hipEventDisableTiming));
-      }
-    }
+    if (ws) DS_PROPAGATE(lane.ensure());
     for (int l = L - 1; l >= 0; --l) {
       const LayerStash& t = ls[l];
       const int b = base(l);
@@ -383,7 +371,7 @@ struct BertStage : ds_stage {
       float* dp = (float*)(ws_base + ws_scores);
       char* dsm = ws_base + ws_ds;
       // the wgrads that read this parity's buffers two layers up must have run
-      if (ws && done_valid[par]) DS_CHECK_HIP(hipStreamWaitEvent(stream, ev_done[par], 0));
+      if (ws) DS_PROPAGATE(lane.reuse(stream, par));
       // output LayerNorm; the column sums of dz2 are the gradient of output/dense/bias
       DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, dy, sp + t.z2, w[b + LN2_G], (const float*)(sp + t.st2), nullptr, dz2,
                                     g[b + LN2_G], g[b + LN2_B], g[b + B_FF2], stream));
@@ -421,8 +409,7 @@ struct BertStage : ds_stage {
       // ---- weight gradients of this layer (on the weight-gradient stream when there is one)
       hipStream_t chain = stream;
       if (ws) {
-        DS_CHECK_HIP(hipEventRecord(ev_ready[par], chain));
-        DS_CHECK_HIP(hipStreamWaitEvent(ws, ev_ready[par], 0));
+        DS_PROPAGATE(lane.begin(chain, ws, par));
         stream = ws;  // gemm_wgrad and the column sums below launch on `stream`
       }
       int rc = DS_OK;
@@ -454,10 +441,7 @@ struct BertStage : ds_stage {
       } while (0);
       stream = chain;
       if (rc != DS_OK) return rc;
-      if (ws) {
-        DS_CHECK_HIP(hipEventRecord(ev_done[par], ws));
-        done_valid[par] = true;
-      }
+      if (ws) DS_PROPAGATE(lane.end(ws, par));
       // dx = dqkv Wqkv^T + dz1 (x also feeds the residual into z1)
       const bool first = (l == 0);
       if (first && !emb && d_in == nullptr) break;  // a first stage takes no input gradient
@@ -466,9 +450,7 @@ struct BertStage : ds_stage {
       dy = dx;
     }
     // the stash slot and the master gradients are released to the caller in the order of `stream`
-    if (ws)
-      for (int p = 0; p < 2; ++p)
-        if (done_valid[p]) DS_CHECK_HIP(hipStreamWaitEvent(stream, ev_done[p], 0));
+    if (ws) DS_PROPAGATE(lane.finish(stream));
     if (emb) {
       // embedding LayerNorm backward, then scatter-add into the three tables
       char* de = ws_base + ws_dz2[0];

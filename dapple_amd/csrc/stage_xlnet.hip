@@ -176,8 +176,10 @@ struct XlnetStage : ds_stage {
   std::vector<char> has_mask, has_seg;
   // workspace
   char* ws_base = nullptr;
-  size_t ws_bytes = 0, ws_qall, ws_ac, ws_dp, ws_bd, ws_ds, ws_dbd, ws_dz2, ws_du, ws_dy1, ws_dz1, ws_dvec, ws_dqw, ws_dqr, ws_dqs, ws_dq,
-         ws_dkv, ws_dkr, ws_deft, ws_dx[2];
+  // buffers the weight-gradient kernels read alternate by layer parity ([2])
+  size_t ws_bytes = 0, ws_qall, ws_ac, ws_dp, ws_bd, ws_ds, ws_dbd, ws_dz2[2], ws_du[2], ws_dy1, ws_dz1[2], ws_dvec, ws_dqw[2], ws_dqr[2],
+         ws_dqs[2], ws_dq[2], ws_dkv[2], ws_dkr[2], ws_deft[2], ws_dx[2];
+  WgradLane lane;
 
   ~XlnetStage() override {
     if (wc_base) (void)hipFree(wc_base);
@@ -254,11 +256,14 @@ struct XlnetStage : ds_stage {
     ws_bd = w.reserve((size_t)B * N * Q * R * 4);
     ws_ds = w.reserve((size_t)B * N * Q * K * esz);
     ws_dbd = w.reserve((size_t)B * N * Q * R * esz);
-    ws_dz2 = w.reserve(act); ws_du = w.reserve(actF); ws_dy1 = w.reserve(act); ws_dz1 = w.reserve(act); ws_dvec = w.reserve(act);
-    ws_dqw = w.reserve(act); ws_dqr = w.reserve(act); ws_dqs = w.reserve(act); ws_dq = w.reserve(act);
-    ws_dkv = w.reserve((size_t)krows * 2 * H * esz);
-    ws_dkr = w.reserve((size_t)R * H * esz);
-    ws_deft = w.reserve((size_t)N * 2 * rows * esz);
+    ws_dy1 = w.reserve(act); ws_dvec = w.reserve(act);
+    for (int p = 0; p < 2; ++p) {
+      ws_dz2[p] = w.reserve(act); ws_du[p] = w.reserve(actF); ws_dz1[p] = w.reserve(act);
+      ws_dqw[p] = w.reserve(act); ws_dqr[p] = w.reserve(act); ws_dqs[p] = w.reserve(act); ws_dq[p] = w.reserve(act);
+      ws_dkv[p] = w.reserve((size_t)krows * 2 * H * esz);
+      ws_dkr[p] = w.reserve((size_t)R * H * esz);
+      ws_deft[p] = w.reserve((size_t)N * 2 * rows * esz);
+    }
     ws_dx[0] = w.reserve(act); ws_dx[1] = w.reserve(act);
     ws_bytes = w.used;
     DS_CHECK_HIP(hipMalloc((void**)&ws_base, ws_bytes));
@@ -413,26 +418,29 @@ struct XlnetStage : ds_stage {
     const float scale = 1.0f / sqrtf((float)D);
     const uint8_t* seg = has_seg[slot] ? (const uint8_t*)(sp + seg_off) : nullptr;
     const char* dy = (const char*)d_out;
-    char* dz2 = ws_base + ws_dz2; char* du = ws_base + ws_du; char* dy1 = ws_base + ws_dy1; char* dz1 = ws_base + ws_dz1;
-    char* dvec = ws_base + ws_dvec; char* dqw = ws_base + ws_dqw; char* dqr = ws_base + ws_dqr; char* dqs = ws_base + ws_dqs;
-    char* dq = ws_base + ws_dq; char* dkv = ws_base + ws_dkv; char* dkr = ws_base + ws_dkr; char* deft = ws_base + ws_deft;
+    char* dy1 = ws_base + ws_dy1; char* dvec = ws_base + ws_dvec;
     float* dp = (float*)(ws_base + ws_dp);
     char* dsm = ws_base + ws_ds; char* dbd = ws_base + ws_dbd;
+    // with a weight-gradient stream, a layer's weight gradients run beside the dgrad chain of the layers below
+    hipStream_t wgs = wgrad_stream;
+    if (wgs) DS_PROPAGATE(lane.ensure());
     for (int l = L - 1; l >= 0; --l) {
       const LayerOff& t = lo[l];
       const int b = base(l);
+      const int par = l & 1;
+      char* dz2 = ws_base + ws_dz2[par]; char* du = ws_base + ws_du[par]; char* dz1 = ws_base + ws_dz1[par];
+      char* dqw = ws_base + ws_dqw[par]; char* dqr = ws_base + ws_dqr[par]; char* dqs = ws_base + ws_dqs[par];
+      char* dq = ws_base + ws_dq[par]; char* dkv = ws_base + ws_dkv[par]; char* dkr = ws_base + ws_dkr[par];
+      char* deft = ws_base + ws_deft[par];
+      if (wgs) DS_PROPAGATE(lane.reuse(stream, par));
       char* x = sp + t.x;
       DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, dy, sp + t.z2, w[b + X_LN2_G], (const float*)(sp + t.st2), nullptr, dz2,
                                     g[b + X_LN2_G], g[b + X_LN2_B], g[b + X_B2], stream));
-      DS_PROPAGATE(gemm(DS_MN_MAJOR, DS_MN_MAJOR, F, H, rows, sp + t.hh, F, dz2, H, g[b + X_W2], H, DS_EPI_ACCUM));
       DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rows, F, H, dz2, H, WT(l, X_W2), H, du, F, DS_EPI_DGELU | DS_EPI_TANH_FORM, nullptr, nullptr, sp + t.u));
-      DS_PROPAGATE(ds_colsum_accum(dtype, rows, F, du, F, g[b + X_B1], stream));
-      DS_PROPAGATE(gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, F, rows, sp + t.y1, H, du, F, g[b + X_W1], F, DS_EPI_ACCUM));
       DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rows, H, F, du, F, WT(l, X_W1), F, dy1, H, DS_EPI_RESIDUAL, nullptr, dz2));
       DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, dy1, sp + t.z1, w[b + X_LN1_G], (const float*)(sp + t.st1), nullptr, dz1,
                                     g[b + X_LN1_G], g[b + X_LN1_B], nullptr, stream));
       // o projection: attn_out[row,h] = sum_nd vec[row,nd] Wo[h,nd]
-      DS_PROPAGATE(gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, rows, dz1, H, sp + t.vec, H, g[b + X_O], H, DS_EPI_ACCUM));
       DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, rows, H, H, dz1, H, WT(l, X_O), H, dvec, H));
       for (int s = 0; s < S; ++s) {
         const size_t so = (size_t)s * rowsS * H * esz;
@@ -478,31 +486,47 @@ struct XlnetStage : ds_stage {
           DS_CHECK_LAUNCH();
         }
       }
-      // relative biases: column sums of the three query-gradient pieces
-      DS_PROPAGATE(ds_colsum_accum(dtype, rows, H, dqw, H, g[b + X_RW], stream));
-      DS_PROPAGATE(ds_colsum_accum(dtype, rows, H, dqr, H, g[b + X_RR], stream));
-      DS_PROPAGATE(ds_colsum_accum(dtype, rows, H, dqs, H, g[b + X_RS], stream));
-      // seg_emb[s][n][:] += sum_rows def[row][n][s] * qs[row][n][:]   (batched over heads)
-      {
-        ds_gemm_desc d;
-        memset(&d, 0, sizeof(d));
-        d.dtype = dtype; d.a_major = DS_K_MAJOR; d.b_major = DS_MN_MAJOR; d.m = 2; d.n = D; d.k = rows;
-        d.lda = rows; d.ldb = H; d.ldc = H; d.batch = N; d.batch_inner = N;
-        d.a_stride_inner = (int64_t)2 * rows; d.b_stride_inner = D; d.c_stride_inner = D;
-        d.flags = DS_EPI_ACCUM; d.alpha = 1.f; d.a = deft; d.b = sp + t.qs; d.c = g[b + X_SEG];
-        DS_PROPAGATE(ds_gemm(&d, stream));
-      }
-      // projections
-      DS_PROPAGATE(gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, rows, x, H, dq, H, g[b + X_Q], H, DS_EPI_ACCUM));
-      DS_PROPAGATE(gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, R, pe, H, dkr, H, g[b + X_R], H, DS_EPI_ACCUM));
+      // ---- weight gradients of this layer (on the weight-gradient stream when there is one)
       const char* dkv_h = dkv + (size_t)Mm * B * 2 * H * esz;
-      for (int j = 0; j < 2; ++j) {  // j = 0: k, 1: v
-        float* gw = g[b + X_K + j];
-        if (Mm > 0)
-          DS_PROPAGATE(gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, Mm * B, sp + mem_off + (size_t)l * Mm * B * H * esz, H, dkv + (size_t)j * H * esz,
-                            2 * H, gw, H, DS_EPI_ACCUM));
-        DS_PROPAGATE(gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, rowsS, x, H, dkv_h + (size_t)j * H * esz, 2 * H, gw, H, DS_EPI_ACCUM));
+      hipStream_t chain = stream;
+      if (wgs) {
+        DS_PROPAGATE(lane.begin(chain, wgs, par));
+        stream = wgs;  // gemm() and the column sums below launch on `stream`
       }
+      int rc = DS_OK;
+      do {
+        if ((rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, F, H, rows, sp + t.hh, F, dz2, H, g[b + X_W2], H, DS_EPI_ACCUM)) != DS_OK) break;
+        if ((rc = ds_colsum_accum(dtype, rows, F, du, F, g[b + X_B1], stream)) != DS_OK) break;
+        if ((rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, F, rows, sp + t.y1, H, du, F, g[b + X_W1], F, DS_EPI_ACCUM)) != DS_OK) break;
+        if ((rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, rows, dz1, H, sp + t.vec, H, g[b + X_O], H, DS_EPI_ACCUM)) != DS_OK) break;
+        // relative biases: column sums of the three query-gradient pieces
+        if ((rc = ds_colsum_accum(dtype, rows, H, dqw, H, g[b + X_RW], stream)) != DS_OK) break;
+        if ((rc = ds_colsum_accum(dtype, rows, H, dqr, H, g[b + X_RR], stream)) != DS_OK) break;
+        if ((rc = ds_colsum_accum(dtype, rows, H, dqs, H, g[b + X_RS], stream)) != DS_OK) break;
+        // seg_emb[s][n][:] += sum_rows def[row][n][s] * qs[row][n][:]   (batched over heads)
+        {
+          ds_gemm_desc d;
+          memset(&d, 0, sizeof(d));
+          d.dtype = dtype; d.a_major = DS_K_MAJOR; d.b_major = DS_MN_MAJOR; d.m = 2; d.n = D; d.k = rows;
+          d.lda = rows; d.ldb = H; d.ldc = H; d.batch = N; d.batch_inner = N;
+          d.a_stride_inner = (int64_t)2 * rows; d.b_stride_inner = D; d.c_stride_inner = D;
+          d.flags = DS_EPI_ACCUM; d.alpha = 1.f; d.a = deft; d.b = sp + t.qs; d.c = g[b + X_SEG];
+          if ((rc = ds_gemm(&d, stream)) != DS_OK) break;
+        }
+        // projections
+        if ((rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, rows, x, H, dq, H, g[b + X_Q], H, DS_EPI_ACCUM)) != DS_OK) break;
+        if ((rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, R, pe, H, dkr, H, g[b + X_R], H, DS_EPI_ACCUM)) != DS_OK) break;
+        for (int j = 0; j < 2 && rc == DS_OK; ++j) {  // j = 0: k, 1: v
+          float* gw = g[b + X_K + j];
+          if (Mm > 0)
+            rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, Mm * B, sp + mem_off + (size_t)l * Mm * B * H * esz, H, dkv + (size_t)j * H * esz,
+                      2 * H, gw, H, DS_EPI_ACCUM);
+          if (rc == DS_OK) rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, rowsS, x, H, dkv_h + (size_t)j * H * esz, 2 * H, gw, H, DS_EPI_ACCUM);
+        }
+      } while (0);
+      stream = chain;
+      if (rc != DS_OK) return rc;
+      if (wgs) DS_PROPAGATE(lane.end(wgs, par));
       // dx = dq Wq^T + dz1 (residual); the content-stream rows also receive dkv Wkv^T
       const bool first = l == 0;
       if (first && d_in == nullptr) break;
@@ -511,6 +535,8 @@ struct XlnetStage : ds_stage {
       DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rowsS, H, 2 * H, dkv_h, 2 * H, wkv[l], 2 * H, dx, H, DS_EPI_RESIDUAL, nullptr, dx));
       dy = dx;
     }
+    // the stash slot and the master gradients are released to the caller in the order of `stream`
+    if (wgs) DS_PROPAGATE(lane.finish(stream));
     return DS_OK;
   }
 };
