@@ -93,6 +93,7 @@ class Stage:
         self.flat_weights = torch.empty(total, dtype=torch.float32, device=self.device)
         self.flat_grads = torch.zeros(total, dtype=torch.float32, device=self.device)
         off = 0
+        self.weight_offsets, self.weight_numels = [], []
         wp = (C.c_void_p * len(sizes))()
         gp = (C.c_void_p * len(sizes))()
         for i, (n, shp, sz) in enumerate(zip(self.weight_names, shapes, sizes)):
@@ -104,6 +105,8 @@ class Stage:
             self.weights[n] = wv
             self.grads[n] = self.flat_grads[off:off + numel].view(*shp)
             wp[i], gp[i] = wv.data_ptr(), self.grads[n].data_ptr()
+            self.weight_offsets.append(off)
+            self.weight_numels.append(numel)
             off += sz
         check(self.lib.ds_stage_bind_weights(self._h, len(sizes), wp, gp), "ds_stage_bind_weights")
 

@@ -278,6 +278,34 @@ int ds_xlnet_stage_create(const ds_xlnet_cfg* cfg, void* stream, ds_stage** out)
  *   mems    [num_layers][mem_len][batch][hidden] in the compute type; required when mem_len > 0 */
 int ds_xlnet_stage_set_inputs(ds_stage* h, int slot, const float* masks, const uint8_t* seg_mat, const void* mems);
 
+/* ---- what the reference runs on the accumulated gradients right after the unroll block ----
+ *
+ * Global-norm clipping, bert/graph.py:162-165 (tf.clip_by_global_norm over all accumulated gradients):
+ * ds_grad_sqnorm_accum adds sum(g^2) of a buffer into a device double (clear it first, call once per
+ * gradient buffer); the update entry points below take that scalar and clip_norm and scale every
+ * gradient by clip_norm / max(sqrt(sum), clip_norm) on the fly (pass NULL for no clipping). */
+int ds_grad_sqnorm_accum(const float* g, size_t n, double* acc, void* stream);
+
+/* The tensors of a flat fp32 master buffer (element offsets, multiples of 4; element counts) and the
+ * decoupled weight-decay rate of each: 0.01 for BERT's matrices, 0 for the names matching
+ * "LayerNorm", "layer_norm", "bias" (bert/graph_helper.py:179-185, _do_use_weight_decay :274-282). */
+typedef struct ds_optim_plan ds_optim_plan;
+int ds_optim_plan_create(int n_tensors, const int64_t* offsets, const int64_t* numels, const float* decay_rates,
+                         ds_optim_plan** out);
+int ds_optim_plan_destroy(ds_optim_plan* plan);
+
+/* AdamWeightDecayOptimizer.apply_gradients, bert/graph_helper.py:213-272:
+ *   m = b1 m + (1-b1) g;  v = b2 v + (1-b2) g^2;  w -= lr * (m / (sqrt(v) + eps) + decay * w)
+ * (no bias correction).  tf.train.AdamOptimizer (xlnet/utils/xlnet_utils.py:195-197) is the same update
+ * with decay 0 and lr replaced by lr * sqrt(1 - b2^t) / (1 - b1^t), which the caller computes.
+ * The hyper-parameters are doubles like the reference's Python floats: 1 - beta is formed in double
+ * and then rounded, as TensorFlow does when it folds `1.0 - self.beta_2` into a float32 constant. */
+int ds_adam_step(const ds_optim_plan* plan, float* w, const float* g, float* m, float* v, double lr, double beta1,
+                 double beta2, double eps, const double* grad_sqnorm, float clip_norm, void* stream);
+/* tf.train.GradientDescentOptimizer (vgg19/tf-keras-dapple.py:187): w -= lr * g */
+int ds_sgd_step(const ds_optim_plan* plan, float* w, const float* g, double lr, const double* grad_sqnorm,
+                float clip_norm, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
