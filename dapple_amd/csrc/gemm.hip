@@ -221,9 +221,29 @@ __device__ __forceinline__ void gemm_epilogue_staged(const GemmArgs& p, f32x16 (
                                                      int wm, int wn, int lane, int tid, int64_t c_off, char* lds) {
   constexpr int TM = BM / 64, TN = BN / 64;
   constexpr int LDW = BN + 4;
+  constexpr int VPR = BN / 8;             // 8-column vectors per tile row
+  constexpr int ITER = BM * VPR / 256;    // vectors per thread
   float* sc = reinterpret_cast<float*>(lds);
   const int flags = p.flags;
   const bool tanh_form = (flags & DS_EPI_TANH_FORM) != 0;
+  float* Cf = reinterpret_cast<float*>(p.c) + c_off;
+  // C += acc with nothing else in the epilogue: fetch this thread's share of C now, in one batch, so
+  // that the round trip to memory runs under the LDS staging below instead of once per vector afterwards
+  const bool preload = (flags & DS_EPI_ACCUM) && p.splitk == 1 &&
+                       (flags & ~(DS_EPI_ACCUM | DS_EPI_BIAS | DS_EPI_OUT_F32)) == 0;
+  f32x4 cpre[ITER][2];
+  if (preload) {
+#pragma unroll
+    for (int it = 0; it < ITER; ++it) {
+      const int v = tid + it * 256;
+      const int row = m0 + v / VPR, col = n0 + (v % VPR) * 8;
+      if (row < p.m && col < p.n) {
+        const float* src = Cf + (int64_t)row * p.ldc + col;
+        cpre[it][0] = *reinterpret_cast<const f32x4*>(src);
+        cpre[it][1] = *reinterpret_cast<const f32x4*>(src + 4);
+      }
+    }
+  }
   __syncthreads();
 #pragma unroll
   for (int i = 0; i < TM; ++i)
@@ -240,11 +260,24 @@ __device__ __forceinline__ void gemm_epilogue_staged(const GemmArgs& p, f32x16 (
     }
   __syncthreads();
   const bool out_f32 = (flags & (DS_EPI_OUT_F32 | DS_EPI_ACCUM)) != 0 || sizeof(T) == 4;
-  float* Cf = reinterpret_cast<float*>(p.c) + c_off;
   T* Ct = reinterpret_cast<T*>(p.c) + c_off;
   const T* R = reinterpret_cast<const T*>(p.residual) + c_off;
   T* C2 = reinterpret_cast<T*>(p.c2) + c_off;
-  constexpr int VPR = BN / 8;  // 8-column vectors per tile row
+  if (preload) {
+#pragma unroll
+    for (int it = 0; it < ITER; ++it) {
+      const int v = tid + it * 256;
+      const int rl = v / VPR, cl = (v % VPR) * 8;
+      const int row = m0 + rl, col = n0 + cl;
+      if (row >= p.m || col >= p.n) continue;
+      const f32x4 lo = *reinterpret_cast<const f32x4*>(sc + rl * LDW + cl);
+      const f32x4 hi = *reinterpret_cast<const f32x4*>(sc + rl * LDW + cl + 4);
+      float* dst = Cf + (int64_t)row * p.ldc + col;
+      *reinterpret_cast<f32x4*>(dst) = cpre[it][0] + lo;
+      *reinterpret_cast<f32x4*>(dst + 4) = cpre[it][1] + hi;
+    }
+    return;
+  }
 #pragma unroll 2
   for (int v = tid; v < BM * VPR; v += 256) {
     const int rl = v / VPR, cl = (v % VPR) * 8;
