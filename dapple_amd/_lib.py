@@ -120,6 +120,8 @@ PROTOTYPES = {
     "ds_stage_overlap_supported": (C.c_int, [C.c_void_p]),
     "ds_stage_enable_overlap": (C.c_int, [C.c_void_p, C.c_int]),
     "ds_stage_join": (C.c_int, [C.c_void_p]),
+    "ds_squad_head": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                C.c_float, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "ds_grad_sqnorm_accum": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p]),
     "ds_optim_plan_create": (C.c_int, [C.c_int, C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_float),
                                         C.POINTER(C.c_void_p)]),

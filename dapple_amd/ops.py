@@ -207,3 +207,28 @@ def attention_bwd(qkv, ctx, lse, dctx, batch, heads, seq, scale, key_mask=None, 
                                        scale, mask_value, ptr(ctx), ptr(lse), ptr(dctx), ptr(dqkv), ptr(delta),
                                        _lib.current_stream()), "ds_attention_bwd")
     return dqkv
+
+
+def squad_head(x, batch, seq, output_weights, output_bias, start_positions, end_positions, d_weights=None, d_bias=None,
+               need_dx=True, loss_scale=1.0):
+    """build_output_layer_squad of bert/models/bert/bert.py:669-718 on the stage's sequence output
+    ``x [batch*seq, hidden]``: returns (loss [1] fp32 on the device, start_logits [batch, seq], end_logits
+    [batch, seq], dx or None).  ``d_weights [2, hidden]`` / ``d_bias [2]`` (fp32) are added to in place."""
+    _need_cuda(x, output_weights, output_bias, start_positions, end_positions)
+    hidden = x.shape[-1]
+    if x.numel() != batch * seq * hidden or tuple(output_weights.shape) != (2, hidden):
+        raise ValueError("squad_head: x must be [batch*seq, hidden] and output_weights [2, hidden]")
+    if start_positions.dtype != torch.int32 or end_positions.dtype != torch.int32:
+        raise ValueError("squad_head: positions must be int32")
+    for t in (output_weights, output_bias, d_weights, d_bias):
+        if t is not None and t.dtype != torch.float32:
+            raise ValueError("squad_head: weights, bias and their gradients must be fp32")
+    loss = torch.empty(1, dtype=torch.float32, device=x.device)
+    logits = torch.empty(batch * seq, 2, dtype=torch.float32, device=x.device)
+    dlogits = torch.empty_like(logits)
+    dx = torch.empty_like(x) if need_dx else None
+    check(_lib.load().ds_squad_head(dtype_code(x), batch, seq, hidden, ptr(x), ptr(output_weights), ptr(output_bias),
+                                    ptr(start_positions), ptr(end_positions), loss_scale, ptr(loss), ptr(logits), ptr(dlogits),
+                                    ptr(dx), ptr(d_weights), ptr(d_bias), _lib.current_stream()), "ds_squad_head")
+    lg = logits.view(batch, seq, 2)
+    return loss, lg[:, :, 0], lg[:, :, 1], dx

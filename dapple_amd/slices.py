@@ -226,6 +226,33 @@ class BertFinetuneSlice(object):
         self.stage.bind(weights)
         self.layers, self.local_device, self.model_type = layers, local_device, model_type
         self.stage_outputs = []
+        self.is_last = (nstage - 1) in mine
+        self.loss = None
+        if self.is_last and model_type == 'mrc':             # bert.py:467-470
+            # cls/squad/output_weights [2, hidden] (truncated normal 0.02), output_bias [2] zeros (bert.py:677-683)
+            g = torch.Generator().manual_seed(seed + 1)
+            H = bert_config.hidden_size
+            self.output_weights = (torch.randn(2, H, generator=g) * 0.02).cuda()
+            self.output_bias = torch.zeros(2, device="cuda")
+            self.d_output_weights = torch.zeros_like(self.output_weights)
+            self.d_output_bias = torch.zeros_like(self.output_bias)
+
+    def build_output_layer_squad(self, sequence_output, is_training=False):
+        """bert.py:669-718 on the last device: start / end logits and the SQuAD loss from
+        ``kwargs["start_positions"]`` / ``kwargs["end_positions"]``.  Returns the gradient of the loss w.r.t.
+        ``sequence_output`` - the upstream gradient of this stage's backward pass; the head's own weight
+        gradients are added into ``d_output_weights`` / ``d_output_bias``."""
+        from . import ops
+        if not (self.is_last and self.model_type == 'mrc'):
+            raise ValueError("build_output_layer_squad: this device does not hold the SQuAD output layer")
+        B, S = self.input_ids.shape
+        sp = torch.as_tensor(self.kwargs["start_positions"], dtype=torch.int32).cuda()
+        ep = torch.as_tensor(self.kwargs["end_positions"], dtype=torch.int32).cuda()
+        x = sequence_output.reshape(B * S, self.bert_config.hidden_size)
+        self.loss, self.start_logits, self.end_logits, dx = ops.squad_head(
+            x, B, S, self.output_weights, self.output_bias, sp, ep, self.d_output_weights, self.d_output_bias)
+        self.stage_outputs = [sequence_output, self.loss]
+        return dx
 
 
 # =========================================================================== VGG19

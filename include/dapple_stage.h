@@ -278,6 +278,18 @@ int ds_xlnet_stage_create(const ds_xlnet_cfg* cfg, void* stream, ds_stage** out)
  *   mems    [num_layers][mem_len][batch][hidden] in the compute type; required when mem_len > 0 */
 int ds_xlnet_stage_set_inputs(ds_stage* h, int slot, const float* masks, const uint8_t* seg_mat, const void* mems);
 
+/* Last-stage head of the SQuAD model, bert/models/bert/bert.py:669-718 (build_output_layer_squad):
+ * logits = X W^T + b with W = cls/squad/output_weights [2, hidden], b = cls/squad/output_bias [2];
+ * loss = (CE(start) + CE(end)) / 2, CE = -mean_batch log_softmax(logits over seq)[position] (:699-713); a
+ * position outside [0, seq) contributes no loss term, like tf.one_hot.
+ *   x [batch*seq, hidden] (compute type): the stage's sequence output; logits, dlogits: fp32 [batch*seq, 2]
+ *   (column 0 start, 1 end) out; loss: device float, overwritten with loss_scale * loss;
+ *   dx (nullable): d loss / d x in the compute type - the d_out of the stage's backward pass;
+ *   dw [2, hidden], dbias [2] (nullable): master gradients, added to (tf.accumulate_n over micro-batches). */
+int ds_squad_head(int dtype, int batch, int seq, int hidden, const void* x, const float* w, const float* bias,
+                  const int32_t* start_positions, const int32_t* end_positions, float loss_scale, float* loss,
+                  float* logits, float* dlogits, void* dx, float* dw, float* dbias, void* stream);
+
 /* ---- what the reference runs on the accumulated gradients right after the unroll block ----
  *
  * Global-norm clipping, bert/graph.py:162-165 (tf.clip_by_global_norm over all accumulated gradients):

@@ -52,6 +52,18 @@ def test_bert_finetune_slice_puts_the_planner_split_on_each_device():
     assert s1.stage.weight_names[0] == "bert/encoder/layer_11/attention/self/query/kernel"
     with pytest.raises(ValueError, match="Cannot use sequence length"):
         slices.BertFinetuneSlice(cfg, 32, False, ids, None, None, None, False)
+    # the last device holds the SQuAD output layer (bert.py:467-470): loss from kwargs' positions, and the gradient
+    # that feeds the stage's backward pass
+    s1.kwargs = {"start_positions": [1, 2], "end_positions": [3, 7]}
+    h = torch.randn(2 * 8, 32, device="cuda")
+    y = torch.empty_like(h)
+    s1.stage.forward(0, h, y)
+    dy = s1.build_output_layer_squad(y.reshape(2, 8, 32))
+    assert s1.stage_outputs[-1] is s1.loss and 0.0 < float(s1.loss) < 10.0
+    assert dy.shape == y.shape and float(s1.d_output_weights.abs().max()) > 0
+    s1.stage.backward(0, dy, torch.empty_like(h))
+    with pytest.raises(ValueError, match="does not hold"):
+        s0.build_output_layer_squad(y)
     s0.stage.close(); s1.stage.close()
 
 
