@@ -77,8 +77,9 @@ struct BertStage : ds_stage {
   size_t esz;
   bool emb;
   bool fused_attn;  // bf16, head size 64: fused attention kernels, no [B,N,S,S] tensors at all
-  // the fused forward pass writes only its stash slot and its output; the workspace belongs to backward
-  bool overlap_safe() const override { return fused_attn; }
+  // the forward pass writes its stash slot, its output and (unfused attention) its own score buffer; the rest
+  // of the workspace belongs to backward
+  bool overlap_safe() const override { return true; }
   // compute copies
   char* wc_base = nullptr;
   std::vector<char*> wqkv, wo, w1, w2;  // element type T
@@ -93,7 +94,7 @@ struct BertStage : ds_stage {
   // workspace
   char* ws_base = nullptr;
   size_t ws_bytes = 0;
-  size_t ws_scores, ws_ds, ws_dz2[2], ws_du[2], ws_da, ws_dz1[2], ws_dctx, ws_dqkv[2], ws_dx[2];
+  size_t ws_scores, ws_fscores, ws_ds, ws_dz2[2], ws_du[2], ws_da, ws_dz1[2], ws_dctx, ws_dqkv[2], ws_dx[2];
   WgradLane lane;
 
   ~BertStage() override {
@@ -197,6 +198,7 @@ struct BertStage : ds_stage {
     // ---- workspace
     Arena w;
     ws_scores = w.reserve(fused_attn ? (size_t)B * NH * S * 4 : (size_t)B * NH * S * S * 4);  // fused: delta
+    ws_fscores = fused_attn ? 0 : w.reserve((size_t)B * NH * S * S * 4);  // forward's own scores: backward keeps ws_scores
     ws_ds = fused_attn ? 0 : w.reserve(probs);
     for (int p = 0; p < 2; ++p) {  // the operands of the weight-gradient GEMMs alternate by layer parity
       ws_dz2[p] = w.reserve(act);
@@ -323,10 +325,10 @@ struct BertStage : ds_stage {
       } else {
       // scores = Q K^T (:499), fp32
       DS_PROPAGATE(gemm_heads(DS_K_MAJOR, DS_K_MAJOR, S, S, D, sp + t.qkv, 3 * H, (int64_t)S * 3 * H, D,
-                              sp + t.qkv + (size_t)H * esz, 3 * H, (int64_t)S * 3 * H, D, ws_base + ws_scores, S,
+                              sp + t.qkv + (size_t)H * esz, 3 * H, (int64_t)S * 3 * H, D, ws_base + ws_fscores, S,
                               (int64_t)NH * S * S, (int64_t)S * S, DS_EPI_OUT_F32));
       // scale, mask adder, softmax (:500-518)
-      DS_PROPAGATE(ds_softmax_fwd(dtype, B, NH, S, S, (const float*)(ws_base + ws_scores), scale, mask, -10000.0f,
+      DS_PROPAGATE(ds_softmax_fwd(dtype, B, NH, S, S, (const float*)(ws_base + ws_fscores), scale, mask, -10000.0f,
                                   sp + t.p, stream));
       // ctx = P V (:533), written head-interleaved as [rows, H] (:536-542)
       DS_PROPAGATE(gemm_heads(DS_K_MAJOR, DS_MN_MAJOR, S, D, S, sp + t.p, S, (int64_t)NH * S * S, (int64_t)S * S,

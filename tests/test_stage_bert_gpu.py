@@ -188,9 +188,42 @@ def test_forward_backward_overlap_matches_serial():
 
 @pytest.mark.gpu
 def test_overlap_refused_where_passes_share_workspace():
-    from dapple_amd import runtime
-    st = runtime.bert_stage(1, 64, 2, 128, 1, 16, "fp32", stash_slots=1)
+    from dapple_amd import runtime, synthetic
+    layers = synthetic.vgg_layers([8, None])
+    st = runtime.vgg_stage(layers, 1, 8, 8, 3, 1)
     assert not st.overlap_supported()
     with pytest.raises(ValueError):
         st.enable_overlap()
     st.close()
+
+
+@pytest.mark.gpu
+def test_forward_backward_overlap_unfused_fp32_with_embedding():
+    """fp32 stage with the embedding (unfused attention, token types set per slot) on three streams against the
+    one-stream run."""
+    from dapple_amd import runtime, synthetic
+    L, H, N, F, B, S, M = 2, 64, 4, 128, 2, 16, 5
+    emb = (50, 2, 16)
+    w = synthetic.bert_weights(41, L, H, F, embeddings=emb)
+    ids = [torch.as_tensor(x).cuda() for x in synthetic.bert_id_inputs(42, M, B, S, emb[0])]
+    dys = [torch.as_tensor(x).cuda() for x in synthetic.upstream_grads(43, M, (B * S, H))]
+    res = []
+    for overlap in (False, True):
+        st = runtime.bert_stage(L, H, N, F, B, S, "fp32", stash_slots=2, embeddings=emb)
+        st.bind(w)
+        if overlap:
+            st.enable_overlap()
+        outs = [torch.empty(B * S, H, device="cuda") for _ in range(M)]
+        rt = runtime.StageRuntime(st, 0, 2, M, needs_input_grad=False)
+        for _ in range(2):
+            st.refresh_weights()
+            st.zero_grads()
+            rt.step(ids, dys, outs)
+        st.sync()
+        res.append(([o.cpu() for o in outs], {k: v.cpu().clone() for k, v in st.grads.items()}))
+        st.close()
+    for a, b in zip(res[0][0], res[1][0]):
+        assert torch.equal(a, b)
+    for k in res[0][1]:
+        a, b = res[0][1][k], res[1][1][k]
+        assert float((a - b).abs().max()) <= 1e-5 * float(a.abs().max()) + 1e-10, k
