@@ -172,6 +172,8 @@ struct GnmtStage : ds_stage {
   }
 
   size_t workspace_bytes() const override { return ws_bytes; }
+  // forward touches its stash slot and its output only; the workspace is backward's
+  bool overlap_safe() const override { return true; }
   size_t stash_bytes(int slots) const override { return slot_bytes * (size_t)slots; }
   int refresh_weights() override { return DS_OK; }  // fp32 kernels are used in place
 

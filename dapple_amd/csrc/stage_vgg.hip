@@ -126,7 +126,7 @@ struct VggStage : ds_stage {
   char* stash_base = nullptr;
   size_t slot_bytes = 0;
   char* ws_base = nullptr;
-  size_t ws_bytes = 0, ws_g[2], ws_col, ws_dwpad;
+  size_t ws_bytes = 0, ws_g[2], ws_col, ws_fcol, ws_dwpad;
   char* wc_base = nullptr;
   std::vector<float*> wflip;  // per op (conv with dgrad), else null
   float* wpad = nullptr;      // first conv when cin % 32 != 0: [kpad, cout]
@@ -180,6 +180,7 @@ struct VggStage : ds_stage {
     if (first.cout > 0 && first.cin % 32 != 0) {
       kpad = ((9 * first.cin + 31) / 32) * 32;
       ws_col = wa.reserve((size_t)N * first.h * first.w * kpad * 4);
+      ws_fcol = wa.reserve((size_t)N * first.h * first.w * kpad * 4);  // forward's own patch matrix: backward keeps ws_col
       ws_dwpad = wa.reserve((size_t)kpad * first.cout * 4);
     }
     ws_bytes = wa.used;
@@ -203,6 +204,8 @@ struct VggStage : ds_stage {
   }
 
   size_t workspace_bytes() const override { return ws_bytes; }
+  // forward writes its stash slot, its output and its own patch matrix; the rest of the workspace is backward's
+  bool overlap_safe() const override { return true; }
   size_t stash_bytes(int slots) const override { return slot_bytes * (size_t)slots; }
 
   int refresh_weights() override {
@@ -241,7 +244,7 @@ struct VggStage : ds_stage {
           DS_PROPAGATE(ds_conv3x3_fwd(DS_F32, N, o.h, o.w, o.cin, o.cout, x, w[o.widx], w[o.widx + 1],
                                       DS_EPI_BIAS | DS_EPI_RELU, nullptr, y, stream));
         } else {
-          float* col = (float*)(ws_base + ws_col);
+          float* col = (float*)(ws_base + ws_fcol);
           DS_PROPAGATE(im2col(o, x, col));
           ds_gemm_desc d;
           memset(&d, 0, sizeof(d));

@@ -187,14 +187,45 @@ def test_forward_backward_overlap_matches_serial():
 
 
 @pytest.mark.gpu
-def test_overlap_refused_where_passes_share_workspace():
+def test_forward_backward_overlap_vgg_and_gnmt():
+    """The convolution and LSTM stages on two streams (their forward passes keep off backward's workspace)
+    against the one-stream run: same outputs bit for bit, gradients up to the order of the atomic adds."""
+    import numpy as np
     from dapple_amd import runtime, synthetic
-    layers = synthetic.vgg_layers([8, None])
-    st = runtime.vgg_stage(layers, 1, 8, 8, 3, 1)
-    assert not st.overlap_supported()
-    with pytest.raises(ValueError):
-        st.enable_overlap()
-    st.close()
+    r = np.random.default_rng(5)
+    layers = synthetic.vgg_layers([32, 32, None, 64])
+    M = 4
+    cases = []
+    imgs = [torch.as_tensor(r.standard_normal((2, 8, 8, 3)).astype(np.float32)).cuda() for _ in range(M)]
+    cases.append(("vgg", lambda: runtime.vgg_stage(layers, 2, 8, 8, 3, 3), synthetic.vgg_weights(6, layers, 3), imgs,
+                  dict(variant="2S-1", needs_input_grad=False)))
+    ids = [torch.as_tensor(r.integers(0, 20, (4, 5)).astype(np.int32)).cuda() for _ in range(M)]
+    cases.append(("gnmt", lambda: runtime.gnmt_stage(3, 16, 20, 4, 5, 2), synthetic.gnmt_weights(7, 3, 16, 20), ids,
+                  dict(needs_input_grad=False)))
+    for name, make, w, xs, kw in cases:
+        res = []
+        for overlap in (False, True):
+            st = make()
+            st.bind(w)
+            assert st.overlap_supported()
+            if overlap:
+                st.enable_overlap()
+            outs = [torch.empty(st.out_shape, device="cuda") for _ in range(M)]
+            dys = [torch.as_tensor(r.standard_normal(tuple(st.out_shape)).astype(np.float32)).cuda() for _ in range(M)] \
+                if not res else res[0][2]
+            rt = runtime.StageRuntime(st, 0, 2, M, **kw)
+            for _ in range(2):
+                st.refresh_weights()
+                st.zero_grads()
+                rt.step(xs, dys, outs)
+            st.sync()
+            res.append(([o.cpu() for o in outs], {k: v.cpu().clone() for k, v in st.grads.items()}, dys))
+            st.close()
+        for a, b in zip(res[0][0], res[1][0]):
+            assert torch.equal(a, b), name
+        for k in res[0][1]:
+            a, b = res[0][1][k], res[1][1][k]
+            assert float((a - b).abs().max()) <= 1e-5 * float(a.abs().max()) + 1e-10, (name, k)
 
 
 @pytest.mark.gpu
