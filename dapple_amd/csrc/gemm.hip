@@ -457,6 +457,17 @@ template <> struct RawFrag<bf16, DS_MN_MAJOR> { s16x4 lo, hi; };
 template <> struct RawFrag<float, DS_MN_MAJOR> { float e0, e1, e2, e3; };
 
 template <typename T> __device__ __forceinline__ void lds_wait(RawFrag<T, DS_K_MAJOR>& r) { lds_wait1(r.v); }
+// Waits until at most N LDS reads are outstanding (they complete in order: everything but the newest N has
+// arrived) and names the fragment registers as in/out operands so that nothing using them moves above it.
+template <int N, typename T> __device__ __forceinline__ void lds_wait_n(RawFrag<T, DS_K_MAJOR>& r) {
+  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(r.v) : "n"(N));
+}
+template <int N> __device__ __forceinline__ void lds_wait_n(RawFrag<bf16, DS_MN_MAJOR>& r) {
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(r.lo), "+v"(r.hi) : "n"(N));
+}
+template <int N> __device__ __forceinline__ void lds_wait_n(RawFrag<float, DS_MN_MAJOR>& r) {
+  asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(r.e0), "+v"(r.e1), "+v"(r.e2), "+v"(r.e3) : "n"(N));
+}
 __device__ __forceinline__ void lds_wait(RawFrag<bf16, DS_MN_MAJOR>& r) {
   asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r.lo), "+v"(r.hi));
 }
@@ -477,6 +488,8 @@ __device__ __forceinline__ f32x4 to_frag(const RawFrag<float, DS_MN_MAJOR>& r) {
 // Per-lane byte offsets (inside one operand tile) of the MFMA fragments a wave reads.
 template <typename T, int W, int MAJOR, int NF> struct FragReader {
   static constexpr int ROW_BYTES = W * (int)sizeof(T);
+  // LDS read instructions per fragment
+  static constexpr int READS = MAJOR == DS_K_MAJOR ? 1 : (sizeof(T) == 2 ? 2 : 4);
   typedef RawFrag<T, MAJOR> Raw;
   uint32_t off[MAJOR == DS_K_MAJOR ? 4 : NF];
 
@@ -527,6 +540,7 @@ template <typename T, int W, int MAJOR, int NF> struct FragReader {
 // accumulators of rows/columns the epilogue never stores.
 typedef __attribute__((address_space(3))) void* lds_vptr;
 typedef __attribute__((address_space(1))) void* glb_vptr;
+__device__ __forceinline__ lds_vptr lds_at(uint32_t a) { return (lds_vptr)(uintptr_t)a; }
 
 template <typename T, int W, int MAJOR> struct PlainDma {
   static constexpr int VEC = Vec16<T>::N;
@@ -561,14 +575,74 @@ template <typename T, int W, int MAJOR> struct PlainDma {
     }
   }
   // load i of the current k-tile (i = 0 .. NV-1, each exactly once per k-tile), then advance()
-  __device__ __forceinline__ void issue_one(char* lds, int wave, int i) {
-    __builtin_amdgcn_global_load_lds((glb_vptr)src[i], (lds_vptr)(lds + (i * 4 + wave) * 1024), 16, 0, 0);
+  __device__ __forceinline__ void issue_one(uint32_t lds_tile, int wave, int i) {
+    __builtin_amdgcn_global_load_lds((glb_vptr)src[i], lds_at(lds_tile + (i * 4 + wave) * 1024), 16, 0, 0);
     src[i] += step;
   }
   __device__ __forceinline__ void advance() {}
-  __device__ __forceinline__ void issue(char* lds, int wave) {
+  __device__ __forceinline__ void issue(uint32_t lds_tile, int wave) {
 #pragma unroll
-    for (int i = 0; i < NV; ++i) issue_one(lds, wave, i);
+    for (int i = 0; i < NV; ++i) issue_one(lds_tile, wave, i);
+    advance();
+  }
+};
+
+// Same tiles as PlainDma, loads written as inline asm in the scalar-base form
+//   global_load_lds_dwordx4 v_offset, s[base:base+1]     (M0 = LDS address of the wave's 1 KiB slot)
+// A lane's 32-bit byte offset inside the operand tile never changes; the tile base is a uniform pointer
+// advanced once per k-tile with scalar adds, so a load costs no vector ALU work at all.  The compiler does
+// not know these are memory operations: every wait on them is an explicit s_waitcnt in the kernel.
+template <typename T, int W, int MAJOR> struct AsmDma {
+  static constexpr int VEC = Vec16<T>::N;
+  static constexpr int KT = Mma<T>::KT;
+  static constexpr int NV = W / 32;
+  static constexpr int ROW_BYTES = W * (int)sizeof(T);
+  static constexpr int CPR = ROW_BYTES / 16;
+  uint32_t voff[NV];
+  uint64_t tile;      // uniform: address of the current k-tile of this block's operand panel
+  int64_t step;       // bytes from one k-tile to the next
+
+  // a value that is the same in every lane, moved to scalar registers so that it can be an asm "s" operand
+  static __device__ __forceinline__ uint64_t uniform64(uint64_t v) {
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return ((uint64_t)hi << 32) | lo;
+  }
+
+  __device__ __forceinline__ void init(const GemmArgs&, const T* base, int64_t ld, int f0, int F, int kt0, int wave, int lane) {
+    const int64_t k0 = (int64_t)kt0 * KT;
+    if (MAJOR == DS_K_MAJOR) {
+      tile = uniform64((uint64_t)(uintptr_t)(base + (int64_t)f0 * ld + k0));
+      step = (int64_t)uniform64((uint64_t)((int64_t)KT * sizeof(T)));
+    } else {
+      tile = uniform64((uint64_t)(uintptr_t)(base + k0 * ld + f0));
+      step = (int64_t)uniform64((uint64_t)((int64_t)KT * ld * sizeof(T)));
+    }
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int p = (i * 4 + wave) * 64 + lane;
+      if (MAJOR == DS_K_MAJOR) {
+        const int row = p >> 3, c = (p & 7) ^ kmajor_swz(row);
+        int f = f0 + row;
+        if (f > F - 1) f = F - 1;
+        voff[i] = (uint32_t)(((int64_t)(f - f0) * ld + c * VEC) * (int64_t)sizeof(T));
+      } else {
+        const int r = p / CPR, pc = p % CPR;
+        const int g = (pc >> 1) ^ mnmajor_swz<ROW_BYTES>(r);
+        int f = f0 + (g * 2 + (pc & 1)) * VEC;
+        if (f > F - VEC) f = F - VEC;
+        voff[i] = (uint32_t)(((int64_t)r * ld + (f - f0)) * (int64_t)sizeof(T));
+      }
+    }
+  }
+  // load i of the current k-tile into the wave's slot of the tile buffer at LDS address `lds_tile`
+  __device__ __forceinline__ void issue_one(uint32_t lds_tile, int wave_s, int i) {
+    const uint32_t m0v = lds_tile + (uint32_t)(i * 4 + wave_s) * 1024u;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0v), "v"(voff[i]), "s"(tile) : "memory", "m0");
+  }
+  __device__ __forceinline__ void advance() { tile += (uint64_t)step; }
+  __device__ __forceinline__ void issue(uint32_t lds_tile, int wave_s) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) issue_one(lds_tile, wave_s, i);
     advance();
   }
 };
@@ -635,13 +709,13 @@ template <typename T, int W, int MODE> struct ConvDma {
     }
   }
   // load i of the current k-tile (i = 0 .. NV-1, each exactly once per k-tile), then advance()
-  __device__ __forceinline__ void issue_one(char* lds, int wave, int i) {
+  __device__ __forceinline__ void issue_one(uint32_t lds_tile, int wave, int i) {
     if (MODE == 1) {
       const int dy = tap / 3 - 1, dx = tap - (tap / 3) * 3 - 1;
       const int sh = (dy * Wd + dx) * C + c0;
       const bool ok = (unsigned)(y[i] + dy) < (unsigned)H && (unsigned)(x[i] + dx) < (unsigned)Wd;
       const T* src = ok ? base + off[i] + sh : reinterpret_cast<const T*>(g_zero16);
-      __builtin_amdgcn_global_load_lds((glb_vptr)src, (lds_vptr)(lds + (i * 4 + wave) * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((glb_vptr)src, lds_at(lds_tile + (i * 4 + wave) * 1024), 16, 0, 0);
     } else {
       const int64_t pix = pix0 + r[i];
       const int q = (int)(pix / Wd);
@@ -649,7 +723,7 @@ template <typename T, int W, int MODE> struct ConvDma {
       const int dy = (dyx[i] >> 2) - 1, dx = (dyx[i] & 3) - 1;
       const bool ok = (unsigned)(yy + dy) < (unsigned)H && (unsigned)(xx + dx) < (unsigned)Wd;
       const T* src = ok ? base + pix * C + shift[i] : reinterpret_cast<const T*>(g_zero16);
-      __builtin_amdgcn_global_load_lds((glb_vptr)src, (lds_vptr)(lds + (i * 4 + wave) * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((glb_vptr)src, lds_at(lds_tile + (i * 4 + wave) * 1024), 16, 0, 0);
     }
   }
   __device__ __forceinline__ void advance() {
@@ -660,14 +734,14 @@ template <typename T, int W, int MODE> struct ConvDma {
       pix0 += KT;
     }
   }
-  __device__ __forceinline__ void issue(char* lds, int wave) {
+  __device__ __forceinline__ void issue(uint32_t lds_tile, int wave) {
 #pragma unroll
-    for (int i = 0; i < NV; ++i) issue_one(lds, wave, i);
+    for (int i = 0; i < NV; ++i) issue_one(lds_tile, wave, i);
     advance();
   }
 };
 
-template <typename T, int W, int MAJOR, int CONV> struct DmaSelect { typedef PlainDma<T, W, MAJOR> type; };
+template <typename T, int W, int MAJOR, int CONV> struct DmaSelect { typedef AsmDma<T, W, MAJOR> type; };
 template <typename T, int W> struct DmaSelect<T, W, DS_K_MAJOR, 1> { typedef ConvDma<T, W, 1> type; };
 template <typename T, int W> struct DmaSelect<T, W, DS_MN_MAJOR, 2> { typedef ConvDma<T, W, 2> type; };
 
@@ -677,7 +751,7 @@ template <typename T, int W> struct DmaSelect<T, W, DS_MN_MAJOR, 2> { typedef Co
 template <typename T, int BM, int BN, int AMAJ, int BMAJ, int STAGES, int CONVA = 0>
 __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
   typedef typename DmaSelect<T, BM, AMAJ, CONVA>::type DA;
-  typedef PlainDma<T, BN, BMAJ> DB;
+  typedef AsmDma<T, BN, BMAJ> DB;
   constexpr int KT = Mma<T>::KT;
   constexpr int TM = BM / 64, TN = BN / 64;
   constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE_BYTES = A_BYTES + B_BYTES;
@@ -713,30 +787,39 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
   DB db;
   da.init(p, A, p.lda, m0, p.m, kt_begin, wave, lane);
   db.init(p, B, p.ldb, n0, p.n, kt_begin, wave, lane);
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);  // scalar copy: LDS slot addresses stay in SGPRs
+  const uint32_t lds0 = lds_addr(lds);
   // Ring of STAGES tile buffers, tile t in buffer t % STAGES.  All STAGES buffers are filled up front.
-  // Inside tile kt, before the MFMAs of its last k-step: every wave has read all of tile kt (its
+  // Inside tile kt, under the first MFMA of its last k-step: every wave has read all of tile kt (its
   // fragment reads are waited for), waits for its own loads of tile kt+1 and meets the others at the
   // one barrier of the k-tile.  After it, tile kt+1 is visible, its first fragments are fetched under
   // the remaining MFMAs of tile kt, and buffer kt % STAGES is free: the loads of tile kt+STAGES go
   // there, issued one at a time between the next 4*TM*TN MFMAs (last k-step of tile kt, first three of
-  // tile kt+1).  A wave stalls on a load instruction while the address unit is busy; issued as one
-  // burst those stalls would sit in front of the MFMAs instead of underneath them.
+  // tile kt+1).  On this part a wave's load instruction and its MFMAs only overlap when they alternate
+  // in ONE instruction stream (a loader wave beside an MFMA wave on the same SIMD makes no progress at
+  // all while the MFMAs run), and a fragment read issued between two MFMAs is free while a block of
+  // reads in front of them is not: the order below is pinned with scheduling barriers.
 #pragma unroll
   for (int s = 0; s < STAGES; ++s) {
     if (s < nkt) {
-      da.issue(lds + s * STAGE_BYTES, wave);
-      db.issue(lds + s * STAGE_BYTES + A_BYTES, wave);
+      da.issue(lds0 + s * STAGE_BYTES, wave_s);
+      db.issue(lds0 + s * STAGE_BYTES + A_BYTES, wave_s);
     }
   }
   FragReader<T, BM, AMAJ, TM> ra;
   FragReader<T, BN, BMAJ, TN> rb;
   ra.init(wm * (BM / 2), lane);
   rb.init(wn * (BN / 2), lane);
-  const uint32_t lds0 = lds_addr(lds);
-  constexpr int NMMA = 4 * TM * TN;   // MFMA groups per k-tile
-  constexpr int TAIL = TM * TN;       // of which the last k-step holds this many
-  RawFrag<T, AMAJ> fa[2][TM];
-  RawFrag<T, BMAJ> fb[2][TN];
+  constexpr int NSLOT = TM * TN;      // MFMA groups per k-step
+  constexpr int NMMA = 4 * NSLOT;     // per k-tile
+  constexpr int NFR = TM + TN;        // fragments per k-step
+  // Fragments run two k-steps ahead of the MFMAs in four register sets (set = k-step).  LDS reads complete
+  // in order, so "at most one k-step's reads outstanding" means the older set has arrived; the lgkmcnt field
+  // has 4 bits, a k-step with more reads than that waits for everything instead.
+  constexpr int RPS = TM * FragReader<T, BM, AMAJ, TM>::READS + TN * FragReader<T, BN, BMAJ, TN>::READS;
+  constexpr int WAITN = RPS <= 15 ? RPS : 0;
+  RawFrag<T, AMAJ> fa[4][TM];
+  RawFrag<T, BMAJ> fb[4][TN];
   {
     // tile 0 is complete once only the tiles issued after it are outstanding
     const int later = (nkt < STAGES ? nkt : STAGES) - 1;
@@ -746,9 +829,12 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
     else __builtin_amdgcn_s_waitcnt(DS_VMCNT(0));
     __builtin_amdgcn_s_barrier();
 #pragma unroll
-    for (int i = 0; i < TM; ++i) ra.read(fa[0][i], lds0, i, 0);
+    for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
-    for (int j = 0; j < TN; ++j) rb.read(fb[0][j], lds0 + A_BYTES, j, 0);
+      for (int i = 0; i < TM; ++i) ra.read(fa[ks][i], lds0, i, ks);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) rb.read(fb[ks][j], lds0 + A_BYTES, j, ks);
+    }
   }
   int buf = 0;  // kt % STAGES
   for (int kt = 0; kt < nkt; ++kt) {
@@ -760,62 +846,80 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
     const bool has_next = kt + 1 < nkt;
     int nbuf = buf + 1;
     if (nbuf == STAGES) nbuf = 0;
+    const uint32_t prev_tile = lds0 + pb * STAGE_BYTES, next_tile = lds0 + nbuf * STAGE_BYTES;
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      const int cur = ks & 1, nxt = cur ^ 1;
-#pragma unroll
-      for (int i = 0; i < TM; ++i) lds_wait(fa[cur][i]);
-#pragma unroll
-      for (int j = 0; j < TN; ++j) lds_wait(fb[cur][j]);
+      // set ks must have arrived; the set issued after it (k-step ks+1) may still be in flight
       if (ks < 3) {
 #pragma unroll
-        for (int i = 0; i < TM; ++i) ra.read(fa[nxt][i], sa, i, ks + 1);
+        for (int i = 0; i < TM; ++i) lds_wait_n<WAITN>(fa[ks][i]);
 #pragma unroll
-        for (int j = 0; j < TN; ++j) rb.read(fb[nxt][j], sb, j, ks + 1);
-      } else if (has_next) {
-        // tile kt+1 is complete once only the tiles issued after it are outstanding:
-        // kt+2 .. kt-1+STAGES, as far as they exist
-        int later = nkt - (kt + 2);
-        if (later > STAGES - 2) later = STAGES - 2;
-        if (later >= 2) __builtin_amdgcn_s_waitcnt(DS_VMCNT(LPT * 2));
-        else if (later == 1) __builtin_amdgcn_s_waitcnt(DS_VMCNT(LPT));
-        else __builtin_amdgcn_s_waitcnt(DS_VMCNT(0));
-        __builtin_amdgcn_s_barrier();
-        const uint32_t na = lds0 + nbuf * STAGE_BYTES;
+        for (int j = 0; j < TN; ++j) lds_wait_n<WAITN>(fb[ks][j]);
+      } else {
 #pragma unroll
-        for (int i = 0; i < TM; ++i) ra.read(fa[nxt][i], na, i, 0);
+        for (int i = 0; i < TM; ++i) lds_wait(fa[ks][i]);
 #pragma unroll
-        for (int j = 0; j < TN; ++j) rb.read(fb[nxt][j], na + A_BYTES, j, 0);
+        for (int j = 0; j < TN; ++j) lds_wait(fb[ks][j]);
       }
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-          Mma<T>::mma(acc[i][j], to_frag(fa[cur][i]), to_frag(fb[cur][j]));
-          const int q = (ks * TM + i) * TN + j;  // compile-time after unrolling
+          const int slot = i * TN + j;            // compile-time after unrolling
+          const int q = ks * NSLOT + slot;
+          Mma<T>::mma(acc[i][j], to_frag(fa[ks][i]), to_frag(fb[ks][j]));
+          __builtin_amdgcn_sched_barrier(0);
+          if (ks == 3 && slot == 0 && has_next) {
+            // tile kt+1 is complete once only the tiles issued after it are outstanding:
+            // kt+2 .. kt-1+STAGES, as far as they exist
+            int later = nkt - (kt + 2);
+            if (later > STAGES - 2) later = STAGES - 2;
+            if (later >= 2) __builtin_amdgcn_s_waitcnt(DS_VMCNT(LPT * 2));
+            else if (later == 1) __builtin_amdgcn_s_waitcnt(DS_VMCNT(LPT));
+            else __builtin_amdgcn_s_waitcnt(DS_VMCNT(0));
+            __builtin_amdgcn_s_barrier();
+          }
+          // this slot's share of the fragment reads: k-steps 2 and 3 of this tile during k-steps 0 and 1, nothing
+          // during k-step 2 (the next tile is not visible yet), k-steps 0 AND 1 of the next tile during k-step 3
+          if (ks < 2) {
+#pragma unroll
+            for (int r = 0; r < NFR; ++r)
+              if ((r * NSLOT) / NFR == slot) {
+                if (r < TM) ra.read(fa[ks + 2][r], sa, r, ks + 2);
+                else rb.read(fb[ks + 2][r - TM], sb, r - TM, ks + 2);
+              }
+          } else if (ks == 3 && has_next) {
+#pragma unroll
+            for (int r = 0; r < 2 * NFR; ++r)
+              if ((r * NSLOT) / (2 * NFR) == slot) {
+                const int nks = r / NFR, rr = r % NFR;
+                if (rr < TM) ra.read(fa[nks][rr], next_tile, rr, nks);
+                else rb.read(fb[nks][rr - TM], next_tile + A_BYTES, rr - TM, nks);
+              }
+          }
+          // this slot's share of the refill loads
           if (ks < 3) {
-            // slots TAIL .. NMMA-1 of the window that refills the buffer of tile kt-1
+            // slots NSLOT .. NMMA-1 of the window that refills the buffer of tile kt-1
             if (refill_prev) {
-              char* const ra_dst = lds + pb * STAGE_BYTES;
 #pragma unroll
               for (int l = 0; l < LPT; ++l)
-                if ((l * NMMA) / LPT == q + TAIL) {
-                  if (l < DA::NV) da.issue_one(ra_dst, wave, l);
-                  else db.issue_one(ra_dst + A_BYTES, wave, l - DA::NV);
+                if ((l * NMMA) / LPT == q + NSLOT) {
+                  if (l < DA::NV) da.issue_one(prev_tile, wave_s, l);
+                  else db.issue_one(prev_tile + A_BYTES, wave_s, l - DA::NV);
                 }
             }
           } else {
-            // slots 0 .. TAIL-1 of the window that refills the buffer of tile kt
+            // slots 0 .. NSLOT-1 of the window that refills the buffer of tile kt
             if (refill_cur) {
-              char* const rc_dst = lds + buf * STAGE_BYTES;
 #pragma unroll
               for (int l = 0; l < LPT; ++l)
-                if ((l * NMMA) / LPT == q - 3 * TAIL) {
-                  if (l < DA::NV) da.issue_one(rc_dst, wave, l);
-                  else db.issue_one(rc_dst + A_BYTES, wave, l - DA::NV);
+                if ((l * NMMA) / LPT == slot) {
+                  if (l < DA::NV) da.issue_one(sa, wave_s, l);
+                  else db.issue_one(sb, wave_s, l - DA::NV);
                 }
             }
           }
+          __builtin_amdgcn_sched_barrier(0);
         }
       if (ks == 2 && refill_prev) { da.advance(); db.advance(); }
     }
