@@ -13,6 +13,7 @@
 //                     g ^ (((r & 3) << 1) & (granules-1)).  bf16 fragments come from
 //                     ds_read_b64_tr_b16 (a 4x16 transpose per 16 lanes), fp32 from 4-byte loads.
 #include <stdlib.h>
+#include <type_traits>
 #include <string.h>
 
 #include "common.h"
@@ -837,13 +838,16 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
     }
   }
   int buf = 0;  // kt % STAGES
-  for (int kt = 0; kt < nkt; ++kt) {
+  // One k-tile.  `steady` (a compile-time flag) says that tile kt-1+STAGES and tile kt+STAGES both exist: then
+  // every refill load and fragment read below is unconditional and the k-tile is one straight run of code.
+  auto k_tile = [&](auto steady, int kt) {
+    constexpr bool ST = decltype(steady)::value;
     const uint32_t sa = lds0 + buf * STAGE_BYTES, sb = sa + A_BYTES;
     int pb = buf - 1;  // buffer of tile kt-1, being refilled with tile kt-1+STAGES
     if (pb < 0) pb += STAGES;
-    const bool refill_prev = kt >= 1 && kt - 1 + STAGES < nkt;
-    const bool refill_cur = kt + STAGES < nkt;
-    const bool has_next = kt + 1 < nkt;
+    const bool refill_prev = ST || (kt >= 1 && kt - 1 + STAGES < nkt);
+    const bool refill_cur = ST || kt + STAGES < nkt;
+    const bool has_next = ST || kt + 1 < nkt;
     int nbuf = buf + 1;
     if (nbuf == STAGES) nbuf = 0;
     const uint32_t prev_tile = lds0 + pb * STAGE_BYTES, next_tile = lds0 + nbuf * STAGE_BYTES;
@@ -872,7 +876,7 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
           if (ks == 3 && slot == 0 && has_next) {
             // tile kt+1 is complete once only the tiles issued after it are outstanding:
             // kt+2 .. kt-1+STAGES, as far as they exist
-            int later = nkt - (kt + 2);
+            int later = ST ? STAGES - 2 : nkt - (kt + 2);
             if (later > STAGES - 2) later = STAGES - 2;
             if (later >= 2) __builtin_amdgcn_s_waitcnt(DS_VMCNT(LPT * 2));
             else if (later == 1) __builtin_amdgcn_s_waitcnt(DS_VMCNT(LPT));
@@ -924,7 +928,12 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
       if (ks == 2 && refill_prev) { da.advance(); db.advance(); }
     }
     buf = nbuf;
-  }
+  };
+  // three loops, so that the straight-line steady state does not share an iteration with the general form
+  int kt = 0;
+  for (; kt < nkt && !(kt >= 1 && kt + STAGES < nkt); ++kt) k_tile(std::false_type(), kt);
+  for (; kt + STAGES < nkt; ++kt) k_tile(std::true_type(), kt);
+  for (; kt < nkt; ++kt) k_tile(std::false_type(), kt);
   if (p.vec_epi) gemm_epilogue_staged<T, BM, BN>(p, acc, m0, n0, wm, wn, lane, tid, c_off, lds);
   else gemm_epilogue<T, BM, BN>(p, acc, m0, n0, wm, wn, lane, c_off);
 }
