@@ -13,6 +13,7 @@ DS_F32, DS_BF16 = 0, 1
 DS_K_MAJOR, DS_MN_MAJOR = 0, 1
 DS_EPI_BIAS, DS_EPI_RESIDUAL, DS_EPI_GELU, DS_EPI_DGELU = 1, 2, 4, 8
 DS_EPI_OUT_F32, DS_EPI_ACCUM, DS_EPI_RELU, DS_EPI_MASK, DS_EPI_TANH_FORM = 16, 32, 64, 128, 256
+DS_EPI_GELU_GRAD, DS_EPI_MUL = 512, 1024
 DS_STAGE_BERT, DS_STAGE_VGG19, DS_STAGE_GNMT, DS_STAGE_XLNET = 0, 1, 2, 3
 
 

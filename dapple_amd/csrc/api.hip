@@ -73,6 +73,7 @@ extern "C" const char* ds_last_error(void) { return g_err; }
 extern "C" const char* ds_build_target(void) { return "gfx950"; }
 
 // ---------------------------------------------------------------- stage handle dispatch
+#include <stdlib.h>
 #include <string.h>
 
 #include "stage.h"

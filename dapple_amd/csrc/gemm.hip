@@ -198,14 +198,16 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, f32x16 (&acc)[B
         float v = acc[i][j][e] * p.alpha + bias;
         if (flags & DS_EPI_RESIDUAL) v += to_f32(R[idx]);
         if (flags & DS_EPI_DGELU) v *= gelu_any_grad(to_f32(C2[idx]), tanh_form);
+        if (flags & DS_EPI_MUL) v *= to_f32(C2[idx]);
         if (flags & DS_EPI_RELU) v = fmaxf(v, 0.f);
         if (flags & DS_EPI_MASK) v = to_f32(C2[idx]) > 0.f ? v : 0.f;
         if (flags & DS_EPI_ACCUM) {
           if (p.splitk > 1) atomicAdd(Cf + idx, v); else Cf[idx] += v;
-        } else if (out_f32) {
-          Cf[idx] = v;
         } else {
-          Ct[idx] = from_f32<T>(v);
+          // with DS_EPI_GELU_GRAD the tensor kept for backward is gelu'(v) instead of the pre-activation v
+          const float keep = (flags & DS_EPI_GELU_GRAD) ? gelu_any_grad(v, tanh_form) : v;
+          if (out_f32) Cf[idx] = keep;
+          else Ct[idx] = from_f32<T>(keep);
         }
         if (flags & DS_EPI_GELU) C2[idx] = from_f32<T>(gelu_any(v, tanh_form));
       }
@@ -314,9 +316,30 @@ __device__ __forceinline__ void gemm_epilogue_staged(const GemmArgs& p, f32x16 (
         for (int e = 0; e < 4; ++e) { x[e] *= gelu_any_grad(a0[e], tanh_form); x[4 + e] *= gelu_any_grad(a1[e], tanh_form); }
       }
     }
+    if (flags & DS_EPI_MUL) {
+      if (sizeof(T) == 2) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(C2 + idx);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] *= (float)a[e];
+      } else {
+        const f32x4 a0 = *reinterpret_cast<const f32x4*>(C2 + idx), a1 = *reinterpret_cast<const f32x4*>(C2 + idx + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { x[e] *= a0[e]; x[4 + e] *= a1[e]; }
+      }
+    }
     if (flags & DS_EPI_RELU) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) x[e] = fmaxf(x[e], 0.f);
+    }
+    // GELU outputs first (they need the pre-activation), then what is kept for backward
+    float act[8];
+    if (flags & DS_EPI_GELU) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) act[e] = gelu_any(x[e], tanh_form);
+      if (flags & DS_EPI_GELU_GRAD) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = gelu_any_grad(x[e], tanh_form);
+      }
     }
     if (flags & DS_EPI_MASK) {
       if (sizeof(T) == 2) {
@@ -356,12 +379,12 @@ __device__ __forceinline__ void gemm_epilogue_staged(const GemmArgs& p, f32x16 (
       if (sizeof(T) == 2) {
         bf16x8 o;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) o[e] = (bf16)gelu_any(x[e], tanh_form);
+        for (int e = 0; e < 8; ++e) o[e] = (bf16)act[e];
         *reinterpret_cast<bf16x8*>(reinterpret_cast<bf16*>(p.c2) + c_off + idx) = o;
       } else {
         f32x4 c0, c1;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) { c0[e] = gelu_any(x[e], tanh_form); c1[e] = gelu_any(x[4 + e], tanh_form); }
+        for (int e = 0; e < 4; ++e) { c0[e] = act[e]; c1[e] = act[4 + e]; }
         *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.c2) + c_off + idx) = c0;
         *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.c2) + c_off + idx + 4) = c1;
       }
@@ -836,6 +859,13 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
 #pragma unroll
       for (int j = 0; j < TN; ++j) rb.read(fb[ks][j], lds0 + A_BYTES, j, ks);
     }
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {  // landed before the loops are entered (see the end of k_tile)
+#pragma unroll
+      for (int i = 0; i < TM; ++i) lds_wait(fa[ks][i]);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) lds_wait(fb[ks][j]);
+    }
   }
   int buf = 0;  // kt % STAGES
   // One k-tile.  `steady` (a compile-time flag) says that tile kt-1+STAGES and tile kt+STAGES both exist: then
@@ -926,6 +956,18 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
           __builtin_amdgcn_sched_barrier(0);
         }
       if (ks == 2 && refill_prev) { da.advance(); db.advance(); }
+    }
+    // No LDS read may be in flight across a loop back-edge or between the loops below: the compiler is free
+    // to copy a fragment register there, and a copy taken before the data has landed copies stale contents.
+    // The first two k-steps of the next tile, fetched under the last four MFMA groups, are waited for here.
+    if (has_next) {
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) lds_wait(fa[ks][i]);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) lds_wait(fb[ks][j]);
+      }
     }
     buf = nbuf;
   };
@@ -1049,7 +1091,8 @@ static int gemm_run(const ds_gemm_desc* d, int splitk_req, void* stream) {
   const int f = d->flags;
   if (f & DS_EPI_BIAS) DS_CHECK_ARG(d->bias != nullptr, "ds_gemm: DS_EPI_BIAS without bias");
   if (f & DS_EPI_RESIDUAL) DS_CHECK_ARG(d->residual != nullptr, "ds_gemm: DS_EPI_RESIDUAL without residual");
-  if (f & (DS_EPI_GELU | DS_EPI_DGELU)) DS_CHECK_ARG(d->c2 != nullptr, "ds_gemm: GELU epilogue without c2");
+  if (f & (DS_EPI_GELU | DS_EPI_DGELU | DS_EPI_MUL)) DS_CHECK_ARG(d->c2 != nullptr, "ds_gemm: GELU / MUL epilogue without c2");
+  DS_CHECK_ARG(!(f & DS_EPI_GELU_GRAD) || (f & DS_EPI_GELU), "ds_gemm: DS_EPI_GELU_GRAD needs DS_EPI_GELU");
   DS_CHECK_ARG(!((f & DS_EPI_GELU) && (f & DS_EPI_DGELU)), "ds_gemm: GELU and DGELU are exclusive");
   DS_CHECK_ARG(!((f & DS_EPI_ACCUM) && (f & (DS_EPI_GELU | DS_EPI_DGELU))), "ds_gemm: ACCUM with GELU");
   (void)esz;

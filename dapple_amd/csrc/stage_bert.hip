@@ -341,7 +341,7 @@ struct BertStage : ds_stage {
       DS_PROPAGATE(ds_layernorm_fwd(dtype, rows, H, sp + t.z1, w[b + LN1_G], w[b + LN1_B], cfg.ln_eps, sp + t.a,
                                     (float*)(sp + t.st1), stream));
       // intermediate dense + gelu (:983-987)
-      DS_PROPAGATE(gemm_fwd(rows, F, H, sp + t.a, weight_T(l, W_FF1), sp + t.u, DS_EPI_BIAS | DS_EPI_GELU, w[b + B_FF1],
+      DS_PROPAGATE(gemm_fwd(rows, F, H, sp + t.a, weight_T(l, W_FF1), sp + t.u, DS_EPI_BIAS | DS_EPI_GELU | DS_EPI_GELU_GRAD, w[b + B_FF1],
                             nullptr, sp + t.h));
       // output dense + residual + layer_norm (:991-996)
       DS_PROPAGATE(gemm_fwd(rows, H, F, sp + t.h, weight_T(l, W_FF2), sp + t.z2, DS_EPI_BIAS | DS_EPI_RESIDUAL,
@@ -378,7 +378,7 @@ struct BertStage : ds_stage {
       DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, dy, sp + t.z2, w[b + LN2_G], (const float*)(sp + t.st2), nullptr, dz2,
                                     g[b + LN2_G], g[b + LN2_B], g[b + B_FF2], stream));
       // du = (dz2 W2^T) * gelu'(u)
-      DS_PROPAGATE(gemm_dgrad(rows, H, F, dz2, weight_T(l, W_FF2), du, DS_EPI_DGELU, nullptr, sp + t.u));
+      DS_PROPAGATE(gemm_dgrad(rows, H, F, dz2, weight_T(l, W_FF2), du, DS_EPI_MUL, nullptr, sp + t.u));
       // da = du W1^T + dz2 (a also feeds the residual into z2)
       DS_PROPAGATE(gemm_dgrad(rows, F, H, du, weight_T(l, W_FF1), da, DS_EPI_RESIDUAL, dz2, nullptr));
       // attention-output LayerNorm; column sums of dz1 = gradient of attention/output/dense/bias

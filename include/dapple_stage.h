@@ -44,6 +44,8 @@ extern "C" {
 #define DS_EPI_RELU 64     /* C = max(acc + bias, 0) */
 #define DS_EPI_TANH_FORM 256 /* GELU / DGELU use the tanh approximation (xlnet/activations/gelu.py:6-11) */
 #define DS_EPI_MASK 128    /* C = aux[m][n] > 0 ? acc : 0 (ReLU backward), aux = c2 */
+#define DS_EPI_GELU_GRAD 512 /* with DS_EPI_GELU: C = gelu'(pre-activation) instead of the pre-activation */
+#define DS_EPI_MUL 1024    /* C = acc * aux[m][n], aux = c2 (backward through a GELU whose derivative was kept) */
 
 const char* ds_last_error(void);
 

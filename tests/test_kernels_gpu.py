@@ -97,6 +97,17 @@ def test_gemm_epilogues(dt):
     a64 = aux.cpu().double().requires_grad_(True)
     (gp,) = torch.autograd.grad(ob.gelu(a64).sum(), a64)
     assert_close(c, (x.cpu().double() @ w.cpu().double()) * gp, TOL[dt], "dgelu")
+    # gelu with its derivative kept for backward, then the multiply epilogue that consumes it
+    from dapple_amd._lib import DS_EPI_GELU_GRAD, DS_EPI_MUL
+    kept = torch.empty(m, n, dtype=DT[dt], device="cuda")
+    act2 = torch.empty_like(kept)
+    ops.gemm(x, w, kept, m, n, k, DS_K_MAJOR, DS_MN_MAJOR, flags=DS_EPI_BIAS | DS_EPI_GELU | DS_EPI_GELU_GRAD, bias=bias, c2=act2)
+    r64 = ref.clone().requires_grad_(True)
+    (gref,) = torch.autograd.grad(ob.gelu(r64).sum(), r64)
+    assert_close(act2, ob.gelu(ref), TOL[dt], "gelu (derivative kept)")
+    assert_close(kept, gref, TOL[dt], "kept gelu derivative")
+    ops.gemm(x, w, c, m, n, k, DS_K_MAJOR, DS_MN_MAJOR, flags=DS_EPI_MUL, c2=aux)
+    assert_close(c, (x.cpu().double() @ w.cpu().double()) * aux.cpu().double(), TOL[dt], "multiply epilogue")
     # fp32 output and accumulate (wgrad form: both operands MN-major), twice -> 2x + initial
     acc0 = r.standard_normal((k, n)).astype(np.float32)
     acc = dev(acc0)

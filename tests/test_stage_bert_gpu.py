@@ -163,7 +163,7 @@ def test_forward_backward_overlap_matches_serial():
     xs = [torch.as_tensor(x).cuda().bfloat16() for x in synthetic.bert_activation_inputs(12, M, B, S, H)]
     dys = [torch.as_tensor(x).cuda().bfloat16() for x in synthetic.upstream_grads(13, M, (B * S, H))]
     res = []
-    for overlap in (False, True):
+    for overlap in (False, True, True, True):     # several overlapped runs: a race would not show every time
         st = runtime.bert_stage(L, H, N, F, B, S, "bf16", stash_slots=2)
         st.bind(w)
         assert st.overlap_supported()
@@ -179,11 +179,12 @@ def test_forward_backward_overlap_matches_serial():
         st.sync()
         res.append(([o.float().cpu() for o in outs], [d.float().cpu() for d in dxs], {k: v.cpu().clone() for k, v in st.grads.items()}))
         st.close()
-    for a, b in zip(res[0][0] + res[0][1], res[1][0] + res[1][1]):
-        assert torch.equal(a, b)
-    for k in res[0][2]:
-        a, b = res[0][2][k], res[1][2][k]
-        assert float((a - b).abs().max()) <= 1e-5 * float(a.abs().max()) + 1e-12, k
+    for other in res[1:]:
+        for a, b in zip(res[0][0] + res[0][1], other[0] + other[1]):
+            assert torch.equal(a, b)
+        for k in res[0][2]:
+            a, b = res[0][2][k], other[2][k]
+            assert float((a - b).abs().max()) <= 1e-5 * float(a.abs().max()) + 1e-12, k
 
 
 @pytest.mark.gpu
