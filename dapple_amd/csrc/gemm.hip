@@ -877,7 +877,6 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
     if (pb < 0) pb += STAGES;
     const bool refill_prev = ST || (kt >= 1 && kt - 1 + STAGES < nkt);
     const bool refill_cur = ST || kt + STAGES < nkt;
-    const bool has_next = ST || kt + 1 < nkt;
     int nbuf = buf + 1;
     if (nbuf == STAGES) nbuf = 0;
     const uint32_t prev_tile = lds0 + pb * STAGE_BYTES, next_tile = lds0 + nbuf * STAGE_BYTES;
@@ -903,11 +902,14 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
           const int q = ks * NSLOT + slot;
           Mma<T>::mma(acc[i][j], to_frag(fa[ks][i]), to_frag(fb[ks][j]));
           __builtin_amdgcn_sched_barrier(0);
-          if (ks == 3 && slot == 0 && has_next) {
+          if (ks == 3 && slot == 0) {
+            // (also after the last tile, where it is a no-op wait and one more barrier: the fragment reads
+            // below must not sit inside a conditional, see the end of k_tile)
             // tile kt+1 is complete once only the tiles issued after it are outstanding:
             // kt+2 .. kt-1+STAGES, as far as they exist
             int later = ST ? STAGES - 2 : nkt - (kt + 2);
             if (later > STAGES - 2) later = STAGES - 2;
+            if (later < 0) later = 0;
             if (later >= 2) __builtin_amdgcn_s_waitcnt(DS_VMCNT(LPT * 2));
             else if (later == 1) __builtin_amdgcn_s_waitcnt(DS_VMCNT(LPT));
             else __builtin_amdgcn_s_waitcnt(DS_VMCNT(0));
@@ -922,7 +924,8 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
                 if (r < TM) ra.read(fa[ks + 2][r], sa, r, ks + 2);
                 else rb.read(fb[ks + 2][r - TM], sb, r - TM, ks + 2);
               }
-          } else if (ks == 3 && has_next) {
+          } else if (ks == 3) {
+            // after the last tile these read a stale buffer into registers nobody uses
 #pragma unroll
             for (int r = 0; r < 2 * NFR; ++r)
               if ((r * NSLOT) / (2 * NFR) == slot) {
@@ -960,14 +963,12 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
     // No LDS read may be in flight across a loop back-edge or between the loops below: the compiler is free
     // to copy a fragment register there, and a copy taken before the data has landed copies stale contents.
     // The first two k-steps of the next tile, fetched under the last four MFMA groups, are waited for here.
-    if (has_next) {
 #pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
+    for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
-        for (int i = 0; i < TM; ++i) lds_wait(fa[ks][i]);
+      for (int i = 0; i < TM; ++i) lds_wait(fa[ks][i]);
 #pragma unroll
-        for (int j = 0; j < TN; ++j) lds_wait(fb[ks][j]);
-      }
+      for (int j = 0; j < TN; ++j) lds_wait(fb[ks][j]);
     }
     buf = nbuf;
   };
