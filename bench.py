@@ -44,7 +44,8 @@ def make_bert(c, args):
     B, S, H, F, N, L, M = c["micro_batch"], c["seq"], c["hidden"], c["ffn"], c["heads"], c["num_layers"], c["num_micro_batches"]
     adt = torch.bfloat16 if c["dtype"] == "bf16" else torch.float32
     K = runtime.stash_depth(0, 2)
-    stage = runtime.bert_stage(L, H, N, F, B, S, c["dtype"], stash_slots=K, embeddings=c["embeddings"])
+    G = max(1, min(args.wgrad_group, M))
+    stage = runtime.bert_stage(L, H, N, F, B, S, c["dtype"], stash_slots=K, embeddings=c["embeddings"], wgrad_group=G)
     stage.bind(synthetic.bert_weights(synthetic.SEED_WEIGHT + c["index"], L, H, F, embeddings=c["embeddings"]))
     if c["embeddings"] is None:
         xs = [torch.as_tensor(x).cuda().to(adt) for x in synthetic.bert_activation_inputs(synthetic.SEED_INPUT + c["index"], M, B, S, H)]
@@ -62,7 +63,8 @@ def make_bert(c, args):
     fwd = 2 * S * (4 * H * H + 2 * H * F) + 4 * S * S * H
     wl.flops_per_sample = 3 * fwd * L
     wl.config = {"layers": L, "hidden": H, "heads": N, "ffn": F, "seq": S, "micro_batch": B, "micro_batches": M,
-                 "embedding": c["embeddings"] is not None, "schedule": "1F1B stage 0 of 2, stash K=%d" % K}
+                 "embedding": c["embeddings"] is not None, "schedule": "1F1B stage 0 of 2, stash K=%d" % K,
+                 "wgrad_group": G}
 
     def cpu():
         from oracle import bert as ob
@@ -221,6 +223,8 @@ def main():
     ap.add_argument("--workload", default="bert48_half")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-overlap", action="store_true", help="keep forward and backward passes on one stream")
+    ap.add_argument("--wgrad-group", type=int, default=4,
+                    help="BERT stages: weight gradients of this many backward passes in one GEMM per weight")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs one pipeline stage on ONE GPU; --gpus %d is not supported "

@@ -43,7 +43,7 @@ class StageCfg(C.Structure):
         ("batch", C.c_int), ("seq", C.c_int), ("with_embedding", C.c_int),
         ("vocab", C.c_int), ("type_vocab", C.c_int), ("max_pos", C.c_int),
         ("ln_eps", C.c_float), ("stash_slots", C.c_int), ("first_layer", C.c_int),
-        ("reserved", C.c_int * 7),
+        ("wgrad_group", C.c_int), ("reserved", C.c_int * 6),
     ]
 
 

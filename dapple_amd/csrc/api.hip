@@ -69,6 +69,8 @@ extern "C" int ds_profile_dump(char* buf, size_t cap) {
   return DS_OK;
 }
 
+thread_local int ds_launch_prio = 0;
+
 extern "C" const char* ds_last_error(void) { return g_err; }
 extern "C" const char* ds_build_target(void) { return "gfx950"; }
 
@@ -107,6 +109,7 @@ extern "C" int ds_stage_overlap_supported(const ds_stage* h) { return h && h->ov
 
 // Orders everything queued on the backward stream before whatever is queued next on the stage's stream.
 static int stage_join(ds_stage* h) {
+  DS_PROPAGATE(h->flush_deferred(true));
   if (h->bwd_stream && h->bwd_pending) {
     DS_CHECK_HIP(hipEventRecord(h->ev_join, h->bwd_stream));
     DS_CHECK_HIP(hipStreamWaitEvent(h->stream, h->ev_join, 0));
@@ -123,8 +126,8 @@ extern "C" int ds_stage_enable_overlap(ds_stage* h, int on) {
   }
   for (char f : h->slot_forwarded)
     if (f) { ds_set_error("ds_stage_enable_overlap: micro-batches in flight"); return DS_ESTATE; }
+  DS_PROPAGATE(stage_join(h));
   if (!on) {
-    DS_PROPAGATE(stage_join(h));
     h->bwd_stream = nullptr;
     h->wgrad_stream = nullptr;
     return DS_OK;

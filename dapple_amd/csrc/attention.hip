@@ -91,6 +91,7 @@ struct AttnArgs {
   float* delta;                  // [B, N, S]
   int B, N, S, H;
   float scale, mask_value;
+  int prio;                      // wave priority (0..3)
 };
 
 // store a transposed 64 x 32 accumulator pair (rows d, columns = this lane's row index) as out[row][d]
@@ -145,6 +146,7 @@ __device__ __forceinline__ void part_xy(const char* slot, float& x, float& y, in
 // ----------------------------------------------------------------------------------- forward
 // grid (S/64, B*N): each wave owns 32 queries and every SPLIT-th 32-key step.
 __global__ __launch_bounds__(NTHREADS) void attn_fwd_kernel(AttnArgs a) {
+  ds_wave_prio(a.prio);
   extern __shared__ __attribute__((aligned(16))) char lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5;
   const int grp = wave & 1, part = wave >> 1;
@@ -229,6 +231,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_fwd_kernel(AttnArgs a) {
 // grid (S/64, B*N): each wave owns 32 queries and every SPLIT-th 32-key step.  Also writes
 // delta[q] = sum_d dO[q,d] O[q,d].
 __global__ __launch_bounds__(NTHREADS) void attn_bwd_dq_kernel(AttnArgs a) {
+  ds_wave_prio(a.prio);
   extern __shared__ __attribute__((aligned(16))) char lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5;
   const int grp = wave & 1, part = wave >> 1;
@@ -299,6 +302,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_bwd_dq_kernel(AttnArgs a) {
 // ----------------------------------------------------------------------------------- backward: dK, dV
 // grid (S/64, B*N): each wave owns 32 keys and every SPLIT-th 32-query step (Q and dO tiles in LDS).
 __global__ __launch_bounds__(NTHREADS) void attn_bwd_dkv_kernel(AttnArgs a) {
+  ds_wave_prio(a.prio);
   extern __shared__ __attribute__((aligned(16))) char lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5;
   const int grp = wave & 1, part = wave >> 1;
@@ -397,6 +401,7 @@ extern "C" int ds_attention_fwd(int dtype, int batch, int heads, int seq, int he
   AttnArgs a;
   a.qkv = (const bf16*)qkv; a.ld = ld; a.key_mask = key_mask; a.ctx = (bf16*)ctx; a.lse = lse; a.dctx = nullptr; a.dqkv = nullptr;
   a.delta = nullptr; a.B = batch; a.N = heads; a.S = seq; a.H = heads * head_dim; a.scale = scale; a.mask_value = mask_value;
+  a.prio = ds_launch_prio;
   static bool attr = false;
   if (!attr) {
     DS_CHECK_HIP(hipFuncSetAttribute((const void*)attn_fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(2048)));
@@ -419,7 +424,7 @@ extern "C" int ds_attention_bwd(int dtype, int batch, int heads, int seq, int he
   AttnArgs a;
   a.qkv = (const bf16*)qkv; a.ld = ld; a.key_mask = key_mask; a.ctx = (bf16*)ctx; a.lse = (float*)lse; a.dctx = (const bf16*)dctx;
   a.dqkv = (bf16*)dqkv; a.delta = delta; a.B = batch; a.N = heads; a.S = seq; a.H = heads * head_dim; a.scale = scale;
-  a.mask_value = mask_value;
+  a.mask_value = mask_value; a.prio = ds_launch_prio;
   static bool attr = false;
   if (!attr) {
     DS_CHECK_HIP(hipFuncSetAttribute((const void*)attn_bwd_dq_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(2048)));

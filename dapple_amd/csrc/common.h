@@ -51,9 +51,24 @@ struct ds_prof_scope {
   ~ds_prof_scope();
 };
 
+// Wave priority of the kernels launched next from this host thread (0..3, the s_setprio scale).  A stage
+// raises it for the passes other work waits on and lowers it for work that only feeds the master gradients,
+// so that waves of both sharing a SIMD are issued in that order.
+extern thread_local int ds_launch_prio;
+struct ds_prio_scope {
+  int keep;
+  explicit ds_prio_scope(int p) : keep(ds_launch_prio) { ds_launch_prio = p; }
+  ~ds_prio_scope() { ds_launch_prio = keep; }
+};
+
 static inline bool ds_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 // ---- device helpers ----
+__device__ __forceinline__ void ds_wave_prio(int p) {  // s_setprio takes an immediate
+  if (p == 1) __builtin_amdgcn_s_setprio(1);
+  else if (p == 2) __builtin_amdgcn_s_setprio(2);
+  else if (p == 3) __builtin_amdgcn_s_setprio(3);
+}
 template <typename T> struct Vec16;  // 16-byte vector of T
 template <> struct Vec16<bf16> { typedef bf16x8 type; static constexpr int N = 8; };
 template <> struct Vec16<float> { typedef f32x4 type; static constexpr int N = 4; };

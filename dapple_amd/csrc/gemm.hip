@@ -57,6 +57,7 @@ struct GemmArgs {
   int xcd_rm, xcd_cn;  // tiles per XCD as an xcd_rm x xcd_cn block of the tile grid (0: contiguous runs)
   int vec_epi;
   int conv_h, conv_w, conv_c;  // implicit 3x3 'same' convolution: extent of the gathered NHWC tensor
+  int prio;                    // wave priority (0..3)
 };
 
 // LDS has 64 banks of 4 bytes: one bank line is 256 bytes = two 128-byte K-major rows.
@@ -782,6 +783,7 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
   constexpr int LPT = DA::NV + DB::NV;  // DMA loads per thread per k-tile
   extern __shared__ __attribute__((aligned(16))) char lds[];
 
+  ds_wave_prio(p.prio);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   int tile_m, tile_n;
@@ -1109,6 +1111,7 @@ static int gemm_run(const ds_gemm_desc* d, int splitk_req, void* stream) {
   a.c_so = d->c_stride_outer; a.c_si = d->c_stride_inner;
   a.flags = f;
   a.alpha = d->alpha;
+  a.prio = ds_launch_prio;
   a.vec_epi = d->n % 8 == 0 && d->ldc % 8 == 0 && d->c_stride_outer % 8 == 0 && d->c_stride_inner % 8 == 0 &&
               ds_aligned16(d->c) && ds_aligned16(d->residual) && ds_aligned16(d->c2);
   const int kt = d->dtype == DS_BF16 ? 64 : 32;
@@ -1192,7 +1195,7 @@ extern "C" int ds_conv3x3_fwd(int dtype, int n, int h, int w, int cin, int cout,
   a.lda = cin; a.ldb = cout; a.ldc = cout;
   a.batch_inner = 1; a.flags = flags; a.alpha = 1.f; a.splitk = 1; a.ktiles_per_split = a.k / 32;
   a.vec_epi = cout % 8 == 0;
-  a.conv_h = h; a.conv_w = w; a.conv_c = cin;
+  a.conv_h = h; a.conv_w = w; a.conv_c = cin; a.prio = ds_launch_prio;
   hipStream_t s = (hipStream_t)stream;
   ds_prof_scope prof(s, cout <= 64 ? "conv3x3_fwd<float,128,64>" : "conv3x3_fwd<float,128,128>", 2.0 * a.m * a.n * a.k, "FLOP");
   if (cout <= 64) return launch_conv_cfg<128, 64, DS_K_MAJOR, 1>(a, s);
@@ -1212,7 +1215,7 @@ extern "C" int ds_conv3x3_wgrad(int dtype, int n, int h, int w, int cin, int cou
   a.m = 9 * cin; a.n = cout; a.k = (int)pixels;
   a.lda = cin; a.ldb = cout; a.ldc = cout;
   a.batch_inner = 1; a.flags = DS_EPI_ACCUM; a.alpha = 1.f;
-  a.conv_h = h; a.conv_w = w; a.conv_c = cin;
+  a.conv_h = h; a.conv_w = w; a.conv_c = cin; a.prio = ds_launch_prio;
   const int bn = cout <= 64 ? 64 : 128;
   const int tiles = ((a.m + 127) / 128) * ((a.n + bn - 1) / bn);
   const int ktiles = a.k / 32;

@@ -49,6 +49,9 @@ struct ds_stage {
   virtual int backward(int slot, const void* d_out, void* d_in) = 0;
   virtual size_t workspace_bytes() const = 0;
   virtual size_t stash_bytes(int slots) const = 0;
+  // queues weight-gradient work that backward passes have deferred; `final`: and orders it before what the
+  // backward stream (or, without one, the stage's stream) runs next
+  virtual int flush_deferred(bool final) { (void)final; return DS_OK; }
 };
 
 // Bookkeeping for running a layer's weight-gradient work on ds_stage::wgrad_stream beside the dgrad

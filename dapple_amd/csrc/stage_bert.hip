@@ -67,8 +67,21 @@ __global__ __launch_bounds__(256) void embed_bwd_kernel(int rows, int H, int seq
   }
 }
 
-struct LayerStash {  // byte offsets into a slot
-  size_t x, qkv, p, ctx, z1, a, u, h, z2, st1, st2, lse;
+// A stashed tensor: `size` bytes per stash position, the positions back to back from byte `off` of the stash.
+// Consecutive positions of a [rows, cols] tensor therefore read as one [n*rows, cols] matrix.
+struct Ten {
+  size_t off = 0, size = 0;
+};
+struct LayerStash {
+  Ten x, qkv, p, ctx, z1, a, u, h, z2, st1, st2, lse;
+};
+// Upstream-gradient operands of a layer's weight-gradient GEMMs when those are deferred: per tensor a ring
+// of positions back to back, byte offsets into dy_base.
+struct LayerDy {
+  size_t dz2, du, dz1, dqkv;
+};
+struct Deferred {
+  int xpos, dypos;
 };
 
 struct BertStage : ds_stage {
@@ -84,11 +97,32 @@ struct BertStage : ds_stage {
   char* wc_base = nullptr;
   std::vector<char*> wqkv, wo, w1, w2;  // element type T
   std::vector<float*> bqkv;
-  // stash
+  // stash: the tensors live at stash positions; with per-pass weight gradients position = slot
   char* stash_base = nullptr;
-  size_t slot_bytes = 0;
-  size_t emb_e = 0, emb_st = 0, emb_ids = 0, emb_tt = 0, mask_off = 0;
+  size_t pos_bytes = 0;  // all tensors of one position
+  Ten emb_e, emb_st;
   std::vector<LayerStash> ls;
+  // small per-slot inputs (mask, token ids, token types)
+  char* small_base = nullptr;
+  size_t small_bytes = 0;
+  size_t emb_ids = 0, emb_tt = 0, mask_off = 0;
+  // Deferred weight gradients (cfg.wgrad_group = G > 1).  A backward pass leaves its upstream-gradient operands
+  // in position (count of backward passes) % 2G of a per-layer ring and the activations where the forward
+  // pass put them; after G passes ONE GEMM per weight contracts over all G micro-batches' rows.  Forward
+  // passes take stash positions round-robin out of K+G, so that G consecutive micro-batches sit back to back.
+  int G = 1, KP = 0, NDY = 0;
+  char* dy_base = nullptr;
+  std::vector<LayerDy> ld;
+  size_t dy_act = 0, dy_actF = 0;
+  std::vector<int> slot_pos, pos_owner;
+  std::vector<char> pos_deferred;
+  int next_pos = 0;
+  long n_backward = 0;
+  std::vector<Deferred> deferred;
+  hipEvent_t ev_chain = nullptr, ev_wg_done = nullptr;
+  std::vector<hipEvent_t> ev_x_bwd, ev_x_wg, ev_dy_wg;
+  std::vector<char> x_bwd_valid, x_wg_valid, dy_wg_valid;
+  bool wg_outstanding = false;
   size_t out_off = 0;  // last layer's y is written straight to the caller's buffer
   std::vector<char> slot_has_mask, slot_has_tt;
   // workspace
@@ -100,10 +134,18 @@ struct BertStage : ds_stage {
   ~BertStage() override {
     if (wc_base) (void)hipFree(wc_base);
     if (stash_base) (void)hipFree(stash_base);
+    if (small_base) (void)hipFree(small_base);
+    if (dy_base) (void)hipFree(dy_base);
+    if (ev_chain) (void)hipEventDestroy(ev_chain);
+    if (ev_wg_done) (void)hipEventDestroy(ev_wg_done);
+    for (hipEvent_t e : ev_x_bwd) (void)hipEventDestroy(e);
+    for (hipEvent_t e : ev_x_wg) (void)hipEventDestroy(e);
+    for (hipEvent_t e : ev_dy_wg) (void)hipEventDestroy(e);
     if (ws_base) (void)hipFree(ws_base);
   }
   int base(int l) const { return (emb ? EMB_NW : 0) + l * LAYER_NW; }
-  char* slotp(int slot) const { return stash_base + (size_t)slot * slot_bytes; }
+  char* at(const Ten& t, int pos) const { return stash_base + t.off + (size_t)pos * t.size; }
+  char* smallp(int slot) const { return small_base + (size_t)slot * small_bytes; }
 
   int init() {
     const ds_stage_cfg& c = cfg;
@@ -160,41 +202,78 @@ struct BertStage : ds_stage {
       bqkv[l] = (float*)(wc_base + o_b[l]);
       if (dtype == DS_BF16) { wo[l] = wc_base + o_wo[l]; w1[l] = wc_base + o_w1[l]; w2[l] = wc_base + o_w2[l]; }
     }
-    // ---- stash layout of one slot
-    Arena sa;
+    // ---- stash layout
+    const int K = c.stash_slots;
+    G = c.wgrad_group > 1 ? c.wgrad_group : 1;
+    KP = G > 1 ? K + G : K;
+    NDY = 2 * G;
     const size_t act = (size_t)rows * H * esz, actF = (size_t)rows * F * esz;
     const size_t probs = (size_t)B * NH * S * S * esz, stats = (size_t)rows * 2 * 4;
-    mask_off = sa.reserve((size_t)B * S * 4);
+    size_t ring_used = 0;
+    auto ring = [&](size_t bytes) {  // rows of 16-byte multiples: no padding between positions
+      Ten t;
+      t.size = (bytes + 15) & ~size_t(15);
+      t.off = ring_used;
+      ring_used += t.size * (size_t)KP;
+      ring_used = (ring_used + 255) & ~size_t(255);
+      pos_bytes += t.size;
+      return t;
+    };
+    Arena sm;
+    mask_off = sm.reserve((size_t)B * S * 4);
     if (emb) {
-      emb_ids = sa.reserve((size_t)rows * 4);
-      emb_tt = sa.reserve((size_t)rows * 4);
-      emb_e = sa.reserve(act);
-      emb_st = sa.reserve(stats);
+      emb_ids = sm.reserve((size_t)rows * 4);
+      emb_tt = sm.reserve((size_t)rows * 4);
+      emb_e = ring(act);
+      emb_st = ring(stats);
     }
+    small_bytes = sm.used;
     ls.resize(L);
-    size_t next_x = L ? sa.reserve(act) : 0;
+    Ten next_x = L ? ring(act) : Ten();
     for (int l = 0; l < L; ++l) {
       LayerStash& t = ls[l];
       t.x = next_x;
-      t.qkv = sa.reserve(3 * act);
-      t.p = fused_attn ? 0 : sa.reserve(probs);
-      t.lse = fused_attn ? sa.reserve((size_t)B * NH * S * 4) : 0;
-      t.ctx = sa.reserve(act);
-      t.z1 = sa.reserve(act);
-      t.a = sa.reserve(act);
-      t.u = sa.reserve(actF);
-      t.h = sa.reserve(actF);
-      t.z2 = sa.reserve(act);
-      t.st1 = sa.reserve(stats);
-      t.st2 = sa.reserve(stats);
-      if (l + 1 < L) next_x = sa.reserve(act);
+      t.qkv = ring(3 * act);
+      if (fused_attn) t.lse = ring((size_t)B * NH * S * 4);
+      else t.p = ring(probs);
+      t.ctx = ring(act);
+      t.z1 = ring(act);
+      t.a = ring(act);
+      t.u = ring(actF);
+      t.h = ring(actF);
+      t.z2 = ring(act);
+      t.st1 = ring(stats);
+      t.st2 = ring(stats);
+      if (l + 1 < L) next_x = ring(act);
     }
-    slot_bytes = sa.used;
-    const int K = c.stash_slots;
-    DS_CHECK_HIP(hipMalloc((void**)&stash_base, slot_bytes * K));
+    DS_CHECK_HIP(hipMalloc((void**)&stash_base, ring_used ? ring_used : 256));
+    DS_CHECK_HIP(hipMalloc((void**)&small_base, small_bytes * K));
     slot_forwarded.assign(K, 0);
     slot_has_mask.assign(K, 0);
     slot_has_tt.assign(K, 0);
+    slot_pos.assign(K, 0);
+    for (int i = 0; i < K; ++i) slot_pos[i] = i;
+    if (G > 1) {
+      pos_owner.assign(KP, -1);
+      pos_deferred.assign(KP, 0);
+      Arena da;
+      ld.resize(L);
+      dy_act = act; dy_actF = actF;
+      for (int l = 0; l < L; ++l) {
+        ld[l].dz2 = da.reserve(act * NDY);
+        ld[l].du = da.reserve(actF * NDY);
+        ld[l].dz1 = da.reserve(act * NDY);
+        ld[l].dqkv = da.reserve(3 * act * NDY);
+      }
+      if (da.used) DS_CHECK_HIP(hipMalloc((void**)&dy_base, da.used));
+      DS_CHECK_HIP(hipEventCreateWithFlags(&ev_chain, hipEventDisableTiming));
+      DS_CHECK_HIP(hipEventCreateWithFlags(&ev_wg_done, hipEventDisableTiming));
+      ev_x_bwd.assign(KP, nullptr); ev_x_wg.assign(KP, nullptr); ev_dy_wg.assign(NDY, nullptr);
+      for (auto& e : ev_x_bwd) DS_CHECK_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+      for (auto& e : ev_x_wg) DS_CHECK_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+      for (auto& e : ev_dy_wg) DS_CHECK_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+      x_bwd_valid.assign(KP, 0); x_wg_valid.assign(KP, 0); dy_wg_valid.assign(NDY, 0);
+    }
     // ---- workspace
     Arena w;
     ws_scores = w.reserve(fused_attn ? (size_t)B * NH * S * 4 : (size_t)B * NH * S * S * 4);  // fused: delta
@@ -216,7 +295,9 @@ struct BertStage : ds_stage {
   }
 
   size_t workspace_bytes() const override { return ws_bytes; }
-  size_t stash_bytes(int slots) const override { return slot_bytes * (size_t)slots; }
+  size_t stash_bytes(int slots) const override {
+    return (pos_bytes + small_bytes) * (size_t)slots + (G > 1 ? pos_bytes * (size_t)G : 0);
+  }
 
   const void* weight_T(int l, int which) const {  // kernel in the element type
     if (dtype == DS_BF16) return which == W_AO ? wo[l] : (which == W_FF1 ? w1[l] : w2[l]);
@@ -284,166 +365,171 @@ struct BertStage : ds_stage {
     return ds_gemm(&d, stream);
   }
 
+  // A stash position for the next forward pass: round-robin, skipping positions whose micro-batch has not
+  // been through backward; a position that deferred weight-gradient work still reads is flushed first.
+  int take_pos(int* out) {
+    for (int tries = 0; tries < KP; ++tries) {
+      const int p = next_pos;
+      next_pos = next_pos + 1 == KP ? 0 : next_pos + 1;
+      if (pos_owner[p] >= 0) continue;
+      if (pos_deferred[p]) DS_PROPAGATE(flush_deferred(false));
+      *out = p;
+      return DS_OK;
+    }
+    ds_set_error("ds_stage_forward: no free stash position");
+    return DS_ESTATE;
+  }
+
   int forward(int slot, const void* in, const float* key_mask, void* out) override {
-    char* sp = slotp(slot);
+    ds_prio_scope prio(1);
+    int pos = slot;
+    if (G > 1) {
+      DS_PROPAGATE(take_pos(&pos));
+      pos_owner[pos] = slot;
+      slot_pos[slot] = pos;
+      // the backward pass and the weight-gradient GEMMs that last read this position
+      if (x_bwd_valid[pos]) DS_CHECK_HIP(hipStreamWaitEvent(stream, ev_x_bwd[pos], 0));
+      if (x_wg_valid[pos]) DS_CHECK_HIP(hipStreamWaitEvent(stream, ev_x_wg[pos], 0));
+    }
+    char* sm = smallp(slot);
     const size_t act = (size_t)rows * H * esz;
     const float scale = 1.0f / sqrtf((float)D);
     const float* mask = nullptr;
     if (key_mask) {
-      DS_CHECK_HIP(hipMemcpyAsync(sp + mask_off, key_mask, (size_t)B * S * 4, hipMemcpyDeviceToDevice, stream));
-      mask = (const float*)(sp + mask_off);
+      DS_CHECK_HIP(hipMemcpyAsync(sm + mask_off, key_mask, (size_t)B * S * 4, hipMemcpyDeviceToDevice, stream));
+      mask = (const float*)(sm + mask_off);
     }
     slot_has_mask[slot] = key_mask != nullptr;
-    char* x0 = L ? sp + ls[0].x : nullptr;
+    char* x0 = L ? at(ls[0].x, pos) : nullptr;
     if (emb) {
-      DS_CHECK_HIP(hipMemcpyAsync(sp + emb_ids, in, (size_t)rows * 4, hipMemcpyDeviceToDevice, stream));
-      const int32_t* tt = slot_has_tt[slot] ? (const int32_t*)(sp + emb_tt) : nullptr;
+      DS_CHECK_HIP(hipMemcpyAsync(sm + emb_ids, in, (size_t)rows * 4, hipMemcpyDeviceToDevice, stream));
+      const int32_t* tt = slot_has_tt[slot] ? (const int32_t*)(sm + emb_tt) : nullptr;
       dim3 grid((rows + 3) / 4);
       if (dtype == DS_BF16)
         hipLaunchKernelGGL(embed_fwd_kernel<bf16>, grid, dim3(256), 0, stream, rows, H, S, cfg.vocab, cfg.type_vocab,
-                           (const int32_t*)(sp + emb_ids), tt, w[E_WORD], w[E_TYPE], w[E_POS], (bf16*)(sp + emb_e));
+                           (const int32_t*)(sm + emb_ids), tt, w[E_WORD], w[E_TYPE], w[E_POS], (bf16*)(at(emb_e, pos)));
       else
         hipLaunchKernelGGL(embed_fwd_kernel<float>, grid, dim3(256), 0, stream, rows, H, S, cfg.vocab, cfg.type_vocab,
-                           (const int32_t*)(sp + emb_ids), tt, w[E_WORD], w[E_TYPE], w[E_POS], (float*)(sp + emb_e));
+                           (const int32_t*)(sm + emb_ids), tt, w[E_WORD], w[E_TYPE], w[E_POS], (float*)(at(emb_e, pos)));
       DS_CHECK_LAUNCH();
-      DS_PROPAGATE(ds_layernorm_fwd(dtype, rows, H, sp + emb_e, w[E_LN_G], w[E_LN_B], cfg.ln_eps, L ? (void*)x0 : out,
-                                    (float*)(sp + emb_st), stream));
+      DS_PROPAGATE(ds_layernorm_fwd(dtype, rows, H, at(emb_e, pos), w[E_LN_G], w[E_LN_B], cfg.ln_eps, L ? (void*)x0 : out,
+                                    (float*)(at(emb_st, pos)), stream));
     } else {
       DS_CHECK_HIP(hipMemcpyAsync(x0, in, act, hipMemcpyDeviceToDevice, stream));
     }
     for (int l = 0; l < L; ++l) {
       const LayerStash& t = ls[l];
       const int b = base(l);
-      char* x = sp + t.x;
-      char* y = (l + 1 < L) ? sp + ls[l + 1].x : (char*)out;
+      char* x = at(t.x, pos);
+      char* y = (l + 1 < L) ? at(ls[l + 1].x, pos) : (char*)out;
       // fused Q|K|V projection (modeling_slice.py:464-485)
-      DS_PROPAGATE(gemm_fwd(rows, 3 * H, H, x, wqkv[l], sp + t.qkv, DS_EPI_BIAS, bqkv[l], nullptr, nullptr));
+      DS_PROPAGATE(gemm_fwd(rows, 3 * H, H, x, wqkv[l], at(t.qkv, pos), DS_EPI_BIAS, bqkv[l], nullptr, nullptr));
       if (fused_attn) {
         // scores, scale, mask adder, softmax and context in one kernel (:499-533)
-        DS_PROPAGATE(ds_attention_fwd(dtype, B, NH, S, D, sp + t.qkv, 3 * H, mask, scale, -10000.0f, sp + t.ctx,
-                                      (float*)(sp + t.lse), stream));
+        DS_PROPAGATE(ds_attention_fwd(dtype, B, NH, S, D, at(t.qkv, pos), 3 * H, mask, scale, -10000.0f, at(t.ctx, pos),
+                                      (float*)(at(t.lse, pos)), stream));
       } else {
       // scores = Q K^T (:499), fp32
-      DS_PROPAGATE(gemm_heads(DS_K_MAJOR, DS_K_MAJOR, S, S, D, sp + t.qkv, 3 * H, (int64_t)S * 3 * H, D,
-                              sp + t.qkv + (size_t)H * esz, 3 * H, (int64_t)S * 3 * H, D, ws_base + ws_fscores, S,
+      DS_PROPAGATE(gemm_heads(DS_K_MAJOR, DS_K_MAJOR, S, S, D, at(t.qkv, pos), 3 * H, (int64_t)S * 3 * H, D,
+                              at(t.qkv, pos) + (size_t)H * esz, 3 * H, (int64_t)S * 3 * H, D, ws_base + ws_fscores, S,
                               (int64_t)NH * S * S, (int64_t)S * S, DS_EPI_OUT_F32));
       // scale, mask adder, softmax (:500-518)
       DS_PROPAGATE(ds_softmax_fwd(dtype, B, NH, S, S, (const float*)(ws_base + ws_fscores), scale, mask, -10000.0f,
-                                  sp + t.p, stream));
+                                  at(t.p, pos), stream));
       // ctx = P V (:533), written head-interleaved as [rows, H] (:536-542)
-      DS_PROPAGATE(gemm_heads(DS_K_MAJOR, DS_MN_MAJOR, S, D, S, sp + t.p, S, (int64_t)NH * S * S, (int64_t)S * S,
-                              sp + t.qkv + (size_t)2 * H * esz, 3 * H, (int64_t)S * 3 * H, D, sp + t.ctx, H,
+      DS_PROPAGATE(gemm_heads(DS_K_MAJOR, DS_MN_MAJOR, S, D, S, at(t.p, pos), S, (int64_t)NH * S * S, (int64_t)S * S,
+                              at(t.qkv, pos) + (size_t)2 * H * esz, 3 * H, (int64_t)S * 3 * H, D, at(t.ctx, pos), H,
                               (int64_t)S * H, D, 0));
       }
       // attention output dense + residual (:974-978), then layer_norm (:979)
-      DS_PROPAGATE(gemm_fwd(rows, H, H, sp + t.ctx, weight_T(l, W_AO), sp + t.z1, DS_EPI_BIAS | DS_EPI_RESIDUAL,
+      DS_PROPAGATE(gemm_fwd(rows, H, H, at(t.ctx, pos), weight_T(l, W_AO), at(t.z1, pos), DS_EPI_BIAS | DS_EPI_RESIDUAL,
                             w[b + B_AO], x, nullptr));
-      DS_PROPAGATE(ds_layernorm_fwd(dtype, rows, H, sp + t.z1, w[b + LN1_G], w[b + LN1_B], cfg.ln_eps, sp + t.a,
-                                    (float*)(sp + t.st1), stream));
+      DS_PROPAGATE(ds_layernorm_fwd(dtype, rows, H, at(t.z1, pos), w[b + LN1_G], w[b + LN1_B], cfg.ln_eps, at(t.a, pos),
+                                    (float*)(at(t.st1, pos)), stream));
       // intermediate dense + gelu (:983-987)
-      DS_PROPAGATE(gemm_fwd(rows, F, H, sp + t.a, weight_T(l, W_FF1), sp + t.u, DS_EPI_BIAS | DS_EPI_GELU | DS_EPI_GELU_GRAD, w[b + B_FF1],
-                            nullptr, sp + t.h));
+      DS_PROPAGATE(gemm_fwd(rows, F, H, at(t.a, pos), weight_T(l, W_FF1), at(t.u, pos), DS_EPI_BIAS | DS_EPI_GELU | DS_EPI_GELU_GRAD, w[b + B_FF1],
+                            nullptr, at(t.h, pos)));
       // output dense + residual + layer_norm (:991-996)
-      DS_PROPAGATE(gemm_fwd(rows, H, F, sp + t.h, weight_T(l, W_FF2), sp + t.z2, DS_EPI_BIAS | DS_EPI_RESIDUAL,
-                            w[b + B_FF2], sp + t.a, nullptr));
-      DS_PROPAGATE(ds_layernorm_fwd(dtype, rows, H, sp + t.z2, w[b + LN2_G], w[b + LN2_B], cfg.ln_eps, y,
-                                    (float*)(sp + t.st2), stream));
+      DS_PROPAGATE(gemm_fwd(rows, H, F, at(t.h, pos), weight_T(l, W_FF2), at(t.z2, pos), DS_EPI_BIAS | DS_EPI_RESIDUAL,
+                            w[b + B_FF2], at(t.a, pos), nullptr));
+      DS_PROPAGATE(ds_layernorm_fwd(dtype, rows, H, at(t.z2, pos), w[b + LN2_G], w[b + LN2_B], cfg.ln_eps, y,
+                                    (float*)(at(t.st2, pos)), stream));
     }
     return DS_OK;
   }
 
   int backward(int slot, const void* d_out, void* d_in) override {
-    char* sp = slotp(slot);
+    ds_prio_scope prio(3);  // the chain every later pass waits on
+    const int pos = slot_pos[slot];
+    char* sm = smallp(slot);
+    const int dypos = (int)(n_backward % NDY);
+    if (G > 1 && dy_wg_valid[dypos]) DS_CHECK_HIP(hipStreamWaitEvent(stream, ev_dy_wg[dypos], 0));
     const float scale = 1.0f / sqrtf((float)D);
     const char* dy = (const char*)d_out;
     // With a weight-gradient stream the wgrad GEMMs and bias column sums of a layer run beside the
     // dgrad chain of the layers below it: they only feed the master gradients.
-    hipStream_t ws = wgrad_stream;
+    hipStream_t ws = G > 1 ? nullptr : wgrad_stream;  // deferred weight gradients go there in flush_deferred
     if (ws) DS_PROPAGATE(lane.ensure());
     for (int l = L - 1; l >= 0; --l) {
       const LayerStash& t = ls[l];
       const int b = base(l);
       const int par = l & 1;
-      char* dz2 = ws_base + ws_dz2[par];
-      char* du = ws_base + ws_du[par];
+      char* dz2 = G > 1 ? dy_base + ld[l].dz2 + dypos * dy_act : ws_base + ws_dz2[par];
+      char* du = G > 1 ? dy_base + ld[l].du + dypos * dy_actF : ws_base + ws_du[par];
       char* da = ws_base + ws_da;
-      char* dz1 = ws_base + ws_dz1[par];
+      char* dz1 = G > 1 ? dy_base + ld[l].dz1 + dypos * dy_act : ws_base + ws_dz1[par];
       char* dctx = ws_base + ws_dctx;
-      char* dqkv = ws_base + ws_dqkv[par];
+      char* dqkv = G > 1 ? dy_base + ld[l].dqkv + dypos * 3 * dy_act : ws_base + ws_dqkv[par];
       float* dp = (float*)(ws_base + ws_scores);
       char* dsm = ws_base + ws_ds;
       // the wgrads that read this parity's buffers two layers up must have run
       if (ws) DS_PROPAGATE(lane.reuse(stream, par));
       // output LayerNorm; the column sums of dz2 are the gradient of output/dense/bias
-      DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, dy, sp + t.z2, w[b + LN2_G], (const float*)(sp + t.st2), nullptr, dz2,
+      DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, dy, at(t.z2, pos), w[b + LN2_G], (const float*)(at(t.st2, pos)), nullptr, dz2,
                                     g[b + LN2_G], g[b + LN2_B], g[b + B_FF2], stream));
       // du = (dz2 W2^T) * gelu'(u)
-      DS_PROPAGATE(gemm_dgrad(rows, H, F, dz2, weight_T(l, W_FF2), du, DS_EPI_MUL, nullptr, sp + t.u));
+      DS_PROPAGATE(gemm_dgrad(rows, H, F, dz2, weight_T(l, W_FF2), du, DS_EPI_MUL, nullptr, at(t.u, pos)));
       // da = du W1^T + dz2 (a also feeds the residual into z2)
       DS_PROPAGATE(gemm_dgrad(rows, F, H, du, weight_T(l, W_FF1), da, DS_EPI_RESIDUAL, dz2, nullptr));
       // attention-output LayerNorm; column sums of dz1 = gradient of attention/output/dense/bias
-      DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, da, sp + t.z1, w[b + LN1_G], (const float*)(sp + t.st1), nullptr, dz1,
+      DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, da, at(t.z1, pos), w[b + LN1_G], (const float*)(at(t.st1, pos)), nullptr, dz1,
                                     g[b + LN1_G], g[b + LN1_B], g[b + B_AO], stream));
       DS_PROPAGATE(gemm_dgrad(rows, H, H, dz1, weight_T(l, W_AO), dctx, 0, nullptr, nullptr));
       // attention backward per (batch, head)
-      const char* q = sp + t.qkv;
+      const char* q = at(t.qkv, pos);
       const char* k = q + (size_t)H * esz;
       const char* v = q + (size_t)2 * H * esz;
       const int64_t so3 = (int64_t)S * 3 * H, soH = (int64_t)S * H, soP = (int64_t)NH * S * S, siP = (int64_t)S * S;
       if (fused_attn) {
-        const float* mask = slot_has_mask[slot] ? (const float*)(sp + mask_off) : nullptr;
-        DS_PROPAGATE(ds_attention_bwd(dtype, B, NH, S, D, q, 3 * H, mask, scale, -10000.0f, sp + t.ctx, (const float*)(sp + t.lse),
+        const float* mask = slot_has_mask[slot] ? (const float*)(sm + mask_off) : nullptr;
+        DS_PROPAGATE(ds_attention_bwd(dtype, B, NH, S, D, q, 3 * H, mask, scale, -10000.0f, at(t.ctx, pos), (const float*)(at(t.lse, pos)),
                                       dctx, dqkv, dp, stream));
       } else {
       // dP = dctx V^T (fp32)
       DS_PROPAGATE(gemm_heads(DS_K_MAJOR, DS_K_MAJOR, S, S, D, dctx, H, soH, D, v, 3 * H, so3, D, dp, S, soP, siP,
                               DS_EPI_OUT_F32));
       // dV = P^T dctx
-      DS_PROPAGATE(gemm_heads(DS_MN_MAJOR, DS_MN_MAJOR, S, D, S, sp + t.p, S, soP, siP, dctx, H, soH, D,
+      DS_PROPAGATE(gemm_heads(DS_MN_MAJOR, DS_MN_MAJOR, S, D, S, at(t.p, pos), S, soP, siP, dctx, H, soH, D,
                               dqkv + (size_t)2 * H * esz, 3 * H, so3, D, 0));
       // dS = scale * P * (dP - rowsum(dP * P))
-      DS_PROPAGATE(ds_softmax_bwd(dtype, (int64_t)B * NH * S, S, sp + t.p, dp, scale, dsm, stream));
+      DS_PROPAGATE(ds_softmax_bwd(dtype, (int64_t)B * NH * S, S, at(t.p, pos), dp, scale, dsm, stream));
       // dQ = dS K ; dK = dS^T Q
       DS_PROPAGATE(gemm_heads(DS_K_MAJOR, DS_MN_MAJOR, S, D, S, dsm, S, soP, siP, k, 3 * H, so3, D, dqkv, 3 * H, so3, D, 0));
       DS_PROPAGATE(gemm_heads(DS_MN_MAJOR, DS_MN_MAJOR, S, D, S, dsm, S, soP, siP, q, 3 * H, so3, D,
                               dqkv + (size_t)H * esz, 3 * H, so3, D, 0));
       }
       // ---- weight gradients of this layer (on the weight-gradient stream when there is one)
-      hipStream_t chain = stream;
-      if (ws) {
-        DS_PROPAGATE(lane.begin(chain, ws, par));
-        stream = ws;  // gemm_wgrad and the column sums below launch on `stream`
-      }
-      int rc = DS_OK;
-      do {
-        if ((rc = gemm_wgrad(rows, H, F, sp + t.h, F, dz2, H, g[b + W_FF2], H)) != DS_OK) break;
-        if ((rc = ds_colsum_accum(dtype, rows, F, du, F, g[b + B_FF1], stream)) != DS_OK) break;
-        if ((rc = gemm_wgrad(rows, F, H, sp + t.a, H, du, F, g[b + W_FF1], F)) != DS_OK) break;
-        if ((rc = gemm_wgrad(rows, H, H, sp + t.ctx, H, dz1, H, g[b + W_AO], H)) != DS_OK) break;
-        // projection gradients: three [H,H] kernels and three biases fed by the columns of dqkv
-        const bool adjacent = g[b + B_K] == g[b + B_Q] + H && g[b + B_V] == g[b + B_Q] + 2 * H &&
-                              g[b + W_K] == g[b + W_Q] + (size_t)H * H && g[b + W_V] == g[b + W_Q] + (size_t)2 * H * H;
-        if (adjacent) {
-          // q, k, v master gradients lie back to back: one column sum over [rows, 3H] and one GEMM batched
-          // over the three column blocks of dqkv
-          if ((rc = ds_colsum_accum(dtype, rows, 3 * H, dqkv, 3 * H, g[b + B_Q], stream)) != DS_OK) break;
-          ds_gemm_desc d;
-          memset(&d, 0, sizeof(d));
-          d.dtype = dtype; d.a_major = DS_MN_MAJOR; d.b_major = DS_MN_MAJOR;
-          d.m = H; d.n = H; d.k = rows; d.lda = H; d.ldb = 3 * H; d.ldc = H; d.batch = 3; d.batch_inner = 3;
-          d.b_stride_inner = H; d.c_stride_inner = (int64_t)H * H;
-          d.flags = DS_EPI_ACCUM; d.alpha = 1.f; d.a = sp + t.x; d.b = dqkv; d.c = g[b + W_Q];
-          if ((rc = ds_gemm(&d, stream)) != DS_OK) break;
-        } else {
-          for (int j = 0; j < 3 && rc == DS_OK; ++j) {
-            rc = ds_colsum_accum(dtype, rows, H, dqkv + (size_t)j * H * esz, 3 * H, g[b + B_Q + j], stream);
-            if (rc == DS_OK) rc = gemm_wgrad(rows, H, H, sp + t.x, H, dqkv + (size_t)j * H * esz, 3 * H, g[b + W_Q + j], H);
-          }
+      if (G == 1) {
+        hipStream_t chain = stream;
+        if (ws) {
+          DS_PROPAGATE(lane.begin(chain, ws, par));
+          stream = ws;  // the GEMMs and column sums of layer_wgrad launch on `stream`
         }
-      } while (0);
-      stream = chain;
-      if (rc != DS_OK) return rc;
-      if (ws) DS_PROPAGATE(lane.end(ws, par));
+        const int rc = layer_wgrad(l, rows, at(t.x, pos), at(t.ctx, pos), at(t.a, pos), at(t.h, pos), dz2, du, dz1, dqkv);
+        stream = chain;
+        if (rc != DS_OK) return rc;
+        if (ws) DS_PROPAGATE(lane.end(ws, par));
+      }
       // dx = dqkv Wqkv^T + dz1 (x also feeds the residual into z1)
       const bool first = (l == 0);
       if (first && !emb && d_in == nullptr) break;  // a first stage takes no input gradient
@@ -453,27 +539,123 @@ struct BertStage : ds_stage {
     }
     // the stash slot and the master gradients are released to the caller in the order of `stream`
     if (ws) DS_PROPAGATE(lane.finish(stream));
+    if (G > 1) {
+      deferred.push_back({pos, dypos});
+      pos_deferred[pos] = 1;
+      pos_owner[pos] = -1;
+      ++n_backward;
+    }
     if (emb) {
       // embedding LayerNorm backward, then scatter-add into the three tables
       char* de = ws_base + ws_dz2[0];
-      DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, dy, sp + emb_e, w[E_LN_G], (const float*)(sp + emb_st), nullptr, de,
+      DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, dy, at(emb_e, pos), w[E_LN_G], (const float*)(at(emb_st, pos)), nullptr, de,
                                     g[E_LN_G], g[E_LN_B], nullptr, stream));
-      const int32_t* tt = slot_has_tt[slot] ? (const int32_t*)(sp + emb_tt) : nullptr;
+      const int32_t* tt = slot_has_tt[slot] ? (const int32_t*)(sm + emb_tt) : nullptr;
       dim3 grid((rows + 3) / 4);
       if (dtype == DS_BF16)
         hipLaunchKernelGGL(embed_bwd_kernel<bf16>, grid, dim3(256), 0, stream, rows, H, S, cfg.vocab, cfg.type_vocab,
-                           (const int32_t*)(sp + emb_ids), tt, (const bf16*)de, g[E_WORD], g[E_TYPE], g[E_POS]);
+                           (const int32_t*)(sm + emb_ids), tt, (const bf16*)de, g[E_WORD], g[E_TYPE], g[E_POS]);
       else
         hipLaunchKernelGGL(embed_bwd_kernel<float>, grid, dim3(256), 0, stream, rows, H, S, cfg.vocab, cfg.type_vocab,
-                           (const int32_t*)(sp + emb_ids), tt, (const float*)de, g[E_WORD], g[E_TYPE], g[E_POS]);
+                           (const int32_t*)(sm + emb_ids), tt, (const float*)de, g[E_WORD], g[E_TYPE], g[E_POS]);
       DS_CHECK_LAUNCH();
+    }
+    if (G > 1) {
+      if (bwd_stream) {
+        DS_CHECK_HIP(hipEventRecord(ev_x_bwd[pos], stream));
+        x_bwd_valid[pos] = 1;
+      } else {
+        x_bwd_valid[pos] = 0;
+      }
+      if ((int)deferred.size() >= G) DS_PROPAGATE(flush_deferred(false));
+    }
+    return DS_OK;
+  }
+
+  // Weight and bias gradients of layer l over m rows (one micro-batch, or several back to back), on `stream`.
+  int layer_wgrad(int l, int m, const char* x, const char* ctx, const char* a, const char* h, const char* dz2,
+                  const char* du, const char* dz1, const char* dqkv) {
+    const int b = base(l);
+    ds_prio_scope prio(0);  // feeds only the master gradients
+    DS_PROPAGATE(gemm_wgrad(m, H, F, h, F, dz2, H, g[b + W_FF2], H));
+    DS_PROPAGATE(ds_colsum_accum(dtype, m, F, du, F, g[b + B_FF1], stream));
+    DS_PROPAGATE(gemm_wgrad(m, F, H, a, H, du, F, g[b + W_FF1], F));
+    DS_PROPAGATE(gemm_wgrad(m, H, H, ctx, H, dz1, H, g[b + W_AO], H));
+    // projection gradients: three [H,H] kernels and three biases fed by the columns of dqkv
+    const bool adjacent = g[b + B_K] == g[b + B_Q] + H && g[b + B_V] == g[b + B_Q] + 2 * H &&
+                          g[b + W_K] == g[b + W_Q] + (size_t)H * H && g[b + W_V] == g[b + W_Q] + (size_t)2 * H * H;
+    if (adjacent) {
+      // q, k, v master gradients lie back to back: one column sum over [m, 3H] and one GEMM batched
+      // over the three column blocks of dqkv
+      DS_PROPAGATE(ds_colsum_accum(dtype, m, 3 * H, dqkv, 3 * H, g[b + B_Q], stream));
+      ds_gemm_desc d;
+      memset(&d, 0, sizeof(d));
+      d.dtype = dtype; d.a_major = DS_MN_MAJOR; d.b_major = DS_MN_MAJOR;
+      d.m = H; d.n = H; d.k = m; d.lda = H; d.ldb = 3 * H; d.ldc = H; d.batch = 3; d.batch_inner = 3;
+      d.b_stride_inner = H; d.c_stride_inner = (int64_t)H * H;
+      d.flags = DS_EPI_ACCUM; d.alpha = 1.f; d.a = x; d.b = dqkv; d.c = g[b + W_Q];
+      DS_PROPAGATE(ds_gemm(&d, stream));
+    } else {
+      for (int j = 0; j < 3; ++j) {
+        DS_PROPAGATE(ds_colsum_accum(dtype, m, H, dqkv + (size_t)j * H * esz, 3 * H, g[b + B_Q + j], stream));
+        DS_PROPAGATE(gemm_wgrad(m, H, H, x, H, dqkv + (size_t)j * H * esz, 3 * H, g[b + W_Q + j], H));
+      }
+    }
+    return DS_OK;
+  }
+
+  int flush_deferred(bool final) override {
+    if (G <= 1) return DS_OK;
+    hipStream_t chain = bwd_stream ? bwd_stream : stream;
+    hipStream_t ws = wgrad_stream ? wgrad_stream : chain;
+    if (!deferred.empty()) {
+      if (ws != chain) {  // the operands the last backward pass wrote
+        DS_CHECK_HIP(hipEventRecord(ev_chain, chain));
+        DS_CHECK_HIP(hipStreamWaitEvent(ws, ev_chain, 0));
+      }
+      hipStream_t keep = stream;
+      stream = ws;
+      int rc = DS_OK;
+      // runs of micro-batches that sit back to back in both rings: one set of GEMMs per run
+      size_t i = 0;
+      while (i < deferred.size() && rc == DS_OK) {
+        size_t j = i + 1;
+        while (j < deferred.size() && deferred[j].xpos == deferred[j - 1].xpos + 1 &&
+               deferred[j].dypos == deferred[j - 1].dypos + 1)
+          ++j;
+        const int n = (int)(j - i), xp = deferred[i].xpos, dp = deferred[i].dypos;
+        for (int l = L - 1; l >= 0 && rc == DS_OK; --l) {
+          const LayerStash& t = ls[l];
+          rc = layer_wgrad(l, n * rows, at(t.x, xp), at(t.ctx, xp), at(t.a, xp), at(t.h, xp),
+                           dy_base + ld[l].dz2 + dp * dy_act, dy_base + ld[l].du + dp * dy_actF,
+                           dy_base + ld[l].dz1 + dp * dy_act, dy_base + ld[l].dqkv + dp * 3 * dy_act);
+        }
+        i = j;
+      }
+      stream = keep;
+      if (rc != DS_OK) return rc;
+      for (const Deferred& e : deferred) {
+        if (ws != chain) {
+          DS_CHECK_HIP(hipEventRecord(ev_x_wg[e.xpos], ws));
+          DS_CHECK_HIP(hipEventRecord(ev_dy_wg[e.dypos], ws));
+        }
+        x_wg_valid[e.xpos] = dy_wg_valid[e.dypos] = ws != chain;
+        pos_deferred[e.xpos] = 0;
+      }
+      deferred.clear();
+      if (ws != chain) wg_outstanding = true;
+    }
+    if (final && wg_outstanding) {
+      DS_CHECK_HIP(hipEventRecord(ev_wg_done, wgrad_owned));
+      DS_CHECK_HIP(hipStreamWaitEvent(chain, ev_wg_done, 0));
+      wg_outstanding = false;
     }
     return DS_OK;
   }
 
   int set_token_types(int slot, const int32_t* tt) {
     if (!emb) { ds_set_error("ds_stage_set_token_types: stage has no embedding"); return DS_ESTATE; }
-    if (tt) DS_CHECK_HIP(hipMemcpyAsync(slotp(slot) + emb_tt, tt, (size_t)rows * 4, hipMemcpyDeviceToDevice, stream));
+    if (tt) DS_CHECK_HIP(hipMemcpyAsync(smallp(slot) + emb_tt, tt, (size_t)rows * 4, hipMemcpyDeviceToDevice, stream));
     slot_has_tt[slot] = tt != nullptr;
     return DS_OK;
   }

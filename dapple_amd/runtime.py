@@ -173,9 +173,11 @@ def _dtype_code(dtype):
 
 
 def bert_stage(num_layers, hidden, heads, ffn, batch, seq, dtype, stash_slots, embeddings=None, first_layer=0,
-               ln_eps=1e-12, device="cuda:0"):
+               ln_eps=1e-12, device="cuda:0", wgrad_group=1):
     """A BERT stage: ``num_layers`` encoder layers, behind the embedding when ``embeddings`` =
-    (vocab, type_vocab, max_pos) is given."""
+    (vocab, type_vocab, max_pos) is given.  ``wgrad_group`` = G > 1: the weight gradients of G consecutive
+    backward passes are formed by one GEMM per weight (G more stash positions; the gradients are complete
+    after ``Stage.join`` / ``Stage.sync``)."""
     if hidden % heads != 0:
         raise ValueError("The hidden size (%d) is not a multiple of the number of attention heads (%d)" % (hidden, heads))
     lib = _lib.load()
@@ -186,6 +188,7 @@ def bert_stage(num_layers, hidden, heads, ffn, batch, seq, dtype, stash_slots, e
         cfg.with_embedding = 1
         cfg.vocab, cfg.type_vocab, cfg.max_pos = embeddings
     cfg.ln_eps, cfg.stash_slots, cfg.first_layer = ln_eps, stash_slots, first_layer
+    cfg.wgrad_group = int(wgrad_group)
     h = C.c_void_p()
     with torch.cuda.device(torch.device(device)):
         check(lib.ds_stage_create(C.byref(cfg), _lib.current_stream(), C.byref(h)), "ds_stage_create")

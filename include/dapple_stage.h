@@ -162,7 +162,13 @@ typedef struct ds_stage_cfg {
   float ln_eps;
   int stash_slots; /* K: in-flight micro-batches (S - i, bert/graph.py:129) */
   int first_layer; /* index of this stage's first encoder layer in the whole model (names only) */
-  int reserved[7];
+  int wgrad_group; /* G: weight gradients of G consecutive backward passes are formed by ONE GEMM per weight
+                    * (contraction over the G micro-batches' rows, one fp32 read-modify-write of the master
+                    * gradient instead of G); 0 or 1: every backward pass accumulates its own.  The sum over
+                    * micro-batches is the one tf.accumulate_n forms (bert/graph.py:159).  With G > 1 the
+                    * handle keeps K+G stash positions and a 2G-deep ring of the upstream-gradient operands,
+                    * and the master gradients are complete only after ds_stage_join / ds_stage_sync. */
+  int reserved[6];
 } ds_stage_cfg;
 
 typedef struct ds_stage ds_stage;
@@ -198,8 +204,9 @@ int ds_stage_sync(ds_stage* h);
  * their weight-gradient GEMMs on a third (default priority); per-slot events keep B(slot) after
  * F(slot) and the next F(slot) after B(slot); (h, 0) returns to one stream (no micro-batch may be
  * in flight for either call).
- * ds_stage_join orders all queued backward work before what is queued next on the stage's stream
- * (call it at the end of a step, before reading gradients on that stream); ds_stage_sync and
+ * ds_stage_join queues the weight-gradient work still deferred (wgrad_group > 1) and orders all queued
+ * backward work before what is queued next on the stage's stream (call it at the end of a step, before
+ * reading gradients on that stream); ds_stage_sync and
  * ds_stage_refresh_weights join by themselves.  Stages whose forward and backward passes share
  * workspace report 0 from ds_stage_overlap_supported and DS_EINVAL from ds_stage_enable_overlap. */
 int ds_stage_overlap_supported(const ds_stage* h);

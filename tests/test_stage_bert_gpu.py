@@ -19,7 +19,7 @@ ADT = {"fp32": torch.float32, "bf16": torch.bfloat16}
 
 
 def run_case(dtype, L, H, N, F, B, S, M, embeddings=None, use_mask=False, K=2, stage_index=0, odtype=torch.float64,
-             seed=0, perturb=True, stddev=0.05):
+             seed=0, perturb=True, stddev=0.05, wgrad_group=1):
     w_np = synthetic.bert_weights(synthetic.SEED_WEIGHT + seed, L, H, F, embeddings=embeddings, stddev=stddev,
                                   perturb=perturb)
     if embeddings is not None:
@@ -35,7 +35,7 @@ def run_case(dtype, L, H, N, F, B, S, M, embeddings=None, use_mask=False, K=2, s
             m[:, 0] = 1.0
 
     # ---- GPU stage
-    stage = runtime.bert_stage(L, H, N, F, B, S, dtype, stash_slots=K, embeddings=embeddings)
+    stage = runtime.bert_stage(L, H, N, F, B, S, dtype, stash_slots=K, embeddings=embeddings, wgrad_group=wgrad_group)
     stage.bind(w_np)
     adt = ADT[dtype]
     xs = [dev(x) if embeddings is not None else dev(x, adt) for x in xs_np]
@@ -259,3 +259,44 @@ def test_forward_backward_overlap_unfused_fp32_with_embedding():
     for k in res[0][1]:
         a, b = res[0][1][k], res[1][1][k]
         assert float((a - b).abs().max()) <= 1e-5 * float(a.abs().max()) + 1e-10, k
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,group", [("fp32", 2), ("fp32", 3), ("bf16", 4)])
+def test_grouped_weight_gradients_match_oracle(dtype, group):
+    """One weight-gradient GEMM per `group` backward passes (5 micro-batches: the last group is short)."""
+    run_case(dtype, 2, 64, 4, 128, 2, 16, 5, use_mask=True, wgrad_group=group)
+    run_case(dtype, 1, 64, 4, 128, 2, 16, 5, embeddings=(50, 2, 32), K=1, wgrad_group=group)
+
+
+@pytest.mark.gpu
+def test_grouped_weight_gradients_over_steps_and_streams():
+    """Grouped weight gradients over several steps (the stash positions and the operand ring wrap, the group
+    boundary falls inside a step) equal the per-pass ones, on one stream and on three."""
+    L, H, N, F, B, S, M = 2, 256, 4, 512, 2, 128, 6
+    w = synthetic.bert_weights(21, L, H, F)
+    xs = [torch.as_tensor(x).cuda().bfloat16() for x in synthetic.bert_activation_inputs(22, M, B, S, H)]
+    dys = [torch.as_tensor(x).cuda().bfloat16() for x in synthetic.upstream_grads(23, M, (B * S, H))]
+    res = []
+    for group, overlap in ((1, False), (4, False), (4, True), (4, True), (6, True), (2, True)):
+        st = runtime.bert_stage(L, H, N, F, B, S, "bf16", stash_slots=2, wgrad_group=group)
+        st.bind(w)
+        if overlap:
+            st.enable_overlap()
+        assert st.stash_bytes() > 0
+        outs = [torch.empty(B * S, H, dtype=torch.bfloat16, device="cuda") for _ in range(M)]
+        dxs = [torch.empty_like(o) for o in outs]
+        rt = runtime.StageRuntime(st, 0, 2, M)
+        for _ in range(3):
+            st.refresh_weights()
+            st.zero_grads()
+            rt.step(xs, dys, outs, dxs)
+        st.sync()
+        res.append(([o.float().cpu() for o in outs], [d.float().cpu() for d in dxs], {k: v.cpu().clone() for k, v in st.grads.items()}))
+        st.close()
+    for other in res[1:]:
+        for a, b in zip(res[0][0] + res[0][1], other[0] + other[1]):
+            assert torch.equal(a, b)
+        for k in res[0][2]:
+            a, b = res[0][2][k], other[2][k]
+            assert float((a - b).abs().max()) <= 2e-5 * float(a.abs().max()) + 1e-12, k
