@@ -204,6 +204,7 @@ struct GnmtStage : ds_stage {
   }
 
   int forward(int slot, const void* in, const float*, void* out) override {
+    ds_prio_scope prio(1);
     char* sp = stash_base + (size_t)slot * slot_bytes;
     DS_CHECK_HIP(hipMemcpyAsync(sp + ids_off, in, (size_t)R * 4, hipMemcpyDeviceToDevice, stream));
     hipLaunchKernelGGL(gnmt_embed_fwd_kernel, dim3((R + 3) / 4), dim3(256), 0, stream, B, T, U, gc.vocab,
@@ -244,6 +245,7 @@ struct GnmtStage : ds_stage {
   }
 
   int backward(int slot, const void* d_out, void*) override {
+    ds_prio_scope prio(3);  // the chain every later pass waits on
     char* sp = stash_base + (size_t)slot * slot_bytes;
     float* dG = (float*)(ws_base + ws_dg);
     float* dc = (float*)(ws_base + ws_dc);

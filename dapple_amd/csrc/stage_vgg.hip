@@ -233,6 +233,7 @@ struct VggStage : ds_stage {
   }
 
   int forward(int slot, const void* in, const float*, void* out) override {
+    ds_prio_scope prio(1);
     char* sp = stash_base + (size_t)slot * slot_bytes;
     DS_CHECK_HIP(hipMemcpyAsync(sp + ops[0].in_off, in, ops[0].in_elems * 4, hipMemcpyDeviceToDevice, stream));
     for (size_t i = 0; i < ops.size(); ++i) {
@@ -267,6 +268,7 @@ struct VggStage : ds_stage {
   }
 
   int backward(int slot, const void* d_out, void* d_in) override {
+    ds_prio_scope prio(3);  // the chain every later pass waits on
     char* sp = stash_base + (size_t)slot * slot_bytes;
     const float* gout = (const float*)d_out;
     int cur = -1;         // which workspace buffer gout lives in (-1: the caller's d_out)

@@ -358,6 +358,7 @@ struct XlnetStage : ds_stage {
   }
 
   int forward(int slot, const void* in, const float*, void* out) override {
+    ds_prio_scope prio(1);
     char* sp = stash_base + (size_t)slot * slot_bytes;
     const size_t act = (size_t)rows * H * esz;
     const float scale = 1.0f / sqrtf((float)D);
@@ -414,6 +415,7 @@ struct XlnetStage : ds_stage {
   }
 
   int backward(int slot, const void* d_out, void* d_in) override {
+    ds_prio_scope prio(3);  // the chain every later pass waits on
     char* sp = stash_base + (size_t)slot * slot_bytes;
     const float scale = 1.0f / sqrtf((float)D);
     const uint8_t* seg = has_seg[slot] ? (const uint8_t*)(sp + seg_off) : nullptr;
@@ -495,6 +497,7 @@ struct XlnetStage : ds_stage {
       }
       int rc = DS_OK;
       do {
+        ds_prio_scope wprio(0);  // feeds only the master gradients
         if ((rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, F, H, rows, sp + t.hh, F, dz2, H, g[b + X_W2], H, DS_EPI_ACCUM)) != DS_OK) break;
         if ((rc = ds_colsum_accum(dtype, rows, F, du, F, g[b + X_B1], stream)) != DS_OK) break;
         if ((rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, F, rows, sp + t.y1, H, du, F, g[b + X_W1], F, DS_EPI_ACCUM)) != DS_OK) break;
