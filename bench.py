@@ -209,6 +209,8 @@ TRAFFIC = {
     "gemm_dma_kernel<bf16,128,128,MN,MN>": 59.0e6,   # ffn weight-gradient shape: 42.2 MB read + 16.8 MB written
     "gemm_dma_kernel<bf16,128,128,K,MN>": 33.9e6,    # ffn1 forward shape
     "gemm_dma_kernel<bf16,128,128,K,K>": 33.8e6,     # ffn2 dgrad shape
+    "gemm_dma_kernel<bf16,64,64,K,K>": 35.8e6,       # mean of the ffn1 / qkv / attention-output dgrad shapes
+    "gemm_dma_kernel<bf16,64,64,K,MN>": 52.6e6,      # ffn2 forward shape
 }
 
 MAKERS = {"bert": make_bert, "vgg": make_vgg, "gnmt": make_gnmt, "xlnet": make_xlnet}
@@ -276,6 +278,9 @@ def main():
         roof = {"bound": "hbm", "achieved": work / (ms * 1e-3) / 1e9, "peak": PEAK["hbm"] / 1e9, "unit": "GB/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
     roof["traffic"] = TRAFFIC.get(dom)
+    if dom == "gemm_dma_kernel<bf16,128,128,MN,MN>" and wl.config.get("wgrad_group", 1) != 1:
+        # measured for four micro-batches per GEMM only
+        roof["traffic"] = 134.5e6 if wl.config["wgrad_group"] == 4 else None
     if roof["traffic"] is not None:
         roof["traffic_unit"] = "bytes per launch (FETCH_SIZE + WRITE_SIZE, scaled by a known-traffic kernel), see " + TRAFFIC_SOURCE
     roof.update({"kernel": dom, "launches": n, "avg_launch_us": ms * 1e3 / n, "share_of_kernel_time": ms / total_ms})

@@ -3,7 +3,7 @@
 ``accumulate N``: ``ds_grad_accumulate`` over N fp32 elements - known traffic (reads 8*N bytes, writes
 4*N bytes), used to scale the FETCH_SIZE / WRITE_SIZE counters.
 ``gemms``: the GEMMs of one BERT-48 half-stage layer at their real shapes (2x512 rows, hidden 1024,
-ffn 4096, bf16), three launches each, so a counter run can report HBM traffic per launch.
+ffn 4096, bf16), three launches each in the order of the list in ``gemms``, so a counter run can report HBM traffic per launch.
 
     rocprofv3 --pmc FETCH_SIZE --output-format csv -d out -o c -- python3 -m dapple_amd.calib accumulate 67108864
     rocprofv3 --pmc FETCH_SIZE --output-format csv -d out -o g -- python3 -m dapple_amd.calib gemms
@@ -33,6 +33,10 @@ def gemms():
         ("fwd ffn2", rows, h, f, DS_K_MAJOR, DS_MN_MAJOR, False),
         ("dgrad ffn2", rows, f, h, DS_K_MAJOR, DS_K_MAJOR, False),
         ("wgrad ffn1", h, f, rows, DS_MN_MAJOR, DS_MN_MAJOR, True),
+        ("dgrad ffn1", rows, h, f, DS_K_MAJOR, DS_K_MAJOR, False),
+        ("dgrad qkv", rows, h, 3 * h, DS_K_MAJOR, DS_K_MAJOR, False),
+        ("dgrad ao", rows, h, h, DS_K_MAJOR, DS_K_MAJOR, False),
+        ("wgrad ffn1 x4", h, f, 4 * rows, DS_MN_MAJOR, DS_MN_MAJOR, True),   # four micro-batches in one GEMM
     ]
     for name, m, n, k, am, bm, acc in shapes:
         a = torch.randn((m, k) if am == DS_K_MAJOR else (k, m), device="cuda").to(bf)

@@ -40,6 +40,7 @@ def pmc(path, needle):
         for c in sorted(per[sel[0]]):
             vals = [per[d][c] for d in sel]
             out.append("%-24s avg %.1f  min %.1f  max %.1f" % (c, sum(vals) / len(vals), min(vals), max(vals)))
+            out.append("%-24s per dispatch, in launch order: %s" % ("", " ".join("%.1f" % v for v in vals)))
     return "\n".join(out)
 
 
