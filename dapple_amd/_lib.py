@@ -103,6 +103,7 @@ PROTOTYPES = {
                                     C.c_void_p]),
     "ds_vgg_stage_create": (C.c_int, [C.POINTER(VggCfg), C.c_void_p, C.POINTER(C.c_void_p)]),
     "ds_gnmt_stage_create": (C.c_int, [C.POINTER(GnmtCfg), C.c_void_p, C.POINTER(C.c_void_p)]),
+    "ds_gnmt_stage_set_lengths": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p]),
     "ds_xlnet_stage_create": (C.c_int, [C.POINTER(XlnetCfg), C.c_void_p, C.POINTER(C.c_void_p)]),
     "ds_xlnet_stage_set_inputs": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
     "ds_stage_create": (C.c_int, [C.POINTER(StageCfg), C.c_void_p, C.POINTER(C.c_void_p)]),

@@ -4,7 +4,11 @@
 // Follows gnmt/nmt/gnmt_model.py:61-221 (DAPPLE branch) and gnmt/nmt/model_helper.py:399-456 of the
 // reference; the cell is TensorFlow's BasicLSTMCell: gates = [x, h] @ kernel[in+U, 4U] + bias, gate
 // order i, j, f, o, c' = c*sigmoid(f + forget_bias) + sigmoid(i)*tanh(j), h' = tanh(c')*sigmoid(o).
-// All sequences are full length (the config passes no lengths), so dynamic_rnn is a plain scan.
+// Without lengths dynamic_rnn is a plain scan.  With source_sequence_length (gnmt_model.py:103, 223-227) a
+// step t >= length[b] emits zeros - also from a residual cell, whose wrapped output is what gets replaced - and
+// keeps the state; the backward direction starts from the zero state at t = length[b] - 1.  Here such a
+// step stores h = c = y = 0 (in either scan order it lies outside the run of live steps, which therefore
+// starts from zeros) and backward gives it zero gate gradients and passes no state gradient on.
 //
 // Per layer: the input half of the gates for all T steps is ONE GEMM [T*B, in] x [in, 4U] (+bias);
 // each step then adds h[t-1] @ Wh (a [B, U] x [U, 4U] GEMM whose epilogue adds the precomputed
@@ -48,10 +52,17 @@ __global__ __launch_bounds__(256) void gnmt_embed_bwd_kernel(int B, int T, int U
 __global__ __launch_bounds__(256) void lstm_cell_fwd_kernel(int B, int U, float forget_bias, float* __restrict__ gates,
                                                            const float* __restrict__ c_prev, float* __restrict__ c,
                                                            float* __restrict__ h, int ldh, const float* __restrict__ x_res,
-                                                           int ldx, float* __restrict__ y, int ldy) {
+                                                           int ldx, float* __restrict__ y, int ldy,
+                                                           const int32_t* __restrict__ len, int t) {
   const int idx = blockIdx.x * 256 + threadIdx.x;
   if (idx >= B * U) return;
   const int b = idx / U, u = idx % U;
+  if (len && t >= len[b]) {  // past the end of sequence b
+    c[idx] = 0.f;
+    h[(int64_t)b * ldh + u] = 0.f;
+    if (y) y[(int64_t)b * ldy + u] = 0.f;
+    return;
+  }
   float* g = gates + (int64_t)b * 4 * U;
   const float i = sigmoidf_(g[u]), j = tanhf(g[U + u]), f = sigmoidf_(g[2 * U + u] + forget_bias), o = sigmoidf_(g[3 * U + u]);
   const float cp = c_prev ? c_prev[idx] : 0.f;
@@ -69,10 +80,17 @@ __global__ __launch_bounds__(256) void lstm_cell_bwd_kernel(int B, int U, const 
                                                            const float* __restrict__ c, const float* __restrict__ c_prev,
                                                            const float* __restrict__ dy, int lddy,
                                                            const float* __restrict__ dh_rec, float* __restrict__ dc_rec,
-                                                           int first, float* __restrict__ dgates) {
+                                                           int first, float* __restrict__ dgates,
+                                                           const int32_t* __restrict__ len, int t) {
   const int idx = blockIdx.x * 256 + threadIdx.x;
   if (idx >= B * U) return;
   const int b = idx / U, u = idx % U;
+  if (len && t >= len[b]) {
+    float* d = dgates + (int64_t)b * 4 * U;
+    d[u] = 0.f; d[U + u] = 0.f; d[2 * U + u] = 0.f; d[3 * U + u] = 0.f;
+    dc_rec[idx] = 0.f;
+    return;
+  }
   const float* g = gact + (int64_t)b * 4 * U;
   const float i = g[u], j = g[U + u], f = g[2 * U + u], o = g[3 * U + u];
   const float tc = tanhf(c[idx]);
@@ -85,6 +103,17 @@ __global__ __launch_bounds__(256) void lstm_cell_bwd_kernel(int B, int U, const 
   d[2 * U + u] = dc * cp * f * (1.f - f);
   d[3 * U + u] = dh * tc * o * (1.f - o);
   dc_rec[idx] = dc * f;
+}
+
+// dst[t, b, :] = t < len[b] ? src[t, b, :] : 0 (the output past the end of a sequence is the constant 0)
+__global__ __launch_bounds__(256) void mask_steps_kernel(int64_t total4, int B, int U4, const int32_t* __restrict__ len,
+                                                        const f32x4* __restrict__ src, f32x4* __restrict__ dst) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total4; i += (int64_t)gridDim.x * 256) {
+    const int64_t row = i / U4;
+    const int t = (int)(row / B), b = (int)(row % B);
+    const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+    dst[i] = t < len[b] ? src[i] : z;
+  }
 }
 
 struct Cell {
@@ -103,9 +132,10 @@ struct GnmtStage : ds_stage {
   int B, T, U, L, R;  // R = T*B rows
   std::vector<Cell> cells;
   char* stash_base = nullptr;
-  size_t slot_bytes = 0, ids_off = 0, x0_off = 0, xb_off = 0;
+  size_t slot_bytes = 0, ids_off = 0, len_off = 0, x0_off = 0, xb_off = 0;
+  std::vector<char> slot_has_len;
   char* ws_base = nullptr;
-  size_t ws_bytes = 0, ws_dg, ws_dx[2], ws_dh[2], ws_dc;
+  size_t ws_bytes = 0, ws_dg, ws_dx[2], ws_dh[2], ws_dc, ws_dym;
 
   ~GnmtStage() override {
     if (stash_base) (void)hipFree(stash_base);
@@ -120,6 +150,7 @@ struct GnmtStage : ds_stage {
     winfo.push_back({name, gc.vocab, U});
     Arena sa;
     ids_off = sa.reserve((size_t)R * 4);
+    len_off = sa.reserve((size_t)B * 4);
     x0_off = sa.reserve((size_t)R * U * 4);
     xb_off = sa.reserve((size_t)R * 2 * U * 4);
     size_t prev_out = 0;
@@ -159,6 +190,7 @@ struct GnmtStage : ds_stage {
     slot_bytes = sa.used;
     DS_CHECK_HIP(hipMalloc((void**)&stash_base, slot_bytes * gc.stash_slots));
     slot_forwarded.assign(gc.stash_slots, 0);
+    slot_has_len.assign(gc.stash_slots, 0);
     Arena wa;
     ws_dg = wa.reserve((size_t)R * 4 * U * 4);
     ws_dx[0] = wa.reserve((size_t)R * 2 * U * 4);
@@ -166,6 +198,7 @@ struct GnmtStage : ds_stage {
     ws_dh[0] = wa.reserve((size_t)B * U * 4);
     ws_dh[1] = wa.reserve((size_t)B * U * 4);
     ws_dc = wa.reserve((size_t)B * U * 4);
+    ws_dym = wa.reserve((size_t)R * U * 4);
     ws_bytes = wa.used;
     DS_CHECK_HIP(hipMalloc((void**)&ws_base, ws_bytes));
     return DS_OK;
@@ -203,9 +236,18 @@ struct GnmtStage : ds_stage {
     return s < 1 ? 1 : s;
   }
 
+  int set_lengths(int slot, const int32_t* lengths) {
+    if (lengths)
+      DS_CHECK_HIP(hipMemcpyAsync(stash_base + (size_t)slot * slot_bytes + len_off, lengths, (size_t)B * 4,
+                                  hipMemcpyDeviceToDevice, stream));
+    slot_has_len[slot] = lengths != nullptr;
+    return DS_OK;
+  }
+
   int forward(int slot, const void* in, const float*, void* out) override {
     ds_prio_scope prio(1);
     char* sp = stash_base + (size_t)slot * slot_bytes;
+    const int32_t* len = slot_has_len[slot] ? (const int32_t*)(sp + len_off) : nullptr;
     DS_CHECK_HIP(hipMemcpyAsync(sp + ids_off, in, (size_t)R * 4, hipMemcpyDeviceToDevice, stream));
     hipLaunchKernelGGL(gnmt_embed_fwd_kernel, dim3((R + 3) / 4), dim3(256), 0, stream, B, T, U, gc.vocab,
                        (const int32_t*)(sp + ids_off), w[0], (float*)(sp + x0_off));
@@ -235,7 +277,8 @@ struct GnmtStage : ds_stage {
         ds_prof_scope prof(stream, "lstm_cell_fwd_kernel", (double)B * U * 4 * (4 + 4 + 2 + (c.residual ? 2 : 1)), "B");
         hipLaunchKernelGGL(lstm_cell_fwd_kernel, dim3(cell_grid), dim3(256), 0, stream, B, U, gc.forget_bias, g,
                            s > 0 ? Cs + (size_t)tp * B * U : nullptr, Cs + (size_t)t * B * U, H + (size_t)t * B * c.ldh, c.ldh,
-                           c.residual ? X + (size_t)t * B * c.ldx : nullptr, c.ldx, Y ? Y + (size_t)t * B * U : nullptr, U);
+                           c.residual ? X + (size_t)t * B * c.ldx : nullptr, c.ldx, Y ? Y + (size_t)t * B * U : nullptr, U,
+                           len, t);
         DS_CHECK_LAUNCH();
       }
       if (last && !c.residual)
@@ -250,8 +293,19 @@ struct GnmtStage : ds_stage {
     float* dG = (float*)(ws_base + ws_dg);
     float* dc = (float*)(ws_base + ws_dc);
     const int cell_grid = (B * U + 255) / 256;
+    const int32_t* len = slot_has_len[slot] ? (const int32_t*)(sp + len_off) : nullptr;
     const float* dY = (const float*)d_out;  // gradient w.r.t. the output of the cell being processed
     int lddy = U;
+    if (len) {
+      // the output past the end of a sequence is constant: no gradient enters there.  With that every gradient
+      // tensor further down has zero rows at those steps by itself (zero gate gradients, masked residual).
+      float* dym = (float*)(ws_base + ws_dym);
+      const int64_t total4 = (int64_t)R * U / 4;
+      hipLaunchKernelGGL(mask_steps_kernel, dim3((unsigned)((total4 + 255) / 256 > 4096 ? 4096 : (total4 + 255) / 256)), dim3(256), 0,
+                         stream, total4, B, U / 4, len, (const f32x4*)d_out, (f32x4*)dym);
+      DS_CHECK_LAUNCH();
+      dY = dym;
+    }
     int pp = 0;
     float* dXB = nullptr;  // gradient w.r.t. the fw|bw concatenation [R, 2U]
     float* dX0 = nullptr;
@@ -274,7 +328,7 @@ struct GnmtStage : ds_stage {
           ds_prof_scope prof(stream, "lstm_cell_bwd_kernel", (double)B * U * 4 * (4 + 4 + 6), "B");
           hipLaunchKernelGGL(lstm_cell_bwd_kernel, dim3(cell_grid), dim3(256), 0, stream, B, U, G + (size_t)t * B * 4 * U,
                              Cs + (size_t)t * B * U, s > 0 ? Cs + (size_t)tp * B * U : nullptr, dY + (size_t)t * B * lddy, lddy,
-                             dh_in, dc, first, dG + (size_t)t * B * 4 * U);
+                             dh_in, dc, first, dG + (size_t)t * B * 4 * U, len, t);
           DS_CHECK_LAUNCH();
         }
         if (s > 0) {  // dh for step tp: dgates[t] @ Wh^T
@@ -336,4 +390,12 @@ extern "C" int ds_gnmt_stage_create(const ds_gnmt_cfg* c, void* stream, ds_stage
   if (rc != DS_OK) { delete s; return rc; }
   *out = s;
   return DS_OK;
+}
+
+extern "C" int ds_gnmt_stage_set_lengths(ds_stage* h, int slot, const int32_t* lengths) {
+  DS_CHECK_ARG(h != nullptr, "ds_gnmt_stage_set_lengths: null handle");
+  DS_CHECK_ARG(h->cfg.kind == DS_STAGE_GNMT, "ds_gnmt_stage_set_lengths: not a GNMT stage");
+  DS_CHECK_ARG(slot >= 0 && slot < h->cfg.stash_slots, "ds_gnmt_stage_set_lengths: slot %d out of range", slot);
+  DS_PROPAGATE(ds_stage_acquire_slot(h, slot));
+  return static_cast<GnmtStage*>(h)->set_lengths(slot, lengths);
 }

@@ -239,10 +239,20 @@ def gnmt_stage(num_layers, units, vocab, batch, seq, stash_slots, forget_bias=1.
     h = C.c_void_p()
     with torch.cuda.device(torch.device(device)):
         check(lib.ds_gnmt_stage_create(C.byref(cfg), _lib.current_stream(), C.byref(h)), "ds_gnmt_stage_create")
-    st = Stage(h, _TORCH_DTYPE[cfg.dtype], batch * seq, seq * batch * units, stash_slots, in_dtype=torch.int32,
-               takes_input_grad=False, device=device, cfg=cfg)
+    st = GnmtStage(h, _TORCH_DTYPE[cfg.dtype], batch * seq, seq * batch * units, stash_slots, in_dtype=torch.int32,
+                   takes_input_grad=False, device=device, cfg=cfg)
     st.out_shape = (seq, batch, units)
     return st
+
+
+class GnmtStage(Stage):
+    def set_lengths(self, slot, lengths=None):
+        """``source_sequence_length`` [batch] int32 of the micro-batch about to be forwarded into ``slot``
+        (None: full length)."""
+        if lengths is not None and (lengths.dtype != torch.int32 or not lengths.is_cuda or not lengths.is_contiguous()
+                                    or lengths.numel() != self.cfg.batch):
+            raise ValueError("lengths must be a contiguous int32 GPU tensor of [batch]")
+        check(self.lib.ds_gnmt_stage_set_lengths(self._h, slot, ptr(lengths)), "ds_gnmt_stage_set_lengths")
 
 
 class XlnetStage(Stage):

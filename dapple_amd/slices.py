@@ -352,8 +352,10 @@ class GNMTEncoderSlice(object):
         self.stage.bind(weights or synthetic.gnmt_weights(seed, n, hparams.num_units, hparams.src_vocab_size,
                                                           init_weight=getattr(hparams, "init_weight", 0.1)))
 
-    def build_graph(self, source_ids, scope=None, dep_outputs=None):
+    def build_graph(self, source_ids, scope=None, dep_outputs=None, source_sequence_length=None):
         out = torch.empty(self.stage.out_shape, device=source_ids.device)
+        self.stage.set_lengths(0, None if source_sequence_length is None else
+                               source_sequence_length.to(torch.int32).contiguous())
         self.stage.forward(0, source_ids.to(torch.int32).contiguous(), out)
         self.stage.backward(0, torch.zeros_like(out))
         return out

@@ -253,7 +253,8 @@ int ds_vgg_stage_create(const ds_vgg_cfg* cfg, void* stream, ds_stage** out);
  * bidirectional BasicLSTMCell layer, then num_layers-1 uni-directional layers, residual from the
  * third layer on (model_helper.py:445-448); ids [batch, seq] int32 in, [seq, batch, units] out
  * (time-major like the reference).  Kernels are TF's [in+units, 4*units] with gate order i, j, f, o.
- * Sequences are full length.  The handle works with every ds_stage_* call; it takes no input gradient. */
+ * Sequences are full length unless ds_gnmt_stage_set_lengths says otherwise.  The handle works with every
+ * ds_stage_* call; it takes no input gradient. */
 typedef struct ds_gnmt_cfg {
   int dtype;       /* DS_F32 */
   int num_layers;  /* encoder layers incl. the bidirectional one (8 for GNMT-16's encoder) */
@@ -263,6 +264,11 @@ typedef struct ds_gnmt_cfg {
   int reserved[8];
 } ds_gnmt_cfg;
 int ds_gnmt_stage_create(const ds_gnmt_cfg* cfg, void* stream, ds_stage** out);
+/* iterator.source_sequence_length (gnmt_model.py:103, 223-227) of the micro-batch that will be forwarded
+ * into `slot`: lengths [batch] int32 on the device, or NULL for full length.  Every layer's dynamic_rnn
+ * gets it: steps t >= lengths[b] emit zeros (residual layers too) and keep the state, the backward
+ * direction of the first layer starts at step lengths[b] - 1.  The setting stays with the slot. */
+int ds_gnmt_stage_set_lengths(ds_stage* h, int slot, const int32_t* lengths);
 
 /* XLNet stage (xlnet/models/slice_xlnet.py:164-180 layer body; xlnet/layers/rel_multihead_attn.py:71-149).
  * Activations are sequence-major like the reference: in/out are [streams][seq][batch][hidden] (stream 0 =

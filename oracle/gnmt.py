@@ -7,12 +7,18 @@ ResidualWrapper).  BasicLSTMCell itself lives in TensorFlow (un-vendored); its p
 algorithm is restated here: one kernel [in+U, 4U] applied to concat([x, h], 1), bias [4U],
 gate order i, j, f, o, c' = c*sigmoid(f + forget_bias) + sigmoid(i)*tanh(j),
 h' = tanh(c')*sigmoid(o).  tf.nn.dynamic_rnn with full-length sequences is a plain scan from a
-zero state; the backward cell of bidirectional_dynamic_rnn scans the reversed sequence.
+zero state; the backward cell of bidirectional_dynamic_rnn scans the reversed sequence.  With
+sequence_length (every layer gets iterator.source_sequence_length, gnmt_model.py:103, 223-227)
+dynamic_rnn emits zeros and copies the state through for t >= length[b] - the output of the WRAPPED
+cell is replaced, so a residual layer emits zeros there too - and the backward direction reverses each
+sequence within its own length (tf.reverse_sequence), i.e. it starts from the zero state at
+t = length[b] - 1.
 
 Pins (tests/test_oracle_gnmt.py): the cell vs torch.nn.LSTMCell after permuting the gate
 blocks (torch order i, f, g, o) and folding forget_bias into the bias; the kernel layout
 [in+U, 4U] vs the shape held by gnmt/nmt/model_test.py:86 ((10, 20) for in = U = 5); the
-scan vs an explicit Python loop; the bidirectional layer vs torch.nn.LSTM(bidirectional=True).
+scan vs an explicit Python loop; the bidirectional layer vs torch.nn.LSTM(bidirectional=True); ragged sequences vs torch.nn.LSTM on a
+packed sequence (pack_padded_sequence / pad_packed_sequence), both directions.
 """
 import torch
 
@@ -36,8 +42,9 @@ def lstm_cell(x, h, c, kernel, bias, forget_bias=1.0):
     return new_h, new_c
 
 
-def dynamic_rnn(x, kernel, bias, forget_bias=1.0, reverse=False):
-    """x [T,B,I] time-major, zero initial state, all sequences full length -> outputs [T,B,U]."""
+def dynamic_rnn(x, kernel, bias, forget_bias=1.0, reverse=False, lengths=None, residual=False):
+    """x [T,B,I] time-major, zero initial state -> outputs [T,B,U] (+ x where the cell has a residual wrapper).
+    lengths [B] int or None (all full length): steps t >= lengths[b] emit zeros and keep the state."""
     T, B, _ = x.shape
     U = kernel.shape[1] // 4
     h = torch.zeros(B, U, dtype=x.dtype)
@@ -45,21 +52,27 @@ def dynamic_rnn(x, kernel, bias, forget_bias=1.0, reverse=False):
     outs = [None] * T
     order = range(T - 1, -1, -1) if reverse else range(T)
     for t in order:
-        h, c = lstm_cell(x[t], h, c, kernel, bias, forget_bias)
-        outs[t] = h
+        nh, nc = lstm_cell(x[t], h, c, kernel, bias, forget_bias)
+        out = nh + x[t] if residual else nh             # ResidualWrapper, model_helper.py:445-448
+        if lengths is not None:
+            live = (t < lengths).to(x.dtype).unsqueeze(1)
+            out = out * live
+            nh = nh * live + h * (1 - live)
+            nc = nc * live + c * (1 - live)
+        h, c = nh, nc
+        outs[t] = out
     return torch.stack(outs)
 
 
-def encoder_forward(ids, w, num_layers, forget_bias=1.0):
-    """ids [B,T] int -> encoder outputs [T,B,U] (gnmt_model.py:78-210)."""
+def encoder_forward(ids, w, num_layers, forget_bias=1.0, lengths=None):
+    """ids [B,T] int -> encoder outputs [T,B,U] (gnmt_model.py:78-210); lengths [B] = source_sequence_length."""
     emb = w[EMB][ids.long().t()]                      # time-major lookup (:78-79, :90-91)
     cells = cell_names(num_layers)
-    fw = dynamic_rnn(emb, w[cells[0][0] + "/kernel"], w[cells[0][0] + "/bias"], forget_bias)
-    bw = dynamic_rnn(emb, w[cells[1][0] + "/kernel"], w[cells[1][0] + "/bias"], forget_bias, reverse=True)
+    fw = dynamic_rnn(emb, w[cells[0][0] + "/kernel"], w[cells[0][0] + "/bias"], forget_bias, lengths=lengths)
+    bw = dynamic_rnn(emb, w[cells[1][0] + "/kernel"], w[cells[1][0] + "/bias"], forget_bias, reverse=True, lengths=lengths)
     x = torch.cat([fw, bw], -1)                       # :108
     for scope, _, residual in cells[2:]:
-        y = dynamic_rnn(x, w[scope + "/kernel"], w[scope + "/bias"], forget_bias)
-        x = y + x if residual else y                  # ResidualWrapper, model_helper.py:445-448
+        x = dynamic_rnn(x, w[scope + "/kernel"], w[scope + "/bias"], forget_bias, lengths=lengths, residual=residual)
     return x
 
 
@@ -67,8 +80,8 @@ def to_torch(weights, dtype=torch.float64, requires_grad=False):
     return {k: torch.as_tensor(v).to(dtype).clone().requires_grad_(requires_grad) for k, v in weights.items()}
 
 
-def stage_vjp(ids, w, d_out, num_layers, forget_bias=1.0):
+def stage_vjp(ids, w, d_out, num_layers, forget_bias=1.0, lengths=None):
     names = sorted(w)
-    out = encoder_forward(ids, w, num_layers, forget_bias)
+    out = encoder_forward(ids, w, num_layers, forget_bias, lengths)
     grads = torch.autograd.grad(out, [w[n] for n in names], grad_outputs=d_out, allow_unused=True)
     return out.detach(), None, {n: g for n, g in zip(names, grads) if g is not None}

@@ -11,7 +11,7 @@ pytestmark = pytest.mark.gpu
 TOL = 1e-4
 
 
-def run_case(L, U, V, B, T, M, K=2, seed=0, init=0.1, perturb=True, odtype=torch.float64, M_check=None):
+def run_case(L, U, V, B, T, M, K=2, seed=0, init=0.1, perturb=True, odtype=torch.float64, M_check=None, lengths=None):
     w_np = synthetic.gnmt_weights(synthetic.SEED_WEIGHT + seed, L, U, V, init_weight=init, perturb=perturb)
     ids_np = synthetic.gnmt_id_inputs(synthetic.SEED_INPUT + seed, M, B, T, V)
     dys_np = synthetic.upstream_grads(synthetic.SEED_GRAD + seed, M, (T, B, U))
@@ -21,12 +21,18 @@ def run_case(L, U, V, B, T, M, K=2, seed=0, init=0.1, perturb=True, odtype=torch
     stage.bind(w_np)
     ids, dys = [dev(i) for i in ids_np], [dev(d) for d in dys_np]
     outs = [torch.empty(T, B, U, device="cuda") for _ in range(M)]
-    runtime.StageRuntime(stage, 0, K, M).step(ids, dys, outs)
+    lens = None if lengths is None else [torch.tensor(l, dtype=torch.int32, device="cuda") for l in lengths]
+    before = None if lens is None else (lambda slot, j: stage.set_lengths(slot, lens[j]))
+    runtime.StageRuntime(stage, 0, K, M).step(ids, dys, outs, before_forward=before)
     stage.sync()
     w_t = og.to_torch(w_np, odtype, requires_grad=True)
     acc = {}
     for j in range(M):
-        out, _, dw = og.stage_vjp(ids[j].cpu(), w_t, dys[j].cpu().to(odtype), L)
+        out, _, dw = og.stage_vjp(ids[j].cpu(), w_t, dys[j].cpu().to(odtype), L,
+                                  lengths=None if lengths is None else torch.tensor(lengths[j]))
+        if lengths is not None:
+            for b, n in enumerate(lengths[j]):
+                assert float(outs[j][n:, b].abs().max() if n < T else 0.0) == 0.0   # zeros past the end, exactly
         assert_close(outs[j], out, TOL, "output mb%d" % j)
         for n, g in dw.items():
             acc[n] = g.clone() if n not in acc else acc[n] + g
@@ -52,3 +58,9 @@ def test_config2_shape_reduced_depth():
     # bidirectional layer, uni layer 1 (2048 -> 1024) and one residual layer; one micro-batch
     c = synthetic.CONFIGS["gnmt16_encoder"]
     run_case(L=3, U=c["units"], V=c["vocab"], B=c["micro_batch"], T=c["seq"], M=1, K=1, seed=c["index"], perturb=False)
+
+
+def test_ragged_sequences():
+    """source_sequence_length per micro-batch: full, single-step, empty and in-between sequences; the second
+    micro-batch reuses a slot whose previous lengths were different, the third goes back to full length."""
+    run_case(L=4, U=32, V=50, B=4, T=6, M=3, init=0.4, seed=3, lengths=[[6, 1, 3, 5], [2, 6, 0, 4], [6, 6, 6, 6]])

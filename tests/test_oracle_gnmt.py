@@ -56,6 +56,39 @@ def test_bidirectional_layer_matches_torch_lstm():
     assert torch.allclose(torch.cat([fw, bw], -1), ref, atol=1e-12)
 
 
+def test_ragged_sequences_match_torch_packed_lstm():
+    """sequence_length: zeros past the end, the backward direction starts at the last valid step
+    (torch.nn.LSTM on a packed sequence does exactly that), including a sequence of length 1 and a full one."""
+    T, B, I, U = 7, 4, 3, 5
+    x = torch.randn(T, B, I, dtype=D)
+    lengths = torch.tensor([7, 1, 4, 6])
+    ks = [torch.randn(I + U, 4 * U, dtype=D) * 0.5 for _ in range(2)]
+    bs = [torch.randn(4 * U, dtype=D) * 0.5 for _ in range(2)]
+    fw = og.dynamic_rnn(x, ks[0], bs[0], 1.0, lengths=lengths)
+    bw = og.dynamic_rnn(x, ks[1], bs[1], 1.0, reverse=True, lengths=lengths)
+    lstm = torch.nn.LSTM(I, U, bidirectional=True).double()
+    with torch.no_grad():
+        for sfx, k, b in (("", ks[0], bs[0]), ("_reverse", ks[1], bs[1])):
+            wih, whh, bb, _ = _to_torch_lstm(k, b, I, 1.0)
+            getattr(lstm, "weight_ih_l0" + sfx).copy_(wih)
+            getattr(lstm, "weight_hh_l0" + sfx).copy_(whh)
+            getattr(lstm, "bias_ih_l0" + sfx).copy_(bb)
+            getattr(lstm, "bias_hh_l0" + sfx).zero_()
+    packed = torch.nn.utils.rnn.pack_padded_sequence(x, lengths, enforce_sorted=False)
+    ref, _ = torch.nn.utils.rnn.pad_packed_sequence(lstm(packed)[0], total_length=T)
+    assert torch.allclose(torch.cat([fw, bw], -1), ref, atol=1e-12)
+    for b in range(B):
+        assert float(fw[lengths[b]:, b].abs().max() if lengths[b] < T else 0.0) == 0.0
+    # a residual layer emits zeros past the end too (the wrapped cell's output is what dynamic_rnn replaces)
+    k2, b2 = torch.randn(U + U, 4 * U, dtype=D) * 0.5, torch.randn(4 * U, dtype=D) * 0.5
+    y = og.dynamic_rnn(fw, k2, b2, 1.0, lengths=lengths, residual=True)
+    assert float(y[1:, 1].abs().max()) == 0.0 and float(y[0, 1].abs().max()) > 0.0
+    # lengths that cover everything change nothing; zero length gives all zeros
+    full = og.dynamic_rnn(x, ks[0], bs[0], 1.0, lengths=torch.full((B,), T))
+    assert torch.equal(full, og.dynamic_rnn(x, ks[0], bs[0], 1.0))
+    assert float(og.dynamic_rnn(x, ks[0], bs[0], 1.0, lengths=torch.zeros(B, dtype=torch.long)).abs().max()) == 0.0
+
+
 def test_encoder_structure_residual_from_third_layer():
     T, B, U, V, L = 4, 2, 4, 9, 4
     w = og.to_torch(synthetic.gnmt_weights(1, L, U, V, init_weight=0.5, perturb=True))
