@@ -193,7 +193,8 @@ def test_colsum(dt):
     assert_close(out, x.cpu().double().sum(0) + 1, 1e-5, "colsum")
 
 
-@pytest.mark.parametrize("B,N,S,use_mask", [(1, 1, 64, False), (2, 3, 128, True), (2, 16, 512, True), (1, 2, 1024, False)])
+@pytest.mark.parametrize("B,N,S,use_mask", [(1, 1, 64, False), (2, 3, 128, True), (2, 16, 512, True), (1, 2, 1024, False),
+                                            (1, 2, 192, True), (2, 1, 320, True), (1, 1, 2048, True)])  # ragged last tile; the maximum
 def test_fused_attention_fwd_bwd(B, N, S, use_mask):
     D, H = 64, N * 64
     r = rng(S + N)
@@ -226,3 +227,27 @@ def test_fused_attention_rejects_other_shapes():
         ops.attention_fwd(qkv, 1, 1, 64, 1.0)
     with pytest.raises(ValueError, match="multiple of 64"):
         ops.attention_fwd(torch.zeros(48, 192, dtype=torch.bfloat16, device="cuda"), 1, 1, 48, 1.0)
+
+
+def test_layernorm_widest_row_and_single_row():
+    """The widest row the kernel takes (64 lanes x 8 vectors x 8 bf16 = 4096 columns), and a single row."""
+    for rows, cols in ((3, 4096), (1, 1024)):
+        r = rng(rows * 7 + cols)
+        x = dev(r.standard_normal((rows, cols)), torch.bfloat16)
+        g = dev(1 + 0.2 * r.standard_normal(cols), torch.float32)
+        b = dev(0.3 * r.standard_normal(cols), torch.float32)
+        dy = dev(r.standard_normal((rows, cols)), torch.bfloat16)
+        y, stats = ops.layernorm_fwd(x, g, b, 1e-12)
+        x64 = x.cpu().double().requires_grad_(True)
+        g64, b64 = g.cpu().double().requires_grad_(True), b.cpu().double().requires_grad_(True)
+        ref = ob.layer_norm(x64, g64, b64)
+        assert_close(y, ref, 1e-2, "ln fwd")
+        dx_ref, dg_ref, db_ref = torch.autograd.grad(ref, [x64, g64, b64], dy.cpu().double())
+        dg, db = torch.zeros(cols, device="cuda"), torch.zeros(cols, device="cuda")
+        dx = ops.layernorm_bwd(dy, x, g, stats, dg, db, None)
+        assert_close(dx, dx_ref, 1e-2, "ln dx")
+        assert_close(dg, dg_ref, 1e-4, "ln dgamma")
+        assert_close(db, db_ref, 1e-4, "ln dbeta")
+    with pytest.raises(ValueError):
+        ops.layernorm_fwd(torch.zeros(2, 4104, dtype=torch.bfloat16, device="cuda"), torch.ones(4104, device="cuda"),
+                          torch.zeros(4104, device="cuda"), 1e-12)
