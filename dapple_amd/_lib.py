@@ -124,6 +124,7 @@ PROTOTYPES = {
     "ds_stage_join": (C.c_int, [C.c_void_p]),
     "ds_squad_head": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                 C.c_float, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "ds_classifier_head": (C.c_int, [C.c_int] * 5 + [C.c_void_p] * 6 + [C.c_float, C.c_float] + [C.c_void_p] * 11),
     "ds_grad_sqnorm_accum": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p]),
     "ds_optim_plan_create": (C.c_int, [C.c_int, C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_float),
                                         C.POINTER(C.c_void_p)]),

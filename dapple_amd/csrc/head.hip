@@ -118,7 +118,179 @@ int squad_head_t(int B, int S, int H, const void* x, const float* w, const float
   return DS_OK;
 }
 
+// ------------------------------------------------------------------ pooler + classification head
+// modeling_slice.py:849-868 (pooler_stage: tanh dense on the first token) and bert.py:642-664
+// (build_output_layer_classification: FC to the labels, mean sparse softmax cross entropy plus the l2
+// regulariser of the FC weights).  The batch is a handful of rows: plain one-thread-per-output kernels.
+
+// pooled[b][j] = tanh(x[b, token 0] . Wp[:, j] + bp[j]); also clears the loss
+template <typename T>
+__global__ __launch_bounds__(256) void pooler_fwd_kernel(int B, int S, int H, const T* __restrict__ x, const float* __restrict__ wp,
+                                                         const float* __restrict__ bp, float* __restrict__ pooled,
+                                                         float* __restrict__ loss) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx == 0) *loss = 0.f;
+  if (idx >= B * H) return;
+  const int b = idx / H, j = idx % H;
+  const T* xr = x + (int64_t)b * S * H;
+  float a = bp[j];
+  for (int i = 0; i < H; ++i) a += to_f32(xr[i]) * wp[(int64_t)i * H + j];
+  pooled[idx] = tanhf(a);
+}
+
+// one block: logits, loss = scale * (mean CE + l2_scale * sum(Wfc^2) / 2), dlogits = d loss / d logits
+__global__ __launch_bounds__(256) void classifier_loss_kernel(int B, int H, int C, const float* __restrict__ pooled,
+                                                              const float* __restrict__ wfc, const float* __restrict__ bfc,
+                                                              const int32_t* __restrict__ labels, float l2_scale, float scale,
+                                                              float* __restrict__ logits, float* __restrict__ dlogits,
+                                                              float* __restrict__ loss) {
+  __shared__ float red[4];
+  __shared__ float lg[64];
+  for (int o = 0; o < B * C; ++o) {  // B*C dot products over H, the block cooperating on each
+    const int b = o / C, c = o % C;
+    float a = 0.f;
+    for (int j = threadIdx.x; j < H; j += 256) a += pooled[(int64_t)b * H + j] * wfc[(int64_t)j * C + c];
+    a = wave_sum(a);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = a;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      const float v = red[0] + red[1] + red[2] + red[3] + bfc[c];
+      logits[o] = v;
+      if (o < 64) lg[o] = v;
+    }
+    __syncthreads();
+  }
+  float sq = 0.f;
+  for (int i = threadIdx.x; i < H * C; i += 256) sq += wfc[i] * wfc[i];
+  sq = wave_sum(sq);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = sq;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float total = l2_scale * 0.5f * (red[0] + red[1] + red[2] + red[3]);
+    for (int b = 0; b < B; ++b) {
+      const float* l = logits + (int64_t)b * C;
+      float mx = l[0];
+      for (int c = 1; c < C; ++c) mx = fmaxf(mx, l[c]);
+      float sum = 0.f;
+      for (int c = 0; c < C; ++c) sum += expf(l[c] - mx);
+      const float lse = mx + logf(sum);
+      const int y = labels[b];
+      const bool ok = y >= 0 && y < C;  // a label outside the classes has no defined loss: NaN, as on TF's GPU kernel
+      total += ok ? -(l[y] - lse) / (float)B : NAN;
+      for (int c = 0; c < C; ++c)
+        dlogits[(int64_t)b * C + c] = ok ? (expf(l[c] - lse) - (c == y ? 1.f : 0.f)) * scale / (float)B : NAN;
+    }
+    *loss = total * scale;
+  }
+}
+
+// dWfc[j][c] += sum_b pooled[b][j] dlogits[b][c] + scale*l2_scale*Wfc[j][c]; dbfc[c] += sum_b dlogits[b][c];
+// dz[b][j] = (sum_c dlogits[b][c] Wfc[j][c]) * (1 - pooled[b][j]^2)
+__global__ __launch_bounds__(256) void classifier_bwd_kernel(int B, int H, int C, const float* __restrict__ pooled,
+                                                             const float* __restrict__ wfc, const float* __restrict__ dlogits,
+                                                             float l2_scale, float scale, float* __restrict__ dwfc,
+                                                             float* __restrict__ dbfc, float* __restrict__ dz) {
+  const int j = blockIdx.x * 256 + threadIdx.x;
+  if (j < C && dbfc) {
+    float s = 0.f;
+    for (int b = 0; b < B; ++b) s += dlogits[(int64_t)b * C + j];
+    dbfc[j] += s;
+  }
+  if (j >= H) return;
+  for (int c = 0; c < C && dwfc; ++c) {
+    float s = scale * l2_scale * wfc[(int64_t)j * C + c];
+    for (int b = 0; b < B; ++b) s += pooled[(int64_t)b * H + j] * dlogits[(int64_t)b * C + c];
+    dwfc[(int64_t)j * C + c] += s;
+  }
+  for (int b = 0; b < B; ++b) {
+    float dp = 0.f;
+    for (int c = 0; c < C; ++c) dp += dlogits[(int64_t)b * C + c] * wfc[(int64_t)j * C + c];
+    const float p = pooled[(int64_t)b * H + j];
+    dz[(int64_t)b * H + j] = dp * (1.f - p * p);
+  }
+}
+
+// dWp[i][j] += sum_b x[b, token 0][i] dz[b][j]; dbp[j] += sum_b dz[b][j]
+template <typename T>
+__global__ __launch_bounds__(256) void pooler_wgrad_kernel(int B, int S, int H, const T* __restrict__ x, const float* __restrict__ dz,
+                                                           float* __restrict__ dwp, float* __restrict__ dbp) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)H * H) return;
+  const int i = (int)(idx / H), j = (int)(idx % H);
+  float s = 0.f;
+  for (int b = 0; b < B; ++b) s += to_f32(x[(int64_t)b * S * H + i]) * dz[(int64_t)b * H + j];
+  dwp[idx] += s;
+  if (i == 0) {
+    float t = 0.f;
+    for (int b = 0; b < B; ++b) t += dz[(int64_t)b * H + j];
+    dbp[j] += t;
+  }
+}
+
+// dx[b, token 0][i] = sum_j dz[b][j] Wp[i][j]; every other token gets no gradient from this head
+template <typename T>
+__global__ __launch_bounds__(256) void pooler_dgrad_kernel(int B, int S, int H, const float* __restrict__ dz, const float* __restrict__ wp,
+                                                           T* __restrict__ dx) {
+  const int64_t total = (int64_t)B * S * H;
+  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
+    const int64_t row = idx / H;
+    const int i = (int)(idx % H);
+    float v = 0.f;
+    if (row % S == 0) {
+      const int b = (int)(row / S);
+      for (int j = 0; j < H; ++j) v += dz[(int64_t)b * H + j] * wp[(int64_t)i * H + j];
+    }
+    dx[idx] = from_f32<T>(v);
+  }
+}
+
+template <typename T>
+int classifier_head_t(int B, int S, int H, int C, const void* x, const float* wp, const float* bp, const float* wfc, const float* bfc,
+                      const int32_t* labels, float l2_scale, float scale, float* loss, float* pooled, float* logits, float* dlogits,
+                      float* dz, void* dx, float* dwp, float* dbp, float* dwfc, float* dbfc, hipStream_t s) {
+  hipLaunchKernelGGL(pooler_fwd_kernel<T>, dim3((B * H + 255) / 256), dim3(256), 0, s, B, S, H, (const T*)x, wp, bp, pooled, loss);
+  DS_CHECK_LAUNCH();
+  hipLaunchKernelGGL(classifier_loss_kernel, dim3(1), dim3(256), 0, s, B, H, C, pooled, wfc, bfc, labels, l2_scale, scale, logits,
+                     dlogits, loss);
+  DS_CHECK_LAUNCH();
+  if (!dx && !dwp) return DS_OK;
+  hipLaunchKernelGGL(classifier_bwd_kernel, dim3(((H > C ? H : C) + 255) / 256), dim3(256), 0, s, B, H, C, pooled, wfc, dlogits,
+                     l2_scale, scale, dwfc, dbfc, dz);
+  DS_CHECK_LAUNCH();
+  if (dwp) {
+    hipLaunchKernelGGL(pooler_wgrad_kernel<T>, dim3((unsigned)(((int64_t)H * H + 255) / 256)), dim3(256), 0, s, B, S, H, (const T*)x,
+                       dz, dwp, dbp);
+    DS_CHECK_LAUNCH();
+  }
+  if (dx) {
+    const int64_t total = (int64_t)B * S * H;
+    hipLaunchKernelGGL(pooler_dgrad_kernel<T>, dim3((unsigned)((total + 255) / 256 > 8192 ? 8192 : (total + 255) / 256)), dim3(256), 0, s,
+                       B, S, H, dz, wp, (T*)dx);
+    DS_CHECK_LAUNCH();
+  }
+  return DS_OK;
+}
+
 }  // namespace
+
+extern "C" int ds_classifier_head(int dtype, int batch, int seq, int hidden, int num_labels, const void* x, const float* pooler_w,
+                                  const float* pooler_b, const float* fc_w, const float* fc_b, const int32_t* labels, float l2_scale,
+                                  float loss_scale, float* loss, float* pooled, float* logits, float* dlogits, float* dz, void* dx,
+                                  float* d_pooler_w, float* d_pooler_b, float* d_fc_w, float* d_fc_b, void* stream) {
+  DS_CHECK_ARG(dtype == DS_F32 || dtype == DS_BF16, "ds_classifier_head: dtype %d", dtype);
+  DS_CHECK_ARG(batch > 0 && seq > 0 && hidden > 0, "ds_classifier_head: non-positive shape");
+  DS_CHECK_ARG(num_labels >= 1 && batch * num_labels <= 64, "ds_classifier_head: batch * num_labels (%d) must be at most 64",
+               batch * num_labels);
+  DS_CHECK_ARG(x && pooler_w && pooler_b && fc_w && fc_b && labels && loss && pooled && logits && dlogits && dz,
+               "ds_classifier_head: null pointer");
+  const bool wg = d_pooler_w || d_pooler_b || d_fc_w || d_fc_b;
+  DS_CHECK_ARG(!wg || (d_pooler_w && d_pooler_b && d_fc_w && d_fc_b), "ds_classifier_head: pass all four weight gradients or none");
+  if (dtype == DS_BF16)
+    return classifier_head_t<bf16>(batch, seq, hidden, num_labels, x, pooler_w, pooler_b, fc_w, fc_b, labels, l2_scale, loss_scale, loss,
+                                   pooled, logits, dlogits, dz, dx, d_pooler_w, d_pooler_b, d_fc_w, d_fc_b, (hipStream_t)stream);
+  return classifier_head_t<float>(batch, seq, hidden, num_labels, x, pooler_w, pooler_b, fc_w, fc_b, labels, l2_scale, loss_scale, loss,
+                                  pooled, logits, dlogits, dz, dx, d_pooler_w, d_pooler_b, d_fc_w, d_fc_b, (hipStream_t)stream);
+}
 
 extern "C" int ds_squad_head(int dtype, int batch, int seq, int hidden, const void* x, const float* w, const float* bias,
                              const int32_t* start_positions, const int32_t* end_positions, float loss_scale, float* loss,

@@ -232,3 +232,30 @@ def squad_head(x, batch, seq, output_weights, output_bias, start_positions, end_
                                     ptr(dx), ptr(d_weights), ptr(d_bias), _lib.current_stream()), "ds_squad_head")
     lg = logits.view(batch, seq, 2)
     return loss, lg[:, :, 0], lg[:, :, 1], dx
+
+
+def classifier_head(x, batch, seq, pooler_w, pooler_b, fc_w, fc_b, labels, grads=None, need_dx=True, l2_scale=1e-3,
+                    loss_scale=1.0):
+    """pooler_stage (modeling_slice.py:849-868) + build_output_layer_classification (bert.py:642-664) on the stage's
+    sequence output ``x [batch*seq, hidden]``: returns (loss [1] fp32 on the device, logits [batch, num_labels], pooled
+    [batch, hidden], dx or None).  ``grads`` = (d_pooler_w, d_pooler_b, d_fc_w, d_fc_b), fp32, added to in place."""
+    _need_cuda(x, pooler_w, pooler_b, fc_w, fc_b, labels)
+    hidden = x.shape[-1]
+    if x.numel() != batch * seq * hidden or tuple(pooler_w.shape) != (hidden, hidden) or fc_w.shape[0] != hidden:
+        raise ValueError("classifier_head: x must be [batch*seq, hidden], pooler_w [hidden, hidden], fc_w [hidden, num_labels]")
+    num_labels = fc_w.shape[1]
+    if labels.dtype != torch.int32 or labels.numel() != batch:
+        raise ValueError("classifier_head: labels must be int32 [batch]")
+    grads = tuple(grads) if grads is not None else (None,) * 4
+    for t in (pooler_w, pooler_b, fc_w, fc_b) + grads:
+        if t is not None and (t.dtype != torch.float32 or not t.is_contiguous()):
+            raise ValueError("classifier_head: weights and their gradients must be contiguous fp32")
+    f32 = dict(dtype=torch.float32, device=x.device)
+    loss, pooled = torch.empty(1, **f32), torch.empty(batch, hidden, **f32)
+    logits, dlogits, dz = torch.empty(batch, num_labels, **f32), torch.empty(batch, num_labels, **f32), torch.empty(batch, hidden, **f32)
+    dx = torch.empty_like(x) if need_dx else None
+    check(_lib.load().ds_classifier_head(dtype_code(x), batch, seq, hidden, num_labels, ptr(x), ptr(pooler_w), ptr(pooler_b), ptr(fc_w),
+                                         ptr(fc_b), ptr(labels), l2_scale, loss_scale, ptr(loss), ptr(pooled), ptr(logits), ptr(dlogits),
+                                         ptr(dz), ptr(dx), ptr(grads[0]), ptr(grads[1]), ptr(grads[2]), ptr(grads[3]),
+                                         _lib.current_stream()), "ds_classifier_head")
+    return loss, logits, pooled, dx

@@ -305,6 +305,22 @@ int ds_squad_head(int dtype, int batch, int seq, int hidden, const void* x, cons
                   const int32_t* start_positions, const int32_t* end_positions, float loss_scale, float* loss,
                   float* logits, float* dlogits, void* dx, float* dw, float* dbias, void* stream);
 
+/* Pooler and classification head of the last BERT stage: pooler_stage, bert/models/bert/modeling_slice.py:849-868
+ * (pooled = tanh(dense(first token)), kernel bert/pooler/dense/kernel [hidden, hidden]) and
+ * build_output_layer_classification, bert/models/bert/bert.py:642-664 (fully_connected to num_labels, weights
+ * src-output-layer/FC/weights [hidden, num_labels]; loss = mean sparse softmax cross entropy + the l2 regulariser
+ * l2_scale * sum(FC weights^2) / 2, 1e-3 in the reference).
+ *   x [batch*seq, hidden] (compute type): the stage's sequence output; labels [batch] int32;
+ *   out: loss (device float, loss_scale * loss), pooled [batch, hidden], logits [batch, num_labels],
+ *   dlogits [batch, num_labels] fp32; dz [batch, hidden] fp32 scratch;
+ *   dx (nullable): d loss / d x, zero except on each sample's first token - the d_out of the stage's backward pass;
+ *   d_pooler_w, d_pooler_b, d_fc_w, d_fc_b (all or none): master gradients, added to.
+ * batch * num_labels <= 64.  A label outside [0, num_labels) gives a NaN loss, as TensorFlow's GPU kernel does. */
+int ds_classifier_head(int dtype, int batch, int seq, int hidden, int num_labels, const void* x, const float* pooler_w,
+                       const float* pooler_b, const float* fc_w, const float* fc_b, const int32_t* labels, float l2_scale,
+                       float loss_scale, float* loss, float* pooled, float* logits, float* dlogits, float* dz, void* dx,
+                       float* d_pooler_w, float* d_pooler_b, float* d_fc_w, float* d_fc_b, void* stream);
+
 /* ---- what the reference runs on the accumulated gradients right after the unroll block ----
  *
  * Global-norm clipping, bert/graph.py:162-165 (tf.clip_by_global_norm over all accumulated gradients):

@@ -92,3 +92,35 @@ def test_last_stage_step_with_the_head():
             floor = float(acc[2 + names.index(n.replace("/beta", "/gamma"))].abs().max())
         assert_close(st.grads[n], g.reshape(st.grads[n].shape), 1e-4, "grad " + n, floor=floor)
     st.close()
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 2e-2)])
+@pytest.mark.parametrize("B,S,H,C", [(2, 16, 64, 2), (3, 128, 1024, 2), (1, 4, 8, 5)])
+def test_classifier_head_matches_oracle(dtype, tol, B, S, H, C):
+    r = np.random.default_rng(B * S + H + C)
+    x = dev(r.standard_normal((B * S, H)), dtype)
+    wp = dev(r.standard_normal((H, H)) / np.sqrt(H), torch.float32)
+    bp = dev(r.standard_normal(H) * 0.1, torch.float32)
+    wf = dev(r.standard_normal((H, C)) * 0.3, torch.float32)
+    bf = dev(np.full(C, 1e-4), torch.float32)                  # biases_initializer=constant(1e-04), bert.py:650
+    y_np = r.integers(0, C, B).astype(np.int32)
+    y = torch.as_tensor(y_np).cuda()
+    grads = [torch.ones_like(t) for t in (wp, bp, wf, bf)]      # pre-filled: the head adds into the master gradients
+    loss, logits, pooled, dx = ops.classifier_head(x, B, S, wp, bp, wf, bf, y, grads)
+    xo = x.cpu().double().reshape(B, S, H).requires_grad_(True)
+    ws = [t.cpu().double().requires_grad_(True) for t in (wp, bp, wf, bf)]
+    lo, lgo, po = oh.classification_loss(xo, ws[0], ws[1], ws[2], ws[3], torch.as_tensor(y_np))
+    gx, *gw = torch.autograd.grad(lo, [xo] + ws)
+    assert_close(loss, lo.reshape(1), tol, "loss")
+    assert_close(logits, lgo, tol, "logits")
+    assert_close(pooled, po, tol, "pooled")
+    assert_close(dx, gx.reshape(B * S, H), tol, "dx")
+    assert float(dx.reshape(B, S, H)[:, 1:].abs().max() if S > 1 else 0.0) == 0.0   # only the first token has a gradient
+    for g, ref, name in zip(grads, gw, ("pooler kernel", "pooler bias", "FC weights", "FC biases")):
+        assert_close(g - 1, ref, tol, "d " + name, floor=float(gw[2].abs().max()) if name == "FC biases" else None)
+    # loss_scale scales loss and gradients; no gradient buffers: forward only
+    loss2, _, _, dx2 = ops.classifier_head(x, B, S, wp, bp, wf, bf, y, None, loss_scale=4.0)
+    assert_close(loss2, 4 * lo.reshape(1), tol, "scaled loss")
+    assert_close(dx2, 4 * gx.reshape(B * S, H), tol, "scaled dx")
+    with pytest.raises(ValueError):
+        ops.classifier_head(x, B, S, wp, bp, wf, bf, y.long())

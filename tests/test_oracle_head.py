@@ -38,3 +38,33 @@ def test_out_of_range_position_gives_no_loss_term():
     part, sl, _ = oh.squad_loss(x, w, b, torch.tensor([1, 9]), torch.tensor([0, 3]))
     missing = -torch.log_softmax(sl[1], -1)[2] / (2 * 2)
     assert abs((full - part).item() - missing.item()) < 1e-12
+
+
+def test_classification_head_matches_library_and_brute_force():
+    torch.manual_seed(2)
+    B, S, H, C = 3, 4, 5, 2
+    x = torch.randn(B, S, H, dtype=torch.float64)
+    wp, bp = torch.randn(H, H, dtype=torch.float64) * 0.5, torch.randn(H, dtype=torch.float64) * 0.1
+    wf = (torch.randn(H, C, dtype=torch.float64) * 0.5).requires_grad_(True)
+    bf = torch.full((C,), 1e-4, dtype=torch.float64)
+    y = torch.tensor([1, 0, 1])
+    loss, logits, pooled = oh.classification_loss(x, wp, bp, wf, bf, y, l2_scale=1e-3)
+    # library routines: Linear + tanh on the FIRST token, mean cross entropy; the regulariser by its closed form
+    lin = torch.nn.Linear(H, H).double()
+    with torch.no_grad():
+        lin.weight.copy_(wp.t()); lin.bias.copy_(bp)
+    assert torch.allclose(pooled, torch.tanh(lin(x[:, 0])), atol=1e-12)
+    ce = torch.nn.functional.cross_entropy(pooled @ wf + bf, y)
+    assert abs(loss.item() - (ce.item() + 1e-3 * 0.5 * float((wf.detach() ** 2).sum()))) < 1e-12
+    # the gradient of the regulariser alone is scale * w (tf.nn.l2_loss = sum(w^2) / 2)
+    (g_all,) = torch.autograd.grad(loss, wf, retain_graph=True)
+    (g_ce,) = torch.autograd.grad(ce, wf)
+    assert torch.allclose(g_all - g_ce, 1e-3 * wf.detach(), atol=1e-12)
+    # brute force on one sample
+    b = 2
+    z = [math.tanh(sum(x[b, 0, i].item() * wp[i, j].item() for i in range(H)) + bp[j].item()) for j in range(H)]
+    lg = [sum(z[j] * wf[j, c].item() for j in range(H)) + bf[c].item() for c in range(C)]
+    assert abs(lg[0] - logits[b, 0].item()) < 1e-12 and abs(lg[1] - logits[b, 1].item()) < 1e-12
+    # tokens other than the first do not enter
+    x2 = x.clone(); x2[:, 1:] += 1.0
+    assert abs(oh.classification_loss(x2, wp, bp, wf, bf, y)[0].item() - loss.item()) < 1e-12

@@ -64,6 +64,18 @@ def test_bert_finetune_slice_puts_the_planner_split_on_each_device():
     s1.stage.backward(0, dy, torch.empty_like(h))
     with pytest.raises(ValueError, match="does not hold"):
         s0.build_output_layer_squad(y)
+    # model_type='classification' (bert.py:463-464): pooler + FC over two classes on the last device
+    s2 = slices.BertFinetuneSlice(cfg, 8, False, ids, None, None, [1, 0], False, model_type="classification",
+                                  slice_devices="/gpu:0,/gpu:1", local_device=1, dtype="fp32")
+    s2.stage.forward(0, h, y)
+    dy = s2.build_output_layer_classification(y.reshape(2, 8, 32))
+    assert s2.stage_outputs[-1] is s2.loss and 0.0 < float(s2.loss) < 10.0
+    assert tuple(s2.logits.shape) == (2, 2) and tuple(s2.pooled_output.shape) == (2, 32) and tuple(s2.predictions.shape) == (2,)
+    assert float(dy.reshape(2, 8, 32)[:, 1:].abs().max()) == 0.0 and float(dy.reshape(2, 8, 32)[:, 0].abs().max()) > 0
+    assert all(float(g.abs().max()) > 0 for g in s2.head_grads)
+    s2.stage.backward(0, dy, torch.empty_like(h))
+    with pytest.raises(ValueError, match="does not hold"):
+        s1.build_output_layer_classification(y)
     s0.stage.close(); s1.stage.close()
 
 
