@@ -83,6 +83,9 @@ struct LayerDy {
 struct Deferred {
   int xpos, dypos;
 };
+struct Run {  // n micro-batches back to back in the stash and in the operand ring
+  int xpos, dypos, n;
+};
 
 struct BertStage : ds_stage {
   int L, H, F, NH, D, B, S, rows;
@@ -468,8 +471,19 @@ struct BertStage : ds_stage {
     const char* dy = (const char*)d_out;
     // With a weight-gradient stream the wgrad GEMMs and bias column sums of a layer run beside the
     // dgrad chain of the layers below it: they only feed the master gradients.
-    hipStream_t ws = G > 1 ? nullptr : wgrad_stream;  // deferred weight gradients go there in flush_deferred
-    if (ws) DS_PROPAGATE(lane.ensure());
+    hipStream_t ws = G > 1 ? nullptr : wgrad_stream;
+    // Grouped weight gradients: the pass that completes a group issues the group's GEMMs layer by layer as its own
+    // chain passes each layer, so that they run beside the chain of the layers below instead of after the pass.
+    const bool closing = G > 1 && (int)deferred.size() + 1 >= G;
+    std::vector<Run> runs;
+    hipStream_t gws = nullptr;
+    if (closing) {
+      std::vector<Deferred> all = deferred;
+      all.push_back({pos, dypos});
+      runs = make_runs(all);
+      gws = wgrad_stream ? wgrad_stream : stream;
+    }
+    if (ws || (gws && gws != stream)) DS_PROPAGATE(lane.ensure());
     for (int l = L - 1; l >= 0; --l) {
       const LayerStash& t = ls[l];
       const int b = base(l);
@@ -529,6 +543,13 @@ struct BertStage : ds_stage {
         stream = chain;
         if (rc != DS_OK) return rc;
         if (ws) DS_PROPAGATE(lane.end(ws, par));
+      } else if (closing) {
+        hipStream_t chain = stream;
+        if (gws != chain) DS_PROPAGATE(lane.begin(chain, gws, par));
+        stream = gws;
+        const int rc = layer_wgrad_runs(l, runs);
+        stream = chain;
+        if (rc != DS_OK) return rc;
       }
       // dx = dqkv Wqkv^T + dz1 (x also feeds the residual into z1)
       const bool first = (l == 0);
@@ -567,8 +588,43 @@ struct BertStage : ds_stage {
       } else {
         x_bwd_valid[pos] = 0;
       }
-      if ((int)deferred.size() >= G) DS_PROPAGATE(flush_deferred(false));
+      if (closing) DS_PROPAGATE(retire_deferred(gws, stream));
     }
+    return DS_OK;
+  }
+
+  // runs of micro-batches that sit back to back in both rings: one set of GEMMs per run
+  static std::vector<Run> make_runs(const std::vector<Deferred>& d) {
+    std::vector<Run> runs;
+    size_t i = 0;
+    while (i < d.size()) {
+      size_t j = i + 1;
+      while (j < d.size() && d[j].xpos == d[j - 1].xpos + 1 && d[j].dypos == d[j - 1].dypos + 1) ++j;
+      runs.push_back({d[i].xpos, d[i].dypos, (int)(j - i)});
+      i = j;
+    }
+    return runs;
+  }
+  int layer_wgrad_runs(int l, const std::vector<Run>& runs) {
+    const LayerStash& t = ls[l];
+    for (const Run& r : runs)
+      DS_PROPAGATE(layer_wgrad(l, r.n * rows, at(t.x, r.xpos), at(t.ctx, r.xpos), at(t.a, r.xpos), at(t.h, r.xpos),
+                               dy_base + ld[l].dz2 + r.dypos * dy_act, dy_base + ld[l].du + r.dypos * dy_actF,
+                               dy_base + ld[l].dz1 + r.dypos * dy_act, dy_base + ld[l].dqkv + r.dypos * 3 * dy_act));
+    return DS_OK;
+  }
+  // the weight-gradient work of every deferred pass has been queued on `ws`
+  int retire_deferred(hipStream_t ws, hipStream_t chain) {
+    for (const Deferred& e : deferred) {
+      if (ws != chain) {
+        DS_CHECK_HIP(hipEventRecord(ev_x_wg[e.xpos], ws));
+        DS_CHECK_HIP(hipEventRecord(ev_dy_wg[e.dypos], ws));
+      }
+      x_wg_valid[e.xpos] = dy_wg_valid[e.dypos] = ws != chain;
+      pos_deferred[e.xpos] = 0;
+    }
+    deferred.clear();
+    if (ws != chain) wg_outstanding = true;
     return DS_OK;
   }
 
@@ -616,34 +672,11 @@ struct BertStage : ds_stage {
       hipStream_t keep = stream;
       stream = ws;
       int rc = DS_OK;
-      // runs of micro-batches that sit back to back in both rings: one set of GEMMs per run
-      size_t i = 0;
-      while (i < deferred.size() && rc == DS_OK) {
-        size_t j = i + 1;
-        while (j < deferred.size() && deferred[j].xpos == deferred[j - 1].xpos + 1 &&
-               deferred[j].dypos == deferred[j - 1].dypos + 1)
-          ++j;
-        const int n = (int)(j - i), xp = deferred[i].xpos, dp = deferred[i].dypos;
-        for (int l = L - 1; l >= 0 && rc == DS_OK; --l) {
-          const LayerStash& t = ls[l];
-          rc = layer_wgrad(l, n * rows, at(t.x, xp), at(t.ctx, xp), at(t.a, xp), at(t.h, xp),
-                           dy_base + ld[l].dz2 + dp * dy_act, dy_base + ld[l].du + dp * dy_actF,
-                           dy_base + ld[l].dz1 + dp * dy_act, dy_base + ld[l].dqkv + dp * 3 * dy_act);
-        }
-        i = j;
-      }
+      const std::vector<Run> runs = make_runs(deferred);
+      for (int l = L - 1; l >= 0 && rc == DS_OK; --l) rc = layer_wgrad_runs(l, runs);
       stream = keep;
       if (rc != DS_OK) return rc;
-      for (const Deferred& e : deferred) {
-        if (ws != chain) {
-          DS_CHECK_HIP(hipEventRecord(ev_x_wg[e.xpos], ws));
-          DS_CHECK_HIP(hipEventRecord(ev_dy_wg[e.dypos], ws));
-        }
-        x_wg_valid[e.xpos] = dy_wg_valid[e.dypos] = ws != chain;
-        pos_deferred[e.xpos] = 0;
-      }
-      deferred.clear();
-      if (ws != chain) wg_outstanding = true;
+      DS_PROPAGATE(retire_deferred(ws, chain));
     }
     if (final && wg_outstanding) {
       DS_CHECK_HIP(hipEventRecord(ev_wg_done, wgrad_owned));
