@@ -300,3 +300,42 @@ def test_grouped_weight_gradients_over_steps_and_streams():
         for k in res[0][2]:
             a, b = res[0][2][k], other[2][k]
             assert float((a - b).abs().max()) <= 2e-5 * float(a.abs().max()) + 1e-12, k
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("overlap", [False, True])
+def test_grouped_weight_gradients_any_call_order(overlap):
+    """Backward passes out of forward order, a slot held across many passes of the others, a join in the middle of a
+    group: the operands of a group then do not sit back to back and the group splits into several GEMMs.  Same
+    gradients as with per-pass weight gradients."""
+    L, H, N, F, B, S = 2, 64, 4, 128, 2, 16
+    w = synthetic.bert_weights(41, L, H, F)
+    n = 9
+    xs = [torch.as_tensor(x).cuda() for x in synthetic.bert_activation_inputs(42, n, B, S, H)]
+    dys = [torch.as_tensor(x).cuda() for x in synthetic.upstream_grads(43, n, (B * S, H))]
+    # (op, slot, micro-batch): slot 2 is held from the start to the end; slots 0/1 go out of order
+    prog = [("F", 2, 0), ("F", 0, 1), ("F", 1, 2), ("B", 1, 2), ("B", 0, 1), ("F", 1, 3), ("F", 0, 4), ("B", 1, 3), ("J",),
+            ("F", 1, 5), ("B", 0, 4), ("B", 1, 5), ("F", 0, 6), ("F", 1, 7), ("B", 0, 6), ("F", 0, 8), ("B", 0, 8), ("B", 1, 7),
+            ("B", 2, 0)]
+    res = []
+    for group in (1, 3):
+        st = runtime.bert_stage(L, H, N, F, B, S, "fp32", stash_slots=3, wgrad_group=group)
+        st.bind(w)
+        if overlap:
+            st.enable_overlap()
+        outs = [torch.empty(B * S, H, device="cuda") for _ in range(n)]
+        dxs = [torch.empty(B * S, H, device="cuda") for _ in range(n)]
+        for op in prog:
+            if op[0] == "F":
+                st.forward(op[1], xs[op[2]], outs[op[2]])
+            elif op[0] == "B":
+                st.backward(op[1], dys[op[2]], dxs[op[2]])
+            else:
+                st.join()
+        st.sync()
+        res.append((torch.stack(outs).cpu(), torch.stack(dxs).cpu(), {k: v.cpu().clone() for k, v in st.grads.items()}))
+        st.close()
+    assert torch.equal(res[0][0], res[1][0]) and torch.equal(res[0][1], res[1][1])
+    for k in res[0][2]:
+        a, b = res[0][2][k], res[1][2][k]
+        assert float((a - b).abs().max()) <= 2e-5 * float(a.abs().max()) + 1e-10, k
