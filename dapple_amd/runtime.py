@@ -314,3 +314,78 @@ class StageRuntime:
                 free.append(slot)
         self.stage.join()
         return outputs
+
+
+class PipelineRuntime:
+    """All S stages of a sliced model on ONE GPU, M micro-batches: the unrolled graph of bert/graph.py:97-161 with the
+    stage boundaries as device tensors instead of sends.  Every stage issues its own early-backward order
+    (``schedule_ops(i, S, M)``, the rule of bert/graph.py:126-132); an operation is issued once its data is there -
+    F(i, j) after F(i-1, j), B(i, j) after B(i+1, j), the last stage's backward after ``loss_fn`` - so the global order
+    is one the reference's control dependencies allow.  ``loss_fn(j, last_output) -> (loss, d_last_output)`` is the
+    last stage's head.  ``step`` returns the per-micro-batch losses (``losses[-1]`` is the reference's ``_loss_fn``,
+    bert/graph.py:166); weight gradients accumulate in each stage's ``grads``; ``all_outputs[j][i]`` keeps the boundary
+    tensor of micro-batch j leaving stage i, like the reference's list of the same name."""
+
+    def __init__(self, stages, num_micro_batches, loss_fn, variant="S"):
+        self.stages, self.m, self.loss_fn = list(stages), num_micro_batches, loss_fn
+        S = len(self.stages)
+        self.ops = [schedule_ops(i, S, num_micro_batches, variant) for i in range(S)]
+        for i, st in enumerate(self.stages):
+            k = min(stash_depth(i, S, variant), num_micro_batches)
+            if st.stash_slots < k:
+                raise ValueError("stage %d has %d stash slots, the schedule needs %d" % (i, st.stash_slots, k))
+            if getattr(st, "overlap", False):
+                raise ValueError("PipelineRuntime hands tensors from stage to stage in the order of one stream: "
+                                 "switch the stages' forward/backward overlap off")
+            if i > 0 and st.in_numel != self.stages[i - 1].out_numel:
+                raise ValueError("stage %d takes %d elements, stage %d hands over %d" % (i, st.in_numel, i - 1, self.stages[i - 1].out_numel))
+        self.issued = []          # (stage, op, micro-batch) in issue order, for inspection
+
+    def step(self, inputs, key_masks=None):
+        S, M = len(self.stages), self.m
+        if len(inputs) != M:
+            raise ValueError("expected %d micro-batches" % M)
+        dev = inputs[0].device
+        self.all_outputs = [[torch.empty(st.out_numel, dtype=st.act_dtype, device=dev) for st in self.stages] for _ in range(M)]
+        in_grads = [[torch.empty(st.in_numel, dtype=st.act_dtype, device=dev) if st.takes_input_grad else None
+                     for st in self.stages] for _ in range(M)]
+        d_last = [None] * M
+        losses = [None] * M
+        fdone = [[False] * M for _ in range(S)]
+        bdone = [[False] * M for _ in range(S)]
+        cursor = [0] * S
+        slot_of = [dict() for _ in range(S)]
+        free = [list(range(st.stash_slots)) for st in self.stages]
+        self.issued = []
+        remaining = sum(len(o) for o in self.ops)
+        while remaining:
+            progressed = False
+            for i, st in enumerate(self.stages):
+                while cursor[i] < len(self.ops[i]):
+                    op, j = self.ops[i][cursor[i]]
+                    if op == "F":
+                        if i > 0 and not fdone[i - 1][j]:
+                            break
+                        slot = free[i].pop(0)
+                        slot_of[i][j] = slot
+                        x = inputs[j] if i == 0 else self.all_outputs[j][i - 1]
+                        st.forward(slot, x, self.all_outputs[j][i], None if key_masks is None else key_masks[j])
+                        fdone[i][j] = True
+                        if i == S - 1:
+                            losses[j], d_last[j] = self.loss_fn(j, self.all_outputs[j][i])
+                    else:
+                        if i < S - 1 and not bdone[i + 1][j]:
+                            break
+                        d_out = d_last[j] if i == S - 1 else in_grads[j][i + 1]
+                        st.backward(slot_of[i][j], d_out.reshape(-1), in_grads[j][i])
+                        free[i].append(slot_of[i].pop(j))
+                        bdone[i][j] = True
+                    self.issued.append((i, op, j))
+                    cursor[i] += 1
+                    remaining -= 1
+                    progressed = True
+            if not progressed:
+                raise RuntimeError("pipeline schedule cannot make progress")
+        for st in self.stages:
+            st.join()
+        return losses

@@ -1,0 +1,91 @@
+"""All stages of a sliced BERT on one GPU under the unrolled early-backward graph (bert/graph.py:97-161): losses,
+boundary tensors and the accumulated gradients of every stage and of the head against autograd through the whole model."""
+import numpy as np
+import pytest
+import torch
+
+from dapple_amd import ops, runtime, synthetic
+from oracle import bert as ob
+from oracle import head as oh
+from util import assert_close, dev
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("split,M", [((1, 2, 1), 5), ((2, 2), 3), ((4,), 2)])
+def test_whole_model_pipeline_matches_autograd(split, M):
+    H, N, F, B, S, V = 64, 4, 128, 2, 16, 50
+    L = sum(split)
+    emb = (V, 2, 32)
+    w_np = synthetic.bert_weights(51, L, H, F, embeddings=emb, stddev=0.05, perturb=True)
+    r = np.random.default_rng(52)
+    hw_np, hb_np = r.standard_normal((2, H)) * 0.05, r.standard_normal(2) * 0.05
+    ids_np = synthetic.bert_id_inputs(53, M, B, S, V)
+    sp_np = r.integers(0, S, (M, B)).astype(np.int32)
+    ep_np = r.integers(0, S, (M, B)).astype(np.int32)
+    nst = len(split)
+    stages, first = [], 0
+    for i, n in enumerate(split):
+        st = runtime.bert_stage(n, H, N, F, B, S, "fp32", stash_slots=runtime.stash_depth(i, nst),
+                                embeddings=emb if i == 0 else None, first_layer=first, wgrad_group=2 if i == 0 else 1)
+        st.bind(w_np)
+        stages.append(st)
+        first += n
+    hw, hb = dev(hw_np, torch.float32), dev(hb_np, torch.float32)
+    dhw, dhb = torch.zeros_like(hw), torch.zeros_like(hb)
+    sp, ep = [dev(x) for x in sp_np], [dev(x) for x in ep_np]
+
+    def loss_fn(j, out):
+        loss, _, _, dx = ops.squad_head(out.reshape(B * S, H), B, S, hw, hb, sp[j], ep[j], dhw, dhb)
+        return loss, dx
+
+    pipe = runtime.PipelineRuntime(stages, M, loss_fn)
+    losses = pipe.step([dev(x) for x in ids_np])
+    torch.cuda.synchronize()
+    # every stage issued its own early-backward order, and nothing ran before its data existed
+    for i in range(nst):
+        assert [(op, j) for (s, op, j) in pipe.issued if s == i] == runtime.schedule_ops(i, nst, M)
+    seen = set()
+    for s, op, j in pipe.issued:
+        if op == "F":
+            assert s == 0 or (s - 1, "F", j) in seen
+        else:
+            assert (s, "F", j) in seen and (s == nst - 1 or (s + 1, "B", j) in seen)
+        seen.add((s, op, j))
+    # oracle: the un-sliced model, one autograd pass per micro-batch, gradients summed (tf.accumulate_n)
+    w_t = ob.to_torch(w_np, torch.float64, requires_grad=True)
+    hw_t = torch.as_tensor(hw_np).double().requires_grad_(True)
+    hb_t = torch.as_tensor(hb_np).double().requires_grad_(True)
+    names = sorted(w_t)
+    acc = None
+    for j in range(M):
+        x = ob.stage_forward(torch.as_tensor(ids_np[j]), w_t, list(range(L)), B, S, N)
+        lo, _, _ = oh.squad_loss(x.reshape(B, S, H), hw_t, hb_t, torch.as_tensor(sp_np[j]), torch.as_tensor(ep_np[j]))
+        assert_close(losses[j], lo.reshape(1), 1e-4, "loss mb%d" % j)
+        assert_close(pipe.all_outputs[j][-1], x.reshape(-1), 1e-4, "last boundary tensor mb%d" % j)
+        g = torch.autograd.grad(lo, [w_t[n] for n in names] + [hw_t, hb_t], allow_unused=True)
+        acc = list(g) if acc is None else [a + b if b is not None else a for a, b in zip(acc, g)]
+    ref = dict(zip(names, acc[:-2]))
+    for st in stages:
+        for n in st.weight_names:
+            floor = ref[n.replace("/key/", "/query/")].abs().max().item() if n.endswith("/key/bias") else None
+            if n == "bert/encoder/layer_%d/output/LayerNorm/beta" % (L - 1):
+                # the head's input gradient sums to zero over the sequence (softmax minus one-hot), so this one
+                # vanishes identically: judge it on the scale of gamma's gradient
+                floor = ref[n.replace("beta", "gamma")].abs().max().item()
+            assert_close(st.grads[n], ref[n], 1e-4, "accumulated grad " + n, floor=floor)
+    assert_close(dhw, acc[-2], 1e-4, "head weights")
+    assert_close(dhb, acc[-1], 1e-4, "head bias", floor=float(acc[-2].abs().max()))
+    for st in stages:
+        st.close()
+
+
+def test_pipeline_rejects_mismatched_stages():
+    a = runtime.bert_stage(1, 64, 4, 128, 2, 16, "fp32", stash_slots=2)
+    b = runtime.bert_stage(1, 32, 4, 64, 2, 16, "fp32", stash_slots=1)
+    with pytest.raises(ValueError, match="hands over"):
+        runtime.PipelineRuntime([a, b], 2, lambda j, out: (None, out))
+    with pytest.raises(ValueError, match="stash slots"):
+        runtime.PipelineRuntime([b, b], 2, lambda j, out: (None, out))
+    a.close()
+    b.close()
