@@ -110,41 +110,73 @@ __global__ __launch_bounds__(256) void xl_softmax_fwd_kernel(int Q, int K, int R
   }
 }
 
-// dbd[i][r] = ds[i][r - Q + i] when that column exists, else 0 (transpose of the rel_shift index map)
-template <typename T>
-__global__ __launch_bounds__(256) void xl_unshift_kernel(int64_t rows, int Q, int K, int R, const T* __restrict__ ds, T* __restrict__ dbd) {
-  const int64_t total = rows * R;
-  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
-    const int r = (int)(idx % R);
-    const int64_t w = idx / R;
-    const int i = (int)(w % Q);
-    const int j = r - Q + i;
-    dbd[idx] = (j >= 0 && j < K) ? ds[w * K + j] : from_f32<T>(0.f);
+// Softmax backward of one score row (b, n, i) per wave, with everything else that needs the row while it is in
+// registers: ds[j] = scale * p[j] * (dp[j] - sum_k p[k] dp[k]);
+//   dbd[i][r] = ds[i][r - Q + i] when that column exists, else 0 (transpose of the rel_shift index map);
+//   def[s] = sum_j [seg(i,j,b) == s] ds[i][j] (gradient of the two segment scores of the row).
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void xl_softmax_bwd_kernel(int Q, int K, int R, int B, int N, const T* __restrict__ p,
+                                                            const float* __restrict__ dp, float scale,
+                                                            const uint8_t* __restrict__ seg_mat, T* __restrict__ ds,
+                                                            T* __restrict__ dbd, float* __restrict__ defs) {
+  const int lane = threadIdx.x & 63;
+  const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (w >= (int64_t)B * N * Q) return;
+  const int i = (int)(w % Q);
+  const int b = (int)(w / Q) / N;
+  const T* pr = p + w * K;
+  const float* dr = dp + w * K;
+  float pv[NV][4], dv[NV][4];
+  float dot = 0.f;
+#pragma unroll
+  for (int v = 0; v < NV; ++v) {
+    const int c = (lane + v * 64) * 4;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (c < K) { pv[v][e] = to_f32(pr[c + e]); dv[v][e] = dr[c + e]; } else { pv[v][e] = 0.f; dv[v][e] = 0.f; }
+      dot += pv[v][e] * dv[v][e];
+    }
   }
+  dot = wave_sum(dot);
+  T* out = ds + w * K;
+  T* brow = dbd + w * R;
+  const int shift = Q - i;  // column j of ds lands in column j + Q - i of dbd
+  float d0 = 0.f, d1 = 0.f;
+#pragma unroll
+  for (int v = 0; v < NV; ++v) {
+    const int c = (lane + v * 64) * 4;
+    if (c < K) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const T val = from_f32<T>(scale * pv[v][e] * (dv[v][e] - dot));
+        out[c + e] = val;
+        brow[c + e + shift] = val;
+        const float f = to_f32(val);
+        if (seg_mat && seg_mat[((int64_t)i * K + c + e) * B + b]) d1 += f; else d0 += f;
+      }
+    }
+  }
+  for (int r = lane; r < shift; r += 64) brow[r] = from_f32<T>(0.f);
+  for (int r = shift + K + lane; r < R; r += 64) brow[r] = from_f32<T>(0.f);
+  d0 = wave_sum(d0);
+  d1 = wave_sum(d1);
+  if (lane == 0) { defs[w * 2] = d0; defs[w * 2 + 1] = d1; }
 }
 
-// One wave per (i, b, n): def[s] = sum_j [seg(i,j,b) == s] ds[i][j]; writes def to deft[(n*2+s)][row] for the
-// seg_emb gradient GEMM, dqs = def[0]*seg_emb[0] + def[1]*seg_emb[1], and dq = dqw + dqr + dqs.
+// One wave per (i, b, n): writes def to deft[(n*2+s)][row] for the seg_emb gradient GEMM,
+// dqs = def[0]*seg_emb[0] + def[1]*seg_emb[1], and dq = dqw + dqr + dqs.
 template <typename T>
-__global__ __launch_bounds__(256) void xl_seg_bwd_kernel(int Q, int K, int B, int N, int D, int64_t rows_total, int64_t row0,
-                                                        const T* __restrict__ ds, const uint8_t* __restrict__ seg_mat,
-                                                        const float* __restrict__ seg_emb, const T* __restrict__ dqw,
-                                                        const T* __restrict__ dqr, T* __restrict__ dqs, T* __restrict__ dq,
-                                                        T* __restrict__ deft) {
+__global__ __launch_bounds__(256) void xl_seg_bwd_kernel(int Q, int B, int N, int D, int64_t rows_total, int64_t row0,
+                                                        const float* __restrict__ defs, const float* __restrict__ seg_emb,
+                                                        const T* __restrict__ dqw, const T* __restrict__ dqr, T* __restrict__ dqs,
+                                                        T* __restrict__ dq, T* __restrict__ deft) {
   const int lane = threadIdx.x & 63;
   const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (w >= (int64_t)B * N * Q) return;
   const int i = (int)(w % Q);
   const int bn = (int)(w / Q), n = bn % N, b = bn / N;
   const int H = N * D;
-  const T* dr = ds + w * K;
-  float d0 = 0.f, d1 = 0.f;
-  for (int j = lane; j < K; j += 64) {
-    const float v = to_f32(dr[j]);
-    if (seg_mat && seg_mat[((int64_t)i * K + j) * B + b]) d1 += v; else d0 += v;
-  }
-  d0 = wave_sum(d0);
-  d1 = wave_sum(d1);
+  const float d0 = defs[w * 2], d1 = defs[w * 2 + 1];
   const int64_t row = (int64_t)i * B + b;  // row inside this stream
   if (lane == 0) {
     deft[(int64_t)(n * 2 + 0) * rows_total + row0 + row] = from_f32<T>(d0);
@@ -177,7 +209,7 @@ struct XlnetStage : ds_stage {
   // workspace
   char* ws_base = nullptr;
   // buffers the weight-gradient kernels read alternate by layer parity ([2])
-  size_t ws_bytes = 0, ws_qall, ws_ac, ws_dp, ws_bd, ws_ds, ws_dbd, ws_dz2[2], ws_du[2], ws_dy1, ws_dz1[2], ws_dvec, ws_dqw[2], ws_dqr[2],
+  size_t ws_bytes = 0, ws_qall, ws_ac, ws_dp, ws_bd, ws_ds, ws_dbd, ws_def, ws_dz2[2], ws_du[2], ws_dy1, ws_dz1[2], ws_dvec, ws_dqw[2], ws_dqr[2],
          ws_dqs[2], ws_dq[2], ws_dkv[2], ws_dkr[2], ws_deft[2], ws_dx[2];
   WgradLane lane;
 
@@ -256,6 +288,7 @@ struct XlnetStage : ds_stage {
     ws_bd = w.reserve((size_t)B * N * Q * R * 4);
     ws_ds = w.reserve((size_t)B * N * Q * K * esz);
     ws_dbd = w.reserve((size_t)B * N * Q * R * esz);
+    ws_def = w.reserve((size_t)B * N * Q * 2 * 4);
     ws_dy1 = w.reserve(act); ws_dvec = w.reserve(act);
     for (int p = 0; p < 2; ++p) {
       ws_dz2[p] = w.reserve(act); ws_du[p] = w.reserve(actF); ws_dz1[p] = w.reserve(act);
@@ -357,6 +390,20 @@ struct XlnetStage : ds_stage {
     return DS_OK;
   }
 
+  template <typename T> int softmax_bwd_t(const T* p, const float* dp, float scale, const uint8_t* seg, T* dsm, T* dbd, float* defs) {
+    const int64_t waves = (int64_t)B * N * Q;
+    dim3 grid((unsigned)((waves + 3) / 4));
+    const int need = (K + 255) / 256;
+    ds_prof_scope prof(stream, sizeof(T) == 2 ? "xl_softmax_bwd_kernel<bf16>" : "xl_softmax_bwd_kernel<float>",
+                       (double)waves * (K * (4 + 2 * sizeof(T)) + R * sizeof(T)), "B");
+    if (need <= 1) hipLaunchKernelGGL((xl_softmax_bwd_kernel<T, 1>), grid, dim3(256), 0, stream, Q, K, R, B, N, p, dp, scale, seg, dsm, dbd, defs);
+    else if (need <= 2) hipLaunchKernelGGL((xl_softmax_bwd_kernel<T, 2>), grid, dim3(256), 0, stream, Q, K, R, B, N, p, dp, scale, seg, dsm, dbd, defs);
+    else if (need <= 4) hipLaunchKernelGGL((xl_softmax_bwd_kernel<T, 4>), grid, dim3(256), 0, stream, Q, K, R, B, N, p, dp, scale, seg, dsm, dbd, defs);
+    else hipLaunchKernelGGL((xl_softmax_bwd_kernel<T, 8>), grid, dim3(256), 0, stream, Q, K, R, B, N, p, dp, scale, seg, dsm, dbd, defs);
+    DS_CHECK_LAUNCH();
+    return DS_OK;
+  }
+
   int forward(int slot, const void* in, const float*, void* out) override {
     ds_prio_scope prio(1);
     char* sp = stash_base + (size_t)slot * slot_bytes;
@@ -453,19 +500,16 @@ struct XlnetStage : ds_stage {
                              2 * H, D, dp, K, (int64_t)N * Q * K, (int64_t)Q * K, DS_EPI_OUT_F32));
         DS_PROPAGATE(gemm_bn(DS_MN_MAJOR, DS_MN_MAJOR, K, D, Q, p, K, (int64_t)N * Q * K, (int64_t)Q * K, dvec + so, (int64_t)B * H, H, D,
                              dkv + (size_t)H * esz, (int64_t)B * 2 * H, 2 * H, D, acc, dkv + (size_t)H * esz));
-        DS_PROPAGATE(ds_softmax_bwd(dtype, (int64_t)B * N * Q, K, p, dp, scale, dsm, stream));
+        // dS, its un-shifted copy for the position term (dbd[i][r] = dS[i][r - Q + i]) and the segment sums, in one pass
+        float* defs = (float*)(ws_base + ws_def);
+        if (dtype == DS_BF16) DS_PROPAGATE(softmax_bwd_t<bf16>((const bf16*)p, dp, scale, seg, (bf16*)dsm, (bf16*)dbd, defs));
+        else DS_PROPAGATE(softmax_bwd_t<float>((const float*)p, dp, scale, seg, (float*)dsm, (float*)dbd, defs));
         // content term: dqw = dS k ; dk (+)= dS^T qw
         DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_MN_MAJOR, Q, D, K, dsm, K, (int64_t)N * Q * K, (int64_t)Q * K, sp + t.kv, (int64_t)B * 2 * H, 2 * H, D,
                              dqw + so, (int64_t)B * H, H, D, 0));
         DS_PROPAGATE(gemm_bn(DS_MN_MAJOR, DS_MN_MAJOR, K, D, Q, dsm, K, (int64_t)N * Q * K, (int64_t)Q * K, sp + t.qw + so, (int64_t)B * H, H, D,
                              dkv, (int64_t)B * 2 * H, 2 * H, D, acc, dkv));
-        // position term through the shift: dbd[i][r] = dS[i][r - Q + i]
-        {
-          const int64_t wr_ = (int64_t)B * N * Q;
-          if (dtype == DS_BF16) hipLaunchKernelGGL(xl_unshift_kernel<bf16>, dim3(g1(wr_ * R)), dim3(256), 0, stream, wr_, Q, K, R, (const bf16*)dsm, (bf16*)dbd);
-          else hipLaunchKernelGGL(xl_unshift_kernel<float>, dim3(g1(wr_ * R)), dim3(256), 0, stream, wr_, Q, K, R, (const float*)dsm, (float*)dbd);
-          DS_CHECK_LAUNCH();
-        }
+        // position term through the shift
         DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_MN_MAJOR, Q, D, R, dbd, R, (int64_t)N * Q * R, (int64_t)Q * R, kr[l], H, 0, D,
                              dqr + so, (int64_t)B * H, H, D, 0));
         for (int bb = 0; bb < B; ++bb) {  // k_r is shared by the batch too: one launch per batch entry, added in place
@@ -478,12 +522,12 @@ struct XlnetStage : ds_stage {
           const int64_t waves = (int64_t)B * N * Q;
           dim3 grid((unsigned)((waves + 3) / 4));
           if (dtype == DS_BF16)
-            hipLaunchKernelGGL(xl_seg_bwd_kernel<bf16>, grid, dim3(256), 0, stream, Q, K, B, N, D, (int64_t)rows, (int64_t)s * rowsS,
-                               (const bf16*)dsm, seg, w[b + X_SEG], (const bf16*)(dqw + so), (const bf16*)(dqr + so), (bf16*)(dqs + so),
+            hipLaunchKernelGGL(xl_seg_bwd_kernel<bf16>, grid, dim3(256), 0, stream, Q, B, N, D, (int64_t)rows, (int64_t)s * rowsS,
+                               defs, w[b + X_SEG], (const bf16*)(dqw + so), (const bf16*)(dqr + so), (bf16*)(dqs + so),
                                (bf16*)(dq + so), (bf16*)deft);
           else
-            hipLaunchKernelGGL(xl_seg_bwd_kernel<float>, grid, dim3(256), 0, stream, Q, K, B, N, D, (int64_t)rows, (int64_t)s * rowsS,
-                               (const float*)dsm, seg, w[b + X_SEG], (const float*)(dqw + so), (const float*)(dqr + so), (float*)(dqs + so),
+            hipLaunchKernelGGL(xl_seg_bwd_kernel<float>, grid, dim3(256), 0, stream, Q, B, N, D, (int64_t)rows, (int64_t)s * rowsS,
+                               defs, w[b + X_SEG], (const float*)(dqw + so), (const float*)(dqr + so), (float*)(dqs + so),
                                (float*)(dq + so), (float*)deft);
           DS_CHECK_LAUNCH();
         }
