@@ -292,24 +292,30 @@ __global__ __launch_bounds__(256) void softmax_bwd_kernel(int64_t rows, int k, c
 
 // ------------------------------------------------------------------ column sums
 // Block = 4 row groups x 64 lanes; a lane owns one 16-byte vector of columns and strides down the
-// rows of its group; groups combine through LDS, then one atomicAdd per column.
+// rows of its group; groups combine through LDS, then one atomicAdd per column.  A matrix narrower than the 64
+// vectors of a wave is read `fold` rows at a time (contiguous rows form one super row of cols * fold elements), so
+// that all lanes have work; the fold copies of a column meet in the final atomic adds.
 template <typename T>
 __global__ __launch_bounds__(256) void colsum_kernel(int rows, int cols, const T* __restrict__ x, int64_t ldx,
-                                                    int rows_per_block, float* __restrict__ out) {
+                                                    int rows_per_block, int fold, float* __restrict__ out) {
   constexpr int VEC = Vec16<T>::N;
   typedef typename Vec16<T>::type V;
   __shared__ float red[4][64 * VEC];
   const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
-  const int c = (blockIdx.x * 64 + lane) * VEC;
+  const int c = (blockIdx.x * 64 + lane) * VEC;  // position inside the super row
+  const int sub = c / cols, cc = c - sub * cols;
   const int r0 = blockIdx.y * rows_per_block;
+  const int nsr = (rows + fold - 1) / fold;
   int r1 = r0 + rows_per_block;
-  if (r1 > rows) r1 = rows;
+  if (r1 > nsr) r1 = nsr;
   float s[VEC];
 #pragma unroll
   for (int e = 0; e < VEC; ++e) s[e] = 0.f;
-  if (c < cols)
+  if (sub < fold)
     for (int r = r0 + g; r < r1; r += 4) {
-      const V v = *reinterpret_cast<const V*>(x + (int64_t)r * ldx + c);
+      const int64_t row = (int64_t)r * fold + sub;
+      if (row >= rows) break;
+      const V v = *reinterpret_cast<const V*>(x + row * ldx + cc);
 #pragma unroll
       for (int e = 0; e < VEC; ++e) s[e] += to_f32(v[e]);
     }
@@ -317,8 +323,8 @@ __global__ __launch_bounds__(256) void colsum_kernel(int rows, int cols, const T
   for (int e = 0; e < VEC; ++e) red[g][lane * VEC + e] = s[e];
   __syncthreads();
   for (int i = threadIdx.x; i < 64 * VEC; i += 256) {
-    const int cc = blockIdx.x * 64 * VEC + i;
-    if (cc < cols) atomicAdd(out + cc, red[0][i] + red[1][i] + red[2][i] + red[3][i]);
+    const int p = blockIdx.x * 64 * VEC + i;
+    if (p < cols * fold) atomicAdd(out + p % cols, red[0][i] + red[1][i] + red[2][i] + red[3][i]);
   }
 }
 
@@ -488,14 +494,20 @@ extern "C" int ds_colsum_accum(int dtype, int rows, int cols, const void* x, int
   DS_CHECK_ARG(rows > 0 && cols > 0 && ldx >= cols && x && out, "ds_colsum_accum: bad argument");
   const int vec = dtype == DS_BF16 ? 8 : 4;
   DS_CHECK_ARG(cols % vec == 0 && ldx % vec == 0 && ds_aligned16(x), "ds_colsum_accum: cols and ldx must be multiples of %d and x 16-byte aligned", vec);
+  // every block ends in one atomic add per column: keep the number of row chunks in the low thousands
+  int fold = 1;
+  if (cols < 64 * vec && (64 * vec) % cols == 0 && ldx == cols) fold = 64 * vec / cols;
+  const int nsr = (rows + fold - 1) / fold;
   int rpb = 32;
-  dim3 grid((cols + 64 * vec - 1) / (64 * vec), (rows + rpb - 1) / rpb);
+  const int strips = (cols * fold + 64 * vec - 1) / (64 * vec);
+  while ((int64_t)strips * ((nsr + rpb - 1) / rpb) > 2048 && rpb < (1 << 20)) rpb *= 2;
+  dim3 grid(strips, (nsr + rpb - 1) / rpb);
   ds_prof_scope prof((hipStream_t)stream, dtype == DS_BF16 ? "colsum_kernel<bf16>" : "colsum_kernel<float>",
                      (double)rows * cols * (dtype == DS_BF16 ? 2 : 4), "B");
   if (dtype == DS_BF16)
-    hipLaunchKernelGGL(colsum_kernel<bf16>, grid, dim3(256), 0, (hipStream_t)stream, rows, cols, (const bf16*)x, ldx, rpb, out);
+    hipLaunchKernelGGL(colsum_kernel<bf16>, grid, dim3(256), 0, (hipStream_t)stream, rows, cols, (const bf16*)x, ldx, rpb, fold, out);
   else
-    hipLaunchKernelGGL(colsum_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, rows, cols, (const float*)x, ldx, rpb, out);
+    hipLaunchKernelGGL(colsum_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, rows, cols, (const float*)x, ldx, rpb, fold, out);
   DS_CHECK_LAUNCH();
   return DS_OK;
 }

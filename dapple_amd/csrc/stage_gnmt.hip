@@ -75,15 +75,16 @@ __global__ __launch_bounds__(256) void lstm_cell_fwd_kernel(int B, int U, float 
 }
 
 // Backward of one step: dh = dy[t] + dh_rec, dc = dc_rec + dh*o*(1 - tanh(c)^2); writes the four
-// pre-activation gate gradients and leaves dc*f in dc_rec for step t-1.
+// pre-activation gate gradients, leaves dc*f in dc_rec for step t-1 and zeroes `clear` [B,U].
 __global__ __launch_bounds__(256) void lstm_cell_bwd_kernel(int B, int U, const float* __restrict__ gact,
                                                            const float* __restrict__ c, const float* __restrict__ c_prev,
                                                            const float* __restrict__ dy, int lddy,
                                                            const float* __restrict__ dh_rec, float* __restrict__ dc_rec,
                                                            int first, float* __restrict__ dgates,
-                                                           const int32_t* __restrict__ len, int t) {
+                                                           const int32_t* __restrict__ len, int t, float* __restrict__ clear) {
   const int idx = blockIdx.x * 256 + threadIdx.x;
   if (idx >= B * U) return;
+  if (clear) clear[idx] = 0.f;  // the buffer the next recurrent product adds into
   const int b = idx / U, u = idx % U;
   if (len && t >= len[b]) {
     float* d = dgates + (int64_t)b * 4 * U;
@@ -328,11 +329,10 @@ struct GnmtStage : ds_stage {
           ds_prof_scope prof(stream, "lstm_cell_bwd_kernel", (double)B * U * 4 * (4 + 4 + 6), "B");
           hipLaunchKernelGGL(lstm_cell_bwd_kernel, dim3(cell_grid), dim3(256), 0, stream, B, U, G + (size_t)t * B * 4 * U,
                              Cs + (size_t)t * B * U, s > 0 ? Cs + (size_t)tp * B * U : nullptr, dY + (size_t)t * B * lddy, lddy,
-                             dh_in, dc, first, dG + (size_t)t * B * 4 * U, len, t);
+                             dh_in, dc, first, dG + (size_t)t * B * 4 * U, len, t, s > 0 ? dh_out : nullptr);
           DS_CHECK_LAUNCH();
         }
         if (s > 0) {  // dh for step tp: dgates[t] @ Wh^T
-          DS_CHECK_HIP(hipMemsetAsync(dh_out, 0, (size_t)B * U * 4, stream));
           DS_PROPAGATE(gemm_accum_splitk(DS_K_MAJOR, B, U, 4 * U, dG + (size_t)t * B * 4 * U, 4 * U, wh, 4 * U, dh_out, U,
                                          split_for(B, U, 4 * U)));
         }

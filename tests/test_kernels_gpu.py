@@ -191,6 +191,12 @@ def test_colsum(dt):
     out = torch.ones(200, device="cuda")
     ops.colsum_accum(x, out)
     assert_close(out, x.cpu().double().sum(0) + 1, 1e-5, "colsum")
+    # narrow matrices (several rows per wave-wide read), a row count that is not a multiple of that, many rows
+    for rows, cols in ((1003, 64), (7, 32), (200001, 64), (4099, 8), (33, 128)):
+        x = dev(rng(rows + cols).standard_normal((rows, cols)), DT[dt])
+        out = torch.ones(cols, device="cuda")
+        ops.colsum_accum(x, out)
+        assert_close(out, x.cpu().double().sum(0) + 1, 1e-4, "colsum %dx%d" % (rows, cols))
 
 
 @pytest.mark.parametrize("B,N,S,use_mask", [(1, 1, 64, False), (2, 3, 128, True), (2, 16, 512, True), (1, 2, 1024, False),
