@@ -5,8 +5,12 @@
 ``gemms``: the GEMMs of one BERT-48 half-stage layer at their real shapes (2x512 rows, hidden 1024,
 ffn 4096, bf16), three launches each in the order of the list in ``gemms``, so a counter run can report HBM traffic per launch.
 
+``elementwise``: the HBM-bound kernels of the path at the BERT-48 half-stage's shapes, five launches each with their
+algorithmic bytes printed, so a kernel trace gives achieved GB/s against the HBM peak.
+
     rocprofv3 --pmc FETCH_SIZE --output-format csv -d out -o c -- python3 -m dapple_amd.calib accumulate 67108864
     rocprofv3 --pmc FETCH_SIZE --output-format csv -d out -o g -- python3 -m dapple_amd.calib gemms
+    rocprofv3 --kernel-trace --stats -d out -o e -- python3 -m dapple_amd.calib elementwise
 """
 import sys
 
@@ -49,8 +53,37 @@ def gemms():
         print("%s: m=%d n=%d k=%d, algorithmic bytes %d" % (name, m, n, k, alg))
 
 
+def elementwise():
+    bf = torch.bfloat16
+    rows, h, f = 1024, 1024, 4096
+    r = torch.randn
+    x, dy = r(rows, h, device="cuda").to(bf), r(rows, h, device="cuda").to(bf)
+    g, b = torch.ones(h, device="cuda"), torch.zeros(h, device="cuda")
+    dg, db, dc = (torch.zeros(h, device="cuda") for _ in range(3))
+    big = r(4 * rows, f, device="cuda").to(bf)
+    out = torch.zeros(f, device="cuda")
+    n_acc = 12596224                     # parameters of one encoder layer
+    acc, grad = torch.zeros(n_acc, device="cuda"), torch.ones(n_acc, device="cuda")
+    src = r(h * f, device="cuda")
+    for _ in range(5):
+        y, st = ops.layernorm_fwd(x, g, b, 1e-12)
+        ops.layernorm_bwd(dy, x, g, st, dg, db, dc)
+        ops.colsum_accum(big, out)
+        ops.grad_accumulate(acc, grad)
+        ops.cast_to_bf16(src)
+    torch.cuda.synchronize()
+    e = 2
+    print("layernorm_fwd_kernel<bf16>  [%d,%d]: %d bytes per launch (read x, write y)" % (rows, h, 2 * rows * h * e))
+    print("layernorm_bwd_kernel<bf16>  [%d,%d]: %d bytes per launch (read dy, x, write dx)" % (rows, h, 3 * rows * h * e))
+    print("colsum_kernel<bf16>         [%d,%d]: %d bytes per launch (read x)" % (4 * rows, f, 4 * rows * f * e))
+    print("accumulate_kernel<float>    %d elements: %d bytes per launch (read acc, g, write acc)" % (n_acc, 12 * n_acc))
+    print("cast_kernel<bf16,float>     %d elements: %d bytes per launch (read fp32, write bf16)" % (h * f, 6 * h * f))
+
+
 if __name__ == "__main__":
     if len(sys.argv) > 1 and sys.argv[1] == "gemms":
         gemms()
+    elif len(sys.argv) > 1 and sys.argv[1] == "elementwise":
+        elementwise()
     else:
         accumulate(int(sys.argv[2]) if len(sys.argv) > 2 else 1 << 26)
