@@ -123,10 +123,13 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(int rows, int cols, 
   for (int i = 0; i < NV; ++i) {
     const int c = (lane + i * 64) * VEC;
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) {
-      g[i][e] = (c < cols) ? gamma[c + e] : 0.f;
-      pg[i][e] = pb[i][e] = ps[i][e] = 0.f;
+    for (int e = 0; e < VEC; e += 4) {  // whole 16-byte vectors: a predicate per element keeps the loads scalar
+      f32x4 gv = {0.f, 0.f, 0.f, 0.f};
+      if (c < cols) gv = *reinterpret_cast<const f32x4*>(gamma + c + e);
+      g[i][e] = gv[0]; g[i][e + 1] = gv[1]; g[i][e + 2] = gv[2]; g[i][e + 3] = gv[3];
     }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) pg[i][e] = pb[i][e] = ps[i][e] = 0.f;
   }
   const int row0 = (blockIdx.x * 4 + wave) * rows_per_wave;
   for (int r = 0; r < rows_per_wave; ++r) {
@@ -179,7 +182,8 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(int rows, int cols, 
     }
   }
   // combine the 4 waves' column partials in LDS, one wave at a time (plain vector stores / read-modify-writes:
-  // LDS float atomics on 32-byte-strided addresses serialise 16 ways)
+  // LDS float atomics on 32-byte-strided addresses serialise 16 ways; parking all four sets and summing them in
+  // one step needs 4x the LDS, which costs more in co-residency with other kernels than the barriers it saves)
   for (int wv = 0; wv < 4; ++wv) {
     if (wave == wv) {
 #pragma unroll
@@ -436,7 +440,7 @@ extern "C" int ds_layernorm_bwd(int dtype, int rows, int cols, const void* dy, c
                                 float* d_colsum, void* stream) {
   DS_PROPAGATE(check_rows("ds_layernorm_bwd", dtype, rows, cols));
   DS_CHECK_ARG(dy && x && gamma && stats && dx && d_gamma && d_beta, "ds_layernorm_bwd: null pointer");
-  DS_CHECK_ARG(ds_aligned16(dy) && ds_aligned16(x) && ds_aligned16(dx) && ds_aligned16(dx_add),
+  DS_CHECK_ARG(ds_aligned16(dy) && ds_aligned16(x) && ds_aligned16(dx) && ds_aligned16(dx_add) && ds_aligned16(gamma),
                "ds_layernorm_bwd: tensors must be 16-byte aligned");
   if (dtype == DS_BF16)
     return layernorm_bwd_t<bf16>(rows, cols, dy, x, gamma, stats, dx_add, dx, d_gamma, d_beta, d_colsum, (hipStream_t)stream);
