@@ -62,6 +62,14 @@ class GnmtCfg(C.Structure):
     ]
 
 
+XLNET_HEAD_TENSORS = ("start_w", "start_b", "end_w0", "end_b0", "ln_gamma", "ln_beta", "end_w1", "end_b1", "ans_w0", "ans_b0",
+                      "ans_w1")
+
+
+class XlnetHeadParams(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in XLNET_HEAD_TENSORS]
+
+
 class XlnetCfg(C.Structure):
     _fields_ = [
         ("dtype", C.c_int), ("num_layers", C.c_int), ("hidden", C.c_int), ("heads", C.c_int), ("ffn", C.c_int),
@@ -125,6 +133,9 @@ PROTOTYPES = {
     "ds_squad_head": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                 C.c_float, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "ds_classifier_head": (C.c_int, [C.c_int] * 5 + [C.c_void_p] * 6 + [C.c_float, C.c_float] + [C.c_void_p] * 11),
+    "ds_xlnet_squad_head_workspace_bytes": (C.c_size_t, [C.c_int] * 4),
+    "ds_xlnet_squad_head": (C.c_int, [C.c_int] * 4 + [C.c_void_p, C.POINTER(XlnetHeadParams)] + [C.c_void_p] * 6 + [C.c_float] +
+                            [C.c_void_p] * 5 + [C.POINTER(XlnetHeadParams), C.c_void_p, C.c_size_t, C.c_void_p]),
     "ds_grad_sqnorm_accum": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p]),
     "ds_optim_plan_create": (C.c_int, [C.c_int, C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_float),
                                         C.POINTER(C.c_void_p)]),

@@ -5,6 +5,7 @@ ctypes and launches on torch's current stream.  Nothing here computes on the
 host and nothing falls back to torch ops.
 """
 import ctypes as C
+import math
 
 import torch
 
@@ -259,3 +260,50 @@ def classifier_head(x, batch, seq, pooler_w, pooler_b, fc_w, fc_b, labels, grads
                                          ptr(dz), ptr(dx), ptr(grads[0]), ptr(grads[1]), ptr(grads[2]), ptr(grads[3]),
                                          _lib.current_stream()), "ds_classifier_head")
     return loss, logits, pooled, dx
+
+
+XLNET_HEAD_SHAPES = {"start_w": lambda h: (h,), "start_b": lambda h: (1,), "end_w0": lambda h: (2 * h, h), "end_b0": lambda h: (h,),
+                     "ln_gamma": lambda h: (h,), "ln_beta": lambda h: (h,), "end_w1": lambda h: (h,), "end_b1": lambda h: (1,),
+                     "ans_w0": lambda h: (2 * h, h), "ans_b0": lambda h: (h,), "ans_w1": lambda h: (h,)}
+
+
+def _xlnet_head_params(tensors, hidden, what):
+    out = _lib.XlnetHeadParams()
+    for name in _lib.XLNET_HEAD_TENSORS:
+        t = tensors[name]
+        if t.dtype != torch.float32 or not t.is_contiguous() or not t.is_cuda or t.numel() != math.prod(XLNET_HEAD_SHAPES[name](hidden)):
+            raise ValueError(f"xlnet_squad_head: {what}[{name!r}] must be a contiguous fp32 device tensor of shape "
+                             f"{XLNET_HEAD_SHAPES[name](hidden)}")
+        setattr(out, name, t.data_ptr())
+    return out
+
+
+def xlnet_squad_head(x, weights, cls_index, start_positions, end_positions, is_impossible, p_mask, dropout_mask=None, grads=None,
+                     need_dx=True, loss_scale=1.0):
+    """XLnetLoss.call (xlnet/losses/xlnet_loss.py:36-120) on the last stage's content stream ``x [seq, batch, hidden]``:
+    returns (loss [1] fp32 on the device, start_logits [batch, seq], end_logits [batch, seq], cls_logits [batch], dx or None).
+    ``weights`` / ``grads``: dicts of fp32 tensors keyed by XLNET_HEAD_SHAPES (Dense kernels with one output as vectors);
+    ``grads`` are added to in place.  ``dropout_mask [batch, hidden]`` is the factor of the dropout at :103 (None = ones)."""
+    _need_cuda(x, cls_index, start_positions, end_positions, is_impossible, p_mask)
+    if x.dim() != 3 or not x.is_contiguous():
+        raise ValueError("xlnet_squad_head: x must be contiguous [seq, batch, hidden]")
+    seq, batch, hidden = x.shape
+    for t in (cls_index, start_positions, end_positions):
+        if t.dtype != torch.int32 or t.numel() != batch:
+            raise ValueError("xlnet_squad_head: cls_index, start_positions, end_positions must be int32 [batch]")
+    for t, n in ((is_impossible, batch), (p_mask, batch * seq)) + (((dropout_mask, batch * hidden),) if dropout_mask is not None else ()):
+        if t.dtype != torch.float32 or not t.is_contiguous() or t.numel() != n:
+            raise ValueError("xlnet_squad_head: is_impossible [batch], p_mask [batch, seq], dropout_mask [batch, hidden] must be contiguous fp32")
+    wp = _xlnet_head_params(weights, hidden, "weights")
+    gp = _xlnet_head_params(grads, hidden, "grads") if grads is not None else None
+    lib = _lib.load()
+    f32 = dict(dtype=torch.float32, device=x.device)
+    nbytes = lib.ds_xlnet_squad_head_workspace_bytes(dtype_code(x), seq, batch, hidden)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    loss, sl, el, cl = torch.empty(1, **f32), torch.empty(batch, seq, **f32), torch.empty(batch, seq, **f32), torch.empty(batch, **f32)
+    dx = torch.empty_like(x) if need_dx else None
+    check(lib.ds_xlnet_squad_head(dtype_code(x), seq, batch, hidden, ptr(x), C.byref(wp), ptr(cls_index), ptr(start_positions),
+                                  ptr(end_positions), ptr(is_impossible), ptr(p_mask), ptr(dropout_mask), loss_scale, ptr(loss), ptr(sl),
+                                  ptr(el), ptr(cl), ptr(dx), C.byref(gp) if gp is not None else None, ptr(ws), nbytes,
+                                  _lib.current_stream()), "ds_xlnet_squad_head")
+    return loss, sl, el, cl, dx

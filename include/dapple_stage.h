@@ -321,6 +321,44 @@ int ds_classifier_head(int dtype, int batch, int seq, int hidden, int num_labels
                        float loss_scale, float* loss, float* pooled, float* logits, float* dlogits, float* dz, void* dx,
                        float* d_pooler_w, float* d_pooler_b, float* d_fc_w, float* d_fc_b, void* stream);
 
+/* SQuAD-2 head of the last XLNet stage: XLnetLoss.call, xlnet/losses/xlnet_loss.py:36-120 (called at
+ * xlnet/models/slice_xlnet.py:238-243 on the content stream).  One struct of device pointers names the eleven
+ * tensors of the layer; it is used twice, for the fp32 weights and for their master gradients.
+ *   start_w [hidden], start_b [1]                     self.dense      (:19)   start logits
+ *   end_w0 [2*hidden, hidden], end_b0 [hidden]        self.dense_0    (:20-23) rows [0, hidden) multiply the
+ *                                                     sequence output, rows [hidden, 2*hidden) the start feature
+ *   ln_gamma, ln_beta [hidden]                        self.layer_norm (:24; layers/layer_normalization.py, eps 1e-14)
+ *   end_w1 [hidden], end_b1 [1]                       self.dense_1    (:25)
+ *   ans_w0 [2*hidden, hidden], ans_b0 [hidden]        self.dense_0_1  (:26-29) rows [0, hidden) multiply the
+ *                                                     probability-weighted start feature, the rest the cls feature
+ *   ans_w1 [hidden]                                   self.dense_1_1  (:30-34, no bias) */
+typedef struct ds_xlnet_head_params {
+  float* start_w; float* start_b;
+  float* end_w0;  float* end_b0;
+  float* ln_gamma; float* ln_beta;
+  float* end_w1;  float* end_b1;
+  float* ans_w0;  float* ans_b0;
+  float* ans_w1;
+} ds_xlnet_head_params;
+/* Bytes of device workspace ds_xlnet_squad_head needs for this shape and element type. */
+size_t ds_xlnet_squad_head_workspace_bytes(int dtype, int seq, int batch, int hidden);
+/* loss = ((start_loss + end_loss) + regression_loss) / 2 (:88, :117-118) and its gradients.
+ *   x [seq, batch, hidden] (compute type, time-major like the stage's output); cls_index, start_positions,
+ *   end_positions int32 [batch] (an index outside [0, seq) is an all-zero one-hot row, like tf.one_hot);
+ *   is_impossible fp32 [batch]; p_mask fp32 [batch, seq];
+ *   dropout_mask fp32 [batch, hidden] or NULL: the factor keras.layers.Dropout(0.1)(., training=True) at :103
+ *   applies to each element (0 or 1/0.9 in the reference, drawn by TensorFlow's generator; NULL = all ones);
+ *   out: loss (device float, loss_scale * loss), start_logits, end_logits fp32 [batch, seq] (unmasked, :51-52 and
+ *   :72-73), cls_logits fp32 [batch];
+ *   dx (nullable): d loss / d x in the compute type - the d_out of the stage's backward pass;
+ *   grads (nullable): master gradients, added to (tf.accumulate_n over micro-batches).
+ * The arithmetic is fp32 whatever the compute type.  hidden must be a multiple of 8. */
+int ds_xlnet_squad_head(int dtype, int seq, int batch, int hidden, const void* x, const ds_xlnet_head_params* weights,
+                        const int32_t* cls_index, const int32_t* start_positions, const int32_t* end_positions,
+                        const float* is_impossible, const float* p_mask, const float* dropout_mask, float loss_scale,
+                        float* loss, float* start_logits, float* end_logits, float* cls_logits, void* dx,
+                        const ds_xlnet_head_params* grads, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- what the reference runs on the accumulated gradients right after the unroll block ----
  *
  * Global-norm clipping, bert/graph.py:162-165 (tf.clip_by_global_norm over all accumulated gradients):
