@@ -339,6 +339,37 @@ class XlnetSlice(object):
                                          K, mem_len=memory_len or 0, streams=streams, first_layer=layers[0])
         w = weights or synthetic.xlnet_weights(seed, len(layers), embedding_dim, num_head, feed_forward_dim, first_layer=layers[0])
         self.stage.bind(w)
+        self.is_last = local_device == xlnet_calc_device(num_layer + 2, num_layer)
+        if self.is_last:
+            # XLnetLoss (losses/xlnet_loss.py:9-34): Dense kernels drawn by keras 'normal' (stddev 0.05), biases 0, LN 1 / 0
+            from . import ops
+            g = torch.Generator().manual_seed(seed + 7)
+            H = embedding_dim
+            self.loss_weights = {}
+            for name, shape in ((n, f(H)) for n, f in ops.XLNET_HEAD_SHAPES.items()):
+                if name in ("start_b", "end_b0", "end_b1", "ans_b0", "ln_beta"):
+                    t = torch.zeros(shape)
+                elif name == "ln_gamma":
+                    t = torch.ones(shape)
+                else:
+                    t = torch.randn(shape, generator=g) * 0.05
+                self.loss_weights[name] = t.cuda()
+            self.loss_grads = {n: torch.zeros_like(t) for n, t in self.loss_weights.items()}
+
+    def xlnet_loss(self, cls_index, start_positions, end_positions, is_impossible, p_mask, output, dropout_mask=None):
+        """slice_xlnet.py:236-244 on the last device: XLnetLoss on the content stream ``output [seq, batch, hidden]``.
+        Sets ``loss`` / ``start_logits`` / ``end_logits`` / ``cls_logits`` and returns the gradient of the loss w.r.t.
+        ``output`` - the upstream gradient of this stage's backward pass; the head's weight gradients are added into
+        ``loss_grads``.  ``dropout_mask [batch, hidden]``: the factor of the dropout inside the loss (None = ones)."""
+        from . import ops
+        if not self.is_last:
+            raise ValueError("xlnet_loss: this device does not hold the loss layer")
+        i32 = lambda t: torch.as_tensor(t, dtype=torch.int32).cuda()
+        f32 = lambda t: None if t is None else torch.as_tensor(t, dtype=torch.float32).cuda().contiguous()
+        self.loss, self.start_logits, self.end_logits, self.cls_logits, dx = ops.xlnet_squad_head(
+            output, self.loss_weights, i32(cls_index), i32(start_positions), i32(end_positions), f32(is_impossible), f32(p_mask),
+            f32(dropout_mask), grads=self.loss_grads)
+        return dx
 
     def build(self, inputs, dep_outputs=None, is_training=True):
         """inputs: the boundary activation(s) [streams, seq, batch, hidden]; returns (None, [stage_output])."""

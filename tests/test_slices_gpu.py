@@ -88,6 +88,23 @@ def test_vgg_xlnet_gnmt_slices_build():
     assert x.layers == list(range(11))
     _, outs = x.build(torch.randn(1, 16, 2, 64, device="cuda"))
     assert outs[0].shape == (1, 16, 2, 64) and torch.isfinite(outs[0]).all()
+    assert not x.is_last
+    with pytest.raises(ValueError):
+        x.xlnet_loss([0, 0], [1, 2], [3, 4], [0.0, 1.0], torch.zeros(2, 16), outs[0][0])
+    x.stage.close()
+    # the last device: layers 11..23, then XLnetLoss on the content stream; its input gradient feeds the backward pass
+    x1 = slices.XlnetSlice(32000, 24, 4, 64, 16, 128, 16, False, memory_len=0, local_device=1, batch_size=2, dtype="fp32", stash_slots=1)
+    assert x1.layers == list(range(11, 24)) and x1.is_last
+    xin = torch.randn(1, 16, 2, 64, device="cuda")
+    y = torch.empty_like(xin)
+    x1.stage.forward(0, xin, y)
+    dy = x1.xlnet_loss([0, 15], [1, 2], [3, 4], [0.0, 1.0], torch.zeros(2, 16), y[0])
+    assert x1.loss.shape == (1,) and torch.isfinite(x1.loss).all() and x1.start_logits.shape == (2, 16) and x1.cls_logits.shape == (2,)
+    dxin = torch.empty_like(xin)
+    x1.stage.backward(0, dy.reshape(1, 16, 2, 64), dxin)
+    x1.stage.sync()
+    assert torch.isfinite(dxin).all() and float(dxin.abs().max()) > 0 and float(x1.loss_grads["end_w0"].abs().max()) > 0
+    x1.stage.close()
     hp = types.SimpleNamespace(unit_type="lstm", num_units=16, forget_bias=1.0, dropout=0.0, num_encoder_layers=3, src_vocab_size=40)
     g = slices.GNMTEncoderSlice(hp, batch_size=4, src_max_len=5)
     assert [c.residual_connection for c in g.cells] == [False, False, False, True]
