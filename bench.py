@@ -227,6 +227,9 @@ def main():
     ap.add_argument("--no-overlap", action="store_true", help="keep forward and backward passes on one stream")
     ap.add_argument("--wgrad-group", type=int, default=4,
                     help="BERT stages: weight gradients of this many backward passes in one GEMM per weight")
+    ap.add_argument("--micro-batch", type=int, default=None,
+                    help="samples per micro-batch instead of the configuration's (a what-if: the headline is the default)")
+    ap.add_argument("--micro-batches", type=int, default=None, help="micro-batches per step instead of the configuration's")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs one pipeline stage on ONE GPU; --gpus %d is not supported "
@@ -237,6 +240,11 @@ def main():
     from dapple_amd import _lib, synthetic
 
     c = dict(synthetic.CONFIGS[args.workload])
+    reshaped = False
+    for key, val in (("micro_batch", args.micro_batch), ("num_micro_batches", args.micro_batches)):
+        if val is not None and val != c[key]:
+            c[key] = val
+            reshaped = True
     dtype = c["dtype"]
     wl = MAKERS[c["kind"]](c, args)
     overlap = not args.no_overlap and wl.stage.overlap_supported()
@@ -295,7 +303,7 @@ def main():
     kernels = {t: {"launches": v[0], "ms": round(v[1], 3),
                    "rate": round(v[2] / (v[1] * 1e-3) / (1e12 if v[3] == "FLOP" else 1e9), 2),
                    "unit": "TFLOP/s" if v[3] == "FLOP" else "GB/s"} for t, v in sorted(prof.items(), key=lambda kv: -kv[1][1])}
-    cfg = {"workload": args.workload, "grad_accum": "fp32 in place", "flops_per_sample": wl.flops_per_sample}
+    cfg = {"workload": args.workload + (" (micro-batching changed on the command line)" if reshaped else ""), "grad_accum": "fp32 in place", "flops_per_sample": wl.flops_per_sample}
     cfg.update(wl.config)
     cfg["fwd_bwd_overlap"] = overlap
     line = {

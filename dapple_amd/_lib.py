@@ -58,7 +58,8 @@ class VggCfg(C.Structure):
 class GnmtCfg(C.Structure):
     _fields_ = [
         ("dtype", C.c_int), ("num_layers", C.c_int), ("units", C.c_int), ("vocab", C.c_int), ("batch", C.c_int),
-        ("seq", C.c_int), ("forget_bias", C.c_float), ("stash_slots", C.c_int), ("reserved", C.c_int * 8),
+        ("seq", C.c_int), ("forget_bias", C.c_float), ("stash_slots", C.c_int), ("decoder_part2", C.c_int), ("first_layer", C.c_int),
+        ("reserved", C.c_int * 6),
     ]
 
 
@@ -112,6 +113,7 @@ PROTOTYPES = {
     "ds_vgg_stage_create": (C.c_int, [C.POINTER(VggCfg), C.c_void_p, C.POINTER(C.c_void_p)]),
     "ds_gnmt_stage_create": (C.c_int, [C.POINTER(GnmtCfg), C.c_void_p, C.POINTER(C.c_void_p)]),
     "ds_gnmt_stage_set_lengths": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p]),
+    "ds_gnmt_stage_set_attention": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p]),
     "ds_xlnet_stage_create": (C.c_int, [C.POINTER(XlnetCfg), C.c_void_p, C.POINTER(C.c_void_p)]),
     "ds_xlnet_stage_set_inputs": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
     "ds_stage_create": (C.c_int, [C.POINTER(StageCfg), C.c_void_p, C.POINTER(C.c_void_p)]),
@@ -133,6 +135,8 @@ PROTOTYPES = {
     "ds_squad_head": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                 C.c_float, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "ds_classifier_head": (C.c_int, [C.c_int] * 5 + [C.c_void_p] * 6 + [C.c_float, C.c_float] + [C.c_void_p] * 11),
+    "ds_nmt_loss_head_workspace_bytes": (C.c_size_t, [C.c_int] * 3),
+    "ds_nmt_loss_head": (C.c_int, [C.c_int] * 4 + [C.c_void_p] * 4 + [C.c_int, C.c_float] + [C.c_void_p] * 4 + [C.c_size_t, C.c_void_p]),
     "ds_xlnet_squad_head_workspace_bytes": (C.c_size_t, [C.c_int] * 4),
     "ds_xlnet_squad_head": (C.c_int, [C.c_int] * 4 + [C.c_void_p, C.POINTER(XlnetHeadParams)] + [C.c_void_p] * 6 + [C.c_float] +
                             [C.c_void_p] * 5 + [C.POINTER(XlnetHeadParams), C.c_void_p, C.c_size_t, C.c_void_p]),

@@ -5,6 +5,7 @@
 //   zero), and its gradient: dX for the stage's backward pass, dW / db added into the master gradients.
 // Everything here is HBM-bound row work: X is read twice (logits, dW) and dX written once.
 #include <math.h>
+#include <string.h>
 
 #include "common.h"
 
@@ -273,6 +274,44 @@ int classifier_head_t(int B, int S, int H, int C, const void* x, const float* wp
 
 }  // namespace
 
+// ------------------------------------------------------------------ GNMT output projection + loss
+// gnmt/nmt/model.py:685-686 (logits = output_layer(rnn_output), a Dense without bias, :497-499) and _compute_loss
+// :824-838: crossent = sparse softmax cross entropy per (step, sample), weighted by sequence_mask(target length),
+// summed and divided by the batch size.  The two products with the [units, vocab] kernel are ds_gemm calls; this
+// kernel turns a row of logits into its loss term and, in place, into d loss / d logits.
+// One block per row r = t*B + b.  Rows past the target length get a zero gradient row and no loss term.
+__global__ __launch_bounds__(256) void nmt_xent_kernel(int B, int T, int V, float* __restrict__ logits, const int32_t* __restrict__ target,
+                                                       const int32_t* __restrict__ lengths, float wgt, float* __restrict__ loss) {
+  __shared__ float red[4];
+  const int r = blockIdx.x, t = r / B, b = r % B;
+  float* lg = logits + (int64_t)r * V;
+  if (t >= lengths[b]) {
+    for (int v = threadIdx.x; v < V; v += 256) lg[v] = 0.f;
+    return;
+  }
+  float mx = -INFINITY;
+  for (int v = threadIdx.x; v < V; v += 256) mx = fmaxf(mx, lg[v]);
+  mx = wave_max(mx);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
+  __syncthreads();
+  mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  __syncthreads();
+  float sum = 0.f;
+  for (int v = threadIdx.x; v < V; v += 256) sum += expf(lg[v] - mx);
+  sum = wave_sum(sum);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = sum;
+  __syncthreads();
+  sum = red[0] + red[1] + red[2] + red[3];
+  const float lse = mx + logf(sum);
+  const int label = target[(int64_t)b * T + t];
+  const bool valid = label >= 0 && label < V;
+  if (threadIdx.x == 0) atomicAdd(loss, valid ? wgt * (lse - lg[label]) : NAN);
+  __syncthreads();  // the label's logit is read before the row is overwritten
+  for (int v = threadIdx.x; v < V; v += 256) lg[v] = wgt * (expf(lg[v] - lse) - (v == label ? 1.f : 0.f));
+}
+
+__global__ void nmt_clear_kernel(float* loss) { *loss = 0.f; }
+
 extern "C" int ds_classifier_head(int dtype, int batch, int seq, int hidden, int num_labels, const void* x, const float* pooler_w,
                                   const float* pooler_b, const float* fc_w, const float* fc_b, const int32_t* labels, float l2_scale,
                                   float loss_scale, float* loss, float* pooled, float* logits, float* dlogits, float* dz, void* dx,
@@ -305,4 +344,49 @@ extern "C" int ds_squad_head(int dtype, int batch, int seq, int hidden, const vo
                               dbias, (hipStream_t)stream);
   return squad_head_t<float>(batch, seq, hidden, x, w, bias, start_positions, end_positions, loss_scale, loss, logits, dlogits, dx, dw,
                              dbias, (hipStream_t)stream);
+}
+
+extern "C" size_t ds_nmt_loss_head_workspace_bytes(int seq, int batch, int vocab) {
+  if (seq <= 0 || batch <= 0 || vocab <= 0) return 0;
+  return (size_t)seq * batch * vocab * sizeof(float);
+}
+
+extern "C" int ds_nmt_loss_head(int seq, int batch, int units, int vocab, const float* x, const float* proj_kernel,
+                                const int32_t* target_output, const int32_t* target_sequence_length, int loss_batch_size,
+                                float loss_scale, float* loss, float* dx, float* d_proj_kernel, void* workspace,
+                                size_t workspace_bytes, void* stream) {
+  DS_CHECK_ARG(seq > 0 && batch > 0 && units > 0 && vocab > 0, "ds_nmt_loss_head: non-positive shape");
+  DS_CHECK_ARG(units % 4 == 0 && vocab % 4 == 0, "ds_nmt_loss_head: units (%d) and vocab (%d) must be multiples of 4", units, vocab);
+  DS_CHECK_ARG(x && proj_kernel && target_output && target_sequence_length && loss && workspace, "ds_nmt_loss_head: null pointer");
+  DS_CHECK_ARG(workspace_bytes >= ds_nmt_loss_head_workspace_bytes(seq, batch, vocab), "ds_nmt_loss_head: workspace of %zu bytes, %zu needed",
+               workspace_bytes, ds_nmt_loss_head_workspace_bytes(seq, batch, vocab));
+  DS_CHECK_ARG(ds_aligned16(x) && ds_aligned16(proj_kernel) && ds_aligned16(workspace) && ds_aligned16(dx) && ds_aligned16(d_proj_kernel),
+               "ds_nmt_loss_head: tensors must be 16-byte aligned");
+  hipStream_t s = (hipStream_t)stream;
+  const int R = seq * batch;
+  float* logits = (float*)workspace;
+  ds_gemm_desc d;
+  memset(&d, 0, sizeof(d));
+  d.dtype = DS_F32; d.batch = 1; d.batch_inner = 1; d.alpha = 1.f;
+  d.a_major = DS_K_MAJOR; d.b_major = DS_MN_MAJOR; d.m = R; d.n = vocab; d.k = units; d.lda = units; d.ldb = vocab; d.ldc = vocab;
+  d.a = x; d.b = proj_kernel; d.c = logits;
+  DS_PROPAGATE(ds_gemm(&d, s));
+  hipLaunchKernelGGL(nmt_clear_kernel, dim3(1), dim3(1), 0, s, loss);
+  {
+    ds_prof_scope prof(s, "nmt_xent_kernel", (double)R * vocab * 4 * 4, "B");
+    hipLaunchKernelGGL(nmt_xent_kernel, dim3(R), dim3(256), 0, s, batch, seq, vocab, logits, target_output, target_sequence_length,
+                       loss_scale / (float)(loss_batch_size > 0 ? loss_batch_size : batch), loss);
+  }
+  DS_CHECK_LAUNCH();
+  if (dx) {  // d loss / d rnn_output = dlogits W^T
+    d.a_major = DS_K_MAJOR; d.b_major = DS_K_MAJOR; d.m = R; d.n = units; d.k = vocab; d.lda = vocab; d.ldb = vocab; d.ldc = units;
+    d.a = logits; d.b = proj_kernel; d.c = dx; d.flags = 0;
+    DS_PROPAGATE(ds_gemm(&d, s));
+  }
+  if (d_proj_kernel) {  // += rnn_output^T dlogits
+    d.a_major = DS_MN_MAJOR; d.b_major = DS_MN_MAJOR; d.m = units; d.n = vocab; d.k = R; d.lda = units; d.ldb = vocab; d.ldc = vocab;
+    d.a = x; d.b = logits; d.c = d_proj_kernel; d.flags = DS_EPI_ACCUM;
+    DS_PROPAGATE(ds_gemm(&d, s));
+  }
+  return DS_OK;
 }

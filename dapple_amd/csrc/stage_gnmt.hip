@@ -368,12 +368,212 @@ struct GnmtStage : ds_stage {
   }
 };
 
+// The decoder cells of the second pipeline device, GNMTAttentionMultiCell_2 (gnmt_model.py:489-537) under
+// dynamic_decode with a TrainingHelper (model.py:641-656): a scan over the padded target steps from the zero state.
+// Cell l reads concat([cur_inp, attention]) - kernel rows [0,U) for the running input, [U,2U) for the attention,
+// [2U,3U) for h - and, for l >= 2, adds the running input to its output (gnmt_residual_fn, :587-613).  The attention is
+// a per-slot side input without gradient (the reference reads it from a non-trainable variable); a slot without one
+// uses zeros and skips the products with the attention rows.
+struct DecCell {
+  int widx;
+  bool residual;
+  size_t g_off, c_off, h_off, y_off;
+};
+
+struct GnmtDecoderStage : ds_stage {
+  ds_gnmt_cfg gc;
+  int B, T, U, L, R;
+  std::vector<DecCell> cells;
+  char* stash_base = nullptr;
+  size_t slot_bytes = 0, x0_off = 0, att_off = 0;
+  std::vector<char> slot_has_att;
+  char* ws_base = nullptr;
+  size_t ws_bytes = 0, ws_dg, ws_dx[2], ws_dh[2], ws_dc;
+
+  ~GnmtDecoderStage() override {
+    if (stash_base) (void)hipFree(stash_base);
+    if (ws_base) (void)hipFree(ws_base);
+  }
+
+  int init() {
+    B = gc.batch; T = gc.seq; U = gc.units; L = gc.num_layers; R = B * T;
+    Arena sa;
+    x0_off = sa.reserve((size_t)R * U * 4);
+    att_off = sa.reserve((size_t)R * U * 4);
+    char name[160];
+    for (int i = 0; i < L; ++i) {
+      const int layer = gc.first_layer + i;
+      DecCell c;
+      memset(&c, 0, sizeof(c));
+      c.residual = layer >= 2;
+      c.widx = (int)winfo.size();
+      snprintf(name, sizeof(name), "dynamic_seq2seq/decoder/multi_rnn_cell_part2/cell_%d/basic_lstm_cell/kernel", layer);
+      winfo.push_back({name, 3 * U, 4 * U});
+      snprintf(name, sizeof(name), "dynamic_seq2seq/decoder/multi_rnn_cell_part2/cell_%d/basic_lstm_cell/bias", layer);
+      winfo.push_back({name, 1, 4 * U});
+      c.g_off = sa.reserve((size_t)R * 4 * U * 4);
+      c.c_off = sa.reserve((size_t)R * U * 4);
+      c.h_off = sa.reserve((size_t)R * U * 4);
+      if (c.residual && i + 1 < L) c.y_off = sa.reserve((size_t)R * U * 4);
+      cells.push_back(c);
+    }
+    slot_bytes = sa.used;
+    DS_CHECK_HIP(hipMalloc((void**)&stash_base, slot_bytes * gc.stash_slots));
+    slot_forwarded.assign(gc.stash_slots, 0);
+    slot_has_att.assign(gc.stash_slots, 0);
+    Arena wa;
+    ws_dg = wa.reserve((size_t)R * 4 * U * 4);
+    ws_dx[0] = wa.reserve((size_t)R * U * 4);
+    ws_dx[1] = wa.reserve((size_t)R * U * 4);
+    ws_dh[0] = wa.reserve((size_t)B * U * 4);
+    ws_dh[1] = wa.reserve((size_t)B * U * 4);
+    ws_dc = wa.reserve((size_t)B * U * 4);
+    ws_bytes = wa.used;
+    DS_CHECK_HIP(hipMalloc((void**)&ws_base, ws_bytes));
+    return DS_OK;
+  }
+
+  size_t workspace_bytes() const override { return ws_bytes; }
+  bool overlap_safe() const override { return true; }  // forward touches its stash slot and its output only
+  size_t stash_bytes(int slots) const override { return slot_bytes * (size_t)slots; }
+  int refresh_weights() override { return DS_OK; }
+
+  int gemm(int am, int bm, int m, int n, int k, const void* a, int64_t lda, const void* b, int64_t ldb, void* c, int64_t ldc,
+           int flags, const float* bias, const void* residual) {
+    ds_gemm_desc d;
+    memset(&d, 0, sizeof(d));
+    d.dtype = DS_F32; d.a_major = am; d.b_major = bm; d.m = m; d.n = n; d.k = k; d.lda = lda; d.ldb = ldb; d.ldc = ldc;
+    d.batch = 1; d.batch_inner = 1; d.flags = flags; d.alpha = 1.f; d.a = a; d.b = b; d.c = c; d.bias = bias; d.residual = residual;
+    return ds_gemm(&d, stream);
+  }
+  int gemm_accum_splitk(int bm, int m, int n, int k, const void* a, int64_t lda, const void* b, int64_t ldb, float* c, int64_t ldc) {
+    ds_gemm_desc d;
+    memset(&d, 0, sizeof(d));
+    d.dtype = DS_F32; d.a_major = DS_K_MAJOR; d.b_major = bm; d.m = m; d.n = n; d.k = k; d.lda = lda; d.ldb = ldb; d.ldc = ldc;
+    d.batch = 1; d.batch_inner = 1; d.flags = DS_EPI_ACCUM; d.alpha = 1.f; d.a = a; d.b = b; d.c = c;
+    return ds_gemm_splitk(&d, GnmtStage::split_for(m, n, k), stream);
+  }
+
+  int set_attention(int slot, const float* attention) {
+    if (attention)
+      DS_CHECK_HIP(hipMemcpyAsync(stash_base + (size_t)slot * slot_bytes + att_off, attention, (size_t)R * U * 4, hipMemcpyDeviceToDevice,
+                                  stream));
+    slot_has_att[slot] = attention != nullptr;
+    return DS_OK;
+  }
+
+  int forward(int slot, const void* in, const float*, void* out) override {
+    ds_prio_scope prio(1);
+    char* sp = stash_base + (size_t)slot * slot_bytes;
+    const float* att = slot_has_att[slot] ? (const float*)(sp + att_off) : nullptr;
+    DS_CHECK_HIP(hipMemcpyAsync(sp + x0_off, in, (size_t)R * U * 4, hipMemcpyDeviceToDevice, stream));
+    const int cell_grid = (B * U + 255) / 256;
+    const float* X = (const float*)(sp + x0_off);
+    for (size_t ci = 0; ci < cells.size(); ++ci) {
+      const DecCell& c = cells[ci];
+      const float* kernel = w[c.widx];
+      const float* wa = kernel + (size_t)U * 4 * U;
+      const float* wh = kernel + (size_t)2 * U * 4 * U;
+      float* G = (float*)(sp + c.g_off);
+      float* Cs = (float*)(sp + c.c_off);
+      float* H = (float*)(sp + c.h_off);
+      const bool last = ci + 1 == cells.size();
+      float* Y = c.residual ? (last ? (float*)out : (float*)(sp + c.y_off)) : nullptr;
+      // input part of the gates for every step: x Wx + bias (+ attention Wa)
+      DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, R, 4 * U, U, X, U, kernel, 4 * U, G, 4 * U, DS_EPI_BIAS, w[c.widx + 1], nullptr));
+      if (att) DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, R, 4 * U, U, att, U, wa, 4 * U, G, 4 * U, DS_EPI_ACCUM, nullptr, nullptr));
+      for (int t = 0; t < T; ++t) {
+        float* g = G + (size_t)t * B * 4 * U;
+        if (t > 0) DS_PROPAGATE(gemm_accum_splitk(DS_MN_MAJOR, B, 4 * U, U, H + (size_t)(t - 1) * B * U, U, wh, 4 * U, g, 4 * U));
+        ds_prof_scope prof(stream, "lstm_cell_fwd_kernel", (double)B * U * 4 * (4 + 4 + 2 + (c.residual ? 2 : 1)), "B");
+        hipLaunchKernelGGL(lstm_cell_fwd_kernel, dim3(cell_grid), dim3(256), 0, stream, B, U, gc.forget_bias, g,
+                           t > 0 ? Cs + (size_t)(t - 1) * B * U : nullptr, Cs + (size_t)t * B * U, H + (size_t)t * B * U, U,
+                           c.residual ? X + (size_t)t * B * U : nullptr, U, Y ? Y + (size_t)t * B * U : nullptr, U,
+                           (const int32_t*)nullptr, t);
+        DS_CHECK_LAUNCH();
+      }
+      if (last && !c.residual) DS_CHECK_HIP(hipMemcpyAsync(out, H, (size_t)R * U * 4, hipMemcpyDeviceToDevice, stream));
+      X = c.residual ? Y : H;
+    }
+    return DS_OK;
+  }
+
+  int backward(int slot, const void* d_out, void* d_in) override {
+    ds_prio_scope prio(3);
+    char* sp = stash_base + (size_t)slot * slot_bytes;
+    const float* att = slot_has_att[slot] ? (const float*)(sp + att_off) : nullptr;
+    float* dG = (float*)(ws_base + ws_dg);
+    float* dc = (float*)(ws_base + ws_dc);
+    const int cell_grid = (B * U + 255) / 256;
+    const float* dY = (const float*)d_out;
+    int pp = 0;
+    for (int ci = (int)cells.size() - 1; ci >= 0; --ci) {
+      const DecCell& c = cells[ci];
+      const float* kernel = w[c.widx];
+      const float* wh = kernel + (size_t)2 * U * 4 * U;
+      const float* G = (const float*)(sp + c.g_off);
+      const float* Cs = (const float*)(sp + c.c_off);
+      const float* H = (const float*)(sp + c.h_off);
+      const float* X = (const float*)(sp + x0_off);
+      if (ci > 0) X = (const float*)(sp + (cells[ci - 1].residual ? cells[ci - 1].y_off : cells[ci - 1].h_off));
+      for (int t = T - 1; t >= 0; --t) {
+        const int first = (t == T - 1);
+        float* dh_in = (float*)(ws_base + ws_dh[t & 1]);
+        float* dh_out = (float*)(ws_base + ws_dh[(t & 1) ^ 1]);
+        {
+          ds_prof_scope prof(stream, "lstm_cell_bwd_kernel", (double)B * U * 4 * (4 + 4 + 6), "B");
+          hipLaunchKernelGGL(lstm_cell_bwd_kernel, dim3(cell_grid), dim3(256), 0, stream, B, U, G + (size_t)t * B * 4 * U,
+                             Cs + (size_t)t * B * U, t > 0 ? Cs + (size_t)(t - 1) * B * U : nullptr, dY + (size_t)t * B * U, U, dh_in, dc,
+                             first, dG + (size_t)t * B * 4 * U, (const int32_t*)nullptr, t, t > 0 ? dh_out : nullptr);
+          DS_CHECK_LAUNCH();
+        }
+        if (t > 0) DS_PROPAGATE(gemm_accum_splitk(DS_K_MAJOR, B, U, 4 * U, dG + (size_t)t * B * 4 * U, 4 * U, wh, 4 * U, dh_out, U));
+      }
+      float* gk = g[c.widx];
+      DS_PROPAGATE(ds_colsum_accum(DS_F32, R, 4 * U, dG, 4 * U, g[c.widx + 1], stream));
+      DS_PROPAGATE(gemm(DS_MN_MAJOR, DS_MN_MAJOR, U, 4 * U, R, X, U, dG, 4 * U, gk, 4 * U, DS_EPI_ACCUM, nullptr, nullptr));
+      if (att)
+        DS_PROPAGATE(gemm(DS_MN_MAJOR, DS_MN_MAJOR, U, 4 * U, R, att, U, dG, 4 * U, gk + (size_t)U * 4 * U, 4 * U, DS_EPI_ACCUM, nullptr, nullptr));
+      if (T > 1)
+        DS_PROPAGATE(gemm(DS_MN_MAJOR, DS_MN_MAJOR, U, 4 * U, (T - 1) * B, H, U, dG + (size_t)B * 4 * U, 4 * U, gk + (size_t)2 * U * 4 * U,
+                          4 * U, DS_EPI_ACCUM, nullptr, nullptr));
+      // gradient of the running input: dG Wx^T (+ dY through the residual connection); none flows into the attention
+      float* dX = ci > 0 ? (float*)(ws_base + ws_dx[pp]) : (float*)d_in;
+      if (dX)
+        DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, R, U, 4 * U, dG, 4 * U, kernel, 4 * U, dX, U, c.residual ? DS_EPI_RESIDUAL : 0, nullptr,
+                          c.residual ? dY : nullptr));
+      dY = dX;
+      pp ^= 1;
+    }
+    return DS_OK;
+  }
+};
+
 }  // namespace
 
 extern "C" int ds_gnmt_stage_create(const ds_gnmt_cfg* c, void* stream, ds_stage** out) {
   DS_CHECK_ARG(c != nullptr && out != nullptr, "ds_gnmt_stage_create: null argument");
   *out = nullptr;
   DS_CHECK_ARG(c->dtype == DS_F32, "ds_gnmt_stage_create: only fp32 is built (dtype %d)", c->dtype);
+  if (c->decoder_part2) {
+    DS_CHECK_ARG(c->num_layers >= 1 && c->first_layer >= 1, "ds_gnmt_stage_create: decoder part 2 holds cells first_layer >= 1 .. (got %d layers from %d)",
+                 c->num_layers, c->first_layer);
+    DS_CHECK_ARG(c->units > 0 && c->units % 4 == 0, "ds_gnmt_stage_create: num_units (%d) must be a positive multiple of 4", c->units);
+    DS_CHECK_ARG(c->batch > 0 && c->seq > 0 && c->batch % 4 == 0, "ds_gnmt_stage_create: batch (%d) must be a positive multiple of 4, seq (%d) positive",
+                 c->batch, c->seq);
+    DS_CHECK_ARG(c->stash_slots >= 1, "ds_gnmt_stage_create: stash_slots must be >= 1");
+    GnmtDecoderStage* s = new GnmtDecoderStage();
+    memset(&s->cfg, 0, sizeof(s->cfg));
+    s->cfg.kind = DS_STAGE_GNMT;
+    s->cfg.dtype = c->dtype;
+    s->cfg.stash_slots = c->stash_slots;
+    s->gc = *c;
+    s->stream = (hipStream_t)stream;
+    const int rc = s->init();
+    if (rc != DS_OK) { delete s; return rc; }
+    *out = s;
+    return DS_OK;
+  }
   DS_CHECK_ARG(c->num_layers >= 2, "ds_gnmt_stage_create: the GNMT encoder has a bidirectional layer and at least one uni-directional layer");
   DS_CHECK_ARG(c->units > 0 && c->units % 4 == 0, "ds_gnmt_stage_create: num_units (%d) must be a positive multiple of 4", c->units);
   DS_CHECK_ARG(c->batch > 0 && c->seq > 0 && c->vocab > 0, "ds_gnmt_stage_create: non-positive shape");
@@ -396,6 +596,17 @@ extern "C" int ds_gnmt_stage_set_lengths(ds_stage* h, int slot, const int32_t* l
   DS_CHECK_ARG(h != nullptr, "ds_gnmt_stage_set_lengths: null handle");
   DS_CHECK_ARG(h->cfg.kind == DS_STAGE_GNMT, "ds_gnmt_stage_set_lengths: not a GNMT stage");
   DS_CHECK_ARG(slot >= 0 && slot < h->cfg.stash_slots, "ds_gnmt_stage_set_lengths: slot %d out of range", slot);
+  GnmtStage* enc = dynamic_cast<GnmtStage*>(h);
+  DS_CHECK_ARG(enc != nullptr, "ds_gnmt_stage_set_lengths: the decoder cells run every padded step (dynamic_decode without impute_finished)");
   DS_PROPAGATE(ds_stage_acquire_slot(h, slot));
-  return static_cast<GnmtStage*>(h)->set_lengths(slot, lengths);
+  return enc->set_lengths(slot, lengths);
+}
+
+extern "C" int ds_gnmt_stage_set_attention(ds_stage* h, int slot, const float* attention) {
+  DS_CHECK_ARG(h != nullptr, "ds_gnmt_stage_set_attention: null handle");
+  GnmtDecoderStage* dec = h->cfg.kind == DS_STAGE_GNMT ? dynamic_cast<GnmtDecoderStage*>(h) : nullptr;
+  DS_CHECK_ARG(dec != nullptr, "ds_gnmt_stage_set_attention: not a GNMT decoder stage");
+  DS_CHECK_ARG(slot >= 0 && slot < h->cfg.stash_slots, "ds_gnmt_stage_set_attention: slot %d out of range", slot);
+  DS_PROPAGATE(ds_stage_acquire_slot(h, slot));
+  return dec->set_attention(slot, attention);
 }

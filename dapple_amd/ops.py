@@ -307,3 +307,32 @@ def xlnet_squad_head(x, weights, cls_index, start_positions, end_positions, is_i
                                   ptr(el), ptr(cl), ptr(dx), C.byref(gp) if gp is not None else None, ptr(ws), nbytes,
                                   _lib.current_stream()), "ds_xlnet_squad_head")
     return loss, sl, el, cl, dx
+
+
+def nmt_loss_head(x, proj_kernel, target_output, target_sequence_length, d_proj_kernel=None, need_dx=True, loss_batch_size=0,
+                  loss_scale=1.0):
+    """GNMT output projection + loss (gnmt/nmt/model.py:685-686, :824-838) on the last decoder cell's outputs
+    ``x [seq, batch, units]`` fp32: returns (loss [1] on the device, dx or None); ``d_proj_kernel`` is added to in place."""
+    _need_cuda(x, proj_kernel, target_output, target_sequence_length)
+    if x.dim() != 3 or x.dtype != torch.float32 or not x.is_contiguous():
+        raise ValueError("nmt_loss_head: x must be contiguous fp32 [seq, batch, units]")
+    seq, batch, units = x.shape
+    if proj_kernel.dtype != torch.float32 or not proj_kernel.is_contiguous() or proj_kernel.dim() != 2 or proj_kernel.shape[0] != units:
+        raise ValueError("nmt_loss_head: proj_kernel must be contiguous fp32 [units, vocab]")
+    vocab = proj_kernel.shape[1]
+    if target_output.dtype != torch.int32 or tuple(target_output.shape) != (batch, seq) or not target_output.is_contiguous():
+        raise ValueError("nmt_loss_head: target_output must be contiguous int32 [batch, seq]")
+    if target_sequence_length.dtype != torch.int32 or target_sequence_length.numel() != batch:
+        raise ValueError("nmt_loss_head: target_sequence_length must be int32 [batch]")
+    if d_proj_kernel is not None and (d_proj_kernel.dtype != torch.float32 or not d_proj_kernel.is_contiguous()
+                                      or d_proj_kernel.shape != proj_kernel.shape):
+        raise ValueError("nmt_loss_head: d_proj_kernel must match proj_kernel")
+    lib = _lib.load()
+    nbytes = lib.ds_nmt_loss_head_workspace_bytes(seq, batch, vocab)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    loss = torch.empty(1, dtype=torch.float32, device=x.device)
+    dx = torch.empty_like(x) if need_dx else None
+    check(lib.ds_nmt_loss_head(seq, batch, units, vocab, ptr(x), ptr(proj_kernel), ptr(target_output), ptr(target_sequence_length),
+                               loss_batch_size, loss_scale, ptr(loss), ptr(dx), ptr(d_proj_kernel), ptr(ws), nbytes,
+                               _lib.current_stream()), "ds_nmt_loss_head")
+    return loss, dx

@@ -245,7 +245,32 @@ def gnmt_stage(num_layers, units, vocab, batch, seq, stash_slots, forget_bias=1.
     return st
 
 
+def gnmt_decoder_stage(num_layers, units, batch, seq, stash_slots, first_layer=1, forget_bias=1.0, dtype="fp32", device="cuda:0"):
+    """Decoder cells ``first_layer .. first_layer + num_layers - 1`` as the reference's second device runs them
+    (GNMTAttentionMultiCell_2, gnmt/nmt/gnmt_model.py:489-537; model.py:641-656): [seq, batch, units] -> [seq, batch, units]."""
+    lib = _lib.load()
+    cfg = GnmtCfg()
+    cfg.dtype, cfg.num_layers, cfg.units, cfg.vocab = _dtype_code(dtype), num_layers, units, 0
+    cfg.batch, cfg.seq, cfg.forget_bias, cfg.stash_slots = batch, seq, forget_bias, stash_slots
+    cfg.decoder_part2, cfg.first_layer = 1, first_layer
+    h = C.c_void_p()
+    with torch.cuda.device(torch.device(device)):
+        check(lib.ds_gnmt_stage_create(C.byref(cfg), _lib.current_stream(), C.byref(h)), "ds_gnmt_stage_create")
+    n = seq * batch * units
+    st = GnmtStage(h, _TORCH_DTYPE[cfg.dtype], n, n, stash_slots, device=device, cfg=cfg)
+    st.out_shape = (seq, batch, units)
+    return st
+
+
 class GnmtStage(Stage):
+    def set_attention(self, slot, attention=None):
+        """Decoder stage: the attention vectors [seq, batch, units] fp32 every cell of the micro-batch about to be
+        forwarded into ``slot`` concatenates to its input (None: zeros).  No gradient flows into them."""
+        if attention is not None and (attention.dtype != torch.float32 or not attention.is_cuda or not attention.is_contiguous()
+                                      or attention.numel() != self.out_numel):
+            raise ValueError("attention must be a contiguous fp32 GPU tensor of [seq, batch, units]")
+        check(self.lib.ds_gnmt_stage_set_attention(self._h, slot, ptr(attention)), "ds_gnmt_stage_set_attention")
+
     def set_lengths(self, slot, lengths=None):
         """``source_sequence_length`` [batch] int32 of the micro-batch about to be forwarded into ``slot``
         (None: full length)."""

@@ -251,3 +251,15 @@ CONFIGS = {
     "xlnet36_half": dict(index=4, kind="xlnet", num_layers=18, hidden=1024, heads=16, ffn=4096, seq=512, mem_len=384,
                          micro_batch=1, num_micro_batches=8, dtype="bf16", streams=2),
 }
+
+
+def gnmt_decoder_weights(seed, first_layer, num_layers, units, init_weight=0.1, perturb=False):
+    """Decoder cells first_layer .. of the second device: kernels [3*units, 4*units] (input | attention | h), biases 0."""
+    rng = _rng(seed)
+    w = {}
+    for l in range(first_layer, first_layer + num_layers):
+        scope = "dynamic_seq2seq/decoder/multi_rnn_cell_part2/cell_%d/basic_lstm_cell" % l
+        w[scope + "/kernel"] = rng.uniform(-init_weight, init_weight, (3 * units, 4 * units)).astype(np.float32)
+        w[scope + "/bias"] = rng.uniform(-init_weight, init_weight, 4 * units).astype(np.float32) if perturb \
+            else np.zeros(4 * units, np.float32)
+    return w

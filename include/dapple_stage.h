@@ -261,7 +261,9 @@ typedef struct ds_gnmt_cfg {
   int units, vocab, batch, seq;
   float forget_bias; /* 1.0 in gnmt/nmt/standard_hparams/wmt16_gnmt_8_layer.json */
   int stash_slots;
-  int reserved[8];
+  int decoder_part2; /* 0: the encoder stage above; 1: the decoder cells of the second device (below) */
+  int first_layer;   /* decoder_part2: index of the first decoder cell held (1 in the reference, gnmt_model.py:346-364) */
+  int reserved[6];
 } ds_gnmt_cfg;
 int ds_gnmt_stage_create(const ds_gnmt_cfg* cfg, void* stream, ds_stage** out);
 /* iterator.source_sequence_length (gnmt_model.py:103, 223-227) of the micro-batch that will be forwarded
@@ -269,6 +271,16 @@ int ds_gnmt_stage_create(const ds_gnmt_cfg* cfg, void* stream, ds_stage** out);
  * gets it: steps t >= lengths[b] emit zeros (residual layers too) and keep the state, the backward
  * direction of the first layer starts at step lengths[b] - 1.  The setting stays with the slot. */
 int ds_gnmt_stage_set_lengths(ds_stage* h, int slot, const int32_t* lengths);
+/* decoder_part2 = 1: decoder cells first_layer .. first_layer + num_layers - 1 as the reference's second device runs
+ * them - GNMTAttentionMultiCell_2, gnmt/nmt/gnmt_model.py:489-537, under dynamic_decode with a TrainingHelper on the
+ * outputs of cell 0 (gnmt/nmt/model.py:641-656): a scan over all `seq` padded target steps from the zero state
+ * (:375).  in / out / d_out / d_in are fp32 [seq, batch, units]; vocab is unused.  Cell l has one kernel
+ * [3*units, 4*units] (rows: running input | attention | h; gate order i, j, f, o) and a bias [4*units], and for
+ * l >= 2 adds the running input to its output (gnmt_residual_fn :587-613).
+ * The attention every cell concatenates to its input (:518, :526) comes from a non-trainable variable in the
+ * reference (:456-459), i.e. it is a constant of the graph: here it is a per-slot side input [seq, batch, units]
+ * on the device that receives no gradient; NULL (the default) stands for zeros, the variable's initial value. */
+int ds_gnmt_stage_set_attention(ds_stage* h, int slot, const float* attention);
 
 /* XLNet stage (xlnet/models/slice_xlnet.py:164-180 layer body; xlnet/layers/rel_multihead_attn.py:71-149).
  * Activations are sequence-major like the reference: in/out are [streams][seq][batch][hidden] (stream 0 =
@@ -320,6 +332,22 @@ int ds_classifier_head(int dtype, int batch, int seq, int hidden, int num_labels
                        const float* pooler_b, const float* fc_w, const float* fc_b, const int32_t* labels, float l2_scale,
                        float loss_scale, float* loss, float* pooled, float* logits, float* dlogits, float* dz, void* dx,
                        float* d_pooler_w, float* d_pooler_b, float* d_fc_w, float* d_fc_b, void* stream);
+
+/* Output projection and loss of the GNMT model on the last device: gnmt/nmt/model.py:685-686 (logits =
+ * output_layer(rnn_output); output_layer is a Dense without bias, :497-499) and _compute_loss :824-838
+ * (loss = sum(sparse_softmax_cross_entropy(target_output, logits) * sequence_mask(target_sequence_length)) / batch_size).
+ *   x fp32 [seq, batch, units]: the outputs of the last decoder cell; proj_kernel fp32 [units, vocab];
+ *   target_output int32 [batch, seq] (the reference transposes it, :827-828), target_sequence_length int32 [batch];
+ *   loss_batch_size: the divisor (hparams batch_size; 0 = batch);
+ *   loss: device float, overwritten with loss_scale * loss; dx (nullable) fp32 [seq, batch, units]: the d_out of the
+ *   decoder stage's backward pass; d_proj_kernel (nullable): master gradient, added to.
+ * workspace holds the [seq*batch, vocab] logits (turned into their gradient in place).  A label outside [0, vocab)
+ * gives a NaN loss, as TensorFlow's GPU kernel does.  units and vocab must be multiples of 4. */
+size_t ds_nmt_loss_head_workspace_bytes(int seq, int batch, int vocab);
+int ds_nmt_loss_head(int seq, int batch, int units, int vocab, const float* x, const float* proj_kernel,
+                     const int32_t* target_output, const int32_t* target_sequence_length, int loss_batch_size,
+                     float loss_scale, float* loss, float* dx, float* d_proj_kernel, void* workspace,
+                     size_t workspace_bytes, void* stream);
 
 /* SQuAD-2 head of the last XLNet stage: XLnetLoss.call, xlnet/losses/xlnet_loss.py:36-120 (called at
  * xlnet/models/slice_xlnet.py:238-243 on the content stream).  One struct of device pointers names the eleven

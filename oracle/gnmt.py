@@ -19,6 +19,11 @@ blocks (torch order i, f, g, o) and folding forget_bias into the bias; the kerne
 [in+U, 4U] vs the shape held by gnmt/nmt/model_test.py:86 ((10, 20) for in = U = 5); the
 scan vs an explicit Python loop; the bidirectional layer vs torch.nn.LSTM(bidirectional=True); ragged sequences vs torch.nn.LSTM on a
 packed sequence (pack_padded_sequence / pad_packed_sequence), both directions.
+
+decoder_part2_forward / nmt_loss restate the second device's share of the decoder (gnmt_model.py:489-537,
+model.py:641-686) and the loss (model.py:791-838).  Pins: a two-cell stack vs torch.nn.LSTMCell fed the concatenated
+input, with the residual taken from the first half of the input; no gradient reaches the attention input; the loss vs
+torch.nn.functional.cross_entropy(reduction="sum") over the unpadded positions divided by the batch size.
 """
 import torch
 
@@ -85,3 +90,52 @@ def stage_vjp(ids, w, d_out, num_layers, forget_bias=1.0, lengths=None):
     out = encoder_forward(ids, w, num_layers, forget_bias, lengths)
     grads = torch.autograd.grad(out, [w[n] for n in names], grad_outputs=d_out, allow_unused=True)
     return out.detach(), None, {n: g for n, g in zip(names, grads) if g is not None}
+
+
+# ---- the decoder layers of the second pipeline device and the loss ----
+# gnmt_model.py:342-383 (DAPPLE branch): decoder cell 0 with the attention wrapper stays on the encoder device
+# (GNMTAttentionMultiCell_1), cells 1.. go to the second device as GNMTAttentionMultiCell_2 (:489-537); cell l has a
+# residual wrapper with gnmt_residual_fn for l >= 2 (:346-364).  model.py:641-656 drives part 2 with
+# dynamic_decode(BasicDecoder(cell2, TrainingHelper(outputs_1, target_sequence_length), zero state)): without
+# impute_finished every step up to the longest target is a plain cell call on the padded input, so it is a scan.
+# Each cell reads concat([cur_inp, new_attention]) (:526); new_attention is global_attention[0], a non-trainable
+# tf.Variable (:456-459): a constant of the graph - no gradient flows into it - that holds whatever was last assigned
+# (its initial value is zero; the assign at :478-479 is fetched by nothing).  Here it is an input, one vector per step.
+DP = "dynamic_seq2seq/decoder/multi_rnn_cell_part2/"
+PROJ = "build_network/decoder/output_projection/output_projection/kernel"
+
+
+def decoder_cell_names(first_layer, num_layers):
+    """[(scope, residual)] of decoder cells first_layer .. first_layer + num_layers - 1 (variable scope "cell_%d", :521)."""
+    return [(DP + "cell_%d/basic_lstm_cell" % l, l >= 2) for l in range(first_layer, first_layer + num_layers)]
+
+
+def decoder_part2_forward(x, attention, w, first_layer, num_layers, forget_bias=1.0):
+    """x [T,B,U]: the outputs of decoder cell 0; attention [T,B,U] or None (zeros) -> outputs of the last cell [T,B,U]."""
+    T, B, U = x.shape
+    cells = decoder_cell_names(first_layer, num_layers)
+    hs = [torch.zeros(B, U, dtype=x.dtype) for _ in cells]         # cell2.zero_state, gnmt_model.py:375
+    cs = [torch.zeros(B, U, dtype=x.dtype) for _ in cells]
+    outs = []
+    for t in range(T):
+        cur_inp = x[t]
+        new_attention = torch.zeros(B, U, dtype=x.dtype) if attention is None else attention[t].detach()   # :518
+        for i, (scope, residual) in enumerate(cells):
+            inp = torch.cat([cur_inp, new_attention], -1)          # :526
+            nh, nc = lstm_cell(inp, hs[i], cs[i], w[scope + "/kernel"], w[scope + "/bias"], forget_bias)
+            hs[i], cs[i] = nh, nc
+            cur_inp = nh + inp[:, :U] if residual else nh          # gnmt_residual_fn :587-613: outputs + actual inputs
+        outs.append(cur_inp)
+    return torch.stack(outs)
+
+
+def nmt_loss(outputs, proj_kernel, target_output, target_sequence_length, batch_size=None):
+    """model.py:685-686 (logits = output_layer(rnn_output), a Dense without bias, :497-499) and _compute_loss :824-838.
+    outputs [T,B,U]; target_output [B,T] ints (transposed at :827-828); returns (loss, logits [T,B,V])."""
+    T, B, _ = outputs.shape
+    logits = outputs @ proj_kernel
+    labels = target_output.long().t()                               # [T,B]
+    crossent = -torch.log_softmax(logits, -1).gather(-1, labels.unsqueeze(-1)).squeeze(-1)    # :820-821
+    target_weights = (torch.arange(T).unsqueeze(0) < target_sequence_length.long().unsqueeze(1)).to(outputs.dtype).t()  # :833-836
+    loss = (crossent * target_weights).sum() / float(batch_size if batch_size is not None else B)   # :837-838
+    return loss, logits

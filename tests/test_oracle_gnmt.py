@@ -114,3 +114,61 @@ def test_parameter_count_of_config():
     cells = sum(v.size for k, v in w.items() if "embedding" not in k)
     assert cells == 2 * (2048 * 4096 + 4096) + (3072 * 4096 + 4096) + 6 * (2048 * 4096 + 4096)
     assert abs(cells - 79.7e6) < 0.1e6
+
+
+def test_decoder_part2_matches_lstmcell_on_the_concatenated_input():
+    torch.manual_seed(7)
+    T, B, U = 4, 3, 5
+    x = torch.randn(T, B, U, dtype=torch.float64)
+    att = torch.randn(T, B, U, dtype=torch.float64, requires_grad=True)
+    cells = og.decoder_cell_names(1, 3)
+    assert [r for _, r in cells] == [False, True, True] and cells[0][0].endswith("multi_rnn_cell_part2/cell_1/basic_lstm_cell")
+    w = {}
+    for scope, _ in cells:
+        w[scope + "/kernel"] = (torch.randn(3 * U, 4 * U, dtype=torch.float64) * 0.3).requires_grad_(True)
+        w[scope + "/bias"] = torch.randn(4 * U, dtype=torch.float64) * 0.1
+    out = og.decoder_part2_forward(x, att, w, 1, 3, forget_bias=1.0)
+    # library cells: torch gate order i, f, g, o; TF order i, j(=g), f, o; forget_bias folded into the bias
+    perm = torch.cat([torch.arange(0, U), torch.arange(2 * U, 3 * U), torch.arange(U, 2 * U), torch.arange(3 * U, 4 * U)])
+    lib = []
+    for scope, _ in cells:
+        c = torch.nn.LSTMCell(2 * U, U).double()
+        k, b = w[scope + "/kernel"].detach(), w[scope + "/bias"].clone()
+        b[2 * U:3 * U] += 1.0
+        with torch.no_grad():
+            c.weight_ih.copy_(k[:2 * U, perm].t()); c.weight_hh.copy_(k[2 * U:, perm].t())
+            c.bias_ih.copy_(b[perm]); c.bias_hh.zero_()
+        lib.append(c)
+    st = [(torch.zeros(B, U, dtype=torch.float64), torch.zeros(B, U, dtype=torch.float64)) for _ in cells]
+    for t in range(T):
+        cur = x[t]
+        for i, (_, residual) in enumerate(cells):
+            h, c = lib[i](torch.cat([cur, att[t].detach()], -1), st[i])
+            st[i] = (h, c)
+            cur = h + cur if residual else h
+        assert torch.allclose(out[t], cur, atol=1e-12)
+    # the attention is a constant of the graph; the kernel rows that multiply it do get a gradient
+    gk = torch.autograd.grad(out.sum(), [w[cells[0][0] + "/kernel"]], retain_graph=True)[0]
+    assert float(gk[U:2 * U].abs().max()) > 0
+    assert torch.autograd.grad(out.sum(), [att], allow_unused=True)[0] is None
+    # zeros for the attention (the variable's initial value) = dropping those kernel rows
+    out0 = og.decoder_part2_forward(x, None, w, 1, 3)
+    w1 = {k: (torch.cat([v[:U], torch.zeros(U, 4 * U, dtype=torch.float64), v[2 * U:]]) if k.endswith("kernel") else v) for k, v in w.items()}
+    assert torch.allclose(out0, og.decoder_part2_forward(x, att, w1, 1, 3), atol=1e-12)
+
+
+def test_nmt_loss_matches_library_cross_entropy():
+    torch.manual_seed(8)
+    T, B, U, V = 5, 3, 4, 7
+    outs = torch.randn(T, B, U, dtype=torch.float64)
+    k = torch.randn(U, V, dtype=torch.float64)
+    tgt = torch.randint(0, V, (B, T))
+    lens = torch.tensor([5, 2, 0])
+    loss, logits = og.nmt_loss(outs, k, tgt, lens)
+    tot = 0.0
+    for b in range(B):
+        n = int(lens[b])
+        if n:
+            tot += torch.nn.functional.cross_entropy(logits[:n, b], tgt[b, :n], reduction="sum").item()
+    assert abs(loss.item() - tot / B) < 1e-12
+    assert torch.allclose(logits[2, 1], outs[2, 1] @ k)
