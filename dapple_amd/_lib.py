@@ -58,8 +58,8 @@ class VggCfg(C.Structure):
 class GnmtCfg(C.Structure):
     _fields_ = [
         ("dtype", C.c_int), ("num_layers", C.c_int), ("units", C.c_int), ("vocab", C.c_int), ("batch", C.c_int),
-        ("seq", C.c_int), ("forget_bias", C.c_float), ("stash_slots", C.c_int), ("decoder_part2", C.c_int), ("first_layer", C.c_int),
-        ("reserved", C.c_int * 6),
+        ("seq", C.c_int), ("forget_bias", C.c_float), ("stash_slots", C.c_int), ("part", C.c_int), ("first_layer", C.c_int),
+        ("src_seq", C.c_int), ("reserved", C.c_int * 5),
     ]
 
 
@@ -114,6 +114,7 @@ PROTOTYPES = {
     "ds_gnmt_stage_create": (C.c_int, [C.POINTER(GnmtCfg), C.c_void_p, C.POINTER(C.c_void_p)]),
     "ds_gnmt_stage_set_lengths": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p]),
     "ds_gnmt_stage_set_attention": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p]),
+    "ds_gnmt_stage_set_decoder_inputs": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
     "ds_xlnet_stage_create": (C.c_int, [C.POINTER(XlnetCfg), C.c_void_p, C.POINTER(C.c_void_p)]),
     "ds_xlnet_stage_set_inputs": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
     "ds_stage_create": (C.c_int, [C.POINTER(StageCfg), C.c_void_p, C.POINTER(C.c_void_p)]),

@@ -549,13 +549,414 @@ struct GnmtDecoderStage : ds_stage {
   }
 };
 
+// ---------------------------------------------------------------------------------------------------------
+// Decoder cell 0 under the attention wrapper: the first device's share of the decoder (gnmt_model.py:309-325,
+// :366-374; model.py:622-640).  Per target step t:
+//   gates = [emb_t | attention_{t-1} | h_{t-1}] K + bias -> (h_t, c_t);  pq = h_t W_q;
+//   score[b, j] = sum_u nv[u] tanh(keys[b, j, u] + pq[b, u] + attention_b[u]) for j < source length, nv = g v / ||v||;
+//   alignments = softmax_j;  attention_t = sum_j alignments[b, j] values[b, j, :]
+// with values = the memory (encoder outputs) zeroed past each source length, keys = values W_mem.
+
+// values[b, j, :] = j < len[b] ? memory[j, b, :] : 0 (batch-major); block 0 also forms nv = g v / ||v||
+__global__ __launch_bounds__(256) void att_prep_kernel(int B, int S, int U, const float* __restrict__ memory, const int32_t* __restrict__ len,
+                                                      float* __restrict__ values, const float* __restrict__ v, const float* __restrict__ gsc,
+                                                      float* __restrict__ nv) {
+  __shared__ float red[4];
+  const int row = blockIdx.x;  // b * S + j
+  const int b = row / S, j = row % S;
+  const bool live = !len || j < len[b];
+  for (int u = threadIdx.x; u < U; u += 256) values[(int64_t)row * U + u] = live ? memory[((int64_t)j * B + b) * U + u] : 0.f;
+  if (row == 0) {
+    float ss = 0.f;
+    for (int u = threadIdx.x; u < U; u += 256) ss += v[u] * v[u];
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const float sc = gsc[0] * rsqrtf(red[0] + red[1] + red[2] + red[3]);
+    for (int u = threadIdx.x; u < U; u += 256) nv[u] = sc * v[u];
+  }
+}
+
+constexpr int ATT_MAX_S = 512;
+
+// one block per sample b: scores over the source steps, softmax, context
+__global__ __launch_bounds__(256) void att_fwd_kernel(int S, int U, const float* __restrict__ keys, const float* __restrict__ values,
+                                                     const float* __restrict__ pq, const float* __restrict__ nv,
+                                                     const float* __restrict__ bias, const int32_t* __restrict__ len,
+                                                     float* __restrict__ align, float* __restrict__ ctx, int ldc) {
+  __shared__ float sc[ATT_MAX_S];
+  __shared__ float red[4];
+  const int b = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int n = len ? len[b] : S;
+  n = n < 0 ? 0 : (n > S ? S : n);
+  for (int j = wave; j < n; j += 4) {
+    const float* k = keys + ((int64_t)b * S + j) * U;
+    float a = 0.f;
+    for (int u = lane * 4; u < U; u += 256) {
+      const f32x4 kv = *reinterpret_cast<const f32x4*>(k + u);
+      const f32x4 qv = *reinterpret_cast<const f32x4*>(pq + (int64_t)b * U + u);
+      const f32x4 bv = *reinterpret_cast<const f32x4*>(bias + u);
+      const f32x4 vv = *reinterpret_cast<const f32x4*>(nv + u);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) a += vv[e] * tanhf(kv[e] + qv[e] + bv[e]);
+    }
+    a = wave_sum(a);
+    if (lane == 0) sc[j] = a;
+  }
+  __syncthreads();
+  float mx = -INFINITY;
+  for (int j = threadIdx.x; j < n; j += 256) mx = fmaxf(mx, sc[j]);
+  mx = wave_max(mx);
+  if (lane == 0) red[wave] = mx;
+  __syncthreads();
+  mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  __syncthreads();
+  float sum = 0.f;
+  for (int j = threadIdx.x; j < n; j += 256) sum += expf(sc[j] - mx);
+  sum = wave_sum(sum);
+  if (lane == 0) red[wave] = sum;
+  __syncthreads();
+  sum = red[0] + red[1] + red[2] + red[3];
+  for (int j = threadIdx.x; j < S; j += 256) {
+    const float p = j < n ? expf(sc[j] - mx) / sum : 0.f;
+    align[(int64_t)b * S + j] = p;
+    if (j < n) sc[j] = p;
+  }
+  __syncthreads();
+  for (int u = threadIdx.x; u < U; u += 256) {
+    float c = 0.f;
+    for (int j = 0; j < n; ++j) c += sc[j] * values[((int64_t)b * S + j) * U + u];
+    ctx[(int64_t)b * ldc + u] = c;
+  }
+}
+
+// one block per sample b: gradient of one step's attention.  datt [B,U] = d loss / d attention_t is consumed and
+// cleared; dkeys / dvalues [B,S,U] are added to; dpq [B,U] is written; dnv / dbias [U] receive atomic adds.
+__global__ __launch_bounds__(256) void att_bwd_kernel(int S, int U, const float* __restrict__ keys, const float* __restrict__ values,
+                                                     const float* __restrict__ pq, const float* __restrict__ nv,
+                                                     const float* __restrict__ bias, const int32_t* __restrict__ len,
+                                                     const float* __restrict__ align, float* __restrict__ datt, float* __restrict__ dpq,
+                                                     float* __restrict__ dkeys, float* __restrict__ dvalues, float* __restrict__ dnv,
+                                                     float* __restrict__ dbias) {
+  __shared__ float ds[ATT_MAX_S];
+  __shared__ float red[4];
+  const int b = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int n = len ? len[b] : S;
+  n = n < 0 ? 0 : (n > S ? S : n);
+  const float* da = datt + (int64_t)b * U;
+  for (int j = wave; j < n; j += 4) {  // d alignment[j] = datt . values[j]
+    const float* vj = values + ((int64_t)b * S + j) * U;
+    float a = 0.f;
+    for (int u = lane * 4; u < U; u += 256) {
+      const f32x4 x = *reinterpret_cast<const f32x4*>(vj + u);
+      const f32x4 d = *reinterpret_cast<const f32x4*>(da + u);
+      a += x[0] * d[0] + x[1] * d[1] + x[2] * d[2] + x[3] * d[3];
+    }
+    a = wave_sum(a);
+    if (lane == 0) ds[j] = a;
+  }
+  __syncthreads();
+  float s = 0.f;
+  for (int j = threadIdx.x; j < n; j += 256) s += align[(int64_t)b * S + j] * ds[j];
+  s = wave_sum(s);
+  if (lane == 0) red[wave] = s;
+  __syncthreads();
+  s = red[0] + red[1] + red[2] + red[3];
+  __syncthreads();
+  for (int j = threadIdx.x; j < n; j += 256) ds[j] = align[(int64_t)b * S + j] * (ds[j] - s);  // d score[j]
+  __syncthreads();
+  for (int u = threadIdx.x; u < U; u += 256) {
+    const float q = pq[(int64_t)b * U + u] + bias[u], v = nv[u], dat = da[u];
+    float acc_pq = 0.f, acc_nv = 0.f;
+    for (int j = 0; j < n; ++j) {
+      const int64_t o = ((int64_t)b * S + j) * U + u;
+      const float th = tanhf(keys[o] + q);
+      const float d = ds[j] * v * (1.f - th * th);
+      dkeys[o] += d;
+      dvalues[o] += align[(int64_t)b * S + j] * dat;
+      acc_pq += d;
+      acc_nv += ds[j] * th;
+    }
+    dpq[(int64_t)b * U + u] = acc_pq;
+    atomicAdd(dbias + u, acc_pq);
+    atomicAdd(dnv + u, acc_nv);
+    datt[(int64_t)b * U + u] = 0.f;
+  }
+}
+
+// d memory[j, b, :] = j < len[b] ? dvalues[b, j, :] : 0
+__global__ __launch_bounds__(256) void att_dmemory_kernel(int B, int S, int U, const float* __restrict__ dvalues, const int32_t* __restrict__ len,
+                                                         float* __restrict__ dmem) {
+  const int row = blockIdx.x, b = row / S, j = row % S;
+  const bool live = !len || j < len[b];
+  for (int u = threadIdx.x; u < U; u += 256) dmem[((int64_t)j * B + b) * U + u] = live ? dvalues[(int64_t)row * U + u] : 0.f;
+}
+
+// nv = g v / ||v||:  dg += dnv . v / ||v||;  dv += g / ||v|| (dnv - (dnv . v) v / ||v||^2)     (one block)
+__global__ __launch_bounds__(256) void att_vg_bwd_kernel(int U, const float* __restrict__ dnv, const float* __restrict__ v,
+                                                        const float* __restrict__ gsc, float* __restrict__ dv, float* __restrict__ dg) {
+  __shared__ float r0[4], r1[4];
+  float dot = 0.f, ss = 0.f;
+  for (int u = threadIdx.x; u < U; u += 256) { dot += dnv[u] * v[u]; ss += v[u] * v[u]; }
+  dot = wave_sum(dot); ss = wave_sum(ss);
+  if ((threadIdx.x & 63) == 0) { r0[threadIdx.x >> 6] = dot; r1[threadIdx.x >> 6] = ss; }
+  __syncthreads();
+  dot = r0[0] + r0[1] + r0[2] + r0[3];
+  ss = r1[0] + r1[1] + r1[2] + r1[3];
+  const float inv = rsqrtf(ss), g = gsc[0];
+  for (int u = threadIdx.x; u < U; u += 256) dv[u] += g * inv * (dnv[u] - dot * v[u] / ss);
+  if (threadIdx.x == 0) dg[0] += dot * inv;
+}
+
+__global__ __launch_bounds__(256) void gnmt_fill0_kernel(float* __restrict__ p, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) p[i] = 0.f;
+}
+
+struct GnmtAttentionStage : ds_stage {
+  ds_gnmt_cfg gc;
+  int B, T, S, U, R, RS;
+  enum { W_EMB, W_K, W_BIAS, W_MEM, W_Q, W_V, W_G, W_B };
+  char* stash_base = nullptr;
+  size_t slot_bytes = 0, ids_off, len_off, nv_off, val_off, key_off, emb_off, ah_off, g_off, c_off, al_off, pq_off;
+  std::vector<char> slot_has_len;
+  std::vector<float*> slot_att_out;
+  char* ws_base = nullptr;
+  size_t ws_bytes = 0, ws_dg, ws_dh[2], ws_dc, ws_datt, ws_dpq, ws_dkeys, ws_dval, ws_dnv, ws_demb;
+
+  ~GnmtAttentionStage() override {
+    if (stash_base) (void)hipFree(stash_base);
+    if (ws_base) (void)hipFree(ws_base);
+  }
+
+  int init() {
+    B = gc.batch; T = gc.seq; S = gc.src_seq; U = gc.units; R = B * T; RS = B * S;
+    const char* P = "dynamic_seq2seq/decoder/";
+    const char* A = "multi_rnn_cell_part1/cell_0_attention/attention/";
+    char name[200];
+    snprintf(name, sizeof(name), "%sembedding_decoder", P); winfo.push_back({name, gc.vocab, U});
+    snprintf(name, sizeof(name), "%s%sbasic_lstm_cell/kernel", P, A); winfo.push_back({name, 3 * U, 4 * U});
+    snprintf(name, sizeof(name), "%s%sbasic_lstm_cell/bias", P, A); winfo.push_back({name, 1, 4 * U});
+    snprintf(name, sizeof(name), "%smemory_layer/kernel", P); winfo.push_back({name, U, U});
+    snprintf(name, sizeof(name), "%s%sbahdanau_attention/query_layer/kernel", P, A); winfo.push_back({name, U, U});
+    snprintf(name, sizeof(name), "%s%sbahdanau_attention/attention_v", P, A); winfo.push_back({name, 1, U});
+    snprintf(name, sizeof(name), "%s%sbahdanau_attention/attention_g", P, A); winfo.push_back({name, 1, 1});
+    snprintf(name, sizeof(name), "%s%sbahdanau_attention/attention_b", P, A); winfo.push_back({name, 1, U});
+    Arena sa;
+    ids_off = sa.reserve((size_t)R * 4);
+    len_off = sa.reserve((size_t)B * 4);
+    nv_off = sa.reserve((size_t)U * 4);
+    val_off = sa.reserve((size_t)RS * U * 4);
+    key_off = sa.reserve((size_t)RS * U * 4);
+    emb_off = sa.reserve((size_t)R * U * 4);
+    ah_off = sa.reserve((size_t)(T + 1) * B * 2 * U * 4);  // block t = [attention_{t-1} | h_{t-1}], block 0 zero
+    g_off = sa.reserve((size_t)R * 4 * U * 4);
+    c_off = sa.reserve((size_t)R * U * 4);
+    al_off = sa.reserve((size_t)T * RS * 4);
+    pq_off = sa.reserve((size_t)R * U * 4);
+    slot_bytes = sa.used;
+    DS_CHECK_HIP(hipMalloc((void**)&stash_base, slot_bytes * gc.stash_slots));
+    slot_forwarded.assign(gc.stash_slots, 0);
+    slot_has_len.assign(gc.stash_slots, 0);
+    slot_att_out.assign(gc.stash_slots, nullptr);
+    Arena wa;
+    ws_dg = wa.reserve((size_t)R * 4 * U * 4);
+    ws_dh[0] = wa.reserve((size_t)B * U * 4);
+    ws_dh[1] = wa.reserve((size_t)B * U * 4);
+    ws_dc = wa.reserve((size_t)B * U * 4);
+    ws_datt = wa.reserve((size_t)B * U * 4);
+    ws_dpq = wa.reserve((size_t)R * U * 4);
+    ws_dkeys = wa.reserve((size_t)RS * U * 4);
+    ws_dval = wa.reserve((size_t)RS * U * 4);
+    ws_dnv = wa.reserve((size_t)U * 4);
+    ws_demb = wa.reserve((size_t)R * U * 4);
+    ws_bytes = wa.used;
+    DS_CHECK_HIP(hipMalloc((void**)&ws_base, ws_bytes));
+    return DS_OK;
+  }
+
+  size_t workspace_bytes() const override { return ws_bytes; }
+  bool overlap_safe() const override { return true; }  // forward touches its stash slot and its outputs only
+  size_t stash_bytes(int slots) const override { return slot_bytes * (size_t)slots; }
+  int refresh_weights() override { return DS_OK; }
+
+  int gemm(int am, int bm, int m, int n, int k, const void* a, int64_t lda, const void* b, int64_t ldb, void* c, int64_t ldc,
+           int flags, const float* bias, const void* residual) {
+    ds_gemm_desc d;
+    memset(&d, 0, sizeof(d));
+    d.dtype = DS_F32; d.a_major = am; d.b_major = bm; d.m = m; d.n = n; d.k = k; d.lda = lda; d.ldb = ldb; d.ldc = ldc;
+    d.batch = 1; d.batch_inner = 1; d.flags = flags; d.alpha = 1.f; d.a = a; d.b = b; d.c = c; d.bias = bias; d.residual = residual;
+    return ds_gemm(&d, stream);
+  }
+  int gemm_accum_splitk(int bm, int m, int n, int k, const void* a, int64_t lda, const void* b, int64_t ldb, float* c, int64_t ldc) {
+    ds_gemm_desc d;
+    memset(&d, 0, sizeof(d));
+    d.dtype = DS_F32; d.a_major = DS_K_MAJOR; d.b_major = bm; d.m = m; d.n = n; d.k = k; d.lda = lda; d.ldb = ldb; d.ldc = ldc;
+    d.batch = 1; d.batch_inner = 1; d.flags = DS_EPI_ACCUM; d.alpha = 1.f; d.a = a; d.b = b; d.c = c;
+    return ds_gemm_splitk(&d, GnmtStage::split_for(m, n, k), stream);
+  }
+  int fill0(float* p, int64_t n) {
+    const int64_t blocks = (n + 255) / 256;
+    hipLaunchKernelGGL(gnmt_fill0_kernel, dim3((unsigned)(blocks > 2048 ? 2048 : blocks)), dim3(256), 0, stream, p, n);
+    DS_CHECK_LAUNCH();
+    return DS_OK;
+  }
+
+  int set_inputs(int slot, const int32_t* target_input, const int32_t* source_lengths, float* attention_out) {
+    char* sp = stash_base + (size_t)slot * slot_bytes;
+    DS_CHECK_HIP(hipMemcpyAsync(sp + ids_off, target_input, (size_t)R * 4, hipMemcpyDeviceToDevice, stream));
+    if (source_lengths) DS_CHECK_HIP(hipMemcpyAsync(sp + len_off, source_lengths, (size_t)B * 4, hipMemcpyDeviceToDevice, stream));
+    slot_has_len[slot] = source_lengths != nullptr;
+    slot_att_out[slot] = attention_out;
+    return DS_OK;
+  }
+
+  int forward(int slot, const void* in, const float*, void* out) override {
+    ds_prio_scope prio(1);
+    char* sp = stash_base + (size_t)slot * slot_bytes;
+    const int32_t* len = slot_has_len[slot] ? (const int32_t*)(sp + len_off) : nullptr;
+    float* values = (float*)(sp + val_off);
+    float* keys = (float*)(sp + key_off);
+    float* nv = (float*)(sp + nv_off);
+    float* emb = (float*)(sp + emb_off);
+    float* AH = (float*)(sp + ah_off);
+    float* G = (float*)(sp + g_off);
+    float* Cs = (float*)(sp + c_off);
+    float* AL = (float*)(sp + al_off);
+    float* PQ = (float*)(sp + pq_off);
+    const float* kernel = w[W_K];
+    hipLaunchKernelGGL(att_prep_kernel, dim3(RS), dim3(256), 0, stream, B, S, U, (const float*)in, len, values, w[W_V], w[W_G], nv);
+    hipLaunchKernelGGL(gnmt_embed_fwd_kernel, dim3((R + 3) / 4), dim3(256), 0, stream, B, T, U, gc.vocab, (const int32_t*)(sp + ids_off),
+                       w[W_EMB], emb);
+    DS_CHECK_LAUNCH();
+    DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, RS, U, U, values, U, w[W_MEM], U, keys, U, 0, nullptr, nullptr));
+    DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, R, 4 * U, U, emb, U, kernel, 4 * U, G, 4 * U, DS_EPI_BIAS, w[W_BIAS], nullptr));
+    DS_PROPAGATE(fill0(AH, (int64_t)B * 2 * U));
+    DS_PROPAGATE(fill0(PQ, (int64_t)R * U));
+    const int cell_grid = (B * U + 255) / 256;
+    for (int t = 0; t < T; ++t) {
+      float* g = G + (size_t)t * B * 4 * U;
+      float* ah = AH + (size_t)t * B * 2 * U;       // [attention_{t-1} | h_{t-1}]
+      float* ah_next = ah + (size_t)B * 2 * U;
+      if (t > 0) DS_PROPAGATE(gemm_accum_splitk(DS_MN_MAJOR, B, 4 * U, 2 * U, ah, 2 * U, kernel + (size_t)U * 4 * U, 4 * U, g, 4 * U));
+      hipLaunchKernelGGL(lstm_cell_fwd_kernel, dim3(cell_grid), dim3(256), 0, stream, B, U, gc.forget_bias, g,
+                         t > 0 ? Cs + (size_t)(t - 1) * B * U : nullptr, Cs + (size_t)t * B * U, ah_next + U, 2 * U, (const float*)nullptr, 0,
+                         (float*)nullptr, 0, (const int32_t*)nullptr, t);
+      DS_CHECK_LAUNCH();
+      float* pq = PQ + (size_t)t * B * U;
+      DS_PROPAGATE(gemm_accum_splitk(DS_MN_MAJOR, B, U, U, ah_next + U, 2 * U, w[W_Q], U, pq, U));
+      ds_prof_scope prof(stream, "att_fwd_kernel", (double)RS * U * 4 * 2, "B");
+      hipLaunchKernelGGL(att_fwd_kernel, dim3(B), dim3(256), 0, stream, S, U, keys, values, pq, nv, w[W_B], len, AL + (size_t)t * RS, ah_next,
+                         2 * U);
+      DS_CHECK_LAUNCH();
+    }
+    // the cell outputs and, if asked for, the attention of every step, out of the [attention | h] blocks 1 .. T
+    DS_CHECK_HIP(hipMemcpy2DAsync(out, (size_t)U * 4, AH + (size_t)B * 2 * U + U, (size_t)2 * U * 4, (size_t)U * 4, R, hipMemcpyDeviceToDevice,
+                                  stream));
+    if (slot_att_out[slot])
+      DS_CHECK_HIP(hipMemcpy2DAsync(slot_att_out[slot], (size_t)U * 4, AH + (size_t)B * 2 * U, (size_t)2 * U * 4, (size_t)U * 4, R,
+                                    hipMemcpyDeviceToDevice, stream));
+    return DS_OK;
+  }
+
+  int backward(int slot, const void* d_out, void* d_in) override {
+    ds_prio_scope prio(3);
+    char* sp = stash_base + (size_t)slot * slot_bytes;
+    const int32_t* len = slot_has_len[slot] ? (const int32_t*)(sp + len_off) : nullptr;
+    const float* values = (const float*)(sp + val_off);
+    const float* keys = (const float*)(sp + key_off);
+    const float* nv = (const float*)(sp + nv_off);
+    const float* emb = (const float*)(sp + emb_off);
+    const float* AH = (const float*)(sp + ah_off);
+    const float* G = (const float*)(sp + g_off);
+    const float* Cs = (const float*)(sp + c_off);
+    const float* AL = (const float*)(sp + al_off);
+    const float* PQ = (const float*)(sp + pq_off);
+    const float* kernel = w[W_K];
+    float* dG = (float*)(ws_base + ws_dg);
+    float* dc = (float*)(ws_base + ws_dc);
+    float* datt = (float*)(ws_base + ws_datt);
+    float* dPQ = (float*)(ws_base + ws_dpq);
+    float* dkeys = (float*)(ws_base + ws_dkeys);
+    float* dval = (float*)(ws_base + ws_dval);
+    float* dnv = (float*)(ws_base + ws_dnv);
+    const float* dY = (const float*)d_out;
+    // datt .. dnv are adjacent: the last step's dpq, the two [B,S,U] accumulators and dnv start at zero
+    DS_PROPAGATE(fill0(datt, (int64_t)((ws_demb - ws_datt) / 4)));
+    const int cell_grid = (B * U + 255) / 256;
+    for (int t = T - 1; t >= 0; --t) {
+      const int first = (t == T - 1);  // nothing downstream reads the last step's state or attention
+      float* dh_in = (float*)(ws_base + ws_dh[t & 1]);
+      float* dh_out = (float*)(ws_base + ws_dh[(t & 1) ^ 1]);
+      float* dpq = dPQ + (size_t)t * B * U;
+      if (!first) {
+        ds_prof_scope prof(stream, "att_bwd_kernel", (double)RS * U * 4 * 6, "B");
+        hipLaunchKernelGGL(att_bwd_kernel, dim3(B), dim3(256), 0, stream, S, U, keys, values, PQ + (size_t)t * B * U, nv, w[W_B], len,
+                           AL + (size_t)t * RS, datt, dpq, dkeys, dval, dnv, g[W_B]);
+        DS_CHECK_LAUNCH();
+        // the query is the cell output: dh_t += dpq W_q^T
+        DS_PROPAGATE(gemm_accum_splitk(DS_K_MAJOR, B, U, U, dpq, U, w[W_Q], U, dh_in, U));
+      }
+      hipLaunchKernelGGL(lstm_cell_bwd_kernel, dim3(cell_grid), dim3(256), 0, stream, B, U, G + (size_t)t * B * 4 * U, Cs + (size_t)t * B * U,
+                         t > 0 ? Cs + (size_t)(t - 1) * B * U : nullptr, dY + (size_t)t * B * U, U, dh_in, dc, first, dG + (size_t)t * B * 4 * U,
+                         (const int32_t*)nullptr, t, t > 0 ? dh_out : nullptr);
+      DS_CHECK_LAUNCH();
+      if (t > 0) {
+        const float* dg = dG + (size_t)t * B * 4 * U;
+        DS_PROPAGATE(gemm_accum_splitk(DS_K_MAJOR, B, U, 4 * U, dg, 4 * U, kernel + (size_t)2 * U * 4 * U, 4 * U, dh_out, U));
+        DS_PROPAGATE(gemm_accum_splitk(DS_K_MAJOR, B, U, 4 * U, dg, 4 * U, kernel + (size_t)U * 4 * U, 4 * U, datt, U));
+      }
+    }
+    // parameter gradients over all steps
+    DS_PROPAGATE(ds_colsum_accum(DS_F32, R, 4 * U, dG, 4 * U, g[W_BIAS], stream));
+    DS_PROPAGATE(gemm(DS_MN_MAJOR, DS_MN_MAJOR, U, 4 * U, R, emb, U, dG, 4 * U, g[W_K], 4 * U, DS_EPI_ACCUM, nullptr, nullptr));
+    DS_PROPAGATE(gemm(DS_MN_MAJOR, DS_MN_MAJOR, 2 * U, 4 * U, R, AH, 2 * U, dG, 4 * U, g[W_K] + (size_t)U * 4 * U, 4 * U, DS_EPI_ACCUM, nullptr,
+                      nullptr));
+    DS_PROPAGATE(gemm(DS_MN_MAJOR, DS_MN_MAJOR, U, U, R, AH + (size_t)B * 2 * U + U, 2 * U, dPQ, U, g[W_Q], U, DS_EPI_ACCUM, nullptr, nullptr));
+    DS_PROPAGATE(gemm(DS_MN_MAJOR, DS_MN_MAJOR, U, U, RS, values, U, dkeys, U, g[W_MEM], U, DS_EPI_ACCUM, nullptr, nullptr));
+    hipLaunchKernelGGL(att_vg_bwd_kernel, dim3(1), dim3(256), 0, stream, U, dnv, w[W_V], w[W_G], g[W_V], g[W_G]);
+    DS_CHECK_LAUNCH();
+    // embedding rows
+    float* demb = (float*)(ws_base + ws_demb);
+    DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, R, U, 4 * U, dG, 4 * U, kernel, 4 * U, demb, U, 0, nullptr, nullptr));
+    hipLaunchKernelGGL(gnmt_embed_bwd_kernel, dim3((R + 3) / 4), dim3(256), 0, stream, B, T, U, gc.vocab, (const int32_t*)(sp + ids_off), demb,
+                       g[W_EMB]);
+    DS_CHECK_LAUNCH();
+    // the memory: through the values directly and through the keys
+    if (d_in) {
+      DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, RS, U, U, dkeys, U, w[W_MEM], U, dval, U, DS_EPI_RESIDUAL, nullptr, dval));
+      hipLaunchKernelGGL(att_dmemory_kernel, dim3(RS), dim3(256), 0, stream, B, S, U, dval, len, (float*)d_in);
+      DS_CHECK_LAUNCH();
+    }
+    return DS_OK;
+  }
+};
+
 }  // namespace
 
 extern "C" int ds_gnmt_stage_create(const ds_gnmt_cfg* c, void* stream, ds_stage** out) {
   DS_CHECK_ARG(c != nullptr && out != nullptr, "ds_gnmt_stage_create: null argument");
   *out = nullptr;
   DS_CHECK_ARG(c->dtype == DS_F32, "ds_gnmt_stage_create: only fp32 is built (dtype %d)", c->dtype);
-  if (c->decoder_part2) {
+  if (c->part == DS_GNMT_ATTENTION_CELL) {
+    DS_CHECK_ARG(c->units > 0 && c->units % 4 == 0, "ds_gnmt_stage_create: num_units (%d) must be a positive multiple of 4", c->units);
+    DS_CHECK_ARG(c->batch > 0 && c->seq > 0 && c->batch % 4 == 0 && c->vocab > 0,
+                 "ds_gnmt_stage_create: batch (%d) must be a positive multiple of 4, seq (%d) and vocab (%d) positive", c->batch, c->seq, c->vocab);
+    DS_CHECK_ARG(c->src_seq >= 1 && c->src_seq <= ATT_MAX_S, "ds_gnmt_stage_create: src_seq (%d) must be in [1, %d]", c->src_seq, ATT_MAX_S);
+    DS_CHECK_ARG(c->stash_slots >= 1, "ds_gnmt_stage_create: stash_slots must be >= 1");
+    GnmtAttentionStage* s = new GnmtAttentionStage();
+    memset(&s->cfg, 0, sizeof(s->cfg));
+    s->cfg.kind = DS_STAGE_GNMT;
+    s->cfg.dtype = c->dtype;
+    s->cfg.stash_slots = c->stash_slots;
+    s->gc = *c;
+    s->stream = (hipStream_t)stream;
+    const int rc = s->init();
+    if (rc != DS_OK) { delete s; return rc; }
+    *out = s;
+    return DS_OK;
+  }
+  DS_CHECK_ARG(c->part == DS_GNMT_ENCODER || c->part == DS_GNMT_DECODER_PART2, "ds_gnmt_stage_create: unknown part %d", c->part);
+  if (c->part == DS_GNMT_DECODER_PART2) {
     DS_CHECK_ARG(c->num_layers >= 1 && c->first_layer >= 1, "ds_gnmt_stage_create: decoder part 2 holds cells first_layer >= 1 .. (got %d layers from %d)",
                  c->num_layers, c->first_layer);
     DS_CHECK_ARG(c->units > 0 && c->units % 4 == 0, "ds_gnmt_stage_create: num_units (%d) must be a positive multiple of 4", c->units);
@@ -609,4 +1010,15 @@ extern "C" int ds_gnmt_stage_set_attention(ds_stage* h, int slot, const float* a
   DS_CHECK_ARG(slot >= 0 && slot < h->cfg.stash_slots, "ds_gnmt_stage_set_attention: slot %d out of range", slot);
   DS_PROPAGATE(ds_stage_acquire_slot(h, slot));
   return dec->set_attention(slot, attention);
+}
+
+extern "C" int ds_gnmt_stage_set_decoder_inputs(ds_stage* h, int slot, const int32_t* target_input, const int32_t* source_sequence_length,
+                                                float* attention_out) {
+  DS_CHECK_ARG(h != nullptr, "ds_gnmt_stage_set_decoder_inputs: null handle");
+  GnmtAttentionStage* st = h->cfg.kind == DS_STAGE_GNMT ? dynamic_cast<GnmtAttentionStage*>(h) : nullptr;
+  DS_CHECK_ARG(st != nullptr, "ds_gnmt_stage_set_decoder_inputs: not a GNMT attention-cell stage");
+  DS_CHECK_ARG(slot >= 0 && slot < h->cfg.stash_slots, "ds_gnmt_stage_set_decoder_inputs: slot %d out of range", slot);
+  DS_CHECK_ARG(target_input != nullptr, "ds_gnmt_stage_set_decoder_inputs: null target_input");
+  DS_PROPAGATE(ds_stage_acquire_slot(h, slot));
+  return st->set_inputs(slot, target_input, source_sequence_length, attention_out);
 }

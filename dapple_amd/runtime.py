@@ -252,7 +252,7 @@ def gnmt_decoder_stage(num_layers, units, batch, seq, stash_slots, first_layer=1
     cfg = GnmtCfg()
     cfg.dtype, cfg.num_layers, cfg.units, cfg.vocab = _dtype_code(dtype), num_layers, units, 0
     cfg.batch, cfg.seq, cfg.forget_bias, cfg.stash_slots = batch, seq, forget_bias, stash_slots
-    cfg.decoder_part2, cfg.first_layer = 1, first_layer
+    cfg.part, cfg.first_layer = 1, first_layer
     h = C.c_void_p()
     with torch.cuda.device(torch.device(device)):
         check(lib.ds_gnmt_stage_create(C.byref(cfg), _lib.current_stream(), C.byref(h)), "ds_gnmt_stage_create")
@@ -262,7 +262,39 @@ def gnmt_decoder_stage(num_layers, units, batch, seq, stash_slots, first_layer=1
     return st
 
 
+def gnmt_attention_stage(units, vocab, batch, seq, src_seq, stash_slots, forget_bias=1.0, dtype="fp32", device="cuda:0"):
+    """Decoder cell 0 under the attention wrapper, on the first device behind the encoder (gnmt/nmt/gnmt_model.py:309-325,
+    :366-374, :440-487; model.py:622-640): memory [src_seq, batch, units] -> cell outputs [seq, batch, units]."""
+    lib = _lib.load()
+    cfg = GnmtCfg()
+    cfg.dtype, cfg.num_layers, cfg.units, cfg.vocab = _dtype_code(dtype), 1, units, vocab
+    cfg.batch, cfg.seq, cfg.forget_bias, cfg.stash_slots = batch, seq, forget_bias, stash_slots
+    cfg.part, cfg.src_seq = 2, src_seq
+    h = C.c_void_p()
+    with torch.cuda.device(torch.device(device)):
+        check(lib.ds_gnmt_stage_create(C.byref(cfg), _lib.current_stream(), C.byref(h)), "ds_gnmt_stage_create")
+    st = GnmtStage(h, _TORCH_DTYPE[cfg.dtype], src_seq * batch * units, seq * batch * units, stash_slots, device=device, cfg=cfg)
+    st.out_shape = (seq, batch, units)
+    return st
+
+
 class GnmtStage(Stage):
+    def set_decoder_inputs(self, slot, target_input, source_sequence_length=None, attention_out=None):
+        """Attention-cell stage: side inputs of the micro-batch about to be forwarded into ``slot``: target_input int32
+        [batch, seq], source_sequence_length int32 [batch] (None: full length), attention_out fp32 [seq, batch, units] that the
+        forward pass fills with every step's attention vector (keep it alive until then)."""
+        b, t = self.cfg.batch, self.cfg.seq
+        if target_input.dtype != torch.int32 or not target_input.is_cuda or not target_input.is_contiguous() or target_input.numel() != b * t:
+            raise ValueError("target_input must be a contiguous int32 GPU tensor of [batch, seq]")
+        if source_sequence_length is not None and (source_sequence_length.dtype != torch.int32 or not source_sequence_length.is_cuda
+                                                   or source_sequence_length.numel() != b):
+            raise ValueError("source_sequence_length must be an int32 GPU tensor of [batch]")
+        if attention_out is not None and (attention_out.dtype != torch.float32 or not attention_out.is_cuda or not attention_out.is_contiguous()
+                                          or attention_out.numel() != self.out_numel):
+            raise ValueError("attention_out must be a contiguous fp32 GPU tensor of [seq, batch, units]")
+        check(self.lib.ds_gnmt_stage_set_decoder_inputs(self._h, slot, ptr(target_input), ptr(source_sequence_length), ptr(attention_out)),
+              "ds_gnmt_stage_set_decoder_inputs")
+
     def set_attention(self, slot, attention=None):
         """Decoder stage: the attention vectors [seq, batch, units] fp32 every cell of the micro-batch about to be
         forwarded into ``slot`` concatenates to its input (None: zeros).  No gradient flows into them."""

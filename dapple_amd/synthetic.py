@@ -263,3 +263,20 @@ def gnmt_decoder_weights(seed, first_layer, num_layers, units, init_weight=0.1, 
         w[scope + "/bias"] = rng.uniform(-init_weight, init_weight, 4 * units).astype(np.float32) if perturb \
             else np.zeros(4 * units, np.float32)
     return w
+
+
+def gnmt_attention_weights(seed, units, vocab, init_weight=0.1, perturb=False):
+    """Decoder cell 0 with its attention wrapper: embedding_decoder, the cell's kernel [3*units, 4*units] and bias, the
+    memory and query layers, attention_v, attention_g (sqrt(1/units), TensorFlow's initial value) and attention_b."""
+    rng = _rng(seed)
+    P = "dynamic_seq2seq/decoder/"
+    A = P + "multi_rnn_cell_part1/cell_0_attention/attention/"
+    u = lambda *shape: rng.uniform(-init_weight, init_weight, shape).astype(np.float32)
+    return {P + "embedding_decoder": u(vocab, units),
+            A + "basic_lstm_cell/kernel": u(3 * units, 4 * units),
+            A + "basic_lstm_cell/bias": u(4 * units) if perturb else np.zeros(4 * units, np.float32),
+            P + "memory_layer/kernel": u(units, units),
+            A + "bahdanau_attention/query_layer/kernel": u(units, units),
+            A + "bahdanau_attention/attention_v": u(units),
+            A + "bahdanau_attention/attention_g": np.array([np.sqrt(1.0 / units) * (1.3 if perturb else 1.0)], np.float32),
+            A + "bahdanau_attention/attention_b": u(units) if perturb else np.zeros(units, np.float32)}

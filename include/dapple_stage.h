@@ -261,17 +261,19 @@ typedef struct ds_gnmt_cfg {
   int units, vocab, batch, seq;
   float forget_bias; /* 1.0 in gnmt/nmt/standard_hparams/wmt16_gnmt_8_layer.json */
   int stash_slots;
-  int decoder_part2; /* 0: the encoder stage above; 1: the decoder cells of the second device (below) */
-  int first_layer;   /* decoder_part2: index of the first decoder cell held (1 in the reference, gnmt_model.py:346-364) */
-  int reserved[6];
+  int part;          /* DS_GNMT_ENCODER (0): the encoder stage above; DS_GNMT_DECODER_PART2; DS_GNMT_ATTENTION_CELL (below) */
+  int first_layer;   /* DS_GNMT_DECODER_PART2: index of the first decoder cell held (1 in the reference, gnmt_model.py:346-364) */
+  int src_seq;       /* DS_GNMT_ATTENTION_CELL: source steps of the memory (seq = target steps) */
+  int reserved[5];
 } ds_gnmt_cfg;
+enum { DS_GNMT_ENCODER = 0, DS_GNMT_DECODER_PART2 = 1, DS_GNMT_ATTENTION_CELL = 2 };
 int ds_gnmt_stage_create(const ds_gnmt_cfg* cfg, void* stream, ds_stage** out);
 /* iterator.source_sequence_length (gnmt_model.py:103, 223-227) of the micro-batch that will be forwarded
  * into `slot`: lengths [batch] int32 on the device, or NULL for full length.  Every layer's dynamic_rnn
  * gets it: steps t >= lengths[b] emit zeros (residual layers too) and keep the state, the backward
  * direction of the first layer starts at step lengths[b] - 1.  The setting stays with the slot. */
 int ds_gnmt_stage_set_lengths(ds_stage* h, int slot, const int32_t* lengths);
-/* decoder_part2 = 1: decoder cells first_layer .. first_layer + num_layers - 1 as the reference's second device runs
+/* part = DS_GNMT_DECODER_PART2: decoder cells first_layer .. first_layer + num_layers - 1 as the reference's second device runs
  * them - GNMTAttentionMultiCell_2, gnmt/nmt/gnmt_model.py:489-537, under dynamic_decode with a TrainingHelper on the
  * outputs of cell 0 (gnmt/nmt/model.py:641-656): a scan over all `seq` padded target steps from the zero state
  * (:375).  in / out / d_out / d_in are fp32 [seq, batch, units]; vocab is unused.  Cell l has one kernel
@@ -281,6 +283,21 @@ int ds_gnmt_stage_set_lengths(ds_stage* h, int slot, const int32_t* lengths);
  * reference (:456-459), i.e. it is a constant of the graph: here it is a per-slot side input [seq, batch, units]
  * on the device that receives no gradient; NULL (the default) stands for zeros, the variable's initial value. */
 int ds_gnmt_stage_set_attention(ds_stage* h, int slot, const float* attention);
+/* part = DS_GNMT_ATTENTION_CELL: decoder cell 0 under the attention wrapper, which the reference keeps on the FIRST
+ * device behind the encoder (GNMTAttentionMultiCell_1, gnmt/nmt/gnmt_model.py:440-487; built at :309-325, :366-374 as
+ * AttentionWrapper(BasicLSTMCell, BahdanauAttention(normalize=True, memory_sequence_length=source_sequence_length),
+ * attention_layer_size=None, output_attention=False); driven by dynamic_decode with a TrainingHelper on the embedded
+ * target_input, gnmt/nmt/model.py:622-640).  The stage input `in` is the memory = the encoder stage's output, fp32
+ * [src_seq, batch, units]; `out` = outputs_1.rnn_output, fp32 [seq, batch, units]; d_in = d loss / d memory (feed it
+ * to the encoder stage's backward pass).  Weights, in ds_stage_weight_info order: embedding_decoder [vocab, units],
+ * the cell's kernel [3*units, 4*units] (rows: embedded input | previous attention | h) and bias, memory_layer/kernel,
+ * query_layer/kernel [units, units], attention_v [units], attention_g [1], attention_b [units].
+ * ds_gnmt_stage_set_decoder_inputs gives the slot its side inputs before the forward pass: target_input int32
+ * [batch, seq]; source_sequence_length int32 [batch] (NULL = src_seq; every length must be >= 1, an empty source gives
+ * NaN in TensorFlow and zeros here); attention_out (nullable) fp32 [seq, batch, units] receives every step's attention
+ * vector (what the second device's cells concatenate to their input). */
+int ds_gnmt_stage_set_decoder_inputs(ds_stage* h, int slot, const int32_t* target_input,
+                                     const int32_t* source_sequence_length, float* attention_out);
 
 /* XLNet stage (xlnet/models/slice_xlnet.py:164-180 layer body; xlnet/layers/rel_multihead_attn.py:71-149).
  * Activations are sequence-major like the reference: in/out are [streams][seq][batch][hidden] (stream 0 =

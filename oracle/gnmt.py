@@ -24,6 +24,12 @@ decoder_part2_forward / nmt_loss restate the second device's share of the decode
 model.py:641-686) and the loss (model.py:791-838).  Pins: a two-cell stack vs torch.nn.LSTMCell fed the concatenated
 input, with the residual taken from the first half of the input; no gradient reaches the attention input; the loss vs
 torch.nn.functional.cross_entropy(reduction="sum") over the unpadded positions divided by the batch size.
+
+attention_cell_forward restates decoder cell 0 under tf.contrib.seq2seq.AttentionWrapper with normed
+BahdanauAttention (both un-vendored TensorFlow: "parity unpinned" against TensorFlow itself).  Pins: the LSTM part vs
+torch.nn.LSTMCell on concat([x_t, previous attention]); the score by scalar loops on a tiny case; alignments sum to one
+over the valid source steps and are exactly zero past them; the context equals torch.bmm(alignments, memory); memory
+rows past the source length influence nothing.
 """
 import torch
 
@@ -139,3 +145,50 @@ def nmt_loss(outputs, proj_kernel, target_output, target_sequence_length, batch_
     target_weights = (torch.arange(T).unsqueeze(0) < target_sequence_length.long().unsqueeze(1)).to(outputs.dtype).t()  # :833-836
     loss = (crossent * target_weights).sum() / float(batch_size if batch_size is not None else B)   # :837-838
     return loss, logits
+
+
+# ---- decoder cell 0 with the attention wrapper: the first device's share of the decoder ----
+# gnmt_model.py:309-325 (memory = encoder outputs, batch-major; normed Bahdanau attention over it with
+# memory_sequence_length = source_sequence_length, attention_model.py:173-178), :366-374 (AttentionWrapper(cell 0,
+# attention_layer_size=None, output_attention=False) inside GNMTAttentionMultiCell_1, zero initial state) and
+# model.py:622-640 (embedding lookup of the time-major target_input, dynamic_decode with a TrainingHelper: a scan over
+# the padded target steps).  AttentionWrapper and BahdanauAttention live in TensorFlow (un-vendored); their published
+# algorithm is restated: values = memory with the steps past each source length zeroed, keys = values W_mem,
+# cell input = concat([x_t, attention_{t-1}]), query = cell output h_t,
+# score[b, j] = sum_u nv[u] tanh(keys[b, j, u] + (h_t W_q)[b, u] + attention_b[u]), nv = attention_g v / ||v||,
+# score = -inf past the source length, alignments = softmax_j, attention_t = context = sum_j alignments values.
+DA = "dynamic_seq2seq/decoder/"
+EMB_DEC = DA + "embedding_decoder"
+ATT_CELL = DA + "multi_rnn_cell_part1/cell_0_attention/attention/basic_lstm_cell"
+ATT_MEM = DA + "memory_layer/kernel"
+ATT_Q = DA + "multi_rnn_cell_part1/cell_0_attention/attention/bahdanau_attention/query_layer/kernel"
+ATT_V = DA + "multi_rnn_cell_part1/cell_0_attention/attention/bahdanau_attention/attention_v"
+ATT_G = DA + "multi_rnn_cell_part1/cell_0_attention/attention/bahdanau_attention/attention_g"
+ATT_B = DA + "multi_rnn_cell_part1/cell_0_attention/attention/bahdanau_attention/attention_b"
+
+
+def attention_cell_forward(target_input, memory, source_sequence_length, w, forget_bias=1.0):
+    """target_input [B,T] ints; memory [S,B,U] (the encoder's time-major outputs); source_sequence_length [B] >= 1.
+    Returns (cell outputs [T,B,U] = outputs_1.rnn_output, attention per step [T,B,U])."""
+    emb = w[EMB_DEC][target_input.long().t()]                       # model.py:624-627
+    mem = memory.transpose(0, 1)                                    # gnmt_model.py:309-312
+    B, S, U = mem.shape
+    mask = torch.arange(S).unsqueeze(0) < source_sequence_length.long().unsqueeze(1)       # [B,S]
+    values = mem * mask.unsqueeze(-1).to(mem.dtype)
+    keys = values @ w[ATT_MEM]
+    v = w[ATT_V]
+    nv = w[ATT_G] * v * torch.rsqrt((v * v).sum())
+    h = torch.zeros(B, U, dtype=mem.dtype)
+    c = torch.zeros(B, U, dtype=mem.dtype)
+    att = torch.zeros(B, U, dtype=mem.dtype)
+    outs, atts = [], []
+    for t in range(emb.shape[0]):
+        h, c = lstm_cell(torch.cat([emb[t], att], -1), h, c, w[ATT_CELL + "/kernel"], w[ATT_CELL + "/bias"], forget_bias)
+        pq = h @ w[ATT_Q]
+        score = (nv * torch.tanh(keys + pq.unsqueeze(1) + w[ATT_B])).sum(-1)
+        score = torch.where(mask, score, torch.full_like(score, float("-inf")))
+        align = torch.softmax(score, -1)
+        att = (align.unsqueeze(-1) * values).sum(1)
+        outs.append(h)
+        atts.append(att)
+    return torch.stack(outs), torch.stack(atts)

@@ -172,3 +172,52 @@ def test_nmt_loss_matches_library_cross_entropy():
             tot += torch.nn.functional.cross_entropy(logits[:n, b], tgt[b, :n], reduction="sum").item()
     assert abs(loss.item() - tot / B) < 1e-12
     assert torch.allclose(logits[2, 1], outs[2, 1] @ k)
+
+
+def _attention_case(seed, T, B, S, U, V):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.rand(*s, generator=g, dtype=torch.float64) * 2 - 1
+    w = {og.EMB_DEC: r(V, U) * 0.5, og.ATT_CELL + "/kernel": r(3 * U, 4 * U) * 0.4, og.ATT_CELL + "/bias": r(4 * U) * 0.1,
+         og.ATT_MEM: r(U, U) * 0.5, og.ATT_Q: r(U, U) * 0.5, og.ATT_V: r(U), og.ATT_G: torch.tensor((1.0 / U) ** 0.5, dtype=torch.float64),
+         og.ATT_B: r(U) * 0.1}
+    ids = torch.randint(0, V, (B, T), generator=g)
+    mem = r(S, B, U)
+    return w, ids, mem
+
+
+def test_attention_cell_against_library_pieces_and_scalar_loops():
+    import math
+    T, B, S, U, V = 3, 2, 4, 3, 6
+    w, ids, mem = _attention_case(9, T, B, S, U, V)
+    lens = torch.tensor([4, 2])
+    outs, atts = og.attention_cell_forward(ids, mem, lens, w)
+    perm = torch.cat([torch.arange(0, U), torch.arange(2 * U, 3 * U), torch.arange(U, 2 * U), torch.arange(3 * U, 4 * U)])
+    cell = torch.nn.LSTMCell(2 * U, U).double()
+    k, b = w[og.ATT_CELL + "/kernel"], w[og.ATT_CELL + "/bias"].clone()
+    b[2 * U:3 * U] += 1.0
+    with torch.no_grad():
+        cell.weight_ih.copy_(k[:2 * U, perm].t()); cell.weight_hh.copy_(k[2 * U:, perm].t()); cell.bias_ih.copy_(b[perm]); cell.bias_hh.zero_()
+    h = c = torch.zeros(B, U, dtype=torch.float64)
+    att = torch.zeros(B, U, dtype=torch.float64)
+    v = w[og.ATT_V].tolist()
+    vn = math.sqrt(sum(x * x for x in v))
+    for t in range(T):
+        h, c = cell(torch.cat([w[og.EMB_DEC][ids[:, t]], att], -1), (h, c))
+        assert torch.allclose(outs[t], h, atol=1e-12)
+        new_att = torch.zeros(B, U, dtype=torch.float64)
+        for bb in range(B):
+            pq = [sum(h[bb, i].item() * w[og.ATT_Q][i, u].item() for i in range(U)) for u in range(U)]
+            sc = []
+            for j in range(int(lens[bb])):
+                key = [sum(mem[j, bb, i].item() * w[og.ATT_MEM][i, u].item() for i in range(U)) for u in range(U)]
+                sc.append(sum(w[og.ATT_G].item() * v[u] / vn * math.tanh(key[u] + pq[u] + w[og.ATT_B][u].item()) for u in range(U)))
+            mx = max(sc)
+            z = sum(math.exp(s - mx) for s in sc)
+            for j, s in enumerate(sc):
+                new_att[bb] += math.exp(s - mx) / z * mem[j, bb]
+        assert torch.allclose(atts[t], new_att, atol=1e-12)
+        att = new_att
+    # memory past the source length influences nothing
+    mem2 = mem.clone(); mem2[2:, 1] += 5.0
+    outs2, atts2 = og.attention_cell_forward(ids, mem2, lens, w)
+    assert torch.equal(outs, outs2) and torch.equal(atts, atts2)
