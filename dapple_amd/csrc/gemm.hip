@@ -1066,6 +1066,45 @@ static void choose_tiling(int m, int n, int k, int kt, int batch, bool can_split
   }
 }
 
+// C (fp32) = alpha * A B^T for bf16 operands with a reduction of exactly 64 (one attention head), both K-major:
+// the score products q k^T / dO v^T.  A 64x64 tile of such a product is 16 KB of operands and 16 KB of output -
+// nothing is reused often enough to stage it: every wave loads its fragments straight from global memory in MFMA
+// operand order (lane = row, 8 consecutive k), multiplies 4 x 4 MFMAs and stores its accumulators, whose lanes run
+// along n (128 contiguous bytes per half wave).  No LDS, no barrier: four such blocks fit a CU beside anything else.
+__global__ __launch_bounds__(256) void gemm_k64_f32out_kernel(GemmArgs p) {
+  ds_wave_prio(p.prio);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5, r = lane & 31;
+  const int tiles_n = p.n / 64;
+  const int64_t wt = (int64_t)blockIdx.x * 4 + wave;
+  if (wt >= (int64_t)(p.m / 64) * tiles_n) return;
+  const int m0 = (int)(wt / tiles_n) * 64, n0 = (int)(wt % tiles_n) * 64;
+  const int z = blockIdx.z, zo = z / p.batch_inner, zi = z % p.batch_inner;
+  const bf16* A = reinterpret_cast<const bf16*>(p.a) + zo * p.a_so + zi * p.a_si + (int64_t)(m0 + r) * p.lda + half * 8;
+  const bf16* B = reinterpret_cast<const bf16*>(p.b) + zo * p.b_so + zi * p.b_si + (int64_t)(n0 + r) * p.ldb + half * 8;
+  float* C = reinterpret_cast<float*>(p.c) + zo * p.c_so + zi * p.c_si;
+  bf16x8 fa[2][4], fb[2][4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      fa[i][ks] = *reinterpret_cast<const bf16x8*>(A + (int64_t)i * 32 * p.lda + ks * 16);
+      fb[i][ks] = *reinterpret_cast<const bf16x8*>(B + (int64_t)i * 32 * p.ldb + ks * 16);
+    }
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      f32x16 acc;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[e] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i][ks], fb[j][ks], acc, 0, 0, 0);
+      float* c = C + (int64_t)(m0 + i * 32) * p.ldc + n0 + j * 32 + r;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) c[(int64_t)((e >> 2) * 8 + half * 4 + (e & 3)) * p.ldc] = acc[e] * p.alpha;
+    }
+}
+
 static int gemm_run(const ds_gemm_desc* d, int splitk_req, void* stream) {
   DS_CHECK_ARG(d != nullptr, "ds_gemm: null descriptor");
   DS_CHECK_ARG(d->dtype == DS_F32 || d->dtype == DS_BF16, "ds_gemm: dtype %d", d->dtype);
@@ -1114,6 +1153,15 @@ static int gemm_run(const ds_gemm_desc* d, int splitk_req, void* stream) {
   a.prio = ds_launch_prio;
   a.vec_epi = d->n % 8 == 0 && d->ldc % 8 == 0 && d->c_stride_outer % 8 == 0 && d->c_stride_inner % 8 == 0 &&
               ds_aligned16(d->c) && ds_aligned16(d->residual) && ds_aligned16(d->c2);
+  if (d->dtype == DS_BF16 && d->a_major == DS_K_MAJOR && d->b_major == DS_K_MAJOR && d->k == 64 && f == DS_EPI_OUT_F32 &&
+      d->m % 64 == 0 && d->n % 64 == 0 && batch <= 65535) {
+    hipStream_t s = (hipStream_t)stream;
+    ds_prof_scope prof(s, "gemm_k64_f32out_kernel<bf16>", 2.0 * d->m * d->n * d->k * batch, "FLOP");
+    const int64_t wave_tiles = (int64_t)(d->m / 64) * (d->n / 64);
+    hipLaunchKernelGGL(gemm_k64_f32out_kernel, dim3((unsigned)((wave_tiles + 3) / 4), 1, batch), dim3(256), 0, s, a);
+    DS_CHECK_LAUNCH();
+    return DS_OK;
+  }
   const int kt = d->dtype == DS_BF16 ? 64 : 32;
   int tile, splitk;
   choose_tiling(d->m, d->n, d->k, kt, batch, (f & DS_EPI_ACCUM) != 0, &tile, &splitk);

@@ -57,23 +57,24 @@ __global__ __launch_bounds__(256) void xl_pos_emb_kernel(int R, int H, int klen,
   }
 }
 
-// One wave per (query row i, batch b, head n) of one stream:
-//   score[j] = (ac[i][j] + bd[i][j + Q - i] + ef[seg(i,j,b)]) * scale - 1e30 * mask[i][j][b],  p = softmax_j
-// with ef[s] = (q + r_s)[i,b,n,:] . seg_emb[s,n,:].  ac is [B*N][Q][K], bd [B*N][Q][R] (fp32).
+// One wave per (stacked query row i', batch b, head n); the streams' query rows are stacked, i' = stream * Q + i
+// (QQ rows in all), as the q buffers and the masks hold them:
+//   score[j] = (ac[i'][j] + bd[i'][j + Q - i] + ef[seg(i,j,b)]) * scale - 1e30 * mask[i'][j][b],  p = softmax_j
+// with ef[s] = (q + r_s)[i',b,n,:] . seg_emb[s,n,:].  ac is [B*N][QQ][K], bd [B*N][QQ][R] (fp32).
 template <typename T, int NV>
-__global__ __launch_bounds__(256) void xl_softmax_fwd_kernel(int Q, int K, int R, int B, int N, int D, const float* __restrict__ ac,
+__global__ __launch_bounds__(256) void xl_softmax_fwd_kernel(int Q, int QQ, int K, int R, int B, int N, int D, const float* __restrict__ ac,
                                                             const float* __restrict__ bd, const T* __restrict__ qs,
                                                             const float* __restrict__ seg_emb, const uint8_t* __restrict__ seg_mat,
                                                             const float* __restrict__ mask, float scale, T* __restrict__ p) {
   const int lane = threadIdx.x & 63;
-  const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // = (b*N + n)*Q + i
-  if (w >= (int64_t)B * N * Q) return;
-  const int i = (int)(w % Q);
-  const int bn = (int)(w / Q), n = bn % N, b = bn / N;
+  const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // = (b*N + n)*QQ + i'
+  if (w >= (int64_t)B * N * QQ) return;
+  const int ii = (int)(w % QQ), i = ii % Q;
+  const int bn = (int)(w / QQ), n = bn % N, b = bn / N;
   const int H = N * D;
   float e0 = 0.f, e1 = 0.f;
   if (lane < D) {
-    const float qv = to_f32(qs[((int64_t)i * B + b) * H + n * D + lane]);
+    const float qv = to_f32(qs[((int64_t)ii * B + b) * H + n * D + lane]);
     e0 = qv * seg_emb[n * D + lane];
     e1 = qv * seg_emb[H + n * D + lane];
   }
@@ -87,10 +88,9 @@ __global__ __launch_bounds__(256) void xl_softmax_fwd_kernel(int Q, int K, int R
   for (int t = 0; t < NV * 4; ++t) {
     const int j = lane + t * 64;
     if (j < K) {
-      const int64_t ijb = ((int64_t)i * K + j) * B + b;
-      const float ef = (seg_mat && seg_mat[ijb]) ? e1 : e0;
+      const float ef = (seg_mat && seg_mat[((int64_t)i * K + j) * B + b]) ? e1 : e0;
       float s = (acr[j] + bdr[j] + ef) * scale;
-      if (mask) s -= 1e30f * mask[ijb];
+      if (mask) s -= 1e30f * mask[((int64_t)ii * K + j) * B + b];
       v[t] = s;
       mx = fmaxf(mx, s);
     } else {
@@ -115,15 +115,15 @@ __global__ __launch_bounds__(256) void xl_softmax_fwd_kernel(int Q, int K, int R
 //   dbd[i][r] = ds[i][r - Q + i] when that column exists, else 0 (transpose of the rel_shift index map);
 //   def[s] = sum_j [seg(i,j,b) == s] ds[i][j] (gradient of the two segment scores of the row).
 template <typename T, int NV>
-__global__ __launch_bounds__(256) void xl_softmax_bwd_kernel(int Q, int K, int R, int B, int N, const T* __restrict__ p,
+__global__ __launch_bounds__(256) void xl_softmax_bwd_kernel(int Q, int QQ, int K, int R, int B, int N, const T* __restrict__ p,
                                                             const float* __restrict__ dp, float scale,
                                                             const uint8_t* __restrict__ seg_mat, T* __restrict__ ds,
                                                             T* __restrict__ dbd, float* __restrict__ defs) {
   const int lane = threadIdx.x & 63;
   const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (w >= (int64_t)B * N * Q) return;
-  const int i = (int)(w % Q);
-  const int b = (int)(w / Q) / N;
+  if (w >= (int64_t)B * N * QQ) return;
+  const int i = (int)(w % QQ) % Q;
+  const int b = (int)(w / QQ) / N;
   const T* pr = p + w * K;
   const float* dr = dp + w * K;
   float pv[NV][4], dv[NV][4];
@@ -163,24 +163,24 @@ __global__ __launch_bounds__(256) void xl_softmax_bwd_kernel(int Q, int K, int R
   if (lane == 0) { defs[w * 2] = d0; defs[w * 2 + 1] = d1; }
 }
 
-// One wave per (i, b, n): writes def to deft[(n*2+s)][row] for the seg_emb gradient GEMM,
+// One wave per (stacked query row i', b, n): writes def to deft[(n*2+s)][row] for the seg_emb gradient GEMM,
 // dqs = def[0]*seg_emb[0] + def[1]*seg_emb[1], and dq = dqw + dqr + dqs.
 template <typename T>
-__global__ __launch_bounds__(256) void xl_seg_bwd_kernel(int Q, int B, int N, int D, int64_t rows_total, int64_t row0,
+__global__ __launch_bounds__(256) void xl_seg_bwd_kernel(int QQ, int B, int N, int D, int64_t rows_total,
                                                         const float* __restrict__ defs, const float* __restrict__ seg_emb,
                                                         const T* __restrict__ dqw, const T* __restrict__ dqr, T* __restrict__ dqs,
                                                         T* __restrict__ dq, T* __restrict__ deft) {
   const int lane = threadIdx.x & 63;
   const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (w >= (int64_t)B * N * Q) return;
-  const int i = (int)(w % Q);
-  const int bn = (int)(w / Q), n = bn % N, b = bn / N;
+  if (w >= (int64_t)B * N * QQ) return;
+  const int ii = (int)(w % QQ);
+  const int bn = (int)(w / QQ), n = bn % N, b = bn / N;
   const int H = N * D;
   const float d0 = defs[w * 2], d1 = defs[w * 2 + 1];
-  const int64_t row = (int64_t)i * B + b;  // row inside this stream
+  const int64_t row = (int64_t)ii * B + b;
   if (lane == 0) {
-    deft[(int64_t)(n * 2 + 0) * rows_total + row0 + row] = from_f32<T>(d0);
-    deft[(int64_t)(n * 2 + 1) * rows_total + row0 + row] = from_f32<T>(d1);
+    deft[(int64_t)(n * 2 + 0) * rows_total + row] = from_f32<T>(d0);
+    deft[(int64_t)(n * 2 + 1) * rows_total + row] = from_f32<T>(d1);
   }
   if (lane < D) {
     const int64_t o = row * H + n * D + lane;
@@ -283,12 +283,13 @@ struct XlnetStage : ds_stage {
     // workspace
     Arena w;
     ws_qall = w.reserve(act);
-    ws_ac = w.reserve((size_t)B * N * Q * K * 4);
-    ws_dp = w.reserve((size_t)B * N * Q * K * 4);  // backward's own score-gradient buffer: forward keeps ws_ac
-    ws_bd = w.reserve((size_t)B * N * Q * R * 4);
-    ws_ds = w.reserve((size_t)B * N * Q * K * esz);
-    ws_dbd = w.reserve((size_t)B * N * Q * R * esz);
-    ws_def = w.reserve((size_t)B * N * Q * 2 * 4);
+    const size_t QQ = (size_t)S * Q;  // the streams' query rows stacked: one product / one softmax launch for all of them
+    ws_ac = w.reserve((size_t)B * N * QQ * K * 4);
+    ws_dp = w.reserve((size_t)B * N * QQ * K * 4);  // backward's own score-gradient buffer: forward keeps ws_ac
+    ws_bd = w.reserve((size_t)B * N * QQ * R * 4);
+    ws_ds = w.reserve((size_t)B * N * QQ * K * esz);
+    ws_dbd = w.reserve((size_t)B * N * QQ * R * esz);
+    ws_def = w.reserve((size_t)B * N * QQ * 2 * 4);
     ws_dy1 = w.reserve(act); ws_dvec = w.reserve(act);
     for (int p = 0; p < 2; ++p) {
       ws_dz2[p] = w.reserve(act); ws_du[p] = w.reserve(actF); ws_dz1[p] = w.reserve(act);
@@ -377,29 +378,31 @@ struct XlnetStage : ds_stage {
 
   template <typename T> int softmax_fwd_t(const float* ac, const float* bd, const T* qs, const float* seg_emb, const uint8_t* seg,
                                           const float* mask, float scale, T* p) {
-    const int64_t waves = (int64_t)B * N * Q;
+    const int QQ = S * Q;
+    const int64_t waves = (int64_t)B * N * QQ;
     dim3 grid((unsigned)((waves + 3) / 4));
     const int need = (K + 255) / 256;
     ds_prof_scope prof(stream, sizeof(T) == 2 ? "xl_softmax_fwd_kernel<bf16>" : "xl_softmax_fwd_kernel<float>",
                        (double)waves * K * (8 + sizeof(T) + 5), "B");
-    if (need <= 1) hipLaunchKernelGGL((xl_softmax_fwd_kernel<T, 1>), grid, dim3(256), 0, stream, Q, K, R, B, N, D, ac, bd, qs, seg_emb, seg, mask, scale, p);
-    else if (need <= 2) hipLaunchKernelGGL((xl_softmax_fwd_kernel<T, 2>), grid, dim3(256), 0, stream, Q, K, R, B, N, D, ac, bd, qs, seg_emb, seg, mask, scale, p);
-    else if (need <= 4) hipLaunchKernelGGL((xl_softmax_fwd_kernel<T, 4>), grid, dim3(256), 0, stream, Q, K, R, B, N, D, ac, bd, qs, seg_emb, seg, mask, scale, p);
-    else hipLaunchKernelGGL((xl_softmax_fwd_kernel<T, 8>), grid, dim3(256), 0, stream, Q, K, R, B, N, D, ac, bd, qs, seg_emb, seg, mask, scale, p);
+    if (need <= 1) hipLaunchKernelGGL((xl_softmax_fwd_kernel<T, 1>), grid, dim3(256), 0, stream, Q, QQ, K, R, B, N, D, ac, bd, qs, seg_emb, seg, mask, scale, p);
+    else if (need <= 2) hipLaunchKernelGGL((xl_softmax_fwd_kernel<T, 2>), grid, dim3(256), 0, stream, Q, QQ, K, R, B, N, D, ac, bd, qs, seg_emb, seg, mask, scale, p);
+    else if (need <= 4) hipLaunchKernelGGL((xl_softmax_fwd_kernel<T, 4>), grid, dim3(256), 0, stream, Q, QQ, K, R, B, N, D, ac, bd, qs, seg_emb, seg, mask, scale, p);
+    else hipLaunchKernelGGL((xl_softmax_fwd_kernel<T, 8>), grid, dim3(256), 0, stream, Q, QQ, K, R, B, N, D, ac, bd, qs, seg_emb, seg, mask, scale, p);
     DS_CHECK_LAUNCH();
     return DS_OK;
   }
 
   template <typename T> int softmax_bwd_t(const T* p, const float* dp, float scale, const uint8_t* seg, T* dsm, T* dbd, float* defs) {
-    const int64_t waves = (int64_t)B * N * Q;
+    const int QQ = S * Q;
+    const int64_t waves = (int64_t)B * N * QQ;
     dim3 grid((unsigned)((waves + 3) / 4));
     const int need = (K + 255) / 256;
     ds_prof_scope prof(stream, sizeof(T) == 2 ? "xl_softmax_bwd_kernel<bf16>" : "xl_softmax_bwd_kernel<float>",
                        (double)waves * (K * (4 + 2 * sizeof(T)) + R * sizeof(T)), "B");
-    if (need <= 1) hipLaunchKernelGGL((xl_softmax_bwd_kernel<T, 1>), grid, dim3(256), 0, stream, Q, K, R, B, N, p, dp, scale, seg, dsm, dbd, defs);
-    else if (need <= 2) hipLaunchKernelGGL((xl_softmax_bwd_kernel<T, 2>), grid, dim3(256), 0, stream, Q, K, R, B, N, p, dp, scale, seg, dsm, dbd, defs);
-    else if (need <= 4) hipLaunchKernelGGL((xl_softmax_bwd_kernel<T, 4>), grid, dim3(256), 0, stream, Q, K, R, B, N, p, dp, scale, seg, dsm, dbd, defs);
-    else hipLaunchKernelGGL((xl_softmax_bwd_kernel<T, 8>), grid, dim3(256), 0, stream, Q, K, R, B, N, p, dp, scale, seg, dsm, dbd, defs);
+    if (need <= 1) hipLaunchKernelGGL((xl_softmax_bwd_kernel<T, 1>), grid, dim3(256), 0, stream, Q, QQ, K, R, B, N, p, dp, scale, seg, dsm, dbd, defs);
+    else if (need <= 2) hipLaunchKernelGGL((xl_softmax_bwd_kernel<T, 2>), grid, dim3(256), 0, stream, Q, QQ, K, R, B, N, p, dp, scale, seg, dsm, dbd, defs);
+    else if (need <= 4) hipLaunchKernelGGL((xl_softmax_bwd_kernel<T, 4>), grid, dim3(256), 0, stream, Q, QQ, K, R, B, N, p, dp, scale, seg, dsm, dbd, defs);
+    else hipLaunchKernelGGL((xl_softmax_bwd_kernel<T, 8>), grid, dim3(256), 0, stream, Q, QQ, K, R, B, N, p, dp, scale, seg, dsm, dbd, defs);
     DS_CHECK_LAUNCH();
     return DS_OK;
   }
@@ -434,20 +437,22 @@ struct XlnetStage : ds_stage {
                              w[b + X_RR], w[b + X_RS], (float*)(sp + t.qw), (float*)(sp + t.qr), (float*)(sp + t.qs));
         DS_CHECK_LAUNCH();
       }
-      for (int s = 0; s < S; ++s) {
-        const size_t so = (size_t)s * rowsS * H * esz;
+      {
+        // The streams' query rows are stacked in the q buffers ([stream][i][b] = row stream*Q + i of stride B*H): every
+        // product below and the softmax run once over all QQ = S*Q rows; probabilities are stashed as [B*N][QQ][K].
+        const int QQ = S * Q;
         // ac = (q + r_w) k^T ; bd (unshifted) = (q + r_r) k_r^T
-        DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_K_MAJOR, Q, K, D, sp + t.qw + so, (int64_t)B * H, H, D, sp + t.kv, (int64_t)B * 2 * H, 2 * H, D,
-                             ac, K, (int64_t)N * Q * K, (int64_t)Q * K, DS_EPI_OUT_F32));
-        DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_K_MAJOR, Q, R, D, sp + t.qr + so, (int64_t)B * H, H, D, kr[l], H, 0, D,
-                             bd, R, (int64_t)N * Q * R, (int64_t)Q * R, DS_EPI_OUT_F32));
-        const float* mask = has_mask[slot] ? (const float*)(sp + mask_off) + (size_t)s * Q * K * B : nullptr;
-        char* p = sp + t.p + (size_t)s * B * N * Q * K * esz;
-        if (dtype == DS_BF16) DS_PROPAGATE(softmax_fwd_t<bf16>(ac, bd, (const bf16*)(sp + t.qs + so), w[b + X_SEG], seg, mask, scale, (bf16*)p));
-        else DS_PROPAGATE(softmax_fwd_t<float>(ac, bd, (const float*)(sp + t.qs + so), w[b + X_SEG], seg, mask, scale, (float*)p));
+        DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_K_MAJOR, QQ, K, D, sp + t.qw, (int64_t)B * H, H, D, sp + t.kv, (int64_t)B * 2 * H, 2 * H, D,
+                             ac, K, (int64_t)N * QQ * K, (int64_t)QQ * K, DS_EPI_OUT_F32));
+        DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_K_MAJOR, QQ, R, D, sp + t.qr, (int64_t)B * H, H, D, kr[l], H, 0, D,
+                             bd, R, (int64_t)N * QQ * R, (int64_t)QQ * R, DS_EPI_OUT_F32));
+        const float* mask = has_mask[slot] ? (const float*)(sp + mask_off) : nullptr;
+        char* p = sp + t.p;
+        if (dtype == DS_BF16) DS_PROPAGATE(softmax_fwd_t<bf16>(ac, bd, (const bf16*)(sp + t.qs), w[b + X_SEG], seg, mask, scale, (bf16*)p));
+        else DS_PROPAGATE(softmax_fwd_t<float>(ac, bd, (const float*)(sp + t.qs), w[b + X_SEG], seg, mask, scale, (float*)p));
         // vec = P v
-        DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_MN_MAJOR, Q, D, K, p, K, (int64_t)N * Q * K, (int64_t)Q * K, sp + t.kv + (size_t)H * esz,
-                             (int64_t)B * 2 * H, 2 * H, D, sp + t.vec + so, (int64_t)B * H, H, D, 0));
+        DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_MN_MAJOR, QQ, D, K, p, K, (int64_t)N * QQ * K, (int64_t)QQ * K, sp + t.kv + (size_t)H * esz,
+                             (int64_t)B * 2 * H, 2 * H, D, sp + t.vec, (int64_t)B * H, H, D, 0));
       }
       // attn_out = vec Wo^T (einsum ibnd,hnd->ibh) + x, LayerNorm
       DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rows, H, H, sp + t.vec, H, WT(l, X_O), H, sp + t.z1, H, DS_EPI_RESIDUAL, nullptr, x));
@@ -491,44 +496,43 @@ struct XlnetStage : ds_stage {
                                     g[b + X_LN1_G], g[b + X_LN1_B], nullptr, stream));
       // o projection: attn_out[row,h] = sum_nd vec[row,nd] Wo[h,nd]
       DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, rows, H, H, dz1, H, WT(l, X_O), H, dvec, H));
-      for (int s = 0; s < S; ++s) {
-        const size_t so = (size_t)s * rowsS * H * esz;
-        const char* p = sp + t.p + (size_t)s * B * N * Q * K * esz;
-        const int acc = s > 0 ? DS_EPI_RESIDUAL : 0;  // k, v, k_r are shared by the streams: add in place
-        // dP = dvec v^T ; dv (+)= P^T dvec
-        DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_K_MAJOR, Q, K, D, dvec + so, (int64_t)B * H, H, D, sp + t.kv + (size_t)H * esz, (int64_t)B * 2 * H,
-                             2 * H, D, dp, K, (int64_t)N * Q * K, (int64_t)Q * K, DS_EPI_OUT_F32));
-        DS_PROPAGATE(gemm_bn(DS_MN_MAJOR, DS_MN_MAJOR, K, D, Q, p, K, (int64_t)N * Q * K, (int64_t)Q * K, dvec + so, (int64_t)B * H, H, D,
-                             dkv + (size_t)H * esz, (int64_t)B * 2 * H, 2 * H, D, acc, dkv + (size_t)H * esz));
+      {
+        // all streams' query rows at once (QQ = S*Q stacked rows, see forward): the sums over the streams that k, v and
+        // k_r receive fall out of the longer reductions
+        const int QQ = S * Q;
+        const char* p = sp + t.p;
+        // dP = dvec v^T ; dv = P^T dvec
+        DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_K_MAJOR, QQ, K, D, dvec, (int64_t)B * H, H, D, sp + t.kv + (size_t)H * esz, (int64_t)B * 2 * H,
+                             2 * H, D, dp, K, (int64_t)N * QQ * K, (int64_t)QQ * K, DS_EPI_OUT_F32));
+        DS_PROPAGATE(gemm_bn(DS_MN_MAJOR, DS_MN_MAJOR, K, D, QQ, p, K, (int64_t)N * QQ * K, (int64_t)QQ * K, dvec, (int64_t)B * H, H, D,
+                             dkv + (size_t)H * esz, (int64_t)B * 2 * H, 2 * H, D, 0));
         // dS, its un-shifted copy for the position term (dbd[i][r] = dS[i][r - Q + i]) and the segment sums, in one pass
         float* defs = (float*)(ws_base + ws_def);
         if (dtype == DS_BF16) DS_PROPAGATE(softmax_bwd_t<bf16>((const bf16*)p, dp, scale, seg, (bf16*)dsm, (bf16*)dbd, defs));
         else DS_PROPAGATE(softmax_bwd_t<float>((const float*)p, dp, scale, seg, (float*)dsm, (float*)dbd, defs));
-        // content term: dqw = dS k ; dk (+)= dS^T qw
-        DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_MN_MAJOR, Q, D, K, dsm, K, (int64_t)N * Q * K, (int64_t)Q * K, sp + t.kv, (int64_t)B * 2 * H, 2 * H, D,
-                             dqw + so, (int64_t)B * H, H, D, 0));
-        DS_PROPAGATE(gemm_bn(DS_MN_MAJOR, DS_MN_MAJOR, K, D, Q, dsm, K, (int64_t)N * Q * K, (int64_t)Q * K, sp + t.qw + so, (int64_t)B * H, H, D,
-                             dkv, (int64_t)B * 2 * H, 2 * H, D, acc, dkv));
+        // content term: dqw = dS k ; dk = dS^T qw
+        DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_MN_MAJOR, QQ, D, K, dsm, K, (int64_t)N * QQ * K, (int64_t)QQ * K, sp + t.kv, (int64_t)B * 2 * H, 2 * H, D,
+                             dqw, (int64_t)B * H, H, D, 0));
+        DS_PROPAGATE(gemm_bn(DS_MN_MAJOR, DS_MN_MAJOR, K, D, QQ, dsm, K, (int64_t)N * QQ * K, (int64_t)QQ * K, sp + t.qw, (int64_t)B * H, H, D,
+                             dkv, (int64_t)B * 2 * H, 2 * H, D, 0));
         // position term through the shift
-        DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_MN_MAJOR, Q, D, R, dbd, R, (int64_t)N * Q * R, (int64_t)Q * R, kr[l], H, 0, D,
-                             dqr + so, (int64_t)B * H, H, D, 0));
-        for (int bb = 0; bb < B; ++bb) {  // k_r is shared by the batch too: one launch per batch entry, added in place
-          const int a2 = (s > 0 || bb > 0) ? DS_EPI_RESIDUAL : 0;
-          DS_PROPAGATE(gemm_bn(DS_MN_MAJOR, DS_MN_MAJOR, R, D, Q, dbd + (size_t)bb * N * Q * R * esz, R, 0, (int64_t)Q * R,
-                               sp + t.qr + so + (size_t)bb * H * esz, (int64_t)B * H, 0, D, dkr, H, 0, D, a2, dkr, 1));
+        DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_MN_MAJOR, QQ, D, R, dbd, R, (int64_t)N * QQ * R, (int64_t)QQ * R, kr[l], H, 0, D,
+                             dqr, (int64_t)B * H, H, D, 0));
+        for (int bb = 0; bb < B; ++bb) {  // k_r is shared by the batch: one launch per batch entry, added in place
+          const int a2 = bb > 0 ? DS_EPI_RESIDUAL : 0;
+          DS_PROPAGATE(gemm_bn(DS_MN_MAJOR, DS_MN_MAJOR, R, D, QQ, dbd + (size_t)bb * N * QQ * R * esz, R, 0, (int64_t)QQ * R,
+                               sp + t.qr + (size_t)bb * H * esz, (int64_t)B * H, 0, D, dkr, H, 0, D, a2, dkr, 1));
         }
         // segment term + dq = dqw + dqr + dqs
         {
-          const int64_t waves = (int64_t)B * N * Q;
+          const int64_t waves = (int64_t)B * N * QQ;
           dim3 grid((unsigned)((waves + 3) / 4));
           if (dtype == DS_BF16)
-            hipLaunchKernelGGL(xl_seg_bwd_kernel<bf16>, grid, dim3(256), 0, stream, Q, B, N, D, (int64_t)rows, (int64_t)s * rowsS,
-                               defs, w[b + X_SEG], (const bf16*)(dqw + so), (const bf16*)(dqr + so), (bf16*)(dqs + so),
-                               (bf16*)(dq + so), (bf16*)deft);
+            hipLaunchKernelGGL(xl_seg_bwd_kernel<bf16>, grid, dim3(256), 0, stream, QQ, B, N, D, (int64_t)rows, defs, w[b + X_SEG],
+                               (const bf16*)dqw, (const bf16*)dqr, (bf16*)dqs, (bf16*)dq, (bf16*)deft);
           else
-            hipLaunchKernelGGL(xl_seg_bwd_kernel<float>, grid, dim3(256), 0, stream, Q, B, N, D, (int64_t)rows, (int64_t)s * rowsS,
-                               defs, w[b + X_SEG], (const float*)(dqw + so), (const float*)(dqr + so), (float*)(dqs + so),
-                               (float*)(dq + so), (float*)deft);
+            hipLaunchKernelGGL(xl_seg_bwd_kernel<float>, grid, dim3(256), 0, stream, QQ, B, N, D, (int64_t)rows, defs, w[b + X_SEG],
+                               (const float*)dqw, (const float*)dqr, (float*)dqs, (float*)dq, (float*)deft);
           DS_CHECK_LAUNCH();
         }
       }

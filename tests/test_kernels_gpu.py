@@ -135,6 +135,22 @@ def test_gemm_batched_head_views(dt):
     assert_close(scores, q @ k.transpose(-1, -2), 1e-5, "scores")
 
 
+@pytest.mark.parametrize("B,N,Q,K", [(1, 16, 512, 896), (2, 3, 64, 192), (1, 1, 128, 64)])
+def test_gemm_head_scores_fp32_out(B, N, Q, K):
+    # bf16, both operands K-major, reduction of exactly 64, fp32 output: the per-head score products (own kernel)
+    D = 64
+    H = N * D
+    r = rng(Q + K + N)
+    q = dev(r.standard_normal((Q, B, H)), torch.bfloat16)           # [i][b][n*D], as the XLNet stage holds q
+    kv = dev(r.standard_normal((K, B, 2 * H)), torch.bfloat16)      # [j][b][k | v]
+    out = torch.full((B, N, Q, K), float("nan"), dtype=torch.float32, device="cuda")
+    ops.gemm(q, kv, out, Q, K, D, DS_K_MAJOR, DS_K_MAJOR, lda=B * H, ldb=B * 2 * H, ldc=K, flags=DS_EPI_OUT_F32, alpha=0.25,
+             batch=B * N, batch_inner=N, a_strides=(H, D), b_strides=(2 * H, D), c_strides=(N * Q * K, Q * K))
+    qh = q.cpu().double().reshape(Q, B, N, D).permute(1, 2, 0, 3)
+    kh = kv[:, :, :H].cpu().double().reshape(K, B, N, D).permute(1, 2, 0, 3)
+    assert_close(out, 0.25 * (qh @ kh.transpose(-1, -2)), 1e-5, "head scores")
+
+
 @pytest.mark.parametrize("dt", ["fp32", "bf16"])
 @pytest.mark.parametrize("rows,cols", [(7, 64), (256, 1024), (33, 512), (5, 2048)])
 def test_layernorm_fwd_bwd(dt, rows, cols):
