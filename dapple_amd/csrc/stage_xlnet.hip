@@ -141,7 +141,7 @@ __global__ __launch_bounds__(256) void xl_softmax_bwd_kernel(int Q, int QQ, int 
   T* out = ds + w * K;
   T* brow = dbd + w * R;
   const int shift = Q - i;  // column j of ds lands in column j + Q - i of dbd
-  float d0 = 0.f, d1 = 0.f;
+  float d0 = 0.f, d1 = 0.f, n1 = 0.f;
 #pragma unroll
   for (int v = 0; v < NV; ++v) {
     const int c = (lane + v * 64) * 4;
@@ -152,7 +152,7 @@ __global__ __launch_bounds__(256) void xl_softmax_bwd_kernel(int Q, int QQ, int 
         out[c + e] = val;
         brow[c + e + shift] = val;
         const float f = to_f32(val);
-        if (seg_mat && seg_mat[((int64_t)i * K + c + e) * B + b]) d1 += f; else d0 += f;
+        if (seg_mat && seg_mat[((int64_t)i * K + c + e) * B + b]) { d1 += f; n1 += 1.f; } else d0 += f;
       }
     }
   }
@@ -160,6 +160,13 @@ __global__ __launch_bounds__(256) void xl_softmax_bwd_kernel(int Q, int QQ, int 
   for (int r = shift + K + lane; r < R; r += 64) brow[r] = from_f32<T>(0.f);
   d0 = wave_sum(d0);
   d1 = wave_sum(d1);
+  n1 = wave_sum(n1);
+  // A softmax row's score gradients sum to zero, so def[0] + def[1] = 0; what the rounded probabilities and the
+  // rounded ds leave of that sum is noise, and it would be multiplied by a whole embedding row.  It is taken out of
+  // the two sums in proportion to the number of keys each one covers.
+  const float excess = (d0 + d1) / (float)K;
+  d0 -= excess * ((float)K - n1);
+  d1 -= excess * n1;
   if (lane == 0) { defs[w * 2] = d0; defs[w * 2 + 1] = d1; }
 }
 

@@ -68,7 +68,18 @@ def run_case(dtype, L, H, N, F, B, Q, Mm, S, M, K=2, seed=0, use_seg=True, mask_
         floor = None
         if not use_seg and n_.endswith(("bias_segment", "seg_emb")):
             floor = acc[n_.rsplit("/", 1)[0] + "/bias_context"].abs().max().item()
-        assert_close(stage.grads[n_], acc[n_].reshape(stage.grads[n_].shape), tol, "accumulated grad " + n_, floor=floor)
+        want = acc[n_].reshape(stage.grads[n_].shape)
+        if use_seg and n_.endswith("bias_segment") and dtype == "bf16":
+            # Each row's two segment-score gradients cancel (a softmax row's score gradients sum to zero), so this
+            # gradient is a small difference - 10 to 40 times below the two sibling biases added to the same q - and
+            # carries the rounding of the bf16 probabilities at their scale, not its own: judged on a tenth of
+            # bias_context's scale where its own maximum is smaller than that.
+            sib = 0.1 * acc[n_.rsplit("/", 1)[0] + "/bias_context"].abs().max().item()
+            if want.abs().max().item() < sib:
+                err = (stage.grads[n_].double().cpu() - want).abs().max().item() / sib
+                assert err <= tol, "accumulated grad %s: %.3e of a tenth of the bias_context scale > tol %.1e" % (n_, err, tol)
+                continue
+        assert_close(stage.grads[n_], want, tol, "accumulated grad " + n_, floor=floor)
     stage.close()
 
 
