@@ -11,6 +11,7 @@
 // Activations are sequence-major rows (stream, i, b) of width H.  Scores are never shifted in memory:
 // the position term is computed unshifted as (q + r_r) k_r^T [qlen, rlen] and the softmax kernel reads
 // column j + qlen - i of it (rel_shift as index arithmetic); backward scatters with the same map.
+#include <stdlib.h>
 #include <string.h>
 
 #include "stage.h"
@@ -197,6 +198,15 @@ __global__ __launch_bounds__(256) void xl_seg_bwd_kernel(int QQ, int B, int N, i
   }
 }
 
+// out[b][j][i] = in[i][j][b]: the key-major copies of the masks / the segment matrix that the fused attention reads
+template <typename T>
+__global__ __launch_bounds__(256) void xl_key_major_kernel(int I, int K, int B, const T* __restrict__ in, T* __restrict__ out) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)I * K * B) return;
+  const int i = (int)(idx % I), j = (int)((idx / I) % K), b = (int)(idx / ((int64_t)I * K));
+  out[idx] = in[((int64_t)i * K + j) * B + b];
+}
+
 struct LayerOff { size_t x, qw, qr, qs, kv, p, vec, z1, y1, u, hh, z2, st1, st2; };
 
 struct XlnetStage : ds_stage {
@@ -210,7 +220,8 @@ struct XlnetStage : ds_stage {
   char* pe = nullptr;
   // stash
   char* stash_base = nullptr;
-  size_t slot_bytes = 0, mask_off = 0, seg_off = 0, mem_off = 0;
+  size_t slot_bytes = 0, mask_off = 0, seg_off = 0, mem_off = 0, maskt_off = 0, segt_off = 0;
+  bool fused_fwd = false;  // forward attention in one kernel (bf16, head size 64, seq a multiple of 64)
   std::vector<LayerOff> lo;
   std::vector<char> has_mask, has_seg;
   // workspace
@@ -269,6 +280,11 @@ struct XlnetStage : ds_stage {
     mask_off = sa.reserve((size_t)S * Q * K * B * 4);
     seg_off = sa.reserve((size_t)Q * K * B);
     mem_off = sa.reserve((size_t)L * (Mm > 0 ? Mm : 1) * B * H * esz);
+    fused_fwd = xc.fused_attention != 0 && ds_xl_attention_fits(dtype, D, Q, K, R);
+    if (fused_fwd) {
+      maskt_off = sa.reserve((size_t)B * K * S * Q * 4);
+      segt_off = sa.reserve((size_t)B * K * Q);
+    }
     lo.resize(L);
     size_t next_x = sa.reserve(act);
     for (int l = 0; l < L; ++l) {
@@ -380,6 +396,19 @@ struct XlnetStage : ds_stage {
     }
     has_mask[slot] = masks != nullptr;
     has_seg[slot] = seg_mat != nullptr;
+    if (fused_fwd) {
+      if (masks) {
+        const int64_t n = (int64_t)S * Q * K * B;
+        hipLaunchKernelGGL(xl_key_major_kernel<float>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, S * Q, K, B,
+                           (const float*)(sp + mask_off), (float*)(sp + maskt_off));
+      }
+      if (seg_mat) {
+        const int64_t n = (int64_t)Q * K * B;
+        hipLaunchKernelGGL(xl_key_major_kernel<uint8_t>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, Q, K, B,
+                           (const uint8_t*)(sp + seg_off), (uint8_t*)(sp + segt_off));
+      }
+      DS_CHECK_LAUNCH();
+    }
     return DS_OK;
   }
 
@@ -444,7 +473,18 @@ struct XlnetStage : ds_stage {
                              w[b + X_RR], w[b + X_RS], (float*)(sp + t.qw), (float*)(sp + t.qr), (float*)(sp + t.qs));
         DS_CHECK_LAUNCH();
       }
-      {
+      if (fused_fwd) {
+        XlAttnArgs xa;
+        xa.qw = sp + t.qw; xa.qr = sp + t.qr; xa.qs = sp + t.qs; xa.ldq = (int64_t)B * H;
+        xa.kv = sp + t.kv; xa.ldkv = (int64_t)B * 2 * H;
+        xa.kr = kr[l]; xa.ldkr = H;
+        xa.seg_emb = w[b + X_SEG];
+        xa.mask_t = has_mask[slot] ? (const float*)(sp + maskt_off) : nullptr;
+        xa.seg_t = has_seg[slot] ? (const uint8_t*)(sp + segt_off) : nullptr;
+        xa.p = sp + t.p; xa.vec = sp + t.vec;
+        xa.Q = Q; xa.QQ = S * Q; xa.K = K; xa.R = R; xa.B = B; xa.N = N; xa.H = H; xa.scale = scale;
+        DS_PROPAGATE(ds_xl_attention_fwd(&xa, stream));
+      } else {
         // The streams' query rows are stacked in the q buffers ([stream][i][b] = row stream*Q + i of stride B*H): every
         // product below and the softmax run once over all QQ = S*Q rows; probabilities are stashed as [B*N][QQ][K].
         const int QQ = S * Q;

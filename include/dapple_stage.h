@@ -313,7 +313,10 @@ typedef struct ds_xlnet_cfg {
   float ln_eps;     /* 1e-14 = K.epsilon()**2 (layer_normalization.py:37-39) */
   int first_layer;  /* names only */
   int stash_slots;
-  int reserved[8];
+  int fused_attention; /* 1: forward attention in one kernel where the shape allows (bf16, head size 64, seq a multiple of
+                          64, mem_len + seq a multiple of 32); 0 (default): products and softmax as separate launches,
+                          which is the faster step at the benchmark shape today.  Results agree to rounding. */
+  int reserved[7];
 } ds_xlnet_cfg;
 int ds_xlnet_stage_create(const ds_xlnet_cfg* cfg, void* stream, ds_stage** out);
 /* Side inputs of the micro-batch that will be forwarded into `slot` (copied into the slot):
