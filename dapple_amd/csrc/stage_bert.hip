@@ -122,7 +122,9 @@ struct BertStage : ds_stage {
   int next_pos = 0;
   long n_backward = 0;
   std::vector<Deferred> deferred;
-  hipEvent_t ev_chain = nullptr, ev_wg_done = nullptr;
+  hipEvent_t ev_chain = nullptr, ev_wg_done = nullptr, ev_refresh = nullptr;
+  std::vector<hipEvent_t> ev_cast;   // compute copies of layer l written (refresh_weights on the weight-gradient stream)
+  std::vector<char> cast_pending;
   std::vector<hipEvent_t> ev_x_bwd, ev_x_wg, ev_dy_wg;
   std::vector<char> x_bwd_valid, x_wg_valid, dy_wg_valid;
   bool wg_outstanding = false;
@@ -141,6 +143,8 @@ struct BertStage : ds_stage {
     if (dy_base) (void)hipFree(dy_base);
     if (ev_chain) (void)hipEventDestroy(ev_chain);
     if (ev_wg_done) (void)hipEventDestroy(ev_wg_done);
+    if (ev_refresh) (void)hipEventDestroy(ev_refresh);
+    for (hipEvent_t e : ev_cast) (void)hipEventDestroy(e);
     for (hipEvent_t e : ev_x_bwd) (void)hipEventDestroy(e);
     for (hipEvent_t e : ev_x_wg) (void)hipEventDestroy(e);
     for (hipEvent_t e : ev_dy_wg) (void)hipEventDestroy(e);
@@ -307,21 +311,50 @@ struct BertStage : ds_stage {
     return w[base(l) + which];
   }
 
+  // The compute copies of layer l are only needed when the next forward pass reaches layer l.  With a weight-gradient
+  // stream at hand (idle between steps) the copies of layers 1.. are made there, one event per layer, and the first
+  // forward pass after the refresh waits for each layer's event as it gets to it: the pass starts after one layer's
+  // casts instead of after all of them.
   int refresh_weights() override {
+    hipStream_t side = wgrad_stream;
+    if (side) {
+      if (ev_cast.empty()) {
+        ev_cast.resize(L);
+        for (int l = 0; l < L; ++l) DS_CHECK_HIP(hipEventCreateWithFlags(&ev_cast[l], hipEventDisableTiming));
+        DS_CHECK_HIP(hipEventCreateWithFlags(&ev_refresh, hipEventDisableTiming));
+      }
+      // everything queued before this call (the master weights' last update among it) precedes the casts
+      DS_CHECK_HIP(hipEventRecord(ev_refresh, stream));
+      DS_CHECK_HIP(hipStreamWaitEvent(side, ev_refresh, 0));
+    }
+    cast_pending.assign(L, 0);
     for (int l = 0; l < L; ++l) {
       const int b = base(l);
+      hipStream_t cs = (side && l > 0) ? side : stream;
       if (dtype == DS_BF16) {
-        hipLaunchKernelGGL(pack_qkv_kernel<bf16>, dim3(1024), dim3(256), 0, stream, H, w[b + W_Q], w[b + W_K], w[b + W_V],
+        hipLaunchKernelGGL(pack_qkv_kernel<bf16>, dim3(1024), dim3(256), 0, cs, H, w[b + W_Q], w[b + W_K], w[b + W_V],
                            w[b + B_Q], w[b + B_K], w[b + B_V], (bf16*)wqkv[l], bqkv[l]);
         DS_CHECK_LAUNCH();
-        DS_PROPAGATE(ds_cast_f32_to_bf16(wo[l], w[b + W_AO], (size_t)H * H, stream));
-        DS_PROPAGATE(ds_cast_f32_to_bf16(w1[l], w[b + W_FF1], (size_t)H * F, stream));
-        DS_PROPAGATE(ds_cast_f32_to_bf16(w2[l], w[b + W_FF2], (size_t)F * H, stream));
+        DS_PROPAGATE(ds_cast_f32_to_bf16(wo[l], w[b + W_AO], (size_t)H * H, cs));
+        DS_PROPAGATE(ds_cast_f32_to_bf16(w1[l], w[b + W_FF1], (size_t)H * F, cs));
+        DS_PROPAGATE(ds_cast_f32_to_bf16(w2[l], w[b + W_FF2], (size_t)F * H, cs));
       } else {
-        hipLaunchKernelGGL(pack_qkv_kernel<float>, dim3(1024), dim3(256), 0, stream, H, w[b + W_Q], w[b + W_K], w[b + W_V],
+        hipLaunchKernelGGL(pack_qkv_kernel<float>, dim3(1024), dim3(256), 0, cs, H, w[b + W_Q], w[b + W_K], w[b + W_V],
                            w[b + B_Q], w[b + B_K], w[b + B_V], (float*)wqkv[l], bqkv[l]);
         DS_CHECK_LAUNCH();
       }
+      if (cs != stream) {
+        DS_CHECK_HIP(hipEventRecord(ev_cast[l], cs));
+        cast_pending[l] = 1;
+      }
+    }
+    return DS_OK;
+  }
+  // called by whatever reads layer l's compute copies first on `s`
+  int await_cast(int l, hipStream_t s) {
+    if (!cast_pending.empty() && cast_pending[l]) {
+      DS_CHECK_HIP(hipStreamWaitEvent(s, ev_cast[l], 0));
+      cast_pending[l] = 0;
     }
     return DS_OK;
   }
@@ -425,6 +458,7 @@ struct BertStage : ds_stage {
       const int b = base(l);
       char* x = at(t.x, pos);
       char* y = (l + 1 < L) ? at(ls[l + 1].x, pos) : (char*)out;
+      DS_PROPAGATE(await_cast(l, stream));
       // fused Q|K|V projection (modeling_slice.py:464-485)
       DS_PROPAGATE(gemm_fwd(rows, 3 * H, H, x, wqkv[l], at(t.qkv, pos), DS_EPI_BIAS, bqkv[l], nullptr, nullptr));
       if (fused_attn) {
