@@ -230,8 +230,13 @@ struct XlnetStage : ds_stage {
   size_t ws_bytes = 0, ws_qall, ws_ac, ws_dp, ws_bd, ws_ds, ws_dbd, ws_def, ws_dz2[2], ws_du[2], ws_dy1, ws_dz1[2], ws_dvec, ws_dqw[2], ws_dqr[2],
          ws_dqs[2], ws_dq[2], ws_dkv[2], ws_dkr[2], ws_deft[2], ws_dx[2];
   WgradLane lane;
+  hipEvent_t ev_refresh = nullptr;
+  std::vector<hipEvent_t> ev_cast;   // layer l's compute copies written (refresh_weights on the weight-gradient stream)
+  std::vector<char> cast_pending;
 
   ~XlnetStage() override {
+    if (ev_refresh) (void)hipEventDestroy(ev_refresh);
+    for (hipEvent_t e : ev_cast) (void)hipEventDestroy(e);
     if (wc_base) (void)hipFree(wc_base);
     if (stash_base) (void)hipFree(stash_base);
     if (ws_base) (void)hipFree(ws_base);
@@ -362,26 +367,58 @@ struct XlnetStage : ds_stage {
   }
   static int g1(int64_t n) { int64_t b = (n + 255) / 256; return (int)(b > 8192 ? 8192 : (b < 1 ? 1 : b)); }
 
+  // Layer l's compute copies (and its k_r) are only needed when the next forward pass reaches layer l: with a
+  // weight-gradient stream at hand those of layers 1.. are made there, one event per layer, and the first forward
+  // pass after the refresh waits for each layer's event as it gets to it.
   int refresh_weights() override {
     if (dtype == DS_BF16) hipLaunchKernelGGL(xl_pos_emb_kernel<bf16>, dim3(g1((int64_t)R * H / 2)), dim3(256), 0, stream, R, H, K, (bf16*)pe);
     else hipLaunchKernelGGL(xl_pos_emb_kernel<float>, dim3(g1((int64_t)R * H / 2)), dim3(256), 0, stream, R, H, K, (float*)pe);
     DS_CHECK_LAUNCH();
-    for (int l = 0; l < L; ++l) {
-      const int b = base(l);
-      if (dtype == DS_BF16) {
-        hipLaunchKernelGGL(xl_pack_kv_kernel<bf16>, dim3(1024), dim3(256), 0, stream, H, w[b + X_K], w[b + X_V], (bf16*)wkv[l]);
-        DS_CHECK_LAUNCH();
-        DS_PROPAGATE(ds_cast_f32_to_bf16(wq[l], w[b + X_Q], (size_t)H * H, stream));
-        DS_PROPAGATE(ds_cast_f32_to_bf16(wr[l], w[b + X_R], (size_t)H * H, stream));
-        DS_PROPAGATE(ds_cast_f32_to_bf16(wo[l], w[b + X_O], (size_t)H * H, stream));
-        DS_PROPAGATE(ds_cast_f32_to_bf16(w1[l], w[b + X_W1], (size_t)H * F, stream));
-        DS_PROPAGATE(ds_cast_f32_to_bf16(w2[l], w[b + X_W2], (size_t)F * H, stream));
-      } else {
-        hipLaunchKernelGGL(xl_pack_kv_kernel<float>, dim3(1024), dim3(256), 0, stream, H, w[b + X_K], w[b + X_V], (float*)wkv[l]);
-        DS_CHECK_LAUNCH();
+    hipStream_t side = wgrad_stream;
+    if (side) {
+      if (ev_cast.empty()) {
+        ev_cast.resize(L);
+        for (int l = 0; l < L; ++l) DS_CHECK_HIP(hipEventCreateWithFlags(&ev_cast[l], hipEventDisableTiming));
+        DS_CHECK_HIP(hipEventCreateWithFlags(&ev_refresh, hipEventDisableTiming));
       }
-      // k_r = pos_emb @ Wr does not depend on the micro-batch: once per refresh
-      DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, R, H, H, pe, H, WT(l, X_R), H, kr[l], H));
+      // everything queued before this call (the master weights' last update, the position table) precedes the copies
+      DS_CHECK_HIP(hipEventRecord(ev_refresh, stream));
+      DS_CHECK_HIP(hipStreamWaitEvent(side, ev_refresh, 0));
+    }
+    cast_pending.assign(L, 0);
+    hipStream_t main_stream = stream;
+    int rc = DS_OK;
+    for (int l = 0; l < L && rc == DS_OK; ++l) {
+      const int b = base(l);
+      hipStream_t cs = (side && l > 0) ? side : main_stream;
+      stream = cs;  // gemm() launches on `stream`
+      do {
+        if (dtype == DS_BF16) {
+          hipLaunchKernelGGL(xl_pack_kv_kernel<bf16>, dim3(1024), dim3(256), 0, cs, H, w[b + X_K], w[b + X_V], (bf16*)wkv[l]);
+          if ((rc = ds_cast_f32_to_bf16(wq[l], w[b + X_Q], (size_t)H * H, cs)) != DS_OK) break;
+          if ((rc = ds_cast_f32_to_bf16(wr[l], w[b + X_R], (size_t)H * H, cs)) != DS_OK) break;
+          if ((rc = ds_cast_f32_to_bf16(wo[l], w[b + X_O], (size_t)H * H, cs)) != DS_OK) break;
+          if ((rc = ds_cast_f32_to_bf16(w1[l], w[b + X_W1], (size_t)H * F, cs)) != DS_OK) break;
+          if ((rc = ds_cast_f32_to_bf16(w2[l], w[b + X_W2], (size_t)F * H, cs)) != DS_OK) break;
+        } else {
+          hipLaunchKernelGGL(xl_pack_kv_kernel<float>, dim3(1024), dim3(256), 0, cs, H, w[b + X_K], w[b + X_V], (float*)wkv[l]);
+        }
+        // k_r = pos_emb @ Wr does not depend on the micro-batch: once per refresh
+        rc = gemm(DS_K_MAJOR, DS_MN_MAJOR, R, H, H, pe, H, WT(l, X_R), H, kr[l], H);
+      } while (0);
+      stream = main_stream;
+      if (rc == DS_OK && cs != main_stream) {
+        if (hipEventRecord(ev_cast[l], cs) != hipSuccess) { ds_set_error("ds_stage_refresh_weights: hipEventRecord failed"); rc = DS_EHIP; }
+        cast_pending[l] = 1;
+      }
+    }
+    if (rc == DS_OK) DS_CHECK_LAUNCH();
+    return rc;
+  }
+  int await_cast(int l, hipStream_t s) {
+    if (!cast_pending.empty() && cast_pending[l]) {
+      DS_CHECK_HIP(hipStreamWaitEvent(s, ev_cast[l], 0));
+      cast_pending[l] = 0;
     }
     return DS_OK;
   }
@@ -458,6 +495,7 @@ struct XlnetStage : ds_stage {
       const int b = base(l);
       char* x = sp + t.x;
       char* y = (l + 1 < L) ? sp + lo[l + 1].x : (char*)out;
+      DS_PROPAGATE(await_cast(l, stream));
       // q for every stream row; k|v for memory rows and for the content-stream rows
       DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, rows, H, H, x, H, WT(l, X_Q), H, qall, H));
       if (Mm > 0)
