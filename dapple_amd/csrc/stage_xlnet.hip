@@ -227,7 +227,7 @@ struct XlnetStage : ds_stage {
   // workspace
   char* ws_base = nullptr;
   // buffers the weight-gradient kernels read alternate by layer parity ([2])
-  size_t ws_bytes = 0, ws_qall, ws_ac, ws_dp, ws_bd, ws_ds, ws_dbd, ws_def, ws_dz2[2], ws_du[2], ws_dy1, ws_dz1[2], ws_dvec, ws_dqw[2], ws_dqr[2],
+  size_t ws_bytes = 0, ws_qall, ws_ac, ws_dp, ws_bd, ws_ds, ws_dbd[2], ws_def, ws_dz2[2], ws_du[2], ws_dy1, ws_dz1[2], ws_dvec, ws_dqw[2], ws_dqr[2],
          ws_dqs[2], ws_dq[2], ws_dkv[2], ws_dkr[2], ws_deft[2], ws_dx[2];
   WgradLane lane;
   hipEvent_t ev_refresh = nullptr;
@@ -316,7 +316,8 @@ struct XlnetStage : ds_stage {
     ws_dp = w.reserve((size_t)B * N * QQ * K * 4);  // backward's own score-gradient buffer: forward keeps ws_ac
     ws_bd = w.reserve((size_t)B * N * QQ * R * 4);
     ws_ds = w.reserve((size_t)B * N * QQ * K * esz);
-    ws_dbd = w.reserve((size_t)B * N * QQ * R * esz);
+    ws_dbd[0] = w.reserve((size_t)B * N * QQ * R * esz);  // read by the weight-gradient stream too (dkr): one per layer parity
+    ws_dbd[1] = w.reserve((size_t)B * N * QQ * R * esz);
     ws_def = w.reserve((size_t)B * N * QQ * 2 * 4);
     ws_dy1 = w.reserve(act); ws_dvec = w.reserve(act);
     for (int p = 0; p < 2; ++p) {
@@ -559,7 +560,7 @@ struct XlnetStage : ds_stage {
     const char* dy = (const char*)d_out;
     char* dy1 = ws_base + ws_dy1; char* dvec = ws_base + ws_dvec;
     float* dp = (float*)(ws_base + ws_dp);
-    char* dsm = ws_base + ws_ds; char* dbd = ws_base + ws_dbd;
+    char* dsm = ws_base + ws_ds;
     // with a weight-gradient stream, a layer's weight gradients run beside the dgrad chain of the layers below
     hipStream_t wgs = wgrad_stream;
     if (wgs) DS_PROPAGATE(lane.ensure());
@@ -570,7 +571,7 @@ struct XlnetStage : ds_stage {
       char* dz2 = ws_base + ws_dz2[par]; char* du = ws_base + ws_du[par]; char* dz1 = ws_base + ws_dz1[par];
       char* dqw = ws_base + ws_dqw[par]; char* dqr = ws_base + ws_dqr[par]; char* dqs = ws_base + ws_dqs[par];
       char* dq = ws_base + ws_dq[par]; char* dkv = ws_base + ws_dkv[par]; char* dkr = ws_base + ws_dkr[par];
-      char* deft = ws_base + ws_deft[par];
+      char* deft = ws_base + ws_deft[par]; char* dbd = ws_base + ws_dbd[par];
       if (wgs) DS_PROPAGATE(lane.reuse(stream, par));
       char* x = sp + t.x;
       DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, dy, sp + t.z2, w[b + X_LN2_G], (const float*)(sp + t.st2), nullptr, dz2,
@@ -603,11 +604,7 @@ struct XlnetStage : ds_stage {
         // position term through the shift
         DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_MN_MAJOR, QQ, D, R, dbd, R, (int64_t)N * QQ * R, (int64_t)QQ * R, kr[l], H, 0, D,
                              dqr, (int64_t)B * H, H, D, 0));
-        for (int bb = 0; bb < B; ++bb) {  // k_r is shared by the batch: one launch per batch entry, added in place
-          const int a2 = bb > 0 ? DS_EPI_RESIDUAL : 0;
-          DS_PROPAGATE(gemm_bn(DS_MN_MAJOR, DS_MN_MAJOR, R, D, QQ, dbd + (size_t)bb * N * QQ * R * esz, R, 0, (int64_t)QQ * R,
-                               sp + t.qr + (size_t)bb * H * esz, (int64_t)B * H, 0, D, dkr, H, 0, D, a2, dkr, 1));
-        }
+        // (dk_r = dbd^T qr feeds only Wr's gradient: it runs with the weight gradients below)
         // segment term + dq = dqw + dqr + dqs
         {
           const int64_t waves = (int64_t)B * N * QQ;
@@ -651,6 +648,12 @@ struct XlnetStage : ds_stage {
         }
         // projections
         if ((rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, rows, x, H, dq, H, g[b + X_Q], H, DS_EPI_ACCUM)) != DS_OK) break;
+        for (int bb = 0; bb < B && rc == DS_OK; ++bb) {  // k_r is shared by the batch: one launch per batch entry, added in place
+          const int a2 = bb > 0 ? DS_EPI_RESIDUAL : 0;
+          rc = gemm_bn(DS_MN_MAJOR, DS_MN_MAJOR, R, D, S * Q, dbd + (size_t)bb * N * S * Q * R * esz, R, 0, (int64_t)S * Q * R,
+                       sp + t.qr + (size_t)bb * H * esz, (int64_t)B * H, 0, D, dkr, H, 0, D, a2, dkr, 1);
+        }
+        if (rc != DS_OK) break;
         if ((rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, R, pe, H, dkr, H, g[b + X_R], H, DS_EPI_ACCUM)) != DS_OK) break;
         for (int j = 0; j < 2 && rc == DS_OK; ++j) {  // j = 0: k, 1: v
           float* gw = g[b + X_K + j];
