@@ -113,7 +113,8 @@ __global__ __launch_bounds__(256) void xl_softmax_fwd_kernel(int Q, int QQ, int 
 
 // Softmax backward of one score row (b, n, i) per wave, with everything else that needs the row while it is in
 // registers: ds[j] = scale * p[j] * (dp[j] - sum_k p[k] dp[k]);
-//   dbd[i][r] = ds[i][r - Q + i] when that column exists, else 0 (transpose of the rel_shift index map);
+//   dbd[i][r] = ds[i][r - Q + i] when that column exists (transpose of the rel_shift index map; the other columns of
+//   dbd hold zeros from the start and are never touched);
 //   def[s] = sum_j [seg(i,j,b) == s] ds[i][j] (gradient of the two segment scores of the row).
 template <typename T, int NV>
 __global__ __launch_bounds__(256) void xl_softmax_bwd_kernel(int Q, int QQ, int K, int R, int B, int N, const T* __restrict__ p,
@@ -157,8 +158,8 @@ __global__ __launch_bounds__(256) void xl_softmax_bwd_kernel(int Q, int QQ, int 
       }
     }
   }
-  for (int r = lane; r < shift; r += 64) brow[r] = from_f32<T>(0.f);
-  for (int r = shift + K + lane; r < R; r += 64) brow[r] = from_f32<T>(0.f);
+  // (columns [0, shift) and [shift + K, R) of the row are zero and stay zero: the band's position depends on i alone,
+  // the buffer is cleared when the stage is created and nothing else is ever written outside the band)
   d0 = wave_sum(d0);
   d1 = wave_sum(d1);
   n1 = wave_sum(n1);
@@ -330,6 +331,10 @@ struct XlnetStage : ds_stage {
     ws_dx[0] = w.reserve(act); ws_dx[1] = w.reserve(act);
     ws_bytes = w.used;
     DS_CHECK_HIP(hipMalloc((void**)&ws_base, ws_bytes));
+    // the un-shifted score gradients: zero outside the band the softmax backward kernel writes
+    // (queued on the stage's stream, ahead of every pass; creation is not something a caller captures in a graph)
+    DS_CHECK_HIP(hipMemsetAsync(ws_base + ws_dbd[0], 0, (size_t)B * N * QQ * R * esz, stream));
+    DS_CHECK_HIP(hipMemsetAsync(ws_base + ws_dbd[1], 0, (size_t)B * N * QQ * R * esz, stream));
     return DS_OK;
   }
 
