@@ -93,6 +93,7 @@ PROTOTYPES = {
                                    C.c_void_p, C.c_void_p, C.c_void_p]),
     "ds_layernorm_bwd": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                    C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "ds_layernorm_param_grads": (C.c_int, [C.c_int, C.c_int, C.c_int] + [C.c_void_p] * 8),
     "ds_softmax_fwd": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_float, C.c_void_p,
                                  C.c_float, C.c_void_p, C.c_void_p]),
     "ds_softmax_bwd": (C.c_int, [C.c_int, C.c_int64, C.c_int, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p,

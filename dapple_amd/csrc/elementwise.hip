@@ -213,6 +213,113 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(int rows, int cols, 
   }
 }
 
+// Backward without the parameter gradients: one wave per row, dx only.  For callers that take d_gamma / d_beta (and the
+// column sums of dx) from layernorm_param_grad_kernel on another stream, off the chain of dependent kernels.
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void layernorm_bwd_rows_kernel(int rows, int cols, const T* __restrict__ dy, const T* __restrict__ x,
+                                                                const float* __restrict__ gamma, const float* __restrict__ stats,
+                                                                const T* __restrict__ dx_add, T* __restrict__ dx) {
+  constexpr int VEC = Vec16<T>::N;
+  typedef typename Vec16<T>::type V;
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const float mean = stats[2 * row], rstd = stats[2 * row + 1];
+  const T* dyr = dy + (int64_t)row * cols;
+  const T* xr = x + (int64_t)row * cols;
+  float dg[NV][VEC], xh[NV][VEC];
+  float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = (lane + i * 64) * VEC;
+    if (c < cols) {
+      const V a = *reinterpret_cast<const V*>(dyr + c);
+      const V b = *reinterpret_cast<const V*>(xr + c);
+#pragma unroll
+      for (int e = 0; e < VEC; e += 4) {
+        const f32x4 gv = *reinterpret_cast<const f32x4*>(gamma + c + e);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          xh[i][e + k] = (to_f32(b[e + k]) - mean) * rstd;
+          dg[i][e + k] = to_f32(a[e + k]) * gv[k];
+          s1 += dg[i][e + k];
+          s2 += dg[i][e + k] * xh[i][e + k];
+        }
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) { dg[i][e] = 0.f; xh[i][e] = 0.f; }
+    }
+  }
+  s1 = wave_sum(s1) / cols;
+  s2 = wave_sum(s2) / cols;
+  T* dxr = dx + (int64_t)row * cols;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = (lane + i * 64) * VEC;
+    if (c < cols) {
+      V o;
+      V add = {};
+      if (dx_add) add = *reinterpret_cast<const V*>(dx_add + (int64_t)row * cols + c);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) o[e] = from_f32<T>(rstd * (dg[i][e] - s1 - xh[i][e] * s2) + (dx_add ? to_f32(add[e]) : 0.f));
+      *reinterpret_cast<V*>(dxr + c) = o;
+    }
+  }
+}
+
+// d_gamma[c] += sum_rows dy x_hat, d_beta[c] += sum_rows dy, d_colsum[c] += sum_rows dx (dx nullable).  A block owns a
+// strip of 64 16-byte vectors and a chunk of rows; its 4 waves take every 4th row and meet in LDS.
+template <typename T>
+__global__ __launch_bounds__(256) void layernorm_param_grad_kernel(int rows, int cols, int rows_per_block, const T* __restrict__ dy,
+                                                                  const T* __restrict__ x, const float* __restrict__ stats,
+                                                                  const T* __restrict__ dx, float* __restrict__ d_gamma,
+                                                                  float* __restrict__ d_beta, float* __restrict__ d_colsum) {
+  constexpr int VEC = Vec16<T>::N;
+  typedef typename Vec16<T>::type V;
+  __shared__ float red[3][4][64 * VEC];
+  const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
+  const int c = (blockIdx.x * 64 + lane) * VEC;
+  const int r0 = blockIdx.y * rows_per_block;
+  int r1 = r0 + rows_per_block;
+  if (r1 > rows) r1 = rows;
+  float pg[VEC], pb[VEC], ps[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) pg[e] = pb[e] = ps[e] = 0.f;
+  if (c < cols)
+    for (int r = r0 + g; r < r1; r += 4) {
+      const float mean = stats[2 * r], rstd = stats[2 * r + 1];
+      const V a = *reinterpret_cast<const V*>(dy + (int64_t)r * cols + c);
+      const V b = *reinterpret_cast<const V*>(x + (int64_t)r * cols + c);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        const float d = to_f32(a[e]);
+        pg[e] += d * (to_f32(b[e]) - mean) * rstd;
+        pb[e] += d;
+      }
+      if (dx) {
+        const V v = *reinterpret_cast<const V*>(dx + (int64_t)r * cols + c);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) ps[e] += to_f32(v[e]);
+      }
+    }
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+    red[0][g][lane * VEC + e] = pg[e];
+    red[1][g][lane * VEC + e] = pb[e];
+    red[2][g][lane * VEC + e] = ps[e];
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < 64 * VEC; i += 256) {
+    const int p = blockIdx.x * 64 * VEC + i;
+    if (p < cols) {
+      atomicAdd(d_gamma + p, red[0][0][i] + red[0][1][i] + red[0][2][i] + red[0][3][i]);
+      atomicAdd(d_beta + p, red[1][0][i] + red[1][1][i] + red[1][2][i] + red[1][3][i]);
+      if (d_colsum) atomicAdd(d_colsum + p, red[2][0][i] + red[2][1][i] + red[2][2][i] + red[2][3][i]);
+    }
+  }
+}
+
 // ------------------------------------------------------------------ softmax
 // One wave per row of fp32 scores; NV 16-byte vectors (4 floats) per lane.
 template <typename T, int NV>
@@ -435,13 +542,55 @@ static int layernorm_bwd_t(int rows, int cols, const void* dy, const void* x, co
   return DS_OK;
 }
 
+template <typename T>
+static int layernorm_bwd_rows_t(int rows, int cols, const void* dy, const void* x, const float* gamma, const float* stats,
+                                const void* dx_add, void* dx, hipStream_t s) {
+  const int need = (cols / Vec16<T>::N + 63) / 64;
+  dim3 grid((rows + 3) / 4);
+  ds_prof_scope prof(s, sizeof(T) == 2 ? "layernorm_bwd_rows_kernel<bf16>" : "layernorm_bwd_rows_kernel<float>",
+                     (double)rows * cols * sizeof(T) * (dx_add ? 4 : 3), "B");
+  DISPATCH_NV(T, need, hipLaunchKernelGGL((layernorm_bwd_rows_kernel<T, NV>), grid, dim3(256), 0, s, rows, cols, (const T*)dy,
+                                          (const T*)x, gamma, stats, (const T*)dx_add, (T*)dx));
+  DS_CHECK_LAUNCH();
+  return DS_OK;
+}
+
+extern "C" int ds_layernorm_param_grads(int dtype, int rows, int cols, const void* dy, const void* x, const float* stats,
+                                        const void* dx, float* d_gamma, float* d_beta, float* d_colsum, void* stream) {
+  DS_CHECK_ARG(dtype == DS_F32 || dtype == DS_BF16, "ds_layernorm_param_grads: dtype %d", dtype);
+  const int vec = dtype == DS_BF16 ? 8 : 4;
+  DS_CHECK_ARG(rows > 0 && cols > 0 && cols % vec == 0, "ds_layernorm_param_grads: rows %d, cols %d (multiple of %d)", rows, cols, vec);
+  DS_CHECK_ARG(dy && x && stats && d_gamma && d_beta && (!d_colsum || dx), "ds_layernorm_param_grads: null pointer (d_colsum needs dx)");
+  DS_CHECK_ARG(ds_aligned16(dy) && ds_aligned16(x) && ds_aligned16(dx), "ds_layernorm_param_grads: tensors must be 16-byte aligned");
+  const int strips = (cols + 64 * vec - 1) / (64 * vec);
+  int rpb = 8;  // every block ends in one atomic add per column and quantity: keep the row chunks in the hundreds
+  while ((int64_t)strips * ((rows + rpb - 1) / rpb) > 512) rpb *= 2;
+  dim3 grid(strips, (rows + rpb - 1) / rpb);
+  hipStream_t s = (hipStream_t)stream;
+  ds_prof_scope prof(s, dtype == DS_BF16 ? "layernorm_param_grad_kernel<bf16>" : "layernorm_param_grad_kernel<float>",
+                     (double)rows * cols * (dtype == DS_BF16 ? 2 : 4) * (d_colsum ? 3 : 2), "B");
+  if (dtype == DS_BF16)
+    hipLaunchKernelGGL(layernorm_param_grad_kernel<bf16>, grid, dim3(256), 0, s, rows, cols, rpb, (const bf16*)dy, (const bf16*)x, stats,
+                       d_colsum ? (const bf16*)dx : nullptr, d_gamma, d_beta, d_colsum);
+  else
+    hipLaunchKernelGGL(layernorm_param_grad_kernel<float>, grid, dim3(256), 0, s, rows, cols, rpb, (const float*)dy, (const float*)x, stats,
+                       d_colsum ? (const float*)dx : nullptr, d_gamma, d_beta, d_colsum);
+  DS_CHECK_LAUNCH();
+  return DS_OK;
+}
+
 extern "C" int ds_layernorm_bwd(int dtype, int rows, int cols, const void* dy, const void* x, const float* gamma,
                                 const float* stats, const void* dx_add, void* dx, float* d_gamma, float* d_beta,
                                 float* d_colsum, void* stream) {
   DS_PROPAGATE(check_rows("ds_layernorm_bwd", dtype, rows, cols));
-  DS_CHECK_ARG(dy && x && gamma && stats && dx && d_gamma && d_beta, "ds_layernorm_bwd: null pointer");
   DS_CHECK_ARG(ds_aligned16(dy) && ds_aligned16(x) && ds_aligned16(dx) && ds_aligned16(dx_add) && ds_aligned16(gamma),
                "ds_layernorm_bwd: tensors must be 16-byte aligned");
+  if (!d_gamma && !d_beta) {  // dx only: the parameter gradients come from ds_layernorm_param_grads
+    DS_CHECK_ARG(dy && x && gamma && stats && dx && !d_colsum, "ds_layernorm_bwd: null pointer (or d_colsum without d_gamma / d_beta)");
+    if (dtype == DS_BF16) return layernorm_bwd_rows_t<bf16>(rows, cols, dy, x, gamma, stats, dx_add, dx, (hipStream_t)stream);
+    return layernorm_bwd_rows_t<float>(rows, cols, dy, x, gamma, stats, dx_add, dx, (hipStream_t)stream);
+  }
+  DS_CHECK_ARG(dy && x && gamma && stats && dx && d_gamma && d_beta, "ds_layernorm_bwd: null pointer");
   if (dtype == DS_BF16)
     return layernorm_bwd_t<bf16>(rows, cols, dy, x, gamma, stats, dx_add, dx, d_gamma, d_beta, d_colsum, (hipStream_t)stream);
   return layernorm_bwd_t<float>(rows, cols, dy, x, gamma, stats, dx_add, dx, d_gamma, d_beta, d_colsum, (hipStream_t)stream);

@@ -113,6 +113,15 @@ def layernorm_bwd(dy, x, gamma, stats, d_gamma, d_beta, d_colsum=None, dx_add=No
     return dx
 
 
+def layernorm_param_grads(dy, x, stats, d_gamma, d_beta, dx=None, d_colsum=None):
+    """d_gamma += sum_rows dy * x_hat, d_beta += sum_rows dy, d_colsum += sum_rows dx: the half of the LayerNorm backward
+    pass that ``layernorm_bwd(..., d_gamma=None, d_beta=None)`` leaves out."""
+    _need_cuda(dy, x, stats, d_gamma, d_beta, dx, d_colsum)
+    rows, cols = x.shape
+    check(_lib.load().ds_layernorm_param_grads(dtype_code(x), rows, cols, ptr(dy), ptr(x), ptr(stats), ptr(dx), ptr(d_gamma),
+                                               ptr(d_beta), ptr(d_colsum), _lib.current_stream()), "ds_layernorm_param_grads")
+
+
 def softmax_fwd(scores, scale, key_mask=None, mask_value=-10000.0, out_dtype=torch.float32):
     """scores fp32 [B, N, Q, K] -> probabilities of out_dtype."""
     _need_cuda(scores, key_mask)

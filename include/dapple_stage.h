@@ -111,6 +111,12 @@ int ds_layernorm_fwd(int dtype, int rows, int cols, const void* x, const float* 
 int ds_layernorm_bwd(int dtype, int rows, int cols, const void* dy, const void* x,
                      const float* gamma, const float* stats, const void* dx_add, void* dx,
                      float* d_gamma, float* d_beta, float* d_colsum, void* stream);
+/* The same backward pass split in two, for callers that keep the parameter gradients off their chain of dependent
+ * kernels: ds_layernorm_bwd with d_gamma = d_beta = d_colsum = NULL writes dx only (one wave per row, no atomics), and
+ * ds_layernorm_param_grads adds d_gamma += sum_rows dy * x_hat, d_beta += sum_rows dy and, when d_colsum is given,
+ * d_colsum += sum_rows dx (dx: the first call's output) - on whatever stream it is given. */
+int ds_layernorm_param_grads(int dtype, int rows, int cols, const void* dy, const void* x, const float* stats,
+                             const void* dx, float* d_gamma, float* d_beta, float* d_colsum, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Softmax over the last axis of fp32 scores [batch*heads*q, k]:

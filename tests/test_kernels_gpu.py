@@ -176,6 +176,17 @@ def test_layernorm_fwd_bwd(dt, rows, cols):
     assert_close(dg, dg_ref + 1, 1e-4, "ln dgamma (accumulates)")
     assert_close(db, db_ref + 1, 1e-4, "ln dbeta")
     assert_close(dcs, dx_ref.sum(0) + 1, 1e-4 if dt == "fp32" else 1e-2, "ln colsum")
+    # the same pass in two calls: dx alone, then the parameter gradients (and the column sums of that dx)
+    dx2 = ops.layernorm_bwd(dy, x, g, stats, None, None, None, dx_add=None)
+    assert_close(dx2, dx_ref, tol, "ln dx (rows only)")
+    dg2, db2, dcs2 = torch.ones(cols, device="cuda"), torch.ones(cols, device="cuda"), torch.ones(cols, device="cuda")
+    ops.layernorm_param_grads(dy, x, stats, dg2, db2, dx=dx2, d_colsum=dcs2)
+    assert_close(dg2, dg_ref + 1, 1e-4, "ln dgamma (separate call)")
+    assert_close(db2, db_ref + 1, 1e-4, "ln dbeta (separate call)")
+    assert_close(dcs2, dx2.double().cpu().sum(0) + 1, 1e-4, "ln colsum (separate call)")
+    dg3, db3 = torch.zeros(cols, device="cuda"), torch.zeros(cols, device="cuda")
+    ops.layernorm_param_grads(dy, x, stats, dg3, db3)
+    assert_close(dg3, dg_ref, 1e-4, "ln dgamma (no colsum)")
 
 
 @pytest.mark.parametrize("dt", ["fp32", "bf16"])
