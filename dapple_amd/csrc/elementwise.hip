@@ -406,12 +406,16 @@ __global__ __launch_bounds__(256) void softmax_bwd_kernel(int64_t rows, int k, c
 // rows of its group; groups combine through LDS, then one atomicAdd per column.  A matrix narrower than the 64
 // vectors of a wave is read `fold` rows at a time (contiguous rows form one super row of cols * fold elements), so
 // that all lanes have work; the fold copies of a column meet in the final atomic adds.
+struct ColsumBatch { const void* x[4]; float* out[4]; };  // matrices of one shape summed by one launch (blockIdx.z)
+
 template <typename T>
-__global__ __launch_bounds__(256) void colsum_kernel(int rows, int cols, const T* __restrict__ x, int64_t ldx,
-                                                    int rows_per_block, int fold, float* __restrict__ out) {
+__global__ __launch_bounds__(256) void colsum_kernel(int rows, int cols, ColsumBatch cb, int64_t ldx,
+                                                    int rows_per_block, int fold) {
   constexpr int VEC = Vec16<T>::N;
   typedef typename Vec16<T>::type V;
   __shared__ float red[4][64 * VEC];
+  const T* __restrict__ x = reinterpret_cast<const T*>(cb.x[blockIdx.z]);
+  float* __restrict__ out = cb.out[blockIdx.z];
   const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
   const int c = (blockIdx.x * 64 + lane) * VEC;  // position inside the super row
   const int sub = c / cols, cc = c - sub * cols;
@@ -642,10 +646,22 @@ extern "C" int ds_softmax_bwd(int dtype, int64_t rows, int k, const void* p, con
   return softmax_bwd_t<float>(rows, k, p, dp, scale, ds, (hipStream_t)stream);
 }
 
+int ds_colsum_accum_multi(int dtype, int rows, int cols, int count, const void* const* xs, int64_t ldx, float* const* outs, void* stream);
+
 extern "C" int ds_colsum_accum(int dtype, int rows, int cols, const void* x, int64_t ldx, float* out, void* stream) {
+  return ds_colsum_accum_multi(dtype, rows, cols, 1, &x, ldx, &out, stream);
+}
+
+int ds_colsum_accum_multi(int dtype, int rows, int cols, int count, const void* const* xs, int64_t ldx, float* const* outs, void* stream) {
   DS_CHECK_ARG(dtype == DS_F32 || dtype == DS_BF16, "ds_colsum_accum: dtype %d", dtype);
-  DS_CHECK_ARG(rows > 0 && cols > 0 && ldx >= cols && x && out, "ds_colsum_accum: bad argument");
+  DS_CHECK_ARG(rows > 0 && cols > 0 && ldx >= cols && count >= 1 && count <= 4, "ds_colsum_accum: bad argument");
   const int vec = dtype == DS_BF16 ? 8 : 4;
+  ColsumBatch cb = {};
+  for (int i = 0; i < count; ++i) {
+    DS_CHECK_ARG(xs[i] && outs[i] && ds_aligned16(xs[i]), "ds_colsum_accum: null or unaligned pointer");
+    cb.x[i] = xs[i]; cb.out[i] = outs[i];
+  }
+  const void* x = xs[0];
   DS_CHECK_ARG(cols % vec == 0 && ldx % vec == 0 && ds_aligned16(x), "ds_colsum_accum: cols and ldx must be multiples of %d and x 16-byte aligned", vec);
   // every block ends in one atomic add per column: keep the number of row chunks in the low thousands
   int fold = 1;
@@ -654,13 +670,13 @@ extern "C" int ds_colsum_accum(int dtype, int rows, int cols, const void* x, int
   int rpb = 32;
   const int strips = (cols * fold + 64 * vec - 1) / (64 * vec);
   while ((int64_t)strips * ((nsr + rpb - 1) / rpb) > 2048 && rpb < (1 << 20)) rpb *= 2;
-  dim3 grid(strips, (nsr + rpb - 1) / rpb);
+  dim3 grid(strips, (nsr + rpb - 1) / rpb, count);
   ds_prof_scope prof((hipStream_t)stream, dtype == DS_BF16 ? "colsum_kernel<bf16>" : "colsum_kernel<float>",
-                     (double)rows * cols * (dtype == DS_BF16 ? 2 : 4), "B");
+                     (double)rows * cols * (dtype == DS_BF16 ? 2 : 4) * count, "B");
   if (dtype == DS_BF16)
-    hipLaunchKernelGGL(colsum_kernel<bf16>, grid, dim3(256), 0, (hipStream_t)stream, rows, cols, (const bf16*)x, ldx, rpb, fold, out);
+    hipLaunchKernelGGL(colsum_kernel<bf16>, grid, dim3(256), 0, (hipStream_t)stream, rows, cols, cb, ldx, rpb, fold);
   else
-    hipLaunchKernelGGL(colsum_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, rows, cols, (const float*)x, ldx, rpb, fold, out);
+    hipLaunchKernelGGL(colsum_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, rows, cols, cb, ldx, rpb, fold);
   DS_CHECK_LAUNCH();
   return DS_OK;
 }

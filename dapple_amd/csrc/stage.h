@@ -131,3 +131,5 @@ struct XlAttnArgs {
 bool ds_xl_attention_fits(int dtype, int head_dim, int Q, int K, int R);
 int ds_xl_attention_fwd(const XlAttnArgs* a, hipStream_t stream);
 int ds_gemm_splitk(const ds_gemm_desc* d, int splitk, void* stream);
+// ds_colsum_accum for up to 4 matrices of one shape in one launch
+int ds_colsum_accum_multi(int dtype, int rows, int cols, int count, const void* const* xs, int64_t ldx, float* const* outs, void* stream);

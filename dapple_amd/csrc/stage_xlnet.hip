@@ -638,9 +638,11 @@ struct XlnetStage : ds_stage {
         if ((rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, F, rows, sp + t.y1, H, du, F, g[b + X_W1], F, DS_EPI_ACCUM)) != DS_OK) break;
         if ((rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, rows, dz1, H, sp + t.vec, H, g[b + X_O], H, DS_EPI_ACCUM)) != DS_OK) break;
         // relative biases: column sums of the three query-gradient pieces
-        if ((rc = ds_colsum_accum(dtype, rows, H, dqw, H, g[b + X_RW], stream)) != DS_OK) break;
-        if ((rc = ds_colsum_accum(dtype, rows, H, dqr, H, g[b + X_RR], stream)) != DS_OK) break;
-        if ((rc = ds_colsum_accum(dtype, rows, H, dqs, H, g[b + X_RS], stream)) != DS_OK) break;
+        {
+          const void* const xs3[3] = {dqw, dqr, dqs};
+          float* const out3[3] = {g[b + X_RW], g[b + X_RR], g[b + X_RS]};
+          if ((rc = ds_colsum_accum_multi(dtype, rows, H, 3, xs3, H, out3, stream)) != DS_OK) break;
+        }
         // seg_emb[s][n][:] += sum_rows def[row][n][s] * qs[row][n][:]   (batched over heads)
         {
           ds_gemm_desc d;
@@ -660,12 +662,28 @@ struct XlnetStage : ds_stage {
         }
         if (rc != DS_OK) break;
         if ((rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, R, pe, H, dkr, H, g[b + X_R], H, DS_EPI_ACCUM)) != DS_OK) break;
-        for (int j = 0; j < 2 && rc == DS_OK; ++j) {  // j = 0: k, 1: v
-          float* gw = g[b + X_K + j];
-          if (Mm > 0)
-            rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, Mm * B, sp + mem_off + (size_t)l * Mm * B * H * esz, H, dkv + (size_t)j * H * esz,
-                      2 * H, gw, H, DS_EPI_ACCUM);
-          if (rc == DS_OK) rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, rowsS, x, H, dkv_h + (size_t)j * H * esz, 2 * H, gw, H, DS_EPI_ACCUM);
+        // Wk and Wv: the two column halves of dkv against the same rows, one batched launch (z = 0: k, 1: v) when the two
+        // master gradients sit one behind the other with no gap
+        if (g[b + X_V] == g[b + X_K] + (size_t)H * H) {
+          ds_gemm_desc d;
+          memset(&d, 0, sizeof(d));
+          d.dtype = dtype; d.a_major = DS_MN_MAJOR; d.b_major = DS_MN_MAJOR; d.m = H; d.n = H; d.lda = H; d.ldb = 2 * H; d.ldc = H;
+          d.batch = 2; d.batch_inner = 2; d.b_stride_inner = H; d.c_stride_inner = (int64_t)H * H;
+          d.flags = DS_EPI_ACCUM; d.alpha = 1.f; d.c = g[b + X_K];
+          if (Mm > 0) {
+            d.k = Mm * B; d.a = sp + mem_off + (size_t)l * Mm * B * H * esz; d.b = dkv;
+            if ((rc = ds_gemm(&d, stream)) != DS_OK) break;
+          }
+          d.k = rowsS; d.a = x; d.b = dkv_h;
+          if ((rc = ds_gemm(&d, stream)) != DS_OK) break;
+        } else {
+          for (int j = 0; j < 2 && rc == DS_OK; ++j) {  // j = 0: k, 1: v
+            float* gw = g[b + X_K + j];
+            if (Mm > 0)
+              rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, Mm * B, sp + mem_off + (size_t)l * Mm * B * H * esz, H, dkv + (size_t)j * H * esz,
+                        2 * H, gw, H, DS_EPI_ACCUM);
+            if (rc == DS_OK) rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, rowsS, x, H, dkv_h + (size_t)j * H * esz, 2 * H, gw, H, DS_EPI_ACCUM);
+          }
         }
       } while (0);
       stream = chain;
