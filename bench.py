@@ -164,7 +164,8 @@ def make_xlnet(c, args):
                                   c["streams"], c["num_micro_batches"])
     adt = torch.bfloat16 if c["dtype"] == "bf16" else torch.float32
     K = runtime.stash_depth(0, 2)
-    stage = runtime.xlnet_stage(L, H, N, F, B, Q, c["dtype"], stash_slots=K, mem_len=Mm, streams=S)
+    stage = runtime.xlnet_stage(L, H, N, F, B, Q, c["dtype"], stash_slots=K, mem_len=Mm, streams=S,
+                                fused_attention=args.xlnet_fused_attention)
     stage.bind(synthetic.xlnet_weights(synthetic.SEED_WEIGHT + c["index"], L, H, N, F))
     xs = [torch.as_tensor(np.stack(x)).cuda().to(adt) for x in synthetic.xlnet_stream_inputs(synthetic.SEED_INPUT + c["index"], M, Q, B, H, S)]
     dys = [torch.as_tensor(np.stack(x)).cuda().to(adt) for x in synthetic.xlnet_stream_inputs(synthetic.SEED_GRAD + c["index"], M, Q, B, H, S)]
@@ -227,6 +228,8 @@ def main():
     ap.add_argument("--no-overlap", action="store_true", help="keep forward and backward passes on one stream")
     ap.add_argument("--wgrad-group", type=int, default=4,
                     help="BERT stages: weight gradients of this many backward passes in one GEMM per weight")
+    ap.add_argument("--xlnet-fused-attention", action="store_true",
+                    help="XLNet stages: forward attention as one kernel (ds_xlnet_cfg.fused_attention)")
     ap.add_argument("--micro-batch", type=int, default=None,
                     help="samples per micro-batch instead of the configuration's (a what-if: the headline is the default)")
     ap.add_argument("--micro-batches", type=int, default=None, help="micro-batches per step instead of the configuration's")
