@@ -117,6 +117,33 @@ __global__ __launch_bounds__(256) void mask_steps_kernel(int64_t total4, int B, 
   }
 }
 
+// fp32 GEMM helpers shared by the three stage kinds of this file
+static int gnmt_gemm(hipStream_t stream, int am, int bm, int m, int n, int k, const void* a, int64_t lda, const void* b, int64_t ldb, void* c,
+                     int64_t ldc, int flags, const float* bias, const void* residual) {
+  ds_gemm_desc d;
+  memset(&d, 0, sizeof(d));
+  d.dtype = DS_F32; d.a_major = am; d.b_major = bm; d.m = m; d.n = n; d.k = k; d.lda = lda; d.ldb = ldb; d.ldc = ldc;
+  d.batch = 1; d.batch_inner = 1; d.flags = flags; d.alpha = 1.f; d.a = a; d.b = b; d.c = c; d.bias = bias; d.residual = residual;
+  return ds_gemm(&d, stream);
+}
+// reduction split of a product with few rows (the per-step recurrent products have only B of them)
+static int gnmt_split_for(int m, int n, int k) {
+  const int tiles = ((m + 63) / 64) * ((n + 63) / 64);
+  int s = 256 / (tiles > 0 ? tiles : 1);
+  const int ktiles = k / 32;
+  if (s > ktiles / 4) s = ktiles / 4;
+  return s < 1 ? 1 : s;
+}
+// c (fp32) += a[m,k] x b: the reduction is split across the chip and added with fp32 atomics
+static int gnmt_gemm_accum_splitk(hipStream_t stream, int bm, int m, int n, int k, const void* a, int64_t lda, const void* b, int64_t ldb,
+                                  float* c, int64_t ldc) {
+  ds_gemm_desc d;
+  memset(&d, 0, sizeof(d));
+  d.dtype = DS_F32; d.a_major = DS_K_MAJOR; d.b_major = bm; d.m = m; d.n = n; d.k = k; d.lda = lda; d.ldb = ldb; d.ldc = ldc;
+  d.batch = 1; d.batch_inner = 1; d.flags = DS_EPI_ACCUM; d.alpha = 1.f; d.a = a; d.b = b; d.c = c;
+  return ds_gemm_splitk(&d, gnmt_split_for(m, n, k), stream);
+}
+
 struct Cell {
   int widx;        // kernel index in the weight list (bias = widx + 1)
   int n_in;        // input width
@@ -213,28 +240,10 @@ struct GnmtStage : ds_stage {
 
   int gemm(int am, int bm, int m, int n, int k, const void* a, int64_t lda, const void* b, int64_t ldb, void* c, int64_t ldc,
            int flags, const float* bias, const void* residual) {
-    ds_gemm_desc d;
-    memset(&d, 0, sizeof(d));
-    d.dtype = DS_F32; d.a_major = am; d.b_major = bm; d.m = m; d.n = n; d.k = k; d.lda = lda; d.ldb = ldb; d.ldc = ldc;
-    d.batch = 1; d.batch_inner = 1; d.flags = flags; d.alpha = 1.f; d.a = a; d.b = b; d.c = c; d.bias = bias; d.residual = residual;
-    return ds_gemm(&d, stream);
+    return gnmt_gemm(stream, am, bm, m, n, k, a, lda, b, ldb, c, ldc, flags, bias, residual);
   }
-  // c (fp32) += a[m,k] x b: the per-step recurrent products have only B rows, so the reduction is
-  // split across the chip and added with fp32 atomics
-  int gemm_accum_splitk(int bm, int m, int n, int k, const void* a, int64_t lda, const void* b, int64_t ldb, float* c,
-                        int64_t ldc, int splitk) {
-    ds_gemm_desc d;
-    memset(&d, 0, sizeof(d));
-    d.dtype = DS_F32; d.a_major = DS_K_MAJOR; d.b_major = bm; d.m = m; d.n = n; d.k = k; d.lda = lda; d.ldb = ldb; d.ldc = ldc;
-    d.batch = 1; d.batch_inner = 1; d.flags = DS_EPI_ACCUM; d.alpha = 1.f; d.a = a; d.b = b; d.c = c;
-    return ds_gemm_splitk(&d, splitk, stream);
-  }
-  static int split_for(int m, int n, int k) {
-    const int tiles = ((m + 63) / 64) * ((n + 63) / 64);
-    int s = 256 / (tiles > 0 ? tiles : 1);
-    const int ktiles = k / 32;
-    if (s > ktiles / 4) s = ktiles / 4;
-    return s < 1 ? 1 : s;
+  int gemm_accum_splitk(int bm, int m, int n, int k, const void* a, int64_t lda, const void* b, int64_t ldb, float* c, int64_t ldc) {
+    return gnmt_gemm_accum_splitk(stream, bm, m, n, k, a, lda, b, ldb, c, ldc);
   }
 
   int set_lengths(int slot, const int32_t* lengths) {
@@ -272,8 +281,7 @@ struct GnmtStage : ds_stage {
         float* g = G + (size_t)t * B * 4 * U;
         if (s > 0) {
           // recurrent half, added in place: g += h[tp] @ Wh
-          DS_PROPAGATE(gemm_accum_splitk(DS_MN_MAJOR, B, 4 * U, U, H + (size_t)tp * B * c.ldh, c.ldh, wh, 4 * U, g, 4 * U,
-                                         split_for(B, 4 * U, U)));
+          DS_PROPAGATE(gemm_accum_splitk(DS_MN_MAJOR, B, 4 * U, U, H + (size_t)tp * B * c.ldh, c.ldh, wh, 4 * U, g, 4 * U));
         }
         ds_prof_scope prof(stream, "lstm_cell_fwd_kernel", (double)B * U * 4 * (4 + 4 + 2 + (c.residual ? 2 : 1)), "B");
         hipLaunchKernelGGL(lstm_cell_fwd_kernel, dim3(cell_grid), dim3(256), 0, stream, B, U, gc.forget_bias, g,
@@ -333,8 +341,7 @@ struct GnmtStage : ds_stage {
           DS_CHECK_LAUNCH();
         }
         if (s > 0) {  // dh for step tp: dgates[t] @ Wh^T
-          DS_PROPAGATE(gemm_accum_splitk(DS_K_MAJOR, B, U, 4 * U, dG + (size_t)t * B * 4 * U, 4 * U, wh, 4 * U, dh_out, U,
-                                         split_for(B, U, 4 * U)));
+          DS_PROPAGATE(gemm_accum_splitk(DS_K_MAJOR, B, U, 4 * U, dG + (size_t)t * B * 4 * U, 4 * U, wh, 4 * U, dh_out, U));
         }
       }
       // parameter gradients over all steps
@@ -440,18 +447,10 @@ struct GnmtDecoderStage : ds_stage {
 
   int gemm(int am, int bm, int m, int n, int k, const void* a, int64_t lda, const void* b, int64_t ldb, void* c, int64_t ldc,
            int flags, const float* bias, const void* residual) {
-    ds_gemm_desc d;
-    memset(&d, 0, sizeof(d));
-    d.dtype = DS_F32; d.a_major = am; d.b_major = bm; d.m = m; d.n = n; d.k = k; d.lda = lda; d.ldb = ldb; d.ldc = ldc;
-    d.batch = 1; d.batch_inner = 1; d.flags = flags; d.alpha = 1.f; d.a = a; d.b = b; d.c = c; d.bias = bias; d.residual = residual;
-    return ds_gemm(&d, stream);
+    return gnmt_gemm(stream, am, bm, m, n, k, a, lda, b, ldb, c, ldc, flags, bias, residual);
   }
   int gemm_accum_splitk(int bm, int m, int n, int k, const void* a, int64_t lda, const void* b, int64_t ldb, float* c, int64_t ldc) {
-    ds_gemm_desc d;
-    memset(&d, 0, sizeof(d));
-    d.dtype = DS_F32; d.a_major = DS_K_MAJOR; d.b_major = bm; d.m = m; d.n = n; d.k = k; d.lda = lda; d.ldb = ldb; d.ldc = ldc;
-    d.batch = 1; d.batch_inner = 1; d.flags = DS_EPI_ACCUM; d.alpha = 1.f; d.a = a; d.b = b; d.c = c;
-    return ds_gemm_splitk(&d, GnmtStage::split_for(m, n, k), stream);
+    return gnmt_gemm_accum_splitk(stream, bm, m, n, k, a, lda, b, ldb, c, ldc);
   }
 
   int set_attention(int slot, const float* attention) {
@@ -781,18 +780,10 @@ struct GnmtAttentionStage : ds_stage {
 
   int gemm(int am, int bm, int m, int n, int k, const void* a, int64_t lda, const void* b, int64_t ldb, void* c, int64_t ldc,
            int flags, const float* bias, const void* residual) {
-    ds_gemm_desc d;
-    memset(&d, 0, sizeof(d));
-    d.dtype = DS_F32; d.a_major = am; d.b_major = bm; d.m = m; d.n = n; d.k = k; d.lda = lda; d.ldb = ldb; d.ldc = ldc;
-    d.batch = 1; d.batch_inner = 1; d.flags = flags; d.alpha = 1.f; d.a = a; d.b = b; d.c = c; d.bias = bias; d.residual = residual;
-    return ds_gemm(&d, stream);
+    return gnmt_gemm(stream, am, bm, m, n, k, a, lda, b, ldb, c, ldc, flags, bias, residual);
   }
   int gemm_accum_splitk(int bm, int m, int n, int k, const void* a, int64_t lda, const void* b, int64_t ldb, float* c, int64_t ldc) {
-    ds_gemm_desc d;
-    memset(&d, 0, sizeof(d));
-    d.dtype = DS_F32; d.a_major = DS_K_MAJOR; d.b_major = bm; d.m = m; d.n = n; d.k = k; d.lda = lda; d.ldb = ldb; d.ldc = ldc;
-    d.batch = 1; d.batch_inner = 1; d.flags = DS_EPI_ACCUM; d.alpha = 1.f; d.a = a; d.b = b; d.c = c;
-    return ds_gemm_splitk(&d, GnmtStage::split_for(m, n, k), stream);
+    return gnmt_gemm_accum_splitk(stream, bm, m, n, k, a, lda, b, ldb, c, ldc);
   }
   int fill0(float* p, int64_t n) {
     const int64_t blocks = (n + 255) / 256;
