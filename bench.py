@@ -156,6 +156,96 @@ def make_gnmt(c, args):
     return wl
 
 
+def make_gnmt_attention(c, args):
+    """Decoder cell 0 under the attention wrapper (device 0, behind the encoder): memory in, cell outputs out."""
+    import numpy as np
+    import torch
+    from dapple_amd import runtime, synthetic
+    U, V, B, T, S, M = c["units"], c["vocab"], c["micro_batch"], c["seq"], c["src_seq"], c["num_micro_batches"]
+    K = runtime.stash_depth(0, 2)
+    stage = runtime.gnmt_attention_stage(U, V, B, T, S, stash_slots=K, forget_bias=c["forget_bias"])
+    stage.bind(synthetic.gnmt_attention_weights(synthetic.SEED_WEIGHT + c["index"], U, V))
+    r = np.random.Generator(np.random.PCG64(synthetic.SEED_INPUT + c["index"]))
+    mems = [torch.as_tensor(r.standard_normal((S, B, U)).astype(np.float32)).cuda() for _ in range(M)]
+    ids = [torch.as_tensor(x).cuda() for x in synthetic.gnmt_id_inputs(synthetic.SEED_INPUT + c["index"], M, B, T, V)]
+    lens = [torch.as_tensor(r.integers(S // 2, S + 1, B).astype(np.int32)).cuda() for _ in range(M)]
+    dys = [torch.as_tensor(x).cuda() for x in synthetic.upstream_grads(synthetic.SEED_GRAD + c["index"], M, (T, B, U))]
+    outs = [torch.empty(T, B, U, device="cuda") for _ in range(M)]
+    dmems = [torch.empty(S, B, U, device="cuda") for _ in range(M)]
+    rt = runtime.StageRuntime(stage, 0, 2, M)
+    wl = Workload()
+    wl.stage = stage
+    wl.step = lambda: (stage.refresh_weights(), stage.zero_grads(),
+                       rt.step(mems, dys, outs, dmems, before_forward=lambda slot, j: stage.set_decoder_inputs(slot, ids[j], lens[j])))
+    wl.samples = B * M
+    # per target step: cell (3U x 4U), query layer (U x U), scores and context over the source (2 S U); once: keys (S U U)
+    wl.flops_per_sample = 3 * (T * 2 * (3 * U * 4 * U + U * U + 2 * S * U) + 2 * S * U * U)
+    wl.config = {"units": U, "vocab": V, "seq": T, "src_seq": S, "micro_batch": B, "micro_batches": M,
+                 "schedule": "1F1B stage 0 of 2, stash K=%d" % K}
+
+    def cpu():
+        from oracle import gnmt as og
+        nb = 16
+        w = {k: torch.tensor(v, dtype=torch.float32) for k, v in synthetic.gnmt_attention_weights(synthetic.SEED_WEIGHT + c["index"], U, V).items()}
+        w[og.ATT_G] = w[og.ATT_G].reshape(())
+        w = {k: v.requires_grad_(True) for k, v in w.items()}
+        mem = mems[0][:, :nb].cpu().contiguous().requires_grad_(True)
+        t0 = time.perf_counter()
+        out, _ = og.attention_cell_forward(ids[0][:nb].cpu(), mem, lens[0][:nb].cpu(), w, c["forget_bias"])
+        torch.autograd.grad(out, [mem] + list(w.values()), grad_outputs=dys[0][:, :nb].cpu().contiguous(), allow_unused=True)
+        dt = time.perf_counter() - t0
+        return dt, nb, "%d of %d sequences of one micro-batch, fwd+BPTT" % (nb, B)
+    wl.cpu = cpu
+    return wl
+
+
+def make_gnmt_decoder(c, args):
+    """Decoder cells 1.. + output projection + loss (device 1, the last stage: K = 1, every forward is followed by its loss
+    and its backward pass)."""
+    import numpy as np
+    import torch
+    from dapple_amd import ops, runtime, synthetic
+    L, F0, U, V, B, T, M = c["num_layers"], c["first_layer"], c["units"], c["vocab"], c["micro_batch"], c["seq"], c["num_micro_batches"]
+    stage = runtime.gnmt_decoder_stage(L, U, B, T, stash_slots=1, first_layer=F0, forget_bias=c["forget_bias"])
+    stage.bind(synthetic.gnmt_decoder_weights(synthetic.SEED_WEIGHT + c["index"], F0, L, U))
+    r = np.random.Generator(np.random.PCG64(synthetic.SEED_INPUT + c["index"]))
+    xs = [torch.as_tensor(r.standard_normal((T, B, U)).astype(np.float32)).cuda() for _ in range(M)]
+    proj = torch.as_tensor(r.uniform(-0.1, 0.1, (U, V)).astype(np.float32)).cuda()
+    dproj = torch.zeros_like(proj)
+    tgt = [torch.as_tensor(x).cuda() for x in synthetic.gnmt_id_inputs(synthetic.SEED_GRAD + c["index"], M, B, T, V)]
+    lens = [torch.as_tensor(r.integers(T // 2, T + 1, B).astype(np.int32)).cuda() for _ in range(M)]
+    y = torch.empty(T, B, U, device="cuda")
+    dxs = [torch.empty(T, B, U, device="cuda") for _ in range(M)]
+
+    def step():
+        stage.refresh_weights(); stage.zero_grads(); dproj.zero_()
+        for j in range(M):
+            stage.forward(0, xs[j], y)
+            _, dy = ops.nmt_loss_head(y, proj, tgt[j], lens[j], d_proj_kernel=dproj)
+            stage.backward(0, dy, dxs[j])
+    wl = Workload()
+    wl.stage = stage
+    wl.step = step
+    wl.samples = B * M
+    wl.flops_per_sample = 3 * T * (L * 2 * 3 * U * 4 * U + 2 * U * V)
+    wl.config = {"layers": L, "first_layer": F0, "units": U, "vocab": V, "seq": T, "micro_batch": B, "micro_batches": M,
+                 "schedule": "last stage (K=1): forward, projection + loss, backward per micro-batch"}
+
+    def cpu():
+        from oracle import gnmt as og
+        nb = 8
+        w = og.to_torch(synthetic.gnmt_decoder_weights(synthetic.SEED_WEIGHT + c["index"], F0, L, U), torch.float32, requires_grad=True)
+        k = proj.cpu().requires_grad_(True)
+        x = xs[0][:, :nb].cpu().contiguous().requires_grad_(True)
+        t0 = time.perf_counter()
+        loss, _ = og.nmt_loss(og.decoder_part2_forward(x, None, w, F0, L, c["forget_bias"]), k, tgt[0][:nb].cpu(), lens[0][:nb].cpu())
+        torch.autograd.grad(loss, [x, k] + list(w.values()))
+        dt = time.perf_counter() - t0
+        return dt, nb, "%d of %d sequences of one micro-batch, fwd+BPTT through all %d cells, projection and loss" % (nb, B, L)
+    wl.cpu = cpu
+    return wl
+
+
 def make_xlnet(c, args):
     import numpy as np
     import torch
@@ -214,7 +304,8 @@ TRAFFIC = {
     "gemm_dma_kernel<bf16,64,64,K,MN>": 52.6e6,      # ffn2 forward shape
 }
 
-MAKERS = {"bert": make_bert, "vgg": make_vgg, "gnmt": make_gnmt, "xlnet": make_xlnet}
+MAKERS = {"bert": make_bert, "vgg": make_vgg, "gnmt": make_gnmt, "xlnet": make_xlnet, "gnmt_attention": make_gnmt_attention,
+          "gnmt_decoder": make_gnmt_decoder}
 METRIC = {"bert48_half": "stage samples/sec fwd+bwd+grad-accum, BERT-48 half-stage; MFMA util %"}
 
 

@@ -578,33 +578,42 @@ __global__ __launch_bounds__(256) void att_prep_kernel(int B, int S, int U, cons
 
 constexpr int ATT_MAX_S = 512;
 
-// one block per sample b: scores over the source steps, softmax, context
-__global__ __launch_bounds__(256) void att_fwd_kernel(int S, int U, const float* __restrict__ keys, const float* __restrict__ values,
-                                                     const float* __restrict__ pq, const float* __restrict__ nv,
-                                                     const float* __restrict__ bias, const int32_t* __restrict__ len,
-                                                     float* __restrict__ align, float* __restrict__ ctx, int ldc) {
+// One wave per (sample b, source step j): score[b][j] = sum_u nv[u] tanh(keys[b,j,u] + pq[b,u] + bias[u]) (raw, unmasked;
+// steps past the source length are skipped: the next kernel never reads them)
+__global__ __launch_bounds__(256) void att_score_kernel(int B, int S, int U, const float* __restrict__ keys, const float* __restrict__ pq,
+                                                       const float* __restrict__ nv, const float* __restrict__ bias,
+                                                       const int32_t* __restrict__ len, float* __restrict__ score) {
+  const int lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= B * S) return;
+  const int b = row / S, j = row % S;
+  if (len && j >= len[b]) return;
+  const float* k = keys + (int64_t)row * U;
+  float a = 0.f;
+  for (int u = lane * 4; u < U; u += 256) {
+    const f32x4 kv = *reinterpret_cast<const f32x4*>(k + u);
+    const f32x4 qv = *reinterpret_cast<const f32x4*>(pq + (int64_t)b * U + u);
+    const f32x4 bv = *reinterpret_cast<const f32x4*>(bias + u);
+    const f32x4 vv = *reinterpret_cast<const f32x4*>(nv + u);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) a += vv[e] * tanhf(kv[e] + qv[e] + bv[e]);
+  }
+  a = wave_sum(a);
+  if (lane == 0) score[row] = a;
+}
+
+// grid (ceil(U/256), B): softmax of sample b's raw scores over its valid source steps (every block of the sample repeats
+// it: at most a few hundred values; the sample's first block writes the alignments, zero past the source length), then
+// the context for the block's 256 units
+__global__ __launch_bounds__(256) void att_context_kernel(int S, int U, const float* __restrict__ score, const float* __restrict__ values,
+                                                         const int32_t* __restrict__ len, float* __restrict__ align,
+                                                         float* __restrict__ ctx, int ldc) {
   __shared__ float sc[ATT_MAX_S];
   __shared__ float red[4];
-  const int b = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int b = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int n = len ? len[b] : S;
   n = n < 0 ? 0 : (n > S ? S : n);
-  for (int j = wave; j < n; j += 4) {
-    const float* k = keys + ((int64_t)b * S + j) * U;
-    float a = 0.f;
-    for (int u = lane * 4; u < U; u += 256) {
-      const f32x4 kv = *reinterpret_cast<const f32x4*>(k + u);
-      const f32x4 qv = *reinterpret_cast<const f32x4*>(pq + (int64_t)b * U + u);
-      const f32x4 bv = *reinterpret_cast<const f32x4*>(bias + u);
-      const f32x4 vv = *reinterpret_cast<const f32x4*>(nv + u);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) a += vv[e] * tanhf(kv[e] + qv[e] + bv[e]);
-    }
-    a = wave_sum(a);
-    if (lane == 0) sc[j] = a;
-  }
-  __syncthreads();
   float mx = -INFINITY;
-  for (int j = threadIdx.x; j < n; j += 256) mx = fmaxf(mx, sc[j]);
+  for (int j = threadIdx.x; j < n; j += 256) { sc[j] = score[(int64_t)b * S + j]; mx = fmaxf(mx, sc[j]); }
   mx = wave_max(mx);
   if (lane == 0) red[wave] = mx;
   __syncthreads();
@@ -618,69 +627,80 @@ __global__ __launch_bounds__(256) void att_fwd_kernel(int S, int U, const float*
   sum = red[0] + red[1] + red[2] + red[3];
   for (int j = threadIdx.x; j < S; j += 256) {
     const float p = j < n ? expf(sc[j] - mx) / sum : 0.f;
-    align[(int64_t)b * S + j] = p;
     if (j < n) sc[j] = p;
+    if (blockIdx.x == 0) align[(int64_t)b * S + j] = p;
   }
   __syncthreads();
-  for (int u = threadIdx.x; u < U; u += 256) {
+  const int u = blockIdx.x * 256 + threadIdx.x;
+  if (u < U) {
     float c = 0.f;
     for (int j = 0; j < n; ++j) c += sc[j] * values[((int64_t)b * S + j) * U + u];
     ctx[(int64_t)b * ldc + u] = c;
   }
 }
 
-// one block per sample b: gradient of one step's attention.  datt [B,U] = d loss / d attention_t is consumed and
-// cleared; dkeys / dvalues [B,S,U] are added to; dpq [B,U] is written; dnv / dbias [U] receive atomic adds.
-__global__ __launch_bounds__(256) void att_bwd_kernel(int S, int U, const float* __restrict__ keys, const float* __restrict__ values,
-                                                     const float* __restrict__ pq, const float* __restrict__ nv,
-                                                     const float* __restrict__ bias, const int32_t* __restrict__ len,
-                                                     const float* __restrict__ align, float* __restrict__ datt, float* __restrict__ dpq,
-                                                     float* __restrict__ dkeys, float* __restrict__ dvalues, float* __restrict__ dnv,
-                                                     float* __restrict__ dbias) {
+// One wave per (b, j): d alignment[b][j] = datt[b] . values[b, j]  (datt = d loss / d attention of this step)
+__global__ __launch_bounds__(256) void att_dalign_kernel(int B, int S, int U, const float* __restrict__ values, const float* __restrict__ datt,
+                                                        const int32_t* __restrict__ len, float* __restrict__ da) {
+  const int lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= B * S) return;
+  const int b = row / S, j = row % S;
+  if (len && j >= len[b]) return;
+  const float* vj = values + (int64_t)row * U;
+  const float* d = datt + (int64_t)b * U;
+  float a = 0.f;
+  for (int u = lane * 4; u < U; u += 256) {
+    const f32x4 x = *reinterpret_cast<const f32x4*>(vj + u);
+    const f32x4 y = *reinterpret_cast<const f32x4*>(d + u);
+    a += x[0] * y[0] + x[1] * y[1] + x[2] * y[2] + x[3] * y[3];
+  }
+  a = wave_sum(a);
+  if (lane == 0) da[row] = a;
+}
+
+// grid (ceil(U/256), B): the rest of one step's attention gradient for the block's 256 units of sample b.  datt [B,U] is
+// consumed and cleared; dkeys / dvalues [B,S,U] are added to; dpq [B,U] is written; dnv / dbias [U] get atomic adds.
+__global__ __launch_bounds__(256) void att_grad_kernel(int S, int U, const float* __restrict__ keys, const float* __restrict__ pq,
+                                                      const float* __restrict__ nv, const float* __restrict__ bias,
+                                                      const int32_t* __restrict__ len, const float* __restrict__ align,
+                                                      const float* __restrict__ da, float* __restrict__ datt, float* __restrict__ dpq,
+                                                      float* __restrict__ dkeys, float* __restrict__ dvalues, float* __restrict__ dnv,
+                                                      float* __restrict__ dbias) {
+  __shared__ float al[ATT_MAX_S];
   __shared__ float ds[ATT_MAX_S];
   __shared__ float red[4];
-  const int b = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int b = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int n = len ? len[b] : S;
   n = n < 0 ? 0 : (n > S ? S : n);
-  const float* da = datt + (int64_t)b * U;
-  for (int j = wave; j < n; j += 4) {  // d alignment[j] = datt . values[j]
-    const float* vj = values + ((int64_t)b * S + j) * U;
-    float a = 0.f;
-    for (int u = lane * 4; u < U; u += 256) {
-      const f32x4 x = *reinterpret_cast<const f32x4*>(vj + u);
-      const f32x4 d = *reinterpret_cast<const f32x4*>(da + u);
-      a += x[0] * d[0] + x[1] * d[1] + x[2] * d[2] + x[3] * d[3];
-    }
-    a = wave_sum(a);
-    if (lane == 0) ds[j] = a;
-  }
-  __syncthreads();
   float s = 0.f;
-  for (int j = threadIdx.x; j < n; j += 256) s += align[(int64_t)b * S + j] * ds[j];
+  for (int j = threadIdx.x; j < n; j += 256) {
+    al[j] = align[(int64_t)b * S + j];
+    ds[j] = da[(int64_t)b * S + j];
+    s += al[j] * ds[j];
+  }
   s = wave_sum(s);
   if (lane == 0) red[wave] = s;
   __syncthreads();
   s = red[0] + red[1] + red[2] + red[3];
+  for (int j = threadIdx.x; j < n; j += 256) ds[j] = al[j] * (ds[j] - s);  // d score[j]
   __syncthreads();
-  for (int j = threadIdx.x; j < n; j += 256) ds[j] = align[(int64_t)b * S + j] * (ds[j] - s);  // d score[j]
-  __syncthreads();
-  for (int u = threadIdx.x; u < U; u += 256) {
-    const float q = pq[(int64_t)b * U + u] + bias[u], v = nv[u], dat = da[u];
-    float acc_pq = 0.f, acc_nv = 0.f;
-    for (int j = 0; j < n; ++j) {
-      const int64_t o = ((int64_t)b * S + j) * U + u;
-      const float th = tanhf(keys[o] + q);
-      const float d = ds[j] * v * (1.f - th * th);
-      dkeys[o] += d;
-      dvalues[o] += align[(int64_t)b * S + j] * dat;
-      acc_pq += d;
-      acc_nv += ds[j] * th;
-    }
-    dpq[(int64_t)b * U + u] = acc_pq;
-    atomicAdd(dbias + u, acc_pq);
-    atomicAdd(dnv + u, acc_nv);
-    datt[(int64_t)b * U + u] = 0.f;
+  const int u = blockIdx.x * 256 + threadIdx.x;
+  if (u >= U) return;
+  const float q = pq[(int64_t)b * U + u] + bias[u], v = nv[u], dat = datt[(int64_t)b * U + u];
+  float acc_pq = 0.f, acc_nv = 0.f;
+  for (int j = 0; j < n; ++j) {
+    const int64_t o = ((int64_t)b * S + j) * U + u;
+    const float th = tanhf(keys[o] + q);
+    const float d = ds[j] * v * (1.f - th * th);
+    dkeys[o] += d;
+    dvalues[o] += al[j] * dat;
+    acc_pq += d;
+    acc_nv += ds[j] * th;
   }
+  dpq[(int64_t)b * U + u] = acc_pq;
+  atomicAdd(dbias + u, acc_pq);
+  atomicAdd(dnv + u, acc_nv);
+  datt[(int64_t)b * U + u] = 0.f;
 }
 
 // d memory[j, b, :] = j < len[b] ? dvalues[b, j, :] : 0
@@ -716,11 +736,11 @@ struct GnmtAttentionStage : ds_stage {
   int B, T, S, U, R, RS;
   enum { W_EMB, W_K, W_BIAS, W_MEM, W_Q, W_V, W_G, W_B };
   char* stash_base = nullptr;
-  size_t slot_bytes = 0, ids_off, len_off, nv_off, val_off, key_off, emb_off, ah_off, g_off, c_off, al_off, pq_off;
+  size_t slot_bytes = 0, ids_off, len_off, nv_off, val_off, key_off, emb_off, ah_off, g_off, c_off, al_off, pq_off, sc_off;
   std::vector<char> slot_has_len;
   std::vector<float*> slot_att_out;
   char* ws_base = nullptr;
-  size_t ws_bytes = 0, ws_dg, ws_dh[2], ws_dc, ws_datt, ws_dpq, ws_dkeys, ws_dval, ws_dnv, ws_demb;
+  size_t ws_bytes = 0, ws_dg, ws_dh[2], ws_dc, ws_datt, ws_dpq, ws_dkeys, ws_dval, ws_dnv, ws_demb, ws_da;
 
   ~GnmtAttentionStage() override {
     if (stash_base) (void)hipFree(stash_base);
@@ -752,6 +772,7 @@ struct GnmtAttentionStage : ds_stage {
     c_off = sa.reserve((size_t)R * U * 4);
     al_off = sa.reserve((size_t)T * RS * 4);
     pq_off = sa.reserve((size_t)R * U * 4);
+    sc_off = sa.reserve((size_t)RS * 4);   // raw scores of the step being computed
     slot_bytes = sa.used;
     DS_CHECK_HIP(hipMalloc((void**)&stash_base, slot_bytes * gc.stash_slots));
     slot_forwarded.assign(gc.stash_slots, 0);
@@ -768,6 +789,7 @@ struct GnmtAttentionStage : ds_stage {
     ws_dval = wa.reserve((size_t)RS * U * 4);
     ws_dnv = wa.reserve((size_t)U * 4);
     ws_demb = wa.reserve((size_t)R * U * 4);
+    ws_da = wa.reserve((size_t)RS * 4);
     ws_bytes = wa.used;
     DS_CHECK_HIP(hipMalloc((void**)&ws_base, ws_bytes));
     return DS_OK;
@@ -835,9 +857,16 @@ struct GnmtAttentionStage : ds_stage {
       DS_CHECK_LAUNCH();
       float* pq = PQ + (size_t)t * B * U;
       DS_PROPAGATE(gemm_accum_splitk(DS_MN_MAJOR, B, U, U, ah_next + U, 2 * U, w[W_Q], U, pq, U));
-      ds_prof_scope prof(stream, "att_fwd_kernel", (double)RS * U * 4 * 2, "B");
-      hipLaunchKernelGGL(att_fwd_kernel, dim3(B), dim3(256), 0, stream, S, U, keys, values, pq, nv, w[W_B], len, AL + (size_t)t * RS, ah_next,
-                         2 * U);
+      float* SC = (float*)(sp + sc_off);
+      {
+        ds_prof_scope prof(stream, "att_score_kernel", (double)RS * U * 4, "B");
+        hipLaunchKernelGGL(att_score_kernel, dim3((RS + 3) / 4), dim3(256), 0, stream, B, S, U, keys, pq, nv, w[W_B], len, SC);
+      }
+      {
+        ds_prof_scope prof(stream, "att_context_kernel", (double)RS * U * 4, "B");
+        hipLaunchKernelGGL(att_context_kernel, dim3((U + 255) / 256, B), dim3(256), 0, stream, S, U, SC, values, len, AL + (size_t)t * RS,
+                           ah_next, 2 * U);
+      }
       DS_CHECK_LAUNCH();
     }
     // the cell outputs and, if asked for, the attention of every step, out of the [attention | h] blocks 1 .. T
@@ -880,9 +909,16 @@ struct GnmtAttentionStage : ds_stage {
       float* dh_out = (float*)(ws_base + ws_dh[(t & 1) ^ 1]);
       float* dpq = dPQ + (size_t)t * B * U;
       if (!first) {
-        ds_prof_scope prof(stream, "att_bwd_kernel", (double)RS * U * 4 * 6, "B");
-        hipLaunchKernelGGL(att_bwd_kernel, dim3(B), dim3(256), 0, stream, S, U, keys, values, PQ + (size_t)t * B * U, nv, w[W_B], len,
-                           AL + (size_t)t * RS, datt, dpq, dkeys, dval, dnv, g[W_B]);
+        float* da = (float*)(ws_base + ws_da);
+        {
+          ds_prof_scope prof(stream, "att_dalign_kernel", (double)RS * U * 4, "B");
+          hipLaunchKernelGGL(att_dalign_kernel, dim3((RS + 3) / 4), dim3(256), 0, stream, B, S, U, values, datt, len, da);
+        }
+        {
+          ds_prof_scope prof(stream, "att_grad_kernel", (double)RS * U * 4 * 5, "B");
+          hipLaunchKernelGGL(att_grad_kernel, dim3((U + 255) / 256, B), dim3(256), 0, stream, S, U, keys, PQ + (size_t)t * B * U, nv, w[W_B],
+                             len, AL + (size_t)t * RS, da, datt, dpq, dkeys, dval, dnv, g[W_B]);
+        }
         DS_CHECK_LAUNCH();
         // the query is the cell output: dh_t += dpq W_q^T
         DS_PROPAGATE(gemm_accum_splitk(DS_K_MAJOR, B, U, U, dpq, U, w[W_Q], U, dh_in, U));

@@ -243,6 +243,12 @@ CONFIGS = {
     # BASELINE configs[2]: GNMT-16 encoder stage (8 LSTM layers, the first bidirectional)
     "gnmt16_encoder": dict(index=2, kind="gnmt", num_layers=8, units=1024, vocab=32000, seq=50, micro_batch=64,
                            num_micro_batches=4, dtype="fp32", forget_bias=1.0),
+    # GNMT-16's two decoder pieces as the reference places them (not BASELINE configurations: the last-stage rows):
+    # decoder cell 0 + attention wrapper behind the encoder on device 0; cells 1..15, projection and loss on device 1
+    "gnmt16_attention_cell": dict(index=5, kind="gnmt_attention", units=1024, vocab=32000, seq=50, src_seq=50, micro_batch=64,
+                                  num_micro_batches=4, dtype="fp32", forget_bias=1.0),
+    "gnmt16_decoder": dict(index=6, kind="gnmt_decoder", num_layers=15, first_layer=1, units=1024, vocab=32000, seq=50,
+                           micro_batch=64, num_micro_batches=4, dtype="fp32", forget_bias=1.0),
     # BASELINE configs[3]: BERT-48 half-stage
     "bert48_half": dict(index=3, kind="bert", num_layers=24, hidden=1024, heads=16, ffn=4096,
                         seq=512, micro_batch=2, num_micro_batches=8, dtype="bf16",
