@@ -740,7 +740,7 @@ struct GnmtAttentionStage : ds_stage {
   std::vector<char> slot_has_len;
   std::vector<float*> slot_att_out;
   char* ws_base = nullptr;
-  size_t ws_bytes = 0, ws_dg, ws_dh[2], ws_dc, ws_datt, ws_dpq, ws_dkeys, ws_dval, ws_dnv, ws_demb, ws_da;
+  size_t ws_bytes = 0, ws_dg, ws_dah[2], ws_dc, ws_dpq, ws_dkeys, ws_dval, ws_dnv, ws_demb, ws_da;
 
   ~GnmtAttentionStage() override {
     if (stash_base) (void)hipFree(stash_base);
@@ -780,10 +780,10 @@ struct GnmtAttentionStage : ds_stage {
     slot_att_out.assign(gc.stash_slots, nullptr);
     Arena wa;
     ws_dg = wa.reserve((size_t)R * 4 * U * 4);
-    ws_dh[0] = wa.reserve((size_t)B * U * 4);
-    ws_dh[1] = wa.reserve((size_t)B * U * 4);
+    // gradient of [attention_{t-1} | h_{t-1}] as two [B, U] blocks, one product fills both; two of them in alternation
+    ws_dah[0] = wa.reserve((size_t)2 * B * U * 4);
+    ws_dah[1] = wa.reserve((size_t)2 * B * U * 4);
     ws_dc = wa.reserve((size_t)B * U * 4);
-    ws_datt = wa.reserve((size_t)B * U * 4);
     ws_dpq = wa.reserve((size_t)R * U * 4);
     ws_dkeys = wa.reserve((size_t)RS * U * 4);
     ws_dval = wa.reserve((size_t)RS * U * 4);
@@ -894,19 +894,21 @@ struct GnmtAttentionStage : ds_stage {
     const float* kernel = w[W_K];
     float* dG = (float*)(ws_base + ws_dg);
     float* dc = (float*)(ws_base + ws_dc);
-    float* datt = (float*)(ws_base + ws_datt);
     float* dPQ = (float*)(ws_base + ws_dpq);
     float* dkeys = (float*)(ws_base + ws_dkeys);
     float* dval = (float*)(ws_base + ws_dval);
     float* dnv = (float*)(ws_base + ws_dnv);
     const float* dY = (const float*)d_out;
-    // datt .. dnv are adjacent: the last step's dpq, the two [B,S,U] accumulators and dnv start at zero
-    DS_PROPAGATE(fill0(datt, (int64_t)((ws_demb - ws_datt) / 4)));
+    // dah .. dnv are adjacent: the state gradients, the last step's dpq, the two [B,S,U] accumulators and dnv start at zero
+    DS_PROPAGATE(fill0((float*)(ws_base + ws_dah[0]), (int64_t)((ws_demb - ws_dah[0]) / 4)));
     const int cell_grid = (B * U + 255) / 256;
     for (int t = T - 1; t >= 0; --t) {
       const int first = (t == T - 1);  // nothing downstream reads the last step's state or attention
-      float* dh_in = (float*)(ws_base + ws_dh[t & 1]);
-      float* dh_out = (float*)(ws_base + ws_dh[(t & 1) ^ 1]);
+      // block (t & 1): [d attention_t | d h_t] from step t + 1; the other block receives this step's
+      float* datt = (float*)(ws_base + ws_dah[t & 1]);
+      float* dh_in = datt + (size_t)B * U;
+      float* datt_out = (float*)(ws_base + ws_dah[(t & 1) ^ 1]);
+      float* dh_out = datt_out + (size_t)B * U;
       float* dpq = dPQ + (size_t)t * B * U;
       if (!first) {
         float* da = (float*)(ws_base + ws_da);
@@ -928,9 +930,14 @@ struct GnmtAttentionStage : ds_stage {
                          (const int32_t*)nullptr, t, t > 0 ? dh_out : nullptr);
       DS_CHECK_LAUNCH();
       if (t > 0) {
-        const float* dg = dG + (size_t)t * B * 4 * U;
-        DS_PROPAGATE(gemm_accum_splitk(DS_K_MAJOR, B, U, 4 * U, dg, 4 * U, kernel + (size_t)2 * U * 4 * U, 4 * U, dh_out, U));
-        DS_PROPAGATE(gemm_accum_splitk(DS_K_MAJOR, B, U, 4 * U, dg, 4 * U, kernel + (size_t)U * 4 * U, 4 * U, datt, U));
+        // [d attention_{t-1} ; d h_{t-1}] = dgates_t x (attention rows ; h rows of the kernel)^T: one batched product.
+        // Both targets are zero here: dh_out by the cell kernel above, datt_out by the att_grad_kernel that last read it.
+        ds_gemm_desc d;
+        memset(&d, 0, sizeof(d));
+        d.dtype = DS_F32; d.a_major = DS_K_MAJOR; d.b_major = DS_K_MAJOR; d.m = B; d.n = U; d.k = 4 * U; d.lda = 4 * U; d.ldb = 4 * U; d.ldc = U;
+        d.batch = 2; d.batch_inner = 2; d.b_stride_inner = (int64_t)U * 4 * U; d.c_stride_inner = (int64_t)B * U;
+        d.flags = DS_EPI_ACCUM; d.alpha = 1.f; d.a = dG + (size_t)t * B * 4 * U; d.b = kernel + (size_t)U * 4 * U; d.c = datt_out;
+        DS_PROPAGATE(ds_gemm_splitk(&d, gnmt_split_for(B, 2 * U, 4 * U), stream));
       }
     }
     // parameter gradients over all steps
