@@ -144,3 +144,32 @@ __device__ __forceinline__ float gelu_tanh_grad(float x) {
 }
 __device__ __forceinline__ float gelu_any(float x, bool tanh_form) { return tanh_form ? gelu_tanh(x) : gelu_erf(x); }
 __device__ __forceinline__ float gelu_any_grad(float x, bool tanh_form) { return tanh_form ? gelu_tanh_grad(x) : gelu_erf_grad(x); }
+
+// A dense layer over a handful of rows: out[b][j] = act(bias[j] + sum_k in[b][k] W[k][j]), W [K0 + K1, N] row-major,
+// in[b] = [in0[b * stride0 .. + K0) | in1[b * stride1 .. + K1)].  grid (ceil(N / 64), rows), 1024 threads: lane = column,
+// the 16 waves split k and meet in LDS.  ACT: 0 none, 1 tanh.
+template <typename TI, int ACT>
+__global__ __launch_bounds__(1024) void ds_small_dense_kernel(int K0, int K1, int N, const TI* __restrict__ in0, int64_t stride0,
+                                                              const float* __restrict__ in1, int64_t stride1,
+                                                              const float* __restrict__ W, const float* __restrict__ bias,
+                                                              float* __restrict__ out) {
+  __shared__ float red[16][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int j = blockIdx.x * 64 + lane, b = blockIdx.y;
+  const int K = K0 + K1, per = (K + 15) / 16;
+  const int k0 = wave * per, k1 = k0 + per < K ? k0 + per : K;
+  float a = 0.f;
+  if (j < N)
+    for (int k = k0; k < k1; ++k) {
+      const float x = k < K0 ? (float)in0[(int64_t)b * stride0 + k] : in1[(int64_t)b * stride1 + (k - K0)];
+      a += x * W[(int64_t)k * N + j];
+    }
+  red[wave][lane] = a;
+  __syncthreads();
+  if (wave == 0 && j < N) {
+    float s = bias ? bias[j] : 0.f;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) s += red[w][lane];
+    out[(int64_t)b * N + j] = ACT == 1 ? tanhf(s) : s;
+  }
+}

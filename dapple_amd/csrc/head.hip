@@ -124,20 +124,7 @@ int squad_head_t(int B, int S, int H, const void* x, const float* w, const float
 // (build_output_layer_classification: FC to the labels, mean sparse softmax cross entropy plus the l2
 // regulariser of the FC weights).  The batch is a handful of rows: plain one-thread-per-output kernels.
 
-// pooled[b][j] = tanh(x[b, token 0] . Wp[:, j] + bp[j]); also clears the loss
-template <typename T>
-__global__ __launch_bounds__(256) void pooler_fwd_kernel(int B, int S, int H, const T* __restrict__ x, const float* __restrict__ wp,
-                                                         const float* __restrict__ bp, float* __restrict__ pooled,
-                                                         float* __restrict__ loss) {
-  const int idx = blockIdx.x * 256 + threadIdx.x;
-  if (idx == 0) *loss = 0.f;
-  if (idx >= B * H) return;
-  const int b = idx / H, j = idx % H;
-  const T* xr = x + (int64_t)b * S * H;
-  float a = bp[j];
-  for (int i = 0; i < H; ++i) a += to_f32(xr[i]) * wp[(int64_t)i * H + j];
-  pooled[idx] = tanhf(a);
-}
+__global__ void head_clear_kernel(float* loss) { *loss = 0.f; }
 
 // one block: logits, loss = scale * (mean CE + l2_scale * sum(Wfc^2) / 2), dlogits = d loss / d logits
 __global__ __launch_bounds__(256) void classifier_loss_kernel(int B, int H, int C, const float* __restrict__ pooled,
@@ -228,28 +215,33 @@ __global__ __launch_bounds__(256) void pooler_wgrad_kernel(int B, int S, int H, 
   }
 }
 
-// dx[b, token 0][i] = sum_j dz[b][j] Wp[i][j]; every other token gets no gradient from this head
+// dx[b, token 0][i] = sum_j dz[b][j] Wp[i][j] (one wave per (b, i): a row of Wp); every other token gets no gradient
+// from this head (zero_rows_kernel)
 template <typename T>
 __global__ __launch_bounds__(256) void pooler_dgrad_kernel(int B, int S, int H, const float* __restrict__ dz, const float* __restrict__ wp,
                                                            T* __restrict__ dx) {
-  const int64_t total = (int64_t)B * S * H;
-  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
-    const int64_t row = idx / H;
-    const int i = (int)(idx % H);
-    float v = 0.f;
-    if (row % S == 0) {
-      const int b = (int)(row / S);
-      for (int j = 0; j < H; ++j) v += dz[(int64_t)b * H + j] * wp[(int64_t)i * H + j];
-    }
-    dx[idx] = from_f32<T>(v);
-  }
+  const int lane = threadIdx.x & 63, o = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (o >= B * H) return;
+  const int b = o / H, i = o % H;
+  float v = 0.f;
+  for (int j = lane; j < H; j += 64) v += dz[(int64_t)b * H + j] * wp[(int64_t)i * H + j];
+  v = wave_sum(v);
+  if (lane == 0) dx[(int64_t)b * S * H + i] = from_f32<T>(v);
+}
+template <typename T>
+__global__ __launch_bounds__(256) void zero_rows_kernel(int64_t total, int S, int H, T* __restrict__ dx) {
+  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256)
+    if ((idx / H) % S != 0) dx[idx] = from_f32<T>(0.f);
 }
 
 template <typename T>
 int classifier_head_t(int B, int S, int H, int C, const void* x, const float* wp, const float* bp, const float* wfc, const float* bfc,
                       const int32_t* labels, float l2_scale, float scale, float* loss, float* pooled, float* logits, float* dlogits,
                       float* dz, void* dx, float* dwp, float* dbp, float* dwfc, float* dbfc, hipStream_t s) {
-  hipLaunchKernelGGL(pooler_fwd_kernel<T>, dim3((B * H + 255) / 256), dim3(256), 0, s, B, S, H, (const T*)x, wp, bp, pooled, loss);
+  // pooled[b][j] = tanh(x[b, token 0] . Wp[:, j] + bp[j])
+  hipLaunchKernelGGL(head_clear_kernel, dim3(1), dim3(1), 0, s, loss);
+  hipLaunchKernelGGL((ds_small_dense_kernel<T, 1>), dim3((H + 63) / 64, B), dim3(1024), 0, s, H, 0, H, (const T*)x, (int64_t)S * H,
+                     (const float*)nullptr, (int64_t)0, wp, bp, pooled);
   DS_CHECK_LAUNCH();
   hipLaunchKernelGGL(classifier_loss_kernel, dim3(1), dim3(256), 0, s, B, H, C, pooled, wfc, bfc, labels, l2_scale, scale, logits,
                      dlogits, loss);
@@ -265,8 +257,9 @@ int classifier_head_t(int B, int S, int H, int C, const void* x, const float* wp
   }
   if (dx) {
     const int64_t total = (int64_t)B * S * H;
-    hipLaunchKernelGGL(pooler_dgrad_kernel<T>, dim3((unsigned)((total + 255) / 256 > 8192 ? 8192 : (total + 255) / 256)), dim3(256), 0, s,
-                       B, S, H, dz, wp, (T*)dx);
+    hipLaunchKernelGGL(zero_rows_kernel<T>, dim3((unsigned)((total + 255) / 256 > 8192 ? 8192 : (total + 255) / 256)), dim3(256), 0, s,
+                       total, S, H, (T*)dx);
+    hipLaunchKernelGGL(pooler_dgrad_kernel<T>, dim3((B * H + 3) / 4), dim3(256), 0, s, B, S, H, dz, wp, (T*)dx);
     DS_CHECK_LAUNCH();
   }
   return DS_OK;

@@ -46,19 +46,6 @@ __global__ __launch_bounds__(256) void xh_pick_kernel(int S, int B, int H, const
   out[(int64_t)b * H + c] = (pos >= 0 && pos < S) ? x[((int64_t)pos * B + b) * H + c] : 0.f;
 }
 
-// thread per (b, j): out[b][j] = act(sum_k in[b][k] W[k][j] + bias[j]); in = [in0 | in1] (in1 null: K = H)
-__global__ __launch_bounds__(256) void xh_dense_fwd_kernel(int B, int H, int N, const float* __restrict__ in0, const float* __restrict__ in1,
-                                                           const float* __restrict__ W, const float* __restrict__ bias, int tanh_act,
-                                                           float* __restrict__ out) {
-  const int j = blockIdx.x * 256 + threadIdx.x, b = blockIdx.y;
-  if (j >= N) return;
-  float a = bias ? bias[j] : 0.f;
-  for (int k = 0; k < H; ++k) a += in0[(int64_t)b * H + k] * W[(int64_t)k * N + j];
-  if (in1)
-    for (int k = 0; k < H; ++k) a += in1[(int64_t)b * H + k] * W[(int64_t)(H + k) * N + j];
-  out[(int64_t)b * N + j] = tanh_act ? tanhf(a) : a;
-}
-
 // one wave per (b, k): din[b][k] = sum_j dout[b][j] W[k][j]
 __global__ __launch_bounds__(256) void xh_dense_din_kernel(int B, int K, int N, const float* __restrict__ dout, const float* __restrict__ W,
                                                            float* __restrict__ din) {
@@ -338,8 +325,8 @@ extern "C" int ds_xlnet_squad_head(int dtype, int seq, int batch, int hidden, co
   hipLaunchKernelGGL(xh_seq_loss_kernel, dim3(B), dim3(256), 0, s, S, start_logits, p_mask, start_positions, wgt, 0, F(L.p), F(L.sl_g), loss);
   // ---- end branch
   hipLaunchKernelGGL(xh_pick_kernel, dim3(cdiv(H, 256), B, 2), dim3(256), 0, s, S, B, H, xf, start_positions, cls_index, F(L.pick0), F(L.pick1));
-  hipLaunchKernelGGL(xh_dense_fwd_kernel, dim3(cdiv(H, 256), B), dim3(256), 0, s, B, H, H, F(L.pick0), (const float*)nullptr,
-                     w->end_w0 + (int64_t)H * H, w->end_b0, 0, F(L.sfw));
+  hipLaunchKernelGGL((ds_small_dense_kernel<float, 0>), dim3(cdiv(H, 64), B), dim3(1024), 0, s, H, 0, H, (const float*)F(L.pick0), (int64_t)H,
+                     (const float*)nullptr, (int64_t)0, (const float*)(w->end_w0 + (int64_t)H * H), (const float*)w->end_b0, F(L.sfw));
   DS_CHECK_LAUNCH();
   DS_PROPAGATE(gemm_f32(DS_K_MAJOR, DS_MN_MAJOR, rows, H, H, xf, H, w->end_w0, H, F(L.t), H, 0, s));
   hipLaunchKernelGGL(xh_addtanh_kernel, dim3(cdiv(big / 4, 256)), dim3(256), 0, s, big / 4, B, H, F(L.t), F(L.sfw));
@@ -349,8 +336,8 @@ extern "C" int ds_xlnet_squad_head(int dtype, int seq, int batch, int hidden, co
   hipLaunchKernelGGL(xh_seq_loss_kernel, dim3(B), dim3(256), 0, s, S, end_logits, p_mask, end_positions, wgt, 1, (float*)nullptr, F(L.del), loss);
   // ---- answerability branch
   hipLaunchKernelGGL(xh_wsum_kernel, dim3(cdiv(H, 256), B, 16), dim3(256), 0, s, S, B, H, xf, F(L.p), F(L.sfeat));
-  hipLaunchKernelGGL(xh_dense_fwd_kernel, dim3(cdiv(H, 256), B), dim3(256), 0, s, B, H, H, F(L.sfeat), F(L.pick1), w->ans_w0, w->ans_b0, 1,
-                     F(L.ans));
+  hipLaunchKernelGGL((ds_small_dense_kernel<float, 1>), dim3(cdiv(H, 64), B), dim3(1024), 0, s, H, H, H, (const float*)F(L.sfeat), (int64_t)H,
+                     (const float*)F(L.pick1), (int64_t)H, (const float*)w->ans_w0, (const float*)w->ans_b0, F(L.ans));
   hipLaunchKernelGGL(xh_answer_kernel, dim3(B), dim3(256), 0, s, H, F(L.ans), dropout_mask, w->ans_w1, is_impossible, wgt, cls_logits, loss,
                      bwd ? F(L.dans) : nullptr, g ? g->ans_w1 : nullptr);
   DS_CHECK_LAUNCH();
