@@ -15,6 +15,7 @@
 // half in place) and runs the fused cell kernel.  Backward walks the steps in reverse with the cell
 // backward kernel and dh = dgates @ Wh^T, then finishes with three big GEMMs over all steps:
 // dX = dG @ Wx^T, dWx += X^T dG, dWh += Hprev^T dG.
+#include <stdlib.h>
 #include <string.h>
 
 #include "stage.h"
@@ -49,11 +50,15 @@ __global__ __launch_bounds__(256) void gnmt_embed_bwd_kernel(int B, int T, int U
 // One time step of the cell.  gates [B,4U] holds the pre-activations (bias included) and is
 // overwritten with the activated gates (sigmoid(i), tanh(j), sigmoid(f + forget_bias), sigmoid(o));
 // h is written with row stride ldh, and y = h + x_res when the cell has a residual connection.
+// part (nullable) [nparts][B][4U]: partial sums of the recurrent product h_{t-1} Wh, one per slice of the reduction,
+// added to the pre-activations here - the product is split so that every CU has work, and summing the slices where
+// they are consumed costs a few reads where atomic adds from the product's epilogue cost as much as the product.
 __global__ __launch_bounds__(256) void lstm_cell_fwd_kernel(int B, int U, float forget_bias, float* __restrict__ gates,
                                                            const float* __restrict__ c_prev, float* __restrict__ c,
                                                            float* __restrict__ h, int ldh, const float* __restrict__ x_res,
                                                            int ldx, float* __restrict__ y, int ldy,
-                                                           const int32_t* __restrict__ len, int t) {
+                                                           const int32_t* __restrict__ len, int t, const float* __restrict__ part,
+                                                           int nparts) {
   const int idx = blockIdx.x * 256 + threadIdx.x;
   if (idx >= B * U) return;
   const int b = idx / U, u = idx % U;
@@ -64,7 +69,12 @@ __global__ __launch_bounds__(256) void lstm_cell_fwd_kernel(int B, int U, float 
     return;
   }
   float* g = gates + (int64_t)b * 4 * U;
-  const float i = sigmoidf_(g[u]), j = tanhf(g[U + u]), f = sigmoidf_(g[2 * U + u] + forget_bias), o = sigmoidf_(g[3 * U + u]);
+  float gi = g[u], gj = g[U + u], gf = g[2 * U + u], go = g[3 * U + u];
+  for (int p = 0; p < nparts; ++p) {
+    const float* q = part + ((int64_t)p * B + b) * 4 * U;
+    gi += q[u]; gj += q[U + u]; gf += q[2 * U + u]; go += q[3 * U + u];
+  }
+  const float i = sigmoidf_(gi), j = tanhf(gj), f = sigmoidf_(gf + forget_bias), o = sigmoidf_(go);
   const float cp = c_prev ? c_prev[idx] : 0.f;
   const float cn = cp * f + i * j;
   const float hn = tanhf(cn) * o;
@@ -76,12 +86,14 @@ __global__ __launch_bounds__(256) void lstm_cell_fwd_kernel(int B, int U, float 
 
 // Backward of one step: dh = dy[t] + dh_rec, dc = dc_rec + dh*o*(1 - tanh(c)^2); writes the four
 // pre-activation gate gradients, leaves dc*f in dc_rec for step t-1 and zeroes `clear` [B,U].
+// The recurrent gradient comes as dh_rec [B,U] (nullable) and / or as part [nparts][B][U], the slices of dgates Wh^T.
 __global__ __launch_bounds__(256) void lstm_cell_bwd_kernel(int B, int U, const float* __restrict__ gact,
                                                            const float* __restrict__ c, const float* __restrict__ c_prev,
                                                            const float* __restrict__ dy, int lddy,
                                                            const float* __restrict__ dh_rec, float* __restrict__ dc_rec,
                                                            int first, float* __restrict__ dgates,
-                                                           const int32_t* __restrict__ len, int t, float* __restrict__ clear) {
+                                                           const int32_t* __restrict__ len, int t, float* __restrict__ clear,
+                                                           const float* __restrict__ part, int nparts) {
   const int idx = blockIdx.x * 256 + threadIdx.x;
   if (idx >= B * U) return;
   if (clear) clear[idx] = 0.f;  // the buffer the next recurrent product adds into
@@ -95,7 +107,11 @@ __global__ __launch_bounds__(256) void lstm_cell_bwd_kernel(int B, int U, const 
   const float* g = gact + (int64_t)b * 4 * U;
   const float i = g[u], j = g[U + u], f = g[2 * U + u], o = g[3 * U + u];
   const float tc = tanhf(c[idx]);
-  const float dh = dy[(int64_t)b * lddy + u] + (first ? 0.f : dh_rec[idx]);
+  float dh = dy[(int64_t)b * lddy + u];
+  if (!first) {
+    if (dh_rec) dh += dh_rec[idx];
+    for (int p = 0; p < nparts; ++p) dh += part[((int64_t)p * B + b) * U + u];
+  }
   const float dc = (first ? 0.f : dc_rec[idx]) + dh * o * (1.f - tc * tc);
   const float cp = c_prev ? c_prev[idx] : 0.f;
   float* d = dgates + (int64_t)b * 4 * U;
@@ -144,6 +160,29 @@ static int gnmt_gemm_accum_splitk(hipStream_t stream, int bm, int m, int n, int 
   return ds_gemm_splitk(&d, gnmt_split_for(m, n, k), stream);
 }
 
+// c[z] = a[:, z-th slice of k] x b[z-th slice of k, :]: the reduction of a product with few rows cut into `slices`
+// independent products (a batched launch, plain stores) whose results the consumer adds up
+static int gnmt_gemm_slices(hipStream_t stream, int bm, int m, int n, int k, int slices, const void* a, int64_t lda, const void* b,
+                            int64_t ldb, float* parts) {
+  ds_gemm_desc d;
+  memset(&d, 0, sizeof(d));
+  const int kc = k / slices;
+  d.dtype = DS_F32; d.a_major = DS_K_MAJOR; d.b_major = bm; d.m = m; d.n = n; d.k = kc; d.lda = lda; d.ldb = ldb; d.ldc = n;
+  d.batch = slices; d.batch_inner = slices;
+  d.a_stride_inner = kc;
+  d.b_stride_inner = bm == DS_K_MAJOR ? (int64_t)kc : (int64_t)kc * ldb;
+  d.c_stride_inner = (int64_t)m * n;
+  d.alpha = 1.f; d.a = a; d.b = b; d.c = parts;
+  return ds_gemm(&d, stream);
+}
+// how many slices: enough 64x64 tiles for every CU, each slice a multiple of 32 (the fp32 k-tile) and at least 128 deep
+static int gnmt_slices_for(int m, int n, int k) {
+  const int tiles = ((m + 63) / 64) * ((n + 63) / 64);
+  int s = 1;
+  while (s < 32 && tiles * s < 256 && k % (2 * s * 32) == 0 && k / (2 * s) >= 128) s *= 2;
+  return s;
+}
+
 struct Cell {
   int widx;        // kernel index in the weight list (bias = widx + 1)
   int n_in;        // input width
@@ -163,7 +202,8 @@ struct GnmtStage : ds_stage {
   size_t slot_bytes = 0, ids_off = 0, len_off = 0, x0_off = 0, xb_off = 0;
   std::vector<char> slot_has_len;
   char* ws_base = nullptr;
-  size_t ws_bytes = 0, ws_dg, ws_dx[2], ws_dh[2], ws_dc, ws_dym;
+  size_t ws_bytes = 0, ws_dg, ws_dx[2], ws_dc, ws_dym, ws_pf, ws_pb;
+  int sl_f = 1, sl_b = 1;  // slices of the recurrent products h Wh (forward) and dgates Wh^T (backward)
 
   ~GnmtStage() override {
     if (stash_base) (void)hipFree(stash_base);
@@ -223,10 +263,12 @@ struct GnmtStage : ds_stage {
     ws_dg = wa.reserve((size_t)R * 4 * U * 4);
     ws_dx[0] = wa.reserve((size_t)R * 2 * U * 4);
     ws_dx[1] = wa.reserve((size_t)R * 2 * U * 4);
-    ws_dh[0] = wa.reserve((size_t)B * U * 4);
-    ws_dh[1] = wa.reserve((size_t)B * U * 4);
     ws_dc = wa.reserve((size_t)B * U * 4);
     ws_dym = wa.reserve((size_t)R * U * 4);
+    sl_f = gnmt_slices_for(B, 4 * U, U);
+    sl_b = gnmt_slices_for(B, U, 4 * U);
+    ws_pf = wa.reserve((size_t)sl_f * B * 4 * U * 4);  // forward's and backward's own: the two may run side by side
+    ws_pb = wa.reserve((size_t)sl_b * B * U * 4);
     ws_bytes = wa.used;
     DS_CHECK_HIP(hipMalloc((void**)&ws_base, ws_bytes));
     return DS_OK;
@@ -279,15 +321,14 @@ struct GnmtStage : ds_stage {
         const int t = c.reverse ? T - 1 - s : s;
         const int tp = c.reverse ? t + 1 : t - 1;  // the step whose state feeds this one
         float* g = G + (size_t)t * B * 4 * U;
-        if (s > 0) {
-          // recurrent half, added in place: g += h[tp] @ Wh
-          DS_PROPAGATE(gemm_accum_splitk(DS_MN_MAJOR, B, 4 * U, U, H + (size_t)tp * B * c.ldh, c.ldh, wh, 4 * U, g, 4 * U));
-        }
+        float* pf = (float*)(ws_base + ws_pf);
+        if (s > 0)  // recurrent half h[tp] @ Wh in sl_f slices of the reduction; the cell kernel adds them to g
+          DS_PROPAGATE(gnmt_gemm_slices(stream, DS_MN_MAJOR, B, 4 * U, U, sl_f, H + (size_t)tp * B * c.ldh, c.ldh, wh, 4 * U, pf));
         ds_prof_scope prof(stream, "lstm_cell_fwd_kernel", (double)B * U * 4 * (4 + 4 + 2 + (c.residual ? 2 : 1)), "B");
         hipLaunchKernelGGL(lstm_cell_fwd_kernel, dim3(cell_grid), dim3(256), 0, stream, B, U, gc.forget_bias, g,
                            s > 0 ? Cs + (size_t)tp * B * U : nullptr, Cs + (size_t)t * B * U, H + (size_t)t * B * c.ldh, c.ldh,
                            c.residual ? X + (size_t)t * B * c.ldx : nullptr, c.ldx, Y ? Y + (size_t)t * B * U : nullptr, U,
-                           len, t);
+                           len, t, pf, s > 0 ? sl_f : 0);
         DS_CHECK_LAUNCH();
       }
       if (last && !c.residual)
@@ -331,18 +372,16 @@ struct GnmtStage : ds_stage {
         const int t = c.reverse ? T - 1 - s : s;
         const int tp = c.reverse ? t + 1 : t - 1;
         const int first = (s == T - 1);  // no recurrent gradient flows into the last step of the scan
-        float* dh_in = (float*)(ws_base + ws_dh[s & 1]);
-        float* dh_out = (float*)(ws_base + ws_dh[(s & 1) ^ 1]);
+        float* pb = (float*)(ws_base + ws_pb);  // slices of dgates Wh^T of the step scanned before this one
         {
           ds_prof_scope prof(stream, "lstm_cell_bwd_kernel", (double)B * U * 4 * (4 + 4 + 6), "B");
           hipLaunchKernelGGL(lstm_cell_bwd_kernel, dim3(cell_grid), dim3(256), 0, stream, B, U, G + (size_t)t * B * 4 * U,
                              Cs + (size_t)t * B * U, s > 0 ? Cs + (size_t)tp * B * U : nullptr, dY + (size_t)t * B * lddy, lddy,
-                             dh_in, dc, first, dG + (size_t)t * B * 4 * U, len, t, s > 0 ? dh_out : nullptr);
+                             (const float*)nullptr, dc, first, dG + (size_t)t * B * 4 * U, len, t, (float*)nullptr, pb, first ? 0 : sl_b);
           DS_CHECK_LAUNCH();
         }
-        if (s > 0) {  // dh for step tp: dgates[t] @ Wh^T
-          DS_PROPAGATE(gemm_accum_splitk(DS_K_MAJOR, B, U, 4 * U, dG + (size_t)t * B * 4 * U, 4 * U, wh, 4 * U, dh_out, U));
-        }
+        if (s > 0)  // dh for step tp: dgates[t] @ Wh^T, in sl_b slices the next cell kernel adds up
+          DS_PROPAGATE(gnmt_gemm_slices(stream, DS_K_MAJOR, B, U, 4 * U, sl_b, dG + (size_t)t * B * 4 * U, 4 * U, wh, 4 * U, pb));
       }
       // parameter gradients over all steps
       DS_PROPAGATE(ds_colsum_accum(DS_F32, R, 4 * U, dG, 4 * U, g[c.widx + 1], stream));
@@ -395,7 +434,8 @@ struct GnmtDecoderStage : ds_stage {
   size_t slot_bytes = 0, x0_off = 0, att_off = 0;
   std::vector<char> slot_has_att;
   char* ws_base = nullptr;
-  size_t ws_bytes = 0, ws_dg, ws_dx[2], ws_dh[2], ws_dc;
+  size_t ws_bytes = 0, ws_dg, ws_dx[2], ws_dc, ws_pf, ws_pb;
+  int sl_f = 1, sl_b = 1;  // slices of the recurrent products (see GnmtStage)
 
   ~GnmtDecoderStage() override {
     if (stash_base) (void)hipFree(stash_base);
@@ -432,9 +472,11 @@ struct GnmtDecoderStage : ds_stage {
     ws_dg = wa.reserve((size_t)R * 4 * U * 4);
     ws_dx[0] = wa.reserve((size_t)R * U * 4);
     ws_dx[1] = wa.reserve((size_t)R * U * 4);
-    ws_dh[0] = wa.reserve((size_t)B * U * 4);
-    ws_dh[1] = wa.reserve((size_t)B * U * 4);
     ws_dc = wa.reserve((size_t)B * U * 4);
+    sl_f = gnmt_slices_for(B, 4 * U, U);
+    sl_b = gnmt_slices_for(B, U, 4 * U);
+    ws_pf = wa.reserve((size_t)sl_f * B * 4 * U * 4);
+    ws_pb = wa.reserve((size_t)sl_b * B * U * 4);
     ws_bytes = wa.used;
     DS_CHECK_HIP(hipMalloc((void**)&ws_base, ws_bytes));
     return DS_OK;
@@ -483,12 +525,13 @@ struct GnmtDecoderStage : ds_stage {
       if (att) DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, R, 4 * U, U, att, U, wa, 4 * U, G, 4 * U, DS_EPI_ACCUM, nullptr, nullptr));
       for (int t = 0; t < T; ++t) {
         float* g = G + (size_t)t * B * 4 * U;
-        if (t > 0) DS_PROPAGATE(gemm_accum_splitk(DS_MN_MAJOR, B, 4 * U, U, H + (size_t)(t - 1) * B * U, U, wh, 4 * U, g, 4 * U));
+        float* pf = (float*)(ws_base + ws_pf);
+        if (t > 0) DS_PROPAGATE(gnmt_gemm_slices(stream, DS_MN_MAJOR, B, 4 * U, U, sl_f, H + (size_t)(t - 1) * B * U, U, wh, 4 * U, pf));
         ds_prof_scope prof(stream, "lstm_cell_fwd_kernel", (double)B * U * 4 * (4 + 4 + 2 + (c.residual ? 2 : 1)), "B");
         hipLaunchKernelGGL(lstm_cell_fwd_kernel, dim3(cell_grid), dim3(256), 0, stream, B, U, gc.forget_bias, g,
                            t > 0 ? Cs + (size_t)(t - 1) * B * U : nullptr, Cs + (size_t)t * B * U, H + (size_t)t * B * U, U,
                            c.residual ? X + (size_t)t * B * U : nullptr, U, Y ? Y + (size_t)t * B * U : nullptr, U,
-                           (const int32_t*)nullptr, t);
+                           (const int32_t*)nullptr, t, pf, t > 0 ? sl_f : 0);
         DS_CHECK_LAUNCH();
       }
       if (last && !c.residual) DS_CHECK_HIP(hipMemcpyAsync(out, H, (size_t)R * U * 4, hipMemcpyDeviceToDevice, stream));
@@ -517,16 +560,16 @@ struct GnmtDecoderStage : ds_stage {
       if (ci > 0) X = (const float*)(sp + (cells[ci - 1].residual ? cells[ci - 1].y_off : cells[ci - 1].h_off));
       for (int t = T - 1; t >= 0; --t) {
         const int first = (t == T - 1);
-        float* dh_in = (float*)(ws_base + ws_dh[t & 1]);
-        float* dh_out = (float*)(ws_base + ws_dh[(t & 1) ^ 1]);
+        float* pb = (float*)(ws_base + ws_pb);
         {
           ds_prof_scope prof(stream, "lstm_cell_bwd_kernel", (double)B * U * 4 * (4 + 4 + 6), "B");
           hipLaunchKernelGGL(lstm_cell_bwd_kernel, dim3(cell_grid), dim3(256), 0, stream, B, U, G + (size_t)t * B * 4 * U,
-                             Cs + (size_t)t * B * U, t > 0 ? Cs + (size_t)(t - 1) * B * U : nullptr, dY + (size_t)t * B * U, U, dh_in, dc,
-                             first, dG + (size_t)t * B * 4 * U, (const int32_t*)nullptr, t, t > 0 ? dh_out : nullptr);
+                             Cs + (size_t)t * B * U, t > 0 ? Cs + (size_t)(t - 1) * B * U : nullptr, dY + (size_t)t * B * U, U,
+                             (const float*)nullptr, dc, first, dG + (size_t)t * B * 4 * U, (const int32_t*)nullptr, t, (float*)nullptr, pb,
+                             first ? 0 : sl_b);
           DS_CHECK_LAUNCH();
         }
-        if (t > 0) DS_PROPAGATE(gemm_accum_splitk(DS_K_MAJOR, B, U, 4 * U, dG + (size_t)t * B * 4 * U, 4 * U, wh, 4 * U, dh_out, U));
+        if (t > 0) DS_PROPAGATE(gnmt_gemm_slices(stream, DS_K_MAJOR, B, U, 4 * U, sl_b, dG + (size_t)t * B * 4 * U, 4 * U, wh, 4 * U, pb));
       }
       float* gk = g[c.widx];
       DS_PROPAGATE(ds_colsum_accum(DS_F32, R, 4 * U, dG, 4 * U, g[c.widx + 1], stream));
@@ -853,7 +896,7 @@ struct GnmtAttentionStage : ds_stage {
       if (t > 0) DS_PROPAGATE(gemm_accum_splitk(DS_MN_MAJOR, B, 4 * U, 2 * U, ah, 2 * U, kernel + (size_t)U * 4 * U, 4 * U, g, 4 * U));
       hipLaunchKernelGGL(lstm_cell_fwd_kernel, dim3(cell_grid), dim3(256), 0, stream, B, U, gc.forget_bias, g,
                          t > 0 ? Cs + (size_t)(t - 1) * B * U : nullptr, Cs + (size_t)t * B * U, ah_next + U, 2 * U, (const float*)nullptr, 0,
-                         (float*)nullptr, 0, (const int32_t*)nullptr, t);
+                         (float*)nullptr, 0, (const int32_t*)nullptr, t, (const float*)nullptr, 0);
       DS_CHECK_LAUNCH();
       float* pq = PQ + (size_t)t * B * U;
       DS_PROPAGATE(gemm_accum_splitk(DS_MN_MAJOR, B, U, U, ah_next + U, 2 * U, w[W_Q], U, pq, U));
@@ -927,7 +970,7 @@ struct GnmtAttentionStage : ds_stage {
       }
       hipLaunchKernelGGL(lstm_cell_bwd_kernel, dim3(cell_grid), dim3(256), 0, stream, B, U, G + (size_t)t * B * 4 * U, Cs + (size_t)t * B * U,
                          t > 0 ? Cs + (size_t)(t - 1) * B * U : nullptr, dY + (size_t)t * B * U, U, dh_in, dc, first, dG + (size_t)t * B * 4 * U,
-                         (const int32_t*)nullptr, t, t > 0 ? dh_out : nullptr);
+                         (const int32_t*)nullptr, t, t > 0 ? dh_out : nullptr, (const float*)nullptr, 0);
       DS_CHECK_LAUNCH();
       if (t > 0) {
         // [d attention_{t-1} ; d h_{t-1}] = dgates_t x (attention rows ; h rows of the kernel)^T: one batched product.
