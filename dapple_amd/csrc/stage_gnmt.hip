@@ -70,18 +70,32 @@ __global__ __launch_bounds__(256) void lstm_cell_fwd_kernel(int B, int U, float 
   }
   float* g = gates + (int64_t)b * 4 * U;
   float gi = g[u], gj = g[U + u], gf = g[2 * U + u], go = g[3 * U + u];
-  for (int p = 0; p < nparts; ++p) {
+  const float cp = c_prev ? c_prev[idx] : 0.f;
+  const float xr = y ? x_res[(int64_t)b * ldx + u] : 0.f;
+  // the slices are read four at a time before any is added (sixteen loads in flight instead of a round trip
+  // to memory per slice); the additions keep the order of the slices
+  int p = 0;
+  for (; p + 4 <= nparts; p += 4) {
+    float v[4][4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const float* q = part + ((int64_t)(p + s) * B + b) * 4 * U;
+      v[s][0] = q[u]; v[s][1] = q[U + u]; v[s][2] = q[2 * U + u]; v[s][3] = q[3 * U + u];
+    }
+#pragma unroll
+    for (int s = 0; s < 4; ++s) { gi += v[s][0]; gj += v[s][1]; gf += v[s][2]; go += v[s][3]; }
+  }
+  for (; p < nparts; ++p) {
     const float* q = part + ((int64_t)p * B + b) * 4 * U;
     gi += q[u]; gj += q[U + u]; gf += q[2 * U + u]; go += q[3 * U + u];
   }
   const float i = sigmoidf_(gi), j = tanhf(gj), f = sigmoidf_(gf + forget_bias), o = sigmoidf_(go);
-  const float cp = c_prev ? c_prev[idx] : 0.f;
   const float cn = cp * f + i * j;
   const float hn = tanhf(cn) * o;
   g[u] = i; g[U + u] = j; g[2 * U + u] = f; g[3 * U + u] = o;
   c[idx] = cn;
   h[(int64_t)b * ldh + u] = hn;
-  if (y) y[(int64_t)b * ldy + u] = hn + x_res[(int64_t)b * ldx + u];
+  if (y) y[(int64_t)b * ldy + u] = hn + xr;
 }
 
 // Backward of one step: dh = dy[t] + dh_rec, dc = dc_rec + dh*o*(1 - tanh(c)^2); writes the four
@@ -106,14 +120,26 @@ __global__ __launch_bounds__(256) void lstm_cell_bwd_kernel(int B, int U, const 
   }
   const float* g = gact + (int64_t)b * 4 * U;
   const float i = g[u], j = g[U + u], f = g[2 * U + u], o = g[3 * U + u];
-  const float tc = tanhf(c[idx]);
+  const float cv = c[idx];
+  const float cp = c_prev ? c_prev[idx] : 0.f;
+  const float dcr = first ? 0.f : dc_rec[idx];
   float dh = dy[(int64_t)b * lddy + u];
   if (!first) {
     if (dh_rec) dh += dh_rec[idx];
-    for (int p = 0; p < nparts; ++p) dh += part[((int64_t)p * B + b) * U + u];
+    // eight slices are read before any is added (one round trip to memory per eight instead of per slice);
+    // the additions keep the order of the slices
+    int p = 0;
+    for (; p + 8 <= nparts; p += 8) {
+      float v[8];
+#pragma unroll
+      for (int s = 0; s < 8; ++s) v[s] = part[((int64_t)(p + s) * B + b) * U + u];
+#pragma unroll
+      for (int s = 0; s < 8; ++s) dh += v[s];
+    }
+    for (; p < nparts; ++p) dh += part[((int64_t)p * B + b) * U + u];
   }
-  const float dc = (first ? 0.f : dc_rec[idx]) + dh * o * (1.f - tc * tc);
-  const float cp = c_prev ? c_prev[idx] : 0.f;
+  const float tc = tanhf(cv);
+  const float dc = dcr + dh * o * (1.f - tc * tc);
   float* d = dgates + (int64_t)b * 4 * U;
   d[u] = dc * j * i * (1.f - i);
   d[U + u] = dc * i * (1.f - j * j);
