@@ -11,6 +11,9 @@ algorithmic bytes printed, so a kernel trace gives achieved GB/s against the HBM
     rocprofv3 --pmc FETCH_SIZE --output-format csv -d out -o c -- python3 -m dapple_amd.calib accumulate 67108864
     rocprofv3 --pmc FETCH_SIZE --output-format csv -d out -o g -- python3 -m dapple_amd.calib gemms
     rocprofv3 --kernel-trace --stats -d out -o e -- python3 -m dapple_amd.calib elementwise
+
+``attention``: the fused attention kernels at the BERT-48 half-stage's shape (2 samples, 16 heads, 512 positions, head
+size 64, bf16), three launches each, for the same counter runs as ``gemms`` (matrix-core busy cycles, HBM traffic).
 """
 import sys
 
@@ -53,6 +56,19 @@ def gemms():
         print("%s: m=%d n=%d k=%d, algorithmic bytes %d" % (name, m, n, k, alg))
 
 
+def attention():
+    batch, heads, seq, d = 2, 16, 512, 64
+    bf = torch.bfloat16
+    qkv = torch.randn(batch * seq, 3 * heads * d, device="cuda").to(bf)
+    dctx = torch.randn(batch * seq, heads * d, device="cuda").to(bf)
+    for _ in range(3):
+        ctx, lse = ops.attention_fwd(qkv, batch, heads, seq, 0.125)
+        ops.attention_bwd(qkv, ctx, lse, dctx, batch, heads, seq, 0.125)
+    torch.cuda.synchronize()
+    unit = batch * heads * seq * seq * d
+    print("attn_fwd_kernel: %d FLOP per launch; attn_bwd_dq_kernel: %d; attn_bwd_dkv_kernel: %d" % (4 * unit, 6 * unit, 8 * unit))
+
+
 def elementwise():
     bf = torch.bfloat16
     rows, h, f = 1024, 1024, 4096
@@ -85,5 +101,7 @@ if __name__ == "__main__":
         gemms()
     elif len(sys.argv) > 1 and sys.argv[1] == "elementwise":
         elementwise()
+    elif len(sys.argv) > 1 and sys.argv[1] == "attention":
+        attention()
     else:
         accumulate(int(sys.argv[2]) if len(sys.argv) > 2 else 1 << 26)
