@@ -137,6 +137,7 @@ PROTOTYPES = {
     "ds_squad_head": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                 C.c_float, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "ds_classifier_head": (C.c_int, [C.c_int] * 5 + [C.c_void_p] * 6 + [C.c_float, C.c_float] + [C.c_void_p] * 11),
+    "ds_regression_head": (C.c_int, [C.c_int] * 4 + [C.c_void_p] * 6 + [C.c_float, C.c_float] + [C.c_void_p] * 11),
     "ds_nmt_loss_head_workspace_bytes": (C.c_size_t, [C.c_int] * 3),
     "ds_nmt_loss_head": (C.c_int, [C.c_int] * 4 + [C.c_void_p] * 4 + [C.c_int, C.c_float] + [C.c_void_p] * 4 + [C.c_size_t, C.c_void_p]),
     "ds_xlnet_squad_head_workspace_bytes": (C.c_size_t, [C.c_int] * 4),

@@ -129,7 +129,8 @@ __global__ void head_clear_kernel(float* loss) { *loss = 0.f; }
 // one block: logits, loss = scale * (mean CE + l2_scale * sum(Wfc^2) / 2), dlogits = d loss / d logits
 __global__ __launch_bounds__(256) void classifier_loss_kernel(int B, int H, int C, const float* __restrict__ pooled,
                                                               const float* __restrict__ wfc, const float* __restrict__ bfc,
-                                                              const int32_t* __restrict__ labels, float l2_scale, float scale,
+                                                              const int32_t* __restrict__ labels, const float* __restrict__ targets,
+                                                              float l2_scale, float scale,
                                                               float* __restrict__ logits, float* __restrict__ dlogits,
                                                               float* __restrict__ loss) {
   __shared__ float red[4];
@@ -155,6 +156,21 @@ __global__ __launch_bounds__(256) void classifier_loss_kernel(int B, int H, int 
   __syncthreads();
   if (threadIdx.x == 0) {
     float total = l2_scale * 0.5f * (red[0] + red[1] + red[2] + red[3]);
+    if (targets) {
+      // regression (bert.py:627-631, C = 1): the prediction is [B, 1] and the labels placeholder is [B]
+      // (bert_finetune.py:212), so `prediction - labels` broadcasts to [B, B] and reduce_mean runs over every pair:
+      // loss = sum_i sum_j (z_i - y_j)^2 / B^2, d loss / d z_i = 2 (z_i - mean(y)) / B
+      float ysum = 0.f;
+      for (int j = 0; j < B; ++j) ysum += targets[j];
+      for (int i = 0; i < B; ++i) {
+        float acc = 0.f;
+        for (int j = 0; j < B; ++j) { const float d = logits[i] - targets[j]; acc += d * d; }
+        total += acc / ((float)B * (float)B);
+        dlogits[i] = 2.f * (logits[i] - ysum / (float)B) * scale / (float)B;
+      }
+      *loss = total * scale;
+      return;
+    }
     for (int b = 0; b < B; ++b) {
       const float* l = logits + (int64_t)b * C;
       float mx = l[0];
@@ -236,14 +252,14 @@ __global__ __launch_bounds__(256) void zero_rows_kernel(int64_t total, int S, in
 
 template <typename T>
 int classifier_head_t(int B, int S, int H, int C, const void* x, const float* wp, const float* bp, const float* wfc, const float* bfc,
-                      const int32_t* labels, float l2_scale, float scale, float* loss, float* pooled, float* logits, float* dlogits,
-                      float* dz, void* dx, float* dwp, float* dbp, float* dwfc, float* dbfc, hipStream_t s) {
+                      const int32_t* labels, const float* targets, float l2_scale, float scale, float* loss, float* pooled, float* logits,
+                      float* dlogits, float* dz, void* dx, float* dwp, float* dbp, float* dwfc, float* dbfc, hipStream_t s) {
   // pooled[b][j] = tanh(x[b, token 0] . Wp[:, j] + bp[j])
   hipLaunchKernelGGL(head_clear_kernel, dim3(1), dim3(1), 0, s, loss);
   hipLaunchKernelGGL((ds_small_dense_kernel<T, 1>), dim3((H + 63) / 64, B), dim3(1024), 0, s, H, 0, H, (const T*)x, (int64_t)S * H,
                      (const float*)nullptr, (int64_t)0, wp, bp, pooled);
   DS_CHECK_LAUNCH();
-  hipLaunchKernelGGL(classifier_loss_kernel, dim3(1), dim3(256), 0, s, B, H, C, pooled, wfc, bfc, labels, l2_scale, scale, logits,
+  hipLaunchKernelGGL(classifier_loss_kernel, dim3(1), dim3(256), 0, s, B, H, C, pooled, wfc, bfc, labels, targets, l2_scale, scale, logits,
                      dlogits, loss);
   DS_CHECK_LAUNCH();
   if (!dx && !dwp) return DS_OK;
@@ -318,10 +334,28 @@ extern "C" int ds_classifier_head(int dtype, int batch, int seq, int hidden, int
   const bool wg = d_pooler_w || d_pooler_b || d_fc_w || d_fc_b;
   DS_CHECK_ARG(!wg || (d_pooler_w && d_pooler_b && d_fc_w && d_fc_b), "ds_classifier_head: pass all four weight gradients or none");
   if (dtype == DS_BF16)
-    return classifier_head_t<bf16>(batch, seq, hidden, num_labels, x, pooler_w, pooler_b, fc_w, fc_b, labels, l2_scale, loss_scale, loss,
-                                   pooled, logits, dlogits, dz, dx, d_pooler_w, d_pooler_b, d_fc_w, d_fc_b, (hipStream_t)stream);
-  return classifier_head_t<float>(batch, seq, hidden, num_labels, x, pooler_w, pooler_b, fc_w, fc_b, labels, l2_scale, loss_scale, loss,
-                                  pooled, logits, dlogits, dz, dx, d_pooler_w, d_pooler_b, d_fc_w, d_fc_b, (hipStream_t)stream);
+    return classifier_head_t<bf16>(batch, seq, hidden, num_labels, x, pooler_w, pooler_b, fc_w, fc_b, labels, nullptr, l2_scale, loss_scale,
+                                   loss, pooled, logits, dlogits, dz, dx, d_pooler_w, d_pooler_b, d_fc_w, d_fc_b, (hipStream_t)stream);
+  return classifier_head_t<float>(batch, seq, hidden, num_labels, x, pooler_w, pooler_b, fc_w, fc_b, labels, nullptr, l2_scale, loss_scale,
+                                  loss, pooled, logits, dlogits, dz, dx, d_pooler_w, d_pooler_b, d_fc_w, d_fc_b, (hipStream_t)stream);
+}
+
+extern "C" int ds_regression_head(int dtype, int batch, int seq, int hidden, const void* x, const float* pooler_w, const float* pooler_b,
+                                  const float* fc_w, const float* fc_b, const float* targets, float l2_scale, float loss_scale,
+                                  float* loss, float* pooled, float* prediction, float* dprediction, float* dz, void* dx,
+                                  float* d_pooler_w, float* d_pooler_b, float* d_fc_w, float* d_fc_b, void* stream) {
+  DS_CHECK_ARG(dtype == DS_F32 || dtype == DS_BF16, "ds_regression_head: dtype %d", dtype);
+  DS_CHECK_ARG(batch > 0 && seq > 0 && hidden > 0, "ds_regression_head: non-positive shape");
+  DS_CHECK_ARG(batch <= 64, "ds_regression_head: batch (%d) must be at most 64", batch);
+  DS_CHECK_ARG(x && pooler_w && pooler_b && fc_w && fc_b && targets && loss && pooled && prediction && dprediction && dz,
+               "ds_regression_head: null pointer");
+  const bool wg = d_pooler_w || d_pooler_b || d_fc_w || d_fc_b;
+  DS_CHECK_ARG(!wg || (d_pooler_w && d_pooler_b && d_fc_w && d_fc_b), "ds_regression_head: pass all four weight gradients or none");
+  if (dtype == DS_BF16)
+    return classifier_head_t<bf16>(batch, seq, hidden, 1, x, pooler_w, pooler_b, fc_w, fc_b, nullptr, targets, l2_scale, loss_scale, loss,
+                                   pooled, prediction, dprediction, dz, dx, d_pooler_w, d_pooler_b, d_fc_w, d_fc_b, (hipStream_t)stream);
+  return classifier_head_t<float>(batch, seq, hidden, 1, x, pooler_w, pooler_b, fc_w, fc_b, nullptr, targets, l2_scale, loss_scale, loss,
+                                  pooled, prediction, dprediction, dz, dx, d_pooler_w, d_pooler_b, d_fc_w, d_fc_b, (hipStream_t)stream);
 }
 
 extern "C" int ds_squad_head(int dtype, int batch, int seq, int hidden, const void* x, const float* w, const float* bias,

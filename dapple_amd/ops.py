@@ -271,6 +271,33 @@ def classifier_head(x, batch, seq, pooler_w, pooler_b, fc_w, fc_b, labels, grads
     return loss, logits, pooled, dx
 
 
+def regression_head(x, batch, seq, pooler_w, pooler_b, fc_w, fc_b, targets, grads=None, need_dx=True, l2_scale=1e-3,
+                    loss_scale=1.0):
+    """pooler_stage (modeling_slice.py:849-868) + build_output_layer_regression (bert.py:615-640) on the stage's sequence
+    output ``x [batch*seq, hidden]``; ``targets`` fp32 [batch].  The loss is the reference graph's: the mean over every
+    (prediction, label) pair of the squared difference (a [batch, 1] - [batch] broadcast) plus the l2 term.  Returns
+    (loss [1] fp32 on the device, prediction [batch, 1], pooled [batch, hidden], dx or None)."""
+    _need_cuda(x, pooler_w, pooler_b, fc_w, fc_b, targets)
+    hidden = x.shape[-1]
+    if x.numel() != batch * seq * hidden or tuple(pooler_w.shape) != (hidden, hidden) or tuple(fc_w.shape) != (hidden, 1):
+        raise ValueError("regression_head: x must be [batch*seq, hidden], pooler_w [hidden, hidden], fc_w [hidden, 1]")
+    if targets.dtype != torch.float32 or targets.numel() != batch:
+        raise ValueError("regression_head: targets must be fp32 [batch]")
+    grads = tuple(grads) if grads is not None else (None,) * 4
+    for t in (pooler_w, pooler_b, fc_w, fc_b) + grads:
+        if t is not None and (t.dtype != torch.float32 or not t.is_contiguous()):
+            raise ValueError("regression_head: weights and their gradients must be contiguous fp32")
+    f32 = dict(dtype=torch.float32, device=x.device)
+    loss, pooled = torch.empty(1, **f32), torch.empty(batch, hidden, **f32)
+    pred, dpred, dz = torch.empty(batch, 1, **f32), torch.empty(batch, 1, **f32), torch.empty(batch, hidden, **f32)
+    dx = torch.empty_like(x) if need_dx else None
+    check(_lib.load().ds_regression_head(dtype_code(x), batch, seq, hidden, ptr(x), ptr(pooler_w), ptr(pooler_b), ptr(fc_w), ptr(fc_b),
+                                         ptr(targets), l2_scale, loss_scale, ptr(loss), ptr(pooled), ptr(pred), ptr(dpred), ptr(dz),
+                                         ptr(dx), ptr(grads[0]), ptr(grads[1]), ptr(grads[2]), ptr(grads[3]),
+                                         _lib.current_stream()), "ds_regression_head")
+    return loss, pred, pooled, dx
+
+
 XLNET_HEAD_SHAPES = {"start_w": lambda h: (h,), "start_b": lambda h: (1,), "end_w0": lambda h: (2 * h, h), "end_b0": lambda h: (h,),
                      "ln_gamma": lambda h: (h,), "ln_beta": lambda h: (h,), "end_w1": lambda h: (h,), "end_b1": lambda h: (1,),
                      "ans_w0": lambda h: (2 * h, h), "ans_b0": lambda h: (h,), "ans_w1": lambda h: (h,)}

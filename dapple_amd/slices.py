@@ -236,16 +236,17 @@ class BertFinetuneSlice(object):
             self.output_bias = torch.zeros(2, device="cuda")
             self.d_output_weights = torch.zeros_like(self.output_weights)
             self.d_output_bias = torch.zeros_like(self.output_bias)
-        elif self.is_last and model_type == 'classification':   # bert.py:463-464
+        elif self.is_last and model_type in ('classification', 'regression'):   # bert.py:463-466
             # bert/pooler/dense (modeling_slice.py:862-866, truncated normal) and src-output-layer/FC
             # (bert.py:644-652: xavier weights [hidden, 2], biases 1e-4)
             g = torch.Generator().manual_seed(seed + 2)
             H = bert_config.hidden_size
             self.pooler_kernel = (torch.randn(H, H, generator=g) * bert_config.initializer_range).cuda()
             self.pooler_bias = torch.zeros(H, device="cuda")
-            limit = (6.0 / (H + 2)) ** 0.5
-            self.fc_weights = ((torch.rand(H, 2, generator=g) * 2 - 1) * limit).cuda()
-            self.fc_biases = torch.full((2,), 1e-4, device="cuda")
+            nout = 2 if model_type == 'classification' else 1        # num_outputs, bert.py:646 / :619
+            limit = (6.0 / (H + nout)) ** 0.5
+            self.fc_weights = ((torch.rand(H, nout, generator=g) * 2 - 1) * limit).cuda()
+            self.fc_biases = torch.full((nout,), 1e-4, device="cuda")
             self.head_grads = [torch.zeros_like(t) for t in (self.pooler_kernel, self.pooler_bias, self.fc_weights, self.fc_biases)]
 
     def build_output_layer_squad(self, sequence_output, is_training=False):
@@ -280,6 +281,23 @@ class BertFinetuneSlice(object):
         self.loss, self.logits, self.pooled_output, dx = ops.classifier_head(
             x, B, S, self.pooler_kernel, self.pooler_bias, self.fc_weights, self.fc_biases, y, self.head_grads)
         self.predictions = torch.softmax(self.logits, -1)[:, 1]          # bert.py:654
+        self.stage_outputs = [sequence_output, self.loss]
+        return dx
+
+    def build_output_layer_regression(self, sequence_output):
+        """pooler_stage and bert.py:615-640 on the last device: one output per sample, loss = the reference graph's
+        ``reduce_mean(pow(prediction - labels, 2))`` (prediction [batch, 1] against the [batch] labels: the mean over every
+        pair) + the FC weights' l2 regulariser.  Returns the gradient of the loss w.r.t. ``sequence_output``; the head's
+        weight gradients are added into ``head_grads``."""
+        from . import ops
+        if not (self.is_last and self.model_type == 'regression'):
+            raise ValueError("build_output_layer_regression: this device does not hold the regression layer")
+        B, S = self.input_ids.shape
+        y = torch.as_tensor(self.labels, dtype=torch.float32).cuda()
+        x = sequence_output.reshape(B * S, self.bert_config.hidden_size)
+        self.loss, self.logits, self.pooled_output, dx = ops.regression_head(
+            x, B, S, self.pooler_kernel, self.pooler_bias, self.fc_weights, self.fc_biases, y, self.head_grads)
+        self.predictions = self.logits                                     # bert.py:634-635
         self.stage_outputs = [sequence_output, self.loss]
         return dx
 

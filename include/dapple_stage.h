@@ -359,6 +359,18 @@ int ds_classifier_head(int dtype, int batch, int seq, int hidden, int num_labels
                        float loss_scale, float* loss, float* pooled, float* logits, float* dlogits, float* dz, void* dx,
                        float* d_pooler_w, float* d_pooler_b, float* d_fc_w, float* d_fc_b, void* stream);
 
+/* Pooler and regression head of the last BERT stage: pooler_stage (bert/models/bert/modeling_slice.py:849-868) and
+ * build_output_layer_regression, bert/models/bert/bert.py:615-640: prediction = fully_connected(pooled) to ONE output
+ * (weights src-output-layer/FC/weights [hidden, 1]), loss = reduce_mean(pow(prediction - labels, 2)) + the l2 regulariser.
+ * The prediction is [batch, 1] and the labels placeholder [batch] (bert_finetune.py:212), so the difference broadcasts to
+ * [batch, batch] and the mean runs over every (prediction, label) pair: loss = sum_i sum_j (z_i - y_j)^2 / batch^2 +
+ * l2_scale * sum(FC weights^2) / 2.  This is what the reference's graph computes and what is computed here.
+ *   targets fp32 [batch]; prediction, dprediction fp32 [batch] out; everything else as ds_classifier_head.  batch <= 64. */
+int ds_regression_head(int dtype, int batch, int seq, int hidden, const void* x, const float* pooler_w, const float* pooler_b,
+                       const float* fc_w, const float* fc_b, const float* targets, float l2_scale, float loss_scale,
+                       float* loss, float* pooled, float* prediction, float* dprediction, float* dz, void* dx,
+                       float* d_pooler_w, float* d_pooler_b, float* d_fc_w, float* d_fc_b, void* stream);
+
 /* Output projection and loss of the GNMT model on the last device: gnmt/nmt/model.py:685-686 (logits =
  * output_layer(rnn_output); output_layer is a Dense without bias, :497-499) and _compute_loss :824-838
  * (loss = sum(sparse_softmax_cross_entropy(target_output, logits) * sequence_mask(target_sequence_length)) / batch_size).

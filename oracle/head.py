@@ -52,6 +52,18 @@ def classification_loss(sequence_output, pooler_kernel, pooler_bias, fc_weights,
     return loss, logits, pooled
 
 
+def regression_loss(sequence_output, pooler_kernel, pooler_bias, fc_weights, fc_biases, labels, l2_scale=1e-3):
+    """build_output_layer_regression, bert/models/bert/bert.py:615-640, behind pooler_stage.  sequence_output
+    [batch, seq, hidden], fc_weights [hidden, 1], labels float [batch] (the placeholder's shape,
+    bert_finetune.py:212).  Returns (loss, prediction [batch, 1], pooled)."""
+    first_token_tensor = sequence_output[:, 0, :]                                    # modeling_slice.py:861
+    pooled = torch.tanh(first_token_tensor @ pooler_kernel + pooler_bias)            # :862-866
+    prediction = pooled @ fc_weights + fc_biases                                     # bert.py:617-625, [batch, 1]
+    # :628-631: [batch, 1] - [batch] broadcasts to [batch, batch]; reduce_mean runs over all of it
+    loss = ((prediction - labels) ** 2).mean() + l2_scale * 0.5 * (fc_weights ** 2).sum()
+    return loss, prediction, pooled
+
+
 def xlnet_squad_loss(output, w, cls_index, start_positions, end_positions, is_impossible, p_mask, dropout_mask=None):
     """XLnetLoss.call, xlnet/losses/xlnet_loss.py:36-120, line by line.
 

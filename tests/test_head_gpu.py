@@ -124,3 +124,33 @@ def test_classifier_head_matches_oracle(dtype, tol, B, S, H, C):
     assert_close(dx2, 4 * gx.reshape(B * S, H), tol, "scaled dx")
     with pytest.raises(ValueError):
         ops.classifier_head(x, B, S, wp, bp, wf, bf, y.long())
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 2e-2)])
+@pytest.mark.parametrize("B,S,H", [(2, 16, 64), (6, 128, 1024), (1, 4, 8)])
+def test_regression_head_matches_oracle(dtype, tol, B, S, H):
+    r = np.random.default_rng(B * S + H)
+    x = dev(r.standard_normal((B * S, H)), dtype)
+    wp = dev(r.standard_normal((H, H)) / np.sqrt(H), torch.float32)
+    bp = dev(r.standard_normal(H) * 0.1, torch.float32)
+    wf = dev(r.standard_normal((H, 1)) * 0.3, torch.float32)
+    bf = dev(np.full(1, 1e-4), torch.float32)
+    y_np = r.standard_normal(B).astype(np.float32)
+    y = torch.as_tensor(y_np).cuda()
+    grads = [torch.ones_like(t) for t in (wp, bp, wf, bf)]
+    loss, pred, pooled, dx = ops.regression_head(x, B, S, wp, bp, wf, bf, y, grads)
+    xo = x.cpu().double().reshape(B, S, H).requires_grad_(True)
+    ws = [t.cpu().double().requires_grad_(True) for t in (wp, bp, wf, bf)]
+    lo, po, zo = oh.regression_loss(xo, ws[0], ws[1], ws[2], ws[3], torch.as_tensor(y_np).double())
+    gx, *gw = torch.autograd.grad(lo, [xo] + ws)
+    assert_close(loss, lo.reshape(1), tol, "loss")
+    assert_close(pred, po, tol, "prediction")
+    assert_close(pooled, zo, tol, "pooled")
+    assert_close(dx, gx.reshape(B * S, H), tol, "dx")
+    for g, ref, name in zip(grads, gw, ("pooler kernel", "pooler bias", "FC weights", "FC biases")):
+        assert_close(g - 1, ref, tol, "d " + name, floor=float(gw[2].abs().max()) if name == "FC biases" else None)
+    loss2, _, _, dx2 = ops.regression_head(x, B, S, wp, bp, wf, bf, y, None, loss_scale=0.5)
+    assert_close(loss2, 0.5 * lo.reshape(1), tol, "scaled loss")
+    assert_close(dx2, 0.5 * gx.reshape(B * S, H), tol, "scaled dx")
+    with pytest.raises(ValueError):
+        ops.regression_head(x, B, S, wp, bp, wf, bf, y.double())

@@ -70,6 +70,38 @@ def test_classification_head_matches_library_and_brute_force():
     assert abs(oh.classification_loss(x2, wp, bp, wf, bf, y)[0].item() - loss.item()) < 1e-12
 
 
+def test_regression_head_is_the_pairwise_mean_of_the_reference_graph():
+    """bert.py:627-631 subtracts the [batch] label placeholder (bert_finetune.py:212) from the [batch, 1] prediction:
+    the difference is [batch, batch].  Pinned by scalar loops over every pair, by the closed form
+    mean_i (z_i - mean y)^2 + var(y), and by the case of one sample, where it is the plain squared error."""
+    torch.manual_seed(5)
+    B, S, H = 4, 3, 6
+    x = torch.randn(B, S, H, dtype=torch.float64)
+    wp, bp = torch.randn(H, H, dtype=torch.float64) * 0.5, torch.randn(H, dtype=torch.float64) * 0.1
+    wf = (torch.randn(H, 1, dtype=torch.float64) * 0.5).requires_grad_(True)
+    bf = torch.full((1,), 1e-4, dtype=torch.float64)
+    y = torch.randn(B, dtype=torch.float64)
+    loss, pred, pooled = oh.regression_loss(x, wp, bp, wf, bf, y, l2_scale=1e-3)
+    assert tuple(pred.shape) == (B, 1)
+    z = []
+    for b in range(B):
+        pz = [math.tanh(sum(x[b, 0, i].item() * wp[i, j].item() for i in range(H)) + bp[j].item()) for j in range(H)]
+        z.append(sum(pz[j] * wf[j, 0].item() for j in range(H)) + bf[0].item())
+        assert abs(z[b] - pred[b, 0].item()) < 1e-12
+    reg = 1e-3 * 0.5 * float((wf.detach() ** 2).sum())
+    brute = sum((z[i] - y[j].item()) ** 2 for i in range(B) for j in range(B)) / (B * B)
+    assert abs(loss.item() - (brute + reg)) < 1e-12
+    ym = float(y.mean())
+    closed = sum((zi - ym) ** 2 for zi in z) / B + float(((y - ym) ** 2).mean())
+    assert abs(loss.item() - (closed + reg)) < 1e-12
+    # d loss / d prediction_i = 2 (z_i - mean y) / B
+    (g,) = torch.autograd.grad(loss, pred, retain_graph=True)
+    assert torch.allclose(g[:, 0], torch.tensor([2 * (zi - ym) / B for zi in z], dtype=torch.float64), atol=1e-12)
+    # one sample: the ordinary squared error
+    l1, p1, _ = oh.regression_loss(x[:1], wp, bp, wf, bf, y[:1], l2_scale=0.0)
+    assert abs(l1.item() - (p1[0, 0].item() - y[0].item()) ** 2) < 1e-12
+
+
 def _xlnet_head_case(seed, S, B, H, std=0.3):
     g = torch.Generator().manual_seed(seed)
     r = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64)
