@@ -7,7 +7,7 @@ sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
 
 
 def pytest_configure(config):
-    config.addinivalue_line("markers", "gpu: needs a real MI355X (run under gpurun)")
+    config.addinivalue_line("markers", "gpu: needs a real MI355X")
 
 
 def pytest_collection_modifyitems(config, items):

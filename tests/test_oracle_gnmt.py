@@ -109,7 +109,7 @@ def test_encoder_structure_residual_from_third_layer():
 
 
 def test_parameter_count_of_config():
-    # C3 = 79.7 M LSTM parameters + 32000 x 1024 embedding
+    # the GNMT-16 encoder configuration = 79.7 M LSTM parameters + 32000 x 1024 embedding
     w = synthetic.gnmt_weights(0, 8, 1024, 32)          # tiny vocab: count the cells only
     cells = sum(v.size for k, v in w.items() if "embedding" not in k)
     assert cells == 2 * (2048 * 4096 + 4096) + (3072 * 4096 + 4096) + 6 * (2048 * 4096 + 4096)

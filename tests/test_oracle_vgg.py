@@ -52,7 +52,7 @@ def test_relu_gradient_is_zero_at_zero():
 
 
 def test_parameter_counts_match_reference_profile():
-    # SURVEY: 16 convs = 20 024 384 parameters, the reference's 14-conv split 15 304 768
+    # 16 convs = 20 024 384 parameters, the reference's 14-conv split 15 304 768
     def count(layers):
         return sum(v.size for v in synthetic.vgg_weights(0, synthetic.scale_layers(layers, 1)).values())
     assert count(synthetic.VGG19_CONV_STACK) == 20024384
