@@ -1,0 +1,196 @@
+"""The stage planner (dapple_amd/planner.py) against closed forms, brute force on small cases, and the plan the
+reference's own model file hard-codes for VGG19 (vgg19/applications/vgg19_slice_model.py:280-335: 15 replicas up to
+block5_conv2, one device from block5_conv3 on), which the planner must find from the reference's profile of that model.
+Host logic only."""
+import itertools
+import os
+
+import pytest
+
+from dapple_amd import planner as P
+
+HERE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "profiles")
+
+
+def chain_profile(times, acts, params):
+    lines = ["node%d -- L%02d -- forward_compute_time=%g, backward_compute_time=%g, activation_size=%g, parameter_size=%g"
+             % (i + 1, i, t / 3.0, 2 * t / 3.0, a, p) for i, (t, a, p) in enumerate(zip(times, acts, params))]
+    lines += ["\tnode%d -- node%d" % (i + 1, i + 2) for i in range(len(times) - 1)]
+    return "\n".join(lines)
+
+
+def test_parse_node_and_list_activation():
+    n = P.parse_node("node5 -- layer_0 -- forward_compute_time=2.69, backward_compute_time=4.47, activation_size=4325376, parameter_size=50384896")
+    assert (n.node_id, n.desc, n.forward_compute_time, n.backward_compute_time) == ("node5", "layer_0", 2.69, 4.47)
+    assert n.activation_size == 4325376.0 and n.parameter_size == 50384896.0
+    m = P.parse_node("node7 -- cell -- forward_compute_time=1.0, backward_compute_time=2.0, activation_size=[10.0; 20.5; 1.5], parameter_size=3.000")
+    assert m.activation_size == 32.0
+    with pytest.raises(ValueError):
+        P.parse_node("node1 -- x -- forward_compute_time=1.0, backward_compute_time=2.0")
+
+
+def test_chain_states_are_prefix_sums():
+    times, acts, params = [3.0, 6.0, 9.0, 12.0], [10.0, 20.0, 30.0, 40.0], [1.0, 2.0, 3.0, 4.0]
+    perf = P.prepare(chain_profile(times, acts, params))
+    assert [s.desc for s in perf.states] == ["L00", "L01", "L02", "L03"]
+    assert perf.all_predecessor_ids == [[], [0], [0, 1], [0, 1, 2]]
+    for j in range(4):
+        assert perf.compute_times[0][j] == pytest.approx(sum(times[:j + 1]) / 1000.0)
+        assert perf.output_activation_sizes[j] == acts[j]
+        for i in range(1, 5):
+            want = sum(times[i:j + 1]) / 1000.0 if j >= i else -1.0
+            assert perf.compute_times[i][j] == pytest.approx(want)
+            assert perf.parameter_sizes[i][j] == pytest.approx(sum(params[i:j + 1]) if j >= i else -1.0)
+    m = P.Model(perf, 2, 8)        # times and activations scale with the batch, parameters do not
+    assert m.perf.compute_times[0][3] == pytest.approx(4 * 0.030)
+    assert m.perf.output_activation_sizes[1] == 80.0 and m.perf.parameter_sizes[0][3] == 10.0
+    assert m.peak_activation_per_batch == 50.0
+
+
+def test_states_of_a_branching_graph_are_the_cuts():
+    """a -> b -> d, a -> c -> d, d -> e.  Every state must be a down-closed set of nodes (a legal set of leading
+    layers), the states must come in an order in which they only grow along the DAG's edges, the bytes crossing a cut are those
+    of its augmented antichain, and the cuts found must be exactly the down-sets with one "frontier": brute force."""
+    node = lambda i, d, t, a: "node%d -- %s -- forward_compute_time=%g, backward_compute_time=0, activation_size=%g, parameter_size=1" % (i, d, t, a)
+    text = "\n".join([node(1, "a", 1, 100), node(2, "b", 2, 10), node(3, "c", 4, 20), node(4, "d", 8, 5), node(5, "e", 16, 1),
+                      "\tnode1 -- node2", "\tnode1 -- node3", "\tnode2 -- node4", "\tnode3 -- node4", "\tnode4 -- node5"])
+    g = P.ProfileGraph.from_str(text)
+    perf = P.prepare(text)
+    t = {"node1": 1, "node2": 2, "node3": 4, "node4": 8, "node5": 16}
+    downsets = []
+    for st in perf.states:
+        members = set(st.antichain)
+        for a in st.antichain:
+            members |= g.predecessors(a)
+        for mnode in members:                                  # down-closed
+            assert g.predecessors(mnode) <= members
+        assert st.compute_time == pytest.approx(sum(t[x] for x in members) / 1000.0)
+        assert st.output_activation_size == sum(g.nodes[x].activation_size for x in st.antichain)
+        downsets.append(frozenset(members))
+    assert downsets[0] == {"node1"} and downsets[-1] == set(t)
+    for i, pre in enumerate(perf.all_predecessor_ids):
+        for k in pre:
+            assert k < i and downsets[k] < downsets[i]
+    # brute force: all non-empty down-closed subsets that contain the source
+    all_down = set()
+    for r in range(1, 6):
+        for sub in itertools.combinations(sorted(t), r):
+            s = set(sub)
+            if "node1" in s and all(g.predecessors(x) <= s for x in s):
+                all_down.add(frozenset(s))
+    assert set(downsets) == all_down and len(downsets) == len(all_down)
+    # the cut {b}: a is still needed by c, so a's output crosses as well
+    b = perf.states[downsets.index(frozenset({"node1", "node2"}))]
+    assert sorted(b.antichain) == ["node1", "node2"] and b.output_activation_size == 110.0
+    # the cut {b, c}: the reference decides per node of the antichain - seen from b, a still feeds c (and from c, b) - so
+    # a's output is counted although both its consumers are before the cut (torch_graph_py.rs:360-376); kept as it is
+    bc = perf.states[downsets.index(frozenset({"node1", "node2", "node3"}))]
+    assert sorted(bc.antichain) == ["node1", "node2", "node3"] and bc.output_activation_size == 130.0
+    # the cut {d}: only d crosses
+    dd = perf.states[downsets.index(frozenset({"node1", "node2", "node3", "node4"}))]
+    assert dd.antichain == ["node4"] and dd.output_activation_size == 5.0
+
+
+def test_device_placements():
+    d = P.Devices(16, [8, 16])
+    empty = tuple([False] * 16)
+    got = {tuple(sorted(p.gids)) for p in d.next_cards(empty, 8)}
+    assert got == {tuple(range(8)), (0, 1, 2, 3, 8, 9, 10, 11)}             # one fresh machine, or scattered over both
+    occ = tuple([True] * 4 + [False] * 12)
+    got = {tuple(sorted(p.gids)) for p in d.next_cards(occ, 2)}
+    assert got == {(8, 9), (4, 5), (4, 8)}                                  # fresh machine, append, scatter
+    got = {tuple(sorted(p.gids)) for p in d.next_cards(occ, 12)}
+    assert got == {tuple(range(4, 16))}
+    with pytest.raises(ValueError):
+        d.next_cards(occ, 13)
+    two = d.next_cards_with_replica(empty, 1, 2)                            # two rounds of one GPU
+    assert {tuple(sorted(p.gids)) for p in two} == {(0, 1), (0, 8)}
+    for p in two:
+        assert sum(p.occupied) == 2 and all(p.occupied[i] for i in p.gids)
+    assert not d.is_cross_machine_within({0, 7}) and d.is_cross_machine_within({7, 8})
+    assert not d.is_cross_machine_from_to({8}, {15}) and d.is_cross_machine_from_to({0}, {15})
+
+
+def test_cost_models_closed_forms():
+    d = P.Devices(16, [8, 16])
+    size = 3.0e9
+    assert d.all_reduce_time({3}, size) == 0.0
+    assert d.all_reduce_time(set(range(8)), size) == pytest.approx(size * 2 * (7 / 8.0) / 25e9 / 4)
+    assert d.all_reduce_time(set(range(16)), size) == pytest.approx(size * 2 * (15 / 16.0) / 3e9)
+    assert d.split_concat_all2all_time({0, 1}, {2, 3}, size) == pytest.approx(size / 25e9)
+    assert d.split_concat_all2all_time({0, 1, 8}, {9}, size) == pytest.approx(size / 3 * 2 / 1e9)   # two of three senders are remote
+    assert d.split_concat_all2all_time({0, 1}, {7, 8}, size) == pytest.approx(size / 3e9)           # receivers span machines
+    other = P.Devices(16, [8, 16], P.Network(intra_p2p=100e9, inter_p2p=50e9, inter_collective=40e9))
+    assert other.split_concat_all2all_time({0}, {8}, size) == pytest.approx(size / 50e9)
+
+
+def test_single_stage_speedup_is_data_parallel_closed_form():
+    text = chain_profile([10.0, 20.0, 30.0], [1e6, 1e6, 1e6], [4e8, 4e8, 4e8])
+    o = P.SyncOrchestrate(text, 1, 64, [4])
+    total = o.m.perf.compute_times[0][-1]
+    gids = frozenset(range(4))
+    s = P.sync_pipeline_speedup_analytical(o.d, o.m, 4, total / 4, [(0, 2, 1, gids)])
+    assert s == pytest.approx(total / (total / 4 + o.d.all_reduce_time(gids, 1.2e9)))
+    assert P.sync_pipeline_speedup_analytical(o.d, o.m, 128, total / 4, [(0, 2, 1, gids)]) == 0.0   # no micro-batch left
+
+
+@pytest.mark.parametrize("seps", [[4], [2, 4]])
+def test_two_stage_plan_is_the_brute_force_optimum(seps):
+    times = [5.0, 9.0, 2.0, 7.0, 11.0, 3.0, 8.0]
+    acts = [4e8, 1e6, 6e8, 2e6, 3e8, 1e6, 1e6]
+    o = P.SyncOrchestrate(chain_profile(times, acts, [1e7] * 7), 1, 32, seps)
+    plan = o.plan_for(2, True)                               # two slots of two replicas, one slot per stage
+    assert plan.replicas == 2 and len(plan.stages) == 2
+    cut = plan.stages[0][1]
+    assert plan.stages[1][0] == cut and plan.stages[0][0] == 0 and plan.stages[1][1] == 6
+    ct, oas = o.m.perf.compute_times, o.m.perf.output_activation_sizes
+    empty = tuple([False] * 4)
+
+    def bottleneck(c):                                       # states 0..c-1 | c..6, best placement of the two stages
+        best = None
+        first = [p for p in o.d.next_cards(empty, 2) if p.strategy == "fresh"] or o.d.next_cards(empty, 2)[:1]
+        for a in first:
+            for b in o.d.next_cards_with_replica(a.occupied, 1, 2):
+                t = max(ct[0][c - 1] / 2, ct[c][6] / 2, o.d.split_concat_all2all_time(a.gids, b.gids, 2 * oas[c - 1]))
+                best = t if best is None else min(best, t)
+        return best
+    brute = {c: bottleneck(c) for c in range(1, 7)}
+    got = max(ct[0][cut - 1] / 2, ct[cut][6] / 2,
+              o.d.split_concat_all2all_time(plan.stages[0][3], plan.stages[1][3], 2 * oas[cut - 1]))
+    assert got == pytest.approx(min(brute.values()))
+    # more freedom cannot make the bottleneck worse
+    full = o.compute_plan_sync(2, 2, False)
+    assert full[6][1][P._BEST].block <= got + 1e-12
+    sp, stages = o.orchestrate()
+    assert sp >= plan.speedup - 1e-12 and stages[0][0] == 0
+
+
+def test_vgg19_profile_gives_the_reference_15_to_1_plan():
+    """vgg-19-pbs-32 at global batch 2048 on two machines of 8 GPUs: the best plan is two stages, 15 GPUs of data
+    parallel replicas for conv1_1 .. conv5_2 and ONE GPU for conv5_3 .. loss - the split and the replica count that
+    vgg19/applications/vgg19_slice_model.py:280-335 and vgg19/run_15_1_pipeline.sh hard-code."""
+    o = P.conductor_from_torch_graph_and_seps(os.path.join(HERE, "vgg-19-pbs-32.txt"), 32, 2048, [8, 16])
+    speedup, stages = o.orchestrate()
+    assert [(s[0], s[1], s[2]) for s in stages] == [(0, 18, 15), (18, 24, 1)]
+    assert stages[0][3] == list(range(15)) and stages[1][3] == [15]
+    names = P.stage_layers(stages, o.m.perf)
+    assert names[0][0] == "Conv2d_1_1" and names[0][-1] == "Conv2d_5_2"
+    assert names[1][0] == "Conv2d_5_3" and names[1][-1] == "Loss"
+    assert 14.0 < speedup < 16.0
+    assert speedup == pytest.approx(max(r.speedup for r in o.res))
+
+
+def test_bert48_profile_two_gpus():
+    """bert-48-pbs-2 on two GPUs of one machine: a two-stage pipeline cut in the middle of the 48 equal encoder layers
+    (the embedding side holds layers 0..23).  The reference's model file hard-codes 23:25 (bert.py:419-430), one layer
+    off the planner's own cost model, which has no term that tells the two halves apart beyond the profile times."""
+    o = P.conductor_from_torch_graph_and_seps(os.path.join(HERE, "bert-48-pbs-2.txt"), 2, 16, [2])
+    perf = o.m.perf
+    assert len(perf.states) == 55 and perf.parameter_sizes[0][-1] == pytest.approx(sum(
+        float(l.split("parameter_size=")[1]) for l in open(os.path.join(HERE, "bert-48-pbs-2.txt")) if "parameter_size=" in l))
+    plan = o.plan_for(2, True)
+    names = P.stage_layers(plan.stages, perf)
+    assert names[0][-1] == "layer_23" and names[1][0] == "layer_24"
+    ct = perf.compute_times
+    cut = plan.stages[0][1]
+    assert max(ct[0][cut - 1], ct[cut][54]) == pytest.approx(min(max(ct[0][c - 1], ct[c][54]) for c in range(1, 55)))
