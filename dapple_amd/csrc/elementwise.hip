@@ -64,13 +64,21 @@ __global__ __launch_bounds__(256) void layernorm_fwd_kernel(int rows, int cols, 
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
   const T* xr = x + (int64_t)row * cols;
-  float v[NV][VEC];
+  float v[NV][VEC], gm[NV][VEC], bt[NV][VEC];
   float sum = 0.f;
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const int c = (lane + i * 64) * VEC;
     if (c < cols) {
       const V t = *reinterpret_cast<const V*>(xr + c);
+      // gamma and beta are fetched here, with x: read where they are used they would cost a second trip to memory
+      // behind the two reductions
+#pragma unroll
+      for (int e = 0; e < VEC; e += 4) {
+        const f32x4 g4 = *reinterpret_cast<const f32x4*>(gamma + c + e), b4 = *reinterpret_cast<const f32x4*>(beta + c + e);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) { gm[i][e + q] = g4[q]; bt[i][e + q] = b4[q]; }
+      }
 #pragma unroll
       for (int e = 0; e < VEC; ++e) { v[i][e] = to_f32(t[e]); sum += v[i][e]; }
     } else {
@@ -97,7 +105,7 @@ __global__ __launch_bounds__(256) void layernorm_fwd_kernel(int rows, int cols, 
     if (c < cols) {
       V o;
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) o[e] = from_f32<T>((v[i][e] - mean) * rstd * gamma[c + e] + beta[c + e]);
+      for (int e = 0; e < VEC; ++e) o[e] = from_f32<T>((v[i][e] - mean) * rstd * gm[i][e] + bt[i][e]);
       *reinterpret_cast<V*>(yr + c) = o;
     }
   }
@@ -132,20 +140,39 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(int rows, int cols, 
     for (int e = 0; e < VEC; ++e) pg[i][e] = pb[i][e] = ps[i][e] = 0.f;
   }
   const int row0 = (blockIdx.x * 4 + wave) * rows_per_wave;
+  // the next row's dy, x and statistics are fetched before this row is reduced and written: one trip to memory per
+  // wave, not one per row
+  V na[NV], nb[NV];
+  float nmean = 0.f, nrstd = 0.f;
+  auto fetch = [&](int row) {
+    if (row >= rows) return;
+    nmean = stats[2 * row]; nrstd = stats[2 * row + 1];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int c = (lane + i * 64) * VEC;
+      if (c < cols) {
+        na[i] = *reinterpret_cast<const V*>(dy + (int64_t)row * cols + c);
+        nb[i] = *reinterpret_cast<const V*>(x + (int64_t)row * cols + c);
+      }
+    }
+  };
+  fetch(row0);
   for (int r = 0; r < rows_per_wave; ++r) {
     const int row = row0 + r;
     if (row >= rows) break;
-    const float mean = stats[2 * row], rstd = stats[2 * row + 1];
-    const T* dyr = dy + (int64_t)row * cols;
-    const T* xr = x + (int64_t)row * cols;
+    const float mean = nmean, rstd = nrstd;
+    V ca[NV], cb[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) { ca[i] = na[i]; cb[i] = nb[i]; }
+    if (r + 1 < rows_per_wave) fetch(row + 1);
     float dyv[NV][VEC], xh[NV][VEC];
     float s1 = 0.f, s2 = 0.f;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int c = (lane + i * 64) * VEC;
       if (c < cols) {
-        const V a = *reinterpret_cast<const V*>(dyr + c);
-        const V b = *reinterpret_cast<const V*>(xr + c);
+        const V a = ca[i];
+        const V b = cb[i];
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
           dyv[i][e] = to_f32(a[e]);
@@ -522,7 +549,8 @@ extern "C" int ds_layernorm_fwd(int dtype, int rows, int cols, const void* x, co
                                 float eps, void* y, float* stats, void* stream) {
   DS_PROPAGATE(check_rows("ds_layernorm_fwd", dtype, rows, cols));
   DS_CHECK_ARG(x && gamma && beta && y, "ds_layernorm_fwd: null pointer");
-  DS_CHECK_ARG(ds_aligned16(x) && ds_aligned16(y), "ds_layernorm_fwd: x/y must be 16-byte aligned");
+  DS_CHECK_ARG(ds_aligned16(x) && ds_aligned16(y) && ds_aligned16(gamma) && ds_aligned16(beta),
+               "ds_layernorm_fwd: x, y, gamma and beta must be 16-byte aligned");
   if (dtype == DS_BF16) return layernorm_fwd_t<bf16>(rows, cols, x, gamma, beta, eps, y, stats, (hipStream_t)stream);
   return layernorm_fwd_t<float>(rows, cols, x, gamma, beta, eps, y, stats, (hipStream_t)stream);
 }
