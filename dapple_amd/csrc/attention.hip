@@ -156,6 +156,10 @@ __global__ __launch_bounds__(NTHREADS) void attn_fwd_kernel(AttnArgs a) {
   char* sk = lds;
   char* sv = lds + CHUNK * ROWB;
   float* adder = reinterpret_cast<float*>(lds + 2 * CHUNK * ROWB);
+  // the first K / V tiles are requested before anything else: the loads below queue behind them and the whole prologue
+  // costs one trip to memory (a mask row staged through LDS would otherwise be waited for before the tiles are asked for)
+  tile_fill(sk, base + a.H, a.ld, a.S < CHUNK ? a.S : CHUNK, wave, lane);
+  tile_fill(sv, base + 2 * a.H, a.ld, a.S < CHUNK ? a.S : CHUNK, wave, lane);
   for (int j = threadIdx.x; j < a.S; j += NTHREADS)
     adder[j] = a.key_mask ? (1.0f - a.key_mask[(int64_t)b * a.S + j]) * a.mask_value : 0.f;
   bf16x8 qf[4];
@@ -168,8 +172,10 @@ __global__ __launch_bounds__(NTHREADS) void attn_fwd_kernel(AttnArgs a) {
   for (int k0 = 0; k0 < a.S; k0 += CHUNK) {
     const int rows = a.S - k0 < CHUNK ? a.S - k0 : CHUNK;
     __syncthreads();
-    tile_fill(sk, base + a.H + (int64_t)k0 * a.ld, a.ld, rows, wave, lane);
-    tile_fill(sv, base + 2 * a.H + (int64_t)k0 * a.ld, a.ld, rows, wave, lane);
+    if (k0 > 0) {  // tile 0 was requested at the top
+      tile_fill(sk, base + a.H + (int64_t)k0 * a.ld, a.ld, rows, wave, lane);
+      tile_fill(sv, base + 2 * a.H + (int64_t)k0 * a.ld, a.ld, rows, wave, lane);
+    }
     __builtin_amdgcn_s_waitcnt(VMCNT0);
     __syncthreads();
     for (int kt = part * 32; kt < rows; kt += 32 * SPLIT) {
@@ -241,6 +247,10 @@ __global__ __launch_bounds__(NTHREADS) void attn_bwd_dq_kernel(AttnArgs a) {
   char* sk = lds;
   char* sv = lds + CHUNK * ROWB;
   float* adder = reinterpret_cast<float*>(lds + 2 * CHUNK * ROWB);
+  // the first K / V tiles are requested first: delta below needs its operands in registers, and waiting for them before
+  // asking for the tiles would cost a second trip to memory
+  tile_fill(sk, base + a.H, a.ld, a.S < CHUNK ? a.S : CHUNK, wave, lane);
+  tile_fill(sv, base + 2 * a.H, a.ld, a.S < CHUNK ? a.S : CHUNK, wave, lane);
   for (int j = threadIdx.x; j < a.S; j += NTHREADS)
     adder[j] = a.key_mask ? (1.0f - a.key_mask[(int64_t)b * a.S + j]) * a.mask_value : 0.f;
   bf16x8 qf[4], dof[4];
@@ -263,8 +273,10 @@ __global__ __launch_bounds__(NTHREADS) void attn_bwd_dq_kernel(AttnArgs a) {
   for (int k0 = 0; k0 < a.S; k0 += CHUNK) {
     const int rows = a.S - k0 < CHUNK ? a.S - k0 : CHUNK;
     __syncthreads();
-    tile_fill(sk, base + a.H + (int64_t)k0 * a.ld, a.ld, rows, wave, lane);
-    tile_fill(sv, base + 2 * a.H + (int64_t)k0 * a.ld, a.ld, rows, wave, lane);
+    if (k0 > 0) {  // tile 0 was requested at the top
+      tile_fill(sk, base + a.H + (int64_t)k0 * a.ld, a.ld, rows, wave, lane);
+      tile_fill(sv, base + 2 * a.H + (int64_t)k0 * a.ld, a.ld, rows, wave, lane);
+    }
     __builtin_amdgcn_s_waitcnt(VMCNT0);
     __syncthreads();
     for (int kt = part * 32; kt < rows; kt += 32 * SPLIT) {
@@ -314,6 +326,10 @@ __global__ __launch_bounds__(NTHREADS) void attn_bwd_dkv_kernel(AttnArgs a) {
   char* sdo = lds + CHUNK * ROWB;
   float* slse = reinterpret_cast<float*>(lds + 2 * CHUNK * ROWB);
   float* sdelta = slse + a.S;
+  // the first Q / dO tiles are requested first: lse and delta go through registers into LDS, and waiting for them before
+  // asking for the tiles would cost a second trip to memory
+  tile_fill(sq, base, a.ld, a.S < CHUNK ? a.S : CHUNK, wave, lane);
+  tile_fill(sdo, dobase, a.H, a.S < CHUNK ? a.S : CHUNK, wave, lane);
   for (int j = threadIdx.x; j < a.S; j += NTHREADS) {
     slse[j] = a.lse[((int64_t)b * a.N + hd) * a.S + j];
     sdelta[j] = a.delta[((int64_t)b * a.N + hd) * a.S + j];
@@ -331,8 +347,10 @@ __global__ __launch_bounds__(NTHREADS) void attn_bwd_dkv_kernel(AttnArgs a) {
   for (int q0 = 0; q0 < a.S; q0 += CHUNK) {
     const int rows = a.S - q0 < CHUNK ? a.S - q0 : CHUNK;
     __syncthreads();
-    tile_fill(sq, base + (int64_t)q0 * a.ld, a.ld, rows, wave, lane);
-    tile_fill(sdo, dobase + (int64_t)q0 * a.H, a.H, rows, wave, lane);
+    if (q0 > 0) {  // tile 0 was requested at the top
+      tile_fill(sq, base + (int64_t)q0 * a.ld, a.ld, rows, wave, lane);
+      tile_fill(sdo, dobase + (int64_t)q0 * a.H, a.H, rows, wave, lane);
+    }
     __builtin_amdgcn_s_waitcnt(VMCNT0);
     __syncthreads();
     for (int qt = part * 32; qt < rows; qt += 32 * SPLIT) {
