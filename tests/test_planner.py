@@ -3,13 +3,25 @@ reference's own model file hard-codes for VGG19 (vgg19/applications/vgg19_slice_
 block5_conv2, one device from block5_conv3 on), which the planner must find from the reference's profile of that model.
 Host logic only."""
 import itertools
+import json
 import os
 
 import pytest
 
 from dapple_amd import planner as P
 
-HERE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "profiles")
+FIXTURE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "planner_profiles.json")
+
+
+def profile_text(name):
+    """The profile in the text form the planner reads, rebuilt from the arrays of the fixture (measurements the reference
+    ships under profiling_results/, written by tests/golden/make_planner_fixtures.py)."""
+    with open(FIXTURE) as f:
+        prof = json.load(f)[name]
+    lines = ["%s -- %s -- forward_compute_time=%s, backward_compute_time=%s, activation_size=%s, parameter_size=%s" % tuple(n)
+             for n in prof["nodes"]]
+    lines += ["\t%s -- %s" % tuple(e) for e in prof["edges"]]
+    return "\n".join(lines)
 
 
 def chain_profile(times, acts, params):
@@ -169,7 +181,7 @@ def test_vgg19_profile_gives_the_reference_15_to_1_plan():
     """vgg-19-pbs-32 at global batch 2048 on two machines of 8 GPUs: the best plan is two stages, 15 GPUs of data
     parallel replicas for conv1_1 .. conv5_2 and ONE GPU for conv5_3 .. loss - the split and the replica count that
     vgg19/applications/vgg19_slice_model.py:280-335 and vgg19/run_15_1_pipeline.sh hard-code."""
-    o = P.conductor_from_torch_graph_and_seps(os.path.join(HERE, "vgg-19-pbs-32.txt"), 32, 2048, [8, 16])
+    o = P.SyncOrchestrate(profile_text("vgg-19-pbs-32"), 32, 2048, [8, 16])
     speedup, stages = o.orchestrate()
     assert [(s[0], s[1], s[2]) for s in stages] == [(0, 18, 15), (18, 24, 1)]
     assert stages[0][3] == list(range(15)) and stages[1][3] == [15]
@@ -184,10 +196,11 @@ def test_bert48_profile_two_gpus():
     """bert-48-pbs-2 on two GPUs of one machine: a two-stage pipeline cut in the middle of the 48 equal encoder layers
     (the embedding side holds layers 0..23).  The reference's model file hard-codes 23:25 (bert.py:419-430), one layer
     off the planner's own cost model, which has no term that tells the two halves apart beyond the profile times."""
-    o = P.conductor_from_torch_graph_and_seps(os.path.join(HERE, "bert-48-pbs-2.txt"), 2, 16, [2])
+    text = profile_text("bert-48-pbs-2")
+    o = P.SyncOrchestrate(text, 2, 16, [2])
     perf = o.m.perf
     assert len(perf.states) == 55 and perf.parameter_sizes[0][-1] == pytest.approx(sum(
-        float(l.split("parameter_size=")[1]) for l in open(os.path.join(HERE, "bert-48-pbs-2.txt")) if "parameter_size=" in l))
+        float(l.split("parameter_size=")[1]) for l in text.split("\n") if "parameter_size=" in l))
     plan = o.plan_for(2, True)
     names = P.stage_layers(plan.stages, perf)
     assert names[0][-1] == "layer_23" and names[1][0] == "layer_24"
