@@ -576,3 +576,22 @@ def stage_layers(plan_stages, perf):
         last = s[1] if i == len(plan_stages) - 1 else s[1] - 1
         out.append([perf.states[j].desc for j in range(s[0], last + 1)])
     return out
+
+
+def encoder_layer_ranges(plan_stages, perf):
+    """(first layer, number of layers) of every stage, from the states named ``layer_<n>`` / ``Layer_<n>`` it covers
+    (BERT and XLNet profiles): the ``first_layer`` / ``num_layers`` a stage of ``runtime.bert_stage`` or
+    ``runtime.xlnet_stage`` is built with.  A stage without such states gets (None, 0)."""
+    import re
+    out = []
+    for names in stage_layers(plan_stages, perf):
+        ids = sorted(int(m.group(1)) for m in (re.match(r"^[Ll]ayer_(\d+)$", n) for n in names) if m)
+        out.append((ids[0], len(ids)) if ids else (None, 0))
+    return out
+
+
+def micro_batches(plan, model):
+    """Micro-batches per step and replica of a plan: global batch / replicas / the micro-batch size
+    (sync_pipeline.rs:39, the count the speed-up model is evaluated with)."""
+    return model.global_batch_size // plan.replicas // model.min_micro_batch_size
+

@@ -204,6 +204,11 @@ def test_bert48_profile_two_gpus():
     plan = o.plan_for(2, True)
     names = P.stage_layers(plan.stages, perf)
     assert names[0][-1] == "layer_23" and names[1][0] == "layer_24"
+    # what a stage of runtime.bert_stage is built with, and the micro-batch count of the step
+    assert P.encoder_layer_ranges(plan.stages, perf) == [(0, 24), (24, 24)]
+    assert plan.replicas == 1 and P.micro_batches(plan, o.m) == 16
+    o.m.min_micro_batch_size = 2
+    assert P.micro_batches(plan, o.m) == 8
     ct = perf.compute_times
     cut = plan.stages[0][1]
     assert max(ct[0][cut - 1], ct[cut][54]) == pytest.approx(min(max(ct[0][c - 1], ct[c][54]) for c in range(1, 55)))
