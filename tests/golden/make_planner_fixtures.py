@@ -8,7 +8,7 @@ import json
 import os
 import sys
 
-NAMES = ["vgg-19-pbs-32", "bert-48-pbs-2"]
+NAMES = ["vgg-19-pbs-32", "bert-48-pbs-2", "xlnet-36-pbs-1"]
 
 
 def read(path):

@@ -212,3 +212,17 @@ def test_bert48_profile_two_gpus():
     ct = perf.compute_times
     cut = plan.stages[0][1]
     assert max(ct[0][cut - 1], ct[cut][54]) == pytest.approx(min(max(ct[0][c - 1], ct[c][54]) for c in range(1, 55)))
+
+
+def test_xlnet36_with_the_call_of_the_reproduction_notes():
+    """The one call the reference documents (PLANNER_REPRODUCTION.md): xlnet-36-pbs-1, profile batch 1, global batch 128,
+    devices [8, 16].  Best plan here: two stages of 8 replicas each, one machine per stage, cut between Layer_17 and
+    Layer_18 (18 : 18 layers).  The reference's model file hard-codes 17 : 19 for this model (slice_xlnet.py:106-121),
+    one layer off: all 36 layers have the same profile, and the planner's cost model has no term that would move the cut."""
+    o = P.SyncOrchestrate(profile_text("xlnet-36-pbs-1"), 1, 128, [8, 16])
+    speedup, stages = o.orchestrate()
+    assert [(s[0], s[2], s[3]) for s in stages] == [(0, 1, list(range(8))), (stages[1][0], 1, list(range(8, 16)))]
+    best = max(o.res, key=lambda r: r.speedup)
+    assert best.replicas == 8 and P.micro_batches(best, o.m) == 16
+    assert P.encoder_layer_ranges(stages, o.m.perf) == [(0, 18), (18, 18)]
+    assert 14.0 < speedup < 15.5
