@@ -308,6 +308,7 @@ class Devices(object):
     def __init__(self, n, seps, network=None):
         self.num_gpus, self.seps, self.num_machines = n, list(seps), len(seps)
         self.network = network or Network()
+        self._replica_memo = {}
 
     def _one_machine(self, lo, hi):
         l = 0
@@ -387,6 +388,9 @@ class Devices(object):
     def next_cards_with_replica(self, occupied, need, replica):
         """``replica`` rounds of ``need`` GPUs, every combination of the rounds' strategies, merged per resulting
         GPU set (device.rs:231-293)."""
+        memo_key = (tuple(occupied), need, replica)
+        if memo_key in self._replica_memo:          # the search asks for the same placement for every pair of cuts
+            return self._replica_memo[memo_key]
         rounds = [([], tuple(occupied))]
         for _ in range(replica):
             nxt = []
@@ -397,7 +401,8 @@ class Devices(object):
         found = {}
         for gids, occ in rounds:
             found[frozenset(gids)] = Placement("fusion", occ, frozenset(gids))
-        return [found[k] for k in sorted(found, key=sorted)]
+        self._replica_memo[memo_key] = [found[k] for k in sorted(found, key=sorted)]
+        return self._replica_memo[memo_key]
 
     # -- cost models
     def all_reduce_time(self, gids, size):
