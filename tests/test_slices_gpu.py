@@ -76,7 +76,21 @@ def test_bert_finetune_slice_puts_the_planner_split_on_each_device():
     s2.stage.backward(0, dy, torch.empty_like(h))
     with pytest.raises(ValueError, match="does not hold"):
         s1.build_output_layer_classification(y)
-    s0.stage.close(); s1.stage.close()
+    # model_type='regression' (bert.py:465-466): pooler + one output, the graph's pairwise squared-error mean
+    s3 = slices.BertFinetuneSlice(cfg, 8, False, ids, None, None, [0.5, -1.25], False, model_type="regression",
+                                  slice_devices="/gpu:0,/gpu:1", local_device=1, dtype="fp32")
+    s3.stage.forward(0, h, y)
+    dy = s3.build_output_layer_regression(y.reshape(2, 8, 32))
+    assert s3.stage_outputs[-1] is s3.loss and float(s3.loss) > 0.0
+    assert tuple(s3.logits.shape) == (2, 1) and tuple(s3.fc_weights.shape) == (32, 1) and s3.predictions is s3.logits
+    z, t = s3.logits[:, 0].double().cpu(), torch.tensor([0.5, -1.25], dtype=torch.float64)
+    want = ((z[:, None] - t[None, :]) ** 2).mean() + 1e-3 * 0.5 * float((s3.fc_weights.double() ** 2).sum())
+    assert abs(float(s3.loss) - float(want)) < 1e-5 * max(1.0, float(want))
+    assert float(dy.reshape(2, 8, 32)[:, 1:].abs().max()) == 0.0 and float(dy.reshape(2, 8, 32)[:, 0].abs().max()) > 0
+    s3.stage.backward(0, dy, torch.empty_like(h))
+    with pytest.raises(ValueError, match="does not hold"):
+        s2.build_output_layer_regression(y)
+    s0.stage.close(); s1.stage.close(); s3.stage.close()
 
 
 def test_vgg_xlnet_gnmt_slices_build():
