@@ -33,6 +33,7 @@ class GemmDesc(C.Structure):
         ("flags", C.c_int), ("alpha", C.c_float),
         ("a", C.c_void_p), ("b", C.c_void_p), ("c", C.c_void_p),
         ("bias", C.c_void_p), ("residual", C.c_void_p), ("c2", C.c_void_p),
+        ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
     ]
 
 
@@ -89,6 +90,7 @@ PROTOTYPES = {
     "ds_cast_f32_to_bf16": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "ds_cast_bf16_to_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "ds_gemm": (C.c_int, [C.POINTER(GemmDesc), C.c_void_p]),
+    "ds_gemm_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int]),
     "ds_layernorm_fwd": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_float,
                                    C.c_void_p, C.c_void_p, C.c_void_p]),
     "ds_layernorm_bwd": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,

@@ -800,6 +800,7 @@ static int gemm_run(const ds_gemm_desc* d, int splitk_req, void* stream) {
   a.flags = f;
   a.alpha = d->alpha;
   a.prio = ds_launch_prio;
+  a.ws_part = nullptr; a.ws_count = nullptr;
   a.vec_epi = d->n % 8 == 0 && d->ldc % 8 == 0 && d->c_stride_outer % 8 == 0 && d->c_stride_inner % 8 == 0 &&
               ds_aligned16(d->c) && ds_aligned16(d->residual) && ds_aligned16(d->c2);
   if (d->dtype == DS_BF16 && d->a_major == DS_K_MAJOR && d->b_major == DS_K_MAJOR && d->k == 64 && f == DS_EPI_OUT_F32 &&
@@ -827,19 +828,53 @@ static int gemm_run(const ds_gemm_desc* d, int splitk_req, void* stream) {
   a.splitk = splitk;
   a.ktiles_per_split = (ktiles + splitk - 1) / splitk;
   hipStream_t s = (hipStream_t)stream;
-  {  // 8-wave kernels (gemm8.hip); DS_GEMM8=0|1|2 forces a block shape where it applies, -1 switches them off
+  if (d->dtype == DS_BF16 && d->k % 64 == 0 && a.vec_epi && splitk == 1) {
+    // 8-wave kernels (gemm8.hip).  Block shape by the number of output tiles: 256x256 and 256x128 blocks need about a
+    // tile per CU to pay (0.8 -> 1.1 PFLOP/s on 4096^3); 128x128 with the same 96 KB of LDS as the 4-wave block it
+    // replaces (what else fits on the CU beside a block decides a multi-stream step more than the block's own speed).
+    // DS_GEMM8 = -1 switches them off, 0..4 forces a shape wherever it applies.
     static const char* env8 = getenv("DS_GEMM8");
-    int cfg8 = env8 ? atoi(env8) : -1;
-    static const char* env_mt = getenv("DS_GEMM8_MIN_TILES");
-    static const char* env_ao = getenv("DS_GEMM8_ACCUM_ONLY");
+    static const char* env_sk = getenv("DS_GEMM_SPLITK_WS");  // 0: never split, n > 1: n slices wherever k divides
     static const int bm8[5] = {256, 256, 128, 128, 128}, bn8[5] = {256, 128, 128, 128, 128};
-    if (cfg8 >= 0 && cfg8 <= 4) {
-      const int tiles8 = ((d->m + bm8[cfg8] - 1) / bm8[cfg8]) * ((d->n + bn8[cfg8] - 1) / bn8[cfg8]) * batch;
-      if (env_mt && tiles8 < atoi(env_mt)) cfg8 = -1;
-      if (env_ao && atoi(env_ao) && !(f & DS_EPI_ACCUM)) cfg8 = -1;
+    auto tiles_of = [&](int c) { return (int64_t)((d->m + bm8[c] - 1) / bm8[c]) * ((d->n + bn8[c] - 1) / bn8[c]) * batch; };
+    int cfg8 = -1;
+    if (env8) {
+      cfg8 = atoi(env8);
+      if (cfg8 > 4) cfg8 = -1;
+    } else if (tiles_of(0) >= 200) {
+      cfg8 = 0;
+    } else if (tiles_of(1) >= 200) {
+      cfg8 = 1;
+    } else if (tiles_of(4) >= 192) {
+      cfg8 = 4;
     }
-    if (cfg8 >= 0 && cfg8 <= 4 && d->dtype == DS_BF16 && d->k % 64 == 0 && a.vec_epi && splitk == 1 &&
-        ktiles > ds_gemm8_stages(cfg8)) {
+    // Split-K through the caller's workspace: a handful of output tiles under a very long k (a few tiles cannot fill
+    // the GPU; the exchange of partial tiles costs about 8 us, so it only pays when a slice is still long).
+    if (batch == 1 && d->workspace != nullptr) {
+      const int64_t tiles = tiles_of(4);
+      int slices = 0;
+      for (int c = 4; c >= 2 && !slices; --c)
+        if (tiles * c <= 64 && ktiles % c == 0 && ktiles / c >= 32) slices = c;
+      if (env_sk) {
+        const int forced = atoi(env_sk);
+        slices = forced <= 1 || forced > 4 || tiles > 1024 ? 0 : (ktiles % forced == 0 && ktiles / forced > ds_gemm8_stages(4) ? forced : 0);
+      }
+      if (slices > 1) {
+        DS_CHECK_ARG(((uintptr_t)d->workspace & 255) == 0 && d->workspace_bytes >= ds_gemm_workspace_bytes(d->m, d->n),
+                     "ds_gemm: workspace must be 256-byte aligned and hold ds_gemm_workspace_bytes(m, n) = %zu bytes (got %zu)",
+                     ds_gemm_workspace_bytes(d->m, d->n), d->workspace_bytes);
+        a.splitk = slices;
+        a.ktiles_per_split = ktiles / slices;
+        a.ws_count = (unsigned*)d->workspace;
+        a.ws_part = (float*)((char*)d->workspace + 4096);
+        char tagk[96];
+        snprintf(tagk, sizeof(tagk), "gemm8_kernel<bf16,128,128,%s,%s>/k%d", d->a_major == DS_K_MAJOR ? "K" : "MN",
+                 d->b_major == DS_K_MAJOR ? "K" : "MN", slices);
+        ds_prof_scope profk(s, tagk, 2.0 * d->m * d->n * d->k, "FLOP");
+        return ds_gemm8_launch(a, 4, d->a_major, d->b_major, 1, s);
+      }
+    }
+    if (cfg8 >= 0 && ktiles > ds_gemm8_stages(cfg8)) {
       char tag8[96];
       snprintf(tag8, sizeof(tag8), "gemm8_kernel<bf16,%d,%d,%s,%s>", bm8[cfg8], bn8[cfg8],
                d->a_major == DS_K_MAJOR ? "K" : "MN", d->b_major == DS_K_MAJOR ? "K" : "MN");
@@ -859,6 +894,13 @@ static int gemm_run(const ds_gemm_desc* d, int splitk_req, void* stream) {
 
 
 extern "C" int ds_gemm(const ds_gemm_desc* d, void* stream) { return gemm_run(d, 1, stream); }
+
+// 4 KiB of arrival counters (one per 128x128 tile, at most 1024 tiles), then up to 4 fp32 partial tiles per tile
+extern "C" size_t ds_gemm_workspace_bytes(int m, int n) {
+  if (m <= 0 || n <= 0) return 0;
+  const size_t tiles = (size_t)((m + 127) / 128) * ((n + 127) / 128);
+  return 4096 + tiles * 4 * 128 * 128 * sizeof(float);
+}
 
 // Split-K variant for accumulating outputs whose reduction dimension dwarfs m*n (atomic fp32 adds).
 int ds_gemm_splitk(const ds_gemm_desc* d, int splitk, void* stream) { return gemm_run(d, splitk, stream); }

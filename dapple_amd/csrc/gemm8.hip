@@ -28,6 +28,20 @@ using namespace dsgemm;
 
 namespace {
 
+// Split-K partials cross from one workgroup to another inside a launch, and the L2 caches of the 8 XCDs are not
+// coherent with each other: the values move as device-scope 8-byte accesses that go past the caches, which costs
+// nothing else in the cache (a release / acquire fence pair would write back and invalidate the whole L2).
+// Split-K partials cross from one workgroup to another inside a launch, and the L2 caches of the 8 XCDs are not
+// coherent with each other: the values move as system-scope 16-byte accesses (sc0 sc1: stores go through to memory,
+// loads come from there), which leaves the rest of the cache alone - a release / acquire fence pair at device scope
+// would write back and invalidate the whole L2 (measured: 60 us per GEMM).
+__device__ __forceinline__ void part_store4(float* p, const f32x4& v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ void part_load4(const float* p, f32x4& v) {
+  asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(v) : "v"(p) : "memory");
+}
+
 template <int BM, int BN, int WM, int WN, int WK, int STAGES, int AMAJ, int BMAJ>
 __global__ __launch_bounds__(512) void gemm8_kernel(GemmArgs p) {
   typedef bf16 T;
@@ -193,10 +207,103 @@ __global__ __launch_bounds__(512) void gemm8_kernel(GemmArgs p) {
   if (STAGES >= 4) k_tile(N(), N(), std::integral_constant<int, (STAGES >= 4 ? STAGES - 4 : 0)>());
   k_tile(N(), N(), std::integral_constant<int, 0>());
 
-  // Epilogue through LDS, one 32-row MFMA block of every wave at a time: the waves park alpha * acc + bias as fp32
-  // rows (with WK == 2 the upper k-half parks its raw partial first and the lower one adds its own), then every
-  // thread streams 8 consecutive columns of a row, so that residual / auxiliary reads and C writes are 16-byte vectors
-  // covering whole rows of the tile.
+  // With WK == 2 the two waves of a SIMD hold the two k-halves of one sub-tile: the upper half parks its accumulators in
+  // LDS as they lie in the registers (16 bytes per lane and store: no bank conflicts), the lower half adds them and
+  // carries the sub-tile from here on.
+  constexpr int WAVE_ACC = TM * TN * 1024;  // floats of one wave's accumulators
+  if (WK == 2) {
+    static_assert(WK == 1 || 4 * WAVE_ACC * 4 <= STAGES * STAGE_BYTES, "pair merge fits the tile ring");
+    float* park = reinterpret_cast<float*>(lds) + wq * WAVE_ACC;
+    __syncthreads();  // every wave is out of the k loop
+    if (wk == 1) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const f32x4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+            *reinterpret_cast<f32x4*>(park + (((i * TN + j) * 4 + g) * 64 + lane) * 4) = v;
+          }
+    }
+    __syncthreads();
+    if (wk == 0) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const f32x4 v = *reinterpret_cast<const f32x4*>(park + (((i * TN + j) * 4 + g) * 64 + lane) * 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[i][j][4 * g + e] += v[e];
+          }
+    }
+  }
+
+  // Split-K through a workspace: every slice stores its accumulators as they lie in the registers (1 KiB per store
+  // instruction), then takes a ticket; the workgroup that draws the last one adds the slices in index order - its own
+  // from registers - so that the result does not depend on which slice came last.
+  if (p.ws_part != nullptr) {
+    constexpr int TILE_ACC = WM * WN * WAVE_ACC;  // = BM * BN
+    const int tile_id = blockIdx.x;
+    float* part = p.ws_part + (size_t)tile_id * p.splitk * TILE_ACC;
+    float* mine = part + (size_t)ks_id * TILE_ACC + wq * WAVE_ACC;
+    if (wk == 0) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const f32x4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+            part_store4(mine + (((i * TN + j) * 4 + g) * 64 + lane) * 4, v);
+          }
+    }
+    // the stores above go through to device-coherent memory; once they are acknowledged the ticket may be drawn
+    __builtin_amdgcn_s_waitcnt(DS_VMCNT(0));
+    __syncthreads();  // every wave is out of the k loop / the pair merge (the ticket word overlays the tile ring)
+    unsigned* ticket = reinterpret_cast<unsigned*>(lds);
+    if (tid == 0) *ticket = __hip_atomic_fetch_add(p.ws_count + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (*ticket != (unsigned)(p.splitk - 1)) return;
+    if (tid == 0) __hip_atomic_store(p.ws_count + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (wk == 0) {
+      // every slice's copy is read back (this workgroup's own too: same bits as its registers), one 32x32 tile of
+      // all slices per round trip; straight-line code, since the loads complete behind the compiler's back
+      const int ns = p.splitk;
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          f32x4 o[4][4];
+#pragma unroll
+          for (int s = 0; s < 4; ++s) {
+            const int sl = s < ns ? s : ns - 1;  // slots past the last slice re-read it and are not added
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+              part_load4(part + (size_t)sl * TILE_ACC + (size_t)wq * WAVE_ACC + (((i * TN + j) * 4 + g) * 64 + lane) * 4, o[s][g]);
+          }
+          asm volatile("s_waitcnt vmcnt(0)"
+                       : "+v"(o[0][0]), "+v"(o[0][1]), "+v"(o[0][2]), "+v"(o[0][3]), "+v"(o[1][0]), "+v"(o[1][1]), "+v"(o[1][2]),
+                         "+v"(o[1][3]), "+v"(o[2][0]), "+v"(o[2][1]), "+v"(o[2][2]), "+v"(o[2][3]), "+v"(o[3][0]), "+v"(o[3][1]),
+                         "+v"(o[3][2]), "+v"(o[3][3]));
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            f32x4 t = o[0][g];
+            if (ns > 1) t += o[1][g];
+            if (ns > 2) t += o[2][g];
+            if (ns > 3) t += o[3][g];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[i][j][4 * g + e] = t[e];
+          }
+        }
+    }
+  }
+
+  // Epilogue through LDS, one 32-row MFMA block of every wave at a time: the waves that carry the sub-tiles park
+  // alpha * acc + bias as fp32 rows, then every thread streams 8 consecutive columns of a row, so that residual /
+  // auxiliary reads and C writes are 16-byte vectors covering whole rows of the tile.
   constexpr int LDW = BN + 4;
   constexpr int SLAB_ROWS = WM * 32;
   constexpr int VPR = BN / 8;
@@ -207,20 +314,6 @@ __global__ __launch_bounds__(512) void gemm8_kernel(GemmArgs p) {
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     __syncthreads();
-    if (WK == 2) {
-      if (wk == 1) {
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-          const int cl = wn * (BN / WN) + j * 32 + (lane & 31);
-#pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            const int rs = wm * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-            sc[rs * LDW + cl] = acc[i][j][e];
-          }
-        }
-      }
-      __syncthreads();
-    }
     if (wk == 0) {
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
@@ -230,9 +323,7 @@ __global__ __launch_bounds__(512) void gemm8_kernel(GemmArgs p) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
           const int rs = wm * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-          float v = acc[i][j][e];
-          if (WK == 2) v += sc[rs * LDW + cl];
-          sc[rs * LDW + cl] = v * p.alpha + bias;
+          sc[rs * LDW + cl] = acc[i][j][e] * p.alpha + bias;
         }
       }
     }
@@ -288,6 +379,8 @@ int ds_gemm8_stages(int cfg) { return cfg == 0 || cfg == 3 ? 2 : cfg == 1 || cfg
 int ds_gemm8_launch(const GemmArgs& a, int cfg, int a_major, int b_major, int batch, hipStream_t stream) {
   DS_CHECK_ARG(a.k % 64 == 0 && a.vec_epi, "ds_gemm8_launch: needs k %% 64 == 0 and the vector epilogue");
   DS_CHECK_ARG(cfg >= 0 && cfg <= 4, "ds_gemm8_launch: cfg %d", cfg);
+  DS_CHECK_ARG(a.splitk == 1 || (a.ws_part && a.ws_count && batch == 1 && a.splitk <= 4),
+               "ds_gemm8_launch: split-K needs a workspace, batch 1 and at most 4 slices");
   DS_CHECK_ARG(a.ktiles_per_split > ds_gemm8_stages(cfg) && (a.k / 64) % a.ktiles_per_split == 0,
                "ds_gemm8_launch: every k-slice needs more than %d k-tiles", ds_gemm8_stages(cfg));
   if (a_major == DS_K_MAJOR && b_major == DS_K_MAJOR) return launch8_cfg<DS_K_MAJOR, DS_K_MAJOR>(a, cfg, batch, stream);

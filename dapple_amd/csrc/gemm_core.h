@@ -44,6 +44,8 @@ struct GemmArgs {
   int vec_epi;
   int conv_h, conv_w, conv_c;  // implicit 3x3 'same' convolution: extent of the gathered NHWC tensor
   int prio;                    // wave priority (0..3)
+  float* ws_part;              // split-K by workspace (8-wave kernels): fp32 partial tiles [tile][slice][BM * BN]
+  unsigned* ws_count;          // and one arrival counter per tile (zero between launches)
 };
 
 

@@ -56,9 +56,10 @@ def cast_to_f32(src):
 
 def gemm(a, b, c, m, n, k, a_major=DS_K_MAJOR, b_major=DS_MN_MAJOR, lda=None, ldb=None, ldc=None, flags=0,
          alpha=1.0, bias=None, residual=None, c2=None, batch=1, batch_inner=1, a_strides=(0, 0), b_strides=(0, 0),
-         c_strides=(0, 0)):
-    """Raw ds_gemm: C[m][n] (+)= alpha * sum_k A(m,k) B(n,k); see include/dapple_stage.h."""
-    _need_cuda(a, b, c, bias, residual, c2)
+         c_strides=(0, 0), workspace=None):
+    """Raw ds_gemm: C[m][n] (+)= alpha * sum_k A(m,k) B(n,k); see include/dapple_stage.h.  `workspace`: a zero-filled
+    uint8 tensor of gemm_workspace_bytes(m, n) bytes that lets the library cut a long k into slices (split-K)."""
+    _need_cuda(a, b, c, bias, residual, c2, workspace)
     d = GemmDesc()
     d.dtype = dtype_code(a)
     d.a_major, d.b_major = a_major, b_major
@@ -75,8 +76,15 @@ def gemm(a, b, c, m, n, k, a_major=DS_K_MAJOR, b_major=DS_MN_MAJOR, lda=None, ld
     d.bias = bias.data_ptr() if bias is not None else None
     d.residual = residual.data_ptr() if residual is not None else None
     d.c2 = c2.data_ptr() if c2 is not None else None
+    if workspace is not None:
+        d.workspace, d.workspace_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
     check(_lib.load().ds_gemm(C.byref(d), _lib.current_stream()), "ds_gemm")
     return c
+
+
+def gemm_workspace_bytes(m, n):
+    """Bytes of split-K workspace ds_gemm wants for an [m, n] output (zero-fill it once before the first use)."""
+    return int(_lib.load().ds_gemm_workspace_bytes(m, n))
 
 
 def dense(x, kernel, bias=None, residual=None, gelu=False):

@@ -95,8 +95,16 @@ typedef struct ds_gemm_desc {
   const float* bias;    /* [n] fp32, DS_EPI_BIAS */
   const void* residual; /* same layout and strides as C, DS_EPI_RESIDUAL */
   void* c2;             /* DS_EPI_GELU second output / DS_EPI_DGELU aux input, layout of C */
+  void* workspace;      /* optional device scratch for split-K (NULL: never split), see ds_gemm_workspace_bytes */
+  size_t workspace_bytes;
 } ds_gemm_desc;
 int ds_gemm(const ds_gemm_desc* d, void* stream);
+/* Split-K: when the output has too few tiles to fill the GPU and k is long (bf16, batch 1), ds_gemm may cut k into
+ * slices that run as separate workgroups; every slice leaves its fp32 partial tile in `workspace`, and the workgroup
+ * that finishes last adds the slices in index order (bit-reproducible) and runs the epilogue.  The workspace must be
+ * at least ds_gemm_workspace_bytes(m, n) bytes, 256-byte aligned, zero-filled once before its first use (the library
+ * leaves its counters at zero), and must not be shared by GEMMs that can run at the same time. */
+size_t ds_gemm_workspace_bytes(int m, int n);
 
 /* ---------------------------------------------------------------------------
  * LayerNorm over the last axis, y = (x - mean) * rsqrt(var + eps) * gamma + beta,

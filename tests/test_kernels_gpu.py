@@ -73,6 +73,64 @@ def test_gemm_layouts(dt, am, bm, m, n, k):
     assert_close(c, Ar @ Br.T, TOL[dt], "gemm")
 
 
+# Shapes that the dispatcher sends to the 512-thread kernels: 128x128 blocks (>= 192 tiles), 256x128 (>= 200), 256x256
+# (>= 200), each with ragged edges and the shortest reduction a block shape accepts.
+BIG_SHAPES = [(1024, 3072, 1024), (1016, 3064, 320), (3584, 2048, 256), (3576, 1800, 256), (4096, 4096, 512),
+              (3992, 4088, 192)]
+
+
+@pytest.mark.parametrize("am,bm", [(0, 0), (0, 1), (1, 1), (1, 0)])
+@pytest.mark.parametrize("m,n,k", BIG_SHAPES)
+def test_gemm_wide_blocks(am, bm, m, n, k):
+    r = rng(m + n * 5 + k * 11 + am * 2 + bm)
+    A = (r.standard_normal((m, k)) * 0.5).astype(np.float32)
+    B = (r.standard_normal((n, k)) * 0.5).astype(np.float32)
+    a = dev(A if am == DS_K_MAJOR else A.T, torch.bfloat16)
+    b = dev(B if bm == DS_K_MAJOR else B.T, torch.bfloat16)
+    bias = dev(r.standard_normal(n), torch.float32)
+    res = dev(r.standard_normal((m, n)), torch.bfloat16)
+    c = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    ops.gemm(a, b, c, m, n, k, am, bm, flags=DS_EPI_BIAS | DS_EPI_RESIDUAL, bias=bias, residual=res, alpha=0.25)
+    Ar = (a if am == DS_K_MAJOR else a.T).float()
+    Br = (b if bm == DS_K_MAJOR else b.T).float()
+    ref = (0.25 * (Ar @ Br.T) + bias + res.float()).cpu().double()   # fp32 on the device: the fp64 host product takes minutes
+    assert_close(c, ref, TOL["bf16"], "gemm, wide blocks")
+    acc0 = dev(r.standard_normal((m, n)), torch.float32)
+    acc = acc0.clone()
+    ops.gemm(a, b, acc, m, n, k, am, bm, flags=DS_EPI_ACCUM)
+    assert_close(acc, (acc0 + Ar @ Br.T).cpu().double(), 1e-5, "gemm accumulate, wide blocks")
+
+
+@pytest.mark.parametrize("am,bm", [(0, 0), (0, 1), (1, 1)])
+@pytest.mark.parametrize("m,n,k", [(128, 256, 8192), (248, 120, 6144), (384, 128, 16384)])
+def test_gemm_split_k_by_workspace(am, bm, m, n, k):
+    """A few output tiles under a long reduction: with a workspace the library cuts k into slices; the result equals the
+    unsplit product up to fp32 summation order, is the same bit for bit on every run, and the workspace comes back zeroed
+    where the library counts arrivals."""
+    r = rng(m + n + k)
+    A = (r.standard_normal((m, k)) * 0.5).astype(np.float32)
+    B = (r.standard_normal((n, k)) * 0.5).astype(np.float32)
+    a = dev(A if am == DS_K_MAJOR else A.T, torch.bfloat16)
+    b = dev(B if bm == DS_K_MAJOR else B.T, torch.bfloat16)
+    bias = dev(r.standard_normal(n), torch.float32)
+    ws = torch.zeros(ops.gemm_workspace_bytes(m, n), dtype=torch.uint8, device="cuda")
+    outs = []
+    for _ in range(3):
+        c = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda")
+        ops.gemm(a, b, c, m, n, k, am, bm, flags=DS_EPI_BIAS | DS_EPI_OUT_F32, bias=bias, workspace=ws)
+        outs.append(c)
+    plain = torch.empty_like(outs[0])
+    ops.gemm(a, b, plain, m, n, k, am, bm, flags=DS_EPI_BIAS | DS_EPI_OUT_F32, bias=bias)
+    Ar = (a if am == DS_K_MAJOR else a.T).cpu().double()
+    Br = (b if bm == DS_K_MAJOR else b.T).cpu().double()
+    assert_close(outs[0], Ar @ Br.T + bias.cpu().double(), 1e-5, "split-K gemm")
+    assert_close(outs[0], plain, 1e-5, "split-K vs unsplit")
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+    assert int(ws[:4096].count_nonzero()) == 0
+    with pytest.raises(Exception):
+        ops.gemm(a, b, outs[0], m, n, k, am, bm, flags=DS_EPI_OUT_F32, workspace=ws[:8192])   # too small
+
+
 @pytest.mark.parametrize("dt", ["fp32", "bf16"])
 def test_gemm_epilogues(dt):
     m, n, k = 192, 160, 96
