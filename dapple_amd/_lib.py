@@ -130,6 +130,9 @@ PROTOTYPES = {
     "ds_stage_forward": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
     "ds_stage_set_token_types": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p]),
     "ds_stage_backward": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
+    "ds_stage_backward_after": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "ds_stage_backward_event": (C.c_void_p, [C.c_void_p, C.c_int]),
+    "ds_stage_wait_backward": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p]),
     "ds_stage_workspace_bytes": (C.c_size_t, [C.c_void_p]),
     "ds_stage_stash_bytes": (C.c_size_t, [C.c_void_p, C.c_int]),
     "ds_stage_sync": (C.c_int, [C.c_void_p]),

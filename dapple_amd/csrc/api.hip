@@ -98,6 +98,7 @@ extern "C" int ds_stage_destroy(ds_stage* h) {
     for (hipEvent_t e : h->ev_forwarded) (void)hipEventDestroy(e);
     for (hipEvent_t e : h->ev_released) (void)hipEventDestroy(e);
     if (h->ev_join) (void)hipEventDestroy(h->ev_join);
+    if (h->ev_dout) (void)hipEventDestroy(h->ev_dout);
     (void)hipStreamDestroy(h->bwd_owned);
     (void)hipStreamDestroy(h->wgrad_owned);
   }
@@ -143,6 +144,7 @@ extern "C" int ds_stage_enable_overlap(ds_stage* h, int on) {
       DS_CHECK_HIP(hipEventCreateWithFlags(&h->ev_released[i], hipEventDisableTiming));
     }
     DS_CHECK_HIP(hipEventCreateWithFlags(&h->ev_join, hipEventDisableTiming));
+    DS_CHECK_HIP(hipEventCreateWithFlags(&h->ev_dout, hipEventDisableTiming));
   }
   h->released_valid.assign(h->cfg.stash_slots, 0);  // everything queued so far is ordered on h->stream
   h->bwd_stream = h->bwd_owned;
@@ -213,7 +215,9 @@ extern "C" int ds_stage_forward(ds_stage* h, int slot, const void* in, const flo
   return rc;
 }
 
-extern "C" int ds_stage_backward(ds_stage* h, int slot, const void* d_out, void* d_in) {
+// after: 0 = the producer of d_out is whatever has been queued on the stage's stream so far; 1 = `ready` (an event, or
+// NULL for "already complete / ordered before F(slot)") says when d_out may be read
+static int stage_backward(ds_stage* h, int slot, const void* d_out, void* d_in, int after, hipEvent_t ready) {
   DS_CHECK_ARG(h != nullptr && d_out != nullptr, "ds_stage_backward: null argument");
   DS_CHECK_ARG(slot >= 0 && slot < h->cfg.stash_slots, "ds_stage_backward: slot %d out of range [0,%d)", slot, h->cfg.stash_slots);
   if (!h->slot_forwarded[slot]) {
@@ -224,6 +228,12 @@ extern "C" int ds_stage_backward(ds_stage* h, int slot, const void* d_out, void*
   int rc;
   if (h->bwd_stream) {
     DS_CHECK_HIP(hipStreamWaitEvent(h->bwd_stream, h->ev_forwarded[slot], 0));
+    if (!after) {
+      DS_CHECK_HIP(hipEventRecord(h->ev_dout, h->stream));
+      DS_CHECK_HIP(hipStreamWaitEvent(h->bwd_stream, h->ev_dout, 0));
+    } else if (ready) {
+      DS_CHECK_HIP(hipStreamWaitEvent(h->bwd_stream, ready, 0));
+    }
     hipStream_t fwd = h->stream;
     h->stream = h->bwd_stream;
     rc = h->backward(slot, d_out, d_in);
@@ -232,10 +242,39 @@ extern "C" int ds_stage_backward(ds_stage* h, int slot, const void* d_out, void*
     h->released_valid[slot] = 1;
     h->bwd_pending = true;
   } else {
+    if (after && ready) DS_CHECK_HIP(hipStreamWaitEvent(h->stream, ready, 0));
     rc = h->backward(slot, d_out, d_in);
   }
   h->slot_forwarded[slot] = 0;
   return rc;
+}
+
+extern "C" int ds_stage_backward(ds_stage* h, int slot, const void* d_out, void* d_in) {
+  return stage_backward(h, slot, d_out, d_in, 0, nullptr);
+}
+
+extern "C" int ds_stage_backward_after(ds_stage* h, int slot, const void* d_out, void* d_in, void* ready_event) {
+  return stage_backward(h, slot, d_out, d_in, 1, (hipEvent_t)ready_event);
+}
+
+extern "C" void* ds_stage_backward_event(ds_stage* h, int slot) {
+  if (!h || slot < 0 || slot >= h->cfg.stash_slots || !h->bwd_stream || !h->released_valid[slot]) return nullptr;
+  return (void*)h->ev_released[slot];
+}
+
+extern "C" int ds_stage_wait_backward(ds_stage* h, int slot, void* stream) {
+  DS_CHECK_ARG(h != nullptr, "ds_stage_wait_backward: null handle");
+  DS_CHECK_ARG(slot >= 0 && slot < h->cfg.stash_slots, "ds_stage_wait_backward: slot %d out of range [0,%d)", slot, h->cfg.stash_slots);
+  if (h->bwd_stream && h->released_valid[slot]) DS_CHECK_HIP(hipStreamWaitEvent((hipStream_t)stream, h->ev_released[slot], 0));
+  else if ((hipStream_t)stream != h->stream) {
+    // one stream: the pass is ordered on the stage's stream; another stream waits for what is queued there
+    hipEvent_t e = nullptr;
+    DS_CHECK_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+    DS_CHECK_HIP(hipEventRecord(e, h->stream));
+    DS_CHECK_HIP(hipStreamWaitEvent((hipStream_t)stream, e, 0));
+    DS_CHECK_HIP(hipEventDestroy(e));
+  }
+  return DS_OK;
 }
 
 extern "C" size_t ds_stage_workspace_bytes(const ds_stage* h) { return h ? h->workspace_bytes() : 0; }

@@ -39,6 +39,7 @@ struct ds_stage {
   std::vector<hipEvent_t> ev_forwarded, ev_released;
   std::vector<char> released_valid;
   hipEvent_t ev_join = nullptr;
+  hipEvent_t ev_dout = nullptr;  // marks what was queued on `stream` when a backward pass was issued
   bool bwd_pending = false;
   virtual ~ds_stage() {}
   // true when forward and backward passes of different slots touch disjoint memory (apart from

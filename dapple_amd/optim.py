@@ -3,8 +3,11 @@
 Same class names and keyword arguments as the reference: ``AdamWeightDecayOptimizer``
 (bert/graph_helper.py:191-272), ``AdamOptimizer`` / ``GradientDescentOptimizer`` (tf.train, as used by
 xlnet/utils/xlnet_utils.py:195-197 and vgg19/tf-keras-dapple.py:187).  ``apply_gradients`` takes the stage
-whose ``grads`` hold the accumulated gradients; ``max_gradient_norm`` is the flag of bert/graph.py:162-165.
-After a step the stage's compute copies are stale: call ``stage.refresh_weights()`` (the next step does).
+whose ``grads`` hold the accumulated gradients - or a list of parameter sets (the stages of a pipeline plus
+``FlatParams`` for head weights kept outside a stage): ``max_gradient_norm`` is the flag of bert/graph.py:162-165,
+``tf.clip_by_global_norm`` over the gradients of ALL slices, so with a list the norm is taken over every set and
+the same factor scales each of them.  After a step a stage's compute copies are stale; ``apply_gradients`` marks
+the stage and its next forward pass rebuilds them (``Stage.refresh_weights``).
 """
 import ctypes as C
 import re
@@ -59,16 +62,26 @@ class _FlatOptimizer:
     def _new_state(self, stage):
         return ()
 
-    def _sqnorm(self, stage, max_gradient_norm):
-        """Device scalar holding sum(g^2) over the stage's gradients, or None without clipping."""
-        if max_gradient_norm is None:
-            return None
+    def global_sqnorm(self, sets):
+        """Device scalar (fp64) holding sum(g^2) over the gradients of every parameter set in ``sets``: the square of
+        the global norm tf.clip_by_global_norm takes over grads_set (bert/graph.py:162-165)."""
+        sets = list(sets)
         if self._sq is None:
-            self._sq = torch.zeros(1, dtype=torch.float64, device=stage.device)
+            self._sq = torch.zeros(1, dtype=torch.float64, device=sets[0].device)
         self._sq.zero_()
-        check(self.lib.ds_grad_sqnorm_accum(_lib.ptr(stage.flat_grads), stage.flat_grads.numel(), _lib.ptr(self._sq),
-                                            _lib.current_stream()), "ds_grad_sqnorm_accum")
+        for st in sets:
+            check(self.lib.ds_grad_sqnorm_accum(_lib.ptr(st.flat_grads), st.flat_grads.numel(), _lib.ptr(self._sq),
+                                                _lib.current_stream()), "ds_grad_sqnorm_accum")
         return self._sq
+
+    def apply_gradients(self, params, max_gradient_norm=None, learning_rate=None):
+        """``params``: a ``runtime.Stage`` / ``FlatParams``, or a list of them clipped by their common global norm."""
+        sets = list(params) if isinstance(params, (list, tuple)) else [params]
+        sq = None if max_gradient_norm is None else self.global_sqnorm(sets)
+        for st in sets:
+            self._apply(st, sq, max_gradient_norm, learning_rate)
+            if hasattr(st, "mark_weights_stale"):
+                st.mark_weights_stale()
 
     def close(self):
         for h, _ in self._plans.values():
@@ -110,9 +123,8 @@ class AdamWeightDecayOptimizer(_FlatOptimizer):
     def _new_state(self, stage):
         return (torch.zeros_like(stage.flat_weights), torch.zeros_like(stage.flat_weights))   # adam_m, adam_v (:223-234)
 
-    def apply_gradients(self, stage, max_gradient_norm=None, learning_rate=None):
+    def _apply(self, stage, sq, max_gradient_norm, learning_rate):
         plan, (m, v) = self._plan(stage)
-        sq = self._sqnorm(stage, max_gradient_norm)
         lr = self.learning_rate if learning_rate is None else learning_rate
         check(self.lib.ds_adam_step(plan, _lib.ptr(stage.flat_weights), _lib.ptr(stage.flat_grads), _lib.ptr(m), _lib.ptr(v),
                                     lr, self.beta_1, self.beta_2, self.epsilon, _lib.ptr(sq),
@@ -133,12 +145,11 @@ class AdamOptimizer(_FlatOptimizer):
     def _new_state(self, stage):
         return (torch.zeros_like(stage.flat_weights), torch.zeros_like(stage.flat_weights))
 
-    def apply_gradients(self, stage, max_gradient_norm=None, learning_rate=None):
+    def _apply(self, stage, sq, max_gradient_norm, learning_rate):
         plan, (m, v) = self._plan(stage)
         t = self._t[id(stage)] = self._t.get(id(stage), 0) + 1
         lr = self.learning_rate if learning_rate is None else learning_rate
         lr_t = lr * (1.0 - self.beta2 ** t) ** 0.5 / (1.0 - self.beta1 ** t)
-        sq = self._sqnorm(stage, max_gradient_norm)
         check(self.lib.ds_adam_step(plan, _lib.ptr(stage.flat_weights), _lib.ptr(stage.flat_grads), _lib.ptr(m), _lib.ptr(v),
                                     lr_t, self.beta1, self.beta2, self.epsilon, _lib.ptr(sq),
                                     0.0 if max_gradient_norm is None else max_gradient_norm, _lib.current_stream()), "ds_adam_step")
@@ -151,9 +162,8 @@ class GradientDescentOptimizer(_FlatOptimizer):
         super().__init__()
         self.learning_rate, self.name = learning_rate, name
 
-    def apply_gradients(self, stage, max_gradient_norm=None, learning_rate=None):
+    def _apply(self, stage, sq, max_gradient_norm, learning_rate):
         plan, _ = self._plan(stage)
-        sq = self._sqnorm(stage, max_gradient_norm)
         lr = self.learning_rate if learning_rate is None else learning_rate
         check(self.lib.ds_sgd_step(plan, _lib.ptr(stage.flat_weights), _lib.ptr(stage.flat_grads), lr, _lib.ptr(sq),
                                    0.0 if max_gradient_norm is None else max_gradient_norm, _lib.current_stream()), "ds_sgd_step")

@@ -67,6 +67,8 @@ class Stage:
             self.weight_shapes.append((cols.value,) if vector else (rows.value, cols.value))
         self.weights, self.grads = {}, {}
         self.flat_weights = self.flat_grads = None
+        self._weights_stale = False
+        self.overlap = False
 
     # -- weights ---------------------------------------------------------------------------
     def bind(self, weights):
@@ -112,28 +114,63 @@ class Stage:
 
     def refresh_weights(self):
         check(self.lib.ds_stage_refresh_weights(self._h), "ds_stage_refresh_weights")
+        self._weights_stale = False
+
+    def mark_weights_stale(self):
+        """The master weights changed (an optimizer step): the next forward pass rebuilds the compute copies first."""
+        self._weights_stale = True
 
     def zero_grads(self):
         self.flat_grads.zero_()
 
     # -- one micro-batch ---------------------------------------------------------------------
+    def _check_tensor(self, t, what, dtype, numel):
+        """The kernels take raw device pointers: anything but a contiguous tensor on this stage's GPU would fault there."""
+        if not t.is_cuda or t.device != torch.device(self.device):
+            raise ValueError("%s must live on %s (got %s)" % (what, self.device, t.device))
+        if not t.is_contiguous():
+            raise ValueError("%s must be contiguous" % what)
+        if t.dtype != dtype or t.numel() != numel:
+            raise ValueError("%s must be %s with %d elements" % (what, dtype, numel))
+
     def forward(self, slot, x, out, key_mask=None, token_type_ids=None):
-        if x.dtype != self.in_dtype or x.numel() != self.in_numel:
-            raise ValueError("stage input must be %s with %d elements" % (self.in_dtype, self.in_numel))
+        self._check_tensor(x, "stage input", self.in_dtype, self.in_numel)
+        self._check_tensor(out, "stage output", self.act_dtype, self.out_numel)
+        if self._weights_stale:
+            self.refresh_weights()
         if token_type_ids is not None:
+            self._check_tensor(token_type_ids, "token_type_ids", torch.int32, self.in_numel)
             check(self.lib.ds_stage_set_token_types(self._h, slot, ptr(token_type_ids)), "ds_stage_set_token_types")
-        if out.dtype != self.act_dtype or out.numel() != self.out_numel:
-            raise ValueError("stage output must be %s with %d elements" % (self.act_dtype, self.out_numel))
-        if key_mask is not None and key_mask.dtype != torch.float32:
-            raise ValueError("key_mask must be fp32 [batch, seq]")
+        if key_mask is not None:
+            if key_mask.dtype != torch.float32 or not key_mask.is_cuda or not key_mask.is_contiguous():
+                raise ValueError("key_mask must be a contiguous fp32 [batch, seq] tensor on the GPU")
         check(self.lib.ds_stage_forward(self._h, slot, ptr(x), ptr(key_mask), ptr(out)), "ds_stage_forward")
 
-    def backward(self, slot, d_out, d_in=None):
-        if d_out.dtype != self.act_dtype or d_out.numel() != self.out_numel:
-            raise ValueError("upstream gradient must be %s with %d elements" % (self.act_dtype, self.out_numel))
-        if d_in is not None and (d_in.dtype != self.act_dtype or d_in.numel() != self.in_numel):
-            raise ValueError("input gradient must be %s with %d elements" % (self.act_dtype, self.in_numel))
-        check(self.lib.ds_stage_backward(self._h, slot, ptr(d_out), ptr(d_in)), "ds_stage_backward")
+    def backward(self, slot, d_out, d_in=None, ready=False):
+        """``ready``: when the upstream gradient may be read.  False (default): after everything queued so far on the
+        stage's stream.  None: it is already complete (synthetic, or produced before this micro-batch's forward pass).
+        A ``torch.cuda.Event`` or a raw event handle (``Stage.backward_event`` of the next stage): after that event -
+        with forward/backward overlap on, the last two keep an earlier-queued forward pass running beside this pass."""
+        self._check_tensor(d_out, "upstream gradient", self.act_dtype, self.out_numel)
+        if d_in is not None:
+            self._check_tensor(d_in, "input gradient", self.act_dtype, self.in_numel)
+        if ready is False:
+            check(self.lib.ds_stage_backward(self._h, slot, ptr(d_out), ptr(d_in)), "ds_stage_backward")
+            return
+        if isinstance(ready, torch.cuda.Event):
+            ready = ready.cuda_event
+        ev = C.c_void_p(ready) if ready is not None else None
+        check(self.lib.ds_stage_backward_after(self._h, slot, ptr(d_out), ptr(d_in), ev), "ds_stage_backward_after")
+
+    def backward_event(self, slot):
+        """Raw handle of the event that completes when the last backward pass of ``slot`` has written its input gradient
+        (None on one stream: the pass is ordered on the stage's stream)."""
+        return self.lib.ds_stage_backward_event(self._h, slot)
+
+    def wait_backward(self, slot, stream=None):
+        """Puts ``stream`` (default: the current one) behind the last backward pass of ``slot``."""
+        s = _lib.current_stream() if stream is None else C.c_void_p(stream.cuda_stream)
+        check(self.lib.ds_stage_wait_backward(self._h, slot, s), "ds_stage_wait_backward")
 
     def sync(self):
         check(self.lib.ds_stage_sync(self._h), "ds_stage_sync")
@@ -359,6 +396,12 @@ class StageRuntime:
         if len(inputs) != self.m or len(upstream) != self.m or len(outputs) != self.m:
             raise ValueError("expected %d micro-batches" % self.m)
         slot_of, free = {}, list(range(self.stage.stash_slots))
+        # the upstream gradients exist when the step starts: with forward/backward overlap a backward pass waits for
+        # this point of the current stream, not for the forward passes queued after it
+        ready = None
+        if self.stage.overlap:
+            ready = torch.cuda.Event()
+            ready.record()
         for op, j in self.ops:
             if op == "F":
                 slot = free.pop(0)
@@ -369,7 +412,7 @@ class StageRuntime:
             else:
                 slot = slot_of.pop(j)
                 d_in = input_grads[j] if (self.needs_input_grad and input_grads is not None) else None
-                self.stage.backward(slot, upstream[j], d_in)
+                self.stage.backward(slot, upstream[j], d_in, ready=ready)
                 free.append(slot)
         self.stage.join()
         return outputs
@@ -381,7 +424,9 @@ class PipelineRuntime:
     (``schedule_ops(i, S, M)``, the rule of bert/graph.py:126-132); an operation is issued once its data is there -
     F(i, j) after F(i-1, j), B(i, j) after B(i+1, j), the last stage's backward after ``loss_fn`` - so the global order
     is one the reference's control dependencies allow.  ``loss_fn(j, last_output) -> (loss, d_last_output)`` is the
-    last stage's head.  ``step`` returns the per-micro-batch losses (``losses[-1]`` is the reference's ``_loss_fn``,
+    last stage's head.  Stages with forward/backward overlap on run their backward passes on streams of their own: the
+    gradient a stage hands down then travels with the event of the pass that wrote it (``Stage.backward_event``), the
+    last stage's with an event recorded behind ``loss_fn``, so a backward pass waits for its data and for nothing else.  ``step`` returns the per-micro-batch losses (``losses[-1]`` is the reference's ``_loss_fn``,
     bert/graph.py:166); weight gradients accumulate in each stage's ``grads``; ``all_outputs[j][i]`` keeps the boundary
     tensor of micro-batch j leaving stage i, like the reference's list of the same name."""
 
@@ -393,9 +438,6 @@ class PipelineRuntime:
             k = min(stash_depth(i, S, variant), num_micro_batches)
             if st.stash_slots < k:
                 raise ValueError("stage %d has %d stash slots, the schedule needs %d" % (i, st.stash_slots, k))
-            if getattr(st, "overlap", False):
-                raise ValueError("PipelineRuntime hands tensors from stage to stage in the order of one stream: "
-                                 "switch the stages' forward/backward overlap off")
             if i > 0 and st.in_numel != self.stages[i - 1].out_numel:
                 raise ValueError("stage %d takes %d elements, stage %d hands over %d" % (i, st.in_numel, i - 1, self.stages[i - 1].out_numel))
         self.issued = []          # (stage, op, micro-batch) in issue order, for inspection
@@ -409,6 +451,8 @@ class PipelineRuntime:
         in_grads = [[torch.empty(st.in_numel, dtype=st.act_dtype, device=dev) if st.takes_input_grad else None
                      for st in self.stages] for _ in range(M)]
         d_last = [None] * M
+        d_ready = [None] * M
+        bwd_event = [dict() for _ in range(S)]
         losses = [None] * M
         fdone = [[False] * M for _ in range(S)]
         bdone = [[False] * M for _ in range(S)]
@@ -432,12 +476,24 @@ class PipelineRuntime:
                         fdone[i][j] = True
                         if i == S - 1:
                             losses[j], d_last[j] = self.loss_fn(j, self.all_outputs[j][i])
+                            d_ready[j] = torch.cuda.Event()
+                            d_ready[j].record()
                     else:
                         if i < S - 1 and not bdone[i + 1][j]:
                             break
                         d_out = d_last[j] if i == S - 1 else in_grads[j][i + 1]
-                        st.backward(slot_of[i][j], d_out.reshape(-1), in_grads[j][i])
-                        free[i].append(slot_of[i].pop(j))
+                        slot = slot_of[i].pop(j)
+                        if i == S - 1:
+                            ready = d_ready[j]
+                        else:
+                            # the pass of the next stage that wrote d_out: its event if it ran on a stream of its own
+                            # (read before that slot is used again), else the order of the shared stream
+                            ready = bwd_event[i + 1].pop(j)
+                            if ready is None:
+                                ready = False
+                        st.backward(slot, d_out.reshape(-1), in_grads[j][i], ready=ready)
+                        bwd_event[i][j] = st.backward_event(slot)
+                        free[i].append(slot)
                         bdone[i][j] = True
                     self.issued.append((i, op, j))
                     cursor[i] += 1

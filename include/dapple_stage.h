@@ -205,8 +205,20 @@ int ds_stage_forward(ds_stage* h, int slot, const void* in, const float* key_mas
  * (segment_ids of bert/models/bert/bert.py:390); NULL or never called: all zeros
  * (modeling_slice.py:785-786).  Only for stages with an embedding. */
 int ds_stage_set_token_types(ds_stage* h, int slot, const int32_t* token_type_ids);
-/* d_in may be NULL for a first stage (bert/graph.py:121 takes no input gradient there). */
+/* d_in may be NULL for a first stage (bert/graph.py:121 takes no input gradient there).
+ * Ordering of d_out and d_in (the data edges prev_grads -> tf.gradients -> y_grads[0] of bert/graph.py:110-143):
+ * on one stream everything follows the stage's stream.  With ds_stage_enable_overlap the pass runs on the handle's
+ * backward stream: ds_stage_backward then waits for everything queued on the stage's stream up to the call (whatever
+ * produced d_out there - a loss head, the next stage - is honoured, at the price that a forward pass queued before the
+ * call also finishes first); ds_stage_backward_after waits only for `ready_event` (a hipEvent_t the caller recorded
+ * behind the producer of d_out, on any stream; NULL: d_out is already complete, or was queued before F(slot) on the
+ * stage's stream), which keeps a forward pass queued earlier running beside this backward pass.  d_in and the
+ * gradients of this pass are ready when the event ds_stage_backward_event returns has completed (NULL on one stream);
+ * ds_stage_wait_backward puts `stream` behind it; ds_stage_join does so for the stage's own stream at the end of a step. */
 int ds_stage_backward(ds_stage* h, int slot, const void* d_out, void* d_in);
+int ds_stage_backward_after(ds_stage* h, int slot, const void* d_out, void* d_in, void* ready_event);
+void* ds_stage_backward_event(ds_stage* h, int slot);
+int ds_stage_wait_backward(ds_stage* h, int slot, void* stream);
 size_t ds_stage_workspace_bytes(const ds_stage* h);
 size_t ds_stage_stash_bytes(const ds_stage* h, int slots);
 int ds_stage_sync(ds_stage* h);

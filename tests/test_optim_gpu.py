@@ -89,6 +89,30 @@ def test_padding_between_tensors_is_left_alone():
     assert torch.all(fp.flat_weights[mask] == 6.0) and torch.all(fp.flat_weights[~mask] == 7.0)
 
 
+def test_clip_by_global_norm_over_several_parameter_sets():
+    """tf.clip_by_global_norm runs over the gradients of all slices (bert/graph.py:162-165): two parameter sets given
+    as a list share one norm and one factor; given one by one each would get its own."""
+    wa, r = make_params(11)
+    wb = {"head/output_weights": r.standard_normal((2, 40)).astype(np.float32), "head/output_bias": r.standard_normal(2).astype(np.float32)}
+    fa, fb = optim.FlatParams(wa), optim.FlatParams(wb)
+    ga = {n: (r.standard_normal(a.shape) * 3).astype(np.float32) for n, a in wa.items()}
+    gb = {n: (r.standard_normal(a.shape) * 0.05).astype(np.float32) for n, a in wb.items()}
+    for fp, g in ((fa, ga), (fb, gb)):
+        for n in g:
+            fp.grads[n].copy_(torch.as_tensor(g[n]))
+    clip = 0.75
+    opt = optim.GradientDescentOptimizer(0.5)
+    opt.apply_gradients([fa, fb], max_gradient_norm=clip)
+    names = list(ga) + list(gb)
+    clipped, norm = oo.clip_by_global_norm([ga[n] for n in ga] + [gb[n] for n in gb], clip)
+    assert norm > clip * 4          # the clip is active, and set b alone would not have been clipped at all
+    assert np.sqrt(sum(float((g.astype(np.float64) ** 2).sum()) for g in gb.values())) < clip
+    ref = dict(zip(names, clipped))
+    for fp, w in ((fa, wa), (fb, wb)):
+        for n in w:
+            assert_close(fp.weights[n], w[n].astype(np.float64) - 0.5 * ref[n], 1e-5, "sgd under the global clip: " + n)
+
+
 def test_stage_step_apply_refresh_forward():
     # one training step of a BERT stage: accumulate over M micro-batches, clip, AdamWeightDecay, refresh; the next
     # forward must equal the oracle's forward with the oracle-updated weights
@@ -105,8 +129,7 @@ def test_stage_step_apply_refresh_forward():
     rt = runtime.StageRuntime(st, 0, 2, M)
     rt.step(xs, dys, outs, dxs)
     opt = optim.AdamWeightDecayOptimizer(1e-3, weight_decay_rate=0.01, exclude_from_weight_decay=EXCLUDE)
-    opt.apply_gradients(st, max_gradient_norm=1.0)
-    st.refresh_weights()
+    opt.apply_gradients(st, max_gradient_norm=1.0)     # marks the stage: its next forward pass rebuilds the compute copies
     st.zero_grads()
     rt.step(xs, dys, outs, dxs)
     st.sync()

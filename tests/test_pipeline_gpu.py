@@ -12,8 +12,11 @@ from util import assert_close, dev
 pytestmark = pytest.mark.gpu
 
 
+@pytest.mark.parametrize("overlap", [False, True])
 @pytest.mark.parametrize("split,M", [((1, 2, 1), 5), ((2, 2), 3), ((4,), 2)])
-def test_whole_model_pipeline_matches_autograd(split, M):
+def test_whole_model_pipeline_matches_autograd(split, M, overlap):
+    """overlap: every stage runs its backward passes on streams of its own; the gradient handed from stage to stage then
+    travels with the event of the pass that wrote it."""
     H, N, F, B, S, V = 64, 4, 128, 2, 16, 50
     L = sum(split)
     emb = (V, 2, 32)
@@ -29,6 +32,9 @@ def test_whole_model_pipeline_matches_autograd(split, M):
         st = runtime.bert_stage(n, H, N, F, B, S, "fp32", stash_slots=runtime.stash_depth(i, nst),
                                 embeddings=emb if i == 0 else None, first_layer=first, wgrad_group=2 if i == 0 else 1)
         st.bind(w_np)
+        if overlap:
+            assert st.overlap_supported()
+            st.enable_overlap()
         stages.append(st)
         first += n
     hw, hb = dev(hw_np, torch.float32), dev(hb_np, torch.float32)
@@ -78,6 +84,62 @@ def test_whole_model_pipeline_matches_autograd(split, M):
     assert_close(dhb, acc[-1], 1e-4, "head bias", floor=float(acc[-2].abs().max()))
     for st in stages:
         st.close()
+
+
+def test_backward_waits_for_upstream_gradient_produced_on_the_stage_stream():
+    """Forward/backward overlap on: the upstream gradient of a pass is written by kernels queued on the stage's stream
+    AFTER that micro-batch's forward pass (a loss head), with the next forward pass queued behind them.  Both ways of
+    saying when it is ready - ds_stage_backward (everything queued so far) and ds_stage_backward_after (an event behind
+    the producer) - give the one-stream result bit for bit."""
+    L, H, N, F, B, S, M = 2, 256, 4, 1024, 2, 128, 4
+    w_np = synthetic.bert_weights(61, L, H, F, stddev=0.05, perturb=True)
+    xs = [dev(x, torch.bfloat16) for x in synthetic.bert_activation_inputs(62, M, B, S, H)]
+    seed = [dev(x, torch.bfloat16) for x in synthetic.upstream_grads(63, M, (B * S, H))]
+
+    def run(mode):
+        st = runtime.bert_stage(L, H, N, F, B, S, "bf16", stash_slots=2)
+        st.bind(w_np)
+        if mode != "one stream":
+            st.enable_overlap()
+        outs = [torch.empty(B * S, H, dtype=torch.bfloat16, device="cuda") for _ in range(M)]
+        dxs = [torch.empty_like(o) for o in outs]
+        douts = [torch.full_like(o, float("nan")) for o in outs]
+        slot_of, free = {}, [0, 1]
+
+        def produce(j):   # a slow elementwise chain standing in for a loss head: d_out = f(out, seed)
+            t = outs[j].float()
+            for _ in range(40):
+                t = t * 0.999 + 0.001
+            douts[j].copy_(t.to(torch.bfloat16) * 0.01 + seed[j])
+            ev = torch.cuda.Event()
+            ev.record()
+            return ev
+
+        evs = {}
+        for op, j in runtime.schedule_ops(0, 2, M):
+            if op == "F":
+                slot_of[j] = free.pop(0)
+                st.forward(slot_of[j], xs[j], outs[j])
+                evs[j] = produce(j)
+            else:
+                st.backward(slot_of[j], douts[j], dxs[j], ready=evs[j] if mode == "event" else False)
+                free.append(slot_of.pop(j))
+        st.sync()
+        res = ([d.clone() for d in dxs], {n: g.clone() for n, g in st.grads.items()})
+        st.close()
+        return res
+
+    ref_dx, ref_g = run("one stream")
+    for mode in ("queued so far", "event"):
+        dx, g = run(mode)
+        for j in range(M):
+            assert torch.equal(dx[j], ref_dx[j]), "%s: input gradient of micro-batch %d" % (mode, j)
+        for n in ref_g:
+            # LayerNorm / bias gradients are fp32 atomic sums whose order is not fixed: compare those at rounding level
+            if n.endswith(("kernel",)):
+                assert torch.equal(g[n], ref_g[n]), "%s: %s" % (mode, n)
+            else:
+                assert_close(g[n], ref_g[n], 1e-5, "%s: %s" % (mode, n), floor=float(ref_g[n].abs().max()) + 1e-30)
 
 
 def test_pipeline_rejects_mismatched_stages():
