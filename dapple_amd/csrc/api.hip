@@ -277,6 +277,18 @@ extern "C" int ds_stage_wait_backward(ds_stage* h, int slot, void* stream) {
   return DS_OK;
 }
 
+extern "C" int ds_stage_release_slot(ds_stage* h, int slot) {
+  DS_CHECK_ARG(h != nullptr, "ds_stage_release_slot: null handle");
+  DS_CHECK_ARG(slot >= 0 && slot < h->cfg.stash_slots, "ds_stage_release_slot: slot %d out of range [0,%d)", slot, h->cfg.stash_slots);
+  if (!h->slot_forwarded[slot]) {
+    ds_set_error("ds_stage_release_slot: slot %d holds no forwarded micro-batch", slot);
+    return DS_ESTATE;
+  }
+  DS_PROPAGATE(h->release(slot));
+  h->slot_forwarded[slot] = 0;
+  return DS_OK;
+}
+
 extern "C" size_t ds_stage_workspace_bytes(const ds_stage* h) { return h ? h->workspace_bytes() : 0; }
 extern "C" size_t ds_stage_stash_bytes(const ds_stage* h, int slots) { return h ? h->stash_bytes(slots) : 0; }
 

@@ -340,6 +340,22 @@ extern "C" int ds_classifier_head(int dtype, int batch, int seq, int hidden, int
                                   loss, pooled, logits, dlogits, dz, dx, d_pooler_w, d_pooler_b, d_fc_w, d_fc_b, (hipStream_t)stream);
 }
 
+extern "C" int ds_pooler(int dtype, int batch, int seq, int hidden, const void* x, const float* pooler_w, const float* pooler_b,
+                         float* pooled, void* stream) {
+  DS_CHECK_ARG(dtype == DS_F32 || dtype == DS_BF16, "ds_pooler: dtype %d", dtype);
+  DS_CHECK_ARG(batch > 0 && seq > 0 && hidden > 0 && batch <= 65535, "ds_pooler: bad shape (%d, %d, %d)", batch, seq, hidden);
+  DS_CHECK_ARG(x && pooler_w && pooler_b && pooled, "ds_pooler: null pointer");
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == DS_BF16)
+    hipLaunchKernelGGL((ds_small_dense_kernel<bf16, 1>), dim3((hidden + 63) / 64, batch), dim3(1024), 0, s, hidden, 0, hidden, (const bf16*)x,
+                       (int64_t)seq * hidden, (const float*)nullptr, (int64_t)0, pooler_w, pooler_b, pooled);
+  else
+    hipLaunchKernelGGL((ds_small_dense_kernel<float, 1>), dim3((hidden + 63) / 64, batch), dim3(1024), 0, s, hidden, 0, hidden, (const float*)x,
+                       (int64_t)seq * hidden, (const float*)nullptr, (int64_t)0, pooler_w, pooler_b, pooled);
+  DS_CHECK_LAUNCH();
+  return DS_OK;
+}
+
 extern "C" int ds_regression_head(int dtype, int batch, int seq, int hidden, const void* x, const float* pooler_w, const float* pooler_b,
                                   const float* fc_w, const float* fc_b, const float* targets, float l2_scale, float loss_scale,
                                   float* loss, float* pooled, float* prediction, float* dprediction, float* dz, void* dx,

@@ -48,6 +48,8 @@ struct ds_stage {
   virtual int refresh_weights() = 0;
   virtual int forward(int slot, const void* in, const float* key_mask, void* out) = 0;
   virtual int backward(int slot, const void* d_out, void* d_in) = 0;
+  // gives up the micro-batch forwarded into `slot` without a backward pass (inference, a forward-only probe)
+  virtual int release(int slot) { (void)slot; return DS_OK; }
   virtual size_t workspace_bytes() const = 0;
   virtual size_t stash_bytes(int slots) const = 0;
   // queues weight-gradient work that backward passes have deferred; `final`: and orders it before what the

@@ -495,6 +495,15 @@ struct BertStage : ds_stage {
     return DS_OK;
   }
 
+  int release(int slot) override {
+    if (G > 1) {  // the stash position goes back to the pool; nothing was deferred for it
+      const int pos = slot_pos[slot];
+      pos_owner[pos] = -1;
+      x_bwd_valid[pos] = 0;
+    }
+    return DS_OK;
+  }
+
   int backward(int slot, const void* d_out, void* d_in) override {
     ds_prio_scope prio(3);  // the chain every later pass waits on
     const int pos = slot_pos[slot];

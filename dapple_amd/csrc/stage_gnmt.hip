@@ -1125,3 +1125,29 @@ extern "C" int ds_gnmt_stage_set_decoder_inputs(ds_stage* h, int slot, const int
   DS_PROPAGATE(ds_stage_acquire_slot(h, slot));
   return st->set_inputs(slot, target_input, source_sequence_length, attention_out);
 }
+
+// ------------------------------------------------------------------ the cell kernels on their own
+extern "C" int ds_lstm_cell_fwd(int batch, int units, float forget_bias, float* gates, const float* c_prev, float* c, float* h,
+                                const float* x_residual, float* y, void* stream) {
+  DS_CHECK_ARG(batch > 0 && units > 0 && (int64_t)batch * units < ((int64_t)1 << 31), "ds_lstm_cell_fwd: bad shape (%d, %d)", batch, units);
+  DS_CHECK_ARG(gates && c && h, "ds_lstm_cell_fwd: null pointer");
+  DS_CHECK_ARG((x_residual == nullptr) == (y == nullptr), "ds_lstm_cell_fwd: x_residual and y come together (ResidualWrapper)");
+  hipStream_t s = (hipStream_t)stream;
+  ds_prof_scope prof(s, "lstm_cell_fwd_kernel", (double)batch * units * 4 * (4 + 4 + 2 + (y ? 2 : 1)), "B");
+  hipLaunchKernelGGL(lstm_cell_fwd_kernel, dim3((batch * units + 255) / 256), dim3(256), 0, s, batch, units, forget_bias, gates, c_prev, c, h,
+                     units, x_residual, units, y, units, (const int32_t*)nullptr, 0, (const float*)nullptr, 0);
+  DS_CHECK_LAUNCH();
+  return DS_OK;
+}
+
+extern "C" int ds_lstm_cell_bwd(int batch, int units, const float* gates_act, const float* c, const float* c_prev, const float* dh,
+                                float* dc, int first, float* dgates, void* stream) {
+  DS_CHECK_ARG(batch > 0 && units > 0 && (int64_t)batch * units < ((int64_t)1 << 31), "ds_lstm_cell_bwd: bad shape (%d, %d)", batch, units);
+  DS_CHECK_ARG(gates_act && c && dh && dc && dgates, "ds_lstm_cell_bwd: null pointer");
+  hipStream_t s = (hipStream_t)stream;
+  ds_prof_scope prof(s, "lstm_cell_bwd_kernel", (double)batch * units * 4 * (4 + 4 + 6), "B");
+  hipLaunchKernelGGL(lstm_cell_bwd_kernel, dim3((batch * units + 255) / 256), dim3(256), 0, s, batch, units, gates_act, c, c_prev, dh, units,
+                     (const float*)nullptr, dc, first, dgates, (const int32_t*)nullptr, 0, (float*)nullptr, (const float*)nullptr, 0);
+  DS_CHECK_LAUNCH();
+  return DS_OK;
+}

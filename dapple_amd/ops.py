@@ -252,6 +252,45 @@ def squad_head(x, batch, seq, output_weights, output_bias, start_positions, end_
     return loss, lg[:, :, 0], lg[:, :, 1], dx
 
 
+def pooler(x, batch, seq, pooler_w, pooler_b):
+    """pooler_stage (modeling_slice.py:849-868): tanh dense on each sample's first token -> fp32 [batch, hidden]."""
+    _need_cuda(x, pooler_w, pooler_b)
+    hidden = pooler_w.shape[1]
+    if x.numel() != batch * seq * hidden or tuple(pooler_w.shape) != (hidden, hidden) or pooler_b.numel() != hidden:
+        raise ValueError("pooler: x must be [batch*seq, hidden], pooler_w [hidden, hidden], pooler_b [hidden]")
+    if pooler_w.dtype != torch.float32 or pooler_b.dtype != torch.float32:
+        raise ValueError("pooler: the dense parameters are fp32")
+    pooled = torch.empty(batch, hidden, dtype=torch.float32, device=x.device)
+    check(_lib.load().ds_pooler(dtype_code(x), batch, seq, hidden, ptr(x), ptr(pooler_w), ptr(pooler_b), ptr(pooled),
+                                _lib.current_stream()), "ds_pooler")
+    return pooled
+
+
+def lstm_cell_fwd(gates, c_prev=None, forget_bias=1.0, x_residual=None):
+    """One BasicLSTMCell step on pre-activations ``gates`` fp32 [batch, 4*units] (overwritten with the activated gates):
+    returns (c, h, y) with y = h + x_residual or None."""
+    _need_cuda(gates, c_prev, x_residual)
+    b, u4 = gates.shape
+    u = u4 // 4
+    c = torch.empty(b, u, dtype=torch.float32, device=gates.device)
+    h = torch.empty_like(c)
+    y = torch.empty_like(c) if x_residual is not None else None
+    check(_lib.load().ds_lstm_cell_fwd(b, u, forget_bias, ptr(gates), ptr(c_prev), ptr(c), ptr(h), ptr(x_residual), ptr(y),
+                                       _lib.current_stream()), "ds_lstm_cell_fwd")
+    return c, h, y
+
+
+def lstm_cell_bwd(gates_act, c, c_prev, dh, dc, first):
+    """Backward of one BasicLSTMCell step: returns dgates [batch, 4*units]; ``dc`` [batch, units] carries the cell-state
+    gradient between steps (read unless ``first``, then overwritten with dc * f)."""
+    _need_cuda(gates_act, c, c_prev, dh, dc)
+    b, u4 = gates_act.shape
+    dgates = torch.empty_like(gates_act)
+    check(_lib.load().ds_lstm_cell_bwd(b, u4 // 4, ptr(gates_act), ptr(c), ptr(c_prev), ptr(dh), ptr(dc), 1 if first else 0,
+                                       ptr(dgates), _lib.current_stream()), "ds_lstm_cell_bwd")
+    return dgates
+
+
 def classifier_head(x, batch, seq, pooler_w, pooler_b, fc_w, fc_b, labels, grads=None, need_dx=True, l2_scale=1e-3,
                     loss_scale=1.0):
     """pooler_stage (modeling_slice.py:849-868) + build_output_layer_classification (bert.py:642-664) on the stage's

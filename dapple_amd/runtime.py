@@ -162,6 +162,10 @@ class Stage:
         ev = C.c_void_p(ready) if ready is not None else None
         check(self.lib.ds_stage_backward_after(self._h, slot, ptr(d_out), ptr(d_in), ev), "ds_stage_backward_after")
 
+    def release(self, slot):
+        """Gives up the micro-batch forwarded into ``slot`` without a backward pass (forward-only use)."""
+        check(self.lib.ds_stage_release_slot(self._h, slot), "ds_stage_release_slot")
+
     def backward_event(self, slot):
         """Raw handle of the event that completes when the last backward pass of ``slot`` has written its input gradient
         (None on one stream: the pass is ordered on the stage's stream)."""

@@ -117,7 +117,7 @@ class BertModelSlice(object):
             st = self._op_stage("emb")
             out = torch.empty(self.batch_size * self.seq_length, config.hidden_size, dtype=st.act_dtype, device=input_ids.device)
             st.forward(0, self.input_ids, out, token_type_ids=self.token_type_ids)
-            st.backward(0, torch.zeros_like(out))         # frees the slot; gradients of a zero upstream are zero
+            st.release(0)
             self.embedding_output = out.reshape(self.batch_size, self.seq_length, config.hidden_size)
             return self.embedding_output
 
@@ -135,7 +135,7 @@ class BertModelSlice(object):
                 st = self._op_stage(idx)
                 out = torch.empty_like(layer_input)
                 st.forward(0, layer_input.contiguous(), out, key_mask=self._key_mask)
-                st.backward(0, torch.zeros_like(out), None)
+                st.release(0)
                 final = out.reshape(self.batch_size, self.seq_length, config.hidden_size)
                 self.all_encoder_layers.append(final)
                 self.sequence_output = final
@@ -143,12 +143,33 @@ class BertModelSlice(object):
             return encoder_layer
 
         def pooler_stage(sequence_output, *args):
-            raise NotImplementedError("the pooler belongs to the last pipeline stage (bert.py:669-718), which this "
-                                      "runtime does not build")
+            # modeling_slice.py:849-868: tanh dense (bert/pooler/dense) on the first token of every sample
+            from . import ops
+            if self.sequence_output is None:
+                self.sequence_output = sequence_output
+            x = self.sequence_output.reshape(self.batch_size * self.seq_length, config.hidden_size).contiguous()
+            kernel, bias = self._pooler_params(x.device)
+            self.pooled_output = ops.pooler(x, self.batch_size, self.seq_length, kernel, bias)
+            return self.pooled_output
 
         self.stages = [embedding_stage, reshape_input]
         self.stages += [create_layer(i) for i in range(config.num_hidden_layers)]
         self.stages.append(pooler_stage)
+
+    def _pooler_params(self, device):
+        """bert/pooler/dense/{kernel, bias} from ``weights`` when present, else truncated-normal-like N(0, initializer_range)
+        and zeros (modeling_slice.py:862-866) drawn once."""
+        if getattr(self, "_pooler", None) is None:
+            H = self.config.hidden_size
+            if "bert/pooler/dense/kernel" in self.weights:
+                k = torch.as_tensor(self.weights["bert/pooler/dense/kernel"], dtype=torch.float32)
+                b = torch.as_tensor(self.weights["bert/pooler/dense/bias"], dtype=torch.float32)
+            else:
+                g = torch.Generator().manual_seed(4321)
+                k = torch.randn(H, H, generator=g) * self.config.initializer_range
+                b = torch.zeros(H)
+            self._pooler = (k.to(device).contiguous(), b.to(device).contiguous())
+        return self._pooler
 
     def _op_stage(self, which):
         """A one-op stage handle (the embedding, or encoder layer ``which``), created on first use."""
@@ -224,6 +245,8 @@ class BertFinetuneSlice(object):
                                                          bert_config.max_position_embeddings),
                                              stddev=bert_config.initializer_range)
         self.stage.bind(weights)
+        self._model_args = (bert_config, is_training, input_ids, input_mask, segment_ids, use_one_hot_embeddings, weights, dtype)
+        self._model = None
         self.layers, self.local_device, self.model_type = layers, local_device, model_type
         self.stage_outputs = []
         self.is_last = (nstage - 1) in mine
@@ -248,6 +271,22 @@ class BertFinetuneSlice(object):
             self.fc_weights = ((torch.rand(H, nout, generator=g) * 2 - 1) * limit).cuda()
             self.fc_biases = torch.full((nout,), 1e-4, device="cuda")
             self.head_grads = [torch.zeros_like(t) for t in (self.pooler_kernel, self.pooler_bias, self.fc_weights, self.fc_biases)]
+
+    @property
+    def model(self):
+        """The ``BertModelSlice`` whose ``stages`` this class places on the devices (bert.py:399-408); built on first
+        use, over the same weights as ``stage`` (its one-op handles are created as they are called)."""
+        if self._model is None:
+            cfg, is_training, ids, mask, seg, one_hot, weights, dtype = self._model_args
+            self._model = BertModelSlice(config=cfg, is_training=False, input_ids=ids, input_mask=mask, token_type_ids=seg,
+                                         use_one_hot_embeddings=one_hot, weights=weights, dtype=dtype)
+        return self._model
+
+    @property
+    def stages(self):
+        """``self.model.stages`` (bert.py:414): the per-op callables [embedding_stage, reshape_input, layer_0 ..,
+        pooler_stage]; ``device_of[i]`` is the device ``calc_device`` gives entry i."""
+        return self.model.stages
 
     def build_output_layer_squad(self, sequence_output, is_training=False):
         """bert.py:669-718 on the last device: start / end logits and the SQuAD loss from
@@ -326,7 +365,7 @@ class SliceVGG19(object):
             self.stage.bind(self._weight_values or synthetic.vgg_weights(self._seed, self.layers, c))
         out = torch.empty(self.stage.out_shape, device=features.device)
         self.stage.forward(0, features.contiguous(), out)
-        self.stage.backward(0, torch.zeros_like(out))
+        self.stage.release(0)
         return None, [out]
 
 
@@ -393,7 +432,7 @@ class XlnetSlice(object):
         """inputs: the boundary activation(s) [streams, seq, batch, hidden]; returns (None, [stage_output])."""
         out = torch.empty(self.stage.out_shape, dtype=self.stage.act_dtype, device=inputs.device)
         self.stage.forward(0, inputs.contiguous(), out)
-        self.stage.backward(0, torch.zeros_like(out), None)
+        self.stage.release(0)
         return None, [out]
 
 
@@ -435,7 +474,7 @@ class GNMTEncoderSlice(object):
         self.stage.set_lengths(0, None if source_sequence_length is None else
                                source_sequence_length.to(torch.int32).contiguous())
         self.stage.forward(0, source_ids.to(torch.int32).contiguous(), out)
-        self.stage.backward(0, torch.zeros_like(out))
+        self.stage.release(0)
         return out
 
 

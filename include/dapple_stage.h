@@ -219,6 +219,9 @@ int ds_stage_backward(ds_stage* h, int slot, const void* d_out, void* d_in);
 int ds_stage_backward_after(ds_stage* h, int slot, const void* d_out, void* d_in, void* ready_event);
 void* ds_stage_backward_event(ds_stage* h, int slot);
 int ds_stage_wait_backward(ds_stage* h, int slot, void* stream);
+/* Gives up the micro-batch forwarded into `slot` without a backward pass: a forward-only use of the stage (the
+ * reference's is_training=False graphs, bert/models/bert/modeling_slice.py:774-776, build no gradients). */
+int ds_stage_release_slot(ds_stage* h, int slot);
 size_t ds_stage_workspace_bytes(const ds_stage* h);
 size_t ds_stage_stash_bytes(const ds_stage* h, int slots);
 int ds_stage_sync(ds_stage* h);
@@ -299,6 +302,18 @@ int ds_gnmt_stage_create(const ds_gnmt_cfg* cfg, void* stream, ds_stage** out);
  * gets it: steps t >= lengths[b] emit zeros (residual layers too) and keep the state, the backward
  * direction of the first layer starts at step lengths[b] - 1.  The setting stays with the slot. */
 int ds_gnmt_stage_set_lengths(ds_stage* h, int slot, const int32_t* lengths);
+/* One time step of BasicLSTMCell (gnmt/nmt/model_helper.py:418-420; TensorFlow's cell: one kernel applied to
+ * concat([x, h]), gates split as i, j, f, o) without the matrix product, for unit parity of the stage's cell kernels.
+ *   fwd: gates fp32 [batch, 4*units] holds the pre-activations (bias included) and is overwritten with sigmoid(i),
+ *        tanh(j), sigmoid(f + forget_bias), sigmoid(o); c = c_prev * f + i * j (c_prev NULL: zero state);
+ *        h = tanh(c) * o; with x_residual and y (ResidualWrapper, :445-448) y = h + x_residual.
+ *   bwd: gates_act / c / c_prev as the forward step left them; dh fp32 [batch, units] = gradient reaching h at this
+ *        step (output plus recurrent); dc in: the cell-state gradient from the step after (ignored when first != 0),
+ *        out: dc * f for the step before; dgates fp32 [batch, 4*units] out: gradients of the pre-activations. */
+int ds_lstm_cell_fwd(int batch, int units, float forget_bias, float* gates, const float* c_prev, float* c, float* h,
+                     const float* x_residual, float* y, void* stream);
+int ds_lstm_cell_bwd(int batch, int units, const float* gates_act, const float* c, const float* c_prev, const float* dh, float* dc,
+                     int first, float* dgates, void* stream);
 /* part = DS_GNMT_DECODER_PART2: decoder cells first_layer .. first_layer + num_layers - 1 as the reference's second device runs
  * them - GNMTAttentionMultiCell_2, gnmt/nmt/gnmt_model.py:489-537, under dynamic_decode with a TrainingHelper on the
  * outputs of cell 0 (gnmt/nmt/model.py:641-656): a scan over all `seq` padded target steps from the zero state
@@ -378,6 +393,11 @@ int ds_classifier_head(int dtype, int batch, int seq, int hidden, int num_labels
                        const float* pooler_b, const float* fc_w, const float* fc_b, const int32_t* labels, float l2_scale,
                        float loss_scale, float* loss, float* pooled, float* logits, float* dlogits, float* dz, void* dx,
                        float* d_pooler_w, float* d_pooler_b, float* d_fc_w, float* d_fc_b, void* stream);
+
+/* pooler_stage alone (bert/models/bert/modeling_slice.py:849-868), the last entry of BertModelSlice.stages:
+ * pooled[b] = tanh(x[b, token 0] . pooler_w + pooler_b), pooled fp32 [batch, hidden]. */
+int ds_pooler(int dtype, int batch, int seq, int hidden, const void* x, const float* pooler_w, const float* pooler_b, float* pooled,
+              void* stream);
 
 /* Pooler and regression head of the last BERT stage: pooler_stage (bert/models/bert/modeling_slice.py:849-868) and
  * build_output_layer_regression, bert/models/bert/bert.py:615-640: prediction = fully_connected(pooled) to ONE output

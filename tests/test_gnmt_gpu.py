@@ -64,3 +64,63 @@ def test_ragged_sequences():
     """source_sequence_length per micro-batch: full, single-step, empty and in-between sequences; the second
     micro-batch reuses a slot whose previous lengths were different, the third goes back to full length."""
     run_case(L=4, U=32, V=50, B=4, T=6, M=3, init=0.4, seed=3, lengths=[[6, 1, 3, 5], [2, 6, 0, 4], [6, 6, 6, 6]])
+
+
+@pytest.mark.parametrize("B,U,residual", [(3, 8, False), (64, 1024, True), (5, 96, True)])
+def test_lstm_cell_kernels_against_torch_lstmcell(B, U, residual):
+    """The cell kernels on their own (ds_lstm_cell_fwd / ds_lstm_cell_bwd): BasicLSTMCell's step - gate order i, j, f, o,
+    forget_bias added to f - is torch.nn.LSTMCell's (order i, f, g, o) after permuting the gate blocks and folding the
+    forget bias into the bias; the backward kernel against autograd through that cell over two chained steps."""
+    from dapple_amd import ops
+    r = np.random.default_rng(B * 7 + U)
+    fb = 1.0
+    pre = [r.standard_normal((B, 4 * U)) for _ in range(2)]          # pre-activations of two consecutive steps (i, j, f, o)
+    xres = [r.standard_normal((B, U)) for _ in range(2)]
+    dys = [r.standard_normal((B, U)) for _ in range(2)]
+
+    def cell_ref(g, c_prev):                                          # fp64 restatement through torch's gate algebra
+        i, j, f, o = g[:, :U], g[:, U:2 * U], g[:, 2 * U:3 * U], g[:, 3 * U:]
+        c = c_prev * torch.sigmoid(f + fb) + torch.sigmoid(i) * torch.tanh(j)
+        return c, torch.tanh(c) * torch.sigmoid(o)
+
+    # pin the restatement above to torch.nn.LSTMCell with zero weights and the pre-activation as its bias
+    cell = torch.nn.LSTMCell(1, U).double()
+    with torch.no_grad():
+        cell.weight_ih.zero_(); cell.weight_hh.zero_(); cell.bias_hh.zero_()
+    g0 = torch.as_tensor(pre[0])
+    perm = torch.cat([g0[:, :U], g0[:, 2 * U:3 * U] + fb, g0[:, U:2 * U], g0[:, 3 * U:]], 1)   # i, f, g, o
+    hs, cs = [], []
+    for b in range(min(B, 3)):
+        with torch.no_grad():
+            cell.bias_ih.copy_(perm[b])
+        h1, c1 = cell(torch.zeros(1, 1).double(), (torch.zeros(1, U).double(), torch.zeros(1, U).double()))
+        hs.append(h1); cs.append(c1)
+    c_chk, h_chk = cell_ref(g0[:min(B, 3)], torch.zeros(min(B, 3), U).double())
+    assert torch.allclose(torch.cat(hs), h_chk, atol=1e-12) and torch.allclose(torch.cat(cs), c_chk, atol=1e-12)
+
+    gt = [torch.as_tensor(p).requires_grad_(True) for p in pre]
+    c1, h1 = cell_ref(gt[0], torch.zeros(B, U).double())
+    # step 2's pre-activation depends on h1 through a fixed linear map, standing in for the recurrent product
+    Wr = torch.as_tensor(r.standard_normal((U, 4 * U)) * 0.1)
+    g2 = gt[1] + h1 @ Wr
+    c2, h2 = cell_ref(g2, c1)
+    y1 = h1 + torch.as_tensor(xres[0]) if residual else h1
+    y2 = h2 + torch.as_tensor(xres[1]) if residual else h2
+    loss = (y1 * torch.as_tensor(dys[0])).sum() + (y2 * torch.as_tensor(dys[1])).sum()
+    dg1_ref, dg2_ref = torch.autograd.grad(loss, [gt[0], g2])
+
+    # GPU: forward step 1, the recurrent product on the host side of the test, forward step 2
+    ga1 = dev(pre[0], torch.float32)
+    cg1, hg1, yg1 = ops.lstm_cell_fwd(ga1, None, fb, dev(xres[0], torch.float32) if residual else None)
+    ga2 = (dev(pre[1], torch.float32).double() + hg1.double() @ Wr.cuda()).float().contiguous()
+    cg2, hg2, yg2 = ops.lstm_cell_fwd(ga2, cg1, fb, dev(xres[1], torch.float32) if residual else None)
+    assert_close(hg1, h1.detach(), 1e-5, "h1"); assert_close(cg2, c2.detach(), 1e-5, "c2"); assert_close(hg2, h2.detach(), 1e-5, "h2")
+    if residual:
+        assert_close(yg2, y2.detach(), 1e-5, "y2 = h2 + x")
+    # backward: step 2 first (no recurrent gradient flows into the last step), then step 1 with dh = dy1 + dgates2 Wr^T
+    dc = torch.zeros(B, U, device="cuda")
+    dgg2 = ops.lstm_cell_bwd(ga2, cg2, cg1, dev(dys[1], torch.float32), dc, first=True)
+    assert_close(dgg2, dg2_ref, 1e-4, "dgates of step 2")
+    dh1 = (dev(dys[0], torch.float32).double() + dgg2.double() @ Wr.cuda().T).float().contiguous()
+    dgg1 = ops.lstm_cell_bwd(ga1, cg1, None, dh1, dc, first=False)
+    assert_close(dgg1, dg1_ref, 1e-4, "dgates of step 1")

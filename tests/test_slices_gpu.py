@@ -28,8 +28,17 @@ def test_bert_model_slice_stages_like_modeling_test():
     w = ob.to_torch(model.weights)
     want = ob.stage_forward(ids.cpu(), w, [0, 1], B, S, 4)
     assert_close(x, want, 1e-4, "stages chained")
-    with pytest.raises(NotImplementedError):
-        model.stages[-1](x)
+    # the last entry is pooler_stage (modeling_slice.py:849-868): tanh dense on the first token
+    pooled = model.stages[-1](x)
+    assert pooled is model.get_pooled_output() and pooled.shape == (B, 32)
+    pk, pb = model._pooler_params(x.device)
+    first = want.reshape(B, S, 32)[:, 0, :].double()
+    assert_close(pooled, torch.tanh(first @ pk.cpu().double() + pb.cpu().double()), 1e-4, "pooler_stage")
+    # calling the stages again works: a forward-only call gives its stash slot back without a backward pass
+    x2 = ids
+    for f in model.stages[:-1]:
+        x2 = f(x2)
+    assert torch.equal(x2, x)
     bad = slices.BertConfig(vocab_size=9, hidden_size=30, num_attention_heads=4)
     with pytest.raises(ValueError, match="not a multiple of the number of attention"):
         slices.BertModelSlice(bad, False, ids)
@@ -46,6 +55,9 @@ def test_bert_finetune_slice_puts_the_planner_split_on_each_device():
     s1 = slices.BertFinetuneSlice(cfg, 8, False, ids, None, None, None, False, model_type="mrc",
                                   slice_devices=["/gpu:0", "/gpu:1"], local_device=1, dtype="fp32")
     assert s0.layers == list(range(11)) and s1.layers == list(range(11, 24))
+    # .stages is the model's list of per-op callables (bert.py:414), 27 entries for BERT-24, placed by calc_device
+    assert len(s1.stages) == 27 and s1.stages is s1.model.stages
+    assert [s1.device_of[i] for i in (0, 12, 13, 26)] == [0, 0, 1, 1]
     assert s0.stage.takes_input_grad is False and s1.stage.takes_input_grad is True
     assert s0.stage.stash_slots == 2 and s1.stage.stash_slots == 1          # K = S - i
     assert s0.stage.weight_names[0] == "bert/embeddings/word_embeddings"
