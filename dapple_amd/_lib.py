@@ -91,6 +91,7 @@ PROTOTYPES = {
     "ds_cast_bf16_to_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "ds_gemm": (C.c_int, [C.POINTER(GemmDesc), C.c_void_p]),
     "ds_gemm_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int]),
+    "ds_gemm_static_scratch": (C.c_int, [C.POINTER(GemmDesc), C.c_void_p]),
     "ds_pooler": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "ds_stage_release_slot": (C.c_int, [C.c_void_p, C.c_int]),
     "ds_lstm_cell_fwd": (C.c_int, [C.c_int, C.c_int, C.c_float] + [C.c_void_p] * 7),

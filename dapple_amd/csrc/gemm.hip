@@ -754,7 +754,7 @@ __global__ __launch_bounds__(256) void gemm_k64_f32out_kernel(GemmArgs p) {
     }
 }
 
-static int gemm_run(const ds_gemm_desc* d, int splitk_req, void* stream) {
+static int gemm_run(const ds_gemm_desc* d, int splitk_req, void* stream, bool must_split = false) {
   DS_CHECK_ARG(d != nullptr, "ds_gemm: null descriptor");
   DS_CHECK_ARG(d->dtype == DS_F32 || d->dtype == DS_BF16, "ds_gemm: dtype %d", d->dtype);
   DS_CHECK_ARG((d->a_major | 1) == 1 && (d->b_major | 1) == 1, "ds_gemm: operand major must be 0 or 1");
@@ -859,6 +859,11 @@ static int gemm_run(const ds_gemm_desc* d, int splitk_req, void* stream) {
         const int forced = atoi(env_sk);
         slices = forced <= 1 || forced > 4 || tiles > 1024 ? 0 : (ktiles % forced == 0 && ktiles / forced > ds_gemm8_stages(4) ? forced : 0);
       }
+      if (must_split && slices <= 1) {
+        ds_set_error("ds_gemm_static_scratch: %d x %d x %d is not a shape that is cut into k slices (at most 64 tile-slices of "
+                     "128 x 128, every slice at least 32 k-tiles of 64)", d->m, d->n, d->k);
+        return DS_EINVAL;
+      }
       if (slices > 1) {
         DS_CHECK_ARG(((uintptr_t)d->workspace & 255) == 0 && d->workspace_bytes >= ds_gemm_workspace_bytes(d->m, d->n),
                      "ds_gemm: workspace must be 256-byte aligned and hold ds_gemm_workspace_bytes(m, n) = %zu bytes (got %zu)",
@@ -874,6 +879,10 @@ static int gemm_run(const ds_gemm_desc* d, int splitk_req, void* stream) {
         return ds_gemm8_launch(a, 4, d->a_major, d->b_major, 1, s);
       }
     }
+    if (must_split) {
+      ds_set_error("ds_gemm_static_scratch: batched GEMMs are not cut into k slices");
+      return DS_EINVAL;
+    }
     if (cfg8 >= 0 && ktiles > ds_gemm8_stages(cfg8)) {
       char tag8[96];
       snprintf(tag8, sizeof(tag8), "gemm8_kernel<bf16,%d,%d,%s,%s>", bm8[cfg8], bn8[cfg8],
@@ -881,6 +890,10 @@ static int gemm_run(const ds_gemm_desc* d, int splitk_req, void* stream) {
       ds_prof_scope prof8(s, tag8, 2.0 * d->m * d->n * d->k * batch, "FLOP");
       return ds_gemm8_launch(a, cfg8, d->a_major, d->b_major, batch, s);
     }
+  }
+  if (must_split) {
+    ds_set_error("ds_gemm_static_scratch: needs bf16 operands, k a multiple of 64 and 16-byte aligned, 8-column outputs");
+    return DS_EINVAL;
   }
   static const int tbm[3] = {128, 128, 64}, tbn[3] = {128, 64, 64};
   char tag[96];
@@ -894,6 +907,44 @@ static int gemm_run(const ds_gemm_desc* d, int splitk_req, void* stream) {
 
 
 extern "C" int ds_gemm(const ds_gemm_desc* d, void* stream) { return gemm_run(d, 1, stream); }
+
+// ------------------------------------------------------------------------------------------
+// ds_gemm for callers that cannot allocate (code under HIP graph capture, serving loops): the split-K workspace is
+// this array instead of caller memory.  Every GPU the library runs on holds its own copy until the process ends.
+namespace {
+constexpr int SCRATCH_MAX_TILES = 16;  // 128x128 output tiles, e.g. 512 x 512 or 128 x 2048
+constexpr size_t SCRATCH_BYTES = 4096 + (size_t)SCRATCH_MAX_TILES * 4 * 128 * 128 * sizeof(float);  // 4 MiB + 4 KiB
+constexpr int SCRATCH_MAX_DEVICES = 64;
+void* g_scratch_ptr[SCRATCH_MAX_DEVICES] = {};
+__global__ void scratch_clear_counters_kernel(unsigned* p) { p[threadIdx.x] = 0u; }
+}  // namespace
+static __device__ __align__(256) unsigned char scratch[SCRATCH_BYTES];
+
+extern "C" int ds_gemm_static_scratch(const ds_gemm_desc* d, void* stream) {
+  DS_CHECK_ARG(d != nullptr, "ds_gemm_static_scratch: null descriptor");
+  DS_CHECK_ARG(d->m > 0 && d->n > 0, "ds_gemm_static_scratch: m, n must be positive (%d %d)", d->m, d->n);
+  const int64_t tiles = (int64_t)((d->m + 127) / 128) * ((d->n + 127) / 128);
+  DS_CHECK_ARG(tiles <= SCRATCH_MAX_TILES,
+               "ds_gemm_static_scratch: a %d x %d output has %lld tiles of 128 x 128, the library's scratch holds %d (%zu bytes)",
+               d->m, d->n, (long long)tiles, SCRATCH_MAX_TILES, SCRATCH_BYTES);
+  int dev = -1;
+  DS_CHECK_HIP(hipGetDevice(&dev));
+  DS_CHECK_ARG(dev >= 0 && dev < SCRATCH_MAX_DEVICES, "ds_gemm_static_scratch: device %d", dev);
+  if (g_scratch_ptr[dev] == nullptr) {
+    // once per device, with that device current: the array's name is only a host-side handle, its device address
+    // comes from the runtime.  The arrival counters start at zero (a kernel, not a memset: callers may capture later
+    // calls into a graph, and every launch leaves the counters at zero again).
+    void* ptr = nullptr;
+    DS_CHECK_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    hipLaunchKernelGGL(scratch_clear_counters_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, (unsigned*)ptr);
+    DS_CHECK_LAUNCH();
+    g_scratch_ptr[dev] = ptr;
+  }
+  ds_gemm_desc c = *d;
+  c.workspace = g_scratch_ptr[dev];
+  c.workspace_bytes = SCRATCH_BYTES;
+  return gemm_run(&c, 1, stream, true);
+}
 
 // 4 KiB of arrival counters (one per 128x128 tile, at most 1024 tiles), then up to 4 fp32 partial tiles per tile
 extern "C" size_t ds_gemm_workspace_bytes(int m, int n) {

@@ -56,9 +56,10 @@ def cast_to_f32(src):
 
 def gemm(a, b, c, m, n, k, a_major=DS_K_MAJOR, b_major=DS_MN_MAJOR, lda=None, ldb=None, ldc=None, flags=0,
          alpha=1.0, bias=None, residual=None, c2=None, batch=1, batch_inner=1, a_strides=(0, 0), b_strides=(0, 0),
-         c_strides=(0, 0), workspace=None):
+         c_strides=(0, 0), workspace=None, static_scratch=False):
     """Raw ds_gemm: C[m][n] (+)= alpha * sum_k A(m,k) B(n,k); see include/dapple_stage.h.  `workspace`: a zero-filled
-    uint8 tensor of gemm_workspace_bytes(m, n) bytes that lets the library cut a long k into slices (split-K)."""
+    uint8 tensor of gemm_workspace_bytes(m, n) bytes that lets the library cut a long k into slices (split-K);
+    `static_scratch`: ds_gemm_static_scratch instead, the variant that allocates nothing (the library's own scratch)."""
     _need_cuda(a, b, c, bias, residual, c2, workspace)
     d = GemmDesc()
     d.dtype = dtype_code(a)
@@ -78,7 +79,10 @@ def gemm(a, b, c, m, n, k, a_major=DS_K_MAJOR, b_major=DS_MN_MAJOR, lda=None, ld
     d.c2 = c2.data_ptr() if c2 is not None else None
     if workspace is not None:
         d.workspace, d.workspace_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
-    check(_lib.load().ds_gemm(C.byref(d), _lib.current_stream()), "ds_gemm")
+    if static_scratch:
+        check(_lib.load().ds_gemm_static_scratch(C.byref(d), _lib.current_stream()), "ds_gemm_static_scratch")
+    else:
+        check(_lib.load().ds_gemm(C.byref(d), _lib.current_stream()), "ds_gemm")
     return c
 
 

@@ -105,6 +105,13 @@ int ds_gemm(const ds_gemm_desc* d, void* stream);
  * at least ds_gemm_workspace_bytes(m, n) bytes, 256-byte aligned, zero-filled once before its first use (the library
  * leaves its counters at zero), and must not be shared by GEMMs that can run at the same time. */
 size_t ds_gemm_workspace_bytes(int m, int n);
+/* ds_gemm cut into k slices with the library's own scratch as the workspace.  No counterpart in the reference: it is
+ * for callers that cannot allocate - code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc - and allocates nothing itself.  Same descriptor and results as ds_gemm with a workspace (d->workspace is
+ * ignored).  Limits: an output of at most 16 tiles of 128 x 128 (4 MiB + 4 KiB of scratch per GPU, held until the
+ * process ends), bf16, batch 1, and a shape that ds_gemm would cut (DS_EINVAL otherwise, with the reason).  All calls
+ * on one GPU share the scratch: calls that overlap in time on one GPU race; calls on one stream do not. */
+int ds_gemm_static_scratch(const ds_gemm_desc* d, void* stream);
 
 /* ---------------------------------------------------------------------------
  * LayerNorm over the last axis, y = (x - mean) * rsqrt(var + eps) * gamma + beta,
