@@ -45,7 +45,8 @@ def make_bert(c, args):
     adt = torch.bfloat16 if c["dtype"] == "bf16" else torch.float32
     K = runtime.stash_depth(0, 2)
     G = max(1, min(args.wgrad_group, M))
-    stage = runtime.bert_stage(L, H, N, F, B, S, c["dtype"], stash_slots=K, embeddings=c["embeddings"], wgrad_group=G)
+    stage = runtime.bert_stage(L, H, N, F, B, S, c["dtype"], stash_slots=K, embeddings=c["embeddings"], wgrad_group=G,
+                               residual_fp32=not args.bf16_residual_stream)
     stage.bind(synthetic.bert_weights(synthetic.SEED_WEIGHT + c["index"], L, H, F, embeddings=c["embeddings"]))
     if c["embeddings"] is None:
         xs = [torch.as_tensor(x).cuda().to(adt) for x in synthetic.bert_activation_inputs(synthetic.SEED_INPUT + c["index"], M, B, S, H)]
@@ -64,7 +65,7 @@ def make_bert(c, args):
     wl.flops_per_sample = 3 * fwd * L
     wl.config = {"layers": L, "hidden": H, "heads": N, "ffn": F, "seq": S, "micro_batch": B, "micro_batches": M,
                  "embedding": c["embeddings"] is not None, "schedule": "1F1B stage 0 of 2, stash K=%d" % K,
-                 "wgrad_group": G}
+                 "wgrad_group": G, "residual_stream": "fp32" if (c["dtype"] != "bf16" or not args.bf16_residual_stream) else "bf16"}
 
     def cpu():
         from oracle import bert as ob
@@ -317,6 +318,8 @@ def main():
     ap.add_argument("--workload", default="bert48_half")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-overlap", action="store_true", help="keep forward and backward passes on one stream")
+    ap.add_argument("--bf16-residual-stream", action="store_true",
+                    help="BERT bf16 workloads: round the residual stream to bf16 too (faster, twice the error at 24 layers)")
     ap.add_argument("--wgrad-group", type=int, default=4,
                     help="BERT stages: weight gradients of this many backward passes in one GEMM per weight")
     ap.add_argument("--xlnet-fused-attention", action="store_true",

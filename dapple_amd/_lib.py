@@ -13,7 +13,7 @@ DS_F32, DS_BF16 = 0, 1
 DS_K_MAJOR, DS_MN_MAJOR = 0, 1
 DS_EPI_BIAS, DS_EPI_RESIDUAL, DS_EPI_GELU, DS_EPI_DGELU = 1, 2, 4, 8
 DS_EPI_OUT_F32, DS_EPI_ACCUM, DS_EPI_RELU, DS_EPI_MASK, DS_EPI_TANH_FORM = 16, 32, 64, 128, 256
-DS_EPI_GELU_GRAD, DS_EPI_MUL = 512, 1024
+DS_EPI_GELU_GRAD, DS_EPI_MUL, DS_EPI_RESIDUAL_F32 = 512, 1024, 2048
 DS_STAGE_BERT, DS_STAGE_VGG19, DS_STAGE_GNMT, DS_STAGE_XLNET = 0, 1, 2, 3
 
 
@@ -44,7 +44,7 @@ class StageCfg(C.Structure):
         ("batch", C.c_int), ("seq", C.c_int), ("with_embedding", C.c_int),
         ("vocab", C.c_int), ("type_vocab", C.c_int), ("max_pos", C.c_int),
         ("ln_eps", C.c_float), ("stash_slots", C.c_int), ("first_layer", C.c_int),
-        ("wgrad_group", C.c_int), ("reserved", C.c_int * 6),
+        ("wgrad_group", C.c_int), ("residual_fp32", C.c_int), ("reserved", C.c_int * 5),
     ]
 
 
@@ -91,6 +91,9 @@ PROTOTYPES = {
     "ds_cast_bf16_to_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "ds_gemm": (C.c_int, [C.POINTER(GemmDesc), C.c_void_p]),
     "ds_gemm_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int]),
+    "ds_layernorm_fwd_mixed": (C.c_int, [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p, C.c_void_p,
+                                          C.c_void_p, C.c_void_p]),
+    "ds_layernorm_bwd_mixed": (C.c_int, [C.c_int, C.c_int] + [C.c_void_p] * 10),
     "ds_gemm_static_scratch": (C.c_int, [C.POINTER(GemmDesc), C.c_void_p]),
     "ds_pooler": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "ds_stage_release_slot": (C.c_int, [C.c_void_p, C.c_int]),

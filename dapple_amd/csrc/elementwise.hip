@@ -240,6 +240,181 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(int rows, int cols, 
   }
 }
 
+// ------------------------------------------------------------------ LayerNorm on an fp32 residual stream
+// A bf16 stage that keeps its residual stream (the sums in front of every LayerNorm and the LayerNorm outputs that
+// feed the next sum) in fp32 rounds to bf16 only where a tensor becomes a GEMM operand.  These kernels read fp32 and
+// write the bf16 operand copy and, optionally, the fp32 carrier; a lane owns groups of 8 consecutive columns.
+__device__ __forceinline__ void ln_load8(const float* p, float (&v)[8]) {
+  const f32x4 a = *reinterpret_cast<const f32x4*>(p), b = *reinterpret_cast<const f32x4*>(p + 4);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) { v[e] = a[e]; v[4 + e] = b[e]; }
+}
+__device__ __forceinline__ void ln_store8(float* p, const float (&v)[8]) {
+  const f32x4 a = {v[0], v[1], v[2], v[3]}, b = {v[4], v[5], v[6], v[7]};
+  *reinterpret_cast<f32x4*>(p) = a;
+  *reinterpret_cast<f32x4*>(p + 4) = b;
+}
+__device__ __forceinline__ void ln_store8(bf16* p, const float (&v)[8]) {
+  bf16x8 o;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = (bf16)v[e];
+  *reinterpret_cast<bf16x8*>(p) = o;
+}
+
+// y = LayerNorm(x): x fp32, y16 bf16, y32 (nullable) fp32.  One wave per row, NG groups of 8 columns per lane.
+template <int NG>
+__global__ __launch_bounds__(256) void layernorm_fwd_mixed_kernel(int rows, int cols, const float* __restrict__ x,
+                                                                 const float* __restrict__ gamma, const float* __restrict__ beta,
+                                                                 float eps, bf16* __restrict__ y16, float* __restrict__ y32,
+                                                                 float* __restrict__ stats) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const float* xr = x + (int64_t)row * cols;
+  float v[NG][8], gm[NG][8], bt[NG][8];
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < NG; ++i) {
+    const int c = (lane + i * 64) * 8;
+    if (c < cols) {
+      ln_load8(xr + c, v[i]);
+      ln_load8(gamma + c, gm[i]);  // with x: read where they are used they would cost a second trip to memory
+      ln_load8(beta + c, bt[i]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sum += v[i][e];
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[i][e] = 0.f;
+    }
+  }
+  const float mean = wave_sum(sum) / cols;
+  float sq = 0.f;
+#pragma unroll
+  for (int i = 0; i < NG; ++i)
+    if ((lane + i * 64) * 8 < cols) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { const float d = v[i][e] - mean; sq += d * d; }
+    }
+  const float rstd = rsqrtf(wave_sum(sq) / cols + eps);
+  if (lane == 0 && stats) { stats[2 * row] = mean; stats[2 * row + 1] = rstd; }
+#pragma unroll
+  for (int i = 0; i < NG; ++i) {
+    const int c = (lane + i * 64) * 8;
+    if (c < cols) {
+      float o[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = (v[i][e] - mean) * rstd * gm[i][e] + bt[i][e];
+      ln_store8(y16 + (int64_t)row * cols + c, o);
+      if (y32) ln_store8(y32 + (int64_t)row * cols + c, o);
+    }
+  }
+}
+
+// Backward of the same: dy, x fp32 in; dx16 bf16 and dx32 (nullable) fp32 out; the parameter gradients and the column
+// sums of dx as in layernorm_bwd_kernel (column partials per wave, combined through LDS, one atomic per column and block).
+template <int NG>
+__global__ __launch_bounds__(256) void layernorm_bwd_mixed_kernel(int rows, int cols, int rows_per_wave, const float* __restrict__ dy,
+                                                                 const float* __restrict__ x, const float* __restrict__ gamma,
+                                                                 const float* __restrict__ stats, bf16* __restrict__ dx16,
+                                                                 float* __restrict__ dx32, float* __restrict__ d_gamma,
+                                                                 float* __restrict__ d_beta, float* __restrict__ d_colsum) {
+  extern __shared__ __attribute__((aligned(16))) float red[];  // [3][cols]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float g[NG][8], pg[NG][8], pb[NG][8], ps[NG][8];
+#pragma unroll
+  for (int i = 0; i < NG; ++i) {
+    const int c = (lane + i * 64) * 8;
+    if (c < cols) ln_load8(gamma + c, g[i]);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      if (c >= cols) g[i][e] = 0.f;
+      pg[i][e] = pb[i][e] = ps[i][e] = 0.f;
+    }
+  }
+  const int row0 = (blockIdx.x * 4 + wave) * rows_per_wave;
+  // the next row's operands are in flight while this row is reduced and written
+  float na[NG][8], nb[NG][8];
+  float nmean = 0.f, nrstd = 0.f;
+  auto fetch = [&](int row) {
+    if (row >= rows) return;
+    nmean = stats[2 * row]; nrstd = stats[2 * row + 1];
+#pragma unroll
+    for (int i = 0; i < NG; ++i) {
+      const int c = (lane + i * 64) * 8;
+      if (c < cols) {
+        ln_load8(dy + (int64_t)row * cols + c, na[i]);
+        ln_load8(x + (int64_t)row * cols + c, nb[i]);
+      }
+    }
+  };
+  fetch(row0);
+  for (int r = 0; r < rows_per_wave; ++r) {
+    const int row = row0 + r;
+    if (row >= rows) break;
+    const float mean = nmean, rstd = nrstd;
+    float dyv[NG][8], xh[NG][8];
+    float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < NG; ++i) {
+      const bool in = (lane + i * 64) * 8 < cols;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        dyv[i][e] = in ? na[i][e] : 0.f;
+        xh[i][e] = in ? (nb[i][e] - mean) * rstd : 0.f;
+        const float dxh = dyv[i][e] * g[i][e];
+        s1 += dxh;
+        s2 += dxh * xh[i][e];
+        pg[i][e] += dyv[i][e] * xh[i][e];
+        pb[i][e] += dyv[i][e];
+      }
+    }
+    if (r + 1 < rows_per_wave) fetch(row + 1);
+    s1 = wave_sum(s1) / cols;
+    s2 = wave_sum(s2) / cols;
+#pragma unroll
+    for (int i = 0; i < NG; ++i) {
+      const int c = (lane + i * 64) * 8;
+      if (c < cols) {
+        float o[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          o[e] = rstd * (dyv[i][e] * g[i][e] - s1 - xh[i][e] * s2);
+          ps[i][e] += o[e];
+        }
+        ln_store8(dx16 + (int64_t)row * cols + c, o);
+        if (dx32) ln_store8(dx32 + (int64_t)row * cols + c, o);
+      }
+    }
+  }
+  for (int wv = 0; wv < 4; ++wv) {
+    if (wave == wv) {
+#pragma unroll
+      for (int i = 0; i < NG; ++i) {
+        const int c = (lane + i * 64) * 8;
+        if (c < cols) {
+#pragma unroll
+          for (int e = 0; e < 8; e += 4) {
+            f32x4* r0 = reinterpret_cast<f32x4*>(&red[c + e]);
+            f32x4* r1 = reinterpret_cast<f32x4*>(&red[cols + c + e]);
+            f32x4* r2 = reinterpret_cast<f32x4*>(&red[2 * cols + c + e]);
+            f32x4 a0 = {pg[i][e], pg[i][e + 1], pg[i][e + 2], pg[i][e + 3]};
+            f32x4 a1 = {pb[i][e], pb[i][e + 1], pb[i][e + 2], pb[i][e + 3]};
+            f32x4 a2 = {ps[i][e], ps[i][e + 1], ps[i][e + 2], ps[i][e + 3]};
+            if (wv > 0) { a0 += *r0; a1 += *r1; a2 += *r2; }
+            *r0 = a0; *r1 = a1; *r2 = a2;
+          }
+        }
+      }
+    }
+    __syncthreads();
+  }
+  for (int c = threadIdx.x; c < cols; c += 256) {
+    atomicAdd(d_gamma + c, red[c]);
+    atomicAdd(d_beta + c, red[cols + c]);
+    if (d_colsum) atomicAdd(d_colsum + c, red[2 * cols + c]);
+  }
+}
+
 // Backward without the parameter gradients: one wave per row, dx only.  For callers that take d_gamma / d_beta (and the
 // column sums of dx) from layernorm_param_grad_kernel on another stream, off the chain of dependent kernels.
 template <typename T, int NV>
@@ -626,6 +801,52 @@ extern "C" int ds_layernorm_bwd(int dtype, int rows, int cols, const void* dy, c
   if (dtype == DS_BF16)
     return layernorm_bwd_t<bf16>(rows, cols, dy, x, gamma, stats, dx_add, dx, d_gamma, d_beta, d_colsum, (hipStream_t)stream);
   return layernorm_bwd_t<float>(rows, cols, dy, x, gamma, stats, dx_add, dx, d_gamma, d_beta, d_colsum, (hipStream_t)stream);
+}
+
+static int check_mixed(const char* who, int rows, int cols) {
+  DS_CHECK_ARG(rows > 0 && cols > 0 && cols % 8 == 0 && cols <= 64 * 8 * 4, "%s: rows %d, cols %d (a multiple of 8, at most 2048)", who, rows, cols);
+  return DS_OK;
+}
+#define DISPATCH_NG(need, CALL)                      \
+  do {                                               \
+    if ((need) <= 1) { constexpr int NG = 1; CALL; } \
+    else if ((need) <= 2) { constexpr int NG = 2; CALL; } \
+    else { constexpr int NG = 4; CALL; }             \
+  } while (0)
+
+extern "C" int ds_layernorm_fwd_mixed(int rows, int cols, const float* x, const float* gamma, const float* beta, float eps,
+                                      void* y_bf16, float* y_f32, float* stats, void* stream) {
+  DS_PROPAGATE(check_mixed("ds_layernorm_fwd_mixed", rows, cols));
+  DS_CHECK_ARG(x && gamma && beta && y_bf16, "ds_layernorm_fwd_mixed: null pointer");
+  DS_CHECK_ARG(ds_aligned16(x) && ds_aligned16(y_bf16) && ds_aligned16(y_f32) && ds_aligned16(gamma) && ds_aligned16(beta),
+               "ds_layernorm_fwd_mixed: tensors must be 16-byte aligned");
+  hipStream_t s = (hipStream_t)stream;
+  const int need = (cols / 8 + 63) / 64;
+  ds_prof_scope prof(s, "layernorm_fwd_mixed_kernel", (double)rows * cols * (4 + 2 + (y_f32 ? 4 : 0)), "B");
+  DISPATCH_NG(need, hipLaunchKernelGGL((layernorm_fwd_mixed_kernel<NG>), dim3((rows + 3) / 4), dim3(256), 0, s, rows, cols, x, gamma, beta,
+                                       eps, (bf16*)y_bf16, y_f32, stats));
+  DS_CHECK_LAUNCH();
+  return DS_OK;
+}
+
+extern "C" int ds_layernorm_bwd_mixed(int rows, int cols, const float* dy, const float* x, const float* gamma, const float* stats,
+                                      void* dx_bf16, float* dx_f32, float* d_gamma, float* d_beta, float* d_colsum, void* stream) {
+  DS_PROPAGATE(check_mixed("ds_layernorm_bwd_mixed", rows, cols));
+  DS_CHECK_ARG(dy && x && gamma && stats && dx_bf16 && d_gamma && d_beta, "ds_layernorm_bwd_mixed: null pointer");
+  DS_CHECK_ARG(ds_aligned16(dy) && ds_aligned16(x) && ds_aligned16(dx_bf16) && ds_aligned16(dx_f32) && ds_aligned16(gamma),
+               "ds_layernorm_bwd_mixed: tensors must be 16-byte aligned");
+  hipStream_t s = (hipStream_t)stream;
+  const int need = (cols / 8 + 63) / 64;
+  int rpw = rows / (128 * 4);
+  if (rpw < 1) rpw = 1;
+  if (rpw > 16) rpw = 16;
+  dim3 grid((rows + 4 * rpw - 1) / (4 * rpw));
+  const size_t lds = 3 * (size_t)cols * sizeof(float);
+  ds_prof_scope prof(s, "layernorm_bwd_mixed_kernel", (double)rows * cols * (4 + 4 + 2 + (dx_f32 ? 4 : 0)), "B");
+  DISPATCH_NG(need, hipLaunchKernelGGL((layernorm_bwd_mixed_kernel<NG>), grid, dim3(256), lds, s, rows, cols, rpw, dy, x, gamma, stats,
+                                       (bf16*)dx_bf16, dx_f32, d_gamma, d_beta, d_colsum));
+  DS_CHECK_LAUNCH();
+  return DS_OK;
 }
 
 template <typename T>

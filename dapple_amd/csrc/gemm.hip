@@ -125,7 +125,8 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, f32x16 (&acc)[B
         if (row >= p.m) continue;
         const int64_t idx = (int64_t)row * p.ldc + col;
         float v = acc[i][j][e] * p.alpha + bias;
-        if (flags & DS_EPI_RESIDUAL) v += to_f32(R[idx]);
+        if (flags & DS_EPI_RESIDUAL)
+          v += (flags & DS_EPI_RESIDUAL_F32) ? (reinterpret_cast<const float*>(p.residual) + c_off)[idx] : to_f32(R[idx]);
         if (flags & DS_EPI_DGELU) v *= gelu_any_grad(to_f32(C2[idx]), tanh_form);
         if (flags & DS_EPI_MUL) v *= to_f32(C2[idx]);
         if (flags & DS_EPI_RELU) v = fmaxf(v, 0.f);
@@ -782,6 +783,7 @@ static int gemm_run(const ds_gemm_desc* d, int splitk_req, void* stream, bool mu
   const int f = d->flags;
   if (f & DS_EPI_BIAS) DS_CHECK_ARG(d->bias != nullptr, "ds_gemm: DS_EPI_BIAS without bias");
   if (f & DS_EPI_RESIDUAL) DS_CHECK_ARG(d->residual != nullptr, "ds_gemm: DS_EPI_RESIDUAL without residual");
+  DS_CHECK_ARG(!(f & DS_EPI_RESIDUAL_F32) || (f & DS_EPI_RESIDUAL), "ds_gemm: DS_EPI_RESIDUAL_F32 needs DS_EPI_RESIDUAL");
   if (f & (DS_EPI_GELU | DS_EPI_DGELU | DS_EPI_MUL)) DS_CHECK_ARG(d->c2 != nullptr, "ds_gemm: GELU / MUL epilogue without c2");
   DS_CHECK_ARG(!(f & DS_EPI_GELU_GRAD) || (f & DS_EPI_GELU), "ds_gemm: DS_EPI_GELU_GRAD needs DS_EPI_GELU");
   DS_CHECK_ARG(!((f & DS_EPI_GELU) && (f & DS_EPI_DGELU)), "ds_gemm: GELU and DGELU are exclusive");

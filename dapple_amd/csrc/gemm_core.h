@@ -266,12 +266,13 @@ __device__ __forceinline__ void gemm_epilogue_vec8(const GemmArgs& p, int64_t c_
   const T* R = reinterpret_cast<const T*>(p.residual) + c_off;
   T* C2 = reinterpret_cast<T*>(p.c2) + c_off;
   if (flags & DS_EPI_RESIDUAL) {
-    if (sizeof(T) == 2) {
+    if (sizeof(T) == 2 && !(flags & DS_EPI_RESIDUAL_F32)) {
       const bf16x8 r = *reinterpret_cast<const bf16x8*>(R + idx);
 #pragma unroll
       for (int e = 0; e < 8; ++e) x[e] += (float)r[e];
     } else {
-      const f32x4 r0 = *reinterpret_cast<const f32x4*>(R + idx), r1 = *reinterpret_cast<const f32x4*>(R + idx + 4);
+      const float* Rf = reinterpret_cast<const float*>(p.residual) + c_off;
+      const f32x4 r0 = *reinterpret_cast<const f32x4*>(Rf + idx), r1 = *reinterpret_cast<const f32x4*>(Rf + idx + 4);
 #pragma unroll
       for (int e = 0; e < 4; ++e) { x[e] += r0[e]; x[4 + e] += r1[e]; }
     }

@@ -93,6 +93,11 @@ struct BertStage : ds_stage {
   size_t esz;
   bool emb;
   bool fused_attn;  // bf16, head size 64: fused attention kernels, no [B,N,S,S] tensors at all
+  // bf16 with cfg.residual_fp32: the residual stream - the sums in front of both LayerNorms, the LayerNorm outputs that
+  // feed the next sum, and the same chain of gradients in backward - stays in fp32; bf16 is only what a GEMM or the
+  // attention kernels read.  The rounding of the stream itself, which otherwise adds up over the layers, is gone.
+  bool rs32 = false;
+  size_t fw_xf[2] = {0, 0}, fw_af = 0, bw_dxf[2] = {0, 0}, bw_dz2f = 0, bw_daf = 0, bw_dz1f = 0;
   // the forward pass writes its stash slot, its output and (unfused attention) its own score buffer; the rest
   // of the workspace belongs to backward
   bool overlap_safe() const override { return true; }
@@ -159,6 +164,7 @@ struct BertStage : ds_stage {
     L = c.num_layers; H = c.hidden; F = c.ffn; NH = c.heads; B = c.batch; S = c.seq;
     D = H / NH; rows = B * S; dtype = c.dtype; esz = dtype == DS_BF16 ? 2 : 4; emb = c.with_embedding != 0;
     fused_attn = dtype == DS_BF16 && D == 64 && S % 64 == 0 && S <= 2048;
+    rs32 = dtype == DS_BF16 && c.residual_fp32 != 0 && L > 0 && H % 8 == 0 && H <= 2048;
     char name[160];
     if (emb) {
       winfo.push_back({"bert/embeddings/word_embeddings", c.vocab, H});
@@ -244,11 +250,11 @@ struct BertStage : ds_stage {
       if (fused_attn) t.lse = ring((size_t)B * NH * S * 4);
       else t.p = ring(probs);
       t.ctx = ring(act);
-      t.z1 = ring(act);
+      t.z1 = ring(rs32 ? (size_t)rows * H * 4 : act);
       t.a = ring(act);
       t.u = ring(actF);
       t.h = ring(actF);
-      t.z2 = ring(act);
+      t.z2 = ring(rs32 ? (size_t)rows * H * 4 : act);
       t.st1 = ring(stats);
       t.st2 = ring(stats);
       if (l + 1 < L) next_x = ring(act);
@@ -296,6 +302,12 @@ struct BertStage : ds_stage {
     ws_dctx = w.reserve(act);
     ws_dx[0] = w.reserve(act);
     ws_dx[1] = w.reserve(act);
+    if (rs32) {
+      const size_t act32 = (size_t)rows * H * 4;
+      fw_xf[0] = w.reserve(act32); fw_xf[1] = w.reserve(act32); fw_af = w.reserve(act32);
+      bw_dxf[0] = w.reserve(act32); bw_dxf[1] = w.reserve(act32);
+      bw_dz2f = w.reserve(act32); bw_daf = w.reserve(act32); bw_dz1f = w.reserve(act32);
+    }
     ws_bytes = w.used;
     DS_CHECK_HIP(hipMalloc((void**)&ws_base, ws_bytes));
     return DS_OK;
@@ -453,6 +465,7 @@ struct BertStage : ds_stage {
     } else {
       DS_CHECK_HIP(hipMemcpyAsync(x0, in, act, hipMemcpyDeviceToDevice, stream));
     }
+    if (rs32) DS_PROPAGATE(ds_cast_bf16_to_f32(ws_base + fw_xf[0], x0, (size_t)rows * H, stream));
     for (int l = 0; l < L; ++l) {
       const LayerStash& t = ls[l];
       const int b = base(l);
@@ -478,19 +491,30 @@ struct BertStage : ds_stage {
                               at(t.qkv, pos) + (size_t)2 * H * esz, 3 * H, (int64_t)S * 3 * H, D, at(t.ctx, pos), H,
                               (int64_t)S * H, D, 0));
       }
+      const int res32 = DS_EPI_RESIDUAL | DS_EPI_RESIDUAL_F32 | DS_EPI_OUT_F32;  // fp32 stream: fp32 residual in, fp32 sum out
+      float* xf = (float*)(ws_base + fw_xf[l & 1]);
+      float* af = (float*)(ws_base + fw_af);
       // attention output dense + residual (:974-978), then layer_norm (:979)
-      DS_PROPAGATE(gemm_fwd(rows, H, H, at(t.ctx, pos), weight_T(l, W_AO), at(t.z1, pos), DS_EPI_BIAS | DS_EPI_RESIDUAL,
-                            w[b + B_AO], x, nullptr));
-      DS_PROPAGATE(ds_layernorm_fwd(dtype, rows, H, at(t.z1, pos), w[b + LN1_G], w[b + LN1_B], cfg.ln_eps, at(t.a, pos),
-                                    (float*)(at(t.st1, pos)), stream));
+      DS_PROPAGATE(gemm_fwd(rows, H, H, at(t.ctx, pos), weight_T(l, W_AO), at(t.z1, pos), DS_EPI_BIAS | (rs32 ? res32 : DS_EPI_RESIDUAL),
+                            w[b + B_AO], rs32 ? (const void*)xf : (const void*)x, nullptr));
+      if (rs32)
+        DS_PROPAGATE(ds_layernorm_fwd_mixed(rows, H, (const float*)at(t.z1, pos), w[b + LN1_G], w[b + LN1_B], cfg.ln_eps, at(t.a, pos), af,
+                                            (float*)(at(t.st1, pos)), stream));
+      else
+        DS_PROPAGATE(ds_layernorm_fwd(dtype, rows, H, at(t.z1, pos), w[b + LN1_G], w[b + LN1_B], cfg.ln_eps, at(t.a, pos),
+                                      (float*)(at(t.st1, pos)), stream));
       // intermediate dense + gelu (:983-987)
       DS_PROPAGATE(gemm_fwd(rows, F, H, at(t.a, pos), weight_T(l, W_FF1), at(t.u, pos), DS_EPI_BIAS | DS_EPI_GELU | DS_EPI_GELU_GRAD, w[b + B_FF1],
                             nullptr, at(t.h, pos)));
       // output dense + residual + layer_norm (:991-996)
-      DS_PROPAGATE(gemm_fwd(rows, H, F, at(t.h, pos), weight_T(l, W_FF2), at(t.z2, pos), DS_EPI_BIAS | DS_EPI_RESIDUAL,
-                            w[b + B_FF2], at(t.a, pos), nullptr));
-      DS_PROPAGATE(ds_layernorm_fwd(dtype, rows, H, at(t.z2, pos), w[b + LN2_G], w[b + LN2_B], cfg.ln_eps, y,
-                                    (float*)(at(t.st2, pos)), stream));
+      DS_PROPAGATE(gemm_fwd(rows, H, F, at(t.h, pos), weight_T(l, W_FF2), at(t.z2, pos), DS_EPI_BIAS | (rs32 ? res32 : DS_EPI_RESIDUAL),
+                            w[b + B_FF2], rs32 ? (const void*)af : (const void*)at(t.a, pos), nullptr));
+      if (rs32)
+        DS_PROPAGATE(ds_layernorm_fwd_mixed(rows, H, (const float*)at(t.z2, pos), w[b + LN2_G], w[b + LN2_B], cfg.ln_eps, y,
+                                            l + 1 < L ? (float*)(ws_base + fw_xf[(l + 1) & 1]) : nullptr, (float*)(at(t.st2, pos)), stream));
+      else
+        DS_PROPAGATE(ds_layernorm_fwd(dtype, rows, H, at(t.z2, pos), w[b + LN2_G], w[b + LN2_B], cfg.ln_eps, y,
+                                      (float*)(at(t.st2, pos)), stream));
     }
     return DS_OK;
   }
@@ -527,6 +551,12 @@ struct BertStage : ds_stage {
       gws = wgrad_stream ? wgrad_stream : stream;
     }
     if (ws || (gws && gws != stream)) DS_PROPAGATE(lane.ensure());
+    // fp32 stream: the gradient that travels down the layers is fp32 (dyf); its bf16 copies feed the GEMMs
+    const float* dyf = nullptr;
+    if (rs32) {
+      DS_PROPAGATE(ds_cast_bf16_to_f32(ws_base + bw_dxf[L & 1], d_out, (size_t)rows * H, stream));
+      dyf = (const float*)(ws_base + bw_dxf[L & 1]);
+    }
     for (int l = L - 1; l >= 0; --l) {
       const LayerStash& t = ls[l];
       const int b = base(l);
@@ -541,16 +571,29 @@ struct BertStage : ds_stage {
       char* dsm = ws_base + ws_ds;
       // the wgrads that read this parity's buffers two layers up must have run
       if (ws) DS_PROPAGATE(lane.reuse(stream, par));
+      const int res32 = DS_EPI_RESIDUAL | DS_EPI_RESIDUAL_F32 | DS_EPI_OUT_F32;
+      float* dz2f = (float*)(ws_base + bw_dz2f);
+      float* daf = (float*)(ws_base + bw_daf);
+      float* dz1f = (float*)(ws_base + bw_dz1f);
       // output LayerNorm; the column sums of dz2 are the gradient of output/dense/bias
-      DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, dy, at(t.z2, pos), w[b + LN2_G], (const float*)(at(t.st2, pos)), nullptr, dz2,
-                                    g[b + LN2_G], g[b + LN2_B], g[b + B_FF2], stream));
+      if (rs32)
+        DS_PROPAGATE(ds_layernorm_bwd_mixed(rows, H, dyf, (const float*)at(t.z2, pos), w[b + LN2_G], (const float*)(at(t.st2, pos)), dz2, dz2f,
+                                            g[b + LN2_G], g[b + LN2_B], g[b + B_FF2], stream));
+      else
+        DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, dy, at(t.z2, pos), w[b + LN2_G], (const float*)(at(t.st2, pos)), nullptr, dz2,
+                                      g[b + LN2_G], g[b + LN2_B], g[b + B_FF2], stream));
       // du = (dz2 W2^T) * gelu'(u)
       DS_PROPAGATE(gemm_dgrad(rows, H, F, dz2, weight_T(l, W_FF2), du, DS_EPI_MUL, nullptr, at(t.u, pos)));
       // da = du W1^T + dz2 (a also feeds the residual into z2)
-      DS_PROPAGATE(gemm_dgrad(rows, F, H, du, weight_T(l, W_FF1), da, DS_EPI_RESIDUAL, dz2, nullptr));
+      if (rs32) DS_PROPAGATE(gemm_dgrad(rows, F, H, du, weight_T(l, W_FF1), daf, res32, dz2f, nullptr));
+      else DS_PROPAGATE(gemm_dgrad(rows, F, H, du, weight_T(l, W_FF1), da, DS_EPI_RESIDUAL, dz2, nullptr));
       // attention-output LayerNorm; column sums of dz1 = gradient of attention/output/dense/bias
-      DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, da, at(t.z1, pos), w[b + LN1_G], (const float*)(at(t.st1, pos)), nullptr, dz1,
-                                    g[b + LN1_G], g[b + LN1_B], g[b + B_AO], stream));
+      if (rs32)
+        DS_PROPAGATE(ds_layernorm_bwd_mixed(rows, H, daf, (const float*)at(t.z1, pos), w[b + LN1_G], (const float*)(at(t.st1, pos)), dz1, dz1f,
+                                            g[b + LN1_G], g[b + LN1_B], g[b + B_AO], stream));
+      else
+        DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, da, at(t.z1, pos), w[b + LN1_G], (const float*)(at(t.st1, pos)), nullptr, dz1,
+                                      g[b + LN1_G], g[b + LN1_B], g[b + B_AO], stream));
       DS_PROPAGATE(gemm_dgrad(rows, H, H, dz1, weight_T(l, W_AO), dctx, 0, nullptr, nullptr));
       // attention backward per (batch, head)
       const char* q = at(t.qkv, pos);
@@ -598,7 +641,15 @@ struct BertStage : ds_stage {
       const bool first = (l == 0);
       if (first && !emb && d_in == nullptr) break;  // a first stage takes no input gradient
       char* dx = first ? (emb ? ws_base + ws_dx[0] : (char*)d_in) : ws_base + ws_dx[l & 1];
-      DS_PROPAGATE(gemm_dgrad(rows, 3 * H, H, dqkv, wqkv[l], dx, DS_EPI_RESIDUAL, dz1, nullptr));
+      if (rs32 && !first) {
+        float* dxf = (float*)(ws_base + bw_dxf[l & 1]);
+        DS_PROPAGATE(gemm_dgrad(rows, 3 * H, H, dqkv, wqkv[l], dxf, res32, dz1f, nullptr));
+        dyf = dxf;
+      } else if (rs32) {  // the stage's input gradient leaves as bf16
+        DS_PROPAGATE(gemm_dgrad(rows, 3 * H, H, dqkv, wqkv[l], dx, DS_EPI_RESIDUAL | DS_EPI_RESIDUAL_F32, dz1f, nullptr));
+      } else {
+        DS_PROPAGATE(gemm_dgrad(rows, 3 * H, H, dqkv, wqkv[l], dx, DS_EPI_RESIDUAL, dz1, nullptr));
+      }
       dy = dx;
     }
     // the stash slot and the master gradients are released to the caller in the order of `stream`

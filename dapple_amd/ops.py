@@ -125,6 +125,33 @@ def layernorm_bwd(dy, x, gamma, stats, d_gamma, d_beta, d_colsum=None, dx_add=No
     return dx
 
 
+def layernorm_fwd_mixed(x, gamma, beta, eps=1e-12, want_f32=True):
+    """LayerNorm on an fp32 residual stream: x fp32 -> (y bf16, y fp32 or None, stats)."""
+    _need_cuda(x, gamma, beta)
+    if x.dtype != torch.float32:
+        raise ValueError("layernorm_fwd_mixed: x must be fp32")
+    rows, cols = x.shape
+    y16 = torch.empty(rows, cols, dtype=torch.bfloat16, device=x.device)
+    y32 = torch.empty_like(x) if want_f32 else None
+    stats = torch.empty(rows, 2, dtype=torch.float32, device=x.device)
+    check(_lib.load().ds_layernorm_fwd_mixed(rows, cols, ptr(x), ptr(gamma), ptr(beta), eps, ptr(y16), ptr(y32), ptr(stats),
+                                             _lib.current_stream()), "ds_layernorm_fwd_mixed")
+    return y16, y32, stats
+
+
+def layernorm_bwd_mixed(dy, x, gamma, stats, d_gamma, d_beta, d_colsum=None, want_f32=True):
+    """Backward of ``layernorm_fwd_mixed``: dy, x fp32 -> (dx bf16, dx fp32 or None); parameter gradients are added to."""
+    _need_cuda(dy, x, gamma, stats, d_gamma, d_beta, d_colsum)
+    if x.dtype != torch.float32 or dy.dtype != torch.float32:
+        raise ValueError("layernorm_bwd_mixed: dy and x must be fp32")
+    rows, cols = x.shape
+    dx16 = torch.empty(rows, cols, dtype=torch.bfloat16, device=x.device)
+    dx32 = torch.empty_like(x) if want_f32 else None
+    check(_lib.load().ds_layernorm_bwd_mixed(rows, cols, ptr(dy), ptr(x), ptr(gamma), ptr(stats), ptr(dx16), ptr(dx32), ptr(d_gamma),
+                                             ptr(d_beta), ptr(d_colsum), _lib.current_stream()), "ds_layernorm_bwd_mixed")
+    return dx16, dx32
+
+
 def layernorm_param_grads(dy, x, stats, d_gamma, d_beta, dx=None, d_colsum=None):
     """d_gamma += sum_rows dy * x_hat, d_beta += sum_rows dy, d_colsum += sum_rows dx: the half of the LayerNorm backward
     pass that ``layernorm_bwd(..., d_gamma=None, d_beta=None)`` leaves out."""

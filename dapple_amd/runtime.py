@@ -214,11 +214,12 @@ def _dtype_code(dtype):
 
 
 def bert_stage(num_layers, hidden, heads, ffn, batch, seq, dtype, stash_slots, embeddings=None, first_layer=0,
-               ln_eps=1e-12, device="cuda:0", wgrad_group=1):
+               ln_eps=1e-12, device="cuda:0", wgrad_group=1, residual_fp32=True):
     """A BERT stage: ``num_layers`` encoder layers, behind the embedding when ``embeddings`` =
     (vocab, type_vocab, max_pos) is given.  ``wgrad_group`` = G > 1: the weight gradients of G consecutive
     backward passes are formed by one GEMM per weight (G more stash positions; the gradients are complete
-    after ``Stage.join`` / ``Stage.sync``)."""
+    after ``Stage.join`` / ``Stage.sync``).  ``residual_fp32`` (bf16 stages): keep the residual stream in fp32 and round
+    to bf16 only the GEMM / attention operands, as the reference's fp32 graph does for the stream."""
     if hidden % heads != 0:
         raise ValueError("The hidden size (%d) is not a multiple of the number of attention heads (%d)" % (hidden, heads))
     lib = _lib.load()
@@ -230,6 +231,7 @@ def bert_stage(num_layers, hidden, heads, ffn, batch, seq, dtype, stash_slots, e
         cfg.vocab, cfg.type_vocab, cfg.max_pos = embeddings
     cfg.ln_eps, cfg.stash_slots, cfg.first_layer = ln_eps, stash_slots, first_layer
     cfg.wgrad_group = int(wgrad_group)
+    cfg.residual_fp32 = 1 if residual_fp32 else 0
     h = C.c_void_p()
     with torch.cuda.device(torch.device(device)):
         check(lib.ds_stage_create(C.byref(cfg), _lib.current_stream(), C.byref(h)), "ds_stage_create")

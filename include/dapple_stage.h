@@ -46,6 +46,8 @@ extern "C" {
 #define DS_EPI_MASK 128    /* C = aux[m][n] > 0 ? acc : 0 (ReLU backward), aux = c2 */
 #define DS_EPI_GELU_GRAD 512 /* with DS_EPI_GELU: C = gelu'(pre-activation) instead of the pre-activation */
 #define DS_EPI_MUL 1024    /* C = acc * aux[m][n], aux = c2 (backward through a GELU whose derivative was kept) */
+#define DS_EPI_RESIDUAL_F32 2048 /* with DS_EPI_RESIDUAL: the residual tensor is fp32 whatever dtype is (a bf16 GEMM adding
+                                  * into an fp32 residual stream; combine with DS_EPI_OUT_F32 to keep the sum in fp32) */
 
 const char* ds_last_error(void);
 
@@ -120,6 +122,13 @@ int ds_gemm_static_scratch(const ds_gemm_desc* d, void* stream);
  * stats receives (mean, rstd) per row for the backward pass. */
 int ds_layernorm_fwd(int dtype, int rows, int cols, const void* x, const float* gamma,
                      const float* beta, float eps, void* y, float* stats, void* stream);
+/* LayerNorm of a bf16 stage that keeps its residual stream in fp32: x (and dy) fp32 in; the result goes out as the bf16
+ * copy the next GEMM reads and, when y_f32 / dx_f32 is given, as the fp32 tensor the next residual sum adds to.
+ * Arithmetic, stats, parameter gradients and d_colsum as ds_layernorm_fwd / ds_layernorm_bwd.  cols % 8 == 0, <= 2048. */
+int ds_layernorm_fwd_mixed(int rows, int cols, const float* x, const float* gamma, const float* beta, float eps,
+                           void* y_bf16, float* y_f32, float* stats, void* stream);
+int ds_layernorm_bwd_mixed(int rows, int cols, const float* dy, const float* x, const float* gamma, const float* stats,
+                           void* dx_bf16, float* dx_f32, float* d_gamma, float* d_beta, float* d_colsum, void* stream);
 /* dx = LN backward; d_gamma/d_beta (fp32, [cols]) are accumulated (+=); d_colsum (nullable,
  * fp32 [cols]) += column sums of dx (the bias gradient of the dense layer that fed x);
  * dx_add (nullable) is added to dx before it is written (gradient of a residual branch). */
@@ -189,7 +198,12 @@ typedef struct ds_stage_cfg {
                     * micro-batches is the one tf.accumulate_n forms (bert/graph.py:159).  With G > 1 the
                     * handle keeps K+G stash positions and a 2G-deep ring of the upstream-gradient operands,
                     * and the master gradients are complete only after ds_stage_join / ds_stage_sync. */
-  int reserved[6];
+  int residual_fp32; /* bf16 stages: 1 keeps the residual stream (the sums in front of both LayerNorms, the LayerNorm
+                      * outputs that feed the next sum, and the same chain of gradients in backward) in fp32 and rounds
+                      * to bf16 only what a GEMM or the attention kernels read: the reference computes all of it in fp32
+                      * (bert/models/bert/modeling_slice.py:942-1001), and the stream's own rounding is what adds up
+                      * over 24 layers.  0: every activation is bf16.  Ignored by fp32 stages. */
+  int reserved[5];
 } ds_stage_cfg;
 
 typedef struct ds_stage ds_stage;

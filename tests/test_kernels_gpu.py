@@ -178,6 +178,25 @@ def test_gemm_epilogues(dt):
     assert_close(out32, 0.5 * (x.cpu().double() @ w.cpu().double()), 1e-5, "out_f32 alpha")
 
 
+@pytest.mark.parametrize("m,n,k", [(192, 160, 96), (1024, 1024, 1024), (1024, 3072, 512)])
+def test_gemm_adds_into_an_fp32_residual_stream(m, n, k):
+    """bf16 operands, fp32 residual in (DS_EPI_RESIDUAL_F32), the sum kept in fp32 (DS_EPI_OUT_F32) or rounded to bf16."""
+    from dapple_amd._lib import DS_EPI_RESIDUAL_F32
+    r = rng(m + n + k)
+    x = dev(r.standard_normal((m, k)), torch.bfloat16)
+    w = dev(r.standard_normal((k, n)) * 0.1, torch.bfloat16)
+    bias = dev(r.standard_normal(n), torch.float32)
+    res = dev(r.standard_normal((m, n)) * 3, torch.float32)
+    ref = x.cpu().double() @ w.cpu().double() + bias.cpu().double() + res.cpu().double()
+    c32 = torch.empty(m, n, dtype=torch.float32, device="cuda")
+    ops.gemm(x, w, c32, m, n, k, DS_K_MAJOR, DS_MN_MAJOR, flags=DS_EPI_BIAS | DS_EPI_RESIDUAL | DS_EPI_RESIDUAL_F32 | DS_EPI_OUT_F32,
+             bias=bias, residual=res)
+    assert_close(c32, ref, 1e-5, "fp32 sum")
+    c16 = torch.empty(m, n, dtype=torch.bfloat16, device="cuda")
+    ops.gemm(x, w, c16, m, n, k, DS_K_MAJOR, DS_MN_MAJOR, flags=DS_EPI_BIAS | DS_EPI_RESIDUAL | DS_EPI_RESIDUAL_F32, bias=bias, residual=res)
+    assert torch.equal(c16, c32.to(torch.bfloat16))
+
+
 @pytest.mark.parametrize("dt", ["fp32", "bf16"])
 def test_gemm_batched_head_views(dt):
     B, N, S, D = 2, 4, 32, 16
@@ -245,6 +264,34 @@ def test_layernorm_fwd_bwd(dt, rows, cols):
     dg3, db3 = torch.zeros(cols, device="cuda"), torch.zeros(cols, device="cuda")
     ops.layernorm_param_grads(dy, x, stats, dg3, db3)
     assert_close(dg3, dg_ref, 1e-4, "ln dgamma (no colsum)")
+
+
+@pytest.mark.parametrize("rows,cols", [(7, 64), (1024, 1024), (33, 520), (5, 2048)])
+def test_layernorm_on_an_fp32_stream(rows, cols):
+    """The kernels of a bf16 stage with an fp32 residual stream: fp32 in, the bf16 operand copy and the fp32 carrier out;
+    both against torch's layer_norm and its autograd in fp64 (the fp32 outputs at 1e-5, their bf16 copies at rounding)."""
+    r = rng(rows + cols)
+    x = dev(r.standard_normal((rows, cols)) * 1.5 + 0.3, torch.float32)
+    gamma = dev(1 + 0.1 * r.standard_normal(cols), torch.float32)
+    beta = dev(0.1 * r.standard_normal(cols), torch.float32)
+    dy = dev(r.standard_normal((rows, cols)), torch.float32)
+    y16, y32, stats = ops.layernorm_fwd_mixed(x, gamma, beta, 1e-12)
+    x64 = x.cpu().double().requires_grad_(True)
+    g64, b64 = gamma.cpu().double().requires_grad_(True), beta.cpu().double().requires_grad_(True)
+    ref = torch.nn.functional.layer_norm(x64, (cols,), g64, b64, 1e-12)
+    assert_close(y32, ref.detach(), 1e-5, "y fp32")
+    assert torch.equal(y16, y32.to(torch.bfloat16))
+    assert ops.layernorm_fwd_mixed(x, gamma, beta, 1e-12, want_f32=False)[1] is None
+    dxr, dgr, dbr = torch.autograd.grad(ref, [x64, g64, b64], dy.cpu().double())
+    dg = torch.full((cols,), 2.0, device="cuda")
+    db = torch.full((cols,), -1.0, device="cuda")
+    dcs = torch.zeros(cols, device="cuda")
+    dx16, dx32 = ops.layernorm_bwd_mixed(dy, x, gamma, stats, dg, db, dcs)
+    assert_close(dx32, dxr, 1e-5, "dx fp32")
+    assert torch.equal(dx16, dx32.to(torch.bfloat16))
+    assert_close(dg - 2.0, dgr, 1e-5, "d_gamma (added to)")
+    assert_close(db + 1.0, dbr, 1e-5, "d_beta (added to)")
+    assert_close(dcs, dxr.sum(0), 1e-4, "column sums of dx", floor=float(dxr.abs().max()) * rows ** 0.5)
 
 
 @pytest.mark.parametrize("dt", ["fp32", "bf16"])

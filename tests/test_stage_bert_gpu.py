@@ -19,7 +19,7 @@ ADT = {"fp32": torch.float32, "bf16": torch.bfloat16}
 
 
 def run_case(dtype, L, H, N, F, B, S, M, embeddings=None, use_mask=False, K=2, stage_index=0, odtype=torch.float64,
-             seed=0, perturb=True, stddev=0.05, wgrad_group=1):
+             seed=0, perturb=True, stddev=0.05, wgrad_group=1, overlap=False):
     w_np = synthetic.bert_weights(synthetic.SEED_WEIGHT + seed, L, H, F, embeddings=embeddings, stddev=stddev,
                                   perturb=perturb)
     if embeddings is not None:
@@ -37,6 +37,8 @@ def run_case(dtype, L, H, N, F, B, S, M, embeddings=None, use_mask=False, K=2, s
     # ---- GPU stage
     stage = runtime.bert_stage(L, H, N, F, B, S, dtype, stash_slots=K, embeddings=embeddings, wgrad_group=wgrad_group)
     stage.bind(w_np)
+    if overlap:
+        stage.enable_overlap()
     adt = ADT[dtype]
     xs = [dev(x) if embeddings is not None else dev(x, adt) for x in xs_np]
     dys = [dev(d, adt) for d in dys_np]
@@ -107,6 +109,13 @@ def test_config0_bert_large_2_layers_fp32():
 def test_config3_shape_two_layers_bf16():
     # BASELINE configs[3] at its real layer shape (seq 512, hidden 1024), depth reduced to 2, M = 2
     run_case("bf16", 2, 1024, 16, 4096, 2, 512, 2, seed=3, perturb=False, stddev=0.02, odtype=torch.float32)
+
+
+def test_config3_shape_two_layers_in_the_benchmark_mode():
+    # the mode bench.py times - weight gradients of 4 passes per GEMM, three streams, 8 micro-batches - at the real layer
+    # shape, depth 2, against the fp32 oracle at the stated 2e-2
+    run_case("bf16", 2, 1024, 16, 4096, 2, 512, 8, seed=3, perturb=False, stddev=0.02, odtype=torch.float32, wgrad_group=4,
+             overlap=True)
 
 
 def test_gradients_do_not_depend_on_stash_depth():
@@ -361,38 +370,49 @@ def _run_config3(dtype, xs_np, dys_np, w, group, overlap, M):
     return res
 
 
-def test_config3_full_size_bf16_against_the_fp32_stage():
-    """BASELINE configs[3] as bench.py runs it (24 layers, 2 x 512 rows, 8 micro-batches, 1F1B K = 2, three streams,
-    weight gradients of 4 passes per GEMM) against the SAME stage in fp32 (the fp32 path is held to 1e-4 of the fp64
-    oracle by the tests above; the oracle itself would take minutes at this size).
+def test_config3_full_size_in_the_benchmark_mode_against_the_oracle():
+    """BASELINE configs[3] exactly as bench.py runs it - 24 layers, 2 x 512 rows, 8 micro-batches, 1F1B K = 2, three streams,
+    weight gradients of 4 passes per GEMM, fp32 residual stream - against the fp32 torch-CPU oracle (bf16 within 2e-2 of the
+    fp32 reference is the stated bar).
 
-    Per layer the bf16 path is within 2e-2 of the oracle (test_config3_shape_two_layers_bf16).  Over 24 layers whose
-    boundary activations are bf16 the rounding of every layer adds up like a random walk: measured 1.3e-2 (L2) / 1.9e-2
-    (max) on the outputs, 2.4e-2 / 3.0e-2 on the input gradients, 1.6e-2 .. 2.4e-2 on the weight gradients.  The bars
-    below are 2e-2 for the outputs and 2e-2 * sqrt(24 / 2) / 2 = 3.5e-2 (L2) for gradients, except the query / key
-    projections: a random-initialised stack of this depth drives the token vectors of a sample towards each other, the
-    softmax is close to uniform, and d scores = P (dP - rowsum(P dP)) then multiplies key vectors that differ from their
-    mean by a fraction of their size - the gradient is a small difference of large terms and bf16 keeps ~1e-1 of it in
-    the last layers (measured 8.7e-2 L2).  The key bias gradient is identically zero (softmax invariance)."""
+    Measured: outputs 7.5e-3 (L2) / 9e-3 (max), input gradients 1.2e-2 / 1.4e-2, every weight gradient <= 1.3e-2 except
+    the query / key projections of the upper layers.  Those are ill-conditioned for ANY bf16 operand: a random-initialised
+    stack of this depth drives the token vectors of a sample towards each other, the rows of d scores sum to zero, and
+    d q = d scores . K (and the weight gradient x^T d k, whose d k sums to zero over the keys) is then a small difference of
+    large terms - the gradient itself is 1-2 orders of magnitude below its sibling, the value projection's.  They are held
+    to 2e-2 on the scale of that sibling (max |error| / max |value gradient|) and to 2e-1 on their own scale (measured
+    8e-2 L2); the key bias gradient is identically zero (softmax invariance) and is judged on the query bias's scale."""
     c = synthetic.CONFIGS["bert48_half"]
-    L, H, F, B, S, M = c["num_layers"], c["hidden"], c["ffn"], c["micro_batch"], c["seq"], c["num_micro_batches"]
+    L, H, N, F, B, S, M = c["num_layers"], c["hidden"], c["heads"], c["ffn"], c["micro_batch"], c["seq"], c["num_micro_batches"]
     w = synthetic.bert_weights(synthetic.SEED_WEIGHT + c["index"], L, H, F)
     xs_np = synthetic.bert_activation_inputs(synthetic.SEED_INPUT + c["index"], M, B, S, H)
     dys_np = synthetic.upstream_grads(synthetic.SEED_GRAD + c["index"], M, (B * S, H))
     got = _run_config3("bf16", xs_np, dys_np, w, 4, True, M)
-    ref = _run_config3("fp32", xs_np, dys_np, w, 1, False, M)
+    w_t = ob.to_torch(w, torch.float32, requires_grad=True)
+    acc = {}
     for j in range(M):
-        assert_close(got[0][j], ref[0][j], 2e-2, "output mb%d" % j)
-        mx, l2 = rel_err(got[1][j], ref[1][j])
-        assert l2 <= 3.5e-2 and mx <= 5e-2, "input grad mb%d: rel max %.3e, l2 %.3e" % (j, mx, l2)
-    for n in ref[2]:
+        x = torch.as_tensor(xs_np[j]).to(torch.bfloat16).float()          # the boundary tensors are bf16 on both sides
+        dy = torch.as_tensor(dys_np[j]).to(torch.bfloat16).float()
+        out, dx, dw = ob.stage_vjp(x, w_t, dy, list(range(L)), B, S, N)
+        assert_close(got[0][j], out, 2e-2, "output mb%d" % j)
+        assert_close(got[1][j], dx, 2e-2, "input grad mb%d" % j)
+        for n, g in dw.items():
+            acc[n] = g.clone() if n not in acc else acc[n] + g
+    worst_own, worst_sib = 0.0, 0.0
+    for n in got[2]:
         if n.endswith("/key/bias"):
-            floor = ref[2][n.replace("/key/", "/query/")].abs().max().item()
-            assert got[2][n].abs().max().item() <= 1.5e-1 * floor, n     # rounding noise, judged like the query bias beside it
+            floor = acc[n.replace("/key/", "/query/")].abs().max().item()
+            assert got[2][n].abs().max().item() <= 2e-1 * floor, n
             continue
-        mx, l2 = rel_err(got[2][n], ref[2][n])
-        bar = 1.5e-1 if "/attention/self/query/" in n or "/attention/self/key/" in n else 3.5e-2
-        assert l2 <= bar, "accumulated grad %s: rel max %.3e, l2 %.3e > %.1e" % (n, mx, l2, bar)
+        mx, l2 = rel_err(got[2][n], acc[n])
+        if "/attention/self/query/" in n or "/attention/self/key/" in n:
+            sibling = acc[n.replace("/query/", "/value/").replace("/key/", "/value/")].abs().max().item()
+            err_sib = (got[2][n].double() - acc[n].double()).abs().max().item() / sibling
+            worst_own, worst_sib = max(worst_own, l2), max(worst_sib, err_sib)
+            assert l2 <= 2e-1 and err_sib <= 2e-2, "%s: rel l2 %.3e (own scale), %.3e of the value gradient's scale" % (n, l2, err_sib)
+        else:
+            assert mx <= 2e-2 and l2 <= 2e-2, "accumulated grad %s: rel max %.3e, l2 %.3e" % (n, mx, l2)
+    print("query/key gradients: worst rel l2 %.3e on their own scale, %.3e of the value gradient's scale" % (worst_own, worst_sib))
 
 
 def test_config3_full_size_exact_properties():
