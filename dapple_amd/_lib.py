@@ -91,6 +91,7 @@ PROTOTYPES = {
     "ds_cast_bf16_to_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "ds_gemm": (C.c_int, [C.POINTER(GemmDesc), C.c_void_p]),
     "ds_gemm_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int]),
+    "ds_vgg_stage_read_activation": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_size_t]),
     "ds_layernorm_fwd_mixed": (C.c_int, [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p, C.c_void_p,
                                           C.c_void_p, C.c_void_p]),
     "ds_layernorm_bwd_mixed": (C.c_int, [C.c_int, C.c_int] + [C.c_void_p] * 10),

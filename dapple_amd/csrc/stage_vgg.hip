@@ -373,6 +373,23 @@ extern "C" int ds_vgg_stage_create(const ds_vgg_cfg* c, void* stream, ds_stage**
 }
 
 // unit entry points -------------------------------------------------------------------------
+extern "C" int ds_vgg_stage_read_activation(ds_stage* h, int slot, int op, float* dst, size_t dst_elems) {
+  DS_CHECK_ARG(h != nullptr && dst != nullptr, "ds_vgg_stage_read_activation: null argument");
+  DS_CHECK_ARG(h->cfg.kind == DS_STAGE_VGG19, "ds_vgg_stage_read_activation: not a VGG stage");
+  VggStage* s = static_cast<VggStage*>(h);
+  DS_CHECK_ARG(slot >= 0 && slot < s->vc.stash_slots, "ds_vgg_stage_read_activation: slot %d out of range", slot);
+  DS_CHECK_ARG(op >= 0 && op < (int)s->ops.size(), "ds_vgg_stage_read_activation: op %d out of range [0,%d)", op, (int)s->ops.size());
+  if (!s->slot_forwarded[slot]) {
+    ds_set_error("ds_vgg_stage_read_activation: slot %d holds no forwarded micro-batch", slot);
+    return DS_ESTATE;
+  }
+  const Op& o = s->ops[op];
+  DS_CHECK_ARG(dst_elems == o.out_elems, "ds_vgg_stage_read_activation: op %d has %zu elements, the buffer %zu", op, o.out_elems, dst_elems);
+  DS_CHECK_HIP(hipMemcpyAsync(dst, s->stash_base + (size_t)slot * s->slot_bytes + o.out_off, o.out_elems * 4, hipMemcpyDeviceToDevice,
+                              s->stream));
+  return DS_OK;
+}
+
 extern "C" int ds_maxpool2x2_fwd(int n, int h, int w, int c, const float* x, float* y, void* stream) {
   DS_CHECK_ARG(n > 0 && h > 0 && w > 0 && c > 0 && h % 2 == 0 && w % 2 == 0 && c % 4 == 0 && x && y,
                "ds_maxpool2x2_fwd: needs even h, w, c %% 4 == 0 and non-null pointers");

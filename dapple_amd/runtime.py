@@ -265,8 +265,8 @@ def vgg_stage(layers, batch, height, width, in_channels, stash_slots, need_input
     h = C.c_void_p()
     with torch.cuda.device(torch.device(device)):
         check(lib.ds_vgg_stage_create(C.byref(cfg), _lib.current_stream(), C.byref(h)), "ds_vgg_stage_create")
-    st = Stage(h, _TORCH_DTYPE[cfg.dtype], batch * height * width * in_channels, batch * h_ * w_ * c_, stash_slots,
-               takes_input_grad=need_input_grad, device=device, cfg=cfg)
+    st = VggStage(h, _TORCH_DTYPE[cfg.dtype], batch * height * width * in_channels, batch * h_ * w_ * c_, stash_slots,
+                  takes_input_grad=need_input_grad, device=device, cfg=cfg)
     st.out_shape = (batch, h_, w_, c_)
     # the stage names convs block%d_conv%d like keras; map the caller's layer names onto them
     st.layer_names = [n for n, c in layers if c is not None]
@@ -319,6 +319,14 @@ def gnmt_attention_stage(units, vocab, batch, seq, src_seq, stash_slots, forget_
     st = GnmtStage(h, _TORCH_DTYPE[cfg.dtype], src_seq * batch * units, seq * batch * units, stash_slots, device=device, cfg=cfg)
     st.out_shape = (seq, batch, units)
     return st
+
+
+class VggStage(Stage):
+    def read_activation(self, slot, op, shape):
+        """The stashed output of op ``op`` (NHWC fp32, ``shape``) of the micro-batch forwarded into ``slot``."""
+        t = torch.empty(shape, dtype=torch.float32, device=self.device)
+        check(self.lib.ds_vgg_stage_read_activation(self._h, slot, op, ptr(t), t.numel()), "ds_vgg_stage_read_activation")
+        return t
 
 
 class GnmtStage(Stage):

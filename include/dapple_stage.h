@@ -298,6 +298,10 @@ typedef struct ds_vgg_cfg {
   int reserved[8];
 } ds_vgg_cfg;
 int ds_vgg_stage_create(const ds_vgg_cfg* cfg, void* stream, ds_stage** out);
+/* Copies the stashed output of op `op` (a conv's post-ReLU activation, a pool's output; NHWC fp32) of the micro-batch
+ * forwarded into `slot` to dst (device memory, dst_elems = its element count), in the order of the stage's stream: the
+ * per-layer outputs a keras model exposes (vgg19/applications/vgg19_slice_model.py:135-213 names every layer). */
+int ds_vgg_stage_read_activation(ds_stage* h, int slot, int op, float* dst, size_t dst_elems);
 
 /* GNMT encoder stage (gnmt/nmt/gnmt_model.py:61-221, DAPPLE branch): embedding lookup, one
  * bidirectional BasicLSTMCell layer, then num_layers-1 uni-directional layers, residual from the

@@ -8,7 +8,8 @@ reached by permutation.  Backward is torch.autograd.
 
 Pins (tests/test_oracle_vgg.py): conv vs a brute-force 7-deep loop; 'same' padding = 1;
 max-pool vs brute force; ReLU gradient 0 at exactly 0; parameter counts vs
-profiling_results/vgg-19-pbs-32.txt of the reference.
+profiling_results/vgg-19-pbs-32.txt of the reference; stage_vjp_forced_branches vs stage_vjp with the
+branches it took itself, and vs brute force on a case with flipped branches.
 """
 import torch
 
@@ -58,3 +59,44 @@ def stage_vjp(x, w, d_out, layers, need_input_grad=False):
     grads = torch.autograd.grad(out, xs, grad_outputs=d_out, allow_unused=True)
     off = 1 if need_input_grad else 0
     return out.detach(), (grads[0] if need_input_grad else None), {n: g for n, g in zip(names, grads[off:]) if g is not None}
+
+
+def branches_of(x, w, layers):
+    """The discrete choices of a forward pass: per conv the ReLU mask (bool, NHWC), per pool the index 0..3 of the
+    window entry that is the maximum (row-major inside the 2x2 window, first maximum on ties)."""
+    masks, picks = {}, {}
+    for name, cout in layers:
+        if cout is None:
+            n, h, wd, c = x.shape
+            win = x.reshape(n, h // 2, 2, wd // 2, 2, c).permute(0, 1, 3, 5, 2, 4).reshape(n, h // 2, wd // 2, c, 4)
+            picks[name] = win.argmax(-1)
+            x = max_pool_2x2(x)
+        else:
+            x = conv3x3_relu(x, w[name + "/kernel"], w[name + "/bias"])
+            masks[name] = x > 0
+    return masks, picks
+
+
+def stage_vjp_forced_branches(x, w, d_out, layers, masks, picks, need_input_grad=False):
+    """stage_vjp along GIVEN branches: ReLU is multiplication by masks[name], max-pool picks window entry picks[name].
+    ReLU and max-pool are the only discontinuities of the stage; a device pass in fp32 takes the other branch than an
+    fp64 pass wherever a pre-activation (or the gap between two window entries) is within rounding of zero, and a
+    flipped branch moves a whole gradient entry.  With the branches of the device pass forced, what is left is smooth
+    (linear in each weight), and fp64 gives the exact derivative of the function the device actually evaluated."""
+    names = sorted(w)
+    if need_input_grad:
+        x = x.clone().requires_grad_(True)
+    h = x
+    for name, cout in layers:
+        if cout is None:
+            n, hh, wd, c = h.shape
+            win = h.reshape(n, hh // 2, 2, wd // 2, 2, c).permute(0, 1, 3, 5, 2, 4).reshape(n, hh // 2, wd // 2, c, 4)
+            h = win.gather(-1, picks[name].unsqueeze(-1)).squeeze(-1)
+        else:
+            z = torch.nn.functional.conv2d(h.permute(0, 3, 1, 2), w[name + "/kernel"].permute(3, 2, 0, 1), w[name + "/bias"],
+                                           stride=1, padding=1).permute(0, 2, 3, 1)
+            h = z * masks[name].to(z.dtype)
+    xs = ([x] if need_input_grad else []) + [w[n] for n in names]
+    grads = torch.autograd.grad(h, xs, grad_outputs=d_out, allow_unused=True)
+    off = 1 if need_input_grad else 0
+    return h.detach(), (grads[0] if need_input_grad else None), {n: g for n, g in zip(names, grads[off:]) if g is not None}

@@ -78,3 +78,42 @@ def test_stage_vjp_finite_differences():
         flat[i] -= 2 * eps
         fm = f(x, wd)
         assert abs((fp - fm) / (2 * eps) - dw[name].reshape(-1)[i].item()) < 1e-5, name
+
+
+def test_forced_branches_reproduce_the_free_pass_and_follow_a_flipped_branch():
+    """stage_vjp_forced_branches: (1) with the branches the oracle's own forward pass took it equals stage_vjp exactly;
+    (2) with one ReLU mask entry and one pool pick flipped it equals finite differences of the function that takes those
+    branches (scalar loops over the layers would say the same: the forced pass is multilinear, so central differences
+    are exact up to rounding)."""
+    r = np.random.Generator(np.random.PCG64(9))
+    layers = [("c1", 4), ("p1", None), ("c2", 3)]
+    x = torch.tensor(r.standard_normal((2, 4, 4, 2)))
+    w = {"c1/kernel": torch.tensor(r.standard_normal((3, 3, 2, 4)) * 0.5), "c1/bias": torch.tensor(r.standard_normal(4) * 0.1),
+         "c2/kernel": torch.tensor(r.standard_normal((3, 3, 4, 3)) * 0.5), "c2/bias": torch.tensor(r.standard_normal(3) * 0.1)}
+    w = {k: v.requires_grad_(True) for k, v in w.items()}
+    dy = torch.tensor(r.standard_normal((2, 2, 2, 3)))
+    masks, picks = ov.branches_of(x, w, layers)
+    out0, dx0, dw0 = ov.stage_vjp(x, w, dy, layers, need_input_grad=True)
+    out1, dx1, dw1 = ov.stage_vjp_forced_branches(x, w, dy, layers, masks, picks, need_input_grad=True)
+    assert torch.equal(out0, out1) and torch.allclose(dx0, dx1, atol=1e-14)
+    for k in dw0:
+        assert torch.allclose(dw0[k], dw1[k], atol=1e-14), k
+    # flip one mask entry and one pick: the forced function changes, and its derivative follows
+    masks["c1"][0, 1, 2, 3] = ~masks["c1"][0, 1, 2, 3]
+    picks["p1"][1, 0, 1, 2] = (picks["p1"][1, 0, 1, 2] + 1) % 4
+    _, _, dwf = ov.stage_vjp_forced_branches(x, w, dy, layers, masks, picks)
+
+    def f(wd):
+        out, _, _ = ov.stage_vjp_forced_branches(x, wd, dy, layers, masks, picks)
+        return float((out * dy).sum())
+
+    for name, idx in (("c1/kernel", (1, 2, 0, 3)), ("c2/kernel", (0, 1, 2, 1)), ("c1/bias", (3,)), ("c2/bias", (0,))):
+        eps = 1e-5
+        wp = {k: v.detach().clone().requires_grad_(True) for k, v in w.items()}
+        wm = {k: v.detach().clone().requires_grad_(True) for k, v in w.items()}
+        with torch.no_grad():
+            wp[name][idx] += eps
+            wm[name][idx] -= eps
+        fd = (f(wp) - f(wm)) / (2 * eps)
+        assert abs(fd - float(dwf[name][idx])) <= 1e-7 * max(1.0, abs(fd)), (name, fd, float(dwf[name][idx]))
+    assert not torch.allclose(dwf["c1/kernel"], dw0["c1/kernel"])       # the flip is visible in the gradient

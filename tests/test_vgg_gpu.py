@@ -128,6 +128,54 @@ def test_stage_vgg19_stack_full_depth_reduced_batch():
               odtype=torch.float64, seed=c["index"], perturb=False, grad_tol=3e-2)
 
 
+def _forced_branch_case(channels, n, h, w, cin, seed, perturb, tol):
+    """One micro-batch through the stage; the oracle walks the branches the GPU took (ReLU masks = stashed activation > 0,
+    pool picks = argmax of the stashed pool input) in fp64: what is left between the two is rounding."""
+    layers = synthetic.vgg_layers(channels)
+    w_np = synthetic.vgg_weights(synthetic.SEED_WEIGHT + seed, layers, cin, perturb=perturb)
+    x_np = synthetic.vgg_inputs(synthetic.SEED_INPUT + seed, 1, n, h, w, cin)[0]
+    stage = runtime.vgg_stage(layers, n, h, w, cin, stash_slots=1)
+    stage.bind(w_np)
+    dy_np = synthetic.upstream_grads(synthetic.SEED_GRAD + seed, 1, stage.out_shape)[0]
+    x, dy = dev(x_np), dev(dy_np)
+    out = torch.empty(stage.out_shape, device="cuda")
+    stage.forward(0, x, out)
+    masks, picks = {}, {}
+    hh, ww, cc = h, w, cin
+    prev = x
+    for i, (name, cout) in enumerate(layers):
+        if cout is None:
+            win = prev.reshape(n, hh // 2, 2, ww // 2, 2, cc).permute(0, 1, 3, 5, 2, 4).reshape(n, hh // 2, ww // 2, cc, 4)
+            picks[name] = win.argmax(-1).cpu()
+            hh, ww = hh // 2, ww // 2
+        else:
+            cc = cout
+        prev = stage.read_activation(0, i, (n, hh, ww, cc))
+        if cout is not None:
+            masks[name] = (prev > 0).cpu()
+    stage.backward(0, dy)
+    stage.sync()
+    w_t = ov.to_torch(w_np, torch.float64, requires_grad=True)
+    o_ref, _, dw = ov.stage_vjp_forced_branches(x.cpu().double(), w_t, dy.cpu().double(), layers, masks, picks)
+    assert_close(out, o_ref, tol, "output")
+    for name in stage.weight_names:
+        assert_close(stage.grads[name], dw[name], tol, "grad " + name)
+    stage.close()
+
+
+def test_forced_branch_oracle_small():
+    _forced_branch_case([32, 32, None, 64, 64, None, 64], n=2, h=16, w=16, cin=3, seed=11, perturb=True, tol=TOL)
+
+
+def test_config1_full_size_along_the_gpus_own_branches():
+    """BASELINE configs[1] at its stated size - conv1_1 .. conv5_4, 4 pools, 32 images of 224 x 224 x 3 - one micro-batch:
+    outputs and all 32 weight / bias gradients at 1e-4 against the fp64 oracle walking the branches the GPU took (the
+    accumulation over 4 micro-batches is the stage-independent sum the smaller cases and the linearity test cover)."""
+    c = synthetic.CONFIGS["vgg19_stage0"]
+    _forced_branch_case([co for _, co in c["layers"]], n=c["micro_batch"], h=c["height"], w=c["width"], cin=c["in_channels"],
+                        seed=c["index"], perturb=False, tol=TOL)
+
+
 @pytest.mark.parametrize("n,h,w,cin,cout", [(8, 224, 224, 64, 64), (8, 28, 28, 256, 512), (32, 14, 14, 512, 512)])
 def test_conv_backward_at_real_layer_shapes(n, h, w, cin, cout):
     # one layer has no downstream discontinuity: the mask is taken from the GPU forward on both sides
