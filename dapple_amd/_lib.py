@@ -94,7 +94,8 @@ PROTOTYPES = {
     "ds_vgg_stage_read_activation": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_size_t]),
     "ds_layernorm_fwd_mixed": (C.c_int, [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p, C.c_void_p,
                                           C.c_void_p, C.c_void_p]),
-    "ds_layernorm_bwd_mixed": (C.c_int, [C.c_int, C.c_int] + [C.c_void_p] * 10),
+    "ds_layernorm_bwd_mixed": (C.c_int, [C.c_int, C.c_int] + [C.c_void_p] * 11),
+    "ds_layernorm_param_grads_mixed": (C.c_int, [C.c_int, C.c_int] + [C.c_void_p] * 8),
     "ds_gemm_static_scratch": (C.c_int, [C.POINTER(GemmDesc), C.c_void_p]),
     "ds_pooler": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "ds_stage_release_slot": (C.c_int, [C.c_void_p, C.c_int]),

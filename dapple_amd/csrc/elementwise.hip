@@ -415,6 +415,129 @@ __global__ __launch_bounds__(256) void layernorm_bwd_mixed_kernel(int rows, int 
   }
 }
 
+// The same backward pass without the parameter gradients: one wave per row, no LDS, no atomics - the form for a chain
+// of dependent kernels.  dy16 (nullable) receives a bf16 copy of dy: with x and stats (kept by the caller) and dx16 it is
+// all layernorm_param_grad_mixed_kernel needs to produce d_gamma, d_beta and the column sums of dx later, elsewhere.
+template <int NG>
+__global__ __launch_bounds__(256) void layernorm_bwd_mixed_rows_kernel(int rows, int cols, const float* __restrict__ dy,
+                                                                      const float* __restrict__ x, const float* __restrict__ gamma,
+                                                                      const float* __restrict__ stats, bf16* __restrict__ dx16,
+                                                                      float* __restrict__ dx32, bf16* __restrict__ dy16) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int64_t ro = (int64_t)row * cols;
+  float a[NG][8], b[NG][8], g[NG][8];
+#pragma unroll
+  for (int i = 0; i < NG; ++i) {
+    const int c = (lane + i * 64) * 8;
+    if (c < cols) {
+      ln_load8(dy + ro + c, a[i]);
+      ln_load8(x + ro + c, b[i]);
+      ln_load8(gamma + c, g[i]);
+    }
+  }
+  const float mean = stats[2 * row], rstd = stats[2 * row + 1];
+  float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+  for (int i = 0; i < NG; ++i) {
+    const int c = (lane + i * 64) * 8;
+    if (c < cols) {
+      if (dy16) ln_store8(dy16 + ro + c, a[i]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        b[i][e] = (b[i][e] - mean) * rstd;
+        a[i][e] *= g[i][e];
+        s1 += a[i][e];
+        s2 += a[i][e] * b[i][e];
+      }
+    }
+  }
+  s1 = wave_sum(s1) / cols;
+  s2 = wave_sum(s2) / cols;
+#pragma unroll
+  for (int i = 0; i < NG; ++i) {
+    const int c = (lane + i * 64) * 8;
+    if (c < cols) {
+      float o[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = rstd * (a[i][e] - s1 - b[i][e] * s2);
+      ln_store8(dx16 + ro + c, o);
+      if (dx32) ln_store8(dx32 + ro + c, o);
+    }
+  }
+}
+
+// d_gamma[c] += sum_rows dy x_hat, d_beta[c] += sum_rows dy, d_colsum[c] += sum_rows dx (dx, d_colsum nullable) from the
+// bf16 copies layernorm_bwd_mixed_rows_kernel left and the fp32 x.  A block owns a strip of 64 x 8 columns and a chunk
+// of rows; its 4 waves take every 4th row and meet in LDS; one atomic per column and block.
+__global__ __launch_bounds__(256) void layernorm_param_grad_mixed_kernel(int rows, int cols, int rows_per_block,
+                                                                        const bf16* __restrict__ dy, const float* __restrict__ x,
+                                                                        const float* __restrict__ stats, const bf16* __restrict__ dx,
+                                                                        float* __restrict__ d_gamma, float* __restrict__ d_beta,
+                                                                        float* __restrict__ d_colsum) {
+  __shared__ float red[3][4][64 * 8];
+  const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
+  const int c = (blockIdx.x * 64 + lane) * 8;
+  const int r0 = blockIdx.y * rows_per_block;
+  int r1 = r0 + rows_per_block;
+  if (r1 > rows) r1 = rows;
+  float pg[8], pb[8], ps[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) pg[e] = pb[e] = ps[e] = 0.f;
+  if (c < cols) {
+    // two rows in flight per wave
+    for (int r = r0 + g; r < r1; r += 8) {
+      const int rb = r + 4;
+      const bool two = rb < r1;
+      const bf16x8 a0 = *reinterpret_cast<const bf16x8*>(dy + (int64_t)r * cols + c);
+      float b0[8], b1[8];
+      ln_load8(x + (int64_t)r * cols + c, b0);
+      const float mean0 = stats[2 * r], rstd0 = stats[2 * r + 1];
+      bf16x8 a1 = {}, v0 = {}, v1 = {};
+      float mean1 = 0.f, rstd1 = 0.f;
+      if (dx) v0 = *reinterpret_cast<const bf16x8*>(dx + (int64_t)r * cols + c);
+      if (two) {
+        a1 = *reinterpret_cast<const bf16x8*>(dy + (int64_t)rb * cols + c);
+        ln_load8(x + (int64_t)rb * cols + c, b1);
+        mean1 = stats[2 * rb]; rstd1 = stats[2 * rb + 1];
+        if (dx) v1 = *reinterpret_cast<const bf16x8*>(dx + (int64_t)rb * cols + c);
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float d = to_f32(a0[e]);
+        pg[e] += d * (b0[e] - mean0) * rstd0;
+        pb[e] += d;
+        ps[e] += to_f32(v0[e]);
+      }
+      if (two) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float d = to_f32(a1[e]);
+          pg[e] += d * (b1[e] - mean1) * rstd1;
+          pb[e] += d;
+          ps[e] += to_f32(v1[e]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    red[0][g][lane * 8 + e] = pg[e];
+    red[1][g][lane * 8 + e] = pb[e];
+    red[2][g][lane * 8 + e] = ps[e];
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < 64 * 8; i += 256) {
+    const int p = blockIdx.x * 64 * 8 + i;
+    if (p < cols) {
+      atomicAdd(d_gamma + p, red[0][0][i] + red[0][1][i] + red[0][2][i] + red[0][3][i]);
+      atomicAdd(d_beta + p, red[1][0][i] + red[1][1][i] + red[1][2][i] + red[1][3][i]);
+      if (d_colsum) atomicAdd(d_colsum + p, red[2][0][i] + red[2][1][i] + red[2][2][i] + red[2][3][i]);
+    }
+  }
+}
+
 // Backward without the parameter gradients: one wave per row, dx only.  For callers that take d_gamma / d_beta (and the
 // column sums of dx) from layernorm_param_grad_kernel on another stream, off the chain of dependent kernels.
 template <typename T, int NV>
@@ -830,13 +953,24 @@ extern "C" int ds_layernorm_fwd_mixed(int rows, int cols, const float* x, const 
 }
 
 extern "C" int ds_layernorm_bwd_mixed(int rows, int cols, const float* dy, const float* x, const float* gamma, const float* stats,
-                                      void* dx_bf16, float* dx_f32, float* d_gamma, float* d_beta, float* d_colsum, void* stream) {
+                                      void* dx_bf16, float* dx_f32, void* dy_bf16, float* d_gamma, float* d_beta, float* d_colsum,
+                                      void* stream) {
   DS_PROPAGATE(check_mixed("ds_layernorm_bwd_mixed", rows, cols));
-  DS_CHECK_ARG(dy && x && gamma && stats && dx_bf16 && d_gamma && d_beta, "ds_layernorm_bwd_mixed: null pointer");
-  DS_CHECK_ARG(ds_aligned16(dy) && ds_aligned16(x) && ds_aligned16(dx_bf16) && ds_aligned16(dx_f32) && ds_aligned16(gamma),
-               "ds_layernorm_bwd_mixed: tensors must be 16-byte aligned");
+  DS_CHECK_ARG(dy && x && gamma && stats && dx_bf16, "ds_layernorm_bwd_mixed: null pointer");
+  DS_CHECK_ARG(ds_aligned16(dy) && ds_aligned16(x) && ds_aligned16(dx_bf16) && ds_aligned16(dx_f32) && ds_aligned16(gamma) &&
+               ds_aligned16(dy_bf16), "ds_layernorm_bwd_mixed: tensors must be 16-byte aligned");
   hipStream_t s = (hipStream_t)stream;
   const int need = (cols / 8 + 63) / 64;
+  if (!d_gamma && !d_beta) {  // dx only: the parameter gradients come from ds_layernorm_param_grads_mixed
+    DS_CHECK_ARG(!d_colsum, "ds_layernorm_bwd_mixed: d_colsum without d_gamma / d_beta");
+    ds_prof_scope prof(s, "layernorm_bwd_mixed_rows_kernel",
+                       (double)rows * cols * (4 + 4 + 2 + (dx_f32 ? 4 : 0) + (dy_bf16 ? 2 : 0)), "B");
+    DISPATCH_NG(need, hipLaunchKernelGGL((layernorm_bwd_mixed_rows_kernel<NG>), dim3((rows + 3) / 4), dim3(256), 0, s, rows, cols, dy, x,
+                                         gamma, stats, (bf16*)dx_bf16, dx_f32, (bf16*)dy_bf16));
+    DS_CHECK_LAUNCH();
+    return DS_OK;
+  }
+  DS_CHECK_ARG(d_gamma && d_beta && !dy_bf16, "ds_layernorm_bwd_mixed: d_gamma and d_beta come together, and without dy_bf16");
   int rpw = rows / (128 * 4);
   if (rpw < 1) rpw = 1;
   if (rpw > 16) rpw = 16;
@@ -845,6 +979,27 @@ extern "C" int ds_layernorm_bwd_mixed(int rows, int cols, const float* dy, const
   ds_prof_scope prof(s, "layernorm_bwd_mixed_kernel", (double)rows * cols * (4 + 4 + 2 + (dx_f32 ? 4 : 0)), "B");
   DISPATCH_NG(need, hipLaunchKernelGGL((layernorm_bwd_mixed_kernel<NG>), grid, dim3(256), lds, s, rows, cols, rpw, dy, x, gamma, stats,
                                        (bf16*)dx_bf16, dx_f32, d_gamma, d_beta, d_colsum));
+  DS_CHECK_LAUNCH();
+  return DS_OK;
+}
+
+extern "C" int ds_layernorm_param_grads_mixed(int rows, int cols, const void* dy_bf16, const float* x, const float* stats,
+                                              const void* dx_bf16, float* d_gamma, float* d_beta, float* d_colsum, void* stream) {
+  DS_CHECK_ARG(rows > 0 && cols > 0 && cols % 8 == 0, "ds_layernorm_param_grads_mixed: rows %d, cols %d (a multiple of 8)", rows, cols);
+  DS_CHECK_ARG(dy_bf16 && x && stats && d_gamma && d_beta && (!d_colsum || dx_bf16),
+               "ds_layernorm_param_grads_mixed: null pointer (d_colsum needs dx_bf16)");
+  DS_CHECK_ARG(ds_aligned16(dy_bf16) && ds_aligned16(x) && ds_aligned16(dx_bf16),
+               "ds_layernorm_param_grads_mixed: tensors must be 16-byte aligned");
+  hipStream_t s = (hipStream_t)stream;
+  const int strips = (cols + 64 * 8 - 1) / (64 * 8);
+  int chunks = 256 / strips;  // about one block per CU
+  if (chunks > (rows + 31) / 32) chunks = (rows + 31) / 32;
+  if (chunks < 1) chunks = 1;
+  const int rpb = (rows + chunks - 1) / chunks;
+  dim3 grid(strips, (rows + rpb - 1) / rpb);
+  ds_prof_scope prof(s, "layernorm_param_grad_mixed_kernel", (double)rows * cols * (2 + 4 + (d_colsum ? 2 : 0)), "B");
+  hipLaunchKernelGGL(layernorm_param_grad_mixed_kernel, grid, dim3(256), 0, s, rows, cols, rpb, (const bf16*)dy_bf16, x, stats,
+                     d_colsum ? (const bf16*)dx_bf16 : nullptr, d_gamma, d_beta, d_colsum);
   DS_CHECK_LAUNCH();
   return DS_OK;
 }

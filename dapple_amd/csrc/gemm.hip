@@ -441,6 +441,17 @@ template <typename T, int W, int MAJOR, int CONV> struct DmaSelect { typedef Asm
 template <typename T, int W> struct DmaSelect<T, W, DS_K_MAJOR, 1> { typedef ConvDma<T, W, 1> type; };
 template <typename T, int W> struct DmaSelect<T, W, DS_MN_MAJOR, 2> { typedef ConvDma<T, W, 2> type; };
 
+// Waits until at most min(later, MAXL) k-tiles' loads (LPT per thread each) are still outstanding.
+template <int LPT, int MAXL> __device__ __forceinline__ void wait_tiles_in_flight(int later) {
+  static_assert(LPT * MAXL <= 63, "the vmcnt field holds 6 bits");
+  if constexpr (MAXL <= 0) {
+    __builtin_amdgcn_s_waitcnt(DS_VMCNT(0));
+  } else {
+    if (later >= MAXL) __builtin_amdgcn_s_waitcnt(DS_VMCNT(LPT * MAXL));
+    else wait_tiles_in_flight<LPT, MAXL - 1>(later);
+  }
+}
+
 template <typename T, int BM, int BN, int AMAJ, int BMAJ, int STAGES, int CONVA = 0>
 __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
   typedef typename DmaSelect<T, BM, AMAJ, CONVA>::type DA;
@@ -517,10 +528,7 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
   {
     // tile 0 is complete once only the tiles issued after it are outstanding
     const int later = (nkt < STAGES ? nkt : STAGES) - 1;
-    if (later >= 3) __builtin_amdgcn_s_waitcnt(DS_VMCNT(LPT * 3));
-    else if (later == 2) __builtin_amdgcn_s_waitcnt(DS_VMCNT(LPT * 2));
-    else if (later == 1) __builtin_amdgcn_s_waitcnt(DS_VMCNT(LPT));
-    else __builtin_amdgcn_s_waitcnt(DS_VMCNT(0));
+    wait_tiles_in_flight<LPT, STAGES - 1>(later);
     __builtin_amdgcn_s_barrier();
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
@@ -577,12 +585,8 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
             // below must not sit inside a conditional, see the end of k_tile)
             // tile kt+1 is complete once only the tiles issued after it are outstanding:
             // kt+2 .. kt-1+STAGES, as far as they exist
-            int later = ST ? STAGES - 2 : nkt - (kt + 2);
-            if (later > STAGES - 2) later = STAGES - 2;
-            if (later < 0) later = 0;
-            if (later >= 2) __builtin_amdgcn_s_waitcnt(DS_VMCNT(LPT * 2));
-            else if (later == 1) __builtin_amdgcn_s_waitcnt(DS_VMCNT(LPT));
-            else __builtin_amdgcn_s_waitcnt(DS_VMCNT(0));
+            if (ST) __builtin_amdgcn_s_waitcnt(DS_VMCNT(LPT * (STAGES - 2)));
+            else wait_tiles_in_flight<LPT, STAGES - 2>(nkt - (kt + 2));
             __builtin_amdgcn_s_barrier();
           }
           // this slot's share of the fragment reads: k-steps 2 and 3 of this tile during k-steps 0 and 1, nothing
@@ -651,6 +655,19 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
   else gemm_epilogue<T, BM, BN>(p, acc, m0, n0, wm, wn, lane, c_off);
 }
 
+template <typename T, int BM, int BN, int AMAJ, int BMAJ, int STAGES>
+int launch_dma(const GemmArgs& a, dim3 grid, hipStream_t stream) {
+  constexpr size_t lds = (size_t)STAGES * (BM + BN) * 128;
+  static bool attr_set = false;
+  if (!attr_set) {
+    DS_CHECK_HIP(hipFuncSetAttribute((const void*)gemm_dma_kernel<T, BM, BN, AMAJ, BMAJ, STAGES>,
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_set = true;
+  }
+  hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, AMAJ, BMAJ, STAGES>), grid, dim3(256), lds, stream, a);
+  return DS_OK;
+}
+
 template <typename T, int BM, int BN, int AMAJ, int BMAJ>
 int launch_cfg(GemmArgs a, int batch, hipStream_t stream) {
   a.grid_m = (a.m + BM - 1) / BM;
@@ -658,17 +675,12 @@ int launch_cfg(GemmArgs a, int batch, hipStream_t stream) {
   choose_xcd_block(a);
   dim3 grid(a.grid_m * a.grid_n, 1, batch * a.splitk);
   if (a.k % Mma<T>::KT == 0) {
-    // 3 buffers: 96 KB for a 128x128 block, 48 KB for 64x64 - a CU's 160 KB of LDS then holds blocks of two
-    // kernels at once, which measured better than a deeper ring when several streams feed the GPU
-    constexpr int STAGES = 3;
-    constexpr size_t lds = (size_t)STAGES * (BM + BN) * 128;
-    static bool attr_set = false;
-    if (!attr_set) {
-      DS_CHECK_HIP(hipFuncSetAttribute((const void*)gemm_dma_kernel<T, BM, BN, AMAJ, BMAJ, STAGES>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-      attr_set = true;
-    }
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, AMAJ, BMAJ, STAGES>), grid, dim3(256), lds, stream, a);
+    // 3 buffers: 96 KB for a 128x128 block, 48 KB for 64x64 - a CU's 160 KB of LDS then holds blocks of two or
+    // three kernels at once.  With several streams feeding the GPU that co-residency is worth more than a deeper
+    // ring: 6 buffers under the 64x64 block (long reductions, one block per CU) made the BERT-48 half-stage step
+    // 3.6 % shorter with all its kernels on one stream and 7 % longer on three.
+    int rc = launch_dma<T, BM, BN, AMAJ, BMAJ, 3>(a, grid, stream);
+    if (rc != DS_OK) return rc;
   } else {
     const size_t lds = 2 * (BM + BN) * 128;
     hipLaunchKernelGGL((gemm_kernel<T, BM, BN, AMAJ, BMAJ>), grid, dim3(256), lds, stream, a);

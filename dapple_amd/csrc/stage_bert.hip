@@ -79,6 +79,7 @@ struct LayerStash {
 // of positions back to back, byte offsets into dy_base.
 struct LayerDy {
   size_t dz2, du, dz1, dqkv;
+  size_t dyn2, dyn1;  // fp32 residual stream: bf16 copies of the gradients that entered the two LayerNorms
 };
 struct Deferred {
   int xpos, dypos;
@@ -277,6 +278,10 @@ struct BertStage : ds_stage {
         ld[l].du = da.reserve(actF * NDY);
         ld[l].dz1 = da.reserve(act * NDY);
         ld[l].dqkv = da.reserve(3 * act * NDY);
+        if (rs32) {
+          ld[l].dyn2 = da.reserve(act * NDY);
+          ld[l].dyn1 = da.reserve(act * NDY);
+        }
       }
       if (da.used) DS_CHECK_HIP(hipMalloc((void**)&dy_base, da.used));
       DS_CHECK_HIP(hipEventCreateWithFlags(&ev_chain, hipEventDisableTiming));
@@ -576,9 +581,15 @@ struct BertStage : ds_stage {
       float* daf = (float*)(ws_base + bw_daf);
       float* dz1f = (float*)(ws_base + bw_dz1f);
       // output LayerNorm; the column sums of dz2 are the gradient of output/dense/bias
-      if (rs32)
+      // (fp32 stream with grouped weight gradients: the chain only computes dz; gamma, beta and bias gradients follow
+      // with the group's weight gradients, from bf16 copies of dy kept beside dz in the operand ring)
+      const bool ln_deferred = rs32 && G > 1;
+      if (ln_deferred)
         DS_PROPAGATE(ds_layernorm_bwd_mixed(rows, H, dyf, (const float*)at(t.z2, pos), w[b + LN2_G], (const float*)(at(t.st2, pos)), dz2, dz2f,
-                                            g[b + LN2_G], g[b + LN2_B], g[b + B_FF2], stream));
+                                            dy_base + ld[l].dyn2 + dypos * dy_act, nullptr, nullptr, nullptr, stream));
+      else if (rs32)
+        DS_PROPAGATE(ds_layernorm_bwd_mixed(rows, H, dyf, (const float*)at(t.z2, pos), w[b + LN2_G], (const float*)(at(t.st2, pos)), dz2, dz2f,
+                                            nullptr, g[b + LN2_G], g[b + LN2_B], g[b + B_FF2], stream));
       else
         DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, dy, at(t.z2, pos), w[b + LN2_G], (const float*)(at(t.st2, pos)), nullptr, dz2,
                                       g[b + LN2_G], g[b + LN2_B], g[b + B_FF2], stream));
@@ -588,9 +599,12 @@ struct BertStage : ds_stage {
       if (rs32) DS_PROPAGATE(gemm_dgrad(rows, F, H, du, weight_T(l, W_FF1), daf, res32, dz2f, nullptr));
       else DS_PROPAGATE(gemm_dgrad(rows, F, H, du, weight_T(l, W_FF1), da, DS_EPI_RESIDUAL, dz2, nullptr));
       // attention-output LayerNorm; column sums of dz1 = gradient of attention/output/dense/bias
-      if (rs32)
+      if (ln_deferred)
         DS_PROPAGATE(ds_layernorm_bwd_mixed(rows, H, daf, (const float*)at(t.z1, pos), w[b + LN1_G], (const float*)(at(t.st1, pos)), dz1, dz1f,
-                                            g[b + LN1_G], g[b + LN1_B], g[b + B_AO], stream));
+                                            dy_base + ld[l].dyn1 + dypos * dy_act, nullptr, nullptr, nullptr, stream));
+      else if (rs32)
+        DS_PROPAGATE(ds_layernorm_bwd_mixed(rows, H, daf, (const float*)at(t.z1, pos), w[b + LN1_G], (const float*)(at(t.st1, pos)), dz1, dz1f,
+                                            nullptr, g[b + LN1_G], g[b + LN1_B], g[b + B_AO], stream));
       else
         DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, da, at(t.z1, pos), w[b + LN1_G], (const float*)(at(t.st1, pos)), nullptr, dz1,
                                       g[b + LN1_G], g[b + LN1_B], g[b + B_AO], stream));
@@ -701,10 +715,22 @@ struct BertStage : ds_stage {
   }
   int layer_wgrad_runs(int l, const std::vector<Run>& runs) {
     const LayerStash& t = ls[l];
-    for (const Run& r : runs)
-      DS_PROPAGATE(layer_wgrad(l, r.n * rows, at(t.x, r.xpos), at(t.ctx, r.xpos), at(t.a, r.xpos), at(t.h, r.xpos),
-                               dy_base + ld[l].dz2 + r.dypos * dy_act, dy_base + ld[l].du + r.dypos * dy_actF,
-                               dy_base + ld[l].dz1 + r.dypos * dy_act, dy_base + ld[l].dqkv + r.dypos * 3 * dy_act));
+    const int b = base(l);
+    for (const Run& r : runs) {
+      const int m = r.n * rows;
+      const char* dz2 = dy_base + ld[l].dz2 + r.dypos * dy_act;
+      const char* dz1 = dy_base + ld[l].dz1 + r.dypos * dy_act;
+      DS_PROPAGATE(layer_wgrad(l, m, at(t.x, r.xpos), at(t.ctx, r.xpos), at(t.a, r.xpos), at(t.h, r.xpos), dz2,
+                               dy_base + ld[l].du + r.dypos * dy_actF, dz1, dy_base + ld[l].dqkv + r.dypos * 3 * dy_act));
+      if (rs32) {  // the LayerNorm parameter gradients and the two bias gradients the chain left out
+        DS_PROPAGATE(ds_layernorm_param_grads_mixed(m, H, dy_base + ld[l].dyn2 + r.dypos * dy_act, (const float*)at(t.z2, r.xpos),
+                                                    (const float*)at(t.st2, r.xpos), dz2, g[b + LN2_G], g[b + LN2_B], g[b + B_FF2],
+                                                    stream));
+        DS_PROPAGATE(ds_layernorm_param_grads_mixed(m, H, dy_base + ld[l].dyn1 + r.dypos * dy_act, (const float*)at(t.z1, r.xpos),
+                                                    (const float*)at(t.st1, r.xpos), dz1, g[b + LN1_G], g[b + LN1_B], g[b + B_AO],
+                                                    stream));
+      }
+    }
     return DS_OK;
   }
   // the weight-gradient work of every deferred pass has been queued on `ws`

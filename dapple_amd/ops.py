@@ -139,17 +139,30 @@ def layernorm_fwd_mixed(x, gamma, beta, eps=1e-12, want_f32=True):
     return y16, y32, stats
 
 
-def layernorm_bwd_mixed(dy, x, gamma, stats, d_gamma, d_beta, d_colsum=None, want_f32=True):
-    """Backward of ``layernorm_fwd_mixed``: dy, x fp32 -> (dx bf16, dx fp32 or None); parameter gradients are added to."""
+def layernorm_bwd_mixed(dy, x, gamma, stats, d_gamma=None, d_beta=None, d_colsum=None, want_f32=True, want_dy_bf16=False):
+    """Backward of ``layernorm_fwd_mixed``: dy, x fp32 -> (dx bf16, dx fp32 or None); parameter gradients are added to.
+    Without ``d_gamma`` / ``d_beta`` only dx is computed (no atomics); ``want_dy_bf16`` then also returns the bf16 copy of
+    dy that ``layernorm_param_grads_mixed`` takes: (dx bf16, dx fp32 or None, dy bf16)."""
     _need_cuda(dy, x, gamma, stats, d_gamma, d_beta, d_colsum)
     if x.dtype != torch.float32 or dy.dtype != torch.float32:
         raise ValueError("layernorm_bwd_mixed: dy and x must be fp32")
     rows, cols = x.shape
     dx16 = torch.empty(rows, cols, dtype=torch.bfloat16, device=x.device)
     dx32 = torch.empty_like(x) if want_f32 else None
-    check(_lib.load().ds_layernorm_bwd_mixed(rows, cols, ptr(dy), ptr(x), ptr(gamma), ptr(stats), ptr(dx16), ptr(dx32), ptr(d_gamma),
-                                             ptr(d_beta), ptr(d_colsum), _lib.current_stream()), "ds_layernorm_bwd_mixed")
-    return dx16, dx32
+    dy16 = torch.empty_like(dx16) if want_dy_bf16 else None
+    check(_lib.load().ds_layernorm_bwd_mixed(rows, cols, ptr(dy), ptr(x), ptr(gamma), ptr(stats), ptr(dx16), ptr(dx32), ptr(dy16),
+                                             ptr(d_gamma), ptr(d_beta), ptr(d_colsum), _lib.current_stream()), "ds_layernorm_bwd_mixed")
+    return (dx16, dx32, dy16) if want_dy_bf16 else (dx16, dx32)
+
+
+def layernorm_param_grads_mixed(dy_bf16, x, stats, d_gamma, d_beta, dx_bf16=None, d_colsum=None):
+    """d_gamma += sum_rows dy * x_hat, d_beta += sum_rows dy, d_colsum += sum_rows dx from the bf16 copies that
+    ``layernorm_bwd_mixed(..., want_dy_bf16=True)`` left and the fp32 x: the deferred half of that backward pass."""
+    _need_cuda(dy_bf16, x, stats, d_gamma, d_beta, dx_bf16, d_colsum)
+    rows, cols = x.shape
+    check(_lib.load().ds_layernorm_param_grads_mixed(rows, cols, ptr(dy_bf16), ptr(x), ptr(stats), ptr(dx_bf16), ptr(d_gamma),
+                                                     ptr(d_beta), ptr(d_colsum), _lib.current_stream()),
+          "ds_layernorm_param_grads_mixed")
 
 
 def layernorm_param_grads(dy, x, stats, d_gamma, d_beta, dx=None, d_colsum=None):

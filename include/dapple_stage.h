@@ -128,7 +128,14 @@ int ds_layernorm_fwd(int dtype, int rows, int cols, const void* x, const float* 
 int ds_layernorm_fwd_mixed(int rows, int cols, const float* x, const float* gamma, const float* beta, float eps,
                            void* y_bf16, float* y_f32, float* stats, void* stream);
 int ds_layernorm_bwd_mixed(int rows, int cols, const float* dy, const float* x, const float* gamma, const float* stats,
-                           void* dx_bf16, float* dx_f32, float* d_gamma, float* d_beta, float* d_colsum, void* stream);
+                           void* dx_bf16, float* dx_f32, void* dy_bf16, float* d_gamma, float* d_beta, float* d_colsum,
+                           void* stream);
+/* With d_gamma = d_beta = NULL ds_layernorm_bwd_mixed writes dx only (one wave per row, no atomics: the form for the
+ * chain of dependent backward kernels) and, when dy_bf16 is given, a bf16 copy of dy.  From that copy, the fp32 x, stats
+ * and dx_bf16 ds_layernorm_param_grads_mixed adds the parameter gradients (and, with d_colsum, the column sums of dx)
+ * later, over any number of rows stacked back to back - on another stream, beside the chain. */
+int ds_layernorm_param_grads_mixed(int rows, int cols, const void* dy_bf16, const float* x, const float* stats,
+                                   const void* dx_bf16, float* d_gamma, float* d_beta, float* d_colsum, void* stream);
 /* dx = LN backward; d_gamma/d_beta (fp32, [cols]) are accumulated (+=); d_colsum (nullable,
  * fp32 [cols]) += column sums of dx (the bias gradient of the dense layer that fed x);
  * dx_add (nullable) is added to dx before it is written (gradient of a residual branch). */

@@ -292,6 +292,28 @@ def test_layernorm_on_an_fp32_stream(rows, cols):
     assert_close(dg - 2.0, dgr, 1e-5, "d_gamma (added to)")
     assert_close(db + 1.0, dbr, 1e-5, "d_beta (added to)")
     assert_close(dcs, dxr.sum(0), 1e-4, "column sums of dx", floor=float(dxr.abs().max()) * rows ** 0.5)
+    # the split form: dx alone (bit-identical to the fused kernel's), then the parameter gradients from the bf16 copy of dy
+    ex16, ex32, dy16 = ops.layernorm_bwd_mixed(dy, x, gamma, stats, want_dy_bf16=True)
+    assert torch.equal(dy16, dy.to(torch.bfloat16))
+    assert_close(ex32, dxr, 1e-5, "dx fp32, rows only")
+    assert torch.equal(ex16, ex32.to(torch.bfloat16))
+    assert ops.layernorm_bwd_mixed(dy, x, gamma, stats, want_f32=False)[1] is None
+    dg2 = torch.full((cols,), 2.0, device="cuda")
+    db2 = torch.full((cols,), -1.0, device="cuda")
+    dcs2 = torch.zeros(cols, device="cuda")
+    ops.layernorm_param_grads_mixed(dy16, x, stats, dg2, db2, ex16, dcs2)
+    # against the same sums taken over the rounded copies in fp64: what the kernel is asked to compute
+    xh = (x64.detach() - x64.detach().mean(1, keepdim=True)) / torch.sqrt(x64.detach().var(1, unbiased=False, keepdim=True) + 1e-12)
+    d16 = dy16.cpu().double()
+    assert_close(dg2 - 2.0, (d16 * xh).sum(0), 1e-5, "d_gamma from the bf16 copy", floor=float(d16.abs().max()) * rows ** 0.5)
+    assert_close(db2 + 1.0, d16.sum(0), 1e-5, "d_beta from the bf16 copy", floor=float(d16.abs().max()) * rows ** 0.5)
+    assert_close(dcs2, ex16.cpu().double().sum(0), 1e-5, "column sums of the bf16 dx", floor=float(dxr.abs().max()) * rows ** 0.5)
+    # and within bf16 rounding of the exact gradients
+    assert_close(dg2 - 2.0, dgr, 2e-2, "d_gamma, deferred", floor=float(dgr.abs().max()))
+    assert_close(db2 + 1.0, dbr, 2e-2, "d_beta, deferred", floor=float(dbr.abs().max()))
+    dg3 = torch.zeros(cols, device="cuda"); db3 = torch.zeros(cols, device="cuda")
+    ops.layernorm_param_grads_mixed(dy16, x, stats, dg3, db3)     # without the column sums
+    assert torch.allclose(dg3, dg2 - 2.0, atol=1e-4 * float(dg3.abs().max())) and torch.allclose(db3, db2 + 1.0, atol=1e-4 * float(db3.abs().max()))
 
 
 @pytest.mark.parametrize("dt", ["fp32", "bf16"])
