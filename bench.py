@@ -295,15 +295,39 @@ def make_xlnet(c, args):
     return wl
 
 
-# HBM bytes per launch from rocprofv3 --pmc runs (counters cannot be read from inside this process)
+# HBM bytes per launch come from rocprofv3 --pmc runs (counters cannot be read from inside this process): the committed
+# summary of those runs holds one machine-readable row per GEMM shape of the headline workload's layer.
 TRAFFIC_SOURCE = "profiles/gemm_bert48_layer_hbm_traffic.txt"
-TRAFFIC = {
-    "gemm_dma_kernel<bf16,128,128,MN,MN>": 59.0e6,   # ffn weight-gradient shape: 42.2 MB read + 16.8 MB written
-    "gemm_dma_kernel<bf16,128,128,K,MN>": 33.9e6,    # ffn1 forward shape
-    "gemm_dma_kernel<bf16,128,128,K,K>": 33.8e6,     # ffn2 dgrad shape
-    "gemm_dma_kernel<bf16,64,64,K,K>": 35.8e6,       # mean of the ffn1 / qkv / attention-output dgrad shapes
-    "gemm_dma_kernel<bf16,64,64,K,MN>": 52.6e6,      # ffn2 forward shape
-}
+
+
+def traffic_rows(path=None):
+    """[(kernel tag, shape name, (m, n, k), bytes read, bytes written, algorithmic bytes)] of the rows 'traffic | ...'."""
+    path = path or os.path.join(os.path.dirname(os.path.abspath(__file__)), TRAFFIC_SOURCE)
+    rows = []
+    if not os.path.exists(path):
+        return rows
+    with open(path) as f:
+        for line in f:
+            if line.startswith("traffic |"):
+                p = [x.strip() for x in line.split("|")]
+                rows.append((p[1], p[2], tuple(int(x) for x in p[3].split("x")), int(p[4]), int(p[5]), int(p[6])))
+    return rows
+
+
+def traffic_of(tag, workload, wgrad_group):
+    """Mean measured HBM bytes per launch of the kernel `tag` over the shapes it runs per layer of `workload`, or None
+    where no counter run covers it (any workload but the headline one; a weight-gradient grouping other than the two
+    measured)."""
+    if workload != "bert48_half":
+        return None
+    rows = [r for r in traffic_rows() if r[0] == tag]
+    if tag.endswith(",MN,MN>"):   # weight gradients: the row of the grouping in use
+        want = {1: "wgrad ffn1 (", 4: "wgrad ffn1 x4 ("}.get(wgrad_group)
+        rows = [r for r in rows if want and r[1].startswith(want)]
+    if not rows:
+        return None
+    return sum(r[3] + r[4] for r in rows) / len(rows)
+
 
 MAKERS = {"bert": make_bert, "vgg": make_vgg, "gnmt": make_gnmt, "xlnet": make_xlnet, "gnmt_attention": make_gnmt_attention,
           "gnmt_decoder": make_gnmt_decoder}
@@ -382,10 +406,7 @@ def main():
     else:
         roof = {"bound": "hbm", "achieved": work / (ms * 1e-3) / 1e9, "peak": PEAK["hbm"] / 1e9, "unit": "GB/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["traffic"] = TRAFFIC.get(dom)
-    if dom == "gemm_dma_kernel<bf16,128,128,MN,MN>" and wl.config.get("wgrad_group", 1) != 1:
-        # measured for four micro-batches per GEMM only
-        roof["traffic"] = 134.5e6 if wl.config["wgrad_group"] == 4 else None
+    roof["traffic"] = None if reshaped else traffic_of(dom, args.workload, wl.config.get("wgrad_group", 1))
     if roof["traffic"] is not None:
         roof["traffic_unit"] = "bytes per launch (FETCH_SIZE + WRITE_SIZE, scaled by a known-traffic kernel), see " + TRAFFIC_SOURCE
     roof.update({"kernel": dom, "launches": n, "avg_launch_us": ms * 1e3 / n, "share_of_kernel_time": ms / total_ms})

@@ -8,9 +8,12 @@ ffn 4096, bf16), three launches each in the order of the list in ``gemms``, so a
 ``elementwise``: the HBM-bound kernels of the path at the BERT-48 half-stage's shapes, five launches each with their
 algorithmic bytes printed, so a kernel trace gives achieved GB/s against the HBM peak.
 
-    rocprofv3 --pmc FETCH_SIZE --output-format csv -d out -o c -- python3 -m dapple_amd.calib accumulate 67108864
-    rocprofv3 --pmc FETCH_SIZE --output-format csv -d out -o g -- python3 -m dapple_amd.calib gemms
-    rocprofv3 --kernel-trace --stats -d out -o e -- python3 -m dapple_amd.calib elementwise
+    rocprofv3 --pmc FETCH_SIZE --output-format csv -d out -o c -- python3 bench_calib.py accumulate 67108864
+    rocprofv3 --pmc FETCH_SIZE --output-format csv -d out -o g -- python3 bench_calib.py gemms
+    rocprofv3 --kernel-trace --stats -d out -o e -- python3 bench_calib.py elementwise
+
+``gemm_table``: the same GEMMs (and 4096 x 4096 x 4096) timed with events, 50 launches back to back on one stream, this
+library beside ``torch.matmul`` (hipBLASLt / rocBLAS) on the same operands: TFLOP/s per shape.
 
 ``attention``: the fused attention kernels at the BERT-48 half-stage's shape (2 samples, 16 heads, 512 positions, head
 size 64, bf16), three launches each, for the same counter runs as ``gemms`` (matrix-core busy cycles, HBM traffic).
@@ -19,8 +22,8 @@ import sys
 
 import torch
 
-from . import ops
-from ._lib import DS_EPI_ACCUM, DS_K_MAJOR, DS_MN_MAJOR
+from dapple_amd import ops
+from dapple_amd._lib import DS_EPI_ACCUM, DS_K_MAJOR, DS_MN_MAJOR
 
 
 def accumulate(n):
@@ -32,10 +35,9 @@ def accumulate(n):
     print("accumulate_kernel<float>: %d elements, reads %d bytes, writes %d bytes per launch" % (n, 8 * n, 4 * n))
 
 
-def gemms():
+def layer_shapes():
     rows, h, f = 1024, 1024, 4096
-    bf = torch.bfloat16
-    shapes = [  # name, m, n, k, a_major, b_major, accumulate
+    return [  # name, m, n, k, a_major, b_major, accumulate
         ("fwd ffn1", rows, f, h, DS_K_MAJOR, DS_MN_MAJOR, False),
         ("fwd ffn2", rows, h, f, DS_K_MAJOR, DS_MN_MAJOR, False),
         ("dgrad ffn2", rows, f, h, DS_K_MAJOR, DS_K_MAJOR, False),
@@ -44,8 +46,15 @@ def gemms():
         ("dgrad qkv", rows, h, 3 * h, DS_K_MAJOR, DS_K_MAJOR, False),
         ("dgrad ao", rows, h, h, DS_K_MAJOR, DS_K_MAJOR, False),
         ("wgrad ffn1 x4", h, f, 4 * rows, DS_MN_MAJOR, DS_MN_MAJOR, True),   # four micro-batches in one GEMM
+        ("fwd qkv", rows, 3 * h, h, DS_K_MAJOR, DS_MN_MAJOR, False),
+        ("fwd ao", rows, h, h, DS_K_MAJOR, DS_MN_MAJOR, False),
+        ("square 4096", 4096, 4096, 4096, DS_K_MAJOR, DS_MN_MAJOR, False),
     ]
-    for name, m, n, k, am, bm, acc in shapes:
+
+
+def gemms():
+    bf = torch.bfloat16
+    for name, m, n, k, am, bm, acc in layer_shapes():
         a = torch.randn((m, k) if am == DS_K_MAJOR else (k, m), device="cuda").to(bf)
         b = torch.randn((n, k) if bm == DS_K_MAJOR else (k, n), device="cuda").to(bf)
         c = torch.zeros(m, n, device="cuda", dtype=torch.float32 if acc else bf)
@@ -54,6 +63,41 @@ def gemms():
         torch.cuda.synchronize()
         alg = 2 * (m * k + n * k) + (8 if acc else 2) * m * n
         print("%s: m=%d n=%d k=%d, algorithmic bytes %d" % (name, m, n, k, alg))
+
+
+def gemm_table():
+    bf = torch.bfloat16
+    reps = 50
+    print("%-16s %-22s %10s %10s %12s %12s" % ("shape", "m x n x k", "ours us", "torch us", "ours TFLOP/s", "torch TFLOP/s"))
+    for name, m, n, k, am, bm, acc in layer_shapes():
+        a = torch.randn((m, k) if am == DS_K_MAJOR else (k, m), device="cuda").to(bf)
+        b = torch.randn((n, k) if bm == DS_K_MAJOR else (k, n), device="cuda").to(bf)
+        c = torch.zeros(m, n, device="cuda", dtype=torch.float32 if acc else bf)
+        ta = a if am == DS_K_MAJOR else a.t()      # [m, k] view
+        tb = b.t() if bm == DS_K_MAJOR else b      # [k, n] view
+        tc = torch.zeros(m, n, device="cuda", dtype=bf)
+
+        def ours():
+            ops.gemm(a, b, c, m, n, k, am, bm, flags=DS_EPI_ACCUM if acc else 0)
+
+        def theirs():
+            # the accumulating product has no single torch call on bf16 operands with an fp32 C: timed as the product alone
+            torch.matmul(ta, tb, out=tc)
+        us = []
+        for fn in (ours, theirs):
+            for _ in range(5):
+                fn()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record()
+            for _ in range(reps):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            us.append(e0.elapsed_time(e1) * 1e3 / reps)
+        fl = 2.0 * m * n * k
+        print("%-16s %-22s %10.2f %10.2f %12.1f %12.1f" % (name + (" C+=" if acc else ""), "%d x %d x %d" % (m, n, k), us[0], us[1],
+                                                          fl / us[0] / 1e6, fl / us[1] / 1e6), flush=True)
 
 
 def attention():
@@ -81,9 +125,14 @@ def elementwise():
     n_acc = 12596224                     # parameters of one encoder layer
     acc, grad = torch.zeros(n_acc, device="cuda"), torch.ones(n_acc, device="cuda")
     src = r(h * f, device="cuda")
+    xf, dyf = x.float(), dy.float()
     for _ in range(5):
         y, st = ops.layernorm_fwd(x, g, b, 1e-12)
         ops.layernorm_bwd(dy, x, g, st, dg, db, dc)
+        y16, y32, stf = ops.layernorm_fwd_mixed(xf, g, b, 1e-12)
+        ops.layernorm_bwd_mixed(dyf, xf, g, stf, dg, db, dc)
+        dx16, dx32, dy16 = ops.layernorm_bwd_mixed(dyf, xf, g, stf, want_dy_bf16=True)
+        ops.layernorm_param_grads_mixed(dy16, xf, stf, dg, db, dx16, dc)
         ops.colsum_accum(big, out)
         ops.grad_accumulate(acc, grad)
         ops.cast_to_bf16(src)
@@ -91,6 +140,10 @@ def elementwise():
     e = 2
     print("layernorm_fwd_kernel<bf16>  [%d,%d]: %d bytes per launch (read x, write y)" % (rows, h, 2 * rows * h * e))
     print("layernorm_bwd_kernel<bf16>  [%d,%d]: %d bytes per launch (read dy, x, write dx)" % (rows, h, 3 * rows * h * e))
+    print("layernorm_fwd_mixed_kernel  [%d,%d]: %d bytes per launch (read x fp32, write y bf16 + fp32)" % (rows, h, 10 * rows * h))
+    print("layernorm_bwd_mixed_kernel  [%d,%d]: %d bytes per launch (read dy, x fp32, write dx bf16 + fp32)" % (rows, h, 14 * rows * h))
+    print("layernorm_bwd_mixed_rows_kernel [%d,%d]: %d bytes per launch (as above + the bf16 copy of dy)" % (rows, h, 16 * rows * h))
+    print("layernorm_param_grad_mixed_kernel [%d,%d]: %d bytes per launch (read dy bf16, x fp32, dx bf16)" % (rows, h, 8 * rows * h))
     print("colsum_kernel<bf16>         [%d,%d]: %d bytes per launch (read x)" % (4 * rows, f, 4 * rows * f * e))
     print("accumulate_kernel<float>    %d elements: %d bytes per launch (read acc, g, write acc)" % (n_acc, 12 * n_acc))
     print("cast_kernel<bf16,float>     %d elements: %d bytes per launch (read fp32, write bf16)" % (h * f, 6 * h * f))
@@ -103,5 +156,7 @@ if __name__ == "__main__":
         elementwise()
     elif len(sys.argv) > 1 and sys.argv[1] == "attention":
         attention()
+    elif len(sys.argv) > 1 and sys.argv[1] == "gemm_table":
+        gemm_table()
     else:
         accumulate(int(sys.argv[2]) if len(sys.argv) > 2 else 1 << 26)

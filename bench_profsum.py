@@ -1,7 +1,7 @@
 """Per-kernel summary of a rocprofv3 ``--kernel-trace`` rocpd database (``*_results.db``).
 
-    python -m dapple_amd.profsum <dir>/bench_results.db
-    python -m dapple_amd.profsum pmc <dir>/x_counter_collection.csv <kernel name substring>
+    python bench_profsum.py <dir>/bench_results.db
+    python bench_profsum.py pmc <dir>/x_counter_collection.csv <kernel name substring>
 """
 import re
 import sqlite3
