@@ -14,6 +14,7 @@ DS_K_MAJOR, DS_MN_MAJOR = 0, 1
 DS_EPI_BIAS, DS_EPI_RESIDUAL, DS_EPI_GELU, DS_EPI_DGELU = 1, 2, 4, 8
 DS_EPI_OUT_F32, DS_EPI_ACCUM, DS_EPI_RELU, DS_EPI_MASK, DS_EPI_TANH_FORM = 16, 32, 64, 128, 256
 DS_EPI_GELU_GRAD, DS_EPI_MUL, DS_EPI_RESIDUAL_F32 = 512, 1024, 2048
+DS_VGG_LOSS_AS_WRITTEN, DS_VGG_LOSS_SPARSE_CE = 0, 1
 DS_STAGE_BERT, DS_STAGE_VGG19, DS_STAGE_GNMT, DS_STAGE_XLNET = 0, 1, 2, 3
 
 
@@ -97,6 +98,8 @@ PROTOTYPES = {
     "ds_layernorm_bwd_mixed": (C.c_int, [C.c_int, C.c_int] + [C.c_void_p] * 11),
     "ds_layernorm_param_grads_mixed": (C.c_int, [C.c_int, C.c_int] + [C.c_void_p] * 8),
     "ds_gemm_static_scratch": (C.c_int, [C.POINTER(GemmDesc), C.c_void_p]),
+    "ds_vgg_head_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int]),
+    "ds_vgg_head": (C.c_int, [C.c_int] * 4 + [C.c_void_p] * 8 + [C.c_int, C.c_float] + [C.c_void_p] * 10 + [C.c_size_t, C.c_void_p]),
     "ds_pooler": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "ds_stage_release_slot": (C.c_int, [C.c_void_p, C.c_int]),
     "ds_lstm_cell_fwd": (C.c_int, [C.c_int, C.c_int, C.c_float] + [C.c_void_p] * 7),

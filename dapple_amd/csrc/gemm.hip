@@ -500,10 +500,9 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
   // one barrier of the k-tile.  After it, tile kt+1 is visible, its first fragments are fetched under
   // the remaining MFMAs of tile kt, and buffer kt % STAGES is free: the loads of tile kt+STAGES go
   // there, issued one at a time between the next 4*TM*TN MFMAs (last k-step of tile kt, first three of
-  // tile kt+1).  On this part a wave's load instruction and its MFMAs only overlap when they alternate
-  // in ONE instruction stream (a loader wave beside an MFMA wave on the same SIMD makes no progress at
-  // all while the MFMAs run), and a fragment read issued between two MFMAs is free while a block of
-  // reads in front of them is not: the order below is pinned with scheduling barriers.
+  // tile kt+1).  With one wave per SIMD a load or fragment read only hides behind an MFMA when it sits
+  // between two MFMAs of the same instruction stream (a block of reads in front of the MFMAs is not
+  // free): the order below is pinned with scheduling barriers.
 #pragma unroll
   for (int s = 0; s < STAGES; ++s) {
     if (s < nkt) {

@@ -463,3 +463,41 @@ def nmt_loss_head(x, proj_kernel, target_output, target_sequence_length, d_proj_
                                loss_batch_size, loss_scale, ptr(loss), ptr(dx), ptr(d_proj_kernel), ptr(ws), nbytes,
                                _lib.current_stream()), "ds_nmt_loss_head")
     return loss, dx
+
+
+VGG_HEAD_NAMES = ("fc1/kernel", "fc1/bias", "fc2/kernel", "fc2/bias", "predictions/kernel", "predictions/bias")
+
+
+def vgg_head(x, weights, labels, grads=None, need_dx=True, loss_mode="as_written", loss_scale=1.0):
+    """Classification block + loss of the last VGG19 stage (vgg19/applications/vgg19_slice_model.py:217-220, 342-355) on
+    the flattened pool output ``x [batch, features]`` fp32.  ``weights``: {keras name: tensor} for ``VGG_HEAD_NAMES``
+    (kernels ``[in, out]``); ``labels`` fp32 ``[batch]``; ``grads`` (optional, same names) are added to in place.
+    ``loss_mode``: "as_written" (the reference's expression: a constant, see ds_vgg_head) or "sparse_ce".
+    Returns (loss [1] on the device, probabilities [batch, classes], dx or None)."""
+    w = [weights[n] for n in VGG_HEAD_NAMES]
+    g = [None] * 6 if grads is None else [grads[n] for n in VGG_HEAD_NAMES]
+    _need_cuda(x, labels, *w, *g)
+    if x.dim() != 2 or x.dtype != torch.float32 or not x.is_contiguous():
+        raise ValueError("vgg_head: x must be contiguous fp32 [batch, features]")
+    batch, features = x.shape
+    fc, classes = w[0].shape[1], w[4].shape[1]
+    want = [(features, fc), (fc,), (fc, fc), (fc,), (fc, classes), (classes,)]
+    for n, t, shp, gt in zip(VGG_HEAD_NAMES, w, want, g):
+        if t.dtype != torch.float32 or not t.is_contiguous() or tuple(t.shape) != shp:
+            raise ValueError("vgg_head: %s must be contiguous fp32 %s" % (n, shp))
+        if gt is not None and (gt.dtype != torch.float32 or not gt.is_contiguous() or gt.shape != t.shape):
+            raise ValueError("vgg_head: gradient of %s must match it" % n)
+    if labels.dtype != torch.float32 or labels.numel() != batch or not labels.is_contiguous():
+        raise ValueError("vgg_head: labels must be contiguous fp32 [batch]")
+    modes = {"as_written": _lib.DS_VGG_LOSS_AS_WRITTEN, "sparse_ce": _lib.DS_VGG_LOSS_SPARSE_CE}
+    if loss_mode not in modes:
+        raise ValueError("vgg_head: loss_mode %r" % (loss_mode,))
+    lib = _lib.load()
+    nbytes = lib.ds_vgg_head_workspace_bytes(batch, fc, classes)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    loss = torch.empty(1, dtype=torch.float32, device=x.device)
+    probs = torch.empty(batch, classes, dtype=torch.float32, device=x.device)
+    dx = torch.empty_like(x) if need_dx else None
+    check(lib.ds_vgg_head(batch, features, fc, classes, ptr(x), *[ptr(t) for t in w], ptr(labels), modes[loss_mode], loss_scale,
+                          ptr(loss), ptr(probs), ptr(dx), *[ptr(t) for t in g], ptr(ws), nbytes, _lib.current_stream()), "ds_vgg_head")
+    return loss, probs, dx

@@ -268,8 +268,11 @@ def vgg_stage(layers, batch, height, width, in_channels, stash_slots, need_input
     st = VggStage(h, _TORCH_DTYPE[cfg.dtype], batch * height * width * in_channels, batch * h_ * w_ * c_, stash_slots,
                   takes_input_grad=need_input_grad, device=device, cfg=cfg)
     st.out_shape = (batch, h_, w_, c_)
-    # the stage names convs block%d_conv%d like keras; map the caller's layer names onto them
+    # the handle numbers its convs block%d_conv%d from block 1; a stage that starts further down the model (the last
+    # device: block5_conv3 ...) goes by the caller's layer names, which are the reference's variable scopes
     st.layer_names = [n for n, c in layers if c is not None]
+    if len(st.weight_names) == 2 * len(st.layer_names):
+        st.weight_names = [n + sfx for n in st.layer_names for sfx in ("/kernel", "/bias")]
     return st
 
 

@@ -343,30 +343,72 @@ class BertFinetuneSlice(object):
 
 # =========================================================================== VGG19
 class SliceVGG19(object):
-    """vgg19_slice_model.py:38-357.  ``build`` runs stage 0 (the replicated conv stack) on one replica's share
-    of the batch and returns ``(None, [stage0_output])`` - the loss is stage 1's."""
+    """vgg19_slice_model.py:38-357.  With ``local_device=0`` ``build`` runs stage 0 (the replicated conv stack) on one
+    replica's share of the batch and returns ``(None, [stage0_output])`` - the loss is the last device's.  With
+    ``local_device=1`` it is the last device (:315-357): the rest of the conv stack, flatten, fc1, fc2, predictions and the
+    loss; ``build(stage0_output, label)`` returns ``(loss, [stage0_output, loss])`` as the reference does and keeps what
+    ``backward`` needs.  ``loss_mode``: "as_written" evaluates the reference's ``K.categorical_crossentropy(x, label)``
+    literally (a constant, ``ops.vgg_head``), "sparse_ce" the cross entropy of the label as a class index."""
 
     def __init__(self, include_top=True, weights='imagenet', input_tensor=None, input_shape=None, pooling=None,
-                 classes=1000, num_replica=15, batch_size=None, weight_values=None, seed=0, stash_slots=3, **kwargs):
+                 classes=1000, num_replica=15, batch_size=None, weight_values=None, seed=0, stash_slots=3, local_device=0,
+                 loss_mode="as_written", fc_units=4096, **kwargs):
         if num_replica not in (2, 15):
             print("For VGG19 only 2:1 and 15:1 pipeline are supported currently!")
             sys.exit(-1)
+        if local_device not in (0, 1):
+            raise ValueError("SliceVGG19: local_device %r (the model has two devices)" % (local_device,))
+        if local_device == 1 and not include_top:
+            raise ValueError("SliceVGG19: the last device is built with the classification block (include_top=True)")
         self.include_top, self.weights, self.pooling, self.classes = include_top, weights, pooling, classes
-        self.num_replica = num_replica
-        # 15:1 keeps conv1_1..conv5_2 on stage 0, 2:1 only blocks 1-3 (:280-302)
-        self.layers = synthetic.VGG19_STAGE0_15_1 if num_replica == 15 else synthetic.VGG19_STAGE0_15_1[:11]
+        self.num_replica, self.local_device, self.loss_mode, self.fc_units = num_replica, local_device, loss_mode, fc_units
+        # 15:1 keeps conv1_1..conv5_2 on stage 0, 2:1 only blocks 1-3 (:280-302); the last device has the rest (:327-340)
+        if local_device == 0:
+            self.layers = synthetic.VGG19_STAGE0_15_1 if num_replica == 15 else synthetic.VGG19_STAGE0_15_1[:11]
+        else:
+            self.layers = synthetic.VGG19_STAGE1_15_1 if num_replica == 15 else synthetic.VGG19_STAGE1_2_1
         self._weight_values, self._seed, self._stash = weight_values, seed, stash_slots
         self.stage = None
+        self.head_weights = self.head_grads = None
+
+    def _make(self, features):
+        n, h, w, c = features.shape
+        last = self.local_device == 1
+        self.stage = runtime.vgg_stage(self.layers, n, h, w, c, 1 if last else self._stash, need_input_grad=last)
+        wv = self._weight_values or synthetic.vgg_weights(self._seed, self.layers, c)
+        self.stage.bind({k: v for k, v in wv.items() if not k.startswith(("fc1/", "fc2/", "predictions/"))})
+        if last:
+            feat = 1
+            for d in self.stage.out_shape[1:]:
+                feat *= d
+            hv = {k: v for k, v in wv.items() if k.startswith(("fc1/", "fc2/", "predictions/"))}
+            if not hv:
+                hv = synthetic.vgg_head_weights(self._seed + 1, feat, self.fc_units, self.classes)
+            self.head_weights = {k: torch.as_tensor(v, dtype=torch.float32).cuda().contiguous() for k, v in hv.items()}
+            self.head_grads = {k: torch.zeros_like(v) for k, v in self.head_weights.items()}
 
     def build(self, features, label, input_shape=None, dep_outputs=None):
-        n, h, w, c = features.shape
         if self.stage is None:
-            self.stage = runtime.vgg_stage(self.layers, n, h, w, c, self._stash)
-            self.stage.bind(self._weight_values or synthetic.vgg_weights(self._seed, self.layers, c))
+            self._make(features)
         out = torch.empty(self.stage.out_shape, device=features.device)
         self.stage.forward(0, features.contiguous(), out)
-        self.stage.release(0)
-        return None, [out]
+        if self.local_device == 0:
+            self.stage.release(0)
+            return None, [out]
+        from . import ops
+        labels = torch.as_tensor(label, dtype=torch.float32).reshape(-1).cuda().contiguous()
+        self.loss, self.predictions, self._dx = ops.vgg_head(out.reshape(out.shape[0], -1), self.head_weights, labels,
+                                                             grads=self.head_grads, loss_mode=self.loss_mode)
+        return self.loss, [features, self.loss]
+
+    def backward(self, d_in=None):
+        """Last device only: the conv layers' backward pass behind the loss of the latest ``build`` (weight gradients into
+        ``stage.grads``; the head's went into ``head_grads`` during ``build``); ``d_in`` receives the gradient of the
+        boundary activation for the device before."""
+        if self.local_device != 1 or self._dx is None:
+            raise ValueError("SliceVGG19.backward: needs the last device and a build() before it")
+        self.stage.backward(0, self._dx.reshape(self.stage.out_shape), d_in)
+        self._dx = None
 
 
 # =========================================================================== XLNet

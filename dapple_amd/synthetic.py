@@ -112,6 +112,10 @@ VGG19_STAGE0_15_1 = [
     ("block5_conv1", 512), ("block5_conv2", 512),
 ]
 VGG19_CONV_STACK = VGG19_STAGE0_15_1 + [("block5_conv3", 512), ("block5_conv4", 512)]
+# what the last device runs in front of the classification block (vgg19_slice_model.py:327-340): with 15 replicas only the end
+# of block 5, with 2 replicas blocks 4 and 5
+VGG19_STAGE1_15_1 = [("block5_conv3", 512), ("block5_conv4", 512), ("block5_pool", None)]
+VGG19_STAGE1_2_1 = VGG19_STAGE0_15_1[11:] + VGG19_STAGE1_15_1
 
 
 def vgg_weights(seed, layers, in_channels=3, perturb=False):
@@ -124,6 +128,18 @@ def vgg_weights(seed, layers, in_channels=3, perturb=False):
         w[name + "/kernel"] = (rng.standard_normal((3, 3, cin, cout)) * np.sqrt(2.0 / (9 * cin))).astype(np.float32)
         w[name + "/bias"] = (0.1 * rng.standard_normal(cout)).astype(np.float32) if perturb else np.zeros(cout, np.float32)
         cin = cout
+    return w
+
+
+def vgg_head_weights(seed, features, fc=4096, classes=1000, perturb=False):
+    """fc1 / fc2 / predictions of vgg19_slice_model.py:218-220 under keras' Dense defaults: glorot-uniform kernels
+    [in, out], zero biases (or small random ones)."""
+    rng = _rng(seed)
+    w = {}
+    for name, (i, o) in (("fc1", (features, fc)), ("fc2", (fc, fc)), ("predictions", (fc, classes))):
+        lim = np.sqrt(6.0 / (i + o))
+        w[name + "/kernel"] = rng.uniform(-lim, lim, (i, o)).astype(np.float32)
+        w[name + "/bias"] = (0.1 * rng.standard_normal(o)).astype(np.float32) if perturb else np.zeros(o, np.float32)
     return w
 
 

@@ -443,6 +443,30 @@ int ds_regression_head(int dtype, int batch, int seq, int hidden, const void* x,
                        float* loss, float* pooled, float* prediction, float* dprediction, float* dz, void* dx,
                        float* d_pooler_w, float* d_pooler_b, float* d_fc_w, float* d_fc_b, void* stream);
 
+/* Classification block and loss of the last VGG19 stage: vgg19/applications/vgg19_slice_model.py:217-220 (flatten; fc1,
+ * fc2 = Dense(4096, relu); predictions = Dense(classes, softmax)) applied at :342-347, and the loss of :354-355,
+ * score_array = K.categorical_crossentropy(x, label); loss = reduce_mean(score_array).
+ *   x fp32 [batch, features]: the flattened NHWC output of block5_pool (keras Flatten keeps the row-major order);
+ *   fc1_w [features, fc], fc2_w [fc, fc], pred_w [fc, classes] in keras' [in, out] layout, biases [out]; all fp32;
+ *   labels fp32 [batch] (the reference feeds a float column, vgg19/tf-keras-dapple.py:57-63);
+ *   loss_mode DS_VGG_LOSS_AS_WRITTEN: the expression of the reference's graph - keras takes its first argument as the
+ *     target, so the softmax output is the target and the label column the "output": label / sum(label) = 1 (NaN for a
+ *     zero label), clipped to 1 - 1e-7, loss = -log(1 - 1e-7) * mean_rows(sum_c x[c]), a constant of about 1.2e-7 whose
+ *     gradient behind the softmax is zero up to rounding;
+ *   loss_mode DS_VGG_LOSS_SPARSE_CE: labels are class indices, loss = mean_rows(-log x[label]) (NaN for a label that is
+ *     no index in [0, classes));
+ *   loss: device float, overwritten with loss_scale * loss; probs fp32 [batch, classes] out;
+ *   dx (nullable) fp32 [batch, features]: the d_out of the conv stage's backward pass; the six weight gradients (all or
+ *   none, nullable) are master gradients, added to.  features, fc, classes multiples of 4. */
+#define DS_VGG_LOSS_AS_WRITTEN 0
+#define DS_VGG_LOSS_SPARSE_CE 1
+size_t ds_vgg_head_workspace_bytes(int batch, int fc, int classes);
+int ds_vgg_head(int batch, int features, int fc, int classes, const float* x, const float* fc1_w, const float* fc1_b,
+                const float* fc2_w, const float* fc2_b, const float* pred_w, const float* pred_b, const float* labels,
+                int loss_mode, float loss_scale, float* loss, float* probs, float* dx, float* d_fc1_w, float* d_fc1_b,
+                float* d_fc2_w, float* d_fc2_b, float* d_pred_w, float* d_pred_b, void* workspace, size_t workspace_bytes,
+                void* stream);
+
 /* Output projection and loss of the GNMT model on the last device: gnmt/nmt/model.py:685-686 (logits =
  * output_layer(rnn_output); output_layer is a Dense without bias, :497-499) and _compute_loss :824-838
  * (loss = sum(sparse_softmax_cross_entropy(target_output, logits) * sequence_mask(target_sequence_length)) / batch_size).

@@ -9,7 +9,8 @@ reached by permutation.  Backward is torch.autograd.
 Pins (tests/test_oracle_vgg.py): conv vs a brute-force 7-deep loop; 'same' padding = 1;
 max-pool vs brute force; ReLU gradient 0 at exactly 0; parameter counts vs
 profiling_results/vgg-19-pbs-32.txt of the reference; stage_vjp_forced_branches vs stage_vjp with the
-branches it took itself, and vs brute force on a case with flipped branches.
+branches it took itself, and vs brute force on a case with flipped branches; the classification block and both
+losses of head_forward / head_loss vs scalar loops, torch's cross_entropy and the closed form of the as-written loss.
 """
 import torch
 
@@ -100,3 +101,31 @@ def stage_vjp_forced_branches(x, w, d_out, layers, masks, picks, need_input_grad
     grads = torch.autograd.grad(h, xs, grad_outputs=d_out, allow_unused=True)
     off = 1 if need_input_grad else 0
     return h.detach(), (grads[0] if need_input_grad else None), {n: g for n, g in zip(names, grads[off:]) if g is not None}
+
+
+# ---------------------------------------------------------------------------------------- last stage: classification block
+def head_forward(x, hw):
+    """vgg19_slice_model.py:217-220 applied at :342-347: Flatten (the caller passes [batch, features]), fc1 and fc2 =
+    Dense(4096, relu), predictions = Dense(classes, softmax); kernels in keras' [in, out] layout."""
+    h1 = torch.relu(x @ hw["fc1/kernel"] + hw["fc1/bias"])
+    h2 = torch.relu(h1 @ hw["fc2/kernel"] + hw["fc2/bias"])
+    return torch.softmax(h2 @ hw["predictions/kernel"] + hw["predictions/bias"], -1)
+
+
+def keras_categorical_crossentropy(target, output, epsilon=1e-7):
+    """keras.backend.categorical_crossentropy(target, output) of the TensorFlow backend for probabilities
+    (from_logits=False), restated from its published definition (keras is not vendored in the reference):
+    output /= reduce_sum(output, -1, keepdims); output = clip(output, eps, 1 - eps); -reduce_sum(target * log(output), -1)."""
+    output = output / output.sum(-1, keepdim=True)
+    output = torch.clamp(output, epsilon, 1.0 - epsilon)
+    return -(target * torch.log(output)).sum(-1)
+
+
+def head_loss(probs, labels, mode="as_written"):
+    """vgg19_slice_model.py:354-355.  "as_written": K.categorical_crossentropy(x, label) exactly as called - the softmax
+    output lands in the `target` slot and the [batch, 1] float label column in the `output` slot - then reduce_mean.
+    "sparse_ce": mean of -log probs[label] with the label as a class index."""
+    if mode == "as_written":
+        return keras_categorical_crossentropy(probs, labels.reshape(-1, 1).to(probs.dtype)).mean()
+    idx = labels.to(torch.int64)
+    return -torch.log(probs[torch.arange(probs.shape[0]), idx]).mean()

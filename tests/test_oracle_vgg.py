@@ -117,3 +117,45 @@ def test_forced_branches_reproduce_the_free_pass_and_follow_a_flipped_branch():
         fd = (f(wp) - f(wm)) / (2 * eps)
         assert abs(fd - float(dwf[name][idx])) <= 1e-7 * max(1.0, abs(fd)), (name, fd, float(dwf[name][idx]))
     assert not torch.allclose(dwf["c1/kernel"], dw0["c1/kernel"])       # the flip is visible in the gradient
+
+
+def _head_weights(r, features, fc, classes):
+    return {"fc1/kernel": torch.tensor(r.standard_normal((features, fc)) * 0.3), "fc1/bias": torch.tensor(r.standard_normal(fc) * 0.1),
+            "fc2/kernel": torch.tensor(r.standard_normal((fc, fc)) * 0.3), "fc2/bias": torch.tensor(r.standard_normal(fc) * 0.1),
+            "predictions/kernel": torch.tensor(r.standard_normal((fc, classes)) * 0.3),
+            "predictions/bias": torch.tensor(r.standard_normal(classes) * 0.1)}
+
+
+def test_classification_block_vs_scalar_loops():
+    r = np.random.Generator(np.random.PCG64(11))
+    B, Fe, Fc, Cl = 3, 5, 4, 6
+    hw = _head_weights(r, Fe, Fc, Cl)
+    x = r.standard_normal((B, Fe))
+    got = ov.head_forward(torch.tensor(x), hw).numpy()
+    for b in range(B):
+        h1 = [max(0.0, sum(x[b, i] * hw["fc1/kernel"][i, j].item() for i in range(Fe)) + hw["fc1/bias"][j].item()) for j in range(Fc)]
+        h2 = [max(0.0, sum(h1[i] * hw["fc2/kernel"][i, j].item() for i in range(Fc)) + hw["fc2/bias"][j].item()) for j in range(Fc)]
+        z = [sum(h2[i] * hw["predictions/kernel"][i, j].item() for i in range(Fc)) + hw["predictions/bias"][j].item() for j in range(Cl)]
+        e = [np.exp(v - max(z)) for v in z]
+        assert np.allclose(got[b], [v / sum(e) for v in e], atol=1e-12)
+
+
+def test_losses_of_the_classification_block():
+    r = np.random.Generator(np.random.PCG64(12))
+    B, Cl = 4, 7
+    z = torch.tensor(r.standard_normal((B, Cl)), requires_grad=True)
+    p = torch.softmax(z, -1)
+    labels = torch.tensor([3.0, 1.0, 6.0, 2.0])
+    # the conventional loss is torch's cross_entropy on the logits
+    want = torch.nn.functional.cross_entropy(z, labels.long())
+    assert torch.allclose(ov.head_loss(p, labels, "sparse_ce"), want, atol=1e-12)
+    # keras' function, used the right way round, is the one-hot cross entropy as well
+    onehot = torch.nn.functional.one_hot(labels.long(), Cl).double()
+    assert torch.allclose(ov.keras_categorical_crossentropy(onehot, p).mean(), want, atol=1e-6)    # (clipping at 1e-7)
+    # as the reference calls it the label column is normalised to 1 and clipped: a constant, whatever the logits
+    loss = ov.head_loss(p, labels, "as_written")
+    assert abs(loss.item() - (-np.log(1.0 - 1e-7))) < 1e-15
+    (g,) = torch.autograd.grad(loss, z)
+    assert g.abs().max().item() < 1e-20 + 1e-7 * 1e-15          # constant upstream gradient dies in the softmax
+    # a zero label is 0/0
+    assert torch.isnan(ov.head_loss(p.detach(), torch.tensor([3.0, 0.0, 6.0, 2.0]), "as_written"))
