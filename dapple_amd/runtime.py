@@ -22,7 +22,11 @@ def stash_depth(stage_index, num_stages, variant="S"):
 
 
 def schedule_ops(stage_index, num_stages, num_micro_batches, variant="S"):
-    """[('F', j) | ('B', j)] in execution order: K warm-up forwards, then one backward per forward."""
+    """[('F', j) | ('B', j)] in execution order: K warm-up forwards, then one backward per forward.  K is the number of
+    forwards the reference's control edges let a stage run ahead (bert/graph.py:126-132: S - i; vgg19/tf-keras-dapple.py:292:
+    2S - 1 - i).  For the first stage this is the order the graph executes in; under the "2S-1" rule a later stage's
+    backward is ready earlier than that, so there the list is the deepest order the edges allow (and what the stash is
+    sized for), one of several valid executions with identical results."""
     if not (0 <= stage_index < num_stages):
         raise ValueError("stage_index %d outside [0, %d)" % (stage_index, num_stages))
     if num_micro_batches < 1:

@@ -86,3 +86,33 @@ def closed_form(stage, num_stages, num_micro_batches, variant="S"):
         if j + K < M:
             ops.append(("F", j + K))
     return ops
+
+
+def runs_to_completion(orders, num_stages, num_micro_batches, variant="S"):
+    """True if every stage can execute exactly its prescribed op list ``orders[i]``, in that order, without deadlock
+    under the graph's edges (the data edges of ``simulate`` and the control edge ``dep_of``): the prescribed lists are
+    then one valid execution of the reference's unrolled graph."""
+    S = num_stages
+    pos = [0] * S
+    done = set()
+    total = sum(len(o) for o in orders)
+    while len(done) < total:
+        fired = []
+        for i in range(S):
+            if pos[i] >= len(orders[i]):
+                continue
+            op, j = orders[i][pos[i]]
+            if op == "F":
+                ok = (i == 0 or ("F", j, i - 1) in done)
+                dep = dep_of(j, i, S, variant)
+                ok = ok and (dep is None or (dep[0], dep[1], i) in done)
+            else:
+                ok = ("F", j, i) in done and (i == S - 1 or ("B", j, i + 1) in done)
+            if ok:
+                fired.append((op, j, i))
+        if not fired:
+            return False
+        for op, j, i in fired:
+            done.add((op, j, i))
+            pos[i] += 1
+    return True
