@@ -256,7 +256,7 @@ def make_xlnet(c, args):
     adt = torch.bfloat16 if c["dtype"] == "bf16" else torch.float32
     K = runtime.stash_depth(0, 2)
     stage = runtime.xlnet_stage(L, H, N, F, B, Q, c["dtype"], stash_slots=K, mem_len=Mm, streams=S,
-                                fused_attention=args.xlnet_fused_attention)
+                                fused_attention=args.xlnet_fused_attention, residual_fp32=not args.bf16_residual_stream)
     stage.bind(synthetic.xlnet_weights(synthetic.SEED_WEIGHT + c["index"], L, H, N, F))
     xs = [torch.as_tensor(np.stack(x)).cuda().to(adt) for x in synthetic.xlnet_stream_inputs(synthetic.SEED_INPUT + c["index"], M, Q, B, H, S)]
     dys = [torch.as_tensor(np.stack(x)).cuda().to(adt) for x in synthetic.xlnet_stream_inputs(synthetic.SEED_GRAD + c["index"], M, Q, B, H, S)]
@@ -277,7 +277,8 @@ def make_xlnet(c, args):
     fwd = 2 * H * H * (S * Q + 2 * Kl + R + S * Q) + S * (2 * 2 * Q * Kl * H + 2 * Q * R * H) + S * 4 * Q * H * F
     wl.flops_per_sample = 3 * fwd * L
     wl.config = {"layers": L, "hidden": H, "heads": N, "ffn": F, "seq": Q, "mem_len": Mm, "streams": S, "micro_batch": B,
-                 "micro_batches": M, "schedule": "1F1B stage 0 of 2, stash K=%d" % K, "flops": "two-stream count"}
+                 "micro_batches": M, "schedule": "1F1B stage 0 of 2, stash K=%d" % K, "flops": "two-stream count",
+                 "residual_stream": "fp32" if (c["dtype"] != "bf16" or not args.bf16_residual_stream) else "bf16"}
 
     def cpu():
         from oracle import xlnet as ox
@@ -343,7 +344,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-overlap", action="store_true", help="keep forward and backward passes on one stream")
     ap.add_argument("--bf16-residual-stream", action="store_true",
-                    help="BERT bf16 workloads: round the residual stream to bf16 too (faster, twice the error at 24 layers)")
+                    help="BERT / XLNet bf16 workloads: round the residual stream to bf16 too (faster, twice the error at full depth)")
     ap.add_argument("--wgrad-group", type=int, default=4,
                     help="BERT stages: weight gradients of this many backward passes in one GEMM per weight")
     ap.add_argument("--xlnet-fused-attention", action="store_true",

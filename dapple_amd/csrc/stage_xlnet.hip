@@ -223,6 +223,10 @@ struct XlnetStage : ds_stage {
   char* stash_base = nullptr;
   size_t slot_bytes = 0, mask_off = 0, seg_off = 0, mem_off = 0, maskt_off = 0, segt_off = 0;
   bool fused_fwd = false;  // forward attention in one kernel (bf16, head size 64, seq a multiple of 64)
+  // bf16 with xc.residual_fp32: the residual stream (the sums in front of both LayerNorms, the LayerNorm outputs that feed
+  // the next sum, and the same chain of gradients in backward) stays in fp32; bf16 is only what a GEMM reads
+  bool rs32 = false;
+  size_t fw_xf[2] = {0, 0}, fw_y1f = 0, bw_dxf[2] = {0, 0}, bw_dz2f = 0, bw_dy1f = 0, bw_dz1f = 0;
   std::vector<LayerOff> lo;
   std::vector<char> has_mask, has_seg;
   // workspace
@@ -287,6 +291,7 @@ struct XlnetStage : ds_stage {
     seg_off = sa.reserve((size_t)Q * K * B);
     mem_off = sa.reserve((size_t)L * (Mm > 0 ? Mm : 1) * B * H * esz);
     fused_fwd = xc.fused_attention != 0 && ds_xl_attention_fits(dtype, D, Q, K, R);
+    rs32 = dtype == DS_BF16 && xc.residual_fp32 != 0 && H % 8 == 0 && H <= 2048;
     if (fused_fwd) {
       maskt_off = sa.reserve((size_t)B * K * S * Q * 4);
       segt_off = sa.reserve((size_t)B * K * Q);
@@ -299,8 +304,8 @@ struct XlnetStage : ds_stage {
       t.qw = sa.reserve(act); t.qr = sa.reserve(act); t.qs = sa.reserve(act);
       t.kv = sa.reserve((size_t)krows * 2 * H * esz);
       t.p = sa.reserve((size_t)S * B * N * Q * K * esz);
-      t.vec = sa.reserve(act); t.z1 = sa.reserve(act); t.y1 = sa.reserve(act);
-      t.u = sa.reserve(actF); t.hh = sa.reserve(actF); t.z2 = sa.reserve(act);
+      t.vec = sa.reserve(act); t.z1 = sa.reserve(rs32 ? (size_t)rows * H * 4 : act); t.y1 = sa.reserve(act);
+      t.u = sa.reserve(actF); t.hh = sa.reserve(actF); t.z2 = sa.reserve(rs32 ? (size_t)rows * H * 4 : act);
       t.st1 = sa.reserve(stats); t.st2 = sa.reserve(stats);
       if (l + 1 < L) next_x = sa.reserve(act);
     }
@@ -329,6 +334,12 @@ struct XlnetStage : ds_stage {
       ws_deft[p] = w.reserve((size_t)N * 2 * rows * esz);
     }
     ws_dx[0] = w.reserve(act); ws_dx[1] = w.reserve(act);
+    if (rs32) {
+      const size_t act32 = (size_t)rows * H * 4;
+      fw_xf[0] = w.reserve(act32); fw_xf[1] = w.reserve(act32); fw_y1f = w.reserve(act32);
+      bw_dxf[0] = w.reserve(act32); bw_dxf[1] = w.reserve(act32);
+      bw_dz2f = w.reserve(act32); bw_dy1f = w.reserve(act32); bw_dz1f = w.reserve(act32);
+    }
     ws_bytes = w.used;
     DS_CHECK_HIP(hipMalloc((void**)&ws_base, ws_bytes));
     // the un-shifted score gradients: zero outside the band the softmax backward kernel writes
@@ -493,6 +504,8 @@ struct XlnetStage : ds_stage {
     const float scale = 1.0f / sqrtf((float)D);
     const uint8_t* seg = has_seg[slot] ? (const uint8_t*)(sp + seg_off) : nullptr;
     DS_CHECK_HIP(hipMemcpyAsync(sp + lo[0].x, in, act, hipMemcpyDeviceToDevice, stream));
+    if (rs32) DS_PROPAGATE(ds_cast_bf16_to_f32(ws_base + fw_xf[0], in, (size_t)rows * H, stream));
+    const int res32 = DS_EPI_RESIDUAL | DS_EPI_RESIDUAL_F32 | DS_EPI_OUT_F32;
     char* qall = ws_base + ws_qall;
     float* ac = (float*)(ws_base + ws_ac);
     float* bd = (float*)(ws_base + ws_bd);
@@ -546,6 +559,22 @@ struct XlnetStage : ds_stage {
                              (int64_t)B * 2 * H, 2 * H, D, sp + t.vec, (int64_t)B * H, H, D, 0));
       }
       // attn_out = vec Wo^T (einsum ibnd,hnd->ibh) + x, LayerNorm
+      if (rs32) {
+        // fp32 stream: x and y1 travel as fp32 beside their bf16 copies (the GEMM operands); z1, z2 are stashed in fp32
+        float* xf = (float*)(ws_base + fw_xf[l & 1]);
+        float* y1f = (float*)(ws_base + fw_y1f);
+        float* yf = (l + 1 < L) ? (float*)(ws_base + fw_xf[(l + 1) & 1]) : nullptr;
+        DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rows, H, H, sp + t.vec, H, WT(l, X_O), H, sp + t.z1, H, res32, nullptr, xf));
+        DS_PROPAGATE(ds_layernorm_fwd_mixed(rows, H, (const float*)(sp + t.z1), w[b + X_LN1_G], w[b + X_LN1_B], xc.ln_eps, sp + t.y1, y1f,
+                                            (float*)(sp + t.st1), stream));
+        DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, rows, F, H, sp + t.y1, H, WT(l, X_W1), F, sp + t.u, F,
+                          DS_EPI_BIAS | DS_EPI_GELU | DS_EPI_TANH_FORM, w[b + X_B1], nullptr, sp + t.hh));
+        DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, rows, H, F, sp + t.hh, F, WT(l, X_W2), H, sp + t.z2, H, DS_EPI_BIAS | res32,
+                          w[b + X_B2], y1f));
+        DS_PROPAGATE(ds_layernorm_fwd_mixed(rows, H, (const float*)(sp + t.z2), w[b + X_LN2_G], w[b + X_LN2_B], xc.ln_eps, y, yf,
+                                            (float*)(sp + t.st2), stream));
+        continue;
+      }
       DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rows, H, H, sp + t.vec, H, WT(l, X_O), H, sp + t.z1, H, DS_EPI_RESIDUAL, nullptr, x));
       DS_PROPAGATE(ds_layernorm_fwd(dtype, rows, H, sp + t.z1, w[b + X_LN1_G], w[b + X_LN1_B], xc.ln_eps, sp + t.y1, (float*)(sp + t.st1), stream));
       DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, rows, F, H, sp + t.y1, H, WT(l, X_W1), F, sp + t.u, F,
@@ -569,6 +598,12 @@ struct XlnetStage : ds_stage {
     // with a weight-gradient stream, a layer's weight gradients run beside the dgrad chain of the layers below
     hipStream_t wgs = wgrad_stream;
     if (wgs) DS_PROPAGATE(lane.ensure());
+    const int res32 = DS_EPI_RESIDUAL | DS_EPI_RESIDUAL_F32 | DS_EPI_OUT_F32;
+    const float* dyf = nullptr;   // fp32 stream: the gradient that travels down the layers
+    if (rs32) {
+      DS_PROPAGATE(ds_cast_bf16_to_f32(ws_base + bw_dxf[L & 1], d_out, (size_t)rows * H, stream));
+      dyf = (const float*)(ws_base + bw_dxf[L & 1]);
+    }
     for (int l = L - 1; l >= 0; --l) {
       const LayerOff& t = lo[l];
       const int b = base(l);
@@ -579,12 +614,24 @@ struct XlnetStage : ds_stage {
       char* deft = ws_base + ws_deft[par]; char* dbd = ws_base + ws_dbd[par];
       if (wgs) DS_PROPAGATE(lane.reuse(stream, par));
       char* x = sp + t.x;
+      float* dz2f = (float*)(ws_base + bw_dz2f);
+      float* dy1f = (float*)(ws_base + bw_dy1f);
+      float* dz1f = (float*)(ws_base + bw_dz1f);
+      if (rs32) {
+        DS_PROPAGATE(ds_layernorm_bwd_mixed(rows, H, dyf, (const float*)(sp + t.z2), w[b + X_LN2_G], (const float*)(sp + t.st2), dz2, dz2f,
+                                            nullptr, g[b + X_LN2_G], g[b + X_LN2_B], g[b + X_B2], stream));
+        DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rows, F, H, dz2, H, WT(l, X_W2), H, du, F, DS_EPI_DGELU | DS_EPI_TANH_FORM, nullptr, nullptr, sp + t.u));
+        DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rows, H, F, du, F, WT(l, X_W1), F, dy1f, H, res32, nullptr, dz2f));
+        DS_PROPAGATE(ds_layernorm_bwd_mixed(rows, H, dy1f, (const float*)(sp + t.z1), w[b + X_LN1_G], (const float*)(sp + t.st1), dz1, dz1f,
+                                            nullptr, g[b + X_LN1_G], g[b + X_LN1_B], nullptr, stream));
+      } else {
       DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, dy, sp + t.z2, w[b + X_LN2_G], (const float*)(sp + t.st2), nullptr, dz2,
                                     g[b + X_LN2_G], g[b + X_LN2_B], g[b + X_B2], stream));
       DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rows, F, H, dz2, H, WT(l, X_W2), H, du, F, DS_EPI_DGELU | DS_EPI_TANH_FORM, nullptr, nullptr, sp + t.u));
       DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rows, H, F, du, F, WT(l, X_W1), F, dy1, H, DS_EPI_RESIDUAL, nullptr, dz2));
       DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, dy1, sp + t.z1, w[b + X_LN1_G], (const float*)(sp + t.st1), nullptr, dz1,
                                     g[b + X_LN1_G], g[b + X_LN1_B], nullptr, stream));
+      }
       // o projection: attn_out[row,h] = sum_nd vec[row,nd] Wo[h,nd]
       DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, rows, H, H, dz1, H, WT(l, X_O), H, dvec, H));
       {
@@ -693,6 +740,14 @@ struct XlnetStage : ds_stage {
       const bool first = l == 0;
       if (first && d_in == nullptr) break;
       char* dx = first ? (char*)d_in : ws_base + ws_dx[l & 1];
+      if (rs32) {
+        float* dxf = (float*)(ws_base + bw_dxf[l & 1]);
+        DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rows, H, H, dq, H, WT(l, X_Q), H, dxf, H, res32, nullptr, dz1f));
+        DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rowsS, H, 2 * H, dkv_h, 2 * H, wkv[l], 2 * H, dxf, H, res32, nullptr, dxf));
+        if (first) DS_PROPAGATE(ds_cast_f32_to_bf16(d_in, dxf, (size_t)rows * H, stream));  // the stage's input gradient leaves as bf16
+        dyf = dxf;
+        continue;
+      }
       DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rows, H, H, dq, H, WT(l, X_Q), H, dx, H, DS_EPI_RESIDUAL, nullptr, dz1));
       DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rowsS, H, 2 * H, dkv_h, 2 * H, wkv[l], 2 * H, dx, H, DS_EPI_RESIDUAL, nullptr, dx));
       dy = dx;

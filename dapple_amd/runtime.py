@@ -381,15 +381,17 @@ class XlnetStage(Stage):
 
 
 def xlnet_stage(num_layers, hidden, heads, ffn, batch, seq, dtype, stash_slots, mem_len=0, streams=1, first_layer=0,
-                ln_eps=1e-14, device="cuda:0", fused_attention=False):
+                ln_eps=1e-14, device="cuda:0", fused_attention=False, residual_fp32=True):
     """An XLNet stage of ``num_layers`` relative-attention layers (xlnet/models/slice_xlnet.py:164-180).
-    ``fused_attention``: run the forward attention as one kernel where the shape allows."""
+    ``fused_attention``: run the forward attention as one kernel where the shape allows.  ``residual_fp32`` (bf16 stages):
+    keep the residual stream in fp32 (``ds_xlnet_cfg.residual_fp32``)."""
     lib = _lib.load()
     cfg = XlnetCfg()
     cfg.dtype, cfg.num_layers, cfg.hidden, cfg.heads, cfg.ffn = _dtype_code(dtype), num_layers, hidden, heads, ffn
     cfg.batch, cfg.seq, cfg.mem_len, cfg.streams = batch, seq, mem_len, streams
     cfg.ln_eps, cfg.first_layer, cfg.stash_slots = ln_eps, first_layer, stash_slots
     cfg.fused_attention = 1 if fused_attention else 0
+    cfg.residual_fp32 = 1 if residual_fp32 else 0
     h = C.c_void_p()
     with torch.cuda.device(torch.device(device)):
         check(lib.ds_xlnet_stage_create(C.byref(cfg), _lib.current_stream(), C.byref(h)), "ds_xlnet_stage_create")

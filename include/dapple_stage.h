@@ -389,7 +389,10 @@ typedef struct ds_xlnet_cfg {
   int fused_attention; /* 1: forward attention in one kernel where the shape allows (bf16, head size 64, seq a multiple of
                           64, mem_len + seq a multiple of 32); 0 (default): products and softmax as separate launches,
                           which is the faster step at the benchmark shape today.  Results agree to rounding. */
-  int reserved[7];
+  int residual_fp32;   /* bf16 only, 1: the residual stream (the sums in front of both LayerNorms, the LayerNorm outputs that
+                          feed the next sum, the same chain of gradients) stays in fp32, bf16 is what the GEMMs read: the
+                          stream's own rounding no longer adds up over the layers (as ds_stage_cfg.residual_fp32) */
+  int reserved[6];
 } ds_xlnet_cfg;
 int ds_xlnet_stage_create(const ds_xlnet_cfg* cfg, void* stream, ds_stage** out);
 /* Side inputs of the micro-batch that will be forwarded into `slot` (copied into the slot):
