@@ -22,7 +22,9 @@ typedef __attribute__((address_space(1))) void* glb_vptr;
 
 constexpr int HD = 64;        // head size
 constexpr int ROWB = 128;     // bytes per tile row (64 bf16)
-constexpr int CHUNK = 256;    // rows of K/V (or Q/dO) resident in LDS at a time
+constexpr int CHUNK = 256;    // rows of K/V (or Q/dO) resident in LDS at a time (XLNet kernel: one buffer of this size)
+constexpr int CH = 128;       // BERT kernels: the same 64 KB as two buffers of 128 rows per tensor; chunk c+2 is loaded while
+                              // chunk c+1 is multiplied, and a chunk is exactly one 32-row step for each of the SPLIT waves
 // A block owns 64 rows of the parallel axis (two groups of 32) and splits the walked axis SPLIT ways:
 // wave w works for group (w & 1) on every SPLIT-th 32-row step starting at (w >> 1).  2*SPLIT waves
 // give every SIMD two waves, so one wave's softmax arithmetic runs under the other's MFMAs.  The
@@ -56,6 +58,16 @@ __device__ __forceinline__ void tile_fill(char* lds, const bf16* src, int64_t ld
   }
 }
 
+// The kernels below never issue another vector-memory load between their prologue and their last chunk, so vmcnt counts
+// tile loads only: a thread issues rows / 64 loads per tensor and chunk.  Waits until only the next chunk's loads (two
+// tensors of next_rows rows) may still be in flight.
+__device__ __forceinline__ void wait_chunk(int next_rows) {
+  const int n = next_rows / 32;  // 2 tensors x next_rows / 64
+  if (n >= 4) __builtin_amdgcn_s_waitcnt((4 & 15) | (7 << 4) | (15 << 8));
+  else if (n >= 2) __builtin_amdgcn_s_waitcnt((2 & 15) | (7 << 4) | (15 << 8));
+  else __builtin_amdgcn_s_waitcnt(VMCNT0);
+}
+
 // A operand, rows = tile rows (row0 + lane%32), k = 8 consecutive columns starting at 16*ks + 8*half
 __device__ __forceinline__ bf16x8 frag_rows(const char* lds, int row0, int ks, int lane) {
   return *reinterpret_cast<const bf16x8*>(lds + tile_off(row0 + (lane & 31), (2 * ks + (lane >> 5)) * 16));
@@ -77,6 +89,8 @@ __device__ __forceinline__ bf16x8 pack8(const float* p) {
   for (int j = 0; j < 8; ++j) r[j] = (bf16)p[j];
   return r;
 }
+constexpr float LOG2E = 1.4426950408889634f, LN2 = 0.6931471805599453f;
+__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ f32x16 mfma(bf16x8 a, bf16x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
 // index along the softmax axis of accumulator element e for this lane's half: (e/4)*8 + 4*half + e%4
 __device__ __forceinline__ int acc_row(int e, int half) { return (e >> 2) * 8 + half * 4 + (e & 3); }
@@ -153,51 +167,59 @@ __global__ __launch_bounds__(NTHREADS) void attn_fwd_kernel(AttnArgs a) {
   const int b = blockIdx.y / a.N, hd = blockIdx.y % a.N;
   const int q = blockIdx.x * 64 + grp * 32 + (lane & 31);
   const bf16* base = a.qkv + (int64_t)b * a.S * a.ld + hd * HD;
-  char* sk = lds;
-  char* sv = lds + CHUNK * ROWB;
-  float* adder = reinterpret_cast<float*>(lds + 2 * CHUNK * ROWB);
-  // the first K / V tiles are requested before anything else: the loads below queue behind them and the whole prologue
+  auto sk = [&](int c) { return lds + (c & 1) * (2 * CH * ROWB); };              // two buffers of CH rows per tensor
+  auto sv = [&](int c) { return lds + (c & 1) * (2 * CH * ROWB) + CH * ROWB; };
+  float* adder = reinterpret_cast<float*>(lds + 4 * CH * ROWB);
+  const int nch = (a.S + CH - 1) / CH;
+  auto rows_of = [&](int c) { return a.S - c * CH < CH ? a.S - c * CH : CH; };
+  auto fill = [&](int c) {
+    tile_fill(sk(c), base + a.H + (int64_t)c * CH * a.ld, a.ld, rows_of(c), wave, lane);
+    tile_fill(sv(c), base + 2 * a.H + (int64_t)c * CH * a.ld, a.ld, rows_of(c), wave, lane);
+  };
+  // the first two K / V chunks are requested before anything else: the loads below queue behind them and the whole prologue
   // costs one trip to memory (a mask row staged through LDS would otherwise be waited for before the tiles are asked for)
-  tile_fill(sk, base + a.H, a.ld, a.S < CHUNK ? a.S : CHUNK, wave, lane);
-  tile_fill(sv, base + 2 * a.H, a.ld, a.S < CHUNK ? a.S : CHUNK, wave, lane);
-  for (int j = threadIdx.x; j < a.S; j += NTHREADS)
-    adder[j] = a.key_mask ? (1.0f - a.key_mask[(int64_t)b * a.S + j]) * a.mask_value : 0.f;
+  fill(0);
+  if (nch > 1) fill(1);
+  const bool masked = a.key_mask != nullptr;
+  if (masked)
+    for (int j = threadIdx.x; j < a.S; j += NTHREADS) adder[j] = (1.0f - a.key_mask[(int64_t)b * a.S + j]) * a.mask_value * LOG2E;
   bf16x8 qf[4];
 #pragma unroll
   for (int ks = 0; ks < 4; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(base + (int64_t)q * a.ld + 16 * ks + 8 * half);
   f32x16 o[2];
 #pragma unroll
   for (int e = 0; e < 16; ++e) { o[0][e] = 0.f; o[1][e] = 0.f; }
+  // running maximum and sum in the base-2 domain: p = exp2(s * scale * log2(e) + adder * log2(e) - m)
   float m = -INFINITY, l = 0.f;
-  for (int k0 = 0; k0 < a.S; k0 += CHUNK) {
-    const int rows = a.S - k0 < CHUNK ? a.S - k0 : CHUNK;
+  const float c2 = a.scale * LOG2E;
+  __builtin_amdgcn_s_waitcnt(VMCNT0);  // q fragments (and the first two chunks): from here on only tile loads are in flight
+  for (int c = 0; c < nch; ++c) {
+    const int rows = rows_of(c);
+    wait_chunk(c + 1 < nch ? rows_of(c + 1) : 0);
     __syncthreads();
-    if (k0 > 0) {  // tile 0 was requested at the top
-      tile_fill(sk, base + a.H + (int64_t)k0 * a.ld, a.ld, rows, wave, lane);
-      tile_fill(sv, base + 2 * a.H + (int64_t)k0 * a.ld, a.ld, rows, wave, lane);
-    }
-    __builtin_amdgcn_s_waitcnt(VMCNT0);
-    __syncthreads();
-    for (int kt = part * 32; kt < rows; kt += 32 * SPLIT) {
+    const char* ck = sk(c);
+    const char* cv = sv(c);
+    const int kt = part * 32;
+    if (kt < rows) {
       f32x16 s;
 #pragma unroll
       for (int e = 0; e < 16; ++e) s[e] = 0.f;
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) s = mfma(frag_rows(sk, kt, ks, lane), qf[ks], s);
+      for (int ks = 0; ks < 4; ++ks) s = mfma(frag_rows(ck, kt, ks, lane), qf[ks], s);
       float p[16];
       float mt = -INFINITY;
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        p[e] = s[e] * a.scale + adder[k0 + kt + acc_row(e, half)];
+        p[e] = masked ? s[e] * c2 + adder[c * CH + kt + acc_row(e, half)] : s[e] * c2;
         mt = fmaxf(mt, p[e]);
       }
       mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
       const float mn = fmaxf(m, mt);
-      const float alpha = __expf(m - mn);
+      const float alpha = exp2_fast(m - mn);
       m = mn;
       float rs = 0.f;
 #pragma unroll
-      for (int e = 0; e < 16; ++e) { p[e] = __expf(p[e] - mn); rs += p[e]; }
+      for (int e = 0; e < 16; ++e) { p[e] = exp2_fast(p[e] - mn); rs += p[e]; }
       l = l * alpha + rs;
 #pragma unroll
       for (int e = 0; e < 16; ++e) { o[0][e] *= alpha; o[1][e] *= alpha; }
@@ -205,8 +227,12 @@ __global__ __launch_bounds__(NTHREADS) void attn_fwd_kernel(AttnArgs a) {
       for (int s2 = 0; s2 < 2; ++s2) {
         const bf16x8 pf = pack8(p + 8 * s2);
 #pragma unroll
-        for (int dt = 0; dt < 2; ++dt) o[dt] = mfma(frag_cols(sv, kt + 16 * s2, dt * 32, lane), pf, o[dt]);
+        for (int dt = 0; dt < 2; ++dt) o[dt] = mfma(frag_cols(cv, kt + 16 * s2, dt * 32, lane), pf, o[dt]);
       }
+    }
+    if (c + 2 < nch) {
+      __syncthreads();  // every wave is done with this buffer
+      fill(c + 2);
     }
   }
   // combine the SPLIT partial softmaxes of each query group (part 0 always saw key step 0: m is finite)
@@ -223,14 +249,14 @@ __global__ __launch_bounds__(NTHREADS) void attn_fwd_kernel(AttnArgs a) {
     float mp, lp;
     part_xy(slot, mp, lp, lane);
     const float mn = fmaxf(m, mp);
-    const float wa = __expf(m - mn), wb = __expf(mp - mn);
+    const float wa = exp2_fast(m - mn), wb = exp2_fast(mp - mn);
     part_merge<2>(slot, o, wa, wb, lane);
     l = l * wa + lp * wb;
     m = mn;
   }
   l += __shfl_xor(l, 32, 64);
   store_t(a.ctx + ((int64_t)b * a.S + q) * a.H + hd * HD, o, 1.0f / l, half);
-  if (half == 0) a.lse[((int64_t)b * a.N + hd) * a.S + q] = m + __logf(l);
+  if (half == 0) a.lse[((int64_t)b * a.N + hd) * a.S + q] = (m + __log2f(l)) * LN2;   // natural-log lse, as backward expects
 }
 
 // ----------------------------------------------------------------------------------- backward: dQ
@@ -244,15 +270,22 @@ __global__ __launch_bounds__(NTHREADS) void attn_bwd_dq_kernel(AttnArgs a) {
   const int b = blockIdx.y / a.N, hd = blockIdx.y % a.N;
   const int q = blockIdx.x * 64 + grp * 32 + (lane & 31);
   const bf16* base = a.qkv + (int64_t)b * a.S * a.ld + hd * HD;
-  char* sk = lds;
-  char* sv = lds + CHUNK * ROWB;
-  float* adder = reinterpret_cast<float*>(lds + 2 * CHUNK * ROWB);
-  // the first K / V tiles are requested first: delta below needs its operands in registers, and waiting for them before
-  // asking for the tiles would cost a second trip to memory
-  tile_fill(sk, base + a.H, a.ld, a.S < CHUNK ? a.S : CHUNK, wave, lane);
-  tile_fill(sv, base + 2 * a.H, a.ld, a.S < CHUNK ? a.S : CHUNK, wave, lane);
-  for (int j = threadIdx.x; j < a.S; j += NTHREADS)
-    adder[j] = a.key_mask ? (1.0f - a.key_mask[(int64_t)b * a.S + j]) * a.mask_value : 0.f;
+  auto sk = [&](int c) { return lds + (c & 1) * (2 * CH * ROWB); };              // two buffers of CH rows per tensor
+  auto sv = [&](int c) { return lds + (c & 1) * (2 * CH * ROWB) + CH * ROWB; };
+  float* adder = reinterpret_cast<float*>(lds + 4 * CH * ROWB);
+  const int nch = (a.S + CH - 1) / CH;
+  auto rows_of = [&](int c) { return a.S - c * CH < CH ? a.S - c * CH : CH; };
+  auto fill = [&](int c) {
+    tile_fill(sk(c), base + a.H + (int64_t)c * CH * a.ld, a.ld, rows_of(c), wave, lane);
+    tile_fill(sv(c), base + 2 * a.H + (int64_t)c * CH * a.ld, a.ld, rows_of(c), wave, lane);
+  };
+  // the first two K / V chunks are requested first: delta below needs its operands in registers, and waiting for them
+  // before asking for the tiles would cost a second trip to memory
+  fill(0);
+  if (nch > 1) fill(1);
+  const bool masked = a.key_mask != nullptr;
+  if (masked)
+    for (int j = threadIdx.x; j < a.S; j += NTHREADS) adder[j] = (1.0f - a.key_mask[(int64_t)b * a.S + j]) * a.mask_value * LOG2E;
   bf16x8 qf[4], dof[4];
   float delta = 0.f;
   const int64_t orow = ((int64_t)b * a.S + q) * a.H + hd * HD;
@@ -265,41 +298,45 @@ __global__ __launch_bounds__(NTHREADS) void attn_bwd_dq_kernel(AttnArgs a) {
     for (int j = 0; j < 8; ++j) delta += (float)dof[ks][j] * (float)of[j];
   }
   delta += __shfl_xor(delta, 32, 64);
-  const float lse = a.lse[((int64_t)b * a.N + hd) * a.S + q];
+  const float lse2 = a.lse[((int64_t)b * a.N + hd) * a.S + q] * LOG2E;
   if (half == 0 && part == 0) a.delta[((int64_t)b * a.N + hd) * a.S + q] = delta;
   f32x16 dq[2];
 #pragma unroll
   for (int e = 0; e < 16; ++e) { dq[0][e] = 0.f; dq[1][e] = 0.f; }
-  for (int k0 = 0; k0 < a.S; k0 += CHUNK) {
-    const int rows = a.S - k0 < CHUNK ? a.S - k0 : CHUNK;
+  const float c2 = a.scale * LOG2E;
+  __builtin_amdgcn_s_waitcnt(VMCNT0);  // the loads and the store above: from here on only tile loads are in flight
+  for (int c = 0; c < nch; ++c) {
+    const int rows = rows_of(c);
+    wait_chunk(c + 1 < nch ? rows_of(c + 1) : 0);
     __syncthreads();
-    if (k0 > 0) {  // tile 0 was requested at the top
-      tile_fill(sk, base + a.H + (int64_t)k0 * a.ld, a.ld, rows, wave, lane);
-      tile_fill(sv, base + 2 * a.H + (int64_t)k0 * a.ld, a.ld, rows, wave, lane);
-    }
-    __builtin_amdgcn_s_waitcnt(VMCNT0);
-    __syncthreads();
-    for (int kt = part * 32; kt < rows; kt += 32 * SPLIT) {
+    const char* ck = sk(c);
+    const char* cv = sv(c);
+    const int kt = part * 32;
+    if (kt < rows) {
       f32x16 s, dp;
 #pragma unroll
       for (int e = 0; e < 16; ++e) { s[e] = 0.f; dp[e] = 0.f; }
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
-        s = mfma(frag_rows(sk, kt, ks, lane), qf[ks], s);     // S^T[key][q]
-        dp = mfma(frag_rows(sv, kt, ks, lane), dof[ks], dp);  // dP^T[key][q] = V dO^T
+        s = mfma(frag_rows(ck, kt, ks, lane), qf[ks], s);     // S^T[key][q]
+        dp = mfma(frag_rows(cv, kt, ks, lane), dof[ks], dp);  // dP^T[key][q] = V dO^T
       }
       float ds[16];
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const float p = __expf(s[e] * a.scale + adder[k0 + kt + acc_row(e, half)] - lse);
-        ds[e] = p * (dp[e] - delta) * a.scale;
+        const float x = masked ? s[e] * c2 + (adder[c * CH + kt + acc_row(e, half)] - lse2) : s[e] * c2 - lse2;
+        ds[e] = exp2_fast(x) * (dp[e] - delta);   // the factor `scale` is applied once, to the sums
       }
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
         const bf16x8 df = pack8(ds + 8 * s2);
 #pragma unroll
-        for (int dt = 0; dt < 2; ++dt) dq[dt] = mfma(frag_cols(sk, kt + 16 * s2, dt * 32, lane), df, dq[dt]);  // dQ^T += K^T dS^T
+        for (int dt = 0; dt < 2; ++dt) dq[dt] = mfma(frag_cols(ck, kt + 16 * s2, dt * 32, lane), df, dq[dt]);  // dQ^T += K^T dS^T
       }
+    }
+    if (c + 2 < nch) {
+      __syncthreads();  // every wave is done with this buffer
+      fill(c + 2);
     }
   }
   __syncthreads();
@@ -308,7 +345,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_bwd_dq_kernel(AttnArgs a) {
   if (part > 0) return;
 #pragma unroll
   for (int pp = 1; pp < SPLIT; ++pp) part_merge<2>(lds + ((pp - 1) * 2 + grp) * PART_BYTES, dq, 1.f, 1.f, lane);
-  store_t(a.dqkv + ((int64_t)b * a.S + q) * a.ld + hd * HD, dq, 1.0f, half);
+  store_t(a.dqkv + ((int64_t)b * a.S + q) * a.ld + hd * HD, dq, a.scale, half);
 }
 
 // ----------------------------------------------------------------------------------- backward: dK, dV
@@ -322,19 +359,25 @@ __global__ __launch_bounds__(NTHREADS) void attn_bwd_dkv_kernel(AttnArgs a) {
   const int key = blockIdx.x * 64 + grp * 32 + (lane & 31);
   const bf16* base = a.qkv + (int64_t)b * a.S * a.ld + hd * HD;
   const bf16* dobase = a.dctx + (int64_t)b * a.S * a.H + hd * HD;
-  char* sq = lds;
-  char* sdo = lds + CHUNK * ROWB;
-  float* slse = reinterpret_cast<float*>(lds + 2 * CHUNK * ROWB);
+  auto sq = [&](int c) { return lds + (c & 1) * (2 * CH * ROWB); };              // two buffers of CH rows per tensor
+  auto sdo = [&](int c) { return lds + (c & 1) * (2 * CH * ROWB) + CH * ROWB; };
+  float* slse = reinterpret_cast<float*>(lds + 4 * CH * ROWB);
   float* sdelta = slse + a.S;
-  // the first Q / dO tiles are requested first: lse and delta go through registers into LDS, and waiting for them before
-  // asking for the tiles would cost a second trip to memory
-  tile_fill(sq, base, a.ld, a.S < CHUNK ? a.S : CHUNK, wave, lane);
-  tile_fill(sdo, dobase, a.H, a.S < CHUNK ? a.S : CHUNK, wave, lane);
+  const int nch = (a.S + CH - 1) / CH;
+  auto rows_of = [&](int c) { return a.S - c * CH < CH ? a.S - c * CH : CH; };
+  auto fill = [&](int c) {
+    tile_fill(sq(c), base + (int64_t)c * CH * a.ld, a.ld, rows_of(c), wave, lane);
+    tile_fill(sdo(c), dobase + (int64_t)c * CH * a.H, a.H, rows_of(c), wave, lane);
+  };
+  // the first two Q / dO chunks are requested first: lse and delta go through registers into LDS, and waiting for them
+  // before asking for the tiles would cost a second trip to memory
+  fill(0);
+  if (nch > 1) fill(1);
   for (int j = threadIdx.x; j < a.S; j += NTHREADS) {
-    slse[j] = a.lse[((int64_t)b * a.N + hd) * a.S + j];
+    slse[j] = a.lse[((int64_t)b * a.N + hd) * a.S + j] * LOG2E;
     sdelta[j] = a.delta[((int64_t)b * a.N + hd) * a.S + j];
   }
-  const float adder = a.key_mask ? (1.0f - a.key_mask[(int64_t)b * a.S + key]) * a.mask_value : 0.f;
+  const float adder = a.key_mask ? (1.0f - a.key_mask[(int64_t)b * a.S + key]) * a.mask_value * LOG2E : 0.f;
   bf16x8 kf[4], vf[4];
 #pragma unroll
   for (int ks = 0; ks < 4; ++ks) {
@@ -344,40 +387,44 @@ __global__ __launch_bounds__(NTHREADS) void attn_bwd_dkv_kernel(AttnArgs a) {
   f32x16 dk[2], dv[2];
 #pragma unroll
   for (int e = 0; e < 16; ++e) { dk[0][e] = 0.f; dk[1][e] = 0.f; dv[0][e] = 0.f; dv[1][e] = 0.f; }
-  for (int q0 = 0; q0 < a.S; q0 += CHUNK) {
-    const int rows = a.S - q0 < CHUNK ? a.S - q0 : CHUNK;
+  const float c2 = a.scale * LOG2E;
+  __builtin_amdgcn_s_waitcnt(VMCNT0);  // the loads above: from here on only tile loads are in flight
+  for (int c = 0; c < nch; ++c) {
+    const int rows = rows_of(c);
+    wait_chunk(c + 1 < nch ? rows_of(c + 1) : 0);
     __syncthreads();
-    if (q0 > 0) {  // tile 0 was requested at the top
-      tile_fill(sq, base + (int64_t)q0 * a.ld, a.ld, rows, wave, lane);
-      tile_fill(sdo, dobase + (int64_t)q0 * a.H, a.H, rows, wave, lane);
-    }
-    __builtin_amdgcn_s_waitcnt(VMCNT0);
-    __syncthreads();
-    for (int qt = part * 32; qt < rows; qt += 32 * SPLIT) {
+    const char* cq = sq(c);
+    const char* cdo = sdo(c);
+    const int qt = part * 32;
+    if (qt < rows) {
       f32x16 s, dp;
 #pragma unroll
       for (int e = 0; e < 16; ++e) { s[e] = 0.f; dp[e] = 0.f; }
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
-        s = mfma(frag_rows(sq, qt, ks, lane), kf[ks], s);      // S[q][key]
-        dp = mfma(frag_rows(sdo, qt, ks, lane), vf[ks], dp);   // dP[q][key] = dO V^T
+        s = mfma(frag_rows(cq, qt, ks, lane), kf[ks], s);      // S[q][key]
+        dp = mfma(frag_rows(cdo, qt, ks, lane), vf[ks], dp);   // dP[q][key] = dO V^T
       }
       float p[16], ds[16];
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const int qq = q0 + qt + acc_row(e, half);
-        p[e] = __expf(s[e] * a.scale + adder - slse[qq]);
-        ds[e] = p[e] * (dp[e] - sdelta[qq]) * a.scale;
+        const int qq = c * CH + qt + acc_row(e, half);
+        p[e] = exp2_fast(s[e] * c2 + (adder - slse[qq]));
+        ds[e] = p[e] * (dp[e] - sdelta[qq]);   // the factor `scale` is applied once, to dK
       }
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
         const bf16x8 pf = pack8(p + 8 * s2), df = pack8(ds + 8 * s2);
 #pragma unroll
         for (int dt = 0; dt < 2; ++dt) {
-          dv[dt] = mfma(frag_cols(sdo, qt + 16 * s2, dt * 32, lane), pf, dv[dt]);  // dV^T += dO^T P
-          dk[dt] = mfma(frag_cols(sq, qt + 16 * s2, dt * 32, lane), df, dk[dt]);   // dK^T += Q^T dS
+          dv[dt] = mfma(frag_cols(cdo, qt + 16 * s2, dt * 32, lane), pf, dv[dt]);  // dV^T += dO^T P
+          dk[dt] = mfma(frag_cols(cq, qt + 16 * s2, dt * 32, lane), df, dk[dt]);   // dK^T += Q^T dS
         }
       }
+    }
+    if (c + 2 < nch) {
+      __syncthreads();  // every wave is done with this buffer
+      fill(c + 2);
     }
   }
   // two merge rounds through the same slots: dK, then dV
@@ -396,7 +443,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_bwd_dkv_kernel(AttnArgs a) {
 #pragma unroll
   for (int pp = 1; pp < SPLIT; ++pp) part_merge<2>(lds + ((pp - 1) * 2 + grp) * PART_BYTES, dv, 1.f, 1.f, lane);
   bf16* orow = a.dqkv + ((int64_t)b * a.S + key) * a.ld + hd * HD;
-  store_t(orow + a.H, dk, 1.0f, half);
+  store_t(orow + a.H, dk, a.scale, half);
   store_t(orow + 2 * a.H, dv, 1.0f, half);
 }
 
@@ -604,7 +651,7 @@ int check(const char* who, int dtype, int B, int N, int S, int D) {
   DS_CHECK_ARG(S <= 2048, "%s: seq %d exceeds 2048", who, S);
   return DS_OK;
 }
-size_t lds_bytes(int S) { return (size_t)2 * CHUNK * ROWB + (size_t)2 * S * sizeof(float); }
+size_t lds_bytes(int S) { return (size_t)4 * CH * ROWB + (size_t)2 * S * sizeof(float); }
 
 }  // namespace
 
