@@ -68,6 +68,22 @@ __device__ __forceinline__ void wait_chunk(int next_rows) {
   else __builtin_amdgcn_s_waitcnt(VMCNT0);
 }
 
+// The mask adders of the 16 accumulator rows of a 32-row step (rows (e/4)*8 + 4*half + e%4): four 16-byte LDS reads, or
+// zeros without a mask - one uniform branch per step instead of one per element.
+__device__ __forceinline__ void step_adders(const float* adder, bool masked, int row0, int half, float (&ad)[16]) {
+  if (masked) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const f32x4 v = *reinterpret_cast<const f32x4*>(adder + row0 + g * 8 + half * 4);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) ad[4 * g + j] = v[j];
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) ad[e] = 0.f;
+  }
+}
+
 // A operand, rows = tile rows (row0 + lane%32), k = 8 consecutive columns starting at 16*ks + 8*half
 __device__ __forceinline__ bf16x8 frag_rows(const char* lds, int row0, int ks, int lane) {
   return *reinterpret_cast<const bf16x8*>(lds + tile_off(row0 + (lane & 31), (2 * ks + (lane >> 5)) * 16));
@@ -206,11 +222,12 @@ __global__ __launch_bounds__(NTHREADS) void attn_fwd_kernel(AttnArgs a) {
       for (int e = 0; e < 16; ++e) s[e] = 0.f;
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) s = mfma(frag_rows(ck, kt, ks, lane), qf[ks], s);
-      float p[16];
+      float p[16], ad[16];
+      step_adders(adder, masked, c * CH + kt, half, ad);
       float mt = -INFINITY;
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        p[e] = masked ? s[e] * c2 + adder[c * CH + kt + acc_row(e, half)] : s[e] * c2;
+        p[e] = s[e] * c2 + ad[e];
         mt = fmaxf(mt, p[e]);
       }
       mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
@@ -321,12 +338,11 @@ __global__ __launch_bounds__(NTHREADS) void attn_bwd_dq_kernel(AttnArgs a) {
         s = mfma(frag_rows(ck, kt, ks, lane), qf[ks], s);     // S^T[key][q]
         dp = mfma(frag_rows(cv, kt, ks, lane), dof[ks], dp);  // dP^T[key][q] = V dO^T
       }
-      float ds[16];
+      float ds[16], ad[16];
+      step_adders(adder, masked, c * CH + kt, half, ad);
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const float x = masked ? s[e] * c2 + (adder[c * CH + kt + acc_row(e, half)] - lse2) : s[e] * c2 - lse2;
-        ds[e] = exp2_fast(x) * (dp[e] - delta);   // the factor `scale` is applied once, to the sums
-      }
+      for (int e = 0; e < 16; ++e)
+        ds[e] = exp2_fast(s[e] * c2 + (ad[e] - lse2)) * (dp[e] - delta);   // the factor `scale` is applied once, to the sums
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
         const bf16x8 df = pack8(ds + 8 * s2);
@@ -405,12 +421,13 @@ __global__ __launch_bounds__(NTHREADS) void attn_bwd_dkv_kernel(AttnArgs a) {
         s = mfma(frag_rows(cq, qt, ks, lane), kf[ks], s);      // S[q][key]
         dp = mfma(frag_rows(cdo, qt, ks, lane), vf[ks], dp);   // dP[q][key] = dO V^T
       }
-      float p[16], ds[16];
+      float p[16], ds[16], ls[16], dl[16];
+      step_adders(slse, true, c * CH + qt, half, ls);     // this step's 16 query rows: log-sum-exp and delta
+      step_adders(sdelta, true, c * CH + qt, half, dl);
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const int qq = c * CH + qt + acc_row(e, half);
-        p[e] = exp2_fast(s[e] * c2 + (adder - slse[qq]));
-        ds[e] = p[e] * (dp[e] - sdelta[qq]);   // the factor `scale` is applied once, to dK
+        p[e] = exp2_fast(s[e] * c2 + (adder - ls[e]));
+        ds[e] = p[e] * (dp[e] - dl[e]);   // the factor `scale` is applied once, to dK
       }
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
