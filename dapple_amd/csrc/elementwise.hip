@@ -266,7 +266,8 @@ template <int NG>
 __global__ __launch_bounds__(256) void layernorm_fwd_mixed_kernel(int rows, int cols, const float* __restrict__ x,
                                                                  const float* __restrict__ gamma, const float* __restrict__ beta,
                                                                  float eps, bf16* __restrict__ y16, float* __restrict__ y32,
-                                                                 float* __restrict__ stats) {
+                                                                 float* __restrict__ stats, int prio) {
+  ds_wave_prio(prio);
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
@@ -422,7 +423,8 @@ template <int NG>
 __global__ __launch_bounds__(256) void layernorm_bwd_mixed_rows_kernel(int rows, int cols, const float* __restrict__ dy,
                                                                       const float* __restrict__ x, const float* __restrict__ gamma,
                                                                       const float* __restrict__ stats, bf16* __restrict__ dx16,
-                                                                      float* __restrict__ dx32, bf16* __restrict__ dy16) {
+                                                                      float* __restrict__ dx32, bf16* __restrict__ dy16, int prio) {
+  ds_wave_prio(prio);
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
@@ -947,7 +949,7 @@ extern "C" int ds_layernorm_fwd_mixed(int rows, int cols, const float* x, const 
   const int need = (cols / 8 + 63) / 64;
   ds_prof_scope prof(s, "layernorm_fwd_mixed_kernel", (double)rows * cols * (4 + 2 + (y_f32 ? 4 : 0)), "B");
   DISPATCH_NG(need, hipLaunchKernelGGL((layernorm_fwd_mixed_kernel<NG>), dim3((rows + 3) / 4), dim3(256), 0, s, rows, cols, x, gamma, beta,
-                                       eps, (bf16*)y_bf16, y_f32, stats));
+                                       eps, (bf16*)y_bf16, y_f32, stats, ds_launch_prio));
   DS_CHECK_LAUNCH();
   return DS_OK;
 }
@@ -966,7 +968,7 @@ extern "C" int ds_layernorm_bwd_mixed(int rows, int cols, const float* dy, const
     ds_prof_scope prof(s, "layernorm_bwd_mixed_rows_kernel",
                        (double)rows * cols * (4 + 4 + 2 + (dx_f32 ? 4 : 0) + (dy_bf16 ? 2 : 0)), "B");
     DISPATCH_NG(need, hipLaunchKernelGGL((layernorm_bwd_mixed_rows_kernel<NG>), dim3((rows + 3) / 4), dim3(256), 0, s, rows, cols, dy, x,
-                                         gamma, stats, (bf16*)dx_bf16, dx_f32, (bf16*)dy_bf16));
+                                         gamma, stats, (bf16*)dx_bf16, dx_f32, (bf16*)dy_bf16, ds_launch_prio));
     DS_CHECK_LAUNCH();
     return DS_OK;
   }
