@@ -182,6 +182,9 @@ def load():
     if not os.path.exists(LIB_PATH):
         raise DappleError("%s not found: build it with `python -m dapple_amd.build` "
                           "(there is no CPU fallback)" % LIB_PATH)
+    # torch first: it ships its own copy of the HIP runtime, and the library's dependency on libamdhip64 must resolve to the
+    # copy torch has loaded - a process with two HIP runtimes sees "no ROCm-capable device" in the second one
+    import torch  # noqa: F401
     lib = C.CDLL(LIB_PATH)
     for name, (res, args) in PROTOTYPES.items():
         fn = getattr(lib, name)          # AttributeError if the symbol is missing
