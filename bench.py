@@ -125,6 +125,65 @@ def make_vgg(c, args):
     return wl
 
 
+def make_vgg_last(c, args):
+    """The last device of the sliced VGG19 (K = 1): conv tail, classification block, loss, backward down to the boundary."""
+    import numpy as np
+    import torch
+    from dapple_amd import ops, runtime, synthetic
+    B, M, layers = c["micro_batch"], c["num_micro_batches"], c["layers"]
+    Hh, Ww, Cin, FC, CL = c["height"], c["width"], c["in_channels"], c["fc"], c["classes"]
+    stage = runtime.vgg_stage(layers, B, Hh, Ww, Cin, stash_slots=1, need_input_grad=True)
+    stage.bind(synthetic.vgg_weights(synthetic.SEED_WEIGHT + c["index"], layers, Cin))
+    feat = 1
+    for d in stage.out_shape[1:]:
+        feat *= d
+    hw = {k: torch.as_tensor(v).cuda() for k, v in synthetic.vgg_head_weights(synthetic.SEED_WEIGHT + c["index"] + 1, feat, FC, CL).items()}
+    hg = {k: torch.zeros_like(v) for k, v in hw.items()}
+    r = np.random.Generator(np.random.PCG64(synthetic.SEED_INPUT + c["index"]))
+    xs = [torch.as_tensor(np.abs(r.standard_normal((B, Hh, Ww, Cin))).astype(np.float32)).cuda() for _ in range(M)]
+    labels = [torch.as_tensor(r.integers(0, CL, B).astype(np.float32)).cuda() for _ in range(M)]
+    y = torch.empty(stage.out_shape, device="cuda")
+    dxs = [torch.empty(B, Hh, Ww, Cin, device="cuda") for _ in range(M)]
+
+    def step():
+        stage.refresh_weights(); stage.zero_grads()
+        for g in hg.values():
+            g.zero_()
+        for j in range(M):
+            stage.forward(0, xs[j], y)
+            _, _, dy = ops.vgg_head(y.reshape(B, feat), hw, labels[j], grads=hg, loss_mode="sparse_ce")
+            stage.backward(0, dy.reshape(stage.out_shape), dxs[j])
+    wl = Workload()
+    wl.stage = stage
+    wl.step = step
+    wl.samples = B * M
+    macs, h, w_, cin = 0, Hh, Ww, Cin
+    for _, cout in layers:
+        if cout is None:
+            h, w_ = h // 2, w_ // 2
+        else:
+            macs += h * w_ * 9 * cin * cout
+            cin = cout
+    wl.flops_per_sample = 2 * 3 * (macs + feat * FC + FC * FC + FC * CL)
+    wl.config = {"convs": sum(1 for _, c_ in layers if c_), "boundary": [Hh, Ww, Cin], "fc": FC, "classes": CL, "micro_batch": B,
+                 "micro_batches": M, "loss": "sparse cross entropy",
+                 "schedule": "last stage (K=1): forward, classification block + loss, backward per micro-batch"}
+
+    def cpu():
+        from oracle import vgg as ov
+        nb = 8
+        w = ov.to_torch({**synthetic.vgg_weights(synthetic.SEED_WEIGHT + c["index"], layers, Cin),
+                         **{k: v.cpu().numpy() for k, v in hw.items()}}, torch.float32, requires_grad=True)
+        x = xs[0][:nb].cpu().requires_grad_(True)
+        t0 = time.perf_counter()
+        loss = ov.head_loss(ov.head_forward(ov.stage_forward(x, w, layers).reshape(nb, -1), w), labels[0][:nb].cpu(), "sparse_ce")
+        torch.autograd.grad(loss, [x] + list(w.values()))
+        dt = time.perf_counter() - t0
+        return dt, nb, "%d of %d images of one micro-batch, conv tail + classification block + loss, fwd+bwd" % (nb, B)
+    wl.cpu = cpu
+    return wl
+
+
 def make_gnmt(c, args):
     import torch
     from dapple_amd import runtime, synthetic
@@ -330,7 +389,7 @@ def traffic_of(tag, workload, wgrad_group):
     return sum(r[3] + r[4] for r in rows) / len(rows)
 
 
-MAKERS = {"bert": make_bert, "vgg": make_vgg, "gnmt": make_gnmt, "xlnet": make_xlnet, "gnmt_attention": make_gnmt_attention,
+MAKERS = {"bert": make_bert, "vgg": make_vgg, "vgg_last": make_vgg_last, "gnmt": make_gnmt, "xlnet": make_xlnet, "gnmt_attention": make_gnmt_attention,
           "gnmt_decoder": make_gnmt_decoder}
 METRIC = {"bert48_half": "stage samples/sec fwd+bwd+grad-accum, BERT-48 half-stage; MFMA util %"}
 

@@ -256,6 +256,10 @@ CONFIGS = {
     # BASELINE configs[1]: VGG19 conv stack (stage 0 of the 15:1 split, widened to conv5_4)
     "vgg19_stage0": dict(index=1, kind="vgg", layers=VGG19_CONV_STACK, height=224, width=224, in_channels=3,
                          micro_batch=32, num_micro_batches=4, dtype="fp32"),
+    # VGG19's last device in the 15:1 split (not a BASELINE configuration: a last-stage row): block5_conv3, block5_conv4,
+    # block5_pool on the concatenated boundary activation, then flatten, fc1, fc2, predictions and the loss
+    "vgg19_last_device": dict(index=7, kind="vgg_last", layers=VGG19_STAGE1_15_1, height=14, width=14, in_channels=512,
+                              fc=4096, classes=1000, micro_batch=32, num_micro_batches=4, dtype="fp32"),
     # BASELINE configs[2]: GNMT-16 encoder stage (8 LSTM layers, the first bidirectional)
     "gnmt16_encoder": dict(index=2, kind="gnmt", num_layers=8, units=1024, vocab=32000, seq=50, micro_batch=64,
                            num_micro_batches=4, dtype="fp32", forget_bias=1.0),
