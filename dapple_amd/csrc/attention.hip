@@ -124,6 +124,20 @@ struct AttnArgs {
   int prio;                      // wave priority (0..3)
 };
 
+// Which (batch, head) pair and which 64-row block of the parallel axis a workgroup takes.  Workgroups go to the 8 XCDs
+// round-robin in launch order (grid x fastest), and the XCDs' L2s are private: with the plain mapping the S/64 blocks of one
+// head land on 8 different XCDs and every one of them fetches that head's K and V (or Q and dO) from memory.  Here the
+// workgroups of one XCD (equal launch index mod 8) take whole heads, one after the other, so a head's tiles are fetched
+// into one L2 once and its other blocks hit there.
+__device__ __forceinline__ void attn_block_map(int& bh, int& blk) {
+  const int nb = gridDim.x, nbh = gridDim.y;
+  if (nbh % 8 != 0) { bh = blockIdx.y; blk = blockIdx.x; return; }
+  const int id = blockIdx.x + nb * blockIdx.y;
+  const int xcd = id & 7, k = id >> 3;
+  bh = (k / nb) * 8 + xcd;
+  blk = k % nb;
+}
+
 // store a transposed 64 x 32 accumulator pair (rows d, columns = this lane's row index) as out[row][d]
 __device__ __forceinline__ void store_t(bf16* out_row, const f32x16 (&acc)[2], float mul, int half) {
 #pragma unroll
@@ -180,8 +194,10 @@ __global__ __launch_bounds__(NTHREADS) void attn_fwd_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5;
   const int grp = wave & 1, part = wave >> 1;
-  const int b = blockIdx.y / a.N, hd = blockIdx.y % a.N;
-  const int q = blockIdx.x * 64 + grp * 32 + (lane & 31);
+  int bh, blk;
+  attn_block_map(bh, blk);
+  const int b = bh / a.N, hd = bh % a.N;
+  const int q = blk * 64 + grp * 32 + (lane & 31);
   const bf16* base = a.qkv + (int64_t)b * a.S * a.ld + hd * HD;
   auto sk = [&](int c) { return lds + (c & 1) * (2 * CH * ROWB); };              // two buffers of CH rows per tensor
   auto sv = [&](int c) { return lds + (c & 1) * (2 * CH * ROWB) + CH * ROWB; };
@@ -284,8 +300,10 @@ __global__ __launch_bounds__(NTHREADS) void attn_bwd_dq_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5;
   const int grp = wave & 1, part = wave >> 1;
-  const int b = blockIdx.y / a.N, hd = blockIdx.y % a.N;
-  const int q = blockIdx.x * 64 + grp * 32 + (lane & 31);
+  int bh, blk;
+  attn_block_map(bh, blk);
+  const int b = bh / a.N, hd = bh % a.N;
+  const int q = blk * 64 + grp * 32 + (lane & 31);
   const bf16* base = a.qkv + (int64_t)b * a.S * a.ld + hd * HD;
   auto sk = [&](int c) { return lds + (c & 1) * (2 * CH * ROWB); };              // two buffers of CH rows per tensor
   auto sv = [&](int c) { return lds + (c & 1) * (2 * CH * ROWB) + CH * ROWB; };
@@ -371,8 +389,10 @@ __global__ __launch_bounds__(NTHREADS) void attn_bwd_dkv_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5;
   const int grp = wave & 1, part = wave >> 1;
-  const int b = blockIdx.y / a.N, hd = blockIdx.y % a.N;
-  const int key = blockIdx.x * 64 + grp * 32 + (lane & 31);
+  int bh, blk;
+  attn_block_map(bh, blk);
+  const int b = bh / a.N, hd = bh % a.N;
+  const int key = blk * 64 + grp * 32 + (lane & 31);
   const bf16* base = a.qkv + (int64_t)b * a.S * a.ld + hd * HD;
   const bf16* dobase = a.dctx + (int64_t)b * a.S * a.H + hd * HD;
   auto sq = [&](int c) { return lds + (c & 1) * (2 * CH * ROWB); };              // two buffers of CH rows per tensor
