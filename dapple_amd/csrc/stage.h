@@ -133,6 +133,34 @@ struct XlAttnArgs {
 // true when the shapes fit the kernel (head size 64, Q a multiple of 64, K a multiple of 32, R = K + Q)
 bool ds_xl_attention_fits(int dtype, int head_dim, int Q, int K, int R);
 int ds_xl_attention_fwd(const XlAttnArgs* a, hipStream_t stream);
+// Scores + softmax of XLNet's relative attention with nothing but bf16 probabilities (forward) or bf16 score gradients
+// (backward) leaving the kernel (attention_xl.hip); operands as in XlAttnArgs.
+struct XlScoreArgs {
+  const void *qw, *qr, *qs;   // bf16 [QQ][B][H]: q + the three biases; row stride ldq, sample b at column b*H
+  int64_t ldq;
+  const void* k;              // bf16 key rows: row stride ldk, sample b at column b*ldk_b, head n at column n*64
+  const void* v;              // bf16 value rows, strides of k (backward)
+  int64_t ldk, ldk_b;
+  const void* kr;             // bf16 [R][H]; row stride ldkr
+  int64_t ldkr;
+  const float* seg_emb;       // fp32 [2][H]
+  const void* meta;           // mask / segment bits packed by ds_xl_pack_meta, or null (no mask, one segment)
+  const float* nseg;          // fp32 [B][Q]: keys of the other segment per query row, or null (backward)
+  void* p;                    // bf16 [B*N][QQ][K]: written by forward, read by backward
+  const void* dvec;           // bf16, layout of qw: gradient of the attention vector (backward)
+  void* ds;                   // bf16 [B*N][QQ][K] (backward out)
+  void* dbd;                  // bf16 [B*N][QQ][R]: ds un-shifted; only the band is written (backward out)
+  float* defs;                // fp32 [B*N][QQ][2] (backward out)
+  int Q, QQ, K, R, B, N, H;
+  float scale;
+};
+// bf16, head size 64, Q and K multiples of 32, K <= 1024, R = K + Q
+bool ds_xl_scores_fit(int dtype, int head_dim, int Q, int K, int R);
+size_t ds_xl_meta_bytes(int QQ, int K, int B);
+// mask fp32 [QQ][K][B] (non-zero = masked) and seg uint8 [Q][K][B], either may be null -> meta; nseg (may be null) <- seg
+int ds_xl_pack_meta(int Q, int QQ, int K, int B, const float* mask, const uint8_t* seg, void* meta, float* nseg, hipStream_t stream);
+int ds_xl_scores_fwd(const XlScoreArgs* a, hipStream_t stream);
+int ds_xl_scores_bwd(const XlScoreArgs* a, hipStream_t stream);
 int ds_gemm_splitk(const ds_gemm_desc* d, int splitk, void* stream);
 // ds_colsum_accum for up to 4 matrices of one shape in one launch
 int ds_colsum_accum_multi(int dtype, int rows, int cols, int count, const void* const* xs, int64_t ldx, float* const* outs, void* stream);

@@ -221,14 +221,17 @@ struct XlnetStage : ds_stage {
   char* pe = nullptr;
   // stash
   char* stash_base = nullptr;
-  size_t slot_bytes = 0, mask_off = 0, seg_off = 0, mem_off = 0, maskt_off = 0, segt_off = 0;
+  size_t slot_bytes = 0, mask_off = 0, seg_off = 0, mem_off = 0, maskt_off = 0, segt_off = 0, meta_off = 0, nseg_off = 0;
   bool fused_fwd = false;  // forward attention in one kernel (bf16, head size 64, seq a multiple of 64)
+  // scores + softmax (forward) and score gradients (backward) in one kernel each, no fp32 score matrices (attention_xl.hip)
+  bool score_fused = false;
   // bf16 with xc.residual_fp32: the residual stream (the sums in front of both LayerNorms, the LayerNorm outputs that feed
   // the next sum, and the same chain of gradients in backward) stays in fp32; bf16 is only what a GEMM reads
   bool rs32 = false;
   size_t fw_xf[2] = {0, 0}, fw_y1f = 0, bw_dxf[2] = {0, 0}, bw_dz2f = 0, bw_dy1f = 0, bw_dz1f = 0;
   std::vector<LayerOff> lo;
   std::vector<char> has_mask, has_seg;
+  // (the packed mask / segment bits of a slot are valid when it has either)
   // workspace
   char* ws_base = nullptr;
   // buffers the weight-gradient kernels read alternate by layer parity ([2])
@@ -290,11 +293,16 @@ struct XlnetStage : ds_stage {
     mask_off = sa.reserve((size_t)S * Q * K * B * 4);
     seg_off = sa.reserve((size_t)Q * K * B);
     mem_off = sa.reserve((size_t)L * (Mm > 0 ? Mm : 1) * B * H * esz);
-    fused_fwd = xc.fused_attention != 0 && ds_xl_attention_fits(dtype, D, Q, K, R);
+    fused_fwd = xc.fused_attention == DS_XL_ATTN_ONE_KERNEL && ds_xl_attention_fits(dtype, D, Q, K, R);
+    score_fused = xc.fused_attention != DS_XL_ATTN_SEPARATE && ds_xl_scores_fit(dtype, D, Q, K, R);
     rs32 = dtype == DS_BF16 && xc.residual_fp32 != 0 && H % 8 == 0 && H <= 2048;
     if (fused_fwd) {
       maskt_off = sa.reserve((size_t)B * K * S * Q * 4);
       segt_off = sa.reserve((size_t)B * K * Q);
+    }
+    if (score_fused) {
+      meta_off = sa.reserve(ds_xl_meta_bytes(S * Q, K, B));
+      nseg_off = sa.reserve((size_t)Q * B * 4);
     }
     lo.resize(L);
     size_t next_x = sa.reserve(act);
@@ -318,9 +326,10 @@ struct XlnetStage : ds_stage {
     Arena w;
     ws_qall = w.reserve(act);
     const size_t QQ = (size_t)S * Q;  // the streams' query rows stacked: one product / one softmax launch for all of them
-    ws_ac = w.reserve((size_t)B * N * QQ * K * 4);
-    ws_dp = w.reserve((size_t)B * N * QQ * K * 4);  // backward's own score-gradient buffer: forward keeps ws_ac
-    ws_bd = w.reserve((size_t)B * N * QQ * R * 4);
+    // fp32 scores: only the path of separate products and softmax launches has them
+    ws_ac = w.reserve(score_fused ? 256 : (size_t)B * N * QQ * K * 4);
+    ws_dp = w.reserve(score_fused ? 256 : (size_t)B * N * QQ * K * 4);  // backward's own score-gradient buffer: forward keeps ws_ac
+    ws_bd = w.reserve(score_fused ? 256 : (size_t)B * N * QQ * R * 4);
     ws_ds = w.reserve((size_t)B * N * QQ * K * esz);
     ws_dbd[0] = w.reserve((size_t)B * N * QQ * R * esz);  // read by the weight-gradient stream too (dkr): one per layer parity
     ws_dbd[1] = w.reserve((size_t)B * N * QQ * R * esz);
@@ -450,6 +459,9 @@ struct XlnetStage : ds_stage {
     }
     has_mask[slot] = masks != nullptr;
     has_seg[slot] = seg_mat != nullptr;
+    if (score_fused && (masks || seg_mat))
+      DS_PROPAGATE(ds_xl_pack_meta(Q, S * Q, K, B, masks ? (const float*)(sp + mask_off) : nullptr,
+                                   seg_mat ? (const uint8_t*)(sp + seg_off) : nullptr, sp + meta_off, (float*)(sp + nseg_off), stream));
     if (fused_fwd) {
       if (masks) {
         const int64_t n = (int64_t)S * Q * K * B;
@@ -541,6 +553,21 @@ struct XlnetStage : ds_stage {
         xa.p = sp + t.p; xa.vec = sp + t.vec;
         xa.Q = Q; xa.QQ = S * Q; xa.K = K; xa.R = R; xa.B = B; xa.N = N; xa.H = H; xa.scale = scale;
         DS_PROPAGATE(ds_xl_attention_fwd(&xa, stream));
+      } else if (score_fused) {
+        const int QQ = S * Q;
+        XlScoreArgs xa;
+        memset(&xa, 0, sizeof(xa));
+        xa.qw = sp + t.qw; xa.qr = sp + t.qr; xa.qs = sp + t.qs; xa.ldq = (int64_t)B * H;
+        xa.k = sp + t.kv; xa.ldk = (int64_t)B * 2 * H; xa.ldk_b = 2 * H;
+        xa.kr = kr[l]; xa.ldkr = H;
+        xa.seg_emb = w[b + X_SEG];
+        xa.meta = (has_mask[slot] || has_seg[slot]) ? sp + meta_off : nullptr;
+        xa.p = sp + t.p;
+        xa.Q = Q; xa.QQ = QQ; xa.K = K; xa.R = R; xa.B = B; xa.N = N; xa.H = H; xa.scale = scale;
+        DS_PROPAGATE(ds_xl_scores_fwd(&xa, stream));
+        // vec = P v
+        DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_MN_MAJOR, QQ, D, K, sp + t.p, K, (int64_t)N * QQ * K, (int64_t)QQ * K, sp + t.kv + (size_t)H * esz,
+                             (int64_t)B * 2 * H, 2 * H, D, sp + t.vec, (int64_t)B * H, H, D, 0));
       } else {
         // The streams' query rows are stacked in the q buffers ([stream][i][b] = row stream*Q + i of stride B*H): every
         // product below and the softmax run once over all QQ = S*Q rows; probabilities are stashed as [B*N][QQ][K].
@@ -639,14 +666,26 @@ struct XlnetStage : ds_stage {
         // k_r receive fall out of the longer reductions
         const int QQ = S * Q;
         const char* p = sp + t.p;
-        // dP = dvec v^T ; dv = P^T dvec
-        DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_K_MAJOR, QQ, K, D, dvec, (int64_t)B * H, H, D, sp + t.kv + (size_t)H * esz, (int64_t)B * 2 * H,
-                             2 * H, D, dp, K, (int64_t)N * QQ * K, (int64_t)QQ * K, DS_EPI_OUT_F32));
+        // dP = dvec v^T (inside the score-gradient kernel where that one runs) ; dv = P^T dvec
+        if (!score_fused)
+          DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_K_MAJOR, QQ, K, D, dvec, (int64_t)B * H, H, D, sp + t.kv + (size_t)H * esz, (int64_t)B * 2 * H,
+                               2 * H, D, dp, K, (int64_t)N * QQ * K, (int64_t)QQ * K, DS_EPI_OUT_F32));
         DS_PROPAGATE(gemm_bn(DS_MN_MAJOR, DS_MN_MAJOR, K, D, QQ, p, K, (int64_t)N * QQ * K, (int64_t)QQ * K, dvec, (int64_t)B * H, H, D,
                              dkv + (size_t)H * esz, (int64_t)B * 2 * H, 2 * H, D, 0));
         // dS, its un-shifted copy for the position term (dbd[i][r] = dS[i][r - Q + i]) and the segment sums, in one pass
         float* defs = (float*)(ws_base + ws_def);
-        if (dtype == DS_BF16) DS_PROPAGATE(softmax_bwd_t<bf16>((const bf16*)p, dp, scale, seg, (bf16*)dsm, (bf16*)dbd, defs));
+        if (score_fused) {
+          XlScoreArgs xa;
+          memset(&xa, 0, sizeof(xa));
+          xa.ldq = (int64_t)B * H;
+          xa.v = sp + t.kv + (size_t)H * esz; xa.ldk = (int64_t)B * 2 * H; xa.ldk_b = 2 * H;
+          xa.ldkr = H;
+          xa.meta = (has_mask[slot] || has_seg[slot]) ? sp + meta_off : nullptr;
+          xa.nseg = has_seg[slot] ? (const float*)(sp + nseg_off) : nullptr;
+          xa.p = (void*)p; xa.dvec = dvec; xa.ds = dsm; xa.dbd = dbd; xa.defs = defs;
+          xa.Q = Q; xa.QQ = QQ; xa.K = K; xa.R = R; xa.B = B; xa.N = N; xa.H = H; xa.scale = scale;
+          DS_PROPAGATE(ds_xl_scores_bwd(&xa, stream));
+        } else if (dtype == DS_BF16) DS_PROPAGATE(softmax_bwd_t<bf16>((const bf16*)p, dp, scale, seg, (bf16*)dsm, (bf16*)dbd, defs));
         else DS_PROPAGATE(softmax_bwd_t<float>((const float*)p, dp, scale, seg, (float*)dsm, (float*)dbd, defs));
         // content term: dqw = dS k ; dk = dS^T qw
         DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_MN_MAJOR, QQ, D, K, dsm, K, (int64_t)N * QQ * K, (int64_t)QQ * K, sp + t.kv, (int64_t)B * 2 * H, 2 * H, D,

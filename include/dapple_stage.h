@@ -379,6 +379,7 @@ int ds_gnmt_stage_set_decoder_inputs(ds_stage* h, int slot, const int32_t* targe
  * seg_emb ([2, hidden]), attn_ln/{gamma,beta}, ff/{W1,b1,W2,b2}, ff_ln/{gamma,beta}.
  * mem_len > 0 and streams == 2 go beyond what the reference builds (it hard-wires memory length 0 and has
  * the content stream only, lambda_funcs.py:20,36) and follow the XLNet formulation. */
+enum { DS_XL_ATTN_AUTO = 0, DS_XL_ATTN_ONE_KERNEL = 1, DS_XL_ATTN_SEPARATE = 2 };
 typedef struct ds_xlnet_cfg {
   int dtype;
   int num_layers, hidden, heads, ffn;
@@ -386,9 +387,15 @@ typedef struct ds_xlnet_cfg {
   float ln_eps;     /* 1e-14 = K.epsilon()**2 (layer_normalization.py:37-39) */
   int first_layer;  /* names only */
   int stash_slots;
-  int fused_attention; /* 1: forward attention in one kernel where the shape allows (bf16, head size 64, seq a multiple of
-                          64, mem_len + seq a multiple of 32); 0 (default): products and softmax as separate launches,
-                          which is the faster step at the benchmark shape today.  Results agree to rounding. */
+  int fused_attention; /* how the attention scores are computed; results agree to rounding:
+                          DS_XL_ATTN_AUTO (0): where the shape allows (bf16, head size 64, seq and mem_len + seq multiples
+                            of 32, mem_len + seq <= 1024) scores, relative shift and softmax are one kernel forward and one
+                            backward, and no fp32 score matrix exists; masks then count as 0 / non-zero.  Other shapes run
+                            as DS_XL_ATTN_SEPARATE.
+                          DS_XL_ATTN_ONE_KERNEL (1): the forward pass also multiplies by v in the same kernel (seq a
+                            multiple of 64); slower in the step at the benchmark shape.
+                          DS_XL_ATTN_SEPARATE (2): every product and the softmax as launches of their own, fp32 scores
+                            in the workspace. */
   int residual_fp32;   /* bf16 only, 1: the residual stream (the sums in front of both LayerNorms, the LayerNorm outputs that
                           feed the next sum, the same chain of gradients) stays in fp32, bf16 is what the GEMMs read: the
                           stream's own rounding no longer adds up over the layers (as ds_stage_cfg.residual_fp32) */

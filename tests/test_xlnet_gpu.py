@@ -125,6 +125,21 @@ def test_fused_forward_attention_shapes(Q, Mm, S, B, mask_kind, use_seg):
              fused=True)
 
 
+@pytest.mark.parametrize("Q,Mm,S,B,mask_kind,use_seg", [(32, 0, 1, 4, "input", True), (64, 32, 2, 2, "perm", True),
+                                                         (32, 96, 2, 1, "perm", False), (96, 160, 1, 2, None, True),
+                                                         (64, 576, 2, 1, "perm", True), (64, 0, 1, 2, None, False)])
+def test_score_kernels_shapes(Q, Mm, S, B, mask_kind, use_seg):
+    # the default path for bf16, head size 64 and seq, mem_len + seq multiples of 32: scores, relative shift and softmax in one
+    # kernel per pass, 32 query rows and all keys per block.  Key counts 32 .. 640 give blocks of one to five waves, waves with
+    # one to four key tiles, a second stream, rows whose every key is masked (permutation masks), no masks / one segment (no
+    # packed bits at all)
+    run_case("bf16", L=2, H=128, N=2, F=256, B=B, Q=Q, Mm=Mm, S=S, M=2, K=1, seed=31 + Q + Mm, use_seg=use_seg, mask_kind=mask_kind)
+
+
+def test_separate_launches_at_a_shape_the_score_kernels_take():
+    run_case("bf16", L=2, H=128, N=2, F=256, B=2, Q=64, Mm=32, S=2, M=2, K=1, seed=5, fused="separate")
+
+
 def test_fused_forward_attention_config4_shape():
     c = synthetic.CONFIGS["xlnet36_half"]
     run_case("bf16", 1, c["hidden"], c["heads"], c["ffn"], c["micro_batch"], c["seq"], c["mem_len"], c["streams"], M=1, K=1,
