@@ -315,7 +315,7 @@ def make_xlnet(c, args):
     adt = torch.bfloat16 if c["dtype"] == "bf16" else torch.float32
     K = runtime.stash_depth(0, 2)
     stage = runtime.xlnet_stage(L, H, N, F, B, Q, c["dtype"], stash_slots=K, mem_len=Mm, streams=S,
-                                fused_attention=args.xlnet_attention, residual_fp32=not args.bf16_residual_stream)
+                                attention=args.xlnet_attention, residual_fp32=not args.bf16_residual_stream)
     stage.bind(synthetic.xlnet_weights(synthetic.SEED_WEIGHT + c["index"], L, H, N, F))
     xs = [torch.as_tensor(np.stack(x)).cuda().to(adt) for x in synthetic.xlnet_stream_inputs(synthetic.SEED_INPUT + c["index"], M, Q, B, H, S)]
     dys = [torch.as_tensor(np.stack(x)).cuda().to(adt) for x in synthetic.xlnet_stream_inputs(synthetic.SEED_GRAD + c["index"], M, Q, B, H, S)]
@@ -406,7 +406,7 @@ def main():
                     help="BERT / XLNet bf16 workloads: round the residual stream to bf16 too (faster, twice the error at full depth)")
     ap.add_argument("--wgrad-group", type=int, default=4,
                     help="BERT stages: weight gradients of this many backward passes in one GEMM per weight")
-    ap.add_argument("--xlnet-attention", choices=["auto", "one_kernel", "separate"], default="auto",
+    ap.add_argument("--xlnet-attention", choices=["auto", "separate"], default="auto",
                     help="XLNet stages: how the attention scores run (ds_xlnet_cfg.fused_attention)")
     ap.add_argument("--micro-batch", type=int, default=None,
                     help="samples per micro-batch instead of the configuration's (a what-if: the headline is the default)")

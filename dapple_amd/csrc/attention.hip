@@ -484,203 +484,6 @@ __global__ __launch_bounds__(NTHREADS) void attn_bwd_dkv_kernel(AttnArgs a) {
   store_t(orow + 2 * a.H, dv, 1.0f, half);
 }
 
-// ----------------------------------------------------------------------------------- XLNet relative attention, forward
-// Same accumulator layout as attn_fwd_kernel (keys down the registers, queries across the lanes).  The position
-// term needs, for query i and key j, row j + Q - i of the projected position embeddings kr: for a 32 x 32 step that is
-// a 63-row window, so the step multiplies the 64 window rows by the queries (T[r'][q], two accumulators) and picks
-// T[jl + 31 - il][il] - a shift of the register index that differs per lane.  Registers cannot be indexed per lane:
-// the wave parks T in a private LDS block laid out [query][r'] and reads it back along the diagonal (row stride 68
-// floats: 16-byte aligned vector writes, and 32 lanes reading at stride 67 hit 32 different banks).
-// Pass 1 walks the keys with the online softmax and accumulates P V; pass 2 walks them again to write the
-// normalised probabilities the backward pass reads.  Masks and segment flags come key-major so that a load
-// instruction (one key, 32 queries) reads contiguous memory.
-constexpr int XCHUNK = 128;                     // keys resident in LDS at a time
-constexpr int XKR_ROWS = XCHUNK + 64;           // window rows of kr for 64 queries x XCHUNK keys
-constexpr int XW_LD = 68;                       // floats per row of a wave's skew block
-constexpr int XW_BYTES = 32 * XW_LD * 4;
-constexpr int X_SV = XCHUNK * ROWB;
-constexpr int X_SKR = 2 * XCHUNK * ROWB;
-constexpr int X_SCR = X_SKR + XKR_ROWS * ROWB;
-constexpr int X_LSE = X_SCR + NWAVES * XW_BYTES;
-constexpr int X_LDS_BYTES = X_LSE + 64 * 4;
-static_assert((SPLIT - 1) * 2 * PART_BYTES <= X_SCR, "merge slots must fit in the tile region");
-static_assert(XCHUNK == 32 * SPLIT, "every wave takes one 32-key step per chunk");
-
-// rows r0 .. r0 + rows - 1 of kr (clamped to [0, R)) -> tile rows 0 .. rows - 1
-__device__ __forceinline__ void xl_fill_kr(char* lds, const bf16* src, int64_t ld, int r0, int rows, int R, int wave, int lane) {
-  for (int c = wave; c < rows / 8; c += NWAVES) {
-    const int p = c * 64 + lane;
-    const int r = p >> 3, pc = p & 7;
-    int gr = r0 + r;
-    gr = gr < 0 ? 0 : (gr >= R ? R - 1 : gr);
-    const bf16* s = src + (int64_t)gr * ld + (pc ^ tile_swz(r)) * 8;
-    __builtin_amdgcn_global_load_lds((glb_vptr)s, (lds_vptr)(lds + c * 1024), 16, 0, 0);
-  }
-}
-
-// scaled, masked scores of one 32-key step for this lane's query: sc[e] belongs to key j0 + acc_row(e, half)
-__device__ __forceinline__ void xl_step_scores(const XlAttnArgs& a, const char* sk, const char* skr, float* W, const bf16x8 (&qwf)[4],
-                                               const bf16x8 (&qrf)[4], int kt, int rb, int lane, int b, int qrow, int i, int j0, float e0,
-                                               float e1, float (&sc)[16]) {
-  const int half = lane >> 5, il = lane & 31;
-  f32x16 s, t0, t1;
-#pragma unroll
-  for (int e = 0; e < 16; ++e) { s[e] = 0.f; t0[e] = 0.f; t1[e] = 0.f; }
-#pragma unroll
-  for (int ks = 0; ks < 4; ++ks) {
-    s = mfma(frag_rows(sk, kt, ks, lane), qwf[ks], s);
-    t0 = mfma(frag_rows(skr, rb, ks, lane), qrf[ks], t0);
-    t1 = mfma(frag_rows(skr, rb + 32, ks, lane), qrf[ks], t1);
-  }
-  float* wr = W + il * XW_LD + half * 4;
-#pragma unroll
-  for (int g = 0; g < 4; ++g) {
-    const f32x4 v0 = {t0[4 * g], t0[4 * g + 1], t0[4 * g + 2], t0[4 * g + 3]};
-    const f32x4 v1 = {t1[4 * g], t1[4 * g + 1], t1[4 * g + 2], t1[4 * g + 3]};
-    *reinterpret_cast<f32x4*>(wr + g * 8) = v0;
-    *reinterpret_cast<f32x4*>(wr + 32 + g * 8) = v1;
-  }
-  __builtin_amdgcn_wave_barrier();  // the block is this wave's own: its LDS operations complete in order
-  const float* rd = W + il * XW_LD + 31 - il;
-  const float* mk = a.mask_t ? a.mask_t + ((int64_t)b * a.K + j0) * a.QQ + qrow : nullptr;
-  const uint8_t* sg = a.seg_t ? a.seg_t + ((int64_t)b * a.K + j0) * a.Q + i : nullptr;
-#pragma unroll
-  for (int e = 0; e < 16; ++e) {
-    const int jl = acc_row(e, half);
-    const float ef = (sg && sg[(int64_t)jl * a.Q]) ? e1 : e0;
-    float v = (s[e] + rd[jl] + ef) * a.scale;
-    if (mk) v -= 1e30f * mk[(int64_t)jl * a.QQ];
-    sc[e] = v;
-  }
-  __builtin_amdgcn_wave_barrier();
-}
-
-// grid (QQ/64, B*N)
-__global__ __launch_bounds__(NTHREADS) void xl_attn_fwd_kernel(XlAttnArgs a, int prio) {
-  ds_wave_prio(prio);
-  extern __shared__ __attribute__((aligned(16))) char lds[];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5, il = lane & 31;
-  const int grp = wave & 1, part = wave >> 1;
-  const int b = blockIdx.y / a.N, hd = blockIdx.y % a.N;
-  const int i0 = (blockIdx.x * 64) % a.Q;                  // stream-relative index of the block's first query
-  const int qrow = blockIdx.x * 64 + grp * 32 + il;        // stacked query row of this lane
-  const int i = i0 + grp * 32 + il;
-  const int64_t hoff = (int64_t)b * a.H + hd * HD;
-  const bf16* kbase = reinterpret_cast<const bf16*>(a.kv) + (int64_t)b * 2 * a.H + hd * HD;
-  const bf16* krbase = reinterpret_cast<const bf16*>(a.kr) + hd * HD;
-  char* sk = lds;
-  char* sv = lds + X_SV;
-  char* skr = lds + X_SKR;
-  float* W = reinterpret_cast<float*>(lds + X_SCR + wave * XW_BYTES);
-  float* slse = reinterpret_cast<float*>(lds + X_LSE);
-  bf16x8 qwf[4], qrf[4];
-  float e0 = 0.f, e1 = 0.f;
-  {
-    const bf16* qwp = reinterpret_cast<const bf16*>(a.qw) + (int64_t)qrow * a.ldq + hoff;
-    const bf16* qrp = reinterpret_cast<const bf16*>(a.qr) + (int64_t)qrow * a.ldq + hoff;
-    const bf16* qsp = reinterpret_cast<const bf16*>(a.qs) + (int64_t)qrow * a.ldq + hoff;
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      qwf[ks] = *reinterpret_cast<const bf16x8*>(qwp + 16 * ks + 8 * half);
-      qrf[ks] = *reinterpret_cast<const bf16x8*>(qrp + 16 * ks + 8 * half);
-      const bf16x8 qv = *reinterpret_cast<const bf16x8*>(qsp + 16 * ks + 8 * half);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int d = 16 * ks + 8 * half + j;
-        e0 += (float)qv[j] * a.seg_emb[hd * HD + d];
-        e1 += (float)qv[j] * a.seg_emb[a.H + hd * HD + d];
-      }
-    }
-    e0 += __shfl_xor(e0, 32, 64);
-    e1 += __shfl_xor(e1, 32, 64);
-  }
-  f32x16 o[2];
-#pragma unroll
-  for (int e = 0; e < 16; ++e) { o[0][e] = 0.f; o[1][e] = 0.f; }
-  float m = -INFINITY, l = 0.f;
-  const int kt = part * 32;               // this wave's key step inside every chunk
-  const int rb = kt + 32 - 32 * grp;      // first window row of that step for this wave's 32 queries
-  for (int k0 = 0; k0 < a.K; k0 += XCHUNK) {
-    const int rows = a.K - k0 < XCHUNK ? a.K - k0 : XCHUNK;
-    __syncthreads();
-    tile_fill(sk, kbase + (int64_t)k0 * a.ldkv, a.ldkv, rows, wave, lane);
-    tile_fill(sv, kbase + a.H + (int64_t)k0 * a.ldkv, a.ldkv, rows, wave, lane);
-    xl_fill_kr(skr, krbase, a.ldkr, k0 + a.Q - i0 - 63, rows + 64, a.R, wave, lane);
-    __builtin_amdgcn_s_waitcnt(VMCNT0);
-    __syncthreads();
-    if (kt < rows) {
-      float p[16];
-      xl_step_scores(a, sk, skr, W, qwf, qrf, kt, rb, lane, b, qrow, i, k0 + kt, e0, e1, p);
-      float mt = -INFINITY;
-#pragma unroll
-      for (int e = 0; e < 16; ++e) mt = fmaxf(mt, p[e]);
-      mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-      const float mn = fmaxf(m, mt);
-      const float alpha = __expf(m - mn);
-      m = mn;
-      float rs = 0.f;
-#pragma unroll
-      for (int e = 0; e < 16; ++e) { p[e] = __expf(p[e] - mn); rs += p[e]; }
-      l = l * alpha + rs;
-#pragma unroll
-      for (int e = 0; e < 16; ++e) { o[0][e] *= alpha; o[1][e] *= alpha; }
-#pragma unroll
-      for (int s2 = 0; s2 < 2; ++s2) {
-        const bf16x8 pf = pack8(p + 8 * s2);
-#pragma unroll
-        for (int dt = 0; dt < 2; ++dt) o[dt] = mfma(frag_cols(sv, kt + 16 * s2, dt * 32, lane), pf, o[dt]);
-      }
-    }
-  }
-  // combine the SPLIT partial softmaxes of each query group (part 0 always saw a key step: K >= 32)
-  __syncthreads();
-  if (part > 0) {
-    part_store<2>(lds + ((part - 1) * 2 + grp) * PART_BYTES, o, lane);
-    part_store_xy(lds + ((part - 1) * 2 + grp) * PART_BYTES, m, l, lane);
-  }
-  __syncthreads();
-  if (part == 0) {
-#pragma unroll
-    for (int pp = 1; pp < SPLIT; ++pp) {
-      const char* slot = lds + ((pp - 1) * 2 + grp) * PART_BYTES;
-      float mp, lp;
-      part_xy(slot, mp, lp, lane);
-      // (a part whose key steps all lay beyond K parked m = -inf, l = 0, o = 0: weight 0)
-      const float mn = fmaxf(m, mp);
-      const float wa = __expf(m - mn), wb = __expf(mp - mn);
-      part_merge<2>(slot, o, wa, wb, lane);
-      l = l * wa + lp * wb;
-      m = mn;
-    }
-    l += __shfl_xor(l, 32, 64);
-    store_t(reinterpret_cast<bf16*>(a.vec) + (int64_t)qrow * a.ldq + hoff, o, 1.0f / l, half);
-    if (half == 0) slse[grp * 32 + il] = m + __logf(l);
-  }
-  __syncthreads();
-  const float lse = slse[grp * 32 + il];
-  // pass 2: the probabilities
-  bf16* prow = reinterpret_cast<bf16*>(a.p) + ((int64_t)blockIdx.y * a.QQ + qrow) * a.K;
-  for (int k0 = 0; k0 < a.K; k0 += XCHUNK) {
-    const int rows = a.K - k0 < XCHUNK ? a.K - k0 : XCHUNK;
-    __syncthreads();
-    tile_fill(sk, kbase + (int64_t)k0 * a.ldkv, a.ldkv, rows, wave, lane);
-    xl_fill_kr(skr, krbase, a.ldkr, k0 + a.Q - i0 - 63, rows + 64, a.R, wave, lane);
-    __builtin_amdgcn_s_waitcnt(VMCNT0);
-    __syncthreads();
-    if (kt < rows) {
-      float p[16];
-      xl_step_scores(a, sk, skr, W, qwf, qrf, kt, rb, lane, b, qrow, i, k0 + kt, e0, e1, p);
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        bf16x4 v;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) v[j] = (bf16)__expf(p[4 * g + j] - lse);
-        *reinterpret_cast<bf16x4*>(prow + k0 + kt + g * 8 + half * 4) = v;
-      }
-    }
-  }
-}
-
 int check(const char* who, int dtype, int B, int N, int S, int D) {
   DS_CHECK_ARG(dtype == DS_BF16, "%s: the fused kernels are bf16 only (dtype %d)", who, dtype);
   DS_CHECK_ARG(D == HD, "%s: head size must be %d (got %d)", who, HD, D);
@@ -741,28 +544,5 @@ extern "C" int ds_attention_bwd(int dtype, int batch, int heads, int seq, int he
     hipLaunchKernelGGL(attn_bwd_dkv_kernel, dim3(seq / 64, batch * heads), dim3(NTHREADS), lds_bytes(seq), s, a);
     DS_CHECK_LAUNCH();
   }
-  return DS_OK;
-}
-
-bool ds_xl_attention_fits(int dtype, int head_dim, int Q, int K, int R) {
-  return dtype == DS_BF16 && head_dim == HD && Q > 0 && Q % 64 == 0 && K >= 32 && K % 32 == 0 && R == K + Q;
-}
-
-int ds_xl_attention_fwd(const XlAttnArgs* a, hipStream_t s) {
-  DS_CHECK_ARG(a && a->qw && a->qr && a->qs && a->kv && a->kr && a->seg_emb && a->p && a->vec, "ds_xl_attention_fwd: null pointer");
-  DS_CHECK_ARG(ds_xl_attention_fits(DS_BF16, a->H / (a->N > 0 ? a->N : 1), a->Q, a->K, a->R) && a->QQ % a->Q == 0 && a->H == a->N * HD,
-               "ds_xl_attention_fwd: shape outside the kernel (Q %d, QQ %d, K %d, R %d, H %d, N %d)", a->Q, a->QQ, a->K, a->R, a->H, a->N);
-  DS_CHECK_ARG(a->ldq % 8 == 0 && a->ldkv % 8 == 0 && a->ldkr % 8 == 0 && ds_aligned16(a->qw) && ds_aligned16(a->qr) && ds_aligned16(a->qs) &&
-               ds_aligned16(a->kv) && ds_aligned16(a->kr) && ds_aligned16(a->p) && ds_aligned16(a->vec), "ds_xl_attention_fwd: bad stride or alignment");
-  DS_CHECK_ARG((int64_t)a->B * a->N <= 65535, "ds_xl_attention_fwd: batch * heads exceeds 65535");
-  static bool attr = false;
-  if (!attr) {
-    DS_CHECK_HIP(hipFuncSetAttribute((const void*)xl_attn_fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, X_LDS_BYTES));
-    attr = true;
-  }
-  // q k^T and q kr^T over the 64-row window (3 products of 32x32x64 per step, twice), P V once
-  ds_prof_scope prof(s, "xl_attn_fwd_kernel", (2.0 * 3 * 2 + 2.0) * a->B * a->N * (double)a->QQ * a->K * HD, "FLOP");
-  hipLaunchKernelGGL(xl_attn_fwd_kernel, dim3(a->QQ / 64, a->B * a->N), dim3(NTHREADS), X_LDS_BYTES, s, *a, ds_launch_prio);
-  DS_CHECK_LAUNCH();
   return DS_OK;
 }

@@ -4,43 +4,62 @@
 //   score[j] = (qw[i'] . k[j] + qr[i'] . kr[j + Q - i] + ef[seg(i, j, b)]) * scale - 1e30 * mask[i'][j][b],   p = softmax_j score
 // and, backward, with dp[j] = dvec[i'] . v[j]:
 //   ds[j] = scale * p[j] * (dp[j] - sum_k p[k] dp[k]),  dbd[i'][j + Q - i] = ds[j],  def[s] = sum_j [seg == s] ds[j].
-// A block owns 32 query rows and ALL keys of one (b, n): wave w keeps the scores of keys [128 w, 128 w + 128) in registers
-// (four 32x32 MFMA accumulators, query rows down the registers, keys across the lanes), so a row's softmax needs one pass and
-// the only thing written is the bf16 probability (forward) or the bf16 score gradients (backward).
-// The relative shift in that orientation: the position product is computed UN-shifted for the 64 consecutive k_r rows a
-// 32 x 32 tile can touch (two accumulators, the second one shared with the next key tile), and the element of row m, key
-// column n is column n + 31 - m of that window - for a fixed register (fixed m) a rotation of the lanes, i.e. one
-// ds_bpermute after the source lanes picked the accumulator they are asked for.
+// A block owns 16 query rows and ALL keys of one (b, n): wave w keeps the scores of keys [128 w, 128 w + 128) in registers
+// (eight 16x16 MFMA accumulators: keys across the 16 lanes of a lane group, four query rows per lane group down the
+// registers), so a row's softmax needs one pass and the only thing written is the bf16 probability (forward) or the bf16
+// score gradients (backward).  At about 110 registers a wave, four waves share a SIMD and two blocks a CU.
+// The relative shift in that orientation: the position product is computed UN-shifted for the 32 consecutive k_r rows a
+// 16 x 16 tile can touch (two accumulators, the second one shared with the next key tile), and the element of row m, key
+// column n is column n + 15 - m of that window - for a fixed register (fixed m within the lane group) a rotation of the
+// group's lanes, i.e. one ds_bpermute after the source lanes picked the accumulator they are asked for.
+// Of the two segment scores only their difference matters (a softmax row ignores a constant), and the mask / segment bits
+// of a lane's 32 scores are two 32-bit words, turned into addends with a bit-field extract and an AND each.
 #include "common.h"
 #include "stage.h"
 
 namespace {
 
 constexpr int HD = 64;    // head size
-constexpr int NT = 4;     // key tiles (of 32 keys) per wave
-constexpr int MAXW = 8;   // waves per block: up to 32 * NT * MAXW = 1024 keys
+constexpr int RB = 16;    // query rows per block
+constexpr int NT = 8;     // key tiles (of 16 keys) per wave
+constexpr int MAXW = 8;   // waves per block: up to 16 * NT * MAXW = 1024 keys
 constexpr float LOG2E = 1.4426950408889634f;
 
-__device__ __forceinline__ f32x16 mfma(bf16x8 a, bf16x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
-// query row (0..31) of accumulator element e in this lane's half
-__device__ __forceinline__ int acc_row(int e, int half) { return (e >> 2) * 8 + half * 4 + (e & 3); }
-__device__ __forceinline__ float lane_read(float v, int src_lane) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src_lane << 2, __builtin_bit_cast(int, v)));
+__device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
+__device__ __forceinline__ float lane_read(float v, int byte_addr) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(byte_addr, __builtin_bit_cast(int, v)));
 }
-// reductions over the 32 lanes of a half wave (the keys of one tile row)
-__device__ __forceinline__ float half_max(float v) {
+// x where bit `idx` of `bits` is set, else 0
+__device__ __forceinline__ float bit_select(uint32_t bits, int idx, float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_sbfe((int)bits, idx, 1) & __builtin_bit_cast(int, x));
+}
+// reductions over the 16 lanes of a lane group (the keys of one tile row): DPP moves only
+__device__ __forceinline__ float group_max(float v) {
   v = fmaxf(v, dpp_move<0xB1>(v));
   v = fmaxf(v, dpp_move<0x4E>(v));
   v = fmaxf(v, dpp_move<0x141>(v));
-  v = fmaxf(v, dpp_move<0x140>(v));
-  return fmaxf(v, __shfl_xor(v, 16, 64));
+  return fmaxf(v, dpp_move<0x140>(v));
 }
-__device__ __forceinline__ float half_sum(float v) {
+__device__ __forceinline__ float group_sum(float v) {
   v += dpp_move<0xB1>(v);
   v += dpp_move<0x4E>(v);
   v += dpp_move<0x141>(v);
-  v += dpp_move<0x140>(v);
-  return v + __shfl_xor(v, 16, 64);
+  return v + dpp_move<0x140>(v);
+}
+
+// Two accumulator registers of a lane (rows m and m + 1 of its key column n) against one bf16 pair per lane: even lanes hold
+// row m, keys (n, n + 1), odd lanes row m + 1, keys (n - 1, n) - so that a 32-bit access per lane covers what two 16-bit
+// accesses would.  The lanes of a pair swap one value through a DPP move.
+__device__ __forceinline__ uint32_t pair_pack(float a, float b, bool odd) {
+  const float recv = dpp_move<0xB1>(odd ? a : b);
+  const bf16x2 v = {(bf16)(odd ? recv : a), (bf16)(odd ? b : recv)};
+  return __builtin_bit_cast(uint32_t, v);
+}
+__device__ __forceinline__ void pair_unpack(uint32_t w, bool odd, float& a, float& b) {
+  const float lo = __builtin_bit_cast(float, w << 16), hi = __builtin_bit_cast(float, w & 0xffff0000u);
+  const float recv = dpp_move<0xB1>(odd ? lo : hi);
+  a = odd ? recv : lo;
+  b = odd ? hi : recv;
 }
 
 // workgroups of one XCD (equal launch index mod 8) take whole heads, so a head's k, k_r and v rows stay in one L2
@@ -53,26 +72,26 @@ __device__ __forceinline__ void block_map(int& bh, int& blk) {
   blk = k % nb;
 }
 
-// meta[b][rb][kt][lane][e]: bit 0 = mask != 0, bit 1 = segment bit of query row rb*32 + acc_row(e, lane/32) and key
-// kt*32 + lane%32: the 16 bytes a lane needs for one tile, in the order of its accumulator registers
+// meta[b][rb][w][lane] = (mask bits, segment bits) of the 32 scores that lane `lane` of wave w holds for row block rb:
+// bit 4 t + v belongs to query row rb*16 + 4 (lane/16) + v and key w*128 + t*16 + lane%16
 __global__ __launch_bounds__(256) void xl_pack_meta_kernel(int Q, int QQ, int K, int B, const float* __restrict__ mask,
-                                                          const uint8_t* __restrict__ seg, u32x4* __restrict__ meta) {
-  const int KT = K >> 5, RB = QQ >> 5;
+                                                          const uint8_t* __restrict__ seg, uint2* __restrict__ meta) {
+  const int NW = (K + 127) >> 7, NRB = QQ / RB;
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= (int64_t)B * RB * KT * 64) return;
-  const int lane = (int)(idx & 63), half = lane >> 5, il = lane & 31;
-  const int kt = (int)((idx >> 6) % KT), rb = (int)((idx >> 6) / KT % RB), b = (int)((idx >> 6) / ((int64_t)KT * RB));
-  const int j = kt * 32 + il;
-  u32x4 out = {0u, 0u, 0u, 0u};
-#pragma unroll
-  for (int e = 0; e < 16; ++e) {
-    const int ii = rb * 32 + acc_row(e, half), i = ii % Q;
-    uint32_t bits = 0;
-    if (mask && mask[((int64_t)ii * K + j) * B + b] != 0.f) bits |= 1u;
-    if (seg && seg[((int64_t)i * K + j) * B + b]) bits |= 2u;
-    out[e >> 2] |= bits << (8 * (e & 3));
+  if (idx >= (int64_t)B * NRB * NW * 64) return;
+  const int lane = (int)(idx & 63), g = lane >> 4, n = lane & 15;
+  const int w = (int)((idx >> 6) % NW), rb = (int)((idx >> 6) / NW % NRB), b = (int)((idx >> 6) / ((int64_t)NW * NRB));
+  uint32_t mb = 0, sb = 0;
+  for (int t = 0; t < NT; ++t) {
+    const int j = w * 128 + t * 16 + n;
+    if (j >= K) break;
+    for (int v = 0; v < 4; ++v) {
+      const int ii = rb * RB + 4 * g + v, i = ii % Q;
+      if (mask && mask[((int64_t)ii * K + j) * B + b] != 0.f) mb |= 1u << (4 * t + v);
+      if (seg && seg[((int64_t)i * K + j) * B + b]) sb |= 1u << (4 * t + v);
+    }
   }
-  meta[idx] = out;
+  meta[idx] = make_uint2(mb, sb);
 }
 
 // nseg[b][i] = number of keys in the other segment (seg bit set) of query row i
@@ -87,141 +106,156 @@ __global__ __launch_bounds__(256) void xl_seg_count_kernel(int Q, int K, int B, 
   if (lane == 0) nseg[w] = n;
 }
 
-// this lane's 16-byte MFMA operand slices of one 64-wide row (k index 16 ks + 8 half .. + 7)
-__device__ __forceinline__ void load_frags(const bf16* row_ptr, bf16x8 (&f)[4]) {
-#pragma unroll
-  for (int ks = 0; ks < 4; ++ks) f[ks] = *reinterpret_cast<const bf16x8*>(row_ptr + 16 * ks);
+// this lane's two 16-byte MFMA operand slices of one 64-wide row (k index 32 ks + 8 (lane / 16) .. + 7; row_ptr includes 8 (lane / 16))
+__device__ __forceinline__ void load_frags(const bf16* row_ptr, bf16x8 (&f)[2]) {
+  f[0] = *reinterpret_cast<const bf16x8*>(row_ptr);
+  f[1] = *reinterpret_cast<const bf16x8*>(row_ptr + 32);
 }
 
-// grid (QQ / 32, B * N), 64 * ceil(K / 128) threads
+// grid (QQ / 16, B * N), 64 * ceil(K / 128) threads.  FULL: K is a multiple of 128, so every wave has all its tiles; META: mask /
+// segment bits exist.
+template <bool FULL, bool META>
 __global__ __launch_bounds__(64 * MAXW) void xl_scores_fwd_kernel(XlScoreArgs a, int prio) {
   ds_wave_prio(prio);
-  __shared__ float sm[MAXW][32], sl[MAXW][32];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5, il = lane & 31;
+  __shared__ float sm[MAXW][RB], sl[MAXW][RB];
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), g = lane >> 4, n = lane & 15;
   const int nw = blockDim.x >> 6;
   int bh, blk;
   block_map(bh, blk);
   const int b = bh / a.N, hd = bh % a.N;
-  const int ii0 = blk * 32, i0 = ii0 % a.Q;
-  const int KT = a.K >> 5;
-  const int64_t hoff = (int64_t)b * a.H + hd * HD;
-  const bf16* qw = reinterpret_cast<const bf16*>(a.qw);
-  const bf16* qr = reinterpret_cast<const bf16*>(a.qr);
-  const bf16* qs = reinterpret_cast<const bf16*>(a.qs);
-  const bf16* kb = reinterpret_cast<const bf16*>(a.k) + (int64_t)b * a.ldk_b + hd * HD + 8 * half;
-  const bf16* krb = reinterpret_cast<const bf16*>(a.kr) + hd * HD + 8 * half;
-  bf16x8 qwf[4], qrf[4];
-  load_frags(qw + (int64_t)(ii0 + il) * a.ldq + hoff + 8 * half, qwf);
-  load_frags(qr + (int64_t)(ii0 + il) * a.ldq + hoff + 8 * half, qrf);
-  // E: lanes 0..31 hold ef[0] of query row `lane`, lanes 32..63 ef[1] of row lane - 32
-  float E = 0.f;
+  const int ii0 = blk * RB, i0 = ii0 % a.Q;
+  const int KT = a.K >> 4;
+  const int kt0 = wave * NT;
+  const int64_t qoff = (int64_t)(ii0 + n) * a.ldq + (int64_t)b * a.H + hd * HD;
+  const bf16* kb = reinterpret_cast<const bf16*>(a.k) + (int64_t)b * a.ldk_b + hd * HD + 8 * g;
+  const bf16* krb = reinterpret_cast<const bf16*>(a.kr) + hd * HD + 8 * g;
+  // The tile loop has no branches (a join would make every wait for operands a wait for all loads in flight): tiles past the
+  // last key read clamped rows and their scores are replaced below.  Operands are requested two tiles ahead.
+  bf16x8 kf[3][2], krf[3][2];
+  auto request = [&](int t) {
+    int j = (kt0 + t) * 16 + n;
+    if (!FULL) j = j < a.K ? j : a.K - 1;
+    load_frags(kb + (int64_t)j * a.ldk, kf[t % 3]);
+    int r = (kt0 + t) * 16 + a.Q - i0 + 1 + n;   // second half of the window: k_r rows j0 + Q - i0 - 15 + 16 + lane
+    r = r < a.R ? r : a.R - 1;
+    load_frags(krb + (int64_t)r * a.ldkr, krf[t % 3]);
+  };
+  bf16x8 qwf[2], qrf[2], f0[2];
+  load_frags(reinterpret_cast<const bf16*>(a.qr) + qoff + 8 * g, qrf);
   {
-    const bf16* qsp = qs + (int64_t)(ii0 + il) * a.ldq + hoff;
-    const float* se = a.seg_emb + (int64_t)half * a.H + hd * HD;
+    int r = kt0 * 16 + a.Q - i0 - 15 + n;   // first half of the first window
+    if (!FULL) r = r < a.R ? r : a.R - 1;
+    load_frags(krb + (int64_t)r * a.ldkr, f0);
+  }
+  load_frags(reinterpret_cast<const bf16*>(a.qw) + qoff + 8 * g, qwf);
+  request(0);
+  request(1);
+  // de[v]: ef[1] - ef[0] of this lane's query row 4 g + v (a row's softmax ignores ef[0])
+  float de[4] = {0.f, 0.f, 0.f, 0.f};
+  uint32_t mbits = 0, sbits = 0;
+  if (META) {
+    const uint2 mw = reinterpret_cast<const uint2*>(a.meta)[(((int64_t)b * (a.QQ / RB) + blk) * nw + wave) * 64 + lane];
+    mbits = mw.x; sbits = mw.y;
+    const bf16* qsp = reinterpret_cast<const bf16*>(a.qs) + qoff + 16 * g;
+    const float* se = a.seg_emb + hd * HD + 16 * g;
+    float d = 0.f;
 #pragma unroll
-    for (int c = 0; c < 8; ++c) {
+    for (int c = 0; c < 2; ++c) {
       const bf16x8 qv = *reinterpret_cast<const bf16x8*>(qsp + 8 * c);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) E += (float)qv[j] * se[8 * c + j];
+      for (int h = 0; h < 2; ++h) {
+        const f32x4 s0 = *reinterpret_cast<const f32x4*>(se + 8 * c + 4 * h), s1 = *reinterpret_cast<const f32x4*>(se + a.H + 8 * c + 4 * h);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) d += (float)qv[4 * h + j] * (s1[j] - s0[j]);
+      }
     }
+    d += __shfl_xor(d, 16, 64);
+    d += __shfl_xor(d, 32, 64);   // every lane: the difference for query row n
+#pragma unroll
+    for (int v = 0; v < 4; ++v) de[v] = lane_read(d, (4 * g + v) << 2);
+  }
+  // column u = n + 15 - m of a tile's window is wanted by lane n of the group: the lane holding it is 16 g + (u & 15), and
+  // that lane serves it from the window's first accumulator when its own column is >= 15 - m
+  int rot[4];
+  bool first[4];
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    const int m = 4 * g + v;
+    rot[v] = (16 * g + ((n + 15 - m) & 15)) << 2;
+    asm volatile("" : "+v"(rot[v]));   // computed once, not once per tile
+    first[v] = n >= 15 - m;
   }
   const float c2 = a.scale * LOG2E;
-  float s[NT][16];
-  f32x16 raw0;
-  const int kt0 = wave * NT;
-  {
-    // the un-shifted position products of the window's first 32 rows: k_r rows kt0*32 + Q - i0 - 31 + lane
-    int r = kt0 * 32 + a.Q - i0 - 31 + il;
-    r = r < a.R ? r : a.R - 1;
-    bf16x8 krf[4];
-    load_frags(krb + (int64_t)r * a.ldkr, krf);
-#pragma unroll
-    for (int e = 0; e < 16; ++e) raw0[e] = 0.f;
-    if (kt0 < KT) {
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks) raw0 = mfma(qrf[ks], krf[ks], raw0);
-    }
-  }
+  float s[NT][4];
+  f32x4 raw0 = {0.f, 0.f, 0.f, 0.f};
+  raw0 = mfma16(qrf[0], f0[0], raw0);
+  raw0 = mfma16(qrf[1], f0[1], raw0);
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
-    const int kt = kt0 + t;
-    if (kt < KT) {
-      const int j0 = kt * 32;
-      bf16x8 kf[4], krf[4];
-      load_frags(kb + (int64_t)(j0 + il) * a.ldk, kf);
-      int r = j0 + a.Q - i0 + 1 + il;   // second half of the window
-      r = r < a.R ? r : a.R - 1;
-      load_frags(krb + (int64_t)r * a.ldkr, krf);
-      u32x4 mw = {0u, 0u, 0u, 0u};
-      if (a.meta) mw = reinterpret_cast<const u32x4*>(a.meta)[(((int64_t)b * (a.QQ >> 5) + blk) * KT + kt) * 64 + lane];
-      f32x16 ac, raw1;
+    if (t + 2 < NT) request(t + 2);
+    f32x4 ac = {0.f, 0.f, 0.f, 0.f}, raw1 = {0.f, 0.f, 0.f, 0.f};
+    ac = mfma16(qwf[0], kf[t % 3][0], ac);
+    raw1 = mfma16(qrf[0], krf[t % 3][0], raw1);
+    ac = mfma16(qwf[1], kf[t % 3][1], ac);
+    raw1 = mfma16(qrf[1], krf[t % 3][1], raw1);
+    float bd[4];
 #pragma unroll
-      for (int e = 0; e < 16; ++e) { ac[e] = 0.f; raw1[e] = 0.f; }
+    for (int v = 0; v < 4; ++v) bd[v] = lane_read(first[v] ? raw0[v] : raw1[v], rot[v]);
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
-        ac = mfma(qwf[ks], kf[ks], ac);
-        raw1 = mfma(qrf[ks], krf[ks], raw1);
+    for (int v = 0; v < 4; ++v) {
+      float x = ac[v] + bd[v];
+      if (META) {
+        x += bit_select(sbits, 4 * t + v, de[v]);
+        s[t][v] = fmaf(x, c2, bit_select(mbits, 4 * t + v, -1e30f));
+      } else {
+        s[t][v] = x * c2;
       }
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int m = acc_row(e, half);
-        // column u = n + 31 - m of the window is wanted by lane n: lanes u >= 31 - m serve it from the first accumulator
-        const float y = il >= 31 - m ? raw0[e] : raw1[e];
-        const float bd = lane_read(y, half * 32 + ((il + 31 - m) & 31));
-        const uint32_t bits = (mw[e >> 2] >> (8 * (e & 3))) & 3u;
-        const float ef = lane_read(E, (int)(bits >> 1) * 32 + m);
-        s[t][e] = (ac[e] + bd + ef) * c2 - ((bits & 1u) ? 1e30f : 0.f);
-      }
-      raw0 = raw1;
-    } else {
-#pragma unroll
-      for (int e = 0; e < 16; ++e) s[t][e] = -INFINITY;
     }
+    raw0 = raw1;
   }
   // the wave's own maxima and sums per row, then the block's
-  float mx[16], l[16];
+  const float dead = -INFINITY;   // tiles past the last key
+  float mx[4], l[4];
 #pragma unroll
-  for (int e = 0; e < 16; ++e) {
-    float v = s[0][e];
+  for (int v = 0; v < 4; ++v) {
+    float x = s[0][v];
 #pragma unroll
-    for (int t = 1; t < NT; ++t) v = fmaxf(v, s[t][e]);
-    mx[e] = half_max(v);
+    for (int t = 1; t < NT; ++t) x = fmaxf(x, FULL || kt0 + t < KT ? s[t][v] : dead);
+    mx[v] = group_max(x);
   }
 #pragma unroll
-  for (int e = 0; e < 16; ++e) {
-    float v = 0.f;
+  for (int v = 0; v < 4; ++v) {
+    float x = 0.f;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-      s[t][e] = kt0 + t < KT ? __builtin_amdgcn_exp2f(s[t][e] - mx[e]) : 0.f;
-      v += s[t][e];
+      s[t][v] = FULL || kt0 + t < KT ? __builtin_amdgcn_exp2f(s[t][v] - mx[v]) : 0.f;
+      x += s[t][v];
     }
-    l[e] = half_sum(v);
+    l[v] = group_sum(x);
   }
-  if (il == 0) {
+  // (a wave of a block always has its first tile: the block has ceil(K / 128) waves)
+  if (n == 0) {
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      sm[wave][acc_row(e, half)] = mx[e];
-      sl[wave][acc_row(e, half)] = l[e];
-    }
+    for (int v = 0; v < 4; ++v) { sm[wave][4 * g + v] = mx[v]; sl[wave][4 * g + v] = l[v]; }
   }
   __syncthreads();
-  if (kt0 >= KT) return;
   float f;
   {
-    float M = sm[0][il];
-    for (int w = 1; w < nw; ++w) M = fmaxf(M, sm[w][il]);
+    float M = sm[0][n];
+    for (int w = 1; w < nw; ++w) M = fmaxf(M, sm[w][n]);
     float L = 0.f;
-    for (int w = 0; w < nw; ++w) L += sl[w][il] * __builtin_amdgcn_exp2f(sm[w][il] - M);
-    f = __builtin_amdgcn_exp2f(sm[wave][il] - M) / L;
+    for (int w = 0; w < nw; ++w) L += sl[w][n] * __builtin_amdgcn_exp2f(sm[w][n] - M);
+    f = __builtin_amdgcn_exp2f(sm[wave][n] - M) / L;
   }
-  bf16* p = reinterpret_cast<bf16*>(a.p) + ((int64_t)bh * a.QQ + ii0) * a.K + il;
+  const bool odd = n & 1;
+  bf16* p = reinterpret_cast<bf16*>(a.p) + ((int64_t)bh * a.QQ + ii0 + 4 * g + (odd ? 1 : 0)) * a.K + (n & ~1);
 #pragma unroll
-  for (int e = 0; e < 16; ++e) {
-    const int m = acc_row(e, half);
-    const float fr = lane_read(f, m);
+  for (int v = 0; v < 4; v += 2) {
+    const float f0s = lane_read(f, (4 * g + v) << 2), f1s = lane_read(f, (4 * g + v + 1) << 2);
 #pragma unroll
     for (int t = 0; t < NT; ++t)
-      if (kt0 + t < KT) p[(int64_t)m * a.K + (kt0 + t) * 32] = (bf16)(s[t][e] * fr);
+      if (FULL || kt0 + t < KT)
+        *reinterpret_cast<uint32_t*>(p + (int64_t)v * a.K + (kt0 + t) * 16) = pair_pack(s[t][v] * f0s, s[t][v + 1] * f1s, odd);
   }
 }
 
@@ -229,110 +263,115 @@ __global__ __launch_bounds__(64 * MAXW) void xl_scores_fwd_kernel(XlScoreArgs a,
 // copy and the two segment sums.  grid and block as the forward kernel.
 __global__ __launch_bounds__(64 * MAXW) void xl_scores_bwd_kernel(XlScoreArgs a, int prio) {
   ds_wave_prio(prio);
-  __shared__ float sd[MAXW][32], st[MAXW][32], s1[MAXW][32];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5, il = lane & 31;
+  __shared__ float sd[MAXW][RB], st[MAXW][RB], s1[MAXW][RB];
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), g = lane >> 4, n = lane & 15;
   const int nw = blockDim.x >> 6;
   int bh, blk;
   block_map(bh, blk);
   const int b = bh / a.N, hd = bh % a.N;
-  const int ii0 = blk * 32, i0 = ii0 % a.Q;
-  const int KT = a.K >> 5;
+  const int ii0 = blk * RB, i0 = ii0 % a.Q;
+  const int KT = a.K >> 4;
   const int kt0 = wave * NT;
-  const int64_t hoff = (int64_t)b * a.H + hd * HD;
-  const bf16* vb = reinterpret_cast<const bf16*>(a.v) + (int64_t)b * a.ldk_b + hd * HD + 8 * half;
-  const bf16* p = reinterpret_cast<const bf16*>(a.p) + ((int64_t)bh * a.QQ + ii0) * a.K + il;
-  bf16x8 dvf[4];
-  load_frags(reinterpret_cast<const bf16*>(a.dvec) + (int64_t)(ii0 + il) * a.ldq + hoff + 8 * half, dvf);
-  float dp[NT][16], pp[NT][16], dot[16];
-#pragma unroll
-  for (int e = 0; e < 16; ++e) dot[e] = 0.f;
-#pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    const int kt = kt0 + t;
-    if (kt < KT) {
-      bf16x8 vf[4];
-      load_frags(vb + (int64_t)(kt * 32 + il) * a.ldk, vf);
-#pragma unroll
-      for (int e = 0; e < 16; ++e) pp[t][e] = (float)p[(int64_t)acc_row(e, half) * a.K + kt * 32];
-      f32x16 acc;
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[e] = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks) acc = mfma(dvf[ks], vf[ks], acc);
-#pragma unroll
-      for (int e = 0; e < 16; ++e) { dp[t][e] = acc[e]; dot[e] += pp[t][e] * acc[e]; }
-    } else {
-#pragma unroll
-      for (int e = 0; e < 16; ++e) { dp[t][e] = 0.f; pp[t][e] = 0.f; }
-    }
-  }
-#pragma unroll
-  for (int e = 0; e < 16; ++e) dot[e] = half_sum(dot[e]);
-  if (il == 0) {
-#pragma unroll
-    for (int e = 0; e < 16; ++e) sd[wave][acc_row(e, half)] = dot[e];
-  }
-  __syncthreads();
-  float D = 0.f;
-  for (int w = 0; w < nw; ++w) D += sd[w][il];
-  float tot[16], d1[16];
-#pragma unroll
-  for (int e = 0; e < 16; ++e) { dot[e] = lane_read(D, acc_row(e, half)); tot[e] = 0.f; d1[e] = 0.f; }
-  bf16* ds = reinterpret_cast<bf16*>(a.ds) + ((int64_t)bh * a.QQ + ii0) * a.K + il;
-  // column j of row i lands in column j + Q - i of the un-shifted copy
-  bf16* dbd = reinterpret_cast<bf16*>(a.dbd) + ((int64_t)bh * a.QQ + ii0) * a.R + il + a.Q - i0;
+  const bool odd = n & 1;
+  const bf16* vb = reinterpret_cast<const bf16*>(a.v) + (int64_t)b * a.ldk_b + hd * HD + 8 * g;
+  const bf16* p = reinterpret_cast<const bf16*>(a.p) + ((int64_t)bh * a.QQ + ii0 + 4 * g + (odd ? 1 : 0)) * a.K + (n & ~1);
+  bf16x8 dvf[2];
+  load_frags(reinterpret_cast<const bf16*>(a.dvec) + (int64_t)(ii0 + n) * a.ldq + (int64_t)b * a.H + hd * HD + 8 * g, dvf);
+  uint32_t sbits = 0;
+  if (a.meta) sbits = reinterpret_cast<const uint2*>(a.meta)[(((int64_t)b * (a.QQ / RB) + blk) * nw + wave) * 64 + lane].y;
+  float dp[NT][4], pp[NT][4], dot[4] = {0.f, 0.f, 0.f, 0.f};
+  bf16x8 vf[2][2];
+  uint32_t pw[2][2];
+  // (no branches in the tile loop: tiles past the last key read the last tile again and count as zeros)
+  auto request = [&](int t) {
+    const int kt = kt0 + t < KT ? kt0 + t : KT - 1;
+    load_frags(vb + (int64_t)(kt * 16 + n) * a.ldk, vf[t & 1]);
+    pw[t & 1][0] = *reinterpret_cast<const uint32_t*>(p + kt * 16);
+    pw[t & 1][1] = *reinterpret_cast<const uint32_t*>(p + 2 * (int64_t)a.K + kt * 16);
+  };
+  request(0);
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
-    const int kt = kt0 + t;
-    if (kt < KT) {
-      u32x4 mw = {0u, 0u, 0u, 0u};
-      if (a.meta) mw = reinterpret_cast<const u32x4*>(a.meta)[(((int64_t)b * (a.QQ >> 5) + blk) * KT + kt) * 64 + lane];
+    {
+      if (t + 1 < NT) request(t + 1);
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+      acc = mfma16(dvf[0], vf[t & 1][0], acc);
+      acc = mfma16(dvf[1], vf[t & 1][1], acc);
+      pair_unpack(pw[t & 1][0], odd, pp[t][0], pp[t][1]);
+      pair_unpack(pw[t & 1][1], odd, pp[t][2], pp[t][3]);
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int m = acc_row(e, half);
-        const bf16 val = (bf16)(a.scale * pp[t][e] * (dp[t][e] - dot[e]));
-        ds[(int64_t)m * a.K + kt * 32] = val;
-        dbd[(int64_t)m * a.R - m + kt * 32] = val;
-        const float f = (float)val;
-        tot[e] += f;
-        if ((mw[e >> 2] >> (8 * (e & 3))) & 2u) d1[e] += f;
+      for (int v = 0; v < 4; ++v) {
+        if (kt0 + t >= KT) pp[t][v] = 0.f;
+        dp[t][v] = acc[v];
+        dot[v] = fmaf(pp[t][v], acc[v], dot[v]);
       }
     }
   }
 #pragma unroll
-  for (int e = 0; e < 16; ++e) { tot[e] = half_sum(tot[e]); d1[e] = half_sum(d1[e]); }
-  if (il == 0) {
+  for (int v = 0; v < 4; ++v) dot[v] = group_sum(dot[v]);
+  if (n == 0) {
 #pragma unroll
-    for (int e = 0; e < 16; ++e) { st[wave][acc_row(e, half)] = tot[e]; s1[wave][acc_row(e, half)] = d1[e]; }
+    for (int v = 0; v < 4; ++v) sd[wave][4 * g + v] = dot[v];
   }
   __syncthreads();
-  if (wave == 0 && half == 0) {
+  float D = 0.f;
+  for (int w = 0; w < nw; ++w) D += sd[w][n];
+  float tot[4], d1[4];
+#pragma unroll
+  for (int v = 0; v < 4; ++v) { dot[v] = lane_read(D, (4 * g + v) << 2); tot[v] = 0.f; d1[v] = 0.f; }
+  bf16* ds = reinterpret_cast<bf16*>(a.ds) + ((int64_t)bh * a.QQ + ii0 + 4 * g + (odd ? 1 : 0)) * a.K + (n & ~1);
+  // column j of row i lands in column j + Q - i of the un-shifted copy
+  bf16* dbd = reinterpret_cast<bf16*>(a.dbd) + ((int64_t)bh * a.QQ + ii0 + 4 * g) * a.R + n + a.Q - i0 - 4 * g;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    if (kt0 + t < KT) {
+      const int kt = kt0 + t;
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const bf16 val = (bf16)(a.scale * pp[t][v] * (dp[t][v] - dot[v]));
+        dbd[(int64_t)v * a.R - v + kt * 16] = val;
+        const float f = (float)val;
+        pp[t][v] = f;
+        tot[v] += f;
+        d1[v] += bit_select(sbits, 4 * t + v, f);
+      }
+      *reinterpret_cast<uint32_t*>(ds + kt * 16) = pair_pack(pp[t][0], pp[t][1], odd);
+      *reinterpret_cast<uint32_t*>(ds + 2 * (int64_t)a.K + kt * 16) = pair_pack(pp[t][2], pp[t][3], odd);
+    }
+  }
+#pragma unroll
+  for (int v = 0; v < 4; ++v) { tot[v] = group_sum(tot[v]); d1[v] = group_sum(d1[v]); }
+  if (n == 0) {
+#pragma unroll
+    for (int v = 0; v < 4; ++v) { st[wave][4 * g + v] = tot[v]; s1[wave][4 * g + v] = d1[v]; }
+  }
+  __syncthreads();
+  if (wave == 0 && g == 0) {
     float T = 0.f, S1 = 0.f;
-    for (int w = 0; w < nw; ++w) { T += st[w][il]; S1 += s1[w][il]; }
+    for (int w = 0; w < nw; ++w) { T += st[w][n]; S1 += s1[w][n]; }
     // A softmax row's score gradients sum to zero; what the rounded probabilities and the rounded ds leave of that sum is
     // noise that would be multiplied by a whole embedding row: it is taken out of the two segment sums in proportion to the
     // number of keys each one covers.
-    const float n1 = a.nseg ? a.nseg[b * a.Q + i0 + il] : 0.f;
+    const float n1 = a.nseg ? a.nseg[b * a.Q + i0 + n] : 0.f;
     const float excess = T / (float)a.K;
     const float o0 = (T - S1) - excess * ((float)a.K - n1);
     const float o1 = S1 - excess * n1;
-    *reinterpret_cast<f32x2*>(a.defs + ((int64_t)bh * a.QQ + ii0 + il) * 2) = f32x2{o0, o1};
+    *reinterpret_cast<f32x2*>(a.defs + ((int64_t)bh * a.QQ + ii0 + n) * 2) = f32x2{o0, o1};
   }
 }
-
 
 }  // namespace
 
 bool ds_xl_scores_fit(int dtype, int head_dim, int Q, int K, int R) {
-  return dtype == DS_BF16 && head_dim == HD && Q > 0 && Q % 32 == 0 && K >= 32 && K % 32 == 0 && K <= 32 * NT * MAXW && R == K + Q;
+  return dtype == DS_BF16 && head_dim == HD && Q > 0 && Q % RB == 0 && K >= 16 && K % 16 == 0 && K <= 16 * NT * MAXW && R == K + Q;
 }
 
-size_t ds_xl_meta_bytes(int QQ, int K, int B) { return (size_t)B * QQ * K; }
+size_t ds_xl_meta_bytes(int QQ, int K, int B) { return (size_t)B * (QQ / RB) * ((K + 127) / 128) * 64 * sizeof(uint2); }
 
 int ds_xl_pack_meta(int Q, int QQ, int K, int B, const float* mask, const uint8_t* seg, void* meta, float* nseg, hipStream_t s) {
-  DS_CHECK_ARG(Q > 0 && QQ % Q == 0 && Q % 32 == 0 && K % 32 == 0 && B > 0 && meta && ds_aligned16(meta), "ds_xl_pack_meta: bad shape or pointer");
-  const int64_t n = (int64_t)B * (QQ / 32) * (K / 32) * 64;
-  hipLaunchKernelGGL(xl_pack_meta_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, Q, QQ, K, B, mask, seg, (u32x4*)meta);
+  DS_CHECK_ARG(Q > 0 && QQ % Q == 0 && Q % RB == 0 && K % 16 == 0 && B > 0 && meta && ds_aligned16(meta), "ds_xl_pack_meta: bad shape or pointer");
+  const int64_t n = (int64_t)B * (QQ / RB) * ((K + 127) / 128) * 64;
+  hipLaunchKernelGGL(xl_pack_meta_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, Q, QQ, K, B, mask, seg, (uint2*)meta);
   if (nseg && seg) hipLaunchKernelGGL(xl_seg_count_kernel, dim3((unsigned)((Q * B + 3) / 4)), dim3(256), 0, s, Q, K, B, seg, nseg);
   DS_CHECK_LAUNCH();
   return DS_OK;
@@ -352,10 +391,15 @@ int ds_xl_scores_fwd(const XlScoreArgs* a, hipStream_t s) {
   DS_CHECK_ARG(a->qw && a->qr && a->qs && a->k && a->kr && a->seg_emb && a->p, "ds_xl_scores_fwd: null pointer");
   DS_CHECK_ARG(ds_aligned16(a->qw) && ds_aligned16(a->qr) && ds_aligned16(a->qs) && ds_aligned16(a->k) && ds_aligned16(a->kr) &&
                ds_aligned16(a->meta), "ds_xl_scores_fwd: operands must be 16-byte aligned");
-  const int nw = (a->K / 32 + NT - 1) / NT;
-  // q k^T once, q k_r^T over 5 window tiles per 4 key tiles
-  ds_prof_scope prof(s, "xl_scores_fwd_kernel", 2.0 * (1.0 + 1.25) * a->B * a->N * (double)a->QQ * a->K * HD, "FLOP");
-  hipLaunchKernelGGL(xl_scores_fwd_kernel, dim3(a->QQ / 32, a->B * a->N), dim3(64 * nw), 0, s, *a, ds_launch_prio);
+  const int nw = (a->K + 127) / 128;
+  // q k^T once, q k_r^T over 9 window tiles per 8 key tiles
+  ds_prof_scope prof(s, "xl_scores_fwd_kernel", 2.0 * (1.0 + 1.125) * a->B * a->N * (double)a->QQ * a->K * HD, "FLOP");
+  const dim3 grid(a->QQ / RB, a->B * a->N), block(64 * nw);
+  const bool full = a->K % 128 == 0;
+  if (full && a->meta) hipLaunchKernelGGL((xl_scores_fwd_kernel<true, true>), grid, block, 0, s, *a, ds_launch_prio);
+  else if (full) hipLaunchKernelGGL((xl_scores_fwd_kernel<true, false>), grid, block, 0, s, *a, ds_launch_prio);
+  else if (a->meta) hipLaunchKernelGGL((xl_scores_fwd_kernel<false, true>), grid, block, 0, s, *a, ds_launch_prio);
+  else hipLaunchKernelGGL((xl_scores_fwd_kernel<false, false>), grid, block, 0, s, *a, ds_launch_prio);
   DS_CHECK_LAUNCH();
   return DS_OK;
 }
@@ -365,9 +409,9 @@ int ds_xl_scores_bwd(const XlScoreArgs* a, hipStream_t s) {
   DS_CHECK_ARG(a->dvec && a->v && a->p && a->ds && a->dbd && a->defs, "ds_xl_scores_bwd: null pointer");
   DS_CHECK_ARG(ds_aligned16(a->dvec) && ds_aligned16(a->v) && ds_aligned16(a->meta) && (reinterpret_cast<uintptr_t>(a->defs) & 7) == 0,
                "ds_xl_scores_bwd: operands must be 16-byte aligned");
-  const int nw = (a->K / 32 + NT - 1) / NT;
+  const int nw = (a->K + 127) / 128;
   ds_prof_scope prof(s, "xl_scores_bwd_kernel", (double)a->B * a->N * a->QQ * (3.0 * a->K * 2 + 0.0), "B");
-  hipLaunchKernelGGL(xl_scores_bwd_kernel, dim3(a->QQ / 32, a->B * a->N), dim3(64 * nw), 0, s, *a, ds_launch_prio);
+  hipLaunchKernelGGL(xl_scores_bwd_kernel, dim3(a->QQ / RB, a->B * a->N), dim3(64 * nw), 0, s, *a, ds_launch_prio);
   DS_CHECK_LAUNCH();
   return DS_OK;
 }

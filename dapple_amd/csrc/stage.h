@@ -111,30 +111,9 @@ static inline int ds_stage_acquire_slot(ds_stage* h, int slot) {
 
 int ds_bert_stage_create(const ds_stage_cfg* cfg, hipStream_t stream, ds_stage** out);
 
-// Fused forward of XLNet's relative attention for bf16 and head size 64 (attention.hip): for every stacked query row
-// i' (stream * Q + i), sample b and head n
-//   score[j] = (qw[i'] . k[j] + qr[i'] . kr[j + Q - i] + ef[seg(i, j, b)]) * scale - 1e30 * mask[i'][j][b]
-//   p = softmax_j score (written out, bf16, for the backward pass),  vec[i'] = sum_j p[j] v[j].
-struct XlAttnArgs {
-  const void *qw, *qr, *qs;   // bf16 [QQ][B][H]: q + the three biases; row stride ldq, head n at column n*64
-  int64_t ldq;
-  const void* kv;             // bf16 [K][B][2H]: k at column 0, v at column H of each row; row stride ldkv
-  int64_t ldkv;
-  const void* kr;             // bf16 [R][H]: the projected position embeddings; row stride ldkr
-  int64_t ldkr;
-  const float* seg_emb;       // fp32 [2][H]
-  const float* mask_t;        // fp32 [B][K][QQ] (key-major copy of the masks) or null
-  const uint8_t* seg_t;       // uint8 [B][K][Q] (key-major copy of the segment matrix) or null
-  void* p;                    // bf16 [B*N][QQ][K]
-  void* vec;                  // bf16, layout of qw
-  int Q, QQ, K, R, B, N, H;
-  float scale;
-};
-// true when the shapes fit the kernel (head size 64, Q a multiple of 64, K a multiple of 32, R = K + Q)
-bool ds_xl_attention_fits(int dtype, int head_dim, int Q, int K, int R);
-int ds_xl_attention_fwd(const XlAttnArgs* a, hipStream_t stream);
 // Scores + softmax of XLNet's relative attention with nothing but bf16 probabilities (forward) or bf16 score gradients
-// (backward) leaving the kernel (attention_xl.hip); operands as in XlAttnArgs.
+// (backward) leaving the kernel (attention_xl.hip): for every stacked query row i' (stream * Q + i), sample b and head n
+//   score[j] = (qw[i'] . k[j] + qr[i'] . kr[j + Q - i] + ef[seg(i, j, b)]) * scale - 1e30 * mask[i'][j][b],  p = softmax_j score
 struct XlScoreArgs {
   const void *qw, *qr, *qs;   // bf16 [QQ][B][H]: q + the three biases; row stride ldq, sample b at column b*H
   int64_t ldq;
@@ -154,7 +133,7 @@ struct XlScoreArgs {
   int Q, QQ, K, R, B, N, H;
   float scale;
 };
-// bf16, head size 64, Q and K multiples of 32, K <= 1024, R = K + Q
+// bf16, head size 64, Q and K multiples of 16, K <= 1024, R = K + Q
 bool ds_xl_scores_fit(int dtype, int head_dim, int Q, int K, int R);
 size_t ds_xl_meta_bytes(int QQ, int K, int B);
 // mask fp32 [QQ][K][B] (non-zero = masked) and seg uint8 [Q][K][B], either may be null -> meta; nseg (may be null) <- seg

@@ -199,15 +199,6 @@ __global__ __launch_bounds__(256) void xl_seg_bwd_kernel(int QQ, int B, int N, i
   }
 }
 
-// out[b][j][i] = in[i][j][b]: the key-major copies of the masks / the segment matrix that the fused attention reads
-template <typename T>
-__global__ __launch_bounds__(256) void xl_key_major_kernel(int I, int K, int B, const T* __restrict__ in, T* __restrict__ out) {
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= (int64_t)I * K * B) return;
-  const int i = (int)(idx % I), j = (int)((idx / I) % K), b = (int)(idx / ((int64_t)I * K));
-  out[idx] = in[((int64_t)i * K + j) * B + b];
-}
-
 struct LayerOff { size_t x, qw, qr, qs, kv, p, vec, z1, y1, u, hh, z2, st1, st2; };
 
 struct XlnetStage : ds_stage {
@@ -221,8 +212,7 @@ struct XlnetStage : ds_stage {
   char* pe = nullptr;
   // stash
   char* stash_base = nullptr;
-  size_t slot_bytes = 0, mask_off = 0, seg_off = 0, mem_off = 0, maskt_off = 0, segt_off = 0, meta_off = 0, nseg_off = 0;
-  bool fused_fwd = false;  // forward attention in one kernel (bf16, head size 64, seq a multiple of 64)
+  size_t slot_bytes = 0, mask_off = 0, seg_off = 0, mem_off = 0, meta_off = 0, nseg_off = 0;
   // scores + softmax (forward) and score gradients (backward) in one kernel each, no fp32 score matrices (attention_xl.hip)
   bool score_fused = false;
   // bf16 with xc.residual_fp32: the residual stream (the sums in front of both LayerNorms, the LayerNorm outputs that feed
@@ -293,13 +283,8 @@ struct XlnetStage : ds_stage {
     mask_off = sa.reserve((size_t)S * Q * K * B * 4);
     seg_off = sa.reserve((size_t)Q * K * B);
     mem_off = sa.reserve((size_t)L * (Mm > 0 ? Mm : 1) * B * H * esz);
-    fused_fwd = xc.fused_attention == DS_XL_ATTN_ONE_KERNEL && ds_xl_attention_fits(dtype, D, Q, K, R);
     score_fused = xc.fused_attention != DS_XL_ATTN_SEPARATE && ds_xl_scores_fit(dtype, D, Q, K, R);
     rs32 = dtype == DS_BF16 && xc.residual_fp32 != 0 && H % 8 == 0 && H <= 2048;
-    if (fused_fwd) {
-      maskt_off = sa.reserve((size_t)B * K * S * Q * 4);
-      segt_off = sa.reserve((size_t)B * K * Q);
-    }
     if (score_fused) {
       meta_off = sa.reserve(ds_xl_meta_bytes(S * Q, K, B));
       nseg_off = sa.reserve((size_t)Q * B * 4);
@@ -462,19 +447,6 @@ struct XlnetStage : ds_stage {
     if (score_fused && (masks || seg_mat))
       DS_PROPAGATE(ds_xl_pack_meta(Q, S * Q, K, B, masks ? (const float*)(sp + mask_off) : nullptr,
                                    seg_mat ? (const uint8_t*)(sp + seg_off) : nullptr, sp + meta_off, (float*)(sp + nseg_off), stream));
-    if (fused_fwd) {
-      if (masks) {
-        const int64_t n = (int64_t)S * Q * K * B;
-        hipLaunchKernelGGL(xl_key_major_kernel<float>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, S * Q, K, B,
-                           (const float*)(sp + mask_off), (float*)(sp + maskt_off));
-      }
-      if (seg_mat) {
-        const int64_t n = (int64_t)Q * K * B;
-        hipLaunchKernelGGL(xl_key_major_kernel<uint8_t>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, Q, K, B,
-                           (const uint8_t*)(sp + seg_off), (uint8_t*)(sp + segt_off));
-      }
-      DS_CHECK_LAUNCH();
-    }
     return DS_OK;
   }
 
@@ -542,18 +514,7 @@ struct XlnetStage : ds_stage {
                              w[b + X_RR], w[b + X_RS], (float*)(sp + t.qw), (float*)(sp + t.qr), (float*)(sp + t.qs));
         DS_CHECK_LAUNCH();
       }
-      if (fused_fwd) {
-        XlAttnArgs xa;
-        xa.qw = sp + t.qw; xa.qr = sp + t.qr; xa.qs = sp + t.qs; xa.ldq = (int64_t)B * H;
-        xa.kv = sp + t.kv; xa.ldkv = (int64_t)B * 2 * H;
-        xa.kr = kr[l]; xa.ldkr = H;
-        xa.seg_emb = w[b + X_SEG];
-        xa.mask_t = has_mask[slot] ? (const float*)(sp + maskt_off) : nullptr;
-        xa.seg_t = has_seg[slot] ? (const uint8_t*)(sp + segt_off) : nullptr;
-        xa.p = sp + t.p; xa.vec = sp + t.vec;
-        xa.Q = Q; xa.QQ = S * Q; xa.K = K; xa.R = R; xa.B = B; xa.N = N; xa.H = H; xa.scale = scale;
-        DS_PROPAGATE(ds_xl_attention_fwd(&xa, stream));
-      } else if (score_fused) {
+      if (score_fused) {
         const int QQ = S * Q;
         XlScoreArgs xa;
         memset(&xa, 0, sizeof(xa));

@@ -381,21 +381,20 @@ class XlnetStage(Stage):
 
 
 def xlnet_stage(num_layers, hidden, heads, ffn, batch, seq, dtype, stash_slots, mem_len=0, streams=1, first_layer=0,
-                ln_eps=1e-14, device="cuda:0", fused_attention=False, residual_fp32=True):
+                ln_eps=1e-14, device="cuda:0", attention="auto", residual_fp32=True):
     """An XLNet stage of ``num_layers`` relative-attention layers (xlnet/models/slice_xlnet.py:164-180).
-    ``fused_attention`` (``ds_xlnet_cfg.fused_attention``): False / "auto" = scores, relative shift and softmax as one kernel
-    per pass where the shape allows; True / "one_kernel" = the forward pass also multiplies by v in that kernel;
-    "separate" = every product and the softmax as launches of their own.  ``residual_fp32`` (bf16 stages): keep the
+    ``attention`` (``ds_xlnet_cfg.fused_attention``): "auto" = scores, relative shift and softmax as one kernel per pass where
+    the shape allows; "separate" = every product and the softmax as launches of their own.  ``residual_fp32`` (bf16 stages): keep the
     residual stream in fp32 (``ds_xlnet_cfg.residual_fp32``)."""
     lib = _lib.load()
     cfg = XlnetCfg()
     cfg.dtype, cfg.num_layers, cfg.hidden, cfg.heads, cfg.ffn = _dtype_code(dtype), num_layers, hidden, heads, ffn
     cfg.batch, cfg.seq, cfg.mem_len, cfg.streams = batch, seq, mem_len, streams
     cfg.ln_eps, cfg.first_layer, cfg.stash_slots = ln_eps, first_layer, stash_slots
-    modes = {False: 0, "auto": 0, True: 1, "one_kernel": 1, "separate": 2}
-    if fused_attention not in modes:
-        raise ValueError("fused_attention must be one of %r" % (list(modes),))
-    cfg.fused_attention = modes[fused_attention]
+    modes = {"auto": 0, "separate": 1}
+    if attention not in modes:
+        raise ValueError("attention must be one of %r" % (list(modes),))
+    cfg.fused_attention = modes[attention]
     cfg.residual_fp32 = 1 if residual_fp32 else 0
     h = C.c_void_p()
     with torch.cuda.device(torch.device(device)):

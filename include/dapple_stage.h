@@ -379,7 +379,7 @@ int ds_gnmt_stage_set_decoder_inputs(ds_stage* h, int slot, const int32_t* targe
  * seg_emb ([2, hidden]), attn_ln/{gamma,beta}, ff/{W1,b1,W2,b2}, ff_ln/{gamma,beta}.
  * mem_len > 0 and streams == 2 go beyond what the reference builds (it hard-wires memory length 0 and has
  * the content stream only, lambda_funcs.py:20,36) and follow the XLNet formulation. */
-enum { DS_XL_ATTN_AUTO = 0, DS_XL_ATTN_ONE_KERNEL = 1, DS_XL_ATTN_SEPARATE = 2 };
+enum { DS_XL_ATTN_AUTO = 0, DS_XL_ATTN_SEPARATE = 1 };
 typedef struct ds_xlnet_cfg {
   int dtype;
   int num_layers, hidden, heads, ffn;
@@ -389,12 +389,10 @@ typedef struct ds_xlnet_cfg {
   int stash_slots;
   int fused_attention; /* how the attention scores are computed; results agree to rounding:
                           DS_XL_ATTN_AUTO (0): where the shape allows (bf16, head size 64, seq and mem_len + seq multiples
-                            of 32, mem_len + seq <= 1024) scores, relative shift and softmax are one kernel forward and one
+                            of 16, mem_len + seq <= 1024) scores, relative shift and softmax are one kernel forward and one
                             backward, and no fp32 score matrix exists; masks then count as 0 / non-zero.  Other shapes run
                             as DS_XL_ATTN_SEPARATE.
-                          DS_XL_ATTN_ONE_KERNEL (1): the forward pass also multiplies by v in the same kernel (seq a
-                            multiple of 64); slower in the step at the benchmark shape.
-                          DS_XL_ATTN_SEPARATE (2): every product and the softmax as launches of their own, fp32 scores
+                          DS_XL_ATTN_SEPARATE (1): every product and the softmax as launches of their own, fp32 scores
                             in the workspace. */
   int residual_fp32;   /* bf16 only, 1: the residual stream (the sums in front of both LayerNorms, the LayerNorm outputs that
                           feed the next sum, the same chain of gradients) stays in fp32, bf16 is what the GEMMs read: the

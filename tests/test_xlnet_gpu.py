@@ -14,7 +14,7 @@ ADT = {"fp32": torch.float32, "bf16": torch.bfloat16}
 
 
 def run_case(dtype, L, H, N, F, B, Q, Mm, S, M, K=2, seed=0, use_seg=True, mask_kind="perm", stddev=0.1, perturb=True,
-             odtype=torch.float64, overlap=False, fused=False):
+             odtype=torch.float64, overlap=False, attention="auto"):
     adt = ADT[dtype]
     klen = Mm + Q
     w_np = synthetic.xlnet_weights(synthetic.SEED_WEIGHT + seed, L, H, N, F, stddev=stddev, perturb=perturb)
@@ -31,7 +31,7 @@ def run_case(dtype, L, H, N, F, B, Q, Mm, S, M, K=2, seed=0, use_seg=True, mask_
     else:
         masks_np = None
 
-    stage = runtime.xlnet_stage(L, H, N, F, B, Q, dtype, stash_slots=K, mem_len=Mm, streams=S, fused_attention=fused)
+    stage = runtime.xlnet_stage(L, H, N, F, B, Q, dtype, stash_slots=K, mem_len=Mm, streams=S, attention=attention)
     stage.bind(w_np)
     if overlap:
         stage.enable_overlap()     # backward passes on the handle's second stream
@@ -115,35 +115,20 @@ def test_config4_shape_one_layer_bf16():
              seed=c["index"], stddev=0.02, perturb=False, odtype=torch.float32)
 
 
-@pytest.mark.parametrize("Q,Mm,S,B,mask_kind,use_seg", [(64, 32, 2, 2, "perm", True), (128, 0, 1, 1, "input", True),
-                                                         (64, 96, 2, 1, "perm", False), (64, 0, 1, 2, None, True)])
-def test_fused_forward_attention_shapes(Q, Mm, S, B, mask_kind, use_seg):
-    # the forward attention as one kernel (scores, relative shift, softmax, P V, probabilities for the backward pass),
-    # an option of the stage for head size 64 and seq a multiple of 64; key counts of 96, 128, 160 and 64 cover partial
-    # and single chunks; the permutation masks include rows whose keys in a 32-key step are all masked
-    run_case("bf16", L=2, H=128, N=2, F=256, B=B, Q=Q, Mm=Mm, S=S, M=2, K=1, seed=11 + Q + Mm, use_seg=use_seg, mask_kind=mask_kind,
-             fused=True)
-
-
 @pytest.mark.parametrize("Q,Mm,S,B,mask_kind,use_seg", [(32, 0, 1, 4, "input", True), (64, 32, 2, 2, "perm", True),
                                                          (32, 96, 2, 1, "perm", False), (96, 160, 1, 2, None, True),
-                                                         (64, 576, 2, 1, "perm", True), (64, 0, 1, 2, None, False)])
+                                                         (64, 576, 2, 1, "perm", True), (64, 0, 1, 2, None, False),
+                                                         (48, 16, 2, 2, "perm", True), (16, 0, 1, 4, "input", True)])
 def test_score_kernels_shapes(Q, Mm, S, B, mask_kind, use_seg):
-    # the default path for bf16, head size 64 and seq, mem_len + seq multiples of 32: scores, relative shift and softmax in one
-    # kernel per pass, 32 query rows and all keys per block.  Key counts 32 .. 640 give blocks of one to five waves, waves with
-    # one to four key tiles, a second stream, rows whose every key is masked (permutation masks), no masks / one segment (no
+    # the default path for bf16, head size 64 and seq, mem_len + seq multiples of 16: scores, relative shift and softmax in one
+    # kernel per pass, 16 query rows and all keys per block.  Key counts 32 .. 640 give blocks of one to five waves, waves with
+    # two to eight key tiles, a second stream, rows whose every key is masked (permutation masks), no masks / one segment (no
     # packed bits at all)
     run_case("bf16", L=2, H=128, N=2, F=256, B=B, Q=Q, Mm=Mm, S=S, M=2, K=1, seed=31 + Q + Mm, use_seg=use_seg, mask_kind=mask_kind)
 
 
 def test_separate_launches_at_a_shape_the_score_kernels_take():
-    run_case("bf16", L=2, H=128, N=2, F=256, B=2, Q=64, Mm=32, S=2, M=2, K=1, seed=5, fused="separate")
-
-
-def test_fused_forward_attention_config4_shape():
-    c = synthetic.CONFIGS["xlnet36_half"]
-    run_case("bf16", 1, c["hidden"], c["heads"], c["ffn"], c["micro_batch"], c["seq"], c["mem_len"], c["streams"], M=1, K=1,
-             seed=c["index"], stddev=0.02, perturb=False, odtype=torch.float32, fused=True)
+    run_case("bf16", L=2, H=128, N=2, F=256, B=2, Q=64, Mm=32, S=2, M=2, K=1, seed=5, attention="separate")
 
 
 @pytest.mark.parametrize("dtype", ["fp32", "bf16"])
