@@ -17,6 +17,10 @@ library beside ``torch.matmul`` (hipBLASLt / rocBLAS) on the same operands: TFLO
 
 ``attention``: the fused attention kernels at the BERT-48 half-stage's shape (2 samples, 16 heads, 512 positions, head
 size 64, bf16), three launches each, for the same counter runs as ``gemms`` (matrix-core busy cycles, HBM traffic).
+
+``xl_scores``: the score kernels of XLNet's relative attention at the XLNet-36 half-stage's shape (two streams of 512
+positions + 384 memory positions, 16 heads, head size 64, bf16, masks and segments), five launches each, with their
+algorithmic bytes and FLOP printed.
 """
 import sys
 
@@ -113,6 +117,27 @@ def attention():
     print("attn_fwd_kernel: %d FLOP per launch; attn_bwd_dq_kernel: %d; attn_bwd_dkv_kernel: %d" % (4 * unit, 6 * unit, 8 * unit))
 
 
+def xl_scores():
+    seq, mem, streams, batch, heads, d = 512, 384, 2, 1, 16, 64
+    rows, klen, H = streams * seq, mem + seq, heads * d
+    bf = torch.bfloat16
+    r = lambda *sh: torch.randn(*sh, device="cuda").to(bf)
+    qw, qr, qs, kv, kr, dvec = r(rows, batch, H), r(rows, batch, H), r(rows, batch, H), r(klen, batch, 2 * H), r(klen + seq, H), r(rows, batch, H)
+    seg_emb = torch.randn(2, H, device="cuda")
+    masks = (torch.rand(rows, klen, batch, device="cuda") < 0.3).float()
+    seg = (torch.rand(seq, klen, batch, device="cuda") < 0.4).to(torch.uint8)
+    meta, nseg = ops.xlnet_scores_pack(seq, rows, klen, batch, masks, seg)
+    dbd = torch.zeros(batch * heads, rows, klen + seq, dtype=bf, device="cuda")
+    for _ in range(5):
+        p = ops.xlnet_scores_fwd(qw, qr, qs, kv, kr, seg_emb, seq, heads, 0.125, meta)
+        ops.xlnet_scores_bwd(kv, p, dvec, seq, heads, 0.125, meta, nseg, dbd)
+    torch.cuda.synchronize()
+    n = batch * heads * rows * klen
+    print("xl_scores_fwd_kernel: %d bytes per launch (write p; operands %d), %d FLOP (q k^T and the 9/8 window of q kr^T)"
+          % (2 * n, 2 * (3 * rows * batch * H + klen * batch * H + (klen + seq) * H), int(2 * 2.125 * n * d)))
+    print("xl_scores_bwd_kernel: %d bytes per launch (read p, write ds and the band of dbd), %d FLOP (dvec v^T)" % (6 * n, 2 * n * d))
+
+
 def elementwise():
     bf = torch.bfloat16
     rows, h, f = 1024, 1024, 4096
@@ -156,6 +181,8 @@ if __name__ == "__main__":
         elementwise()
     elif len(sys.argv) > 1 and sys.argv[1] == "attention":
         attention()
+    elif len(sys.argv) > 1 and sys.argv[1] == "xl_scores":
+        xl_scores()
     elif len(sys.argv) > 1 and sys.argv[1] == "gemm_table":
         gemm_table()
     else:

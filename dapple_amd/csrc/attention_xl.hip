@@ -12,8 +12,14 @@
 // 16 x 16 tile can touch (two accumulators, the second one shared with the next key tile), and the element of row m, key
 // column n is column n + 15 - m of that window - for a fixed register (fixed m within the lane group) a rotation of the
 // group's lanes, i.e. one ds_bpermute after the source lanes picked the accumulator they are asked for.
+// Key, position and value rows reach the MFMA operand registers through LDS: a lane-per-row load straight into operand order
+// is one 16-byte request per lane to the vector cache (64 per instruction, four times what contiguous lanes cost), which made
+// the cache's request rate the limit of both kernels.  Every wave stages its own 16-row tiles (LDS DMA, eight lanes per row,
+// chunks XOR-swizzled by the row, two stages) and reads them back in operand order; no barrier is involved.
 // Of the two segment scores only their difference matters (a softmax row ignores a constant), and the mask / segment bits
 // of a lane's 32 scores are two 32-bit words, turned into addends with a bit-field extract and an AND each.
+#include <string.h>
+
 #include "common.h"
 #include "stage.h"
 
@@ -106,6 +112,45 @@ __global__ __launch_bounds__(256) void xl_seg_count_kernel(int Q, int K, int B, 
   if (lane == 0) nseg[w] = n;
 }
 
+typedef __attribute__((address_space(3))) void* lds_vptr;
+typedef __attribute__((address_space(1))) void* glb_vptr;
+constexpr int TILE_BYTES = 16 * HD * 2;   // 16 rows of 64 bf16
+// vmcnt(n): at most n of this wave's vector-memory operations still in flight
+__device__ __forceinline__ void wait_vm4() { __builtin_amdgcn_s_waitcnt((4 & 15) | (7 << 4) | (15 << 8)); }
+__device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt((0 & 15) | (7 << 4) | (15 << 8)); }
+// Before a stage is handed to the DMA again every LDS read of it must have RETURNED: LDS DMA writes do not queue behind the
+// wave's ds_read instructions, and the compiler, which orders the two only by issue, otherwise moves the next request above
+// the wait that completes the previous tile's last read.
+__device__ __forceinline__ void stage_free() {
+  __builtin_amdgcn_s_waitcnt(15 | (3 << 14) | (7 << 4) | (0 << 8));   // lgkmcnt(0)
+  __builtin_amdgcn_sched_barrier(0);
+}
+// LDS tile: [16 rows][8 chunks of 16 bytes], chunk index XOR-swizzled by the row so that the 16 lanes reading one chunk
+// column of 16 rows spread over the banks (64 banks: a 256-byte line is two rows)
+__device__ __forceinline__ int tile_swz(int row) {
+  const int t = (row >> 1) & 7;
+  return ((t & 1) << 2) | (t >> 1);
+}
+// rows row0 .. row0 + 15 (clamped to last_row) of a row-major matrix, 64 columns from `base` -> one LDS tile; two instructions,
+// eight lanes per row
+__device__ __forceinline__ void tile16_fill(char* lds, const bf16* base, int64_t ld, int row0, int last_row, int lane) {
+#pragma unroll
+  for (int c = 0; c < 2; ++c) {
+    const int r = c * 8 + (lane >> 3), pc = lane & 7;
+    int gr = row0 + r;
+    gr = gr < last_row ? gr : last_row;
+    const bf16* src = base + (int64_t)gr * ld + (pc ^ tile_swz(r)) * 8;
+    __builtin_amdgcn_global_load_lds((glb_vptr)src, (lds_vptr)(lds + c * 1024), 16, 0, 0);
+  }
+}
+// MFMA operand slices of lane (g, n) from a tile: row n, k index 32 ks + 8 g .. + 7
+__device__ __forceinline__ void tile16_frags(const char* lds, int g, int n, bf16x8 (&f)[2]) {
+  const char* row = lds + n * (HD * 2);
+  const int z = tile_swz(n);
+  f[0] = *reinterpret_cast<const bf16x8*>(row + ((g ^ z) << 4));
+  f[1] = *reinterpret_cast<const bf16x8*>(row + (((g + 4) ^ z) << 4));
+}
+
 // this lane's two 16-byte MFMA operand slices of one 64-wide row (k index 32 ks + 8 (lane / 16) .. + 7; row_ptr includes 8 (lane / 16))
 __device__ __forceinline__ void load_frags(const bf16* row_ptr, bf16x8 (&f)[2]) {
   f[0] = *reinterpret_cast<const bf16x8*>(row_ptr);
@@ -117,7 +162,7 @@ __device__ __forceinline__ void load_frags(const bf16* row_ptr, bf16x8 (&f)[2]) 
 template <bool FULL, bool META>
 __global__ __launch_bounds__(64 * MAXW) void xl_scores_fwd_kernel(XlScoreArgs a, int prio) {
   ds_wave_prio(prio);
-  __shared__ float sm[MAXW][RB], sl[MAXW][RB];
+  extern __shared__ __attribute__((aligned(16))) char lds[];
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), g = lane >> 4, n = lane & 15;
   const int nw = blockDim.x >> 6;
   int bh, blk;
@@ -127,29 +172,27 @@ __global__ __launch_bounds__(64 * MAXW) void xl_scores_fwd_kernel(XlScoreArgs a,
   const int KT = a.K >> 4;
   const int kt0 = wave * NT;
   const int64_t qoff = (int64_t)(ii0 + n) * a.ldq + (int64_t)b * a.H + hd * HD;
-  const bf16* kb = reinterpret_cast<const bf16*>(a.k) + (int64_t)b * a.ldk_b + hd * HD + 8 * g;
-  const bf16* krb = reinterpret_cast<const bf16*>(a.kr) + hd * HD + 8 * g;
-  // The tile loop has no branches (a join would make every wait for operands a wait for all loads in flight): tiles past the
-  // last key read clamped rows and their scores are replaced below.  Operands are requested two tiles ahead.
-  bf16x8 kf[3][2], krf[3][2];
+  const bf16* kb = reinterpret_cast<const bf16*>(a.k) + (int64_t)b * a.ldk_b + hd * HD;
+  const bf16* krb = reinterpret_cast<const bf16*>(a.kr) + hd * HD;
+  float (*sm)[RB] = reinterpret_cast<float (*)[RB]>(lds + nw * 4 * TILE_BYTES);
+  float (*sl)[RB] = sm + MAXW;
+  char* stage = lds + wave * 4 * TILE_BYTES;   // two stages of (key tile, position tile)
+  // The tile loop has no branches: tiles past the last key stage clamped rows and their scores are replaced below.  The
+  // next tile's rows are requested before the current tile is worked on.
   auto request = [&](int t) {
-    int j = (kt0 + t) * 16 + n;
-    if (!FULL) j = j < a.K ? j : a.K - 1;
-    load_frags(kb + (int64_t)j * a.ldk, kf[t % 3]);
-    int r = (kt0 + t) * 16 + a.Q - i0 + 1 + n;   // second half of the window: k_r rows j0 + Q - i0 - 15 + 16 + lane
-    r = r < a.R ? r : a.R - 1;
-    load_frags(krb + (int64_t)r * a.ldkr, krf[t % 3]);
+    char* st = stage + (t & 1) * 2 * TILE_BYTES;
+    tile16_fill(st, kb, a.ldk, (kt0 + t) * 16, a.K - 1, lane);
+    tile16_fill(st + TILE_BYTES, krb, a.ldkr, (kt0 + t) * 16 + a.Q - i0 + 1, a.R - 1, lane);   // second half of the window
   };
   bf16x8 qwf[2], qrf[2], f0[2];
   load_frags(reinterpret_cast<const bf16*>(a.qr) + qoff + 8 * g, qrf);
   {
     int r = kt0 * 16 + a.Q - i0 - 15 + n;   // first half of the first window
     if (!FULL) r = r < a.R ? r : a.R - 1;
-    load_frags(krb + (int64_t)r * a.ldkr, f0);
+    load_frags(krb + (int64_t)r * a.ldkr + 8 * g, f0);
   }
   load_frags(reinterpret_cast<const bf16*>(a.qw) + qoff + 8 * g, qwf);
   request(0);
-  request(1);
   // de[v]: ef[1] - ef[0] of this lane's query row 4 g + v (a row's softmax ignores ef[0])
   float de[4] = {0.f, 0.f, 0.f, 0.f};
   uint32_t mbits = 0, sbits = 0;
@@ -192,12 +235,17 @@ __global__ __launch_bounds__(64 * MAXW) void xl_scores_fwd_kernel(XlScoreArgs a,
   raw0 = mfma16(qrf[1], f0[1], raw0);
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
-    if (t + 2 < NT) request(t + 2);
+    stage_free();
+    if (t + 1 < NT) { request(t + 1); wait_vm4(); } else wait_vm0();   // tile t has landed; only tile t + 1 may be in flight
+    const char* st = stage + (t & 1) * 2 * TILE_BYTES;
+    bf16x8 kf[2], krf[2];
+    tile16_frags(st, g, n, kf);
+    tile16_frags(st + TILE_BYTES, g, n, krf);
     f32x4 ac = {0.f, 0.f, 0.f, 0.f}, raw1 = {0.f, 0.f, 0.f, 0.f};
-    ac = mfma16(qwf[0], kf[t % 3][0], ac);
-    raw1 = mfma16(qrf[0], krf[t % 3][0], raw1);
-    ac = mfma16(qwf[1], kf[t % 3][1], ac);
-    raw1 = mfma16(qrf[1], krf[t % 3][1], raw1);
+    ac = mfma16(qwf[0], kf[0], ac);
+    raw1 = mfma16(qrf[0], krf[0], raw1);
+    ac = mfma16(qwf[1], kf[1], ac);
+    raw1 = mfma16(qrf[1], krf[1], raw1);
     float bd[4];
 #pragma unroll
     for (int v = 0; v < 4; ++v) bd[v] = lane_read(first[v] ? raw0[v] : raw1[v], rot[v]);
@@ -263,7 +311,7 @@ __global__ __launch_bounds__(64 * MAXW) void xl_scores_fwd_kernel(XlScoreArgs a,
 // copy and the two segment sums.  grid and block as the forward kernel.
 __global__ __launch_bounds__(64 * MAXW) void xl_scores_bwd_kernel(XlScoreArgs a, int prio) {
   ds_wave_prio(prio);
-  __shared__ float sd[MAXW][RB], st[MAXW][RB], s1[MAXW][RB];
+  extern __shared__ __attribute__((aligned(16))) char lds[];
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), g = lane >> 4, n = lane & 15;
   const int nw = blockDim.x >> 6;
   int bh, blk;
@@ -273,19 +321,22 @@ __global__ __launch_bounds__(64 * MAXW) void xl_scores_bwd_kernel(XlScoreArgs a,
   const int KT = a.K >> 4;
   const int kt0 = wave * NT;
   const bool odd = n & 1;
-  const bf16* vb = reinterpret_cast<const bf16*>(a.v) + (int64_t)b * a.ldk_b + hd * HD + 8 * g;
+  const bf16* vb = reinterpret_cast<const bf16*>(a.v) + (int64_t)b * a.ldk_b + hd * HD;
+  float (*sd)[RB] = reinterpret_cast<float (*)[RB]>(lds + nw * 2 * TILE_BYTES);
+  float (*st)[RB] = sd + MAXW;
+  float (*s1)[RB] = st + MAXW;
+  char* stage = lds + wave * 2 * TILE_BYTES;   // two stages of a value tile
   const bf16* p = reinterpret_cast<const bf16*>(a.p) + ((int64_t)bh * a.QQ + ii0 + 4 * g + (odd ? 1 : 0)) * a.K + (n & ~1);
   bf16x8 dvf[2];
   load_frags(reinterpret_cast<const bf16*>(a.dvec) + (int64_t)(ii0 + n) * a.ldq + (int64_t)b * a.H + hd * HD + 8 * g, dvf);
   uint32_t sbits = 0;
   if (a.meta) sbits = reinterpret_cast<const uint2*>(a.meta)[(((int64_t)b * (a.QQ / RB) + blk) * nw + wave) * 64 + lane].y;
   float dp[NT][4], pp[NT][4], dot[4] = {0.f, 0.f, 0.f, 0.f};
-  bf16x8 vf[2][2];
   uint32_t pw[2][2];
   // (no branches in the tile loop: tiles past the last key read the last tile again and count as zeros)
   auto request = [&](int t) {
     const int kt = kt0 + t < KT ? kt0 + t : KT - 1;
-    load_frags(vb + (int64_t)(kt * 16 + n) * a.ldk, vf[t & 1]);
+    tile16_fill(stage + (t & 1) * TILE_BYTES, vb, a.ldk, kt * 16, a.K - 1, lane);
     pw[t & 1][0] = *reinterpret_cast<const uint32_t*>(p + kt * 16);
     pw[t & 1][1] = *reinterpret_cast<const uint32_t*>(p + 2 * (int64_t)a.K + kt * 16);
   };
@@ -293,10 +344,13 @@ __global__ __launch_bounds__(64 * MAXW) void xl_scores_bwd_kernel(XlScoreArgs a,
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     {
-      if (t + 1 < NT) request(t + 1);
+      stage_free();
+      if (t + 1 < NT) { request(t + 1); wait_vm4(); } else wait_vm0();   // tile t (two tile loads, two probability loads) has landed
+      bf16x8 vf[2];
+      tile16_frags(stage + (t & 1) * TILE_BYTES, g, n, vf);
       f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-      acc = mfma16(dvf[0], vf[t & 1][0], acc);
-      acc = mfma16(dvf[1], vf[t & 1][1], acc);
+      acc = mfma16(dvf[0], vf[0], acc);
+      acc = mfma16(dvf[1], vf[1], acc);
       pair_unpack(pw[t & 1][0], odd, pp[t][0], pp[t][1]);
       pair_unpack(pw[t & 1][1], odd, pp[t][2], pp[t][3]);
 #pragma unroll
@@ -396,10 +450,20 @@ int ds_xl_scores_fwd(const XlScoreArgs* a, hipStream_t s) {
   ds_prof_scope prof(s, "xl_scores_fwd_kernel", 2.0 * (1.0 + 1.125) * a->B * a->N * (double)a->QQ * a->K * HD, "FLOP");
   const dim3 grid(a->QQ / RB, a->B * a->N), block(64 * nw);
   const bool full = a->K % 128 == 0;
-  if (full && a->meta) hipLaunchKernelGGL((xl_scores_fwd_kernel<true, true>), grid, block, 0, s, *a, ds_launch_prio);
-  else if (full) hipLaunchKernelGGL((xl_scores_fwd_kernel<true, false>), grid, block, 0, s, *a, ds_launch_prio);
-  else if (a->meta) hipLaunchKernelGGL((xl_scores_fwd_kernel<false, true>), grid, block, 0, s, *a, ds_launch_prio);
-  else hipLaunchKernelGGL((xl_scores_fwd_kernel<false, false>), grid, block, 0, s, *a, ds_launch_prio);
+  const size_t lds = (size_t)nw * 4 * TILE_BYTES + 2 * MAXW * RB * sizeof(float);
+  static bool attr = false;
+  if (!attr) {
+    const int most = MAXW * 4 * TILE_BYTES + 2 * MAXW * RB * (int)sizeof(float);
+    DS_CHECK_HIP(hipFuncSetAttribute((const void*)xl_scores_fwd_kernel<true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, most));
+    DS_CHECK_HIP(hipFuncSetAttribute((const void*)xl_scores_fwd_kernel<true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, most));
+    DS_CHECK_HIP(hipFuncSetAttribute((const void*)xl_scores_fwd_kernel<false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, most));
+    DS_CHECK_HIP(hipFuncSetAttribute((const void*)xl_scores_fwd_kernel<false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, most));
+    attr = true;
+  }
+  if (full && a->meta) hipLaunchKernelGGL((xl_scores_fwd_kernel<true, true>), grid, block, lds, s, *a, ds_launch_prio);
+  else if (full) hipLaunchKernelGGL((xl_scores_fwd_kernel<true, false>), grid, block, lds, s, *a, ds_launch_prio);
+  else if (a->meta) hipLaunchKernelGGL((xl_scores_fwd_kernel<false, true>), grid, block, lds, s, *a, ds_launch_prio);
+  else hipLaunchKernelGGL((xl_scores_fwd_kernel<false, false>), grid, block, lds, s, *a, ds_launch_prio);
   DS_CHECK_LAUNCH();
   return DS_OK;
 }
@@ -411,7 +475,46 @@ int ds_xl_scores_bwd(const XlScoreArgs* a, hipStream_t s) {
                "ds_xl_scores_bwd: operands must be 16-byte aligned");
   const int nw = (a->K + 127) / 128;
   ds_prof_scope prof(s, "xl_scores_bwd_kernel", (double)a->B * a->N * a->QQ * (3.0 * a->K * 2 + 0.0), "B");
-  hipLaunchKernelGGL(xl_scores_bwd_kernel, dim3(a->QQ / RB, a->B * a->N), dim3(64 * nw), 0, s, *a, ds_launch_prio);
+  hipLaunchKernelGGL(xl_scores_bwd_kernel, dim3(a->QQ / RB, a->B * a->N), dim3(64 * nw), (size_t)nw * 2 * TILE_BYTES + 3 * MAXW * RB * sizeof(float), s,
+                     *a, ds_launch_prio);
   DS_CHECK_LAUNCH();
   return DS_OK;
+}
+
+// ---- the same kernels as operators of the C ABI (dense layouts: q rows [QQ][B][H], kv rows [K][B][2H], kr rows [R][H])
+static void xl_dense_args(XlScoreArgs& a, int seq, int rows, int klen, int batch, int heads, float scale) {
+  memset(&a, 0, sizeof(a));
+  const int H = heads * HD;
+  a.ldq = (int64_t)batch * H; a.ldk = (int64_t)batch * 2 * H; a.ldk_b = 2 * H; a.ldkr = H;
+  a.Q = seq; a.QQ = rows; a.K = klen; a.R = klen + seq; a.B = batch; a.N = heads; a.H = H; a.scale = scale;
+}
+
+extern "C" size_t ds_xlnet_scores_meta_bytes(int rows, int klen, int batch) {
+  return rows > 0 && klen > 0 && batch > 0 ? ds_xl_meta_bytes(rows, klen, batch) : 0;
+}
+
+extern "C" int ds_xlnet_scores_pack(int seq, int rows, int klen, int batch, const float* masks, const uint8_t* seg_mat, void* meta,
+                                    float* nseg, void* stream) {
+  DS_CHECK_ARG(ds_xl_scores_fit(DS_BF16, HD, seq, klen, klen + seq), "ds_xlnet_scores_pack: seq %d / klen %d outside the kernels", seq, klen);
+  return ds_xl_pack_meta(seq, rows, klen, batch, masks, seg_mat, meta, nseg, (hipStream_t)stream);
+}
+
+extern "C" int ds_xlnet_scores_fwd(int seq, int rows, int klen, int batch, int heads, const void* qw, const void* qr, const void* qs,
+                                   const void* kv, const void* kr, const float* seg_emb, const void* meta, float scale, void* p,
+                                   void* stream) {
+  DS_CHECK_ARG(heads > 0 && batch > 0, "ds_xlnet_scores_fwd: non-positive shape");
+  XlScoreArgs a;
+  xl_dense_args(a, seq, rows, klen, batch, heads, scale);
+  a.qw = qw; a.qr = qr; a.qs = qs; a.k = kv; a.kr = kr; a.seg_emb = seg_emb; a.meta = meta; a.p = p;
+  return ds_xl_scores_fwd(&a, (hipStream_t)stream);
+}
+
+extern "C" int ds_xlnet_scores_bwd(int seq, int rows, int klen, int batch, int heads, const void* kv, const void* p, const void* dvec,
+                                   const void* meta, const float* nseg, float scale, void* ds, void* dbd, float* defs, void* stream) {
+  DS_CHECK_ARG(heads > 0 && batch > 0 && kv, "ds_xlnet_scores_bwd: bad argument");
+  XlScoreArgs a;
+  xl_dense_args(a, seq, rows, klen, batch, heads, scale);
+  a.v = (const char*)kv + (size_t)a.H * sizeof(bf16); a.p = (void*)p; a.dvec = dvec; a.meta = meta; a.nseg = nseg;
+  a.ds = ds; a.dbd = dbd; a.defs = defs;
+  return ds_xl_scores_bwd(&a, (hipStream_t)stream);
 }

@@ -271,6 +271,48 @@ def attention_bwd(qkv, ctx, lse, dctx, batch, heads, seq, scale, key_mask=None, 
     return dqkv
 
 
+def xlnet_scores_pack(seq, rows, klen, batch, masks=None, seg_mat=None):
+    """Mask (fp32 [rows, klen, batch], non-zero = masked) and segment matrix (uint8 [seq, klen, batch]) as the packed bits
+    ``xlnet_scores_fwd`` / ``xlnet_scores_bwd`` read -> (meta, nseg); (None, None) when both are None."""
+    if masks is None and seg_mat is None:
+        return None, None
+    _need_cuda(masks, seg_mat)
+    lib = _lib.load()
+    dev = (masks if masks is not None else seg_mat).device
+    meta = torch.empty(lib.ds_xlnet_scores_meta_bytes(rows, klen, batch), dtype=torch.uint8, device=dev)
+    nseg = torch.zeros(batch, seq, dtype=torch.float32, device=dev) if seg_mat is not None else None
+    check(lib.ds_xlnet_scores_pack(seq, rows, klen, batch, ptr(masks), ptr(seg_mat), ptr(meta), ptr(nseg), _lib.current_stream()),
+          "ds_xlnet_scores_pack")
+    return meta, nseg
+
+
+def xlnet_scores_fwd(qw, qr, qs, kv, kr, seg_emb, seq, heads, scale, meta=None):
+    """Probabilities of XLNet's relative attention (bf16, head size 64): ``qw, qr, qs [rows, batch, H]``, ``kv [klen, batch,
+    2H]``, ``kr [klen + seq, H]``, ``seg_emb`` fp32 ``[2, H]`` -> ``p [batch*heads, rows, klen]``."""
+    _need_cuda(qw, qr, qs, kv, kr, seg_emb, meta)
+    rows, batch, _ = qw.shape
+    klen = kv.shape[0]
+    p = torch.empty(batch * heads, rows, klen, dtype=qw.dtype, device=qw.device)
+    check(_lib.load().ds_xlnet_scores_fwd(seq, rows, klen, batch, heads, ptr(qw), ptr(qr), ptr(qs), ptr(kv), ptr(kr), ptr(seg_emb),
+                                          ptr(meta), scale, ptr(p), _lib.current_stream()), "ds_xlnet_scores_fwd")
+    return p
+
+
+def xlnet_scores_bwd(kv, p, dvec, seq, heads, scale, meta=None, nseg=None, dbd=None):
+    """Score gradients of the same rows from ``dvec [rows, batch, H]`` (gradient of ``p v``): -> (ds, dbd, defs); ``dbd``
+    ``[batch*heads, rows, klen + seq]`` is written only inside its band (pass a cleared buffer to reuse it)."""
+    _need_cuda(kv, p, dvec, meta, nseg, dbd)
+    rows, batch, _ = dvec.shape
+    klen = kv.shape[0]
+    ds = torch.empty_like(p)
+    if dbd is None:
+        dbd = torch.zeros(batch * heads, rows, klen + seq, dtype=p.dtype, device=p.device)
+    defs = torch.empty(batch * heads, rows, 2, dtype=torch.float32, device=p.device)
+    check(_lib.load().ds_xlnet_scores_bwd(seq, rows, klen, batch, heads, ptr(kv), ptr(p), ptr(dvec), ptr(meta), ptr(nseg), scale,
+                                          ptr(ds), ptr(dbd), ptr(defs), _lib.current_stream()), "ds_xlnet_scores_bwd")
+    return ds, dbd, defs
+
+
 def squad_head(x, batch, seq, output_weights, output_bias, start_positions, end_positions, d_weights=None, d_bias=None,
                need_dx=True, loss_scale=1.0):
     """build_output_layer_squad of bert/models/bert/bert.py:669-718 on the stage's sequence output

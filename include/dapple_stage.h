@@ -400,6 +400,30 @@ typedef struct ds_xlnet_cfg {
   int reserved[6];
 } ds_xlnet_cfg;
 int ds_xlnet_stage_create(const ds_xlnet_cfg* cfg, void* stream, ds_stage** out);
+
+/* Scores and softmax of XLNet's relative attention as operators (xlnet/layers/rel_multihead_attn.py:71-115 with the relative
+ * shift of lambda_funcs.py:85-93): what an XLNet stage runs per layer under DS_XL_ATTN_AUTO.  bf16, head size 64; seq and klen
+ * multiples of 16, klen <= 1024.  rows = streams * seq stacked query rows (row stream*seq + i is position i).  Layouts:
+ *   qw, qr, qs [rows][batch][heads*64]   q + bias_context / bias_relative / bias_segment
+ *   kv         [klen][batch][2*heads*64] k at column 0, v at column heads*64 of a row
+ *   kr         [klen + seq][heads*64]    projected position embeddings
+ *   seg_emb    fp32 [2][heads*64];  p, ds bf16 [batch*heads][rows][klen];  dbd bf16 [batch*heads][rows][klen + seq]
+ * forward:  p = softmax_j((qw.k[j] + qr.kr[j + seq - i] + qs.seg_emb[seg(i,j,b)]) * scale - 1e30 * mask(i',j,b))
+ * backward: dp = dvec v^T, ds = scale * p * (dp - sum_j p dp), dbd[i'][j + seq - i] = ds[i'][j] (only that band is written:
+ *           clear dbd once), defs fp32 [batch*heads][rows][2] = the sums of ds over the keys of either segment.
+ * ds_xlnet_scores_pack turns masks fp32 [rows][klen][batch] (non-zero = masked; may be NULL) and seg_mat uint8
+ * [seq][klen][batch] (may be NULL) into the packed bits both kernels read (meta, ds_xlnet_scores_meta_bytes bytes, 16-byte
+ * aligned) and nseg fp32 [batch][seq] (keys of the other segment per row; may be NULL when seg_mat is).  meta = NULL in
+ * forward / backward means no mask and one segment. */
+size_t ds_xlnet_scores_meta_bytes(int rows, int klen, int batch);
+int ds_xlnet_scores_pack(int seq, int rows, int klen, int batch, const float* masks, const uint8_t* seg_mat, void* meta,
+                         float* nseg, void* stream);
+int ds_xlnet_scores_fwd(int seq, int rows, int klen, int batch, int heads, const void* qw, const void* qr, const void* qs,
+                        const void* kv, const void* kr, const float* seg_emb, const void* meta, float scale, void* p,
+                        void* stream);
+int ds_xlnet_scores_bwd(int seq, int rows, int klen, int batch, int heads, const void* kv, const void* p, const void* dvec,
+                        const void* meta, const float* nseg, float scale, void* ds, void* dbd, float* defs, void* stream);
+
 /* Side inputs of the micro-batch that will be forwarded into `slot` (copied into the slot):
  *   masks   [streams][seq][mem_len+seq][batch] fp32, 1 = masked (get_attn_mask, lambda_funcs.py:7-44); NULL = none
  *   seg_mat [seq][mem_len+seq][batch] uint8, 1 = different segment (segment_embed.py:41-52); NULL = all equal
