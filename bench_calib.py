@@ -122,17 +122,20 @@ def xl_scores():
     rows, klen, H = streams * seq, mem + seq, heads * d
     bf = torch.bfloat16
     r = lambda *sh: torch.randn(*sh, device="cuda").to(bf)
-    qw, qr, qs, kv, kr, dvec = r(rows, batch, H), r(rows, batch, H), r(rows, batch, H), r(klen, batch, 2 * H), r(klen + seq, H), r(rows, batch, H)
+    q, kv, kr, dvec = r(rows, batch, H), r(klen, batch, 2 * H), r(klen + seq, H), r(rows, batch, H)
     seg_emb = torch.randn(2, H, device="cuda")
+    biases = [torch.randn(H, device="cuda") for _ in range(3)]
     masks = (torch.rand(rows, klen, batch, device="cuda") < 0.3).float()
     seg = (torch.rand(seq, klen, batch, device="cuda") < 0.4).to(torch.uint8)
     meta, nseg = ops.xlnet_scores_pack(seq, rows, klen, batch, masks, seg)
     dbd = torch.zeros(batch * heads, rows, klen + seq, dtype=bf, device="cuda")
     for _ in range(5):
-        p = ops.xlnet_scores_fwd(qw, qr, qs, kv, kr, seg_emb, seq, heads, 0.125, meta)
+        qw, qr, qs, de = ops.xlnet_bias_q(q, biases[0], biases[1], biases[2], seg_emb, heads)
+        p = ops.xlnet_scores_fwd(qw, qr, de, kv, kr, seq, heads, 0.125, meta)
         ops.xlnet_scores_bwd(kv, p, dvec, seq, heads, 0.125, meta, nseg, dbd)
     torch.cuda.synchronize()
     n = batch * heads * rows * klen
+    print("xl_bias_q_de_kernel: %d bytes per launch (read q, write qw, qr, qs)" % (8 * rows * batch * H))
     print("xl_scores_fwd_kernel: %d bytes per launch (write p; operands %d), %d FLOP (q k^T and the 9/8 window of q kr^T)"
           % (2 * n, 2 * (3 * rows * batch * H + klen * batch * H + (klen + seq) * H), int(2 * 2.125 * n * d)))
     print("xl_scores_bwd_kernel: %d bytes per launch (read p, write ds and the band of dbd), %d FLOP (dvec v^T)" % (6 * n, 2 * n * d))

@@ -121,8 +121,9 @@ PROTOTYPES = {
     "ds_colsum_accum": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]),
     "ds_xlnet_scores_meta_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int]),
     "ds_xlnet_scores_pack": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "ds_xlnet_bias_q": (C.c_int, [C.c_int, C.c_int, C.c_int] + [C.c_void_p] * 10),
     "ds_xlnet_scores_fwd": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
-                                      C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p, C.c_void_p]),
+                                      C.c_void_p, C.c_void_p, C.c_float, C.c_void_p, C.c_void_p]),
     "ds_xlnet_scores_bwd": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                       C.c_void_p, C.c_float, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "ds_conv3x3_fwd": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p,

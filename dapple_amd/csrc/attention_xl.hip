@@ -151,6 +151,46 @@ __device__ __forceinline__ void tile16_frags(const char* lds, int g, int n, bf16
   f[1] = *reinterpret_cast<const bf16x8*>(row + (((g + 4) ^ z) << 4));
 }
 
+// qw, qr, qs = q + r_w, q + r_r, q + r_s (bf16) for one row [H] per wave, and de[b][n][i'] = qs . (seg_emb[1] - seg_emb[0]) over
+// head n's 64 columns: the difference of the row's two segment scores, from the ROUNDED qs like every other use of it.
+// A lane owns 8 consecutive columns, so a head is 8 lanes.
+__global__ __launch_bounds__(256) void xl_bias_q_de_kernel(int rows, int B, int N, int QQ, const bf16* __restrict__ q,
+                                                          const float* __restrict__ rw, const float* __restrict__ rr,
+                                                          const float* __restrict__ rs, const float* __restrict__ seg_emb,
+                                                          bf16* __restrict__ qw, bf16* __restrict__ qr, bf16* __restrict__ qs,
+                                                          float* __restrict__ de) {
+  const int lane = threadIdx.x & 63;
+  const int r = blockIdx.x * 4 + (threadIdx.x >> 6);   // row ii * B + b
+  if (r >= rows) return;
+  const int ii = r / B, b = r % B, H = N * HD;
+  for (int c0 = lane * 8; c0 < H; c0 += 512) {
+    const bf16x8 x = *reinterpret_cast<const bf16x8*>(q + (int64_t)r * H + c0);
+    bf16x8 ow, orr, os;
+    float d = 0.f;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const f32x4 bw = *reinterpret_cast<const f32x4*>(rw + c0 + 4 * h), br = *reinterpret_cast<const f32x4*>(rr + c0 + 4 * h);
+      const f32x4 bs = *reinterpret_cast<const f32x4*>(rs + c0 + 4 * h);
+      const f32x4 s0 = *reinterpret_cast<const f32x4*>(seg_emb + c0 + 4 * h), s1 = *reinterpret_cast<const f32x4*>(seg_emb + H + c0 + 4 * h);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float v = (float)x[4 * h + j];
+        ow[4 * h + j] = (bf16)(v + bw[j]);
+        orr[4 * h + j] = (bf16)(v + br[j]);
+        os[4 * h + j] = (bf16)(v + bs[j]);
+        d += (float)os[4 * h + j] * (s1[j] - s0[j]);
+      }
+    }
+    *reinterpret_cast<bf16x8*>(qw + (int64_t)r * H + c0) = ow;
+    *reinterpret_cast<bf16x8*>(qr + (int64_t)r * H + c0) = orr;
+    *reinterpret_cast<bf16x8*>(qs + (int64_t)r * H + c0) = os;
+    d += dpp_move<0xB1>(d);    // lane ^ 1
+    d += dpp_move<0x4E>(d);    // lane ^ 2
+    d += dpp_move<0x141>(d);   // mirror within 8 lanes: the other quad
+    if ((lane & 7) == 0) de[((int64_t)b * N + c0 / HD) * QQ + ii] = d;
+  }
+}
+
 // this lane's two 16-byte MFMA operand slices of one 64-wide row (k index 32 ks + 8 (lane / 16) .. + 7; row_ptr includes 8 (lane / 16))
 __device__ __forceinline__ void load_frags(const bf16* row_ptr, bf16x8 (&f)[2]) {
   f[0] = *reinterpret_cast<const bf16x8*>(row_ptr);
@@ -193,29 +233,15 @@ __global__ __launch_bounds__(64 * MAXW) void xl_scores_fwd_kernel(XlScoreArgs a,
   }
   load_frags(reinterpret_cast<const bf16*>(a.qw) + qoff + 8 * g, qwf);
   request(0);
-  // de[v]: ef[1] - ef[0] of this lane's query row 4 g + v (a row's softmax ignores ef[0])
+  // de[v]: ef[1] - ef[0] of this lane's query row 4 g + v (a row's softmax ignores ef[0]), from ds_xl_bias_q
   float de[4] = {0.f, 0.f, 0.f, 0.f};
   uint32_t mbits = 0, sbits = 0;
   if (META) {
     const uint2 mw = reinterpret_cast<const uint2*>(a.meta)[(((int64_t)b * (a.QQ / RB) + blk) * nw + wave) * 64 + lane];
     mbits = mw.x; sbits = mw.y;
-    const bf16* qsp = reinterpret_cast<const bf16*>(a.qs) + qoff + 16 * g;
-    const float* se = a.seg_emb + hd * HD + 16 * g;
-    float d = 0.f;
+    const f32x4 dv = *reinterpret_cast<const f32x4*>(a.de + ((int64_t)b * a.N + hd) * a.QQ + ii0 + 4 * g);
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
-      const bf16x8 qv = *reinterpret_cast<const bf16x8*>(qsp + 8 * c);
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const f32x4 s0 = *reinterpret_cast<const f32x4*>(se + 8 * c + 4 * h), s1 = *reinterpret_cast<const f32x4*>(se + a.H + 8 * c + 4 * h);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) d += (float)qv[4 * h + j] * (s1[j] - s0[j]);
-      }
-    }
-    d += __shfl_xor(d, 16, 64);
-    d += __shfl_xor(d, 32, 64);   // every lane: the difference for query row n
-#pragma unroll
-    for (int v = 0; v < 4; ++v) de[v] = lane_read(d, (4 * g + v) << 2);
+    for (int v = 0; v < 4; ++v) de[v] = dv[v];
   }
   // column u = n + 15 - m of a tile's window is wanted by lane n of the group: the lane holding it is 16 g + (u & 15), and
   // that lane serves it from the window's first accumulator when its own column is >= 15 - m
@@ -431,6 +457,17 @@ int ds_xl_pack_meta(int Q, int QQ, int K, int B, const float* mask, const uint8_
   return DS_OK;
 }
 
+int ds_xl_bias_q(int rows, int B, int N, const void* q, const float* rw, const float* rr, const float* rs, const float* seg_emb,
+                 void* qw, void* qr, void* qs, float* de, hipStream_t s) {
+  DS_CHECK_ARG(rows > 0 && B > 0 && N > 0 && q && rw && rr && rs && seg_emb && qw && qr && qs && de, "ds_xl_bias_q: bad argument");
+  DS_CHECK_ARG(ds_aligned16(q) && ds_aligned16(rw) && ds_aligned16(rr) && ds_aligned16(rs) && ds_aligned16(seg_emb) && ds_aligned16(qw) &&
+               ds_aligned16(qr) && ds_aligned16(qs), "ds_xl_bias_q: operands must be 16-byte aligned");
+  hipLaunchKernelGGL(xl_bias_q_de_kernel, dim3((unsigned)((rows * B + 3) / 4)), dim3(256), 0, s, rows * B, B, N, rows, (const bf16*)q, rw, rr, rs,
+                     seg_emb, (bf16*)qw, (bf16*)qr, (bf16*)qs, de);
+  DS_CHECK_LAUNCH();
+  return DS_OK;
+}
+
 static int xl_scores_check(const char* who, const XlScoreArgs* a) {
   DS_CHECK_ARG(a && a->N > 0 && a->H == a->N * HD && ds_xl_scores_fit(DS_BF16, HD, a->Q, a->K, a->R) && a->QQ % a->Q == 0 && a->B > 0,
                "%s: shape outside the kernel (Q %d, QQ %d, K %d, R %d, H %d, N %d)", who, a ? a->Q : 0, a ? a->QQ : 0, a ? a->K : 0,
@@ -442,8 +479,8 @@ static int xl_scores_check(const char* who, const XlScoreArgs* a) {
 
 int ds_xl_scores_fwd(const XlScoreArgs* a, hipStream_t s) {
   DS_PROPAGATE(xl_scores_check("ds_xl_scores_fwd", a));
-  DS_CHECK_ARG(a->qw && a->qr && a->qs && a->k && a->kr && a->seg_emb && a->p, "ds_xl_scores_fwd: null pointer");
-  DS_CHECK_ARG(ds_aligned16(a->qw) && ds_aligned16(a->qr) && ds_aligned16(a->qs) && ds_aligned16(a->k) && ds_aligned16(a->kr) &&
+  DS_CHECK_ARG(a->qw && a->qr && a->k && a->kr && a->p && (a->de || !a->meta), "ds_xl_scores_fwd: null pointer");
+  DS_CHECK_ARG(ds_aligned16(a->qw) && ds_aligned16(a->qr) && ds_aligned16(a->de) && ds_aligned16(a->k) && ds_aligned16(a->kr) &&
                ds_aligned16(a->meta), "ds_xl_scores_fwd: operands must be 16-byte aligned");
   const int nw = (a->K + 127) / 128;
   // q k^T once, q k_r^T over 9 window tiles per 8 key tiles
@@ -499,13 +536,17 @@ extern "C" int ds_xlnet_scores_pack(int seq, int rows, int klen, int batch, cons
   return ds_xl_pack_meta(seq, rows, klen, batch, masks, seg_mat, meta, nseg, (hipStream_t)stream);
 }
 
-extern "C" int ds_xlnet_scores_fwd(int seq, int rows, int klen, int batch, int heads, const void* qw, const void* qr, const void* qs,
-                                   const void* kv, const void* kr, const float* seg_emb, const void* meta, float scale, void* p,
-                                   void* stream) {
+extern "C" int ds_xlnet_bias_q(int rows, int batch, int heads, const void* q, const float* bias_context, const float* bias_relative,
+                               const float* bias_segment, const float* seg_emb, void* qw, void* qr, void* qs, float* de, void* stream) {
+  return ds_xl_bias_q(rows, batch, heads, q, bias_context, bias_relative, bias_segment, seg_emb, qw, qr, qs, de, (hipStream_t)stream);
+}
+
+extern "C" int ds_xlnet_scores_fwd(int seq, int rows, int klen, int batch, int heads, const void* qw, const void* qr, const float* de,
+                                   const void* kv, const void* kr, const void* meta, float scale, void* p, void* stream) {
   DS_CHECK_ARG(heads > 0 && batch > 0, "ds_xlnet_scores_fwd: non-positive shape");
   XlScoreArgs a;
   xl_dense_args(a, seq, rows, klen, batch, heads, scale);
-  a.qw = qw; a.qr = qr; a.qs = qs; a.k = kv; a.kr = kr; a.seg_emb = seg_emb; a.meta = meta; a.p = p;
+  a.qw = qw; a.qr = qr; a.de = de; a.k = kv; a.kr = kr; a.meta = meta; a.p = p;
   return ds_xl_scores_fwd(&a, (hipStream_t)stream);
 }
 

@@ -115,14 +115,14 @@ int ds_bert_stage_create(const ds_stage_cfg* cfg, hipStream_t stream, ds_stage**
 // (backward) leaving the kernel (attention_xl.hip): for every stacked query row i' (stream * Q + i), sample b and head n
 //   score[j] = (qw[i'] . k[j] + qr[i'] . kr[j + Q - i] + ef[seg(i, j, b)]) * scale - 1e30 * mask[i'][j][b],  p = softmax_j score
 struct XlScoreArgs {
-  const void *qw, *qr, *qs;   // bf16 [QQ][B][H]: q + the three biases; row stride ldq, sample b at column b*H
+  const void *qw, *qr;        // bf16 [QQ][B][H]: q + bias_context, q + bias_relative; row stride ldq, sample b at column b*H
   int64_t ldq;
+  const float* de;            // fp32 [B][N][QQ]: (q + bias_segment) . (seg_emb[1] - seg_emb[0]) per head, from ds_xl_bias_q (forward)
   const void* k;              // bf16 key rows: row stride ldk, sample b at column b*ldk_b, head n at column n*64
   const void* v;              // bf16 value rows, strides of k (backward)
   int64_t ldk, ldk_b;
   const void* kr;             // bf16 [R][H]; row stride ldkr
   int64_t ldkr;
-  const float* seg_emb;       // fp32 [2][H]
   const void* meta;           // mask / segment bits packed by ds_xl_pack_meta, or null (no mask, one segment)
   const float* nseg;          // fp32 [B][Q]: keys of the other segment per query row, or null (backward)
   void* p;                    // bf16 [B*N][QQ][K]: written by forward, read by backward
@@ -138,6 +138,9 @@ bool ds_xl_scores_fit(int dtype, int head_dim, int Q, int K, int R);
 size_t ds_xl_meta_bytes(int QQ, int K, int B);
 // mask fp32 [QQ][K][B] (non-zero = masked) and seg uint8 [Q][K][B], either may be null -> meta; nseg (may be null) <- seg
 int ds_xl_pack_meta(int Q, int QQ, int K, int B, const float* mask, const uint8_t* seg, void* meta, float* nseg, hipStream_t stream);
+// q bf16 [rows][B][N*64] -> qw, qr, qs (same layout) and de fp32 [B][N][rows]
+int ds_xl_bias_q(int rows, int B, int N, const void* q, const float* rw, const float* rr, const float* rs, const float* seg_emb,
+                 void* qw, void* qr, void* qs, float* de, hipStream_t stream);
 int ds_xl_scores_fwd(const XlScoreArgs* a, hipStream_t stream);
 int ds_xl_scores_bwd(const XlScoreArgs* a, hipStream_t stream);
 int ds_gemm_splitk(const ds_gemm_desc* d, int splitk, void* stream);

@@ -225,7 +225,7 @@ struct XlnetStage : ds_stage {
   // workspace
   char* ws_base = nullptr;
   // buffers the weight-gradient kernels read alternate by layer parity ([2])
-  size_t ws_bytes = 0, ws_qall, ws_ac, ws_dp, ws_bd, ws_ds, ws_dbd[2], ws_def, ws_dz2[2], ws_du[2], ws_dy1, ws_dz1[2], ws_dvec, ws_dqw[2], ws_dqr[2],
+  size_t ws_bytes = 0, ws_de = 0, ws_qall, ws_ac, ws_dp, ws_bd, ws_ds, ws_dbd[2], ws_def, ws_dz2[2], ws_du[2], ws_dy1, ws_dz1[2], ws_dvec, ws_dqw[2], ws_dqr[2],
          ws_dqs[2], ws_dq[2], ws_dkv[2], ws_dkr[2], ws_deft[2], ws_dx[2];
   WgradLane lane;
   hipEvent_t ev_refresh = nullptr;
@@ -310,6 +310,7 @@ struct XlnetStage : ds_stage {
     // workspace
     Arena w;
     ws_qall = w.reserve(act);
+    if (score_fused) ws_de = w.reserve((size_t)B * N * S * Q * 4);   // forward only, like qall
     const size_t QQ = (size_t)S * Q;  // the streams' query rows stacked: one product / one softmax launch for all of them
     // fp32 scores: only the path of separate products and softmax launches has them
     ws_ac = w.reserve(score_fused ? 256 : (size_t)B * N * QQ * K * 4);
@@ -506,7 +507,10 @@ struct XlnetStage : ds_stage {
       DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, rowsS, 2 * H, H, x, H, wkv[l], 2 * H, sp + t.kv + (size_t)Mm * B * 2 * H * esz, 2 * H));
       {
         const int64_t total = (int64_t)rows * H;
-        if (dtype == DS_BF16)
+        if (score_fused)
+          DS_PROPAGATE(ds_xl_bias_q(S * Q, B, N, qall, w[b + X_RW], w[b + X_RR], w[b + X_RS], w[b + X_SEG], sp + t.qw, sp + t.qr, sp + t.qs,
+                                    (float*)(ws_base + ws_de), stream));
+        else if (dtype == DS_BF16)
           hipLaunchKernelGGL(xl_bias_q_kernel<bf16>, dim3(g1(total)), dim3(256), 0, stream, total, H, (const bf16*)qall, w[b + X_RW],
                              w[b + X_RR], w[b + X_RS], (bf16*)(sp + t.qw), (bf16*)(sp + t.qr), (bf16*)(sp + t.qs));
         else
@@ -518,10 +522,9 @@ struct XlnetStage : ds_stage {
         const int QQ = S * Q;
         XlScoreArgs xa;
         memset(&xa, 0, sizeof(xa));
-        xa.qw = sp + t.qw; xa.qr = sp + t.qr; xa.qs = sp + t.qs; xa.ldq = (int64_t)B * H;
+        xa.qw = sp + t.qw; xa.qr = sp + t.qr; xa.de = (const float*)(ws_base + ws_de); xa.ldq = (int64_t)B * H;
         xa.k = sp + t.kv; xa.ldk = (int64_t)B * 2 * H; xa.ldk_b = 2 * H;
         xa.kr = kr[l]; xa.ldkr = H;
-        xa.seg_emb = w[b + X_SEG];
         xa.meta = (has_mask[slot] || has_seg[slot]) ? sp + meta_off : nullptr;
         xa.p = sp + t.p;
         xa.Q = Q; xa.QQ = QQ; xa.K = K; xa.R = R; xa.B = B; xa.N = N; xa.H = H; xa.scale = scale;

@@ -286,15 +286,27 @@ def xlnet_scores_pack(seq, rows, klen, batch, masks=None, seg_mat=None):
     return meta, nseg
 
 
-def xlnet_scores_fwd(qw, qr, qs, kv, kr, seg_emb, seq, heads, scale, meta=None):
-    """Probabilities of XLNet's relative attention (bf16, head size 64): ``qw, qr, qs [rows, batch, H]``, ``kv [klen, batch,
-    2H]``, ``kr [klen + seq, H]``, ``seg_emb`` fp32 ``[2, H]`` -> ``p [batch*heads, rows, klen]``."""
-    _need_cuda(qw, qr, qs, kv, kr, seg_emb, meta)
+def xlnet_bias_q(q, bias_context, bias_relative, bias_segment, seg_emb, heads):
+    """``q [rows, batch, H]`` (bf16) -> (qw, qr, qs, de): q plus the three relative-attention biases (fp32 ``[H]``) and
+    ``de [batch, heads, rows]`` = qs . (seg_emb[1] - seg_emb[0]) per head."""
+    _need_cuda(q, bias_context, bias_relative, bias_segment, seg_emb)
+    rows, batch, _ = q.shape
+    qw, qr, qs = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+    de = torch.empty(batch, heads, rows, dtype=torch.float32, device=q.device)
+    check(_lib.load().ds_xlnet_bias_q(rows, batch, heads, ptr(q), ptr(bias_context), ptr(bias_relative), ptr(bias_segment), ptr(seg_emb),
+                                      ptr(qw), ptr(qr), ptr(qs), ptr(de), _lib.current_stream()), "ds_xlnet_bias_q")
+    return qw, qr, qs, de
+
+
+def xlnet_scores_fwd(qw, qr, de, kv, kr, seq, heads, scale, meta=None):
+    """Probabilities of XLNet's relative attention (bf16, head size 64): ``qw, qr [rows, batch, H]`` and ``de`` from
+    ``xlnet_bias_q``, ``kv [klen, batch, 2H]``, ``kr [klen + seq, H]`` -> ``p [batch*heads, rows, klen]``."""
+    _need_cuda(qw, qr, de, kv, kr, meta)
     rows, batch, _ = qw.shape
     klen = kv.shape[0]
     p = torch.empty(batch * heads, rows, klen, dtype=qw.dtype, device=qw.device)
-    check(_lib.load().ds_xlnet_scores_fwd(seq, rows, klen, batch, heads, ptr(qw), ptr(qr), ptr(qs), ptr(kv), ptr(kr), ptr(seg_emb),
-                                          ptr(meta), scale, ptr(p), _lib.current_stream()), "ds_xlnet_scores_fwd")
+    check(_lib.load().ds_xlnet_scores_fwd(seq, rows, klen, batch, heads, ptr(qw), ptr(qr), ptr(de), ptr(kv), ptr(kr), ptr(meta), scale,
+                                          ptr(p), _lib.current_stream()), "ds_xlnet_scores_fwd")
     return p
 
 

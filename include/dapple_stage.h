@@ -404,11 +404,14 @@ int ds_xlnet_stage_create(const ds_xlnet_cfg* cfg, void* stream, ds_stage** out)
 /* Scores and softmax of XLNet's relative attention as operators (xlnet/layers/rel_multihead_attn.py:71-115 with the relative
  * shift of lambda_funcs.py:85-93): what an XLNet stage runs per layer under DS_XL_ATTN_AUTO.  bf16, head size 64; seq and klen
  * multiples of 16, klen <= 1024.  rows = streams * seq stacked query rows (row stream*seq + i is position i).  Layouts:
- *   qw, qr, qs [rows][batch][heads*64]   q + bias_context / bias_relative / bias_segment
+ *   q, qw, qr, qs [rows][batch][heads*64] the projected queries; q + bias_context / bias_relative / bias_segment
+ *   de         fp32 [batch][heads][rows]  qs . (seg_emb[1] - seg_emb[0]) per head: the difference of a row's two segment
+ *                                         scores (ds_xlnet_bias_q writes qw, qr, qs and de from q)
  *   kv         [klen][batch][2*heads*64] k at column 0, v at column heads*64 of a row
  *   kr         [klen + seq][heads*64]    projected position embeddings
  *   seg_emb    fp32 [2][heads*64];  p, ds bf16 [batch*heads][rows][klen];  dbd bf16 [batch*heads][rows][klen + seq]
- * forward:  p = softmax_j((qw.k[j] + qr.kr[j + seq - i] + qs.seg_emb[seg(i,j,b)]) * scale - 1e30 * mask(i',j,b))
+ * forward:  p = softmax_j((qw.k[j] + qr.kr[j + seq - i] + qs.seg_emb[seg(i,j,b)]) * scale - 1e30 * mask(i',j,b)),
+ *           evaluated with de * seg(i,j,b) in place of the segment score (a softmax row ignores the common qs.seg_emb[0])
  * backward: dp = dvec v^T, ds = scale * p * (dp - sum_j p dp), dbd[i'][j + seq - i] = ds[i'][j] (only that band is written:
  *           clear dbd once), defs fp32 [batch*heads][rows][2] = the sums of ds over the keys of either segment.
  * ds_xlnet_scores_pack turns masks fp32 [rows][klen][batch] (non-zero = masked; may be NULL) and seg_mat uint8
@@ -418,9 +421,10 @@ int ds_xlnet_stage_create(const ds_xlnet_cfg* cfg, void* stream, ds_stage** out)
 size_t ds_xlnet_scores_meta_bytes(int rows, int klen, int batch);
 int ds_xlnet_scores_pack(int seq, int rows, int klen, int batch, const float* masks, const uint8_t* seg_mat, void* meta,
                          float* nseg, void* stream);
-int ds_xlnet_scores_fwd(int seq, int rows, int klen, int batch, int heads, const void* qw, const void* qr, const void* qs,
-                        const void* kv, const void* kr, const float* seg_emb, const void* meta, float scale, void* p,
-                        void* stream);
+int ds_xlnet_bias_q(int rows, int batch, int heads, const void* q, const float* bias_context, const float* bias_relative,
+                    const float* bias_segment, const float* seg_emb, void* qw, void* qr, void* qs, float* de, void* stream);
+int ds_xlnet_scores_fwd(int seq, int rows, int klen, int batch, int heads, const void* qw, const void* qr, const float* de,
+                        const void* kv, const void* kr, const void* meta, float scale, void* p, void* stream);
 int ds_xlnet_scores_bwd(int seq, int rows, int klen, int batch, int heads, const void* kv, const void* p, const void* dvec,
                         const void* meta, const float* nseg, float scale, void* ds, void* dbd, float* defs, void* stream);
 

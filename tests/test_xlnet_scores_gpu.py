@@ -17,12 +17,16 @@ def make_case(seq, mem, streams, batch, heads, mask_kind, use_seg, seed):
     g = torch.Generator().manual_seed(seed)
     rows, klen, H = streams * seq, mem + seq, heads * D
     r = lambda *s: torch.randn(*s, generator=g)
-    t = {
-        "qw": r(rows, batch, H), "qr": r(rows, batch, H), "qs": r(rows, batch, H), "kv": r(klen, batch, 2 * H),
-        "kr": r(klen + seq, H), "dvec": r(rows, batch, H),
-    }
+    t = {"q": r(rows, batch, H), "kv": r(klen, batch, 2 * H), "kr": r(klen + seq, H), "dvec": r(rows, batch, H)}
     t = {k: v.to(torch.bfloat16).cuda() for k, v in t.items()}
     t["seg_emb"] = (0.5 * r(2, H)).cuda()
+    biases = [(0.5 * r(H)).cuda() for _ in range(3)]
+    t["qw"], t["qr"], t["qs"], t["de"] = ops.xlnet_bias_q(t["q"], biases[0], biases[1], biases[2], t["seg_emb"], heads)
+    for name, bias in zip(("qw", "qr", "qs"), biases):      # q + bias, rounded once
+        assert torch.equal(t[name], (t["q"].float() + bias).to(torch.bfloat16)), name
+    want_de = torch.einsum("ibnd,nd->bni", t["qs"].double().view(rows, batch, heads, D),
+                           (t["seg_emb"][1] - t["seg_emb"][0]).double().view(heads, D))
+    assert rel_err(t["de"], want_de.cpu())[0] <= 1e-5
     masks = None
     if mask_kind == "random":       # about a third masked, some rows entirely
         masks = (torch.rand(rows, klen, batch, generator=g) < 0.35).float()
@@ -69,7 +73,7 @@ def test_scores_forward_and_backward(seq, mem, streams, batch, heads, mask_kind,
     t, rows, klen = make_case(seq, mem, streams, batch, heads, mask_kind, use_seg, seed=seq + mem)
     scale = 1.0 / np.sqrt(D)
     meta, nseg = ops.xlnet_scores_pack(seq, rows, klen, batch, t["masks"], t["seg"])
-    p = ops.xlnet_scores_fwd(t["qw"], t["qr"], t["qs"], t["kv"], t["kr"], t["seg_emb"], seq, heads, scale, meta)
+    p = ops.xlnet_scores_fwd(t["qw"], t["qr"], t["de"], t["kv"], t["kr"], seq, heads, scale, meta)
     want = reference_p(t, seq, heads, scale)
     mx, l2 = rel_err(p, want.cpu())
     assert mx <= 1e-2 and l2 <= 1e-2, "probabilities: rel max %.3e, l2 %.3e" % (mx, l2)
@@ -106,4 +110,4 @@ def test_scores_forward_and_backward(seq, mem, streams, batch, heads, mask_kind,
 def test_scores_reject_shapes_outside_the_kernels():
     t, rows, klen = make_case(16, 8, 1, 1, 2, None, False, seed=1)       # klen 24: not a multiple of 16
     with pytest.raises(Exception, match="outside the kernel"):
-        ops.xlnet_scores_fwd(t["qw"], t["qr"], t["qs"], t["kv"], t["kr"], t["seg_emb"], 16, 2, 0.125)
+        ops.xlnet_scores_fwd(t["qw"], t["qr"], t["de"], t["kv"], t["kr"], 16, 2, 0.125)
