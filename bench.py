@@ -337,7 +337,8 @@ def make_xlnet(c, args):
     wl.flops_per_sample = 3 * fwd * L
     wl.config = {"layers": L, "hidden": H, "heads": N, "ffn": F, "seq": Q, "mem_len": Mm, "streams": S, "micro_batch": B,
                  "micro_batches": M, "schedule": "1F1B stage 0 of 2, stash K=%d" % K, "flops": "two-stream count",
-                 "residual_stream": "fp32" if (c["dtype"] != "bf16" or not args.bf16_residual_stream) else "bf16"}
+                 "residual_stream": "fp32" if (c["dtype"] != "bf16" or not args.bf16_residual_stream) else "bf16",
+                 "attention_scores": "one kernel per pass" if args.xlnet_attention == "auto" else "separate launches, fp32 scores"}
 
     def cpu():
         from oracle import xlnet as ox
