@@ -677,7 +677,8 @@ int launch_cfg(GemmArgs a, int batch, hipStream_t stream) {
     // 3 buffers: 96 KB for a 128x128 block, 48 KB for 64x64 - a CU's 160 KB of LDS then holds blocks of two or
     // three kernels at once.  With several streams feeding the GPU that co-residency is worth more than a deeper
     // ring: 6 buffers under the 64x64 block (long reductions, one block per CU) made the BERT-48 half-stage step
-    // 3.6 % shorter with all its kernels on one stream and 7 % longer on three.
+    // 3.6 % shorter with all its kernels on one stream and 7 % longer on three; 4 buffers (64 KB: the products of
+    // 1024 x 1024 x 3072..4096 run 2 us faster alone) still 6 % longer - a third block no longer fits beside two.
     int rc = launch_dma<T, BM, BN, AMAJ, BMAJ, 3>(a, grid, stream);
     if (rc != DS_OK) return rc;
   } else {
