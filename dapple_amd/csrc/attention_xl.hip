@@ -214,8 +214,10 @@ __global__ __launch_bounds__(64 * MAXW) void xl_scores_fwd_kernel(XlScoreArgs a,
   const int64_t qoff = (int64_t)(ii0 + n) * a.ldq + (int64_t)b * a.H + hd * HD;
   const bf16* kb = reinterpret_cast<const bf16*>(a.k) + (int64_t)b * a.ldk_b + hd * HD;
   const bf16* krb = reinterpret_cast<const bf16*>(a.kr) + hd * HD;
-  float (*sm)[RB] = reinterpret_cast<float (*)[RB]>(lds + nw * 4 * TILE_BYTES);
-  float (*sl)[RB] = sm + MAXW;
+  // the per-wave maxima and sums meet in the first 128 bytes of every wave's own stage area, once its tiles are done with:
+  // the block then needs exactly 8 KB per wave, and two blocks of 7 waves leave room for a 48 KB GEMM block on the CU
+  auto sm = [&](int w) { return reinterpret_cast<float*>(lds + w * 4 * TILE_BYTES); };
+  auto sl = [&](int w) { return reinterpret_cast<float*>(lds + w * 4 * TILE_BYTES) + RB; };
   char* stage = lds + wave * 4 * TILE_BYTES;   // two stages of (key tile, position tile)
   // The tile loop has no branches: tiles past the last key stage clamped rows and their scores are replaced below.  The
   // next tile's rows are requested before the current tile is worked on.
@@ -310,16 +312,16 @@ __global__ __launch_bounds__(64 * MAXW) void xl_scores_fwd_kernel(XlScoreArgs a,
   // (a wave of a block always has its first tile: the block has ceil(K / 128) waves)
   if (n == 0) {
 #pragma unroll
-    for (int v = 0; v < 4; ++v) { sm[wave][4 * g + v] = mx[v]; sl[wave][4 * g + v] = l[v]; }
+    for (int v = 0; v < 4; ++v) { sm(wave)[4 * g + v] = mx[v]; sl(wave)[4 * g + v] = l[v]; }
   }
   __syncthreads();
   float f;
   {
-    float M = sm[0][n];
-    for (int w = 1; w < nw; ++w) M = fmaxf(M, sm[w][n]);
+    float M = sm(0)[n];
+    for (int w = 1; w < nw; ++w) M = fmaxf(M, sm(w)[n]);
     float L = 0.f;
-    for (int w = 0; w < nw; ++w) L += sl[w][n] * __builtin_amdgcn_exp2f(sm[w][n] - M);
-    f = __builtin_amdgcn_exp2f(sm[wave][n] - M) / L;
+    for (int w = 0; w < nw; ++w) L += sl(w)[n] * __builtin_amdgcn_exp2f(sm(w)[n] - M);
+    f = __builtin_amdgcn_exp2f(sm(wave)[n] - M) / L;
   }
   const bool odd = n & 1;
   bf16* p = reinterpret_cast<bf16*>(a.p) + ((int64_t)bh * a.QQ + ii0 + 4 * g + (odd ? 1 : 0)) * a.K + (n & ~1);
@@ -487,10 +489,10 @@ int ds_xl_scores_fwd(const XlScoreArgs* a, hipStream_t s) {
   ds_prof_scope prof(s, "xl_scores_fwd_kernel", 2.0 * (1.0 + 1.125) * a->B * a->N * (double)a->QQ * a->K * HD, "FLOP");
   const dim3 grid(a->QQ / RB, a->B * a->N), block(64 * nw);
   const bool full = a->K % 128 == 0;
-  const size_t lds = (size_t)nw * 4 * TILE_BYTES + 2 * MAXW * RB * sizeof(float);
+  const size_t lds = (size_t)nw * 4 * TILE_BYTES;
   static bool attr = false;
   if (!attr) {
-    const int most = MAXW * 4 * TILE_BYTES + 2 * MAXW * RB * (int)sizeof(float);
+    const int most = MAXW * 4 * TILE_BYTES;
     DS_CHECK_HIP(hipFuncSetAttribute((const void*)xl_scores_fwd_kernel<true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, most));
     DS_CHECK_HIP(hipFuncSetAttribute((const void*)xl_scores_fwd_kernel<true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, most));
     DS_CHECK_HIP(hipFuncSetAttribute((const void*)xl_scores_fwd_kernel<false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, most));
