@@ -491,7 +491,9 @@ int check(const char* who, int dtype, int B, int N, int S, int D) {
   DS_CHECK_ARG(S <= 2048, "%s: seq %d exceeds 2048", who, S);
   return DS_OK;
 }
-size_t lds_bytes(int S) { return (size_t)4 * CH * ROWB + (size_t)2 * S * sizeof(float); }
+// K / V (or Q / dO) tiles, two buffers each, plus `vectors` per-position fp32 arrays (mask adders; log-sum-exp and delta).
+// Every 4 KB counts: at 64 KB two 48 KB GEMM blocks of other streams fit on the CU beside an attention block, at 68 KB one.
+size_t lds_bytes(int S, int vectors) { return (size_t)4 * CH * ROWB + (size_t)vectors * S * sizeof(float); }
 
 }  // namespace
 
@@ -506,12 +508,12 @@ extern "C" int ds_attention_fwd(int dtype, int batch, int heads, int seq, int he
   a.prio = ds_launch_prio;
   static bool attr = false;
   if (!attr) {
-    DS_CHECK_HIP(hipFuncSetAttribute((const void*)attn_fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(2048)));
+    DS_CHECK_HIP(hipFuncSetAttribute((const void*)attn_fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(2048, 2)));
     attr = true;
   }
   hipStream_t s = (hipStream_t)stream;
   ds_prof_scope prof(s, "attn_fwd_kernel", 4.0 * batch * heads * (double)seq * seq * head_dim, "FLOP");
-  hipLaunchKernelGGL(attn_fwd_kernel, dim3(seq / 64, batch * heads), dim3(NTHREADS), lds_bytes(seq), s, a);
+  hipLaunchKernelGGL(attn_fwd_kernel, dim3(seq / 64, batch * heads), dim3(NTHREADS), lds_bytes(seq, key_mask ? 1 : 0), s, a);
   DS_CHECK_LAUNCH();
   return DS_OK;
 }
@@ -529,19 +531,19 @@ extern "C" int ds_attention_bwd(int dtype, int batch, int heads, int seq, int he
   a.mask_value = mask_value; a.prio = ds_launch_prio;
   static bool attr = false;
   if (!attr) {
-    DS_CHECK_HIP(hipFuncSetAttribute((const void*)attn_bwd_dq_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(2048)));
-    DS_CHECK_HIP(hipFuncSetAttribute((const void*)attn_bwd_dkv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(2048)));
+    DS_CHECK_HIP(hipFuncSetAttribute((const void*)attn_bwd_dq_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(2048, 2)));
+    DS_CHECK_HIP(hipFuncSetAttribute((const void*)attn_bwd_dkv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(2048, 2)));
     attr = true;
   }
   hipStream_t s = (hipStream_t)stream;
   {
     ds_prof_scope prof(s, "attn_bwd_dq_kernel", 6.0 * batch * heads * (double)seq * seq * head_dim, "FLOP");
-    hipLaunchKernelGGL(attn_bwd_dq_kernel, dim3(seq / 64, batch * heads), dim3(NTHREADS), lds_bytes(seq), s, a);
+    hipLaunchKernelGGL(attn_bwd_dq_kernel, dim3(seq / 64, batch * heads), dim3(NTHREADS), lds_bytes(seq, key_mask ? 1 : 0), s, a);
     DS_CHECK_LAUNCH();
   }
   {
     ds_prof_scope prof(s, "attn_bwd_dkv_kernel", 8.0 * batch * heads * (double)seq * seq * head_dim, "FLOP");
-    hipLaunchKernelGGL(attn_bwd_dkv_kernel, dim3(seq / 64, batch * heads), dim3(NTHREADS), lds_bytes(seq), s, a);
+    hipLaunchKernelGGL(attn_bwd_dkv_kernel, dim3(seq / 64, batch * heads), dim3(NTHREADS), lds_bytes(seq, 2), s, a);
     DS_CHECK_LAUNCH();
   }
   return DS_OK;
