@@ -1,7 +1,8 @@
 // Measured rates of the parts of a CU the GEMM kernels are built from (MI355X, gfx950): LDS read rate per instruction
 // form, LDS-DMA (global_load_lds_dwordx4) rate under several address patterns, MFMA rate with 1 and 2 waves per SIMD and
 // with one or all CUs busy, an MFMA wave beside a loader wave on one SIMD, and loads interleaved with MFMAs in one wave.
-// A stand-alone program, not part of libdapple_hip.so:  make -C dapple_amd/csrc microbench && dapple_amd/csrc/microbench/hw_rates
+// A stand-alone program, not part of libdapple_hip.so:
+//   hipcc -O3 -std=c++17 --offload-arch=gfx950 -Wno-inline-asm -Xclang -target-feature -Xclang -packed-fp32-ops bench_hw_rates.hip -o bench_hw_rates && ./bench_hw_rates
 #include <hip/hip_runtime.h>
 #include <stdio.h>
 #include <stdlib.h>
