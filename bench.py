@@ -56,7 +56,7 @@ def make_bert(c, args):
         dxs = None
     dys = [torch.as_tensor(x).cuda().to(adt) for x in synthetic.upstream_grads(synthetic.SEED_GRAD + c["index"], M, (B * S, H))]
     outs = [torch.empty(B * S, H, dtype=adt, device="cuda") for _ in range(M)]
-    rt = runtime.StageRuntime(stage, 0, 2, M)
+    rt = runtime.StageRuntime(stage, 0, 2, M, pair_passes=args.pair_passes)
     wl = Workload()
     wl.stage = stage
     wl.step = lambda: (stage.refresh_weights(), stage.zero_grads(), rt.step(xs, dys, outs, dxs))
@@ -65,7 +65,8 @@ def make_bert(c, args):
     wl.flops_per_sample = 3 * fwd * L
     wl.config = {"layers": L, "hidden": H, "heads": N, "ffn": F, "seq": S, "micro_batch": B, "micro_batches": M,
                  "embedding": c["embeddings"] is not None, "schedule": "1F1B stage 0 of 2, stash K=%d" % K,
-                 "wgrad_group": G, "residual_stream": "fp32" if (c["dtype"] != "bf16" or not args.bf16_residual_stream) else "bf16"}
+                 "wgrad_group": G, "residual_stream": "fp32" if (c["dtype"] != "bf16" or not args.bf16_residual_stream) else "bf16",
+                 "pair_passes": args.pair_passes}
 
     def cpu():
         from oracle import bert as ob
@@ -407,6 +408,9 @@ def main():
                     help="BERT / XLNet bf16 workloads: round the residual stream to bf16 too (faster, twice the error at full depth)")
     ap.add_argument("--wgrad-group", type=int, default=4,
                     help="BERT stages: weight gradients of this many backward passes in one GEMM per weight")
+    ap.add_argument("--pair-passes", action="store_true",
+                    help="BERT stages: issue F(j+1) and B(j) as ONE call that walks both chains level by level, one grouped launch "
+                         "per level (ds_stage_forward_backward), instead of two calls on two streams (measured slower: a what-if)")
     ap.add_argument("--xlnet-attention", choices=["auto", "separate"], default="auto",
                     help="XLNet stages: how the attention scores run (ds_xlnet_cfg.fused_attention)")
     ap.add_argument("--micro-batch", type=int, default=None,

@@ -21,6 +21,11 @@ size 64, bf16), three launches each, for the same counter runs as ``gemms`` (mat
 ``xl_scores``: the score kernels of XLNet's relative attention at the XLNet-36 half-stage's shape (two streams of 512
 positions + 384 memory positions, 16 heads, head size 64, bf16, masks and segments), five launches each, with their
 algorithmic bytes and FLOP printed.
+
+``grouped``: pairs and triples of the layer's GEMMs that a stage in steady state holds at the same time (a forward product
+of micro-batch j+1, an input-gradient product of micro-batch j, a weight-gradient product over four micro-batches), timed
+three ways - back to back on one stream, side by side on two / three streams, and as ONE ``ds_gemm_grouped`` launch per
+tile-shape choice.
 """
 import sys
 
@@ -102,6 +107,87 @@ def gemm_table():
         fl = 2.0 * m * n * k
         print("%-16s %-22s %10.2f %10.2f %12.1f %12.1f" % (name + (" C+=" if acc else ""), "%d x %d x %d" % (m, n, k), us[0], us[1],
                                                           fl / us[0] / 1e6, fl / us[1] / 1e6), flush=True)
+
+
+def grouped():
+    bf = torch.bfloat16
+    shapes = {name: (m, n, k, am, bm, acc) for name, m, n, k, am, bm, acc in layer_shapes()}
+    sets = [
+        ("fwd ffn1", "dgrad ffn2"),
+        ("fwd qkv", "dgrad ffn2"),
+        ("fwd ffn2", "dgrad ffn1"),
+        ("fwd ffn2", "dgrad qkv"),
+        ("fwd ao", "dgrad ao"),
+        ("fwd ffn1", "dgrad ffn2", "wgrad ffn1 x4"),
+        ("fwd ffn2", "dgrad ffn1", "wgrad ffn1 x4"),
+        ("fwd ao", "dgrad ao", "wgrad ffn1 x4"),
+        ("wgrad ffn1 x4",),
+        ("fwd ffn1",),
+        ("fwd ffn2",),
+    ]
+    reps = 20
+    streams = [torch.cuda.Stream() for _ in range(3)]
+    main = torch.cuda.Stream()
+
+    def operands(name):
+        m, n, k, am, bm, acc = shapes[name]
+        a = torch.randn((m, k) if am == DS_K_MAJOR else (k, m), device="cuda").to(bf)
+        b = torch.randn((n, k) if bm == DS_K_MAJOR else (k, n), device="cuda").to(bf)
+        c = torch.zeros(m, n, device="cuda", dtype=torch.float32 if acc else bf)
+        return dict(a=a, b=b, c=c, m=m, n=n, k=k, a_major=am, b_major=bm, flags=DS_EPI_ACCUM if acc else 0)
+
+    def timed(fn):
+        """`reps` rounds of fn captured into a graph (so that the host's issue rate is out of the picture), replayed."""
+        with torch.cuda.stream(main):
+            fn()
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=main):
+                for _ in range(reps):
+                    fn()
+            graph.replay()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(3):
+                graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / (3 * reps)
+
+    print("%-44s %9s %9s | grouped launch, us (tile shape per problem: 0=256x256 1=256x128 2=128x128 3=128x64, 4/5 = 2/3 with two "
+          "tile buffers)" % ("set", "1 stream", "n streams"))
+    for names in sets:
+        probs = [operands(nm) for nm in names]
+        flop = sum(2.0 * p["m"] * p["n"] * p["k"] for p in probs)
+
+        def serial():
+            for p in probs:
+                ops.gemm(**p)
+
+        def side_by_side():
+            cur = torch.cuda.current_stream()
+            for p, st in zip(probs[1:], streams):
+                st.wait_stream(cur)
+                with torch.cuda.stream(st):
+                    ops.gemm(**p)
+            ops.gemm(**probs[0])
+            for p, st in zip(probs[1:], streams):
+                cur.wait_stream(st)
+
+        t1 = timed(serial)
+        tn = timed(side_by_side) if len(probs) > 1 else float("nan")
+        cells = []
+        narrow = [p["n"] == 1024 and p["m"] == 1024 for p in probs]
+        choices = set()
+        for wide_cfg in (1, 2, 4):
+            for narrow_cfg in (2, 3, 4, 5):
+                for wg_cfg in (0, 1, 2, 4):
+                    choices.add(tuple((wg_cfg if p["flags"] else (narrow_cfg if nr else wide_cfg)) for p, nr in zip(probs, narrow)))
+        for cfgs in sorted(choices):
+            plist = [dict(p, cfg=c) for p, c in zip(probs, cfgs)]
+            cells.append("%s:%.1f" % ("".join(str(c) for c in cfgs), timed(lambda: ops.gemm_grouped(plist))))
+        print("%-44s %9.1f %9.1f | %s   [%.1f GFLOP]" % (" + ".join(names), t1, tn, "  ".join(cells), flop / 1e9), flush=True)
 
 
 def attention():
@@ -188,5 +274,7 @@ if __name__ == "__main__":
         xl_scores()
     elif len(sys.argv) > 1 and sys.argv[1] == "gemm_table":
         gemm_table()
+    elif len(sys.argv) > 1 and sys.argv[1] == "grouped":
+        grouped()
     else:
         accumulate(int(sys.argv[2]) if len(sys.argv) > 2 else 1 << 26)

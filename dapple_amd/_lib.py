@@ -93,6 +93,7 @@ PROTOTYPES = {
     "ds_cast_bf16_to_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "ds_gemm": (C.c_int, [C.POINTER(GemmDesc), C.c_void_p]),
     "ds_gemm_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int]),
+    "ds_gemm_grouped": (C.c_int, [C.POINTER(GemmDesc), C.POINTER(C.c_int), C.c_int, C.c_void_p]),
     "ds_vgg_stage_read_activation": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_size_t]),
     "ds_layernorm_fwd_mixed": (C.c_int, [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p, C.c_void_p,
                                           C.c_void_p, C.c_void_p]),
@@ -151,6 +152,7 @@ PROTOTYPES = {
     "ds_stage_forward": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
     "ds_stage_set_token_types": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p]),
     "ds_stage_backward": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
+    "ds_stage_forward_backward": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
     "ds_stage_backward_after": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
     "ds_stage_backward_event": (C.c_void_p, [C.c_void_p, C.c_int]),
     "ds_stage_wait_backward": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p]),

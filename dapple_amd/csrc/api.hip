@@ -99,6 +99,7 @@ extern "C" int ds_stage_destroy(ds_stage* h) {
     for (hipEvent_t e : h->ev_released) (void)hipEventDestroy(e);
     if (h->ev_join) (void)hipEventDestroy(h->ev_join);
     if (h->ev_dout) (void)hipEventDestroy(h->ev_dout);
+    if (h->ev_pair) (void)hipEventDestroy(h->ev_pair);
     (void)hipStreamDestroy(h->bwd_owned);
     (void)hipStreamDestroy(h->wgrad_owned);
   }
@@ -215,6 +216,52 @@ extern "C" int ds_stage_forward(ds_stage* h, int slot, const void* in, const flo
   return rc;
 }
 
+// F(fslot) and B(bslot) of different micro-batches in one call.  Stages that pair passes walk both chains together on
+// the stage's stream (one grouped launch per level); the others get the two calls one after the other.
+extern "C" int ds_stage_forward_backward(ds_stage* h, int fslot, const void* in, const float* key_mask, void* out, int bslot,
+                                         const void* d_out, void* d_in) {
+  DS_CHECK_ARG(h != nullptr && in != nullptr && out != nullptr && d_out != nullptr, "ds_stage_forward_backward: null argument");
+  if (!h->pairs_passes()) {
+    DS_PROPAGATE(ds_stage_forward(h, fslot, in, key_mask, out));
+    return ds_stage_backward(h, bslot, d_out, d_in);
+  }
+  const int K = h->cfg.stash_slots;
+  DS_CHECK_ARG(fslot >= 0 && fslot < K && bslot >= 0 && bslot < K && fslot != bslot,
+               "ds_stage_forward_backward: slots %d and %d must be two different slots in [0,%d)", fslot, bslot, K);
+  if (!h->bound) { ds_set_error("ds_stage_forward_backward: weights not bound"); return DS_ESTATE; }
+  if (h->slot_forwarded[fslot]) {
+    ds_set_error("ds_stage_forward_backward: slot %d still holds a micro-batch whose backward has not run", fslot);
+    return DS_ESTATE;
+  }
+  if (!h->slot_forwarded[bslot]) {
+    ds_set_error("ds_stage_forward_backward: slot %d holds no forwarded micro-batch", bslot);
+    return DS_ESTATE;
+  }
+  DS_CHECK_ARG(ds_aligned16(in) && ds_aligned16(out) && ds_aligned16(d_out) && ds_aligned16(d_in),
+               "ds_stage_forward_backward: in/out/d_out/d_in must be 16-byte aligned");
+  if (h->bwd_stream && h->bwd_pending) {
+    // the backward half shares its workspace with earlier backward passes: everything on the backward stream first
+    DS_CHECK_HIP(hipEventRecord(h->ev_join, h->bwd_stream));
+    DS_CHECK_HIP(hipStreamWaitEvent(h->stream, h->ev_join, 0));
+  }
+  DS_PROPAGATE(ds_stage_acquire_slot(h, fslot));
+  const int rc = h->forward_backward(fslot, in, key_mask, out, bslot, d_out, d_in);
+  if (rc != DS_OK) return rc;
+  h->slot_forwarded[fslot] = 1;
+  h->slot_forwarded[bslot] = 0;
+  if (h->bwd_stream) {
+    DS_CHECK_HIP(hipEventRecord(h->ev_forwarded[fslot], h->stream));
+    DS_CHECK_HIP(hipEventRecord(h->ev_released[bslot], h->stream));
+    h->released_valid[bslot] = 1;
+    h->bwd_pending = true;  // ds_stage_join orders the weight-gradient stream behind the backward stream, and that before the caller
+    // a backward pass issued on its own after this call runs on the backward stream and reuses this pass's workspace
+    if (!h->ev_pair) DS_CHECK_HIP(hipEventCreateWithFlags(&h->ev_pair, hipEventDisableTiming));
+    DS_CHECK_HIP(hipEventRecord(h->ev_pair, h->stream));
+    h->pair_valid = true;
+  }
+  return DS_OK;
+}
+
 // after: 0 = the producer of d_out is whatever has been queued on the stage's stream so far; 1 = `ready` (an event, or
 // NULL for "already complete / ordered before F(slot)") says when d_out may be read
 static int stage_backward(ds_stage* h, int slot, const void* d_out, void* d_in, int after, hipEvent_t ready) {
@@ -228,6 +275,10 @@ static int stage_backward(ds_stage* h, int slot, const void* d_out, void* d_in, 
   int rc;
   if (h->bwd_stream) {
     DS_CHECK_HIP(hipStreamWaitEvent(h->bwd_stream, h->ev_forwarded[slot], 0));
+    if (h->pair_valid) {
+      DS_CHECK_HIP(hipStreamWaitEvent(h->bwd_stream, h->ev_pair, 0));
+      h->pair_valid = false;  // the backward stream is behind it from here on
+    }
     if (!after) {
       DS_CHECK_HIP(hipEventRecord(h->ev_dout, h->stream));
       DS_CHECK_HIP(hipStreamWaitEvent(h->bwd_stream, h->ev_dout, 0));

@@ -767,7 +767,8 @@ __global__ __launch_bounds__(256) void gemm_k64_f32out_kernel(GemmArgs p) {
     }
 }
 
-static int gemm_run(const ds_gemm_desc* d, int splitk_req, void* stream, bool must_split = false) {
+// Checks a descriptor and turns it into launch arguments (tiling, slicing and workspace fields are left to the caller).
+int ds_gemm_make_args(const ds_gemm_desc* d, GemmArgs* out, int* batch_out) {
   DS_CHECK_ARG(d != nullptr, "ds_gemm: null descriptor");
   DS_CHECK_ARG(d->dtype == DS_F32 || d->dtype == DS_BF16, "ds_gemm: dtype %d", d->dtype);
   DS_CHECK_ARG((d->a_major | 1) == 1 && (d->b_major | 1) == 1, "ds_gemm: operand major must be 0 or 1");
@@ -800,9 +801,11 @@ static int gemm_run(const ds_gemm_desc* d, int splitk_req, void* stream, bool mu
   DS_CHECK_ARG(!(f & DS_EPI_GELU_GRAD) || (f & DS_EPI_GELU), "ds_gemm: DS_EPI_GELU_GRAD needs DS_EPI_GELU");
   DS_CHECK_ARG(!((f & DS_EPI_GELU) && (f & DS_EPI_DGELU)), "ds_gemm: GELU and DGELU are exclusive");
   DS_CHECK_ARG(!((f & DS_EPI_ACCUM) && (f & (DS_EPI_GELU | DS_EPI_DGELU))), "ds_gemm: ACCUM with GELU");
+  DS_CHECK_ARG((f & ~0xFFF) == 0, "ds_gemm: unknown epilogue flags 0x%x", f & ~0xFFF);
   (void)esz;
 
   GemmArgs a;
+  memset(&a, 0, sizeof(a));
   a.a = (const char*)d->a; a.b = (const char*)d->b; a.c = (char*)d->c;
   a.bias = d->bias; a.residual = (const char*)d->residual; a.c2 = (char*)d->c2;
   a.m = d->m; a.n = d->n; a.k = d->k;
@@ -817,6 +820,17 @@ static int gemm_run(const ds_gemm_desc* d, int splitk_req, void* stream, bool mu
   a.ws_part = nullptr; a.ws_count = nullptr;
   a.vec_epi = d->n % 8 == 0 && d->ldc % 8 == 0 && d->c_stride_outer % 8 == 0 && d->c_stride_inner % 8 == 0 &&
               ds_aligned16(d->c) && ds_aligned16(d->residual) && ds_aligned16(d->c2);
+  a.splitk = 1;
+  *out = a;
+  *batch_out = batch;
+  return DS_OK;
+}
+
+static int gemm_run(const ds_gemm_desc* d, int splitk_req, void* stream, bool must_split = false) {
+  GemmArgs a;
+  int batch = 1;
+  DS_PROPAGATE(ds_gemm_make_args(d, &a, &batch));
+  const int f = d->flags;
   if (d->dtype == DS_BF16 && d->a_major == DS_K_MAJOR && d->b_major == DS_K_MAJOR && d->k == 64 && f == DS_EPI_OUT_F32 &&
       d->m % 64 == 0 && d->n % 64 == 0 && batch <= 65535) {
     hipStream_t s = (hipStream_t)stream;
@@ -849,12 +863,12 @@ static int gemm_run(const ds_gemm_desc* d, int splitk_req, void* stream, bool mu
     // DS_GEMM8 = -1 switches them off, 0..4 forces a shape wherever it applies.
     static const char* env8 = getenv("DS_GEMM8");
     static const char* env_sk = getenv("DS_GEMM_SPLITK_WS");  // 0: never split, n > 1: n slices wherever k divides
-    static const int bm8[5] = {256, 256, 128, 128, 128}, bn8[5] = {256, 128, 128, 128, 128};
+    static const int bm8[6] = {256, 256, 128, 128, 128, 128}, bn8[6] = {256, 128, 128, 128, 128, 64};
     auto tiles_of = [&](int c) { return (int64_t)((d->m + bm8[c] - 1) / bm8[c]) * ((d->n + bn8[c] - 1) / bn8[c]) * batch; };
     int cfg8 = -1;
     if (env8) {
       cfg8 = atoi(env8);
-      if (cfg8 > 4) cfg8 = -1;
+      if (cfg8 > 5) cfg8 = -1;
     } else if (tiles_of(0) >= 200) {
       cfg8 = 0;
     } else if (tiles_of(1) >= 200) {

@@ -6,7 +6,8 @@
 // the other waits), and the block shapes keep LDS and vector-memory traffic per MFMA low:
 //   cfg 0: 256x256 block, waves 2(m) x 4(n), 128x64 per wave, 2 tile buffers (128 KB)
 //   cfg 1: 256x128 block, waves 2 x 2 x 2(k), 128x64 per wave pair, 3 tile buffers (144 KB)
-//   cfg 2: 128x128 block, waves 2 x 2 x 2(k),  64x64 per wave pair, 4 tile buffers (128 KB)
+//   cfg 2: 128x128 block, waves 2 x 2 x 2(k),  64x64 per wave pair, 4 tile buffers (128 KB; cfg 3 / 4: 2 / 3 buffers)
+//   cfg 5: 128x64  block, waves 2 x 2 x 2(k),  64x32 per wave pair, 4 tile buffers (96 KB)
 // In the 2 x 2 x 2 shapes the two waves of a SIMD own the same output sub-tile and split the four 16-deep k-steps of
 // every 64-deep k-tile between them (each fragment is still read from LDS once); their partial sums meet in LDS in
 // the epilogue.  Tiles move global -> LDS by LDS-DMA, one barrier per k-tile, fragments one k-step ahead of the
@@ -49,17 +50,18 @@ int launch8_cfg(const GemmArgs& a, int cfg, int batch, hipStream_t stream) {
     case 1: return launch8<256, 128, 2, 2, 2, 3, AMAJ, BMAJ>(a, batch, stream);
     case 3: return launch8<128, 128, 2, 2, 2, 2, AMAJ, BMAJ>(a, batch, stream);
     case 4: return launch8<128, 128, 2, 2, 2, 3, AMAJ, BMAJ>(a, batch, stream);
+    case 5: return launch8<128, 64, 2, 2, 2, 4, AMAJ, BMAJ>(a, batch, stream);
     default: return launch8<128, 128, 2, 2, 2, 4, AMAJ, BMAJ>(a, batch, stream);
   }
 }
 
 }  // namespace
 
-int ds_gemm8_stages(int cfg) { return cfg == 0 || cfg == 3 ? 2 : cfg == 1 || cfg == 4 ? 3 : 4; }
+int ds_gemm8_stages(int cfg) { return cfg == 0 || cfg == 3 ? 2 : cfg == 1 || cfg == 4 ? 3 : 4; }  // cfg 2 and 5: 4
 
 int ds_gemm8_launch(const GemmArgs& a, int cfg, int a_major, int b_major, int batch, hipStream_t stream) {
   DS_CHECK_ARG(a.k % 64 == 0 && a.vec_epi, "ds_gemm8_launch: needs k %% 64 == 0 and the vector epilogue");
-  DS_CHECK_ARG(cfg >= 0 && cfg <= 4, "ds_gemm8_launch: cfg %d", cfg);
+  DS_CHECK_ARG(cfg >= 0 && cfg <= 5, "ds_gemm8_launch: cfg %d", cfg);
   DS_CHECK_ARG(a.splitk == 1 || (a.ws_part && a.ws_count && batch == 1 && a.splitk <= 4),
                "ds_gemm8_launch: split-K needs a workspace, batch 1 and at most 4 slices");
   DS_CHECK_ARG(a.ktiles_per_split > ds_gemm8_stages(cfg) && (a.k / 64) % a.ktiles_per_split == 0,

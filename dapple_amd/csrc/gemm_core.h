@@ -46,7 +46,16 @@ struct GemmArgs {
   int prio;                    // wave priority (0..3)
   float* ws_part;              // split-K by workspace (8-wave kernels): fp32 partial tiles [tile][slice][BM * BN]
   unsigned* ws_count;          // and one arrival counter per tile (zero between launches)
+  float* rowdot;               // DS_EPI_ROWDOT (grouped launches only): see gemm_epilogue_vec8
+  int rowdot_seq;
 };
+
+// Internal epilogue flag: besides C, write for every row and every block of 64 columns the dot product of the bf16 values
+// stored to C with the bf16 tensor c2 (layout of C):
+//   rowdot[((row / rowdot_seq) * (n / 64) + col / 64) * rowdot_seq + row % rowdot_seq]
+// With C = d ctx and c2 = ctx of an attention layer (rows = samples x positions, 64 columns per head) that is the
+// delta[b][head][position] = sum_d dO O of the softmax backward.  Needs n % 64 == 0 and no other use of c2.
+#define DS_EPI_ROWDOT 4096
 
 
 // LDS has 64 banks of 4 bytes: one bank line is 256 bytes = two 128-byte K-major rows.
@@ -346,6 +355,19 @@ __device__ __forceinline__ void gemm_epilogue_vec8(const GemmArgs& p, int64_t c_
 #pragma unroll
     for (int e = 0; e < 8; ++e) o[e] = (bf16)x[e];
     *reinterpret_cast<bf16x8*>(reinterpret_cast<bf16*>(p.c) + c_off + idx) = o;
+    if (sizeof(T) == 2 && (flags & DS_EPI_ROWDOT)) {
+      // 8 neighbouring lanes hold the 64 columns of one head of this row (the vector index runs along the row first)
+      const bf16x8 a = *reinterpret_cast<const bf16x8*>(C2 + idx);
+      float d = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) d += (float)o[e] * (float)a[e];
+      d += __shfl_xor(d, 1, 64);
+      d += __shfl_xor(d, 2, 64);
+      d += __shfl_xor(d, 4, 64);
+      const int64_t row = idx / p.ldc, col = idx % p.ldc;
+      if ((col & 63) == 0)
+        p.rowdot[((row / p.rowdot_seq) * (p.n >> 6) + (col >> 6)) * p.rowdot_seq + row % p.rowdot_seq] = d;
+    }
   }
   if (flags & DS_EPI_GELU) {
     if (sizeof(T) == 2) {
@@ -387,4 +409,7 @@ inline void choose_xcd_block(GemmArgs& a) {
 // vector epilogue (GemmArgs::vec_epi).  splitk, ktiles_per_split, flags as for the 4-wave kernels.
 // every k-slice must hold more than ds_gemm8_stages(cfg) k-tiles (the depth of the tile ring), all slices equal.
 int ds_gemm8_stages(int cfg);
+// Checks a ds_gemm descriptor and fills the launch arguments that follow from it alone (operands, shapes, strides,
+// epilogue, vec_epi, wave priority); tiling, slicing and workspace fields are the caller's.
+int ds_gemm_make_args(const ds_gemm_desc* d, dsgemm::GemmArgs* out, int* batch_out);
 int ds_gemm8_launch(const dsgemm::GemmArgs& a, int cfg, int a_major, int b_major, int batch, hipStream_t stream);

@@ -41,6 +41,8 @@ struct ds_stage {
   hipEvent_t ev_join = nullptr;
   hipEvent_t ev_dout = nullptr;  // marks what was queued on `stream` when a backward pass was issued
   bool bwd_pending = false;
+  hipEvent_t ev_pair = nullptr;  // end of the latest ds_stage_forward_backward on `stream`: later backward passes share its workspace
+  bool pair_valid = false;
   virtual ~ds_stage() {}
   // true when forward and backward passes of different slots touch disjoint memory (apart from
   // read-only weights), so they may run concurrently
@@ -48,6 +50,13 @@ struct ds_stage {
   virtual int refresh_weights() = 0;
   virtual int forward(int slot, const void* in, const float* key_mask, void* out) = 0;
   virtual int backward(int slot, const void* d_out, void* d_in) = 0;
+  // true when forward_backward runs a forward and a backward pass of different slots as one walk over both chains on
+  // `stream` (grouped launches); otherwise the two passes are issued one after the other
+  virtual bool pairs_passes() const { return false; }
+  virtual int forward_backward(int fslot, const void* in, const float* key_mask, void* out, int bslot, const void* d_out, void* d_in) {
+    DS_PROPAGATE(forward(fslot, in, key_mask, out));
+    return backward(bslot, d_out, d_in);
+  }
   // gives up the micro-batch forwarded into `slot` without a backward pass (inference, a forward-only probe)
   virtual int release(int slot) { (void)slot; return DS_OK; }
   virtual size_t workspace_bytes() const = 0;

@@ -4,8 +4,13 @@
 // Follows bert/models/bert/modeling_slice.py of the reference: embedding_stage :794-821,
 // encoder_layer :942-1001 (attention_layer :357-549, dense+residual+layer_norm, gelu FFN).
 // Dropout is the identity (is_training=False zeroes it, :774-776).
+#include <stdlib.h>
 #include <string.h>
 
+#include <functional>
+#include <memory>
+
+#include "group.h"
 #include "stage.h"
 
 namespace {
@@ -377,31 +382,36 @@ struct BertStage : ds_stage {
   }
 
   // C[rows_m, n] = A[rows_m, k] (K-major) x W[k, n] (MN-major) with an epilogue
-  int gemm_fwd(int m, int n, int k, const void* a, const void* wt, void* c, int flags, const float* bias,
-               const void* residual, void* c2) {
+  ds_gemm_desc desc_fwd(int m, int n, int k, const void* a, const void* wt, void* c, int flags, const float* bias,
+                        const void* residual, void* c2) const {
     ds_gemm_desc d;
     memset(&d, 0, sizeof(d));
     d.dtype = dtype; d.a_major = DS_K_MAJOR; d.b_major = DS_MN_MAJOR;
     d.m = m; d.n = n; d.k = k; d.lda = k; d.ldb = n; d.ldc = n; d.batch = 1; d.batch_inner = 1;
     d.flags = flags; d.alpha = 1.f; d.a = a; d.b = wt; d.c = c; d.bias = bias; d.residual = residual; d.c2 = c2;
-    return ds_gemm(&d, stream);
+    return d;
   }
   // dX[m, k] = dY[m, n] x W[k, n]^T (+ residual) (* gelu'(aux))
-  int gemm_dgrad(int m, int n, int k, const void* dy, const void* wt, void* dx, int flags, const void* residual, void* aux) {
+  ds_gemm_desc desc_dgrad(int m, int n, int k, const void* dy, const void* wt, void* dx, int flags, const void* residual,
+                          void* aux) const {
     ds_gemm_desc d;
     memset(&d, 0, sizeof(d));
     d.dtype = dtype; d.a_major = DS_K_MAJOR; d.b_major = DS_K_MAJOR;
     d.m = m; d.n = k; d.k = n; d.lda = n; d.ldb = n; d.ldc = k; d.batch = 1; d.batch_inner = 1;
     d.flags = flags; d.alpha = 1.f; d.a = dy; d.b = wt; d.c = dx; d.residual = residual; d.c2 = aux;
-    return ds_gemm(&d, stream);
+    return d;
   }
   // dW[k, n] (fp32) += X[m, k]^T x dY[m, n]
-  int gemm_wgrad(int m, int n, int k, const void* x, int64_t ldx, const void* dy, int64_t ldy, float* dw, int64_t lddw) {
+  ds_gemm_desc desc_wgrad(int m, int n, int k, const void* x, int64_t ldx, const void* dy, int64_t ldy, float* dw, int64_t lddw) const {
     ds_gemm_desc d;
     memset(&d, 0, sizeof(d));
     d.dtype = dtype; d.a_major = DS_MN_MAJOR; d.b_major = DS_MN_MAJOR;
     d.m = k; d.n = n; d.k = m; d.lda = ldx; d.ldb = ldy; d.ldc = lddw; d.batch = 1; d.batch_inner = 1;
     d.flags = DS_EPI_ACCUM; d.alpha = 1.f; d.a = x; d.b = dy; d.c = dw;
+    return d;
+  }
+  int gemm_wgrad(int m, int n, int k, const void* x, int64_t ldx, const void* dy, int64_t ldy, float* dw, int64_t lddw) {
+    const ds_gemm_desc d = desc_wgrad(m, n, k, x, ldx, dy, ldy, dw, lddw);
     return ds_gemm(&d, stream);
   }
   // per-(batch, head) GEMM on [rows, ld] matrices whose head h owns columns h*D..h*D+D-1
@@ -433,8 +443,148 @@ struct BertStage : ds_stage {
     return DS_ESTATE;
   }
 
+  // ---- a pass as a sequence of steps
+  // A step is one link of a pass's chain of dependent kernels.  `solo` launches it as kernels of its own on `stream`;
+  // `ops` describe the same work as tasks of a grouped launch (group.h) where the stage's configuration allows - then
+  // a forward and a backward pass of different micro-batches advance level by level, one launch per level carrying a
+  // step of each.  `before` / `after` are the host's work around the step: event waits, launches on other streams.
+  struct Step {
+    std::function<int()> before, solo, after;
+    int nops = 0;
+    GroupOp ops[2];
+  };
+  typedef std::vector<Step> Steps;
+  // grouped launches exist for the bf16 kernels of the benchmarked configuration: fused attention, fp32 residual stream
+  // and deferred weight gradients (whose backward LayerNorm is the row kernel)
+  bool groupable() const { return fused_attn && rs32 && G > 1 && H % 64 == 0 && F % 64 == 0 && H >= 192 && F >= 192; }
+  bool pairs_passes() const override { return groupable(); }
+
+  static Step& add(Steps& st, std::function<int()> solo) {
+    st.emplace_back();
+    st.back().solo = std::move(solo);
+    return st.back();
+  }
+  Step& add_gemm(Steps& st, const ds_gemm_desc& d, int prio) {
+    Step& s = add(st, [this, d]() { return ds_gemm(&d, stream); });
+    if (groupable()) {
+      s.nops = 1;
+      s.ops[0].kind = GOP_GEMM;
+      s.ops[0].gemm = d;
+      s.ops[0].prio = prio;
+    }
+    return s;
+  }
+  Step& add_ln_fwd(Steps& st, int prio, const float* x, const float* gamma, const float* beta, void* y16, float* y32, float* stats) {
+    Step& s = add(st, [=]() { return ds_layernorm_fwd_mixed(rows, H, x, gamma, beta, cfg.ln_eps, y16, y32, stats, stream); });
+    if (groupable()) {
+      GroupOp& o = s.ops[0];
+      s.nops = 1;
+      o.kind = GOP_LN_FWD; o.prio = prio; o.rows = rows; o.cols = H; o.x = x; o.gamma = gamma; o.beta = beta; o.eps = cfg.ln_eps;
+      o.y16 = y16; o.y32 = y32; o.stats = stats;
+    }
+    return s;
+  }
+  Step& add_ln_bwd_rows(Steps& st, int prio, const float* dy, const float* x, const float* gamma, const float* stats, void* dx16, float* dx32,
+                        void* dy16) {
+    Step& s = add(st, [=]() { return ds_layernorm_bwd_mixed(rows, H, dy, x, gamma, stats, dx16, dx32, dy16, nullptr, nullptr, nullptr, stream); });
+    if (groupable()) {
+      GroupOp& o = s.ops[0];
+      s.nops = 1;
+      o.kind = GOP_LN_BWD; o.prio = prio; o.rows = rows; o.cols = H; o.x = x; o.gamma = gamma; o.stats = (float*)stats; o.dy = dy;
+      o.y16 = dx16; o.y32 = dx32; o.dy16 = dy16;
+    }
+    return s;
+  }
+  void attn_op(GroupOp& o, int kind, int prio, const void* qkv, const float* mask, void* ctx, float* lse, const void* dctx, void* dqkv,
+               float* delta) const {
+    o.kind = kind; o.prio = prio; o.B = B; o.N = NH; o.S = S; o.qkv = qkv; o.ld = 3 * H; o.key_mask = mask;
+    o.scale = 1.0f / sqrtf((float)D); o.mask_value = -10000.0f; o.ctx = ctx; o.lse = lse; o.dctx = dctx; o.dqkv = dqkv; o.delta = delta;
+  }
+
+  // one pass alone: every step as launches of its own, in order
+  int play(const Steps& st) {
+    for (const Step& s : st) {
+      if (s.before) DS_PROPAGATE(s.before());
+      DS_PROPAGATE(s.solo());
+      if (s.after) DS_PROPAGATE(s.after());
+    }
+    return DS_OK;
+  }
+
+  // Tile shapes of the grouped launches (DS_GROUP_CFG_WIDE / _NARROW: tuning overrides, group.h numbering).
+  void choose_cfg(GroupOp& o) const {
+    if (o.kind != GOP_GEMM || o.cfg >= 0) return;
+    static const char* env_w = getenv("DS_GROUP_CFG_WIDE");
+    static const char* env_n = getenv("DS_GROUP_CFG_NARROW");
+    const bool narrow = o.gemm.n <= 1024 && o.gemm.m <= 1024;
+    if (narrow) o.cfg = env_n ? atoi(env_n) : 3;
+    else o.cfg = env_w ? atoi(env_w) : 4;
+    // a tile ring must be shorter than the reduction: the two-buffer shapes take anything from three k-tiles on
+    const int ktiles = o.gemm.k / 64;
+    if (o.cfg == 3 && ktiles <= 4) o.cfg = 5;
+    if ((o.cfg == 1 || o.cfg == 2) && ktiles <= 3) o.cfg = 4;
+  }
+
+  // A forward and a backward pass of different micro-batches side by side on `stream`: steps that exist as tasks go
+  // out as ONE launch per level - the next step of either chain - the others as launches of their own.  The backward
+  // chain runs `lead` levels ahead so that steps of different kinds meet (DS_GROUP_LEAD).
+  int play_pair(Steps& f, Steps& b) {
+    static const char* env_lead = getenv("DS_GROUP_LEAD");
+    int lead = env_lead ? atoi(env_lead) : 1;
+    size_t fi = 0, bi = 0;
+    while (fi < f.size() || bi < b.size()) {
+      // steps that only exist as launches of their own go first, forward chain first
+      if (fi < f.size() && f[fi].nops == 0) {
+        DS_PROPAGATE(play_one(f[fi++], 1));
+        continue;
+      }
+      if (bi < b.size() && b[bi].nops == 0) {
+        DS_PROPAGATE(play_one(b[bi++], 3));
+        continue;
+      }
+      Step* sf = fi < f.size() ? &f[fi] : nullptr;
+      Step* sb = bi < b.size() ? &b[bi] : nullptr;
+      if (lead > 0 && sb) { sf = nullptr; --lead; }
+      GroupOp ops[4];
+      int n = 0;
+      if (sb) {
+        if (sb->before) DS_PROPAGATE(sb->before());
+        for (int i = 0; i < sb->nops; ++i) ops[n++] = sb->ops[i];
+      }
+      if (sf) {
+        if (sf->before) DS_PROPAGATE(sf->before());
+        for (int i = 0; i < sf->nops; ++i) ops[n++] = sf->ops[i];
+      }
+      for (int i = 0; i < n; ++i) choose_cfg(ops[i]);
+      DS_PROPAGATE(ds_group_launch(ops, n, stream));
+      if (sb) {
+        if (sb->after) DS_PROPAGATE(sb->after());
+        ++bi;
+      }
+      if (sf) {
+        if (sf->after) DS_PROPAGATE(sf->after());
+        ++fi;
+      }
+    }
+    return DS_OK;
+  }
+  int play_one(const Step& s, int prio) {
+    ds_prio_scope scope(prio);
+    if (s.before) DS_PROPAGATE(s.before());
+    DS_PROPAGATE(s.solo());
+    if (s.after) DS_PROPAGATE(s.after());
+    return DS_OK;
+  }
+
   int forward(int slot, const void* in, const float* key_mask, void* out) override {
     ds_prio_scope prio(1);
+    Steps st;
+    DS_PROPAGATE(forward_steps(slot, in, key_mask, out, st));
+    return play(st);
+  }
+
+  int forward_steps(int slot, const void* in, const float* key_mask, void* out, Steps& st) {
+    const int prio = 1;
     int pos = slot;
     if (G > 1) {
       DS_PROPAGATE(take_pos(&pos));
@@ -447,79 +597,87 @@ struct BertStage : ds_stage {
     char* sm = smallp(slot);
     const size_t act = (size_t)rows * H * esz;
     const float scale = 1.0f / sqrtf((float)D);
-    const float* mask = nullptr;
-    if (key_mask) {
-      DS_CHECK_HIP(hipMemcpyAsync(sm + mask_off, key_mask, (size_t)B * S * 4, hipMemcpyDeviceToDevice, stream));
-      mask = (const float*)(sm + mask_off);
-    }
+    const float* mask = key_mask ? (const float*)(sm + mask_off) : nullptr;
     slot_has_mask[slot] = key_mask != nullptr;
     char* x0 = L ? at(ls[0].x, pos) : nullptr;
-    if (emb) {
-      DS_CHECK_HIP(hipMemcpyAsync(sm + emb_ids, in, (size_t)rows * 4, hipMemcpyDeviceToDevice, stream));
-      const int32_t* tt = slot_has_tt[slot] ? (const int32_t*)(sm + emb_tt) : nullptr;
-      dim3 grid((rows + 3) / 4);
-      if (dtype == DS_BF16)
-        hipLaunchKernelGGL(embed_fwd_kernel<bf16>, grid, dim3(256), 0, stream, rows, H, S, cfg.vocab, cfg.type_vocab,
-                           (const int32_t*)(sm + emb_ids), tt, w[E_WORD], w[E_TYPE], w[E_POS], (bf16*)(at(emb_e, pos)));
-      else
-        hipLaunchKernelGGL(embed_fwd_kernel<float>, grid, dim3(256), 0, stream, rows, H, S, cfg.vocab, cfg.type_vocab,
-                           (const int32_t*)(sm + emb_ids), tt, w[E_WORD], w[E_TYPE], w[E_POS], (float*)(at(emb_e, pos)));
-      DS_CHECK_LAUNCH();
-      DS_PROPAGATE(ds_layernorm_fwd(dtype, rows, H, at(emb_e, pos), w[E_LN_G], w[E_LN_B], cfg.ln_eps, L ? (void*)x0 : out,
-                                    (float*)(at(emb_st, pos)), stream));
-    } else {
-      DS_CHECK_HIP(hipMemcpyAsync(x0, in, act, hipMemcpyDeviceToDevice, stream));
-    }
-    if (rs32) DS_PROPAGATE(ds_cast_bf16_to_f32(ws_base + fw_xf[0], x0, (size_t)rows * H, stream));
+    add(st, [=]() {  // the micro-batch's inputs into the slot, the embedding if the stage has it
+      if (key_mask) DS_CHECK_HIP(hipMemcpyAsync(sm + mask_off, key_mask, (size_t)B * S * 4, hipMemcpyDeviceToDevice, stream));
+      if (emb) {
+        DS_CHECK_HIP(hipMemcpyAsync(sm + emb_ids, in, (size_t)rows * 4, hipMemcpyDeviceToDevice, stream));
+        const int32_t* tt = slot_has_tt[slot] ? (const int32_t*)(sm + emb_tt) : nullptr;
+        dim3 grid((rows + 3) / 4);
+        if (dtype == DS_BF16)
+          hipLaunchKernelGGL(embed_fwd_kernel<bf16>, grid, dim3(256), 0, stream, rows, H, S, cfg.vocab, cfg.type_vocab,
+                             (const int32_t*)(sm + emb_ids), tt, w[E_WORD], w[E_TYPE], w[E_POS], (bf16*)(at(emb_e, pos)));
+        else
+          hipLaunchKernelGGL(embed_fwd_kernel<float>, grid, dim3(256), 0, stream, rows, H, S, cfg.vocab, cfg.type_vocab,
+                             (const int32_t*)(sm + emb_ids), tt, w[E_WORD], w[E_TYPE], w[E_POS], (float*)(at(emb_e, pos)));
+        DS_CHECK_LAUNCH();
+        DS_PROPAGATE(ds_layernorm_fwd(dtype, rows, H, at(emb_e, pos), w[E_LN_G], w[E_LN_B], cfg.ln_eps, L ? (void*)x0 : out,
+                                      (float*)(at(emb_st, pos)), stream));
+      } else {
+        DS_CHECK_HIP(hipMemcpyAsync(x0, in, act, hipMemcpyDeviceToDevice, stream));
+      }
+      if (rs32) DS_PROPAGATE(ds_cast_bf16_to_f32(ws_base + fw_xf[0], x0, (size_t)rows * H, stream));
+      return DS_OK;
+    });
     for (int l = 0; l < L; ++l) {
       const LayerStash& t = ls[l];
       const int b = base(l);
       char* x = at(t.x, pos);
       char* y = (l + 1 < L) ? at(ls[l + 1].x, pos) : (char*)out;
-      DS_PROPAGATE(await_cast(l, stream));
+      char* qkv = at(t.qkv, pos);
       // fused Q|K|V projection (modeling_slice.py:464-485)
-      DS_PROPAGATE(gemm_fwd(rows, 3 * H, H, x, wqkv[l], at(t.qkv, pos), DS_EPI_BIAS, bqkv[l], nullptr, nullptr));
+      add_gemm(st, desc_fwd(rows, 3 * H, H, x, wqkv[l], qkv, DS_EPI_BIAS, bqkv[l], nullptr, nullptr), prio).before =
+          [this, l]() { return await_cast(l, stream); };
       if (fused_attn) {
         // scores, scale, mask adder, softmax and context in one kernel (:499-533)
-        DS_PROPAGATE(ds_attention_fwd(dtype, B, NH, S, D, at(t.qkv, pos), 3 * H, mask, scale, -10000.0f, at(t.ctx, pos),
-                                      (float*)(at(t.lse, pos)), stream));
+        char* ctx = at(t.ctx, pos);
+        float* lse = (float*)(at(t.lse, pos));
+        Step& s = add(st, [=]() { return ds_attention_fwd(dtype, B, NH, S, D, qkv, 3 * H, mask, scale, -10000.0f, ctx, lse, stream); });
+        if (groupable()) {
+          s.nops = 1;
+          attn_op(s.ops[0], GOP_ATTN_FWD, prio, qkv, mask, ctx, lse, nullptr, nullptr, nullptr);
+        }
       } else {
-      // scores = Q K^T (:499), fp32
-      DS_PROPAGATE(gemm_heads(DS_K_MAJOR, DS_K_MAJOR, S, S, D, at(t.qkv, pos), 3 * H, (int64_t)S * 3 * H, D,
-                              at(t.qkv, pos) + (size_t)H * esz, 3 * H, (int64_t)S * 3 * H, D, ws_base + ws_fscores, S,
-                              (int64_t)NH * S * S, (int64_t)S * S, DS_EPI_OUT_F32));
-      // scale, mask adder, softmax (:500-518)
-      DS_PROPAGATE(ds_softmax_fwd(dtype, B, NH, S, S, (const float*)(ws_base + ws_fscores), scale, mask, -10000.0f,
-                                  at(t.p, pos), stream));
-      // ctx = P V (:533), written head-interleaved as [rows, H] (:536-542)
-      DS_PROPAGATE(gemm_heads(DS_K_MAJOR, DS_MN_MAJOR, S, D, S, at(t.p, pos), S, (int64_t)NH * S * S, (int64_t)S * S,
-                              at(t.qkv, pos) + (size_t)2 * H * esz, 3 * H, (int64_t)S * 3 * H, D, at(t.ctx, pos), H,
-                              (int64_t)S * H, D, 0));
+        char* p = at(t.p, pos);
+        char* ctx = at(t.ctx, pos);
+        add(st, [=]() {
+          // scores = Q K^T (:499), fp32
+          DS_PROPAGATE(gemm_heads(DS_K_MAJOR, DS_K_MAJOR, S, S, D, qkv, 3 * H, (int64_t)S * 3 * H, D, qkv + (size_t)H * esz, 3 * H,
+                                  (int64_t)S * 3 * H, D, ws_base + ws_fscores, S, (int64_t)NH * S * S, (int64_t)S * S, DS_EPI_OUT_F32));
+          // scale, mask adder, softmax (:500-518)
+          DS_PROPAGATE(ds_softmax_fwd(dtype, B, NH, S, S, (const float*)(ws_base + ws_fscores), scale, mask, -10000.0f, p, stream));
+          // ctx = P V (:533), written head-interleaved as [rows, H] (:536-542)
+          return gemm_heads(DS_K_MAJOR, DS_MN_MAJOR, S, D, S, p, S, (int64_t)NH * S * S, (int64_t)S * S, qkv + (size_t)2 * H * esz, 3 * H,
+                            (int64_t)S * 3 * H, D, ctx, H, (int64_t)S * H, D, 0);
+        });
       }
       const int res32 = DS_EPI_RESIDUAL | DS_EPI_RESIDUAL_F32 | DS_EPI_OUT_F32;  // fp32 stream: fp32 residual in, fp32 sum out
       float* xf = (float*)(ws_base + fw_xf[l & 1]);
       float* af = (float*)(ws_base + fw_af);
       // attention output dense + residual (:974-978), then layer_norm (:979)
-      DS_PROPAGATE(gemm_fwd(rows, H, H, at(t.ctx, pos), weight_T(l, W_AO), at(t.z1, pos), DS_EPI_BIAS | (rs32 ? res32 : DS_EPI_RESIDUAL),
-                            w[b + B_AO], rs32 ? (const void*)xf : (const void*)x, nullptr));
-      if (rs32)
-        DS_PROPAGATE(ds_layernorm_fwd_mixed(rows, H, (const float*)at(t.z1, pos), w[b + LN1_G], w[b + LN1_B], cfg.ln_eps, at(t.a, pos), af,
-                                            (float*)(at(t.st1, pos)), stream));
-      else
-        DS_PROPAGATE(ds_layernorm_fwd(dtype, rows, H, at(t.z1, pos), w[b + LN1_G], w[b + LN1_B], cfg.ln_eps, at(t.a, pos),
-                                      (float*)(at(t.st1, pos)), stream));
+      add_gemm(st, desc_fwd(rows, H, H, at(t.ctx, pos), weight_T(l, W_AO), at(t.z1, pos), DS_EPI_BIAS | (rs32 ? res32 : DS_EPI_RESIDUAL),
+                            w[b + B_AO], rs32 ? (const void*)xf : (const void*)x, nullptr), prio);
+      if (rs32) {
+        add_ln_fwd(st, prio, (const float*)at(t.z1, pos), w[b + LN1_G], w[b + LN1_B], at(t.a, pos), af, (float*)(at(t.st1, pos)));
+      } else {
+        char *z1 = at(t.z1, pos), *a = at(t.a, pos), *st1 = at(t.st1, pos);
+        add(st, [=]() { return ds_layernorm_fwd(dtype, rows, H, z1, w[b + LN1_G], w[b + LN1_B], cfg.ln_eps, a, (float*)st1, stream); });
+      }
       // intermediate dense + gelu (:983-987)
-      DS_PROPAGATE(gemm_fwd(rows, F, H, at(t.a, pos), weight_T(l, W_FF1), at(t.u, pos), DS_EPI_BIAS | DS_EPI_GELU | DS_EPI_GELU_GRAD, w[b + B_FF1],
-                            nullptr, at(t.h, pos)));
+      add_gemm(st, desc_fwd(rows, F, H, at(t.a, pos), weight_T(l, W_FF1), at(t.u, pos), DS_EPI_BIAS | DS_EPI_GELU | DS_EPI_GELU_GRAD,
+                            w[b + B_FF1], nullptr, at(t.h, pos)), prio);
       // output dense + residual + layer_norm (:991-996)
-      DS_PROPAGATE(gemm_fwd(rows, H, F, at(t.h, pos), weight_T(l, W_FF2), at(t.z2, pos), DS_EPI_BIAS | (rs32 ? res32 : DS_EPI_RESIDUAL),
-                            w[b + B_FF2], rs32 ? (const void*)af : (const void*)at(t.a, pos), nullptr));
-      if (rs32)
-        DS_PROPAGATE(ds_layernorm_fwd_mixed(rows, H, (const float*)at(t.z2, pos), w[b + LN2_G], w[b + LN2_B], cfg.ln_eps, y,
-                                            l + 1 < L ? (float*)(ws_base + fw_xf[(l + 1) & 1]) : nullptr, (float*)(at(t.st2, pos)), stream));
-      else
-        DS_PROPAGATE(ds_layernorm_fwd(dtype, rows, H, at(t.z2, pos), w[b + LN2_G], w[b + LN2_B], cfg.ln_eps, y,
-                                      (float*)(at(t.st2, pos)), stream));
+      add_gemm(st, desc_fwd(rows, H, F, at(t.h, pos), weight_T(l, W_FF2), at(t.z2, pos), DS_EPI_BIAS | (rs32 ? res32 : DS_EPI_RESIDUAL),
+                            w[b + B_FF2], rs32 ? (const void*)af : (const void*)at(t.a, pos), nullptr), prio);
+      if (rs32) {
+        add_ln_fwd(st, prio, (const float*)at(t.z2, pos), w[b + LN2_G], w[b + LN2_B], y,
+                   l + 1 < L ? (float*)(ws_base + fw_xf[(l + 1) & 1]) : nullptr, (float*)(at(t.st2, pos)));
+      } else {
+        char *z2 = at(t.z2, pos), *st2 = at(t.st2, pos);
+        add(st, [=]() { return ds_layernorm_fwd(dtype, rows, H, z2, w[b + LN2_G], w[b + LN2_B], cfg.ln_eps, y, (float*)st2, stream); });
+      }
     }
     return DS_OK;
   }
@@ -535,33 +693,59 @@ struct BertStage : ds_stage {
 
   int backward(int slot, const void* d_out, void* d_in) override {
     ds_prio_scope prio(3);  // the chain every later pass waits on
+    Steps st;
+    DS_PROPAGATE(backward_steps(slot, d_out, d_in, st));
+    return play(st);
+  }
+
+  // A forward pass (slot fslot) and a backward pass (slot bslot) of different micro-batches as one walk over both
+  // chains on `stream`: the reference's graph leaves them unordered (bert/graph.py:126-132).
+  int forward_backward(int fslot, const void* in, const float* key_mask, void* out, int bslot, const void* d_out, void* d_in) override {
+    if (!groupable()) {
+      {
+        ds_prio_scope prio(1);
+        Steps f;
+        DS_PROPAGATE(forward_steps(fslot, in, key_mask, out, f));
+        DS_PROPAGATE(play(f));
+      }
+      return backward(bslot, d_out, d_in);
+    }
+    Steps f, b;
+    DS_PROPAGATE(forward_steps(fslot, in, key_mask, out, f));
+    DS_PROPAGATE(backward_steps(bslot, d_out, d_in, b));
+    return play_pair(f, b);
+  }
+
+  int backward_steps(int slot, const void* d_out, void* d_in, Steps& st) {
+    const int prio = 3;
     const int pos = slot_pos[slot];
     char* sm = smallp(slot);
     const int dypos = (int)(n_backward % NDY);
     if (G > 1 && dy_wg_valid[dypos]) DS_CHECK_HIP(hipStreamWaitEvent(stream, ev_dy_wg[dypos], 0));
     const float scale = 1.0f / sqrtf((float)D);
-    const char* dy = (const char*)d_out;
     // With a weight-gradient stream the wgrad GEMMs and bias column sums of a layer run beside the
     // dgrad chain of the layers below it: they only feed the master gradients.
     hipStream_t ws = G > 1 ? nullptr : wgrad_stream;
     // Grouped weight gradients: the pass that completes a group issues the group's GEMMs layer by layer as its own
     // chain passes each layer, so that they run beside the chain of the layers below instead of after the pass.
     const bool closing = G > 1 && (int)deferred.size() + 1 >= G;
-    std::vector<Run> runs;
+    std::shared_ptr<std::vector<Run>> runs = std::make_shared<std::vector<Run>>();
     hipStream_t gws = nullptr;
     if (closing) {
       std::vector<Deferred> all = deferred;
       all.push_back({pos, dypos});
-      runs = make_runs(all);
+      *runs = make_runs(all);
       gws = wgrad_stream ? wgrad_stream : stream;
     }
     if (ws || (gws && gws != stream)) DS_PROPAGATE(lane.ensure());
     // fp32 stream: the gradient that travels down the layers is fp32 (dyf); its bf16 copies feed the GEMMs
     const float* dyf = nullptr;
     if (rs32) {
-      DS_PROPAGATE(ds_cast_bf16_to_f32(ws_base + bw_dxf[L & 1], d_out, (size_t)rows * H, stream));
-      dyf = (const float*)(ws_base + bw_dxf[L & 1]);
+      float* dst = (float*)(ws_base + bw_dxf[L & 1]);
+      add(st, [=]() { return ds_cast_bf16_to_f32(dst, d_out, (size_t)rows * H, stream); });
+      dyf = dst;
     }
+    const char* dy = (const char*)d_out;
     for (int l = L - 1; l >= 0; --l) {
       const LayerStash& t = ls[l];
       const int b = base(l);
@@ -574,82 +758,118 @@ struct BertStage : ds_stage {
       char* dqkv = G > 1 ? dy_base + ld[l].dqkv + dypos * 3 * dy_act : ws_base + ws_dqkv[par];
       float* dp = (float*)(ws_base + ws_scores);
       char* dsm = ws_base + ws_ds;
-      // the wgrads that read this parity's buffers two layers up must have run
-      if (ws) DS_PROPAGATE(lane.reuse(stream, par));
       const int res32 = DS_EPI_RESIDUAL | DS_EPI_RESIDUAL_F32 | DS_EPI_OUT_F32;
       float* dz2f = (float*)(ws_base + bw_dz2f);
       float* daf = (float*)(ws_base + bw_daf);
       float* dz1f = (float*)(ws_base + bw_dz1f);
+      const float* z2 = (const float*)at(t.z2, pos);
+      const float* z1 = (const float*)at(t.z1, pos);
+      const float* st2 = (const float*)(at(t.st2, pos));
+      const float* st1 = (const float*)(at(t.st1, pos));
       // output LayerNorm; the column sums of dz2 are the gradient of output/dense/bias
       // (fp32 stream with grouped weight gradients: the chain only computes dz; gamma, beta and bias gradients follow
       // with the group's weight gradients, from bf16 copies of dy kept beside dz in the operand ring)
       const bool ln_deferred = rs32 && G > 1;
-      if (ln_deferred)
-        DS_PROPAGATE(ds_layernorm_bwd_mixed(rows, H, dyf, (const float*)at(t.z2, pos), w[b + LN2_G], (const float*)(at(t.st2, pos)), dz2, dz2f,
-                                            dy_base + ld[l].dyn2 + dypos * dy_act, nullptr, nullptr, nullptr, stream));
-      else if (rs32)
-        DS_PROPAGATE(ds_layernorm_bwd_mixed(rows, H, dyf, (const float*)at(t.z2, pos), w[b + LN2_G], (const float*)(at(t.st2, pos)), dz2, dz2f,
-                                            nullptr, g[b + LN2_G], g[b + LN2_B], g[b + B_FF2], stream));
-      else
-        DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, dy, at(t.z2, pos), w[b + LN2_G], (const float*)(at(t.st2, pos)), nullptr, dz2,
-                                      g[b + LN2_G], g[b + LN2_B], g[b + B_FF2], stream));
+      Step* first_step;
+      if (ln_deferred) {
+        first_step = &add_ln_bwd_rows(st, prio, dyf, z2, w[b + LN2_G], st2, dz2, dz2f, dy_base + ld[l].dyn2 + dypos * dy_act);
+      } else if (rs32) {
+        const float* dyin = dyf;
+        first_step = &add(st, [=]() {
+          return ds_layernorm_bwd_mixed(rows, H, dyin, z2, w[b + LN2_G], st2, dz2, dz2f, nullptr, g[b + LN2_G], g[b + LN2_B], g[b + B_FF2], stream);
+        });
+      } else {
+        const char* dyin = dy;
+        first_step = &add(st, [=]() {
+          return ds_layernorm_bwd(dtype, rows, H, dyin, z2, w[b + LN2_G], st2, nullptr, dz2, g[b + LN2_G], g[b + LN2_B], g[b + B_FF2], stream);
+        });
+      }
+      // the wgrads that read this parity's buffers two layers up must have run
+      if (ws) first_step->before = [this, par]() { return lane.reuse(stream, par); };
       // du = (dz2 W2^T) * gelu'(u)
-      DS_PROPAGATE(gemm_dgrad(rows, H, F, dz2, weight_T(l, W_FF2), du, DS_EPI_MUL, nullptr, at(t.u, pos)));
+      add_gemm(st, desc_dgrad(rows, H, F, dz2, weight_T(l, W_FF2), du, DS_EPI_MUL, nullptr, at(t.u, pos)), prio);
       // da = du W1^T + dz2 (a also feeds the residual into z2)
-      if (rs32) DS_PROPAGATE(gemm_dgrad(rows, F, H, du, weight_T(l, W_FF1), daf, res32, dz2f, nullptr));
-      else DS_PROPAGATE(gemm_dgrad(rows, F, H, du, weight_T(l, W_FF1), da, DS_EPI_RESIDUAL, dz2, nullptr));
+      if (rs32) add_gemm(st, desc_dgrad(rows, F, H, du, weight_T(l, W_FF1), daf, res32, dz2f, nullptr), prio);
+      else add_gemm(st, desc_dgrad(rows, F, H, du, weight_T(l, W_FF1), da, DS_EPI_RESIDUAL, dz2, nullptr), prio);
       // attention-output LayerNorm; column sums of dz1 = gradient of attention/output/dense/bias
-      if (ln_deferred)
-        DS_PROPAGATE(ds_layernorm_bwd_mixed(rows, H, daf, (const float*)at(t.z1, pos), w[b + LN1_G], (const float*)(at(t.st1, pos)), dz1, dz1f,
-                                            dy_base + ld[l].dyn1 + dypos * dy_act, nullptr, nullptr, nullptr, stream));
-      else if (rs32)
-        DS_PROPAGATE(ds_layernorm_bwd_mixed(rows, H, daf, (const float*)at(t.z1, pos), w[b + LN1_G], (const float*)(at(t.st1, pos)), dz1, dz1f,
-                                            nullptr, g[b + LN1_G], g[b + LN1_B], g[b + B_AO], stream));
-      else
-        DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, da, at(t.z1, pos), w[b + LN1_G], (const float*)(at(t.st1, pos)), nullptr, dz1,
-                                      g[b + LN1_G], g[b + LN1_B], g[b + B_AO], stream));
-      DS_PROPAGATE(gemm_dgrad(rows, H, H, dz1, weight_T(l, W_AO), dctx, 0, nullptr, nullptr));
+      if (ln_deferred) {
+        add_ln_bwd_rows(st, prio, daf, z1, w[b + LN1_G], st1, dz1, dz1f, dy_base + ld[l].dyn1 + dypos * dy_act);
+      } else if (rs32) {
+        add(st, [=]() {
+          return ds_layernorm_bwd_mixed(rows, H, daf, z1, w[b + LN1_G], st1, dz1, dz1f, nullptr, g[b + LN1_G], g[b + LN1_B], g[b + B_AO], stream);
+        });
+      } else {
+        add(st, [=]() {
+          return ds_layernorm_bwd(dtype, rows, H, da, z1, w[b + LN1_G], st1, nullptr, dz1, g[b + LN1_G], g[b + LN1_B], g[b + B_AO], stream);
+        });
+      }
+      // d ctx = dz1 Wo^T; as a task of a grouped launch it also leaves delta = rowsum(d ctx * ctx) per head, which lets the
+      // two attention-backward kernels run side by side (alone, the dQ kernel computes delta and the dK/dV kernel waits for it)
+      {
+        Step& s = add_gemm(st, desc_dgrad(rows, H, H, dz1, weight_T(l, W_AO), dctx, 0, nullptr, nullptr), prio);
+        if (s.nops) {
+          s.ops[0].gemm.c2 = at(t.ctx, pos);
+          s.ops[0].rowdot = dp;
+          s.ops[0].rowdot_seq = S;
+        }
+      }
       // attention backward per (batch, head)
       const char* q = at(t.qkv, pos);
       const char* k = q + (size_t)H * esz;
       const char* v = q + (size_t)2 * H * esz;
       const int64_t so3 = (int64_t)S * 3 * H, soH = (int64_t)S * H, soP = (int64_t)NH * S * S, siP = (int64_t)S * S;
+      Step* attn_step;
       if (fused_attn) {
         const float* mask = slot_has_mask[slot] ? (const float*)(sm + mask_off) : nullptr;
-        DS_PROPAGATE(ds_attention_bwd(dtype, B, NH, S, D, q, 3 * H, mask, scale, -10000.0f, at(t.ctx, pos), (const float*)(at(t.lse, pos)),
-                                      dctx, dqkv, dp, stream));
+        char* ctx = at(t.ctx, pos);
+        const float* lse = (const float*)(at(t.lse, pos));
+        attn_step = &add(st, [=]() {
+          return ds_attention_bwd(dtype, B, NH, S, D, q, 3 * H, mask, scale, -10000.0f, ctx, lse, dctx, dqkv, dp, stream);
+        });
+        if (groupable()) {
+          attn_step->nops = 2;
+          attn_op(attn_step->ops[0], GOP_ATTN_DKV, prio, q, mask, ctx, (float*)lse, dctx, dqkv, dp);
+          attn_op(attn_step->ops[1], GOP_ATTN_DQ, prio, q, mask, ctx, (float*)lse, dctx, dqkv, nullptr);
+        }
       } else {
-      // dP = dctx V^T (fp32)
-      DS_PROPAGATE(gemm_heads(DS_K_MAJOR, DS_K_MAJOR, S, S, D, dctx, H, soH, D, v, 3 * H, so3, D, dp, S, soP, siP,
-                              DS_EPI_OUT_F32));
-      // dV = P^T dctx
-      DS_PROPAGATE(gemm_heads(DS_MN_MAJOR, DS_MN_MAJOR, S, D, S, at(t.p, pos), S, soP, siP, dctx, H, soH, D,
-                              dqkv + (size_t)2 * H * esz, 3 * H, so3, D, 0));
-      // dS = scale * P * (dP - rowsum(dP * P))
-      DS_PROPAGATE(ds_softmax_bwd(dtype, (int64_t)B * NH * S, S, at(t.p, pos), dp, scale, dsm, stream));
-      // dQ = dS K ; dK = dS^T Q
-      DS_PROPAGATE(gemm_heads(DS_K_MAJOR, DS_MN_MAJOR, S, D, S, dsm, S, soP, siP, k, 3 * H, so3, D, dqkv, 3 * H, so3, D, 0));
-      DS_PROPAGATE(gemm_heads(DS_MN_MAJOR, DS_MN_MAJOR, S, D, S, dsm, S, soP, siP, q, 3 * H, so3, D,
-                              dqkv + (size_t)H * esz, 3 * H, so3, D, 0));
+        char* p = at(t.p, pos);
+        attn_step = &add(st, [=]() {
+          // dP = dctx V^T (fp32)
+          DS_PROPAGATE(gemm_heads(DS_K_MAJOR, DS_K_MAJOR, S, S, D, dctx, H, soH, D, v, 3 * H, so3, D, dp, S, soP, siP, DS_EPI_OUT_F32));
+          // dV = P^T dctx
+          DS_PROPAGATE(gemm_heads(DS_MN_MAJOR, DS_MN_MAJOR, S, D, S, p, S, soP, siP, dctx, H, soH, D, dqkv + (size_t)2 * H * esz, 3 * H, so3, D, 0));
+          // dS = scale * P * (dP - rowsum(dP * P))
+          DS_PROPAGATE(ds_softmax_bwd(dtype, (int64_t)B * NH * S, S, p, dp, scale, dsm, stream));
+          // dQ = dS K ; dK = dS^T Q
+          DS_PROPAGATE(gemm_heads(DS_K_MAJOR, DS_MN_MAJOR, S, D, S, dsm, S, soP, siP, k, 3 * H, so3, D, dqkv, 3 * H, so3, D, 0));
+          return gemm_heads(DS_MN_MAJOR, DS_MN_MAJOR, S, D, S, dsm, S, soP, siP, q, 3 * H, so3, D, dqkv + (size_t)H * esz, 3 * H, so3, D, 0);
+        });
       }
       // ---- weight gradients of this layer (on the weight-gradient stream when there is one)
       if (G == 1) {
-        hipStream_t chain = stream;
-        if (ws) {
-          DS_PROPAGATE(lane.begin(chain, ws, par));
-          stream = ws;  // the GEMMs and column sums of layer_wgrad launch on `stream`
-        }
-        const int rc = layer_wgrad(l, rows, at(t.x, pos), at(t.ctx, pos), at(t.a, pos), at(t.h, pos), dz2, du, dz1, dqkv);
-        stream = chain;
-        if (rc != DS_OK) return rc;
-        if (ws) DS_PROPAGATE(lane.end(ws, par));
+        const char *x = at(t.x, pos), *ctx = at(t.ctx, pos), *a = at(t.a, pos), *h = at(t.h, pos);
+        attn_step->after = [=]() {
+          hipStream_t chain = stream;
+          if (ws) {
+            DS_PROPAGATE(lane.begin(chain, ws, par));
+            stream = ws;  // the GEMMs and column sums of layer_wgrad launch on `stream`
+          }
+          const int rc = layer_wgrad(l, rows, x, ctx, a, h, dz2, du, dz1, dqkv);
+          stream = chain;
+          if (rc != DS_OK) return rc;
+          if (ws) DS_PROPAGATE(lane.end(ws, par));
+          return (int)DS_OK;
+        };
       } else if (closing) {
-        hipStream_t chain = stream;
-        if (gws != chain) DS_PROPAGATE(lane.begin(chain, gws, par));
-        stream = gws;
-        const int rc = layer_wgrad_runs(l, runs);
-        stream = chain;
-        if (rc != DS_OK) return rc;
+        attn_step->after = [=]() {
+          hipStream_t chain = stream;
+          hipStream_t side = wgrad_stream ? wgrad_stream : chain;
+          if (side != chain) DS_PROPAGATE(lane.begin(chain, side, par));
+          stream = side;
+          const int rc = layer_wgrad_runs(l, *runs);
+          stream = chain;
+          return rc;
+        };
       }
       // dx = dqkv Wqkv^T + dz1 (x also feeds the residual into z1)
       const bool first = (l == 0);
@@ -657,47 +877,51 @@ struct BertStage : ds_stage {
       char* dx = first ? (emb ? ws_base + ws_dx[0] : (char*)d_in) : ws_base + ws_dx[l & 1];
       if (rs32 && !first) {
         float* dxf = (float*)(ws_base + bw_dxf[l & 1]);
-        DS_PROPAGATE(gemm_dgrad(rows, 3 * H, H, dqkv, wqkv[l], dxf, res32, dz1f, nullptr));
+        add_gemm(st, desc_dgrad(rows, 3 * H, H, dqkv, wqkv[l], dxf, res32, dz1f, nullptr), prio);
         dyf = dxf;
       } else if (rs32) {  // the stage's input gradient leaves as bf16
-        DS_PROPAGATE(gemm_dgrad(rows, 3 * H, H, dqkv, wqkv[l], dx, DS_EPI_RESIDUAL | DS_EPI_RESIDUAL_F32, dz1f, nullptr));
+        add_gemm(st, desc_dgrad(rows, 3 * H, H, dqkv, wqkv[l], dx, DS_EPI_RESIDUAL | DS_EPI_RESIDUAL_F32, dz1f, nullptr), prio);
       } else {
-        DS_PROPAGATE(gemm_dgrad(rows, 3 * H, H, dqkv, wqkv[l], dx, DS_EPI_RESIDUAL, dz1, nullptr));
+        add_gemm(st, desc_dgrad(rows, 3 * H, H, dqkv, wqkv[l], dx, DS_EPI_RESIDUAL, dz1, nullptr), prio);
       }
       dy = dx;
     }
     // the stash slot and the master gradients are released to the caller in the order of `stream`
-    if (ws) DS_PROPAGATE(lane.finish(stream));
-    if (G > 1) {
-      deferred.push_back({pos, dypos});
-      pos_deferred[pos] = 1;
-      pos_owner[pos] = -1;
-      ++n_backward;
-    }
-    if (emb) {
-      // embedding LayerNorm backward, then scatter-add into the three tables
-      char* de = ws_base + ws_dz2[0];
-      DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, dy, at(emb_e, pos), w[E_LN_G], (const float*)(at(emb_st, pos)), nullptr, de,
-                                    g[E_LN_G], g[E_LN_B], nullptr, stream));
-      const int32_t* tt = slot_has_tt[slot] ? (const int32_t*)(sm + emb_tt) : nullptr;
-      dim3 grid((rows + 3) / 4);
-      if (dtype == DS_BF16)
-        hipLaunchKernelGGL(embed_bwd_kernel<bf16>, grid, dim3(256), 0, stream, rows, H, S, cfg.vocab, cfg.type_vocab,
-                           (const int32_t*)(sm + emb_ids), tt, (const bf16*)de, g[E_WORD], g[E_TYPE], g[E_POS]);
-      else
-        hipLaunchKernelGGL(embed_bwd_kernel<float>, grid, dim3(256), 0, stream, rows, H, S, cfg.vocab, cfg.type_vocab,
-                           (const int32_t*)(sm + emb_ids), tt, (const float*)de, g[E_WORD], g[E_TYPE], g[E_POS]);
-      DS_CHECK_LAUNCH();
-    }
-    if (G > 1) {
-      if (bwd_stream) {
-        DS_CHECK_HIP(hipEventRecord(ev_x_bwd[pos], stream));
-        x_bwd_valid[pos] = 1;
-      } else {
-        x_bwd_valid[pos] = 0;
+    const char* dy_last = dy;
+    add(st, [=]() {
+      if (ws) DS_PROPAGATE(lane.finish(stream));
+      if (G > 1) {
+        deferred.push_back({pos, dypos});
+        pos_deferred[pos] = 1;
+        pos_owner[pos] = -1;
+        ++n_backward;
       }
-      if (closing) DS_PROPAGATE(retire_deferred(gws, stream));
-    }
+      if (emb) {
+        // embedding LayerNorm backward, then scatter-add into the three tables
+        char* de = ws_base + ws_dz2[0];
+        DS_PROPAGATE(ds_layernorm_bwd(dtype, rows, H, dy_last, at(emb_e, pos), w[E_LN_G], (const float*)(at(emb_st, pos)), nullptr, de,
+                                      g[E_LN_G], g[E_LN_B], nullptr, stream));
+        const int32_t* tt = slot_has_tt[slot] ? (const int32_t*)(sm + emb_tt) : nullptr;
+        dim3 grid((rows + 3) / 4);
+        if (dtype == DS_BF16)
+          hipLaunchKernelGGL(embed_bwd_kernel<bf16>, grid, dim3(256), 0, stream, rows, H, S, cfg.vocab, cfg.type_vocab,
+                             (const int32_t*)(sm + emb_ids), tt, (const bf16*)de, g[E_WORD], g[E_TYPE], g[E_POS]);
+        else
+          hipLaunchKernelGGL(embed_bwd_kernel<float>, grid, dim3(256), 0, stream, rows, H, S, cfg.vocab, cfg.type_vocab,
+                             (const int32_t*)(sm + emb_ids), tt, (const float*)de, g[E_WORD], g[E_TYPE], g[E_POS]);
+        DS_CHECK_LAUNCH();
+      }
+      if (G > 1) {
+        if (bwd_stream) {
+          DS_CHECK_HIP(hipEventRecord(ev_x_bwd[pos], stream));
+          x_bwd_valid[pos] = 1;
+        } else {
+          x_bwd_valid[pos] = 0;
+        }
+        if (closing) DS_PROPAGATE(retire_deferred(wgrad_stream ? wgrad_stream : stream, stream));
+      }
+      return (int)DS_OK;
+    });
     return DS_OK;
   }
 

@@ -54,6 +54,73 @@ def cast_to_f32(src):
     return dst
 
 
+def _check_gemm_operands(a, b, c, m, n, k, a_major, b_major, lda, ldb, ldc, flags, batch, a_strides, b_strides, c_strides,
+                         bias, residual, c2):
+    """Every element the kernels may touch must lie inside the tensors handed in: a wrong shape would fault the GPU."""
+    if a.dtype != b.dtype:
+        raise ValueError("A and B must have one element type")
+    want_c = torch.float32 if (flags & (DS_EPI_OUT_F32 | DS_EPI_ACCUM)) or a.dtype == torch.float32 else torch.bfloat16
+    if c.dtype != want_c:
+        raise ValueError("C must be %s for these flags" % want_c)
+    zmax = batch - 1
+
+    def extent(rows, cols, ld, strides):
+        return (rows - 1) * ld + cols + zmax * (abs(strides[0]) + abs(strides[1]))
+    need_a = extent(m, k, lda, a_strides) if a_major == DS_K_MAJOR else extent(k, m, lda, a_strides)
+    need_b = extent(n, k, ldb, b_strides) if b_major == DS_K_MAJOR else extent(k, n, ldb, b_strides)
+    need_c = extent(m, n, ldc, c_strides)
+    if a.numel() < need_a or b.numel() < need_b or c.numel() < need_c:
+        raise ValueError("operand too small: A %d < %d, B %d < %d or C %d < %d elements" %
+                         (a.numel(), need_a, b.numel(), need_b, c.numel(), need_c))
+    if bias is not None and (bias.dtype != torch.float32 or bias.numel() < n):
+        raise ValueError("bias must be fp32 with at least n elements")
+    if residual is not None and residual.numel() < need_c:
+        raise ValueError("residual too small")
+    if c2 is not None and c2.numel() < need_c:
+        raise ValueError("c2 too small")
+
+
+def _gemm_desc(a, b, c, m, n, k, a_major, b_major, lda, ldb, ldc, flags, alpha, bias, residual, c2, batch, batch_inner,
+               a_strides, b_strides, c_strides):
+    _need_cuda(a, b, c, bias, residual, c2)
+    d = GemmDesc()
+    d.dtype = dtype_code(a)
+    d.a_major, d.b_major = a_major, b_major
+    d.m, d.n, d.k = m, n, k
+    d.lda = lda if lda is not None else (k if a_major == DS_K_MAJOR else m)
+    d.ldb = ldb if ldb is not None else (k if b_major == DS_K_MAJOR else n)
+    d.ldc = ldc if ldc is not None else n
+    _check_gemm_operands(a, b, c, m, n, k, a_major, b_major, d.lda, d.ldb, d.ldc, flags, batch, a_strides, b_strides,
+                         c_strides, bias, residual, c2)
+    d.batch, d.batch_inner = batch, batch_inner
+    d.a_stride_outer, d.a_stride_inner = a_strides
+    d.b_stride_outer, d.b_stride_inner = b_strides
+    d.c_stride_outer, d.c_stride_inner = c_strides
+    d.flags, d.alpha = flags, alpha
+    d.a, d.b, d.c = a.data_ptr(), b.data_ptr(), c.data_ptr()
+    d.bias = bias.data_ptr() if bias is not None else None
+    d.residual = residual.data_ptr() if residual is not None else None
+    d.c2 = c2.data_ptr() if c2 is not None else None
+    return d
+
+
+def gemm_grouped(problems):
+    """ds_gemm_grouped: `problems` is a list of dicts with the keyword arguments of `gemm` (a, b, c, m, n, k, a_major,
+    b_major, flags, bias, residual, c2, ...) plus `cfg`, the tile shape (0 = 256x256, 1 = 256x128, 2 = 128x128,
+    3 = 128x64); all of them run as one launch, workgroups starting in list order."""
+    n = len(problems)
+    descs = (GemmDesc * n)()
+    cfgs = (C.c_int * n)()
+    for i, p in enumerate(problems):
+        p = dict(p)
+        cfgs[i] = p.pop("cfg", 2)
+        args = dict(a_major=DS_K_MAJOR, b_major=DS_MN_MAJOR, lda=None, ldb=None, ldc=None, flags=0, alpha=1.0, bias=None,
+                    residual=None, c2=None, batch=1, batch_inner=1, a_strides=(0, 0), b_strides=(0, 0), c_strides=(0, 0))
+        args.update(p)
+        descs[i] = _gemm_desc(**args)
+    check(_lib.load().ds_gemm_grouped(descs, cfgs, n, _lib.current_stream()), "ds_gemm_grouped")
+
+
 def gemm(a, b, c, m, n, k, a_major=DS_K_MAJOR, b_major=DS_MN_MAJOR, lda=None, ldb=None, ldc=None, flags=0,
          alpha=1.0, bias=None, residual=None, c2=None, batch=1, batch_inner=1, a_strides=(0, 0), b_strides=(0, 0),
          c_strides=(0, 0), workspace=None, static_scratch=False):

@@ -166,6 +166,23 @@ class Stage:
         ev = C.c_void_p(ready) if ready is not None else None
         check(self.lib.ds_stage_backward_after(self._h, slot, ptr(d_out), ptr(d_in), ev), "ds_stage_backward_after")
 
+    def forward_backward(self, fslot, x, out, bslot, d_out, d_in=None, key_mask=None):
+        """F(fslot) and B(bslot) of two different micro-batches as one call (``ds_stage_forward_backward``): stages that
+        pair passes walk both chains together, one launch per level; the others run the two passes one after the other.
+        The upstream gradient must already be ordered on the current stream."""
+        self._check_tensor(x, "stage input", self.in_dtype, self.in_numel)
+        self._check_tensor(out, "stage output", self.act_dtype, self.out_numel)
+        self._check_tensor(d_out, "upstream gradient", self.act_dtype, self.out_numel)
+        if d_in is not None:
+            self._check_tensor(d_in, "input gradient", self.act_dtype, self.in_numel)
+        if key_mask is not None:
+            if key_mask.dtype != torch.float32 or not key_mask.is_cuda or not key_mask.is_contiguous():
+                raise ValueError("key_mask must be a contiguous fp32 [batch, seq] tensor on the GPU")
+        if self._weights_stale:
+            self.refresh_weights()
+        check(self.lib.ds_stage_forward_backward(self._h, fslot, ptr(x), ptr(key_mask), ptr(out), bslot, ptr(d_out), ptr(d_in)),
+              "ds_stage_forward_backward")
+
     def release(self, slot):
         """Gives up the micro-batch forwarded into ``slot`` without a backward pass (forward-only use)."""
         check(self.lib.ds_stage_release_slot(self._h, slot), "ds_stage_release_slot")
@@ -408,8 +425,12 @@ def xlnet_stage(num_layers, hidden, heads, ffn, batch, seq, dtype, stash_slots, 
 class StageRuntime:
     """Runs one stage over M micro-batches in the early-backward order."""
 
-    def __init__(self, stage, stage_index=0, num_stages=2, num_micro_batches=8, variant="S", needs_input_grad=True):
+    def __init__(self, stage, stage_index=0, num_stages=2, num_micro_batches=8, variant="S", needs_input_grad=True,
+                 pair_passes=False):
+        """``pair_passes``: where the order has F(j+1) directly in front of B(j) - its steady state - issue the two as one
+        ``Stage.forward_backward`` call (same results; stages that pair passes run them level by level in one launch each)."""
         self.stage = stage
+        self.pair_passes = bool(pair_passes)
         self.ops = schedule_ops(stage_index, num_stages, num_micro_batches, variant)
         self.k = min(stash_depth(stage_index, num_stages, variant), num_micro_batches)
         if stage.stash_slots < self.k:
@@ -429,13 +450,25 @@ class StageRuntime:
         if self.stage.overlap:
             ready = torch.cuda.Event()
             ready.record()
-        for op, j in self.ops:
+        i = 0
+        while i < len(self.ops):
+            op, j = self.ops[i]
+            i += 1
             if op == "F":
                 slot = free.pop(0)
                 slot_of[j] = slot
                 if before_forward is not None:
                     before_forward(slot, j)          # e.g. XlnetStage.set_inputs for this micro-batch
-                self.stage.forward(slot, inputs[j], outputs[j], None if key_masks is None else key_masks[j])
+                mask = None if key_masks is None else key_masks[j]
+                if self.pair_passes and i < len(self.ops) and self.ops[i][0] == "B":
+                    jb = self.ops[i][1]
+                    i += 1
+                    bslot = slot_of.pop(jb)
+                    d_in = input_grads[jb] if (self.needs_input_grad and input_grads is not None) else None
+                    self.stage.forward_backward(slot, inputs[j], outputs[j], bslot, upstream[jb], d_in, key_mask=mask)
+                    free.append(bslot)
+                    continue
+                self.stage.forward(slot, inputs[j], outputs[j], mask)
             else:
                 slot = slot_of.pop(j)
                 d_in = input_grads[j] if (self.needs_input_grad and input_grads is not None) else None

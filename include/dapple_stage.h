@@ -114,6 +114,14 @@ size_t ds_gemm_workspace_bytes(int m, int n);
  * process ends), bf16, batch 1, and a shape that ds_gemm would cut (DS_EINVAL otherwise, with the reason).  All calls
  * on one GPU share the scratch: calls that overlap in time on one GPU race; calls on one stream do not. */
 int ds_gemm_static_scratch(const ds_gemm_desc* d, void* stream);
+/* Several independent GEMMs as ONE launch (bf16, k % 64 == 0, the operand-major pairs (K, MN), (K, K), (MN, MN); at
+ * most 8 problems).  What a stage holds in steady state - a forward product of one micro-batch, an input-gradient
+ * product of another (the reference's graph orders them only by control dependencies, bert/graph.py:126-132) and
+ * weight-gradient products nothing waits for (bert/graph.py:145-161) - is too small per problem to fill the GPU
+ * with large tiles; together it is not.  cfgs[i] is the tile shape of problem i: 0 = 256 x 256, 1 = 256 x 128,
+ * 2 = 128 x 128, 3 = 128 x 64.  Workgroups start in the order of the list: put what other work waits for first.
+ * Results are those of ds_gemm on each descriptor (d->workspace is ignored: no k slicing). */
+int ds_gemm_grouped(const ds_gemm_desc* descs, const int* cfgs, int n, void* stream);
 
 /* ---------------------------------------------------------------------------
  * LayerNorm over the last axis, y = (x - mean) * rsqrt(var + eps) * gamma + beta,
@@ -247,6 +255,16 @@ int ds_stage_backward(ds_stage* h, int slot, const void* d_out, void* d_in);
 int ds_stage_backward_after(ds_stage* h, int slot, const void* d_out, void* d_in, void* ready_event);
 void* ds_stage_backward_event(ds_stage* h, int slot);
 int ds_stage_wait_backward(ds_stage* h, int slot, void* stream);
+/* The forward pass of one micro-batch into `fslot` and the backward pass of another out of `bslot` as ONE call
+ * (arguments of ds_stage_forward and ds_stage_backward).  The reference's graph leaves the two unordered: only the
+ * control dependencies of bert/graph.py:126-132 constrain them.  A BERT stage in bf16 with fused attention, the fp32
+ * residual stream and wgrad_group > 1 walks both chains together on the stage's stream, one launch per level carrying
+ * the next operation of either chain (large tiles for both instead of small ones for each); every other stage runs
+ * the two calls one after the other.  d_out must be ordered before the call on the stage's stream; d_in, out and the
+ * gradients follow the stage's stream (ds_stage_join / ds_stage_sync at the end of a step, as for separate calls).
+ * Results equal those of the separate calls up to the rounding of a different tile order in the GEMMs. */
+int ds_stage_forward_backward(ds_stage* h, int fslot, const void* in, const float* key_mask, void* out, int bslot,
+                              const void* d_out, void* d_in);
 /* Gives up the micro-batch forwarded into `slot` without a backward pass: a forward-only use of the stage (the
  * reference's is_training=False graphs, bert/models/bert/modeling_slice.py:774-776, build no gradients). */
 int ds_stage_release_slot(ds_stage* h, int slot);

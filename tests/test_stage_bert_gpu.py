@@ -19,7 +19,7 @@ ADT = {"fp32": torch.float32, "bf16": torch.bfloat16}
 
 
 def run_case(dtype, L, H, N, F, B, S, M, embeddings=None, use_mask=False, K=2, stage_index=0, odtype=torch.float64,
-             seed=0, perturb=True, stddev=0.05, wgrad_group=1, overlap=False):
+             seed=0, perturb=True, stddev=0.05, wgrad_group=1, overlap=False, pair_passes=False):
     w_np = synthetic.bert_weights(synthetic.SEED_WEIGHT + seed, L, H, F, embeddings=embeddings, stddev=stddev,
                                   perturb=perturb)
     if embeddings is not None:
@@ -45,7 +45,7 @@ def run_case(dtype, L, H, N, F, B, S, M, embeddings=None, use_mask=False, K=2, s
     outs = [torch.empty(B * S, H, dtype=adt, device="cuda") for _ in range(M)]
     dxs = None if embeddings is not None else [torch.empty(B * S, H, dtype=adt, device="cuda") for _ in range(M)]
     masks = None if masks_np is None else [dev(m) for m in masks_np]
-    rt = runtime.StageRuntime(stage, stage_index=stage_index, num_stages=stage_index + K, num_micro_batches=M)
+    rt = runtime.StageRuntime(stage, stage_index=stage_index, num_stages=stage_index + K, num_micro_batches=M, pair_passes=pair_passes)
     rt.step(xs, dys, outs, dxs, masks)
     stage.sync()
     torch.cuda.synchronize()
