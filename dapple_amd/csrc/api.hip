@@ -111,6 +111,10 @@ extern "C" int ds_stage_overlap_supported(const ds_stage* h) { return h && h->ov
 
 // Orders everything queued on the backward stream before whatever is queued next on the stage's stream.
 static int stage_join(ds_stage* h) {
+  if (h->bwd_stream && h->pair_valid) {  // what a paired pass queued on the stage's stream precedes what follows on the backward stream
+    DS_CHECK_HIP(hipStreamWaitEvent(h->bwd_stream, h->ev_pair, 0));
+    h->pair_valid = false;
+  }
   DS_PROPAGATE(h->flush_deferred(true));
   if (h->bwd_stream && h->bwd_pending) {
     DS_CHECK_HIP(hipEventRecord(h->ev_join, h->bwd_stream));

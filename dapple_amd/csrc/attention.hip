@@ -40,6 +40,7 @@ int check(const char* who, int dtype, int B, int N, int S, int D) {
   DS_CHECK_ARG(D == HD, "%s: head size must be %d (got %d)", who, HD, D);
   DS_CHECK_ARG(B > 0 && N > 0 && S > 0 && S % 64 == 0, "%s: seq (%d) must be a positive multiple of 64", who, S);
   DS_CHECK_ARG(S <= 2048, "%s: seq %d exceeds 2048", who, S);
+  DS_CHECK_ARG((int64_t)B * N <= 65535, "%s: batch * heads = %lld exceeds the 65535 a launch grid holds", who, (long long)B * N);
   return DS_OK;
 }
 
@@ -53,7 +54,7 @@ extern "C" int ds_attention_fwd(int dtype, int batch, int heads, int seq, int he
   AttnArgs a;
   a.qkv = (const bf16*)qkv; a.ld = ld; a.key_mask = key_mask; a.ctx = (bf16*)ctx; a.lse = lse; a.dctx = nullptr; a.dqkv = nullptr;
   a.delta = nullptr; a.B = batch; a.N = heads; a.S = seq; a.H = heads * head_dim; a.scale = scale; a.mask_value = mask_value;
-  a.prio = ds_launch_prio;
+  a.prio = ds_launch_prio; a.kbar = nullptr;
   static bool attr = false;
   if (!attr) {
     DS_CHECK_HIP(hipFuncSetAttribute((const void*)attn_fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(2048, 2)));
@@ -69,14 +70,31 @@ extern "C" int ds_attention_fwd(int dtype, int batch, int heads, int seq, int he
 extern "C" int ds_attention_bwd(int dtype, int batch, int heads, int seq, int head_dim, const void* qkv, int64_t ld,
                                 const float* key_mask, float scale, float mask_value, const void* ctx, const float* lse,
                                 const void* dctx, void* dqkv, float* delta, void* stream) {
+  return ds_attention_bwd_centered(dtype, batch, heads, seq, head_dim, qkv, ld, key_mask, scale, mask_value, ctx, lse, dctx, dqkv, delta,
+                                   nullptr, stream);
+}
+
+extern "C" int ds_attention_key_mean(int dtype, int batch, int heads, int seq, int head_dim, const void* qkv, int64_t ld, float* key_mean,
+                                     void* stream) {
+  DS_PROPAGATE(check("ds_attention_key_mean", dtype, batch, heads, seq, head_dim));
+  DS_CHECK_ARG(qkv && key_mean && ld >= 3 * heads * head_dim && ld % 8 == 0 && ds_aligned16(qkv) && ds_aligned16(key_mean),
+               "ds_attention_key_mean: null pointer, bad ld or alignment");
+  const int H = heads * head_dim;
+  return ds_sample_colsum(batch, seq, H, (const bf16*)qkv + H, ld, 1.0f / seq, key_mean, stream);
+}
+
+extern "C" int ds_attention_bwd_centered(int dtype, int batch, int heads, int seq, int head_dim, const void* qkv, int64_t ld,
+                                         const float* key_mask, float scale, float mask_value, const void* ctx, const float* lse,
+                                         const void* dctx, void* dqkv, float* delta, const float* key_mean, void* stream) {
   DS_PROPAGATE(check("ds_attention_bwd", dtype, batch, heads, seq, head_dim));
+  DS_CHECK_ARG(ds_aligned16(key_mean), "ds_attention_bwd: key_mean must be 16-byte aligned");
   DS_CHECK_ARG(qkv && ctx && lse && dctx && dqkv && delta, "ds_attention_bwd: null pointer");
   DS_CHECK_ARG(ld >= 3 * heads * head_dim && ld % 8 == 0 && ds_aligned16(qkv) && ds_aligned16(ctx) && ds_aligned16(dctx) &&
                ds_aligned16(dqkv), "ds_attention_bwd: bad ld or alignment");
   AttnArgs a;
   a.qkv = (const bf16*)qkv; a.ld = ld; a.key_mask = key_mask; a.ctx = (bf16*)ctx; a.lse = (float*)lse; a.dctx = (const bf16*)dctx;
   a.dqkv = (bf16*)dqkv; a.delta = delta; a.B = batch; a.N = heads; a.S = seq; a.H = heads * head_dim; a.scale = scale;
-  a.mask_value = mask_value; a.prio = ds_launch_prio;
+  a.mask_value = mask_value; a.prio = ds_launch_prio; a.kbar = key_mean;
   static bool attr = false;
   if (!attr) {
     DS_CHECK_HIP(hipFuncSetAttribute((const void*)attn_bwd_dq_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(2048, 2)));

@@ -112,6 +112,7 @@ struct AttnArgs {
   int B, N, S, H;
   float scale, mask_value;
   int prio;                      // wave priority (0..3)
+  const float* kbar;             // backward, nullable: [B, H] mean key of every sample and head (see attn_bwd_dq_body)
 };
 
 // Which (batch, head) pair and which 64-row block of the parallel axis a workgroup takes.  Workgroups go to the 8 XCDs
@@ -324,6 +325,14 @@ __device__ __forceinline__ void attn_bwd_dq_body(const AttnArgs& a, char* lds, i
   f32x16 dq[2];
 #pragma unroll
   for (int e = 0; e < 16; ++e) { dq[0][e] = 0.f; dq[1][e] = 0.f; }
+  // row sums of the bf16 dS that enter the dQ products, by the matrix pipe (it has time to spare; the vector ALU does not):
+  // ones[32 x 16] dS^T[16 x 32] puts the sum over a step's keys for query `lane % 32` into every register of rs
+  f32x16 rs;
+  bf16x8 ones;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) rs[e] = 0.f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) ones[j] = (bf16)1.0f;
   const float c2 = a.scale * LOG2E;
   __builtin_amdgcn_s_waitcnt(VMCNT0);  // the loads and the store above: from here on only tile loads are in flight
   for (int c = 0; c < nch; ++c) {
@@ -350,6 +359,7 @@ __device__ __forceinline__ void attn_bwd_dq_body(const AttnArgs& a, char* lds, i
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
         const bf16x8 df = pack8(ds + 8 * s2);
+        if (a.kbar != nullptr) rs = mfma(ones, df, rs);   // every row: what the rounded rows of dS sum to (exactly 0 before rounding)
 #pragma unroll
         for (int dt = 0; dt < 2; ++dt) dq[dt] = mfma(frag_cols(ck, kt + 16 * s2, dt * 32, lane), df, dq[dt]);  // dQ^T += K^T dS^T
       }
@@ -359,12 +369,42 @@ __device__ __forceinline__ void attn_bwd_dq_body(const AttnArgs& a, char* lds, i
       fill(c + 2);
     }
   }
+  // the mean key of this head, asked for now so that the trip to memory runs under the merge
+  f32x4 kv[2][4];
+  if (a.kbar != nullptr && part == 0) {
+    const float* kb = a.kbar + (int64_t)b * a.H + hd * HD;
+#pragma unroll
+    for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) kv[dt][g] = *reinterpret_cast<const f32x4*>(kb + dt * 32 + g * 8 + half * 4);
+  }
   __syncthreads();
-  if (part > 0) part_store<2>(lds + ((part - 1) * 2 + grp) * PART_BYTES, dq, lane);
+  if (part > 0) {
+    part_store<2>(lds + ((part - 1) * 2 + grp) * PART_BYTES, dq, lane);
+    part_store_xy(lds + ((part - 1) * 2 + grp) * PART_BYTES, rs[0], 0.f, lane);
+  }
   __syncthreads();
   if (part > 0) return;
+  float rsum = rs[0];
 #pragma unroll
-  for (int pp = 1; pp < SPLIT; ++pp) part_merge<2>(lds + ((pp - 1) * 2 + grp) * PART_BYTES, dq, 1.f, 1.f, lane);
+  for (int pp = 1; pp < SPLIT; ++pp) {
+    const char* slot = lds + ((pp - 1) * 2 + grp) * PART_BYTES;
+    part_merge<2>(slot, dq, 1.f, 1.f, lane);
+    float r1, unused;
+    part_xy(slot, r1, unused, lane);
+    rsum += r1;
+  }
+  if (a.kbar != nullptr) {
+    // Every row of dS sums to zero, so dQ = dS K = dS (K - 1 kbar^T) for any vector kbar.  The dS that entered the
+    // products above were rounded to bf16 and sum to rsum instead: against keys that share a large common part (token
+    // vectors that have grown alike over the layers) rsum * kbar is the bulk of dQ's rounding error, and it is known.
+#pragma unroll
+    for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dq[dt][g * 4 + j] -= rsum * kv[dt][g][j];
+  }
   store_t(a.dqkv + ((int64_t)b * a.S + q) * a.ld + hd * HD, dq, a.scale, half);
 }
 

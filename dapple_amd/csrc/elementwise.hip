@@ -1,6 +1,7 @@
 // HBM-bound kernels: gradient accumulation, casts, LayerNorm, softmax, column sums.
 // All move data as 16-byte vectors per lane with grid-stride or one-wave-per-row mappings.
 #include <stdlib.h>
+#include <string.h>
 
 #include "common.h"
 #include "rows_core.h"
@@ -989,4 +990,125 @@ int ds_colsum_accum_multi(int dtype, int rows, int cols, int count, const void* 
     hipLaunchKernelGGL(colsum_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, rows, cols, cb, ldx, rpb, fold);
   DS_CHECK_LAUNCH();
   return DS_OK;
+}
+
+// ------------------------------------------------------------------ per-sample column sums, rank-k correction
+// out[s][c] = scale * sum over the `seq` rows of sample s of x[s * seq + r][c] (bf16 x, row stride ldx).  Every row of
+// the score gradient of a softmax sums to zero, so a query gradient dS K only sees the keys' deviation from their mean,
+// and every head's key gradients sum to zero over a sample, so a key-projection weight gradient X^T dK only sees the
+// deviation of the layer's inputs from their mean: the means (and the column sums the rounded gradients are left with)
+// are what this kernel gives.  A block owns 64 columns of one sample: 8 lanes per row, 32 rows in flight.
+namespace {
+constexpr int SAMPLE_COLSUM_MAX = 64;
+struct SampleColsumArgs {
+  const bf16* x[SAMPLE_COLSUM_MAX];
+  float* out[SAMPLE_COLSUM_MAX];
+  int64_t ldx[SAMPLE_COLSUM_MAX];
+  float scale[SAMPLE_COLSUM_MAX];
+};
+// grid (ceil(cols / 64), samples, problems)
+__global__ __launch_bounds__(256) void sample_colsum_kernel(int seq, int cols, SampleColsumArgs a) {
+  __shared__ float red[32][65];
+  const int cg = threadIdx.x & 7, rg = threadIdx.x >> 3;
+  const int c = blockIdx.x * 64 + cg * 8, s = blockIdx.y, z = blockIdx.z;
+  const int64_t ldx = a.ldx[z];
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  if (c < cols) {
+    const bf16* base = a.x[z] + (int64_t)s * seq * ldx + c;
+#pragma unroll 4
+    for (int r = rg; r < seq; r += 32) {
+      const bf16x8 v = *reinterpret_cast<const bf16x8*>(base + (int64_t)r * ldx);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += (float)v[e];
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) red[rg][cg * 8 + e] = acc[e];
+  __syncthreads();
+  if (threadIdx.x < 64 && blockIdx.x * 64 + threadIdx.x < cols) {
+    float t = 0.f;
+#pragma unroll
+    for (int r = 0; r < 32; ++r) t += red[r][threadIdx.x];
+    a.out[z][(int64_t)s * cols + blockIdx.x * 64 + threadIdx.x] = t * a.scale[z];
+  }
+}
+
+// For every problem z: w[i][n] -= sum_{s < ns} a[s][i] * b[s][n] and, with v, v[n] -= sum_s b[s][n].
+// grid (ceil(cols / 1024), rows, problems), a thread owns 4 consecutive columns.
+constexpr int RANK_UPDATE_MAX = 32;
+struct RankUpdateArgs {
+  const float* a[RANK_UPDATE_MAX];
+  const float* b[RANK_UPDATE_MAX];
+  float* w[RANK_UPDATE_MAX];
+  float* v[RANK_UPDATE_MAX];
+};
+__global__ __launch_bounds__(256) void rank_update_kernel(int rows, int cols, int ns, int64_t ldw, RankUpdateArgs p) {
+  const int i = blockIdx.y, n = (blockIdx.x * 256 + threadIdx.x) * 4, z = blockIdx.z;
+  if (n >= cols) return;
+  const float* a = p.a[z];
+  const float* b = p.b[z];
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f}, tot = {0.f, 0.f, 0.f, 0.f};
+  for (int s = 0; s < ns; ++s) {
+    const float ai = a[(int64_t)s * rows + i];
+    const f32x4 bv = *reinterpret_cast<const f32x4*>(b + (int64_t)s * cols + n);
+    acc += ai * bv;
+    tot += bv;
+  }
+  f32x4* q = reinterpret_cast<f32x4*>(p.w[z] + (int64_t)i * ldw + n);
+  *q = *q - acc;
+  if (p.v[z] != nullptr && i == 0) {
+    f32x4* r = reinterpret_cast<f32x4*>(p.v[z] + n);
+    *r = *r - tot;
+  }
+}
+}  // namespace
+
+// `count` matrices of one shape (samples * seq rows, cols columns) in one launch: outs[i][s][c] = scales[i] * column sum of sample s of xs[i]
+int ds_sample_colsum_multi(int count, int samples, int seq, int cols, const void* const* xs, const int64_t* ldxs, const float* scales,
+                           float* const* outs, void* stream) {
+  DS_CHECK_ARG(count > 0 && samples > 0 && samples <= 65535 && seq > 0 && cols > 0 && cols % 8 == 0, "ds_sample_colsum: bad shape");
+  for (int first = 0; first < count; first += SAMPLE_COLSUM_MAX) {
+    const int n = count - first < SAMPLE_COLSUM_MAX ? count - first : SAMPLE_COLSUM_MAX;
+    SampleColsumArgs a;
+    memset(&a, 0, sizeof(a));
+    for (int i = 0; i < n; ++i) {
+      DS_CHECK_ARG(xs[first + i] && outs[first + i] && ds_aligned16(xs[first + i]) && ldxs[first + i] % 8 == 0 && ldxs[first + i] >= cols,
+                   "ds_sample_colsum: null or unaligned pointer, or a bad row stride");
+      a.x[i] = (const bf16*)xs[first + i]; a.out[i] = outs[first + i]; a.ldx[i] = ldxs[first + i]; a.scale[i] = scales[first + i];
+    }
+    ds_prof_scope prof((hipStream_t)stream, "sample_colsum_kernel", (double)n * samples * seq * cols * 2, "B");
+    hipLaunchKernelGGL(sample_colsum_kernel, dim3((cols + 63) / 64, samples, n), dim3(256), 0, (hipStream_t)stream, seq, cols, a);
+    DS_CHECK_LAUNCH();
+  }
+  return DS_OK;
+}
+
+int ds_sample_colsum(int samples, int seq, int cols, const void* x, int64_t ldx, float scale, float* out, void* stream) {
+  return ds_sample_colsum_multi(1, samples, seq, cols, &x, &ldx, &scale, &out, stream);
+}
+
+// `count` updates of one shape in one launch; the w (and v) of different problems must not overlap
+int ds_rank_update_multi(int count, int rows, int cols, int ns, const float* const* as, const float* const* bs, float* const* ws, int64_t ldw,
+                         float* const* vs, void* stream) {
+  DS_CHECK_ARG(count > 0 && rows > 0 && rows <= 65535 && cols > 0 && cols % 4 == 0 && ns > 0 && ldw % 4 == 0 && ldw >= cols, "ds_rank_update: bad shape");
+  for (int first = 0; first < count; first += RANK_UPDATE_MAX) {
+    const int n = count - first < RANK_UPDATE_MAX ? count - first : RANK_UPDATE_MAX;
+    RankUpdateArgs p;
+    memset(&p, 0, sizeof(p));
+    for (int i = 0; i < n; ++i) {
+      p.a[i] = as[first + i]; p.b[i] = bs[first + i]; p.w[i] = ws[first + i]; p.v[i] = vs ? vs[first + i] : nullptr;
+      DS_CHECK_ARG(p.a[i] && p.b[i] && p.w[i] && ds_aligned16(p.b[i]) && ds_aligned16(p.w[i]) && ds_aligned16(p.v[i]),
+                   "ds_rank_update: null or unaligned pointer");
+    }
+    ds_prof_scope prof((hipStream_t)stream, "rank_update_kernel", (double)n * rows * cols * 8, "B");
+    hipLaunchKernelGGL(rank_update_kernel, dim3((cols + 1023) / 1024, rows, n), dim3(256), 0, (hipStream_t)stream, rows, cols, ns, ldw, p);
+    DS_CHECK_LAUNCH();
+  }
+  return DS_OK;
+}
+
+int ds_rank_update(int rows, int cols, int ns, const float* a, const float* b, float* w, int64_t ldw, float* v, void* stream) {
+  return ds_rank_update_multi(1, rows, cols, ns, &a, &b, &w, ldw, &v, stream);
 }

@@ -36,6 +36,7 @@ struct GroupOp {
   const void* dctx = nullptr;
   void* dqkv = nullptr;
   float* delta = nullptr;
+  const float* key_mean = nullptr;  // GOP_ATTN_DQ, nullable: ds_attention_bwd_centered
   // GOP_LN_*: arguments of ds_layernorm_fwd_mixed / ds_layernorm_bwd_mixed
   int rows = 0, cols = 0;
   const float* x = nullptr;

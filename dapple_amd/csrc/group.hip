@@ -150,7 +150,7 @@ int fill_attention(const GroupOp& op, GroupTask& t, size_t* lds) {
   DS_CHECK_ARG((int64_t)op.B * op.N * (op.S / 64) < (1 << 24), "ds_group_launch: attention: too many workgroups");
   dsattn::AttnArgs& a = t.at;
   a.qkv = (const bf16*)op.qkv; a.ld = op.ld; a.key_mask = op.key_mask; a.ctx = (bf16*)op.ctx; a.lse = op.lse;
-  a.dctx = (const bf16*)op.dctx; a.dqkv = (bf16*)op.dqkv; a.delta = op.delta;
+  a.dctx = (const bf16*)op.dctx; a.dqkv = (bf16*)op.dqkv; a.delta = op.delta; a.kbar = op.key_mean;
   a.B = op.B; a.N = op.N; a.S = op.S; a.H = (int)H; a.scale = op.scale; a.mask_value = op.mask_value; a.prio = op.prio;
   DS_CHECK_ARG(a.ctx && a.lse && ds_aligned16(a.ctx), "ds_group_launch: attention: ctx and lse are needed");
   int vectors = op.key_mask ? 1 : 0;

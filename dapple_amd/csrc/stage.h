@@ -153,5 +153,15 @@ int ds_xl_bias_q(int rows, int B, int N, const void* q, const float* rw, const f
 int ds_xl_scores_fwd(const XlScoreArgs* a, hipStream_t stream);
 int ds_xl_scores_bwd(const XlScoreArgs* a, hipStream_t stream);
 int ds_gemm_splitk(const ds_gemm_desc* d, int splitk, void* stream);
+// out[s][c] = scale * sum over the seq rows of sample s of the bf16 matrix x (row stride ldx): per-sample column sums / means
+int ds_sample_colsum(int samples, int seq, int cols, const void* x, int64_t ldx, float scale, float* out, void* stream);
+// the same for `count` matrices of one shape in one launch
+int ds_sample_colsum_multi(int count, int samples, int seq, int cols, const void* const* xs, const int64_t* ldxs, const float* scales,
+                           float* const* outs, void* stream);
+// w[i][n] -= sum_{s < ns} a[s][i] * b[s][n] and, with v, v[n] -= sum_s b[s][n]   (a [ns][rows], b [ns][cols], w fp32 with row stride ldw)
+int ds_rank_update(int rows, int cols, int ns, const float* a, const float* b, float* w, int64_t ldw, float* v, void* stream);
+// `count` such updates of one shape in one launch (no two of them on the same w)
+int ds_rank_update_multi(int count, int rows, int cols, int ns, const float* const* as, const float* const* bs, float* const* ws, int64_t ldw,
+                         float* const* vs, void* stream);
 // ds_colsum_accum for up to 4 matrices of one shape in one launch
 int ds_colsum_accum_multi(int dtype, int rows, int cols, int count, const void* const* xs, int64_t ldx, float* const* outs, void* stream);

@@ -78,13 +78,14 @@ struct Ten {
   size_t off = 0, size = 0;
 };
 struct LayerStash {
-  Ten x, qkv, p, ctx, z1, a, u, h, z2, st1, st2, lse;
+  Ten x, qkv, p, ctx, z1, a, u, h, z2, st1, st2, lse, kbar, xbar;
 };
 // Upstream-gradient operands of a layer's weight-gradient GEMMs when those are deferred: per tensor a ring
 // of positions back to back, byte offsets into dy_base.
 struct LayerDy {
   size_t dz2, du, dz1, dqkv;
   size_t dyn2, dyn1;  // fp32 residual stream: bf16 copies of the gradients that entered the two LayerNorms
+  size_t dksum;       // fused attention: per sample, the column sums of the pass's key gradients (fp32 [B][H])
 };
 struct Deferred {
   int xpos, dypos;
@@ -99,6 +100,9 @@ struct BertStage : ds_stage {
   size_t esz;
   bool emb;
   bool fused_attn;  // bf16, head size 64: fused attention kernels, no [B,N,S,S] tensors at all
+  // fused attention: query gradients through ds_attention_bwd_centered, key parameter gradients from key gradients
+  // centred over each sample (DS_BERT_CENTRED=0 switches both off, for measurements)
+  bool centred = false, centre_q = false, centre_k = false;
   // bf16 with cfg.residual_fp32: the residual stream - the sums in front of both LayerNorms, the LayerNorm outputs that
   // feed the next sum, and the same chain of gradients in backward - stays in fp32; bf16 is only what a GEMM or the
   // attention kernels read.  The rounding of the stream itself, which otherwise adds up over the layers, is gone.
@@ -145,6 +149,7 @@ struct BertStage : ds_stage {
   char* ws_base = nullptr;
   size_t ws_bytes = 0;
   size_t ws_scores, ws_fscores, ws_ds, ws_dz2[2], ws_du[2], ws_da, ws_dz1[2], ws_dctx, ws_dqkv[2], ws_dx[2];
+  size_t ws_dksum = 0;
   WgradLane lane;
 
   ~BertStage() override {
@@ -170,6 +175,12 @@ struct BertStage : ds_stage {
     L = c.num_layers; H = c.hidden; F = c.ffn; NH = c.heads; B = c.batch; S = c.seq;
     D = H / NH; rows = B * S; dtype = c.dtype; esz = dtype == DS_BF16 ? 2 : 4; emb = c.with_embedding != 0;
     fused_attn = dtype == DS_BF16 && D == 64 && S % 64 == 0 && S <= 2048;
+    {
+      const char* env = getenv("DS_BERT_CENTRED");
+      centred = fused_attn && !(env && atoi(env) == 0);
+      centre_q = centred && !(env && atoi(env) == 3);
+      centre_k = centred && !(env && atoi(env) == 2);
+    }
     rs32 = dtype == DS_BF16 && c.residual_fp32 != 0 && L > 0 && H % 8 == 0 && H <= 2048;
     char name[160];
     if (emb) {
@@ -253,7 +264,11 @@ struct BertStage : ds_stage {
       LayerStash& t = ls[l];
       t.x = next_x;
       t.qkv = ring(3 * act);
-      if (fused_attn) t.lse = ring((size_t)B * NH * S * 4);
+      if (fused_attn) {
+        t.lse = ring((size_t)B * NH * S * 4);
+        t.kbar = ring((size_t)B * H * 4);  // mean key per sample and head
+        t.xbar = ring((size_t)B * H * 4);  // mean input row per sample
+      }
       else t.p = ring(probs);
       t.ctx = ring(act);
       t.z1 = ring(rs32 ? (size_t)rows * H * 4 : act);
@@ -287,6 +302,7 @@ struct BertStage : ds_stage {
           ld[l].dyn2 = da.reserve(act * NDY);
           ld[l].dyn1 = da.reserve(act * NDY);
         }
+        ld[l].dksum = da.reserve((size_t)B * H * 4 * NDY);
       }
       if (da.used) DS_CHECK_HIP(hipMalloc((void**)&dy_base, da.used));
       DS_CHECK_HIP(hipEventCreateWithFlags(&ev_chain, hipEventDisableTiming));
@@ -317,6 +333,10 @@ struct BertStage : ds_stage {
       fw_xf[0] = w.reserve(act32); fw_xf[1] = w.reserve(act32); fw_af = w.reserve(act32);
       bw_dxf[0] = w.reserve(act32); bw_dxf[1] = w.reserve(act32);
       bw_dz2f = w.reserve(act32); bw_daf = w.reserve(act32); bw_dz1f = w.reserve(act32);
+    }
+    if (fused_attn) {  // per-sample means of a layer's inputs and column sums of its key gradients (weight-gradient side)
+      const size_t ns = (size_t)(G > 1 ? G : 1) * B;
+      ws_dksum = w.reserve(ns * H * 4);
     }
     ws_bytes = w.used;
     DS_CHECK_HIP(hipMalloc((void**)&ws_base, ws_bytes));
@@ -576,6 +596,22 @@ struct BertStage : ds_stage {
     return DS_OK;
   }
 
+  // Per sample, the mean key of every head (what ds_attention_bwd_centered wants) and the mean input row (for the key
+  // kernel's weight gradient) of every layer, in one launch at the end of the forward pass that wrote them.  (On the
+  // weight-gradient stream it would queue behind a whole group's GEMMs, and the slot's backward pass would wait for it.)
+  int sample_means(int pos) {
+    std::vector<const void*> xs;
+    std::vector<int64_t> lds;
+    std::vector<float> scales;
+    std::vector<float*> outs;
+    for (int l = 0; l < L; ++l) {
+      xs.push_back(at(ls[l].qkv, pos) + (size_t)H * esz); lds.push_back(3 * H); outs.push_back((float*)at(ls[l].kbar, pos));
+      xs.push_back(at(ls[l].x, pos)); lds.push_back(H); outs.push_back((float*)at(ls[l].xbar, pos));
+      scales.push_back(1.0f / S); scales.push_back(1.0f / S);
+    }
+    return ds_sample_colsum_multi((int)xs.size(), B, S, H, xs.data(), lds.data(), scales.data(), outs.data(), stream);
+  }
+
   int forward(int slot, const void* in, const float* key_mask, void* out) override {
     ds_prio_scope prio(1);
     Steps st;
@@ -628,8 +664,10 @@ struct BertStage : ds_stage {
       char* y = (l + 1 < L) ? at(ls[l + 1].x, pos) : (char*)out;
       char* qkv = at(t.qkv, pos);
       // fused Q|K|V projection (modeling_slice.py:464-485)
-      add_gemm(st, desc_fwd(rows, 3 * H, H, x, wqkv[l], qkv, DS_EPI_BIAS, bqkv[l], nullptr, nullptr), prio).before =
-          [this, l]() { return await_cast(l, stream); };
+      {
+        Step& s = add_gemm(st, desc_fwd(rows, 3 * H, H, x, wqkv[l], qkv, DS_EPI_BIAS, bqkv[l], nullptr, nullptr), prio);
+        s.before = [this, l]() { return await_cast(l, stream); };
+      }
       if (fused_attn) {
         // scores, scale, mask adder, softmax and context in one kernel (:499-533)
         char* ctx = at(t.ctx, pos);
@@ -679,6 +717,7 @@ struct BertStage : ds_stage {
         add(st, [=]() { return ds_layernorm_fwd(dtype, rows, H, z2, w[b + LN2_G], w[b + LN2_B], cfg.ln_eps, y, (float*)st2, stream); });
       }
     }
+    if (centred && L > 0) st.back().after = [this, pos]() { return sample_means(pos); };
     return DS_OK;
   }
 
@@ -823,13 +862,15 @@ struct BertStage : ds_stage {
         const float* mask = slot_has_mask[slot] ? (const float*)(sm + mask_off) : nullptr;
         char* ctx = at(t.ctx, pos);
         const float* lse = (const float*)(at(t.lse, pos));
+        const float* kbar = centre_q ? (const float*)at(t.kbar, pos) : nullptr;
         attn_step = &add(st, [=]() {
-          return ds_attention_bwd(dtype, B, NH, S, D, q, 3 * H, mask, scale, -10000.0f, ctx, lse, dctx, dqkv, dp, stream);
+          return ds_attention_bwd_centered(dtype, B, NH, S, D, q, 3 * H, mask, scale, -10000.0f, ctx, lse, dctx, dqkv, dp, kbar, stream);
         });
         if (groupable()) {
           attn_step->nops = 2;
           attn_op(attn_step->ops[0], GOP_ATTN_DKV, prio, q, mask, ctx, (float*)lse, dctx, dqkv, dp);
           attn_op(attn_step->ops[1], GOP_ATTN_DQ, prio, q, mask, ctx, (float*)lse, dctx, dqkv, nullptr);
+          attn_step->ops[1].key_mean = kbar;
         }
       } else {
         char* p = at(t.p, pos);
@@ -848,13 +889,14 @@ struct BertStage : ds_stage {
       // ---- weight gradients of this layer (on the weight-gradient stream when there is one)
       if (G == 1) {
         const char *x = at(t.x, pos), *ctx = at(t.ctx, pos), *a = at(t.a, pos), *h = at(t.h, pos);
+        const float* xbar = centred ? (const float*)at(t.xbar, pos) : nullptr;
         attn_step->after = [=]() {
           hipStream_t chain = stream;
           if (ws) {
             DS_PROPAGATE(lane.begin(chain, ws, par));
             stream = ws;  // the GEMMs and column sums of layer_wgrad launch on `stream`
           }
-          const int rc = layer_wgrad(l, rows, x, ctx, a, h, dz2, du, dz1, dqkv);
+          const int rc = layer_wgrad(l, rows, x, xbar, ctx, a, h, dz2, du, dz1, dqkv);
           stream = chain;
           if (rc != DS_OK) return rc;
           if (ws) DS_PROPAGATE(lane.end(ws, par));
@@ -911,6 +953,7 @@ struct BertStage : ds_stage {
                              (const int32_t*)(sm + emb_ids), tt, (const float*)de, g[E_WORD], g[E_TYPE], g[E_POS]);
         DS_CHECK_LAUNCH();
       }
+      if (G > 1 && centre_k) DS_PROPAGATE(key_gradient_sums(dypos));
       if (G > 1) {
         if (bwd_stream) {
           DS_CHECK_HIP(hipEventRecord(ev_x_bwd[pos], stream));
@@ -918,7 +961,21 @@ struct BertStage : ds_stage {
         } else {
           x_bwd_valid[pos] = 0;
         }
-        if (closing) DS_PROPAGATE(retire_deferred(wgrad_stream ? wgrad_stream : stream, stream));
+        if (closing) {
+          hipStream_t side = wgrad_stream ? wgrad_stream : stream;
+          if (centre_k) {
+            hipStream_t chain = stream;
+            if (side != chain) {  // the key-gradient sums this pass has just queued
+              DS_CHECK_HIP(hipEventRecord(ev_chain, chain));
+              DS_CHECK_HIP(hipStreamWaitEvent(side, ev_chain, 0));
+            }
+            stream = side;
+            const int rc = key_corrections(*runs);
+            stream = chain;
+            if (rc != DS_OK) return rc;
+          }
+          DS_PROPAGATE(retire_deferred(side, stream));
+        }
       }
       return (int)DS_OK;
     });
@@ -937,6 +994,34 @@ struct BertStage : ds_stage {
     }
     return runs;
   }
+  // Deferred weight gradients: per sample, the column sums of the key gradients a backward pass left in the operand ring,
+  // all layers in one launch at the end of the pass; and, when the group's GEMMs have been queued, the centring of the
+  // key projections' parameter gradients (see layer_wgrad) for all layers in one launch per run.
+  int key_gradient_sums(int dypos) {
+    std::vector<const void*> xs;
+    std::vector<int64_t> lds(L, 3 * H);
+    std::vector<float> scales(L, 1.0f);
+    std::vector<float*> outs;
+    for (int l = 0; l < L; ++l) {
+      xs.push_back(dy_base + ld[l].dqkv + (size_t)dypos * 3 * dy_act + (size_t)H * esz);
+      outs.push_back((float*)(dy_base + ld[l].dksum + (size_t)dypos * B * H * 4));
+    }
+    return ds_sample_colsum_multi(L, B, S, H, xs.data(), lds.data(), scales.data(), outs.data(), stream);
+  }
+  int key_corrections(const std::vector<Run>& runs) {
+    for (const Run& r : runs) {
+      std::vector<const float*> as, bs;
+      std::vector<float*> ws, vs;
+      for (int l = 0; l < L; ++l) {
+        as.push_back((const float*)at(ls[l].xbar, r.xpos));
+        bs.push_back((const float*)(dy_base + ld[l].dksum + (size_t)r.dypos * B * H * 4));
+        ws.push_back(g[base(l) + W_K]);
+        vs.push_back(g[base(l) + B_K]);
+      }
+      DS_PROPAGATE(ds_rank_update_multi(L, H, H, r.n * B, as.data(), bs.data(), ws.data(), H, vs.data(), stream));
+    }
+    return DS_OK;
+  }
   int layer_wgrad_runs(int l, const std::vector<Run>& runs) {
     const LayerStash& t = ls[l];
     const int b = base(l);
@@ -944,7 +1029,8 @@ struct BertStage : ds_stage {
       const int m = r.n * rows;
       const char* dz2 = dy_base + ld[l].dz2 + r.dypos * dy_act;
       const char* dz1 = dy_base + ld[l].dz1 + r.dypos * dy_act;
-      DS_PROPAGATE(layer_wgrad(l, m, at(t.x, r.xpos), at(t.ctx, r.xpos), at(t.a, r.xpos), at(t.h, r.xpos), dz2,
+      DS_PROPAGATE(layer_wgrad(l, m, at(t.x, r.xpos), centred ? (const float*)at(t.xbar, r.xpos) : nullptr, at(t.ctx, r.xpos), at(t.a, r.xpos),
+                               at(t.h, r.xpos), dz2,
                                dy_base + ld[l].du + r.dypos * dy_actF, dz1, dy_base + ld[l].dqkv + r.dypos * 3 * dy_act));
       if (rs32) {  // the LayerNorm parameter gradients and the two bias gradients the chain left out
         DS_PROPAGATE(ds_layernorm_param_grads_mixed(m, H, dy_base + ld[l].dyn2 + r.dypos * dy_act, (const float*)at(t.z2, r.xpos),
@@ -973,7 +1059,7 @@ struct BertStage : ds_stage {
   }
 
   // Weight and bias gradients of layer l over m rows (one micro-batch, or several back to back), on `stream`.
-  int layer_wgrad(int l, int m, const char* x, const char* ctx, const char* a, const char* h, const char* dz2,
+  int layer_wgrad(int l, int m, const char* x, const float* xbar, const char* ctx, const char* a, const char* h, const char* dz2,
                   const char* du, const char* dz1, const char* dqkv) {
     const int b = base(l);
     ds_prio_scope prio(0);  // feeds only the master gradients
@@ -1001,6 +1087,17 @@ struct BertStage : ds_stage {
         DS_PROPAGATE(gemm_wgrad(m, H, H, x, H, dqkv + (size_t)j * H * esz, 3 * H, g[b + W_Q + j], H));
       }
     }
+    if (centre_k && G == 1) {
+      // The key gradients of a sample sum to zero per head (every row of dS does, and dK = dS^T Q adds the rows up), so
+      // X^T dK only depends on the inputs' deviation from their per-sample mean and the key bias gets no gradient at all.
+      // The stored dK are rounded to bf16 (from bf16-rounded dS) and sum to a residue instead; against inputs that share a
+      // large common part, mean (x) residue is the bulk of the key kernel's gradient error.  The residue is known: the
+      // parameter gradients are those of dK centred over each sample's keys - the mean's share goes out again.
+      const int ns = m / S;
+      float* dksum = (float*)(ws_base + ws_dksum);
+      DS_PROPAGATE(ds_sample_colsum(ns, S, H, dqkv + (size_t)H * esz, 3 * H, 1.0f, dksum, stream));
+      DS_PROPAGATE(ds_rank_update(H, H, ns, xbar, dksum, g[b + W_K], H, g[b + B_K], stream));
+    }
     return DS_OK;
   }
 
@@ -1018,6 +1115,7 @@ struct BertStage : ds_stage {
       int rc = DS_OK;
       const std::vector<Run> runs = make_runs(deferred);
       for (int l = L - 1; l >= 0 && rc == DS_OK; --l) rc = layer_wgrad_runs(l, runs);
+      if (rc == DS_OK && centre_k) rc = key_corrections(runs);
       stream = keep;
       if (rc != DS_OK) return rc;
       DS_PROPAGATE(retire_deferred(ws, chain));

@@ -319,6 +319,7 @@ def maxpool2x2_bwd(x, dy, relu_mask=False):
 def attention_fwd(qkv, batch, heads, seq, scale, key_mask=None, mask_value=-10000.0):
     """Fused bf16 attention on the fused projection qkv [batch*seq, 3*heads*64] -> (ctx, lse)."""
     _need_cuda(qkv, key_mask)
+    _check_attention(qkv, batch, heads, seq, key_mask=key_mask)
     hidden = qkv.shape[1] // 3
     ctx = torch.empty(batch * seq, hidden, dtype=qkv.dtype, device=qkv.device)
     lse = torch.empty(batch, heads, seq, dtype=torch.float32, device=qkv.device)
@@ -327,14 +328,43 @@ def attention_fwd(qkv, batch, heads, seq, scale, key_mask=None, mask_value=-1000
     return ctx, lse
 
 
-def attention_bwd(qkv, ctx, lse, dctx, batch, heads, seq, scale, key_mask=None, mask_value=-10000.0):
-    _need_cuda(qkv, ctx, lse, dctx, key_mask)
+def _check_attention(qkv, batch, heads, seq, others=(), key_mask=None):
+    """Shapes the fused attention kernels index by: a wrong one reads or writes outside the tensors."""
+    if qkv.dim() != 2 or qkv.shape[0] != batch * seq or qkv.shape[1] % (3 * heads) != 0:
+        raise ValueError("qkv must be [batch * seq, 3 * heads * head_size]")
+    for t in others:
+        if t.dtype != qkv.dtype or tuple(t.shape) != (batch * seq, qkv.shape[1] // 3):
+            raise ValueError("ctx / dctx must be [batch * seq, heads * head_size] of qkv's element type")
+    if key_mask is not None and (key_mask.dtype != torch.float32 or key_mask.numel() != batch * seq):
+        raise ValueError("key_mask must be fp32 [batch, seq]")
+
+
+def attention_key_mean(qkv, batch, heads, seq):
+    """Mean key of every sample and head, fp32 [batch, heads * 64] (ds_attention_key_mean)."""
+    _need_cuda(qkv)
+    _check_attention(qkv, batch, heads, seq)
+    hidden = qkv.shape[1] // 3
+    out = torch.empty(batch, hidden, dtype=torch.float32, device=qkv.device)
+    check(_lib.load().ds_attention_key_mean(dtype_code(qkv), batch, heads, seq, hidden // heads, ptr(qkv), qkv.shape[1], ptr(out), _lib.current_stream()),
+          "ds_attention_key_mean")
+    return out
+
+
+def attention_bwd(qkv, ctx, lse, dctx, batch, heads, seq, scale, key_mask=None, mask_value=-10000.0, key_mean=None):
+    """``key_mean`` (from ``attention_key_mean``): ds_attention_bwd_centered, which keeps the rounding of the score gradients
+    out of dq."""
+    _need_cuda(qkv, ctx, lse, dctx, key_mask, key_mean)
+    _check_attention(qkv, batch, heads, seq, (ctx, dctx), key_mask)
+    if lse.dtype != torch.float32 or lse.numel() != batch * heads * seq:
+        raise ValueError("lse must be fp32 [batch, heads, seq]")
+    if key_mean is not None and (key_mean.dtype != torch.float32 or key_mean.numel() != batch * (qkv.shape[1] // 3)):
+        raise ValueError("key_mean must be fp32 [batch, heads * head_size]")
     hidden = qkv.shape[1] // 3
     dqkv = torch.empty_like(qkv)
     delta = torch.empty_like(lse)
-    check(_lib.load().ds_attention_bwd(dtype_code(qkv), batch, heads, seq, hidden // heads, ptr(qkv), qkv.shape[1], ptr(key_mask),
-                                       scale, mask_value, ptr(ctx), ptr(lse), ptr(dctx), ptr(dqkv), ptr(delta),
-                                       _lib.current_stream()), "ds_attention_bwd")
+    check(_lib.load().ds_attention_bwd_centered(dtype_code(qkv), batch, heads, seq, hidden // heads, ptr(qkv), qkv.shape[1],
+                                                ptr(key_mask), scale, mask_value, ptr(ctx), ptr(lse), ptr(dctx), ptr(dqkv), ptr(delta),
+                                                ptr(key_mean), _lib.current_stream()), "ds_attention_bwd")
     return dqkv
 
 

@@ -180,6 +180,17 @@ int ds_attention_fwd(int dtype, int batch, int heads, int seq, int head_dim, con
 int ds_attention_bwd(int dtype, int batch, int heads, int seq, int head_dim, const void* qkv, int64_t ld,
                      const float* key_mask, float scale, float mask_value, const void* ctx,
                      const float* lse, const void* dctx, void* dqkv, float* delta, void* stream);
+/* The same backward pass with the rounding of the score gradients kept out of dq.  Every row of dS = P (dP - delta) sums to
+ * zero, so dq = dS k only depends on the keys' deviation from their mean; the kernel multiplies bf16-rounded dS, whose rows
+ * no longer sum to zero, and against keys that share a large common part (token vectors that have grown alike over many
+ * layers) that residue times the mean key is the bulk of dq's error.  With key_mean ([batch, heads * 64] fp32, from
+ * ds_attention_key_mean on the same qkv; NULL = ds_attention_bwd) the kernel subtracts it: dq -= rowsum(rounded dS) * mean.
+ * Same arithmetic otherwise (tf.gradients of modeling_slice.py:499-533). */
+int ds_attention_key_mean(int dtype, int batch, int heads, int seq, int head_dim, const void* qkv, int64_t ld, float* key_mean,
+                          void* stream);
+int ds_attention_bwd_centered(int dtype, int batch, int heads, int seq, int head_dim, const void* qkv, int64_t ld,
+                              const float* key_mask, float scale, float mask_value, const void* ctx, const float* lse,
+                              const void* dctx, void* dqkv, float* delta, const float* key_mean, void* stream);
 
 /* Column sums: out[n] (fp32) += sum_m x[m][n]; the bias gradient of tf.layers.dense. */
 int ds_colsum_accum(int dtype, int rows, int cols, const void* x, int64_t ldx, float* out,

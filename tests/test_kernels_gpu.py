@@ -13,7 +13,7 @@ from dapple_amd import ops
 from dapple_amd._lib import (DS_EPI_ACCUM, DS_EPI_BIAS, DS_EPI_DGELU, DS_EPI_GELU, DS_EPI_OUT_F32, DS_EPI_RELU,
                              DS_EPI_RESIDUAL, DS_K_MAJOR, DS_MN_MAJOR)
 from oracle import bert as ob
-from util import assert_close, dev
+from util import assert_close, dev, rel_err
 
 pytestmark = pytest.mark.gpu
 DT = {"fp32": torch.float32, "bf16": torch.bfloat16}
@@ -379,6 +379,37 @@ def test_fused_attention_fwd_bwd(B, N, S, use_mask):
     dqkv = ops.attention_bwd(qkv, ctx, lse, dctx, B, N, S, scale, mask)
     for i, name in enumerate(("dq", "dk", "dv")):
         assert_close(dqkv[:, i * H:(i + 1) * H], dx[:, i * H:(i + 1) * H], 2e-2, "fused attention " + name)
+
+
+def test_fused_attention_backward_with_keys_that_share_a_common_part():
+    """Keys = a large common vector + small differences (what a deep, randomly initialised stack drives its token vectors
+    to): dq = dS k is then a small difference of large terms.  The plain kernel's dq carries the row sums of the
+    bf16-rounded dS times the common part; ds_attention_bwd_centered takes that out: its dq meets the 2e-2 bar of its own
+    scale where the plain kernel misses it by a wide margin.  dk and dv are untouched."""
+    B, N, S, D = 2, 4, 256, 64
+    H = N * D
+    r = rng(91)
+    common = r.standard_normal((1, 3 * H)) * np.concatenate([np.zeros(H), np.full(H, 4.0), np.zeros(H)])
+    qkv = dev(r.standard_normal((B * S, 3 * H)) * 0.5 + common, torch.bfloat16)
+    dctx = dev(r.standard_normal((B * S, H)), torch.bfloat16)
+    scale = 1.0 / math.sqrt(D)
+    ctx, lse = ops.attention_fwd(qkv, B, N, S, scale)
+    x = qkv.cpu().double().requires_grad_(True)
+    q, k, v = (x[:, i * H:(i + 1) * H].reshape(B, S, N, D).permute(0, 2, 1, 3) for i in range(3))
+    ref = (torch.softmax(q @ k.transpose(-1, -2) * scale, -1) @ v).permute(0, 2, 1, 3).reshape(B * S, H)
+    (dx,) = torch.autograd.grad(ref, x, dctx.cpu().double())
+    kmean = ops.attention_key_mean(qkv, B, N, S)
+    want_mean = qkv[:, H:2 * H].float().reshape(B, S, H).mean(1)
+    assert_close(kmean, want_mean, 1e-5, "key mean")
+    plain = ops.attention_bwd(qkv, ctx, lse, dctx, B, N, S, scale)
+    centred = ops.attention_bwd(qkv, ctx, lse, dctx, B, N, S, scale, key_mean=kmean)
+    err_plain = rel_err(plain[:, :H], dx[:, :H])[1]
+    err_centred = rel_err(centred[:, :H], dx[:, :H])[1]
+    print("dq rel l2: plain %.3e, centred %.3e" % (err_plain, err_centred))
+    assert err_centred <= 2e-2 and err_plain > 3 * err_centred
+    assert torch.equal(plain[:, H:], centred[:, H:])
+    for i, name in ((1, "dk"), (2, "dv")):
+        assert_close(centred[:, i * H:(i + 1) * H], dx[:, i * H:(i + 1) * H], 2e-2, "fused attention " + name)
 
 
 def test_fused_attention_rejects_other_shapes():

@@ -139,7 +139,9 @@ def test_backward_waits_for_upstream_gradient_produced_on_the_stage_stream():
             if n.endswith(("kernel",)):
                 assert torch.equal(g[n], ref_g[n]), "%s: %s" % (mode, n)
             else:
-                assert_close(g[n], ref_g[n], 1e-5, "%s: %s" % (mode, n), floor=float(ref_g[n].abs().max()) + 1e-30)
+                # (the key bias gradient is zero up to what two fp32 sums of the same terms differ by: judged on the query bias's scale)
+                scale = float(ref_g[n.replace("/key/bias", "/query/bias")].abs().max()) + 1e-30
+                assert float((g[n] - ref_g[n]).abs().max()) <= 1e-5 * scale, "%s: %s" % (mode, n)
 
 
 def test_pipeline_rejects_mismatched_stages():

@@ -11,7 +11,7 @@ import torch
 from dapple_amd import runtime, synthetic
 from oracle import bert as ob
 from oracle import runtime as ort
-from util import assert_close, dev, rel_err
+from util import assert_close, dev, grad_scale, rel_err
 
 pytestmark = pytest.mark.gpu
 TOL = {"fp32": 1e-4, "bf16": 2e-2}
@@ -193,7 +193,7 @@ def test_forward_backward_overlap_matches_serial():
             assert torch.equal(a, b)
         for k in res[0][2]:
             a, b = res[0][2][k], other[2][k]
-            assert float((a - b).abs().max()) <= 1e-5 * float(a.abs().max()) + 1e-12, k
+            assert float((a - b).abs().max()) <= 1e-5 * grad_scale(res[0][2], k) + 1e-12, k
 
 
 @pytest.mark.gpu
@@ -235,7 +235,7 @@ def test_forward_backward_overlap_vgg_and_gnmt():
             assert torch.equal(a, b), name
         for k in res[0][1]:
             a, b = res[0][1][k], res[1][1][k]
-            assert float((a - b).abs().max()) <= 1e-5 * float(a.abs().max()) + 1e-10, (name, k)
+            assert float((a - b).abs().max()) <= 1e-5 * grad_scale(res[0][1], k) + 1e-10, (name, k)
 
 
 @pytest.mark.gpu
@@ -267,7 +267,7 @@ def test_forward_backward_overlap_unfused_fp32_with_embedding():
         assert torch.equal(a, b)
     for k in res[0][1]:
         a, b = res[0][1][k], res[1][1][k]
-        assert float((a - b).abs().max()) <= 1e-5 * float(a.abs().max()) + 1e-10, k
+        assert float((a - b).abs().max()) <= 1e-5 * grad_scale(res[0][1], k) + 1e-10, k
 
 
 @pytest.mark.gpu
@@ -313,7 +313,7 @@ def test_grouped_weight_gradients_over_steps_and_streams():
             # the one leaving it) beside the chain, where the per-pass form sums the fp32 values: bf16 rounding of the
             # terms, not of the sum.  Everything else only differs in fp32 summation order.
             from_copies = "LayerNorm" in k or k.endswith("output/dense/bias")
-            assert float((a - b).abs().max()) <= (1e-2 if from_copies else 2e-5) * float(a.abs().max()) + 1e-12, k
+            assert float((a - b).abs().max()) <= (1e-2 if from_copies else 2e-5) * grad_scale(res[0][2], k) + 1e-12, k
 
 
 @pytest.mark.gpu
@@ -352,7 +352,7 @@ def test_grouped_weight_gradients_any_call_order(overlap):
     assert torch.equal(res[0][0], res[1][0]) and torch.equal(res[0][1], res[1][1])
     for k in res[0][2]:
         a, b = res[0][2][k], res[1][2][k]
-        assert float((a - b).abs().max()) <= 2e-5 * float(a.abs().max()) + 1e-10, k
+        assert float((a - b).abs().max()) <= 2e-5 * grad_scale(res[0][2], k) + 1e-10, k
 
 
 def _run_config3(dtype, xs_np, dys_np, w, group, overlap, M):
@@ -378,15 +378,16 @@ def _run_config3(dtype, xs_np, dys_np, w, group, overlap, M):
 def test_config3_full_size_in_the_benchmark_mode_against_the_oracle():
     """BASELINE configs[3] exactly as bench.py runs it - 24 layers, 2 x 512 rows, 8 micro-batches, 1F1B K = 2, three streams,
     weight gradients of 4 passes per GEMM, fp32 residual stream - against the fp32 torch-CPU oracle (bf16 within 2e-2 of the
-    fp32 reference is the stated bar).
+    fp32 reference is the stated bar), every tensor on its own scale.
 
-    Measured: outputs 7.5e-3 (L2) / 9e-3 (max), input gradients 1.2e-2 / 1.4e-2, every weight gradient <= 1.3e-2 except
-    the query / key projections of the upper layers.  Those are ill-conditioned for ANY bf16 operand: a random-initialised
+    Measured: outputs 7.5e-3 (L2) / 9e-3 (max), input gradients 1.2e-2 / 1.4e-2, every weight gradient <= 1.5e-2, the
+    query / key projections included (1.2e-2..1.4e-2 L2).  Those two are the ill-conditioned ones: a random-initialised
     stack of this depth drives the token vectors of a sample towards each other, the rows of d scores sum to zero, and
-    d q = d scores . K (and the weight gradient x^T d k, whose d k sums to zero over the keys) is then a small difference of
-    large terms - the gradient itself is 1-2 orders of magnitude below its sibling, the value projection's.  They are held
-    to 2e-2 on the scale of that sibling (max |error| / max |value gradient|) and to 2e-1 on their own scale (measured
-    8e-2 L2); the key bias gradient is identically zero (softmax invariance) and is judged on the query bias's scale."""
+    d q = d scores . K (and the weight gradient x^T d k, whose d k sums to zero over the keys) is a small difference of
+    large terms, 1-2 orders of magnitude below the value projection's gradient.  The stage removes the part of the
+    rounding error that the common component amplifies (ds_attention_bwd_centered for d q, the per-sample rank-one
+    correction of the key kernel's gradient); without it they sit at 8e-2.  The key bias gradient is identically zero
+    (softmax invariance) and is judged on the query bias's scale."""
     c = synthetic.CONFIGS["bert48_half"]
     L, H, N, F, B, S, M = c["num_layers"], c["hidden"], c["heads"], c["ffn"], c["micro_batch"], c["seq"], c["num_micro_batches"]
     w = synthetic.bert_weights(synthetic.SEED_WEIGHT + c["index"], L, H, F)
@@ -403,21 +404,21 @@ def test_config3_full_size_in_the_benchmark_mode_against_the_oracle():
         assert_close(got[1][j], dx, 2e-2, "input grad mb%d" % j)
         for n, g in dw.items():
             acc[n] = g.clone() if n not in acc else acc[n] + g
-    worst_own, worst_sib = 0.0, 0.0
+    worst_qk, worst_rest, worst_kb = 0.0, 0.0, 0.0
     for n in got[2]:
         if n.endswith("/key/bias"):
             floor = acc[n.replace("/key/", "/query/")].abs().max().item()
-            assert got[2][n].abs().max().item() <= 2e-1 * floor, n
+            worst_kb = max(worst_kb, got[2][n].abs().max().item() / floor)
+            assert got[2][n].abs().max().item() <= 2e-2 * floor, n
             continue
         mx, l2 = rel_err(got[2][n], acc[n])
+        assert mx <= 2e-2 and l2 <= 2e-2, "accumulated grad %s: rel max %.3e, l2 %.3e" % (n, mx, l2)
         if "/attention/self/query/" in n or "/attention/self/key/" in n:
-            sibling = acc[n.replace("/query/", "/value/").replace("/key/", "/value/")].abs().max().item()
-            err_sib = (got[2][n].double() - acc[n].double()).abs().max().item() / sibling
-            worst_own, worst_sib = max(worst_own, l2), max(worst_sib, err_sib)
-            assert l2 <= 2e-1 and err_sib <= 2e-2, "%s: rel l2 %.3e (own scale), %.3e of the value gradient's scale" % (n, l2, err_sib)
+            worst_qk = max(worst_qk, mx, l2)
         else:
-            assert mx <= 2e-2 and l2 <= 2e-2, "accumulated grad %s: rel max %.3e, l2 %.3e" % (n, mx, l2)
-    print("query/key gradients: worst rel l2 %.3e on their own scale, %.3e of the value gradient's scale" % (worst_own, worst_sib))
+            worst_rest = max(worst_rest, mx, l2)
+    print("weight gradients, worst of rel max / rel l2 on their own scale: query and key projections %.3e, all others %.3e; "
+          "key bias %.3e of the query bias's scale" % (worst_qk, worst_rest, worst_kb))
 
 
 def test_config3_full_size_exact_properties():

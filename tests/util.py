@@ -32,3 +32,10 @@ def dev(a, dtype=None):
     if dtype is not None:
         t = t.to(dtype)
     return t.cuda().contiguous()
+
+
+def grad_scale(grads, name):
+    """Magnitude a weight gradient is judged on: its own largest entry, except for the key bias of an attention layer, whose
+    gradient vanishes identically (a key bias shifts every score of a row equally) - that one is judged on the query bias's."""
+    ref = name.replace("/key/bias", "/query/bias") if name.endswith("/key/bias") else name
+    return float(grads[ref].abs().max())
