@@ -413,6 +413,9 @@ def main():
                          "per level (ds_stage_forward_backward), instead of two calls on two streams (measured slower: a what-if)")
     ap.add_argument("--xlnet-attention", choices=["auto", "separate"], default="auto",
                     help="XLNet stages: how the attention scores run (ds_xlnet_cfg.fused_attention)")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="default workload only: skip the three-step runs of the other BASELINE configurations that are attached "
+                         "to the line as `workloads`")
     ap.add_argument("--micro-batch", type=int, default=None,
                     help="samples per micro-batch instead of the configuration's (a what-if: the headline is the default)")
     ap.add_argument("--micro-batches", type=int, default=None, help="micro-batches per step instead of the configuration's")
@@ -499,6 +502,29 @@ def main():
     wl.stage.close()
     del wl
     torch.cuda.empty_cache()
+    if args.workload == "bert48_half" and not reshaped and not args.no_other_workloads:
+        # the other BASELINE configurations, a few steps each, in the same process: throughput and whole-stage fraction of
+        # the matrix peak of their arithmetic (no CPU legs, no per-kernel timing)
+        others = {}
+        for name in ("bert_large_2l", "vgg19_stage0", "gnmt16_encoder", "xlnet36_half"):
+            oc = dict(synthetic.CONFIGS[name])
+            ow = MAKERS[oc["kind"]](oc, args)
+            o_overlap = not args.no_overlap and ow.stage.overlap_supported()
+            if o_overlap:
+                ow.stage.enable_overlap()
+            ow.step()
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            for _ in range(3):
+                ow.step()
+            torch.cuda.synchronize()
+            odt = (time.perf_counter() - t1) / 3
+            others[name] = {"value": ow.samples / odt, "unit": "samples/s", "ms_per_step": odt * 1e3, "steps": 3, "dtype": oc["dtype"],
+                            "stage_frac_of_peak": ow.flops_per_sample * ow.samples / odt / PEAK[oc["dtype"]]}
+            ow.stage.close()
+            del ow
+            torch.cuda.empty_cache()
+        line["workloads"] = others
     if not args.no_cpu_baseline:
         cores = host_cores()
         torch.set_num_threads(cores)

@@ -99,7 +99,10 @@ PROTOTYPES = {
                                           C.c_void_p, C.c_void_p]),
     "ds_layernorm_bwd_mixed": (C.c_int, [C.c_int, C.c_int] + [C.c_void_p] * 11),
     "ds_layernorm_param_grads_mixed": (C.c_int, [C.c_int, C.c_int] + [C.c_void_p] * 8),
+    "ds_layernorm_bwd_mixed_rows": (C.c_int, [C.c_int, C.c_int] + [C.c_void_p] * 9),
+    "ds_layernorm_param_grads_exact": (C.c_int, [C.c_int, C.c_int] + [C.c_void_p] * 9),
     "ds_gemm_static_scratch": (C.c_int, [C.POINTER(GemmDesc), C.c_void_p]),
+    "ds_gemm_static_scratch_init": (C.c_int, []),
     "ds_vgg_head_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int]),
     "ds_vgg_head": (C.c_int, [C.c_int] * 4 + [C.c_void_p] * 8 + [C.c_int, C.c_float] + [C.c_void_p] * 10 + [C.c_size_t, C.c_void_p]),
     "ds_pooler": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),

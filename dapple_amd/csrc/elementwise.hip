@@ -370,9 +370,11 @@ template <int NG>
 __global__ __launch_bounds__(256) void layernorm_bwd_mixed_rows_kernel(int rows, int cols, const float* __restrict__ dy,
                                                                       const float* __restrict__ x, const float* __restrict__ gamma,
                                                                       const float* __restrict__ stats, bf16* __restrict__ dx16,
-                                                                      float* __restrict__ dx32, bf16* __restrict__ dy16, int prio) {
+                                                                      float* __restrict__ dx32, bf16* __restrict__ dy16, float* __restrict__ dy32,
+                                                                      float* __restrict__ rowsums, int prio) {
   ds_wave_prio(prio);
-  dsrows::layernorm_bwd_mixed_rows_row<NG>(blockIdx.x * 4 + (threadIdx.x >> 6), threadIdx.x & 63, rows, cols, dy, x, gamma, stats, dx16, dx32, dy16);
+  dsrows::layernorm_bwd_mixed_rows_row<NG>(blockIdx.x * 4 + (threadIdx.x >> 6), threadIdx.x & 63, rows, cols, dy, x, gamma, stats, dx16, dx32, dy16,
+                                           dy32, rowsums);
 }
 
 // d_gamma[c] += sum_rows dy x_hat, d_beta[c] += sum_rows dy, d_colsum[c] += sum_rows dx (dx, d_colsum nullable) from the
@@ -424,6 +426,74 @@ __global__ __launch_bounds__(256) void layernorm_param_grad_mixed_kernel(int row
           pg[e] += d * (b1[e] - mean1) * rstd1;
           pb[e] += d;
           ps[e] += to_f32(v1[e]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    red[0][g][lane * 8 + e] = pg[e];
+    red[1][g][lane * 8 + e] = pb[e];
+    red[2][g][lane * 8 + e] = ps[e];
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < 64 * 8; i += 256) {
+    const int p = blockIdx.x * 64 * 8 + i;
+    if (p < cols) {
+      atomicAdd(d_gamma + p, red[0][0][i] + red[0][1][i] + red[0][2][i] + red[0][3][i]);
+      atomicAdd(d_beta + p, red[1][0][i] + red[1][1][i] + red[1][2][i] + red[1][3][i]);
+      if (d_colsum) atomicAdd(d_colsum + p, red[2][0][i] + red[2][1][i] + red[2][2][i] + red[2][3][i]);
+    }
+  }
+}
+
+// The same sums without rounding: dy comes as the fp32 copy, and dx is rebuilt in fp32 from the two per-row means the
+// row kernel left (dx = rstd (dy gamma - s1 - x_hat s2)), so the results equal those of layernorm_bwd_mixed_kernel up
+// to the order of the fp32 additions.  Same block shape as layernorm_param_grad_mixed_kernel.
+__global__ __launch_bounds__(256) void layernorm_param_grad_exact_kernel(int rows, int cols, int rows_per_block, const float* __restrict__ dy,
+                                                                        const float* __restrict__ x, const float* __restrict__ gamma,
+                                                                        const float* __restrict__ stats, const float* __restrict__ rowsums,
+                                                                        float* __restrict__ d_gamma, float* __restrict__ d_beta,
+                                                                        float* __restrict__ d_colsum) {
+  __shared__ float red[3][4][64 * 8];
+  const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
+  const int c = (blockIdx.x * 64 + lane) * 8;
+  const int r0 = blockIdx.y * rows_per_block;
+  int r1 = r0 + rows_per_block;
+  if (r1 > rows) r1 = rows;
+  float pg[8], pb[8], ps[8], gm[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) pg[e] = pb[e] = ps[e] = gm[e] = 0.f;
+  if (c < cols) {
+    ln_load8(gamma + c, gm);
+    // two rows in flight per wave
+    for (int r = r0 + g; r < r1; r += 8) {
+      const int rb = r + 4;
+      const bool two = rb < r1;
+      float a0[8], b0[8], a1[8], b1[8];
+      ln_load8(dy + (int64_t)r * cols + c, a0);
+      ln_load8(x + (int64_t)r * cols + c, b0);
+      const float mean0 = stats[2 * r], rstd0 = stats[2 * r + 1], s10 = rowsums[2 * r], s20 = rowsums[2 * r + 1];
+      float mean1 = 0.f, rstd1 = 0.f, s11 = 0.f, s21 = 0.f;
+      if (two) {
+        ln_load8(dy + (int64_t)rb * cols + c, a1);
+        ln_load8(x + (int64_t)rb * cols + c, b1);
+        mean1 = stats[2 * rb]; rstd1 = stats[2 * rb + 1]; s11 = rowsums[2 * rb]; s21 = rowsums[2 * rb + 1];
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float xh = (b0[e] - mean0) * rstd0;
+        pg[e] += a0[e] * xh;
+        pb[e] += a0[e];
+        ps[e] += rstd0 * (a0[e] * gm[e] - s10 - xh * s20);
+      }
+      if (two) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float xh = (b1[e] - mean1) * rstd1;
+          pg[e] += a1[e] * xh;
+          pb[e] += a1[e];
+          ps[e] += rstd1 * (a1[e] * gm[e] - s11 - xh * s21);
         }
       }
     }
@@ -873,7 +943,7 @@ extern "C" int ds_layernorm_bwd_mixed(int rows, int cols, const float* dy, const
     ds_prof_scope prof(s, "layernorm_bwd_mixed_rows_kernel",
                        (double)rows * cols * (4 + 4 + 2 + (dx_f32 ? 4 : 0) + (dy_bf16 ? 2 : 0)), "B");
     DISPATCH_NG(need, hipLaunchKernelGGL((layernorm_bwd_mixed_rows_kernel<NG>), dim3((rows + 3) / 4), dim3(256), 0, s, rows, cols, dy, x,
-                                         gamma, stats, (bf16*)dx_bf16, dx_f32, (bf16*)dy_bf16, ds_launch_prio));
+                                         gamma, stats, (bf16*)dx_bf16, dx_f32, (bf16*)dy_bf16, nullptr, nullptr, ds_launch_prio));
     DS_CHECK_LAUNCH();
     return DS_OK;
   }
@@ -907,6 +977,41 @@ extern "C" int ds_layernorm_param_grads_mixed(int rows, int cols, const void* dy
   ds_prof_scope prof(s, "layernorm_param_grad_mixed_kernel", (double)rows * cols * (2 + 4 + (d_colsum ? 2 : 0)), "B");
   hipLaunchKernelGGL(layernorm_param_grad_mixed_kernel, grid, dim3(256), 0, s, rows, cols, rpb, (const bf16*)dy_bf16, x, stats,
                      d_colsum ? (const bf16*)dx_bf16 : nullptr, d_gamma, d_beta, d_colsum);
+  DS_CHECK_LAUNCH();
+  return DS_OK;
+}
+
+// The row kernel with the hand-over that loses nothing: an fp32 copy of dy and the two per-row means (see rows_core.h).
+extern "C" int ds_layernorm_bwd_mixed_rows(int rows, int cols, const float* dy, const float* x, const float* gamma, const float* stats,
+                                           void* dx_bf16, float* dx_f32, float* dy_copy, float* row_sums, void* stream) {
+  DS_PROPAGATE(check_mixed("ds_layernorm_bwd_mixed_rows", rows, cols));
+  DS_CHECK_ARG(dy && x && gamma && stats && dx_bf16 && dy_copy && row_sums, "ds_layernorm_bwd_mixed_rows: null pointer");
+  DS_CHECK_ARG(ds_aligned16(dy) && ds_aligned16(x) && ds_aligned16(dx_bf16) && ds_aligned16(dx_f32) && ds_aligned16(gamma) && ds_aligned16(dy_copy),
+               "ds_layernorm_bwd_mixed_rows: tensors must be 16-byte aligned");
+  hipStream_t s = (hipStream_t)stream;
+  const int need = (cols / 8 + 63) / 64;
+  ds_prof_scope prof(s, "layernorm_bwd_mixed_rows_kernel", (double)rows * cols * (4 + 4 + 2 + (dx_f32 ? 4 : 0) + 4), "B");
+  DISPATCH_NG(need, hipLaunchKernelGGL((layernorm_bwd_mixed_rows_kernel<NG>), dim3((rows + 3) / 4), dim3(256), 0, s, rows, cols, dy, x, gamma,
+                                       stats, (bf16*)dx_bf16, dx_f32, (bf16*)nullptr, dy_copy, row_sums, ds_launch_prio));
+  DS_CHECK_LAUNCH();
+  return DS_OK;
+}
+
+extern "C" int ds_layernorm_param_grads_exact(int rows, int cols, const float* dy_copy, const float* x, const float* gamma, const float* stats,
+                                              const float* row_sums, float* d_gamma, float* d_beta, float* d_colsum, void* stream) {
+  DS_CHECK_ARG(rows > 0 && cols > 0 && cols % 8 == 0, "ds_layernorm_param_grads_exact: rows %d, cols %d (a multiple of 8)", rows, cols);
+  DS_CHECK_ARG(dy_copy && x && gamma && stats && row_sums && d_gamma && d_beta, "ds_layernorm_param_grads_exact: null pointer");
+  DS_CHECK_ARG(ds_aligned16(dy_copy) && ds_aligned16(x) && ds_aligned16(gamma), "ds_layernorm_param_grads_exact: tensors must be 16-byte aligned");
+  hipStream_t s = (hipStream_t)stream;
+  const int strips = (cols + 64 * 8 - 1) / (64 * 8);
+  int chunks = 256 / strips;  // about one block per CU
+  if (chunks > (rows + 31) / 32) chunks = (rows + 31) / 32;
+  if (chunks < 1) chunks = 1;
+  const int rpb = (rows + chunks - 1) / chunks;
+  dim3 grid(strips, (rows + rpb - 1) / rpb);
+  ds_prof_scope prof(s, "layernorm_param_grad_exact_kernel", (double)rows * cols * 8, "B");
+  hipLaunchKernelGGL(layernorm_param_grad_exact_kernel, grid, dim3(256), 0, s, rows, cols, rpb, dy_copy, x, gamma, stats, row_sums, d_gamma,
+                     d_beta, d_colsum);
   DS_CHECK_LAUNCH();
   return DS_OK;
 }

@@ -900,6 +900,7 @@ static int gemm_run(const ds_gemm_desc* d, int splitk_req, void* stream, bool mu
         a.ktiles_per_split = ktiles / slices;
         a.ws_count = (unsigned*)d->workspace;
         a.ws_part = (float*)((char*)d->workspace + 4096);
+        a.ws_bytes = d->workspace_bytes - 4096;
         char tagk[96];
         snprintf(tagk, sizeof(tagk), "gemm8_kernel<bf16,128,128,%s,%s>/k%d", d->a_major == DS_K_MAJOR ? "K" : "MN",
                  d->b_major == DS_K_MAJOR ? "K" : "MN", slices);
@@ -944,9 +945,24 @@ constexpr int SCRATCH_MAX_TILES = 16;  // 128x128 output tiles, e.g. 512 x 512 o
 constexpr size_t SCRATCH_BYTES = 4096 + (size_t)SCRATCH_MAX_TILES * 4 * 128 * 128 * sizeof(float);  // 4 MiB + 4 KiB
 constexpr int SCRATCH_MAX_DEVICES = 64;
 void* g_scratch_ptr[SCRATCH_MAX_DEVICES] = {};
-__global__ void scratch_clear_counters_kernel(unsigned* p) { p[threadIdx.x] = 0u; }
 }  // namespace
 static __device__ __align__(256) unsigned char scratch[SCRATCH_BYTES];
+
+// Resolves the device address of the library's scratch on the current device (once per device; the array's name is only
+// a host-side handle).  Launches nothing and allocates nothing: a file-scope device array is zero when its code object
+// is loaded, and every split-K launch leaves the arrival counters at zero again.  A caller that is going to capture
+// ds_gemm_static_scratch into a graph calls this first, outside the capture; otherwise the first call does it.
+extern "C" int ds_gemm_static_scratch_init(void) {
+  int dev = -1;
+  DS_CHECK_HIP(hipGetDevice(&dev));
+  DS_CHECK_ARG(dev >= 0 && dev < SCRATCH_MAX_DEVICES, "ds_gemm_static_scratch: device %d", dev);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    DS_CHECK_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    g_scratch_ptr[dev] = ptr;
+  }
+  return DS_OK;
+}
 
 extern "C" int ds_gemm_static_scratch(const ds_gemm_desc* d, void* stream) {
   DS_CHECK_ARG(d != nullptr, "ds_gemm_static_scratch: null descriptor");
@@ -955,19 +971,9 @@ extern "C" int ds_gemm_static_scratch(const ds_gemm_desc* d, void* stream) {
   DS_CHECK_ARG(tiles <= SCRATCH_MAX_TILES,
                "ds_gemm_static_scratch: a %d x %d output has %lld tiles of 128 x 128, the library's scratch holds %d (%zu bytes)",
                d->m, d->n, (long long)tiles, SCRATCH_MAX_TILES, SCRATCH_BYTES);
+  DS_PROPAGATE(ds_gemm_static_scratch_init());
   int dev = -1;
   DS_CHECK_HIP(hipGetDevice(&dev));
-  DS_CHECK_ARG(dev >= 0 && dev < SCRATCH_MAX_DEVICES, "ds_gemm_static_scratch: device %d", dev);
-  if (g_scratch_ptr[dev] == nullptr) {
-    // once per device, with that device current: the array's name is only a host-side handle, its device address
-    // comes from the runtime.  The arrival counters start at zero (a kernel, not a memset: callers may capture later
-    // calls into a graph, and every launch leaves the counters at zero again).
-    void* ptr = nullptr;
-    DS_CHECK_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
-    hipLaunchKernelGGL(scratch_clear_counters_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, (unsigned*)ptr);
-    DS_CHECK_LAUNCH();
-    g_scratch_ptr[dev] = ptr;
-  }
   ds_gemm_desc c = *d;
   c.workspace = g_scratch_ptr[dev];
   c.workspace_bytes = SCRATCH_BYTES;

@@ -31,6 +31,14 @@ int launch8(GemmArgs a, int batch, hipStream_t stream) {
   a.grid_n = (a.n + BN - 1) / BN;
   choose_xcd_block(a);
   dim3 grid(a.grid_m * a.grid_n, 1, batch * a.splitk);
+  if (a.ws_part != nullptr) {
+    // every k-slice of every tile parks BM x BN floats at ws_part[(tile * splitk + slice) * BM * BN]; the counters (one
+    // unsigned per tile) sit in the 4096 bytes in front of ws_part
+    const size_t need = (size_t)a.grid_m * a.grid_n * a.splitk * BM * BN * sizeof(float);
+    DS_CHECK_ARG((size_t)a.grid_m * a.grid_n * sizeof(unsigned) <= 4096 && need <= a.ws_bytes,
+                 "ds_gemm8_launch: %d x %d tiles in %d slices need %zu bytes of workspace behind the counters, the caller's holds %zu",
+                 a.grid_m, a.grid_n, a.splitk, need, a.ws_bytes);
+  }
   constexpr size_t lds = (size_t)STAGES * (BM + BN) * 128;
   static bool attr_set = false;
   if (!attr_set) {

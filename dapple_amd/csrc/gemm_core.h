@@ -46,6 +46,7 @@ struct GemmArgs {
   int prio;                    // wave priority (0..3)
   float* ws_part;              // split-K by workspace (8-wave kernels): fp32 partial tiles [tile][slice][BM * BN]
   unsigned* ws_count;          // and one arrival counter per tile (zero between launches)
+  size_t ws_bytes;             // bytes behind ws_part (host side: the launcher checks them against the grid it is about to start)
   float* rowdot;               // DS_EPI_ROWDOT (grouped launches only): see gemm_epilogue_vec8
   int rowdot_seq;
 };

@@ -48,6 +48,8 @@ struct GroupOp {
   float* stats = nullptr;
   const float* dy = nullptr;
   void* dy16 = nullptr;  // nullable: bf16 copy of dy
+  float* dy32 = nullptr;      // nullable: fp32 copy of dy and
+  float* row_sums = nullptr;  // the two per-row means (ds_layernorm_bwd_mixed_rows)
   GroupOp() { memset(&gemm, 0, sizeof(gemm)); }
 };
 

@@ -32,6 +32,8 @@ struct RowArgs {
   float* stats;
   const float* dy;
   bf16* dy16;
+  float* dy32;
+  float* rowsums;
 };
 
 enum { ROLE_ATTN_FWD = 64, ROLE_ATTN_DQ, ROLE_ATTN_DKV, ROLE_LN_FWD, ROLE_LN_BWD };
@@ -78,7 +80,7 @@ __device__ __forceinline__ void run_tile(const GemmArgs& g, char* lds, int bx, i
 
 template <int NG>
 __device__ __forceinline__ void run_rows(const RowArgs& r, bool backward, int row, int lane) {
-  if (backward) dsrows::layernorm_bwd_mixed_rows_row<NG>(row, lane, r.rows, r.cols, r.dy, r.x, r.gamma, r.stats, r.y16, r.y32, r.dy16);
+  if (backward) dsrows::layernorm_bwd_mixed_rows_row<NG>(row, lane, r.rows, r.cols, r.dy, r.x, r.gamma, r.stats, r.y16, r.y32, r.dy16, r.dy32, r.rowsums);
   else dsrows::layernorm_fwd_mixed_row<NG>(row, lane, r.rows, r.cols, r.x, r.gamma, r.beta, r.eps, r.y16, r.y32, r.stats);
 }
 
@@ -173,10 +175,10 @@ int fill_rows(const GroupOp& op, GroupTask& t) {
                op.cols);
   DS_CHECK_ARG(op.x && op.gamma && op.y16 && op.stats, "ds_group_launch: LayerNorm: null argument");
   DS_CHECK_ARG(ds_aligned16(op.x) && ds_aligned16(op.gamma) && ds_aligned16(op.y16) && ds_aligned16(op.y32) && ds_aligned16(op.dy) &&
-               ds_aligned16(op.dy16) && ds_aligned16(op.beta), "ds_group_launch: LayerNorm: operands must be 16-byte aligned");
+               ds_aligned16(op.dy16) && ds_aligned16(op.beta) && ds_aligned16(op.dy32), "ds_group_launch: LayerNorm: operands must be 16-byte aligned");
   RowArgs& r = t.r;
   r.rows = op.rows; r.cols = op.cols; r.x = op.x; r.gamma = op.gamma; r.beta = op.beta; r.eps = op.eps; r.y16 = (bf16*)op.y16;
-  r.y32 = op.y32; r.stats = op.stats; r.dy = op.dy; r.dy16 = (bf16*)op.dy16;
+  r.y32 = op.y32; r.stats = op.stats; r.dy = op.dy; r.dy16 = (bf16*)op.dy16; r.dy32 = op.dy32; r.rowsums = op.row_sums;
   if (op.kind == GOP_LN_FWD) {
     DS_CHECK_ARG(op.beta != nullptr, "ds_group_launch: LayerNorm forward: beta is needed");
     t.role = ROLE_LN_FWD;

@@ -72,11 +72,14 @@ __device__ __forceinline__ void layernorm_fwd_mixed_row(int row, int lane, int r
 // The same backward pass without the parameter gradients: one wave per row, no LDS, no atomics - the form for a chain
 // of dependent kernels.  dy16 (nullable) receives a bf16 copy of dy: with x and stats (kept by the caller) and dx16 it is
 // all layernorm_param_grad_mixed_kernel needs to produce d_gamma, d_beta and the column sums of dx later, elsewhere.
+// dy32 / rowsums (nullable) are the same hand-over without rounding: an fp32 copy of dy and, per row, the two means
+// (of dy gamma and of dy gamma x_hat) from which layernorm_param_grad_exact_kernel rebuilds the fp32 dx.
 template <int NG>
 __device__ __forceinline__ void layernorm_bwd_mixed_rows_row(int row, int lane, int rows, int cols, const float* __restrict__ dy,
                                                                       const float* __restrict__ x, const float* __restrict__ gamma,
                                                                       const float* __restrict__ stats, bf16* __restrict__ dx16,
-                                                                      float* __restrict__ dx32, bf16* __restrict__ dy16) {
+                                                                      float* __restrict__ dx32, bf16* __restrict__ dy16,
+                                                                      float* __restrict__ dy32 = nullptr, float* __restrict__ rowsums = nullptr) {
   if (row >= rows) return;
   const int64_t ro = (int64_t)row * cols;
   float a[NG][8], b[NG][8], g[NG][8];
@@ -96,6 +99,7 @@ __device__ __forceinline__ void layernorm_bwd_mixed_rows_row(int row, int lane, 
     const int c = (lane + i * 64) * 8;
     if (c < cols) {
       if (dy16) ln_store8(dy16 + ro + c, a[i]);
+      if (dy32) ln_store8(dy32 + ro + c, a[i]);
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         b[i][e] = (b[i][e] - mean) * rstd;
@@ -107,6 +111,7 @@ __device__ __forceinline__ void layernorm_bwd_mixed_rows_row(int row, int lane, 
   }
   s1 = wave_sum(s1) / cols;
   s2 = wave_sum(s2) / cols;
+  if (rowsums && lane == 0) { rowsums[2 * row] = s1; rowsums[2 * row + 1] = s2; }
 #pragma unroll
   for (int i = 0; i < NG; ++i) {
     const int c = (lane + i * 64) * 8;

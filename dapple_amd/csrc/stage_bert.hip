@@ -84,7 +84,8 @@ struct LayerStash {
 // of positions back to back, byte offsets into dy_base.
 struct LayerDy {
   size_t dz2, du, dz1, dqkv;
-  size_t dyn2, dyn1;  // fp32 residual stream: bf16 copies of the gradients that entered the two LayerNorms
+  size_t dyn2, dyn1;  // fp32 residual stream: fp32 copies of the gradients that entered the two LayerNorms
+  size_t rs2, rs1;    // and the two per-row means of each LayerNorm's backward pass
   size_t dksum;       // fused attention: per sample, the column sums of the pass's key gradients (fp32 [B][H])
 };
 struct Deferred {
@@ -131,7 +132,7 @@ struct BertStage : ds_stage {
   int G = 1, KP = 0, NDY = 0;
   char* dy_base = nullptr;
   std::vector<LayerDy> ld;
-  size_t dy_act = 0, dy_actF = 0;
+  size_t dy_act = 0, dy_actF = 0, dy_act32 = 0;
   std::vector<int> slot_pos, pos_owner;
   std::vector<char> pos_deferred;
   int next_pos = 0;
@@ -292,15 +293,17 @@ struct BertStage : ds_stage {
       pos_deferred.assign(KP, 0);
       Arena da;
       ld.resize(L);
-      dy_act = act; dy_actF = actF;
+      dy_act = act; dy_actF = actF; dy_act32 = (size_t)rows * H * 4;
       for (int l = 0; l < L; ++l) {
         ld[l].dz2 = da.reserve(act * NDY);
         ld[l].du = da.reserve(actF * NDY);
         ld[l].dz1 = da.reserve(act * NDY);
         ld[l].dqkv = da.reserve(3 * act * NDY);
         if (rs32) {
-          ld[l].dyn2 = da.reserve(act * NDY);
-          ld[l].dyn1 = da.reserve(act * NDY);
+          ld[l].dyn2 = da.reserve(dy_act32 * NDY);
+          ld[l].dyn1 = da.reserve(dy_act32 * NDY);
+          ld[l].rs2 = da.reserve((size_t)rows * 8 * NDY);
+          ld[l].rs1 = da.reserve((size_t)rows * 8 * NDY);
         }
         ld[l].dksum = da.reserve((size_t)B * H * 4 * NDY);
       }
@@ -505,13 +508,13 @@ struct BertStage : ds_stage {
     return s;
   }
   Step& add_ln_bwd_rows(Steps& st, int prio, const float* dy, const float* x, const float* gamma, const float* stats, void* dx16, float* dx32,
-                        void* dy16) {
-    Step& s = add(st, [=]() { return ds_layernorm_bwd_mixed(rows, H, dy, x, gamma, stats, dx16, dx32, dy16, nullptr, nullptr, nullptr, stream); });
+                        float* dy32, float* row_sums) {
+    Step& s = add(st, [=]() { return ds_layernorm_bwd_mixed_rows(rows, H, dy, x, gamma, stats, dx16, dx32, dy32, row_sums, stream); });
     if (groupable()) {
       GroupOp& o = s.ops[0];
       s.nops = 1;
       o.kind = GOP_LN_BWD; o.prio = prio; o.rows = rows; o.cols = H; o.x = x; o.gamma = gamma; o.stats = (float*)stats; o.dy = dy;
-      o.y16 = dx16; o.y32 = dx32; o.dy16 = dy16;
+      o.y16 = dx16; o.y32 = dx32; o.dy32 = dy32; o.row_sums = row_sums;
     }
     return s;
   }
@@ -811,7 +814,8 @@ struct BertStage : ds_stage {
       const bool ln_deferred = rs32 && G > 1;
       Step* first_step;
       if (ln_deferred) {
-        first_step = &add_ln_bwd_rows(st, prio, dyf, z2, w[b + LN2_G], st2, dz2, dz2f, dy_base + ld[l].dyn2 + dypos * dy_act);
+        first_step = &add_ln_bwd_rows(st, prio, dyf, z2, w[b + LN2_G], st2, dz2, dz2f, (float*)(dy_base + ld[l].dyn2 + dypos * dy_act32),
+                                      (float*)(dy_base + ld[l].rs2 + (size_t)dypos * rows * 8));
       } else if (rs32) {
         const float* dyin = dyf;
         first_step = &add(st, [=]() {
@@ -832,7 +836,8 @@ struct BertStage : ds_stage {
       else add_gemm(st, desc_dgrad(rows, F, H, du, weight_T(l, W_FF1), da, DS_EPI_RESIDUAL, dz2, nullptr), prio);
       // attention-output LayerNorm; column sums of dz1 = gradient of attention/output/dense/bias
       if (ln_deferred) {
-        add_ln_bwd_rows(st, prio, daf, z1, w[b + LN1_G], st1, dz1, dz1f, dy_base + ld[l].dyn1 + dypos * dy_act);
+        add_ln_bwd_rows(st, prio, daf, z1, w[b + LN1_G], st1, dz1, dz1f, (float*)(dy_base + ld[l].dyn1 + dypos * dy_act32),
+                        (float*)(dy_base + ld[l].rs1 + (size_t)dypos * rows * 8));
       } else if (rs32) {
         add(st, [=]() {
           return ds_layernorm_bwd_mixed(rows, H, daf, z1, w[b + LN1_G], st1, dz1, dz1f, nullptr, g[b + LN1_G], g[b + LN1_B], g[b + B_AO], stream);
@@ -1032,13 +1037,15 @@ struct BertStage : ds_stage {
       DS_PROPAGATE(layer_wgrad(l, m, at(t.x, r.xpos), centred ? (const float*)at(t.xbar, r.xpos) : nullptr, at(t.ctx, r.xpos), at(t.a, r.xpos),
                                at(t.h, r.xpos), dz2,
                                dy_base + ld[l].du + r.dypos * dy_actF, dz1, dy_base + ld[l].dqkv + r.dypos * 3 * dy_act));
-      if (rs32) {  // the LayerNorm parameter gradients and the two bias gradients the chain left out
-        DS_PROPAGATE(ds_layernorm_param_grads_mixed(m, H, dy_base + ld[l].dyn2 + r.dypos * dy_act, (const float*)at(t.z2, r.xpos),
-                                                    (const float*)at(t.st2, r.xpos), dz2, g[b + LN2_G], g[b + LN2_B], g[b + B_FF2],
-                                                    stream));
-        DS_PROPAGATE(ds_layernorm_param_grads_mixed(m, H, dy_base + ld[l].dyn1 + r.dypos * dy_act, (const float*)at(t.z1, r.xpos),
-                                                    (const float*)at(t.st1, r.xpos), dz1, g[b + LN1_G], g[b + LN1_B], g[b + B_AO],
-                                                    stream));
+      if (rs32) {  // the LayerNorm parameter gradients and the two bias gradients the chain left out, from its fp32 hand-over
+        DS_PROPAGATE(ds_layernorm_param_grads_exact(m, H, (const float*)(dy_base + ld[l].dyn2 + r.dypos * dy_act32), (const float*)at(t.z2, r.xpos),
+                                                    w[b + LN2_G], (const float*)at(t.st2, r.xpos),
+                                                    (const float*)(dy_base + ld[l].rs2 + (size_t)r.dypos * rows * 8), g[b + LN2_G], g[b + LN2_B],
+                                                    g[b + B_FF2], stream));
+        DS_PROPAGATE(ds_layernorm_param_grads_exact(m, H, (const float*)(dy_base + ld[l].dyn1 + r.dypos * dy_act32), (const float*)at(t.z1, r.xpos),
+                                                    w[b + LN1_G], (const float*)at(t.st1, r.xpos),
+                                                    (const float*)(dy_base + ld[l].rs1 + (size_t)r.dypos * rows * 8), g[b + LN1_G], g[b + LN1_B],
+                                                    g[b + B_AO], stream));
       }
     }
     return DS_OK;

@@ -211,9 +211,10 @@ def layernorm_bwd_mixed(dy, x, gamma, stats, d_gamma=None, d_beta=None, d_colsum
     Without ``d_gamma`` / ``d_beta`` only dx is computed (no atomics); ``want_dy_bf16`` then also returns the bf16 copy of
     dy that ``layernorm_param_grads_mixed`` takes: (dx bf16, dx fp32 or None, dy bf16)."""
     _need_cuda(dy, x, gamma, stats, d_gamma, d_beta, d_colsum)
-    if x.dtype != torch.float32 or dy.dtype != torch.float32:
-        raise ValueError("layernorm_bwd_mixed: dy and x must be fp32")
-    rows, cols = x.shape
+    rows, cols = _check_ln_mixed(x, gamma, stats, [(dy, torch.float32)])
+    for t in (d_gamma, d_beta, d_colsum):
+        if t is not None and (t.dtype != torch.float32 or t.numel() != cols):
+            raise ValueError("parameter gradients must be fp32 [cols]")
     dx16 = torch.empty(rows, cols, dtype=torch.bfloat16, device=x.device)
     dx32 = torch.empty_like(x) if want_f32 else None
     dy16 = torch.empty_like(dx16) if want_dy_bf16 else None
@@ -222,11 +223,58 @@ def layernorm_bwd_mixed(dy, x, gamma, stats, d_gamma=None, d_beta=None, d_colsum
     return (dx16, dx32, dy16) if want_dy_bf16 else (dx16, dx32)
 
 
+def _check_ln_mixed(x, gamma, stats, others=()):
+    """The row kernels index every tensor by x's shape: anything smaller is read or written out of bounds."""
+    if x.dim() != 2 or x.dtype != torch.float32:
+        raise ValueError("x must be a 2-D fp32 tensor")
+    rows, cols = x.shape
+    if gamma.dtype != torch.float32 or gamma.numel() != cols or stats.dtype != torch.float32 or stats.numel() != 2 * rows:
+        raise ValueError("gamma must be fp32 [cols] and stats fp32 [rows, 2]")
+    for t, dt in others:
+        if t is not None and (t.dtype != dt or t.numel() != rows * cols):
+            raise ValueError("tensor of %s with x's shape expected" % dt)
+    return rows, cols
+
+
+def layernorm_bwd_mixed_rows(dy, x, gamma, stats, want_f32=True):
+    """ds_layernorm_bwd_mixed_rows: dy, x fp32 -> (dx bf16, dx fp32 or None, fp32 copy of dy, per-row means [rows, 2])."""
+    _need_cuda(dy, x, gamma, stats)
+    rows, cols = _check_ln_mixed(x, gamma, stats, [(dy, torch.float32)])
+    dx16 = torch.empty(rows, cols, dtype=torch.bfloat16, device=x.device)
+    dx32 = torch.empty_like(x) if want_f32 else None
+    dyc = torch.empty_like(x)
+    row_sums = torch.empty(rows, 2, dtype=torch.float32, device=x.device)
+    check(_lib.load().ds_layernorm_bwd_mixed_rows(rows, cols, ptr(dy), ptr(x), ptr(gamma), ptr(stats), ptr(dx16), ptr(dx32), ptr(dyc),
+                                                  ptr(row_sums), _lib.current_stream()), "ds_layernorm_bwd_mixed_rows")
+    return dx16, dx32, dyc, row_sums
+
+
+def layernorm_param_grads_exact(dy_copy, x, gamma, stats, row_sums, d_gamma, d_beta, d_colsum=None):
+    """ds_layernorm_param_grads_exact: the deferred half of ``layernorm_bwd_mixed_rows``, without rounding."""
+    _need_cuda(dy_copy, x, gamma, stats, row_sums, d_gamma, d_beta, d_colsum)
+    rows, cols = _check_ln_mixed(x, gamma, stats, [(dy_copy, torch.float32)])
+    if row_sums.dtype != torch.float32 or row_sums.numel() != 2 * rows:
+        raise ValueError("row_sums must be fp32 [rows, 2]")
+    for t in (d_gamma, d_beta, d_colsum):
+        if t is not None and (t.dtype != torch.float32 or t.numel() != cols):
+            raise ValueError("parameter gradients must be fp32 [cols]")
+    check(_lib.load().ds_layernorm_param_grads_exact(rows, cols, ptr(dy_copy), ptr(x), ptr(gamma), ptr(stats), ptr(row_sums), ptr(d_gamma),
+                                                     ptr(d_beta), ptr(d_colsum), _lib.current_stream()), "ds_layernorm_param_grads_exact")
+
+
 def layernorm_param_grads_mixed(dy_bf16, x, stats, d_gamma, d_beta, dx_bf16=None, d_colsum=None):
     """d_gamma += sum_rows dy * x_hat, d_beta += sum_rows dy, d_colsum += sum_rows dx from the bf16 copies that
     ``layernorm_bwd_mixed(..., want_dy_bf16=True)`` left and the fp32 x: the deferred half of that backward pass."""
     _need_cuda(dy_bf16, x, stats, d_gamma, d_beta, dx_bf16, d_colsum)
+    if x.dim() != 2 or x.dtype != torch.float32 or stats.numel() != 2 * x.shape[0]:
+        raise ValueError("x must be 2-D fp32 and stats [rows, 2]")
     rows, cols = x.shape
+    for t in (dy_bf16, dx_bf16):
+        if t is not None and (t.dtype != torch.bfloat16 or t.numel() != rows * cols):
+            raise ValueError("dy_bf16 / dx_bf16 must be bf16 with x's shape")
+    for t in (d_gamma, d_beta, d_colsum):
+        if t is not None and (t.dtype != torch.float32 or t.numel() != cols):
+            raise ValueError("parameter gradients must be fp32 [cols]")
     check(_lib.load().ds_layernorm_param_grads_mixed(rows, cols, ptr(dy_bf16), ptr(x), ptr(stats), ptr(dx_bf16), ptr(d_gamma),
                                                      ptr(d_beta), ptr(d_colsum), _lib.current_stream()),
           "ds_layernorm_param_grads_mixed")

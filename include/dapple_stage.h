@@ -114,6 +114,10 @@ size_t ds_gemm_workspace_bytes(int m, int n);
  * process ends), bf16, batch 1, and a shape that ds_gemm would cut (DS_EINVAL otherwise, with the reason).  All calls
  * on one GPU share the scratch: calls that overlap in time on one GPU race; calls on one stream do not. */
 int ds_gemm_static_scratch(const ds_gemm_desc* d, void* stream);
+/* Looks up the scratch's device address on the current device (once per device; launches and allocates nothing).
+ * ds_gemm_static_scratch does it on its first call; a caller that captures that call into a HIP graph calls this
+ * first, outside the capture. */
+int ds_gemm_static_scratch_init(void);
 /* Several independent GEMMs as ONE launch (bf16, k % 64 == 0, the operand-major pairs (K, MN), (K, K), (MN, MN); at
  * most 8 problems).  What a stage holds in steady state - a forward product of one micro-batch, an input-gradient
  * product of another (the reference's graph orders them only by control dependencies, bert/graph.py:126-132) and
@@ -144,6 +148,14 @@ int ds_layernorm_bwd_mixed(int rows, int cols, const float* dy, const float* x, 
  * later, over any number of rows stacked back to back - on another stream, beside the chain. */
 int ds_layernorm_param_grads_mixed(int rows, int cols, const void* dy_bf16, const float* x, const float* stats,
                                    const void* dx_bf16, float* d_gamma, float* d_beta, float* d_colsum, void* stream);
+/* The same split with nothing rounded on the way: ds_layernorm_bwd_mixed_rows writes dx (bf16, and fp32 when dx_f32 is
+ * given), an fp32 copy of dy and, per row, the two means of the backward formula (row_sums [rows][2]); from those, x,
+ * stats and gamma ds_layernorm_param_grads_exact adds d_gamma, d_beta and (d_colsum given) the column sums of the fp32 dx,
+ * which it rebuilds - the sums ds_layernorm_bwd_mixed itself would have formed, up to the order of the additions. */
+int ds_layernorm_bwd_mixed_rows(int rows, int cols, const float* dy, const float* x, const float* gamma, const float* stats,
+                                void* dx_bf16, float* dx_f32, float* dy_copy, float* row_sums, void* stream);
+int ds_layernorm_param_grads_exact(int rows, int cols, const float* dy_copy, const float* x, const float* gamma, const float* stats,
+                                   const float* row_sums, float* d_gamma, float* d_beta, float* d_colsum, void* stream);
 /* dx = LN backward; d_gamma/d_beta (fp32, [cols]) are accumulated (+=); d_colsum (nullable,
  * fp32 [cols]) += column sums of dx (the bias gradient of the dense layer that fed x);
  * dx_add (nullable) is added to dx before it is written (gradient of a residual branch). */

@@ -314,6 +314,16 @@ def test_layernorm_on_an_fp32_stream(rows, cols):
     dg3 = torch.zeros(cols, device="cuda"); db3 = torch.zeros(cols, device="cuda")
     ops.layernorm_param_grads_mixed(dy16, x, stats, dg3, db3)     # without the column sums
     assert torch.allclose(dg3, dg2 - 2.0, atol=1e-4 * float(dg3.abs().max())) and torch.allclose(db3, db2 + 1.0, atol=1e-4 * float(db3.abs().max()))
+    # the split form that rounds nothing on the way: fp32 copy of dy + the two per-row means, then the exact sums
+    fx16, fx32, dyc, row_sums = ops.layernorm_bwd_mixed_rows(dy, x, gamma, stats)
+    assert torch.equal(fx16, ex16) and torch.equal(fx32, ex32) and torch.equal(dyc, dy)
+    dg4 = torch.full((cols,), 2.0, device="cuda")
+    db4 = torch.full((cols,), -1.0, device="cuda")
+    dcs4 = torch.zeros(cols, device="cuda")
+    ops.layernorm_param_grads_exact(dyc, x, gamma, stats, row_sums, dg4, db4, dcs4)
+    assert_close(dg4 - 2.0, dgr, 1e-5, "d_gamma, exact hand-over")
+    assert_close(db4 + 1.0, dbr, 1e-5, "d_beta, exact hand-over")
+    assert_close(dcs4, dxr.sum(0), 1e-4, "column sums of dx, exact hand-over", floor=float(dxr.abs().max()) * rows ** 0.5)
 
 
 @pytest.mark.parametrize("dt", ["fp32", "bf16"])

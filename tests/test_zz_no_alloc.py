@@ -25,13 +25,19 @@ def test_static_scratch_gemm_equals_workspace_gemm_on_two_calls_in_a_row():
     """Two calls back to back through the C ABI, the second on a smaller problem that reuses the front of the scratch the
     first one filled: both equal ds_gemm with a caller workspace bit for bit (same kernel, same slices, same order of
     the fixed-order reduction), and the product itself is right."""
+    from dapple_amd import _lib
+    _lib.check(_lib.load().ds_gemm_static_scratch_init(), "ds_gemm_static_scratch_init")
     for seed, (m, n, k, am, bm) in enumerate([(512, 512, 8192, DS_K_MAJOR, DS_MN_MAJOR), (128, 256, 8192, DS_K_MAJOR, DS_K_MAJOR)]):
         a, b, bias, res = _case(70 + seed, m, n, k, am, bm)
         ws = torch.zeros(ops.gemm_workspace_bytes(m, n), dtype=torch.uint8, device="cuda")
         want = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
         ops.gemm(a, b, want, m, n, k, am, bm, flags=DS_EPI_BIAS | DS_EPI_RESIDUAL, bias=bias, residual=res, workspace=ws)
         got = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
         ops.gemm(a, b, got, m, n, k, am, bm, flags=DS_EPI_BIAS | DS_EPI_RESIDUAL, bias=bias, residual=res, static_scratch=True)
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before, "call %d changed the free device memory" % seed
         assert torch.equal(got, want), "call %d" % seed
         Ar = (a if am == DS_K_MAJOR else a.T).float()
         Br = (b if bm == DS_K_MAJOR else b.T).float()
