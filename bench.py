@@ -406,7 +406,7 @@ def main():
     ap.add_argument("--no-overlap", action="store_true", help="keep forward and backward passes on one stream")
     ap.add_argument("--bf16-residual-stream", action="store_true",
                     help="BERT / XLNet bf16 workloads: round the residual stream to bf16 too (faster, twice the error at full depth)")
-    ap.add_argument("--wgrad-group", type=int, default=4,
+    ap.add_argument("--wgrad-group", type=int, default=8,
                     help="BERT stages: weight gradients of this many backward passes in one GEMM per weight")
     ap.add_argument("--pair-passes", action="store_true",
                     help="BERT stages: issue F(j+1) and B(j) as ONE call that walks both chains level by level, one grouped launch "

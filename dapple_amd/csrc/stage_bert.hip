@@ -236,7 +236,8 @@ struct BertStage : ds_stage {
     // ---- stash layout
     const int K = c.stash_slots;
     G = c.wgrad_group > 1 ? c.wgrad_group : 1;
-    KP = G > 1 ? K + G : K;
+    // (a multiple of G: the G micro-batches of a group then always sit back to back, one GEMM per weight and group)
+    KP = G > 1 ? (K + G + G - 1) / G * G : K;
     NDY = 2 * G;
     const size_t act = (size_t)rows * H * esz, actF = (size_t)rows * F * esz;
     const size_t probs = (size_t)B * NH * S * S * esz, stats = (size_t)rows * 2 * 4;
@@ -968,6 +969,13 @@ struct BertStage : ds_stage {
         }
         if (closing) {
           hipStream_t side = wgrad_stream ? wgrad_stream : stream;
+          {
+            hipStream_t chain = stream;
+            stream = side;
+            const int rc = launch_pending_wgrads();
+            stream = chain;
+            if (rc != DS_OK) return rc;
+          }
           if (centre_k) {
             hipStream_t chain = stream;
             if (side != chain) {  // the key-gradient sums this pass has just queued
@@ -1027,6 +1035,16 @@ struct BertStage : ds_stage {
     }
     return DS_OK;
   }
+  // weight-gradient GEMMs collected for one grouped launch (on `stream`, the stream they were collected for)
+  std::vector<GroupOp> wg_pending;
+  int launch_pending_wgrads() {
+    if (wg_pending.empty()) return DS_OK;
+    static const char* env_skip = getenv("DS_BERT_SKIP_WGRAD_TIMING_ONLY");
+    if (env_skip) { wg_pending.clear(); return DS_OK; }
+    const int rc = ds_group_launch(wg_pending.data(), (int)wg_pending.size(), stream);
+    wg_pending.clear();
+    return rc;
+  }
   int layer_wgrad_runs(int l, const std::vector<Run>& runs) {
     const LayerStash& t = ls[l];
     const int b = base(l);
@@ -1070,13 +1088,36 @@ struct BertStage : ds_stage {
                   const char* du, const char* dz1, const char* dqkv) {
     const int b = base(l);
     ds_prio_scope prio(0);  // feeds only the master gradients
+    // projection gradients: three [H,H] kernels and three biases fed by the columns of dqkv
+    const bool adjacent = g[b + B_K] == g[b + B_Q] + H && g[b + B_V] == g[b + B_Q] + 2 * H &&
+                          g[b + W_K] == g[b + W_Q] + (size_t)H * H && g[b + W_V] == g[b + W_Q] + (size_t)2 * H * H;
+    // Long reductions (several micro-batches' rows per weight): the layer's four weight-gradient GEMMs are independent, so
+    // one launch carries all their 256 x 128 tiles - no hand-over between them, their tails fill each other - and, with
+    // deferred weight gradients, those of two layers (measured on the BERT-48 half-stage: 40.25 -> 38.3 ms per step with
+    // all 8 micro-batches in one group).  DS_BERT_GROUP_WGRAD = -1 switches it off, 0..5 forces a tile shape.
+    static const char* env_gw = getenv("DS_BERT_GROUP_WGRAD");
+    const int group_cfg = env_gw ? atoi(env_gw) : (m >= 2048 ? 1 : -1);
+    if (group_cfg >= 0 && adjacent && dtype == DS_BF16 && m % 64 == 0 && m > 256 && H % 8 == 0 && F % 8 == 0) {
+      GroupOp ops[4];
+      ops[0].gemm = desc_wgrad(m, H, F, h, F, dz2, H, g[b + W_FF2], H);
+      ops[1].gemm = desc_wgrad(m, F, H, a, H, du, F, g[b + W_FF1], F);
+      ops[2].gemm = desc_wgrad(m, H, H, ctx, H, dz1, H, g[b + W_AO], H);
+      ds_gemm_desc& d = ops[3].gemm;
+      d = desc_wgrad(m, H, H, x, H, dqkv, 3 * H, g[b + W_Q], H);
+      d.batch = 3; d.batch_inner = 3; d.b_stride_inner = H; d.c_stride_inner = (int64_t)H * H;
+      for (GroupOp& o : ops) { o.kind = GOP_GEMM; o.cfg = group_cfg; o.prio = 0; wg_pending.push_back(o); }
+      static const char* env_gl = getenv("DS_BERT_GROUP_LAYERS");
+      // (per-pass weight gradients hand their operand buffers back layer by layer: nothing is held over)
+      const size_t per_launch = G > 1 && !(env_gl && atoi(env_gl) == 1) ? 8 : 4;
+      if (wg_pending.size() >= per_launch) DS_PROPAGATE(launch_pending_wgrads());
+      DS_PROPAGATE(ds_colsum_accum(dtype, m, F, du, F, g[b + B_FF1], stream));
+      DS_PROPAGATE(ds_colsum_accum(dtype, m, 3 * H, dqkv, 3 * H, g[b + B_Q], stream));
+      return DS_OK;
+    }
     DS_PROPAGATE(gemm_wgrad(m, H, F, h, F, dz2, H, g[b + W_FF2], H));
     DS_PROPAGATE(ds_colsum_accum(dtype, m, F, du, F, g[b + B_FF1], stream));
     DS_PROPAGATE(gemm_wgrad(m, F, H, a, H, du, F, g[b + W_FF1], F));
     DS_PROPAGATE(gemm_wgrad(m, H, H, ctx, H, dz1, H, g[b + W_AO], H));
-    // projection gradients: three [H,H] kernels and three biases fed by the columns of dqkv
-    const bool adjacent = g[b + B_K] == g[b + B_Q] + H && g[b + B_V] == g[b + B_Q] + 2 * H &&
-                          g[b + W_K] == g[b + W_Q] + (size_t)H * H && g[b + W_V] == g[b + W_Q] + (size_t)2 * H * H;
     if (adjacent) {
       // q, k, v master gradients lie back to back: one column sum over [m, 3H] and one GEMM batched
       // over the three column blocks of dqkv
@@ -1122,6 +1163,7 @@ struct BertStage : ds_stage {
       int rc = DS_OK;
       const std::vector<Run> runs = make_runs(deferred);
       for (int l = L - 1; l >= 0 && rc == DS_OK; --l) rc = layer_wgrad_runs(l, runs);
+      if (rc == DS_OK) rc = launch_pending_wgrads();
       if (rc == DS_OK && centre_k) rc = key_corrections(runs);
       stream = keep;
       if (rc != DS_OK) return rc;
