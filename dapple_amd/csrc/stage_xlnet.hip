@@ -14,6 +14,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include "group.h"
 #include "stage.h"
 
 namespace {
@@ -365,9 +366,9 @@ struct XlnetStage : ds_stage {
     return ds_gemm(&d, stream);
   }
   // batched over (b, n): zo = b, zi = n
-  int gemm_bn(int am, int bm, int m, int n, int k, const void* a, int64_t lda, int64_t a_so, int64_t a_si, const void* b,
-              int64_t ldb, int64_t b_so, int64_t b_si, void* c, int64_t ldc, int64_t c_so, int64_t c_si, int flags,
-              const void* residual = nullptr, int nb = -1) {
+  ds_gemm_desc desc_bn(int am, int bm, int m, int n, int k, const void* a, int64_t lda, int64_t a_so, int64_t a_si, const void* b,
+                       int64_t ldb, int64_t b_so, int64_t b_si, void* c, int64_t ldc, int64_t c_so, int64_t c_si, int flags,
+                       const void* residual = nullptr, int nb = -1) const {
     ds_gemm_desc d;
     memset(&d, 0, sizeof(d));
     d.dtype = dtype; d.a_major = am; d.b_major = bm; d.m = m; d.n = n; d.k = k; d.lda = lda; d.ldb = ldb; d.ldc = ldc;
@@ -375,7 +376,19 @@ struct XlnetStage : ds_stage {
     d.a_stride_outer = a_so; d.a_stride_inner = a_si; d.b_stride_outer = b_so; d.b_stride_inner = b_si;
     d.c_stride_outer = c_so; d.c_stride_inner = c_si;
     d.flags = flags; d.alpha = 1.f; d.a = a; d.b = b; d.c = c; d.residual = residual;
+    return d;
+  }
+  int gemm_bn(int am, int bm, int m, int n, int k, const void* a, int64_t lda, int64_t a_so, int64_t a_si, const void* b,
+              int64_t ldb, int64_t b_so, int64_t b_si, void* c, int64_t ldc, int64_t c_so, int64_t c_si, int flags,
+              const void* residual = nullptr, int nb = -1) {
+    const ds_gemm_desc d = desc_bn(am, bm, m, n, k, a, lda, a_so, a_si, b, ldb, b_so, b_si, c, ldc, c_so, c_si, flags, residual, nb);
     return ds_gemm(&d, stream);
+  }
+  // The per-head products of a backward pass that read the score gradients do not depend on each other: with bf16 and
+  // reductions of whole 64-deep k-tiles they go out as ONE launch of 128 x 64 tiles (DS_XL_GROUP_PRODUCTS=0: one each).
+  bool group_products(int QQ) const {
+    static const char* env = getenv("DS_XL_GROUP_PRODUCTS");
+    return dtype == DS_BF16 && D == 64 && QQ % 64 == 0 && K % 64 == 0 && R % 64 == 0 && QQ > 256 && K > 256 && !(env && atoi(env) == 0);
   }
   static int g1(int64_t n) { int64_t b = (n + 255) / 256; return (int)(b > 8192 ? 8192 : (b < 1 ? 1 : b)); }
 
@@ -634,8 +647,10 @@ struct XlnetStage : ds_stage {
         if (!score_fused)
           DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_K_MAJOR, QQ, K, D, dvec, (int64_t)B * H, H, D, sp + t.kv + (size_t)H * esz, (int64_t)B * 2 * H,
                                2 * H, D, dp, K, (int64_t)N * QQ * K, (int64_t)QQ * K, DS_EPI_OUT_F32));
-        DS_PROPAGATE(gemm_bn(DS_MN_MAJOR, DS_MN_MAJOR, K, D, QQ, p, K, (int64_t)N * QQ * K, (int64_t)QQ * K, dvec, (int64_t)B * H, H, D,
-                             dkv + (size_t)H * esz, (int64_t)B * 2 * H, 2 * H, D, 0));
+        const bool grouped = group_products(QQ);
+        const ds_gemm_desc d_dv = desc_bn(DS_MN_MAJOR, DS_MN_MAJOR, K, D, QQ, p, K, (int64_t)N * QQ * K, (int64_t)QQ * K, dvec, (int64_t)B * H, H, D,
+                                          dkv + (size_t)H * esz, (int64_t)B * 2 * H, 2 * H, D, 0);
+        if (!grouped) DS_PROPAGATE(ds_gemm(&d_dv, stream));
         // dS, its un-shifted copy for the position term (dbd[i][r] = dS[i][r - Q + i]) and the segment sums, in one pass
         float* defs = (float*)(ws_base + ws_def);
         if (score_fused) {
@@ -652,13 +667,23 @@ struct XlnetStage : ds_stage {
         } else if (dtype == DS_BF16) DS_PROPAGATE(softmax_bwd_t<bf16>((const bf16*)p, dp, scale, seg, (bf16*)dsm, (bf16*)dbd, defs));
         else DS_PROPAGATE(softmax_bwd_t<float>((const float*)p, dp, scale, seg, (float*)dsm, (float*)dbd, defs));
         // content term: dqw = dS k ; dk = dS^T qw
-        DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_MN_MAJOR, QQ, D, K, dsm, K, (int64_t)N * QQ * K, (int64_t)QQ * K, sp + t.kv, (int64_t)B * 2 * H, 2 * H, D,
-                             dqw, (int64_t)B * H, H, D, 0));
-        DS_PROPAGATE(gemm_bn(DS_MN_MAJOR, DS_MN_MAJOR, K, D, QQ, dsm, K, (int64_t)N * QQ * K, (int64_t)QQ * K, sp + t.qw, (int64_t)B * H, H, D,
-                             dkv, (int64_t)B * 2 * H, 2 * H, D, 0));
+        const ds_gemm_desc d_dqw = desc_bn(DS_K_MAJOR, DS_MN_MAJOR, QQ, D, K, dsm, K, (int64_t)N * QQ * K, (int64_t)QQ * K, sp + t.kv,
+                                           (int64_t)B * 2 * H, 2 * H, D, dqw, (int64_t)B * H, H, D, 0);
+        const ds_gemm_desc d_dk = desc_bn(DS_MN_MAJOR, DS_MN_MAJOR, K, D, QQ, dsm, K, (int64_t)N * QQ * K, (int64_t)QQ * K, sp + t.qw, (int64_t)B * H,
+                                          H, D, dkv, (int64_t)B * 2 * H, 2 * H, D, 0);
         // position term through the shift
-        DS_PROPAGATE(gemm_bn(DS_K_MAJOR, DS_MN_MAJOR, QQ, D, R, dbd, R, (int64_t)N * QQ * R, (int64_t)QQ * R, kr[l], H, 0, D,
-                             dqr, (int64_t)B * H, H, D, 0));
+        const ds_gemm_desc d_dqr = desc_bn(DS_K_MAJOR, DS_MN_MAJOR, QQ, D, R, dbd, R, (int64_t)N * QQ * R, (int64_t)QQ * R, kr[l], H, 0, D,
+                                           dqr, (int64_t)B * H, H, D, 0);
+        if (grouped) {
+          GroupOp ops[4];
+          ops[0].gemm = d_dqr; ops[1].gemm = d_dqw; ops[2].gemm = d_dk; ops[3].gemm = d_dv;
+          for (GroupOp& o : ops) { o.kind = GOP_GEMM; o.cfg = 3; o.prio = ds_launch_prio; }
+          DS_PROPAGATE(ds_group_launch(ops, 4, stream));
+        } else {
+          DS_PROPAGATE(ds_gemm(&d_dqw, stream));
+          DS_PROPAGATE(ds_gemm(&d_dk, stream));
+          DS_PROPAGATE(ds_gemm(&d_dqr, stream));
+        }
         // (dk_r = dbd^T qr feeds only Wr's gradient: it runs with the weight gradients below)
         // segment term + dq = dqw + dqr + dqs
         {
