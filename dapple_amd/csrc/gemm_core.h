@@ -46,7 +46,8 @@ struct GemmArgs {
   int prio;                    // wave priority (0..3)
   float* ws_part;              // split-K by workspace (8-wave kernels): fp32 partial tiles [tile][slice][BM * BN]
   unsigned* ws_count;          // and one arrival counter per tile (zero between launches)
-  size_t ws_bytes;             // bytes behind ws_part (host side: the launcher checks them against the grid it is about to start)
+  size_t ws_bytes;
+  int flush_each;  // fp32 products: 1 = fold the partial sums after every k-tile (32 terms) instead of every fourth             // bytes behind ws_part (host side: the launcher checks them against the grid it is about to start)
   float* rowdot;               // DS_EPI_ROWDOT (grouped launches only): see gemm_epilogue_vec8
   int rowdot_seq;
 };

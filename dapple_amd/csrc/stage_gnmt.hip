@@ -22,7 +22,7 @@
 
 namespace {
 
-__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + __expf(-x)); }
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
 
 // table rows -> time-major activations: x[(t*B + b), :] = table[ids[b*T + t], :]
 __global__ __launch_bounds__(256) void gnmt_embed_fwd_kernel(int B, int T, int U, int vocab, const int32_t* __restrict__ ids,

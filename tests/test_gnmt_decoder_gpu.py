@@ -98,12 +98,12 @@ def test_projection_and_loss_match_oracle(T, B, U, V, lens):
     x, k = dev(x_np), dev(k_np)
     dk = torch.ones_like(k)                                    # pre-filled: the head adds into the master gradient
     loss, dx = ops.nmt_loss_head(x, k, dev(tgt_np), dev(lens_np), d_proj_kernel=dk, loss_scale=3.0)
-    odt = torch.float64 if V < 1000 else torch.float32          # the full-size case checks against an fp32 CPU run
+    odt = torch.float64
     xo = torch.tensor(x_np, dtype=odt, requires_grad=True)
     ko = torch.tensor(k_np, dtype=odt, requires_grad=True)
     lo, _ = og.nmt_loss(xo, ko, torch.tensor(tgt_np), torch.tensor(lens_np))
     gx, gk = torch.autograd.grad(lo, [xo, ko])
-    tol = TOL if V < 1000 else 5e-4
+    tol = TOL
     assert_close(loss, 3.0 * lo.detach().double().reshape(1), tol, "loss")
     assert_close(dx, 3.0 * gx.double(), tol, "dx")
     assert_close(dk - 1, 3.0 * gk.double(), tol, "d output_projection")

@@ -12,7 +12,7 @@ TOL = 1e-4
 
 
 def run_case(L, U, V, B, T, M, K=2, seed=0, init=0.1, perturb=True, odtype=torch.float64, M_check=None, lengths=None, tol=TOL,
-             tol_l2=None):
+             tol_l2=None, tol_out=None):
     w_np = synthetic.gnmt_weights(synthetic.SEED_WEIGHT + seed, L, U, V, init_weight=init, perturb=perturb)
     ids_np = synthetic.gnmt_id_inputs(synthetic.SEED_INPUT + seed, M, B, T, V)
     dys_np = synthetic.upstream_grads(synthetic.SEED_GRAD + seed, M, (T, B, U))
@@ -34,7 +34,7 @@ def run_case(L, U, V, B, T, M, K=2, seed=0, init=0.1, perturb=True, odtype=torch
         if lengths is not None:
             for b, n in enumerate(lengths[j]):
                 assert float(outs[j][n:, b].abs().max() if n < T else 0.0) == 0.0   # zeros past the end, exactly
-        _close(outs[j], out, tol, tol_l2, "output mb%d" % j)
+        _close(outs[j], out, tol_out or tol, tol_l2, "output mb%d" % j)
         for n, g in dw.items():
             acc[n] = g.clone() if n not in acc else acc[n] + g
     for n in stage.weight_names:
@@ -48,6 +48,7 @@ def _close(got, want, tol, tol_l2, what):
         return
     from util import rel_err
     mx, l2 = rel_err(got, want)
+    print("%-90s rel max %.2e  rel l2 %.2e" % (what, mx, l2), flush=True)
     assert mx <= tol and l2 <= tol_l2, "%s: rel max %.3e (bar %.1e), rel l2 %.3e (bar %.1e)" % (what, mx, tol, l2, tol_l2)
 
 
@@ -77,13 +78,14 @@ def test_config2_full_size():
 
     At this depth (400 chained cell steps with reductions of 2048-3072 terms) fp32 arithmetic itself sits at the 1e-4 bar:
     the same oracle run in fp32 on the CPU (MKL) differs from its fp64 self by 0.9e-4 (max) / 1e-5 (L2) on the outputs and by
-    0.5e-4 .. 1.2e-4 (max), 5e-5 .. 7e-5 (L2) on the weight gradients.  The stage's MFMA products add their terms in
-    plain k order where MKL adds blocked partial sums, which costs about a factor two: measured 1.8e-4 / 1.6e-5 on the outputs,
-    1e-4 .. 3.6e-4 (max) and 1.0e-4 .. 1.5e-4 (L2) on the gradients.  Bars: 5e-4 max-norm, 2e-4 L2; the 1e-4 bar of the
-    stated tolerance is held at depth 3 (test_config2_shape_reduced_depth) and on every smaller case."""
+    0.5e-4 .. 1.2e-4 (max), 5e-5 .. 7e-5 (L2) on the weight gradients.  The stage's fp32 products add blocked partial sums
+    (128 terms at a time) as MKL does; measured: outputs 1.2e-4 (max: single elements behind a saturating gate) / 9e-6 (L2),
+    gradients 4.6e-5 .. 9.4e-5 (max) and 4.9e-5 .. 6.6e-5 (L2).  Bars: the stated 1e-4 on the L2 error of every tensor and on
+    the max-norm of every gradient, 1.5e-4 on the max-norm of the outputs; the 1e-4 max-norm bar is held on the outputs too
+    at depth 3 (test_config2_shape_reduced_depth) and on every smaller case."""
     c = synthetic.CONFIGS["gnmt16_encoder"]
     run_case(L=c["num_layers"], U=c["units"], V=c["vocab"], B=c["micro_batch"], T=c["seq"], M=c["num_micro_batches"], K=2,
-             seed=c["index"], perturb=False, tol=5e-4, tol_l2=2e-4)
+             seed=c["index"], perturb=False, tol=1e-4, tol_l2=1e-4, tol_out=1.5e-4)
 
 
 def test_ragged_sequences():
