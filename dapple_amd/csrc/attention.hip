@@ -55,7 +55,7 @@ extern "C" int ds_attention_fwd(int dtype, int batch, int heads, int seq, int he
   a.qkv = (const bf16*)qkv; a.ld = ld; a.key_mask = key_mask; a.ctx = (bf16*)ctx; a.lse = lse; a.dctx = nullptr; a.dqkv = nullptr;
   a.delta = nullptr; a.B = batch; a.N = heads; a.S = seq; a.H = heads * head_dim; a.scale = scale; a.mask_value = mask_value;
   a.prio = ds_launch_prio; a.kbar = nullptr;
-  static bool attr = false;
+  static std::atomic<bool> attr(false);  // two threads may both set the (idempotent) attribute; neither launches before it is set
   if (!attr) {
     DS_CHECK_HIP(hipFuncSetAttribute((const void*)attn_fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(2048, 2)));
     attr = true;
@@ -95,7 +95,7 @@ extern "C" int ds_attention_bwd_centered(int dtype, int batch, int heads, int se
   a.qkv = (const bf16*)qkv; a.ld = ld; a.key_mask = key_mask; a.ctx = (bf16*)ctx; a.lse = (float*)lse; a.dctx = (const bf16*)dctx;
   a.dqkv = (bf16*)dqkv; a.delta = delta; a.B = batch; a.N = heads; a.S = seq; a.H = heads * head_dim; a.scale = scale;
   a.mask_value = mask_value; a.prio = ds_launch_prio; a.kbar = key_mean;
-  static bool attr = false;
+  static std::atomic<bool> attr(false);  // two threads may both set the (idempotent) attribute; neither launches before it is set
   if (!attr) {
     DS_CHECK_HIP(hipFuncSetAttribute((const void*)attn_bwd_dq_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(2048, 2)));
     DS_CHECK_HIP(hipFuncSetAttribute((const void*)attn_bwd_dkv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(2048, 2)));

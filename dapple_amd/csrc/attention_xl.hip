@@ -490,7 +490,7 @@ int ds_xl_scores_fwd(const XlScoreArgs* a, hipStream_t s) {
   const dim3 grid(a->QQ / RB, a->B * a->N), block(64 * nw);
   const bool full = a->K % 128 == 0;
   const size_t lds = (size_t)nw * 4 * TILE_BYTES;
-  static bool attr = false;
+  static std::atomic<bool> attr(false);  // two threads may both set the (idempotent) attribute; neither launches before it is set
   if (!attr) {
     const int most = MAXW * 4 * TILE_BYTES;
     DS_CHECK_HIP(hipFuncSetAttribute((const void*)xl_scores_fwd_kernel<true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, most));

@@ -693,7 +693,7 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
 template <typename T, int BM, int BN, int AMAJ, int BMAJ, int STAGES>
 int launch_dma(const GemmArgs& a, dim3 grid, hipStream_t stream) {
   constexpr size_t lds = (size_t)STAGES * (BM + BN) * 128;
-  static bool attr_set = false;
+  static std::atomic<bool> attr_set(false);  // two threads may both set the (idempotent) attribute; neither launches before it is set
   if (!attr_set) {
     DS_CHECK_HIP(hipFuncSetAttribute((const void*)gemm_dma_kernel<T, BM, BN, AMAJ, BMAJ, STAGES>,
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
@@ -1037,7 +1037,7 @@ int launch_conv_cfg(GemmArgs a, hipStream_t stream) {
   dim3 grid(a.grid_m * a.grid_n, 1, a.splitk);
   constexpr int STAGES = 4;
   constexpr size_t lds = (size_t)STAGES * (BM + BN) * 128;
-  static bool attr_set = false;
+  static std::atomic<bool> attr_set(false);  // two threads may both set the (idempotent) attribute; neither launches before it is set
   if (!attr_set) {
     DS_CHECK_HIP(hipFuncSetAttribute((const void*)gemm_dma_kernel<float, BM, BN, AMAJ, DS_MN_MAJOR, STAGES, MODE>,
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));

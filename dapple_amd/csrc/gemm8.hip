@@ -40,7 +40,7 @@ int launch8(GemmArgs a, int batch, hipStream_t stream) {
                  a.grid_m, a.grid_n, a.splitk, need, a.ws_bytes);
   }
   constexpr size_t lds = (size_t)STAGES * (BM + BN) * 128;
-  static bool attr_set = false;
+  static std::atomic<bool> attr_set(false);  // two threads may both set the (idempotent) attribute; neither launches before it is set
   if (!attr_set) {
     DS_CHECK_HIP(hipFuncSetAttribute((const void*)gemm8_kernel<BM, BN, WM, WN, WK, STAGES, AMAJ, BMAJ>,
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));

@@ -265,7 +265,7 @@ int ds_group_launch(const GroupOp* ops, int n, hipStream_t stream) {
     next += (t.count + 7) & ~7;
     if (need > lds) lds = need;
   }
-  static bool attr_set = false;
+  static std::atomic<bool> attr_set(false);  // two threads may both set the (idempotent) attribute; neither launches before it is set
   if (!attr_set) {
     DS_CHECK_HIP(hipFuncSetAttribute((const void*)group_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 147456));
     DS_CHECK_HIP(hipFuncSetAttribute((const void*)group_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 98304));

@@ -1039,8 +1039,6 @@ struct BertStage : ds_stage {
   std::vector<GroupOp> wg_pending;
   int launch_pending_wgrads() {
     if (wg_pending.empty()) return DS_OK;
-    static const char* env_skip = getenv("DS_BERT_SKIP_WGRAD_TIMING_ONLY");
-    if (env_skip) { wg_pending.clear(); return DS_OK; }
     const int rc = ds_group_launch(wg_pending.data(), (int)wg_pending.size(), stream);
     wg_pending.clear();
     return rc;

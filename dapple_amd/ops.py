@@ -30,6 +30,14 @@ def _need_cuda(*ts):
             raise ValueError("tensor must be contiguous")
 
 
+def _expect(what, t, dtype, shape):
+    """``t`` (None allowed) must have exactly this element type and shape: the kernels index by these sizes unchecked."""
+    if t is None:
+        return
+    if t.dtype != dtype or tuple(t.shape) != tuple(shape):
+        raise ValueError("%s must be %s %s, got %s %s" % (what, dtype, list(shape), t.dtype, list(t.shape)))
+
+
 def grad_accumulate(acc, g):
     """acc (fp32) += g, in place (tf.accumulate_n of bert/graph.py:159, one micro-batch at a time)."""
     _need_cuda(acc, g)
@@ -293,6 +301,9 @@ def softmax_fwd(scores, scale, key_mask=None, mask_value=-10000.0, out_dtype=tor
     """scores fp32 [B, N, Q, K] -> probabilities of out_dtype."""
     _need_cuda(scores, key_mask)
     b, n, q, k = scores.shape
+    if scores.dtype != torch.float32 or out_dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("softmax_fwd: fp32 scores, fp32 or bf16 probabilities")
+    _expect("softmax_fwd: key_mask", key_mask, torch.float32, (b, k))
     p = torch.empty(b, n, q, k, dtype=out_dtype, device=scores.device)
     check(_lib.load().ds_softmax_fwd(dtype_code(p), b, n, q, k, ptr(scores), scale, ptr(key_mask), mask_value, ptr(p),
                                      _lib.current_stream()), "ds_softmax_fwd")
@@ -301,6 +312,8 @@ def softmax_fwd(scores, scale, key_mask=None, mask_value=-10000.0, out_dtype=tor
 
 def softmax_bwd(p, dp, scale):
     _need_cuda(p, dp)
+    if dp.dtype != torch.float32 or dp.shape != p.shape:
+        raise ValueError("softmax_bwd: dp must be fp32 with the shape of p")
     k = p.shape[-1]
     rows = p.numel() // k
     ds = torch.empty_like(p)
@@ -312,6 +325,7 @@ def softmax_bwd(p, dp, scale):
 def colsum_accum(x, out):
     _need_cuda(x, out)
     rows, cols = x.shape
+    _expect("colsum_accum: out", out, torch.float32, (cols,))
     check(_lib.load().ds_colsum_accum(dtype_code(x), rows, cols, ptr(x), cols, ptr(out), _lib.current_stream()),
           "ds_colsum_accum")
     return out
@@ -422,6 +436,10 @@ def xlnet_scores_pack(seq, rows, klen, batch, masks=None, seg_mat=None):
     if masks is None and seg_mat is None:
         return None, None
     _need_cuda(masks, seg_mat)
+    _expect("xlnet_scores_pack: masks", masks, torch.float32, (rows, klen, batch))
+    _expect("xlnet_scores_pack: seg_mat", seg_mat, torch.uint8, (seq, klen, batch))
+    if rows % seq:
+        raise ValueError("xlnet_scores_pack: rows must be a multiple of seq (the streams are stacked)")
     lib = _lib.load()
     dev = (masks if masks is not None else seg_mat).device
     meta = torch.empty(lib.ds_xlnet_scores_meta_bytes(rows, klen, batch), dtype=torch.uint8, device=dev)
@@ -435,7 +453,14 @@ def xlnet_bias_q(q, bias_context, bias_relative, bias_segment, seg_emb, heads):
     """``q [rows, batch, H]`` (bf16) -> (qw, qr, qs, de): q plus the three relative-attention biases (fp32 ``[H]``) and
     ``de [batch, heads, rows]`` = qs . (seg_emb[1] - seg_emb[0]) per head."""
     _need_cuda(q, bias_context, bias_relative, bias_segment, seg_emb)
-    rows, batch, _ = q.shape
+    rows, batch, hidden = q.shape
+    if q.dtype != torch.bfloat16 or hidden != heads * 64:
+        raise ValueError("xlnet_bias_q: q must be bf16 [rows, batch, heads * 64]")
+    for name, t in (("bias_context", bias_context), ("bias_relative", bias_relative), ("bias_segment", bias_segment)):
+        if t.dtype != torch.float32 or t.numel() != hidden:
+            raise ValueError("xlnet_bias_q: %s must be fp32 with heads * 64 elements" % name)
+    if seg_emb.dtype != torch.float32 or seg_emb.numel() != 2 * hidden:
+        raise ValueError("xlnet_bias_q: seg_emb must be fp32 [2, heads, 64]")
     qw, qr, qs = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
     de = torch.empty(batch, heads, rows, dtype=torch.float32, device=q.device)
     check(_lib.load().ds_xlnet_bias_q(rows, batch, heads, ptr(q), ptr(bias_context), ptr(bias_relative), ptr(bias_segment), ptr(seg_emb),
@@ -443,12 +468,25 @@ def xlnet_bias_q(q, bias_context, bias_relative, bias_segment, seg_emb, heads):
     return qw, qr, qs, de
 
 
+def _xlnet_scores_check(what, seq, rows, klen, batch, heads, hidden, kv, meta):
+    if hidden != heads * 64 or rows % seq or klen < seq:
+        raise ValueError("%s: head size 64, rows a multiple of seq and klen >= seq are required" % what)
+    _expect(what + ": kv", kv, torch.bfloat16, (klen, batch, 2 * hidden))
+    if meta is not None and (meta.dtype != torch.uint8 or meta.numel() != _lib.load().ds_xlnet_scores_meta_bytes(rows, klen, batch)):
+        raise ValueError("%s: meta must be what xlnet_scores_pack returned for these sizes" % what)
+
+
 def xlnet_scores_fwd(qw, qr, de, kv, kr, seq, heads, scale, meta=None):
     """Probabilities of XLNet's relative attention (bf16, head size 64): ``qw, qr [rows, batch, H]`` and ``de`` from
     ``xlnet_bias_q``, ``kv [klen, batch, 2H]``, ``kr [klen + seq, H]`` -> ``p [batch*heads, rows, klen]``."""
     _need_cuda(qw, qr, de, kv, kr, meta)
-    rows, batch, _ = qw.shape
+    rows, batch, hidden = qw.shape
     klen = kv.shape[0]
+    _xlnet_scores_check("xlnet_scores_fwd", seq, rows, klen, batch, heads, hidden, kv, meta)
+    _expect("xlnet_scores_fwd: qw", qw, torch.bfloat16, (rows, batch, hidden))
+    _expect("xlnet_scores_fwd: qr", qr, torch.bfloat16, (rows, batch, hidden))
+    _expect("xlnet_scores_fwd: de", de, torch.float32, (batch, heads, rows))
+    _expect("xlnet_scores_fwd: kr", kr, torch.bfloat16, (klen + seq, hidden))
     p = torch.empty(batch * heads, rows, klen, dtype=qw.dtype, device=qw.device)
     check(_lib.load().ds_xlnet_scores_fwd(seq, rows, klen, batch, heads, ptr(qw), ptr(qr), ptr(de), ptr(kv), ptr(kr), ptr(meta), scale,
                                           ptr(p), _lib.current_stream()), "ds_xlnet_scores_fwd")
@@ -459,8 +497,13 @@ def xlnet_scores_bwd(kv, p, dvec, seq, heads, scale, meta=None, nseg=None, dbd=N
     """Score gradients of the same rows from ``dvec [rows, batch, H]`` (gradient of ``p v``): -> (ds, dbd, defs); ``dbd``
     ``[batch*heads, rows, klen + seq]`` is written only inside its band (pass a cleared buffer to reuse it)."""
     _need_cuda(kv, p, dvec, meta, nseg, dbd)
-    rows, batch, _ = dvec.shape
+    rows, batch, hidden = dvec.shape
     klen = kv.shape[0]
+    _xlnet_scores_check("xlnet_scores_bwd", seq, rows, klen, batch, heads, hidden, kv, meta)
+    _expect("xlnet_scores_bwd: dvec", dvec, torch.bfloat16, (rows, batch, hidden))
+    _expect("xlnet_scores_bwd: p", p, torch.bfloat16, (batch * heads, rows, klen))
+    _expect("xlnet_scores_bwd: nseg", nseg, torch.float32, (batch, seq))
+    _expect("xlnet_scores_bwd: dbd", dbd, torch.bfloat16, (batch * heads, rows, klen + seq))
     ds = torch.empty_like(p)
     if dbd is None:
         dbd = torch.zeros(batch * heads, rows, klen + seq, dtype=p.dtype, device=p.device)
@@ -515,6 +558,10 @@ def lstm_cell_fwd(gates, c_prev=None, forget_bias=1.0, x_residual=None):
     _need_cuda(gates, c_prev, x_residual)
     b, u4 = gates.shape
     u = u4 // 4
+    if gates.dtype != torch.float32 or u4 != 4 * u or u == 0:
+        raise ValueError("lstm_cell_fwd: gates must be fp32 [batch, 4 * units]")
+    _expect("lstm_cell_fwd: c_prev", c_prev, torch.float32, (b, u))
+    _expect("lstm_cell_fwd: x_residual", x_residual, torch.float32, (b, u))
     c = torch.empty(b, u, dtype=torch.float32, device=gates.device)
     h = torch.empty_like(c)
     y = torch.empty_like(c) if x_residual is not None else None
@@ -528,6 +575,13 @@ def lstm_cell_bwd(gates_act, c, c_prev, dh, dc, first):
     gradient between steps (read unless ``first``, then overwritten with dc * f)."""
     _need_cuda(gates_act, c, c_prev, dh, dc)
     b, u4 = gates_act.shape
+    u = u4 // 4
+    if gates_act.dtype != torch.float32 or u4 != 4 * u or u == 0:
+        raise ValueError("lstm_cell_bwd: gates_act must be fp32 [batch, 4 * units]")
+    for name, t in (("c", c), ("c_prev", c_prev), ("dh", dh), ("dc", dc)):
+        _expect("lstm_cell_bwd: " + name, t, torch.float32, (b, u))
+    if c is None or dh is None or dc is None:
+        raise ValueError("lstm_cell_bwd: c, dh and dc are required")
     dgates = torch.empty_like(gates_act)
     check(_lib.load().ds_lstm_cell_bwd(b, u4 // 4, ptr(gates_act), ptr(c), ptr(c_prev), ptr(dh), ptr(dc), 1 if first else 0,
                                        ptr(dgates), _lib.current_stream()), "ds_lstm_cell_bwd")

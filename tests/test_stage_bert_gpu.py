@@ -112,9 +112,9 @@ def test_config3_shape_two_layers_bf16():
 
 
 def test_config3_shape_two_layers_in_the_benchmark_mode():
-    # the mode bench.py times - weight gradients of 4 passes per GEMM, three streams, 8 micro-batches - at the real layer
+    # the mode bench.py times - weight gradients of all 8 passes per GEMM, three streams, 8 micro-batches - at the real layer
     # shape, depth 2, against the fp32 oracle at the stated 2e-2
-    run_case("bf16", 2, 1024, 16, 4096, 2, 512, 8, seed=3, perturb=False, stddev=0.02, odtype=torch.float32, wgrad_group=4,
+    run_case("bf16", 2, 1024, 16, 4096, 2, 512, 8, seed=3, perturb=False, stddev=0.02, odtype=torch.float32, wgrad_group=8,
              overlap=True)
 
 
