@@ -35,6 +35,7 @@ class GemmDesc(C.Structure):
         ("a", C.c_void_p), ("b", C.c_void_p), ("c", C.c_void_p),
         ("bias", C.c_void_p), ("residual", C.c_void_p), ("c2", C.c_void_p),
         ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
+        ("k_segment", C.c_int), ("a_segment_stride", C.c_int64), ("b_segment_stride", C.c_int64),
     ]
 
 

@@ -370,7 +370,7 @@ template <typename T, int W, int MODE> struct ConvDma {
   int r[NV];
   int64_t pix0;
 
-  __device__ __forceinline__ void init(const GemmArgs& p, const T* b, int64_t, int f0, int F, int kt0, int wave, int lane) {
+  __device__ __forceinline__ void init(const GemmArgs& p, const T* b, int64_t, int f0, int F, int kt0, int wave, int lane, int64_t = 0) {
     base = b; H = p.conv_h; Wd = p.conv_w; C = p.conv_c;
     if (MODE == 1) {
       const int kpt = C / KT;
@@ -490,8 +490,8 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs p) {
 
   DA da;
   DB db;
-  da.init(p, A, p.lda, m0, p.m, kt_begin, wave, lane);
-  db.init(p, B, p.ldb, n0, p.n, kt_begin, wave, lane);
+  da.init(p, A, p.lda, m0, p.m, kt_begin, wave, lane, p.a_seg);
+  db.init(p, B, p.ldb, n0, p.n, kt_begin, wave, lane, p.b_seg);
   const int wave_s = __builtin_amdgcn_readfirstlane(wave);  // scalar copy: LDS slot addresses stay in SGPRs
   const uint32_t lds0 = lds_addr(lds);
   // Ring of STAGES tile buffers, tile t in buffer t % STAGES.  All STAGES buffers are filled up front.
@@ -839,6 +839,13 @@ int ds_gemm_make_args(const ds_gemm_desc* d, GemmArgs* out, int* batch_out) {
   DS_CHECK_ARG(!((f & DS_EPI_ACCUM) && (f & (DS_EPI_GELU | DS_EPI_DGELU))), "ds_gemm: ACCUM with GELU");
   DS_CHECK_ARG((f & ~0xFFF) == 0, "ds_gemm: unknown epilogue flags 0x%x", f & ~0xFFF);
   (void)esz;
+  if (d->k_segment != 0) {
+    const int kt = d->dtype == DS_BF16 ? 64 : 32;
+    DS_CHECK_ARG(d->a_major == DS_MN_MAJOR && d->b_major == DS_MN_MAJOR, "ds_gemm: a segmented reduction needs MN-major A and B");
+    DS_CHECK_ARG(d->k_segment > 0 && d->k_segment % kt == 0 && d->k % d->k_segment == 0,
+                 "ds_gemm: k_segment %d must be a multiple of %d that divides k = %d", d->k_segment, kt, d->k);
+    DS_CHECK_ARG(d->a_segment_stride % vec == 0 && d->b_segment_stride % vec == 0, "ds_gemm: segment strides must be multiples of %d", vec);
+  }
 
   GemmArgs a;
   memset(&a, 0, sizeof(a));
@@ -854,6 +861,10 @@ int ds_gemm_make_args(const ds_gemm_desc* d, GemmArgs* out, int* batch_out) {
   a.alpha = d->alpha;
   a.prio = ds_launch_prio;
   a.ws_part = nullptr; a.ws_count = nullptr;
+  if (d->k_segment != 0 && d->k_segment != d->k) {
+    a.seg_ktiles = d->k_segment / (d->dtype == DS_BF16 ? 64 : 32);
+    a.a_seg = d->a_segment_stride; a.b_seg = d->b_segment_stride;
+  }
   a.vec_epi = d->n % 8 == 0 && d->ldc % 8 == 0 && d->c_stride_outer % 8 == 0 && d->c_stride_inner % 8 == 0 &&
               ds_aligned16(d->c) && ds_aligned16(d->residual) && ds_aligned16(d->c2);
   a.splitk = 1;

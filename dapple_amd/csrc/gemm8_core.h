@@ -64,8 +64,8 @@ __device__ __forceinline__ void gemm8_tile(const GemmArgs& p, char* lds, int bx,
 
   DA da;
   DB db;
-  da.init(p, A, p.lda, m0, p.m, kt_begin, wave, lane);
-  db.init(p, B, p.ldb, n0, p.n, kt_begin, wave, lane);
+  da.init(p, A, p.lda, m0, p.m, kt_begin, wave, lane, p.a_seg);
+  db.init(p, B, p.ldb, n0, p.n, kt_begin, wave, lane, p.b_seg);
   const int wave_s = __builtin_amdgcn_readfirstlane(wave);
   const uint32_t lds0 = lds_addr(lds);
 #pragma unroll

@@ -46,8 +46,11 @@ struct GemmArgs {
   int prio;                    // wave priority (0..3)
   float* ws_part;              // split-K by workspace (8-wave kernels): fp32 partial tiles [tile][slice][BM * BN]
   unsigned* ws_count;          // and one arrival counter per tile (zero between launches)
-  size_t ws_bytes;
-  int flush_each;  // fp32 products: 1 = fold the partial sums after every k-tile (32 terms) instead of every fourth             // bytes behind ws_part (host side: the launcher checks them against the grid it is about to start)
+  size_t ws_bytes;             // bytes behind ws_part (host side: the launcher checks them against the grid it is about to start)
+  // Segmented reduction (MN-major operands): k runs over segments of seg_ktiles k-tiles; segment s of A / B starts
+  // a_seg / b_seg elements behind segment s - 1 (0 for both = every segment reads the same rows).  seg_ktiles = 0: one run.
+  int seg_ktiles;
+  int64_t a_seg, b_seg;
   float* rowdot;               // DS_EPI_ROWDOT (grouped launches only): see gemm_epilogue_vec8
   int rowdot_seq;
 };
@@ -215,6 +218,8 @@ template <typename T, int W, int MAJOR, int NW = 4> struct AsmDma {
   uint32_t voff[NV];
   uint64_t tile;      // uniform: address of the current k-tile of this block's operand panel
   int64_t step;       // bytes from one k-tile to the next
+  int64_t seg_jump;   // segmented reduction: what to add on top of `step` when a segment ends
+  int seg_tiles, seg_left;  // k-tiles per segment (0: no segments), k-tiles left in the current one
 
   // a value that is the same in every lane, moved to scalar registers so that it can be an asm "s" operand
   static __device__ __forceinline__ uint64_t uniform64(uint64_t v) {
@@ -222,11 +227,21 @@ template <typename T, int W, int MAJOR, int NW = 4> struct AsmDma {
     return ((uint64_t)hi << 32) | lo;
   }
 
-  __device__ __forceinline__ void init(const GemmArgs&, const T* base, int64_t ld, int f0, int F, int kt0, int wave, int lane) {
+  __device__ __forceinline__ void init(const GemmArgs& p, const T* base, int64_t ld, int f0, int F, int kt0, int wave, int lane,
+                                       int64_t seg_stride = 0) {
     const int64_t k0 = (int64_t)kt0 * KT;
+    seg_tiles = 0; seg_left = 0; seg_jump = 0;
     if (MAJOR == DS_K_MAJOR) {
       tile = uniform64((uint64_t)(uintptr_t)(base + (int64_t)f0 * ld + k0));
       step = (int64_t)uniform64((uint64_t)((int64_t)KT * sizeof(T)));
+    } else if (p.seg_ktiles > 0) {
+      // k-tile kt0 is tile `within` of segment `seg`; a segment's rows are contiguous (stride ld)
+      const int seg = kt0 / p.seg_ktiles, within = kt0 - seg * p.seg_ktiles;
+      tile = uniform64((uint64_t)(uintptr_t)(base + (int64_t)seg * seg_stride + (int64_t)within * KT * ld + f0));
+      step = (int64_t)uniform64((uint64_t)((int64_t)KT * ld * sizeof(T)));
+      seg_tiles = __builtin_amdgcn_readfirstlane(p.seg_ktiles);
+      seg_left = __builtin_amdgcn_readfirstlane(p.seg_ktiles - within);
+      seg_jump = (int64_t)uniform64((uint64_t)((seg_stride - (int64_t)p.seg_ktiles * KT * ld) * (int64_t)sizeof(T)));
     } else {
       tile = uniform64((uint64_t)(uintptr_t)(base + k0 * ld + f0));
       step = (int64_t)uniform64((uint64_t)((int64_t)KT * ld * sizeof(T)));
@@ -253,7 +268,13 @@ template <typename T, int W, int MAJOR, int NW = 4> struct AsmDma {
     const uint32_t m0v = lds_tile + (uint32_t)(i * NW + wave_s) * 1024u;
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0v), "v"(voff[i]), "s"(tile) : "memory", "m0");
   }
-  __device__ __forceinline__ void advance() { tile += (uint64_t)step; }
+  __device__ __forceinline__ void advance() {
+    tile += (uint64_t)step;
+    if (MAJOR != DS_K_MAJOR && seg_tiles > 0 && --seg_left == 0) {  // uniform: scalar compare and add
+      tile += (uint64_t)seg_jump;
+      seg_left = seg_tiles;
+    }
+  }
   __device__ __forceinline__ void issue(uint32_t lds_tile, int wave_s) {
 #pragma unroll
     for (int i = 0; i < NV; ++i) issue_one(lds_tile, wave_s, i);

@@ -63,19 +63,28 @@ def cast_to_f32(src):
 
 
 def _check_gemm_operands(a, b, c, m, n, k, a_major, b_major, lda, ldb, ldc, flags, batch, a_strides, b_strides, c_strides,
-                         bias, residual, c2):
+                         bias, residual, c2, k_segment=0, a_segment_stride=0, b_segment_stride=0, batch_inner=1):
     """Every element the kernels may touch must lie inside the tensors handed in: a wrong shape would fault the GPU."""
     if a.dtype != b.dtype:
         raise ValueError("A and B must have one element type")
     want_c = torch.float32 if (flags & (DS_EPI_OUT_F32 | DS_EPI_ACCUM)) or a.dtype == torch.float32 else torch.bfloat16
     if c.dtype != want_c:
         raise ValueError("C must be %s for these flags" % want_c)
-    zmax = batch - 1
+    inner = max(batch_inner, 1)
+    if batch % inner:
+        raise ValueError("batch must be a multiple of batch_inner")
 
-    def extent(rows, cols, ld, strides):
-        return (rows - 1) * ld + cols + zmax * (abs(strides[0]) + abs(strides[1]))
-    need_a = extent(m, k, lda, a_strides) if a_major == DS_K_MAJOR else extent(k, m, lda, a_strides)
-    need_b = extent(n, k, ldb, b_strides) if b_major == DS_K_MAJOR else extent(k, n, ldb, b_strides)
+    def extent(rows, cols, ld, strides):   # batch entry z sits at (z // inner) * strides[0] + (z % inner) * strides[1]
+        return (rows - 1) * ld + cols + (batch // inner - 1) * abs(strides[0]) + (inner - 1) * abs(strides[1])
+    if k_segment:
+        if a_major != DS_MN_MAJOR or b_major != DS_MN_MAJOR or k_segment <= 0 or k % k_segment or a_segment_stride < 0 or b_segment_stride < 0:
+            raise ValueError("a segmented reduction needs MN-major operands, k_segment dividing k and non-negative segment strides")
+        nseg = k // k_segment
+        need_a = extent(k_segment, m, lda, a_strides) + (nseg - 1) * a_segment_stride
+        need_b = extent(k_segment, n, ldb, b_strides) + (nseg - 1) * b_segment_stride
+    else:
+        need_a = extent(m, k, lda, a_strides) if a_major == DS_K_MAJOR else extent(k, m, lda, a_strides)
+        need_b = extent(n, k, ldb, b_strides) if b_major == DS_K_MAJOR else extent(k, n, ldb, b_strides)
     need_c = extent(m, n, ldc, c_strides)
     if a.numel() < need_a or b.numel() < need_b or c.numel() < need_c:
         raise ValueError("operand too small: A %d < %d, B %d < %d or C %d < %d elements" %
@@ -89,7 +98,7 @@ def _check_gemm_operands(a, b, c, m, n, k, a_major, b_major, lda, ldb, ldc, flag
 
 
 def _gemm_desc(a, b, c, m, n, k, a_major, b_major, lda, ldb, ldc, flags, alpha, bias, residual, c2, batch, batch_inner,
-               a_strides, b_strides, c_strides):
+               a_strides, b_strides, c_strides, k_segment=0, a_segment_stride=0, b_segment_stride=0):
     _need_cuda(a, b, c, bias, residual, c2)
     d = GemmDesc()
     d.dtype = dtype_code(a)
@@ -99,7 +108,8 @@ def _gemm_desc(a, b, c, m, n, k, a_major, b_major, lda, ldb, ldc, flags, alpha, 
     d.ldb = ldb if ldb is not None else (k if b_major == DS_K_MAJOR else n)
     d.ldc = ldc if ldc is not None else n
     _check_gemm_operands(a, b, c, m, n, k, a_major, b_major, d.lda, d.ldb, d.ldc, flags, batch, a_strides, b_strides,
-                         c_strides, bias, residual, c2)
+                         c_strides, bias, residual, c2, k_segment, a_segment_stride, b_segment_stride, batch_inner)
+    d.k_segment, d.a_segment_stride, d.b_segment_stride = k_segment, a_segment_stride, b_segment_stride
     d.batch, d.batch_inner = batch, batch_inner
     d.a_stride_outer, d.a_stride_inner = a_strides
     d.b_stride_outer, d.b_stride_inner = b_strides
@@ -131,34 +141,21 @@ def gemm_grouped(problems):
 
 def gemm(a, b, c, m, n, k, a_major=DS_K_MAJOR, b_major=DS_MN_MAJOR, lda=None, ldb=None, ldc=None, flags=0,
          alpha=1.0, bias=None, residual=None, c2=None, batch=1, batch_inner=1, a_strides=(0, 0), b_strides=(0, 0),
-         c_strides=(0, 0), workspace=None, static_scratch=False):
+         c_strides=(0, 0), workspace=None, static_scratch=False, k_segment=0, a_segment_stride=0, b_segment_stride=0):
     """Raw ds_gemm: C[m][n] (+)= alpha * sum_k A(m,k) B(n,k); see include/dapple_stage.h.  `workspace`: a zero-filled
     uint8 tensor of gemm_workspace_bytes(m, n) bytes that lets the library cut a long k into slices (split-K);
-    `static_scratch`: ds_gemm_static_scratch instead, the variant that allocates nothing (the library's own scratch)."""
-    _need_cuda(a, b, c, bias, residual, c2, workspace)
-    d = GemmDesc()
-    d.dtype = dtype_code(a)
-    d.a_major, d.b_major = a_major, b_major
-    d.m, d.n, d.k = m, n, k
-    d.lda = lda if lda is not None else (k if a_major == DS_K_MAJOR else m)
-    d.ldb = ldb if ldb is not None else (k if b_major == DS_K_MAJOR else n)
-    d.ldc = ldc if ldc is not None else n
-    d.batch, d.batch_inner = batch, batch_inner
-    d.a_stride_outer, d.a_stride_inner = a_strides
-    d.b_stride_outer, d.b_stride_inner = b_strides
-    d.c_stride_outer, d.c_stride_inner = c_strides
-    d.flags, d.alpha = flags, alpha
-    d.a, d.b, d.c = a.data_ptr(), b.data_ptr(), c.data_ptr()
-    d.bias = bias.data_ptr() if bias is not None else None
-    d.residual = residual.data_ptr() if residual is not None else None
-    d.c2 = c2.data_ptr() if c2 is not None else None
+    `static_scratch`: ds_gemm_static_scratch instead, the variant that allocates nothing (the library's own scratch).
+    `k_segment` (MN-major operands): the reduction runs over k / k_segment segments whose first rows are
+    `a_segment_stride` / `b_segment_stride` elements apart."""
+    _need_cuda(workspace)
+    d = _gemm_desc(a, b, c, m, n, k, a_major, b_major, lda, ldb, ldc, flags, alpha, bias, residual, c2, batch, batch_inner,
+                   a_strides, b_strides, c_strides, k_segment, a_segment_stride, b_segment_stride)
     if workspace is not None:
         d.workspace, d.workspace_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
     if static_scratch:
         check(_lib.load().ds_gemm_static_scratch(C.byref(d), _lib.current_stream()), "ds_gemm_static_scratch")
     else:
         check(_lib.load().ds_gemm(C.byref(d), _lib.current_stream()), "ds_gemm")
-    return c
 
 
 def gemm_workspace_bytes(m, n):

@@ -101,6 +101,46 @@ def test_gemm_wide_blocks(am, bm, m, n, k):
     assert_close(acc, (acc0 + Ar @ Br.T).cpu().double(), 1e-5, "gemm accumulate, wide blocks")
 
 
+@pytest.mark.parametrize("dt,m,n,kseg,nseg,agap,bgap", [
+    ("bf16", 1024, 2048, 512, 4, 3, 0),      # 8-wave tiles; A's segments 3 rows apart beyond their length, B's back to back
+    ("bf16", 256, 192, 128, 3, 0, 5),        # 4-wave tiles
+    ("bf16", 4096, 1024, 1024, 8, 2, 1),     # a weight gradient over 8 micro-batches
+    ("bf16", 1024, 1024, 1408, 2, -1, 0),    # A's segment stride 0: both segments read the same rows
+    ("fp32", 512, 256, 96, 5, 1, 2),
+])
+def test_gemm_segmented_reduction(dt, m, n, kseg, nseg, agap, bgap):
+    """ds_gemm_desc.k_segment: C += sum over segments s of A_s^T B_s with the segments' first rows a fixed stride apart (rows
+    of other tensors in between, as in a stash whose slots hold one micro-batch each); against the sum of the per-segment
+    products, through the plain launch, the accumulate epilogue and a grouped launch."""
+    r = rng(m + n + kseg * nseg)
+    tdt = DT[dt]
+    arows = kseg + agap if agap >= 0 else 0          # rows from one segment's start to the next
+    brows = kseg + bgap
+    a = dev(r.standard_normal((max(arows, 1) * (nseg - 1) + kseg, m)) * 0.5, tdt)
+    b = dev(r.standard_normal((brows * (nseg - 1) + kseg, n)) * 0.5, tdt)
+    ref = torch.zeros(m, n, dtype=torch.float64)
+    for s_ in range(nseg):
+        As = a[s_ * arows: s_ * arows + kseg].float().cpu().double()
+        Bs = b[s_ * brows: s_ * brows + kseg].float().cpu().double()
+        ref += As.T @ Bs
+    kw = dict(k_segment=kseg, a_segment_stride=arows * m, b_segment_stride=brows * n)
+    c = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda")
+    ops.gemm(a, b, c, m, n, kseg * nseg, DS_MN_MAJOR, DS_MN_MAJOR, flags=DS_EPI_OUT_F32, **kw)
+    assert_close(c, ref, 1e-5 if dt == "bf16" else 1e-5, "segmented reduction")
+    acc0 = dev(r.standard_normal((m, n)), torch.float32)
+    acc = acc0.clone()
+    ops.gemm(a, b, acc, m, n, kseg * nseg, DS_MN_MAJOR, DS_MN_MAJOR, flags=DS_EPI_ACCUM, **kw)
+    assert_close(acc, acc0.cpu().double() + ref, 1e-5, "segmented reduction, accumulate")
+    if dt == "bf16":
+        for cfg in (1, 3):
+            g = acc0.clone()
+            ops.gemm_grouped([dict(a=a, b=b, c=g, m=m, n=n, k=kseg * nseg, a_major=DS_MN_MAJOR, b_major=DS_MN_MAJOR, flags=DS_EPI_ACCUM,
+                                   cfg=cfg, **kw)])
+            assert_close(g, acc0.cpu().double() + ref, 1e-5, "segmented reduction, grouped launch cfg %d" % cfg)
+    with pytest.raises((ValueError, RuntimeError)):
+        ops.gemm(a, b, c, m, n, kseg * nseg, DS_MN_MAJOR, DS_MN_MAJOR, flags=DS_EPI_OUT_F32, k_segment=kseg + 8, a_segment_stride=0, b_segment_stride=0)
+
+
 @pytest.mark.parametrize("am,bm", [(0, 0), (0, 1), (1, 1)])
 @pytest.mark.parametrize("m,n,k", [(128, 256, 8192), (248, 120, 6144), (384, 128, 16384)])
 def test_gemm_split_k_by_workspace(am, bm, m, n, k):
