@@ -315,8 +315,9 @@ def make_xlnet(c, args):
                                   c["streams"], c["num_micro_batches"])
     adt = torch.bfloat16 if c["dtype"] == "bf16" else torch.float32
     K = runtime.stash_depth(0, 2)
+    G = max(1, min(args.wgrad_group, M)) if c["dtype"] == "bf16" else 1
     stage = runtime.xlnet_stage(L, H, N, F, B, Q, c["dtype"], stash_slots=K, mem_len=Mm, streams=S,
-                                attention=args.xlnet_attention, residual_fp32=not args.bf16_residual_stream)
+                                attention=args.xlnet_attention, residual_fp32=not args.bf16_residual_stream, wgrad_group=G)
     stage.bind(synthetic.xlnet_weights(synthetic.SEED_WEIGHT + c["index"], L, H, N, F))
     xs = [torch.as_tensor(np.stack(x)).cuda().to(adt) for x in synthetic.xlnet_stream_inputs(synthetic.SEED_INPUT + c["index"], M, Q, B, H, S)]
     dys = [torch.as_tensor(np.stack(x)).cuda().to(adt) for x in synthetic.xlnet_stream_inputs(synthetic.SEED_GRAD + c["index"], M, Q, B, H, S)]
@@ -337,7 +338,7 @@ def make_xlnet(c, args):
     fwd = 2 * H * H * (S * Q + 2 * Kl + R + S * Q) + S * (2 * 2 * Q * Kl * H + 2 * Q * R * H) + S * 4 * Q * H * F
     wl.flops_per_sample = 3 * fwd * L
     wl.config = {"layers": L, "hidden": H, "heads": N, "ffn": F, "seq": Q, "mem_len": Mm, "streams": S, "micro_batch": B,
-                 "micro_batches": M, "schedule": "1F1B stage 0 of 2, stash K=%d" % K, "flops": "two-stream count",
+                 "micro_batches": M, "schedule": "1F1B stage 0 of 2, stash K=%d" % K, "flops": "two-stream count", "wgrad_group": G,
                  "residual_stream": "fp32" if (c["dtype"] != "bf16" or not args.bf16_residual_stream) else "bf16",
                  "attention_scores": "one kernel per pass" if args.xlnet_attention == "auto" else "separate launches, fp32 scores"}
 

@@ -79,7 +79,7 @@ class XlnetCfg(C.Structure):
         ("dtype", C.c_int), ("num_layers", C.c_int), ("hidden", C.c_int), ("heads", C.c_int), ("ffn", C.c_int),
         ("batch", C.c_int), ("seq", C.c_int), ("mem_len", C.c_int), ("streams", C.c_int), ("ln_eps", C.c_float),
         ("first_layer", C.c_int), ("stash_slots", C.c_int), ("fused_attention", C.c_int), ("residual_fp32", C.c_int),
-        ("reserved", C.c_int * 6),
+        ("wgrad_group", C.c_int), ("reserved", C.c_int * 5),
     ]
 
 

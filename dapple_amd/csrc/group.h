@@ -53,7 +53,7 @@ struct GroupOp {
   GroupOp() { memset(&gemm, 0, sizeof(gemm)); }
 };
 
-constexpr int DS_GROUP_MAX_TASKS = 8;
+constexpr int DS_GROUP_MAX_TASKS = 12;  // (288 bytes of kernel arguments each, 4 KB in all)
 // All tasks as one launch; workgroups start in list order.
 int ds_group_launch(const GroupOp* ops, int n, hipStream_t stream);
 // The tile shape ds_group_launch picks for a GEMM when GroupOp::cfg < 0.

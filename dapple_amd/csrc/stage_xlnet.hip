@@ -200,7 +200,9 @@ __global__ __launch_bounds__(256) void xl_seg_bwd_kernel(int QQ, int B, int N, i
   }
 }
 
-struct LayerOff { size_t x, qw, qr, qs, kv, p, vec, z1, y1, u, hh, z2, st1, st2; };
+// (mem directly in front of x: the memory rows followed by the content stream's rows are the [klen * batch, hidden] input of
+// the key / value projection, read as one matrix)
+struct LayerOff { size_t mem, x, qw, qr, qs, kv, p, vec, z1, y1, u, hh, z2, st1, st2; };
 
 struct XlnetStage : ds_stage {
   ds_xlnet_cfg xc;
@@ -213,7 +215,7 @@ struct XlnetStage : ds_stage {
   char* pe = nullptr;
   // stash
   char* stash_base = nullptr;
-  size_t slot_bytes = 0, mask_off = 0, seg_off = 0, mem_off = 0, meta_off = 0, nseg_off = 0;
+  size_t slot_bytes = 0, mask_off = 0, seg_off = 0, meta_off = 0, nseg_off = 0, mem_bytes = 0, layer_stride = 0;
   // scores + softmax (forward) and score gradients (backward) in one kernel each, no fp32 score matrices (attention_xl.hip)
   bool score_fused = false;
   // bf16 with xc.residual_fp32: the residual stream (the sums in front of both LayerNorms, the LayerNorm outputs that feed
@@ -229,13 +231,40 @@ struct XlnetStage : ds_stage {
   size_t ws_bytes = 0, ws_de = 0, ws_qall, ws_ac, ws_dp, ws_bd, ws_ds, ws_dbd[2], ws_def, ws_dz2[2], ws_du[2], ws_dy1, ws_dz1[2], ws_dvec, ws_dqw[2], ws_dqr[2],
          ws_dqs[2], ws_dq[2], ws_dkv[2], ws_dkr[2], ws_deft[2], ws_dx[2];
   WgradLane lane;
+  // Deferred weight gradients (xc.wgrad_group = G > 1, bf16): a backward pass leaves the operands of its weight-gradient
+  // products in a ring of 2G positions per layer and its activations stay in their stash position; after every G passes
+  // ONE product per weight runs over all G micro-batches (a segmented reduction: the micro-batches' rows sit one stash
+  // position / one ring position apart), the products of two layers as one grouped launch.  There are then more stash
+  // positions than slots (slots + G, rounded up to a multiple of G), handed out round-robin in forward order.
+  int G = 1, KP = 0, NDY = 0;
+  struct LayerDy { size_t dz2, du, dz1, dq, dqw, dqr, dqs, dkv, dkr; };
+  std::vector<LayerDy> ld;
+  char* dy_base = nullptr;
+  size_t dy_act = 0, dy_actF = 0, dy_kv = 0, dy_kr = 0;
+  struct Deferred { int xpos, dypos; };
+  struct Run { int xpos, dypos, n; };
+  std::vector<Deferred> deferred;
+  std::vector<int> slot_pos, pos_owner;
+  std::vector<char> slot_fresh, pos_deferred, x_bwd_valid, x_wg_valid, dy_wg_valid;
+  std::vector<hipEvent_t> ev_x_bwd, ev_x_wg, ev_dy_wg;
+  hipEvent_t ev_chain = nullptr, ev_wg_done = nullptr;
+  bool wg_outstanding = false;
+  int next_pos = 0;
+  int64_t n_backward = 0;
+  std::vector<GroupOp> wg_pending;
   hipEvent_t ev_refresh = nullptr;
   std::vector<hipEvent_t> ev_cast;   // layer l's compute copies written (refresh_weights on the weight-gradient stream)
   std::vector<char> cast_pending;
 
   ~XlnetStage() override {
     if (ev_refresh) (void)hipEventDestroy(ev_refresh);
+    if (ev_chain) (void)hipEventDestroy(ev_chain);
+    if (ev_wg_done) (void)hipEventDestroy(ev_wg_done);
     for (hipEvent_t e : ev_cast) (void)hipEventDestroy(e);
+    for (hipEvent_t e : ev_x_bwd) (void)hipEventDestroy(e);
+    for (hipEvent_t e : ev_x_wg) (void)hipEventDestroy(e);
+    for (hipEvent_t e : ev_dy_wg) (void)hipEventDestroy(e);
+    if (dy_base) (void)hipFree(dy_base);
     if (wc_base) (void)hipFree(wc_base);
     if (stash_base) (void)hipFree(stash_base);
     if (ws_base) (void)hipFree(ws_base);
@@ -283,7 +312,6 @@ struct XlnetStage : ds_stage {
     const size_t act = (size_t)rows * H * esz, actF = (size_t)rows * F * esz, stats = (size_t)rows * 2 * 4;
     mask_off = sa.reserve((size_t)S * Q * K * B * 4);
     seg_off = sa.reserve((size_t)Q * K * B);
-    mem_off = sa.reserve((size_t)L * (Mm > 0 ? Mm : 1) * B * H * esz);
     score_fused = xc.fused_attention != DS_XL_ATTN_SEPARATE && ds_xl_scores_fit(dtype, D, Q, K, R);
     rs32 = dtype == DS_BF16 && xc.residual_fp32 != 0 && H % 8 == 0 && H <= 2048;
     if (score_fused) {
@@ -291,20 +319,52 @@ struct XlnetStage : ds_stage {
       nseg_off = sa.reserve((size_t)Q * B * 4);
     }
     lo.resize(L);
-    size_t next_x = sa.reserve(act);
+    mem_bytes = (size_t)Mm * B * H * esz;   // a multiple of 16: x stays aligned for vector loads
+    size_t next_x = sa.reserve(mem_bytes + act);
     for (int l = 0; l < L; ++l) {
       LayerOff& t = lo[l];
-      t.x = next_x;
+      t.mem = next_x;
+      t.x = next_x + mem_bytes;
       t.qw = sa.reserve(act); t.qr = sa.reserve(act); t.qs = sa.reserve(act);
       t.kv = sa.reserve((size_t)krows * 2 * H * esz);
       t.p = sa.reserve((size_t)S * B * N * Q * K * esz);
       t.vec = sa.reserve(act); t.z1 = sa.reserve(rs32 ? (size_t)rows * H * 4 : act); t.y1 = sa.reserve(act);
       t.u = sa.reserve(actF); t.hh = sa.reserve(actF); t.z2 = sa.reserve(rs32 ? (size_t)rows * H * 4 : act);
       t.st1 = sa.reserve(stats); t.st2 = sa.reserve(stats);
-      if (l + 1 < L) next_x = sa.reserve(act);
+      if (l + 1 < L) next_x = sa.reserve(mem_bytes + act);
     }
+    layer_stride = L > 1 ? lo[1].mem - lo[0].mem : mem_bytes + act;
     slot_bytes = sa.used;
-    DS_CHECK_HIP(hipMalloc((void**)&stash_base, slot_bytes * xc.stash_slots));
+    // deferred weight gradients need whole k-tiles per segment of every reduction (bf16: 64 rows)
+    G = xc.wgrad_group > 1 && dtype == DS_BF16 && rows % 64 == 0 && krows % 64 == 0 && R % 64 == 0 && H % 8 == 0 && F % 8 == 0 ? xc.wgrad_group : 1;
+    KP = G > 1 ? (xc.stash_slots + G + G - 1) / G * G : xc.stash_slots;
+    NDY = 2 * G;
+    DS_CHECK_HIP(hipMalloc((void**)&stash_base, slot_bytes * KP));
+    slot_pos.assign(xc.stash_slots, -1);
+    slot_fresh.assign(xc.stash_slots, 0);
+    if (G <= 1) for (int i = 0; i < xc.stash_slots; ++i) slot_pos[i] = i;
+    if (G > 1) {
+      pos_owner.assign(KP, -1);
+      pos_deferred.assign(KP, 0);
+      Arena da;
+      dy_act = act; dy_actF = actF; dy_kv = (size_t)krows * 2 * H * esz; dy_kr = (size_t)R * H * esz;
+      ld.resize(L);
+      for (int l = 0; l < L; ++l) {
+        ld[l].dz2 = da.reserve(dy_act * NDY); ld[l].du = da.reserve(dy_actF * NDY); ld[l].dz1 = da.reserve(dy_act * NDY);
+        ld[l].dq = da.reserve(dy_act * NDY); ld[l].dqw = da.reserve(dy_act * NDY); ld[l].dqr = da.reserve(dy_act * NDY);
+        ld[l].dqs = da.reserve(dy_act * NDY); ld[l].dkv = da.reserve(dy_kv * NDY); ld[l].dkr = da.reserve(dy_kr * NDY);
+      }
+      DS_CHECK_HIP(hipMalloc((void**)&dy_base, da.used));
+      ev_x_bwd.assign(KP, nullptr); ev_x_wg.assign(KP, nullptr); ev_dy_wg.assign(NDY, nullptr);
+      for (int i = 0; i < KP; ++i) {
+        DS_CHECK_HIP(hipEventCreateWithFlags(&ev_x_bwd[i], hipEventDisableTiming));
+        DS_CHECK_HIP(hipEventCreateWithFlags(&ev_x_wg[i], hipEventDisableTiming));
+      }
+      for (int i = 0; i < NDY; ++i) DS_CHECK_HIP(hipEventCreateWithFlags(&ev_dy_wg[i], hipEventDisableTiming));
+      DS_CHECK_HIP(hipEventCreateWithFlags(&ev_chain, hipEventDisableTiming));
+      DS_CHECK_HIP(hipEventCreateWithFlags(&ev_wg_done, hipEventDisableTiming));
+      x_bwd_valid.assign(KP, 0); x_wg_valid.assign(KP, 0); dy_wg_valid.assign(NDY, 0);
+    }
     slot_forwarded.assign(xc.stash_slots, 0);
     has_mask.assign(xc.stash_slots, 0);
     has_seg.assign(xc.stash_slots, 0);
@@ -348,7 +408,7 @@ struct XlnetStage : ds_stage {
   size_t workspace_bytes() const override { return ws_bytes; }
   // forward writes qall / ac / bd and its stash slot, backward everything else: disjoint
   bool overlap_safe() const override { return true; }
-  size_t stash_bytes(int slots) const override { return slot_bytes * (size_t)slots; }
+  size_t stash_bytes(int slots) const override { return slot_bytes * (size_t)(G > 1 ? (slots + G + G - 1) / G * G : slots); }
 
   const void* WT(int l, int which) const {
     if (dtype == DS_BF16) {
@@ -448,13 +508,38 @@ struct XlnetStage : ds_stage {
     return DS_OK;
   }
 
+  // A stash position for the micro-batch that enters `slot` next (deferred weight gradients only): round-robin over the
+  // positions no micro-batch owns; a position that deferred weight-gradient work still reads is flushed first, and
+  // `s` - the stream that will write the position - waits for the kernels that last read it.
+  int assign_pos(int slot, hipStream_t s) {
+    for (int tries = 0; tries < KP; ++tries) {
+      const int p = next_pos;
+      next_pos = next_pos + 1 == KP ? 0 : next_pos + 1;
+      if (pos_owner[p] >= 0) continue;
+      if (pos_deferred[p]) DS_PROPAGATE(flush_deferred(false));
+      if (x_bwd_valid[p]) DS_CHECK_HIP(hipStreamWaitEvent(s, ev_x_bwd[p], 0));
+      if (x_wg_valid[p]) DS_CHECK_HIP(hipStreamWaitEvent(s, ev_x_wg[p], 0));
+      x_bwd_valid[p] = x_wg_valid[p] = 0;
+      pos_owner[p] = slot;
+      slot_pos[slot] = p;
+      return DS_OK;
+    }
+    ds_set_error("ds_stage_forward: no free stash position");
+    return DS_ESTATE;
+  }
+  char* slot_base(int slot) const { return stash_base + (size_t)slot_pos[slot] * slot_bytes; }
+
   int set_aux(int slot, const float* masks, const uint8_t* seg_mat, const void* mems) {
-    char* sp = stash_base + (size_t)slot * slot_bytes;
+    if (G > 1 && !slot_fresh[slot]) {  // the side inputs of a micro-batch travel with its stash position
+      DS_PROPAGATE(assign_pos(slot, stream));
+      slot_fresh[slot] = 1;
+    }
+    char* sp = slot_base(slot);
     if (masks) DS_CHECK_HIP(hipMemcpyAsync(sp + mask_off, masks, (size_t)S * Q * K * B * 4, hipMemcpyDeviceToDevice, stream));
     if (seg_mat) DS_CHECK_HIP(hipMemcpyAsync(sp + seg_off, seg_mat, (size_t)Q * K * B, hipMemcpyDeviceToDevice, stream));
     if (Mm > 0) {
       if (!mems) { ds_set_error("ds_xlnet_stage_set_inputs: mem_len is %d but mems is NULL", Mm); return DS_EINVAL; }
-      DS_CHECK_HIP(hipMemcpyAsync(sp + mem_off, mems, (size_t)L * Mm * B * H * esz, hipMemcpyDeviceToDevice, stream));
+      DS_CHECK_HIP(hipMemcpy2DAsync(sp + lo[0].mem, layer_stride, mems, mem_bytes, mem_bytes, L, hipMemcpyDeviceToDevice, stream));
     }
     has_mask[slot] = masks != nullptr;
     has_seg[slot] = seg_mat != nullptr;
@@ -497,7 +582,18 @@ struct XlnetStage : ds_stage {
 
   int forward(int slot, const void* in, const float*, void* out) override {
     ds_prio_scope prio(1);
-    char* sp = stash_base + (size_t)slot * slot_bytes;
+    if (G > 1) {
+      if (!slot_fresh[slot]) {
+        if (has_mask[slot] || has_seg[slot] || Mm > 0) {
+          ds_set_error("ds_stage_forward: with wgrad_group > 1 a micro-batch's masks, segments and memories live in its own stash "
+                       "position: call ds_xlnet_stage_set_inputs before every forward pass");
+          return DS_ESTATE;
+        }
+        DS_PROPAGATE(assign_pos(slot, stream));
+      }
+      slot_fresh[slot] = 0;
+    }
+    char* sp = slot_base(slot);
     const size_t act = (size_t)rows * H * esz;
     const float scale = 1.0f / sqrtf((float)D);
     const uint8_t* seg = has_seg[slot] ? (const uint8_t*)(sp + seg_off) : nullptr;
@@ -515,9 +611,7 @@ struct XlnetStage : ds_stage {
       DS_PROPAGATE(await_cast(l, stream));
       // q for every stream row; k|v for memory rows and for the content-stream rows
       DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, rows, H, H, x, H, WT(l, X_Q), H, qall, H));
-      if (Mm > 0)
-        DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, Mm * B, 2 * H, H, sp + mem_off + (size_t)l * Mm * B * H * esz, H, wkv[l], 2 * H, sp + t.kv, 2 * H));
-      DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, rowsS, 2 * H, H, x, H, wkv[l], 2 * H, sp + t.kv + (size_t)Mm * B * 2 * H * esz, 2 * H));
+      DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, krows, 2 * H, H, sp + t.mem, H, wkv[l], 2 * H, sp + t.kv, 2 * H));
       {
         const int64_t total = (int64_t)rows * H;
         if (score_fused)
@@ -590,9 +684,145 @@ struct XlnetStage : ds_stage {
     return DS_OK;
   }
 
+  int release(int slot) override {
+    if (G > 1 && slot_pos[slot] >= 0) {  // the stash position goes back to the pool; nothing was deferred for it
+      const int pos = slot_pos[slot];
+      pos_owner[pos] = -1;
+      x_bwd_valid[pos] = 0;
+    }
+    return DS_OK;
+  }
+
+  // runs of micro-batches that sit in consecutive stash positions and consecutive ring positions: one product per run
+  static std::vector<Run> make_runs(const std::vector<Deferred>& d) {
+    std::vector<Run> runs;
+    size_t i = 0;
+    while (i < d.size()) {
+      size_t j = i + 1;
+      while (j < d.size() && d[j].xpos == d[j - 1].xpos + 1 && d[j].dypos == d[j - 1].dypos + 1) ++j;
+      runs.push_back({d[i].xpos, d[i].dypos, (int)(j - i)});
+      i = j;
+    }
+    return runs;
+  }
+  int launch_pending_wgrads() {
+    if (wg_pending.empty()) return DS_OK;
+    const int rc = ds_group_launch(wg_pending.data(), (int)wg_pending.size(), stream);
+    wg_pending.clear();
+    return rc;
+  }
+  // The deferred weight gradients of layer l for every run, on `stream`: six products per run - W2, W1, o, q, r, k|v - each
+  // a segmented reduction over the run's micro-batches (activations one stash position apart, gradients one ring position
+  // apart), queued for a grouped launch of 256 x 128 tiles (two layers per launch) where the reduction is long enough,
+  // and the bias column sums over the run's rows.
+  int layer_wgrad_runs(int l, const std::vector<Run>& runs) {
+    const LayerOff& t = lo[l];
+    const int b = base(l);
+    ds_prio_scope prio(0);
+    const int64_t sstride = (int64_t)(slot_bytes / esz);
+    const bool kv_adjacent = g[b + X_V] == g[b + X_K] + (size_t)H * H;
+    for (const Run& r : runs) {
+      const char* sp0 = stash_base + (size_t)r.xpos * slot_bytes;
+      const char* dz2 = dy_base + ld[l].dz2 + r.dypos * dy_act; const char* du = dy_base + ld[l].du + r.dypos * dy_actF;
+      const char* dz1 = dy_base + ld[l].dz1 + r.dypos * dy_act; const char* dq = dy_base + ld[l].dq + r.dypos * dy_act;
+      const char* dkv = dy_base + ld[l].dkv + r.dypos * dy_kv; const char* dkr = dy_base + ld[l].dkr + r.dypos * dy_kr;
+      ds_gemm_desc ds[7];
+      int nd = 0;
+      auto wg = [&](int m, int n, int kseg, const void* a, int64_t lda, int64_t aseg, const void* bb, int64_t ldb, int64_t bseg, float* c,
+                    int64_t ldc) -> ds_gemm_desc& {
+        ds_gemm_desc& d = ds[nd++];
+        memset(&d, 0, sizeof(d));
+        d.dtype = dtype; d.a_major = DS_MN_MAJOR; d.b_major = DS_MN_MAJOR; d.m = m; d.n = n; d.k = kseg * r.n; d.lda = lda; d.ldb = ldb; d.ldc = ldc;
+        d.batch = 1; d.batch_inner = 1; d.flags = DS_EPI_ACCUM; d.alpha = 1.f; d.a = a; d.b = bb; d.c = c;
+        if (r.n > 1) { d.k_segment = kseg; d.a_segment_stride = aseg; d.b_segment_stride = bseg; }
+        return d;
+      };
+      wg(F, H, rows, sp0 + t.hh, F, sstride, dz2, H, (int64_t)rows * H, g[b + X_W2], H);
+      wg(H, F, rows, sp0 + t.y1, H, sstride, du, F, (int64_t)rows * F, g[b + X_W1], F);
+      wg(H, H, rows, dz1, H, (int64_t)rows * H, sp0 + t.vec, H, sstride, g[b + X_O], H);
+      wg(H, H, rows, sp0 + t.x, H, sstride, dq, H, (int64_t)rows * H, g[b + X_Q], H);
+      wg(H, H, R, pe, H, 0, dkr, H, (int64_t)R * H, g[b + X_R], H);   // every micro-batch against the same position table
+      if (kv_adjacent) {  // k and v: the two column halves of dkv, batched (z = 0: k, 1: v)
+        ds_gemm_desc& d = wg(H, H, krows, sp0 + t.mem, H, sstride, dkv, 2 * H, (int64_t)krows * 2 * H, g[b + X_K], H);
+        d.batch = 2; d.batch_inner = 2; d.b_stride_inner = H; d.c_stride_inner = (int64_t)H * H;
+      } else {
+        for (int j = 0; j < 2; ++j)
+          wg(H, H, krows, sp0 + t.mem, H, sstride, dkv + (size_t)j * H * esz, 2 * H, (int64_t)krows * 2 * H, g[b + X_K + j], H);
+      }
+      for (int i = 0; i < nd; ++i) {
+        // (one launch never carries two products into the same master gradient: runs of one layer are flushed apart)
+        const bool grouped = ds[i].k / 64 > 3 && ds[i].m >= 128 && ds[i].n >= 128;
+        if (grouped) {
+          GroupOp o;
+          o.kind = GOP_GEMM; o.gemm = ds[i]; o.cfg = ds[i].m >= 256 ? 1 : 2; o.prio = 0;
+          wg_pending.push_back(o);
+        } else {
+          DS_PROPAGATE(ds_gemm(&ds[i], stream));
+        }
+      }
+      if (runs.size() > 1 || wg_pending.size() + nd > (size_t)DS_GROUP_MAX_TASKS) DS_PROPAGATE(launch_pending_wgrads());
+      DS_PROPAGATE(ds_colsum_accum(dtype, rows * r.n, F, du, F, g[b + X_B1], stream));
+      const void* const xs3[3] = {dy_base + ld[l].dqw + r.dypos * dy_act, dy_base + ld[l].dqr + r.dypos * dy_act, dy_base + ld[l].dqs + r.dypos * dy_act};
+      float* const out3[3] = {g[b + X_RW], g[b + X_RR], g[b + X_RS]};
+      DS_PROPAGATE(ds_colsum_accum_multi(dtype, rows * r.n, H, 3, xs3, H, out3, stream));
+    }
+    return DS_OK;
+  }
+  // the weight-gradient work of every deferred pass has been queued on `ws`
+  int retire_deferred(hipStream_t ws, hipStream_t chain) {
+    for (const Deferred& e : deferred) {
+      if (ws != chain) {
+        DS_CHECK_HIP(hipEventRecord(ev_x_wg[e.xpos], ws));
+        DS_CHECK_HIP(hipEventRecord(ev_dy_wg[e.dypos], ws));
+      }
+      x_wg_valid[e.xpos] = dy_wg_valid[e.dypos] = ws != chain;
+      pos_deferred[e.xpos] = 0;
+    }
+    deferred.clear();
+    if (ws != chain) wg_outstanding = true;
+    return DS_OK;
+  }
+  int flush_deferred(bool final) override {
+    if (G <= 1) return DS_OK;
+    hipStream_t chain = bwd_stream ? bwd_stream : stream;
+    hipStream_t ws = wgrad_stream ? wgrad_stream : chain;
+    if (!deferred.empty()) {
+      if (ws != chain) {  // the operands the last backward pass wrote
+        DS_CHECK_HIP(hipEventRecord(ev_chain, chain));
+        DS_CHECK_HIP(hipStreamWaitEvent(ws, ev_chain, 0));
+      }
+      hipStream_t keep = stream;
+      stream = ws;
+      int rc = DS_OK;
+      const std::vector<Run> runs = make_runs(deferred);
+      for (int l = L - 1; l >= 0 && rc == DS_OK; --l) rc = layer_wgrad_runs(l, runs);
+      if (rc == DS_OK) rc = launch_pending_wgrads();
+      stream = keep;
+      if (rc != DS_OK) return rc;
+      DS_PROPAGATE(retire_deferred(ws, chain));
+    }
+    if (final && wg_outstanding) {
+      DS_CHECK_HIP(hipEventRecord(ev_wg_done, wgrad_owned));
+      DS_CHECK_HIP(hipStreamWaitEvent(chain, ev_wg_done, 0));
+      wg_outstanding = false;
+    }
+    return DS_OK;
+  }
+
   int backward(int slot, const void* d_out, void* d_in) override {
     ds_prio_scope prio(3);  // the chain every later pass waits on
-    char* sp = stash_base + (size_t)slot * slot_bytes;
+    char* sp = slot_base(slot);
+    const int pos = slot_pos[slot];
+    const int dypos = G > 1 ? (int)(n_backward % NDY) : 0;
+    if (G > 1 && dy_wg_valid[dypos]) DS_CHECK_HIP(hipStreamWaitEvent(stream, ev_dy_wg[dypos], 0));
+    // the pass that completes a group queues the group's products layer by layer as its own chain passes each layer
+    const bool closing = G > 1 && (int)deferred.size() + 1 >= G;
+    std::vector<Run> runs;
+    if (closing) {
+      std::vector<Deferred> all = deferred;
+      all.push_back({pos, dypos});
+      runs = make_runs(all);
+    }
     const float scale = 1.0f / sqrtf((float)D);
     const uint8_t* seg = has_seg[slot] ? (const uint8_t*)(sp + seg_off) : nullptr;
     const char* dy = (const char*)d_out;
@@ -612,9 +842,17 @@ struct XlnetStage : ds_stage {
       const LayerOff& t = lo[l];
       const int b = base(l);
       const int par = l & 1;
-      char* dz2 = ws_base + ws_dz2[par]; char* du = ws_base + ws_du[par]; char* dz1 = ws_base + ws_dz1[par];
-      char* dqw = ws_base + ws_dqw[par]; char* dqr = ws_base + ws_dqr[par]; char* dqs = ws_base + ws_dqs[par];
-      char* dq = ws_base + ws_dq[par]; char* dkv = ws_base + ws_dkv[par]; char* dkr = ws_base + ws_dkr[par];
+      // with deferred weight gradients their operands go to the layer's ring position of this pass
+      auto ringp = [&](size_t off, size_t per) { return dy_base + off + (size_t)dypos * per; };
+      char* dz2 = G > 1 ? ringp(ld[l].dz2, dy_act) : ws_base + ws_dz2[par];
+      char* du = G > 1 ? ringp(ld[l].du, dy_actF) : ws_base + ws_du[par];
+      char* dz1 = G > 1 ? ringp(ld[l].dz1, dy_act) : ws_base + ws_dz1[par];
+      char* dqw = G > 1 ? ringp(ld[l].dqw, dy_act) : ws_base + ws_dqw[par];
+      char* dqr = G > 1 ? ringp(ld[l].dqr, dy_act) : ws_base + ws_dqr[par];
+      char* dqs = G > 1 ? ringp(ld[l].dqs, dy_act) : ws_base + ws_dqs[par];
+      char* dq = G > 1 ? ringp(ld[l].dq, dy_act) : ws_base + ws_dq[par];
+      char* dkv = G > 1 ? ringp(ld[l].dkv, dy_kv) : ws_base + ws_dkv[par];
+      char* dkr = G > 1 ? ringp(ld[l].dkr, dy_kr) : ws_base + ws_dkr[par];
       char* deft = ws_base + ws_deft[par]; char* dbd = ws_base + ws_dbd[par];
       if (wgs) DS_PROPAGATE(lane.reuse(stream, par));
       char* x = sp + t.x;
@@ -708,12 +946,14 @@ struct XlnetStage : ds_stage {
       int rc = DS_OK;
       do {
         ds_prio_scope wprio(0);  // feeds only the master gradients
+        if (G <= 1) {
         if ((rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, F, H, rows, sp + t.hh, F, dz2, H, g[b + X_W2], H, DS_EPI_ACCUM)) != DS_OK) break;
         if ((rc = ds_colsum_accum(dtype, rows, F, du, F, g[b + X_B1], stream)) != DS_OK) break;
         if ((rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, F, rows, sp + t.y1, H, du, F, g[b + X_W1], F, DS_EPI_ACCUM)) != DS_OK) break;
         if ((rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, rows, dz1, H, sp + t.vec, H, g[b + X_O], H, DS_EPI_ACCUM)) != DS_OK) break;
+        }
         // relative biases: column sums of the three query-gradient pieces
-        {
+        if (G <= 1) {
           const void* const xs3[3] = {dqw, dqr, dqs};
           float* const out3[3] = {g[b + X_RW], g[b + X_RR], g[b + X_RS]};
           if ((rc = ds_colsum_accum_multi(dtype, rows, H, 3, xs3, H, out3, stream)) != DS_OK) break;
@@ -729,13 +969,14 @@ struct XlnetStage : ds_stage {
           if ((rc = ds_gemm(&d, stream)) != DS_OK) break;
         }
         // projections
-        if ((rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, rows, x, H, dq, H, g[b + X_Q], H, DS_EPI_ACCUM)) != DS_OK) break;
+        if (G <= 1 && (rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, rows, x, H, dq, H, g[b + X_Q], H, DS_EPI_ACCUM)) != DS_OK) break;
         for (int bb = 0; bb < B && rc == DS_OK; ++bb) {  // k_r is shared by the batch: one launch per batch entry, added in place
           const int a2 = bb > 0 ? DS_EPI_RESIDUAL : 0;
           rc = gemm_bn(DS_MN_MAJOR, DS_MN_MAJOR, R, D, S * Q, dbd + (size_t)bb * N * S * Q * R * esz, R, 0, (int64_t)S * Q * R,
                        sp + t.qr + (size_t)bb * H * esz, (int64_t)B * H, 0, D, dkr, H, 0, D, a2, dkr, 1);
         }
         if (rc != DS_OK) break;
+        if (G > 1) break;  // the rest comes from the ring, once per group
         if ((rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, R, pe, H, dkr, H, g[b + X_R], H, DS_EPI_ACCUM)) != DS_OK) break;
         // Wk and Wv: the two column halves of dkv against the same rows, one batched launch (z = 0: k, 1: v) when the two
         // master gradients sit one behind the other with no gap
@@ -745,25 +986,22 @@ struct XlnetStage : ds_stage {
           d.dtype = dtype; d.a_major = DS_MN_MAJOR; d.b_major = DS_MN_MAJOR; d.m = H; d.n = H; d.lda = H; d.ldb = 2 * H; d.ldc = H;
           d.batch = 2; d.batch_inner = 2; d.b_stride_inner = H; d.c_stride_inner = (int64_t)H * H;
           d.flags = DS_EPI_ACCUM; d.alpha = 1.f; d.c = g[b + X_K];
-          if (Mm > 0) {
-            d.k = Mm * B; d.a = sp + mem_off + (size_t)l * Mm * B * H * esz; d.b = dkv;
-            if ((rc = ds_gemm(&d, stream)) != DS_OK) break;
-          }
-          d.k = rowsS; d.a = x; d.b = dkv_h;
+          d.k = krows; d.a = sp + t.mem; d.b = dkv;   // memory rows and content rows in one reduction
           if ((rc = ds_gemm(&d, stream)) != DS_OK) break;
         } else {
-          for (int j = 0; j < 2 && rc == DS_OK; ++j) {  // j = 0: k, 1: v
-            float* gw = g[b + X_K + j];
-            if (Mm > 0)
-              rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, Mm * B, sp + mem_off + (size_t)l * Mm * B * H * esz, H, dkv + (size_t)j * H * esz,
-                        2 * H, gw, H, DS_EPI_ACCUM);
-            if (rc == DS_OK) rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, rowsS, x, H, dkv_h + (size_t)j * H * esz, 2 * H, gw, H, DS_EPI_ACCUM);
-          }
+          for (int j = 0; j < 2 && rc == DS_OK; ++j)  // j = 0: k, 1: v
+            rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, krows, sp + t.mem, H, dkv + (size_t)j * H * esz, 2 * H, g[b + X_K + j], H, DS_EPI_ACCUM);
         }
       } while (0);
+      if (wgs) {
+        stream = chain;
+        if (rc != DS_OK) return rc;
+        DS_PROPAGATE(lane.end(wgs, par));   // (the chain's next use of the parity's buffers does not wait for the group's products)
+        stream = wgs;
+      }
+      if (rc == DS_OK && closing) rc = layer_wgrad_runs(l, runs);
       stream = chain;
       if (rc != DS_OK) return rc;
-      if (wgs) DS_PROPAGATE(lane.end(wgs, par));
       // dx = dq Wq^T + dz1 (residual); the content-stream rows also receive dkv Wkv^T
       const bool first = l == 0;
       if (first && d_in == nullptr) break;
@@ -782,6 +1020,27 @@ struct XlnetStage : ds_stage {
     }
     // the stash slot and the master gradients are released to the caller in the order of `stream`
     if (wgs) DS_PROPAGATE(lane.finish(stream));
+    if (G > 1) {
+      deferred.push_back({pos, dypos});
+      pos_deferred[pos] = 1;
+      pos_owner[pos] = -1;
+      ++n_backward;
+      if (bwd_stream) {
+        DS_CHECK_HIP(hipEventRecord(ev_x_bwd[pos], stream));
+        x_bwd_valid[pos] = 1;
+      } else {
+        x_bwd_valid[pos] = 0;
+      }
+      if (closing) {
+        hipStream_t side = wgs ? wgs : stream;
+        hipStream_t chain = stream;
+        stream = side;
+        const int rc = launch_pending_wgrads();
+        stream = chain;
+        if (rc != DS_OK) return rc;
+        DS_PROPAGATE(retire_deferred(side, stream));
+      }
+    }
     return DS_OK;
   }
 };

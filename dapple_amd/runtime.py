@@ -398,11 +398,12 @@ class XlnetStage(Stage):
 
 
 def xlnet_stage(num_layers, hidden, heads, ffn, batch, seq, dtype, stash_slots, mem_len=0, streams=1, first_layer=0,
-                ln_eps=1e-14, device="cuda:0", attention="auto", residual_fp32=True):
+                ln_eps=1e-14, device="cuda:0", attention="auto", residual_fp32=True, wgrad_group=1):
     """An XLNet stage of ``num_layers`` relative-attention layers (xlnet/models/slice_xlnet.py:164-180).
     ``attention`` (``ds_xlnet_cfg.fused_attention``): "auto" = scores, relative shift and softmax as one kernel per pass where
     the shape allows; "separate" = every product and the softmax as launches of their own.  ``residual_fp32`` (bf16 stages): keep the
-    residual stream in fp32 (``ds_xlnet_cfg.residual_fp32``)."""
+    residual stream in fp32 (``ds_xlnet_cfg.residual_fp32``).  ``wgrad_group`` = G > 1 (bf16): weight gradients once per G
+    backward passes, one product per weight over all G micro-batches; call ``set_inputs`` before every forward pass then."""
     lib = _lib.load()
     cfg = XlnetCfg()
     cfg.dtype, cfg.num_layers, cfg.hidden, cfg.heads, cfg.ffn = _dtype_code(dtype), num_layers, hidden, heads, ffn
@@ -413,6 +414,7 @@ def xlnet_stage(num_layers, hidden, heads, ffn, batch, seq, dtype, stash_slots, 
         raise ValueError("attention must be one of %r" % (list(modes),))
     cfg.fused_attention = modes[attention]
     cfg.residual_fp32 = 1 if residual_fp32 else 0
+    cfg.wgrad_group = wgrad_group
     h = C.c_void_p()
     with torch.cuda.device(torch.device(device)):
         check(lib.ds_xlnet_stage_create(C.byref(cfg), _lib.current_stream(), C.byref(h)), "ds_xlnet_stage_create")

@@ -445,7 +445,12 @@ typedef struct ds_xlnet_cfg {
   int residual_fp32;   /* bf16 only, 1: the residual stream (the sums in front of both LayerNorms, the LayerNorm outputs that
                           feed the next sum, the same chain of gradients) stays in fp32, bf16 is what the GEMMs read: the
                           stream's own rounding no longer adds up over the layers (as ds_stage_cfg.residual_fp32) */
-  int reserved[6];
+  int wgrad_group;     /* G > 1 (bf16; rows, klen * batch and klen + seq multiples of 64; otherwise taken as 1): weight gradients
+                          are formed once per G backward passes, one product per weight over all G micro-batches (as
+                          ds_stage_cfg.wgrad_group: the sum tf.accumulate_n forms happens inside the matrix cores).  Master
+                          gradients are complete after ds_stage_join / ds_stage_sync; masks, segments and memories then travel
+                          with a micro-batch's stash position: ds_xlnet_stage_set_inputs before every forward pass. */
+  int reserved[5];
 } ds_xlnet_cfg;
 int ds_xlnet_stage_create(const ds_xlnet_cfg* cfg, void* stream, ds_stage** out);
 

@@ -14,7 +14,7 @@ ADT = {"fp32": torch.float32, "bf16": torch.bfloat16}
 
 
 def run_case(dtype, L, H, N, F, B, Q, Mm, S, M, K=2, seed=0, use_seg=True, mask_kind="perm", stddev=0.1, perturb=True,
-             odtype=torch.float64, overlap=False, attention="auto"):
+             odtype=torch.float64, overlap=False, attention="auto", wgrad_group=1):
     adt = ADT[dtype]
     klen = Mm + Q
     w_np = synthetic.xlnet_weights(synthetic.SEED_WEIGHT + seed, L, H, N, F, stddev=stddev, perturb=perturb)
@@ -31,7 +31,8 @@ def run_case(dtype, L, H, N, F, B, Q, Mm, S, M, K=2, seed=0, use_seg=True, mask_
     else:
         masks_np = None
 
-    stage = runtime.xlnet_stage(L, H, N, F, B, Q, dtype, stash_slots=K, mem_len=Mm, streams=S, attention=attention)
+    stage = runtime.xlnet_stage(L, H, N, F, B, Q, dtype, stash_slots=K, mem_len=Mm, streams=S, attention=attention,
+                                wgrad_group=wgrad_group)
     stage.bind(w_np)
     if overlap:
         stage.enable_overlap()     # backward passes on the handle's second stream
@@ -137,12 +138,51 @@ def test_forward_backward_overlap(dtype):
     run_case(dtype, L=2, H=64, N=4, F=128, B=2, Q=16, Mm=8, S=2, M=6, seed=3, overlap=True)
 
 
-def _run_config4(dtype, M, dy_scale=1.0, repeat_first=False, overlap=True):
+@pytest.mark.parametrize("M,G,overlap", [(4, 2, False), (4, 4, True), (6, 4, True), (8, 8, True), (3, 8, False)])
+def test_grouped_weight_gradients(M, G, overlap):
+    # ds_xlnet_cfg.wgrad_group: weight gradients once per G backward passes, one segmented product per weight over the G
+    # micro-batches' stash and ring positions (two layers' products per grouped launch); groups that fill, a short last group
+    # flushed by the join, a group larger than the step; on one stream and on three
+    run_case("bf16", L=3, H=128, N=2, F=256, B=2, Q=64, Mm=64, S=2, M=M, K=2, seed=40 + M + G, overlap=overlap, wgrad_group=G)
+
+
+def test_grouped_weight_gradients_over_steps():
+    # two steps on one handle (positions and ring wrap around), gradients zeroed in between, against the ungrouped handle
+    from dapple_amd import runtime as rt_
+    L, H, N, F, B, Q, Mm, S, M = 2, 128, 2, 256, 1, 64, 64, 2, 5
+    w_np = synthetic.xlnet_weights(synthetic.SEED_WEIGHT + 77, L, H, N, F, stddev=0.1, perturb=True)
+    xs = [dev(np.stack(x), torch.bfloat16) for x in synthetic.xlnet_stream_inputs(synthetic.SEED_INPUT + 77, M, Q, B, H, streams=S)]
+    dys = [dev(np.stack(x), torch.bfloat16) for x in synthetic.xlnet_stream_inputs(synthetic.SEED_GRAD + 77, M, Q, B, H, streams=S)]
+    masks = dev(np.stack(list(synthetic.xlnet_perm_masks(97, Q, Mm, B))[:S]))
+    mems = dev(np.stack(synthetic.xlnet_mems(57, L, Mm, B, H)), torch.bfloat16)
+    res = {}
+    for G in (1, 4):
+        st = rt_.xlnet_stage(L, H, N, F, B, Q, "bf16", stash_slots=2, mem_len=Mm, streams=S, wgrad_group=G)
+        st.bind(w_np)
+        st.enable_overlap()
+        outs = [torch.empty(S, Q, B, H, dtype=torch.bfloat16, device="cuda") for _ in range(M)]
+        dxs = [torch.empty_like(o) for o in outs]
+        run = rt_.StageRuntime(st, 0, 2, M)
+        for step in range(3):
+            st.zero_grads()
+            run.step(xs, dys, outs, dxs, before_forward=lambda slot, j: st.set_inputs(slot, masks, None, mems))
+        st.sync()
+        res[G] = ([o.float().cpu() for o in outs], [d.float().cpu() for d in dxs], {n: st.grads[n].cpu().clone() for n in st.weight_names})
+        st.close()
+    for a, b in zip(res[1][0] + res[1][1], res[4][0] + res[4][1]):
+        assert torch.equal(a, b)                     # the passes themselves do not change
+    for n in res[1][2]:
+        scale = res[1][2][n].abs().max().item()
+        if scale > 0:
+            assert (res[1][2][n] - res[4][2][n]).abs().max().item() <= 2e-3 * scale, n   # one fp32 sum order against another
+
+
+def _run_config4(dtype, M, dy_scale=1.0, repeat_first=False, overlap=True, wgrad_group=8):
     """BASELINE configs[4] at its full size (18 layers, seq 512 + memory 384, two streams) as bench.py runs it."""
     c = synthetic.CONFIGS["xlnet36_half"]
     L, H, N, F, B, Q, Mm, S = c["num_layers"], c["hidden"], c["heads"], c["ffn"], c["micro_batch"], c["seq"], c["mem_len"], c["streams"]
     adt = torch.bfloat16 if dtype == "bf16" else torch.float32
-    st = runtime.xlnet_stage(L, H, N, F, B, Q, dtype, stash_slots=2, mem_len=Mm, streams=S)
+    st = runtime.xlnet_stage(L, H, N, F, B, Q, dtype, stash_slots=2, mem_len=Mm, streams=S, wgrad_group=wgrad_group)
     st.bind(synthetic.xlnet_weights(synthetic.SEED_WEIGHT + c["index"], L, H, N, F))
     if overlap:
         st.enable_overlap()
