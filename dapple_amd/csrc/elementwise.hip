@@ -450,11 +450,13 @@ __global__ __launch_bounds__(256) void layernorm_param_grad_mixed_kernel(int row
 // The same sums without rounding: dy comes as the fp32 copy, and dx is rebuilt in fp32 from the two per-row means the
 // row kernel left (dx = rstd (dy gamma - s1 - x_hat s2)), so the results equal those of layernorm_bwd_mixed_kernel up
 // to the order of the fp32 additions.  Same block shape as layernorm_param_grad_mixed_kernel.
+// x and stats may come in segments of seg_rows rows whose starts are x_seg / st_seg elements apart (activations of several
+// micro-batches in different stash slots); dy and rowsums are always one run of rows.
 __global__ __launch_bounds__(256) void layernorm_param_grad_exact_kernel(int rows, int cols, int rows_per_block, const float* __restrict__ dy,
                                                                         const float* __restrict__ x, const float* __restrict__ gamma,
                                                                         const float* __restrict__ stats, const float* __restrict__ rowsums,
                                                                         float* __restrict__ d_gamma, float* __restrict__ d_beta,
-                                                                        float* __restrict__ d_colsum) {
+                                                                        float* __restrict__ d_colsum, int seg_rows, int64_t x_seg, int64_t st_seg) {
   __shared__ float red[3][4][64 * 8];
   const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
   const int c = (blockIdx.x * 64 + lane) * 8;
@@ -471,14 +473,18 @@ __global__ __launch_bounds__(256) void layernorm_param_grad_exact_kernel(int row
       const int rb = r + 4;
       const bool two = rb < r1;
       float a0[8], b0[8], a1[8], b1[8];
+      const int sg0 = r / seg_rows, w0 = r - sg0 * seg_rows;
+      const float* st0 = stats + sg0 * st_seg + 2 * w0;
       ln_load8(dy + (int64_t)r * cols + c, a0);
-      ln_load8(x + (int64_t)r * cols + c, b0);
-      const float mean0 = stats[2 * r], rstd0 = stats[2 * r + 1], s10 = rowsums[2 * r], s20 = rowsums[2 * r + 1];
+      ln_load8(x + sg0 * x_seg + (int64_t)w0 * cols + c, b0);
+      const float mean0 = st0[0], rstd0 = st0[1], s10 = rowsums[2 * r], s20 = rowsums[2 * r + 1];
       float mean1 = 0.f, rstd1 = 0.f, s11 = 0.f, s21 = 0.f;
       if (two) {
+        const int sg1 = rb / seg_rows, w1 = rb - sg1 * seg_rows;
+        const float* st1 = stats + sg1 * st_seg + 2 * w1;
         ln_load8(dy + (int64_t)rb * cols + c, a1);
-        ln_load8(x + (int64_t)rb * cols + c, b1);
-        mean1 = stats[2 * rb]; rstd1 = stats[2 * rb + 1]; s11 = rowsums[2 * rb]; s21 = rowsums[2 * rb + 1];
+        ln_load8(x + sg1 * x_seg + (int64_t)w1 * cols + c, b1);
+        mean1 = st1[0]; rstd1 = st1[1]; s11 = rowsums[2 * rb]; s21 = rowsums[2 * rb + 1];
       }
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
@@ -997,9 +1003,20 @@ extern "C" int ds_layernorm_bwd_mixed_rows(int rows, int cols, const float* dy, 
   return DS_OK;
 }
 
+int ds_layernorm_param_grads_exact_seg(int rows, int cols, const float* dy_copy, const float* x, const float* gamma, const float* stats,
+                                       const float* row_sums, float* d_gamma, float* d_beta, float* d_colsum, int seg_rows, int64_t x_seg,
+                                       int64_t st_seg, void* stream);
+
 extern "C" int ds_layernorm_param_grads_exact(int rows, int cols, const float* dy_copy, const float* x, const float* gamma, const float* stats,
                                               const float* row_sums, float* d_gamma, float* d_beta, float* d_colsum, void* stream) {
+  return ds_layernorm_param_grads_exact_seg(rows, cols, dy_copy, x, gamma, stats, row_sums, d_gamma, d_beta, d_colsum, rows, 0, 0, stream);
+}
+
+int ds_layernorm_param_grads_exact_seg(int rows, int cols, const float* dy_copy, const float* x, const float* gamma, const float* stats,
+                                       const float* row_sums, float* d_gamma, float* d_beta, float* d_colsum, int seg_rows, int64_t x_seg,
+                                       int64_t st_seg, void* stream) {
   DS_CHECK_ARG(rows > 0 && cols > 0 && cols % 8 == 0, "ds_layernorm_param_grads_exact: rows %d, cols %d (a multiple of 8)", rows, cols);
+  DS_CHECK_ARG(seg_rows > 0 && rows % seg_rows == 0 && x_seg % 4 == 0, "ds_layernorm_param_grads_exact: %d rows in segments of %d", rows, seg_rows);
   DS_CHECK_ARG(dy_copy && x && gamma && stats && row_sums && d_gamma && d_beta, "ds_layernorm_param_grads_exact: null pointer");
   DS_CHECK_ARG(ds_aligned16(dy_copy) && ds_aligned16(x) && ds_aligned16(gamma), "ds_layernorm_param_grads_exact: tensors must be 16-byte aligned");
   hipStream_t s = (hipStream_t)stream;
@@ -1011,7 +1028,7 @@ extern "C" int ds_layernorm_param_grads_exact(int rows, int cols, const float* d
   dim3 grid(strips, (rows + rpb - 1) / rpb);
   ds_prof_scope prof(s, "layernorm_param_grad_exact_kernel", (double)rows * cols * 8, "B");
   hipLaunchKernelGGL(layernorm_param_grad_exact_kernel, grid, dim3(256), 0, s, rows, cols, rpb, dy_copy, x, gamma, stats, row_sums, d_gamma,
-                     d_beta, d_colsum);
+                     d_beta, d_colsum, seg_rows, x_seg, st_seg);
   DS_CHECK_LAUNCH();
   return DS_OK;
 }

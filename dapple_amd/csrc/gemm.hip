@@ -841,7 +841,8 @@ int ds_gemm_make_args(const ds_gemm_desc* d, GemmArgs* out, int* batch_out) {
   (void)esz;
   if (d->k_segment != 0) {
     const int kt = d->dtype == DS_BF16 ? 64 : 32;
-    DS_CHECK_ARG(d->a_major == DS_MN_MAJOR && d->b_major == DS_MN_MAJOR, "ds_gemm: a segmented reduction needs MN-major A and B");
+    // (a K-major operand runs on along its rows whatever the segments: its segment stride is not used)
+    DS_CHECK_ARG(d->a_major == DS_MN_MAJOR || d->b_major == DS_MN_MAJOR, "ds_gemm: a segmented reduction needs an MN-major operand");
     DS_CHECK_ARG(d->k_segment > 0 && d->k_segment % kt == 0 && d->k % d->k_segment == 0,
                  "ds_gemm: k_segment %d must be a multiple of %d that divides k = %d", d->k_segment, kt, d->k);
     DS_CHECK_ARG(d->a_segment_stride % vec == 0 && d->b_segment_stride % vec == 0, "ds_gemm: segment strides must be multiples of %d", vec);

@@ -163,5 +163,9 @@ int ds_rank_update(int rows, int cols, int ns, const float* a, const float* b, f
 // `count` such updates of one shape in one launch (no two of them on the same w)
 int ds_rank_update_multi(int count, int rows, int cols, int ns, const float* const* as, const float* const* bs, float* const* ws, int64_t ldw,
                          float* const* vs, void* stream);
+// ds_layernorm_param_grads_exact with x and stats in segments of seg_rows rows, x_seg / st_seg elements apart
+int ds_layernorm_param_grads_exact_seg(int rows, int cols, const float* dy_copy, const float* x, const float* gamma, const float* stats,
+                                       const float* row_sums, float* d_gamma, float* d_beta, float* d_colsum, int seg_rows, int64_t x_seg,
+                                       int64_t st_seg, void* stream);
 // ds_colsum_accum for up to 4 matrices of one shape in one launch
 int ds_colsum_accum_multi(int dtype, int rows, int cols, int count, const void* const* xs, int64_t ldx, float* const* outs, void* stream);

@@ -237,10 +237,10 @@ struct XlnetStage : ds_stage {
   // position / one ring position apart), the products of two layers as one grouped launch.  There are then more stash
   // positions than slots (slots + G, rounded up to a multiple of G), handed out round-robin in forward order.
   int G = 1, KP = 0, NDY = 0;
-  struct LayerDy { size_t dz2, du, dz1, dq, dqw, dqr, dqs, dkv, dkr; };
+  struct LayerDy { size_t dz2, du, dz1, dq, dqw, dqr, dqs, dkv, dbd, deft, dkr, dyn2, dyn1, rs2, rs1; };  // (deft: [heads * 2][2G * rows]; dkr: one per layer)
   std::vector<LayerDy> ld;
   char* dy_base = nullptr;
-  size_t dy_act = 0, dy_actF = 0, dy_kv = 0, dy_kr = 0;
+  size_t dy_act = 0, dy_actF = 0, dy_kv = 0, dy_bd = 0;
   struct Deferred { int xpos, dypos; };
   struct Run { int xpos, dypos, n; };
   std::vector<Deferred> deferred;
@@ -347,14 +347,21 @@ struct XlnetStage : ds_stage {
       pos_owner.assign(KP, -1);
       pos_deferred.assign(KP, 0);
       Arena da;
-      dy_act = act; dy_actF = actF; dy_kv = (size_t)krows * 2 * H * esz; dy_kr = (size_t)R * H * esz;
+      dy_act = act; dy_actF = actF; dy_kv = (size_t)krows * 2 * H * esz; dy_bd = (size_t)B * N * S * Q * R * esz;
       ld.resize(L);
       for (int l = 0; l < L; ++l) {
         ld[l].dz2 = da.reserve(dy_act * NDY); ld[l].du = da.reserve(dy_actF * NDY); ld[l].dz1 = da.reserve(dy_act * NDY);
         ld[l].dq = da.reserve(dy_act * NDY); ld[l].dqw = da.reserve(dy_act * NDY); ld[l].dqr = da.reserve(dy_act * NDY);
-        ld[l].dqs = da.reserve(dy_act * NDY); ld[l].dkv = da.reserve(dy_kv * NDY); ld[l].dkr = da.reserve(dy_kr * NDY);
+        ld[l].dqs = da.reserve(dy_act * NDY); ld[l].dkv = da.reserve(dy_kv * NDY); ld[l].dbd = da.reserve(dy_bd * NDY);
+        ld[l].deft = da.reserve((size_t)N * 2 * rows * esz * NDY); ld[l].dkr = da.reserve((size_t)R * H * esz);
+        if (rs32) {  // the fp32 gradients entering the two LayerNorms and two sums per row: their parameter gradients are formed per group
+          ld[l].dyn2 = da.reserve((size_t)rows * H * 4 * NDY); ld[l].dyn1 = da.reserve((size_t)rows * H * 4 * NDY);
+          ld[l].rs2 = da.reserve((size_t)rows * 8 * NDY); ld[l].rs1 = da.reserve((size_t)rows * 8 * NDY);
+        }
       }
       DS_CHECK_HIP(hipMalloc((void**)&dy_base, da.used));
+      // the un-shifted score gradients are zero outside the band the score-gradient kernel writes, in every ring position
+      for (int l = 0; l < L; ++l) DS_CHECK_HIP(hipMemsetAsync(dy_base + ld[l].dbd, 0, dy_bd * NDY, stream));
       ev_x_bwd.assign(KP, nullptr); ev_x_wg.assign(KP, nullptr); ev_dy_wg.assign(NDY, nullptr);
       for (int i = 0; i < KP; ++i) {
         DS_CHECK_HIP(hipEventCreateWithFlags(&ev_x_bwd[i], hipEventDisableTiming));
@@ -725,7 +732,29 @@ struct XlnetStage : ds_stage {
       const char* sp0 = stash_base + (size_t)r.xpos * slot_bytes;
       const char* dz2 = dy_base + ld[l].dz2 + r.dypos * dy_act; const char* du = dy_base + ld[l].du + r.dypos * dy_actF;
       const char* dz1 = dy_base + ld[l].dz1 + r.dypos * dy_act; const char* dq = dy_base + ld[l].dq + r.dypos * dy_act;
-      const char* dkv = dy_base + ld[l].dkv + r.dypos * dy_kv; const char* dkr = dy_base + ld[l].dkr + r.dypos * dy_kr;
+      const char* dkv = dy_base + ld[l].dkv + r.dypos * dy_kv;
+      char* dkr = dy_base + ld[l].dkr;
+      const int QQ = S * Q;
+      // dk_r = sum over micro-batches and samples of dbd^T (q + r_r), per head: k_r is shared by the batch, so one launch per
+      // batch entry, added in place (launched before the grouped products: W_r's needs it)
+      for (int bb = 0; bb < B; ++bb) {
+        ds_gemm_desc d = desc_bn(DS_MN_MAJOR, DS_MN_MAJOR, R, D, QQ * r.n, dy_base + ld[l].dbd + r.dypos * dy_bd + (size_t)bb * N * QQ * R * esz, R, 0,
+                                 (int64_t)QQ * R, sp0 + t.qr + (size_t)bb * H * esz, (int64_t)B * H, 0, D, dkr, H, 0, D,
+                                 bb > 0 ? DS_EPI_RESIDUAL : 0, dkr, 1);
+        if (r.n > 1) { d.k_segment = QQ; d.a_segment_stride = (int64_t)(dy_bd / esz); d.b_segment_stride = sstride; }
+        DS_PROPAGATE(ds_gemm(&d, stream));
+      }
+      // seg_emb[s][n][:] += sum_rows def[row][n][s] * qs[row][n][:]   (batched over heads; the run's rows are contiguous in deft)
+      {
+        ds_gemm_desc d;
+        memset(&d, 0, sizeof(d));
+        d.dtype = dtype; d.a_major = DS_K_MAJOR; d.b_major = DS_MN_MAJOR; d.m = 2; d.n = D; d.k = rows * r.n;
+        d.lda = (int64_t)NDY * rows; d.ldb = H; d.ldc = H; d.batch = N; d.batch_inner = N;
+        d.a_stride_inner = (int64_t)2 * NDY * rows; d.b_stride_inner = D; d.c_stride_inner = D;
+        d.flags = DS_EPI_ACCUM; d.alpha = 1.f; d.a = dy_base + ld[l].deft + (size_t)r.dypos * rows * esz; d.b = sp0 + t.qs; d.c = g[b + X_SEG];
+        if (r.n > 1) { d.k_segment = rows; d.b_segment_stride = sstride; }
+        DS_PROPAGATE(ds_gemm(&d, stream));
+      }
       ds_gemm_desc ds[7];
       int nd = 0;
       auto wg = [&](int m, int n, int kseg, const void* a, int64_t lda, int64_t aseg, const void* bb, int64_t ldb, int64_t bseg, float* c,
@@ -741,7 +770,7 @@ struct XlnetStage : ds_stage {
       wg(H, F, rows, sp0 + t.y1, H, sstride, du, F, (int64_t)rows * F, g[b + X_W1], F);
       wg(H, H, rows, dz1, H, (int64_t)rows * H, sp0 + t.vec, H, sstride, g[b + X_O], H);
       wg(H, H, rows, sp0 + t.x, H, sstride, dq, H, (int64_t)rows * H, g[b + X_Q], H);
-      wg(H, H, R, pe, H, 0, dkr, H, (int64_t)R * H, g[b + X_R], H);   // every micro-batch against the same position table
+      { ds_gemm_desc& d = wg(H, H, R, pe, H, 0, dkr, H, 0, g[b + X_R], H); d.k = R; d.k_segment = 0; }   // dk_r already holds the run's sum
       if (kv_adjacent) {  // k and v: the two column halves of dkv, batched (z = 0: k, 1: v)
         ds_gemm_desc& d = wg(H, H, krows, sp0 + t.mem, H, sstride, dkv, 2 * H, (int64_t)krows * 2 * H, g[b + X_K], H);
         d.batch = 2; d.batch_inner = 2; d.b_stride_inner = H; d.c_stride_inner = (int64_t)H * H;
@@ -762,6 +791,16 @@ struct XlnetStage : ds_stage {
       }
       if (runs.size() > 1 || wg_pending.size() + nd > (size_t)DS_GROUP_MAX_TASKS) DS_PROPAGATE(launch_pending_wgrads());
       DS_PROPAGATE(ds_colsum_accum(dtype, rows * r.n, F, du, F, g[b + X_B1], stream));
+      if (rs32) {
+        const size_t a32 = (size_t)rows * H * 4, r8 = (size_t)rows * 8;
+        const int64_t s4 = (int64_t)(slot_bytes / 4);
+        DS_PROPAGATE(ds_layernorm_param_grads_exact_seg(rows * r.n, H, (const float*)(dy_base + ld[l].dyn2 + r.dypos * a32), (const float*)(sp0 + t.z2),
+                                                        w[b + X_LN2_G], (const float*)(sp0 + t.st2), (const float*)(dy_base + ld[l].rs2 + r.dypos * r8),
+                                                        g[b + X_LN2_G], g[b + X_LN2_B], g[b + X_B2], rows, s4, s4, stream));
+        DS_PROPAGATE(ds_layernorm_param_grads_exact_seg(rows * r.n, H, (const float*)(dy_base + ld[l].dyn1 + r.dypos * a32), (const float*)(sp0 + t.z1),
+                                                        w[b + X_LN1_G], (const float*)(sp0 + t.st1), (const float*)(dy_base + ld[l].rs1 + r.dypos * r8),
+                                                        g[b + X_LN1_G], g[b + X_LN1_B], nullptr, rows, s4, s4, stream));
+      }
       const void* const xs3[3] = {dy_base + ld[l].dqw + r.dypos * dy_act, dy_base + ld[l].dqr + r.dypos * dy_act, dy_base + ld[l].dqs + r.dypos * dy_act};
       float* const out3[3] = {g[b + X_RW], g[b + X_RR], g[b + X_RS]};
       DS_PROPAGATE(ds_colsum_accum_multi(dtype, rows * r.n, H, 3, xs3, H, out3, stream));
@@ -852,14 +891,25 @@ struct XlnetStage : ds_stage {
       char* dqs = G > 1 ? ringp(ld[l].dqs, dy_act) : ws_base + ws_dqs[par];
       char* dq = G > 1 ? ringp(ld[l].dq, dy_act) : ws_base + ws_dq[par];
       char* dkv = G > 1 ? ringp(ld[l].dkv, dy_kv) : ws_base + ws_dkv[par];
-      char* dkr = G > 1 ? ringp(ld[l].dkr, dy_kr) : ws_base + ws_dkr[par];
-      char* deft = ws_base + ws_deft[par]; char* dbd = ws_base + ws_dbd[par];
-      if (wgs) DS_PROPAGATE(lane.reuse(stream, par));
+      char* dkr = ws_base + ws_dkr[par];
+      char* deft = G > 1 ? dy_base + ld[l].deft + (size_t)dypos * rows * esz : ws_base + ws_deft[par];
+      const int64_t deft_ld = G > 1 ? (int64_t)NDY * rows : (int64_t)rows;
+      char* dbd = G > 1 ? ringp(ld[l].dbd, dy_bd) : ws_base + ws_dbd[par];
+      if (wgs && G <= 1) DS_PROPAGATE(lane.reuse(stream, par));
       char* x = sp + t.x;
       float* dz2f = (float*)(ws_base + bw_dz2f);
       float* dy1f = (float*)(ws_base + bw_dy1f);
       float* dz1f = (float*)(ws_base + bw_dz1f);
-      if (rs32) {
+      if (rs32 && G > 1) {
+        // rows only on the chain (no atomics); gamma / beta / bias gradients come from the fp32 copy and the row sums, per group
+        const size_t a32 = (size_t)rows * H * 4, r8 = (size_t)rows * 8;
+        DS_PROPAGATE(ds_layernorm_bwd_mixed_rows(rows, H, dyf, (const float*)(sp + t.z2), w[b + X_LN2_G], (const float*)(sp + t.st2), dz2, dz2f,
+                                                 (float*)(dy_base + ld[l].dyn2 + dypos * a32), (float*)(dy_base + ld[l].rs2 + dypos * r8), stream));
+        DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rows, F, H, dz2, H, WT(l, X_W2), H, du, F, DS_EPI_DGELU | DS_EPI_TANH_FORM, nullptr, nullptr, sp + t.u));
+        DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rows, H, F, du, F, WT(l, X_W1), F, dy1f, H, res32, nullptr, dz2f));
+        DS_PROPAGATE(ds_layernorm_bwd_mixed_rows(rows, H, dy1f, (const float*)(sp + t.z1), w[b + X_LN1_G], (const float*)(sp + t.st1), dz1, dz1f,
+                                                 (float*)(dy_base + ld[l].dyn1 + dypos * a32), (float*)(dy_base + ld[l].rs1 + dypos * r8), stream));
+      } else if (rs32) {
         DS_PROPAGATE(ds_layernorm_bwd_mixed(rows, H, dyf, (const float*)(sp + t.z2), w[b + X_LN2_G], (const float*)(sp + t.st2), dz2, dz2f,
                                             nullptr, g[b + X_LN2_G], g[b + X_LN2_B], g[b + X_B2], stream));
         DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rows, F, H, dz2, H, WT(l, X_W2), H, du, F, DS_EPI_DGELU | DS_EPI_TANH_FORM, nullptr, nullptr, sp + t.u));
@@ -928,10 +978,10 @@ struct XlnetStage : ds_stage {
           const int64_t waves = (int64_t)B * N * QQ;
           dim3 grid((unsigned)((waves + 3) / 4));
           if (dtype == DS_BF16)
-            hipLaunchKernelGGL(xl_seg_bwd_kernel<bf16>, grid, dim3(256), 0, stream, QQ, B, N, D, (int64_t)rows, defs, w[b + X_SEG],
+            hipLaunchKernelGGL(xl_seg_bwd_kernel<bf16>, grid, dim3(256), 0, stream, QQ, B, N, D, deft_ld, defs, w[b + X_SEG],
                                (const bf16*)dqw, (const bf16*)dqr, (bf16*)dqs, (bf16*)dq, (bf16*)deft);
           else
-            hipLaunchKernelGGL(xl_seg_bwd_kernel<float>, grid, dim3(256), 0, stream, QQ, B, N, D, (int64_t)rows, defs, w[b + X_SEG],
+            hipLaunchKernelGGL(xl_seg_bwd_kernel<float>, grid, dim3(256), 0, stream, QQ, B, N, D, deft_ld, defs, w[b + X_SEG],
                                (const float*)dqw, (const float*)dqr, (float*)dqs, (float*)dq, (float*)deft);
           DS_CHECK_LAUNCH();
         }
@@ -939,21 +989,21 @@ struct XlnetStage : ds_stage {
       // ---- weight gradients of this layer (on the weight-gradient stream when there is one)
       const char* dkv_h = dkv + (size_t)Mm * B * 2 * H * esz;
       hipStream_t chain = stream;
-      if (wgs) {
+      if (wgs && (G <= 1 || closing)) {
         DS_PROPAGATE(lane.begin(chain, wgs, par));
         stream = wgs;  // gemm() and the column sums below launch on `stream`
       }
       int rc = DS_OK;
-      do {
+      if (G <= 1) do {
         ds_prio_scope wprio(0);  // feeds only the master gradients
-        if (G <= 1) {
+        {
         if ((rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, F, H, rows, sp + t.hh, F, dz2, H, g[b + X_W2], H, DS_EPI_ACCUM)) != DS_OK) break;
         if ((rc = ds_colsum_accum(dtype, rows, F, du, F, g[b + X_B1], stream)) != DS_OK) break;
         if ((rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, F, rows, sp + t.y1, H, du, F, g[b + X_W1], F, DS_EPI_ACCUM)) != DS_OK) break;
         if ((rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, rows, dz1, H, sp + t.vec, H, g[b + X_O], H, DS_EPI_ACCUM)) != DS_OK) break;
         }
         // relative biases: column sums of the three query-gradient pieces
-        if (G <= 1) {
+        {
           const void* const xs3[3] = {dqw, dqr, dqs};
           float* const out3[3] = {g[b + X_RW], g[b + X_RR], g[b + X_RS]};
           if ((rc = ds_colsum_accum_multi(dtype, rows, H, 3, xs3, H, out3, stream)) != DS_OK) break;
@@ -969,14 +1019,13 @@ struct XlnetStage : ds_stage {
           if ((rc = ds_gemm(&d, stream)) != DS_OK) break;
         }
         // projections
-        if (G <= 1 && (rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, rows, x, H, dq, H, g[b + X_Q], H, DS_EPI_ACCUM)) != DS_OK) break;
+        if ((rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, rows, x, H, dq, H, g[b + X_Q], H, DS_EPI_ACCUM)) != DS_OK) break;
         for (int bb = 0; bb < B && rc == DS_OK; ++bb) {  // k_r is shared by the batch: one launch per batch entry, added in place
           const int a2 = bb > 0 ? DS_EPI_RESIDUAL : 0;
           rc = gemm_bn(DS_MN_MAJOR, DS_MN_MAJOR, R, D, S * Q, dbd + (size_t)bb * N * S * Q * R * esz, R, 0, (int64_t)S * Q * R,
                        sp + t.qr + (size_t)bb * H * esz, (int64_t)B * H, 0, D, dkr, H, 0, D, a2, dkr, 1);
         }
         if (rc != DS_OK) break;
-        if (G > 1) break;  // the rest comes from the ring, once per group
         if ((rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, R, pe, H, dkr, H, g[b + X_R], H, DS_EPI_ACCUM)) != DS_OK) break;
         // Wk and Wv: the two column halves of dkv against the same rows, one batched launch (z = 0: k, 1: v) when the two
         // master gradients sit one behind the other with no gap
@@ -993,13 +1042,14 @@ struct XlnetStage : ds_stage {
             rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, krows, sp + t.mem, H, dkv + (size_t)j * H * esz, 2 * H, g[b + X_K + j], H, DS_EPI_ACCUM);
         }
       } while (0);
-      if (wgs) {
+      if (wgs && G <= 1) {
         stream = chain;
         if (rc != DS_OK) return rc;
-        DS_PROPAGATE(lane.end(wgs, par));   // (the chain's next use of the parity's buffers does not wait for the group's products)
-        stream = wgs;
+        DS_PROPAGATE(lane.end(wgs, par));
       }
-      if (rc == DS_OK && closing) rc = layer_wgrad_runs(l, runs);
+      // deferred weight gradients: nothing per pass; the pass that completes a group queues the group's work for this layer,
+      // behind what the chain has just left in the ring
+      if (closing) rc = layer_wgrad_runs(l, runs);
       stream = chain;
       if (rc != DS_OK) return rc;
       // dx = dq Wq^T + dz1 (residual); the content-stream rows also receive dkv Wkv^T

@@ -77,11 +77,11 @@ def _check_gemm_operands(a, b, c, m, n, k, a_major, b_major, lda, ldb, ldc, flag
     def extent(rows, cols, ld, strides):   # batch entry z sits at (z // inner) * strides[0] + (z % inner) * strides[1]
         return (rows - 1) * ld + cols + (batch // inner - 1) * abs(strides[0]) + (inner - 1) * abs(strides[1])
     if k_segment:
-        if a_major != DS_MN_MAJOR or b_major != DS_MN_MAJOR or k_segment <= 0 or k % k_segment or a_segment_stride < 0 or b_segment_stride < 0:
-            raise ValueError("a segmented reduction needs MN-major operands, k_segment dividing k and non-negative segment strides")
+        if (a_major != DS_MN_MAJOR and b_major != DS_MN_MAJOR) or k_segment <= 0 or k % k_segment or a_segment_stride < 0 or b_segment_stride < 0:
+            raise ValueError("a segmented reduction needs an MN-major operand, k_segment dividing k and non-negative segment strides")
         nseg = k // k_segment
-        need_a = extent(k_segment, m, lda, a_strides) + (nseg - 1) * a_segment_stride
-        need_b = extent(k_segment, n, ldb, b_strides) + (nseg - 1) * b_segment_stride
+        need_a = extent(m, k, lda, a_strides) if a_major == DS_K_MAJOR else extent(k_segment, m, lda, a_strides) + (nseg - 1) * a_segment_stride
+        need_b = extent(n, k, ldb, b_strides) if b_major == DS_K_MAJOR else extent(k_segment, n, ldb, b_strides) + (nseg - 1) * b_segment_stride
     else:
         need_a = extent(m, k, lda, a_strides) if a_major == DS_K_MAJOR else extent(k, m, lda, a_strides)
         need_b = extent(n, k, ldb, b_strides) if b_major == DS_K_MAJOR else extent(k, n, ldb, b_strides)

@@ -99,9 +99,10 @@ typedef struct ds_gemm_desc {
   void* c2;             /* DS_EPI_GELU second output / DS_EPI_DGELU aux input, layout of C */
   void* workspace;      /* optional device scratch for split-K (NULL: never split), see ds_gemm_workspace_bytes */
   size_t workspace_bytes;
-  /* Segmented reduction (0: none).  With MN-major A and B the k index may run over k / k_segment segments of k_segment
+  /* Segmented reduction (0: none).  For an MN-major operand the k index may run over k / k_segment segments of k_segment
    * rows each: rows inside a segment are lda / ldb apart as usual, segment s starts a_segment_stride / b_segment_stride
-   * elements behind segment s - 1 (a stride of 0 reads the same rows for every segment).  This is how ONE weight-gradient
+   * elements behind segment s - 1 (a stride of 0 reads the same rows for every segment); a K-major operand beside it runs
+   * on along its rows and its stride is ignored; at least one operand must be MN-major.  This is how ONE weight-gradient
    * product X^T dY sums over several micro-batches whose activations sit in different stash slots
    * (tf.accumulate_n over the micro-batches, bert/graph.py:145-161).  k_segment must be a multiple of 64 (bf16) or 32 (fp32). */
   int k_segment;

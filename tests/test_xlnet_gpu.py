@@ -174,7 +174,10 @@ def test_grouped_weight_gradients_over_steps():
     for n in res[1][2]:
         scale = res[1][2][n].abs().max().item()
         if scale > 0:
-            assert (res[1][2][n] - res[4][2][n]).abs().max().item() <= 2e-3 * scale, n   # one fp32 sum order against another
+            # one fp32 sum order against another; W_r's gradient goes through dk_r, which the ungrouped handle rounds to bf16
+            # once per pass and the grouped one once per group
+            bar = 8e-3 if n.endswith("/r") else 2e-3
+            assert (res[1][2][n] - res[4][2][n]).abs().max().item() <= bar * scale, n
 
 
 def _run_config4(dtype, M, dy_scale=1.0, repeat_first=False, overlap=True, wgrad_group=8):
