@@ -617,8 +617,22 @@ struct XlnetStage : ds_stage {
       char* y = (l + 1 < L) ? sp + lo[l + 1].x : (char*)out;
       DS_PROPAGATE(await_cast(l, stream));
       // q for every stream row; k|v for memory rows and for the content-stream rows
+      // The two projections do not depend on each other: one grouped launch of 128 x 128 tiles (64 + 112 of them at the
+      // XLNet-36 shape) instead of two launches of 64 x 64 tiles, 1 % of the step.  DS_XL_GROUP_QKV = -1: two launches; 0..5: tile shape.
+      static const char* env_qkv = getenv("DS_XL_GROUP_QKV");
+      const int qkv_cfg = env_qkv ? atoi(env_qkv) : 2;
+      if (qkv_cfg >= 0 && dtype == DS_BF16 && H % 64 == 0 && H > 256) {
+        GroupOp ops[2];
+        for (GroupOp& o : ops) { o.kind = GOP_GEMM; o.cfg = qkv_cfg; o.prio = ds_launch_prio; memset(&o.gemm, 0, sizeof(o.gemm)); }
+        ds_gemm_desc& dq_ = ops[1].gemm; ds_gemm_desc& dk_ = ops[0].gemm;
+        dq_.dtype = dtype; dq_.a_major = DS_K_MAJOR; dq_.b_major = DS_MN_MAJOR; dq_.m = rows; dq_.n = H; dq_.k = H; dq_.lda = H; dq_.ldb = H; dq_.ldc = H;
+        dq_.batch = 1; dq_.batch_inner = 1; dq_.alpha = 1.f; dq_.a = x; dq_.b = WT(l, X_Q); dq_.c = qall;
+        dk_ = dq_; dk_.m = krows; dk_.n = 2 * H; dk_.ldb = 2 * H; dk_.ldc = 2 * H; dk_.a = sp + t.mem; dk_.b = wkv[l]; dk_.c = sp + t.kv;
+        DS_PROPAGATE(ds_group_launch(ops, 2, stream));
+      } else {
       DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, rows, H, H, x, H, WT(l, X_Q), H, qall, H));
       DS_PROPAGATE(gemm(DS_K_MAJOR, DS_MN_MAJOR, krows, 2 * H, H, sp + t.mem, H, wkv[l], 2 * H, sp + t.kv, 2 * H));
+      }
       {
         const int64_t total = (int64_t)rows * H;
         if (score_fused)
