@@ -108,6 +108,20 @@ PROTOTYPES = {
     "ds_vgg_head": (C.c_int, [C.c_int] * 4 + [C.c_void_p] * 8 + [C.c_int, C.c_float] + [C.c_void_p] * 10 + [C.c_size_t, C.c_void_p]),
     "ds_pooler": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "ds_stage_release_slot": (C.c_int, [C.c_void_p, C.c_int]),
+    "ds_relu_fwd": (C.c_int, [C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "ds_relu_bwd": (C.c_int, [C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
+    "ds_add": (C.c_int, [C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "ds_copy2d": (C.c_int, [C.c_int64, C.c_int, C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_int, C.c_void_p]),
+    "ds_batchnorm_workspace_bytes": (C.c_size_t, [C.c_int]),
+    "ds_batchnorm_train_fwd": (C.c_int, [C.c_int64, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_float] + [C.c_void_p] * 5 +
+                               [C.c_float, C.c_void_p, C.c_void_p]),
+    "ds_batchnorm_train_bwd": (C.c_int, [C.c_int64, C.c_int] + [C.c_void_p] * 6 + [C.c_int] + [C.c_void_p] * 4),
+    "ds_pool3x3_fwd": (C.c_int, [C.c_int] * 5 + [C.c_void_p] * 3),
+    "ds_pool3x3_bwd": (C.c_int, [C.c_int] * 5 + [C.c_void_p] * 3 + [C.c_int, C.c_void_p]),
+    "ds_depthwise_conv_fwd": (C.c_int, [C.c_int] * 5 + [C.c_void_p] * 4),
+    "ds_depthwise_conv_bwd": (C.c_int, [C.c_int] * 5 + [C.c_void_p] * 4 + [C.c_int, C.c_void_p, C.c_void_p]),
+    "ds_gather1d": (C.c_int, [C.c_int] * 6 + [C.c_void_p] * 3),
+    "ds_scatter1d": (C.c_int, [C.c_int] * 6 + [C.c_void_p] * 2 + [C.c_int, C.c_void_p]),
     "ds_lstm_cell_fwd": (C.c_int, [C.c_int, C.c_int, C.c_float] + [C.c_void_p] * 7),
     "ds_lstm_cell_bwd": (C.c_int, [C.c_int, C.c_int] + [C.c_void_p] * 5 + [C.c_int, C.c_void_p, C.c_void_p]),
     "ds_layernorm_fwd": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_float,

@@ -531,9 +531,13 @@ def calc_reduction_layers(num_cells, num_reduction_layers):
 
 
 class BaseCell(object):
-    """network_utils_slice.py:294-313: a NAS cell cut by the pipeline at ``cell_3``/``cell_7`` with two boundary
-    tensors (``cut_outputs``).  Shape of the interface only: no BASELINE config exercises AmoebaNet and its
-    kernels (separable / dilated conv, batch norm) are not built."""
+    """network_utils_slice.py:294-428: a NAS cell, cut by the pipeline inside ``cell_3`` (6 cells) / ``cell_7`` (12 cells) with
+    two boundary tensors (``cut_outputs``, :335, :365).  Normal cells (stride 1) run on the GPU through ``dapple_amd.amoeba``:
+    separable, 1 x k / k x 1 and 1 x 1 convolutions, 3 x 3 average / max pooling, train-mode batch normalisation, the sums of
+    the five combinations and the concatenation of the unused states.  TensorFlow keeps a cell's variables in its variable
+    scope; here they are handed over with ``bind`` (names as in ``amoeba.cell_variable_shapes``).  Not built: reduction
+    cells (stride 2, ``factorized_reduction``), dilated convolutions, drop path with a keep probability below 1 (the
+    driver's default is 1.0, amoeba-dapple.py:128)."""
 
     def __init__(self, num_conv_filters, operations, used_hiddenstates, hiddenstate_indices, drop_path_keep_prob,
                  total_num_cells, drop_path_burn_in_steps, dep_outputs=None):
@@ -542,11 +546,42 @@ class BaseCell(object):
         self._drop_path_keep_prob, self._total_num_cells = drop_path_keep_prob, total_num_cells
         self._drop_path_burn_in_steps, self._dep_outputs = drop_path_burn_in_steps, dep_outputs
         self.cut_outputs = []
+        # total_num_cells counts the two reduction cells (:580-581); FLAGS.num_cells 6 / 12 put the cut in cell_3 / cell_7 (:309-312)
+        self.cut_cell_name = {6: "cell_3", 12: "cell_7"}.get(total_num_cells - 2, "")
+        self._variables, self._gradients, self._cells = None, None, []
+
+    def bind(self, variables, gradients=None):
+        """``variables`` / ``gradients``: name -> fp32 tensor on the GPU; gradients are added to in place by ``backward``."""
+        self._variables, self._gradients = variables, gradients
+        return self
 
     def __call__(self, net, scope=None, filter_scaling=1, stride=1, prev_layer=None, cell_num=-1):
-        raise NotImplementedError("AmoebaNet cells are not built: none of the measured configurations runs them")
+        from . import amoeba
+        if self._variables is None:
+            raise RuntimeError("BaseCell: bind(variables) before the first call")
+        if stride != 1:
+            raise NotImplementedError("reduction cells (stride %d) are not built" % stride)
+        if self._drop_path_keep_prob < 1.0:
+            raise NotImplementedError("drop path with a keep probability below 1 draws from TensorFlow's generator and is not built")
+        self._cell_num, self._filter_scaling = cell_num, filter_scaling
+        self._filter_size = int(self._num_conv_filters * filter_scaling)
+        cell = amoeba.Cell(scope, self._filter_size, self._operations, self._hiddenstate_indices, self._used_hiddenstates,
+                           self._variables, self._gradients)
+        out = cell.forward(net, prev_layer)
+        if scope == self.cut_cell_name:
+            self.cut_outputs.extend(cell.cut_outputs)
+        self._cells.append(cell)
+        return out
+
+    def backward(self, d_out):
+        """Backward pass of the latest call not yet walked back: -> (d_net, d_prev_layer or None)."""
+        if not self._cells:
+            raise RuntimeError("BaseCell.backward without a forward call")
+        return self._cells.pop().backward(d_out)
 
 
 def build_network(inputs, num_classes, is_training=True, hparams=None, dep_outputs=None):
-    """model_builder_slice.py:292-345 (signature only)."""
-    raise NotImplementedError("AmoebaNet is an interface shell in this runtime: none of the measured configurations runs it")
+    """model_builder_slice.py:292-345 (signature only): the stem, the reduction cells and the classifier around the cells are
+    not built - ``BaseCell`` runs single normal cells."""
+    raise NotImplementedError("the AmoebaNet network around the cells (stem, reduction cells, classifier) is not built: "
+                              "BaseCell runs single normal cells; none of the measured configurations runs the network")

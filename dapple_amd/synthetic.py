@@ -306,3 +306,38 @@ def gnmt_attention_weights(seed, units, vocab, init_weight=0.1, perturb=False):
             A + "bahdanau_attention/attention_v": u(units),
             A + "bahdanau_attention/attention_g": np.array([np.sqrt(1.0 / units) * (1.3 if perturb else 1.0)], np.float32),
             A + "bahdanau_attention/attention_b": u(units) if perturb else np.zeros(units, np.float32)}
+
+
+# ---- AmoebaNet cells (amoeba_net/model_specs.py:22-87: normal cells of the four published networks)
+AMOEBA_NORMAL_CELLS = {
+    "amoeba_net_a": (["avg_pool_3x3", "max_pool_3x3", "separable_3x3_2", "none", "none", "avg_pool_3x3", "separable_3x3_2",
+                      "separable_5x5_2", "avg_pool_3x3", "separable_3x3_2"], [0, 0, 1, 1, 0, 1, 0, 2, 5, 0], [1, 0, 1, 0, 0, 1, 0]),
+    "amoeba_net_b": (["1x1", "max_pool_3x3", "none", "separable_3x3_2", "1x1", "separable_3x3_2", "1x1", "none", "avg_pool_3x3",
+                      "1x1"], [1, 1, 1, 0, 1, 0, 2, 2, 1, 5], [0, 1, 1, 0, 0, 1, 0]),
+    "amoeba_net_c": (["avg_pool_3x3", "separable_3x3_2", "none", "separable_3x3_2", "avg_pool_3x3", "separable_3x3_2", "none",
+                      "separable_3x3_2", "avg_pool_3x3", "separable_3x3_2"], [0, 0, 0, 0, 2, 1, 0, 1, 3, 0], [1, 0, 0, 1, 0, 0, 0]),
+    "amoeba_net_d": (["1x1", "max_pool_3x3", "none", "1x7_7x1", "1x1", "1x7_7x1", "max_pool_3x3", "none", "avg_pool_3x3", "1x1"],
+                     [1, 1, 1, 0, 0, 0, 2, 2, 1, 5], [0, 1, 1, 0, 0, 1, 0]),
+}
+
+
+def amoeba_cell_weights(seed, shapes, perturb=True):
+    """name -> fp32 array for the shapes of ``dapple_amd.amoeba.cell_variable_shapes``: kernels from a variance-scaling normal
+    (fan-out), gamma = 1, beta = 0 (perturbed on request so their gradients are exercised), moving statistics at their
+    initial 0 / 1."""
+    rng = _rng(seed)
+    w = {}
+    for name in sorted(shapes):
+        shp = shapes[name]
+        if name.endswith("gamma"):
+            w[name] = (1 + 0.2 * rng.standard_normal(shp)).astype(np.float32) if perturb else np.ones(shp, np.float32)
+        elif name.endswith("beta"):
+            w[name] = (0.2 * rng.standard_normal(shp)).astype(np.float32) if perturb else np.zeros(shp, np.float32)
+        elif name.endswith("moving_mean"):
+            w[name] = np.zeros(shp, np.float32)
+        elif name.endswith("moving_variance"):
+            w[name] = np.ones(shp, np.float32)
+        else:
+            fan_out = shp[-1] if not name.endswith("depthwise_weights") else shp[0] * shp[1]
+            w[name] = (rng.standard_normal(shp) * np.sqrt(2.0 / fan_out)).astype(np.float32)
+    return w

@@ -421,6 +421,47 @@ int ds_gnmt_stage_set_attention(ds_stage* h, int slot, const float* attention);
 int ds_gnmt_stage_set_decoder_inputs(ds_stage* h, int slot, const int32_t* target_input,
                                      const int32_t* source_sequence_length, float* attention_out);
 
+/* ---- Operators of an AmoebaNet cell (amoeba_net/network_utils_slice.py), fp32, NHWC ([n, h, w, c] = [rows, c] matrices).
+ * The cell itself (BaseCell.__call__, :394-428) is composed from these and ds_gemm on the host side (dapple_amd/amoeba.py).
+ * `accumulate` != 0: the result is added to what the output holds (a tensor that feeds several operations collects their
+ * gradients). */
+/* tf.nn.relu (:321, :353, ...) and its gradient (dx (+)= dy where x > 0) */
+int ds_relu_fwd(int64_t n, const float* x, float* y, void* stream);
+int ds_relu_bwd(int64_t n, const float* x, const float* dy, float* dx, int accumulate, void* stream);
+/* h = h1 + h2 (:418) */
+int ds_add(int64_t n, const float* a, const float* b, float* y, void* stream);
+/* dst[r][0..cols) (+)= src[r][0..cols) with row strides ld_src / ld_dst: tf.concat of the unused states along the channels
+ * (:553-554) writes each state into its column block; the gradient reads the block back */
+int ds_copy2d(int64_t rows, int cols, const float* src, int64_t ld_src, float* dst, int64_t ld_dst, int accumulate, void* stream);
+/* batch_norm in training mode (:600-806: tf.nn.fused_batch_norm on the batch's own moments, :765-766): per channel
+ * mean and biased variance over the rows, y = (x - mean) rsqrt(var + eps) gamma + beta; save_mean / save_rstd [c] are
+ * kept for the backward pass; moving_mean / moving_var (nullable) follow assign_moving_average (:779-790):
+ * m -= (1 - decay) (m - value), the variance entering as the unbiased estimate.  workspace: ds_batchnorm_workspace_bytes. */
+size_t ds_batchnorm_workspace_bytes(int channels);
+int ds_batchnorm_train_fwd(int64_t rows, int channels, const float* x, const float* gamma, const float* beta, float eps, float* y,
+                           float* save_mean, float* save_rstd, float* moving_mean, float* moving_var, float decay, void* workspace,
+                           void* stream);
+/* dx (+)= gamma rstd (dy - mean_r dy - x_hat mean_r(dy x_hat)); d_gamma += sum_r dy x_hat, d_beta += sum_r dy (nullable) */
+int ds_batchnorm_train_bwd(int64_t rows, int channels, const float* dy, const float* x, const float* gamma, const float* save_mean,
+                           const float* save_rstd, float* dx, int accumulate_dx, float* d_gamma, float* d_beta, void* workspace,
+                           void* stream);
+/* slim.avg_pool2d / slim.max_pool2d, 3 x 3, stride 1, 'SAME' (_pooling, :262-276): kind 0 averages over the taps inside the
+ * image, 1 takes the maximum ('min' pooling is max pooling of -x).  The backward call takes the forward INPUT x. */
+int ds_pool3x3_fwd(int kind, int n, int h, int w, int c, const float* x, float* y, void* stream);
+int ds_pool3x3_bwd(int kind, int n, int h, int w, int c, const float* x, const float* dy, float* dx, int accumulate, void* stream);
+/* The depthwise half of slim.separable_conv2d(..., depth_multiplier=1) (_stacked_separable_conv, :213-238): k x k (k odd),
+ * stride 1, 'SAME'; kernel [k, k, c] (TensorFlow's [k, k, c, 1]).  The pointwise half is ds_gemm on [rows, c]. */
+int ds_depthwise_conv_fwd(int n, int h, int w, int c, int k, const float* x, const float* kernel, float* y, void* stream);
+/* dx (nullable) (+)= input gradient; d_kernel (nullable) += kernel gradient */
+int ds_depthwise_conv_bwd(int n, int h, int w, int c, int k, const float* x, const float* kernel, const float* dy, float* dx,
+                          int accumulate_dx, float* d_kernel, void* stream);
+/* The factorised convolutions slim.conv2d(net, f, [1, k]) / [k, 1] (_apply_conv_operation, :446-459) as GEMMs:
+ * col[pixel][t * c + ch] = x at the pixel shifted by t - k/2 along the width (axis 1) or the height (axis 0), zero outside
+ * the image, so the convolution is col [pixels, k c] x kernel [k c, f] (the kernel as TensorFlow stores it);
+ * ds_scatter1d is the transpose of the gather: dx (+)= the input gradient from d col. */
+int ds_gather1d(int n, int h, int w, int c, int k, int axis, const float* x, float* col, void* stream);
+int ds_scatter1d(int n, int h, int w, int c, int k, int axis, const float* dcol, float* dx, int accumulate, void* stream);
+
 /* XLNet stage (xlnet/models/slice_xlnet.py:164-180 layer body; xlnet/layers/rel_multihead_attn.py:71-149).
  * Activations are sequence-major like the reference: in/out are [streams][seq][batch][hidden] (stream 0 =
  * content stream h, stream 1 = query stream g).  Per-layer weights, in ds_stage_weight_info order:

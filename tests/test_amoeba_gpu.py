@@ -1,0 +1,184 @@
+"""AmoebaNet cell on the GPU through the C ABI against the fp64 CPU oracle (fp32: 1e-4 relative): the operators one by one,
+then whole normal cells of the four published networks - output, both input gradients, every parameter gradient, the two
+tensors at the pipeline cut, gradients accumulated over micro-batches."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from dapple_amd import _lib, amoeba, slices, synthetic
+from dapple_amd._lib import check, ptr
+from oracle import amoeba as oa
+from util import assert_close, dev
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+
+def _rand(shape, seed, scale=1.0):
+    return (np.random.default_rng(seed).standard_normal(shape) * scale).astype(np.float32)
+
+
+def _vjp(fn, inputs, d_out):
+    ins = [torch.tensor(a, dtype=torch.float64, requires_grad=True) for a in inputs]
+    out = fn(*ins)
+    return out.detach(), torch.autograd.grad(out, ins, torch.tensor(d_out, dtype=torch.float64))
+
+
+@pytest.mark.parametrize("n,h,w,c", [(2, 7, 5, 8), (3, 14, 14, 64), (1, 1, 1, 4)])
+def test_batch_norm_training_mode(n, h, w, c):
+    lib, st = _lib.load(), _lib.current_stream()
+    x, g, b, dy = _rand((n, h, w, c), 1) * 2 + 0.5, 1 + _rand((c,), 2, 0.3), _rand((c,), 3), _rand((n, h, w, c), 4)
+    xd, gd, bd, dyd = dev(x), dev(g), dev(b), dev(dy)
+    y, mean, rstd = torch.empty_like(xd), torch.empty(c, device="cuda"), torch.empty(c, device="cuda")
+    mm, mv = torch.zeros(c, device="cuda"), torch.ones(c, device="cuda")
+    ws = torch.empty(lib.ds_batchnorm_workspace_bytes(c), dtype=torch.uint8, device="cuda")
+    rows = n * h * w
+    check(lib.ds_batchnorm_train_fwd(rows, c, ptr(xd), ptr(gd), ptr(bd), 1e-3, ptr(y), ptr(mean), ptr(rstd), ptr(mm), ptr(mv), 0.9, ptr(ws), st), "fwd")
+    ref, (dx_r, dg_r, db_r) = _vjp(lambda a, g_, b_: oa.batch_norm_train(a, g_, b_), [x, g, b], dy)
+    assert_close(y, ref, TOL, "batch norm output")
+    mm_r, mv_r = oa.moving_average_update(torch.zeros(c, dtype=torch.float64), torch.ones(c, dtype=torch.float64), torch.tensor(x, dtype=torch.float64), 0.9)
+    assert_close(mm, mm_r, TOL, "moving mean")
+    if rows > 1:
+        assert_close(mv, mv_r, TOL, "moving variance")
+    dx, dg, db = torch.empty_like(xd), torch.ones(c, device="cuda"), torch.ones(c, device="cuda")
+    check(lib.ds_batchnorm_train_bwd(rows, c, ptr(dyd), ptr(xd), ptr(gd), ptr(mean), ptr(rstd), ptr(dx), 0, ptr(dg), ptr(db), ptr(ws), st), "bwd")
+    if rows > 1:
+        assert_close(dx, dx_r, TOL, "batch norm dx")
+        assert_close(dg - 1, dg_r, TOL, "d gamma (added)")
+    assert_close(db - 1, db_r, TOL, "d beta (added)")
+    keep = dx.clone()
+    check(lib.ds_batchnorm_train_bwd(rows, c, ptr(dyd), ptr(xd), ptr(gd), ptr(mean), ptr(rstd), ptr(dx), 1, None, None, ptr(ws), st), "bwd")
+    assert_close(dx, 2 * keep.double().cpu(), 1e-6, "dx accumulated")
+
+
+@pytest.mark.parametrize("kind", ["avg", "max"])
+@pytest.mark.parametrize("n,h,w,c", [(2, 6, 5, 8), (1, 1, 3, 4), (2, 14, 14, 32)])
+def test_pool3x3(kind, n, h, w, c):
+    lib, st = _lib.load(), _lib.current_stream()
+    x, dy = _rand((n, h, w, c), 5), _rand((n, h, w, c), 6)
+    xd, dyd = dev(x), dev(dy)
+    code = 0 if kind == "avg" else 1
+    y, dx = torch.empty_like(xd), torch.empty_like(xd)
+    check(lib.ds_pool3x3_fwd(code, n, h, w, c, ptr(xd), ptr(y), st), "fwd")
+    check(lib.ds_pool3x3_bwd(code, n, h, w, c, ptr(xd), ptr(dyd), ptr(dx), 0, st), "bwd")
+    ref, (dx_r,) = _vjp(lambda a: oa.pool3x3(a, kind), [x], dy)
+    assert_close(y, ref, 1e-6, kind + " pool")
+    assert_close(dx, dx_r, 1e-5, kind + " pool dx")
+
+
+@pytest.mark.parametrize("n,h,w,c,k", [(2, 6, 5, 8, 3), (1, 9, 9, 16, 5), (2, 7, 7, 4, 7), (1, 2, 2, 4, 5)])
+def test_depthwise_convolution(n, h, w, c, k):
+    lib, st = _lib.load(), _lib.current_stream()
+    x, wt, dy = _rand((n, h, w, c), 7), _rand((k, k, c), 8, 0.3), _rand((n, h, w, c), 9)
+    xd, wd, dyd = dev(x), dev(wt), dev(dy)
+    y, dx, dw = torch.empty_like(xd), torch.empty_like(xd), torch.ones_like(wd)
+    check(lib.ds_depthwise_conv_fwd(n, h, w, c, k, ptr(xd), ptr(wd), ptr(y), st), "fwd")
+    check(lib.ds_depthwise_conv_bwd(n, h, w, c, k, ptr(xd), ptr(wd), ptr(dyd), ptr(dx), 0, ptr(dw), st), "bwd")
+    ref, (dx_r, dw_r) = _vjp(oa.depthwise_same, [x, wt], dy)
+    assert_close(y, ref, 1e-5, "depthwise")
+    assert_close(dx, dx_r, 1e-5, "depthwise dx")
+    assert_close(dw - 1, dw_r, TOL, "depthwise d kernel (added)")
+
+
+@pytest.mark.parametrize("axis,k", [(1, 7), (0, 7), (1, 3), (0, 3)])
+def test_factorised_convolution_as_gather_and_gemm(axis, k):
+    from dapple_amd import ops
+    from dapple_amd._lib import DS_K_MAJOR, DS_MN_MAJOR
+    lib, st = _lib.load(), _lib.current_stream()
+    n, h, w, cin, cout = 2, 9, 8, 8, 12
+    x, wt = _rand((n, h, w, cin), 10), _rand((k * cin, cout), 11, 0.2)
+    xd, wd = dev(x), dev(wt)
+    col = torch.empty(n * h * w, k * cin, device="cuda")
+    check(lib.ds_gather1d(n, h, w, cin, k, axis, ptr(xd), ptr(col), st), "gather")
+    y = torch.empty(n * h * w, cout, device="cuda")
+    ops.gemm(col, wd, y, n * h * w, cout, k * cin, DS_K_MAJOR, DS_MN_MAJOR)
+    w4 = wt.reshape((1, k, cin, cout) if axis == 1 else (k, 1, cin, cout))
+    ref = oa.conv2d_same(torch.tensor(x, dtype=torch.float64), torch.tensor(w4, dtype=torch.float64))
+    assert_close(y.view(n, h, w, cout), ref, 1e-5, "1 x k / k x 1 convolution")
+    dcol = dev(_rand((n * h * w, k * cin), 12))
+    dx = torch.empty_like(xd)
+    check(lib.ds_scatter1d(n, h, w, cin, k, axis, ptr(dcol), ptr(dx), 0, st), "scatter")
+    # the scatter is the transpose of the gather: <gather(x), dcol> == <x, scatter(dcol)>
+    lhs = (col.double() * dcol.double()).sum().item()
+    rhs = (xd.double() * dx.double()).sum().item()
+    assert abs(lhs - rhs) <= 1e-5 * max(1.0, abs(lhs))
+
+
+def _run_cell(name, f, cin, cprev, n, h, w, seed, micro_batches=1, scope="cell_0", total_num_cells=8):
+    ops_, idx, used = synthetic.AMOEBA_NORMAL_CELLS[name]
+    shapes = amoeba.cell_variable_shapes(scope, cin, cprev, f, ops_, idx, used)
+    w_np = synthetic.amoeba_cell_weights(seed, shapes)
+    variables = {k: dev(v) for k, v in w_np.items()}
+    grads = {k: torch.zeros_like(v) for k, v in variables.items() if "moving_" not in k}
+    cell = slices.BaseCell(f, ops_, used, idx, 1.0, total_num_cells, 0).bind(variables, grads)
+    p64 = {k: torch.tensor(v, dtype=torch.float64) for k, v in w_np.items()}
+    acc = {}
+    for m in range(micro_batches):
+        net, d_out = _rand((n, h, w, cin), seed + 10 * m + 1), None
+        prev = None if cprev is None else _rand((n, h, w, cprev), seed + 10 * m + 2)
+        out = cell(dev(net), scope=scope, prev_layer=None if prev is None else dev(prev), cell_num=0)
+        d_out = _rand(tuple(out.shape), seed + 10 * m + 3)
+        d_net, d_prev = cell.backward(dev(d_out))
+        o_r, dn_r, dp_r, dw_r = oa.cell_vjp(torch.tensor(net, dtype=torch.float64), None if prev is None else torch.tensor(prev, dtype=torch.float64),
+                                            p64, torch.tensor(d_out, dtype=torch.float64), scope, f, ops_, idx, used)
+        assert_close(out, o_r, TOL, "%s output mb%d" % (name, m))
+        assert_close(d_net, dn_r, TOL, "%s d net mb%d" % (name, m))
+        if prev is not None:
+            assert_close(d_prev, dp_r, TOL, "%s d prev_layer mb%d" % (name, m))
+        for k, g in dw_r.items():
+            acc[k] = g if k not in acc else acc[k] + g
+    for k, g in acc.items():
+        scale = None
+        assert_close(grads[k], g, TOL, "%s accumulated grad %s" % (name, k), floor=scale)
+    return cell, variables
+
+
+@pytest.mark.parametrize("name", ["amoeba_net_a", "amoeba_net_b", "amoeba_net_c", "amoeba_net_d"])
+def test_normal_cells_small(name):
+    _run_cell(name, f=16, cin=24, cprev=32, n=2, h=6, w=6, seed=20)
+
+
+def test_cell_without_prev_layer_and_with_matching_prev_layer():
+    _run_cell("amoeba_net_a", f=16, cin=24, cprev=None, n=2, h=5, w=5, seed=30)     # prev_layer = None: net stands in, other widths are reduced
+    _run_cell("amoeba_net_d", f=16, cin=16, cprev=16, n=2, h=5, w=5, seed=31)       # equal widths: no prev_1x1 / prev_bn
+
+
+def test_gradients_accumulate_over_micro_batches():
+    _run_cell("amoeba_net_d", f=16, cin=24, cprev=32, n=2, h=6, w=6, seed=40, micro_batches=3)
+
+
+def test_reference_cell_shape_amoeba_net_d():
+    # the reference's driver: amoeba_net_d, reduction_size 256 (amoeba-dapple.py:132-136): the normal cells behind the first
+    # reduction cell run 256 filters on 28 x 28 maps of 4 x 256 channels; batch 8 (amoeba_net/run.sh)
+    _run_cell("amoeba_net_d", f=256, cin=1024, cprev=1024, n=8, h=28, w=28, seed=50)
+
+
+def test_pipeline_cut_yields_two_tensors():
+    # 6 cells: the cut sits inside cell_3 (network_utils_slice.py:309-312): prev_layer after relu + prev_1x1 and net after
+    # relu + 1x1 leave the first device; the second resumes at the two batch norms
+    cell, variables = _run_cell("amoeba_net_a", f=16, cin=24, cprev=32, n=2, h=6, w=6, seed=60, scope="cell_3", total_num_cells=8)
+    assert len(cell.cut_outputs) == 2
+    cut_prev, cut_net = cell.cut_outputs
+    assert tuple(cut_prev.shape) == (2, 6, 6, 16) and tuple(cut_net.shape) == (2, 6, 6, 16)
+    ops_, idx, used = synthetic.AMOEBA_NORMAL_CELLS["amoeba_net_a"]
+    p64 = {k: v.double().cpu() for k, v in variables.items()}
+    net, prev = _rand((2, 6, 6, 24), 61), _rand((2, 6, 6, 32), 62)
+    cp, cn = oa.cell_head(torch.tensor(net, dtype=torch.float64), torch.tensor(prev, dtype=torch.float64), p64, "cell_3", 16)
+    assert_close(cut_prev, cp, TOL, "cut tensor prev")
+    assert_close(cut_net, cn, TOL, "cut tensor net")
+    other, _ = _run_cell("amoeba_net_a", f=16, cin=24, cprev=32, n=2, h=6, w=6, seed=60, scope="cell_2", total_num_cells=8)
+    assert other.cut_outputs == []
+
+
+def test_unbuilt_parts_say_so():
+    ops_, idx, used = synthetic.AMOEBA_NORMAL_CELLS["amoeba_net_a"]
+    cell = slices.BaseCell(16, ops_, used, idx, 1.0, 8, 0).bind({}, None)
+    x = torch.zeros(1, 4, 4, 16, device="cuda")
+    with pytest.raises(NotImplementedError):
+        cell(x, scope="reduction_cell_0", stride=2)
+    with pytest.raises(NotImplementedError):
+        slices.BaseCell(16, ops_, used, idx, 0.7, 8, 0).bind({}, None)(x, scope="cell_0")
+    with pytest.raises(RuntimeError):
+        slices.BaseCell(16, ops_, used, idx, 1.0, 8, 0)(x, scope="cell_0")
