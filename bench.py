@@ -377,6 +377,59 @@ def traffic_rows(path=None):
     return rows
 
 
+def make_amoeba(c, args):
+    import numpy as np
+    import torch
+    from dapple_amd import amoeba, slices, synthetic
+    ops_, idx, used = synthetic.AMOEBA_NORMAL_CELLS[c["cell"]]
+    f, cin, B, Hh, Ww, M = c["filters"], c["in_channels"], c["micro_batch"], c["height"], c["width"], c["num_micro_batches"]
+    shapes = amoeba.cell_variable_shapes("cell_1", cin, cin, f, ops_, idx, used)
+    w_np = synthetic.amoeba_cell_weights(synthetic.SEED_WEIGHT + c["index"], shapes)
+    variables = {k: torch.as_tensor(v).cuda() for k, v in w_np.items()}
+    grads = {k: torch.zeros_like(v) for k, v in variables.items() if "moving_" not in k}
+    cell = slices.BaseCell(f, ops_, used, idx, 1.0, 14, 0).bind(variables, grads)
+    rng = np.random.default_rng(synthetic.SEED_INPUT + c["index"])
+    nets = [torch.as_tensor(rng.standard_normal((B, Hh, Ww, cin)).astype(np.float32)).cuda() for _ in range(M)]
+    prevs = [torch.as_tensor(rng.standard_normal((B, Hh, Ww, cin)).astype(np.float32)).cuda() for _ in range(M)]
+    n_out = f * sum(1 for u in used if not u)
+    dys = [torch.as_tensor(rng.standard_normal((B, Hh, Ww, n_out)).astype(np.float32)).cuda() for _ in range(M)]
+
+    def step():
+        for g in grads.values():
+            g.zero_()
+        for j in range(M):                      # K = 1: F0 B0 F1 B1 ... (a cell keeps one micro-batch's activations)
+            cell(nets[j], scope="cell_1", prev_layer=prevs[j], cell_num=1)
+            cell.backward(dys[j])
+
+    class _NoStage:
+        def overlap_supported(self):
+            return False
+
+        def close(self):
+            pass
+    wl = Workload()
+    wl.stage = _NoStage()
+    wl.step = step
+    wl.samples = B * M
+    rows = Hh * Ww
+    flops = 0
+    for name, shp in shapes.items():            # every kernel that is a matrix of a GEMM: 2 * rows * cin * cout forward
+        if name.endswith("weights") and len(shp) == 2:
+            flops += 2 * rows * shp[0] * shp[1]
+    wl.flops_per_sample = 3 * flops
+    wl.config = {"cell": c["cell"], "filters": f, "in_channels": cin, "map": [Hh, Ww], "micro_batch": B, "micro_batches": M,
+                 "schedule": "F0 B0 F1 B1 ... (one micro-batch in flight)", "flops": "the cell's convolutions as GEMMs, x 3 for the backward pass"}
+
+    def cpu():
+        from oracle import amoeba as oa
+        p = {k: torch.as_tensor(v) for k, v in w_np.items()}
+        t0 = time.perf_counter()
+        oa.cell_vjp(nets[0].cpu(), prevs[0].cpu(), p, dys[0].cpu(), "cell_1", f, ops_, idx, used)
+        return time.perf_counter() - t0, B, "1 of %d micro-batches (%d samples) forward + backward through the cell" % (M, B)
+    wl.cpu = cpu
+    return wl
+
+
 def traffic_of(tag, workload, wgrad_group):
     """Mean measured HBM bytes per launch of the kernel `tag` over the shapes it runs per layer of `workload`, or None
     where no counter run covers it (any workload but the headline one; a weight-gradient grouping other than the two
@@ -392,7 +445,7 @@ def traffic_of(tag, workload, wgrad_group):
     return sum(r[3] + r[4] for r in rows) / len(rows)
 
 
-MAKERS = {"bert": make_bert, "vgg": make_vgg, "vgg_last": make_vgg_last, "gnmt": make_gnmt, "xlnet": make_xlnet, "gnmt_attention": make_gnmt_attention,
+MAKERS = {"amoeba": make_amoeba, "bert": make_bert, "vgg": make_vgg, "vgg_last": make_vgg_last, "gnmt": make_gnmt, "xlnet": make_xlnet, "gnmt_attention": make_gnmt_attention,
           "gnmt_decoder": make_gnmt_decoder}
 METRIC = {"bert48_half": "stage samples/sec fwd+bwd+grad-accum, BERT-48 half-stage; MFMA util %"}
 

@@ -267,8 +267,8 @@ __global__ __launch_bounds__(TPB) void scatter1d_kernel(int64_t n, int H, int W,
 }
 
 int chunks_for(int64_t rows, int C, int64_t* per) {
-  int64_t chunks = 2048 / ((C + TPB - 1) / TPB);
-  if (chunks > (rows + 63) / 64) chunks = (rows + 63) / 64;
+  int64_t chunks = 2048 / ((C + TPB - 1) / TPB);   // enough blocks for every CU to hold several
+  if (chunks > (rows + 15) / 16) chunks = (rows + 15) / 16;
   if (chunks < 1) chunks = 1;
   if (chunks > 65535) chunks = 65535;
   *per = (rows + chunks - 1) / chunks;

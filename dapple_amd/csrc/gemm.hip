@@ -752,15 +752,24 @@ int launch_major(const GemmArgs& a, int batch, int tile, int am, int bm, hipStre
 static void choose_tiling(int m, int n, int k, int kt, int batch, bool can_split, int* tile, int* splitk) {
   static const int bm[3] = {128, 128, 64}, bn[3] = {128, 64, 64};
   static const double slots[3] = {256, 512, 512}, t_round[3] = {0.6, 1.06, 0.45};
-  (void)k; (void)kt; (void)can_split;
   double best = 1e300;
   *tile = 0;
   *splitk = 1;
+  double best_blocks = 0;
   for (int t = 0; t < 3; ++t) {
     const double blocks = (double)((m + bm[t] - 1) / bm[t]) * ((n + bn[t] - 1) / bn[t]) * batch;
     const double rounds = (double)((long long)((blocks + slots[t] - 1) / slots[t]));
     const double cost = rounds * t_round[t];
-    if (cost < best) { best = cost; *tile = t; }
+    if (cost < best) { best = cost; *tile = t; best_blocks = blocks; }
+  }
+  // fp32 accumulation (C += A B^T) of a few tiles under a long reduction - a weight gradient over thousands of pixels
+  // into a small kernel: the reduction is cut into slices that add their parts atomically, so that every CU has work
+  if (can_split && kt == 32 && best_blocks <= 64 && k / kt >= 64) {
+    int sk = (int)(256 / best_blocks);
+    const int most = k / kt / 8;
+    if (sk > most) sk = most;
+    if (sk > 64) sk = 64;
+    if (sk > 1) *splitk = sk;
   }
 }
 
@@ -901,8 +910,9 @@ static int gemm_run(const ds_gemm_desc* d, int splitk_req, void* stream, bool mu
   const int ktiles = (d->k + kt - 1) / kt;
   if (splitk_req > 1 && (f & DS_EPI_ACCUM)) splitk = splitk_req < ktiles ? splitk_req : ktiles;
   if (splitk > 1) a.vec_epi = 0;  // atomics want neighbouring lanes on neighbouring addresses
-  a.splitk = splitk;
   a.ktiles_per_split = (ktiles + splitk - 1) / splitk;
+  splitk = (ktiles + a.ktiles_per_split - 1) / a.ktiles_per_split;   // no slice without a k-tile
+  a.splitk = splitk;
   hipStream_t s = (hipStream_t)stream;
   if (d->dtype == DS_BF16 && d->k % 64 == 0 && a.vec_epi && splitk == 1) {
     // 8-wave kernels (gemm8.hip).  Block shape by the number of output tiles: 256x256 and 256x128 blocks need about a

@@ -276,6 +276,10 @@ CONFIGS = {
     # BASELINE configs[4]: XLNet-36 half-stage, two streams, memory 384
     "xlnet36_half": dict(index=4, kind="xlnet", num_layers=18, hidden=1024, heads=16, ffn=4096, seq=512, mem_len=384,
                          micro_batch=1, num_micro_batches=8, dtype="bf16", streams=2),
+    # one normal cell of the reference driver's AmoebaNet (not a BASELINE configuration): amoeba_net_d, reduction_size 256
+    # (amoeba_net/amoeba-dapple.py:132-136), a cell behind the first reduction cell: 28 x 28 maps, 4 x 256 channels in, batch 8
+    "amoeba_net_d_cell": dict(index=8, kind="amoeba", cell="amoeba_net_d", filters=256, in_channels=1024, height=28, width=28,
+                              micro_batch=8, num_micro_batches=4, dtype="fp32"),
 }
 
 

@@ -97,6 +97,6 @@ def test_grouped_launch_rejects_what_it_cannot_run():
         p["a"], p["b"], p["c"] = p["a"].float(), p["b"].float(), p["c"].float()
         ops.gemm_grouped([dict(p, cfg=2)])
     with pytest.raises(ValueError):
-        ops.gemm_grouped([ok] * 9)
+        ops.gemm_grouped([ok] * 13)           # more tasks than one launch carries
     with pytest.raises(ValueError):   # an operand smaller than its shape says
         ops.gemm_grouped([dict(ok, m=256)])
