@@ -756,7 +756,13 @@ struct XlnetStage : ds_stage {
                                  (int64_t)QQ * R, sp0 + t.qr + (size_t)bb * H * esz, (int64_t)B * H, 0, D, dkr, H, 0, D,
                                  bb > 0 ? DS_EPI_RESIDUAL : 0, dkr, 1);
         if (r.n > 1) { d.k_segment = QQ; d.a_segment_stride = (int64_t)(dy_bd / esz); d.b_segment_stride = sstride; }
-        DS_PROPAGATE(ds_gemm(&d, stream));
+        if (D == 64 && R >= 128 && d.k / 64 > 4) {  // a long reduction into 64 columns per head: 8-wave 128 x 64 tiles
+          GroupOp o;
+          o.kind = GOP_GEMM; o.gemm = d; o.cfg = 3; o.prio = 0;
+          DS_PROPAGATE(ds_group_launch(&o, 1, stream));
+        } else {
+          DS_PROPAGATE(ds_gemm(&d, stream));
+        }
       }
       // seg_emb[s][n][:] += sum_rows def[row][n][s] * qs[row][n][:]   (batched over heads; the run's rows are contiguous in deft)
       {
