@@ -180,6 +180,38 @@ def test_grouped_weight_gradients_over_steps():
             assert (res[1][2][n] - res[4][2][n]).abs().max().item() <= bar * scale, n
 
 
+def test_grouped_weight_gradients_after_forward_only_passes():
+    # forward-only passes (released without a backward pass) walk the stash positions round before a training step: the
+    # positions they took are free again, nothing of them reaches the master gradients
+    L, H, N, F, B, Q, Mm, S, M = 2, 128, 2, 256, 1, 64, 64, 2, 4
+    w_np = synthetic.xlnet_weights(synthetic.SEED_WEIGHT + 78, L, H, N, F, stddev=0.1, perturb=True)
+    xs = [dev(np.stack(x), torch.bfloat16) for x in synthetic.xlnet_stream_inputs(synthetic.SEED_INPUT + 78, M, Q, B, H, streams=S)]
+    dys = [dev(np.stack(x), torch.bfloat16) for x in synthetic.xlnet_stream_inputs(synthetic.SEED_GRAD + 78, M, Q, B, H, streams=S)]
+    masks = dev(np.stack(list(synthetic.xlnet_perm_masks(98, Q, Mm, B))[:S]))
+    mems = dev(np.stack(synthetic.xlnet_mems(58, L, Mm, B, H)), torch.bfloat16)
+    res = {}
+    for warm in (0, 11):
+        st = runtime.xlnet_stage(L, H, N, F, B, Q, "bf16", stash_slots=2, mem_len=Mm, streams=S, wgrad_group=4)
+        st.bind(w_np)
+        st.enable_overlap()
+        outs = [torch.empty(S, Q, B, H, dtype=torch.bfloat16, device="cuda") for _ in range(M)]
+        dxs = [torch.empty_like(o) for o in outs]
+        for i in range(warm):
+            st.set_inputs(i % 2, masks, None, mems)
+            st.forward(i % 2, xs[i % M], outs[0])
+            st.release(i % 2)
+        st.zero_grads()
+        runtime.StageRuntime(st, 0, 2, M).step(xs, dys, outs, dxs, before_forward=lambda slot, j: st.set_inputs(slot, masks, None, mems))
+        st.sync()
+        res[warm] = ([o.float().cpu() for o in outs + dxs], {n: st.grads[n].cpu().clone() for n in st.weight_names})
+        st.close()
+    for a, b in zip(res[0][0], res[11][0]):
+        assert torch.equal(a, b)
+    for n in res[0][1]:
+        scale = res[0][1][n].abs().max().item()
+        assert (res[0][1][n] - res[11][1][n]).abs().max().item() <= 1e-5 * max(scale, 1e-30), n   # (atomic sums: order only)
+
+
 def _run_config4(dtype, M, dy_scale=1.0, repeat_first=False, overlap=True, wgrad_group=8):
     """BASELINE configs[4] at its full size (18 layers, seq 512 + memory 384, two streams) as bench.py runs it."""
     c = synthetic.CONFIGS["xlnet36_half"]
