@@ -46,6 +46,18 @@ __global__ __launch_bounds__(256) void xl_pack_kv_kernel(int H, const float* __r
   }
 }
 
+// wqkv[h][0:H] = wq[h][:], [H:2H] = wk[h][:], [2H:3H] = wv[h][:]: as a K-major operand, row h of the three kernels side by side
+template <typename T>
+__global__ __launch_bounds__(256) void xl_pack_qkv_kernel(int H, const float* __restrict__ wq, const float* __restrict__ wk,
+                                                         const float* __restrict__ wv, T* __restrict__ wqkv) {
+  const int64_t total = (int64_t)H * 3 * H;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int h = (int)(i / (3 * H)), j = (int)(i % (3 * H));
+    const float* src = j < H ? wq : (j < 2 * H ? wk : wv);
+    wqkv[i] = from_f32<T>(src[(int64_t)h * H + j % H]);
+  }
+}
+
 // pe[r][t] = sin((klen - r) * f_t), pe[r][H/2 + t] = cos(...), f_t = 10000^(-2t/H)  (lambda_funcs.py:50-79)
 template <typename T>
 __global__ __launch_bounds__(256) void xl_pos_emb_kernel(int R, int H, int klen, T* __restrict__ pe) {
@@ -179,7 +191,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void xl_seg_bwd_kernel(int QQ, int B, int N, int D, int64_t rows_total,
                                                         const float* __restrict__ defs, const float* __restrict__ seg_emb,
                                                         const T* __restrict__ dqw, const T* __restrict__ dqr, T* __restrict__ dqs,
-                                                        T* __restrict__ dq, T* __restrict__ deft) {
+                                                        T* __restrict__ dq, int64_t ld_dq, T* __restrict__ deft) {
   const int lane = threadIdx.x & 63;
   const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (w >= (int64_t)B * N * QQ) return;
@@ -196,7 +208,7 @@ __global__ __launch_bounds__(256) void xl_seg_bwd_kernel(int QQ, int B, int N, i
     const int64_t o = row * H + n * D + lane;
     const float s = d0 * seg_emb[n * D + lane] + d1 * seg_emb[H + n * D + lane];
     dqs[o] = from_f32<T>(s);
-    dq[o] = from_f32<T>(to_f32(dqw[o]) + to_f32(dqr[o]) + s);
+    dq[row * ld_dq + n * D + lane] = from_f32<T>(to_f32(dqw[o]) + to_f32(dqr[o]) + s);
   }
 }
 
@@ -211,7 +223,7 @@ struct XlnetStage : ds_stage {
   size_t esz;
   // compute copies
   char* wc_base = nullptr;
-  std::vector<char*> wq, wkv, wr, wo, w1, w2, kr;
+  std::vector<char*> wq, wkv, wqkv, wr, wo, w1, w2, kr;
   char* pe = nullptr;
   // stash
   char* stash_base = nullptr;
@@ -229,7 +241,7 @@ struct XlnetStage : ds_stage {
   char* ws_base = nullptr;
   // buffers the weight-gradient kernels read alternate by layer parity ([2])
   size_t ws_bytes = 0, ws_de = 0, ws_qall, ws_ac, ws_dp, ws_bd, ws_ds, ws_dbd[2], ws_def, ws_dz2[2], ws_du[2], ws_dy1, ws_dz1[2], ws_dvec, ws_dqw[2], ws_dqr[2],
-         ws_dqs[2], ws_dq[2], ws_dkv[2], ws_dkr[2], ws_deft[2], ws_dx[2];
+         ws_dqs[2], ws_dqkv[2], ws_dkr[2], ws_deft[2], ws_dx[2];
   WgradLane lane;
   // Deferred weight gradients (xc.wgrad_group = G > 1, bf16): a backward pass leaves the operands of its weight-gradient
   // products in a ring of 2G positions per layer and its activations stay in their stash position; after every G passes
@@ -237,10 +249,14 @@ struct XlnetStage : ds_stage {
   // position / one ring position apart), the products of two layers as one grouped launch.  There are then more stash
   // positions than slots (slots + G, rounded up to a multiple of G), handed out round-robin in forward order.
   int G = 1, KP = 0, NDY = 0;
-  struct LayerDy { size_t dz2, du, dz1, dq, dqw, dqr, dqs, dkv, dbd, deft, dkr, dyn2, dyn1, rs2, rs1; };  // (deft: [heads * 2][2G * rows]; dkr: one per layer)
+  struct LayerDy { size_t dz2, du, dz1, dqkv, dqw, dqr, dqs, dbd, deft, dkr, dyn2, dyn1, rs2, rs1; };  // (deft: [heads * 2][2G * rows]; dkr: one per layer)
   std::vector<LayerDy> ld;
   char* dy_base = nullptr;
-  size_t dy_act = 0, dy_actF = 0, dy_kv = 0, dy_bd = 0;
+  // The query gradients and the key | value gradients of a pass share one matrix of (mem_len * batch + rows) rows and 3 H
+  // columns: dq in columns [0, H) of the rows behind the memory rows, dk | dv in columns [H, 3 H) of the first klen * batch
+  // rows - so the content stream's rows hold [dq | dk | dv] side by side and the input gradient
+  // dx = dq Wq^T + (dk | dv) Wkv^T is ONE product over 3 H (the query stream's k | v columns are never written and stay zero).
+  size_t dy_act = 0, dy_actF = 0, dy_qkv = 0, dy_bd = 0;
   struct Deferred { int xpos, dypos; };
   struct Run { int xpos, dypos, n; };
   std::vector<Deferred> deferred;
@@ -290,10 +306,11 @@ struct XlnetStage : ds_stage {
         winfo.push_back({name, r, c});
       }
     Arena ca;
-    std::vector<size_t> o_q(L), o_kv(L), o_r(L), o_o(L), o_1(L), o_2(L), o_kr(L);
+    std::vector<size_t> o_q(L), o_kv(L), o_qkv(L), o_r(L), o_o(L), o_1(L), o_2(L), o_kr(L);
     const size_t o_pe = ca.reserve((size_t)R * H * esz);
     for (int l = 0; l < L; ++l) {
       o_kv[l] = ca.reserve((size_t)H * 2 * H * esz);
+      o_qkv[l] = ca.reserve((size_t)H * 3 * H * esz);
       o_kr[l] = ca.reserve((size_t)R * H * esz);
       if (dtype == DS_BF16) {
         o_q[l] = ca.reserve((size_t)H * H * esz); o_r[l] = ca.reserve((size_t)H * H * esz); o_o[l] = ca.reserve((size_t)H * H * esz);
@@ -302,9 +319,9 @@ struct XlnetStage : ds_stage {
     }
     DS_CHECK_HIP(hipMalloc((void**)&wc_base, ca.used));
     pe = wc_base + o_pe;
-    wq.resize(L); wkv.resize(L); wr.resize(L); wo.resize(L); w1.resize(L); w2.resize(L); kr.resize(L);
+    wq.resize(L); wkv.resize(L); wqkv.resize(L); wr.resize(L); wo.resize(L); w1.resize(L); w2.resize(L); kr.resize(L);
     for (int l = 0; l < L; ++l) {
-      wkv[l] = wc_base + o_kv[l]; kr[l] = wc_base + o_kr[l];
+      wkv[l] = wc_base + o_kv[l]; wqkv[l] = wc_base + o_qkv[l]; kr[l] = wc_base + o_kr[l];
       if (dtype == DS_BF16) { wq[l] = wc_base + o_q[l]; wr[l] = wc_base + o_r[l]; wo[l] = wc_base + o_o[l]; w1[l] = wc_base + o_1[l]; w2[l] = wc_base + o_2[l]; }
     }
     // stash
@@ -347,12 +364,12 @@ struct XlnetStage : ds_stage {
       pos_owner.assign(KP, -1);
       pos_deferred.assign(KP, 0);
       Arena da;
-      dy_act = act; dy_actF = actF; dy_kv = (size_t)krows * 2 * H * esz; dy_bd = (size_t)B * N * S * Q * R * esz;
+      dy_act = act; dy_actF = actF; dy_qkv = ((size_t)Mm * B + rows) * 3 * H * esz; dy_bd = (size_t)B * N * S * Q * R * esz;
       ld.resize(L);
       for (int l = 0; l < L; ++l) {
         ld[l].dz2 = da.reserve(dy_act * NDY); ld[l].du = da.reserve(dy_actF * NDY); ld[l].dz1 = da.reserve(dy_act * NDY);
-        ld[l].dq = da.reserve(dy_act * NDY); ld[l].dqw = da.reserve(dy_act * NDY); ld[l].dqr = da.reserve(dy_act * NDY);
-        ld[l].dqs = da.reserve(dy_act * NDY); ld[l].dkv = da.reserve(dy_kv * NDY); ld[l].dbd = da.reserve(dy_bd * NDY);
+        ld[l].dqkv = da.reserve(dy_qkv * NDY); ld[l].dqw = da.reserve(dy_act * NDY); ld[l].dqr = da.reserve(dy_act * NDY);
+        ld[l].dqs = da.reserve(dy_act * NDY); ld[l].dbd = da.reserve(dy_bd * NDY);
         ld[l].deft = da.reserve((size_t)N * 2 * rows * esz * NDY); ld[l].dkr = da.reserve((size_t)R * H * esz);
         if (rs32) {  // the fp32 gradients entering the two LayerNorms and two sums per row: their parameter gradients are formed per group
           ld[l].dyn2 = da.reserve((size_t)rows * H * 4 * NDY); ld[l].dyn1 = da.reserve((size_t)rows * H * 4 * NDY);
@@ -361,7 +378,10 @@ struct XlnetStage : ds_stage {
       }
       DS_CHECK_HIP(hipMalloc((void**)&dy_base, da.used));
       // the un-shifted score gradients are zero outside the band the score-gradient kernel writes, in every ring position
-      for (int l = 0; l < L; ++l) DS_CHECK_HIP(hipMemsetAsync(dy_base + ld[l].dbd, 0, dy_bd * NDY, stream));
+      for (int l = 0; l < L; ++l) {
+        DS_CHECK_HIP(hipMemsetAsync(dy_base + ld[l].dbd, 0, dy_bd * NDY, stream));
+        DS_CHECK_HIP(hipMemsetAsync(dy_base + ld[l].dqkv, 0, dy_qkv * NDY, stream));
+      }
       ev_x_bwd.assign(KP, nullptr); ev_x_wg.assign(KP, nullptr); ev_dy_wg.assign(NDY, nullptr);
       for (int i = 0; i < KP; ++i) {
         DS_CHECK_HIP(hipEventCreateWithFlags(&ev_x_bwd[i], hipEventDisableTiming));
@@ -391,8 +411,8 @@ struct XlnetStage : ds_stage {
     ws_dy1 = w.reserve(act); ws_dvec = w.reserve(act);
     for (int p = 0; p < 2; ++p) {
       ws_dz2[p] = w.reserve(act); ws_du[p] = w.reserve(actF); ws_dz1[p] = w.reserve(act);
-      ws_dqw[p] = w.reserve(act); ws_dqr[p] = w.reserve(act); ws_dqs[p] = w.reserve(act); ws_dq[p] = w.reserve(act);
-      ws_dkv[p] = w.reserve((size_t)krows * 2 * H * esz);
+      ws_dqw[p] = w.reserve(act); ws_dqr[p] = w.reserve(act); ws_dqs[p] = w.reserve(act);
+      ws_dqkv[p] = w.reserve(((size_t)Mm * B + rows) * 3 * H * esz);
       ws_dkr[p] = w.reserve((size_t)R * H * esz);
       ws_deft[p] = w.reserve((size_t)N * 2 * rows * esz);
     }
@@ -409,6 +429,7 @@ struct XlnetStage : ds_stage {
     // (queued on the stage's stream, ahead of every pass; creation is not something a caller captures in a graph)
     DS_CHECK_HIP(hipMemsetAsync(ws_base + ws_dbd[0], 0, (size_t)B * N * QQ * R * esz, stream));
     DS_CHECK_HIP(hipMemsetAsync(ws_base + ws_dbd[1], 0, (size_t)B * N * QQ * R * esz, stream));
+    for (int p = 0; p < 2; ++p) DS_CHECK_HIP(hipMemsetAsync(ws_base + ws_dqkv[p], 0, ((size_t)Mm * B + rows) * 3 * H * esz, stream));
     return DS_OK;
   }
 
@@ -487,6 +508,7 @@ struct XlnetStage : ds_stage {
       do {
         if (dtype == DS_BF16) {
           hipLaunchKernelGGL(xl_pack_kv_kernel<bf16>, dim3(1024), dim3(256), 0, cs, H, w[b + X_K], w[b + X_V], (bf16*)wkv[l]);
+          hipLaunchKernelGGL(xl_pack_qkv_kernel<bf16>, dim3(1024), dim3(256), 0, cs, H, w[b + X_Q], w[b + X_K], w[b + X_V], (bf16*)wqkv[l]);
           if ((rc = ds_cast_f32_to_bf16(wq[l], w[b + X_Q], (size_t)H * H, cs)) != DS_OK) break;
           if ((rc = ds_cast_f32_to_bf16(wr[l], w[b + X_R], (size_t)H * H, cs)) != DS_OK) break;
           if ((rc = ds_cast_f32_to_bf16(wo[l], w[b + X_O], (size_t)H * H, cs)) != DS_OK) break;
@@ -494,6 +516,7 @@ struct XlnetStage : ds_stage {
           if ((rc = ds_cast_f32_to_bf16(w2[l], w[b + X_W2], (size_t)F * H, cs)) != DS_OK) break;
         } else {
           hipLaunchKernelGGL(xl_pack_kv_kernel<float>, dim3(1024), dim3(256), 0, cs, H, w[b + X_K], w[b + X_V], (float*)wkv[l]);
+          hipLaunchKernelGGL(xl_pack_qkv_kernel<float>, dim3(1024), dim3(256), 0, cs, H, w[b + X_Q], w[b + X_K], w[b + X_V], (float*)wqkv[l]);
         }
         // k_r = pos_emb @ Wr does not depend on the micro-batch: once per refresh
         rc = gemm(DS_K_MAJOR, DS_MN_MAJOR, R, H, H, pe, H, WT(l, X_R), H, kr[l], H);
@@ -745,8 +768,11 @@ struct XlnetStage : ds_stage {
     for (const Run& r : runs) {
       const char* sp0 = stash_base + (size_t)r.xpos * slot_bytes;
       const char* dz2 = dy_base + ld[l].dz2 + r.dypos * dy_act; const char* du = dy_base + ld[l].du + r.dypos * dy_actF;
-      const char* dz1 = dy_base + ld[l].dz1 + r.dypos * dy_act; const char* dq = dy_base + ld[l].dq + r.dypos * dy_act;
-      const char* dkv = dy_base + ld[l].dkv + r.dypos * dy_kv;
+      const char* dz1 = dy_base + ld[l].dz1 + r.dypos * dy_act;
+      const char* dqkv = dy_base + ld[l].dqkv + r.dypos * dy_qkv;
+      const char* dq = dqkv + (size_t)Mm * B * 3 * H * esz;   // columns [0, H) behind the memory rows
+      const char* dkv = dqkv + (size_t)H * esz;                // columns [H, 3 H) from the first row
+      const int64_t qkv_seg = (int64_t)(dy_qkv / esz);
       char* dkr = dy_base + ld[l].dkr;
       const int QQ = S * Q;
       // dk_r = sum over micro-batches and samples of dbd^T (q + r_r), per head: k_r is shared by the batch, so one launch per
@@ -789,14 +815,14 @@ struct XlnetStage : ds_stage {
       wg(F, H, rows, sp0 + t.hh, F, sstride, dz2, H, (int64_t)rows * H, g[b + X_W2], H);
       wg(H, F, rows, sp0 + t.y1, H, sstride, du, F, (int64_t)rows * F, g[b + X_W1], F);
       wg(H, H, rows, dz1, H, (int64_t)rows * H, sp0 + t.vec, H, sstride, g[b + X_O], H);
-      wg(H, H, rows, sp0 + t.x, H, sstride, dq, H, (int64_t)rows * H, g[b + X_Q], H);
+      wg(H, H, rows, sp0 + t.x, H, sstride, dq, 3 * H, qkv_seg, g[b + X_Q], H);
       { ds_gemm_desc& d = wg(H, H, R, pe, H, 0, dkr, H, 0, g[b + X_R], H); d.k = R; d.k_segment = 0; }   // dk_r already holds the run's sum
       if (kv_adjacent) {  // k and v: the two column halves of dkv, batched (z = 0: k, 1: v)
-        ds_gemm_desc& d = wg(H, H, krows, sp0 + t.mem, H, sstride, dkv, 2 * H, (int64_t)krows * 2 * H, g[b + X_K], H);
+        ds_gemm_desc& d = wg(H, H, krows, sp0 + t.mem, H, sstride, dkv, 3 * H, qkv_seg, g[b + X_K], H);
         d.batch = 2; d.batch_inner = 2; d.b_stride_inner = H; d.c_stride_inner = (int64_t)H * H;
       } else {
         for (int j = 0; j < 2; ++j)
-          wg(H, H, krows, sp0 + t.mem, H, sstride, dkv + (size_t)j * H * esz, 2 * H, (int64_t)krows * 2 * H, g[b + X_K + j], H);
+          wg(H, H, krows, sp0 + t.mem, H, sstride, dkv + (size_t)j * H * esz, 3 * H, qkv_seg, g[b + X_K + j], H);
       }
       for (int i = 0; i < nd; ++i) {
         // (one launch never carries two products into the same master gradient: runs of one layer are flushed apart)
@@ -909,8 +935,9 @@ struct XlnetStage : ds_stage {
       char* dqw = G > 1 ? ringp(ld[l].dqw, dy_act) : ws_base + ws_dqw[par];
       char* dqr = G > 1 ? ringp(ld[l].dqr, dy_act) : ws_base + ws_dqr[par];
       char* dqs = G > 1 ? ringp(ld[l].dqs, dy_act) : ws_base + ws_dqs[par];
-      char* dq = G > 1 ? ringp(ld[l].dq, dy_act) : ws_base + ws_dq[par];
-      char* dkv = G > 1 ? ringp(ld[l].dkv, dy_kv) : ws_base + ws_dkv[par];
+      char* dqkv = G > 1 ? ringp(ld[l].dqkv, dy_qkv) : ws_base + ws_dqkv[par];
+      char* dq = dqkv + (size_t)Mm * B * 3 * H * esz;   // [rows, H] at row stride 3 H
+      char* dkv = dqkv + (size_t)H * esz;                // [klen * batch, 2 H] at row stride 3 H
       char* dkr = ws_base + ws_dkr[par];
       char* deft = G > 1 ? dy_base + ld[l].deft + (size_t)dypos * rows * esz : ws_base + ws_deft[par];
       const int64_t deft_ld = G > 1 ? (int64_t)NDY * rows : (int64_t)rows;
@@ -957,7 +984,7 @@ struct XlnetStage : ds_stage {
                                2 * H, D, dp, K, (int64_t)N * QQ * K, (int64_t)QQ * K, DS_EPI_OUT_F32));
         const bool grouped = group_products(QQ);
         const ds_gemm_desc d_dv = desc_bn(DS_MN_MAJOR, DS_MN_MAJOR, K, D, QQ, p, K, (int64_t)N * QQ * K, (int64_t)QQ * K, dvec, (int64_t)B * H, H, D,
-                                          dkv + (size_t)H * esz, (int64_t)B * 2 * H, 2 * H, D, 0);
+                                          dkv + (size_t)H * esz, (int64_t)B * 3 * H, 3 * H, D, 0);
         if (!grouped) DS_PROPAGATE(ds_gemm(&d_dv, stream));
         // dS, its un-shifted copy for the position term (dbd[i][r] = dS[i][r - Q + i]) and the segment sums, in one pass
         float* defs = (float*)(ws_base + ws_def);
@@ -978,7 +1005,7 @@ struct XlnetStage : ds_stage {
         const ds_gemm_desc d_dqw = desc_bn(DS_K_MAJOR, DS_MN_MAJOR, QQ, D, K, dsm, K, (int64_t)N * QQ * K, (int64_t)QQ * K, sp + t.kv,
                                            (int64_t)B * 2 * H, 2 * H, D, dqw, (int64_t)B * H, H, D, 0);
         const ds_gemm_desc d_dk = desc_bn(DS_MN_MAJOR, DS_MN_MAJOR, K, D, QQ, dsm, K, (int64_t)N * QQ * K, (int64_t)QQ * K, sp + t.qw, (int64_t)B * H,
-                                          H, D, dkv, (int64_t)B * 2 * H, 2 * H, D, 0);
+                                          H, D, dkv, (int64_t)B * 3 * H, 3 * H, D, 0);
         // position term through the shift
         const ds_gemm_desc d_dqr = desc_bn(DS_K_MAJOR, DS_MN_MAJOR, QQ, D, R, dbd, R, (int64_t)N * QQ * R, (int64_t)QQ * R, kr[l], H, 0, D,
                                            dqr, (int64_t)B * H, H, D, 0);
@@ -999,15 +1026,14 @@ struct XlnetStage : ds_stage {
           dim3 grid((unsigned)((waves + 3) / 4));
           if (dtype == DS_BF16)
             hipLaunchKernelGGL(xl_seg_bwd_kernel<bf16>, grid, dim3(256), 0, stream, QQ, B, N, D, deft_ld, defs, w[b + X_SEG],
-                               (const bf16*)dqw, (const bf16*)dqr, (bf16*)dqs, (bf16*)dq, (bf16*)deft);
+                               (const bf16*)dqw, (const bf16*)dqr, (bf16*)dqs, (bf16*)dq, (int64_t)3 * H, (bf16*)deft);
           else
             hipLaunchKernelGGL(xl_seg_bwd_kernel<float>, grid, dim3(256), 0, stream, QQ, B, N, D, deft_ld, defs, w[b + X_SEG],
-                               (const float*)dqw, (const float*)dqr, (float*)dqs, (float*)dq, (float*)deft);
+                               (const float*)dqw, (const float*)dqr, (float*)dqs, (float*)dq, (int64_t)3 * H, (float*)deft);
           DS_CHECK_LAUNCH();
         }
       }
       // ---- weight gradients of this layer (on the weight-gradient stream when there is one)
-      const char* dkv_h = dkv + (size_t)Mm * B * 2 * H * esz;
       hipStream_t chain = stream;
       if (wgs && (G <= 1 || closing)) {
         DS_PROPAGATE(lane.begin(chain, wgs, par));
@@ -1039,7 +1065,7 @@ struct XlnetStage : ds_stage {
           if ((rc = ds_gemm(&d, stream)) != DS_OK) break;
         }
         // projections
-        if ((rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, rows, x, H, dq, H, g[b + X_Q], H, DS_EPI_ACCUM)) != DS_OK) break;
+        if ((rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, rows, x, H, dq, 3 * H, g[b + X_Q], H, DS_EPI_ACCUM)) != DS_OK) break;
         for (int bb = 0; bb < B && rc == DS_OK; ++bb) {  // k_r is shared by the batch: one launch per batch entry, added in place
           const int a2 = bb > 0 ? DS_EPI_RESIDUAL : 0;
           rc = gemm_bn(DS_MN_MAJOR, DS_MN_MAJOR, R, D, S * Q, dbd + (size_t)bb * N * S * Q * R * esz, R, 0, (int64_t)S * Q * R,
@@ -1052,14 +1078,14 @@ struct XlnetStage : ds_stage {
         if (g[b + X_V] == g[b + X_K] + (size_t)H * H) {
           ds_gemm_desc d;
           memset(&d, 0, sizeof(d));
-          d.dtype = dtype; d.a_major = DS_MN_MAJOR; d.b_major = DS_MN_MAJOR; d.m = H; d.n = H; d.lda = H; d.ldb = 2 * H; d.ldc = H;
+          d.dtype = dtype; d.a_major = DS_MN_MAJOR; d.b_major = DS_MN_MAJOR; d.m = H; d.n = H; d.lda = H; d.ldb = 3 * H; d.ldc = H;
           d.batch = 2; d.batch_inner = 2; d.b_stride_inner = H; d.c_stride_inner = (int64_t)H * H;
           d.flags = DS_EPI_ACCUM; d.alpha = 1.f; d.c = g[b + X_K];
           d.k = krows; d.a = sp + t.mem; d.b = dkv;   // memory rows and content rows in one reduction
           if ((rc = ds_gemm(&d, stream)) != DS_OK) break;
         } else {
           for (int j = 0; j < 2 && rc == DS_OK; ++j)  // j = 0: k, 1: v
-            rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, krows, sp + t.mem, H, dkv + (size_t)j * H * esz, 2 * H, g[b + X_K + j], H, DS_EPI_ACCUM);
+            rc = gemm(DS_MN_MAJOR, DS_MN_MAJOR, H, H, krows, sp + t.mem, H, dkv + (size_t)j * H * esz, 3 * H, g[b + X_K + j], H, DS_EPI_ACCUM);
         }
       } while (0);
       if (wgs && G <= 1) {
@@ -1072,20 +1098,18 @@ struct XlnetStage : ds_stage {
       if (closing) rc = layer_wgrad_runs(l, runs);
       stream = chain;
       if (rc != DS_OK) return rc;
-      // dx = dq Wq^T + dz1 (residual); the content-stream rows also receive dkv Wkv^T
+      // dx = dq Wq^T + dz1 (residual) and, on the content stream's rows, + (dk | dv) Wkv^T: one product over [dq | dk | dv]
       const bool first = l == 0;
       if (first && d_in == nullptr) break;
       char* dx = first ? (char*)d_in : ws_base + ws_dx[l & 1];
       if (rs32) {
         float* dxf = (float*)(ws_base + bw_dxf[l & 1]);
-        DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rows, H, H, dq, H, WT(l, X_Q), H, dxf, H, res32, nullptr, dz1f));
-        DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rowsS, H, 2 * H, dkv_h, 2 * H, wkv[l], 2 * H, dxf, H, res32, nullptr, dxf));
+        DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rows, H, 3 * H, dq, 3 * H, wqkv[l], 3 * H, dxf, H, res32, nullptr, dz1f));
         if (first) DS_PROPAGATE(ds_cast_f32_to_bf16(d_in, dxf, (size_t)rows * H, stream));  // the stage's input gradient leaves as bf16
         dyf = dxf;
         continue;
       }
-      DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rows, H, H, dq, H, WT(l, X_Q), H, dx, H, DS_EPI_RESIDUAL, nullptr, dz1));
-      DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rowsS, H, 2 * H, dkv_h, 2 * H, wkv[l], 2 * H, dx, H, DS_EPI_RESIDUAL, nullptr, dx));
+      DS_PROPAGATE(gemm(DS_K_MAJOR, DS_K_MAJOR, rows, H, 3 * H, dq, 3 * H, wqkv[l], 3 * H, dx, H, DS_EPI_RESIDUAL, nullptr, dz1));
       dy = dx;
     }
     // the stash slot and the master gradients are released to the caller in the order of `stream`
