@@ -560,7 +560,7 @@ def main():
         # the other BASELINE configurations, a few steps each, in the same process: throughput and whole-stage fraction of
         # the matrix peak of their arithmetic (no CPU legs, no per-kernel timing)
         others = {}
-        for name in ("bert_large_2l", "vgg19_stage0", "gnmt16_encoder", "xlnet36_half"):
+        for name in ("bert_large_2l", "vgg19_stage0", "gnmt16_encoder", "xlnet36_half", "amoeba_net_d_cell"):
             oc = dict(synthetic.CONFIGS[name])
             ow = MAKERS[oc["kind"]](oc, args)
             o_overlap = not args.no_overlap and ow.stage.overlap_supported()
