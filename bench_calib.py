@@ -27,6 +27,7 @@ of micro-batch j+1, an input-gradient product of micro-batch j, a weight-gradien
 three ways - back to back on one stream, side by side on two / three streams, and as ONE ``ds_gemm_grouped`` launch per
 tile-shape choice.
 """
+import time
 import sys
 
 import torch
@@ -190,6 +191,33 @@ def grouped():
         print("%-44s %9.1f %9.1f | %s   [%.1f GFLOP]" % (" + ".join(names), t1, tn, "  ".join(cells), flop / 1e9), flush=True)
 
 
+def wgrad_group():
+    """The weight-gradient products of two BERT-48 layers over all 8 micro-batches of a step (8192 rows) as ONE grouped launch
+    of 256 x 128 tiles - what the stage queues twelve times per step - three launches, for counter and trace runs."""
+    bf = torch.bfloat16
+    rows, h, f = 8 * 1024, 1024, 4096
+    probs, flop = [], 0
+    for layer in range(2):
+        x, ctx, a1, hh = (torch.randn(rows, w, device="cuda").to(bf) for w in (h, h, h, f))
+        dz2, du, dz1, dqkv = (torch.randn(rows, w, device="cuda").to(bf) for w in (h, f, h, 3 * h))
+        for a, b, m, n, extra in ((hh, dz2, f, h, {}), (a1, du, h, f, {}), (ctx, dz1, h, h, {}),
+                                  (x, dqkv, h, h, dict(ldb=3 * h, batch=3, batch_inner=3, b_strides=(0, h), c_strides=(0, h * h)))):
+            nb = extra.get("batch", 1)
+            c = torch.zeros(nb * m, n, device="cuda")
+            probs.append(dict(a=a, b=b, c=c, m=m, n=n, k=rows, a_major=DS_MN_MAJOR, b_major=DS_MN_MAJOR, flags=DS_EPI_ACCUM, cfg=1, **extra))
+            flop += 2 * m * n * rows * nb
+    for _ in range(3):
+        ops.gemm_grouped(probs)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(5):
+        ops.gemm_grouped(probs)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / 5
+    print("grouped weight gradients of two layers over 8192 rows: %d tasks, %.2f GFLOP per launch, %.1f us, %.0f TFLOP/s"
+          % (len(probs), flop / 1e9, dt * 1e6, flop / dt / 1e12))
+
+
 def attention():
     batch, heads, seq, d = 2, 16, 512, 64
     bf = torch.bfloat16
@@ -276,5 +304,7 @@ if __name__ == "__main__":
         gemm_table()
     elif len(sys.argv) > 1 and sys.argv[1] == "grouped":
         grouped()
+    elif len(sys.argv) > 1 and sys.argv[1] == "wgrad_group":
+        wgrad_group()
     else:
         accumulate(int(sys.argv[2]) if len(sys.argv) > 2 else 1 << 26)
