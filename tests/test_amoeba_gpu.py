@@ -155,6 +155,42 @@ def test_reference_cell_shape_amoeba_net_d():
     _run_cell("amoeba_net_d", f=256, cin=1024, cprev=1024, n=8, h=28, w=28, seed=50)
 
 
+def test_two_chained_cells_forward_and_backward():
+    # cells feed each other as in _build_network_base (model_builder_slice.py:399-417): cell n takes the previous cell's
+    # output as net and the output before that as prev_layer; the backward pass hands d_net and d_prev_layer back the same way
+    ops_, idx, used = synthetic.AMOEBA_NORMAL_CELLS["amoeba_net_d"]
+    f, c0, n, h, w = 16, 24, 2, 6, 6
+    c1 = f * sum(1 for u in used if not u)                      # width of a cell's output
+    shapes = {}
+    shapes.update(amoeba.cell_variable_shapes("cell_0", c0, c0, f, ops_, idx, used))
+    shapes.update(amoeba.cell_variable_shapes("cell_1", c1, c0, f, ops_, idx, used))
+    w_np = synthetic.amoeba_cell_weights(70, shapes)
+    variables = {k: dev(v) for k, v in w_np.items()}
+    grads = {k: torch.zeros_like(v) for k, v in variables.items() if "moving_" not in k}
+    cell = slices.BaseCell(f, ops_, used, idx, 1.0, 8, 0).bind(variables, grads)
+    x0, x1, d_out = _rand((n, h, w, c0), 71), _rand((n, h, w, c0), 72), _rand((n, h, w, c1), 73)
+    x0d, x1d = dev(x0), dev(x1)
+    y0 = cell(x1d, scope="cell_0", prev_layer=x0d, cell_num=0)
+    y1 = cell(y0, scope="cell_1", prev_layer=x1d, cell_num=1)
+    d_y0, d_x1_b = cell.backward(dev(d_out))                    # cell_1: d net (= d y0), d prev_layer (= part of d x1)
+    d_x1_a, d_x0 = cell.backward(d_y0)                          # cell_0
+    p64 = {k: torch.tensor(v, dtype=torch.float64) for k, v in w_np.items()}
+    a0 = torch.tensor(x0, dtype=torch.float64, requires_grad=True)
+    a1 = torch.tensor(x1, dtype=torch.float64, requires_grad=True)
+    names = sorted(k for k in p64 if "moving_" not in k)
+    params = {k: p64[k].clone().requires_grad_(True) for k in names}
+    full = dict(p64)
+    full.update(params)
+    r0, _ = oa.cell_forward(a1, a0, full, "cell_0", f, ops_, idx, used)
+    r1, _ = oa.cell_forward(r0, a1, full, "cell_1", f, ops_, idx, used)
+    g = torch.autograd.grad(r1, [a0, a1] + [params[k] for k in names], torch.tensor(d_out, dtype=torch.float64))
+    assert_close(y1, r1.detach(), TOL, "output of the second cell")
+    assert_close(d_x0, g[0], TOL, "gradient of the first input")
+    assert_close(d_x1_a + d_x1_b, g[1], TOL, "gradient of the second input (through both cells)")
+    for k, gk in zip(names, g[2:]):
+        assert_close(grads[k], gk, TOL, "grad " + k)
+
+
 def test_pipeline_cut_yields_two_tensors():
     # 6 cells: the cut sits inside cell_3 (network_utils_slice.py:309-312): prev_layer after relu + prev_1x1 and net after
     # relu + 1x1 leave the first device; the second resumes at the two batch norms
