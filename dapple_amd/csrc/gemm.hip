@@ -982,6 +982,20 @@ static int gemm_run(const ds_gemm_desc* d, int splitk_req, void* stream, bool mu
     ds_set_error("ds_gemm_static_scratch: needs bf16 operands, k a multiple of 64 and 16-byte aligned, 8-column outputs");
     return DS_EINVAL;
   }
+  {
+    // 64x64 blocks under a long reduction: the four waves split the k-steps of every k-tile instead of the tile (half the
+    // LDS fragment reads for the same 48 KB; gemm8_core.h).  DS_GEMM_KS4 = 0 switches it off, n sets the least number of k-tiles.
+    static const char* env_ks = getenv("DS_GEMM_KS4");
+    const int least = env_ks ? atoi(env_ks) : 16;
+    if (least > 0 && tile == 2 && d->dtype == DS_BF16 && d->k % 64 == 0 && a.vec_epi && splitk == 1 && ktiles % 2 == 0 && ktiles >= 4 &&
+        ktiles >= least) {
+      char tagk[96];
+      snprintf(tagk, sizeof(tagk), "gemm_ks4_kernel<bf16,64,64,%s,%s>", d->a_major == DS_K_MAJOR ? "K" : "MN",
+               d->b_major == DS_K_MAJOR ? "K" : "MN");
+      ds_prof_scope profk(s, tagk, 2.0 * d->m * d->n * d->k * batch, "FLOP");
+      return ds_gemm_ks4_launch(a, d->a_major, d->b_major, batch, s);
+    }
+  }
   static const int tbm[3] = {128, 128, 64}, tbn[3] = {128, 64, 64};
   char tag[96];
   snprintf(tag, sizeof(tag), "%s<%s,%d,%d,%s,%s>", d->k % kt == 0 ? "gemm_dma_kernel" : "gemm_kernel",

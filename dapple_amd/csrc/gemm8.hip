@@ -51,6 +51,32 @@ int launch8(GemmArgs a, int batch, hipStream_t stream) {
   return DS_OK;
 }
 
+// The 64x64 block of four waves that split the k-steps of every k-tile (gemm8_core.h): 48 KB of LDS like the 4-wave
+// kernel of gemm.hip, half its fragment reads.
+template <int AMAJ, int BMAJ>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void gemm_ks4_kernel(GemmArgs p) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  ds_wave_prio(p.prio);
+  gemm8_tile<64, 64, 1, 1, 4, 3, AMAJ, BMAJ>(p, lds, blockIdx.x, blockIdx.z);
+}
+
+template <int AMAJ, int BMAJ>
+int launch_ks4(GemmArgs a, int batch, hipStream_t stream) {
+  a.grid_m = (a.m + 63) / 64;
+  a.grid_n = (a.n + 63) / 64;
+  choose_xcd_block(a);
+  dim3 grid(a.grid_m * a.grid_n, 1, batch);
+  constexpr size_t lds = (size_t)3 * (64 + 64) * 128;
+  static std::atomic<bool> attr_set(false);  // two threads may both set the (idempotent) attribute; neither launches before it is set
+  if (!attr_set) {
+    DS_CHECK_HIP(hipFuncSetAttribute((const void*)gemm_ks4_kernel<AMAJ, BMAJ>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_set = true;
+  }
+  hipLaunchKernelGGL((gemm_ks4_kernel<AMAJ, BMAJ>), grid, dim3(256), lds, stream, a);
+  DS_CHECK_LAUNCH();
+  return DS_OK;
+}
+
 template <int AMAJ, int BMAJ>
 int launch8_cfg(const GemmArgs& a, int cfg, int batch, hipStream_t stream) {
   switch (cfg) {
@@ -78,4 +104,14 @@ int ds_gemm8_launch(const GemmArgs& a, int cfg, int a_major, int b_major, int ba
   if (a_major == DS_K_MAJOR && b_major == DS_MN_MAJOR) return launch8_cfg<DS_K_MAJOR, DS_MN_MAJOR>(a, cfg, batch, stream);
   if (a_major == DS_MN_MAJOR && b_major == DS_MN_MAJOR) return launch8_cfg<DS_MN_MAJOR, DS_MN_MAJOR>(a, cfg, batch, stream);
   return launch8_cfg<DS_MN_MAJOR, DS_K_MAJOR>(a, cfg, batch, stream);
+}
+
+int ds_gemm_ks4_launch(const GemmArgs& a, int a_major, int b_major, int batch, hipStream_t stream) {
+  const int nkt = a.k / 64;
+  DS_CHECK_ARG(a.k % 64 == 0 && a.vec_epi && a.splitk == 1 && a.ws_part == nullptr && nkt >= 4 && nkt % 2 == 0 && a.ktiles_per_split == nkt,
+               "ds_gemm_ks4_launch: needs the vector epilogue, no k-slices and an even number (at least 4) of 64-deep k-tiles");
+  if (a_major == DS_K_MAJOR && b_major == DS_K_MAJOR) return launch_ks4<DS_K_MAJOR, DS_K_MAJOR>(a, batch, stream);
+  if (a_major == DS_K_MAJOR && b_major == DS_MN_MAJOR) return launch_ks4<DS_K_MAJOR, DS_MN_MAJOR>(a, batch, stream);
+  if (a_major == DS_MN_MAJOR && b_major == DS_MN_MAJOR) return launch_ks4<DS_MN_MAJOR, DS_MN_MAJOR>(a, batch, stream);
+  return launch_ks4<DS_MN_MAJOR, DS_K_MAJOR>(a, batch, stream);
 }

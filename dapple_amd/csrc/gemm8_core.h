@@ -17,14 +17,21 @@ __device__ __forceinline__ void part_load4(const float* p, f32x4& v) {
   asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(v) : "v"(p) : "memory");
 }
 
-// One output tile of C by one 512-thread workgroup.  `lds` is the workgroup's dynamic LDS (STAGES * (BM + BN) * 128 bytes),
-// bx the workgroup's index among the tiles of the problem (what a launch of its own passes as blockIdx.x), bz its index
-// among batch entries x k-slices (blockIdx.z).  All 512 threads must enter.
+// One output tile of C by one workgroup of WM x WN x WK waves (512 threads; 256 in the 1 x 1 x 4 shape).  `lds` is the
+// workgroup's dynamic LDS (STAGES * (BM + BN) * 128 bytes), bx the workgroup's index among the tiles of the problem (what a
+// launch of its own passes as blockIdx.x), bz its index among batch entries x k-slices (blockIdx.z).  All threads must enter.
+// The 1 x 1 x 4 shape (a 64x64 block of four waves, 3 tile buffers = the 48 KB of the 4-wave kernel of gemm.hip): every
+// wave multiplies the WHOLE 64x64 tile over one of the four 16-deep k-steps of each k-tile, so a fragment is read from LDS
+// once per block instead of twice (16 KB of fragment reads per k-tile instead of 32 - with the 16 KB the tile loads write,
+// the LDS port is what bounds that block); the four partial tiles meet in LDS at the end, every wave summing one 32x32
+// quadrant.  Its k-tile has a single k-step, so the two fragment register sets alternate from k-tile to k-tile (PAR below)
+// and the number of k-tiles must be even.
 template <int BM, int BN, int WM, int WN, int WK, int STAGES, int AMAJ, int BMAJ>
 __device__ __forceinline__ void gemm8_tile(const GemmArgs& p, char* lds, int bx, int bz) {
   typedef bf16 T;
-  typedef AsmDma<T, BM, AMAJ, 8> DA;
-  typedef AsmDma<T, BN, BMAJ, 8> DB;
+  constexpr int NW = WM * WN * WK;                     // waves of the workgroup
+  typedef AsmDma<T, BM, AMAJ, NW> DA;
+  typedef AsmDma<T, BN, BMAJ, NW> DB;
   constexpr int KT = 64;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;  // 32x32 MFMA tiles per wave
   constexpr int KS = 4 / WK;                           // k-steps of a k-tile that one wave multiplies
@@ -33,7 +40,8 @@ __device__ __forceinline__ void gemm8_tile(const GemmArgs& p, char* lds, int bx,
   constexpr int NSLOT = TM * TN;                       // MFMAs per k-step
   constexpr int NMMA = KS * NSLOT;                     // MFMAs per k-tile and wave
   constexpr int NFR = TM + TN;                         // fragments per k-step
-  static_assert(WM * WN * WK == 8 && (WK == 1 || WK == 2), "8 waves");
+  static_assert((NW == 8 && (WK == 1 || WK == 2)) || (NW == 4 && WK == 4 && TM == 2 && TN == 2 && STAGES == 3),
+                "8 waves, or the 64x64 block of four k-step waves");
   static_assert((STAGES - 2) * LPT <= 63, "vmcnt range");
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   // waves w and w + 4 share a SIMD: with WK == 2 they are the two k-halves of one output sub-tile
@@ -109,9 +117,10 @@ __device__ __forceinline__ void gemm8_tile(const GemmArgs& p, char* lds, int bx,
   // tile kt-1+STAGES / kt+STAGES exist (their loads are issued in this k-tile), LATER is the number of tiles issued
   // after tile kt+1 that may still be in flight at the barrier.  No LDS read is in flight at the end (the compiler may
   // copy fragment registers where control flow joins; a copy taken before the data has landed would be stale).
-  auto k_tile = [&](auto rp, auto rc, auto later) {
+  auto k_tile = [&](auto rp, auto rc, auto later, auto par) {
     constexpr bool RP = decltype(rp)::value, RC = decltype(rc)::value;
     constexpr int LATER = decltype(later)::value;
+    constexpr int PAR = decltype(par)::value;   // register set that holds this k-tile's first fragments
     const uint32_t sa = lds0 + buf * STAGE_BYTES, sb = sa + A_BYTES;
     int pb = buf - 1;
     if (pb < 0) pb += STAGES;
@@ -120,7 +129,7 @@ __device__ __forceinline__ void gemm8_tile(const GemmArgs& p, char* lds, int bx,
     const uint32_t prev_tile = lds0 + pb * STAGE_BYTES, next_tile = lds0 + nbuf * STAGE_BYTES;
 #pragma unroll
     for (int ksl = 0; ksl < KS; ++ksl) {
-      const int cur = ksl & 1, nxt = cur ^ 1;
+      const int cur = (ksl + PAR) & 1, nxt = cur ^ 1;
       const bool last = ksl == KS - 1;
 #pragma unroll
       for (int i = 0; i < TM; ++i)
@@ -162,7 +171,7 @@ __device__ __forceinline__ void gemm8_tile(const GemmArgs& p, char* lds, int bx,
           }
           __builtin_amdgcn_sched_barrier(0);
         }
-      if (ksl == KS - 2 && RP) { da.advance(); db.advance(); }
+      if ((KS > 1 && ksl == KS - 2 && RP) || (KS == 1 && RC)) { da.advance(); db.advance(); }
 #pragma unroll
       for (int i = 0; i < TM; ++i) lds_wait(fa[nxt][i]);
 #pragma unroll
@@ -173,19 +182,34 @@ __device__ __forceinline__ void gemm8_tile(const GemmArgs& p, char* lds, int bx,
   // nkt > STAGES (checked on the host): head tile, steady loop, then the last STAGES tiles with compile-time counts
   typedef std::true_type Y;
   typedef std::false_type N;
-  k_tile(N(), Y(), std::integral_constant<int, STAGES - 2>());
-  for (int kt = 1; kt + STAGES < nkt; ++kt) k_tile(Y(), Y(), std::integral_constant<int, STAGES - 2>());
-  k_tile(Y(), N(), std::integral_constant<int, STAGES - 2>());
-  if (STAGES >= 3) k_tile(N(), N(), std::integral_constant<int, (STAGES >= 3 ? STAGES - 3 : 0)>());
-  if (STAGES >= 4) k_tile(N(), N(), std::integral_constant<int, (STAGES >= 4 ? STAGES - 4 : 0)>());
-  k_tile(N(), N(), std::integral_constant<int, 0>());
+  typedef std::integral_constant<int, 0> P0;
+  typedef std::integral_constant<int, 1> P1;
+  if constexpr (KS % 2 == 0) {
+    k_tile(N(), Y(), std::integral_constant<int, STAGES - 2>(), P0());
+    for (int kt = 1; kt + STAGES < nkt; ++kt) k_tile(Y(), Y(), std::integral_constant<int, STAGES - 2>(), P0());
+    k_tile(Y(), N(), std::integral_constant<int, STAGES - 2>(), P0());
+    if (STAGES >= 3) k_tile(N(), N(), std::integral_constant<int, (STAGES >= 3 ? STAGES - 3 : 0)>(), P0());
+    if (STAGES >= 4) k_tile(N(), N(), std::integral_constant<int, (STAGES >= 4 ? STAGES - 4 : 0)>(), P0());
+    k_tile(N(), N(), std::integral_constant<int, 0>(), P0());
+  } else {
+    // one k-step per k-tile: the register sets alternate; nkt is even (checked on the host) and STAGES is 3, so the steady
+    // loop runs an even number of times and the last three tiles start from sets 1, 0, 1
+    k_tile(N(), Y(), std::integral_constant<int, STAGES - 2>(), P0());
+    for (int kt = 1; kt + STAGES < nkt; kt += 2) {
+      k_tile(Y(), Y(), std::integral_constant<int, STAGES - 2>(), P1());
+      k_tile(Y(), Y(), std::integral_constant<int, STAGES - 2>(), P0());
+    }
+    k_tile(Y(), N(), std::integral_constant<int, STAGES - 2>(), P1());
+    k_tile(N(), N(), std::integral_constant<int, (STAGES >= 3 ? STAGES - 3 : 0)>(), P0());
+    k_tile(N(), N(), std::integral_constant<int, 0>(), P1());
+  }
 
   // With WK == 2 the two waves of a SIMD hold the two k-halves of one sub-tile: the upper half parks its accumulators in
   // LDS as they lie in the registers (16 bytes per lane and store: no bank conflicts), the lower half adds them and
   // carries the sub-tile from here on.
   constexpr int WAVE_ACC = TM * TN * 1024;  // floats of one wave's accumulators
   if (WK == 2) {
-    static_assert(WK == 1 || 4 * WAVE_ACC * 4 <= STAGES * STAGE_BYTES, "pair merge fits the tile ring");
+    static_assert(WK != 2 || 4 * WAVE_ACC * 4 <= STAGES * STAGE_BYTES, "pair merge fits the tile ring");
     float* park = reinterpret_cast<float*>(lds) + wq * WAVE_ACC;
     __syncthreads();  // every wave is out of the k loop
     if (wk == 1) {
@@ -274,37 +298,79 @@ __device__ __forceinline__ void gemm8_tile(const GemmArgs& p, char* lds, int bx,
     }
   }
 
+  // With WK == 4 every wave holds a partial sum of the whole 64x64 tile: each parks the three 32x32 quadrants that are
+  // not its own (as they lie in the registers; 4 x 12 KB = the tile ring), then adds to its own quadrant the three
+  // copies of it, in the order of the waves that wrote them, and carries that quadrant through the epilogue as wave
+  // (wave / 2, wave % 2) of a 2 x 2 grid.
+  if constexpr (WK == 4) {
+    static_assert(WK != 4 || 4 * 3 * 4096 <= STAGES * STAGE_BYTES, "quadrant merge fits the tile ring");
+    // copy s (0..2) of quadrant q: 4 KB at lds + (q * 3 + s) * 4096, piece g of lane l at ((g * 64) + l) * 16
+    auto park = [&](const f32x16& a, int q, int sl) {
+      char* dst = lds + (q * 3 + sl) * 4096;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 v = {a[4 * g], a[4 * g + 1], a[4 * g + 2], a[4 * g + 3]};
+        *reinterpret_cast<f32x4*>(dst + (g * 64 + lane) * 16) = v;
+      }
+    };
+    auto gather = [&](f32x16& a, int q) {
+#pragma unroll
+      for (int sl = 0; sl < 3; ++sl)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const f32x4 v = *reinterpret_cast<const f32x4*>(lds + (q * 3 + sl) * 4096 + (g * 64 + lane) * 16);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) a[4 * g + e] += v[e];
+        }
+    };
+    __syncthreads();  // every wave is out of the k loop
+    // wave w is copy (w < q ? w : w - 1) of quadrant q != w
+    if (wk == 0) { park(acc[0][1], 1, 0); park(acc[1][0], 2, 0); park(acc[1][1], 3, 0); }
+    else if (wk == 1) { park(acc[0][0], 0, 0); park(acc[1][0], 2, 1); park(acc[1][1], 3, 1); }
+    else if (wk == 2) { park(acc[0][0], 0, 1); park(acc[0][1], 1, 1); park(acc[1][1], 3, 2); }
+    else { park(acc[0][0], 0, 2); park(acc[0][1], 1, 2); park(acc[1][0], 2, 2); }
+    __syncthreads();
+    if (wk == 1) acc[0][0] = acc[0][1];
+    else if (wk == 2) acc[0][0] = acc[1][0];
+    else if (wk == 3) acc[0][0] = acc[1][1];
+    gather(acc[0][0], wk);
+  }
+  // the wave grid and the sub-tiles per wave as the epilogue sees them
+  constexpr int EWM = WK == 4 ? 2 : WM, EWN = WK == 4 ? 2 : WN, ETM = WK == 4 ? 1 : TM, ETN = WK == 4 ? 1 : TN;
+  const int ewm = WK == 4 ? (wk >> 1) : wm, ewn = WK == 4 ? (wk & 1) : wn;
+  const bool carries = WK == 4 || wk == 0;
+
   // Epilogue through LDS, one 32-row MFMA block of every wave at a time: the waves that carry the sub-tiles park
   // alpha * acc + bias as fp32 rows, then every thread streams 8 consecutive columns of a row, so that residual /
   // auxiliary reads and C writes are 16-byte vectors covering whole rows of the tile.
   constexpr int LDW = BN + 4;
-  constexpr int SLAB_ROWS = WM * 32;
+  constexpr int SLAB_ROWS = EWM * 32;
   constexpr int VPR = BN / 8;
   constexpr int VECS = SLAB_ROWS * VPR;
   static_assert(SLAB_ROWS * LDW * 4 <= STAGES * STAGE_BYTES, "staging slab fits the tile ring");
   float* sc = reinterpret_cast<float*>(lds);
   const int flags = p.flags;
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
+  for (int i = 0; i < ETM; ++i) {
     __syncthreads();
-    if (wk == 0) {
+    if (carries) {
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int cl = wn * (BN / WN) + j * 32 + (lane & 31);
+      for (int j = 0; j < ETN; ++j) {
+        const int cl = ewn * (BN / EWN) + j * 32 + (lane & 31);
         const int col = n0 + cl;
         const float bias = ((flags & DS_EPI_BIAS) && col < p.n) ? p.bias[col] : 0.f;
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-          const int rs = wm * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+          const int rs = ewm * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
           sc[rs * LDW + cl] = acc[i][j][e] * p.alpha + bias;
         }
       }
     }
     __syncthreads();
 #pragma unroll 2
-    for (int v = tid; v < VECS; v += 512) {
+    for (int v = tid; v < VECS; v += 64 * NW) {
       const int rs = v / VPR, cl = (v % VPR) * 8;
-      const int row = m0 + (rs >> 5) * (BM / WM) + i * 32 + (rs & 31), col = n0 + cl;
+      const int row = m0 + (rs >> 5) * (BM / EWM) + i * 32 + (rs & 31), col = n0 + cl;
       if (row >= p.m || col >= p.n) continue;
       float x[8];
       const f32x4 lo = *reinterpret_cast<const f32x4*>(sc + rs * LDW + cl);

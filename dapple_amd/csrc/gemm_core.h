@@ -436,3 +436,6 @@ int ds_gemm8_stages(int cfg);
 // epilogue, vec_epi, wave priority); tiling, slicing and workspace fields are the caller's.
 int ds_gemm_make_args(const ds_gemm_desc* d, dsgemm::GemmArgs* out, int* batch_out);
 int ds_gemm8_launch(const dsgemm::GemmArgs& a, int cfg, int a_major, int b_major, int batch, hipStream_t stream);
+// The 64x64 block whose four waves split the k-steps of every k-tile (gemm8.hip): bf16, vector epilogue, no k-slices, an
+// even number (at least 4) of 64-deep k-tiles.
+int ds_gemm_ks4_launch(const dsgemm::GemmArgs& a, int a_major, int b_major, int batch, hipStream_t stream);

@@ -21,9 +21,9 @@ def test_traffic_rows_parse_and_cover_the_layer():
         acc = "C +=" in name
         assert alg == 2 * (m * k + n * k) + (8 if acc else 2) * m * n
         assert wr >= (4 if acc else 2) * m * n and rd >= 2 * (m * k + n * k)      # nothing moves less than the operands once
-    dom = bench.traffic_of("gemm_dma_kernel<bf16,64,64,K,K>", "bert48_half", 4)
+    dom = bench.traffic_of("gemm_ks4_kernel<bf16,64,64,K,K>", "bert48_half", 4)
     assert dom is not None and 30e6 < dom < 45e6
-    assert bench.traffic_of("gemm_dma_kernel<bf16,64,64,K,K>", "xlnet36_half", 4) is None
+    assert bench.traffic_of("gemm_ks4_kernel<bf16,64,64,K,K>", "xlnet36_half", 4) is None
     assert bench.traffic_of("gemm8_kernel<bf16,128,128,MN,MN>", "bert48_half", 3) is None   # grouping without a counter run
 
 

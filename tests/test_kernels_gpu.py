@@ -10,7 +10,7 @@ import pytest
 import torch
 
 from dapple_amd import ops
-from dapple_amd._lib import (DS_EPI_ACCUM, DS_EPI_BIAS, DS_EPI_DGELU, DS_EPI_GELU, DS_EPI_OUT_F32, DS_EPI_RELU,
+from dapple_amd._lib import (DS_EPI_ACCUM, DS_EPI_BIAS, DS_EPI_DGELU, DS_EPI_GELU, DS_EPI_OUT_F32, DS_EPI_RELU, DS_EPI_RESIDUAL_F32,
                              DS_EPI_RESIDUAL, DS_K_MAJOR, DS_MN_MAJOR)
 from oracle import bert as ob
 from util import assert_close, dev, rel_err
@@ -99,6 +99,40 @@ def test_gemm_wide_blocks(am, bm, m, n, k):
     acc = acc0.clone()
     ops.gemm(a, b, acc, m, n, k, am, bm, flags=DS_EPI_ACCUM)
     assert_close(acc, (acc0 + Ar @ Br.T).cpu().double(), 1e-5, "gemm accumulate, wide blocks")
+
+
+@pytest.mark.parametrize("am,bm,m,n,k", [
+    (DS_K_MAJOR, DS_K_MAJOR, 1024, 1024, 4096),     # the BERT-48 layer's narrow input gradients
+    (DS_K_MAJOR, DS_MN_MAJOR, 1024, 1024, 1024),    # its attention output projection
+    (DS_K_MAJOR, DS_K_MAJOR, 200, 328, 2048),       # ragged edge tiles
+    (DS_MN_MAJOR, DS_MN_MAJOR, 320, 192, 1152),     # 18 k-tiles
+    (DS_MN_MAJOR, DS_K_MAJOR, 64, 64, 1024),        # one block
+    (DS_K_MAJOR, DS_MN_MAJOR, 448, 1024, 3072),
+])
+def test_gemm_blocks_whose_waves_split_the_k_steps(am, bm, m, n, k):
+    """64x64 blocks under a reduction of at least 16 (an even number of) k-tiles: each of the four waves multiplies the whole
+    tile over one 16-deep k-step of every k-tile and the partial tiles meet in LDS.  All operand-major pairs, ragged edges,
+    the vector epilogue's terms and the fp32 accumulate."""
+    r = rng(m * 3 + n * 5 + k * 7 + am * 2 + bm)
+    A = (r.standard_normal((m, k)) * 0.5).astype(np.float32)
+    B = (r.standard_normal((n, k)) * 0.5).astype(np.float32)
+    a = dev(A if am == DS_K_MAJOR else A.T, torch.bfloat16)
+    b = dev(B if bm == DS_K_MAJOR else B.T, torch.bfloat16)
+    bias = dev(r.standard_normal(n), torch.float32)
+    res = dev(r.standard_normal((m, n)), torch.float32)
+    Ar = (a if am == DS_K_MAJOR else a.T).float().cpu().double()
+    Br = (b if bm == DS_K_MAJOR else b.T).float().cpu().double()
+    prod = Ar @ Br.T
+    c = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    ops.gemm(a, b, c, m, n, k, am, bm, flags=DS_EPI_BIAS, bias=bias, alpha=0.125)
+    assert_close(c, 0.125 * prod + bias.cpu().double(), TOL["bf16"], "gemm, k-step waves, bf16 output")
+    c32 = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda")
+    ops.gemm(a, b, c32, m, n, k, am, bm, flags=DS_EPI_OUT_F32 | DS_EPI_RESIDUAL | DS_EPI_RESIDUAL_F32, residual=res)
+    assert_close(c32, prod + res.cpu().double(), 1e-5, "gemm, k-step waves, fp32 output + fp32 residual")
+    acc0 = dev(r.standard_normal((m, n)), torch.float32)
+    acc = acc0.clone()
+    ops.gemm(a, b, acc, m, n, k, am, bm, flags=DS_EPI_ACCUM)
+    assert_close(acc, acc0.cpu().double() + prod, 1e-5, "gemm accumulate, k-step waves")
 
 
 @pytest.mark.parametrize("dt,m,n,kseg,nseg,agap,bgap", [
@@ -433,6 +467,28 @@ def test_fused_attention_fwd_bwd(B, N, S, use_mask, spread):
     dqkv = ops.attention_bwd(qkv, ctx, lse, dctx, B, N, S, scale, mask)
     for i, name in enumerate(("dq", "dk", "dv")):
         assert_close(dqkv[:, i * H:(i + 1) * H], dx[:, i * H:(i + 1) * H], 2e-2, "fused attention " + name)
+
+
+def test_fused_attention_with_a_negative_scale():
+    """The mask-free short form of the steps takes the maximum of the raw scores, which is the maximum of the scaled ones
+    only for a positive scale: any other scale must take the general form and still be right."""
+    B, N, S, D = 1, 2, 128, 64
+    H = N * D
+    r = rng(17)
+    qkv = dev(r.standard_normal((B * S, 3 * H)) * 0.7, torch.bfloat16)
+    dctx = dev(r.standard_normal((B * S, H)), torch.bfloat16)
+    scale = -0.2
+    ctx, lse = ops.attention_fwd(qkv, B, N, S, scale)
+    x = qkv.cpu().double().requires_grad_(True)
+    q, k, v = (x[:, i * H:(i + 1) * H].reshape(B, S, N, D).permute(0, 2, 1, 3) for i in range(3))
+    sc = q @ k.transpose(-1, -2) * scale
+    ref = (torch.softmax(sc, -1) @ v).permute(0, 2, 1, 3).reshape(B * S, H)
+    assert_close(ctx, ref, 1e-2, "fused attention fwd, negative scale")
+    assert_close(lse, torch.logsumexp(sc, -1), 1e-3, "logsumexp, negative scale")
+    (dx,) = torch.autograd.grad(ref, x, dctx.cpu().double())
+    dqkv = ops.attention_bwd(qkv, ctx, lse, dctx, B, N, S, scale)
+    for i, name in enumerate(("dq", "dk", "dv")):
+        assert_close(dqkv[:, i * H:(i + 1) * H], dx[:, i * H:(i + 1) * H], 2e-2, "fused attention %s, negative scale" % name)
 
 
 def test_fused_attention_backward_with_keys_that_share_a_common_part():
