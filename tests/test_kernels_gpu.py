@@ -138,6 +138,7 @@ def test_gemm_blocks_whose_waves_split_the_k_steps(am, bm, m, n, k):
 @pytest.mark.parametrize("dt,m,n,kseg,nseg,agap,bgap", [
     ("bf16", 1024, 2048, 512, 4, 3, 0),      # 8-wave tiles; A's segments 3 rows apart beyond their length, B's back to back
     ("bf16", 256, 192, 128, 3, 0, 5),        # 4-wave tiles
+    ("bf16", 256, 192, 256, 4, 2, 1),        # 16 k-tiles under 64x64 blocks: the waves split the k-steps
     ("bf16", 4096, 1024, 1024, 8, 2, 1),     # a weight gradient over 8 micro-batches
     ("bf16", 1024, 1024, 1408, 2, -1, 0),    # A's segment stride 0: both segments read the same rows
     ("fp32", 512, 256, 96, 5, 1, 2),
