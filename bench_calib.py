@@ -26,6 +26,10 @@ algorithmic bytes and FLOP printed.
 of micro-batch j+1, an input-gradient product of micro-batch j, a weight-gradient product over four micro-batches), timed
 three ways - back to back on one stream, side by side on two / three streams, and as ONE ``ds_gemm_grouped`` launch per
 tile-shape choice.
+
+``timeline [workload]``: where a step of ``bench.py``'s workload (default bert48_half) spends its time - the moment every
+backward pass's chain of kernels ends (an event on a probe stream behind ``ds_stage_wait_backward``), the distance from
+one to the next and what is left after the last; three steps, no profiler.
 """
 import time
 import sys
@@ -291,8 +295,52 @@ def elementwise():
     print("cast_kernel<bf16,float>     %d elements: %d bytes per launch (read fp32, write bf16)" % (h * f, 6 * h * f))
 
 
+def timeline(workload):
+    import types
+    import bench
+    from dapple_amd import synthetic
+    args = types.SimpleNamespace(wgrad_group=8, bf16_residual_stream=False, pair_passes=False, xlnet_attention="auto")
+    c = dict(synthetic.CONFIGS[workload])
+    wl = bench.MAKERS[c["kind"]](c, args)
+    stage = wl.stage
+    if stage.overlap_supported():
+        stage.enable_overlap()
+    for _ in range(3):
+        wl.step()
+    torch.cuda.synchronize()
+    probe = torch.cuda.Stream()
+    plain_backward = stage.backward
+    marks = []
+
+    def backward(slot, d_out, d_in=None, ready=False):
+        plain_backward(slot, d_out, d_in, ready=ready)
+        stage.wait_backward(slot, probe)
+        e = torch.cuda.Event(enable_timing=True)
+        e.record(probe)
+        marks.append(e)
+    stage.backward = backward
+    for _ in range(3):
+        marks.clear()
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        t0 = time.perf_counter()
+        wl.step()
+        e1 = torch.cuda.Event(enable_timing=True)
+        e1.record()
+        host = time.perf_counter() - t0
+        torch.cuda.synchronize()
+        tot = e0.elapsed_time(e1)
+        ts = [e0.elapsed_time(e) for e in marks]
+        print("%s: step %.2f ms (the host queued it in %.2f ms); backward chains end at %s ms" % (workload, tot, host * 1e3, " ".join("%.2f" % t for t in ts)))
+        print("   from one chain's end to the next: %s ms; after the last chain: %.2f ms"
+              % (" ".join("%.2f" % (b - a) for a, b in zip([0.0] + ts[:-1], ts)), tot - ts[-1]))
+
+
 if __name__ == "__main__":
-    if len(sys.argv) > 1 and sys.argv[1] == "gemms":
+    if len(sys.argv) > 1 and sys.argv[1] == "timeline":
+        timeline(sys.argv[2] if len(sys.argv) > 2 else "bert48_half")
+    elif len(sys.argv) > 1 and sys.argv[1] == "gemms":
         gemms()
     elif len(sys.argv) > 1 and sys.argv[1] == "elementwise":
         elementwise()
