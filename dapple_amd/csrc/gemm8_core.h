@@ -26,7 +26,10 @@ __device__ __forceinline__ void part_load4(const float* p, f32x4& v) {
 // the LDS port is what bounds that block); the four partial tiles meet in LDS at the end, every wave summing one 32x32
 // quadrant.  Its k-tile has a single k-step, so the two fragment register sets alternate from k-tile to k-tile (PAR below)
 // and the number of k-tiles must be even.
-template <int BM, int BN, int WM, int WN, int WK, int STAGES, int AMAJ, int BMAJ>
+// COLSUM: the workgroups of the first tile row also sum the B operand over k (GemmArgs::colsum) - one more MFMA per B
+// fragment with an A operand of ones, by the waves that hold the tile's first rows: all 32 rows of the result are the
+// column sums of the 16 x 32 fragment.
+template <int BM, int BN, int WM, int WN, int WK, int STAGES, int AMAJ, int BMAJ, bool COLSUM = false>
 __device__ __forceinline__ void gemm8_tile(const GemmArgs& p, char* lds, int bx, int bz) {
   typedef bf16 T;
   constexpr int NW = WM * WN * WK;                     // waves of the workgroup
@@ -69,6 +72,19 @@ __device__ __forceinline__ void gemm8_tile(const GemmArgs& p, char* lds, int bx,
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  static_assert(!COLSUM || (WK == 2 && NW == 8), "column sums: the 2 x 2 x 2 shapes");
+  const bool cs_wave = COLSUM && tile_m == 0 && wm == 0;   // wave-uniform
+  f32x16 cs[COLSUM ? TN : 1];
+  bf16x8 ones;
+  if (COLSUM) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) cs[j][e] = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ones[e] = (bf16)1.0f;
+  }
 
   DA da;
   DB db;
@@ -137,6 +153,9 @@ __device__ __forceinline__ void gemm8_tile(const GemmArgs& p, char* lds, int bx,
         for (int j = 0; j < TN; ++j) {
           const int slot = i * TN + j;
           Mma<T>::mma(acc[i][j], to_frag(fa[cur][i]), to_frag(fb[cur][j]));
+          if (COLSUM && i == 0) {
+            if (cs_wave) Mma<T>::mma(cs[COLSUM ? j : 0], ones, to_frag(fb[cur][j]));
+          }
           __builtin_amdgcn_sched_barrier(0);
           if (last && slot == 0) {
             __builtin_amdgcn_s_waitcnt(DS_VMCNT(LPT * LATER));
@@ -235,6 +254,31 @@ __device__ __forceinline__ void gemm8_tile(const GemmArgs& p, char* lds, int bx,
 #pragma unroll
             for (int e = 0; e < 4; ++e) acc[i][j][4 * g + e] += v[e];
           }
+    }
+  }
+
+  if constexpr (COLSUM) {
+    // the two k-halves of the column sums meet like the accumulators above (one more round through the same LDS), then
+    // lane n of the lower half adds column n of each of its 32-column blocks - row 0 of the result, like every row
+    float* parkc = reinterpret_cast<float*>(lds) + wn * (TN * 1024);
+    __syncthreads();
+    if (cs_wave && wk == 1) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const f32x4 v = {cs[j][4 * g], cs[j][4 * g + 1], cs[j][4 * g + 2], cs[j][4 * g + 3]};
+          *reinterpret_cast<f32x4*>(parkc + ((j * 4 + g) * 64 + lane) * 4) = v;
+        }
+    }
+    __syncthreads();
+    if (cs_wave && wk == 0 && lane < 32) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int col = n0 + wn * (BN / WN) + j * 32 + lane;
+        const float other = parkc[(j * 4 * 64 + lane) * 4];   // element 0 of piece 0: row 0 of the upper half's sums
+        if (col < p.n) p.colsum[zi * p.colsum_si + col] += cs[j][0] + other;
+      }
     }
   }
 

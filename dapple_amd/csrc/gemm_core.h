@@ -53,6 +53,10 @@ struct GemmArgs {
   int64_t a_seg, b_seg;
   float* rowdot;               // DS_EPI_ROWDOT (grouped launches only): see gemm_epilogue_vec8
   int rowdot_seq;
+  // Column sums of the B operand beside the product (grouped launches, 256x128 tiles): colsum[zi * colsum_si + col] +=
+  // sum_k B(col, k) - with B = dY of a weight gradient X^T dY that is the gradient of the layer's bias.  null: none.
+  float* colsum;
+  int64_t colsum_si;
 };
 
 // Internal epilogue flag: besides C, write for every row and every block of 64 columns the dot product of the bf16 values

@@ -25,6 +25,10 @@ struct GroupOp {
   // of a column block of bf16(C[row][col]) * c2[row][col] (c2 bf16, layout of C; no other epilogue that reads c2)
   float* rowdot = nullptr;
   int rowdot_seq = 0;
+  // with colsum (256x128 tiles, operand majors (MN, MN), batch == batch_inner): colsum[z * colsum_stride + col] += sum over
+  // k of B(col, k) for batch entry z - the bias gradient beside the weight gradient X^T dY that reads the same dY
+  float* colsum = nullptr;
+  int64_t colsum_stride = 0;
   // GOP_ATTN_*: arguments of ds_attention_fwd / ds_attention_bwd (bf16, head size 64)
   int B = 0, N = 0, S = 0;
   const void* qkv = nullptr;
@@ -53,7 +57,7 @@ struct GroupOp {
   GroupOp() { memset(&gemm, 0, sizeof(gemm)); }
 };
 
-constexpr int DS_GROUP_MAX_TASKS = 12;  // (288 bytes of kernel arguments each, 4 KB in all)
+constexpr int DS_GROUP_MAX_TASKS = 12;  // (304 bytes of kernel arguments each, 4 KB in all)
 // All tasks as one launch; workgroups start in list order.
 int ds_group_launch(const GroupOp* ops, int n, hipStream_t stream);
 // The tile shape ds_group_launch picks for a GEMM when GroupOp::cfg < 0.

@@ -71,7 +71,10 @@ constexpr TileCfg tile_cfg(int cfg) {
 template <int CFG, int AMAJ, int BMAJ>
 __device__ __forceinline__ void run_tile(const GemmArgs& g, char* lds, int bx, int bz) {
   if (CFG == 0) gemm8_tile<256, 256, 2, 4, 1, 2, AMAJ, BMAJ>(g, lds, bx, bz);
-  else if (CFG == 1) gemm8_tile<256, 128, 2, 2, 2, 3, AMAJ, BMAJ>(g, lds, bx, bz);
+  else if (CFG == 1) {
+    if (AMAJ == DS_MN_MAJOR && BMAJ == DS_MN_MAJOR && g.colsum != nullptr) gemm8_tile<256, 128, 2, 2, 2, 3, AMAJ, BMAJ, true>(g, lds, bx, bz);
+    else gemm8_tile<256, 128, 2, 2, 2, 3, AMAJ, BMAJ>(g, lds, bx, bz);
+  }
   else if (CFG == 2) gemm8_tile<128, 128, 2, 2, 2, 3, AMAJ, BMAJ>(g, lds, bx, bz);
   else if (CFG == 3) gemm8_tile<128, 64, 2, 2, 2, 4, AMAJ, BMAJ>(g, lds, bx, bz);
   else if (CFG == 4) gemm8_tile<128, 128, 2, 2, 2, 2, AMAJ, BMAJ>(g, lds, bx, bz);
@@ -243,6 +246,12 @@ int ds_group_launch(const GroupOp* ops, int n, hipStream_t stream) {
         t.g.flags |= DS_EPI_ROWDOT;
         t.g.rowdot = op.rowdot;
         t.g.rowdot_seq = op.rowdot_seq;
+      }
+      if (op.colsum) {
+        DS_CHECK_ARG(cfg == 1 && wgrad && (batch == 1 || batch == (d->batch_inner > 0 ? d->batch_inner : 1)) && ds_aligned16(op.colsum),
+                     "ds_group_launch: task %d: column sums need 256x128 tiles, operand majors (MN, MN) and a batch that is all inner", i);
+        t.g.colsum = op.colsum;
+        t.g.colsum_si = op.colsum_stride;
       }
       t.role = GROUP_ROLE(cfg, d->a_major, d->b_major);
       t.per_z = t.g.grid_m * t.g.grid_n;

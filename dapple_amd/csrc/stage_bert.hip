@@ -1103,13 +1103,23 @@ struct BertStage : ds_stage {
       ds_gemm_desc& d = ops[3].gemm;
       d = desc_wgrad(m, H, H, x, H, dqkv, 3 * H, g[b + W_Q], H);
       d.batch = 3; d.batch_inner = 3; d.b_stride_inner = H; d.c_stride_inner = (int64_t)H * H;
+      // the two bias gradients that are column sums of a GEMM's dY operand come out of that GEMM (256x128 tiles only)
+      static const char* env_cs = getenv("DS_BERT_GROUP_COLSUM");
+      const bool fused_colsum = group_cfg == 1 && !(env_cs && atoi(env_cs) == 0);
+      if (fused_colsum) {
+        ops[1].colsum = g[b + B_FF1];
+        ops[3].colsum = g[b + B_Q];
+        ops[3].colsum_stride = H;
+      }
       for (GroupOp& o : ops) { o.kind = GOP_GEMM; o.cfg = group_cfg; o.prio = 0; wg_pending.push_back(o); }
       static const char* env_gl = getenv("DS_BERT_GROUP_LAYERS");
       // (per-pass weight gradients hand their operand buffers back layer by layer: nothing is held over)
       const size_t per_launch = G > 1 && !(env_gl && atoi(env_gl) == 1) ? 8 : 4;
       if (wg_pending.size() >= per_launch) DS_PROPAGATE(launch_pending_wgrads());
-      DS_PROPAGATE(ds_colsum_accum(dtype, m, F, du, F, g[b + B_FF1], stream));
-      DS_PROPAGATE(ds_colsum_accum(dtype, m, 3 * H, dqkv, 3 * H, g[b + B_Q], stream));
+      if (!fused_colsum) {
+        DS_PROPAGATE(ds_colsum_accum(dtype, m, F, du, F, g[b + B_FF1], stream));
+        DS_PROPAGATE(ds_colsum_accum(dtype, m, 3 * H, dqkv, 3 * H, g[b + B_Q], stream));
+      }
       return DS_OK;
     }
     DS_PROPAGATE(gemm_wgrad(m, H, F, h, F, dz2, H, g[b + W_FF2], H));

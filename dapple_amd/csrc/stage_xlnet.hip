@@ -824,19 +824,24 @@ struct XlnetStage : ds_stage {
         for (int j = 0; j < 2; ++j)
           wg(H, H, krows, sp0 + t.mem, H, sstride, dkv + (size_t)j * H * esz, 3 * H, qkv_seg, g[b + X_K + j], H);
       }
+      bool b1_fused = false;   // the first FFN bias gradient = column sums of du, the dY operand of W1's product
       for (int i = 0; i < nd; ++i) {
         // (one launch never carries two products into the same master gradient: runs of one layer are flushed apart)
         const bool grouped = ds[i].k / 64 > 3 && ds[i].m >= 128 && ds[i].n >= 128;
         if (grouped) {
           GroupOp o;
           o.kind = GOP_GEMM; o.gemm = ds[i]; o.cfg = ds[i].m >= 256 ? 1 : 2; o.prio = 0;
+          if (i == 1 && o.cfg == 1) {
+            o.colsum = g[b + X_B1];
+            b1_fused = true;
+          }
           wg_pending.push_back(o);
         } else {
           DS_PROPAGATE(ds_gemm(&ds[i], stream));
         }
       }
       if (runs.size() > 1 || wg_pending.size() + nd > (size_t)DS_GROUP_MAX_TASKS) DS_PROPAGATE(launch_pending_wgrads());
-      DS_PROPAGATE(ds_colsum_accum(dtype, rows * r.n, F, du, F, g[b + X_B1], stream));
+      if (!b1_fused) DS_PROPAGATE(ds_colsum_accum(dtype, rows * r.n, F, du, F, g[b + X_B1], stream));
       if (rs32) {
         const size_t a32 = (size_t)rows * H * 4, r8 = (size_t)rows * 8;
         const int64_t s4 = (int64_t)(slot_bytes / 4);
