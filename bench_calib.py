@@ -319,8 +319,19 @@ def timeline(workload):
         e.record(probe)
         marks.append(e)
     stage.backward = backward
+    plain_forward = stage.forward
+    fmarks = []
+
+    def forward(*a, **k):
+        r = plain_forward(*a, **k)
+        e = torch.cuda.Event(enable_timing=True)
+        e.record()     # the forward passes run on the stream the step is queued on
+        fmarks.append(e)
+        return r
+    stage.forward = forward
     for _ in range(3):
         marks.clear()
+        fmarks.clear()
         torch.cuda.synchronize()
         e0 = torch.cuda.Event(enable_timing=True)
         e0.record()
@@ -333,6 +344,7 @@ def timeline(workload):
         tot = e0.elapsed_time(e1)
         ts = [e0.elapsed_time(e) for e in marks]
         print("%s: step %.2f ms (the host queued it in %.2f ms); backward chains end at %s ms" % (workload, tot, host * 1e3, " ".join("%.2f" % t for t in ts)))
+        print("   forward passes end at %s ms" % " ".join("%.2f" % e0.elapsed_time(e) for e in fmarks))
         print("   from one chain's end to the next: %s ms; after the last chain: %.2f ms"
               % (" ".join("%.2f" % (b - a) for a, b in zip([0.0] + ts[:-1], ts)), tot - ts[-1]))
 
