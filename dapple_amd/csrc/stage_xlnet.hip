@@ -1017,7 +1017,13 @@ struct XlnetStage : ds_stage {
         if (grouped) {
           GroupOp ops[4];
           ops[0].gemm = d_dqr; ops[1].gemm = d_dqw; ops[2].gemm = d_dk; ops[3].gemm = d_dv;
-          for (GroupOp& o : ops) { o.kind = GOP_GEMM; o.cfg = 3; o.prio = ds_launch_prio; }
+          // 128x64 tiles with two buffers (48 KB: three workgroups per CU, or room beside the forward pass's blocks) - these
+          // products stream 130 MB of score gradients for 7.5 GFLOP, so what counts is loads in flight per CU, not the
+          // depth of one block's ring (measured on the XLNet-36 half-stage: 42.27 ms per step against 42.96 with four
+          // buffers, 43.7 / 44.3 with 128x128 tiles of three / two buffers).  DS_XL_PRODUCTS_CFG = 2..5 forces a shape.
+          static const char* env_pc = getenv("DS_XL_PRODUCTS_CFG");
+          const int pcfg = env_pc ? atoi(env_pc) : 5;
+          for (GroupOp& o : ops) { o.kind = GOP_GEMM; o.cfg = pcfg; o.prio = ds_launch_prio; }
           DS_PROPAGATE(ds_group_launch(ops, 4, stream));
         } else {
           DS_PROPAGATE(ds_gemm(&d_dqw, stream));
